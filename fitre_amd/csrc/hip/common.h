@@ -1,0 +1,161 @@
+// Shared plumbing of the gfx950 device layer: status reporting, the launch
+// stream, per-class launch accounting, wave64 reductions and fast division.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include "fitre_hip.h"
+
+namespace fitre {
+
+constexpr int kWave = 64;
+
+// ---- status -------------------------------------------------------------
+void set_error(const char *fmt, ...);
+int fail(int code, const char *fmt, ...);
+hipStream_t stream();
+bool ready();
+
+#define FITRE_HIP_TRY(expr)                                                                          \
+	do {                                                                                             \
+		hipError_t e_ = (expr);                                                                      \
+		if (e_ != hipSuccess)                                                                        \
+			return ::fitre::fail(FITRE_E_DEVICE, "%s failed at %s:%d: %s", #expr, __FILE__,          \
+			                     __LINE__, hipGetErrorString(e_));                                   \
+	} while (0)
+
+#define FITRE_REQUIRE(cond, ...)                                                                     \
+	do {                                                                                             \
+		if (!(cond)) return ::fitre::fail(FITRE_E_ARGUMENT, __VA_ARGS__);                            \
+	} while (0)
+
+#define FITRE_NEED_INIT()                                                                            \
+	do {                                                                                             \
+		if (!::fitre::ready())                                                                       \
+			return ::fitre::fail(FITRE_E_DEVICE, "%s: fitre_hip_init has not been called", __func__); \
+	} while (0)
+
+// ---- per-class launch accounting ------------------------------------------
+// A LaunchScope brackets the launches made while it is alive with two events
+// when accounting is on; otherwise it costs one branch.
+struct LaunchScope {
+	LaunchScope(int kernelClass, double work);
+	~LaunchScope();
+	int slot;
+};
+
+int check_launch(const char *what);
+
+// ---- integer division by a run-time constant ------------------------------
+// q = n / d for 0 <= n < 2^31 via one 32x32->64 multiply.
+struct FastDiv {
+	uint32_t mul;
+	uint32_t shift;
+	uint32_t div;
+	__host__ __device__ FastDiv() : mul(0), shift(0), div(1) {}
+	__host__ __device__ explicit FastDiv(uint32_t d) : div(d)
+	{
+		if (d == 1) {
+			mul = 0;
+			shift = 0;
+			return;
+		}
+		uint32_t l = 0;
+		while ((1ull << l) < d) l++;
+		shift = l;
+		mul = (uint32_t)(((1ull << 32) * ((1ull << l) - d)) / d + 1);
+	}
+	__device__ __forceinline__ uint32_t quot(uint32_t n) const
+	{
+		if (div == 1) return n;
+		uint32_t t = __umulhi(n, mul);
+		return (t + ((n - t) >> 1)) >> (shift - 1);
+	}
+	__device__ __forceinline__ void divmod(uint32_t n, uint32_t &q, uint32_t &r) const
+	{
+		q = quot(n);
+		r = n - q * div;
+	}
+};
+
+// ---- wave64 reductions ------------------------------------------------------
+// Butterfly over the 64 lanes: DPP inside a row of 16 lanes, ds_swizzle across
+// rows of a 32-lane half, one bpermute across halves.  Every lane ends with
+// the total.
+__device__ __forceinline__ int dpp_quad_xor1(int v) { return __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xf, 0xf, false); }
+__device__ __forceinline__ int dpp_quad_xor2(int v) { return __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xf, 0xf, false); }
+__device__ __forceinline__ int dpp_half_mirror(int v) { return __builtin_amdgcn_update_dpp(0, v, 0x141, 0xf, 0xf, false); }
+__device__ __forceinline__ int dpp_row_mirror(int v) { return __builtin_amdgcn_update_dpp(0, v, 0x140, 0xf, 0xf, false); }
+__device__ __forceinline__ int swz_xor16(int v) { return __builtin_amdgcn_ds_swizzle(v, 0x401F); }
+__device__ __forceinline__ int xor32(int v) { return __shfl_xor(v, 32, 64); }
+
+template <typename F>
+__device__ __forceinline__ float wave_shuffle_f(float v, F f)
+{
+	return __int_as_float(f(__float_as_int(v)));
+}
+template <typename F>
+__device__ __forceinline__ double wave_shuffle_d(double v, F f)
+{
+	int lo = __double2loint(v), hi = __double2hiint(v);
+	return __hiloint2double(f(hi), f(lo));
+}
+
+__device__ __forceinline__ float wave_sum(float v)
+{
+	v += wave_shuffle_f(v, dpp_quad_xor1);
+	v += wave_shuffle_f(v, dpp_quad_xor2);
+	v += wave_shuffle_f(v, dpp_half_mirror);
+	v += wave_shuffle_f(v, dpp_row_mirror);
+	v += wave_shuffle_f(v, swz_xor16);
+	v += wave_shuffle_f(v, xor32);
+	return v;
+}
+__device__ __forceinline__ double wave_sum(double v)
+{
+	v += wave_shuffle_d(v, dpp_quad_xor1);
+	v += wave_shuffle_d(v, dpp_quad_xor2);
+	v += wave_shuffle_d(v, dpp_half_mirror);
+	v += wave_shuffle_d(v, dpp_row_mirror);
+	v += wave_shuffle_d(v, swz_xor16);
+	v += wave_shuffle_d(v, xor32);
+	return v;
+}
+__device__ __forceinline__ float wave_max(float v)
+{
+	v = fmaxf(v, wave_shuffle_f(v, dpp_quad_xor1));
+	v = fmaxf(v, wave_shuffle_f(v, dpp_quad_xor2));
+	v = fmaxf(v, wave_shuffle_f(v, dpp_half_mirror));
+	v = fmaxf(v, wave_shuffle_f(v, dpp_row_mirror));
+	v = fmaxf(v, wave_shuffle_f(v, swz_xor16));
+	v = fmaxf(v, wave_shuffle_f(v, xor32));
+	return v;
+}
+
+// Sum over a workgroup of BLOCK threads (BLOCK a multiple of 64, <= 1024);
+// every thread gets the total.  lds must hold BLOCK/64 values of T.
+template <int BLOCK, typename T>
+__device__ __forceinline__ T block_sum(T v, T *lds)
+{
+	constexpr int WAVES = BLOCK / kWave;
+	v = wave_sum(v);
+	if constexpr (WAVES == 1) return v;
+	const int wave = threadIdx.x / kWave;
+	__syncthreads();
+	if ((threadIdx.x % kWave) == 0) lds[wave] = v;
+	__syncthreads();
+	T total = lds[0];
+#pragma unroll
+	for (int w = 1; w < WAVES; w++) total += lds[w];
+	return total;
+}
+
+inline unsigned blocks_for(long n, int perBlock, unsigned cap = 1u << 20)
+{
+	long b = (n + perBlock - 1) / perBlock;
+	if (b < 1) b = 1;
+	if (b > (long)cap) b = cap;
+	return (unsigned)b;
+}
+
+} // namespace fitre

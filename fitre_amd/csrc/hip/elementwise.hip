@@ -1,0 +1,366 @@
+// Bandwidth-bound elementwise kernels, level-1 helpers and scalar reductions.
+// One templated grid-stride kernel per arity; 16-byte accesses whenever every
+// pointer is 16-byte aligned, scalar accesses otherwise.
+#include <math.h>
+#include "common.h"
+#include "fitre_nn.h"
+
+namespace fitre {
+
+constexpr int kEwBlock = 256;
+
+template <typename T>
+struct Vec;
+template <>
+struct Vec<float> {
+	static constexpr int N = 1;
+};
+template <>
+struct Vec<float4> {
+	static constexpr int N = 4;
+};
+
+__device__ __forceinline__ float comp(const float &v, int) { return v; }
+__device__ __forceinline__ float comp(const float4 &v, int i) { return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w; }
+__device__ __forceinline__ void setc(float &v, int, float x) { v = x; }
+__device__ __forceinline__ void setc(float4 &v, int i, float x)
+{
+	if (i == 0) v.x = x;
+	else if (i == 1) v.y = x;
+	else if (i == 2) v.z = x;
+	else v.w = x;
+}
+
+// out[i] = f(in0[i], in1[i], in2[i], in3[i]) for up to four inputs (unused ones alias in0).
+template <typename V, int NIN, typename F>
+__global__ void __launch_bounds__(kEwBlock) map_kernel(const V *a, const V *b, const V *c, const V *d, V *out, long nvec, F f)
+{
+	long stride = (long)gridDim.x * blockDim.x;
+	for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < nvec; i += stride) {
+		V va = a[i], vb = va, vc = va, vd = va, vo;
+		if constexpr (NIN > 1) vb = b[i];
+		if constexpr (NIN > 2) vc = c[i];
+		if constexpr (NIN > 3) vd = d[i];
+#pragma unroll
+		for (int k = 0; k < Vec<V>::N; k++) setc(vo, k, f(comp(va, k), comp(vb, k), comp(vc, k), comp(vd, k)));
+		out[i] = vo;
+	}
+}
+
+static inline bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
+
+template <int NIN, typename F>
+static int launch_map(const char *name, int cls, const float *a, const float *b, const float *c, const float *d,
+                      float *out, long n, F f)
+{
+	if (n == 0) return FITRE_OK;
+	LaunchScope scope(cls, (double)(NIN + 1) * 4.0 * (double)n);
+	bool vec = (n % 4 == 0) && aligned16(a) && aligned16(out) && (NIN < 2 || aligned16(b)) &&
+	           (NIN < 3 || aligned16(c)) && (NIN < 4 || aligned16(d));
+	if (vec) {
+		long nv = n / 4;
+		map_kernel<float4, NIN, F><<<blocks_for(nv, kEwBlock * 2, 8192), kEwBlock, 0, stream()>>>(
+		    (const float4 *)a, (const float4 *)b, (const float4 *)c, (const float4 *)d, (float4 *)out, nv, f);
+	} else {
+		map_kernel<float, NIN, F><<<blocks_for(n, kEwBlock * 4, 8192), kEwBlock, 0, stream()>>>(a, b, c, d, out, n, f);
+	}
+	return check_launch(name);
+}
+
+// ---- functors ---------------------------------------------------------------
+struct FAxpy { float alpha; __device__ float operator()(float x, float y, float, float) const { return y + alpha * x; } };
+struct FScal { float alpha; __device__ float operator()(float x, float, float, float) const { return alpha * x; } };
+struct FCopy { __device__ float operator()(float x, float, float, float) const { return x; } };
+struct FMul { __device__ float operator()(float x, float y, float, float) const { return x * y; } };
+struct FMulAdd2 { __device__ float operator()(float a, float b, float c, float d) const { return a * b + c * d; } };
+struct FInvScale { float eps; __device__ float operator()(float x, float y, float, float) const { return x / (sqrtf(y) + eps); } };
+struct FSqr { __device__ float operator()(float x, float, float, float) const { return x * x; } };
+struct FSqrDecay { float decay; __device__ float operator()(float x, float y, float, float) const { return decay * x + (1.f - decay) * y * y; } };
+
+__device__ __forceinline__ float sigmoidf(float x) { return 1.f / (1.f + expf(-x)); }
+
+struct ActRelu { __device__ float operator()(float x, float, float, float) const { return x < 0.f ? 0.f : x; } };
+struct ActSoftplus { __device__ float operator()(float x, float, float, float) const { return x < 20.f ? logf(1.f + expf(x)) : x; } };
+struct ActElu { __device__ float operator()(float x, float, float, float) const { return x < 0.f ? (expf(x) - 1.f) : x; } };
+struct ActSwish { __device__ float operator()(float x, float, float, float) const { return x / (1.f + expf(-x)); } };
+struct ActLogistic { __device__ float operator()(float x, float, float, float) const { return sigmoidf(x); } };
+struct ActTanh { __device__ float operator()(float x, float, float, float) const { return tanhf(x); } };
+
+// backward functors take (delta, z_in, z_out)
+struct DLogistic { __device__ float operator()(float d, float, float zo, float) const { return d * zo * (1.f - zo); } };
+struct DTanh { __device__ float operator()(float d, float, float zo, float) const { return d * ((1.f + zo) * (1.f - zo)); } };
+struct DSoftplus { __device__ float operator()(float d, float zi, float, float) const { return d * sigmoidf(zi); } };
+struct DSwish { __device__ float operator()(float d, float zi, float zo, float) const { float t = sigmoidf(zi); return d * (zo + t * (1.f - zo)); } };
+struct DRelu { __device__ float operator()(float d, float, float zo, float) const { return zo > 0.f ? d : 0.f; } };
+struct DElu { __device__ float operator()(float d, float, float zo, float) const { return zo < 0.f ? d * (zo + 1.f) : d; } };
+
+// ---- scalar reductions --------------------------------------------------------
+enum RedOp { RED_SUM = 0, RED_DOT = 1, RED_SQR = 2, RED_ABS = 3, RED_ABSMAX = 4 };
+
+template <int OP>
+__global__ void __launch_bounds__(256) reduce_stage1(const float *x, const float *y, long n, double *partial)
+{
+	__shared__ double lds[4];
+	double acc = 0.0;
+	long stride = (long)gridDim.x * blockDim.x;
+	for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+		float v = x[i];
+		if constexpr (OP == RED_SUM) acc += (double)v;
+		if constexpr (OP == RED_DOT) acc += (double)v * (double)y[i];
+		if constexpr (OP == RED_SQR) acc += (double)v * (double)v;
+		if constexpr (OP == RED_ABS) acc += (double)fabsf(v);
+		if constexpr (OP == RED_ABSMAX) acc = fmax(acc, (double)fabsf(v));
+	}
+	if constexpr (OP == RED_ABSMAX) {
+		float m = wave_max((float)acc);
+		__shared__ float ldsm[4];
+		if (threadIdx.x % kWave == 0) ldsm[threadIdx.x / kWave] = m;
+		__syncthreads();
+		if (threadIdx.x == 0) partial[blockIdx.x] = (double)fmaxf(fmaxf(ldsm[0], ldsm[1]), fmaxf(ldsm[2], ldsm[3]));
+	} else {
+		double t = block_sum<256>(acc, lds);
+		if (threadIdx.x == 0) partial[blockIdx.x] = t;
+	}
+}
+
+template <int OP>
+__global__ void __launch_bounds__(256) reduce_stage2(const double *partial, int count, float *result)
+{
+	__shared__ double lds[4];
+	double acc = 0.0;
+	for (int i = threadIdx.x; i < count; i += 256) {
+		if constexpr (OP == RED_ABSMAX) acc = fmax(acc, partial[i]);
+		else acc += partial[i];
+	}
+	if constexpr (OP == RED_ABSMAX) {
+		float m = wave_max((float)acc);
+		__shared__ float ldsm[4];
+		if (threadIdx.x % kWave == 0) ldsm[threadIdx.x / kWave] = m;
+		__syncthreads();
+		if (threadIdx.x == 0) result[0] = fmaxf(fmaxf(ldsm[0], ldsm[1]), fmaxf(ldsm[2], ldsm[3]));
+	} else {
+		double t = block_sum<256>(acc, lds);
+		if (threadIdx.x == 0) result[0] = (OP == RED_SQR) ? (float)sqrt(t) : (float)t;
+	}
+}
+
+constexpr int kRedBlocks = 1024;
+static double *g_partials = nullptr; // kRedBlocks doubles + 1 float result slot
+static float *g_host_result = nullptr;
+
+static int ensure_reduce_buffers()
+{
+	if (g_partials) return FITRE_OK;
+	FITRE_HIP_TRY(hipMalloc((void **)&g_partials, (kRedBlocks + 2) * sizeof(double)));
+	FITRE_HIP_TRY(hipHostMalloc((void **)&g_host_result, 64, hipHostMallocDefault));
+	return FITRE_OK;
+}
+
+template <int OP>
+static int scalar_reduce(const char *name, int n, const float *x, const float *y, float *result)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(n >= 0 && x && result && (OP != RED_DOT || y), "%s: bad argument", name);
+	if (n == 0) {
+		*result = 0.f;
+		return FITRE_OK;
+	}
+	int rc = ensure_reduce_buffers();
+	if (rc) return rc;
+	{
+		LaunchScope scope(FITRE_KC_BLAS1, 4.0 * n * (OP == RED_DOT ? 2 : 1));
+		unsigned blocks = blocks_for(n, 256 * 8, kRedBlocks);
+		float *devResult = (float *)(g_partials + kRedBlocks);
+		reduce_stage1<OP><<<blocks, 256, 0, stream()>>>(x, y, n, g_partials);
+		reduce_stage2<OP><<<1, 256, 0, stream()>>>(g_partials, (int)blocks, devResult);
+		rc = check_launch(name);
+		if (rc) return rc;
+		FITRE_HIP_TRY(hipMemcpyAsync(g_host_result, devResult, sizeof(float), hipMemcpyDeviceToHost, stream()));
+	}
+	FITRE_HIP_TRY(hipStreamSynchronize(stream()));
+	*result = *g_host_result;
+	return FITRE_OK;
+}
+
+// column-major rows x cols: out[i] = x[i] * y[i / rows]
+__global__ void __launch_bounds__(256) col_scale_kernel(const float *x, int rows, long n, const float *y, float *out)
+{
+	long stride = (long)gridDim.x * blockDim.x;
+	for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) out[i] = x[i] * y[i / rows];
+}
+// column-major rows x cols: mat[i] += vec[i % rows]
+__global__ void __launch_bounds__(256) add_column_kernel(float *mat, int rows, long n, const float *vec)
+{
+	long stride = (long)gridDim.x * blockDim.x;
+	for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) mat[i] += vec[i % rows];
+}
+// [channels][perChannel]: x[c][i] += bias[c]
+__global__ void __launch_bounds__(256) add_channel_bias_kernel(float *x, long perChannel, const float *bias)
+{
+	float b = bias[blockIdx.y];
+	float *p = x + (size_t)blockIdx.y * perChannel;
+	long stride = (long)gridDim.x * blockDim.x;
+	for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < perChannel; i += stride) p[i] += b;
+}
+// out[r] = sum_c mat[r + c*rows]  (one wave per row group; rows are the fast index)
+__global__ void __launch_bounds__(256) row_sum_kernel(const float *mat, int rows, int cols, float *out)
+{
+	int r = blockIdx.x * blockDim.x + threadIdx.x;
+	if (r >= rows) return;
+	double acc = 0.0;
+	for (int c = 0; c < cols; c++) acc += (double)mat[(size_t)c * rows + r];
+	out[r] = (float)acc;
+}
+
+} // namespace fitre
+
+using namespace fitre;
+
+#define EW_CHECK(name, cond)                                                                         \
+	FITRE_NEED_INIT();                                                                               \
+	FITRE_REQUIRE(cond, "%s: null pointer or negative size", name)
+
+extern "C" {
+
+int fitre_hip_axpy(int n, float alpha, const float *x, float *y)
+{
+	EW_CHECK("fitre_hip_axpy", x && y && n >= 0);
+	return launch_map<2>("axpy", FITRE_KC_BLAS1, x, y, nullptr, nullptr, y, n, FAxpy{ alpha });
+}
+int fitre_hip_scal(int n, float alpha, float *x)
+{
+	EW_CHECK("fitre_hip_scal", x && n >= 0);
+	return launch_map<1>("scal", FITRE_KC_BLAS1, x, nullptr, nullptr, nullptr, x, n, FScal{ alpha });
+}
+int fitre_hip_copy(int n, const float *x, float *y)
+{
+	EW_CHECK("fitre_hip_copy", x && y && n >= 0);
+	return launch_map<1>("copy", FITRE_KC_BLAS1, x, nullptr, nullptr, nullptr, y, n, FCopy{});
+}
+int fitre_hip_dot(int n, const float *x, const float *y, float *result) { return scalar_reduce<RED_DOT>("fitre_hip_dot", n, x, y, result); }
+int fitre_hip_nrm2(int n, const float *x, float *result) { return scalar_reduce<RED_SQR>("fitre_hip_nrm2", n, x, nullptr, result); }
+int fitre_hip_asum(int n, const float *x, float *result) { return scalar_reduce<RED_ABS>("fitre_hip_asum", n, x, nullptr, result); }
+int fitre_hip_norm_inf(int n, const float *x, float *result) { return scalar_reduce<RED_ABSMAX>("fitre_hip_norm_inf", n, x, nullptr, result); }
+int fitre_hip_sum(int n, const float *x, float *result) { return scalar_reduce<RED_SUM>("fitre_hip_sum", n, x, nullptr, result); }
+
+int fitre_hip_fill(float *x, long n, float value)
+{
+	EW_CHECK("fitre_hip_fill", x && n >= 0);
+	// y = 0*x + value would read x; use a scaled copy of a constant instead
+	struct FConst { float v; __device__ float operator()(float, float, float, float) const { return v; } };
+	return launch_map<1>("fill", FITRE_KC_BLAS1, x, nullptr, nullptr, nullptr, x, n, FConst{ value });
+}
+int fitre_hip_hadamard(const float *x, float *y, long n)
+{
+	EW_CHECK("fitre_hip_hadamard", x && y && n >= 0);
+	return launch_map<2>("hadamard", FITRE_KC_BLAS1, x, y, nullptr, nullptr, y, n, FMul{});
+}
+int fitre_hip_hadamard2(const float *m1, const float *m2, const float *m3, const float *m4, long n, float *out)
+{
+	EW_CHECK("fitre_hip_hadamard2", m1 && m2 && m3 && m4 && out && n >= 0);
+	return launch_map<4>("hadamard2", FITRE_KC_BLAS1, m1, m2, m3, m4, out, n, FMulAdd2{});
+}
+int fitre_hip_elem_inv_scale(const float *x, const float *y, float eps, long n, float *out)
+{
+	EW_CHECK("fitre_hip_elem_inv_scale", x && y && out && n >= 0);
+	return launch_map<2>("elem_inv_scale", FITRE_KC_BLAS1, x, y, nullptr, nullptr, out, n, FInvScale{ eps });
+}
+int fitre_hip_elem_sqr(const float *x, long n, float *out)
+{
+	EW_CHECK("fitre_hip_elem_sqr", x && out && n >= 0);
+	return launch_map<1>("elem_sqr", FITRE_KC_BLAS1, x, nullptr, nullptr, nullptr, out, n, FSqr{});
+}
+int fitre_hip_elem_sqr_decay(const float *x, const float *y, float decay, long n, float *out)
+{
+	EW_CHECK("fitre_hip_elem_sqr_decay", x && y && out && n >= 0);
+	return launch_map<2>("elem_sqr_decay", FITRE_KC_BLAS1, x, y, nullptr, nullptr, out, n, FSqrDecay{ decay });
+}
+int fitre_hip_mat_mat_scale(const float *x, const float *y, long n, float *out)
+{
+	EW_CHECK("fitre_hip_mat_mat_scale", x && y && out && n >= 0);
+	return launch_map<2>("mat_mat_scale", FITRE_KC_BLAS1, x, y, nullptr, nullptr, out, n, FMul{});
+}
+int fitre_hip_mat_row_vec_scale(const float *x, int rows, int cols, const float *y, float *out)
+{
+	EW_CHECK("fitre_hip_mat_row_vec_scale", x && y && out && rows > 0 && cols > 0);
+	long n = (long)rows * cols;
+	LaunchScope scope(FITRE_KC_BLAS1, 8.0 * n);
+	col_scale_kernel<<<blocks_for(n, 1024, 8192), 256, 0, stream()>>>(x, rows, n, y, out);
+	return check_launch("col_scale_kernel");
+}
+int fitre_hip_add_column(float *mat, int rows, int cols, const float *vec)
+{
+	EW_CHECK("fitre_hip_add_column", mat && vec && rows > 0 && cols > 0);
+	long n = (long)rows * cols;
+	LaunchScope scope(FITRE_KC_BLAS1, 8.0 * n);
+	add_column_kernel<<<blocks_for(n, 1024, 8192), 256, 0, stream()>>>(mat, rows, n, vec);
+	return check_launch("add_column_kernel");
+}
+int fitre_hip_add_channel_bias(float *x, int channels, long perChannel, const float *bias)
+{
+	EW_CHECK("fitre_hip_add_channel_bias", x && bias && channels > 0 && perChannel > 0);
+	FITRE_REQUIRE(channels <= 65535, "fitre_hip_add_channel_bias: %d channels exceed the grid limit", channels);
+	LaunchScope scope(FITRE_KC_BLAS1, 8.0 * channels * perChannel);
+	dim3 grid(blocks_for(perChannel, 1024, 1024), channels);
+	add_channel_bias_kernel<<<grid, 256, 0, stream()>>>(x, perChannel, bias);
+	return check_launch("add_channel_bias_kernel");
+}
+int fitre_hip_row_sum(const float *mat, int rows, int cols, float *out)
+{
+	EW_CHECK("fitre_hip_row_sum", mat && out && rows > 0 && cols > 0);
+	LaunchScope scope(FITRE_KC_BIAS_GRAD, 4.0 * rows * cols);
+	row_sum_kernel<<<blocks_for(rows, 256), 256, 0, stream()>>>(mat, rows, cols, out);
+	return check_launch("row_sum_kernel");
+}
+
+int fitre_hip_activation_forward(int actFun, const float *in, float *out, long n)
+{
+	EW_CHECK("fitre_hip_activation_forward", in && out && n >= 0);
+	const int cls = FITRE_KC_ACT_FWD;
+	switch (actFun) {
+	case CNN_ACT_RELU: return launch_map<1>("relu", cls, in, nullptr, nullptr, nullptr, out, n, ActRelu{});
+	case CNN_ACT_SOFTPLUS: return launch_map<1>("softplus", cls, in, nullptr, nullptr, nullptr, out, n, ActSoftplus{});
+	case CNN_ACT_ELU: return launch_map<1>("elu", cls, in, nullptr, nullptr, nullptr, out, n, ActElu{});
+	case CNN_ACT_SWISH: return launch_map<1>("swish", cls, in, nullptr, nullptr, nullptr, out, n, ActSwish{});
+	case ACT_LOGISTIC: return launch_map<1>("logistic", cls, in, nullptr, nullptr, nullptr, out, n, ActLogistic{});
+	case ACT_TANH: return launch_map<1>("tanh", cls, in, nullptr, nullptr, nullptr, out, n, ActTanh{});
+	case ACT_LINEAR:
+	case CNN_ACT_NONE:
+		if (in == out) return FITRE_OK;
+		return launch_map<1>("copy", cls, in, nullptr, nullptr, nullptr, out, n, FCopy{});
+	default: return fail(FITRE_E_UNSUPPORTED, "fitre_hip_activation_forward: unknown activation code %d", actFun);
+	}
+}
+
+int fitre_hip_activation_backward(int actFun, const float *delta, const float *z_in, const float *z_out, float *out, long n)
+{
+	EW_CHECK("fitre_hip_activation_backward", delta && out && n >= 0);
+	const int cls = FITRE_KC_ACT_BWD;
+	switch (actFun) {
+	case ACT_LOGISTIC:
+		FITRE_REQUIRE(z_out, "activation backward (logistic): z_out is null");
+		return launch_map<3>("dlogistic", cls, delta, z_out, z_out, nullptr, out, n, DLogistic{});
+	case ACT_TANH:
+		FITRE_REQUIRE(z_out, "activation backward (tanh): z_out is null");
+		return launch_map<3>("dtanh", cls, delta, z_out, z_out, nullptr, out, n, DTanh{});
+	case CNN_ACT_SOFTPLUS:
+		FITRE_REQUIRE(z_in, "activation backward (softplus): z_in is null");
+		return launch_map<2>("dsoftplus", cls, delta, z_in, nullptr, nullptr, out, n, DSoftplus{});
+	case CNN_ACT_SWISH:
+		FITRE_REQUIRE(z_in && z_out, "activation backward (swish): z_in or z_out is null");
+		return launch_map<3>("dswish", cls, delta, z_in, z_out, nullptr, out, n, DSwish{});
+	case CNN_ACT_RELU:
+		FITRE_REQUIRE(z_out, "activation backward (relu): z_out is null");
+		return launch_map<3>("drelu", cls, delta, z_out, z_out, nullptr, out, n, DRelu{});
+	case CNN_ACT_ELU:
+		FITRE_REQUIRE(z_out, "activation backward (elu): z_out is null");
+		return launch_map<3>("delu", cls, delta, z_out, z_out, nullptr, out, n, DElu{});
+	case ACT_LINEAR:
+	case CNN_ACT_NONE:
+		if (delta == out) return FITRE_OK;
+		return launch_map<1>("copy", cls, delta, nullptr, nullptr, nullptr, out, n, FCopy{});
+	default: return fail(FITRE_E_UNSUPPORTED, "fitre_hip_activation_backward: unknown activation code %d", actFun);
+	}
+}
+
+} // extern "C"

@@ -1,0 +1,840 @@
+// Bandwidth-bound layer kernels on [C][N][A][B] tensors: pooling, batch
+// normalisation, per-channel sums, softmax cross entropy and the layout change
+// at the convolution / fully-connected boundary.
+#include <float.h>
+#include <math.h>
+#include "common.h"
+#include "fitre_nn.h"
+
+namespace fitre {
+
+// =====================================================================
+// pooling
+// =====================================================================
+
+struct PoolGeom {
+	int inA, inB, outA, outB, ksize, stride, padding;
+	FastDiv divOutB, divOutA, divInB, divInA;
+};
+
+static PoolGeom make_geom(int inA, int inB, int ksize, int stride, int padding, int outA, int outB)
+{
+	PoolGeom g;
+	g.inA = inA;
+	g.inB = inB;
+	g.outA = outA;
+	g.outB = outB;
+	g.ksize = ksize;
+	g.stride = stride;
+	g.padding = padding;
+	g.divOutB = FastDiv((uint32_t)outB);
+	g.divOutA = FastDiv((uint32_t)outA);
+	g.divInB = FastDiv((uint32_t)inB);
+	g.divInA = FastDiv((uint32_t)inA);
+	return g;
+}
+
+// First maximum of one window in memory order (A outer, B inner, strict >);
+// returns the offset inside the map, or -1 for a window with no valid cell.
+__device__ __forceinline__ int window_argmax(const float *map, const PoolGeom &g, int oa, int ob, float &best)
+{
+	int a0 = oa * g.stride - g.padding, b0 = ob * g.stride - g.padding;
+	int arg = -1;
+	best = -FLT_MAX;
+	for (int da = 0; da < g.ksize; da++) {
+		int a = a0 + da;
+		if (a < 0 || a >= g.inA) continue;
+		for (int db = 0; db < g.ksize; db++) {
+			int b = b0 + db;
+			if (b < 0 || b >= g.inB) continue;
+			float t = map[a * g.inB + b];
+			if (t > best) {
+				best = t;
+				arg = a * g.inB + b;
+			}
+		}
+	}
+	return arg;
+}
+
+// one thread per pooled cell
+template <int MODE> // 0 max value, 1 average, 2 argmax index
+__global__ void __launch_bounds__(256) pool_forward_kernel(const float *in, PoolGeom g, long maps, float *out, int *index)
+{
+	long total = maps * g.outA * g.outB;
+	long stride = (long)gridDim.x * blockDim.x;
+	for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+		uint32_t q, ob, oa, map;
+		g.divOutB.divmod((uint32_t)i, q, ob);
+		g.divOutA.divmod(q, map, oa);
+		const float *src = in + (size_t)map * g.inA * g.inB;
+		if constexpr (MODE == 1) {
+			int a0 = (int)oa * g.stride - g.padding, b0 = (int)ob * g.stride - g.padding;
+			float s = 0.f;
+			for (int da = 0; da < g.ksize; da++) {
+				int a = a0 + da;
+				if (a < 0 || a >= g.inA) continue;
+				for (int db = 0; db < g.ksize; db++) {
+					int b = b0 + db;
+					if (b < 0 || b >= g.inB) continue;
+					s += src[a * g.inB + b];
+				}
+			}
+			out[i] = s / (float)(g.ksize * g.ksize);
+		} else {
+			float best;
+			int arg = window_argmax(src, g, (int)oa, (int)ob, best);
+			if constexpr (MODE == 0) out[i] = best;
+			else index[i] = (arg < 0) ? INT_MAX : arg;
+		}
+	}
+}
+
+// Gradient reaching input cell (a, b) of one map: sum over the windows that
+// contain the cell.  No atomics: every input cell is owned by one thread.
+template <int POOL> // 0 max, 1 average
+__device__ __forceinline__ float pool_gather(const float *dmap, const float *zmap, const PoolGeom &g, int a, int b)
+{
+	// windows oa with oa*stride - padding <= a <= oa*stride - padding + ksize - 1
+	int oaHi = (a + g.padding) / g.stride;
+	int obHi = (b + g.padding) / g.stride;
+	int oaLo = (a + g.padding - g.ksize + g.stride) / g.stride; // ceil((a+p-k+1)/s) for a+p-k+1 >= 1-s
+	int obLo = (b + g.padding - g.ksize + g.stride) / g.stride;
+	if (a + g.padding - g.ksize + 1 <= 0) oaLo = 0;
+	if (b + g.padding - g.ksize + 1 <= 0) obLo = 0;
+	if (oaHi >= g.outA) oaHi = g.outA - 1;
+	if (obHi >= g.outB) obHi = g.outB - 1;
+	float acc = 0.f;
+	const int self = a * g.inB + b;
+	for (int oa = oaLo; oa <= oaHi; oa++) {
+		for (int ob = obLo; ob <= obHi; ob++) {
+			if constexpr (POOL == 0) {
+				float best;
+				if (window_argmax(zmap, g, oa, ob, best) == self) acc += dmap[oa * g.outB + ob];
+			} else {
+				acc += dmap[oa * g.outB + ob] * (1.f / (float)(g.ksize * g.ksize));
+			}
+		}
+	}
+	return acc;
+}
+
+__device__ __forceinline__ float act_derivative(int actFun, float zi, float zo)
+{
+	switch (actFun) {
+	case ACT_LOGISTIC: return zo * (1.f - zo);
+	case ACT_TANH: return (1.f + zo) * (1.f - zo);
+	case CNN_ACT_SOFTPLUS: return 1.f / (1.f + expf(-zi));
+	case CNN_ACT_SWISH: {
+		float t = 1.f / (1.f + expf(-zi));
+		return zo + t * (1.f - zo);
+	}
+	case CNN_ACT_RELU: return zo > 0.f ? 1.f : 0.f;
+	case CNN_ACT_ELU: return zo < 0.f ? zo + 1.f : 1.f;
+	default: return 1.f;
+	}
+}
+
+// One thread per input cell.  POOL: 0 max, 1 average, 2 none.  FUSE_ACT: also
+// write dxAct = gradient * f'(.).
+template <int POOL, bool FUSE_ACT>
+__global__ void __launch_bounds__(256)
+pool_backward_kernel(const float *delta, const float *z_in, const float *z_act, PoolGeom g, long maps, int actFun,
+                     float *dxPool, float *dxAct)
+{
+	long perMap = (long)g.inA * g.inB;
+	long total = maps * perMap;
+	long stride = (long)gridDim.x * blockDim.x;
+	for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+		float gval;
+		if constexpr (POOL == 2) {
+			gval = delta[i];
+		} else {
+			uint32_t q, b, a, map;
+			g.divInB.divmod((uint32_t)i, q, b);
+			g.divInA.divmod(q, map, a);
+			gval = pool_gather<POOL>(delta + (size_t)map * g.outA * g.outB, z_act + (size_t)map * perMap, g, (int)a, (int)b);
+		}
+		if (dxPool) dxPool[i] = gval;
+		if constexpr (FUSE_ACT) {
+			float zo = z_act ? z_act[i] : 0.f;
+			float zi = z_in ? z_in[i] : 0.f;
+			dxAct[i] = gval * act_derivative(actFun, zi, zo);
+		}
+	}
+}
+
+// strict-> scan of four values in order, starting below every finite float
+__device__ __forceinline__ int scan2x2(float v0, float v1, float v2, float v3)
+{
+	float best = -FLT_MAX;
+	int arg = -1;
+	if (v0 > best) { best = v0; arg = 0; }
+	if (v1 > best) { best = v1; arg = 1; }
+	if (v2 > best) { best = v2; arg = 2; }
+	if (v3 > best) { best = v3; arg = 3; }
+	return arg;
+}
+
+// Non-overlapping 2x2 / stride 2 / no padding max pool, even extents: one
+// thread per pair of pooled cells adjacent along B, i.e. a 2 x 4 input patch
+// moved with 16-byte accesses.  Fused with the activation derivative.
+template <bool FUSE_ACT>
+__global__ void __launch_bounds__(256)
+maxpool2_backward_kernel(const float *delta, const float *z_in, const float *z_act, int inA, int inB, long maps,
+                         int actFun, float *dxPool, float *dxAct)
+{
+	const int outB2 = inB / 4; // pairs of pooled cells per pooled row
+	const int outA = inA / 2;
+	long total = maps * outA * outB2;
+	long stride = (long)gridDim.x * blockDim.x;
+	for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+		long map = i / ((long)outA * outB2);
+		int rem = (int)(i - map * outA * outB2);
+		int oa = rem / outB2, pb = rem - oa * outB2;
+		size_t inOff = (size_t)map * inA * inB + (size_t)(2 * oa) * inB + 4 * pb;
+		size_t dOff = (size_t)map * outA * (inB / 2) + (size_t)oa * (inB / 2) + 2 * pb;
+		float4 r0 = *reinterpret_cast<const float4 *>(z_act + inOff);
+		float4 r1 = *reinterpret_cast<const float4 *>(z_act + inOff + inB);
+		float2 d = *reinterpret_cast<const float2 *>(delta + dOff);
+		// memory-order scan of each 2x2 window: (a0,b0), (a0,b1), (a1,b0), (a1,b1)
+		float4 g0 = make_float4(0.f, 0.f, 0.f, 0.f), g1 = g0;
+		int arg = scan2x2(r0.x, r0.y, r1.x, r1.y);
+		if (arg == 0) g0.x = d.x;
+		else if (arg == 1) g0.y = d.x;
+		else if (arg == 2) g1.x = d.x;
+		else if (arg == 3) g1.y = d.x;
+		arg = scan2x2(r0.z, r0.w, r1.z, r1.w);
+		if (arg == 0) g0.z = d.y;
+		else if (arg == 1) g0.w = d.y;
+		else if (arg == 2) g1.z = d.y;
+		else if (arg == 3) g1.w = d.y;
+		if (dxPool) {
+			*reinterpret_cast<float4 *>(dxPool + inOff) = g0;
+			*reinterpret_cast<float4 *>(dxPool + inOff + inB) = g1;
+		}
+		if constexpr (FUSE_ACT) {
+			float4 i0 = r0, i1 = r1;
+			if (z_in) {
+				i0 = *reinterpret_cast<const float4 *>(z_in + inOff);
+				i1 = *reinterpret_cast<const float4 *>(z_in + inOff + inB);
+			}
+			g0.x *= act_derivative(actFun, i0.x, r0.x);
+			g0.y *= act_derivative(actFun, i0.y, r0.y);
+			g0.z *= act_derivative(actFun, i0.z, r0.z);
+			g0.w *= act_derivative(actFun, i0.w, r0.w);
+			g1.x *= act_derivative(actFun, i1.x, r1.x);
+			g1.y *= act_derivative(actFun, i1.y, r1.y);
+			g1.z *= act_derivative(actFun, i1.z, r1.z);
+			g1.w *= act_derivative(actFun, i1.w, r1.w);
+			*reinterpret_cast<float4 *>(dxAct + inOff) = g0;
+			*reinterpret_cast<float4 *>(dxAct + inOff + inB) = g1;
+		}
+	}
+}
+
+static bool act_known(int actFun)
+{
+	switch (actFun) {
+	case ACT_LOGISTIC:
+	case ACT_TANH:
+	case ACT_LINEAR:
+	case CNN_ACT_NONE:
+	case CNN_ACT_SOFTPLUS:
+	case CNN_ACT_ELU:
+	case CNN_ACT_RELU:
+	case CNN_ACT_SWISH: return true;
+	default: return false;
+	}
+}
+static bool act_needs_zin(int actFun) { return actFun == CNN_ACT_SOFTPLUS || actFun == CNN_ACT_SWISH; }
+static bool act_needs_zout(int actFun)
+{
+	return actFun == ACT_LOGISTIC || actFun == ACT_TANH || actFun == CNN_ACT_SWISH || actFun == CNN_ACT_RELU ||
+	       actFun == CNN_ACT_ELU;
+}
+
+static int check_pool_shape(const char *fn, int channels, int samples, int inA, int inB, int ksize, int stride,
+                            int padding, int outA, int outB)
+{
+	FITRE_REQUIRE(channels > 0 && samples > 0 && inA > 0 && inB > 0 && ksize > 0 && stride > 0 && padding >= 0,
+	              "%s: non-positive shape (C=%d N=%d A=%d B=%d k=%d s=%d p=%d)", fn, channels, samples, inA, inB,
+	              ksize, stride, padding);
+	FITRE_REQUIRE(outA == (inA + 2 * padding - ksize) / stride + 1 && outB == (inB + 2 * padding - ksize) / stride + 1 &&
+	                  outA > 0 && outB > 0,
+	              "%s: pooled extent %dx%d does not match input %dx%d, k=%d s=%d p=%d", fn, outA, outB, inA, inB, ksize,
+	              stride, padding);
+	FITRE_REQUIRE(padding < ksize, "%s: padding %d >= window %d leaves empty windows", fn, padding, ksize);
+	FITRE_REQUIRE((double)channels * samples * inA * inB < 2147483647.0, "%s: tensor exceeds 2^31 elements", fn);
+	return FITRE_OK;
+}
+
+// =====================================================================
+// per-channel reductions and batch normalisation
+// =====================================================================
+
+constexpr int kRedBlock = 256;
+
+// number of segments each channel is cut into
+static int segments_for(int channels, long perChannel)
+{
+	long perBlockMin = 4096; // at least 16 elements per thread
+	long s = (perChannel + perBlockMin - 1) / perBlockMin;
+	long want = (2048 + channels - 1) / channels; // aim at >= 2048 workgroups
+	if (s > want) s = want;
+	if (s > 256) s = 256;
+	if (s < 1) s = 1;
+	return (int)s;
+}
+
+// Segment [lo, hi) of a channel handled by block (blockIdx.x of gridDim.x), in units of 4 elements
+// so that 16-byte accesses stay aligned.
+__device__ __forceinline__ void segment_range(long perChannel, long &lo, long &hi)
+{
+	long quads = (perChannel + 3) / 4;
+	long per = (quads + gridDim.x - 1) / gridDim.x;
+	lo = (long)blockIdx.x * per * 4;
+	hi = lo + per * 4;
+	if (hi > perChannel) hi = perChannel;
+	if (lo > perChannel) lo = perChannel;
+}
+
+// NOUT sums per (channel, segment): MODE 0: sum x; 1: sum x, sum x*y; 2: sum x, sum x^2
+template <int MODE, bool VEC>
+__global__ void __launch_bounds__(kRedBlock)
+channel_partial_kernel(const float *x, const float *y, long perChannel, double *partial)
+{
+	__shared__ double lds[kRedBlock / kWave];
+	const int c = blockIdx.y;
+	const float *px = x + (size_t)c * perChannel;
+	const float *py = (MODE == 1) ? y + (size_t)c * perChannel : nullptr;
+	long lo, hi;
+	segment_range(perChannel, lo, hi);
+	double s0 = 0.0, s1 = 0.0;
+	if constexpr (VEC) {
+		for (long i = lo + 4 * (long)threadIdx.x; i + 3 < hi; i += 4 * kRedBlock) {
+			float4 a = *reinterpret_cast<const float4 *>(px + i);
+			float t0 = (a.x + a.y) + (a.z + a.w);
+			s0 += (double)t0;
+			if constexpr (MODE == 1) {
+				float4 b = *reinterpret_cast<const float4 *>(py + i);
+				s1 += (double)(a.x * b.x) + (double)(a.y * b.y) + (double)(a.z * b.z) + (double)(a.w * b.w);
+			}
+			if constexpr (MODE == 2)
+				s1 += (double)a.x * a.x + (double)a.y * a.y + (double)a.z * a.z + (double)a.w * a.w;
+		}
+		long tail = lo + ((hi - lo) / 4) * 4;
+		for (long i = tail + threadIdx.x; i < hi; i += kRedBlock) {
+			float a = px[i];
+			s0 += (double)a;
+			if constexpr (MODE == 1) s1 += (double)(a * py[i]);
+			if constexpr (MODE == 2) s1 += (double)a * a;
+		}
+	} else {
+		for (long i = lo + threadIdx.x; i < hi; i += kRedBlock) {
+			float a = px[i];
+			s0 += (double)a;
+			if constexpr (MODE == 1) s1 += (double)(a * py[i]);
+			if constexpr (MODE == 2) s1 += (double)a * a;
+		}
+	}
+	double t0 = block_sum<kRedBlock>(s0, lds);
+	double t1 = 0.0;
+	if constexpr (MODE != 0) t1 = block_sum<kRedBlock>(s1, lds);
+	if (threadIdx.x == 0) {
+		size_t slot = ((size_t)c * gridDim.x + blockIdx.x) * 2;
+		partial[slot] = t0;
+		partial[slot + 1] = t1;
+	}
+}
+
+// out[c] = sum over segments of partial[c][s][which]
+__global__ void channel_finish_kernel(const double *partial, int segments, int which, int channels, float *out)
+{
+	int c = blockIdx.x * blockDim.x + threadIdx.x;
+	if (c >= channels) return;
+	double acc = 0.0;
+	for (int s = 0; s < segments; s++) acc += partial[((size_t)c * segments + s) * 2 + which];
+	out[c] = (float)acc;
+}
+
+// batch-norm forward, statistics: mean, biased variance, running statistics
+__global__ void bn_stats_kernel(const double *partial, int segments, int channels, long perChannel, float momentum,
+                                float *mean, float *variance, float *runMean, float *runVar)
+{
+	int c = blockIdx.x * blockDim.x + threadIdx.x;
+	if (c >= channels) return;
+	double s = 0.0, ss = 0.0;
+	for (int k = 0; k < segments; k++) {
+		s += partial[((size_t)c * segments + k) * 2];
+		ss += partial[((size_t)c * segments + k) * 2 + 1];
+	}
+	double m = s / (double)perChannel;
+	double v = ss / (double)perChannel - m * m;
+	if (v < 0.0) v = 0.0;
+	mean[c] = (float)m;
+	variance[c] = (float)v;
+	runMean[c] = momentum * runMean[c] + (1.f - momentum) * (float)m;
+	runVar[c] = momentum * runVar[c] + (1.f - momentum) * (float)v;
+}
+
+template <bool VEC>
+__global__ void __launch_bounds__(kRedBlock)
+bn_normalize_kernel(const float *x, const float *mean, const float *variance, float epsilon, long perChannel, float *zhat)
+{
+	const int c = blockIdx.y;
+	const float mu = mean[c];
+	const float inv = 1.f / sqrtf(variance[c] + epsilon);
+	const float *px = x + (size_t)c * perChannel;
+	float *po = zhat + (size_t)c * perChannel;
+	long lo, hi;
+	segment_range(perChannel, lo, hi);
+	if constexpr (VEC) {
+		for (long i = lo + 4 * (long)threadIdx.x; i + 3 < hi; i += 4 * kRedBlock) {
+			float4 a = *reinterpret_cast<const float4 *>(px + i);
+			a.x = (a.x - mu) * inv;
+			a.y = (a.y - mu) * inv;
+			a.z = (a.z - mu) * inv;
+			a.w = (a.w - mu) * inv;
+			*reinterpret_cast<float4 *>(po + i) = a;
+		}
+		long tail = lo + ((hi - lo) / 4) * 4;
+		for (long i = tail + threadIdx.x; i < hi; i += kRedBlock) po[i] = (px[i] - mu) * inv;
+	} else {
+		for (long i = lo + threadIdx.x; i < hi; i += kRedBlock) po[i] = (px[i] - mu) * inv;
+	}
+}
+
+// batch-norm backward, elementwise part; also leaves the per-segment sum of the
+// result in partialOut (for the bias gradient).
+template <bool VEC>
+__global__ void __launch_bounds__(kRedBlock)
+bn_backward_apply_kernel(const float *delta, const float *zhat, const float *variance, const double *partial,
+                         int segmentsIn, float epsilon, long perChannel, float *out, double *partialOut)
+{
+	__shared__ double lds[kRedBlock / kWave];
+	const int c = blockIdx.y;
+	double d1 = 0.0, d2 = 0.0;
+	for (int k = 0; k < segmentsIn; k++) {
+		d1 += partial[((size_t)c * segmentsIn + k) * 2];
+		d2 += partial[((size_t)c * segmentsIn + k) * 2 + 1];
+	}
+	const float m = (float)perChannel;
+	const float sum1 = (float)d1, sum2 = (float)d2;
+	const float scale = 1.f / (m * sqrtf(epsilon + variance[c]));
+	const float *pd = delta + (size_t)c * perChannel;
+	const float *pz = zhat + (size_t)c * perChannel;
+	float *po = out + (size_t)c * perChannel;
+	long lo, hi;
+	segment_range(perChannel, lo, hi);
+	double acc = 0.0;
+	if constexpr (VEC) {
+		for (long i = lo + 4 * (long)threadIdx.x; i + 3 < hi; i += 4 * kRedBlock) {
+			float4 d = *reinterpret_cast<const float4 *>(pd + i);
+			float4 z = *reinterpret_cast<const float4 *>(pz + i);
+			float4 r;
+			r.x = (m * d.x - sum1 - sum2 * z.x) * scale;
+			r.y = (m * d.y - sum1 - sum2 * z.y) * scale;
+			r.z = (m * d.z - sum1 - sum2 * z.z) * scale;
+			r.w = (m * d.w - sum1 - sum2 * z.w) * scale;
+			*reinterpret_cast<float4 *>(po + i) = r;
+			acc += (double)((r.x + r.y) + (r.z + r.w));
+		}
+		long tail = lo + ((hi - lo) / 4) * 4;
+		for (long i = tail + threadIdx.x; i < hi; i += kRedBlock) {
+			float r = (m * pd[i] - sum1 - sum2 * pz[i]) * scale;
+			po[i] = r;
+			acc += (double)r;
+		}
+	} else {
+		for (long i = lo + threadIdx.x; i < hi; i += kRedBlock) {
+			float r = (m * pd[i] - sum1 - sum2 * pz[i]) * scale;
+			po[i] = r;
+			acc += (double)r;
+		}
+	}
+	if (partialOut) {
+		double t = block_sum<kRedBlock>(acc, lds);
+		if (threadIdx.x == 0) partialOut[((size_t)c * gridDim.x + blockIdx.x) * 2] = t;
+	}
+}
+
+static inline bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
+
+// =====================================================================
+// softmax cross entropy
+// =====================================================================
+
+// one wave per row; classes strided over the lanes
+__global__ void __launch_bounds__(256)
+softmax_ce_kernel(const float *logits, const float *target, int rows, int classes, float *probs, float *errors, float *nll)
+{
+	const int lane = threadIdx.x % kWave;
+	const int row = blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
+	if (row >= rows) return;
+	const float *in = logits + (size_t)row * classes;
+	float mx = -FLT_MAX;
+	for (int c = lane; c < classes; c += kWave) mx = fmaxf(mx, in[c]);
+	mx = wave_max(mx);
+	float s = 0.f;
+	for (int c = lane; c < classes; c += kWave) s += expf(in[c] - mx);
+	s = wave_sum(s);
+	const float inv = 1.f / s;
+	const int label = (int)target[row]; // 1-based
+	const float invRows = 1.f / (float)rows;
+	for (int c = lane; c < classes; c += kWave) {
+		float p = expf(in[c] - mx) * inv + 1e-10f;
+		probs[(size_t)row * classes + c] = p;
+		if (errors) errors[(size_t)row * classes + c] = (((c + 1) == label) ? p - 1.f : p) * invRows;
+		if ((c + 1) == label) nll[row] = -logf(p);
+	}
+	if (lane == 0 && (label < 1 || label > classes)) nll[row] = 0.f;
+}
+
+__global__ void cross_entropy_error_kernel(const float *probs, const float *target, int rows, int classes, float *errors)
+{
+	long total = (long)rows * classes;
+	long stride = (long)gridDim.x * blockDim.x;
+	const float invRows = 1.f / (float)rows;
+	for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+		int r = (int)(i / classes), c = (int)(i - (long)r * classes);
+		float p = probs[i];
+		errors[i] = (((float)(c + 1) == target[r]) ? p - 1.f : p) * invRows;
+	}
+}
+
+__global__ void __launch_bounds__(256) mean_kernel(const float *x, int n, float *out)
+{
+	__shared__ double lds[4];
+	double acc = 0.0;
+	for (int i = threadIdx.x; i < n; i += 256) acc += (double)x[i];
+	double t = block_sum<256>(acc, lds);
+	if (threadIdx.x == 0) out[0] = (float)(t / (double)n);
+}
+
+static float *g_nll = nullptr;
+static int g_nll_rows = 0;
+static float *g_loss_host = nullptr;
+
+// =====================================================================
+// layout changes
+// =====================================================================
+
+// [right][left][chunk] -> [left][right][chunk]
+__global__ void reshape_kernel(const float *in, int right, int left, int chunk, float *out)
+{
+	long total = (long)right * left * chunk;
+	long stride = (long)gridDim.x * blockDim.x;
+	for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+		long t = i % chunk;
+		long q = i / chunk;
+		long l = q % left, r = q / left;
+		out[(l * right + r) * chunk + t] = in[i];
+	}
+}
+
+// TO_FC: in [C][N][a*B+b] -> out [N][C][b*A+a];  otherwise the inverse.
+template <bool TO_FC>
+__global__ void boundary_permute_kernel(const float *in, int C, int N, int A, int B, float *out)
+{
+	long total = (long)C * N * A * B;
+	long stride = (long)gridDim.x * blockDim.x;
+	for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+		// i enumerates the output
+		long inner = i % ((long)A * B);
+		long outer = i / ((long)A * B);
+		if constexpr (TO_FC) {
+			long c = outer % C, n = outer / C;
+			long a = inner % A, b = inner / A;
+			out[i] = in[((c * N + n) * A + a) * B + b];
+		} else {
+			long n = outer % N, c = outer / N;
+			long b = inner % B, a = inner / B;
+			out[i] = in[((n * C + c) * B + b) * A + a];
+		}
+	}
+}
+
+} // namespace fitre
+
+using namespace fitre;
+
+extern "C" {
+
+int fitre_hip_pool_forward(int poolType, const float *in, int channels, int samples, int inA, int inB, int ksize,
+                           int stride, int padding, int outA, int outB, float *out)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(in && out, "fitre_hip_pool_forward: null pointer");
+	int rc = check_pool_shape("fitre_hip_pool_forward", channels, samples, inA, inB, ksize, stride, padding, outA, outB);
+	if (rc) return rc;
+	PoolGeom g = make_geom(inA, inB, ksize, stride, padding, outA, outB);
+	long maps = (long)channels * samples;
+	long total = maps * outA * outB;
+	LaunchScope scope(FITRE_KC_POOL_FWD, 4.0 * (double)(maps * inA * inB + total));
+	if (poolType == MAX_POOL)
+		pool_forward_kernel<0><<<blocks_for(total, 512, 8192), 256, 0, stream()>>>(in, g, maps, out, nullptr);
+	else if (poolType == AVG_POOL)
+		pool_forward_kernel<1><<<blocks_for(total, 512, 8192), 256, 0, stream()>>>(in, g, maps, out, nullptr);
+	else
+		return fail(FITRE_E_UNSUPPORTED, "fitre_hip_pool_forward: unknown pool type %d", poolType);
+	return check_launch("pool_forward_kernel");
+}
+
+int fitre_hip_max_pool_argmax(const float *z_in, int channels, int samples, int inA, int inB, int ksize, int stride,
+                              int padding, int outA, int outB, int *index)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(z_in && index, "fitre_hip_max_pool_argmax: null pointer");
+	int rc = check_pool_shape("fitre_hip_max_pool_argmax", channels, samples, inA, inB, ksize, stride, padding, outA, outB);
+	if (rc) return rc;
+	PoolGeom g = make_geom(inA, inB, ksize, stride, padding, outA, outB);
+	long maps = (long)channels * samples;
+	long total = maps * outA * outB;
+	LaunchScope scope(FITRE_KC_POOL_FWD, 4.0 * (double)(maps * inA * inB + total));
+	pool_forward_kernel<2><<<blocks_for(total, 512, 8192), 256, 0, stream()>>>(z_in, g, maps, nullptr, index);
+	return check_launch("pool_forward_kernel<argmax>");
+}
+
+int fitre_hip_pool_act_backward(int poolType, int actFun, const float *delta, const float *z_in, const float *z_act,
+                                int channels, int samples, int inA, int inB, int ksize, int stride, int padding,
+                                int outA, int outB, float *dxPool, float *dxAct)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(delta && dxAct, "fitre_hip_pool_act_backward: null pointer");
+	FITRE_REQUIRE(act_known(actFun), "fitre_hip_pool_act_backward: unknown activation code %d", actFun);
+	FITRE_REQUIRE(!act_needs_zin(actFun) || z_in, "fitre_hip_pool_act_backward: activation %d needs z_in", actFun);
+	FITRE_REQUIRE(!(act_needs_zout(actFun) || poolType == MAX_POOL) || z_act,
+	              "fitre_hip_pool_act_backward: z_act is required");
+	long maps = (long)channels * samples;
+	long total = maps * inA * inB;
+	if (poolType == NO_POOL) {
+		FITRE_REQUIRE(channels > 0 && samples > 0 && inA > 0 && inB > 0, "fitre_hip_pool_act_backward: non-positive shape");
+		FITRE_REQUIRE((double)total < 2147483647.0, "fitre_hip_pool_act_backward: tensor exceeds 2^31 elements");
+	} else {
+		int rc = check_pool_shape("fitre_hip_pool_act_backward", channels, samples, inA, inB, ksize, stride, padding, outA, outB);
+		if (rc) return rc;
+	}
+	PoolGeom g = make_geom(inA, inB, ksize > 0 ? ksize : 1, stride > 0 ? stride : 1, padding, outA > 0 ? outA : 1, outB > 0 ? outB : 1);
+	double bytes = 4.0 * (double)total * (1 + (dxPool ? 1 : 0) + (act_needs_zin(actFun) ? 1 : 0) + 1) +
+	               4.0 * (double)maps * (poolType == NO_POOL ? inA * inB : outA * outB);
+	LaunchScope scope(FITRE_KC_POOL_ACT_BWD, bytes);
+	unsigned blocks = blocks_for(total, 512, 16384);
+	if (poolType == MAX_POOL) {
+		bool fast = ksize == 2 && stride == 2 && padding == 0 && (inB % 4 == 0) && (inA % 2 == 0) && aligned16(z_act) &&
+		            aligned16(dxAct) && (!dxPool || aligned16(dxPool)) && (!z_in || aligned16(z_in)) &&
+		            (((uintptr_t)delta & 7) == 0);
+		if (fast)
+			maxpool2_backward_kernel<true><<<blocks_for(total / 8, 256, 16384), 256, 0, stream()>>>(
+			    delta, act_needs_zin(actFun) ? z_in : nullptr, z_act, inA, inB, maps, actFun, dxPool, dxAct);
+		else
+			pool_backward_kernel<0, true><<<blocks, 256, 0, stream()>>>(delta, z_in, z_act, g, maps, actFun, dxPool, dxAct);
+	} else if (poolType == AVG_POOL) {
+		pool_backward_kernel<1, true><<<blocks, 256, 0, stream()>>>(delta, z_in, z_act, g, maps, actFun, dxPool, dxAct);
+	} else if (poolType == NO_POOL) {
+		pool_backward_kernel<2, true><<<blocks, 256, 0, stream()>>>(delta, z_in, z_act, g, maps, actFun, dxPool, dxAct);
+	} else {
+		return fail(FITRE_E_UNSUPPORTED, "fitre_hip_pool_act_backward: unknown pool type %d", poolType);
+	}
+	return check_launch("pool_act_backward");
+}
+
+int fitre_hip_pool_backward(int poolType, const float *delta, const float *z_in, int channels, int samples, int inA,
+                            int inB, int ksize, int stride, int padding, int outA, int outB, float *out)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(delta && out, "fitre_hip_pool_backward: null pointer");
+	FITRE_REQUIRE(poolType != MAX_POOL || z_in, "fitre_hip_pool_backward: max pooling needs the pool input");
+	int rc = check_pool_shape("fitre_hip_pool_backward", channels, samples, inA, inB, ksize, stride, padding, outA, outB);
+	if (rc) return rc;
+	PoolGeom g = make_geom(inA, inB, ksize, stride, padding, outA, outB);
+	long maps = (long)channels * samples;
+	long total = maps * inA * inB;
+	LaunchScope scope(FITRE_KC_POOL_BWD, 4.0 * (double)(total * (poolType == MAX_POOL ? 2 : 1) + maps * outA * outB));
+	unsigned blocks = blocks_for(total, 512, 16384);
+	if (poolType == MAX_POOL) {
+		bool fast = ksize == 2 && stride == 2 && padding == 0 && (inB % 4 == 0) && (inA % 2 == 0) && aligned16(z_in) &&
+		            aligned16(out) && (((uintptr_t)delta & 7) == 0);
+		if (fast)
+			maxpool2_backward_kernel<false><<<blocks_for(total / 8, 256, 16384), 256, 0, stream()>>>(
+			    delta, nullptr, z_in, inA, inB, maps, CNN_ACT_NONE, out, nullptr);
+		else
+			pool_backward_kernel<0, false><<<blocks, 256, 0, stream()>>>(delta, nullptr, z_in, g, maps, CNN_ACT_NONE, out, nullptr);
+	} else if (poolType == AVG_POOL) {
+		pool_backward_kernel<1, false><<<blocks, 256, 0, stream()>>>(delta, nullptr, nullptr, g, maps, CNN_ACT_NONE, out, nullptr);
+	} else {
+		return fail(FITRE_E_UNSUPPORTED, "fitre_hip_pool_backward: unknown pool type %d", poolType);
+	}
+	return check_launch("pool_backward_kernel");
+}
+
+size_t fitre_hip_batch_norm_workspace(int channels, long perChannel)
+{
+	if (channels <= 0 || perChannel <= 0) return 0;
+	return (size_t)channels * segments_for(channels, perChannel) * 2 * sizeof(double) * 2 + 64;
+}
+
+size_t fitre_hip_channel_sum_workspace(int channels, long perChannel)
+{
+	return fitre_hip_batch_norm_workspace(channels, perChannel);
+}
+
+static int check_channels(const char *fn, int channels, long perChannel, void *ws, size_t wsBytes)
+{
+	FITRE_REQUIRE(channels > 0 && perChannel > 0, "%s: non-positive shape (channels=%d, perChannel=%ld)", fn, channels, perChannel);
+	FITRE_REQUIRE(channels <= 65535, "%s: %d channels exceed the grid limit", fn, channels);
+	FITRE_REQUIRE(ws != nullptr && (((uintptr_t)ws) & 7) == 0, "%s: workspace is null or not 8-byte aligned", fn);
+	if (wsBytes < fitre_hip_batch_norm_workspace(channels, perChannel))
+		return fail(FITRE_E_WORKSPACE, "%s: workspace of %zu bytes is smaller than the %zu required", fn, wsBytes,
+		            fitre_hip_batch_norm_workspace(channels, perChannel));
+	return FITRE_OK;
+}
+
+int fitre_hip_channel_sum(const float *x, int channels, long perChannel, float *out, void *ws, size_t wsBytes)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(x && out, "fitre_hip_channel_sum: null pointer");
+	int rc = check_channels("fitre_hip_channel_sum", channels, perChannel, ws, wsBytes);
+	if (rc) return rc;
+	int S = segments_for(channels, perChannel);
+	double *partial = (double *)ws;
+	LaunchScope scope(FITRE_KC_BIAS_GRAD, 4.0 * (double)channels * (double)perChannel);
+	dim3 grid(S, channels);
+	bool vec = aligned16(x) && (perChannel % 4 == 0);
+	if (vec)
+		channel_partial_kernel<0, true><<<grid, kRedBlock, 0, stream()>>>(x, nullptr, perChannel, partial);
+	else
+		channel_partial_kernel<0, false><<<grid, kRedBlock, 0, stream()>>>(x, nullptr, perChannel, partial);
+	channel_finish_kernel<<<blocks_for(channels, 64), 64, 0, stream()>>>(partial, S, 0, channels, out);
+	return check_launch("channel_sum");
+}
+
+int fitre_hip_batch_norm_forward(const float *in, int channels, long perChannel, float *zhat, float *mean, float *variance,
+                                 float *runningMean, float *runningVariance, float epsilon, float momentum, int train,
+                                 void *ws, size_t wsBytes)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(in && zhat && mean && variance && runningMean && runningVariance, "fitre_hip_batch_norm_forward: null pointer");
+	int rc = check_channels("fitre_hip_batch_norm_forward", channels, perChannel, ws, wsBytes);
+	if (rc) return rc;
+	int S = segments_for(channels, perChannel);
+	double *partial = (double *)ws;
+	LaunchScope scope(FITRE_KC_BN_FWD, 4.0 * (double)channels * (double)perChannel * (train ? 3 : 2));
+	dim3 grid(S, channels);
+	bool vec = aligned16(in) && aligned16(zhat) && (perChannel % 4 == 0);
+	if (train) {
+		if (vec)
+			channel_partial_kernel<2, true><<<grid, kRedBlock, 0, stream()>>>(in, nullptr, perChannel, partial);
+		else
+			channel_partial_kernel<2, false><<<grid, kRedBlock, 0, stream()>>>(in, nullptr, perChannel, partial);
+		bn_stats_kernel<<<blocks_for(channels, 64), 64, 0, stream()>>>(partial, S, channels, perChannel, momentum, mean,
+		                                                            variance, runningMean, runningVariance);
+	}
+	const float *mu = train ? mean : runningMean;
+	const float *var = train ? variance : runningVariance;
+	if (vec)
+		bn_normalize_kernel<true><<<grid, kRedBlock, 0, stream()>>>(in, mu, var, epsilon, perChannel, zhat);
+	else
+		bn_normalize_kernel<false><<<grid, kRedBlock, 0, stream()>>>(in, mu, var, epsilon, perChannel, zhat);
+	return check_launch("batch_norm_forward");
+}
+
+int fitre_hip_batch_norm_backward(const float *delta, const float *zhat, const float *variance, int channels,
+                                  long perChannel, float epsilon, float *out, float *biasGrad, void *ws, size_t wsBytes)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(delta && zhat && variance && out, "fitre_hip_batch_norm_backward: null pointer");
+	int rc = check_channels("fitre_hip_batch_norm_backward", channels, perChannel, ws, wsBytes);
+	if (rc) return rc;
+	int S = segments_for(channels, perChannel);
+	double *partial = (double *)ws;
+	double *partialOut = partial + (size_t)channels * S * 2;
+	LaunchScope scope(FITRE_KC_BN_BWD, 12.0 * (double)channels * (double)perChannel + 8.0 * channels);
+	dim3 grid(S, channels);
+	bool vec = aligned16(delta) && aligned16(zhat) && aligned16(out) && (perChannel % 4 == 0);
+	if (vec) {
+		channel_partial_kernel<1, true><<<grid, kRedBlock, 0, stream()>>>(delta, zhat, perChannel, partial);
+		bn_backward_apply_kernel<true><<<grid, kRedBlock, 0, stream()>>>(delta, zhat, variance, partial, S, epsilon, perChannel,
+		                                                                 out, biasGrad ? partialOut : nullptr);
+	} else {
+		channel_partial_kernel<1, false><<<grid, kRedBlock, 0, stream()>>>(delta, zhat, perChannel, partial);
+		bn_backward_apply_kernel<false><<<grid, kRedBlock, 0, stream()>>>(delta, zhat, variance, partial, S, epsilon, perChannel,
+		                                                                  out, biasGrad ? partialOut : nullptr);
+	}
+	if (biasGrad) channel_finish_kernel<<<blocks_for(channels, 64), 64, 0, stream()>>>(partialOut, S, 0, channels, biasGrad);
+	return check_launch("batch_norm_backward");
+}
+
+int fitre_hip_softmax_cross_entropy(const float *logits, const float *target, int rows, int classes, float *probs,
+                                    float *errors, float *lossHost)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(logits && target && probs && lossHost, "fitre_hip_softmax_cross_entropy: null pointer");
+	FITRE_REQUIRE(rows > 0 && classes > 0, "fitre_hip_softmax_cross_entropy: non-positive shape (%d x %d)", rows, classes);
+	if (rows > g_nll_rows) {
+		FITRE_HIP_TRY(hipStreamSynchronize(stream()));
+		if (g_nll) FITRE_HIP_TRY(hipFree(g_nll));
+		g_nll = nullptr;
+		g_nll_rows = 0;
+		int cap = rows < 4096 ? 4096 : rows;
+		FITRE_HIP_TRY(hipMalloc((void **)&g_nll, sizeof(float) * ((size_t)cap + 16)));
+		g_nll_rows = cap;
+	}
+	if (!g_loss_host) FITRE_HIP_TRY(hipHostMalloc((void **)&g_loss_host, 64, hipHostMallocDefault));
+	{
+		LaunchScope scope(FITRE_KC_SOFTMAX, 4.0 * rows * classes * 2);
+		softmax_ce_kernel<<<blocks_for(rows, 4), 256, 0, stream()>>>(logits, target, rows, classes, probs, errors, g_nll);
+		mean_kernel<<<1, 256, 0, stream()>>>(g_nll, rows, g_nll + g_nll_rows);
+		int rc = check_launch("softmax_ce_kernel");
+		if (rc) return rc;
+	}
+	FITRE_HIP_TRY(hipMemcpyAsync(g_loss_host, g_nll + g_nll_rows, sizeof(float), hipMemcpyDeviceToHost, stream()));
+	FITRE_HIP_TRY(hipStreamSynchronize(stream()));
+	*lossHost = *g_loss_host;
+	return FITRE_OK;
+}
+
+int fitre_hip_cross_entropy_error(const float *probs, const float *target, int rows, int classes, float *errors)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(probs && target && errors, "fitre_hip_cross_entropy_error: null pointer");
+	FITRE_REQUIRE(rows > 0 && classes > 0, "fitre_hip_cross_entropy_error: non-positive shape (%d x %d)", rows, classes);
+	LaunchScope scope(FITRE_KC_SOFTMAX, 8.0 * rows * classes);
+	cross_entropy_error_kernel<<<blocks_for((long)rows * classes, 256, 4096), 256, 0, stream()>>>(probs, target, rows, classes, errors);
+	return check_launch("cross_entropy_error_kernel");
+}
+
+int fitre_hip_reshape(const float *in, int right, int left, int chunk, float *out)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(in && out && in != out, "fitre_hip_reshape: null or aliased pointers");
+	FITRE_REQUIRE(right > 0 && left > 0 && chunk > 0, "fitre_hip_reshape: non-positive shape");
+	long total = (long)right * left * chunk;
+	LaunchScope scope(FITRE_KC_PERMUTE, 8.0 * total);
+	reshape_kernel<<<blocks_for(total, 512, 8192), 256, 0, stream()>>>(in, right, left, chunk, out);
+	return check_launch("reshape_kernel");
+}
+
+int fitre_hip_conv_to_fc(const float *in, int channels, int samples, int extA, int extB, float *out)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(in && out && in != out, "fitre_hip_conv_to_fc: null or aliased pointers");
+	FITRE_REQUIRE(channels > 0 && samples > 0 && extA > 0 && extB > 0, "fitre_hip_conv_to_fc: non-positive shape");
+	long total = (long)channels * samples * extA * extB;
+	LaunchScope scope(FITRE_KC_PERMUTE, 8.0 * total);
+	boundary_permute_kernel<true><<<blocks_for(total, 512, 8192), 256, 0, stream()>>>(in, channels, samples, extA, extB, out);
+	return check_launch("boundary_permute_kernel");
+}
+
+int fitre_hip_fc_to_conv(const float *in, int channels, int samples, int extA, int extB, float *out)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(in && out && in != out, "fitre_hip_fc_to_conv: null or aliased pointers");
+	FITRE_REQUIRE(channels > 0 && samples > 0 && extA > 0 && extB > 0, "fitre_hip_fc_to_conv: non-positive shape");
+	long total = (long)channels * samples * extA * extB;
+	LaunchScope scope(FITRE_KC_PERMUTE, 8.0 * total);
+	boundary_permute_kernel<false><<<blocks_for(total, 512, 8192), 256, 0, stream()>>>(in, channels, samples, extA, extB, out);
+	return check_launch("boundary_permute_kernel");
+}
+
+} // extern "C"

@@ -1,0 +1,326 @@
+// Environment, memory and timing entry points of the device layer.
+// Replaces device/cuda_environment.c, device/cuda_utils.c and device/query.c
+// of the reference (handles become one stream owned by this file).
+#include <stdarg.h>
+#include <string.h>
+#include <vector>
+#include "common.h"
+
+namespace fitre {
+
+static thread_local char g_error[512] = "";
+static hipStream_t g_stream = nullptr;
+static bool g_ready = false;
+static int g_device = -1;
+
+// accounting state
+struct ClassTotals {
+	long launches;
+	double ms;
+	double work;
+};
+static bool g_profile = false;
+static ClassTotals g_totals[FITRE_KC_COUNT];
+struct Pending {
+	hipEvent_t start, stop;
+	int cls;
+};
+static std::vector<Pending> g_pending;
+static std::vector<hipEvent_t> g_event_pool;
+
+void set_error(const char *fmt, ...)
+{
+	va_list ap;
+	va_start(ap, fmt);
+	vsnprintf(g_error, sizeof(g_error), fmt, ap);
+	va_end(ap);
+}
+
+int fail(int code, const char *fmt, ...)
+{
+	va_list ap;
+	va_start(ap, fmt);
+	vsnprintf(g_error, sizeof(g_error), fmt, ap);
+	va_end(ap);
+	return code;
+}
+
+hipStream_t stream() { return g_stream; }
+bool ready() { return g_ready; }
+
+int check_launch(const char *what)
+{
+	hipError_t e = hipGetLastError();
+	if (e != hipSuccess) return fail(FITRE_E_DEVICE, "launch of %s failed: %s", what, hipGetErrorString(e));
+	return FITRE_OK;
+}
+
+static hipEvent_t take_event()
+{
+	if (!g_event_pool.empty()) {
+		hipEvent_t e = g_event_pool.back();
+		g_event_pool.pop_back();
+		return e;
+	}
+	hipEvent_t e = nullptr;
+	if (hipEventCreate(&e) != hipSuccess) return nullptr;
+	return e;
+}
+
+static void drain_pending()
+{
+	for (Pending &p : g_pending) {
+		float ms = 0.f;
+		if (hipEventSynchronize(p.stop) == hipSuccess && hipEventElapsedTime(&ms, p.start, p.stop) == hipSuccess)
+			g_totals[p.cls].ms += ms;
+		g_event_pool.push_back(p.start);
+		g_event_pool.push_back(p.stop);
+	}
+	g_pending.clear();
+}
+
+LaunchScope::LaunchScope(int kernelClass, double work) : slot(-1)
+{
+	if (!g_profile || kernelClass < 0 || kernelClass >= FITRE_KC_COUNT) return;
+	Pending p;
+	p.start = take_event();
+	p.stop = take_event();
+	p.cls = kernelClass;
+	if (!p.start || !p.stop) return;
+	g_totals[kernelClass].launches += 1;
+	g_totals[kernelClass].work += work;
+	(void)hipEventRecord(p.start, g_stream);
+	g_pending.push_back(p);
+	slot = (int)g_pending.size() - 1;
+}
+
+LaunchScope::~LaunchScope()
+{
+	if (slot < 0) return;
+	(void)hipEventRecord(g_pending[slot].stop, g_stream);
+	if (g_pending.size() >= 2048) drain_pending();
+}
+
+// Byte fill as a kernel: a memset node recorded into a captured graph is not
+// reliable on this platform, a kernel node is.
+__global__ void fill_bytes_kernel(unsigned char *p, unsigned char v, size_t n)
+{
+	size_t words = n / 16;
+	uint4 *p16 = reinterpret_cast<uint4 *>(p);
+	unsigned w = v * 0x01010101u;
+	size_t stride = (size_t)gridDim.x * blockDim.x;
+	for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < words; i += stride)
+		p16[i] = make_uint4(w, w, w, w);
+	for (size_t i = words * 16 + (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) p[i] = v;
+}
+
+} // namespace fitre
+
+using namespace fitre;
+
+extern "C" {
+
+int fitre_hip_init(int device)
+{
+	int count = 0;
+	FITRE_HIP_TRY(hipGetDeviceCount(&count));
+	if (device < 0 || device >= count)
+		return fail(FITRE_E_ARGUMENT, "fitre_hip_init: device %d out of range (%d visible)", device, count);
+	FITRE_HIP_TRY(hipSetDevice(device));
+	if (g_ready && g_device == device) return FITRE_OK;
+	if (g_ready) fitre_hip_shutdown();
+	FITRE_HIP_TRY(hipStreamCreate(&g_stream)); // default priority, ordered with the null stream
+	g_device = device;
+	g_ready = true;
+	memset(g_totals, 0, sizeof(g_totals));
+	return FITRE_OK;
+}
+
+int fitre_hip_shutdown(void)
+{
+	if (!g_ready) return FITRE_OK;
+	(void)hipStreamSynchronize(g_stream);
+	drain_pending();
+	for (hipEvent_t e : g_event_pool) (void)hipEventDestroy(e);
+	g_event_pool.clear();
+	(void)hipStreamDestroy(g_stream);
+	g_stream = nullptr;
+	g_ready = false;
+	g_profile = false;
+	return FITRE_OK;
+}
+
+int fitre_hip_sync(void)
+{
+	FITRE_NEED_INIT();
+	FITRE_HIP_TRY(hipStreamSynchronize(g_stream));
+	return FITRE_OK;
+}
+
+const char *fitre_hip_last_error(void) { return g_error; }
+
+void *fitre_hip_stream(void) { return (void *)g_stream; }
+
+int fitre_hip_device_info(int *computeUnits, int *waveSize, int *maxThreadsPerBlock, size_t *totalBytes,
+                          size_t *freeBytes, char *name, int nameLen)
+{
+	FITRE_NEED_INIT();
+	hipDeviceProp_t prop;
+	FITRE_HIP_TRY(hipGetDeviceProperties(&prop, g_device));
+	if (computeUnits) *computeUnits = prop.multiProcessorCount;
+	if (waveSize) *waveSize = prop.warpSize;
+	if (maxThreadsPerBlock) *maxThreadsPerBlock = prop.maxThreadsPerBlock;
+	size_t fr = 0, tot = 0;
+	FITRE_HIP_TRY(hipMemGetInfo(&fr, &tot));
+	if (totalBytes) *totalBytes = tot;
+	if (freeBytes) *freeBytes = fr;
+	if (name && nameLen > 0) {
+		snprintf(name, (size_t)nameLen, "%s (%s)", prop.name, prop.gcnArchName);
+	}
+	return FITRE_OK;
+}
+
+int fitre_hip_malloc(void **ptr, size_t bytes)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(ptr != nullptr, "fitre_hip_malloc: null result pointer");
+	FITRE_REQUIRE(bytes > 0, "fitre_hip_malloc: zero bytes requested");
+	FITRE_HIP_TRY(hipMalloc(ptr, bytes));
+	return FITRE_OK;
+}
+
+int fitre_hip_free(void *ptr)
+{
+	FITRE_NEED_INIT();
+	if (!ptr) return FITRE_OK;
+	FITRE_HIP_TRY(hipStreamSynchronize(g_stream));
+	FITRE_HIP_TRY(hipFree(ptr));
+	return FITRE_OK;
+}
+
+int fitre_hip_malloc_host(void **ptr, size_t bytes)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(ptr != nullptr, "fitre_hip_malloc_host: null result pointer");
+	FITRE_REQUIRE(bytes > 0, "fitre_hip_malloc_host: zero bytes requested");
+	FITRE_HIP_TRY(hipHostMalloc(ptr, bytes, hipHostMallocDefault));
+	return FITRE_OK;
+}
+
+int fitre_hip_free_host(void *ptr)
+{
+	FITRE_NEED_INIT();
+	if (!ptr) return FITRE_OK;
+	FITRE_HIP_TRY(hipStreamSynchronize(g_stream));
+	FITRE_HIP_TRY(hipHostFree(ptr));
+	return FITRE_OK;
+}
+
+int fitre_hip_memset(void *ptr, int value, size_t bytes)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(ptr != nullptr, "fitre_hip_memset: null pointer");
+	if (bytes == 0) return FITRE_OK;
+	unsigned char *p = (unsigned char *)ptr;
+	// head up to 16-byte alignment, then the aligned body
+	size_t head = (16 - ((uintptr_t)p & 15)) & 15;
+	if (head > bytes) head = bytes;
+	if (head) {
+		fill_bytes_kernel<<<1, 64, 0, g_stream>>>(p, (unsigned char)value, head);
+		p += head;
+		bytes -= head;
+	}
+	if (bytes) {
+		unsigned blocks = blocks_for((long)(bytes / 16 + 1), 256, 4096);
+		fill_bytes_kernel<<<blocks, 256, 0, g_stream>>>(p, (unsigned char)value, bytes);
+	}
+	return check_launch("fill_bytes_kernel");
+}
+
+int fitre_hip_copy_h2d(void *dev, const void *host, size_t bytes)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(dev && host, "fitre_hip_copy_h2d: null pointer");
+	if (bytes == 0) return FITRE_OK;
+	FITRE_HIP_TRY(hipMemcpyAsync(dev, host, bytes, hipMemcpyHostToDevice, g_stream));
+	FITRE_HIP_TRY(hipStreamSynchronize(g_stream));
+	return FITRE_OK;
+}
+
+int fitre_hip_copy_d2h(void *host, const void *dev, size_t bytes)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(dev && host, "fitre_hip_copy_d2h: null pointer");
+	if (bytes == 0) return FITRE_OK;
+	FITRE_HIP_TRY(hipMemcpyAsync(host, dev, bytes, hipMemcpyDeviceToHost, g_stream));
+	FITRE_HIP_TRY(hipStreamSynchronize(g_stream));
+	return FITRE_OK;
+}
+
+int fitre_hip_copy_d2d(void *dst, const void *src, size_t bytes)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(dst && src, "fitre_hip_copy_d2d: null pointer");
+	if (bytes == 0 || dst == src) return FITRE_OK;
+	FITRE_HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, g_stream));
+	return FITRE_OK;
+}
+
+int fitre_hip_event_create(void **event)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(event != nullptr, "fitre_hip_event_create: null result pointer");
+	hipEvent_t e;
+	FITRE_HIP_TRY(hipEventCreate(&e));
+	*event = (void *)e;
+	return FITRE_OK;
+}
+
+int fitre_hip_event_destroy(void *event)
+{
+	FITRE_NEED_INIT();
+	if (!event) return FITRE_OK;
+	FITRE_HIP_TRY(hipEventDestroy((hipEvent_t)event));
+	return FITRE_OK;
+}
+
+int fitre_hip_event_record(void *event)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(event != nullptr, "fitre_hip_event_record: null event");
+	FITRE_HIP_TRY(hipEventRecord((hipEvent_t)event, g_stream));
+	return FITRE_OK;
+}
+
+int fitre_hip_event_elapsed_ms(void *start, void *stop, float *ms)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(start && stop && ms, "fitre_hip_event_elapsed_ms: null argument");
+	FITRE_HIP_TRY(hipEventSynchronize((hipEvent_t)stop));
+	FITRE_HIP_TRY(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
+	return FITRE_OK;
+}
+
+int fitre_hip_profile_enable(int on)
+{
+	FITRE_NEED_INIT();
+	FITRE_HIP_TRY(hipStreamSynchronize(g_stream));
+	drain_pending();
+	if (on) memset(g_totals, 0, sizeof(g_totals));
+	g_profile = (on != 0);
+	return FITRE_OK;
+}
+
+int fitre_hip_profile_read(int kernelClass, long *launches, double *milliseconds, double *work)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(kernelClass >= 0 && kernelClass < FITRE_KC_COUNT, "fitre_hip_profile_read: class %d unknown", kernelClass);
+	FITRE_HIP_TRY(hipStreamSynchronize(g_stream));
+	drain_pending();
+	if (launches) *launches = g_totals[kernelClass].launches;
+	if (milliseconds) *milliseconds = g_totals[kernelClass].ms;
+	if (work) *work = g_totals[kernelClass].work;
+	return FITRE_OK;
+}
+
+} // extern "C"

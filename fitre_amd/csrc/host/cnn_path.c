@@ -1,0 +1,313 @@
+/*
+ * cnnForward / cnnBackward / computeCNNGradient: the model-level passes of the
+ * gradient path, as C host code over the C-ABI device layer.
+ *
+ * Data flow and z / dx contents follow functions/cnn_forward.cu:49-383,
+ * functions/cnn_backward.cu:76-857 and functions/cnn_gradient.cu:13-64 of the
+ * reference; what differs is below the layer calls: no patch matrices, no
+ * ones-vector products, no staging copies -- the dx slots themselves are the
+ * working buffers of the backward pass.
+ */
+#include <stdio.h>
+#include <stdlib.h>
+#include "fitre_cnn.h"
+#include "fitre_hip.h"
+
+#define HIP_CALL(expr)                                                                               \
+	do {                                                                                             \
+		int rc_ = (expr);                                                                            \
+		if (rc_ != FITRE_OK) {                                                                       \
+			fprintf(stderr, "%s:%d: %s -> error %d: %s\n", __FILE__, __LINE__, #expr, rc_,           \
+			        fitre_hip_last_error());                                                         \
+			exit(-1);                                                                                \
+		}                                                                                            \
+	} while (0)
+
+static int has_bn(const CONV_LAYER *c) { return c->batchNorm != PERFORM_NO_BATCH_NORM; }
+
+static fitre_conv_shape conv_shape(const CONV_LAYER *l, int samples)
+{
+	fitre_conv_shape s;
+	s.samples = samples;
+	s.inChannels = l->inChannels;
+	s.outChannels = l->outChannels;
+	s.inA = l->width; /* A = image column index, B = image row index (fastest) */
+	s.inB = l->height;
+	s.outA = l->outWidth;
+	s.outB = l->outHeight;
+	s.ksize = l->kSize;
+	s.stride = l->stride;
+	s.padding = l->padding;
+	return s;
+}
+
+static size_t max_sz(size_t a, size_t b) { return a > b ? a : b; }
+
+/* extent of the feature map handed to the first FC layer */
+static void feature_extent(const CNN_MODEL *model, int *extA, int *extB)
+{
+	const CONV_LAYER *c = &model->convLayer[model->cLayers - 1];
+	const POOL_LAYER *p = &model->poolLayer[model->cLayers - 1];
+	if (p->type != NO_POOL) {
+		*extA = p->outWidth;
+		*extB = p->outHeight;
+	} else {
+		*extA = c->outWidth;
+		*extB = c->outHeight;
+	}
+}
+
+static size_t forward_ws_bytes(const CNN_MODEL *model, int batch)
+{
+	size_t need = 256;
+	for (int i = 0; i < model->cLayers; i++) {
+		const CONV_LAYER *c = &model->convLayer[i];
+		fitre_conv_shape s = conv_shape(c, batch);
+		need = max_sz(need, fitre_hip_conv_forward_workspace(&s));
+		if (has_bn(c)) need = max_sz(need, fitre_hip_batch_norm_workspace(c->outChannels, (long)batch * c->outWidth * c->outHeight));
+	}
+	if (model->cLayers > 0) {
+		int extA, extB;
+		feature_extent(model, &extA, &extB);
+		need = max_sz(need, sizeof(real) * (size_t)extA * extB * batch * model->convLayer[model->cLayers - 1].outChannels);
+	}
+	for (int i = 0; i < model->lLayers; i++)
+		need = max_sz(need, fitre_hip_gemm_workspace(model->fcLayer[i].out, batch, model->fcLayer[i].in));
+	return need;
+}
+
+static size_t backward_ws_bytes(const CNN_MODEL *model, int batch)
+{
+	size_t need = 256;
+	for (int i = 0; i < model->cLayers; i++) {
+		const CONV_LAYER *c = &model->convLayer[i];
+		fitre_conv_shape s = conv_shape(c, batch);
+		need = max_sz(need, fitre_hip_conv_weight_grad_workspace(&s));
+		if (i != 0) need = max_sz(need, fitre_hip_conv_input_grad_workspace(&s));
+		need = max_sz(need, fitre_hip_batch_norm_workspace(c->outChannels, (long)batch * c->outWidth * c->outHeight));
+	}
+	for (int i = 0; i < model->lLayers; i++) {
+		const FC_LAYER *f = &model->fcLayer[i];
+		need = max_sz(need, fitre_hip_gemm_workspace(f->out, f->in, batch));
+		need = max_sz(need, fitre_hip_gemm_workspace(f->in, batch, f->out));
+	}
+	return need;
+}
+
+long cnnForwardMemRequired(CNN_MODEL *model)
+{
+	return (long)((forward_ws_bytes(model, model->batchSize) + sizeof(real) - 1) / sizeof(real));
+}
+
+long cnnBackwardMemRequired(CNN_MODEL *model)
+{
+	return (long)((backward_ws_bytes(model, model->batchSize) + sizeof(real) - 1) / sizeof(real));
+}
+
+real cnnForward(CNN_MODEL *model, DEVICE_DATASET *data, SCRATCH_AREA *scratch, real *z, real *probs, real *errors,
+                int s, int curBatchSize, EVAL_TYPE forTesting)
+{
+	(void)s;
+	const int *wOffsets = model->wOffsets, *bOffsets = model->bOffsets, *zOffsets = model->zOffsets;
+	const real *weights = data->weights;
+	const int nc = model->cLayers, n = curBatchSize;
+	void *ws = (void *)scratch->nextDevPtr;
+	const size_t wsBytes = sizeof(real) * (size_t)cnnForwardMemRequired(model);
+
+	if (forTesting != MODEL_TRAIN && forTesting != MODEL_TRAIN_ACCURACY && forTesting != MODEL_TEST_ACCURACY) {
+		fprintf(stderr, "Unknown EVAL_TYPE... \n\n");
+		exit(-1);
+	}
+	if (nc < 1 || n < 1 || n > model->batchSize) {
+		fprintf(stderr, "cnnForward: needs at least one convolution layer and 1 <= batch (%d) <= model batch (%d)\n", n,
+		        model->batchSize);
+		exit(-1);
+	}
+
+	for (int l = 0; l < nc; l++) {
+		const CONV_LAYER *cv = &model->convLayer[l];
+		const POOL_LAYER *pl = &model->poolLayer[l];
+		const real *in = (l == 0) ? data->currentBatch : z + zOffsets[l] + model->convLayer[l - 1].outputOffset;
+		real *slab = z + zOffsets[l + 1];
+		real *actOut = slab + cv->activationOffset;
+		const long perChannel = (long)n * cv->outWidth * cv->outHeight;
+		const long count = perChannel * cv->outChannels;
+		fitre_conv_shape shape = conv_shape(cv, n);
+
+		HIP_CALL(fitre_hip_conv_forward(&shape, in, weights + wOffsets[l],
+		                                (model->bias == 0) ? NULL : weights + bOffsets[l], slab, ws, wsBytes));
+		if (has_bn(cv)) {
+			real *bnOut = slab + cv->batchNormOffset;
+			HIP_CALL(fitre_hip_batch_norm_forward(slab, cv->outChannels, perChannel, bnOut, bnOut + cv->meansOffset,
+			                                      bnOut + cv->variancesOffset, bnOut + cv->runningMeansOffset,
+			                                      bnOut + cv->runningVariancesOffset, (real)BATCH_NORM_EPSILON,
+			                                      (real)BATCH_NORM_MOMENTUM, forTesting == MODEL_TRAIN, ws, wsBytes));
+			HIP_CALL(fitre_hip_activation_forward(model->actFuns[l], bnOut, actOut, count));
+		} else {
+			HIP_CALL(fitre_hip_activation_forward(model->actFuns[l], slab, actOut, count));
+		}
+		if (pl->type != NO_POOL)
+			HIP_CALL(fitre_hip_pool_forward(pl->type, actOut, cv->outChannels, n, pl->width, pl->height, pl->pSize,
+			                                pl->stride, pl->padding, pl->outWidth, pl->outHeight,
+			                                slab + cv->poolOffset));
+	}
+
+	/* [C][N][a*B+b] -> [N][C][b*A+a], in place through the workspace */
+	const CONV_LAYER *last = &model->convLayer[nc - 1];
+	int extA, extB;
+	feature_extent(model, &extA, &extB);
+	real *feat = z + zOffsets[nc] + last->outputOffset;
+	const size_t featCount = (size_t)extA * extB * n * last->outChannels;
+	HIP_CALL(fitre_hip_conv_to_fc(feat, last->outChannels, n, extA, extB, (real *)ws));
+	HIP_CALL(fitre_hip_copy_d2d(feat, ws, sizeof(real) * featCount));
+
+	int outputOffset = last->outputOffset;
+	for (int l = 0; l < model->lLayers; l++) {
+		if (l != 0) outputOffset = 0;
+		const FC_LAYER *f = &model->fcLayer[l];
+		real *out = z + zOffsets[l + 1 + nc];
+		const long count = (long)f->out * n;
+		/* W z + b, then the saved copy behind it, then the activation in place */
+		HIP_CALL(fitre_hip_gemm(0, 0, f->out, n, f->in, 1.f, weights + wOffsets[l + nc], f->out,
+		                        z + zOffsets[l + nc] + outputOffset, f->in, 0.f, out, f->out,
+		                        (model->bias == 0) ? NULL : weights + bOffsets[l + nc], ws, wsBytes));
+		HIP_CALL(fitre_hip_copy_d2d(out + count, out, sizeof(real) * (size_t)count));
+		HIP_CALL(fitre_hip_activation_forward(f->actFun, out, out, count));
+	}
+
+	const real *logits = (model->lLayers == 0) ? feat : z + zOffsets[model->lLayers + nc];
+	real loss = 0;
+	HIP_CALL(fitre_hip_softmax_cross_entropy(logits, data->sampledTrainY, n, data->numClasses, probs, errors, &loss));
+	HIP_CALL(fitre_hip_sync());
+	return loss;
+}
+
+void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, real *gradient, real *dx, real *delta,
+                 real *delta_new, int offset, int batchSize, real *hostPtr)
+{
+	(void)offset;
+	(void)hostPtr;
+	const int *wOffsets = model->wOffsets, *bOffsets = model->bOffsets, *zOffsets = model->zOffsets;
+	const real *weights = data->weights;
+	const int n = batchSize, nc = model->cLayers;
+	void *ws = (void *)devPtr;
+	const size_t wsBytes = sizeof(real) * (size_t)cnnBackwardMemRequired(model);
+	real *temp;
+
+	if (nc < 1 || n < 1 || n > model->batchSize) {
+		fprintf(stderr, "cnnBackward: needs at least one convolution layer and 1 <= batch (%d) <= model batch (%d)\n", n,
+		        model->batchSize);
+		exit(-1);
+	}
+	const CONV_LAYER *last = &model->convLayer[nc - 1];
+
+	for (int f = model->lLayers - 1; f >= 0; f--) {
+		const FC_LAYER *l = &model->fcLayer[f];
+		real *zl = z + zOffsets[f + nc + 1];
+		const long count = (long)l->out * n;
+		const real *zin = z + zOffsets[f + nc] + ((f == 0) ? last->outputOffset : 0);
+
+		/* delta *= f'(.) */
+		HIP_CALL(fitre_hip_activation_backward(l->actFun, delta, zl + l->offset, zl, delta, count));
+		/* dW = delta * z' */
+		HIP_CALL(fitre_hip_gemm(0, 1, l->out, l->in, n, 1.f, delta, l->out, zin, l->in, 0.f,
+		                        gradient + wOffsets[f + nc], l->out, NULL, ws, wsBytes));
+		/* db = delta * 1 */
+		if (model->bias != 0) HIP_CALL(fitre_hip_row_sum(delta, l->out, n, gradient + bOffsets[f + nc]));
+		/* snapshot kept for the Hessian-vector product and the KFAC factors */
+		HIP_CALL(fitre_hip_copy_d2d(dx + zOffsets[f + nc + 1], delta, sizeof(real) * (size_t)count));
+		/* delta = W' * delta */
+		HIP_CALL(fitre_hip_gemm(1, 0, l->in, n, l->out, 1.f, weights + wOffsets[f + nc], l->out, delta, l->out, 0.f,
+		                        delta_new, l->in, NULL, ws, wsBytes));
+		temp = delta_new;
+		delta_new = delta;
+		delta = temp;
+	}
+
+	/* [N][C][b*A+a] -> [C][N][a*B+b] */
+	{
+		int extA, extB;
+		feature_extent(model, &extA, &extB);
+		HIP_CALL(fitre_hip_fc_to_conv(delta, last->outChannels, n, extA, extB, delta_new));
+		temp = delta_new;
+		delta_new = delta;
+		delta = temp;
+	}
+
+	for (int c = nc - 1; c >= 0; c--) {
+		const CONV_LAYER *l = &model->convLayer[c];
+		const POOL_LAYER *p = &model->poolLayer[c];
+		const real *slab = z + zOffsets[c + 1];
+		real *dslab = dx + zOffsets[c + 1];
+		const long perChannel = (long)n * l->outWidth * l->outHeight;
+		const int act = model->actFuns[c];
+
+		if (p->type != MAX_POOL && p->type != AVG_POOL && p->type != NO_POOL) {
+			fprintf(stderr, "Unknown Pool Function... \n");
+			exit(-1);
+		}
+		const real *actIn = has_bn(l) ? slab + l->batchNormOffset : slab;
+		const real *actOut = slab + l->activationOffset;
+		if (c == nc - 1 && p->type == NO_POOL) {
+			/* The forward pass rewrote this layer's activation output into the FC layout in place;
+			 * rebuild it from the activation input (the reference reads the permuted buffer,
+			 * functions/cnn_backward.cu:574-580). */
+			HIP_CALL(fitre_hip_activation_forward(act, actIn, delta_new, perChannel * l->outChannels));
+			actOut = delta_new;
+		}
+		/* pool backward -> dx slab + 0; times f'(.) -> dx slab + activationOffset */
+		HIP_CALL(fitre_hip_pool_act_backward(p->type, act, delta, actIn, actOut, l->outChannels, n, p->width, p->height,
+		                                     p->pSize, p->stride, p->padding, p->outWidth, p->outHeight, dslab,
+		                                     dslab + l->activationOffset));
+		const real *cur = dslab + l->activationOffset;
+
+		if (has_bn(l)) {
+			/* batch-norm backward -> dx slab + batchNormOffset; its column sums are the bias gradient */
+			HIP_CALL(fitre_hip_batch_norm_backward(cur, slab + l->batchNormOffset,
+			                                       slab + l->batchNormOffset + l->variancesOffset, l->outChannels,
+			                                       perChannel, (real)BATCH_NORM_EPSILON, dslab + l->batchNormOffset,
+			                                       (model->bias != 0) ? gradient + bOffsets[c] : NULL, ws, wsBytes));
+			cur = dslab + l->batchNormOffset;
+		} else if (model->bias != 0) {
+			HIP_CALL(fitre_hip_channel_sum(cur, l->outChannels, perChannel, gradient + bOffsets[c], ws, wsBytes));
+		}
+
+		const real *input = (c == 0) ? data->currentBatch : z + zOffsets[c] + model->convLayer[c - 1].outputOffset;
+		fitre_conv_shape shape = conv_shape(l, n);
+		HIP_CALL(fitre_hip_conv_weight_grad(&shape, input, cur, gradient + wOffsets[c], ws, wsBytes));
+		if (c != 0) HIP_CALL(fitre_hip_conv_input_grad(&shape, cur, weights + wOffsets[c], delta, ws, wsBytes));
+	}
+	HIP_CALL(fitre_hip_sync());
+}
+
+real evaluateCNNModel(CNN_MODEL *model, DEVICE_DATASET *data, SCRATCH_AREA *scratch, real *z, real *probs,
+                      real *lossFuncErrors, int offset, int curBatchSize)
+{
+	return cnnForward(model, data, scratch, z, probs, lossFuncErrors, offset, curBatchSize, MODEL_TRAIN);
+}
+
+real computeCNNGradient(CNN_MODEL *model, DEVICE_DATASET *data, SCRATCH_AREA *scratch, real *z, real *dx, real *probs,
+                        real *lossFuncErrors, real *gradient, int offset, int curBatchSize, real weightDecay)
+{
+	real *oldDevPtr = scratch->nextDevPtr;
+	real *oldHostPtr = scratch->nextHostPtr;
+	real *oldPagePtr = scratch->nextPageLckPtr;
+
+	real *errors = scratch->nextDevPtr;
+	real *errors_1 = errors + model->maxDeltaSize;
+	real *nextDevPtr = errors_1 + model->maxDeltaSize;
+	scratch->nextDevPtr = nextDevPtr;
+
+	real lossVal = evaluateCNNModel(model, data, scratch, z, probs, lossFuncErrors, offset, curBatchSize);
+
+	HIP_CALL(fitre_hip_copy_d2d(errors, lossFuncErrors, sizeof(real) * (size_t)data->numClasses * curBatchSize));
+	cnnBackward(model, data, nextDevPtr, z, gradient, dx, errors, errors_1, offset, curBatchSize, scratch->nextHostPtr);
+
+	if (weightDecay != 0) HIP_CALL(fitre_hip_axpy(model->pSize, weightDecay, data->weights, gradient));
+	HIP_CALL(fitre_hip_sync());
+
+	scratch->nextDevPtr = oldDevPtr;
+	scratch->nextHostPtr = oldHostPtr;
+	scratch->nextPageLckPtr = oldPagePtr;
+	return lossVal;
+}

@@ -1,0 +1,150 @@
+"""Loads the two in-tree shared libraries and declares their C-ABI to ctypes.
+
+There is no fallback: if a library is missing or a symbol is not exported the
+import fails with the reason.  Build with ``python -m fitre_amd.build``.
+"""
+import ctypes as C
+import os
+
+from .structs import (CNN_MODEL, CONV_LAYER, DEVICE_DATASET, POOL_LAYER, SCRATCH_AREA, fitre_conv_shape)
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+HIP_LIB_PATH = os.path.join(_PKG, "libfitre_hip.so")
+CNN_LIB_PATH = os.path.join(_PKG, "libfitre_cnn.so")
+
+vp, i32, f32, lng, sz = C.c_void_p, C.c_int, C.c_float, C.c_long, C.c_size_t
+pvp, pi32, pf32 = C.POINTER(C.c_void_p), C.POINTER(C.c_int), C.POINTER(C.c_float)
+pshape = C.POINTER(fitre_conv_shape)
+pmodel, pdata, pscratch = C.POINTER(CNN_MODEL), C.POINTER(DEVICE_DATASET), C.POINTER(SCRATCH_AREA)
+
+# name -> (restype, argtypes); mirrors include/fitre_hip.h
+HIP_API = {
+    "fitre_hip_init": (i32, [i32]),
+    "fitre_hip_shutdown": (i32, []),
+    "fitre_hip_sync": (i32, []),
+    "fitre_hip_last_error": (C.c_char_p, []),
+    "fitre_hip_device_info": (i32, [pi32, pi32, pi32, C.POINTER(sz), C.POINTER(sz), C.c_char_p, i32]),
+    "fitre_hip_stream": (vp, []),
+    "fitre_hip_malloc": (i32, [pvp, sz]),
+    "fitre_hip_free": (i32, [vp]),
+    "fitre_hip_malloc_host": (i32, [pvp, sz]),
+    "fitre_hip_free_host": (i32, [vp]),
+    "fitre_hip_memset": (i32, [vp, i32, sz]),
+    "fitre_hip_copy_h2d": (i32, [vp, vp, sz]),
+    "fitre_hip_copy_d2h": (i32, [vp, vp, sz]),
+    "fitre_hip_copy_d2d": (i32, [vp, vp, sz]),
+    "fitre_hip_event_create": (i32, [pvp]),
+    "fitre_hip_event_destroy": (i32, [vp]),
+    "fitre_hip_event_record": (i32, [vp]),
+    "fitre_hip_event_elapsed_ms": (i32, [vp, vp, pf32]),
+    "fitre_hip_profile_enable": (i32, [i32]),
+    "fitre_hip_profile_read": (i32, [i32, C.POINTER(lng), C.POINTER(C.c_double), C.POINTER(C.c_double)]),
+    "fitre_hip_axpy": (i32, [i32, f32, vp, vp]),
+    "fitre_hip_scal": (i32, [i32, f32, vp]),
+    "fitre_hip_copy": (i32, [i32, vp, vp]),
+    "fitre_hip_dot": (i32, [i32, vp, vp, pf32]),
+    "fitre_hip_nrm2": (i32, [i32, vp, pf32]),
+    "fitre_hip_asum": (i32, [i32, vp, pf32]),
+    "fitre_hip_norm_inf": (i32, [i32, vp, pf32]),
+    "fitre_hip_sum": (i32, [i32, vp, pf32]),
+    "fitre_hip_fill": (i32, [vp, lng, f32]),
+    "fitre_hip_hadamard": (i32, [vp, vp, lng]),
+    "fitre_hip_hadamard2": (i32, [vp, vp, vp, vp, lng, vp]),
+    "fitre_hip_elem_inv_scale": (i32, [vp, vp, f32, lng, vp]),
+    "fitre_hip_elem_sqr": (i32, [vp, lng, vp]),
+    "fitre_hip_elem_sqr_decay": (i32, [vp, vp, f32, lng, vp]),
+    "fitre_hip_mat_mat_scale": (i32, [vp, vp, lng, vp]),
+    "fitre_hip_mat_row_vec_scale": (i32, [vp, i32, i32, vp, vp]),
+    "fitre_hip_add_column": (i32, [vp, i32, i32, vp]),
+    "fitre_hip_add_channel_bias": (i32, [vp, i32, lng, vp]),
+    "fitre_hip_activation_forward": (i32, [i32, vp, vp, lng]),
+    "fitre_hip_activation_backward": (i32, [i32, vp, vp, vp, vp, lng]),
+    "fitre_hip_pool_forward": (i32, [i32, vp] + [i32] * 9 + [vp]),
+    "fitre_hip_pool_backward": (i32, [i32, vp, vp] + [i32] * 9 + [vp]),
+    "fitre_hip_max_pool_argmax": (i32, [vp] + [i32] * 9 + [vp]),
+    "fitre_hip_pool_act_backward": (i32, [i32, i32, vp, vp, vp] + [i32] * 9 + [vp, vp]),
+    "fitre_hip_batch_norm_workspace": (sz, [i32, lng]),
+    "fitre_hip_batch_norm_forward": (i32, [vp, i32, lng, vp, vp, vp, vp, vp, f32, f32, i32, vp, sz]),
+    "fitre_hip_batch_norm_backward": (i32, [vp, vp, vp, i32, lng, f32, vp, vp, vp, sz]),
+    "fitre_hip_channel_sum_workspace": (sz, [i32, lng]),
+    "fitre_hip_channel_sum": (i32, [vp, i32, lng, vp, vp, sz]),
+    "fitre_hip_row_sum": (i32, [vp, i32, i32, vp]),
+    "fitre_hip_softmax_cross_entropy": (i32, [vp, vp, i32, i32, vp, vp, pf32]),
+    "fitre_hip_cross_entropy_error": (i32, [vp, vp, i32, i32, vp]),
+    "fitre_hip_reshape": (i32, [vp, i32, i32, i32, vp]),
+    "fitre_hip_conv_to_fc": (i32, [vp, i32, i32, i32, i32, vp]),
+    "fitre_hip_fc_to_conv": (i32, [vp, i32, i32, i32, i32, vp]),
+    "fitre_hip_conv_forward_workspace": (sz, [pshape]),
+    "fitre_hip_conv_forward": (i32, [pshape, vp, vp, vp, vp, vp, sz]),
+    "fitre_hip_conv_weight_grad_workspace": (sz, [pshape]),
+    "fitre_hip_conv_weight_grad": (i32, [pshape, vp, vp, vp, vp, sz]),
+    "fitre_hip_conv_input_grad_workspace": (sz, [pshape]),
+    "fitre_hip_conv_input_grad": (i32, [pshape, vp, vp, vp, vp, sz]),
+    "fitre_hip_gemm_workspace": (sz, [i32, i32, i32]),
+    "fitre_hip_gemm": (i32, [i32, i32, i32, i32, i32, f32, vp, i32, vp, i32, f32, vp, i32, vp, vp, sz]),
+}
+
+pconv, ppool = C.POINTER(CONV_LAYER), C.POINTER(POOL_LAYER)
+# mirrors include/fitre_cnn.h and include/fitre_shim.h
+CNN_API = {
+    "getDimensions": (None, [i32, i32, i32, i32, i32, pi32, pi32]),
+    "computeParamSize": (None, [pmodel]),
+    "computeWeightOffsets": (None, [pmodel]),
+    "computeWeightBiasOffsets": (None, [pmodel]),
+    "computeZOffsets": (None, [pmodel, i32, i32, i32]),
+    "makeLayer": (None, [pconv, ppool, i32, i32, i32, i32, i32, pi32, pi32, i32, i32]),
+    "readVGG11": (None, [pmodel, i32, i32, i32, i32, i32, i32, i32, i32]),
+    "fitre_make_conv_layer": (None, [pconv, ppool] + [i32] * 13 + [pi32, pi32]),
+    "fitre_finalize_model": (None, [pmodel, i32, i32, i32]),
+    "fitre_build_lenet": (None, [pmodel] + [i32] * 9),
+    "fitre_build_vgg11": (None, [pmodel] + [i32] * 8),
+    "fitre_build_alexnet": (None, [pmodel] + [i32] * 8),
+    "cnnForwardMemRequired": (lng, [pmodel]),
+    "cnnForward": (f32, [pmodel, pdata, pscratch, vp, vp, vp, i32, i32, i32]),
+    "cnnBackwardMemRequired": (lng, [pmodel]),
+    "cnnBackward": (None, [pmodel, pdata, vp, vp, vp, vp, vp, vp, i32, i32, vp]),
+    "evaluateCNNModel": (f32, [pmodel, pdata, pscratch, vp, vp, vp, i32, i32]),
+    "computeCNNGradient": (f32, [pmodel, pdata, pscratch, vp, vp, vp, vp, vp, i32, i32, f32]),
+    "getDeviceParameters": (None, []),
+    "fitre_env_init": (None, [pscratch, i32, sz]),
+    "cuda_env_init": (None, [pscratch, i32]),
+    "cuda_allocate_workspace": (None, [pscratch, i32]),
+    "fitre_allocate_workspace": (None, [pscratch, sz]),
+    "cuda_env_cleanup": (None, [pscratch]),
+    "cuda_malloc": (None, [pvp, sz, i32, i32]),
+    "cuda_malloc_host": (None, [pvp, sz, i32, i32]),
+    "cuda_free": (None, [vp, i32]),
+    "cuda_free_host": (None, [vp, i32]),
+    "cuda_memset": (None, [vp, i32, sz, i32]),
+    "copy_host_device": (None, [vp, vp, sz, i32, i32]),
+    "copy_device": (None, [vp, vp, sz, i32]),
+    "print_device_mem_usage": (None, []),
+}
+
+
+def _load(path, api):
+    if not os.path.exists(path):
+        raise ImportError("%s is missing: build it with `python -m fitre_amd.build`" % path)
+    lib = C.CDLL(path, mode=C.RTLD_GLOBAL)
+    for name, (restype, argtypes) in api.items():
+        try:
+            fn = getattr(lib, name)
+        except AttributeError:
+            raise ImportError("%s does not export %s" % (path, name))
+        fn.restype = restype
+        fn.argtypes = argtypes
+    return lib
+
+
+hip = _load(HIP_LIB_PATH, HIP_API)
+cnn = _load(CNN_LIB_PATH, CNN_API)
+
+
+class FitreError(RuntimeError):
+    pass
+
+
+def check(rc, what=""):
+    """Raises FitreError with the device layer's message when rc is not 0."""
+    if rc != 0:
+        raise FitreError("%s failed with code %d: %s" % (what or "device call", rc, hip.fitre_hip_last_error().decode()))

@@ -1,0 +1,87 @@
+"""ctypes mirrors of the records in include/fitre_types.h and include/fitre_nn.h.
+
+Field names and order are those of the reference's nn/nn_decl.h:64-155 and
+core/structdefs.h:25-83; `real` is float.
+"""
+import ctypes as C
+
+MAX_LAYERS = 20
+real = C.c_float
+real_p = C.POINTER(real)
+
+# enumerators (nn/nn_decl.h:13-62, 97-101)
+PERFORM_NO_BATCH_NORM, PERFORM_BATCH_NORM, PERFORM_BATCH_NORM_TRAINABLE = 0, 10, 20
+MODEL_TRAIN, MODEL_TRAIN_ACCURACY, MODEL_TEST_ACCURACY = 10, 20, 30
+ACT_NONE, ACT_LOGISTIC, ACT_TANH, ACT_LINEAR, ACT_SOFTMAX = 0, 1, 2, 3, 4
+CNN_ACT_NONE, CNN_ACT_SOFTPLUS, CNN_ACT_ELU, CNN_ACT_RELU, CNN_ACT_SWISH = 10, 11, 12, 13, 14
+MAX_POOL, AVG_POOL, NO_POOL = 0, 1, 2
+CIFAR10, CIFAR100, IMAGENET = 10, 20, 30
+INT_MAX = 2 ** 31 - 1
+
+
+class CONV_LAYER(C.Structure):
+    _fields_ = [(n, C.c_int) for n in (
+        "inChannels", "outChannels", "width", "height", "outWidth", "outHeight", "kSize", "stride",
+        "padding", "activationOffset", "poolOffset", "batchNormOffset", "outputOffset", "batchNorm",
+        "meansOffset", "variancesOffset", "runningMeansOffset", "runningVariancesOffset", "convVolumn",
+        "activationVolumn", "poolVolumn", "batchNormVolumn")]
+
+
+class POOL_LAYER(C.Structure):
+    _fields_ = [(n, C.c_int) for n in (
+        "height", "width", "outHeight", "outWidth", "type", "pSize", "padding", "stride")]
+
+
+class FC_LAYER(C.Structure):
+    _fields_ = [(n, C.c_int) for n in ("in_", "out", "actFun", "batchNorm", "offset")]
+
+
+class CNN_MODEL(C.Structure):
+    _fields_ = [
+        ("convLayer", CONV_LAYER * MAX_LAYERS),
+        ("actFuns", C.c_int * MAX_LAYERS),
+        ("poolLayer", POOL_LAYER * MAX_LAYERS),
+        ("cLayers", C.c_int),
+        ("lLayers", C.c_int),
+        ("fcLayer", FC_LAYER * MAX_LAYERS),
+        ("bias", C.c_int),
+        ("pSize", C.c_int),
+        ("zSize", C.c_int),
+        ("batchSize", C.c_int),
+        ("maxDeltaSize", C.c_int),
+        ("name", C.c_int),
+        ("enableBatchNorm", C.c_int),
+        ("wOffsets", C.c_int * MAX_LAYERS),
+        ("bOffsets", C.c_int * MAX_LAYERS),
+        ("zOffsets", C.c_int * MAX_LAYERS),
+        ("zztSize", C.c_int),
+        ("zztOffsets", C.c_int * MAX_LAYERS),
+        ("rZOffsets", C.c_int * MAX_LAYERS),
+    ]
+
+
+class SCRATCH_AREA(C.Structure):
+    _fields_ = [(n, C.c_void_p) for n in (
+        "hostWorkspace", "devWorkspace", "pageLckWorkspace", "nextDevPtr", "nextHostPtr", "nextPageLckPtr")]
+
+
+class SparseDataset(C.Structure):
+    _fields_ = [("rowPtr", C.c_void_p), ("colPtr", C.c_void_p), ("rowCsrPtr", C.c_void_p),
+                ("valPtr", C.c_void_p), ("nnz", C.c_int), ("sortedVals", C.c_void_p), ("P", C.c_void_p),
+                ("descr", C.c_void_p)]
+
+
+class DEVICE_DATASET(C.Structure):
+    _fields_ = [
+        ("trainSetX", C.c_void_p), ("trainSetY", C.c_void_p), ("testSetX", C.c_void_p),
+        ("testSetY", C.c_void_p), ("weights", C.c_void_p), ("numClasses", C.c_int),
+        ("datasetType", C.c_int), ("features", C.c_int), ("height", C.c_int), ("width", C.c_int),
+        ("testSizeX", C.c_int), ("testSizeY", C.c_int), ("trainSizeX", C.c_int), ("trainSizeY", C.c_int),
+        ("sampleSize", C.c_int), ("sampledTrainX", C.c_void_p), ("sampledTrainY", C.c_void_p),
+        ("currentBatch", C.c_void_p), ("spSamplingMatrix", SparseDataset),
+    ]
+
+
+class fitre_conv_shape(C.Structure):
+    _fields_ = [(n, C.c_int) for n in (
+        "samples", "inChannels", "outChannels", "inA", "inB", "outA", "outB", "ksize", "stride", "padding")]

@@ -1,0 +1,88 @@
+/*
+ * fitre_cnn.h -- host-side C interface of the CNN gradient path.
+ *
+ * These are the free functions the reference's solvers and drivers call
+ * (solvers/kfac_trust_region.cu:352,361,395; utilities/cnn_derivative_test.cu:158-168).
+ * Names, argument order and argument meaning are the reference's; every
+ * function is device-complete when it returns.  On an unrecoverable error a
+ * message goes to stderr and the process exits, as in the reference
+ * (functions/cnn_backward.cu:171-174).
+ *
+ * All pointers named z, dx, probs, errors, gradient, delta, devPtr and the
+ * DEVICE_DATASET members are DEVICE pointers owned by the caller.
+ */
+#ifndef FITRE_CNN_H
+#define FITRE_CNN_H
+
+#include "fitre_nn.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- shape and flat-layout arithmetic (reference: nn/utils.c:12-172) ---- */
+
+/* (height + 2*padding - kernel)/stride + 1, integer division. nn/utils.c:12-17 */
+void getDimensions(int height, int width, int padding, int stride, int kernel, int *h, int *w);
+/* pSize = number of reals in the flat parameter vector. nn/utils.c:19-42 */
+void computeParamSize(CNN_MODEL *model);
+/* wOffsets for a model without biases; bOffsets := INT_MAX. nn/utils.c:44-71 */
+void computeWeightOffsets(CNN_MODEL *model);
+/* interleaved [W_l | b_l] offsets for a model with biases. nn/utils.c:74-105 */
+void computeWeightBiasOffsets(CNN_MODEL *model);
+/* zOffsets, zztOffsets, zSize, zztSize, maxDeltaSize. nn/utils.c:108-172 */
+void computeZOffsets(CNN_MODEL *model, int height, int width, int batchSize);
+/* 3x3 / stride 1 / pad 1 convolution + optional 2x2 pool, with the slab
+ * offsets of nn/read_vgg.c:25-120. */
+void makeLayer(CONV_LAYER *conv, POOL_LAYER *pool, POOL_TYPE poolFun, int inChannels, int outChannels,
+               int height, int width, int *outHeight, int *outWidth, int batchSize,
+               BATCH_NORM_TYPES batchnorm);
+/* VGG-11 as the reference builds it (swish; nn/read_vgg.c:216-300). */
+void readVGG11(CNN_MODEL *model, int batchSize, int height, int width, int numClasses, int inChannels,
+               int bias, int enableBatchNorm, DATASET_TYPE datasetType);
+
+/* ---- builders that have no counterpart in the reference: the same slab
+ * scheme as makeLayer for arbitrary kernel / stride / padding / pooling ---- */
+void fitre_make_conv_layer(CONV_LAYER *conv, POOL_LAYER *pool, int inChannels, int outChannels,
+                           int height, int width, int kSize, int stride, int padding,
+                           POOL_TYPE poolFun, int poolSize, int poolStride, int poolPadding,
+                           int batchSize, BATCH_NORM_TYPES batchnorm, int *outHeight, int *outWidth);
+/* Fills pSize, w/b/z offsets and sizes once cLayers/lLayers/layers/bias are set. */
+void fitre_finalize_model(CNN_MODEL *model, int height, int width, int batchSize);
+/* LeNet-style: conv5x5 C->6, pool2, conv5x5 6->16, pool2, FC 400-120-84-classes (32x32 input). */
+void fitre_build_lenet(CNN_MODEL *model, int batchSize, int height, int width, int inChannels,
+                       int numClasses, int bias, int enableBatchNorm, int convAct, int fcAct);
+/* VGG-11-style with a chosen activation. */
+void fitre_build_vgg11(CNN_MODEL *model, int batchSize, int height, int width, int inChannels,
+                       int numClasses, int bias, int enableBatchNorm, int convAct);
+/* ImageNet AlexNet-style: 11x11/s4/p2, 5x5/p2, 3x3 x3, maxpool 3/2 after 1,2,5; FC 9216-4096-4096-classes. */
+void fitre_build_alexnet(CNN_MODEL *model, int batchSize, int height, int width, int inChannels,
+                         int numClasses, int bias, int convAct, int fcAct);
+
+/* ---- the gradient path (reference: functions/cnn_forward.h:9-13,
+ * functions/cnn_backward.h:11-16, functions/cnn_gradient.h:9-12,
+ * functions/cnn_eval_model.cu:7-13) ---- */
+
+/* Scratch (in reals) the forward pass may carve from scratch->nextDevPtr. */
+long cnnForwardMemRequired(CNN_MODEL *model);
+/* Fills z, probs (classes x batch, class fastest) and errors = (p - onehot)/batch;
+ * returns the mean negative log-likelihood. */
+real cnnForward(CNN_MODEL *model, DEVICE_DATASET *data, SCRATCH_AREA *scratch, real *z, real *probs,
+                real *errors, int s, int curBatchSize, EVAL_TYPE forTesting);
+/* Scratch (in reals) cnnBackward may carve from devPtr. */
+long cnnBackwardMemRequired(CNN_MODEL *model);
+/* gradient[pSize] and the dx snapshots from z and delta (= errors of cnnForward).
+ * delta and delta_new (each >= maxDeltaSize reals) are clobbered. */
+void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, real *gradient, real *dx,
+                 real *delta, real *delta_new, int offset, int batchSize, real *hostPtr);
+real evaluateCNNModel(CNN_MODEL *model, DEVICE_DATASET *data, SCRATCH_AREA *scratch, real *z,
+                      real *probs, real *lossFuncErrors, int offset, int curBatchSize);
+/* forward + backward + gradient += weightDecay * weights; returns the loss. */
+real computeCNNGradient(CNN_MODEL *model, DEVICE_DATASET *data, SCRATCH_AREA *scratch, real *z, real *dx,
+                        real *probs, real *lossFuncErrors, real *gradient, int offset, int curBatchSize,
+                        real weightDecay);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

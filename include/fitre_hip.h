@@ -1,0 +1,224 @@
+/*
+ * fitre_hip.h -- C-ABI of the MI355X (gfx950) device layer.
+ *
+ * This is the whole boundary between the C host code and the HIP kernels:
+ * plain pointers and sizes, no C++ or framework types.  It replaces the
+ * reference's device/cuda_environment.[ch], device/cuda_utils.[ch],
+ * device/handles.h, device/query.c, and every cuBLAS call and __global__
+ * kernel reached from cnnForward / cnnBackward.
+ *
+ * Conventions
+ *   - every function returns 0 on success and a non-zero FITRE_E_* code on
+ *     failure; fitre_hip_last_error() then describes the failure;
+ *   - all tensor pointers are device pointers; work is queued on the layer's
+ *     own stream and is NOT complete on return unless stated -- call
+ *     fitre_hip_sync() before reading results on the host;
+ *   - activations are [C][N][A][B] reals, B fastest (the reference's
+ *     column-major (N*H*W) x C matrix with A = image column, B = image row);
+ *   - "ws" arguments are caller-provided device workspaces of at least the
+ *     number of bytes the matching *_workspace() function returns.
+ */
+#ifndef FITRE_HIP_H
+#define FITRE_HIP_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FITRE_OK            0
+#define FITRE_E_DEVICE      1 /* a HIP runtime call failed */
+#define FITRE_E_ARGUMENT    2 /* null pointer, non-positive size, inconsistent shape */
+#define FITRE_E_UNSUPPORTED 3 /* activation / pooling code or shape the kernels do not cover */
+#define FITRE_E_WORKSPACE   4 /* workspace smaller than required */
+
+/* ---------------- environment (device/cuda_environment.c:29-77, device/query.c:7-49) ---------------- */
+int fitre_hip_init(int device);
+int fitre_hip_shutdown(void);
+int fitre_hip_sync(void);
+const char *fitre_hip_last_error(void);
+/* compute units, wavefront size, max threads per block, total and free bytes; name may be NULL */
+int fitre_hip_device_info(int *computeUnits, int *waveSize, int *maxThreadsPerBlock, size_t *totalBytes,
+                          size_t *freeBytes, char *name, int nameLen);
+/* the hipStream_t the layer launches on, as an opaque pointer */
+void *fitre_hip_stream(void);
+
+/* ---------------- memory (device/cuda_utils.c; device/cuda_utils.h:15-26) ---------------- */
+int fitre_hip_malloc(void **ptr, size_t bytes);
+int fitre_hip_free(void *ptr);
+int fitre_hip_malloc_host(void **ptr, size_t bytes); /* pinned */
+int fitre_hip_free_host(void *ptr);
+int fitre_hip_memset(void *ptr, int value, size_t bytes);          /* stream-ordered */
+int fitre_hip_copy_h2d(void *dev, const void *host, size_t bytes); /* complete on return */
+int fitre_hip_copy_d2h(void *host, const void *dev, size_t bytes); /* complete on return */
+int fitre_hip_copy_d2d(void *dst, const void *src, size_t bytes);  /* stream-ordered */
+
+/* ---------------- timing ---------------- */
+/* Events on the layer's stream. */
+int fitre_hip_event_create(void **event);
+int fitre_hip_event_destroy(void *event);
+int fitre_hip_event_record(void *event);
+int fitre_hip_event_elapsed_ms(void *start, void *stop, float *ms); /* waits for stop */
+
+/* Per-kernel-class accounting: while enabled, every launch is bracketed by
+ * events on the stream and attributed to one FITRE_KC_* class together with
+ * its algorithmic work (flops for GEMM classes, bytes for the others). */
+enum fitre_kernel_class {
+	FITRE_KC_CONV_DW = 0,
+	FITRE_KC_CONV_DX = 1,
+	FITRE_KC_CONV_FWD = 2,
+	FITRE_KC_FC_GEMM = 3,
+	FITRE_KC_SPLITK_REDUCE = 4,
+	FITRE_KC_BN_BWD = 5,
+	FITRE_KC_BN_FWD = 6,
+	FITRE_KC_POOL_BWD = 7,
+	FITRE_KC_POOL_FWD = 8,
+	FITRE_KC_ACT_BWD = 9,
+	FITRE_KC_ACT_FWD = 10,
+	FITRE_KC_BIAS_GRAD = 11,
+	FITRE_KC_SOFTMAX = 12,
+	FITRE_KC_PERMUTE = 13,
+	FITRE_KC_BLAS1 = 14,
+	FITRE_KC_POOL_ACT_BWD = 15,
+	FITRE_KC_KFAC_FACTOR = 16,
+	FITRE_KC_COUNT = 17
+};
+int fitre_hip_profile_enable(int on); /* on=1 clears the counters and starts; on=0 stops */
+/* launches, summed milliseconds and summed algorithmic work of one class (syncs first) */
+int fitre_hip_profile_read(int kernelClass, long *launches, double *milliseconds, double *work);
+
+/* ---------------- level-1 helpers (the cublasD* calls of the solvers and of
+ * functions/cnn_gradient.cu:54-56, functions/softmax_loss.cu:243) ---------------- */
+int fitre_hip_axpy(int n, float alpha, const float *x, float *y);         /* y += alpha x */
+int fitre_hip_scal(int n, float alpha, float *x);                         /* x *= alpha */
+int fitre_hip_copy(int n, const float *x, float *y);                      /* y = x */
+int fitre_hip_dot(int n, const float *x, const float *y, float *result);  /* host result, complete on return */
+int fitre_hip_nrm2(int n, const float *x, float *result);                 /* host result */
+int fitre_hip_asum(int n, const float *x, float *result);                 /* host result */
+int fitre_hip_norm_inf(int n, const float *x, float *result);             /* device/reduce.cu:110-153 kerNormInf */
+int fitre_hip_sum(int n, const float *x, float *result);                  /* utilities/reduce.cu:32-84 */
+
+/* ---------------- elementwise helpers ---------------- */
+int fitre_hip_fill(float *x, long n, float value);                        /* dev_initializations.cu:7-14, dev_activations.cu:89-95 */
+int fitre_hip_hadamard(const float *x, float *y, long n);                 /* y *= x                  dev_hadamard.cu:4-10 */
+int fitre_hip_hadamard2(const float *m1, const float *m2, const float *m3, const float *m4, long n,
+                        float *out);                                      /* out = m1*m2 + m3*m4     dev_hadamard.cu:12-20 */
+int fitre_hip_elem_inv_scale(const float *x, const float *y, float eps, long n, float *out);
+                                                                          /* out = x/(sqrt(y)+eps)   dev_elem_scale.cu */
+int fitre_hip_elem_sqr(const float *x, long n, float *out);               /* out = x*x               dev_elem_sqr.cu */
+int fitre_hip_elem_sqr_decay(const float *x, const float *y, float decay, long n, float *out);
+                                                                          /* out = decay*x+(1-decay)*y*y  dev_elem_sqr_decay.cu */
+int fitre_hip_mat_mat_scale(const float *x, const float *y, long n, float *out); /* out = x*y        dev_mat_mat_scale.cu */
+int fitre_hip_mat_row_vec_scale(const float *x, int rows, int cols, const float *y, float *out);
+                                                                          /* out[i] = x[i]*y[i/rows] dev_mat_vec_scale.cu */
+int fitre_hip_add_column(float *mat, int rows, int cols, const float *vec); /* mat[:,c] += vec; column-major  dev_mat_vec_addition.cu:6-17 */
+int fitre_hip_add_channel_bias(float *x, int channels, long perChannel, const float *bias); /* eval_convolution.cu:26-34 */
+
+/* ---------------- activations (codes of ACTIVATION_FUNCTIONS / CNN_ACTIVATION_FUNCTIONS) ---------------- */
+/* out = f(in); in == out allowed.  dev_activations.cu:8-95, swish.cu:14-23 */
+int fitre_hip_activation_forward(int actFun, const float *in, float *out, long n);
+/* out = delta * f'(.) ; z_in = activation input, z_out = activation output; out == delta allowed.
+ * swish.cu:34-43, dev_layer_error.cu:13-48; ReLU uses z_out > 0. */
+int fitre_hip_activation_backward(int actFun, const float *delta, const float *z_in, const float *z_out,
+                                  float *out, long n);
+
+/* ---------------- pooling on [C][N][A][B] (functions/dev_pool.cu) ---------------- */
+/* poolType: 0 max, 1 average.  inA/inB = input extent along A/B; window origin k*stride - padding. */
+int fitre_hip_pool_forward(int poolType, const float *in, int channels, int samples, int inA, int inB,
+                           int ksize, int stride, int padding, int outA, int outB, float *out);
+/* Max pool: delta at the first maximum in memory order (strict >), zero elsewhere; overlapping
+ * windows add.  Average pool: delta / ksize^2 spread over the window.  dev_pool.cu:269-298,346-398 */
+int fitre_hip_pool_backward(int poolType, const float *delta, const float *z_in, int channels, int samples,
+                            int inA, int inB, int ksize, int stride, int padding, int outA, int outB,
+                            float *out);
+/* argmax offset inside each A x B map for every pooled cell (int32, layout of the pooled tensor) */
+int fitre_hip_max_pool_argmax(const float *z_in, int channels, int samples, int inA, int inB, int ksize,
+                              int stride, int padding, int outA, int outB, int *index);
+/* Fused max/avg/no pool backward + activation backward: writes dxPool (pool-backward result) and
+ * dxAct = dxPool * f'(.).  poolType 2 = no pooling (delta has the input extent). */
+int fitre_hip_pool_act_backward(int poolType, int actFun, const float *delta, const float *z_in,
+                                const float *z_act, int channels, int samples, int inA, int inB,
+                                int ksize, int stride, int padding, int outA, int outB, float *dxPool,
+                                float *dxAct);
+
+/* ---------------- batch normalisation, non-affine, per channel over N*A*B (functions/dev_batch_norm.cu) ---------------- */
+size_t fitre_hip_batch_norm_workspace(int channels, long perChannel);
+/* train != 0: batch mean / biased variance, running = momentum*running + (1-momentum)*batch,
+ * zhat = (x-mean)/sqrt(var+eps); train == 0: normalise with the running statistics.  :263-393 */
+int fitre_hip_batch_norm_forward(const float *in, int channels, long perChannel, float *zhat, float *mean,
+                                 float *variance, float *runningMean, float *runningVariance,
+                                 float epsilon, float momentum, int train, void *ws, size_t wsBytes);
+/* out = (m*delta - sum(delta) - zhat*sum(delta*zhat)) / (m*sqrt(eps+var)), m = perChannel.  :550-621.
+ * biasGrad (may be NULL) receives the per-channel sum of out. */
+int fitre_hip_batch_norm_backward(const float *delta, const float *zhat, const float *variance,
+                                  int channels, long perChannel, float epsilon, float *out,
+                                  float *biasGrad, void *ws, size_t wsBytes);
+
+/* ---------------- reductions ---------------- */
+/* out[c] = sum of the perChannel contiguous values of channel c (conv bias gradient,
+ * functions/cnn_backward.cu:662-689). */
+size_t fitre_hip_channel_sum_workspace(int channels, long perChannel);
+int fitre_hip_channel_sum(const float *x, int channels, long perChannel, float *out, void *ws,
+                          size_t wsBytes);
+/* out[r] = sum over columns of a column-major rows x cols matrix (FC bias gradient, :212-224). */
+int fitre_hip_row_sum(const float *mat, int rows, int cols, float *out);
+
+/* ---------------- softmax cross entropy (functions/softmax_loss.cu:17-79,141-245) ---------------- */
+/* logits/probs/errors: classes x rows, class fastest; target: 1-based class ids as float.
+ * probs = softmax + 1e-10; errors = (probs - onehot)/rows; *lossHost = mean(-log probs[target]),
+ * written to host memory, complete on return.  errors may be NULL. */
+int fitre_hip_softmax_cross_entropy(const float *logits, const float *target, int rows, int classes,
+                                    float *probs, float *errors, float *lossHost);
+/* errors = (probs - onehot)/rows only (computeCrossEntropyError, :231-245) */
+int fitre_hip_cross_entropy_error(const float *probs, const float *target, int rows, int classes,
+                                  float *errors);
+
+/* ---------------- layout changes at the conv <-> FC boundary ---------------- */
+/* [right][left][chunk] -> [left][right][chunk]   (dev_backprop_convolution.cu:140-168) */
+int fitre_hip_reshape(const float *in, int right, int left, int chunk, float *out);
+/* [C][N][a*B+b] -> [N][C][b*A+a]  (reshape + ker_transpose, cnn_forward.cu:238-261); in != out */
+int fitre_hip_conv_to_fc(const float *in, int channels, int samples, int extA, int extB, float *out);
+/* [N][C][b*A+a] -> [C][N][a*B+b]  (cnn_backward.cu:310-326); in != out */
+int fitre_hip_fc_to_conv(const float *in, int channels, int samples, int extA, int extB, float *out);
+
+/* ---------------- fp32-MFMA contractions ---------------- */
+/* Convolution geometry shared by the three convolution entry points. */
+typedef struct fitre_conv_shape {
+	int samples;      /* N */
+	int inChannels;   /* Cin */
+	int outChannels;  /* Cout */
+	int inA, inB;     /* input extent along A (image column) and B (image row) */
+	int outA, outB;   /* output extent */
+	int ksize, stride, padding;
+} fitre_conv_shape;
+
+/* y[Cout][N][outA][outB] = conv(x[Cin][N][inA][inB], w[Cout][Cin][k][k]) + bias (bias may be NULL).
+ * Replaces im2col + GEMM + bias of functions/eval_convolution.cu:110-121. */
+size_t fitre_hip_conv_forward_workspace(const fitre_conv_shape *s);
+int fitre_hip_conv_forward(const fitre_conv_shape *s, const float *x, const float *w, const float *bias,
+                           float *y, void *ws, size_t wsBytes);
+/* dW[Cout][Cin*k*k] = sum over (n,a,b) of patch(x) * delta.  Replaces im2col + GEMM of
+ * functions/cnn_backward.cu:771-783. */
+size_t fitre_hip_conv_weight_grad_workspace(const fitre_conv_shape *s);
+int fitre_hip_conv_weight_grad(const fitre_conv_shape *s, const float *x, const float *delta, float *dW,
+                               void *ws, size_t wsBytes);
+/* dx[Cin][N][inA][inB] = transposed convolution of delta with w; stride must be 1.  Replaces
+ * functions/dev_backprop_convolution.cu:173-247. */
+size_t fitre_hip_conv_input_grad_workspace(const fitre_conv_shape *s);
+int fitre_hip_conv_input_grad(const fitre_conv_shape *s, const float *delta, const float *w, float *dx,
+                              void *ws, size_t wsBytes);
+
+/* Column-major GEMM C(MxN) = alpha*op(A)*op(B) + beta*C with the argument meaning of cublasDgemm
+ * (transA/transB: 0 = N, 1 = T).  Used for the FC layers (eval_gradient.cu:63-67,
+ * cnn_backward.cu:189-197,250-254) and the KFAC factor products (kfac_inverses.cu:531-536,808-813).
+ * bias (may be NULL) is added to every column (length M) after the product when beta == 0. */
+size_t fitre_hip_gemm_workspace(int M, int N, int K);
+int fitre_hip_gemm(int transA, int transB, int M, int N, int K, float alpha, const float *A, int lda,
+                   const float *B, int ldb, float beta, float *C, int ldc, const float *bias, void *ws,
+                   size_t wsBytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,848 @@
+/*
+ * fitre_oracle.c -- CPU restatement of the reference's CNN forward/backward
+ * path.  TEST INFRASTRUCTURE ONLY: it is the checker the HIP kernels are
+ * compared with, and the timed CPU baseline of the benchmark.  Nothing in
+ * the shipped library links, loads or calls it.
+ *
+ * Built twice from this one file: real = double (the parity oracle) and
+ * real = float (the CPU baseline), see oracle/Makefile.
+ *
+ * Each function cites the reference lines it follows.  It keeps the
+ * reference's data flow on purpose -- materialised patch matrices, BLAS-style
+ * GEMM calls with the reference's own argument lists, one pass per kernel --
+ * so that it can be audited against the reference line by line, and so that
+ * it shares no structure with the implicit-GEMM kernels it checks.
+ *
+ * Deliberate departures from the reference (each is a reference defect; the
+ * HIP path makes the same choice):
+ *   D1  ReLU / ELU backward multiply by the true derivative; the reference
+ *       leaves delta unchanged (functions/cnn_backward.cu:561-565).
+ *   D2  pooling windows start at k*stride - padding; the reference's
+ *       (k-1)*stride + ksize - 2*padding (functions/dev_pool.cu:94-95) equals
+ *       it only when ksize = stride + padding.
+ *   D3  average-pool backward is the adjoint of the forward for any window;
+ *       the reference's kernel is valid only for ksize = stride, no padding,
+ *       extent divisible by ksize (functions/dev_pool.cu:269-298), where the
+ *       two agree.
+ *   D4  the FC<->conv boundary transpose uses row*width + col; the
+ *       reference's row*height + col (functions/dev_transpose.cu:26-28) is
+ *       the same for square maps, the only ones it is run on.
+ *   D5  ReLU / ELU are applied on fully connected layers; the reference
+ *       prints "not implemented" and leaves the values unchanged
+ *       (functions/eval_gradient.cu:205-211).
+ *   D6  when the last convolution layer has no pooling stage, its activation
+ *       output has been rewritten in place into the fully connected layout by
+ *       the forward pass (functions/cnn_forward.cu:238-261); the backward pass
+ *       then recomputes that layer's activation output from its input instead
+ *       of reading the permuted buffer as the reference does
+ *       (functions/cnn_backward.cu:574-580).  No shipped network of the
+ *       reference ends in an unpooled layer.
+ *
+ * Parity pins (tests/test_oracle_*.py): the stored batch-norm known answer
+ * pytorch/testing/my.out:9; brute-force direct convolution and its adjoint
+ * identities; float64 autograd of the textbook layers; a Taylor remainder
+ * test of the whole gradient (utilities/cnn_derivative_test.cu:197-199);
+ * the logged LeNet parameter offsets.  No function here is "parity unpinned".
+ */
+#include <float.h>
+#include <limits.h>
+#include <math.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include "fitre_nn.h"
+
+#ifdef FITRE_REAL_DOUBLE
+#define REAL_MAX DBL_MAX
+#else
+#define REAL_MAX FLT_MAX
+#endif
+
+#define OP_N 0
+#define OP_T 1
+
+/* ------------------------------------------------------------------ */
+/* BLAS-shaped helpers (column-major), standing in for the cuBLAS calls */
+/* ------------------------------------------------------------------ */
+
+/* C(MxN) = alpha * op(A)(MxK) * op(B)(KxN) + beta * C, column-major, as cublasDgemm. */
+void oracle_gemm(int transA, int transB, int M, int N, int K, real alpha, const real *A, int lda,
+                 const real *B, int ldb, real beta, real *C, int ldc)
+{
+#pragma omp parallel for schedule(static)
+	for (int j = 0; j < N; j++) {
+		real *c = C + (size_t)j * ldc;
+		if (beta == 0) {
+			for (int i = 0; i < M; i++) c[i] = 0;
+		} else if (beta != 1) {
+			for (int i = 0; i < M; i++) c[i] *= beta;
+		}
+		if (transA == OP_N) {
+			for (int k = 0; k < K; k++) {
+				real b = alpha * (transB == OP_N ? B[(size_t)j * ldb + k] : B[(size_t)k * ldb + j]);
+				const real *a = A + (size_t)k * lda;
+#pragma omp simd
+				for (int i = 0; i < M; i++) c[i] += a[i] * b;
+			}
+		} else {
+			for (int i = 0; i < M; i++) {
+				const real *a = A + (size_t)i * lda;
+				real s = 0;
+				if (transB == OP_N) {
+					const real *b = B + (size_t)j * ldb;
+#pragma omp simd reduction(+ : s)
+					for (int k = 0; k < K; k++) s += a[k] * b[k];
+				} else {
+					for (int k = 0; k < K; k++) s += a[k] * B[(size_t)k * ldb + j];
+				}
+				c[i] += alpha * s;
+			}
+		}
+	}
+}
+
+/* y = alpha * op(A) x + beta * y, as cublasDgemv (A is MxN column-major). */
+static void oracle_gemv(int trans, int M, int N, real alpha, const real *A, int lda, const real *x,
+                        real beta, real *y)
+{
+	if (trans == OP_N)
+		oracle_gemm(OP_N, OP_N, M, 1, N, alpha, A, lda, x, N, beta, y, M);
+	else
+		oracle_gemm(OP_T, OP_N, N, 1, M, alpha, A, lda, x, M, beta, y, N);
+}
+
+/* ------------------------------------------------------------------ */
+/* patch matrices                                                      */
+/* ------------------------------------------------------------------ */
+
+/* functions/dev_image.cu:12-51 (ker_im2col) with the launch of :114-141.
+ * data_im is [C][N][width][height] (height fastest); data_col is the
+ * (N*Hc*Wc) x (C*k*k) column-major patch matrix, column index
+ * c*k*k + j*k + i with j the window column and i the window row. */
+void oracle_im2col(const real *data_im, int samples, int channels, int height, int width, int ksize,
+                   int pad, int stride, real *data_col)
+{
+	int height_col = (height + 2 * pad - ksize) / stride + 1;
+	int width_col = (width + 2 * pad - ksize) / stride + 1;
+	size_t plane = (size_t)height_col * width_col * samples;
+#pragma omp parallel for collapse(2) schedule(static)
+	for (int channel_in = 0; channel_in < channels; channel_in++) {
+		for (int n = 0; n < samples; n++) {
+			for (int w_out = 0; w_out < width_col; w_out++) {
+				for (int h_out = 0; h_out < height_col; h_out++) {
+					int h_in = h_out * stride - pad;
+					int w_in = w_out * stride - pad;
+					real *col = data_col + (size_t)channel_in * ksize * ksize * plane +
+					            (size_t)n * height_col * width_col + (size_t)w_out * height_col + h_out;
+					const real *im = data_im + ((size_t)channel_in * samples + n) * height * width;
+					for (int j = 0; j < ksize; j++) {
+						for (int i = 0; i < ksize; i++) {
+							int h = h_in + i, w = w_in + j;
+							*col = (h >= 0 && w >= 0 && h < height && w < width)
+							           ? im[(size_t)w * height + h]
+							           : 0;
+							col += plane;
+						}
+					}
+				}
+			}
+		}
+	}
+}
+
+/* functions/dev_backprop_convolution.cu:60-96 (kerBackPropConvolutionBatchHelper):
+ * patch matrix of delta for the input gradient, (N*H*W) x (dChannels*fH*fW),
+ * window walked from (col+pad, row+pad) downwards. */
+static void oracle_delta_cols(const real *delta, int dHeight, int dWidth, int dChannels, int fHeight,
+                              int fWidth, real *img, int height, int width, int padding, int samples)
+{
+	size_t plane = (size_t)height * width * samples;
+#pragma omp parallel for collapse(2) schedule(static)
+	for (int chId = 0; chId < dChannels; chId++) {
+		for (int imgId = 0; imgId < samples; imgId++) {
+			for (int myCol = 0; myCol < width; myCol++) {
+				for (int myRow = 0; myRow < height; myRow++) {
+					size_t imgOffset = (size_t)chId * fHeight * fWidth * plane +
+					                   (size_t)imgId * height * width + (size_t)myCol * height + myRow;
+					size_t deltaOffset =
+					    (size_t)chId * samples * dHeight * dWidth + (size_t)imgId * dHeight * dWidth;
+					for (int c = myCol + padding; c > myCol + padding - fWidth; c--) {
+						for (int r = myRow + padding; r > myRow + padding - fHeight; r--) {
+							int ok = (c < dWidth) && (c >= 0) && (r >= 0) && (r < dHeight);
+							img[imgOffset] = ok ? delta[deltaOffset + (size_t)c * dHeight + r] : 0;
+							imgOffset += plane;
+						}
+					}
+				}
+			}
+		}
+	}
+}
+
+/* functions/dev_backprop_convolution.cu:140-168 (kerReshapeMatrix / reshapeMatrix):
+ * [right][left][chunk] -> [left][right][chunk]. */
+void oracle_reshape(const real *input, int rightChannels, int leftChannels, int chunk, real *output)
+{
+	for (int nId = 0; nId < rightChannels; nId++)
+		for (int cId = 0; cId < leftChannels; cId++)
+			for (int t = 0; t < chunk; t++)
+				output[(size_t)cId * chunk * rightChannels + (size_t)nId * chunk + t] =
+				    input[((size_t)nId * leftChannels + cId) * chunk + t];
+}
+
+/* functions/dev_transpose.cu:8-30 (ker_transpose): every height x width map,
+ * stored column-major, is rewritten row-major (departure D4). */
+void oracle_transpose(const real *input, int maps, int height, int width, real *output)
+{
+	for (int m = 0; m < maps; m++)
+		for (int col = 0; col < width; col++)
+			for (int row = 0; row < height; row++)
+				output[(size_t)m * height * width + (size_t)row * width + col] =
+				    input[(size_t)m * height * width + (size_t)col * height + row];
+}
+
+/* functions/dev_transpose.cu:36-58 (ker_transpose_rc): row-major -> column-major. */
+void oracle_transpose_rc(const real *input, int maps, int height, int width, real *output)
+{
+	for (int m = 0; m < maps; m++)
+		for (int row = 0; row < height; row++)
+			for (int col = 0; col < width; col++)
+				output[(size_t)m * height * width + (size_t)col * height + row] =
+				    input[(size_t)m * height * width + (size_t)row * width + col];
+}
+
+/* ------------------------------------------------------------------ */
+/* activations                                                         */
+/* ------------------------------------------------------------------ */
+
+/* Forward activations in place: functions/dev_activations.cu:8-95,
+ * functions/swish.cu:14-23; switch of functions/eval_convolution.cu:172-205
+ * and functions/eval_gradient.cu:141-229.  Returns -1 for an unknown code. */
+int oracle_activation_forward(int actFun, real *x, size_t n)
+{
+	switch (actFun) {
+	case CNN_ACT_RELU:
+		for (size_t i = 0; i < n; i++)
+			if (x[i] < 0) x[i] = 0;
+		break;
+	case CNN_ACT_SOFTPLUS:
+		for (size_t i = 0; i < n; i++)
+			if (x[i] < 20) x[i] = log(1 + exp(x[i]));
+		break;
+	case CNN_ACT_ELU:
+		for (size_t i = 0; i < n; i++)
+			if (x[i] < 0) x[i] = 1.0 * (exp(x[i]) - 1);
+		break;
+	case CNN_ACT_SWISH:
+		for (size_t i = 0; i < n; i++) x[i] = x[i] / (1 + exp(-x[i]));
+		break;
+	case ACT_LOGISTIC:
+		for (size_t i = 0; i < n; i++) x[i] = 1. / (1. + exp(-x[i]));
+		break;
+	case ACT_TANH:
+		for (size_t i = 0; i < n; i++) x[i] = tanh(x[i]);
+		break;
+	case ACT_LINEAR:
+	case CNN_ACT_NONE:
+		break;
+	default:
+		return -1;
+	}
+	return 0;
+}
+
+/* delta *= f'(.) : functions/swish.cu:34-43, functions/dev_layer_error.cu:13-48,
+ * switches of functions/cnn_backward.cu:120-175 and :523-592.  z_in is the
+ * activation's input, z_out its output.  ReLU/ELU: departure D1. */
+int oracle_activation_backward(int actFun, real *delta, const real *z_in, const real *z_out, size_t n)
+{
+	switch (actFun) {
+	case ACT_LOGISTIC:
+		for (size_t i = 0; i < n; i++) delta[i] = delta[i] * z_out[i] * (1.0 - z_out[i]);
+		break;
+	case ACT_TANH:
+		for (size_t i = 0; i < n; i++) delta[i] *= (1.0 + z_out[i]) * (1.0 - z_out[i]);
+		break;
+	case CNN_ACT_SOFTPLUS:
+		for (size_t i = 0; i < n; i++) delta[i] *= 1. / (1. + exp(-z_in[i]));
+		break;
+	case CNN_ACT_SWISH:
+		for (size_t i = 0; i < n; i++) {
+			real t = 1. / (1. + exp(-z_in[i]));
+			delta[i] *= (z_out[i] + t * (1. - z_out[i]));
+		}
+		break;
+	case CNN_ACT_RELU:
+		for (size_t i = 0; i < n; i++)
+			if (!(z_out[i] > 0)) delta[i] = 0;
+		break;
+	case CNN_ACT_ELU:
+		for (size_t i = 0; i < n; i++)
+			if (z_out[i] < 0) delta[i] *= (z_out[i] + 1.0);
+		break;
+	case ACT_LINEAR:
+	case CNN_ACT_NONE:
+		break;
+	default:
+		return -1;
+	}
+	return 0;
+}
+
+/* ------------------------------------------------------------------ */
+/* pooling                                                             */
+/* ------------------------------------------------------------------ */
+
+/* functions/dev_pool.cu:79-121 (ker_max_pool_layer), window origin per D2. */
+void oracle_max_pool_forward(const real *input, int samples, int channels, int height, int width,
+                             int ksize, int stride, int padding, int p_height, int p_width, real *output)
+{
+#pragma omp parallel for collapse(2) schedule(static)
+	for (int ch = 0; ch < channels; ch++) {
+		for (int idx = 0; idx < samples; idx++) {
+			const real *in = input + ((size_t)ch * samples + idx) * height * width;
+			real *out = output + ((size_t)ch * samples + idx) * p_height * p_width;
+			for (int l = 0; l < p_width; l++) {
+				for (int k = 0; k < p_height; k++) {
+					int i = k * stride - padding, j = l * stride - padding;
+					real val = -REAL_MAX;
+					for (int r = 0; r < ksize; r++) {
+						for (int c = 0; c < ksize; c++) {
+							int frow = i + r, fcol = j + c;
+							if (frow < 0 || fcol < 0 || frow >= height || fcol >= width) continue;
+							real t = in[frow + (size_t)fcol * height];
+							if (t > val) val = t;
+						}
+					}
+					out[(size_t)l * p_height + k] = val;
+				}
+			}
+		}
+	}
+}
+
+/* functions/dev_pool.cu:41-77 (ker_avg_pool_layer): sum of the in-range cells / ksize^2. */
+void oracle_avg_pool_forward(const real *input, int samples, int channels, int height, int width,
+                             int ksize, int stride, int padding, int p_height, int p_width, real *output)
+{
+	for (int ch = 0; ch < channels; ch++) {
+		for (int idx = 0; idx < samples; idx++) {
+			const real *in = input + ((size_t)ch * samples + idx) * height * width;
+			real *out = output + ((size_t)ch * samples + idx) * p_height * p_width;
+			for (int l = 0; l < p_width; l++) {
+				for (int k = 0; k < p_height; k++) {
+					int i = k * stride - padding, j = l * stride - padding;
+					real val = 0;
+					for (int r = 0; r < ksize; r++) {
+						for (int c = 0; c < ksize; c++) {
+							int frow = i + r, fcol = j + c;
+							if (frow < 0 || fcol < 0 || frow >= height || fcol >= width) continue;
+							val += in[frow + (size_t)fcol * height];
+						}
+					}
+					out[(size_t)l * p_height + k] = val / (ksize * ksize);
+				}
+			}
+		}
+	}
+}
+
+/* Position (offset inside one height x width map) selected by the reference's
+ * backward scan, functions/dev_pool.cu:374-391: window columns outer, rows
+ * inner, strict '>' -- i.e. the first maximum in memory order. */
+static int argmax_in_window(const real *in, int height, int width, int ksize, int i, int j)
+{
+	int best = INT_MAX;
+	real maxVal = -REAL_MAX;
+	for (int c = 0; c < ksize; c++) {
+		for (int r = 0; r < ksize; r++) {
+			int fcol = j + c, frow = i + r;
+			if (fcol < 0 || fcol >= width || frow < 0 || frow >= height) continue;
+			int tid = frow + fcol * height;
+			if (in[tid] > maxVal) {
+				maxVal = in[tid];
+				best = tid;
+			}
+		}
+	}
+	return best;
+}
+
+/* argmax offsets for every pooled cell, same layout as the pooled tensor. */
+void oracle_max_pool_argmax(const real *z_in, int samples, int channels, int height, int width,
+                            int ksize, int stride, int padding, int p_height, int p_width, int *index)
+{
+	for (int ch = 0; ch < channels; ch++)
+		for (int idx = 0; idx < samples; idx++)
+			for (int l = 0; l < p_width; l++)
+				for (int k = 0; k < p_height; k++)
+					index[((size_t)ch * samples + idx) * p_height * p_width + (size_t)l * p_height + k] =
+					    argmax_in_window(z_in + ((size_t)ch * samples + idx) * height * width, height,
+					                     width, ksize, k * stride - padding, l * stride - padding);
+}
+
+/* functions/dev_pool.cu:346-398 + :474-497 (memset, then add delta at the argmax). */
+void oracle_max_pool_backward(const real *delta, const real *z_in, int channels, int height, int width,
+                              int ksize, int stride, int padding, int p_height, int p_width, int samples,
+                              real *output)
+{
+	memset(output, 0, sizeof(real) * (size_t)height * width * channels * samples);
+#pragma omp parallel for collapse(2) schedule(static)
+	for (int ch = 0; ch < channels; ch++) {
+		for (int idx = 0; idx < samples; idx++) {
+			const real *in = z_in + ((size_t)ch * samples + idx) * height * width;
+			real *out = output + ((size_t)ch * samples + idx) * height * width;
+			const real *d = delta + ((size_t)ch * samples + idx) * p_height * p_width;
+			for (int l = 0; l < p_width; l++) {
+				for (int k = 0; k < p_height; k++) {
+					int t = argmax_in_window(in, height, width, ksize, k * stride - padding,
+					                         l * stride - padding);
+					if (t != INT_MAX) out[t] += d[(size_t)l * p_height + k];
+				}
+			}
+		}
+	}
+}
+
+/* functions/cnn_backward.cu:465-481 (scale by 1/ksize^2) + functions/dev_pool.cu:269-298
+ * (spread over the window), written as the adjoint of the forward (D3). */
+void oracle_avg_pool_backward(const real *delta, int channels, int height, int width, int ksize,
+                              int stride, int padding, int p_height, int p_width, int samples,
+                              real *output)
+{
+	memset(output, 0, sizeof(real) * (size_t)height * width * channels * samples);
+	real scale = 1. / (ksize * ksize);
+	for (int ch = 0; ch < channels; ch++) {
+		for (int idx = 0; idx < samples; idx++) {
+			real *out = output + ((size_t)ch * samples + idx) * height * width;
+			const real *d = delta + ((size_t)ch * samples + idx) * p_height * p_width;
+			for (int l = 0; l < p_width; l++) {
+				for (int k = 0; k < p_height; k++) {
+					int i = k * stride - padding, j = l * stride - padding;
+					for (int c = 0; c < ksize; c++) {
+						for (int r = 0; r < ksize; r++) {
+							int fcol = j + c, frow = i + r;
+							if (fcol < 0 || fcol >= width || frow < 0 || frow >= height) continue;
+							out[frow + (size_t)fcol * height] += scale * d[(size_t)l * p_height + k];
+						}
+					}
+				}
+			}
+		}
+	}
+}
+
+/* ------------------------------------------------------------------ */
+/* batch normalisation (spatial, non-affine)                           */
+/* ------------------------------------------------------------------ */
+
+/* functions/dev_batch_norm.cu:263-315 (mean, biased variance, running
+ * statistics), :27-38 (z-hat), :331-393 (train / evaluation switch).
+ * output holds rows*channels reals followed by the four per-channel vectors
+ * at the given offsets (relative to output). */
+void oracle_batch_norm_forward(const real *input, int height, int width, int channels, int samples,
+                               real *output, int meansOffset, int variancesOffset, real epsilon,
+                               int forTesting, real momentum, int runningMeansOffset,
+                               int runningVariancesOffset)
+{
+	size_t rows = (size_t)height * width * samples;
+	real *batch_mean = output + meansOffset;
+	real *batch_variance = output + variancesOffset;
+	real *dataset_mean = output + runningMeansOffset;
+	real *dataset_variance = output + runningVariancesOffset;
+
+	if (forTesting == MODEL_TRAIN) {
+		for (int c = 0; c < channels; c++) {
+			const real *x = input + (size_t)c * rows;
+			real s = 0;
+			for (size_t i = 0; i < rows; i++) s += x[i];
+			batch_mean[c] = s * (1. / (real)rows);
+			real v = 0;
+			for (size_t i = 0; i < rows; i++) {
+				real t = x[i] - batch_mean[c];
+				v += t * t;
+			}
+			batch_variance[c] = v * (1. / (real)rows);
+			dataset_mean[c] = momentum * dataset_mean[c] + (1. - momentum) * batch_mean[c];
+			dataset_variance[c] = momentum * dataset_variance[c] + (1. - momentum) * batch_variance[c];
+		}
+	}
+	const real *mu = (forTesting == MODEL_TRAIN) ? batch_mean : dataset_mean;
+	const real *var = (forTesting == MODEL_TRAIN) ? batch_variance : dataset_variance;
+	for (int c = 0; c < channels; c++)
+		for (size_t i = 0; i < rows; i++)
+			output[(size_t)c * rows + i] = (input[(size_t)c * rows + i] - mu[c]) / sqrt(var[c] + epsilon);
+}
+
+/* functions/dev_batch_norm.cu:550-621 with the helper :398-466 and the kernel
+ * :132-150: out = (m*delta - sum(delta) - zhat * sum(delta*zhat)) / (m*sqrt(eps+var)). */
+void oracle_batch_norm_backward(const real *delta, int height, int width, int channels, int samples,
+                                const real *variance, real *output, const real *zout, real epsilon)
+{
+	size_t rows = (size_t)height * width * samples;
+#pragma omp parallel for schedule(static)
+	for (int c = 0; c < channels; c++) {
+		const real *d = delta + (size_t)c * rows;
+		const real *zh = zout + (size_t)c * rows;
+		real *o = output + (size_t)c * rows;
+		real sum1 = 0, sum2 = 0;
+		for (size_t i = 0; i < rows; i++) {
+			sum1 += d[i];
+			sum2 += d[i] * zh[i];
+		}
+		real m = (real)rows;
+		for (size_t i = 0; i < rows; i++)
+			o[i] = (m * d[i] - sum1 - sum2 * zh[i]) / (m * sqrt(epsilon + variance[c]));
+	}
+}
+
+/* ------------------------------------------------------------------ */
+/* softmax cross entropy                                               */
+/* ------------------------------------------------------------------ */
+
+/* functions/softmax_loss.cu:17-79 + :141-213: probs (class fastest), mean
+ * negative log-likelihood.  maxdot starts at 0 and 1e-10 is added to every
+ * probability, as in the reference.  target holds 1-based class ids. */
+real oracle_softmax_loss(const real *input, const real *target, int rows, int num_classes, real *probs)
+{
+	real total = 0;
+	for (int r = 0; r < rows; r++) {
+		real maxdot = 0;
+		for (int i = 0; i < num_classes; i++)
+			if (maxdot < input[i + (size_t)r * num_classes]) maxdot = input[i + (size_t)r * num_classes];
+		real s = 0;
+		for (int i = 0; i < num_classes; i++) {
+			probs[i + (size_t)r * num_classes] = exp(input[i + (size_t)r * num_classes] - maxdot);
+			s += probs[i + (size_t)r * num_classes];
+		}
+		for (int i = 0; i < num_classes; i++)
+			probs[i + (size_t)r * num_classes] = probs[i + (size_t)r * num_classes] / s + 1e-10;
+		real ind = 0;
+		for (int i = 0; i < num_classes; i++)
+			if ((int)target[r] == (i + 1)) ind = -log(probs[i + (size_t)r * num_classes]);
+		total += ind;
+	}
+	return total / rows;
+}
+
+/* functions/softmax_loss.cu:215-245: errors = (probs - onehot) / rows. */
+void oracle_cross_entropy_error(const real *probs, int rows, int numclasses, const real *target,
+                                real *errors)
+{
+	real alpha = 1. / (real)rows;
+	for (int r = 0; r < rows; r++)
+		for (int c = 0; c < numclasses; c++) {
+			real v = probs[c + (size_t)r * numclasses];
+			if ((real)(c + 1) == target[r]) v -= 1.;
+			errors[c + (size_t)r * numclasses] = v * alpha;
+		}
+}
+
+/* ------------------------------------------------------------------ */
+/* layers                                                              */
+/* ------------------------------------------------------------------ */
+
+/* functions/eval_convolution.cu:52-267 (applyConvolutionLayer): patch matrix,
+ * GEMM (:115-119), bias (:26-34), batch norm (:132-161), activation
+ * (:172-205), pooling (:215-219).  devScratch >= M*K reals. */
+int oracle_conv_layer_forward(const real *input, int samples, int in_channels, int height, int width,
+                              int ksize, int pad, int stride, int col_height, int col_width,
+                              const real *weights, const real *bias, real *output, int out_channels,
+                              int actFun, int pkSize, int pkStride, int pkPad, int poolFun,
+                              int poolOutHeight, int poolOutWidth, int performBatchNorm, real epsilon,
+                              int activationOffset, int poolOffset, int batchNormOffset, int meansOffset,
+                              int variancesOffset, real *devScratch, int forTesting,
+                              int runningMeansOffset, int runningVariancesOffset)
+{
+	real *imgCols = devScratch;
+	real *imgColWtOut = output;
+	real *actOut = output + activationOffset;
+	size_t M = (size_t)samples * col_height * col_width;
+	int K = ksize * ksize * in_channels;
+
+	oracle_im2col(input, samples, in_channels, height, width, ksize, pad, stride, imgCols);
+	oracle_gemm(OP_N, OP_N, (int)M, out_channels, K, 1, imgCols, (int)M, weights, K, 0, imgColWtOut, (int)M);
+	if (bias)
+		for (int c = 0; c < out_channels; c++)
+			for (size_t i = 0; i < M; i++) imgColWtOut[(size_t)c * M + i] += bias[c];
+
+	if (performBatchNorm != PERFORM_NO_BATCH_NORM) {
+		real *batchOut = output + batchNormOffset;
+		oracle_batch_norm_forward(imgColWtOut, col_height, col_width, out_channels, samples, batchOut,
+		                          meansOffset, variancesOffset, epsilon, forTesting, BATCH_NORM_MOMENTUM,
+		                          runningMeansOffset, runningVariancesOffset);
+		memcpy(actOut, batchOut, sizeof(real) * M * out_channels);
+	} else {
+		memcpy(actOut, imgColWtOut, sizeof(real) * M * out_channels);
+	}
+	if (oracle_activation_forward(actFun, actOut, M * out_channels)) return -1;
+
+	if (poolFun == MAX_POOL)
+		oracle_max_pool_forward(actOut, samples, out_channels, col_height, col_width, pkSize, pkStride,
+		                        pkPad, poolOutHeight, poolOutWidth, output + poolOffset);
+	else if (poolFun == AVG_POOL)
+		oracle_avg_pool_forward(actOut, samples, out_channels, col_height, col_width, pkSize, pkStride,
+		                        pkPad, poolOutHeight, poolOutWidth, output + poolOffset);
+	else if (poolFun != NO_POOL)
+		return -1;
+	return 0;
+}
+
+/* functions/eval_gradient.cu:29-229 (applyLayerActivation): W z + b, saved
+ * pre-activation copy behind the output, activation in place. */
+int oracle_fc_layer_forward(int actFunction, const real *W, int wRows, int wCols, const real *b,
+                            const real *z, int zRows, int zCols, real *output)
+{
+	oracle_gemm(OP_N, OP_N, wRows, zCols, wCols, 1, W, wRows, z, zRows, 0, output, wRows);
+	if (b)
+		for (int n = 0; n < zCols; n++)
+			for (int r = 0; r < wRows; r++) output[(size_t)n * wRows + r] += b[r];
+	memcpy(output + (size_t)wRows * zCols, output, sizeof(real) * (size_t)wRows * zCols);
+	return oracle_activation_forward(actFunction, output, (size_t)wRows * zCols);
+}
+
+/* functions/cnn_backward.cu:771-783: dW = im2col(X)^T * delta (K x Cout, ld K). */
+void oracle_conv_weight_gradient(const real *input, const real *delta, int samples, int in_channels,
+                                 int height, int width, int ksize, int pad, int stride,
+                                 int out_channels, real *dW, real *devScratch)
+{
+	int col_h = (height + 2 * pad - ksize) / stride + 1;
+	int col_w = (width + 2 * pad - ksize) / stride + 1;
+	int M = col_h * col_w * samples, K = ksize * ksize * in_channels;
+	oracle_im2col(input, samples, in_channels, height, width, ksize, pad, stride, devScratch);
+	oracle_gemm(OP_T, OP_N, K, out_channels, M, 1, devScratch, M, delta, M, 0, dW, K);
+}
+
+/* functions/dev_backprop_convolution.cu:173-247 (backpropConvolution):
+ * delta patch matrix, weight reorder [Cout][Cin][k*k]->[Cin][Cout][k*k], GEMM. */
+void oracle_conv_input_gradient(const real *delta, int dHeight, int dWidth, int dChannels,
+                                const real *filter, int fHeight, int fWidth, int height, int width,
+                                int padding, int channels, int samples, real *delta_1, real *devPtr)
+{
+	real *imgCols = devPtr;
+	real *reordered = imgCols + (size_t)samples * height * width * fHeight * fWidth * dChannels;
+	oracle_delta_cols(delta, dHeight, dWidth, dChannels, fHeight, fWidth, imgCols, height, width,
+	                  padding, samples);
+	oracle_reshape(filter, dChannels, channels, fHeight * fWidth, reordered);
+	int M = samples * height * width, R = fHeight * fWidth * dChannels;
+	oracle_gemm(OP_N, OP_N, M, channels, R, 1, imgCols, M, reordered, R, 0, delta_1, M);
+}
+
+/* ------------------------------------------------------------------ */
+/* whole model                                                         */
+/* ------------------------------------------------------------------ */
+
+static size_t max_patch_reals(const CNN_MODEL *model, int batch)
+{
+	size_t best = 0;
+	for (int i = 0; i < model->cLayers; i++) {
+		const CONV_LAYER *c = &model->convLayer[i];
+		const POOL_LAYER *p = &model->poolLayer[i];
+		size_t kk = (size_t)c->kSize * c->kSize;
+		size_t fwd = (size_t)p->height * p->width * batch * c->inChannels * kk;
+		size_t bwd = (size_t)c->height * c->width * batch * c->outChannels * kk +
+		             (size_t)c->outChannels * c->inChannels * kk;
+		if (fwd > best) best = fwd;
+		if (bwd > best) best = bwd;
+	}
+	return best + 16;
+}
+
+/* functions/cnn_forward.cu:49-383 (cnnForward).  x is the batch
+ * [C][N][W][H]; y the 1-based labels; returns the mean NLL, or NAN on an
+ * unknown activation / pool code. */
+real oracle_cnn_forward(const CNN_MODEL *model, const real *weights, const real *x, const real *y,
+                        int numClasses, real *z, real *probs, real *errors, int curBatchSize,
+                        int forTesting)
+{
+	const int *wOffsets = model->wOffsets, *bOffsets = model->bOffsets, *zOffsets = model->zOffsets;
+	int nc = model->cLayers;
+	real *scratch = (real *)malloc(sizeof(real) * max_patch_reals(model, curBatchSize));
+	if (!scratch) return NAN;
+
+	for (int l = 0; l < nc; l++) {
+		const CONV_LAYER *cv = &model->convLayer[l];
+		const POOL_LAYER *pl = &model->poolLayer[l];
+		const real *in = (l == 0) ? x : z + zOffsets[l] + model->convLayer[l - 1].outputOffset;
+		int rc = oracle_conv_layer_forward(
+		    in, curBatchSize, cv->inChannels, cv->height, cv->width, cv->kSize, cv->padding, cv->stride,
+		    cv->outHeight, cv->outWidth, weights + wOffsets[l],
+		    (model->bias == 0) ? NULL : weights + bOffsets[l], z + zOffsets[l + 1], cv->outChannels,
+		    model->actFuns[l], pl->pSize, pl->stride, pl->padding, pl->type, pl->outHeight, pl->outWidth,
+		    cv->batchNorm, BATCH_NORM_EPSILON, cv->activationOffset, cv->poolOffset, cv->batchNormOffset,
+		    cv->meansOffset, cv->variancesOffset, scratch, forTesting, cv->runningMeansOffset,
+		    cv->runningVariancesOffset);
+		if (rc) {
+			free(scratch);
+			return NAN;
+		}
+	}
+
+	/* [C][N][w*H+h] -> [N][C][h*W+w], in place (cnn_forward.cu:238-261) */
+	const CONV_LAYER *c = &model->convLayer[nc - 1];
+	const POOL_LAYER *p = &model->poolLayer[nc - 1];
+	int fh = (p->type != NO_POOL) ? p->outHeight : c->outHeight;
+	int fw = (p->type != NO_POOL) ? p->outWidth : c->outWidth;
+	real *feat = z + zOffsets[nc] + c->outputOffset;
+	size_t featCount = (size_t)fh * fw * curBatchSize * c->outChannels;
+	oracle_reshape(feat, c->outChannels, curBatchSize, fh * fw, scratch);
+	oracle_transpose(scratch, c->outChannels * curBatchSize, fh, fw, feat);
+	(void)featCount;
+
+	int outputOffset = c->outputOffset;
+	for (int l = 0; l < model->lLayers; l++) {
+		if (l != 0) outputOffset = 0;
+		const FC_LAYER *f = &model->fcLayer[l];
+		if (oracle_fc_layer_forward(f->actFun, weights + wOffsets[l + nc], f->out, f->in,
+		                            (model->bias == 0) ? NULL : weights + bOffsets[l + nc],
+		                            z + zOffsets[l + nc] + outputOffset, f->in, curBatchSize,
+		                            z + zOffsets[l + 1 + nc])) {
+			free(scratch);
+			return NAN;
+		}
+	}
+	const real *logits = (model->lLayers == 0) ? z + zOffsets[nc] + c->outputOffset
+	                                           : z + zOffsets[model->lLayers + nc];
+	real loss = oracle_softmax_loss(logits, y, curBatchSize, numClasses, probs);
+	oracle_cross_entropy_error(probs, curBatchSize, numClasses, y, errors);
+	free(scratch);
+	return loss;
+}
+
+/* functions/cnn_backward.cu:76-857 (cnnBackward).  delta holds the loss
+ * errors on entry; delta and delta_new are clobbered.  Returns 0, or -1 on an
+ * unknown activation / pool code (where the reference exits). */
+int oracle_cnn_backward(const CNN_MODEL *model, const real *weights, const real *x, const real *z,
+                        real *gradient, real *dx, real *delta, real *delta_new, int batchSize)
+{
+	const int *wOffsets = model->wOffsets, *bOffsets = model->bOffsets, *zOffsets = model->zOffsets;
+	int n = batchSize, cLayers = model->cLayers;
+	real *scratch = (real *)malloc(sizeof(real) * max_patch_reals(model, batchSize));
+	if (!scratch) return -1;
+	const CONV_LAYER *cLayer = &model->convLayer[cLayers - 1];
+	const POOL_LAYER *pLayer = &model->poolLayer[cLayers - 1];
+	real *temp;
+
+	for (int f = model->lLayers - 1; f >= 0; f--) {
+		FC_LAYER l = model->fcLayer[f];
+		const real *zl = z + zOffsets[f + cLayers + 1];
+		if (oracle_activation_backward(l.actFun, delta, zl + l.offset, zl, (size_t)l.out * n)) {
+			free(scratch);
+			return -1;
+		}
+		/* dW = delta * z' (:189-197) */
+		oracle_gemm(OP_N, OP_T, l.out, l.in, n, 1, delta, l.out,
+		            z + zOffsets[f + cLayers] + ((f == 0) ? cLayer->outputOffset : 0), l.in, 0,
+		            gradient + wOffsets[f + cLayers], l.out);
+		if (model->bias != 0) {
+			/* db = delta * 1 (:212-224) */
+			for (int i = 0; i < n; i++) scratch[i] = 1;
+			oracle_gemv(OP_N, l.out, n, 1, delta, l.out, scratch, 0, gradient + bOffsets[f + cLayers]);
+		}
+		memcpy(dx + zOffsets[f + cLayers + 1], delta, sizeof(real) * (size_t)l.out * n);
+		/* delta = W' * delta (:250-254) */
+		oracle_gemm(OP_T, OP_N, l.in, n, l.out, 1, weights + wOffsets[f + cLayers], l.out, delta, l.out, 0,
+		            delta_new, l.in);
+		temp = delta_new;
+		delta_new = delta;
+		delta = temp;
+	}
+
+	/* [N][C][h*W+w] -> [C][N][w*H+h] (:310-326) */
+	{
+		int fh = (pLayer->type != NO_POOL) ? pLayer->outHeight : cLayer->outHeight;
+		int fw = (pLayer->type != NO_POOL) ? pLayer->outWidth : cLayer->outWidth;
+		oracle_reshape(delta, n, cLayer->outChannels, fh * fw, scratch);
+		oracle_transpose_rc(scratch, cLayer->outChannels * n, fh, fw, delta);
+	}
+
+	for (int c = cLayers - 1; c >= 0; c--) {
+		CONV_LAYER l = model->convLayer[c];
+		POOL_LAYER p = model->poolLayer[c];
+		const real *slab = z + zOffsets[c + 1];
+		size_t actCount = (size_t)n * l.activationVolumn;
+
+		switch (p.type) {
+		case MAX_POOL:
+			oracle_max_pool_backward(delta, slab + l.activationOffset, l.outChannels, p.height, p.width,
+			                         p.pSize, p.stride, p.padding, p.outHeight, p.outWidth, n, delta_new);
+			break;
+		case AVG_POOL:
+			oracle_avg_pool_backward(delta, l.outChannels, p.height, p.width, p.pSize, p.stride,
+			                         p.padding, p.outHeight, p.outWidth, n, delta_new);
+			break;
+		case NO_POOL:
+			memcpy(delta_new, delta, sizeof(real) * actCount);
+			break;
+		default:
+			free(scratch);
+			return -1;
+		}
+		memcpy(dx + zOffsets[c + 1], delta_new, sizeof(real) * actCount);
+
+		const real *actIn = (l.batchNorm != PERFORM_NO_BATCH_NORM) ? slab + l.batchNormOffset : slab;
+		const real *actOut = slab + l.activationOffset;
+		if (c == cLayers - 1 && p.type == NO_POOL) {
+			/* departure D6: the stored activation output is in the FC layout */
+			memcpy(scratch, actIn, sizeof(real) * actCount);
+			if (oracle_activation_forward(model->actFuns[c], scratch, actCount)) {
+				free(scratch);
+				return -1;
+			}
+			actOut = scratch;
+		}
+		if (oracle_activation_backward(model->actFuns[c], delta_new, actIn, actOut, actCount)) {
+			free(scratch);
+			return -1;
+		}
+		memcpy(dx + zOffsets[c + 1] + l.activationOffset, delta_new, sizeof(real) * actCount);
+
+		if (l.batchNorm != PERFORM_NO_BATCH_NORM) {
+			oracle_batch_norm_backward(delta_new, l.outHeight, l.outWidth, l.outChannels, n,
+			                           slab + l.batchNormOffset + l.variancesOffset, delta,
+			                           slab + l.batchNormOffset, BATCH_NORM_EPSILON);
+			memcpy(dx + zOffsets[c + 1] + l.batchNormOffset, delta, sizeof(real) * actCount);
+			memcpy(delta_new, delta, sizeof(real) * actCount);
+		}
+
+		int M = p.height * p.width * n;
+		if (model->bias != 0) {
+			/* db = 1' * delta (:662-689) */
+			for (int i = 0; i < M; i++) scratch[i] = 1;
+			oracle_gemm(OP_N, OP_N, 1, l.outChannels, M, 1, scratch, 1, delta_new, M, 0,
+			            gradient + bOffsets[c], 1);
+		}
+
+		const real *dataset = (c == 0) ? x : z + zOffsets[c] + model->convLayer[c - 1].outputOffset;
+		oracle_conv_weight_gradient(dataset, delta_new, n, l.inChannels, l.height, l.width, l.kSize,
+		                            l.padding, l.stride, l.outChannels, gradient + wOffsets[c], scratch);
+		if (c != 0)
+			oracle_conv_input_gradient(delta_new, p.height, p.width, l.outChannels,
+			                           weights + wOffsets[c], l.kSize, l.kSize, l.height, l.width,
+			                           l.padding, l.inChannels, n, delta, scratch);
+	}
+	free(scratch);
+	return 0;
+}
+
+/* functions/cnn_gradient.cu:13-64 (computeCNNGradient): forward, backward,
+ * gradient += weightDecay * weights.  Returns the loss. */
+real oracle_cnn_gradient(const CNN_MODEL *model, const real *weights, const real *x, const real *y,
+                         int numClasses, real *z, real *dx, real *probs, real *lossFuncErrors,
+                         real *gradient, int curBatchSize, real weightDecay)
+{
+	real loss = oracle_cnn_forward(model, weights, x, y, numClasses, z, probs, lossFuncErrors,
+	                               curBatchSize, MODEL_TRAIN);
+	size_t dsz = (size_t)model->maxDeltaSize;
+	real *errors = (real *)calloc(2 * dsz, sizeof(real));
+	if (!errors) return NAN;
+	memcpy(errors, lossFuncErrors, sizeof(real) * (size_t)numClasses * curBatchSize);
+	if (oracle_cnn_backward(model, weights, x, z, gradient, dx, errors, errors + dsz, curBatchSize))
+		loss = NAN;
+	for (int i = 0; i < model->pSize; i++) gradient[i] += weightDecay * weights[i];
+	free(errors);
+	return loss;
+}
+
+int oracle_sizeof_real(void) { return (int)sizeof(real); }

@@ -1,0 +1,219 @@
+"""ctypes front end of the CPU oracle (oracle/fitre_oracle.c).
+
+TEST INFRASTRUCTURE ONLY.  Imported by tests/, by __graft_entry__.smoke() and by
+the cpu_baseline leg of bench.py; never by the fitre_amd package.
+
+Two builds of the same C file: float64 (`f64`, the parity checker) and float32
+(`f32`, the timed CPU baseline).  Arrays are numpy arrays in the reference's
+flat layouts; see the C file for the reference lines each function follows.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+from fitre_amd.structs import CNN_MODEL
+
+_DIR = os.path.dirname(os.path.abspath(__file__))
+
+
+def build():
+    """Compiles both oracle libraries with the Makefile next to this file."""
+    subprocess.run(["make", "-s", "-C", _DIR, "all"], check=True)
+
+
+class Oracle:
+    def __init__(self, double=True):
+        name = "libfitre_oracle_f64.so" if double else "libfitre_oracle_f32.so"
+        path = os.path.join(_DIR, name)
+        if not os.path.exists(path):
+            build()
+        self.lib = C.CDLL(path)
+        self.dtype = np.float64 if double else np.float32
+        self.creal = C.c_double if double else C.c_float
+        assert self.lib.oracle_sizeof_real() == np.dtype(self.dtype).itemsize
+        self.lib.oracle_cnn_forward.restype = self.creal
+        self.lib.oracle_cnn_gradient.restype = self.creal
+        self.lib.oracle_softmax_loss.restype = self.creal
+
+    # ---- helpers -------------------------------------------------------
+    def arr(self, a):
+        return np.ascontiguousarray(a, dtype=self.dtype)
+
+    def zeros(self, n):
+        return np.zeros(int(n), dtype=self.dtype)
+
+    @staticmethod
+    def p(a):
+        return a.ctypes.data_as(C.c_void_p)
+
+    def r(self, v):
+        return self.creal(v)
+
+    # ---- whole model ---------------------------------------------------
+    def forward(self, model: CNN_MODEL, weights, x, y, classes, batch, mode=10, z=None):
+        """Returns (loss, z, probs, errors).  Pass z to carry running batch-norm statistics."""
+        weights, x, y = self.arr(weights), self.arr(x), self.arr(y)
+        z = self.zeros(model.zSize) if z is None else z
+        probs, errors = self.zeros(classes * batch), self.zeros(classes * batch)
+        loss = self.lib.oracle_cnn_forward(C.byref(model), self.p(weights), self.p(x), self.p(y), classes,
+                                           self.p(z), self.p(probs), self.p(errors), batch, mode)
+        return float(loss), z, probs, errors
+
+    def backward(self, model: CNN_MODEL, weights, x, z, errors, batch):
+        """Returns (gradient, dx)."""
+        weights, x = self.arr(weights), self.arr(x)
+        grad, dx = self.zeros(model.pSize), self.zeros(model.zSize)
+        delta = self.zeros(model.maxDeltaSize)
+        delta[:errors.size] = errors
+        delta_new = self.zeros(model.maxDeltaSize)
+        rc = self.lib.oracle_cnn_backward(C.byref(model), self.p(weights), self.p(x), self.p(z), self.p(grad),
+                                          self.p(dx), self.p(delta), self.p(delta_new), batch)
+        if rc != 0:
+            raise ValueError("oracle_cnn_backward: unknown activation or pooling code")
+        return grad, dx
+
+    def gradient(self, model: CNN_MODEL, weights, x, y, classes, batch, weight_decay=0.0):
+        """computeCNNGradient: returns dict(loss, gradient, z, dx, probs, errors)."""
+        weights, x, y = self.arr(weights), self.arr(x), self.arr(y)
+        z, dx = self.zeros(model.zSize), self.zeros(model.zSize)
+        probs, errors = self.zeros(classes * batch), self.zeros(classes * batch)
+        grad = self.zeros(model.pSize)
+        loss = self.lib.oracle_cnn_gradient(C.byref(model), self.p(weights), self.p(x), self.p(y), classes,
+                                            self.p(z), self.p(dx), self.p(probs), self.p(errors), self.p(grad),
+                                            batch, self.r(weight_decay))
+        return dict(loss=float(loss), gradient=grad, z=z, dx=dx, probs=probs, errors=errors)
+
+    # ---- single operations ------------------------------------------------
+    def gemm(self, ta, tb, M, N, K, alpha, A, lda, B, ldb, beta, Cm, ldc):
+        A, B, Cm = self.arr(A), self.arr(B), self.arr(Cm).copy()
+        self.lib.oracle_gemm(ta, tb, M, N, K, self.r(alpha), self.p(A), lda, self.p(B), ldb, self.r(beta),
+                             self.p(Cm), ldc)
+        return Cm
+
+    def im2col(self, x, samples, channels, height, width, k, pad, stride):
+        x = self.arr(x)
+        hc, wc = (height + 2 * pad - k) // stride + 1, (width + 2 * pad - k) // stride + 1
+        col = self.zeros(hc * wc * samples * channels * k * k)
+        self.lib.oracle_im2col(self.p(x), samples, channels, height, width, k, pad, stride, self.p(col))
+        return col
+
+    def conv_forward(self, x, w, bias, samples, cin, height, width, k, pad, stride, cout):
+        """Convolution output only ([Cout][N][Wc][Hc])."""
+        x, w = self.arr(x), self.arr(w)
+        hc, wc = (height + 2 * pad - k) // stride + 1, (width + 2 * pad - k) // stride + 1
+        M, K = hc * wc * samples, k * k * cin
+        col = self.im2col(x, samples, cin, height, width, k, pad, stride)
+        out = self.gemm(0, 0, M, cout, K, 1.0, col, M, w, K, 0.0, self.zeros(M * cout), M)
+        if bias is not None:
+            out = (out.reshape(cout, M) + self.arr(bias)[:, None]).reshape(-1)
+        return out
+
+    def conv_weight_grad(self, x, delta, samples, cin, height, width, k, pad, stride, cout):
+        x, delta = self.arr(x), self.arr(delta)
+        hc, wc = (height + 2 * pad - k) // stride + 1, (width + 2 * pad - k) // stride + 1
+        dW = self.zeros(cout * cin * k * k)
+        scratch = self.zeros(hc * wc * samples * cin * k * k)
+        self.lib.oracle_conv_weight_gradient(self.p(x), self.p(delta), samples, cin, height, width, k, pad, stride,
+                                             cout, self.p(dW), self.p(scratch))
+        return dW
+
+    def conv_input_grad(self, delta, w, samples, cin, height, width, k, pad, cout):
+        delta, w = self.arr(delta), self.arr(w)
+        dh, dw = height + 2 * pad - k + 1, width + 2 * pad - k + 1
+        out = self.zeros(samples * height * width * cin)
+        scratch = self.zeros(samples * height * width * k * k * cout + cout * cin * k * k)
+        self.lib.oracle_conv_input_gradient(self.p(delta), dh, dw, cout, self.p(w), k, k, height, width, pad, cin,
+                                            samples, self.p(out), self.p(scratch))
+        return out
+
+    def activation_forward(self, act, x):
+        x = self.arr(x).copy()
+        rc = self.lib.oracle_activation_forward(act, self.p(x), C.c_size_t(x.size))
+        if rc:
+            raise ValueError("unknown activation %d" % act)
+        return x
+
+    def activation_backward(self, act, delta, z_in, z_out):
+        d = self.arr(delta).copy()
+        z_in, z_out = self.arr(z_in), self.arr(z_out)
+        rc = self.lib.oracle_activation_backward(act, self.p(d), self.p(z_in), self.p(z_out), C.c_size_t(d.size))
+        if rc:
+            raise ValueError("unknown activation %d" % act)
+        return d
+
+    def pool_forward(self, kind, x, samples, channels, height, width, k, stride, pad):
+        x = self.arr(x)
+        ph, pw = (height + 2 * pad - k) // stride + 1, (width + 2 * pad - k) // stride + 1
+        out = self.zeros(ph * pw * samples * channels)
+        fn = self.lib.oracle_max_pool_forward if kind == 0 else self.lib.oracle_avg_pool_forward
+        fn(self.p(x), samples, channels, height, width, k, stride, pad, ph, pw, self.p(out))
+        return out
+
+    def max_pool_argmax(self, x, samples, channels, height, width, k, stride, pad):
+        x = self.arr(x)
+        ph, pw = (height + 2 * pad - k) // stride + 1, (width + 2 * pad - k) // stride + 1
+        idx = np.zeros(ph * pw * samples * channels, dtype=np.int32)
+        self.lib.oracle_max_pool_argmax(self.p(x), samples, channels, height, width, k, stride, pad, ph, pw,
+                                        idx.ctypes.data_as(C.c_void_p))
+        return idx
+
+    def pool_backward(self, kind, delta, z_in, samples, channels, height, width, k, stride, pad):
+        delta = self.arr(delta)
+        ph, pw = (height + 2 * pad - k) // stride + 1, (width + 2 * pad - k) // stride + 1
+        out = self.zeros(height * width * samples * channels)
+        if kind == 0:
+            z_in = self.arr(z_in)
+            self.lib.oracle_max_pool_backward(self.p(delta), self.p(z_in), channels, height, width, k, stride, pad,
+                                              ph, pw, samples, self.p(out))
+        else:
+            self.lib.oracle_avg_pool_backward(self.p(delta), channels, height, width, k, stride, pad, ph, pw,
+                                              samples, self.p(out))
+        return out
+
+    def batch_norm_forward(self, x, height, width, channels, samples, eps=1e-5, train=True, momentum=0.9,
+                           running=None):
+        """Returns (zhat, mean, var, running_mean, running_var)."""
+        x = self.arr(x)
+        n = height * width * samples * channels
+        out = self.zeros(n + 4 * channels)
+        if running is not None:
+            out[n + 2 * channels:n + 3 * channels] = running[0]
+            out[n + 3 * channels:] = running[1]
+        self.lib.oracle_batch_norm_forward(self.p(x), height, width, channels, samples, self.p(out), n, n + channels,
+                                           self.r(eps), 10 if train else 20, self.r(momentum), n + 2 * channels,
+                                           n + 3 * channels)
+        c = channels
+        return out[:n], out[n:n + c], out[n + c:n + 2 * c], out[n + 2 * c:n + 3 * c], out[n + 3 * c:]
+
+    def batch_norm_backward(self, delta, zhat, variance, height, width, channels, samples, eps=1e-5):
+        delta, zhat, variance = self.arr(delta), self.arr(zhat), self.arr(variance)
+        out = self.zeros(delta.size)
+        self.lib.oracle_batch_norm_backward(self.p(delta), height, width, channels, samples, self.p(variance),
+                                            self.p(out), self.p(zhat), self.r(eps))
+        return out
+
+    def softmax_loss(self, logits, target, rows, classes):
+        logits, target = self.arr(logits), self.arr(target)
+        probs = self.zeros(rows * classes)
+        loss = self.lib.oracle_softmax_loss(self.p(logits), self.p(target), rows, classes, self.p(probs))
+        return float(loss), probs
+
+    def cross_entropy_error(self, probs, target, rows, classes):
+        probs, target = self.arr(probs), self.arr(target)
+        err = self.zeros(rows * classes)
+        self.lib.oracle_cross_entropy_error(self.p(probs), rows, classes, self.p(target), self.p(err))
+        return err
+
+    def reshape(self, x, right, left, chunk):
+        x = self.arr(x)
+        out = self.zeros(x.size)
+        self.lib.oracle_reshape(self.p(x), right, left, chunk, self.p(out))
+        return out
+
+    def transpose(self, x, maps, height, width, rc=False):
+        x = self.arr(x)
+        out = self.zeros(x.size)
+        (self.lib.oracle_transpose_rc if rc else self.lib.oracle_transpose)(self.p(x), maps, height, width, self.p(out))
+        return out

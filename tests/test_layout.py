@@ -1,0 +1,123 @@
+"""Flat parameter / activation-store layout (nn/utils.c:12-172, nn/read_vgg.c:25-120) and ABI surface."""
+import ctypes as C
+import json
+import os
+import re
+
+import numpy as np
+
+from fitre_amd import lib as L
+from fitre_amd.structs import (CNN_ACT_RELU, CNN_ACT_SWISH, CNN_MODEL, INT_MAX, MAX_POOL, NO_POOL)
+from helpers import build_alexnet, build_custom, build_lenet, build_vgg11
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+
+
+def test_lenet_offsets_match_reference_log():
+    want = json.load(open(os.path.join(HERE, "golden", "lenet_offsets.json")))["offsets"]
+    m = build_lenet(128, bn=False, bias=1)
+    got = []
+    for l in range(m.cLayers + m.lLayers):
+        got += [m.wOffsets[l], m.bOffsets[l]]
+    got.append(m.pSize)
+    assert got == want
+
+
+def test_param_sizes_of_the_benchmark_configs():
+    # 3x3 convs 3-64-128-256-256-512-512-512-512 + FC 512->10, with biases
+    convs = [(3, 64), (64, 128), (128, 256), (256, 256), (256, 512), (512, 512), (512, 512), (512, 512)]
+    want = sum(9 * a * b + b for a, b in convs) + 512 * 10 + 10
+    m = build_vgg11(256)
+    assert m.pSize == want == 9225610
+    assert m.zSize == 124403456
+    assert build_alexnet(64).pSize == 62378344
+    # AlexNet extents 224 -> 55 -> 27 -> 27 -> 13 -> 13/13/13 -> 6
+    a = build_alexnet(64)
+    assert [a.convLayer[i].outHeight for i in range(5)] == [55, 27, 13, 13, 13]
+    assert [a.poolLayer[i].outHeight for i in range(5)] == [27, 13, 13, 13, 6]
+    assert a.fcLayer[0].in_ == 9216
+
+
+def test_no_bias_offsets():
+    m = build_lenet(4, bias=0)
+    assert m.pSize == 450 + 2400 + 48000 + 10080 + 840
+    assert [m.wOffsets[i] for i in range(6)] == [0, 450, 2850, 50850, 60930, 61770]
+    assert all(m.bOffsets[i] == INT_MAX for i in range(5))
+
+
+def test_slab_offsets_with_and_without_batch_norm():
+    B = 4
+    # one pooled and one unpooled 3x3 layer on 8x8, 2 -> 3 -> 5 channels
+    for bn in (False, True):
+        m = build_custom(B, 8, 8, 2, [dict(cout=3, k=3, pad=1, pool=(MAX_POOL, 2, 2, 0), bn=bn),
+                                      dict(cout=5, k=3, pad=1, pool=None, bn=bn)], [(7, 10)])
+        c0, c1 = m.convLayer[0], m.convLayer[1]
+        V0, P0, V1 = 8 * 8 * 3 * B, 4 * 4 * 3 * B, 4 * 4 * 5 * B
+        if not bn:
+            assert (c0.activationOffset, c0.poolOffset, c0.outputOffset) == (V0, 2 * V0, 2 * V0)
+            assert c0.batchNormOffset == INT_MAX and c0.meansOffset == INT_MAX
+            assert (c1.activationOffset, c1.poolOffset, c1.outputOffset) == (V1, INT_MAX, V1)
+            slab0, slab1 = 2 * V0 + P0, 2 * V1
+        else:
+            assert c0.batchNormOffset == V0 and c0.meansOffset == V0 and c0.variancesOffset == V0 + 3
+            assert c0.runningMeansOffset == V0 + 6 and c0.runningVariancesOffset == V0 + 9
+            assert c0.activationOffset == 2 * V0 + 12 and c0.poolOffset == 3 * V0 + 12
+            assert c1.activationOffset == 2 * V1 + 20 and c1.outputOffset == c1.activationOffset
+            slab0, slab1 = 3 * V0 + 12 + P0, 3 * V1 + 20
+        assert [m.zOffsets[i] for i in range(5)] == [0, 0, slab0, slab0 + slab1, slab0 + slab1 + 2 * 7 * B]
+        assert m.zSize == slab0 + slab1 + 2 * 7 * B
+        assert m.maxDeltaSize == max(slab0, slab1)
+        assert m.fcLayer[0].in_ == 5 * 4 * 4 and m.fcLayer[0].offset == 7 * B
+
+
+def test_readVGG11_is_the_swish_network():
+    m = CNN_MODEL()
+    L.cnn.readVGG11(C.byref(m), 8, 32, 32, 10, 3, 0, 0, 10)
+    assert m.cLayers == 8 and m.lLayers == 1 and all(m.actFuns[i] == CNN_ACT_SWISH for i in range(8))
+    assert [m.poolLayer[i].type for i in range(8)] == [MAX_POOL, MAX_POOL, NO_POOL, MAX_POOL, NO_POOL, MAX_POOL, NO_POOL, MAX_POOL]
+    assert m.fcLayer[0].in_ == 512
+
+
+def test_get_dimensions():
+    h, w = C.c_int(), C.c_int()
+    L.cnn.getDimensions(224, 224, 2, 4, 11, C.byref(h), C.byref(w))
+    assert (h.value, w.value) == (55, 55)
+    L.cnn.getDimensions(27, 13, 0, 2, 3, C.byref(h), C.byref(w))
+    assert (h.value, w.value) == (13, 6)
+
+
+def _declared(header, pattern):
+    text = open(os.path.join(ROOT, "include", header)).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(pattern, text)))
+
+
+def test_libraries_export_every_declared_symbol():
+    hip_names = _declared("fitre_hip.h", r"\b(fitre_hip_\w+)\s*\(")
+    assert len(hip_names) > 50
+    for n in hip_names:
+        assert hasattr(L.hip, n), n
+        assert n in L.HIP_API, "ctypes table lacks %s" % n
+    cnn_names = _declared("fitre_cnn.h", r"\b([A-Za-z_]\w*)\s*\(") + _declared("fitre_shim.h", r"\b([A-Za-z_]\w*)\s*\(")
+    cnn_names = [n for n in cnn_names if n not in ("defined",)]
+    assert "cnnBackward" in cnn_names and "computeCNNGradient" in cnn_names and "copy_host_device" in cnn_names
+    for n in cnn_names:
+        assert hasattr(L.cnn, n), n
+    for g in ("BLOCK_SIZE", "WARP_SIZE", "DEVICE_NUM_BLOCKS"):
+        assert C.c_int.in_dll(L.cnn, g) is not None
+
+
+def test_struct_sizes_match_the_c_side():
+    # a C-side check would need a compiler run; the builders fill every field through C, so a
+    # mismatch in field order shows as garbage here
+    m = build_vgg11(2)
+    assert m.batchSize == 2 and m.bias == 1 and m.cLayers == 8
+    assert m.convLayer[7].outChannels == 512 and m.poolLayer[7].outHeight == 1
+    assert C.sizeof(CNN_MODEL) == 20 * 22 * 4 + 20 * 4 + 20 * 8 * 4 + 8 + 20 * 5 * 4 + 7 * 4 + 3 * 80 + 4 + 2 * 80
+
+
+def test_workspace_requirements_are_positive_and_modest():
+    m = build_vgg11(256)
+    fwd, bwd = L.cnn.cnnForwardMemRequired(C.byref(m)), L.cnn.cnnBackwardMemRequired(C.byref(m))
+    assert 0 < fwd * 4 < 512e6 and 0 < bwd * 4 < 512e6
