@@ -1,0 +1,220 @@
+#!/usr/bin/env python3
+"""Benchmark of the CNN backward pass on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu]
+
+Workload: VGG-11-style network, fp32, batch 256, 3x32x32 N(0,1) inputs, 10 uniform classes, eight
+3x3/pad-1 convolutions (64,128,256,256,512,512,512,512) each with non-affine batch norm and ReLU,
+max-pool 2 after convolutions 1,2,4,6,8, FC 512->10, softmax cross entropy; He-normal weights.
+A step is one cnnBackward call through the C boundary (copy of the loss errors into the delta
+buffer included), device-complete on return; the forward pass runs once, untimed, to produce z.
+Inputs, weights and z are resident in HBM before the timed region starts.
+
+Prints ONE JSON line: backward images/sec, plus
+  roofline      the dominant kernel (largest summed time): algorithmic FLOPs / its average launch
+                duration, measured with HIP events on the library's stream in a second pass of the
+                same K steps (the first, timed pass runs without per-launch events), against the
+                157.3 TFLOP/s fp32-MFMA peak;
+  kernels       the same accounting for every kernel class of the backward pass;
+  cpu_baseline  the C restatement of the reference's algorithm (float32, OpenMP) timed on the host
+                cores on a bounded sample (same network, smaller batch);
+  torch_cpu     torch autograd of the same network on the host cores (float32), for orientation.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+PEAK_MFMA_F32_TFLOPS = 157.3
+PEAK_HBM_GBS = 8000.0
+
+KC = dict(conv_dw=0, conv_dx=1, conv_fwd=2, fc_gemm=3, splitk_reduce=4, bn_bwd=5, bn_fwd=6, pool_bwd=7, pool_fwd=8,
+          act_bwd=9, act_fwd=10, bias_grad=11, softmax=12, permute=13, blas1=14, pool_act_bwd=15, kfac_factor=16)
+MFMA_CLASSES = ("conv_dw", "conv_dx", "conv_fwd", "fc_gemm", "kfac_factor")
+TILES = {0: "", 1: "64x64", 2: "64x128", 3: "128x64", 4: "128x128"}
+
+
+def read_profile(L):
+    rows = []
+    for name, cls in KC.items():
+        for tile in range(5):
+            n, ms, work = C.c_long(), C.c_double(), C.c_double()
+            L.check(L.hip.fitre_hip_profile_read_tile(cls, tile, C.byref(n), C.byref(ms), C.byref(work)))
+            if n.value:
+                rows.append(dict(kernel=name + ("/" + TILES[tile] if tile else ""), cls=name, launches=n.value,
+                                 ms=ms.value, work=work.value))
+    return rows
+
+
+def gpu_leg(args):
+    from fitre_amd import lib as L
+    from helpers import Device, GpuModel, at, batch_inputs, build_vgg11, he_weights
+
+    batch = 256
+    dev = Device(0)
+    name = C.create_string_buffer(128)
+    cus = C.c_int()
+    L.check(L.hip.fitre_hip_device_info(C.byref(cus), None, None, None, None, name, 128))
+    model = build_vgg11(batch, bn=True)
+    rng = np.random.default_rng(0xF17E0003)
+    w = he_weights(model, rng).astype(np.float32)
+    x, y = batch_inputs(model, batch, rng)
+    gm = GpuModel(dev, model, w, x.astype(np.float32), y, batch)
+    loss = gm.forward()  # untimed: produces z, probs and the loss errors
+
+    def run(steps):
+        for _ in range(steps):
+            gm.backward()  # copies errors -> delta, calls cnnBackward; device-complete on return
+
+    run(args.warmup)
+    dev.sync()
+    ev0, ev1 = C.c_void_p(), C.c_void_p()
+    L.check(L.hip.fitre_hip_event_create(C.byref(ev0)))
+    L.check(L.hip.fitre_hip_event_create(C.byref(ev1)))
+    dev.sync()
+    L.check(L.hip.fitre_hip_event_record(ev0))
+    t0 = time.perf_counter()
+    run(args.steps)
+    dev.sync()
+    t1 = time.perf_counter()
+    L.check(L.hip.fitre_hip_event_record(ev1))
+    ms_events = C.c_float()
+    L.check(L.hip.fitre_hip_event_elapsed_ms(ev0, ev1, C.byref(ms_events)))
+    wall = t1 - t0
+
+    # second pass of the same steps with per-launch events
+    L.check(L.hip.fitre_hip_profile_enable(1))
+    run(args.steps)
+    dev.sync()
+    L.check(L.hip.fitre_hip_profile_enable(0))
+    rows = read_profile(L)
+    grad = gm.get("grad")
+    finite = bool(np.isfinite(grad).all() and np.isfinite(loss))
+    gm.release()
+    dev.close()
+
+    kernels = {}
+    for r in rows:
+        avg_us = 1e3 * r["ms"] / r["launches"]
+        per_step = r["launches"] / args.steps
+        if r["cls"] in MFMA_CLASSES:
+            rate = r["work"] / (r["ms"] * 1e-3) / 1e12 if r["ms"] > 0 else 0.0
+            kernels[r["kernel"]] = dict(bound="mfma", launches_per_step=per_step, avg_us=round(avg_us, 2),
+                                        ms_per_step=round(r["ms"] / args.steps, 4), achieved=round(rate, 2),
+                                        unit="TFLOP/s", frac=round(rate / PEAK_MFMA_F32_TFLOPS, 4))
+        else:
+            rate = r["work"] / (r["ms"] * 1e-3) / 1e9 if r["ms"] > 0 else 0.0
+            kernels[r["kernel"]] = dict(bound="hbm", launches_per_step=per_step, avg_us=round(avg_us, 2),
+                                        ms_per_step=round(r["ms"] / args.steps, 4), achieved=round(rate, 1),
+                                        unit="GB/s", frac=round(rate / PEAK_HBM_GBS, 4))
+    dom = max(rows, key=lambda r: r["ms"])
+    dk = kernels[dom["kernel"]]
+    roofline = dict(kernel=dom["kernel"], bound=dk["bound"], achieved=dk["achieved"],
+                    peak=PEAK_MFMA_F32_TFLOPS if dk["bound"] == "mfma" else PEAK_HBM_GBS, unit=dk["unit"],
+                    frac=dk["frac"], traffic=None, avg_launch_us=dk["avg_us"],
+                    launches_per_step=dk["launches_per_step"])
+    conv_rows = [r for r in rows if r["cls"] in ("conv_dw", "conv_dx")]
+    conv_ms, conv_work = sum(r["ms"] for r in conv_rows), sum(r["work"] for r in conv_rows)
+    conv = dict(ms_per_step=round(conv_ms / args.steps, 4), gflop_per_step=round(conv_work / args.steps / 1e9, 2),
+                achieved=round(conv_work / (conv_ms * 1e-3) / 1e12, 2) if conv_ms else 0.0, unit="TFLOP/s")
+    conv["frac"] = round(conv["achieved"] / PEAK_MFMA_F32_TFLOPS, 4)
+    return dict(wall=wall, ms_events=ms_events.value, batch=batch, loss=loss, finite=finite,
+                device=name.value.decode(), compute_units=cus.value, roofline=roofline, kernels=kernels,
+                conv_backward_gemms=conv)
+
+
+def cpu_leg(batch=64, repeats=10):
+    """float32 build of the oracle (the reference's algorithm restated in C, OpenMP over the host
+    cores): one forward, then `repeats` backward passes on the same network at a smaller batch."""
+    from helpers import batch_inputs, build_vgg11, he_weights
+    from oracle.oracle import Oracle
+
+    o = Oracle(double=False)
+    model = build_vgg11(batch, bn=True)
+    rng = np.random.default_rng(1)
+    w = he_weights(model, rng).astype(np.float32)
+    x, y = batch_inputs(model, batch, rng)
+    _, z, _, errors = o.forward(model, w, x, y, 10, batch)
+    o.backward(model, w, x, z, errors, batch)  # warm-up
+    t0 = time.perf_counter()
+    for _ in range(repeats):
+        o.backward(model, w, x, z, errors, batch)
+    dt = time.perf_counter() - t0
+    cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    return dict(value=round(batch * repeats / dt, 2), unit="images/s", cores=cores, kind="port",
+                sample="VGG-11 backward, float32, batch %d x %d passes, C restatement with OpenMP" % (batch, repeats))
+
+
+def torch_leg(batch=32, repeats=3):
+    import torch
+    import torchref
+    from helpers import batch_inputs, build_vgg11, he_weights
+
+    model = build_vgg11(batch, bn=True)
+    rng = np.random.default_rng(1)
+    w = he_weights(model, rng)
+    x, y = batch_inputs(model, batch, rng)
+    torchref.run(model, w, x, y, batch, dtype=torch.float32, want_intermediates=False)
+    t0 = time.perf_counter()
+    for _ in range(repeats):
+        torchref.run(model, w, x, y, batch, dtype=torch.float32, want_intermediates=False)
+    dt = time.perf_counter() - t0
+    return dict(value=round(batch * repeats / dt, 2), unit="images/s (forward+backward)", threads=torch.get_num_threads(),
+                sample="torch %s autograd, float32, batch %d x %d" % (torch.__version__, batch, repeats))
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU (the reference path is single-device and every "
+                 "box here has one GPU); --gpus %d is not supported" % args.gpus)
+
+    g = gpu_leg(args)
+    seconds = g["ms_events"] * 1e-3
+    value = g["batch"] * args.steps / seconds
+    line = {
+        "metric": "backward images/sec, VGG-11 fp32 b=256 on 1 MI355X",
+        "value": round(value, 1),
+        "unit": "images/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(1e3 * seconds / args.steps, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "VGG-11-style CNN backward (cnnBackward), fp32, batch 256, 3x32x32, BN+ReLU, 10 classes",
+                   "batch": g["batch"], "device": g["device"], "compute_units": g["compute_units"]},
+        "roofline": g["roofline"],
+        "conv_backward_gemms": g["conv_backward_gemms"],
+        "kernels": g["kernels"],
+        "wall_ms_per_step": round(1e3 * g["wall"] / args.steps, 4),
+        "loss": round(g["loss"], 6),
+        "finite": g["finite"],
+    }
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_leg()
+        try:
+            line["torch_cpu"] = torch_leg()
+        except Exception as exc:  # torch is optional on the box
+            line["torch_cpu"] = {"error": str(exc)}
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -39,7 +39,7 @@ bool ready();
 // A LaunchScope brackets the launches made while it is alive with two events
 // when accounting is on; otherwise it costs one branch.
 struct LaunchScope {
-	LaunchScope(int kernelClass, double work);
+	LaunchScope(int kernelClass, double work, int tile = 0);
 	~LaunchScope();
 	int slot;
 };

@@ -79,8 +79,7 @@ int fitre_hip_conv_forward(const fitre_conv_shape *s, const float *x, const floa
 	PlainParams pa{ w, (long)R, I };
 	PatchGeom pb = make_patch_geom(x, s->inChannels, s->samples, s->inA, s->inB, s->outA, s->outB, s->ksize, s->stride, s->padding);
 	OutParams out{ y, (long)J, 0, bias, nullptr, 1.f, 0.f };
-	LaunchScope scope(FITRE_KC_CONV_FWD, conv_flops(s));
-	return launch_gemm<PlainKContig, PatchRowContig>(pa, pb, out, I, J, R, plan, ws, wsBytes);
+	return launch_gemm<PlainKContig, PatchRowContig>(pa, pb, out, I, J, R, plan, ws, wsBytes, FITRE_KC_CONV_FWD, conv_flops(s));
 }
 
 // ---- weight gradient: I = Cout, J = Cin*k*k, R = positions -------------------
@@ -101,8 +100,7 @@ int fitre_hip_conv_weight_grad(const fitre_conv_shape *s, const float *x, const 
 	PlainParams pa{ delta, (long)R, I };
 	PatchGeom pb = make_patch_geom(x, s->inChannels, s->samples, s->inA, s->inB, s->outA, s->outB, s->ksize, s->stride, s->padding);
 	OutParams out{ dW, (long)J, 0, nullptr, nullptr, 1.f, 0.f };
-	LaunchScope scope(FITRE_KC_CONV_DW, conv_flops(s));
-	return launch_gemm<PlainKContig, PatchKContig>(pa, pb, out, I, J, R, plan, ws, wsBytes);
+	return launch_gemm<PlainKContig, PatchKContig>(pa, pb, out, I, J, R, plan, ws, wsBytes, FITRE_KC_CONV_DW, conv_flops(s));
 }
 
 // ---- input gradient: I = Cin, J = input positions, R = Cout*k*k ----------------
@@ -133,8 +131,7 @@ int fitre_hip_conv_input_grad(const fitre_conv_shape *s, const float *delta, con
 	PatchGeom pb = make_patch_geom(delta, s->outChannels, s->samples, s->outA, s->outB, s->inA, s->inB, s->ksize, 1,
 	                               s->ksize - 1 - s->padding);
 	OutParams out{ dx, (long)J, 0, nullptr, nullptr, 1.f, 0.f };
-	LaunchScope scope(FITRE_KC_CONV_DX, conv_flops(s));
-	return launch_gemm<FlipWeightKContig, PatchRowContig>(pa, pb, out, I, J, R, plan, ws, wsBytes);
+	return launch_gemm<FlipWeightKContig, PatchRowContig>(pa, pb, out, I, J, R, plan, ws, wsBytes, FITRE_KC_CONV_DX, conv_flops(s));
 }
 
 // ---- general column-major GEMM ---------------------------------------------------
@@ -157,17 +154,17 @@ int fitre_hip_gemm(int transA, int transB, int M, int N, int K, float alpha, con
 	const int I = N, J = M, R = K;
 	GemmPlan plan = plan_gemm(I, J, R);
 	OutParams out{ C, (long)ldc, 0, nullptr, bias, alpha, beta };
-	LaunchScope scope(FITRE_KC_FC_GEMM, 2.0 * (double)M * N * K);
+	const double flops = 2.0 * (double)M * N * K;
 	// engine A(i = n, k): op(B)(k, n).  transB == 0: B[n*ldb + k] (contiguous along k); else B[k*ldb + n]
 	// engine B(j = m, k): op(A)(m, k).  transA == 0: A[k*lda + m] (contiguous along m); else A[m*lda + k]
 	PlainParams bk{ B, (long)ldb, I };
 	PlainParams br{ B, (long)ldb, I };
 	PlainParams ar{ A, (long)lda, J };
 	PlainParams ak{ A, (long)lda, J };
-	if (!transB && !transA) return launch_gemm<PlainKContig, PlainRowContig>(bk, ar, out, I, J, R, plan, ws, wsBytes);
-	if (!transB && transA) return launch_gemm<PlainKContig, PlainKContig>(bk, ak, out, I, J, R, plan, ws, wsBytes);
-	if (transB && !transA) return launch_gemm<PlainRowContig, PlainRowContig>(br, ar, out, I, J, R, plan, ws, wsBytes);
-	return launch_gemm<PlainRowContig, PlainKContig>(br, ak, out, I, J, R, plan, ws, wsBytes);
+	if (!transB && !transA) return launch_gemm<PlainKContig, PlainRowContig>(bk, ar, out, I, J, R, plan, ws, wsBytes, FITRE_KC_FC_GEMM, flops);
+	if (!transB && transA) return launch_gemm<PlainKContig, PlainKContig>(bk, ak, out, I, J, R, plan, ws, wsBytes, FITRE_KC_FC_GEMM, flops);
+	if (transB && !transA) return launch_gemm<PlainRowContig, PlainRowContig>(br, ar, out, I, J, R, plan, ws, wsBytes, FITRE_KC_FC_GEMM, flops);
+	return launch_gemm<PlainRowContig, PlainKContig>(br, ak, out, I, J, R, plan, ws, wsBytes, FITRE_KC_FC_GEMM, flops);
 }
 
 } // extern "C"

@@ -446,9 +446,10 @@ inline GemmPlan fit_plan(GemmPlan p, long I, long J, long R, const void *ws, siz
 
 template <template <int, int, int> class OpA, template <int, int, int> class OpB, int BM, int BN>
 static int launch_tile(const typename OpA<BM, kGemmBK, BM + 1>::Params &pa, const typename OpB<BN, kGemmBK, BN + 1>::Params &pb,
-                       const OutParams &out, int I, int J, int R, const GemmPlan &plan, void *ws)
+                       const OutParams &out, int I, int J, int R, const GemmPlan &plan, void *ws, int kernelClass, double flops)
 {
 	typedef TileCfg<BM, BN, kGemmBK> Cfg;
+	constexpr int tileId = (BM == 64 ? (BN == 64 ? 1 : 2) : (BN == 64 ? 3 : 4));
 	typedef OpA<BM, kGemmBK, Cfg::LDA> A;
 	typedef OpB<BN, kGemmBK, Cfg::LDB> B;
 	dim3 grid((J + BN - 1) / BN, (I + BM - 1) / BM, plan.splits);
@@ -458,13 +459,18 @@ static int launch_tile(const typename OpA<BM, kGemmBK, BM + 1>::Params &pa, cons
 		part.C = (float *)ws;
 		part.ldc = J;
 		part.splitStride = (long)I * J;
-		mfma_gemm_kernel<Cfg, A, B><<<grid, kGemmThreads, 0, stream()>>>(pa, pb, part, I, J, R, plan.kChunk);
+		{
+			LaunchScope scope(kernelClass, flops, tileId);
+			mfma_gemm_kernel<Cfg, A, B><<<grid, kGemmThreads, 0, stream()>>>(pa, pb, part, I, J, R, plan.kChunk);
+		}
 		OutParams fin = out;
 		fin.splitStride = 0;
+		LaunchScope scope(FITRE_KC_SPLITK_REDUCE, 4.0 * (double)I * J * (plan.splits + 1));
 		splitk_reduce_kernel<<<blocks_for((long)I * J, 256, 4096), 256, 0, stream()>>>((const float *)ws, plan.splits, I, J, fin);
 	} else {
 		OutParams direct = out;
 		direct.splitStride = 0;
+		LaunchScope scope(kernelClass, flops, tileId);
 		mfma_gemm_kernel<Cfg, A, B><<<grid, kGemmThreads, 0, stream()>>>(pa, pb, direct, I, J, R, plan.kChunk);
 	}
 	return check_launch("mfma_gemm_kernel");
@@ -473,7 +479,7 @@ static int launch_tile(const typename OpA<BM, kGemmBK, BM + 1>::Params &pa, cons
 // Picks the tile instantiation the plan names.
 template <template <int, int, int> class OpA, template <int, int, int> class OpB, class PA, class PB>
 static int launch_gemm(const PA &pa, const PB &pb, const OutParams &out, int I, int J, int R, const GemmPlan &ideal, void *ws,
-                       size_t wsBytes)
+                       size_t wsBytes, int kernelClass, double flops)
 {
 	const GemmPlan plan = fit_plan(ideal, I, J, R, ws, wsBytes);
 	if (plan.wsBytes > 0) {
@@ -481,10 +487,10 @@ static int launch_gemm(const PA &pa, const PB &pb, const OutParams &out, int I, 
 		if (wsBytes < plan.wsBytes)
 			return fail(FITRE_E_WORKSPACE, "split-K workspace of %zu bytes is smaller than the %zu required", wsBytes, plan.wsBytes);
 	}
-	if (plan.bm == 128 && plan.bn == 128) return launch_tile<OpA, OpB, 128, 128>(pa, pb, out, I, J, R, plan, ws);
-	if (plan.bm == 64 && plan.bn == 128) return launch_tile<OpA, OpB, 64, 128>(pa, pb, out, I, J, R, plan, ws);
-	if (plan.bm == 128 && plan.bn == 64) return launch_tile<OpA, OpB, 128, 64>(pa, pb, out, I, J, R, plan, ws);
-	return launch_tile<OpA, OpB, 64, 64>(pa, pb, out, I, J, R, plan, ws);
+	if (plan.bm == 128 && plan.bn == 128) return launch_tile<OpA, OpB, 128, 128>(pa, pb, out, I, J, R, plan, ws, kernelClass, flops);
+	if (plan.bm == 64 && plan.bn == 128) return launch_tile<OpA, OpB, 64, 128>(pa, pb, out, I, J, R, plan, ws, kernelClass, flops);
+	if (plan.bm == 128 && plan.bn == 64) return launch_tile<OpA, OpB, 128, 64>(pa, pb, out, I, J, R, plan, ws, kernelClass, flops);
+	return launch_tile<OpA, OpB, 64, 64>(pa, pb, out, I, J, R, plan, ws, kernelClass, flops);
 }
 
 } // namespace fitre

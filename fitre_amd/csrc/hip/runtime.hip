@@ -20,10 +20,10 @@ struct ClassTotals {
 	double work;
 };
 static bool g_profile = false;
-static ClassTotals g_totals[FITRE_KC_COUNT];
+static ClassTotals g_totals[FITRE_KC_COUNT][FITRE_TILE_VARIANTS];
 struct Pending {
 	hipEvent_t start, stop;
-	int cls;
+	int cls, tile;
 };
 static std::vector<Pending> g_pending;
 static std::vector<hipEvent_t> g_event_pool;
@@ -72,23 +72,24 @@ static void drain_pending()
 	for (Pending &p : g_pending) {
 		float ms = 0.f;
 		if (hipEventSynchronize(p.stop) == hipSuccess && hipEventElapsedTime(&ms, p.start, p.stop) == hipSuccess)
-			g_totals[p.cls].ms += ms;
+			g_totals[p.cls][p.tile].ms += ms;
 		g_event_pool.push_back(p.start);
 		g_event_pool.push_back(p.stop);
 	}
 	g_pending.clear();
 }
 
-LaunchScope::LaunchScope(int kernelClass, double work) : slot(-1)
+LaunchScope::LaunchScope(int kernelClass, double work, int tile) : slot(-1)
 {
-	if (!g_profile || kernelClass < 0 || kernelClass >= FITRE_KC_COUNT) return;
+	if (!g_profile || kernelClass < 0 || kernelClass >= FITRE_KC_COUNT || tile < 0 || tile >= FITRE_TILE_VARIANTS) return;
 	Pending p;
 	p.start = take_event();
 	p.stop = take_event();
 	p.cls = kernelClass;
+	p.tile = tile;
 	if (!p.start || !p.stop) return;
-	g_totals[kernelClass].launches += 1;
-	g_totals[kernelClass].work += work;
+	g_totals[kernelClass][tile].launches += 1;
+	g_totals[kernelClass][tile].work += work;
 	(void)hipEventRecord(p.start, g_stream);
 	g_pending.push_back(p);
 	slot = (int)g_pending.size() - 1;
@@ -317,9 +318,29 @@ int fitre_hip_profile_read(int kernelClass, long *launches, double *milliseconds
 	FITRE_REQUIRE(kernelClass >= 0 && kernelClass < FITRE_KC_COUNT, "fitre_hip_profile_read: class %d unknown", kernelClass);
 	FITRE_HIP_TRY(hipStreamSynchronize(g_stream));
 	drain_pending();
-	if (launches) *launches = g_totals[kernelClass].launches;
-	if (milliseconds) *milliseconds = g_totals[kernelClass].ms;
-	if (work) *work = g_totals[kernelClass].work;
+	long n = 0;
+	double ms = 0.0, wk = 0.0;
+	for (int t = 0; t < FITRE_TILE_VARIANTS; t++) {
+		n += g_totals[kernelClass][t].launches;
+		ms += g_totals[kernelClass][t].ms;
+		wk += g_totals[kernelClass][t].work;
+	}
+	if (launches) *launches = n;
+	if (milliseconds) *milliseconds = ms;
+	if (work) *work = wk;
+	return FITRE_OK;
+}
+
+int fitre_hip_profile_read_tile(int kernelClass, int tile, long *launches, double *milliseconds, double *work)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(kernelClass >= 0 && kernelClass < FITRE_KC_COUNT && tile >= 0 && tile < FITRE_TILE_VARIANTS,
+	              "fitre_hip_profile_read_tile: class %d / tile %d unknown", kernelClass, tile);
+	FITRE_HIP_TRY(hipStreamSynchronize(g_stream));
+	drain_pending();
+	if (launches) *launches = g_totals[kernelClass][tile].launches;
+	if (milliseconds) *milliseconds = g_totals[kernelClass][tile].ms;
+	if (work) *work = g_totals[kernelClass][tile].work;
 	return FITRE_OK;
 }
 

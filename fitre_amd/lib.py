@@ -39,6 +39,7 @@ HIP_API = {
     "fitre_hip_event_elapsed_ms": (i32, [vp, vp, pf32]),
     "fitre_hip_profile_enable": (i32, [i32]),
     "fitre_hip_profile_read": (i32, [i32, C.POINTER(lng), C.POINTER(C.c_double), C.POINTER(C.c_double)]),
+    "fitre_hip_profile_read_tile": (i32, [i32, i32, C.POINTER(lng), C.POINTER(C.c_double), C.POINTER(C.c_double)]),
     "fitre_hip_axpy": (i32, [i32, f32, vp, vp]),
     "fitre_hip_scal": (i32, [i32, f32, vp]),
     "fitre_hip_copy": (i32, [i32, vp, vp]),

@@ -87,6 +87,10 @@ enum fitre_kernel_class {
 int fitre_hip_profile_enable(int on); /* on=1 clears the counters and starts; on=0 stops */
 /* launches, summed milliseconds and summed algorithmic work of one class (syncs first) */
 int fitre_hip_profile_read(int kernelClass, long *launches, double *milliseconds, double *work);
+/* The MFMA classes run one of several tile instantiations of the same kernel template; tile selects
+ * one: 0 = not tiled, 1 = 64x64, 2 = 64x128, 3 = 128x64, 4 = 128x128 (channel rows x contiguous columns). */
+#define FITRE_TILE_VARIANTS 5
+int fitre_hip_profile_read_tile(int kernelClass, int tile, long *launches, double *milliseconds, double *work);
 
 /* ---------------- level-1 helpers (the cublasD* calls of the solvers and of
  * functions/cnn_gradient.cu:54-56, functions/softmax_loss.cu:243) ---------------- */

@@ -1,0 +1,153 @@
+"""fp32-MFMA contractions against the float64 oracle: convolution forward, weight gradient, input
+gradient and the column-major GEMM, over tile-edge, split-K and layout edge cases."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from fitre_amd import lib as L
+from helpers import conv_shape, rel_err
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-4
+hip = L.hip
+
+# N, Cin, Cout, A(width), B(height), k, stride, pad
+CONV_CASES = [
+    (2, 3, 6, 32, 32, 5, 1, 0),      # LeNet conv1
+    (2, 6, 16, 14, 14, 5, 1, 0),     # LeNet conv2
+    (4, 3, 64, 32, 32, 3, 1, 1),     # VGG conv1
+    (2, 64, 128, 16, 16, 3, 1, 1),   # VGG conv2
+    (4, 130, 70, 8, 8, 3, 1, 1),     # channel counts off the tile grid
+    (8, 256, 256, 4, 4, 3, 1, 1),    # deep reduction, small map
+    (16, 96, 200, 2, 2, 3, 1, 1),    # 2x2 maps (VGG conv8 shape class)
+    (2, 3, 8, 67, 67, 11, 4, 2),     # AlexNet conv1 (strided)
+    (2, 8, 12, 13, 13, 5, 1, 2),     # AlexNet conv2
+    (3, 5, 7, 9, 6, 3, 1, 1),        # rectangular
+    (1, 1, 1, 5, 5, 3, 1, 0),        # degenerate
+    (2, 4, 5, 7, 7, 1, 1, 0),        # 1x1 window
+    (2, 4, 6, 9, 9, 3, 2, 1),        # stride 2
+]
+
+
+def run_conv(dev, oracle64, case, which):
+    N, Cin, Cout, A, B, k, s, p = case
+    shape = conv_shape(N, Cin, Cout, A, B, k, s, p)
+    oA, oB = shape.outA, shape.outB
+    rng = np.random.default_rng(sum(case))
+    x = rng.standard_normal(Cin * N * A * B).astype(np.float32)
+    w = (rng.standard_normal(Cout * Cin * k * k) / np.sqrt(Cin * k * k)).astype(np.float32)
+    b = rng.standard_normal(Cout).astype(np.float32)
+    d = rng.standard_normal(Cout * N * oA * oB).astype(np.float32)
+    px, pw, pb, pd = dev.upload(x), dev.upload(w), dev.upload(b), dev.upload(d)
+    bufs = [px, pw, pb, pd]
+    if which == "fwd":
+        nb = hip.fitre_hip_conv_forward_workspace(C.byref(shape))
+        ws, out = dev.alloc(nb), dev.zeros(d.size)
+        L.check(hip.fitre_hip_conv_forward(C.byref(shape), px, pw, pb, out, ws, nb))
+        got, want = dev.download(out, d.size), oracle64.conv_forward(x, w, b, N, Cin, B, A, k, p, s, Cout)
+    elif which == "dw":
+        nb = hip.fitre_hip_conv_weight_grad_workspace(C.byref(shape))
+        ws, out = dev.alloc(nb), dev.zeros(w.size)
+        L.check(hip.fitre_hip_conv_weight_grad(C.byref(shape), px, pd, out, ws, nb))
+        got, want = dev.download(out, w.size), oracle64.conv_weight_grad(x, d, N, Cin, B, A, k, p, s, Cout)
+    else:
+        nb = hip.fitre_hip_conv_input_grad_workspace(C.byref(shape))
+        ws, out = dev.alloc(nb), dev.zeros(x.size)
+        L.check(hip.fitre_hip_conv_input_grad(C.byref(shape), pd, pw, out, ws, nb))
+        got, want = dev.download(out, x.size), oracle64.conv_input_grad(d, w, N, Cin, B, A, k, p, Cout)
+    for q in bufs + [ws, out]:
+        dev.free(q)
+    return got, want
+
+
+@pytest.mark.parametrize("case", CONV_CASES)
+def test_conv_forward(dev, oracle64, case):
+    got, want = run_conv(dev, oracle64, case, "fwd")
+    assert rel_err(got, want) < TOL
+
+
+@pytest.mark.parametrize("case", CONV_CASES)
+def test_conv_weight_gradient(dev, oracle64, case):
+    got, want = run_conv(dev, oracle64, case, "dw")
+    assert rel_err(got, want) < TOL
+
+
+@pytest.mark.parametrize("case", [c for c in CONV_CASES if c[6] == 1])
+def test_conv_input_gradient(dev, oracle64, case):
+    got, want = run_conv(dev, oracle64, case, "dx")
+    assert rel_err(got, want) < TOL
+
+
+def test_conv_input_gradient_refuses_stride(dev):
+    shape = conv_shape(2, 4, 6, 9, 9, 3, 2, 1)
+    p = dev.zeros(4096)
+    assert hip.fitre_hip_conv_input_grad(C.byref(shape), p, p, p, p, 4096) == 3
+    assert b"stride" in hip.fitre_hip_last_error()
+
+
+def test_conv_shape_is_validated(dev):
+    shape = conv_shape(2, 4, 6, 9, 9, 3, 1, 1)
+    shape.outA = 5
+    p = dev.zeros(4096)
+    assert hip.fitre_hip_conv_forward(C.byref(shape), p, p, None, p, p, 4096) == 2
+
+
+def test_split_k_is_deterministic_and_workspace_independent(dev, oracle64):
+    # long reduction, one output tile: planned with many splits; a tiny workspace forces fewer
+    case = (32, 3, 16, 32, 32, 3, 1, 1)
+    N, Cin, Cout, A, B, k, s, p = case
+    shape = conv_shape(*case)
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal(Cin * N * A * B).astype(np.float32)
+    d = rng.standard_normal(Cout * N * A * B).astype(np.float32)
+    px, pd = dev.upload(x), dev.upload(d)
+    nb = hip.fitre_hip_conv_weight_grad_workspace(C.byref(shape))
+    assert nb > 0
+    ws, out = dev.alloc(nb), dev.zeros(Cout * Cin * k * k)
+    res = []
+    for _ in range(3):
+        L.check(hip.fitre_hip_conv_weight_grad(C.byref(shape), px, pd, out, ws, nb))
+        res.append(dev.download(out, Cout * Cin * k * k))
+    np.testing.assert_array_equal(res[0], res[1])
+    np.testing.assert_array_equal(res[0], res[2])
+    want = oracle64.conv_weight_grad(x, d, N, Cin, B, A, k, p, s, Cout)
+    assert rel_err(res[0], want) < TOL
+    small = 3 * Cout * Cin * k * k * 4  # room for three partial tiles only
+    L.check(hip.fitre_hip_conv_weight_grad(C.byref(shape), px, pd, out, ws, small))
+    assert rel_err(dev.download(out, Cout * Cin * k * k), want) < TOL
+    L.check(hip.fitre_hip_conv_weight_grad(C.byref(shape), px, pd, out, None, 0))  # unsplit
+    assert rel_err(dev.download(out, Cout * Cin * k * k), want) < TOL
+
+
+GEMM_CASES = [  # M, N, K
+    (10, 256, 512), (512, 256, 10), (120, 7, 400), (84, 128, 120), (1, 1, 1), (129, 65, 33), (300, 200, 64), (64, 64, 4096),
+]
+
+
+@pytest.mark.parametrize("M,N,K", GEMM_CASES)
+@pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
+def test_gemm(dev, oracle64, M, N, K, ta, tb):
+    rng = np.random.default_rng(M + N + K)
+    lda = (K if ta else M) + 3
+    ldb = (N if tb else K) + 1
+    ldc = M + 2
+    A = rng.standard_normal(lda * (M if ta else K)).astype(np.float32)
+    Bm = rng.standard_normal(ldb * (K if tb else N)).astype(np.float32)
+    C0 = rng.standard_normal(ldc * N).astype(np.float32)
+    pa, pb, pc = dev.upload(A), dev.upload(Bm), dev.upload(C0)
+    nb = hip.fitre_hip_gemm_workspace(M, N, K)
+    ws = dev.alloc(nb)
+    L.check(hip.fitre_hip_gemm(ta, tb, M, N, K, 0.5, pa, lda, pb, ldb, 2.0, pc, ldc, None, ws, nb))
+    want = oracle64.gemm(ta, tb, M, N, K, 0.5, A, lda, Bm, ldb, 2.0, C0, ldc)
+    got = dev.download(pc, ldc * N)
+    assert rel_err(got, want) < TOL
+    # padding rows of C (ldc > M) are untouched
+    np.testing.assert_array_equal(got.reshape(N, ldc)[:, M:], C0.reshape(N, ldc)[:, M:])
+    # beta = 0 with a bias column added
+    bias = rng.standard_normal(M).astype(np.float32)
+    L.check(hip.fitre_hip_gemm(ta, tb, M, N, K, 1.0, pa, lda, pb, ldb, 0.0, pc, ldc, dev.upload(bias), ws, nb))
+    want = oracle64.gemm(ta, tb, M, N, K, 1.0, A, lda, Bm, ldb, 0.0, np.zeros(ldc * N), ldc).reshape(N, ldc)[:, :M] + bias[None, :]
+    assert rel_err(dev.download(pc, ldc * N).reshape(N, ldc)[:, :M], want) < TOL
+    for q in (pa, pb, pc, ws):
+        dev.free(q)

@@ -1,0 +1,219 @@
+"""cnnForward / cnnBackward / computeCNNGradient through the C boundary against the float64 oracle:
+loss, probabilities, every z and dx slot and the flat gradient; then size-independent properties at
+the full benchmark shapes."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from fitre_amd import lib as L
+from fitre_amd.structs import (CNN_ACT_NONE, CNN_ACT_RELU, CNN_ACT_SWISH, MAX_POOL, NO_POOL, PERFORM_NO_BATCH_NORM)
+from helpers import GpuModel, batch_inputs, build_alexnet, build_custom, build_lenet, build_vgg11, he_weights, num_classes, rel_err
+from test_oracle_model import MODELS, slot, smooth_models
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-4
+
+
+def compare_with_oracle(dev, oracle64, model, batch, seed, weight_decay=0.0, tol=TOL, end_to_end=False):
+    """Forward: every z slot, probabilities, errors and the loss against the float64 forward.
+    Backward: the flat gradient and every dx slot against the float64 cnnBackward restatement run on
+    the SAME inputs cnnBackward received (the z the GPU produced, and its loss errors) -- ReLU masks
+    and pooling selections are functions of z, so both sides then take identical decisions and the
+    comparison measures arithmetic only.  end_to_end additionally compares with the all-float64
+    pipeline (small models, where no pre-activation sits within rounding of a kink)."""
+    rng = np.random.default_rng(seed)
+    w = he_weights(model, rng, bias_scale=0.05)
+    x, y = batch_inputs(model, batch, rng)
+    w32, x32 = w.astype(np.float32), x.astype(np.float32)
+    classes = num_classes(model)
+    gm = GpuModel(dev, model, w32, x32, y, batch)
+    loss = gm.gradient(weight_decay)
+    z, dx, grad = gm.get("z"), gm.get("dx"), gm.get("grad")
+    probs, errors = gm.get("probs"), gm.get("errors")
+    gm.release()
+
+    # ---- forward
+    fl, fz, fprobs, ferrors = oracle64.forward(model, w32, x32, y, classes, batch)
+    assert abs(loss - fl) < 1e-5 * max(1.0, abs(fl))
+    assert rel_err(probs, fprobs) < tol and rel_err(errors, ferrors) < tol
+    for l in range(model.cLayers):
+        c, p = model.convLayer[l], model.poolLayer[l]
+        names = ["conv", "act"] + (["bn"] if c.batchNorm != PERFORM_NO_BATCH_NORM else []) + (["pool"] if p.type != NO_POOL else [])
+        for nme in names:
+            assert rel_err(slot(z, model, l, nme), slot(fz, model, l, nme)) < tol, "z %s of layer %d" % (nme, l)
+    for f in range(model.lLayers):
+        base = model.zOffsets[model.cLayers + f + 1]
+        cnt = model.fcLayer[f].out * batch
+        assert rel_err(z[base:base + 2 * cnt], fz[base:base + 2 * cnt]) < tol, "z of FC layer %d" % f
+
+    # ---- backward on identical inputs
+    rgrad, rdx = oracle64.backward(model, w32, x32, z.astype(np.float64), errors.astype(np.float64), batch)
+    rgrad = rgrad + weight_decay * w32.astype(np.float64)
+    assert rel_err(grad, rgrad) < tol, "flat gradient"
+    nl = model.cLayers + model.lLayers
+    for l in range(nl):  # per-layer blocks: a small layer must not hide behind a large one
+        a = model.wOffsets[l]
+        b = model.bOffsets[l] if model.bias else (model.wOffsets[l + 1] if l + 1 < nl else model.pSize)
+        assert rel_err(grad[a:b], rgrad[a:b]) < tol, "weight gradient of layer %d" % l
+        if model.bias:
+            e = model.wOffsets[l + 1] if l + 1 < nl else model.pSize
+            if l < model.cLayers and model.convLayer[l].batchNorm != PERFORM_NO_BATCH_NORM:
+                # behind batch norm the bias gradient is a sum that cancels to zero; what is left is rounding
+                cl = model.convLayer[l]
+                cancel = np.abs(slot(rdx, model, l, "bn")).reshape(cl.outChannels, -1).sum(1).max()
+                assert np.abs(grad[b:e] - rgrad[b:e]).max() < 1e-5 * cancel, "bias gradient of layer %d" % l
+            else:
+                assert rel_err(grad[b:e], rgrad[b:e]) < tol, "bias gradient of layer %d" % l
+    for l in range(model.cLayers):
+        c = model.convLayer[l]
+        for nme in ["conv", "act"] + (["bn"] if c.batchNorm != PERFORM_NO_BATCH_NORM else []):
+            assert rel_err(slot(dx, model, l, nme), slot(rdx, model, l, nme)) < tol, "dx %s of layer %d" % (nme, l)
+    for f in range(model.lLayers):
+        base = model.zOffsets[model.cLayers + f + 1]
+        cnt = model.fcLayer[f].out * batch
+        assert rel_err(dx[base:base + cnt], rdx[base:base + cnt]) < tol, "dx of FC layer %d" % f
+
+    if end_to_end:
+        ref = oracle64.gradient(model, w32, x32, y, classes, batch, weight_decay)
+        assert rel_err(grad, ref["gradient"]) < tol, "flat gradient, all-float64 pipeline"
+    return grad, rgrad
+
+
+@pytest.mark.parametrize("name,model,batch", MODELS, ids=[m[0] for m in MODELS])
+def test_small_models_every_slot(dev, oracle64, name, model, batch):
+    compare_with_oracle(dev, oracle64, model, batch, seed=sum(map(ord, name)), end_to_end=True)
+
+
+@pytest.mark.parametrize("idx", [0, 1, 2])
+def test_smooth_models(dev, oracle64, idx):
+    model, batch = list(smooth_models())[idx]
+    compare_with_oracle(dev, oracle64, model, batch, seed=idx, weight_decay=0.01, end_to_end=True)
+
+
+def test_lenet_batch128(dev, oracle64):
+    compare_with_oracle(dev, oracle64, build_lenet(128, bn=False), 128, seed=11)
+
+
+def test_lenet_bn_batch1024(dev, oracle64):
+    compare_with_oracle(dev, oracle64, build_lenet(1024, bn=True), 1024, seed=12)
+
+
+def test_vgg11_bn_reduced_batch(dev, oracle64):
+    # the benchmark network at its real layer shapes; batch trimmed so that the oracle takes seconds
+    compare_with_oracle(dev, oracle64, build_vgg11(16, bn=True), 16, seed=13)
+
+
+def test_vgg11_swish_reference_network(dev, oracle64):
+    compare_with_oracle(dev, oracle64, build_vgg11(8, bn=True, act=CNN_ACT_SWISH, bias=0), 8, seed=14)
+
+
+def test_alexnet_reduced(dev, oracle64):
+    # AlexNet layer types at a reduced image (67 -> 16 -> 7 -> 3 -> 1): 11x11/s4/p2, 5x5/p2, 3x3, maxpool 3/2
+    compare_with_oracle(dev, oracle64, build_alexnet(4, classes=50, size=67), 4, seed=15)
+
+
+def test_smaller_batch_than_model(dev, oracle64):
+    """The solvers call with curBatchSize <= model->batchSize (last mini-batch of an epoch)."""
+    model = build_custom(8, 8, 8, 3, [dict(cout=4, k=3, pad=1, pool=(MAX_POOL, 2, 2, 0), bn=True)], [(5, CNN_ACT_NONE)])
+    rng = np.random.default_rng(5)
+    w = he_weights(model, rng).astype(np.float32)
+    x, y = batch_inputs(model, 5, rng)
+    gm = GpuModel(dev, model, w, x.astype(np.float32), y, 5)
+    loss = gm.gradient()
+    ref_model = build_custom(8, 8, 8, 3, [dict(cout=4, k=3, pad=1, pool=(MAX_POOL, 2, 2, 0), bn=True)], [(5, CNN_ACT_NONE)])
+    ref = oracle64.gradient(ref_model, w, x.astype(np.float32), y, 5, 5)
+    assert abs(loss - ref["loss"]) < 1e-5
+    assert rel_err(gm.get("grad"), ref["gradient"]) < TOL
+    gm.release()
+
+
+def test_scratch_cursors_are_restored(dev):
+    model = build_lenet(4)
+    rng = np.random.default_rng(6)
+    x, y = batch_inputs(model, 4, rng)
+    gm = GpuModel(dev, model, he_weights(model, rng).astype(np.float32), x.astype(np.float32), y, 4)
+    before = (gm.scratch.nextDevPtr, gm.scratch.nextHostPtr, gm.scratch.nextPageLckPtr)
+    gm.gradient()
+    assert (gm.scratch.nextDevPtr, gm.scratch.nextHostPtr, gm.scratch.nextPageLckPtr) == before
+    gm.release()
+
+
+# ------------------------------------------------------------------ full benchmark shapes: properties
+@pytest.fixture(scope="module")
+def vgg_full(dev):
+    batch = 256
+    model = build_vgg11(batch, bn=True)
+    rng = np.random.default_rng(2024)
+    w = he_weights(model, rng).astype(np.float32)
+    x, y = batch_inputs(model, batch, rng)
+    gm = GpuModel(dev, model, w, x.astype(np.float32), y, batch)
+    yield gm, w
+    gm.release()
+
+
+def test_vgg11_full_size_properties(vgg_full, dev):
+    gm, w = vgg_full
+    model, batch = gm.model, gm.batch
+    loss = gm.forward()
+    assert np.isfinite(loss) and 1.0 < loss < 10.0
+    probs = gm.get("probs").reshape(batch, 10)
+    np.testing.assert_allclose(probs.sum(1), 1.0, atol=1e-5)
+    err = gm.get("errors").reshape(batch, 10)
+    np.testing.assert_allclose(err.sum(1), 0.0, atol=1e-7)
+    gm.backward()
+    g1 = gm.get("grad")
+    assert np.isfinite(g1).all() and np.abs(g1).max() > 0
+    # bitwise run-to-run determinism (no atomics anywhere on the path)
+    gm.backward()
+    np.testing.assert_array_equal(g1, gm.get("grad"))
+    # batch-norm backward invariants per channel: sum(dx) = 0 = the bias gradient, sum(dx * zhat) ~ 0
+    z, dx = gm.get("z"), gm.get("dx")
+    for l in (0, 3, 7):
+        c = model.convLayer[l]
+        per = batch * c.outHeight * c.outWidth
+        d = slot(dx, model, l, "bn").reshape(c.outChannels, per).astype(np.float64)
+        zh = slot(z, model, l, "bn").reshape(c.outChannels, per).astype(np.float64)
+        scale = np.abs(d).sum(1).max()
+        assert np.abs(d.sum(1)).max() < 1e-5 * scale
+        assert np.abs((d * zh).sum(1)).max() < 1e-3 * scale
+        b = g1[model.bOffsets[l]:model.bOffsets[l] + c.outChannels]
+        assert np.abs(b).max() < 1e-5 * scale
+    # FC bias gradient = column sums of the loss errors; FC weight gradient = errors x features
+    fcw = g1[model.wOffsets[8]:model.wOffsets[8] + 5120].reshape(512, 10).astype(np.float64)
+    feat = z[model.zOffsets[8] + model.convLayer[7].outputOffset:][:512 * batch].reshape(batch, 512).astype(np.float64)
+    want = feat.T @ err.astype(np.float64)
+    assert rel_err(fcw, want) < TOL
+    np.testing.assert_allclose(g1[model.bOffsets[8]:model.bOffsets[8] + 10], err.astype(np.float64).sum(0), atol=1e-6)
+
+
+def test_vgg11_full_size_backward_is_linear_in_delta(vgg_full, dev):
+    """cnnBackward is linear in the incoming errors: B(2*delta) = 2*B(delta) up to rounding,
+    and exactly so for a power-of-two factor."""
+    gm, w = vgg_full
+    gm.forward()
+    gm.backward()
+    g1 = gm.get("grad")
+    L.check(L.hip.fitre_hip_scal(10 * gm.batch, 2.0, gm.errors))
+    gm.backward()
+    g2 = gm.get("grad")
+    np.testing.assert_array_equal(g2, 2 * g1)
+
+
+def test_vgg11_full_size_directional_derivative(vgg_full, dev):
+    """g'd against a central difference of the loss along a random direction d (fp32 forward)."""
+    gm, w = vgg_full
+    gm.forward()
+    gm.backward()
+    g = gm.get("grad").astype(np.float64)
+    rng = np.random.default_rng(99)
+    d = rng.standard_normal(w.size)
+    d *= 1.0 / np.linalg.norm(d)
+    h = 2e-2
+    losses = []
+    for sgn in (+1, -1):
+        L.check(L.hip.fitre_hip_copy_h2d(gm.w, (w + np.float32(sgn * h) * d.astype(np.float32)).ctypes.data_as(C.c_void_p), 4 * w.size))
+        losses.append(gm.forward())
+    L.check(L.hip.fitre_hip_copy_h2d(gm.w, w.ctypes.data_as(C.c_void_p), 4 * w.size))
+    fd = (losses[0] - losses[1]) / (2 * h)
+    assert abs(fd - np.dot(g, d)) < 0.05 * abs(np.dot(g, d)) + 1e-3

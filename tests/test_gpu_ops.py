@@ -1,0 +1,328 @@
+"""Parity of every C-ABI kernel entry point with the float64 oracle on seeded inputs.
+Tolerance: max-abs error relative to the largest reference magnitude <= 1e-4 (fp32 arithmetic);
+pooling selections are bit-exact."""
+import ctypes as C
+import json
+import os
+
+import numpy as np
+import pytest
+
+from fitre_amd import lib as L
+from fitre_amd.structs import (ACT_LINEAR, ACT_LOGISTIC, ACT_TANH, AVG_POOL, CNN_ACT_ELU, CNN_ACT_NONE, CNN_ACT_RELU,
+                               CNN_ACT_SOFTPLUS, CNN_ACT_SWISH, MAX_POOL, NO_POOL)
+from helpers import at, conv_shape, rel_err
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-4
+HERE = os.path.dirname(os.path.abspath(__file__))
+hip = L.hip
+
+
+def ok(rc):
+    L.check(rc)
+
+
+# ------------------------------------------------------------------ level 1 and elementwise
+def test_level1(dev):
+    rng = np.random.default_rng(1)
+    for n in (1, 63, 1000, 262147):
+        x, y = rng.standard_normal(n).astype(np.float32), rng.standard_normal(n).astype(np.float32)
+        dx_, dy_ = dev.upload(x), dev.upload(y)
+        ok(hip.fitre_hip_axpy(n, 0.75, dx_, dy_))
+        np.testing.assert_allclose(dev.download(dy_, n), y + np.float32(0.75) * x, rtol=1e-6, atol=1e-6)
+        ok(hip.fitre_hip_scal(n, -2.0, dx_))
+        np.testing.assert_array_equal(dev.download(dx_, n), -2 * x)
+        out = C.c_float()
+        x2 = -2 * x.astype(np.float64)
+        y2 = dev.download(dy_, n).astype(np.float64)
+        ok(hip.fitre_hip_dot(n, dx_, dy_, C.byref(out)))
+        assert abs(out.value - np.dot(x2, y2)) <= 1e-5 * max(1, np.abs(x2 * y2).sum())
+        ok(hip.fitre_hip_nrm2(n, dx_, C.byref(out)))
+        assert abs(out.value - np.linalg.norm(x2)) <= 1e-6 * np.linalg.norm(x2)
+        ok(hip.fitre_hip_asum(n, dx_, C.byref(out)))
+        assert abs(out.value - np.abs(x2).sum()) <= 1e-6 * np.abs(x2).sum()
+        ok(hip.fitre_hip_norm_inf(n, dx_, C.byref(out)))
+        assert out.value == np.float32(np.abs(x2).max())
+        ok(hip.fitre_hip_sum(n, dx_, C.byref(out)))
+        assert abs(out.value - x2.sum()) <= 1e-6 * np.abs(x2).sum()
+        ok(hip.fitre_hip_copy(n, dx_, dy_))
+        np.testing.assert_array_equal(dev.download(dy_, n), -2 * x)
+        dev.free(dx_), dev.free(dy_)
+
+
+def test_elementwise_helpers(dev):
+    rng = np.random.default_rng(2)
+    n = 4099
+    a, b, c, d = (rng.standard_normal(n).astype(np.float32) for _ in range(4))
+    pos = np.abs(b) + np.float32(0.1)
+    da, db, dc, dd, dpos, out = (dev.upload(v) for v in (a, b, c, d, pos, np.zeros(n)))
+    ok(hip.fitre_hip_hadamard2(da, db, dc, dd, n, out))
+    np.testing.assert_allclose(dev.download(out, n), a * b + c * d, rtol=1e-6, atol=1e-6)
+    ok(hip.fitre_hip_elem_inv_scale(da, dpos, 1e-3, n, out))
+    np.testing.assert_allclose(dev.download(out, n), a / (np.sqrt(pos) + np.float32(1e-3)), rtol=1e-6)
+    ok(hip.fitre_hip_elem_sqr(da, n, out))
+    np.testing.assert_array_equal(dev.download(out, n), a * a)
+    ok(hip.fitre_hip_elem_sqr_decay(da, db, 0.8, n, out))
+    np.testing.assert_allclose(dev.download(out, n), np.float32(0.8) * a + np.float32(0.2) * b * b, rtol=1e-5, atol=1e-6)
+    ok(hip.fitre_hip_mat_mat_scale(da, db, n, out))
+    np.testing.assert_array_equal(dev.download(out, n), a * b)
+    ok(hip.fitre_hip_hadamard(da, db, n))
+    np.testing.assert_array_equal(dev.download(db, n), a * b)
+    ok(hip.fitre_hip_fill(out, n, 1.0))
+    assert (dev.download(out, n) == 1).all()
+    rows, cols = 7, 13
+    m = rng.standard_normal(rows * cols).astype(np.float32)
+    v = rng.standard_normal(cols).astype(np.float32)
+    dm, dv, o2 = dev.upload(m), dev.upload(v), dev.zeros(rows * cols)
+    ok(hip.fitre_hip_mat_row_vec_scale(dm, rows, cols, dv, o2))
+    np.testing.assert_array_equal(dev.download(o2, rows * cols), (m.reshape(cols, rows) * v[:, None]).reshape(-1))
+    vr = rng.standard_normal(rows).astype(np.float32)
+    dvr = dev.upload(vr)
+    ok(hip.fitre_hip_add_column(dm, rows, cols, dvr))
+    np.testing.assert_array_equal(dev.download(dm, rows * cols), (m.reshape(cols, rows) + vr[None, :]).reshape(-1))
+    x = rng.standard_normal(5 * 33).astype(np.float32)
+    bias = rng.standard_normal(5).astype(np.float32)
+    dxx, dbb = dev.upload(x), dev.upload(bias)
+    ok(hip.fitre_hip_add_channel_bias(dxx, 5, 33, dbb))
+    np.testing.assert_array_equal(dev.download(dxx, x.size), (x.reshape(5, 33) + bias[:, None]).reshape(-1))
+    dsum = dev.zeros(rows)
+    ok(hip.fitre_hip_row_sum(dev.upload(m), rows, cols, dsum))
+    np.testing.assert_allclose(dev.download(dsum, rows), m.reshape(cols, rows).astype(np.float64).sum(0), rtol=1e-6, atol=1e-6)
+
+
+def test_memset_and_copies(dev):
+    n = 1003
+    p = dev.upload(np.arange(n, dtype=np.float32))
+    ok(hip.fitre_hip_memset(at(p, 3), 0, 4 * 500))
+    got = dev.download(p, n)
+    want = np.arange(n, dtype=np.float32)
+    want[3:503] = 0
+    np.testing.assert_array_equal(got, want)
+    q = dev.zeros(n)
+    ok(hip.fitre_hip_copy_d2d(q, p, 4 * n))
+    np.testing.assert_array_equal(dev.download(q, n), want)
+
+
+ACTS = [CNN_ACT_RELU, CNN_ACT_SWISH, CNN_ACT_SOFTPLUS, CNN_ACT_ELU, ACT_LOGISTIC, ACT_TANH, CNN_ACT_NONE, ACT_LINEAR]
+
+
+@pytest.mark.parametrize("act", ACTS)
+@pytest.mark.parametrize("n,misalign", [(4096, 0), (1001, 1)])
+def test_activations(dev, oracle64, act, n, misalign):
+    rng = np.random.default_rng(act)
+    x = (rng.standard_normal(n) * 3).astype(np.float32)
+    x[:4] = [25.0, -25.0, 0.0, -0.0]
+    d = rng.standard_normal(n).astype(np.float32)
+    buf = dev.upload(np.concatenate([np.zeros(misalign, np.float32), x]))
+    px = at(buf, misalign)
+    out = dev.zeros(n + misalign)
+    po = at(out, misalign)
+    ok(hip.fitre_hip_activation_forward(act, px, po, n))
+    y = dev.download(po, n)
+    want = oracle64.activation_forward(act, x.astype(np.float64))
+    assert rel_err(y, want) < 1e-6
+    dd = dev.upload(np.concatenate([np.zeros(misalign, np.float32), d]))
+    res = dev.zeros(n + misalign)
+    ok(hip.fitre_hip_activation_backward(act, at(dd, misalign), px, po, at(res, misalign), n))
+    wantb = oracle64.activation_backward(act, d.astype(np.float64), x.astype(np.float64), want)
+    assert rel_err(dev.download(at(res, misalign), n), wantb) < 1e-5
+    for b in (buf, out, dd, res):
+        dev.free(b)
+
+
+def test_unknown_activation_code_is_an_error(dev):
+    p = dev.zeros(16)
+    assert hip.fitre_hip_activation_forward(99, p, p, 16) == 3
+    assert b"unknown activation" in hip.fitre_hip_last_error()
+    assert hip.fitre_hip_activation_backward(99, p, p, p, p, 16) == 3
+    assert hip.fitre_hip_activation_forward(CNN_ACT_RELU, None, p, 16) == 2
+
+
+# ------------------------------------------------------------------ pooling
+POOL_GEOMS = [  # C, N, A(width), B(height), k, s, p
+    (3, 2, 8, 8, 2, 2, 0),      # the 16-byte fast path
+    (2, 3, 6, 10, 2, 2, 0),     # 2x2 but B % 4 != 0
+    (2, 2, 7, 5, 3, 2, 1),      # the reference's 3/2/1
+    (3, 2, 13, 13, 3, 2, 0),    # AlexNet 3/2/0
+    (2, 2, 6, 6, 3, 1, 0),      # heavily overlapping
+    (8, 1, 2, 2, 3, 2, 1),      # drivers/pool_driver.cu
+    (2, 2, 5, 5, 2, 2, 0),      # odd extent: last row/column unpooled
+]
+
+
+@pytest.mark.parametrize("geom", POOL_GEOMS)
+@pytest.mark.parametrize("kind", [MAX_POOL, AVG_POOL])
+def test_pool_forward_backward(dev, oracle64, geom, kind):
+    Cn, N, A, B, k, s, p = geom
+    oA, oB = (A + 2 * p - k) // s + 1, (B + 2 * p - k) // s + 1
+    rng = np.random.default_rng(k * 100 + s * 10 + p)
+    x = rng.standard_normal(Cn * N * A * B).astype(np.float32)
+    d = rng.standard_normal(Cn * N * oA * oB).astype(np.float32)
+    px, pd = dev.upload(x), dev.upload(d)
+    out, back = dev.zeros(d.size), dev.upload(np.full(x.size, 7.0))
+    ok(hip.fitre_hip_pool_forward(kind, px, Cn, N, A, B, k, s, p, oA, oB, out))
+    want = oracle64.pool_forward(kind, x, N, Cn, B, A, k, s, p)
+    if kind == MAX_POOL:
+        np.testing.assert_array_equal(dev.download(out, d.size), want.astype(np.float32))
+        idx = dev.zeros(d.size, np.int32)
+        ok(hip.fitre_hip_max_pool_argmax(px, Cn, N, A, B, k, s, p, oA, oB, idx))
+        np.testing.assert_array_equal(dev.download(idx, d.size, np.int32), oracle64.max_pool_argmax(x, N, Cn, B, A, k, s, p))
+    else:
+        assert rel_err(dev.download(out, d.size), want) < 1e-6
+    ok(hip.fitre_hip_pool_backward(kind, pd, px, Cn, N, A, B, k, s, p, oA, oB, back))
+    wantb = oracle64.pool_backward(kind, d, x, N, Cn, B, A, k, s, p)
+    got = dev.download(back, x.size)
+    assert rel_err(got, wantb) < 1e-6
+    if kind == MAX_POOL:  # the routing itself is exact: same zero pattern
+        np.testing.assert_array_equal(got != 0, wantb != 0)
+
+
+def test_max_pool_ties_are_bit_exact(dev, oracle64):
+    # all-equal windows (post-ReLU zeros), two-way ties, negative ties; 2x2 fast path and generic path
+    for (A, B, k, s, p) in [(4, 4, 2, 2, 0), (4, 8, 2, 2, 0), (5, 5, 3, 2, 1), (6, 6, 3, 1, 0)]:
+        rng = np.random.default_rng(A * B)
+        x = rng.integers(-1, 2, size=3 * 2 * A * B).astype(np.float32)  # values in {-1, 0, 1}: ties everywhere
+        oA, oB = (A + 2 * p - k) // s + 1, (B + 2 * p - k) // s + 1
+        d = np.arange(1, 3 * 2 * oA * oB + 1, dtype=np.float32)
+        px, pd = dev.upload(x), dev.upload(d)
+        idx = dev.zeros(d.size, np.int32)
+        ok(hip.fitre_hip_max_pool_argmax(px, 3, 2, A, B, k, s, p, oA, oB, idx))
+        np.testing.assert_array_equal(dev.download(idx, d.size, np.int32), oracle64.max_pool_argmax(x, 2, 3, B, A, k, s, p))
+        back = dev.zeros(x.size)
+        ok(hip.fitre_hip_pool_backward(MAX_POOL, pd, px, 3, 2, A, B, k, s, p, oA, oB, back))
+        np.testing.assert_array_equal(dev.download(back, x.size), oracle64.pool_backward(0, d, x, 2, 3, B, A, k, s, p).astype(np.float32))
+
+
+@pytest.mark.parametrize("geom", POOL_GEOMS[:4])
+@pytest.mark.parametrize("act", [CNN_ACT_RELU, CNN_ACT_SWISH, CNN_ACT_SOFTPLUS, CNN_ACT_NONE])
+@pytest.mark.parametrize("kind", [MAX_POOL, AVG_POOL, NO_POOL])
+def test_fused_pool_activation_backward(dev, oracle64, geom, act, kind):
+    Cn, N, A, B, k, s, p = geom
+    oA, oB = ((A + 2 * p - k) // s + 1, (B + 2 * p - k) // s + 1) if kind != NO_POOL else (A, B)
+    rng = np.random.default_rng(act + kind)
+    zin = rng.standard_normal(Cn * N * A * B).astype(np.float32)
+    zact = oracle64.activation_forward(act, zin.astype(np.float64)).astype(np.float32)
+    d = rng.standard_normal(Cn * N * oA * oB).astype(np.float32)
+    pz, pa, pd = dev.upload(zin), dev.upload(zact), dev.upload(d)
+    dxp, dxa = dev.zeros(zin.size), dev.zeros(zin.size)
+    ok(hip.fitre_hip_pool_act_backward(kind, act, pd, pz, pa, Cn, N, A, B, k, s, p, oA, oB, dxp, dxa))
+    if kind == NO_POOL:
+        wantp = d.astype(np.float64)
+    else:
+        wantp = oracle64.pool_backward(kind, d, zact, N, Cn, B, A, k, s, p)
+    wanta = oracle64.activation_backward(act, wantp, zin.astype(np.float64), zact.astype(np.float64))
+    assert rel_err(dev.download(dxp, zin.size), wantp) < 1e-6
+    assert rel_err(dev.download(dxa, zin.size), wanta) < 1e-5
+
+
+def test_pool_shape_mismatch_is_rejected(dev):
+    p = dev.zeros(64)
+    assert hip.fitre_hip_pool_forward(MAX_POOL, p, 1, 1, 8, 8, 2, 2, 0, 3, 4, p) == 2
+    assert hip.fitre_hip_pool_forward(5, p, 1, 1, 8, 8, 2, 2, 0, 4, 4, p) == 3
+
+
+# ------------------------------------------------------------------ batch norm and reductions
+def bn_ws(dev, Cn, per):
+    nbytes = hip.fitre_hip_batch_norm_workspace(Cn, per)
+    return dev.alloc(nbytes), nbytes
+
+
+def test_bn_backward_reference_known_answer(dev):
+    g = json.load(open(os.path.join(HERE, "golden", "bn_backward_known_answer.json")))
+    ws, nb = bn_ws(dev, 1, 4)
+    out = dev.zeros(4)
+    ok(hip.fitre_hip_batch_norm_backward(dev.upload(g["err"]), dev.upload(g["zout"]), dev.upload([g["variance"]]), 1, 4,
+                                         g["epsilon"], out, None, ws, nb))
+    np.testing.assert_allclose(dev.download(out, 4), g["expected"], rtol=2e-5)
+
+
+@pytest.mark.parametrize("Cn,N,A,B,mis", [(3, 5, 4, 6, 0), (64, 8, 32, 32, 0), (6, 37, 28, 28, 0), (5, 3, 3, 3, 1), (16, 1024, 28, 28, 0)])
+def test_batch_norm_forward_backward(dev, oracle64, Cn, N, A, B, mis):
+    per = N * A * B
+    rng = np.random.default_rng(per % 1000)
+    x = (rng.standard_normal(Cn * per) * 1.7 + 0.4).astype(np.float32)
+    d = rng.standard_normal(Cn * per).astype(np.float32) * np.float32(1e-3)
+    ws, nb = bn_ws(dev, Cn, per)
+    xbuf = dev.upload(np.concatenate([np.zeros(mis, np.float32), x]))
+    px = at(xbuf, mis)
+    zh = dev.zeros(Cn * per + mis)
+    pz = at(zh, mis)
+    stats = dev.upload(np.concatenate([np.zeros(2 * Cn), np.full(Cn, 0.5), np.full(Cn, 2.0)]))
+    mean, var, rmean, rvar = (at(stats, i * Cn) for i in range(4))
+    ok(hip.fitre_hip_batch_norm_forward(px, Cn, per, pz, mean, var, rmean, rvar, 1e-5, 0.9, 1, ws, nb))
+    zhat, wmean, wvar, wrm, wrv = oracle64.batch_norm_forward(x, B, A, Cn, N, running=(np.full(Cn, 0.5), np.full(Cn, 2.0)))
+    got_stats = dev.download(stats, 4 * Cn)
+    assert rel_err(got_stats[:Cn], wmean) < 1e-5 and rel_err(got_stats[Cn:2 * Cn], wvar) < 1e-5
+    assert rel_err(got_stats[2 * Cn:3 * Cn], wrm) < 1e-5 and rel_err(got_stats[3 * Cn:], wrv) < 1e-5
+    assert rel_err(dev.download(pz, Cn * per), zhat) < 1e-5
+    # evaluation mode: running statistics, which the call must leave unchanged
+    ok(hip.fitre_hip_batch_norm_forward(px, Cn, per, pz, mean, var, rmean, rvar, 1e-5, 0.9, 0, ws, nb))
+    ze, *_ = oracle64.batch_norm_forward(x, B, A, Cn, N, train=False, running=(wrm, wrv))
+    assert rel_err(dev.download(pz, Cn * per), ze) < 1e-5
+    np.testing.assert_array_equal(dev.download(stats, 4 * Cn), got_stats)
+    # backward on the oracle's zhat (isolates the backward kernel)
+    dbuf = dev.upload(np.concatenate([np.zeros(mis, np.float32), d]))
+    zbuf = dev.upload(np.concatenate([np.zeros(mis, np.float32), zhat.astype(np.float32)]))
+    out = dev.zeros(Cn * per + mis)
+    db_ = dev.zeros(Cn)
+    ok(hip.fitre_hip_batch_norm_backward(at(dbuf, mis), at(zbuf, mis), dev.upload(wvar), Cn, per, 1e-5, at(out, mis), db_, ws, nb))
+    want = oracle64.batch_norm_backward(d, zhat.astype(np.float32), wvar.astype(np.float32), B, A, Cn, N)
+    got = dev.download(at(out, mis), Cn * per)
+    assert rel_err(got, want) < TOL
+    # bias gradient = column sums of the result; mathematically zero, so compare with the sums of what was written
+    np.testing.assert_allclose(dev.download(db_, Cn), got.astype(np.float64).reshape(Cn, per).sum(1), atol=1e-5 * np.abs(got).max() * np.sqrt(per))
+    for b in (xbuf, zh, dbuf, zbuf, out, ws):
+        dev.free(b)
+
+
+def test_workspace_too_small_is_reported(dev):
+    p = dev.zeros(4096)
+    assert hip.fitre_hip_batch_norm_backward(p, p, p, 4, 1024, 1e-5, p, None, p, 8) == 4
+    assert b"workspace" in hip.fitre_hip_last_error()
+
+
+@pytest.mark.parametrize("Cn,per", [(6, 100352), (16, 12800), (64, 262144), (3, 17), (512, 1024)])
+def test_channel_sum(dev, Cn, per):
+    rng = np.random.default_rng(Cn)
+    x = rng.standard_normal(Cn * per).astype(np.float32)
+    nb = hip.fitre_hip_channel_sum_workspace(Cn, per)
+    ws, out = dev.alloc(nb), dev.zeros(Cn)
+    ok(hip.fitre_hip_channel_sum(dev.upload(x), Cn, per, out, ws, nb))
+    want = x.astype(np.float64).reshape(Cn, per).sum(1)
+    np.testing.assert_allclose(dev.download(out, Cn), want, atol=2e-7 * np.abs(x).astype(np.float64).reshape(Cn, per).sum(1).max())
+
+
+# ------------------------------------------------------------------ softmax cross entropy
+@pytest.mark.parametrize("rows,classes", [(4, 10), (256, 10), (64, 1000), (1024, 10), (3, 70)])
+def test_softmax_cross_entropy(dev, oracle64, rows, classes):
+    rng = np.random.default_rng(rows + classes)
+    logits = (rng.standard_normal(rows * classes) * 2).astype(np.float32)
+    y = rng.integers(1, classes + 1, rows).astype(np.float32)
+    pl, py = dev.upload(logits), dev.upload(y)
+    probs, err = dev.zeros(rows * classes), dev.zeros(rows * classes)
+    loss = C.c_float()
+    ok(hip.fitre_hip_softmax_cross_entropy(pl, py, rows, classes, probs, err, C.byref(loss)))
+    wl, wp = oracle64.softmax_loss(logits, y, rows, classes)
+    we = oracle64.cross_entropy_error(wp, y, rows, classes)
+    assert abs(loss.value - wl) < 1e-5 * max(1, abs(wl))
+    assert rel_err(dev.download(probs, rows * classes), wp) < 1e-5
+    assert rel_err(dev.download(err, rows * classes), we) < 1e-5
+    err2 = dev.zeros(rows * classes)
+    ok(hip.fitre_hip_cross_entropy_error(probs, py, rows, classes, err2))
+    np.testing.assert_allclose(dev.download(err2, rows * classes), dev.download(err, rows * classes), rtol=1e-6, atol=1e-9)
+
+
+# ------------------------------------------------------------------ layout changes
+def test_boundary_permutes(dev, oracle64):
+    Cn, N, A, B = 5, 3, 4, 2
+    x = np.arange(Cn * N * A * B, dtype=np.float32)
+    px, out, back = dev.upload(x), dev.zeros(x.size), dev.zeros(x.size)
+    ok(hip.fitre_hip_conv_to_fc(px, Cn, N, A, B, out))
+    want = oracle64.transpose(oracle64.reshape(x, Cn, N, A * B), Cn * N, B, A)
+    np.testing.assert_array_equal(dev.download(out, x.size), want)
+    ok(hip.fitre_hip_fc_to_conv(out, Cn, N, A, B, back))
+    np.testing.assert_array_equal(dev.download(back, x.size), x)
+    ok(hip.fitre_hip_reshape(px, Cn, N, A * B, out))
+    np.testing.assert_array_equal(dev.download(out, x.size), oracle64.reshape(x, Cn, N, A * B))
+    assert hip.fitre_hip_conv_to_fc(px, Cn, N, A, B, px) == 2  # in place is refused
