@@ -50,26 +50,22 @@ int check_launch(const char *what);
 // q = n / d for 0 <= n < 2^31 via one 32x32->64 multiply.
 struct FastDiv {
 	uint32_t mul;
-	uint32_t shift;
+	uint32_t shiftm1; // ceil(log2 d) - 1 (0 for d <= 2)
 	uint32_t div;
-	__host__ __device__ FastDiv() : mul(0), shift(0), div(1) {}
-	__host__ __device__ explicit FastDiv(uint32_t d) : div(d)
+	__host__ __device__ FastDiv() : mul(0), shiftm1(0), div(1) {}
+	__host__ __device__ explicit FastDiv(uint32_t d) : mul(0), shiftm1(0), div(d)
 	{
-		if (d == 1) {
-			mul = 0;
-			shift = 0;
-			return;
-		}
+		if (d <= 1) return;
 		uint32_t l = 0;
 		while ((1ull << l) < d) l++;
-		shift = l;
+		shiftm1 = l - 1;
 		mul = (uint32_t)(((1ull << 32) * ((1ull << l) - d)) / d + 1);
 	}
 	__device__ __forceinline__ uint32_t quot(uint32_t n) const
 	{
-		if (div == 1) return n;
 		uint32_t t = __umulhi(n, mul);
-		return (t + ((n - t) >> 1)) >> (shift - 1);
+		uint32_t q = (t + ((n - t) >> 1)) >> shiftm1;
+		return (div == 1) ? n : q; // a select, not a branch
 	}
 	__device__ __forceinline__ void divmod(uint32_t n, uint32_t &q, uint32_t &r) const
 	{

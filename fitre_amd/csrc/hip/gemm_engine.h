@@ -30,7 +30,6 @@ struct TileCfg {
 	static constexpr int BM = BM_, BN = BN_, BK = BK_;
 	static constexpr int WM = BM / 2, WN = BN / 2; // wave tile
 	static constexpr int TM = WM / 32, TN = WN / 32; // 32x32 blocks per wave
-	static constexpr int LDA = BM + 1, LDB = BN + 1; // odd strides: conflict-light for both access patterns
 	static_assert(BM % 64 == 0 && BN % 64 == 0 && BK % 2 == 0, "tile shape");
 	static_assert((BM * BK) % kGemmThreads == 0 && (BN * BK) % kGemmThreads == 0, "tile shape");
 	static_assert(kGemmThreads % BK == 0, "BK must divide the workgroup");
@@ -41,31 +40,58 @@ struct TileCfg {
 //   init(params, row0, tid)      once per workgroup
 //   load(k0, kend, regs)         global -> registers, zero outside the matrix
 //   store(lds, regs)             registers -> LDS [k][row], row stride LD
+//
+// Global reads go through a raw buffer resource: an element outside the matrix
+// or the image gets the byte offset 0xFFFFFFFF, which the hardware range check
+// answers with zero -- no branch and no 64-bit address arithmetic per element.
+// Every tensor an operand reads must therefore be smaller than 4 GiB.
 // ---------------------------------------------------------------------------
+
+constexpr uint32_t kOutOfRange = 0xFFFFFFFFu;
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const float *p, uint32_t bytes)
+{
+	return __builtin_amdgcn_make_buffer_rsrc((void *)p, 0, bytes, 0x00020000);
+}
+__device__ __forceinline__ float buffer_load(__amdgpu_buffer_rsrc_t r, uint32_t byteOffset)
+{
+	return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, (int)byteOffset, 0, 0));
+}
+
+// LDS row stride for a tile of ROWS rows: stores of the k-contiguous operands
+// put 16 (BK = 16) or 32 (BK = 32) consecutive k of a few rows into one
+// instruction; stride = 2 (resp. 1) mod 32 spreads them over all banks.  Reads
+// (32 consecutive rows of one k) are conflict-free for any stride.
+template <int ROWS, int BK>
+struct LdsStride {
+	static constexpr int value = ROWS + (BK == 16 ? 2 : 1);
+};
 
 // a strided matrix operand: rows along the non-reduction index
 struct PlainParams {
 	const float *p;
-	long ld;
+	uint32_t bytes; // extent of the matrix in memory
+	int ld;
 	int rows;
 };
 
 // element(row, k) = p[k * ld + row]   (contiguous along the non-reduction index)
-template <int ROWS, int BK, int LD>
+template <int ROWS, int BK>
 struct PlainRowContig {
 	static constexpr int E = ROWS * BK / kGemmThreads;
 	static constexpr int KSTEP = kGemmThreads / ROWS;
+	static constexpr int LD = LdsStride<ROWS, BK>::value;
 	typedef PlainParams Params;
-	const float *p;
-	long ld;
-	int rowL, kL;
+	__amdgpu_buffer_rsrc_t rsrc;
+	int ld, rowL, kL, row;
 	bool rowOk;
 	__device__ __forceinline__ void init(const Params &pr, int row0, int tid)
 	{
+		rsrc = make_rsrc(pr.p, pr.bytes);
 		rowL = tid % ROWS;
 		kL = tid / ROWS;
-		rowOk = (row0 + rowL) < pr.rows;
-		p = pr.p + (row0 + rowL);
+		row = row0 + rowL;
+		rowOk = row < pr.rows;
 		ld = pr.ld;
 	}
 	__device__ __forceinline__ void load(int k0, int kend, float (&r)[E]) const
@@ -73,7 +99,8 @@ struct PlainRowContig {
 #pragma unroll
 		for (int e = 0; e < E; e++) {
 			int k = k0 + kL + KSTEP * e;
-			r[e] = (rowOk && k < kend) ? p[(size_t)k * ld] : 0.f;
+			uint32_t off = (rowOk & (k < kend)) ? 4u * (uint32_t)(k * ld + row) : kOutOfRange;
+			r[e] = buffer_load(rsrc, off);
 		}
 	}
 	__device__ __forceinline__ void store(float *lds, const float (&r)[E]) const
@@ -84,21 +111,25 @@ struct PlainRowContig {
 };
 
 // element(row, k) = p[row * ld + k]   (contiguous along the reduction index)
-template <int ROWS, int BK, int LD>
+template <int ROWS, int BK>
 struct PlainKContig {
 	static constexpr int E = ROWS * BK / kGemmThreads;
 	static constexpr int RSTEP = kGemmThreads / BK;
+	static constexpr int LD = LdsStride<ROWS, BK>::value;
 	typedef PlainParams Params;
-	const float *p;
-	long ld;
-	int rowL, kL, rowsLeft;
+	__amdgpu_buffer_rsrc_t rsrc;
+	int rowL, kL;
+	uint32_t rowOff[E]; // 4 * row * ld, or out of range
 	__device__ __forceinline__ void init(const Params &pr, int row0, int tid)
 	{
+		rsrc = make_rsrc(pr.p, pr.bytes);
 		kL = tid % BK;
 		rowL = tid / BK;
-		rowsLeft = pr.rows - row0;
-		p = pr.p + (size_t)row0 * pr.ld;
-		ld = pr.ld;
+#pragma unroll
+		for (int e = 0; e < E; e++) {
+			int row = row0 + rowL + RSTEP * e;
+			rowOff[e] = (row < pr.rows) ? 4u * (uint32_t)(row * pr.ld) : kOutOfRange;
+		}
 	}
 	__device__ __forceinline__ void load(int k0, int kend, float (&r)[E]) const
 	{
@@ -106,8 +137,8 @@ struct PlainKContig {
 		bool kOk = k < kend;
 #pragma unroll
 		for (int e = 0; e < E; e++) {
-			int row = rowL + RSTEP * e;
-			r[e] = (kOk && row < rowsLeft) ? p[(size_t)row * ld + k] : 0.f;
+			uint32_t off = (kOk & (rowOff[e] != kOutOfRange)) ? rowOff[e] + 4u * (uint32_t)k : kOutOfRange;
+			r[e] = buffer_load(rsrc, off);
 		}
 	}
 	__device__ __forceinline__ void store(float *lds, const float (&r)[E]) const
@@ -123,21 +154,53 @@ struct PlainKContig {
 // image read as zero.
 struct PatchGeom {
 	const float *src; // [channels][samples][srcA][srcB]
+	uint32_t bytes;   // extent of src
 	int samples, srcA, srcB, outA, outB, ksize, stride, pad;
-	int positions;      // samples * outA * outB
-	int taps;           // ksize * ksize
-	int patchLen;       // channels * taps
-	long chanStride;    // samples * srcA * srcB
+	int positions;   // samples * outA * outB
+	int taps;        // ksize * ksize
+	int patchLen;    // channels * taps
+	int chanStride;  // samples * srcA * srcB
+	// Decode of the reduction index k = (c, ta, tb) for the operand whose k is uniform across a
+	// wave: low word c*chanStride + ta*srcB + tb, high word ta << 16 | tb.  Entries are stored in
+	// the order the waves consume them (see patch_table_slot) and read with scalar loads.
+	const unsigned long long *ktable;
 	FastDiv divOutB, divOutA, divTaps, divK;
 };
 
+// A wave of the row-contiguous patch operand handles, in every BK-deep slice, the indices
+// k0 + kL + kstep*e (e = 0..BK/kstep-1); their table entries sit next to each other.
+__host__ __device__ inline int patch_table_slot(int k, int bk, int kstep)
+{
+	int in = k % bk;
+	return (k - in) + (in % kstep) * (bk / kstep) + in / kstep;
+}
+
+// fills PatchGeom::ktable for slices of depth bk read with stride kstep; `padded` entries
+__global__ void patch_table_kernel(unsigned long long *table, int padded, int patchLen, int chanStride, int srcB,
+                                   FastDiv divTaps, FastDiv divK, int bk, int kstep)
+{
+	int k = blockIdx.x * blockDim.x + threadIdx.x;
+	if (k >= padded) return;
+	unsigned long long entry = 0;
+	if (k < patchLen) {
+		uint32_t c, tap, ta, tb;
+		divTaps.divmod((uint32_t)k, c, tap);
+		divK.divmod(tap, ta, tb);
+		uint32_t off = (uint32_t)((int)c * chanStride + (int)ta * srcB + (int)tb);
+		entry = ((unsigned long long)((ta << 16) | tb) << 32) | off;
+	}
+	table[patch_table_slot(k, bk, kstep)] = entry;
+}
+
 // element(row = m, k = (c, ta, tb)) of the patch matrix; contiguous along m.
-template <int ROWS, int BK, int LD>
+template <int ROWS, int BK>
 struct PatchRowContig {
 	static constexpr int E = ROWS * BK / kGemmThreads;
 	static constexpr int KSTEP = kGemmThreads / ROWS;
+	static constexpr int LD = LdsStride<ROWS, BK>::value;
 	typedef PatchGeom Params;
 	PatchGeom g; // copy of the kernel argument: stays in scalar registers
+	__amdgpu_buffer_rsrc_t rsrc;
 	int rowL, kL;
 	int a0, b0;  // source cell of tap (0,0)
 	int base;    // offset of that cell inside a channel plane (may be negative)
@@ -145,6 +208,7 @@ struct PatchRowContig {
 	__device__ __forceinline__ void init(const Params &pr, int row0, int tid)
 	{
 		g = pr;
+		rsrc = make_rsrc(pr.src, pr.bytes);
 		rowL = tid % ROWS;
 		kL = __builtin_amdgcn_readfirstlane(tid / ROWS); // the same for a whole wave (ROWS >= 64)
 		uint32_t m = (uint32_t)(row0 + rowL);
@@ -158,16 +222,19 @@ struct PatchRowContig {
 	}
 	__device__ __forceinline__ void load(int k0, int kend, float (&r)[E]) const
 	{
+		// the E entries of this wave are contiguous and 8*E-byte aligned: one wide scalar load
+		const unsigned long long *p =
+		    (const unsigned long long *)__builtin_assume_aligned(g.ktable + (k0 + kL * E), 8 * E);
+		unsigned long long t[E];
+#pragma unroll
+		for (int e = 0; e < E; e++) t[e] = p[e];
 #pragma unroll
 		for (int e = 0; e < E; e++) {
 			int k = k0 + kL + KSTEP * e; // wave-uniform
-			uint32_t c, tap, ta, tb;
-			g.divTaps.divmod((uint32_t)k, c, tap);
-			g.divK.divmod(tap, ta, tb);
-			int a = a0 + (int)ta, b = b0 + (int)tb;
-			bool ok = rowOk && k < kend && (unsigned)a < (unsigned)g.srcA && (unsigned)b < (unsigned)g.srcB;
-			long off = (long)c * g.chanStride + base + (int)ta * g.srcB + (int)tb;
-			r[e] = ok ? g.src[off] : 0.f;
+			int tap = (int)(t[e] >> 32), kOff = (int)(uint32_t)t[e];
+			int a = a0 + (tap >> 16), b = b0 + (tap & 0xffff);
+			bool ok = rowOk & (k < kend) & ((unsigned)a < (unsigned)g.srcA) & ((unsigned)b < (unsigned)g.srcB);
+			r[e] = buffer_load(rsrc, ok ? 4u * (uint32_t)(base + kOff) : kOutOfRange);
 		}
 	}
 	__device__ __forceinline__ void store(float *lds, const float (&r)[E]) const
@@ -179,18 +246,21 @@ struct PatchRowContig {
 
 // element(row = (c, ta, tb), k = m) of the transposed patch matrix; the reduction
 // index m is the contiguous one.  Used for the weight gradient.
-template <int ROWS, int BK, int LD>
+template <int ROWS, int BK>
 struct PatchKContig {
 	static constexpr int E = ROWS * BK / kGemmThreads;
 	static constexpr int RSTEP = kGemmThreads / BK;
+	static constexpr int LD = LdsStride<ROWS, BK>::value;
 	typedef PatchGeom Params;
 	PatchGeom g;
+	__amdgpu_buffer_rsrc_t rsrc;
 	int rowL, kL;
-	long rowOff[E]; // c*chanStride + ta*srcB + tb, or -1 for rows past the patch length
-	int rowTap[E];  // ta << 16 | tb
+	int rowOff[E]; // c*chanStride + ta*srcB + tb, or -1 for rows past the patch length
+	int rowTap[E]; // ta << 16 | tb
 	__device__ __forceinline__ void init(const Params &pr, int row0, int tid)
 	{
 		g = pr;
+		rsrc = make_rsrc(pr.src, pr.bytes);
 		kL = tid % BK;
 		rowL = tid / BK;
 #pragma unroll
@@ -199,7 +269,7 @@ struct PatchKContig {
 			uint32_t c, tap, ta, tb;
 			pr.divTaps.divmod(row, c, tap);
 			pr.divK.divmod(tap, ta, tb);
-			rowOff[e] = (row < (uint32_t)pr.patchLen) ? (long)c * pr.chanStride + (long)ta * pr.srcB + tb : -1;
+			rowOff[e] = (row < (uint32_t)pr.patchLen) ? (int)c * pr.chanStride + (int)ta * pr.srcB + (int)tb : -1;
 			rowTap[e] = (int)((ta << 16) | tb);
 		}
 	}
@@ -211,12 +281,12 @@ struct PatchKContig {
 		g.divOutB.divmod(m, q, ob);
 		g.divOutA.divmod(q, n, oa);
 		int a0 = (int)oa * g.stride - g.pad, b0 = (int)ob * g.stride - g.pad;
-		long base = (long)n * g.srcA * g.srcB + (long)a0 * g.srcB + b0;
+		int base = (int)n * g.srcA * g.srcB + a0 * g.srcB + b0;
 #pragma unroll
 		for (int e = 0; e < E; e++) {
 			int a = a0 + (rowTap[e] >> 16), b = b0 + (rowTap[e] & 0xffff);
-			bool ok = kOk && rowOff[e] >= 0 && (unsigned)a < (unsigned)g.srcA && (unsigned)b < (unsigned)g.srcB;
-			r[e] = ok ? g.src[rowOff[e] + base] : 0.f;
+			bool ok = kOk & (rowOff[e] >= 0) & ((unsigned)a < (unsigned)g.srcA) & ((unsigned)b < (unsigned)g.srcB);
+			r[e] = buffer_load(rsrc, ok ? 4u * (uint32_t)(rowOff[e] + base) : kOutOfRange);
 		}
 	}
 	__device__ __forceinline__ void store(float *lds, const float (&r)[E]) const
@@ -230,23 +300,32 @@ struct PatchKContig {
 // w[o][ci][ksize-1-ta][ksize-1-tb]  (w is [Cout][Cin][k][k]).
 struct FlipWeightParams {
 	const float *w;
-	int cin, taps;   // taps = ksize*ksize
-	long outStride;  // cin * taps
+	uint32_t bytes;
+	int cin, taps;  // taps = ksize*ksize
+	int outStride;  // cin * taps
 	FastDiv divTaps;
 };
-template <int ROWS, int BK, int LD>
+template <int ROWS, int BK>
 struct FlipWeightKContig {
 	static constexpr int E = ROWS * BK / kGemmThreads;
 	static constexpr int RSTEP = kGemmThreads / BK;
+	static constexpr int LD = LdsStride<ROWS, BK>::value;
 	typedef FlipWeightParams Params;
 	FlipWeightParams g;
-	int rowL, kL, row0;
-	__device__ __forceinline__ void init(const Params &pr, int r0, int tid)
+	__amdgpu_buffer_rsrc_t rsrc;
+	int rowL, kL;
+	int rowOff[E]; // row * taps, or -1
+	__device__ __forceinline__ void init(const Params &pr, int row0, int tid)
 	{
 		g = pr;
+		rsrc = make_rsrc(pr.w, pr.bytes);
 		kL = tid % BK;
 		rowL = tid / BK;
-		row0 = r0;
+#pragma unroll
+		for (int e = 0; e < E; e++) {
+			int row = row0 + rowL + RSTEP * e;
+			rowOff[e] = (row < pr.cin) ? row * pr.taps : -1;
+		}
 	}
 	__device__ __forceinline__ void load(int k0, int kend, float (&r)[E]) const
 	{
@@ -254,12 +333,10 @@ struct FlipWeightKContig {
 		bool kOk = k < kend;
 		uint32_t o, tap;
 		g.divTaps.divmod((uint32_t)k, o, tap);
-		long off = (long)o * g.outStride + (g.taps - 1 - (int)tap);
+		int off = (int)o * g.outStride + (g.taps - 1 - (int)tap);
 #pragma unroll
-		for (int e = 0; e < E; e++) {
-			int row = row0 + rowL + RSTEP * e;
-			r[e] = (kOk && row < g.cin) ? g.w[off + (long)row * g.taps] : 0.f;
-		}
+		for (int e = 0; e < E; e++)
+			r[e] = buffer_load(rsrc, (kOk & (rowOff[e] >= 0)) ? 4u * (uint32_t)(off + rowOff[e]) : kOutOfRange);
 	}
 	__device__ __forceinline__ void store(float *lds, const float (&r)[E]) const
 	{
@@ -290,8 +367,9 @@ mfma_gemm_kernel(const typename OpA::Params pa, const typename OpB::Params pb, c
 {
 	constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK;
 	constexpr int TM = Cfg::TM, TN = Cfg::TN;
-	__shared__ float As[BK * Cfg::LDA];
-	__shared__ float Bs[BK * Cfg::LDB];
+	constexpr int LDA = OpA::LD, LDB = OpB::LD;
+	__shared__ float As[BK * LDA];
+	__shared__ float Bs[BK * LDB];
 
 	const int tid = threadIdx.x;
 	const int lane = tid & 63;
@@ -317,9 +395,9 @@ mfma_gemm_kernel(const typename OpA::Params pa, const typename OpB::Params pb, c
 	opA.load(kbeg, kend, ra);
 	opB.load(kbeg, kend, rb);
 
-	const int wi = (wave >> 1) * Cfg::WM + (lane & 31);
-	const int wj = (wave & 1) * Cfg::WN + (lane & 31);
 	const int khalf = lane >> 5;
+	const float *aRd = As + khalf * LDA + (wave >> 1) * Cfg::WM + (lane & 31);
+	const float *bRd = Bs + khalf * LDB + (wave & 1) * Cfg::WN + (lane & 31);
 
 	for (int k0 = kbeg; k0 < kend; k0 += BK) {
 		__syncthreads(); // everyone is done reading the previous slice
@@ -330,19 +408,33 @@ mfma_gemm_kernel(const typename OpA::Params pa, const typename OpB::Params pb, c
 			opA.load(k0 + BK, kend, ra);
 			opB.load(k0 + BK, kend, rb);
 		}
+		// the fragments of step kk+1 are read from LDS while the MFMAs of step kk run
+		float a[2][TM], b[2][TN];
+#pragma unroll
+		for (int tm = 0; tm < TM; tm++) a[0][tm] = aRd[tm * 32];
+#pragma unroll
+		for (int tn = 0; tn < TN; tn++) b[0][tn] = bRd[tn * 32];
 #pragma unroll
 		for (int kk = 0; kk < BK / 2; kk++) {
-			const int krow = 2 * kk + khalf;
-			float a[TM], b[TN];
+			const int cur = kk & 1, nxt = cur ^ 1;
+			if (kk + 1 < BK / 2) {
 #pragma unroll
-			for (int tm = 0; tm < TM; tm++) a[tm] = As[krow * Cfg::LDA + wi + tm * 32];
+				for (int tm = 0; tm < TM; tm++) a[nxt][tm] = aRd[(2 * kk + 2) * LDA + tm * 32];
 #pragma unroll
-			for (int tn = 0; tn < TN; tn++) b[tn] = Bs[krow * Cfg::LDB + wj + tn * 32];
+				for (int tn = 0; tn < TN; tn++) b[nxt][tn] = bRd[(2 * kk + 2) * LDB + tn * 32];
+			}
 #pragma unroll
 			for (int tm = 0; tm < TM; tm++)
 #pragma unroll
 				for (int tn = 0; tn < TN; tn++)
-					acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[tm], b[tn], acc[tm][tn], 0, 0, 0);
+					acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][tm], b[cur][tn], acc[tm][tn], 0, 0, 0);
+			// issue order: the LDS reads of the next step go out right behind the first MFMAs
+			// of this one, so that their latency is covered by the 64-cycle matrix operations
+			__builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+			__builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+			__builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+			__builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+			__builtin_amdgcn_sched_group_barrier(0x008, TM * TN, 0);
 		}
 	}
 
@@ -375,21 +467,55 @@ mfma_gemm_kernel(const typename OpA::Params pa, const typename OpB::Params pb, c
 }
 
 // C[i*ldc + j] = alpha * sum_s ws[s][i][j] (+bias) + beta*C, partials summed in split order.
+// VEC = 4: four consecutive j per thread with 16-byte reads (J % 4 == 0, aligned workspace).
+template <int VEC>
 __global__ void __launch_bounds__(256)
 splitk_reduce_kernel(const float *ws, int splits, int I, int J, OutParams out)
 {
-	long total = (long)I * J;
-	long stride = (long)gridDim.x * blockDim.x;
-	for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
-		int i = (int)(idx / J), j = (int)(idx - (long)i * J);
-		double acc = 0.0;
-		for (int s = 0; s < splits; s++) acc += (double)ws[(size_t)s * total + idx];
-		float val = (float)acc * out.alpha;
-		if (out.biasI) val += out.biasI[i];
-		if (out.biasJ) val += out.biasJ[j];
-		float *dst = out.C + (size_t)i * out.ldc + j;
-		if (out.beta != 0.f) val += out.beta * *dst;
-		*dst = val;
+	const long total = (long)I * J;
+	const long groups = total / VEC;
+	const long stride = (long)gridDim.x * blockDim.x;
+	for (long gidx = (long)blockIdx.x * blockDim.x + threadIdx.x; gidx < groups; gidx += stride) {
+		const long idx = gidx * VEC;
+		const int i = (int)(idx / J), j = (int)(idx - (long)i * J);
+		double acc[VEC];
+#pragma unroll
+		for (int v = 0; v < VEC; v++) acc[v] = 0.0;
+		const float *p = ws + idx;
+		int s = 0;
+		for (; s + 4 <= splits; s += 4) { // four independent reads in flight
+			float part[4][VEC];
+#pragma unroll
+			for (int u = 0; u < 4; u++) {
+				if constexpr (VEC == 4) {
+					float4 t = *reinterpret_cast<const float4 *>(p + (size_t)(s + u) * total);
+					part[u][0] = t.x, part[u][1] = t.y, part[u][2] = t.z, part[u][3] = t.w;
+				} else {
+					part[u][0] = p[(size_t)(s + u) * total];
+				}
+			}
+#pragma unroll
+			for (int u = 0; u < 4; u++)
+#pragma unroll
+				for (int v = 0; v < VEC; v++) acc[v] += (double)part[u][v];
+		}
+		for (; s < splits; s++) {
+			if constexpr (VEC == 4) {
+				float4 t = *reinterpret_cast<const float4 *>(p + (size_t)s * total);
+				acc[0] += (double)t.x, acc[1] += (double)t.y, acc[2] += (double)t.z, acc[3] += (double)t.w;
+			} else {
+				acc[0] += (double)p[(size_t)s * total];
+			}
+		}
+#pragma unroll
+		for (int v = 0; v < VEC; v++) {
+			float val = (float)acc[v] * out.alpha;
+			if (out.biasI) val += out.biasI[i];
+			if (out.biasJ) val += out.biasJ[j + v];
+			float *dst = out.C + (size_t)i * out.ldc + j + v;
+			if (out.beta != 0.f) val += out.beta * *dst;
+			*dst = val;
+		}
 	}
 }
 
@@ -404,6 +530,28 @@ struct GemmPlan {
 };
 
 constexpr int kGemmBK = 16;
+constexpr int kComputeUnits = 256; // MI355X
+
+// Estimated duration (microseconds) of a product cut into `splits` reduction ranges.
+// Workgroups are spread evenly over the compute units; a compute unit runs up to three of
+// them at once, and the more it holds the better the matrix pipes stay fed.  A split
+// product pays for writing and re-reading its partial tiles.
+inline double estimate_us(long tiles, int bm, int bn, long I, long J, long R, long splits, long *chunkOut, long *splitsOut)
+{
+	long chunk = (R + splits - 1) / splits;
+	chunk = ((chunk + kGemmBK - 1) / kGemmBK) * kGemmBK;
+	long s = (R + chunk - 1) / chunk;
+	long groups = tiles * s;
+	long perCu = (groups + kComputeUnits - 1) / kComputeUnits;
+	// one k-step of a bm x bn tile keeps the four matrix pipes of a compute unit busy for this long
+	double stepUs = (double)(bm / 32) * (bn / 32) * (kGemmBK / 2) * 64.0 / 4.0 / 2400.0;
+	double eff = perCu >= 3 ? 0.80 : (perCu == 2 ? 0.68 : 0.52);
+	double t = (double)perCu * (double)(chunk / kGemmBK) * stepUs / eff + 3.0;
+	if (s > 1) t += 4.0 + (double)(s + 1) * (double)I * (double)J * 4.0 / 3.0e6; // ~3 TB/s, bytes -> us
+	*chunkOut = chunk;
+	*splitsOut = s;
+	return t;
+}
 
 inline GemmPlan plan_gemm(long I, long J, long R)
 {
@@ -411,18 +559,23 @@ inline GemmPlan plan_gemm(long I, long J, long R)
 	p.bm = (I <= 64) ? 64 : 128;
 	p.bn = (J <= 64) ? 64 : 128;
 	long tiles = ((I + p.bm - 1) / p.bm) * ((J + p.bn - 1) / p.bn);
-	long want = (768 + tiles - 1) / tiles; // aim at three workgroups per compute unit
-	long maxByDepth = R / (4 * kGemmBK);    // keep at least four slices per split
-	if (maxByDepth < 1) maxByDepth = 1;
-	long splits = want < maxByDepth ? want : maxByDepth;
-	if (splits > 1024) splits = 1024;
-	if (splits < 1) splits = 1;
-	long chunk = (R + splits - 1) / splits;
-	chunk = ((chunk + kGemmBK - 1) / kGemmBK) * kGemmBK;
-	splits = (R + chunk - 1) / chunk;
-	p.splits = (int)splits;
-	p.kChunk = (int)chunk;
-	p.wsBytes = (splits > 1) ? (size_t)splits * I * J * sizeof(float) : 0;
+	long maxSplits = R / (2 * kGemmBK); // at least two slices per split
+	if (maxSplits > 1024) maxSplits = 1024;
+	if (maxSplits < 1) maxSplits = 1;
+	double best = 1e30;
+	long bestChunk = ((R + kGemmBK - 1) / kGemmBK) * kGemmBK, bestSplits = 1;
+	for (long s = 1; s <= maxSplits; s++) {
+		long chunk, eff;
+		double t = estimate_us(tiles, p.bm, p.bn, I, J, R, s, &chunk, &eff);
+		if (t < best) {
+			best = t;
+			bestChunk = chunk;
+			bestSplits = eff;
+		}
+	}
+	p.splits = (int)bestSplits;
+	p.kChunk = (int)bestChunk;
+	p.wsBytes = (bestSplits > 1) ? (size_t)bestSplits * I * J * sizeof(float) : 0;
 	return p;
 }
 
@@ -444,14 +597,14 @@ inline GemmPlan fit_plan(GemmPlan p, long I, long J, long R, const void *ws, siz
 	return p;
 }
 
-template <template <int, int, int> class OpA, template <int, int, int> class OpB, int BM, int BN>
-static int launch_tile(const typename OpA<BM, kGemmBK, BM + 1>::Params &pa, const typename OpB<BN, kGemmBK, BN + 1>::Params &pb,
+template <template <int, int> class OpA, template <int, int> class OpB, int BM, int BN>
+static int launch_tile(const typename OpA<BM, kGemmBK>::Params &pa, const typename OpB<BN, kGemmBK>::Params &pb,
                        const OutParams &out, int I, int J, int R, const GemmPlan &plan, void *ws, int kernelClass, double flops)
 {
 	typedef TileCfg<BM, BN, kGemmBK> Cfg;
 	constexpr int tileId = (BM == 64 ? (BN == 64 ? 1 : 2) : (BN == 64 ? 3 : 4));
-	typedef OpA<BM, kGemmBK, Cfg::LDA> A;
-	typedef OpB<BN, kGemmBK, Cfg::LDB> B;
+	typedef OpA<BM, kGemmBK> A;
+	typedef OpB<BN, kGemmBK> B;
 	dim3 grid((J + BN - 1) / BN, (I + BM - 1) / BM, plan.splits);
 	if (grid.y > 65535 || grid.z > 65535) return fail(FITRE_E_UNSUPPORTED, "gemm grid %u x %u x %u too large", grid.x, grid.y, grid.z);
 	if (plan.splits > 1) {
@@ -466,7 +619,11 @@ static int launch_tile(const typename OpA<BM, kGemmBK, BM + 1>::Params &pa, cons
 		OutParams fin = out;
 		fin.splitStride = 0;
 		LaunchScope scope(FITRE_KC_SPLITK_REDUCE, 4.0 * (double)I * J * (plan.splits + 1));
-		splitk_reduce_kernel<<<blocks_for((long)I * J, 256, 4096), 256, 0, stream()>>>((const float *)ws, plan.splits, I, J, fin);
+		const bool vec = (J % 4 == 0) && ((((uintptr_t)ws) & 15) == 0);
+		if (vec)
+			splitk_reduce_kernel<4><<<blocks_for((long)I * J / 4, 256, 8192), 256, 0, stream()>>>((const float *)ws, plan.splits, I, J, fin);
+		else
+			splitk_reduce_kernel<1><<<blocks_for((long)I * J, 256, 8192), 256, 0, stream()>>>((const float *)ws, plan.splits, I, J, fin);
 	} else {
 		OutParams direct = out;
 		direct.splitStride = 0;
@@ -477,7 +634,7 @@ static int launch_tile(const typename OpA<BM, kGemmBK, BM + 1>::Params &pa, cons
 }
 
 // Picks the tile instantiation the plan names.
-template <template <int, int, int> class OpA, template <int, int, int> class OpB, class PA, class PB>
+template <template <int, int> class OpA, template <int, int> class OpB, class PA, class PB>
 static int launch_gemm(const PA &pa, const PB &pb, const OutParams &out, int I, int J, int R, const GemmPlan &ideal, void *ws,
                        size_t wsBytes, int kernelClass, double flops)
 {
