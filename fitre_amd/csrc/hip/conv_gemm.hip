@@ -1,6 +1,6 @@
 // Convolution forward / weight gradient / input gradient and the general
 // column-major GEMM, all on the fp32-MFMA tile engine.
-#include "gemm_engine.h"
+#include "conv3x3.h"
 
 namespace fitre {
 
@@ -81,6 +81,188 @@ static double conv_flops(const fitre_conv_shape *s)
 	return 2.0 * (double)s->samples * s->outA * s->outB * (double)s->inChannels * s->ksize * s->ksize * (double)s->outChannels;
 }
 
+// ---- 3x3 / stride 1 / pad 1 fast paths -------------------------------------------------------
+constexpr int kC3CB = 8; // reduction channels per LDS block of the position-contiguous kernels
+
+struct BlockPlan {
+	int splits, perSplit;
+	size_t wsBytes;
+};
+
+// Splits a reduction of nBlocks equal blocks (blockUs microseconds of matrix-pipe time each) over
+// workgroups so that the compute units are evenly loaded; same cost model as plan_gemm.
+static BlockPlan plan_blocks(long tiles, long nBlocks, double blockUs, int residentPerCu, long I, long J)
+{
+	BlockPlan best{ 1, (int)nBlocks, 0 };
+	double bestT = 1e30;
+	for (long s = 1; s <= nBlocks && s <= 1024; s++) {
+		long per = (nBlocks + s - 1) / s;
+		long eff = (nBlocks + per - 1) / per;
+		long groups = tiles * eff;
+		long perCu = (groups + kComputeUnits - 1) / kComputeUnits;
+		double e = perCu >= residentPerCu ? 0.85 : (perCu * 2 >= residentPerCu + 1 ? 0.72 : 0.55);
+		double t = (double)perCu * (double)per * blockUs / e + 3.0;
+		if (eff > 1) t += 4.0 + (double)(eff + 1) * (double)I * (double)J * 4.0 / 3.0e6;
+		if (t < bestT) {
+			bestT = t;
+			best.splits = (int)eff;
+			best.perSplit = (int)per;
+			best.wsBytes = eff > 1 ? (size_t)eff * I * J * sizeof(float) : 0;
+		}
+	}
+	return best;
+}
+
+static BlockPlan fit_blocks(BlockPlan p, long nBlocks, long I, long J, const void *ws, size_t wsBytes)
+{
+	if (p.splits <= 1) return p;
+	size_t per = (size_t)I * J * sizeof(float);
+	long fit = ws ? (long)(wsBytes / per) : 0;
+	if (fit >= p.splits) return p;
+	long s = fit >= 2 ? fit : 1;
+	p.perSplit = (int)((nBlocks + s - 1) / s);
+	p.splits = (int)((nBlocks + p.perSplit - 1) / p.perSplit);
+	p.wsBytes = p.splits > 1 ? (size_t)p.splits * per : 0;
+	return p;
+}
+
+static bool c3_geometry(const fitre_conv_shape *s)
+{
+	return s->ksize == 3 && s->stride == 1 && s->padding == 1 && s->inB <= 64 && s->outA == s->inA && s->outB == s->inB;
+}
+// forward: reduce over Cin; input gradient: reduce over Cout
+static bool c3_pos_eligible(const fitre_conv_shape *s, bool dx)
+{
+	int cred = dx ? s->outChannels : s->inChannels;
+	return c3_geometry(s) && cred % kC3CB == 0;
+}
+static bool c3_dw_eligible(const fitre_conv_shape *s) { return c3_geometry(s) && s->inChannels >= 16 && s->outChannels >= 32; }
+
+static BlockPlan c3_pos_plan(const fitre_conv_shape *s, bool dx)
+{
+	long I = dx ? s->inChannels : s->outChannels, J = (long)s->samples * s->inA * s->inB;
+	long cred = dx ? s->outChannels : s->inChannels;
+	long it = I <= 64 ? 64 : kC3Tile;
+	long tiles = ((I + it - 1) / it) * ((J + kC3Tile - 1) / kC3Tile);
+	double blockUs = (9.0 * kC3CB / 2.0) * (it / 32.0) * 64.0 / 2400.0; // MFMA steps x blocks per wave x 64 cycles
+	return plan_blocks(tiles, cred / kC3CB, blockUs, it == 64 ? 3 : 2, I, J);
+}
+static BlockPlan c3_dw_plan(const fitre_conv_shape *s)
+{
+	long J = (long)s->samples * s->inA * s->inB;
+	long tiles = ((s->inChannels + kC3DwCin - 1) / kC3DwCin) * ((s->outChannels + kC3Tile - 1) / kC3Tile);
+	double stageUs = (kC3Stage / 2.0) * 9.0 * 64.0 / 2400.0;
+	return plan_blocks(tiles, (J + kC3Stage - 1) / kC3Stage, stageUs, 2, s->outChannels, (long)s->inChannels * 9);
+}
+
+static void launch_reduce(const float *ws, int splits, int I, int J, const OutParams &fin)
+{
+	LaunchScope scope(FITRE_KC_SPLITK_REDUCE, 4.0 * (double)I * J * (splits + 1));
+	const bool vec = (J % 4 == 0) && ((((uintptr_t)ws) & 15) == 0);
+	if (vec)
+		splitk_reduce_kernel<4><<<blocks_for((long)I * J / 4, 256, 8192), 256, 0, stream()>>>(ws, splits, I, J, fin);
+	else
+		splitk_reduce_kernel<1><<<blocks_for((long)I * J, 256, 8192), 256, 0, stream()>>>(ws, splits, I, J, fin);
+}
+
+template <bool DX>
+static int launch_c3_pos(const fitre_conv_shape *s, const float *src, const float *w, const float *bias, float *outPtr, void *ws,
+                         size_t wsBytes)
+{
+	const int I = DX ? s->inChannels : s->outChannels, cred = DX ? s->outChannels : s->inChannels;
+	const int J = s->samples * s->inA * s->inB;
+	BlockPlan plan = fit_blocks(c3_pos_plan(s, DX), cred / kC3CB, I, J, ws, wsBytes);
+	if (plan.wsBytes > 0 && (((uintptr_t)ws) & 3)) return fail(FITRE_E_WORKSPACE, "split workspace is misaligned");
+	Conv3x3Params p;
+	p.src = src;
+	p.w = w;
+	p.srcBytes = (uint32_t)((size_t)cred * J * sizeof(float));
+	p.wBytes = (uint32_t)((size_t)s->outChannels * s->inChannels * 9 * sizeof(float));
+	p.I = I;
+	p.cred = cred;
+	p.J = J;
+	p.A = s->inA;
+	p.B = s->inB;
+	p.perSplit = plan.perSplit;
+	p.divB = FastDiv((uint32_t)s->inB);
+	p.divA = FastDiv((uint32_t)s->inA);
+	OutParams out{ outPtr, (long)J, 0, bias, nullptr, 1.f, 0.f };
+	OutParams part = out;
+	if (plan.splits > 1) {
+		part.C = (float *)ws;
+		part.splitStride = (long)I * J;
+	}
+	const bool vecw = ((((uintptr_t)w) & 15) == 0) && (DX ? (I % 4 == 0) : true);
+	const int it = I <= 64 ? 64 : kC3Tile;
+	dim3 grid((J + kC3Tile - 1) / kC3Tile, (I + it - 1) / it, plan.splits);
+	if (grid.y > 65535 || grid.z > 65535) return fail(FITRE_E_UNSUPPORTED, "conv3x3 grid too large");
+	{
+		LaunchScope scope(DX ? FITRE_KC_CONV_DX : FITRE_KC_CONV_FWD, conv_flops(s), it == 64 ? 2 : 4);
+		const bool narrow = s->inB <= 32;
+#define C3_LAUNCH(V, MB, IT_) conv3x3_pos_kernel<kC3CB, DX, V, MB, IT_><<<grid, kGemmThreads, 0, stream()>>>(p, part)
+		if (it == 64) {
+			if (vecw && narrow) C3_LAUNCH(true, 32, 64);
+			else if (vecw) C3_LAUNCH(true, 64, 64);
+			else if (narrow) C3_LAUNCH(false, 32, 64);
+			else C3_LAUNCH(false, 64, 64);
+		} else {
+			if (vecw && narrow) C3_LAUNCH(true, 32, 128);
+			else if (vecw) C3_LAUNCH(true, 64, 128);
+			else if (narrow) C3_LAUNCH(false, 32, 128);
+			else C3_LAUNCH(false, 64, 128);
+		}
+#undef C3_LAUNCH
+	}
+	if (plan.splits > 1) launch_reduce((const float *)ws, plan.splits, I, J, out);
+	return check_launch("conv3x3_pos_kernel");
+}
+
+static int launch_c3_dw(const fitre_conv_shape *s, const float *x, const float *delta, float *dW, void *ws, size_t wsBytes)
+{
+	const int I = s->outChannels, cin = s->inChannels, K = cin * 9;
+	const int J = s->samples * s->inA * s->inB;
+	const int stages = (J + kC3Stage - 1) / kC3Stage;
+	BlockPlan plan = fit_blocks(c3_dw_plan(s), stages, I, K, ws, wsBytes);
+	if (plan.wsBytes > 0 && (((uintptr_t)ws) & 3)) return fail(FITRE_E_WORKSPACE, "split workspace is misaligned");
+	Conv3x3Params p;
+	p.src = x;
+	p.w = nullptr;
+	p.srcBytes = (uint32_t)((size_t)cin * J * sizeof(float));
+	p.wBytes = 0;
+	p.I = I;
+	p.cred = cin;
+	p.J = J;
+	p.A = s->inA;
+	p.B = s->inB;
+	p.perSplit = plan.perSplit;
+	p.divB = FastDiv((uint32_t)s->inB);
+	p.divA = FastDiv((uint32_t)s->inA);
+	OutParams out{ dW, (long)K, 0, nullptr, nullptr, 1.f, 0.f };
+	OutParams part = out;
+	if (plan.splits > 1) {
+		part.C = (float *)ws;
+		part.splitStride = (long)I * K;
+	}
+	const uint32_t deltaBytes = (uint32_t)((size_t)I * J * sizeof(float));
+	const bool vecd = ((((uintptr_t)delta) & 15) == 0) && (J % 4 == 0);
+	dim3 grid((cin + kC3DwCin - 1) / kC3DwCin, (I + kC3Tile - 1) / kC3Tile, plan.splits);
+	if (grid.y > 65535 || grid.z > 65535) return fail(FITRE_E_UNSUPPORTED, "conv3x3 grid too large");
+	{
+		LaunchScope scope(FITRE_KC_CONV_DW, conv_flops(s), 4);
+		const bool narrow = s->inB <= 32;
+		if (vecd && narrow)
+			conv3x3_dw_kernel<true, 32><<<grid, kGemmThreads, 0, stream()>>>(p, delta, deltaBytes, part);
+		else if (vecd)
+			conv3x3_dw_kernel<true, 64><<<grid, kGemmThreads, 0, stream()>>>(p, delta, deltaBytes, part);
+		else if (narrow)
+			conv3x3_dw_kernel<false, 32><<<grid, kGemmThreads, 0, stream()>>>(p, delta, deltaBytes, part);
+		else
+			conv3x3_dw_kernel<false, 64><<<grid, kGemmThreads, 0, stream()>>>(p, delta, deltaBytes, part);
+	}
+	if (plan.splits > 1) launch_reduce((const float *)ws, plan.splits, I, K, out);
+	return check_launch("conv3x3_dw_kernel");
+}
+
 } // namespace fitre
 
 using namespace fitre;
@@ -91,6 +273,7 @@ extern "C" {
 size_t fitre_hip_conv_forward_workspace(const fitre_conv_shape *s)
 {
 	if (!s) return 0;
+	if (c3_pos_eligible(s, false)) return c3_pos_plan(s, false).wsBytes;
 	return plan_gemm(s->outChannels, (long)s->samples * s->outA * s->outB, (long)s->inChannels * s->ksize * s->ksize).wsBytes;
 }
 
@@ -101,6 +284,7 @@ int fitre_hip_conv_forward(const fitre_conv_shape *s, const float *x, const floa
 	int rc = check_conv("fitre_hip_conv_forward", s);
 	if (rc) return rc;
 	FITRE_REQUIRE(x && w && y, "fitre_hip_conv_forward: null pointer");
+	if (c3_pos_eligible(s, false)) return launch_c3_pos<false>(s, x, w, bias, y, ws, wsBytes);
 	const int I = s->outChannels, J = s->samples * s->outA * s->outB, R = s->inChannels * s->ksize * s->ksize;
 	GemmPlan plan = plan_gemm(I, J, R);
 	PlainParams pa{ w, (uint32_t)((size_t)I * R * sizeof(float)), R, I };
@@ -115,6 +299,7 @@ int fitre_hip_conv_forward(const fitre_conv_shape *s, const float *x, const floa
 size_t fitre_hip_conv_weight_grad_workspace(const fitre_conv_shape *s)
 {
 	if (!s) return 0;
+	if (c3_dw_eligible(s)) return c3_dw_plan(s).wsBytes;
 	return plan_gemm(s->outChannels, (long)s->inChannels * s->ksize * s->ksize, (long)s->samples * s->outA * s->outB).wsBytes;
 }
 
@@ -124,6 +309,7 @@ int fitre_hip_conv_weight_grad(const fitre_conv_shape *s, const float *x, const 
 	int rc = check_conv("fitre_hip_conv_weight_grad", s);
 	if (rc) return rc;
 	FITRE_REQUIRE(x && delta && dW, "fitre_hip_conv_weight_grad: null pointer");
+	if (c3_dw_eligible(s)) return launch_c3_dw(s, x, delta, dW, ws, wsBytes);
 	const int I = s->outChannels, J = s->inChannels * s->ksize * s->ksize, R = s->samples * s->outA * s->outB;
 	GemmPlan plan = plan_gemm(I, J, R);
 	PlainParams pa{ delta, (uint32_t)((size_t)I * R * sizeof(float)), R, I };
@@ -136,6 +322,7 @@ int fitre_hip_conv_weight_grad(const fitre_conv_shape *s, const float *x, const 
 size_t fitre_hip_conv_input_grad_workspace(const fitre_conv_shape *s)
 {
 	if (!s) return 0;
+	if (c3_pos_eligible(s, true)) return c3_pos_plan(s, true).wsBytes;
 	return plan_gemm(s->inChannels, (long)s->samples * s->inA * s->inB, (long)s->outChannels * s->ksize * s->ksize).wsBytes;
 }
 
@@ -148,6 +335,7 @@ int fitre_hip_conv_input_grad(const fitre_conv_shape *s, const float *delta, con
 	if (s->stride != 1)
 		return fail(FITRE_E_UNSUPPORTED, "fitre_hip_conv_input_grad: stride %d (only stride 1 is back-propagated through)", s->stride);
 	FITRE_REQUIRE(s->padding < s->ksize, "fitre_hip_conv_input_grad: padding %d >= window %d", s->padding, s->ksize);
+	if (c3_pos_eligible(s, true)) return launch_c3_pos<true>(s, delta, w, nullptr, dx, ws, wsBytes);
 	const int I = s->inChannels, J = s->samples * s->inA * s->inB, R = s->outChannels * s->ksize * s->ksize;
 	GemmPlan plan = plan_gemm(I, J, R);
 	FlipWeightParams pa;

@@ -27,6 +27,15 @@ CONV_CASES = [
     (1, 1, 1, 5, 5, 3, 1, 0),        # degenerate
     (2, 4, 5, 7, 7, 1, 1, 0),        # 1x1 window
     (2, 4, 6, 9, 9, 3, 2, 1),        # stride 2
+    # 3x3 / stride 1 / pad 1 fast paths: tile edges in every dimension
+    (3, 8, 16, 8, 8, 3, 1, 1),       # 192 positions: not a multiple of the 128-position tile
+    (2, 16, 40, 6, 10, 3, 1, 1),     # rectangular maps, 40 output channels
+    (5, 24, 136, 4, 4, 3, 1, 1),     # 136 channels: one full and one partial channel tile
+    (2, 32, 32, 32, 32, 3, 1, 1),    # 32-wide rows
+    (1, 8, 8, 64, 64, 3, 1, 1),      # widest row the LDS window holds
+    (1, 8, 8, 66, 66, 3, 1, 1),      # one wider: general engine
+    (7, 48, 64, 3, 5, 3, 1, 1),      # odd extents, 105 positions
+    (64, 64, 64, 2, 2, 3, 1, 1),     # 2x2 maps
 ]
 
 
@@ -77,6 +86,29 @@ def test_conv_weight_gradient(dev, oracle64, case):
 def test_conv_input_gradient(dev, oracle64, case):
     got, want = run_conv(dev, oracle64, case, "dx")
     assert rel_err(got, want) < TOL
+
+
+def test_conv3x3_with_unaligned_weight_and_delta_pointers(dev, oracle64):
+    """Flat parameter vectors put weight blocks at arbitrary offsets: the fast paths must fall back to
+    4-byte accesses when a pointer is not 16-byte aligned."""
+    from helpers import at
+    N, Cin, Cout, A, B = 4, 16, 32, 8, 8
+    shape = conv_shape(N, Cin, Cout, A, B, 3, 1, 1)
+    rng = np.random.default_rng(77)
+    x = rng.standard_normal(Cin * N * A * B).astype(np.float32)
+    w = rng.standard_normal(Cout * Cin * 9).astype(np.float32)
+    d = rng.standard_normal(Cout * N * A * B).astype(np.float32)
+    pw = at(dev.upload(np.concatenate([np.zeros(3, np.float32), w])), 3)
+    pd = at(dev.upload(np.concatenate([np.zeros(1, np.float32), d])), 1)
+    px = dev.upload(x)
+    ws = dev.alloc(1 << 24)
+    out = dev.zeros(max(d.size, x.size, w.size))
+    L.check(hip.fitre_hip_conv_forward(C.byref(shape), px, pw, None, out, ws, 1 << 24))
+    assert rel_err(dev.download(out, d.size), oracle64.conv_forward(x, w, None, N, Cin, B, A, 3, 1, 1, Cout)) < TOL
+    L.check(hip.fitre_hip_conv_input_grad(C.byref(shape), pd, pw, out, ws, 1 << 24))
+    assert rel_err(dev.download(out, x.size), oracle64.conv_input_grad(d, w, N, Cin, B, A, 3, 1, Cout)) < TOL
+    L.check(hip.fitre_hip_conv_weight_grad(C.byref(shape), px, pd, out, ws, 1 << 24))
+    assert rel_err(dev.download(out, w.size), oracle64.conv_weight_grad(x, d, N, Cin, B, A, 3, 1, 1, Cout)) < TOL
 
 
 def test_conv_input_gradient_refuses_stride(dev):
