@@ -1,55 +1,9 @@
 // Convolution forward / weight gradient / input gradient and the general
 // column-major GEMM, all on the fp32-MFMA tile engine.
 #include "conv3x3.h"
+#include "conv_common.h"
 
 namespace fitre {
-
-static int check_conv(const char *fn, const fitre_conv_shape *s)
-{
-	FITRE_REQUIRE(s != nullptr, "%s: null shape", fn);
-	FITRE_REQUIRE(s->samples > 0 && s->inChannels > 0 && s->outChannels > 0 && s->inA > 0 && s->inB > 0 && s->ksize > 0 &&
-	                  s->stride > 0 && s->padding >= 0,
-	              "%s: non-positive shape (N=%d Cin=%d Cout=%d A=%d B=%d k=%d s=%d p=%d)", fn, s->samples, s->inChannels,
-	              s->outChannels, s->inA, s->inB, s->ksize, s->stride, s->padding);
-	FITRE_REQUIRE(s->outA == (s->inA + 2 * s->padding - s->ksize) / s->stride + 1 &&
-	                  s->outB == (s->inB + 2 * s->padding - s->ksize) / s->stride + 1 && s->outA > 0 && s->outB > 0,
-	              "%s: output extent %dx%d does not follow from input %dx%d, k=%d s=%d p=%d", fn, s->outA, s->outB, s->inA,
-	              s->inB, s->ksize, s->stride, s->padding);
-	FITRE_REQUIRE(s->ksize < 256, "%s: window %d too large", fn, s->ksize);
-	double lim = 1073741823.0; /* operands are read through 32-bit byte offsets */
-	FITRE_REQUIRE((double)s->samples * s->inA * s->inB * s->inChannels < lim &&
-	                  (double)s->samples * s->outA * s->outB * s->outChannels < lim &&
-	                  (double)s->inChannels * s->ksize * s->ksize * s->outChannels < lim,
-	              "%s: a tensor exceeds 2^30 elements", fn);
-	return FITRE_OK;
-}
-
-// patches of `src` (srcA x srcB per map) taken on an outA x outB grid
-static PatchGeom make_patch_geom(const float *src, int channels, int samples, int srcA, int srcB, int outA, int outB, int ksize,
-                                 int stride, int pad)
-{
-	PatchGeom g;
-	g.src = src;
-	g.bytes = (uint32_t)((size_t)channels * samples * srcA * srcB * sizeof(float));
-	g.samples = samples;
-	g.srcA = srcA;
-	g.srcB = srcB;
-	g.outA = outA;
-	g.outB = outB;
-	g.ksize = ksize;
-	g.stride = stride;
-	g.pad = pad;
-	g.positions = samples * outA * outB;
-	g.taps = ksize * ksize;
-	g.patchLen = channels * g.taps;
-	g.chanStride = samples * srcA * srcB;
-	g.divOutB = FastDiv((uint32_t)outB);
-	g.divOutA = FastDiv((uint32_t)outA);
-	g.divTaps = FastDiv((uint32_t)g.taps);
-	g.divK = FastDiv((uint32_t)ksize);
-	g.ktable = nullptr;
-	return g;
-}
 
 // Device table of the patch decode, owned by the layer and grown on demand; every use is
 // ordered on the layer's stream.
@@ -76,10 +30,6 @@ static int attach_patch_table(PatchGeom &g, int bn)
 	return check_launch("patch_table_kernel");
 }
 
-static double conv_flops(const fitre_conv_shape *s)
-{
-	return 2.0 * (double)s->samples * s->outA * s->outB * (double)s->inChannels * s->ksize * s->ksize * (double)s->outChannels;
-}
 
 // ---- 3x3 / stride 1 / pad 1 fast paths -------------------------------------------------------
 constexpr int kC3CB = 8; // reduction channels per LDS block of the position-contiguous kernels
@@ -155,16 +105,6 @@ static BlockPlan c3_dw_plan(const fitre_conv_shape *s)
 	return plan_blocks(tiles, (J + kC3Stage - 1) / kC3Stage, stageUs, 2, s->outChannels, (long)s->inChannels * 9);
 }
 
-static void launch_reduce(const float *ws, int splits, int I, int J, const OutParams &fin)
-{
-	LaunchScope scope(FITRE_KC_SPLITK_REDUCE, 4.0 * (double)I * J * (splits + 1));
-	const bool vec = (J % 4 == 0) && ((((uintptr_t)ws) & 15) == 0);
-	if (vec)
-		splitk_reduce_kernel<4><<<blocks_for((long)I * J / 4, 256, 8192), 256, 0, stream()>>>(ws, splits, I, J, fin);
-	else
-		splitk_reduce_kernel<1><<<blocks_for((long)I * J, 256, 8192), 256, 0, stream()>>>(ws, splits, I, J, fin);
-}
-
 template <bool DX>
 static int launch_c3_pos(const fitre_conv_shape *s, const float *src, const float *w, const float *bias, float *outPtr, void *ws,
                          size_t wsBytes)
@@ -213,7 +153,7 @@ static int launch_c3_pos(const fitre_conv_shape *s, const float *src, const floa
 		}
 #undef C3_LAUNCH
 	}
-	if (plan.splits > 1) launch_reduce((const float *)ws, plan.splits, I, J, out);
+	if (plan.splits > 1) launch_splitk_reduce((const float *)ws, plan.splits, I, J, out);
 	return check_launch("conv3x3_pos_kernel");
 }
 
@@ -259,7 +199,7 @@ static int launch_c3_dw(const fitre_conv_shape *s, const float *x, const float *
 		else
 			conv3x3_dw_kernel<false, 64><<<grid, kGemmThreads, 0, stream()>>>(p, delta, deltaBytes, part);
 	}
-	if (plan.splits > 1) launch_reduce((const float *)ws, plan.splits, I, K, out);
+	if (plan.splits > 1) launch_splitk_reduce((const float *)ws, plan.splits, I, K, out);
 	return check_launch("conv3x3_dw_kernel");
 }
 

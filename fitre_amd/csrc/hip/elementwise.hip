@@ -202,14 +202,31 @@ __global__ void __launch_bounds__(256) add_channel_bias_kernel(float *x, long pe
 	long stride = (long)gridDim.x * blockDim.x;
 	for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < perChannel; i += stride) p[i] += b;
 }
-// out[r] = sum_c mat[r + c*rows]  (one wave per row group; rows are the fast index)
+// out[r] = sum_c mat[r + c*rows]  (rows are the fast index).  A workgroup owns 16 rows; its 16
+// column phases each add every 16th column in double, then the phases are combined in a fixed order.
 __global__ void __launch_bounds__(256) row_sum_kernel(const float *mat, int rows, int cols, float *out)
 {
-	int r = blockIdx.x * blockDim.x + threadIdx.x;
-	if (r >= rows) return;
+	__shared__ double part[16][17];
+	const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+	const int r = blockIdx.x * 16 + tx;
 	double acc = 0.0;
-	for (int c = 0; c < cols; c++) acc += (double)mat[(size_t)c * rows + r];
-	out[r] = (float)acc;
+	if (r < rows) {
+		int c = ty;
+		for (; c + 48 < cols; c += 64) { // four loads in flight
+			float v0 = mat[(size_t)c * rows + r], v1 = mat[(size_t)(c + 16) * rows + r];
+			float v2 = mat[(size_t)(c + 32) * rows + r], v3 = mat[(size_t)(c + 48) * rows + r];
+			acc += (double)v0, acc += (double)v1, acc += (double)v2, acc += (double)v3;
+		}
+		for (; c < cols; c += 16) acc += (double)mat[(size_t)c * rows + r];
+	}
+	part[ty][tx] = acc;
+	__syncthreads();
+	if (ty == 0 && r < rows) {
+		double total = 0.0;
+#pragma unroll
+		for (int q = 0; q < 16; q++) total += part[q][tx];
+		out[r] = (float)total;
+	}
 }
 
 } // namespace fitre
@@ -309,7 +326,7 @@ int fitre_hip_row_sum(const float *mat, int rows, int cols, float *out)
 {
 	EW_CHECK("fitre_hip_row_sum", mat && out && rows > 0 && cols > 0);
 	LaunchScope scope(FITRE_KC_BIAS_GRAD, 4.0 * rows * cols);
-	row_sum_kernel<<<blocks_for(rows, 256), 256, 0, stream()>>>(mat, rows, cols, out);
+	row_sum_kernel<<<(rows + 15) / 16, 256, 0, stream()>>>(mat, rows, cols, out);
 	return check_launch("row_sum_kernel");
 }
 

@@ -160,6 +160,7 @@ struct PatchGeom {
 	int taps;        // ksize * ksize
 	int patchLen;    // channels * taps
 	int chanStride;  // samples * srcA * srcB
+	float onesValue; // value of the constant row that PatchKContigOnes appends after the patch rows
 	// Decode of the reduction index k = (c, ta, tb) for the operand whose k is uniform across a
 	// wave: low word c*chanStride + ta*srcB + tb, high word ta << 16 | tb.  Entries are stored in
 	// the order the waves consume them (see patch_table_slot) and read with scalar loads.
@@ -176,7 +177,7 @@ __host__ __device__ inline int patch_table_slot(int k, int bk, int kstep)
 }
 
 // fills PatchGeom::ktable for slices of depth bk read with stride kstep; `padded` entries
-__global__ void patch_table_kernel(unsigned long long *table, int padded, int patchLen, int chanStride, int srcB,
+static __global__ void patch_table_kernel(unsigned long long *table, int padded, int patchLen, int chanStride, int srcB,
                                    FastDiv divTaps, FastDiv divK, int bk, int kstep)
 {
 	int k = blockIdx.x * blockDim.x + threadIdx.x;
@@ -245,9 +246,11 @@ struct PatchRowContig {
 };
 
 // element(row = (c, ta, tb), k = m) of the transposed patch matrix; the reduction
-// index m is the contiguous one.  Used for the weight gradient.
-template <int ROWS, int BK>
-struct PatchKContig {
+// index m is the contiguous one.  Used for the weight gradient and the Kronecker factors.
+// ONES: row patchLen is a constant row (onesValue at every position) -- the bias column
+// of the augmented patch matrix.
+template <int ROWS, int BK, bool ONES>
+struct PatchKContigT {
 	static constexpr int E = ROWS * BK / kGemmThreads;
 	static constexpr int RSTEP = kGemmThreads / BK;
 	static constexpr int LD = LdsStride<ROWS, BK>::value;
@@ -270,6 +273,7 @@ struct PatchKContig {
 			pr.divTaps.divmod(row, c, tap);
 			pr.divK.divmod(tap, ta, tb);
 			rowOff[e] = (row < (uint32_t)pr.patchLen) ? (int)c * pr.chanStride + (int)ta * pr.srcB + (int)tb : -1;
+			if (ONES && row == (uint32_t)pr.patchLen) rowOff[e] = -2;
 			rowTap[e] = (int)((ta << 16) | tb);
 		}
 	}
@@ -287,6 +291,7 @@ struct PatchKContig {
 			int a = a0 + (rowTap[e] >> 16), b = b0 + (rowTap[e] & 0xffff);
 			bool ok = kOk & (rowOff[e] >= 0) & ((unsigned)a < (unsigned)g.srcA) & ((unsigned)b < (unsigned)g.srcB);
 			r[e] = buffer_load(rsrc, ok ? 4u * (uint32_t)(rowOff[e] + base) : kOutOfRange);
+			if (ONES) r[e] = (kOk & (rowOff[e] == -2)) ? g.onesValue : r[e];
 		}
 	}
 	__device__ __forceinline__ void store(float *lds, const float (&r)[E]) const
@@ -295,6 +300,8 @@ struct PatchKContig {
 		for (int e = 0; e < E; e++) lds[kL * LD + rowL + RSTEP * e] = r[e];
 	}
 };
+template <int ROWS, int BK> using PatchKContig = PatchKContigT<ROWS, BK, false>;
+template <int ROWS, int BK> using PatchKContigOnes = PatchKContigT<ROWS, BK, true>;
 
 // Weights as seen by the input gradient: element(row = ci, k = (o, ta, tb)) =
 // w[o][ci][ksize-1-ta][ksize-1-tb]  (w is [Cout][Cin][k][k]).
@@ -355,6 +362,10 @@ struct OutParams {
 	const float *biasI; // added per i (may be null); ignored when split
 	const float *biasJ; // added per j (may be null); ignored when split
 	float alpha, beta;  // C = alpha * acc (+ bias) + beta * C; ignored when split
+	// Symmetric product (both operands are the same matrix, I == J): tiles entirely below the
+	// diagonal are skipped, elements with j < i are not stored and every stored element with
+	// j > i is also written to C[j][i].  With split-K the mirroring happens in the reduction.
+	int mirror;
 };
 
 // ---------------------------------------------------------------------------
@@ -377,6 +388,7 @@ mfma_gemm_kernel(const typename OpA::Params pa, const typename OpB::Params pb, c
 	const int i0 = blockIdx.y * BM, j0 = blockIdx.x * BN;
 	const int kbeg = blockIdx.z * kChunk;
 	const int kend = (kbeg + kChunk < R) ? kbeg + kChunk : R;
+	if (out.mirror && j0 + BN <= i0) return; // the mirror tile produces these elements
 
 	OpA opA;
 	OpB opB;
@@ -452,6 +464,7 @@ mfma_gemm_kernel(const typename OpA::Params pa, const typename OpB::Params pb, c
 			for (int v = 0; v < 16; v++) {
 				const int i = i0 + (wave >> 1) * Cfg::WM + tm * 32 + 8 * (v / 4) + 4 * khalf + (v % 4);
 				if (i >= I) continue;
+				if (out.mirror && j < i) continue;
 				float val = acc[tm][tn][v];
 				float *dst = C + (size_t)i * out.ldc + j;
 				if (!split) {
@@ -459,6 +472,7 @@ mfma_gemm_kernel(const typename OpA::Params pa, const typename OpB::Params pb, c
 					if (out.biasI) val += out.biasI[i];
 					if (out.biasJ) val += out.biasJ[j];
 					if (out.beta != 0.f) val += out.beta * *dst;
+					if (out.mirror && j > i) C[(size_t)j * out.ldc + i] = val; // bias and beta are not used with mirror
 				}
 				*dst = val;
 			}
@@ -509,13 +523,81 @@ splitk_reduce_kernel(const float *ws, int splits, int I, int J, OutParams out)
 		}
 #pragma unroll
 		for (int v = 0; v < VEC; v++) {
+			if (out.mirror && j + v < i) continue; // no partials below the diagonal
 			float val = (float)acc[v] * out.alpha;
 			if (out.biasI) val += out.biasI[i];
 			if (out.biasJ) val += out.biasJ[j + v];
 			float *dst = out.C + (size_t)i * out.ldc + j + v;
 			if (out.beta != 0.f) val += out.beta * *dst;
 			*dst = val;
+			if (out.mirror && j + v > i) out.C[(size_t)(j + v) * out.ldc + i] = val;
 		}
+	}
+}
+
+// The same sum for a SMALL output with MANY partials (a weight gradient of a thin layer): a
+// workgroup owns 16 output groups, its 16 phases each add every 16th partial, and the phases are
+// combined in a fixed order -- the parallelism comes from the partials, not from the output.
+template <int VEC>
+__global__ void __launch_bounds__(256)
+splitk_reduce_wide_kernel(const float *ws, int splits, int I, int J, OutParams out)
+{
+	__shared__ double part[16][16 * VEC + 1];
+	const long total = (long)I * J;
+	const long groups = total / VEC;
+	const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+	const long gidx = (long)blockIdx.x * 16 + tx;
+	double acc[VEC];
+#pragma unroll
+	for (int v = 0; v < VEC; v++) acc[v] = 0.0;
+	if (gidx < groups) {
+		const float *p = ws + gidx * VEC;
+		for (int s = ty; s < splits; s += 16) {
+			if constexpr (VEC == 4) {
+				float4 t = *reinterpret_cast<const float4 *>(p + (size_t)s * total);
+				acc[0] += (double)t.x, acc[1] += (double)t.y, acc[2] += (double)t.z, acc[3] += (double)t.w;
+			} else {
+				acc[0] += (double)p[(size_t)s * total];
+			}
+		}
+	}
+#pragma unroll
+	for (int v = 0; v < VEC; v++) part[ty][tx * VEC + v] = acc[v];
+	__syncthreads();
+	if (ty == 0 && gidx < groups) {
+		const long idx = gidx * VEC;
+		const int i = (int)(idx / J), j = (int)(idx - (long)i * J);
+#pragma unroll
+		for (int v = 0; v < VEC; v++) {
+			if (out.mirror && j + v < i) continue;
+			double sum = 0.0;
+#pragma unroll
+			for (int q = 0; q < 16; q++) sum += part[q][tx * VEC + v];
+			float val = (float)sum * out.alpha;
+			if (out.biasI) val += out.biasI[i];
+			if (out.biasJ) val += out.biasJ[j + v];
+			float *dst = out.C + (size_t)i * out.ldc + j + v;
+			if (out.beta != 0.f) val += out.beta * *dst;
+			*dst = val;
+			if (out.mirror && j + v > i) out.C[(size_t)(j + v) * out.ldc + i] = val;
+		}
+	}
+}
+
+// Sums `splits` partial I x J matrices from ws into fin (alpha, beta and biases applied once).
+static inline void launch_splitk_reduce(const float *ws, int splits, int I, int J, const OutParams &fin)
+{
+	LaunchScope scope(FITRE_KC_SPLITK_REDUCE, 4.0 * (double)I * J * (splits + 1));
+	const bool vec = (J % 4 == 0) && ((((uintptr_t)ws) & 15) == 0);
+	const long groups = (long)I * J / (vec ? 4 : 1);
+	const bool wide = splits >= 32 && groups <= 64 * 1024; // too few outputs to fill the chip one thread each
+	if (wide) {
+		const unsigned blocks = (unsigned)((groups + 15) / 16);
+		if (vec) splitk_reduce_wide_kernel<4><<<blocks, 256, 0, stream()>>>(ws, splits, I, J, fin);
+		else splitk_reduce_wide_kernel<1><<<blocks, 256, 0, stream()>>>(ws, splits, I, J, fin);
+	} else {
+		if (vec) splitk_reduce_kernel<4><<<blocks_for(groups, 256, 8192), 256, 0, stream()>>>(ws, splits, I, J, fin);
+		else splitk_reduce_kernel<1><<<blocks_for(groups, 256, 8192), 256, 0, stream()>>>(ws, splits, I, J, fin);
 	}
 }
 
@@ -553,12 +635,17 @@ inline double estimate_us(long tiles, int bm, int bn, long I, long J, long R, lo
 	return t;
 }
 
-inline GemmPlan plan_gemm(long I, long J, long R)
+// mirror: a symmetric product (I == J) that only computes the tiles on and above the diagonal
+inline GemmPlan plan_gemm(long I, long J, long R, bool mirror = false)
 {
 	GemmPlan p;
 	p.bm = (I <= 64) ? 64 : 128;
 	p.bn = (J <= 64) ? 64 : 128;
 	long tiles = ((I + p.bm - 1) / p.bm) * ((J + p.bn - 1) / p.bn);
+	if (mirror) {
+		long t = (I + p.bm - 1) / p.bm;
+		tiles = t * (t + 1) / 2;
+	}
 	long maxSplits = R / (2 * kGemmBK); // at least two slices per split
 	if (maxSplits > 1024) maxSplits = 1024;
 	if (maxSplits < 1) maxSplits = 1;
@@ -618,12 +705,7 @@ static int launch_tile(const typename OpA<BM, kGemmBK>::Params &pa, const typena
 		}
 		OutParams fin = out;
 		fin.splitStride = 0;
-		LaunchScope scope(FITRE_KC_SPLITK_REDUCE, 4.0 * (double)I * J * (plan.splits + 1));
-		const bool vec = (J % 4 == 0) && ((((uintptr_t)ws) & 15) == 0);
-		if (vec)
-			splitk_reduce_kernel<4><<<blocks_for((long)I * J / 4, 256, 8192), 256, 0, stream()>>>((const float *)ws, plan.splits, I, J, fin);
-		else
-			splitk_reduce_kernel<1><<<blocks_for((long)I * J, 256, 8192), 256, 0, stream()>>>((const float *)ws, plan.splits, I, J, fin);
+		launch_splitk_reduce((const float *)ws, plan.splits, I, J, fin);
 	} else {
 		OutParams direct = out;
 		direct.splitStride = 0;

@@ -83,6 +83,12 @@ HIP_API = {
     "fitre_hip_conv_input_grad": (i32, [pshape, vp, vp, vp, vp, sz]),
     "fitre_hip_gemm_workspace": (sz, [i32, i32, i32]),
     "fitre_hip_gemm": (i32, [i32, i32, i32, i32, i32, f32, vp, i32, vp, i32, f32, vp, i32, vp, vp, sz]),
+    "fitre_hip_kfac_conv_input_factor_workspace": (sz, [vp, i32]),
+    "fitre_hip_kfac_conv_input_factor": (i32, [vp, vp, i32, vp, vp, sz]),
+    "fitre_hip_kfac_gram_workspace": (sz, [i32, C.c_long]),
+    "fitre_hip_kfac_conv_output_factor": (i32, [vp, vp, vp, vp, sz]),
+    "fitre_hip_kfac_fc_input_factor": (i32, [vp, i32, i32, i32, vp, vp, sz]),
+    "fitre_hip_kfac_fc_output_factor": (i32, [vp, i32, i32, vp, vp, sz]),
 }
 
 pconv, ppool = C.POINTER(CONV_LAYER), C.POINTER(POOL_LAYER)

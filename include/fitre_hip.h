@@ -222,6 +222,32 @@ int fitre_hip_gemm(int transA, int transB, int M, int N, int K, float alpha, con
                    const float *B, int ldb, float beta, float *C, int ldc, const float *bias, void *ws,
                    size_t wsBytes);
 
+/* ---- Kronecker factors of the KFAC curvature approximation --------------------------------------
+ * Each factor is a dense symmetric matrix, written in full (row-major == column-major).  The
+ * products are symmetric, so only the tiles on and above the diagonal are computed.
+ *
+ * Convolution, input side (solvers/kfac_inverses.cu:489-540): A = P^T P / samples with
+ * P = [ im2col(x) / (outA*outB) , 1 ], order Cin*k*k (+1 with bias); patch column order
+ * (c, ta, tb) as in the weight layout.  The patch matrix is not materialised. */
+size_t fitre_hip_kfac_conv_input_factor_workspace(const fitre_conv_shape *s, int withBias);
+int fitre_hip_kfac_conv_input_factor(const fitre_conv_shape *s, const float *x, int withBias, float *factor,
+                                     void *ws, size_t wsBytes);
+/* Workspace of the three factors below: order = matrix order, reduce = length of the sum
+ * (positions = samples*outA*outB for a convolution, samples for a fully connected layer). */
+size_t fitre_hip_kfac_gram_workspace(int order, long reduce);
+/* Convolution, output side (kfac_inverses.cu:806-816): G = D^T D * (samples*outA*outB), D = delta
+ * [Cout][samples*outA*outB] seen as positions x Cout; order Cout. */
+int fitre_hip_kfac_conv_output_factor(const fitre_conv_shape *s, const float *delta, float *factor, void *ws,
+                                      size_t wsBytes);
+/* Fully connected, input side (kfac_inverses.cu:596-625): A = Z Z^T / samples, Z = [ z ; 1 ] with z
+ * column-major in x samples; order in (+1 with bias).  Workspace: fitre_hip_kfac_gram_workspace(in, samples). */
+int fitre_hip_kfac_fc_input_factor(const float *z, int in, int samples, int withBias, float *factor, void *ws,
+                                   size_t wsBytes);
+/* Fully connected, output side (kfac_inverses.cu:838-852): G = D D^T * samples, D = delta column-major
+ * out x samples; order out. */
+int fitre_hip_kfac_fc_output_factor(const float *delta, int out, int samples, float *factor, void *ws,
+                                    size_t wsBytes);
+
 #ifdef __cplusplus
 }
 #endif

@@ -630,6 +630,67 @@ void oracle_conv_input_gradient(const real *delta, int dHeight, int dWidth, int 
 }
 
 /* ------------------------------------------------------------------ */
+/* KFAC Kronecker factors (the products only; inverses are not restated) */
+/* ------------------------------------------------------------------ */
+
+/* solvers/kfac_inverses.cu:489-540 (computeOmegaZ, convolution layers): patch matrix scaled by
+ * 1/(outHeight*outWidth), a column of ones when the model has a bias, Z^T Z, then 1/samples.
+ * factor is zCols x zCols column-major (symmetric); devScratch holds zRows*zCols reals. */
+void oracle_kfac_conv_input_factor(const real *input, int samples, int in_channels, int height, int width,
+                                   int ksize, int pad, int stride, int bias, real *factor, real *devScratch)
+{
+	int col_h = (height + 2 * pad - ksize) / stride + 1;
+	int col_w = (width + 2 * pad - ksize) / stride + 1;
+	int zRows = samples * col_h * col_w;
+	int zCols = in_channels * ksize * ksize + (bias ? 1 : 0);
+	real *expanded = devScratch;
+	oracle_im2col(input, samples, in_channels, height, width, ksize, pad, stride, expanded);
+	real alpha = (real)1 / (real)(col_h * col_w);
+	size_t scaled = (size_t)zRows * (bias ? zCols - 1 : zCols);
+	for (size_t i = 0; i < scaled; i++) expanded[i] *= alpha;
+	if (bias)
+		for (int i = 0; i < zRows; i++) expanded[(size_t)zRows * (zCols - 1) + i] = 1;
+	oracle_gemm(OP_T, OP_N, zCols, zCols, zRows, 1, expanded, zRows, expanded, zRows, 0, factor, zCols);
+	alpha = (real)1 / (real)samples;
+	for (size_t i = 0; i < (size_t)zCols * zCols; i++) factor[i] *= alpha;
+}
+
+/* solvers/kfac_inverses.cu:782-816 (computeLambdaDelta, convolution layers): delta is
+ * (samples*outHeight*outWidth) x outChannels column-major; G = delta^T delta scaled by the row count. */
+void oracle_kfac_conv_output_factor(const real *delta, int samples, int out_height, int out_width,
+                                    int out_channels, real *factor)
+{
+	int rows = samples * out_height * out_width;
+	oracle_gemm(OP_T, OP_N, out_channels, out_channels, rows, 1, delta, rows, delta, rows, 0, factor, out_channels);
+	real alpha = (real)out_height * (real)out_width * (real)samples;
+	for (size_t i = 0; i < (size_t)out_channels * out_channels; i++) factor[i] *= alpha;
+}
+
+/* solvers/kfac_inverses.cu:596-625 (computeOmegaZ, linear layers): z is in x samples column-major,
+ * a row of ones is appended when the model has a bias; A = Z (Z/samples)^T.
+ * devScratch holds 2*zRows*samples reals. */
+void oracle_kfac_fc_input_factor(const real *z, int in, int samples, int bias, real *factor, real *devScratch)
+{
+	int zRows = in + (bias ? 1 : 0);
+	real *zMatrix = devScratch, *scaledZ = devScratch + (size_t)zRows * samples;
+	for (int n = 0; n < samples; n++) {
+		for (int r = 0; r < in; r++) zMatrix[(size_t)n * zRows + r] = z[(size_t)n * in + r];
+		if (bias) zMatrix[(size_t)n * zRows + in] = 1;
+	}
+	real alpha = (real)1 / (real)samples;
+	for (size_t i = 0; i < (size_t)zRows * samples; i++) scaledZ[i] = zMatrix[i] * alpha;
+	oracle_gemm(OP_N, OP_T, zRows, zRows, samples, 1, zMatrix, zRows, scaledZ, zRows, 0, factor, zRows);
+}
+
+/* solvers/kfac_inverses.cu:838-852 (computeLambdaDelta, linear layers): delta is out x samples
+ * column-major; G = delta delta^T scaled by samples. */
+void oracle_kfac_fc_output_factor(const real *delta, int out, int samples, real *factor)
+{
+	oracle_gemm(OP_N, OP_T, out, out, samples, 1, delta, out, delta, out, 0, factor, out);
+	for (size_t i = 0; i < (size_t)out * out; i++) factor[i] *= (real)samples;
+}
+
+/* ------------------------------------------------------------------ */
 /* whole model                                                         */
 /* ------------------------------------------------------------------ */
 

@@ -128,6 +128,37 @@ class Oracle:
                                             samples, self.p(out), self.p(scratch))
         return out
 
+    # ---- KFAC factors ---------------------------------------------------
+    def kfac_conv_input_factor(self, x, samples, cin, height, width, k, pad, stride, bias):
+        x = self.arr(x)
+        hc, wc = (height + 2 * pad - k) // stride + 1, (width + 2 * pad - k) // stride + 1
+        n = cin * k * k + (1 if bias else 0)
+        factor = self.zeros(n * n)
+        scratch = self.zeros(hc * wc * samples * n)
+        self.lib.oracle_kfac_conv_input_factor(self.p(x), samples, cin, height, width, k, pad, stride, int(bool(bias)),
+                                               self.p(factor), self.p(scratch))
+        return factor.reshape(n, n)
+
+    def kfac_conv_output_factor(self, delta, samples, out_height, out_width, cout):
+        delta = self.arr(delta)
+        factor = self.zeros(cout * cout)
+        self.lib.oracle_kfac_conv_output_factor(self.p(delta), samples, out_height, out_width, cout, self.p(factor))
+        return factor.reshape(cout, cout)
+
+    def kfac_fc_input_factor(self, z, n_in, samples, bias):
+        z = self.arr(z)
+        n = n_in + (1 if bias else 0)
+        factor = self.zeros(n * n)
+        scratch = self.zeros(2 * n * samples)
+        self.lib.oracle_kfac_fc_input_factor(self.p(z), n_in, samples, int(bool(bias)), self.p(factor), self.p(scratch))
+        return factor.reshape(n, n)
+
+    def kfac_fc_output_factor(self, delta, n_out, samples):
+        delta = self.arr(delta)
+        factor = self.zeros(n_out * n_out)
+        self.lib.oracle_kfac_fc_output_factor(self.p(delta), n_out, samples, self.p(factor))
+        return factor.reshape(n_out, n_out)
+
     def activation_forward(self, act, x):
         x = self.arr(x).copy()
         rc = self.lib.oracle_activation_forward(act, self.p(x), C.c_size_t(x.size))

@@ -292,3 +292,62 @@ def test_reshape_and_transposes(oracle64):
     t = oracle64.transpose(m, 2, 3, 5).reshape(2, 3, 5)
     np.testing.assert_array_equal(t, m.reshape(2, 5, 3).transpose(0, 2, 1))
     np.testing.assert_array_equal(oracle64.transpose(t.reshape(-1), 2, 3, 5, rc=True), m)
+
+
+# ------------------------------------------------------------------ KFAC factors
+def unfold_patches(x_nchw, k, pad, stride):
+    """(N*L) x (C*k*k) patch matrix from the library unfold, columns re-ordered from torch's
+    (c, kh, kw) to the weight layout's (c, window column, window row); pytorch/testing/test_expanded.py:13-35
+    builds the same matrix and forms exp^T exp."""
+    N, C = x_nchw.shape[:2]
+    u = F.unfold(x_nchw, k, padding=pad, stride=stride)                    # N, C*k*k, L
+    u = u.reshape(N, C, k, k, -1).permute(0, 4, 1, 3, 2).reshape(-1, C * k * k)  # rows (n, l); cols (c, kw, kh)
+    return u.numpy()
+
+
+@pytest.mark.parametrize("case", [(3, 2, 5, 4, 3, 1, 1, True), (2, 3, 6, 6, 3, 0, 1, False), (2, 1, 7, 5, 2, 1, 2, True),
+                                  (1, 2, 4, 4, 5, 2, 1, True)])
+def test_kfac_conv_input_factor_against_unfold(oracle64, case):
+    N, C, H, W, k, pad, stride, bias = case
+    rng = np.random.default_rng(11)
+    xt = torch.from_numpy(rng.standard_normal((N, C, H, W)))
+    OH, OW = (H + 2 * pad - k) // stride + 1, (W + 2 * pad - k) // stride + 1
+    P = unfold_patches(xt, k, pad, stride) / (OH * OW)
+    if bias:
+        P = np.concatenate([P, np.ones((P.shape[0], 1))], axis=1)
+    want = P.T @ P / N
+    got = oracle64.kfac_conv_input_factor(from_nchw(xt), N, C, H, W, k, pad, stride, bias)
+    np.testing.assert_allclose(got, want, atol=1e-13)
+    np.testing.assert_allclose(got, got.T, atol=0)
+    assert np.linalg.eigvalsh(got).min() > -1e-12
+    if bias:
+        assert abs(got[-1, -1] - OH * OW) < 1e-12  # ones^T ones / N
+
+
+def test_kfac_conv_input_factor_closed_form_for_constant_image(oracle64):
+    # x = 1 without padding: every patch entry is 1, so each patch-patch entry is
+    # (1/L)^2 * N*L / N = 1/L, each patch-bias entry is 1 and the corner is L  (L = OH*OW)
+    N, C, H, W, k = 3, 2, 6, 5, 3
+    L = (H - k + 1) * (W - k + 1)
+    got = oracle64.kfac_conv_input_factor(np.ones(N * C * H * W), N, C, H, W, k, 0, 1, True)
+    K = C * k * k
+    np.testing.assert_allclose(got[:K, :K], 1.0 / L, atol=1e-14)
+    np.testing.assert_allclose(got[K, :K], 1.0, atol=1e-14)
+    assert abs(got[K, K] - L) < 1e-12
+
+
+def test_kfac_output_and_fc_factors_against_numpy(oracle64):
+    rng = np.random.default_rng(12)
+    N, Cout, OH, OW = 3, 4, 2, 5
+    d = rng.standard_normal((Cout, N * OH * OW))               # [Cout][N][OW][OH] flattened
+    got = oracle64.kfac_conv_output_factor(d.reshape(-1), N, OH, OW, Cout)
+    np.testing.assert_allclose(got, d @ d.T * (N * OH * OW), atol=1e-11)
+    n_in, n_out = 5, 3
+    z = rng.standard_normal((N, n_in))                         # column-major in x N: sample-major memory
+    for bias in (False, True):
+        Z = np.concatenate([z, np.ones((N, 1))], axis=1) if bias else z
+        got = oracle64.kfac_fc_input_factor(z.reshape(-1), n_in, N, bias)
+        np.testing.assert_allclose(got, Z.T @ Z / N, atol=1e-13)
+    dl = rng.standard_normal((N, n_out))
+    got = oracle64.kfac_fc_output_factor(dl.reshape(-1), n_out, N)
+    np.testing.assert_allclose(got, dl.T @ dl * N, atol=1e-12)
