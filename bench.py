@@ -98,6 +98,7 @@ def gpu_leg(args):
     rows = read_profile(L)
     grad = gm.get("grad")
     finite = bool(np.isfinite(grad).all() and np.isfinite(loss))
+    kfac = kfac_leg(L, dev, gm, model, batch, max(2, args.steps // 4))
     gm.release()
     dev.close()
 
@@ -128,7 +129,48 @@ def gpu_leg(args):
     conv["frac"] = round(conv["achieved"] / PEAK_MFMA_F32_TFLOPS, 4)
     return dict(wall=wall, ms_events=ms_events.value, batch=batch, loss=loss, finite=finite,
                 device=name.value.decode(), compute_units=cus.value, roofline=roofline, kernels=kernels,
-                conv_backward_gemms=conv)
+                conv_backward_gemms=conv, kfac_factors=kfac)
+
+
+def kfac_leg(L, dev, gm, model, batch, passes):
+    """Kronecker factors of every layer from the z / dx the backward pass left behind (not part of the
+    images/sec metric): computeOmegaZFactors + computeLambdaDeltaFactors, `passes` times."""
+    from fitre_amd.structs import KFAC_CURVATURE_INFO
+
+    info = KFAC_CURVATURE_INFO()
+    L.cnn.computeKFACStorageIndices(C.byref(model), C.byref(info))
+    last = model.cLayers + model.lLayers
+    omega = dev.zeros(info.OmegaZOffsets[last])
+    lam = dev.zeros(info.LambdaGOffsets[last])
+    ws = dev.alloc(4 * L.cnn.kfacFactorsMemRequired(C.byref(model), batch))
+
+    def run():
+        L.cnn.computeOmegaZFactors(C.byref(info), C.byref(model), C.byref(gm.data), batch, None, gm.z, omega,
+                                   model.zOffsets, model.zztOffsets, ws)
+        L.cnn.computeLambdaDeltaFactors(C.byref(info), C.byref(model), batch, gm.dx, None, lam, model.zOffsets,
+                                        model.zztOffsets, ws)
+
+    run()
+    dev.sync()
+    t0 = time.perf_counter()
+    for _ in range(passes):
+        run()
+    dev.sync()
+    wall_ms = 1e3 * (time.perf_counter() - t0) / passes
+    L.check(L.hip.fitre_hip_profile_enable(1))  # resets the tables
+    for _ in range(passes):
+        run()
+    dev.sync()
+    L.check(L.hip.fitre_hip_profile_enable(0))
+    rows = [r for r in read_profile(L) if r["cls"] == "kfac_factor"]
+    ms, work = sum(r["ms"] for r in rows), sum(r["work"] for r in rows)
+    for q in (omega, lam, ws):
+        dev.free(q)
+    rate = work / (ms * 1e-3) / 1e12 if ms else 0.0
+    return dict(ms_per_pass=round(wall_ms, 4), kernel_ms_per_pass=round(ms / passes, 4),
+                gflop_per_pass=round(work / passes / 1e9, 2), achieved=round(rate, 2), unit="TFLOP/s",
+                frac=round(rate / PEAK_MFMA_F32_TFLOPS, 4),
+                note="upper-triangle flops n(n+1)*positions; all %d layers, both sides" % last)
 
 
 def cpu_leg(batch=64, repeats=10):
@@ -202,6 +244,7 @@ def main():
                    "batch": g["batch"], "device": g["device"], "compute_units": g["compute_units"]},
         "roofline": g["roofline"],
         "conv_backward_gemms": g["conv_backward_gemms"],
+        "kfac_factors": g["kfac_factors"],
         "kernels": g["kernels"],
         "wall_ms_per_step": round(1e3 * g["wall"] / args.steps, 4),
         "loss": round(g["loss"], 6),

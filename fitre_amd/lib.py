@@ -6,7 +6,8 @@ import fails with the reason.  Build with ``python -m fitre_amd.build``.
 import ctypes as C
 import os
 
-from .structs import (CNN_MODEL, CONV_LAYER, DEVICE_DATASET, POOL_LAYER, SCRATCH_AREA, fitre_conv_shape)
+from .structs import (CNN_MODEL, CONV_LAYER, DEVICE_DATASET, KFAC_CURVATURE_INFO, POOL_LAYER, SCRATCH_AREA,
+                      fitre_conv_shape)
 
 _PKG = os.path.dirname(os.path.abspath(__file__))
 HIP_LIB_PATH = os.path.join(_PKG, "libfitre_hip.so")
@@ -16,6 +17,7 @@ vp, i32, f32, lng, sz = C.c_void_p, C.c_int, C.c_float, C.c_long, C.c_size_t
 pvp, pi32, pf32 = C.POINTER(C.c_void_p), C.POINTER(C.c_int), C.POINTER(C.c_float)
 pshape = C.POINTER(fitre_conv_shape)
 pmodel, pdata, pscratch = C.POINTER(CNN_MODEL), C.POINTER(DEVICE_DATASET), C.POINTER(SCRATCH_AREA)
+pkfac = C.POINTER(KFAC_CURVATURE_INFO)
 
 # name -> (restype, argtypes); mirrors include/fitre_hip.h
 HIP_API = {
@@ -112,6 +114,11 @@ CNN_API = {
     "cnnBackward": (None, [pmodel, pdata, vp, vp, vp, vp, vp, vp, i32, i32, vp]),
     "evaluateCNNModel": (f32, [pmodel, pdata, pscratch, vp, vp, vp, i32, i32]),
     "computeCNNGradient": (f32, [pmodel, pdata, pscratch, vp, vp, vp, vp, vp, i32, i32, f32]),
+    # include/fitre_kfac.h
+    "computeKFACStorageIndices": (None, [pmodel, pkfac]),
+    "kfacFactorsMemRequired": (lng, [pmodel, i32]),
+    "computeOmegaZFactors": (None, [pkfac, pmodel, pdata, i32, vp, vp, vp, pi32, pi32, vp]),
+    "computeLambdaDeltaFactors": (None, [pkfac, pmodel, i32, vp, vp, vp, pi32, pi32, vp]),
     "getDeviceParameters": (None, []),
     "fitre_env_init": (None, [pscratch, i32, sz]),
     "cuda_env_init": (None, [pscratch, i32]),

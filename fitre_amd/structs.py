@@ -82,6 +82,17 @@ class DEVICE_DATASET(C.Structure):
     ]
 
 
+class KFAC_CURVATURE_INFO(C.Structure):
+    """include/fitre_kfac.h (solvers/kfac_structs.h:13-52 of the reference)."""
+    _fields_ = ([(n, C.c_void_p) for n in ("OmegaZZT", "LambdaGGT", "OmegaZInv", "LambdaGInv", "vec", "nGradient",
+                                           "gradient")] +
+                [("OmegaZOffsets", C.c_int * MAX_LAYERS), ("LambdaGOffsets", C.c_int * MAX_LAYERS)] +
+                [(n, C.c_float) for n in ("stats_decay", "momentum", "regLambda", "dampGamma")] +
+                [("checkGrad", C.c_int), ("dampedInputSize", C.c_int)] +
+                [(n, C.c_void_p) for n in ("dampedInput", "dampedZ", "dampedLambda")] +
+                [("inverseFreq", C.c_int)])
+
+
 class fitre_conv_shape(C.Structure):
     _fields_ = [(n, C.c_int) for n in (
         "samples", "inChannels", "outChannels", "inA", "inB", "outA", "outB", "ksize", "stride", "padding")]

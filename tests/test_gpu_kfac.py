@@ -101,3 +101,77 @@ def test_factor_argument_errors(dev):
     assert hip.fitre_hip_kfac_conv_input_factor(C.byref(shape), None, 1, None, None, 0) == 2
     assert hip.fitre_hip_kfac_fc_input_factor(None, 4, 4, 1, None, None, 0) == 2
     assert hip.fitre_hip_kfac_fc_output_factor(None, 0, 4, None, None, 0) == 2
+
+
+# ---------------------------------------------------------------------------- model level
+def _model_cases():
+    from fitre_amd.structs import AVG_POOL, CNN_ACT_NONE, CNN_ACT_RELU, CNN_ACT_SWISH, MAX_POOL
+    from helpers import build_custom, build_lenet
+    yield "lenet_bias", build_lenet(16, bias=1, bn=False), 16
+    yield "small_vgg_bn", build_custom(12, 8, 8, 3, [dict(cout=6, k=3, pad=1, pool=(MAX_POOL, 2, 2, 0), bn=True, act=CNN_ACT_RELU),
+                                                      dict(cout=9, k=3, pad=1, pool=None, bn=True, act=CNN_ACT_SWISH),
+                                                      dict(cout=5, k=3, pad=1, pool=(MAX_POOL, 2, 2, 0), bn=False, act=CNN_ACT_RELU)],
+                                       [(7, CNN_ACT_NONE)], bias=1), 12
+    yield "no_bias", build_custom(5, 6, 6, 2, [dict(cout=4, k=3, pad=0, pool=(AVG_POOL, 2, 2, 0), bn=False, act=CNN_ACT_SWISH)],
+                                  [(6, CNN_ACT_SWISH), (3, CNN_ACT_NONE)], bias=0), 5
+
+
+@pytest.mark.parametrize("name", ["lenet_bias", "small_vgg_bn", "no_bias"])
+def test_model_factor_passes(dev, oracle64, name):
+    """computeOmegaZFactors / computeLambdaDeltaFactors after a forward and a backward pass: every layer's
+    factor against the oracle's factor of the same z / dx contents, at the offsets of computeKFACStorageIndices."""
+    from fitre_amd.structs import KFAC_CURVATURE_INFO
+    from helpers import GpuModel, batch_inputs, he_weights
+    model, batch = next((m, b) for n, m, b in _model_cases() if n == name)
+    rng = np.random.default_rng(sum(map(ord, name)))
+    w = he_weights(model, rng).astype(np.float32)
+    x, y = batch_inputs(model, batch, rng)
+    x = x.astype(np.float32)
+    gm = GpuModel(dev, model, w, x, y, batch)
+    gm.forward()
+    gm.backward()
+    z, dxs = gm.get("z"), gm.get("dx")
+    info = KFAC_CURVATURE_INFO()
+    L.cnn.computeKFACStorageIndices(C.byref(model), C.byref(info))
+    nc, nl = model.cLayers, model.lLayers
+    tot_o, tot_l = info.OmegaZOffsets[nc + nl], info.LambdaGOffsets[nc + nl]
+    omega = dev.upload(np.full(tot_o, np.nan, dtype=np.float32))
+    lam = dev.upload(np.full(tot_l, np.nan, dtype=np.float32))
+    ws = dev.alloc(4 * L.cnn.kfacFactorsMemRequired(C.byref(model), batch))
+    L.cnn.computeOmegaZFactors(C.byref(info), C.byref(model), C.byref(gm.data), batch, None, gm.z, omega, model.zOffsets,
+                               model.zztOffsets, ws)
+    L.cnn.computeLambdaDeltaFactors(C.byref(info), C.byref(model), batch, gm.dx, None, lam, model.zOffsets, model.zztOffsets, ws)
+    got_o, got_l = dev.download(omega, tot_o), dev.download(lam, tot_l)
+    bias = model.bias != 0
+    zo = model.zOffsets
+    for l in range(nc):
+        c = model.convLayer[l]
+        if l == 0:
+            src = x.reshape(-1)
+        else:
+            prev = model.convLayer[l - 1]
+            start = zo[l] + prev.outputOffset
+            src = z[start:start + c.inChannels * batch * c.height * c.width]
+        n = c.inChannels * c.kSize ** 2 + (1 if bias else 0)
+        want = oracle64.kfac_conv_input_factor(src, batch, c.inChannels, c.height, c.width, c.kSize, c.padding, c.stride, bias)
+        got = got_o[info.OmegaZOffsets[l]:info.OmegaZOffsets[l] + n * n].reshape(n, n)
+        assert rel_err(got, want) < TOL, ("omega conv", l)
+        off = zo[l + 1] + (c.batchNormOffset if c.batchNorm else c.activationOffset)
+        count = c.outChannels * batch * c.outHeight * c.outWidth
+        want = oracle64.kfac_conv_output_factor(dxs[off:off + count], batch, c.outHeight, c.outWidth, c.outChannels)
+        got = got_l[info.LambdaGOffsets[l]:info.LambdaGOffsets[l] + c.outChannels ** 2].reshape(c.outChannels, -1)
+        assert rel_err(got, want) < TOL, ("lambda conv", l)
+    for l in range(nl):
+        f = model.fcLayer[l]
+        start = zo[nc] + model.convLayer[nc - 1].outputOffset if l == 0 else zo[nc + l]
+        n = f.in_ + (1 if bias else 0)
+        want = oracle64.kfac_fc_input_factor(z[start:start + f.in_ * batch], f.in_, batch, bias)
+        got = got_o[info.OmegaZOffsets[nc + l]:info.OmegaZOffsets[nc + l] + n * n].reshape(n, n)
+        assert rel_err(got, want) < TOL, ("omega fc", l)
+        start = zo[nc + l + 1]
+        want = oracle64.kfac_fc_output_factor(dxs[start:start + f.out * batch], f.out, batch)
+        got = got_l[info.LambdaGOffsets[nc + l]:info.LambdaGOffsets[nc + l] + f.out ** 2].reshape(f.out, -1)
+        assert rel_err(got, want) < TOL, ("lambda fc", l)
+    for q in (omega, lam, ws):
+        dev.free(q)
+    gm.release()
