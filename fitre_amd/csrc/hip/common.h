@@ -13,7 +13,8 @@ constexpr int kWave = 64;
 // ---- status -------------------------------------------------------------
 void set_error(const char *fmt, ...);
 int fail(int code, const char *fmt, ...);
-hipStream_t stream();
+hipStream_t stream(); // the selected lane
+int lane();           // its index (0 or 1)
 bool ready();
 
 #define FITRE_HIP_TRY(expr)                                                                          \

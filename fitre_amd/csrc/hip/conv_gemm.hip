@@ -7,14 +7,16 @@ namespace fitre {
 
 // Device table of the patch decode, owned by the layer and grown on demand; every use is
 // ordered on the layer's stream.
-static unsigned long long *g_ktable = nullptr;
-static int g_ktable_cap = 0;
+static unsigned long long *g_ktables[2] = { nullptr, nullptr }; // one per lane
+static int g_ktable_caps[2] = { 0, 0 };
 
 // bn = tile extent along the positions, which fixes how the waves stride through a slice
 static int attach_patch_table(PatchGeom &g, int bn)
 {
 	const int kstep = kGemmThreads / bn;
 	const int padded = ((g.patchLen + kGemmBK - 1) / kGemmBK) * kGemmBK;
+	unsigned long long *&g_ktable = g_ktables[lane()];
+	int &g_ktable_cap = g_ktable_caps[lane()];
 	if (padded > g_ktable_cap) {
 		FITRE_HIP_TRY(hipStreamSynchronize(stream()));
 		if (g_ktable) FITRE_HIP_TRY(hipFree(g_ktable));

@@ -1,6 +1,8 @@
 // Environment, memory and timing entry points of the device layer.
 // Replaces device/cuda_environment.c, device/cuda_utils.c and device/query.c
-// of the reference (handles become one stream owned by this file).
+// of the reference (handles become two streams -- "lanes" -- owned by this file:
+// everything is queued on the selected lane, lane 0 unless a caller overlaps
+// independent work on lane 1).
 #include <stdarg.h>
 #include <string.h>
 #include <vector>
@@ -9,7 +11,13 @@
 namespace fitre {
 
 static thread_local char g_error[512] = "";
-static hipStream_t g_stream = nullptr;
+constexpr int kLanes = 2;
+static hipStream_t g_lanes[kLanes] = { nullptr, nullptr };
+static hipStream_t g_stream = nullptr; // the selected lane
+static int g_lane = 0;
+constexpr int kJoinEvents = 64;
+static hipEvent_t g_join[kJoinEvents];
+static int g_join_next = 0;
 static bool g_ready = false;
 static int g_device = -1;
 
@@ -46,6 +54,7 @@ int fail(int code, const char *fmt, ...)
 }
 
 hipStream_t stream() { return g_stream; }
+int lane() { return g_lane; }
 bool ready() { return g_ready; }
 
 int check_launch(const char *what)
@@ -130,7 +139,11 @@ int fitre_hip_init(int device)
 	FITRE_HIP_TRY(hipSetDevice(device));
 	if (g_ready && g_device == device) return FITRE_OK;
 	if (g_ready) fitre_hip_shutdown();
-	FITRE_HIP_TRY(hipStreamCreate(&g_stream)); // default priority, ordered with the null stream
+	for (int i = 0; i < kLanes; i++) FITRE_HIP_TRY(hipStreamCreate(&g_lanes[i])); // default priority
+	for (int i = 0; i < kJoinEvents; i++) FITRE_HIP_TRY(hipEventCreateWithFlags(&g_join[i], hipEventDisableTiming));
+	g_join_next = 0;
+	g_stream = g_lanes[0];
+	g_lane = 0;
 	g_device = device;
 	g_ready = true;
 	memset(g_totals, 0, sizeof(g_totals));
@@ -140,11 +153,15 @@ int fitre_hip_init(int device)
 int fitre_hip_shutdown(void)
 {
 	if (!g_ready) return FITRE_OK;
-	(void)hipStreamSynchronize(g_stream);
+	for (int i = 0; i < kLanes; i++) (void)hipStreamSynchronize(g_lanes[i]);
 	drain_pending();
 	for (hipEvent_t e : g_event_pool) (void)hipEventDestroy(e);
 	g_event_pool.clear();
-	(void)hipStreamDestroy(g_stream);
+	for (int i = 0; i < kJoinEvents; i++) (void)hipEventDestroy(g_join[i]);
+	for (int i = 0; i < kLanes; i++) {
+		(void)hipStreamDestroy(g_lanes[i]);
+		g_lanes[i] = nullptr;
+	}
 	g_stream = nullptr;
 	g_ready = false;
 	g_profile = false;
@@ -154,7 +171,30 @@ int fitre_hip_shutdown(void)
 int fitre_hip_sync(void)
 {
 	FITRE_NEED_INIT();
-	FITRE_HIP_TRY(hipStreamSynchronize(g_stream));
+	for (int i = 0; i < kLanes; i++) FITRE_HIP_TRY(hipStreamSynchronize(g_lanes[i]));
+	return FITRE_OK;
+}
+
+int fitre_hip_lane_select(int laneIndex)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(laneIndex >= 0 && laneIndex < kLanes, "fitre_hip_lane_select: lane %d out of range", laneIndex);
+	// with per-launch accounting on, everything runs on lane 0 so that durations are not shared
+	g_lane = g_profile ? 0 : laneIndex;
+	g_stream = g_lanes[g_lane];
+	return FITRE_OK;
+}
+
+int fitre_hip_lane_wait(int waiter, int signaller)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(waiter >= 0 && waiter < kLanes && signaller >= 0 && signaller < kLanes,
+	              "fitre_hip_lane_wait: lane out of range (%d waits for %d)", waiter, signaller);
+	if (waiter == signaller) return FITRE_OK;
+	hipEvent_t e = g_join[g_join_next];
+	g_join_next = (g_join_next + 1) % kJoinEvents;
+	FITRE_HIP_TRY(hipEventRecord(e, g_lanes[signaller]));
+	FITRE_HIP_TRY(hipStreamWaitEvent(g_lanes[waiter], e, 0));
 	return FITRE_OK;
 }
 
@@ -194,7 +234,7 @@ int fitre_hip_free(void *ptr)
 {
 	FITRE_NEED_INIT();
 	if (!ptr) return FITRE_OK;
-	FITRE_HIP_TRY(hipStreamSynchronize(g_stream));
+	for (int i = 0; i < kLanes; i++) FITRE_HIP_TRY(hipStreamSynchronize(g_lanes[i]));
 	FITRE_HIP_TRY(hipFree(ptr));
 	return FITRE_OK;
 }
@@ -212,7 +252,7 @@ int fitre_hip_free_host(void *ptr)
 {
 	FITRE_NEED_INIT();
 	if (!ptr) return FITRE_OK;
-	FITRE_HIP_TRY(hipStreamSynchronize(g_stream));
+	for (int i = 0; i < kLanes; i++) FITRE_HIP_TRY(hipStreamSynchronize(g_lanes[i]));
 	FITRE_HIP_TRY(hipHostFree(ptr));
 	return FITRE_OK;
 }
@@ -305,10 +345,14 @@ int fitre_hip_event_elapsed_ms(void *start, void *stop, float *ms)
 int fitre_hip_profile_enable(int on)
 {
 	FITRE_NEED_INIT();
-	FITRE_HIP_TRY(hipStreamSynchronize(g_stream));
+	for (int i = 0; i < kLanes; i++) FITRE_HIP_TRY(hipStreamSynchronize(g_lanes[i]));
 	drain_pending();
 	if (on) memset(g_totals, 0, sizeof(g_totals));
 	g_profile = (on != 0);
+	if (g_profile) {
+		g_lane = 0;
+		g_stream = g_lanes[0];
+	}
 	return FITRE_OK;
 }
 

@@ -76,13 +76,15 @@ static size_t forward_ws_bytes(const CNN_MODEL *model, int batch)
 	return need;
 }
 
-static size_t backward_ws_bytes(const CNN_MODEL *model, int batch)
+/* cnnBackward carves two workspaces from devPtr: one for the chain that produces each layer's
+ * delta (pool / activation / batch norm / input gradient, lane 0) and one for the weight gradients,
+ * which run beside that chain on lane 1. */
+static size_t backward_chain_ws_bytes(const CNN_MODEL *model, int batch)
 {
 	size_t need = 256;
 	for (int i = 0; i < model->cLayers; i++) {
 		const CONV_LAYER *c = &model->convLayer[i];
 		fitre_conv_shape s = conv_shape(c, batch);
-		need = max_sz(need, fitre_hip_conv_weight_grad_workspace(&s));
 		if (i != 0) need = max_sz(need, fitre_hip_conv_input_grad_workspace(&s));
 		need = max_sz(need, fitre_hip_batch_norm_workspace(c->outChannels, (long)batch * c->outWidth * c->outHeight));
 	}
@@ -91,7 +93,22 @@ static size_t backward_ws_bytes(const CNN_MODEL *model, int batch)
 		need = max_sz(need, fitre_hip_gemm_workspace(f->out, f->in, batch));
 		need = max_sz(need, fitre_hip_gemm_workspace(f->in, batch, f->out));
 	}
-	return need;
+	return (need + 255) & ~(size_t)255;
+}
+
+static size_t backward_side_ws_bytes(const CNN_MODEL *model, int batch)
+{
+	size_t need = 256;
+	for (int i = 0; i < model->cLayers; i++) {
+		fitre_conv_shape s = conv_shape(&model->convLayer[i], batch);
+		need = max_sz(need, fitre_hip_conv_weight_grad_workspace(&s));
+	}
+	return (need + 255) & ~(size_t)255;
+}
+
+static size_t backward_ws_bytes(const CNN_MODEL *model, int batch)
+{
+	return backward_chain_ws_bytes(model, batch) + backward_side_ws_bytes(model, batch);
 }
 
 long cnnForwardMemRequired(CNN_MODEL *model)
@@ -191,7 +208,9 @@ void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, 
 	const real *weights = data->weights;
 	const int n = batchSize, nc = model->cLayers;
 	void *ws = (void *)devPtr;
-	const size_t wsBytes = sizeof(real) * (size_t)cnnBackwardMemRequired(model);
+	const size_t wsBytes = backward_chain_ws_bytes(model, model->batchSize);
+	void *sideWs = (void *)((char *)devPtr + wsBytes);
+	const size_t sideBytes = backward_side_ws_bytes(model, model->batchSize);
 	real *temp;
 
 	if (nc < 1 || n < 1 || n > model->batchSize) {
@@ -274,7 +293,12 @@ void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, 
 
 		const real *input = (c == 0) ? data->currentBatch : z + zOffsets[c] + model->convLayer[c - 1].outputOffset;
 		fitre_conv_shape shape = conv_shape(l, n);
-		HIP_CALL(fitre_hip_conv_weight_grad(&shape, input, cur, gradient + wOffsets[c], ws, wsBytes));
+		/* The weight gradient needs this layer's delta and input, both final by now, and nothing
+		 * later reads its result: it runs on lane 1 beside the chain that goes on to the layers below. */
+		HIP_CALL(fitre_hip_lane_wait(1, 0));
+		HIP_CALL(fitre_hip_lane_select(1));
+		HIP_CALL(fitre_hip_conv_weight_grad(&shape, input, cur, gradient + wOffsets[c], sideWs, sideBytes));
+		HIP_CALL(fitre_hip_lane_select(0));
 		if (c != 0) HIP_CALL(fitre_hip_conv_input_grad(&shape, cur, weights + wOffsets[c], delta, ws, wsBytes));
 	}
 	HIP_CALL(fitre_hip_sync());

@@ -41,8 +41,17 @@ const char *fitre_hip_last_error(void);
 /* compute units, wavefront size, max threads per block, total and free bytes; name may be NULL */
 int fitre_hip_device_info(int *computeUnits, int *waveSize, int *maxThreadsPerBlock, size_t *totalBytes,
                           size_t *freeBytes, char *name, int nameLen);
-/* the hipStream_t the layer launches on, as an opaque pointer */
+/* the hipStream_t of the selected lane, as an opaque pointer */
 void *fitre_hip_stream(void);
+/* The layer owns two streams ("lanes", both at default priority).  Every call queues its work on the
+ * selected lane (0 after init).  A caller that has two independent chains of work may put one on
+ * lane 1 and order the chains with fitre_hip_lane_wait(waiter, signaller): work queued on `waiter`
+ * after the call starts only when everything queued on `signaller` before the call has finished.
+ * fitre_hip_sync() waits for both lanes.  While per-launch accounting is on (fitre_hip_profile_enable)
+ * lane selection is ignored and everything runs on lane 0, so that launch durations are unshared.
+ * No counterpart in the reference, which runs on the null stream and synchronises after every launch. */
+int fitre_hip_lane_select(int lane);
+int fitre_hip_lane_wait(int waiter, int signaller);
 
 /* ---------------- memory (device/cuda_utils.c; device/cuda_utils.h:15-26) ---------------- */
 int fitre_hip_malloc(void **ptr, size_t bytes);
