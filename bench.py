@@ -69,6 +69,14 @@ def gpu_leg(args):
     x, y = batch_inputs(model, batch, rng)
     gm = GpuModel(dev, model, w, x.astype(np.float32), y, batch)
     loss = gm.forward()  # untimed: produces z, probs and the loss errors
+    # one plain copy of known size (64 Mi floats: 256 MiB read, 256 MiB written), outside the timed
+    # region: the kernel that hardware traffic counters of the same run are scaled by
+    cal_n = 1 << 26
+    cal_src, cal_dst = dev.zeros(cal_n), dev.zeros(cal_n)
+    L.check(L.hip.fitre_hip_copy(cal_n, cal_src, cal_dst))
+    dev.sync()
+    dev.free(cal_src)
+    dev.free(cal_dst)
 
     def run(steps):
         for _ in range(steps):

@@ -16,10 +16,10 @@
 //
 // Weight gradient ("reduction over positions"):
 //     dW[o][c][ta][tb] = sum_m delta[o][m] * src[c][m + (ta-1)*B + (tb-1)]
-//   A workgroup owns 128 output channels x 32 input channels x all nine taps: each wave
-//   keeps nine 32x32 accumulator blocks (one per tap).  A stage brings 32 positions of
-//   delta (128 rows) and of the source (32 rows, plus the halo) into LDS; every MFMA
-//   step then reads ONE delta fragment and nine shifted source fragments.
+//   A workgroup of twelve waves owns 128 output channels x 32 input channels x all nine taps:
+//   each wave keeps three 32x32 accumulator blocks (the taps of one window row).  A stage brings
+//   64 positions of delta (128 rows) and of the source (32 rows, plus the halo) into LDS; every
+//   MFMA step then reads one delta fragment and three shifted source fragments.
 //
 // The code avoids everything the compiler turns into control flow or private memory in
 // the hot loops: no conditional loads or stores (invalid cells go to an out-of-range
@@ -264,28 +264,37 @@ conv3x3_pos_kernel(const Conv3x3Params p, const OutParams out)
 // ---------------------------------------------------------------------------------
 // weight gradient
 // ---------------------------------------------------------------------------------
-constexpr int kC3Stage = 32;               // positions per LDS stage
+constexpr int kC3DwThreads = 768;          // 12 waves: (output-channel block 0..3) x (tap row 0..2)
+constexpr int kC3Stage = 64;               // positions per LDS stage
 constexpr int kC3DwCin = 32;               // input channels per workgroup
 constexpr int kC3DeltaLd = kC3Stage + 1;   // odd row stride of the delta stage
 
+// One workgroup per compute unit: 128 output channels x 32 input channels x 9 taps, i.e. 36
+// accumulator blocks of 32x32, three per wave (the three taps of one window row).  Twelve waves
+// keep three wavefronts on every SIMD while the accumulators of the whole chip -- the volume a
+// split reduction has to write out and sum again -- stay at half of what two four-wave
+// workgroups per compute unit would hold.  LDS stages are double buffered: one barrier per stage.
 // MAXB: widest image row this instantiation's source window holds (32 or 64)
 template <bool VECD, int MAXB>
-__global__ void __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(2, 2)))
+__global__ void __launch_bounds__(kC3DwThreads)
 conv3x3_dw_kernel(const Conv3x3Params p, const float *delta, uint32_t deltaBytes, const OutParams out)
 {
+	constexpr int T = kC3DwThreads;
 	constexpr int WIN_MAX = kC3Stage + 2 * (MAXB + 1);
 	constexpr int SRC_LD = WIN_MAX + 1 - (WIN_MAX & 1); // odd row stride of the source stage
-	constexpr int X_DUMMY = kC3DwCin * SRC_LD;
-	constexpr int CH_PER_WAVE = kC3DwCin / 4;
-	constexpr int XI = (WIN_MAX + 63) / 64;
-	constexpr int XE = CH_PER_WAVE * XI;
-	constexpr int DE = kC3Tile * kC3Stage / 4 / kGemmThreads; // 4-float groups of delta per thread (4)
-	__shared__ float Ds[kC3Tile * kC3DeltaLd];
-	__shared__ float Xs[kC3DwCin * SRC_LD + 1];
-	__shared__ uint32_t Ms[kC3Stage];
+	constexpr int X_DUMMY = kC3DwCin * SRC_LD;          // swallows the stores of threads without a cell
+	constexpr int D_DUMMY = kC3Tile * kC3DeltaLd;
+	constexpr int DGROUPS = kC3Tile * kC3Stage / 4;     // 4-float groups of delta per stage
+	constexpr int DE = (DGROUPS + T - 1) / T;
+	constexpr int XE = (kC3DwCin * WIN_MAX + T - 1) / T;
+	static_assert(T % (kC3Stage / 4) == 0, "a thread keeps its column group in every round");
+	__shared__ float Ds[2][D_DUMMY + 4];
+	__shared__ float Xs[2][X_DUMMY + 1];
+	__shared__ uint32_t Ms[2][kC3Stage];
 
 	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 	const int khalf = lane >> 5, l32 = lane & 31;
+	const int ob = wave & 3, ta = wave >> 2; // output-channel block, tap row
 	const int c0 = blockIdx.x * kC3DwCin, o0 = blockIdx.y * kC3Tile;
 	const int halo = p.B + 1;
 	const int win = kC3Stage + 2 * halo;
@@ -297,6 +306,31 @@ conv3x3_dw_kernel(const Conv3x3Params p, const float *delta, uint32_t deltaBytes
 	const __amdgpu_buffer_rsrc_t srcRs = make_rsrc(p.src, p.srcBytes);
 	const __amdgpu_buffer_rsrc_t dRs = make_rsrc(delta, deltaBytes);
 
+	// what this thread stages, fixed for all stages
+	const int dCol = 4 * (tid % (kC3Stage / 4)); // first position of its delta groups inside the stage
+	int dRowOff[DE];                             // (o0 + row) * plane, or -1 for no group / row past the tensor
+	int dLds[DE];
+#pragma unroll
+	for (int e = 0; e < DE; e++) {
+		const int idx = tid + T * e;
+		const int row = idx / (kC3Stage / 4);
+		const bool has = idx < DGROUPS;
+		dRowOff[e] = (has & ((o0 + row) < p.I)) ? (o0 + row) * plane : -1;
+		dLds[e] = has ? row * kC3DeltaLd + dCol : D_DUMMY;
+	}
+	int xChanOff[XE]; // (c0 + c) * plane, or -1
+	int xRel[XE];     // cell position relative to the first position of the stage
+	int xLds[XE];
+#pragma unroll
+	for (int e = 0; e < XE; e++) {
+		const int idx = tid + T * e;
+		const int c = idx / win, x = idx - c * win;
+		const bool has = c < kC3DwCin;
+		xChanOff[e] = (has & ((c0 + c) < p.cred)) ? (c0 + c) * plane : -1;
+		xRel[e] = x - halo;
+		xLds[e] = has ? c * SRC_LD + x : X_DUMMY;
+	}
+
 	float dreg[DE * 4];
 	float xreg[XE];
 	uint32_t mreg = 0;
@@ -306,17 +340,15 @@ conv3x3_dw_kernel(const Conv3x3Params p, const float *delta, uint32_t deltaBytes
 		const int m0_ = (ST) * kC3Stage;                                                                              \
 		_Pragma("unroll") for (int e = 0; e < DE; e++)                                                                \
 		{                                                                                                             \
-			const int idx = tid + kGemmThreads * e;                                                                   \
-			const int row = idx / (kC3Stage / 4), qd = idx % (kC3Stage / 4);                                          \
-			const int m = m0_ + 4 * qd;                                                                               \
-			const bool rowOk = (o0 + row) < p.I;                                                                      \
+			const int m = m0_ + dCol;                                                                                 \
 			if constexpr (VECD) { /* plane % 4 == 0: a group is inside the row or past its end as a whole */          \
-				const bool ok = rowOk & (m < plane);                                                                  \
-				const float4 v4 = *reinterpret_cast<const float4 *>(delta + (ok ? (o0 + row) * plane + m : 0));       \
+				const bool ok = (dRowOff[e] >= 0) & (m < plane);                                                      \
+				const float4 v4 = *reinterpret_cast<const float4 *>(delta + (ok ? dRowOff[e] + m : 0));               \
 				dreg[4 * e + 0] = ok ? v4.x : 0.f, dreg[4 * e + 1] = ok ? v4.y : 0.f;                                 \
 				dreg[4 * e + 2] = ok ? v4.z : 0.f, dreg[4 * e + 3] = ok ? v4.w : 0.f;                                 \
 			} else {                                                                                                  \
-				const uint32_t off = 4u * (uint32_t)((o0 + row) * plane + m);                                         \
+				const bool rowOk = dRowOff[e] >= 0;                                                                   \
+				const uint32_t off = 4u * (uint32_t)(dRowOff[e] + m);                                                 \
 				dreg[4 * e + 0] = buffer_load(dRs, (rowOk & (m + 0 < plane)) ? off : kOutOfRange);                    \
 				dreg[4 * e + 1] = buffer_load(dRs, (rowOk & (m + 1 < plane)) ? off + 4u : kOutOfRange);               \
 				dreg[4 * e + 2] = buffer_load(dRs, (rowOk & (m + 2 < plane)) ? off + 8u : kOutOfRange);               \
@@ -325,83 +357,90 @@ conv3x3_dw_kernel(const Conv3x3Params p, const float *delta, uint32_t deltaBytes
 		}                                                                                                             \
 		_Pragma("unroll") for (int e = 0; e < XE; e++)                                                                \
 		{                                                                                                             \
-			const int c = wave * CH_PER_WAVE + e / XI, x = lane + 64 * (e % XI);                                      \
-			const int m = m0_ - halo + x;                                                                             \
-			const bool ok = (x < win) & ((c0 + c) < p.cred) & (m >= 0) & (m < plane);                                 \
-			xreg[e] = buffer_load(srcRs, ok ? 4u * (uint32_t)((c0 + c) * plane + m) : kOutOfRange);                   \
+			const int m = m0_ + xRel[e];                                                                              \
+			const bool ok = (xChanOff[e] >= 0) & (m >= 0) & (m < plane);                                              \
+			xreg[e] = buffer_load(srcRs, ok ? 4u * (uint32_t)(xChanOff[e] + m) : kOutOfRange);                        \
 		}                                                                                                             \
-		mreg = border_bits(p, (uint32_t)(m0_ + (tid & (kC3Stage - 1))));                                              \
+		if (tid < kC3Stage) mreg = border_bits(p, (uint32_t)(m0_ + tid));                                             \
 	}
 
-	v16f acc[9];
+#define C3_STORE_STAGE(BUF)                                                                                           \
+	{                                                                                                                 \
+		_Pragma("unroll") for (int e = 0; e < DE; e++)                                                                \
+		{                                                                                                             \
+			float *dst = Ds[BUF] + dLds[e];                                                                           \
+			dst[0] = dreg[4 * e], dst[1] = dreg[4 * e + 1], dst[2] = dreg[4 * e + 2], dst[3] = dreg[4 * e + 3];       \
+		}                                                                                                             \
+		_Pragma("unroll") for (int e = 0; e < XE; e++) Xs[BUF][xLds[e]] = xreg[e];                                    \
+		if (tid < kC3Stage) Ms[BUF][tid] = mreg;                                                                      \
+	}
+
+	v16f acc[3];
 #pragma unroll
-	for (int t = 0; t < 9; t++)
+	for (int t = 0; t < 3; t++)
 #pragma unroll
 		for (int v = 0; v < 16; v++) acc[t][v] = 0.f;
 
-	const float *aBase = Ds + (wave * 32 + l32) * kC3DeltaLd + khalf;
-	const float *bBase = Xs + l32 * SRC_LD + halo + khalf;
+	const int aOff = (ob * 32 + l32) * kC3DeltaLd + khalf;
+	const int bOff = l32 * SRC_LD + halo + khalf + (ta - 1) * p.B - 1; // tap (ta, 0); +1, +2 for the other two
+	const int tap0 = ta * 3;
 
-	if (stBeg < stEnd) C3_LOAD_STAGE(stBeg);
+	if (stBeg < stEnd) {
+		C3_LOAD_STAGE(stBeg);
+		C3_STORE_STAGE(0);
+	}
+	__syncthreads();
 	for (int st = stBeg; st < stEnd; st++) {
-		__syncthreads();
-#pragma unroll
-		for (int e = 0; e < DE; e++) {
-			const int idx = tid + kGemmThreads * e;
-			const int row = idx / (kC3Stage / 4), qd = idx % (kC3Stage / 4);
-			float *dst = Ds + row * kC3DeltaLd + 4 * qd;
-			dst[0] = dreg[4 * e], dst[1] = dreg[4 * e + 1], dst[2] = dreg[4 * e + 2], dst[3] = dreg[4 * e + 3];
-		}
-#pragma unroll
-		for (int e = 0; e < XE; e++) {
-			const int c = wave * CH_PER_WAVE + e / XI, x = lane + 64 * (e % XI);
-			Xs[(x < win) ? c * SRC_LD + x : X_DUMMY] = xreg[e];
-		}
-		Ms[tid & (kC3Stage - 1)] = mreg; // every group of 32 threads holds the same 32 values
-		__syncthreads();
+		const int buf = (st - stBeg) & 1;
 		if (st + 1 < stEnd) C3_LOAD_STAGE(st + 1);
 
-		// 16 MFMA steps of two positions; per step one delta fragment, the border bits of the
-		// two positions and nine shifted source fragments, read one step ahead
-		float fa[2], fb[2][9];
+		// 32 MFMA steps of two positions; per step one delta fragment, the border bits of the two
+		// positions and three shifted source fragments, read one step ahead
+		const float *aBase = Ds[buf] + aOff;
+		const float *bBase = Xs[buf] + bOff;
+		const uint32_t *mBase = Ms[buf] + khalf;
+		float fa[2], fb[2][3];
 		uint32_t fbits[2];
 		fa[0] = aBase[0];
-		fbits[0] = Ms[khalf];
+		fbits[0] = mBase[0];
 #pragma unroll
-		for (int tap = 0; tap < 9; tap++) fb[0][tap] = bBase[(tap / 3 - 1) * p.B + (tap % 3 - 1)];
+		for (int tb = 0; tb < 3; tb++) fb[0][tb] = bBase[tb];
 #pragma unroll
 		for (int s = 0; s < kC3Stage / 2; s++) {
 			const int cur = s & 1, nxt = cur ^ 1;
-			float bm[9];
+			float bm[3];
 #pragma unroll
-			for (int tap = 0; tap < 9; tap++) bm[tap] = keep_if(fb[cur][tap], fbits[cur], tap);
+			for (int tb = 0; tb < 3; tb++) bm[tb] = keep_if(fb[cur][tb], fbits[cur], tap0 + tb);
 			if (s + 1 < kC3Stage / 2) {
 				fa[nxt] = aBase[2 * (s + 1)];
-				fbits[nxt] = Ms[2 * (s + 1) + khalf];
+				fbits[nxt] = mBase[2 * (s + 1)];
 #pragma unroll
-				for (int tap = 0; tap < 9; tap++) fb[nxt][tap] = bBase[2 * (s + 1) + (tap / 3 - 1) * p.B + (tap % 3 - 1)];
+				for (int tb = 0; tb < 3; tb++) fb[nxt][tb] = bBase[2 * (s + 1) + tb];
 			}
 #pragma unroll
-			for (int tap = 0; tap < 9; tap++) acc[tap] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[cur], bm[tap], acc[tap], 0, 0, 0);
-			__builtin_amdgcn_sched_group_barrier(0x002, 18, 0); // border masking of this step
+			for (int tb = 0; tb < 3; tb++) acc[tb] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[cur], bm[tb], acc[tb], 0, 0, 0);
+			__builtin_amdgcn_sched_group_barrier(0x002, 6, 0); // border masking of this step
 			__builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-			__builtin_amdgcn_sched_group_barrier(0x100, 11, 0); // LDS reads of the next step
-			__builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
+			__builtin_amdgcn_sched_group_barrier(0x100, 5, 0); // LDS reads of the next step
+			__builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
 		}
+		if (st + 1 < stEnd) C3_STORE_STAGE(buf ^ 1);
+		__syncthreads();
 	}
 #undef C3_LOAD_STAGE
+#undef C3_STORE_STAGE
 
-	// ---- store: dW[o][c][tap], nine consecutive floats per (o, c) -----------------------------
+	// ---- store: dW[o][c][tap]; this wave holds taps (ta, 0..2) of 32 output x 32 input channels ----
 	float *C = out.C + (size_t)blockIdx.z * out.splitStride;
 	const int c = c0 + l32;
 	if (c < p.cred) {
 #pragma unroll
 		for (int v = 0; v < 16; v++) {
-			const int o = o0 + wave * 32 + 8 * (v / 4) + 4 * khalf + (v % 4);
+			const int o = o0 + ob * 32 + 8 * (v / 4) + 4 * khalf + (v % 4);
 			if (o >= p.I) continue;
-			float *dst = C + (size_t)o * out.ldc + c * 9;
+			float *dst = C + (size_t)o * out.ldc + c * 9 + tap0;
 #pragma unroll
-			for (int tap = 0; tap < 9; tap++) dst[tap] = acc[tap][v];
+			for (int tb = 0; tb < 3; tb++) dst[tb] = acc[tb][v];
 		}
 	}
 }

@@ -103,8 +103,8 @@ static BlockPlan c3_dw_plan(const fitre_conv_shape *s)
 {
 	long J = (long)s->samples * s->inA * s->inB;
 	long tiles = ((s->inChannels + kC3DwCin - 1) / kC3DwCin) * ((s->outChannels + kC3Tile - 1) / kC3Tile);
-	double stageUs = (kC3Stage / 2.0) * 9.0 * 64.0 / 2400.0;
-	return plan_blocks(tiles, (J + kC3Stage - 1) / kC3Stage, stageUs, 2, s->outChannels, (long)s->inChannels * 9);
+	double stageUs = (kC3Stage / 2.0) * 9.0 * 64.0 / 2400.0; // three waves per SIMD, three MFMAs per step each
+	return plan_blocks(tiles, (J + kC3Stage - 1) / kC3Stage, stageUs, 1, s->outChannels, (long)s->inChannels * 9);
 }
 
 template <bool DX>
@@ -193,13 +193,13 @@ static int launch_c3_dw(const fitre_conv_shape *s, const float *x, const float *
 		LaunchScope scope(FITRE_KC_CONV_DW, conv_flops(s), 4);
 		const bool narrow = s->inB <= 32;
 		if (vecd && narrow)
-			conv3x3_dw_kernel<true, 32><<<grid, kGemmThreads, 0, stream()>>>(p, delta, deltaBytes, part);
+			conv3x3_dw_kernel<true, 32><<<grid, kC3DwThreads, 0, stream()>>>(p, delta, deltaBytes, part);
 		else if (vecd)
-			conv3x3_dw_kernel<true, 64><<<grid, kGemmThreads, 0, stream()>>>(p, delta, deltaBytes, part);
+			conv3x3_dw_kernel<true, 64><<<grid, kC3DwThreads, 0, stream()>>>(p, delta, deltaBytes, part);
 		else if (narrow)
-			conv3x3_dw_kernel<false, 32><<<grid, kGemmThreads, 0, stream()>>>(p, delta, deltaBytes, part);
+			conv3x3_dw_kernel<false, 32><<<grid, kC3DwThreads, 0, stream()>>>(p, delta, deltaBytes, part);
 		else
-			conv3x3_dw_kernel<false, 64><<<grid, kGemmThreads, 0, stream()>>>(p, delta, deltaBytes, part);
+			conv3x3_dw_kernel<false, 64><<<grid, kC3DwThreads, 0, stream()>>>(p, delta, deltaBytes, part);
 	}
 	if (plan.splits > 1) launch_splitk_reduce((const float *)ws, plan.splits, I, K, out);
 	return check_launch("conv3x3_dw_kernel");
