@@ -27,6 +27,7 @@ HIPCC_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-function",
 ]
+HIPCC_FLAGS += os.environ.get("FITRE_HIPCC_EXTRA", "").split()  # e.g. -D switches while tuning a kernel
 GCC_FLAGS = ["-O2", "-std=c11", "-fPIC", "-Wall", "-Wextra", "-I" + INC]
 
 

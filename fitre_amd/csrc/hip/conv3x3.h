@@ -21,10 +21,11 @@
 //   64 positions of delta (128 rows) and of the source (32 rows, plus the halo) into LDS; every
 //   MFMA step then reads one delta fragment and three shifted source fragments.
 //
-// The code avoids everything the compiler turns into control flow or private memory in
-// the hot loops: no conditional loads or stores (invalid cells go to an out-of-range
-// buffer offset, resp. a dummy LDS word), border zeroing with v_bfe/v_and instead of a
-// select, staging registers as plain float arrays filled by unrolled loops.
+// The code avoids everything the compiler turns into control flow, private memory or vector
+// arithmetic in the hot loops: no conditional loads or stores (invalid cells go to an
+// out-of-range buffer offset, resp. a dummy LDS word), image borders as zero words in the LDS
+// layout instead of per-element tests, per-thread staging offsets computed once, staging
+// registers as plain float arrays filled by unrolled loops.
 #pragma once
 #include "gemm_engine.h"
 
@@ -44,61 +45,68 @@ struct Conv3x3Params {
 	FastDiv divB, divA; // position -> (n, a, b)
 };
 
-// nine border bits of flat position m: bit ta*3+tb is set when (a+ta-1, b+tb-1) is inside the image
-__device__ __forceinline__ uint32_t border_bits(const Conv3x3Params &p, uint32_t m)
+// Index of flat position m = (n, a, b) in the zero-padded layout: every image row is followed by
+// one zero cell and every image by one zero row, so that a window tap that leaves the image on
+// any side lands on a zero:  (n*(A+1) + a)*(B+1) + b.  `m` is taken one image late (callers add
+// 2*A*B) so that positions a little before the tensor map consistently too.
+__device__ __forceinline__ uint32_t padded_index(const Conv3x3Params &p, uint32_t m)
 {
 	uint32_t q, b, n, a;
 	p.divB.divmod(m, q, b);
 	p.divA.divmod(q, n, a);
-	uint32_t bits = 0;
-#pragma unroll
-	for (int ta = 0; ta < 3; ta++)
-#pragma unroll
-		for (int tb = 0; tb < 3; tb++) {
-			int aa = (int)a + ta - 1, bb = (int)b + tb - 1;
-			bool ok = ((int)m < p.J) & ((unsigned)aa < (unsigned)p.A) & ((unsigned)bb < (unsigned)p.B);
-			bits |= ok ? (1u << (ta * 3 + tb)) : 0u;
-		}
-	return bits;
+	return (n * (uint32_t)(p.A + 1) + a) * (uint32_t)(p.B + 1) + b;
 }
 
-// value if bit `tap` of bits is set, +0.0f otherwise: sign-extending 1-bit field extract, then AND
-__device__ __forceinline__ float keep_if(float value, uint32_t bits, int tap)
-{
-	int m = __builtin_amdgcn_sbfe((int)bits, tap, 1); // 0 or -1
-	return __int_as_float(__float_as_int(value) & m);
-}
+// offset that marks a 16-byte group as out of range for all four of its words
+constexpr uint32_t kGroupOutOfRange = 0xFFFFFFF0u;
 
 // ---------------------------------------------------------------------------------
 // position-contiguous product (forward: DX = false, input gradient: DX = true)
 // CB reduction channels per block; MAXB = widest image row the window is sized for.
+//
+// The source window of a block sits in LDS in the zero-padded layout above, so the B fragment
+// of tap (ta, tb) is the lane's own cell address plus (ta-1)*(B+1) + (tb-1): no border test in
+// the MFMA loop.  Which LDS word a staged cell goes to, which global offsets a thread loads and
+// where they are stored do not depend on the channel block: all of it is computed once, and a
+// block only moves the (uniform) base of the buffer resources.
 // ---------------------------------------------------------------------------------
 // IT = channel rows per workgroup tile (128, or 64 for products with at most 64 output channels).
 template <int CB, bool DX, int MAXB, int IT>
 struct C3Pos {
 	static constexpr int TM = IT / 64, TN = 2;
-	// weights in LDS.  forward: 128 rows (output channel) x CB*9, odd row stride.
-	// input gradient: CB rows (reduction channel) x 128*9 weights of the tile's channels.
+	// weights in LDS.  forward: IT rows (output channel) x CB*9, odd row stride.
+	// input gradient: CB rows (reduction channel) x IT*9 weights of the tile's channels.
 	static constexpr int A_LD = DX ? (IT * 9 + 4) : (CB * 9 + 1);
 	static constexpr int A_FLOATS = DX ? CB * A_LD : IT * A_LD;
 	static constexpr int WQ = DX ? (IT * 9 / 4) : (CB * 9 / 4); // 4-float groups per LDS row
 	static constexpr int WROWS = DX ? CB : IT;
 	static constexpr int WGROUPS = WROWS * WQ;
 	static constexpr int WE = (WGROUPS + kGemmThreads - 1) / kGemmThreads; // groups per thread
-	static constexpr bool WEXACT = WGROUPS % kGemmThreads == 0;            // else the last round is partial
-	static constexpr int A_DUMMY = A_FLOATS;                               // four spare words for the idle threads of that round
-	// source window in LDS: CB channels x (128 + 2*(B+1)) cells, odd channel stride; one spare
-	// word at the end swallows the writes of threads that have no cell
-	static constexpr int WIN_MAX = kC3Tile + 2 * (MAXB + 1);
-	static constexpr int WIN_LD = WIN_MAX + 1 - (WIN_MAX & 1); // odd
+	static constexpr int A_DUMMY = A_FLOATS;                               // four spare words for threads without a group
+	// flat cells staged per channel: 128 positions plus B+1 on either side
+	static constexpr int CELLS_MAX = kC3Tile + 2 * (MAXB + 1);
+	// the same cells in the padded layout (the host checks that the shape fits)
+	static constexpr int PAD_MAX = MAXB <= 32 ? 384 : 512;
+	static constexpr int WIN_LD = PAD_MAX + 1; // odd channel stride
 	static constexpr int B_FLOATS = CB * WIN_LD + 1;
 	static constexpr int B_DUMMY = CB * WIN_LD;
 	// window staging: each wave owns CB/4 channels, lanes walk the cells 64 at a time
 	static constexpr int CH_PER_WAVE = CB / 4;
-	static constexpr int XI = (WIN_MAX + 63) / 64;
+	static constexpr int XI = (CELLS_MAX + 63) / 64;
 	static constexpr int SE = CH_PER_WAVE * XI;
 	static_assert(CB % 4 == 0, "CB must be a multiple of the wave count");
 };
+
+// words of the padded window a tile needs: what lies before the tile's first position
+// (B+1 cells, at most two row ends and two image ends) ...
+__host__ __device__ inline int c3_pad_before(int B) { return 3 * (B + 1) + 2; }
+// ... plus 128 + B+1 positions forward with every row end and image end they can cross
+inline int c3_pad_window(int A, int B)
+{
+	const int span = kC3Tile - 1 + B + 1;
+	const int rowEnds = (span + B - 1) / B, imageEnds = (span + A * B - 1) / (A * B);
+	return c3_pad_before(B) + span + rowEnds + imageEnds * (B + 1) + 2;
+}
 
 template <int CB, bool DX, bool VECW, int MAXB, int IT>
 __global__ void __launch_bounds__(kGemmThreads)
@@ -118,17 +126,50 @@ conv3x3_pos_kernel(const Conv3x3Params p, const OutParams out)
 	const int cbTotal = p.cred / CB;
 	const int cbBeg = blockIdx.z * p.perSplit;
 	const int cbEnd = (cbBeg + p.perSplit < cbTotal) ? cbBeg + p.perSplit : cbTotal;
+	const int rowLen = DX ? p.I * 9 : p.cred * 9;
+	const uint32_t late = (uint32_t)(2 * p.A * p.B);              // see padded_index; covers the B+1 cells before position 0
+	const uint32_t ref = padded_index(p, (uint32_t)j0 + late);    // the tile's first position
+	const int before = c3_pad_before(p.B);
 
-	const __amdgpu_buffer_rsrc_t srcRs = make_rsrc(p.src, p.srcBytes);
-	const __amdgpu_buffer_rsrc_t wRs = make_rsrc(p.w, p.wBytes);
+	// the padded window starts out all zero; staging only ever writes the cells of real positions
+	for (int i = tid; i < K::B_FLOATS; i += kGemmThreads) Bs[i] = 0.f;
 
-	uint32_t bits[TN];
+	// ---- what this thread stages, the same for every channel block -------------------------
+	// weights: 16-byte groups idx = tid + 256*e of the block's WROWS x WQ group matrix
+	uint32_t wOff[K::WE]; // byte offset inside the block's weights
+	int wLds[K::WE];
 #pragma unroll
-	for (int tn = 0; tn < TN; tn++) bits[tn] = border_bits(p, (uint32_t)(j0 + (wave & 1) * 64 + tn * 32 + l32));
+	for (int e = 0; e < K::WE; e++) {
+		const int idx = tid + kGemmThreads * e;
+		const int row = idx / K::WQ, qd = idx - row * K::WQ;
+		const bool has = idx < K::WGROUPS;
+		// forward: row = output channel, w[(i0+row)*cred*9 + c0*9 + 4*qd ..]
+		// input gradient: row = reduction channel, w[(c0+row)*I*9 + i0*9 + 4*qd ..]
+		// Rows or columns past the tensor's extent only feed accumulator rows that are never stored:
+		// they may read any valid address (vector loads) or be answered with zero (buffer loads).
+		const int rowG = DX ? row : (i0 + row);
+		const int colG = DX ? (i0 * 9 + 4 * qd) : (4 * qd);
+		const bool inside = has & (DX ? (colG + 3 < rowLen) : (rowG < p.I));
+		const uint32_t off = 4u * (uint32_t)(rowG * rowLen + colG);
+		wOff[e] = VECW ? (inside ? off : 0u) : (has ? off : kGroupOutOfRange);
+		wLds[e] = has ? row * K::A_LD + 4 * qd : K::A_DUMMY;
+	}
+	// window cells x = lane + 64*xi of CH_PER_WAVE channels
+	uint32_t sOff[K::SE]; // byte offset inside the block's channels
+	int sLds[K::SE];
+#pragma unroll
+	for (int e = 0; e < K::SE; e++) {
+		const int c = wave * K::CH_PER_WAVE + e / K::XI, x = lane + 64 * (e % K::XI);
+		const int m = j0 - halo + x; // flat position inside the channel plane
+		const bool has = x < win;
+		const bool inside = has & (m >= 0) & (m < plane);
+		sOff[e] = inside ? 4u * (uint32_t)(c * plane + m) : kOutOfRange;
+		const int cell = (int)(padded_index(p, (uint32_t)m + late) - ref) + before;
+		sLds[e] = has ? c * K::WIN_LD + cell : K::B_DUMMY;
+	}
 
 	float wreg[K::WE * 4];
 	float sreg[K::SE];
-	const int rowLen = DX ? p.I * 9 : p.cred * 9;
 
 	v16f acc[TM][TN];
 #pragma unroll
@@ -138,46 +179,46 @@ conv3x3_pos_kernel(const Conv3x3Params p, const OutParams out)
 #pragma unroll
 			for (int v = 0; v < 16; v++) acc[tm][tn][v] = 0.f;
 
-	// fragment base addresses; the channel pair (2*cp + khalf) and the tap are added per step
+	// fragment base addresses; the channel pair, the tap column and (A side) the tap are
+	// compile-time offsets from these
 	const int rowA = (wave >> 1) * (IT / 2) + l32; // channel row inside the tile (+32 for tm = 1)
 	const float *aBase = DX ? (As + khalf * K::A_LD + rowA * 9) : (As + rowA * K::A_LD + khalf * 9);
 	constexpr int aTmStep = DX ? 32 * 9 : 32 * K::A_LD;
 	constexpr int aCpStep = DX ? 2 * K::A_LD : 18;
-	const float *bBase = Bs + khalf * K::WIN_LD + halo + (wave & 1) * 64 + l32;
+	const float *bRow[TN][3]; // per tap row: the lane's cell one row up / same row / one row down, one column left
+#pragma unroll
+	for (int tn = 0; tn < TN; tn++) {
+		const uint32_t m = (uint32_t)(j0 + (wave & 1) * 64 + tn * 32 + l32);
+		const int cell = (int)(padded_index(p, m + late) - ref) + before;
+#pragma unroll
+		for (int r = 0; r < 3; r++) bRow[tn][r] = Bs + khalf * K::WIN_LD + cell + (r - 1) * (p.B + 1) - 1;
+	}
 
 // global -> registers for channel block CBI (a macro: the register arrays must stay registers)
 #define C3_LOAD_BLOCK(CBI)                                                                                            \
 	{                                                                                                                 \
 		const int c0_ = (CBI) * CB;                                                                                   \
-		_Pragma("unroll") for (int e = 0; e < K::WE; e++)                                                             \
-		{                                                                                                             \
-			const int idx = tid + kGemmThreads * e;                                                                   \
-			const int row = idx / K::WQ, qd = idx - row * K::WQ;                                                      \
-			/* forward: row = output channel, w[(i0+row)*cred*9 + c0*9 + 4*qd ..]                                    \
-			   input gradient: row = reduction channel, w[(c0+row)*I*9 + i0*9 + 4*qd ..] */                           \
-			const int rowG = DX ? (c0_ + row) : (i0 + row);                                                           \
-			const int colG = DX ? (i0 * 9 + 4 * qd) : (c0_ * 9 + 4 * qd);                                             \
-			const bool ok = (DX ? (colG < rowLen) : (rowG < p.I)) & (K::WEXACT | (idx < K::WGROUPS));                 \
-			if constexpr (VECW) {                                                                                     \
-				/* rows / columns past the tensor are clamped to element 0: their products land in                   \
-				   accumulator rows that are never stored */                                                          \
-				const float4 v4 = *reinterpret_cast<const float4 *>(p.w + (ok ? rowG * rowLen + colG : 0));           \
+		const size_t wShift = DX ? (size_t)c0_ * rowLen : (size_t)c0_ * 9; /* floats, uniform */                      \
+		if constexpr (VECW) {                                                                                         \
+			const char *wBlk = reinterpret_cast<const char *>(p.w + wShift);                                          \
+			_Pragma("unroll") for (int e = 0; e < K::WE; e++)                                                         \
+			{                                                                                                         \
+				const float4 v4 = *reinterpret_cast<const float4 *>(wBlk + wOff[e]);                                  \
 				wreg[4 * e + 0] = v4.x, wreg[4 * e + 1] = v4.y, wreg[4 * e + 2] = v4.z, wreg[4 * e + 3] = v4.w;       \
-			} else {                                                                                                  \
-				const uint32_t off = ok ? 4u * (uint32_t)(rowG * rowLen + colG) : kOutOfRange;                        \
-				wreg[4 * e + 0] = buffer_load(wRs, off);                                                              \
-				wreg[4 * e + 1] = buffer_load(wRs, ok ? off + 4u : kOutOfRange);                                      \
-				wreg[4 * e + 2] = buffer_load(wRs, ok ? off + 8u : kOutOfRange);                                      \
-				wreg[4 * e + 3] = buffer_load(wRs, ok ? off + 12u : kOutOfRange);                                     \
+			}                                                                                                         \
+		} else {                                                                                                      \
+			const __amdgpu_buffer_rsrc_t wRs = make_rsrc(p.w + wShift, p.wBytes - (uint32_t)(4 * wShift));            \
+			_Pragma("unroll") for (int e = 0; e < K::WE; e++)                                                         \
+			{                                                                                                         \
+				wreg[4 * e + 0] = buffer_load(wRs, wOff[e]);                                                          \
+				wreg[4 * e + 1] = buffer_load(wRs, wOff[e] + 4u);                                                     \
+				wreg[4 * e + 2] = buffer_load(wRs, wOff[e] + 8u);                                                     \
+				wreg[4 * e + 3] = buffer_load(wRs, wOff[e] + 12u);                                                    \
 			}                                                                                                         \
 		}                                                                                                             \
-		_Pragma("unroll") for (int e = 0; e < K::SE; e++)                                                             \
-		{                                                                                                             \
-			const int c = wave * K::CH_PER_WAVE + e / K::XI, x = lane + 64 * (e % K::XI);                             \
-			const int m = j0 - halo + x; /* flat position inside the channel plane */                                 \
-			const bool ok = (x < win) & (m >= 0) & (m < plane);                                                       \
-			sreg[e] = buffer_load(srcRs, ok ? 4u * (uint32_t)((c0_ + c) * plane + m) : kOutOfRange);                  \
-		}                                                                                                             \
+		const size_t sShift = (size_t)c0_ * plane;                                                                    \
+		const __amdgpu_buffer_rsrc_t sRs = make_rsrc(p.src + sShift, p.srcBytes - (uint32_t)(4 * sShift));            \
+		_Pragma("unroll") for (int e = 0; e < K::SE; e++) sreg[e] = buffer_load(sRs, sOff[e]);                        \
 	}
 
 	if (cbBeg < cbEnd) C3_LOAD_BLOCK(cbBeg);
@@ -186,9 +227,7 @@ conv3x3_pos_kernel(const Conv3x3Params p, const OutParams out)
 		__syncthreads();
 #pragma unroll
 		for (int e = 0; e < K::WE; e++) {
-			const int idx = tid + kGemmThreads * e;
-			const int row = idx / K::WQ, qd = idx - row * K::WQ;
-			float *dst = As + ((K::WEXACT | (idx < K::WGROUPS)) ? row * K::A_LD + 4 * qd : K::A_DUMMY);
+			float *dst = As + wLds[e];
 			if constexpr (DX) { // A_LD is a multiple of four
 				*reinterpret_cast<float4 *>(dst) = make_float4(wreg[4 * e], wreg[4 * e + 1], wreg[4 * e + 2], wreg[4 * e + 3]);
 			} else {
@@ -196,10 +235,7 @@ conv3x3_pos_kernel(const Conv3x3Params p, const OutParams out)
 			}
 		}
 #pragma unroll
-		for (int e = 0; e < K::SE; e++) {
-			const int c = wave * K::CH_PER_WAVE + e / K::XI, x = lane + 64 * (e % K::XI);
-			Bs[(x < win) ? c * K::WIN_LD + x : K::B_DUMMY] = sreg[e];
-		}
+		for (int e = 0; e < K::SE; e++) Bs[sLds[e]] = sreg[e];
 		__syncthreads();
 		if (cb + 1 < cbEnd) C3_LOAD_BLOCK(cb + 1);
 
@@ -210,29 +246,23 @@ conv3x3_pos_kernel(const Conv3x3Params p, const OutParams out)
 #pragma unroll
 		for (int tm = 0; tm < TM; tm++) a[0][tm] = aBase[tm * aTmStep + (DX ? 8 : 0)];
 #pragma unroll
-		for (int tn = 0; tn < TN; tn++) b[0][tn] = bBase[tn * 32 - p.B - 1];
+		for (int tn = 0; tn < TN; tn++) b[0][tn] = bRow[tn][0][0];
 #pragma unroll
 		for (int step = 0; step < STEPS; step++) {
 			const int cur = step & 1, nxt = cur ^ 1;
-			const int tap = step / (CB / 2);
-			float bm[TN];
-#pragma unroll
-			for (int tn = 0; tn < TN; tn++) bm[tn] = keep_if(b[cur][tn], bits[tn], tap);
 			if (step + 1 < STEPS) {
 				const int tapN = (step + 1) / (CB / 2), cpN = (step + 1) % (CB / 2);
-				const int shiftN = (tapN / 3 - 1) * p.B + (tapN % 3 - 1);
 				const int aTapN = DX ? (8 - tapN) : tapN;
 #pragma unroll
 				for (int tm = 0; tm < TM; tm++) a[nxt][tm] = aBase[tm * aTmStep + cpN * aCpStep + aTapN];
 #pragma unroll
-				for (int tn = 0; tn < TN; tn++) b[nxt][tn] = bBase[cpN * 2 * K::WIN_LD + tn * 32 + shiftN];
+				for (int tn = 0; tn < TN; tn++) b[nxt][tn] = bRow[tn][tapN / 3][cpN * 2 * K::WIN_LD + tapN % 3];
 			}
 #pragma unroll
 			for (int tm = 0; tm < TM; tm++)
 #pragma unroll
 				for (int tn = 0; tn < TN; tn++)
-					acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][tm], bm[tn], acc[tm][tn], 0, 0, 0);
-			__builtin_amdgcn_sched_group_barrier(0x002, 2 * TN, 0);  // border masking of this step
+					acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][tm], b[cur][tn], acc[tm][tn], 0, 0, 0);
 			__builtin_amdgcn_sched_group_barrier(0x008, 1, 0);       // first MFMA
 			__builtin_amdgcn_sched_group_barrier(0x100, TM + TN, 0); // LDS reads of the next step
 			__builtin_amdgcn_sched_group_barrier(0x008, TM * TN - 1, 0);
@@ -273,24 +303,38 @@ constexpr int kC3DeltaLd = kC3Stage + 1;   // odd row stride of the delta stage
 // accumulator blocks of 32x32, three per wave (the three taps of one window row).  Twelve waves
 // keep three wavefronts on every SIMD while the accumulators of the whole chip -- the volume a
 // split reduction has to write out and sum again -- stay at half of what two four-wave
-// workgroups per compute unit would hold.  LDS stages are double buffered: one barrier per stage.
-// MAXB: widest image row this instantiation's source window holds (32 or 64)
+// workgroups per compute unit would hold.  LDS stages are double buffered: one barrier per
+// stage, and the next stage is written half way through the current one.
+//
+// Border handling costs two vector instructions per MFMA step:
+//   * the source stage keeps every image row followed by one zero word ("row pads"), so the
+//     taps one column left / right of the row ends read zeros; the word of flat window cell r
+//     is r + (bs + r) / B with bs = column of the window's first cell;
+//   * taps one row up / down are invalid on the first / last row of an image; that depends on
+//     the position only, i.e. on the reduction index, so the mask is applied to the delta
+//     fragment (one AND per step) with a per-position mask table;
+//   * the padded word of a position comes from a second table (one add per step).
+// Requires positions % 64 == 0 (no partial stage).
+// MAXB: widest image row this instantiation's source window holds: 16 (for 2 <= B <= 16) or 32
 template <bool VECD, int MAXB>
 __global__ void __launch_bounds__(kC3DwThreads)
 conv3x3_dw_kernel(const Conv3x3Params p, const float *delta, uint32_t deltaBytes, const OutParams out)
 {
 	constexpr int T = kC3DwThreads;
-	constexpr int WIN_MAX = kC3Stage + 2 * (MAXB + 1);
-	constexpr int SRC_LD = WIN_MAX + 1 - (WIN_MAX & 1); // odd row stride of the source stage
-	constexpr int X_DUMMY = kC3DwCin * SRC_LD;          // swallows the stores of threads without a cell
+	constexpr int CELLS_MAX = kC3Stage + 2 * (MAXB + 1);               // flat window cells per channel
+	constexpr int XP_MAX = CELLS_MAX + (CELLS_MAX + MAXB - 2) / MAXB + 1; // with row pads (largest at B = MAXB)
+	constexpr int XP_LD = XP_MAX + 1 - (XP_MAX & 1);                    // odd row stride
+	constexpr int X_DUMMY = kC3DwCin * XP_LD;                           // swallows stores that have no target
 	constexpr int D_DUMMY = kC3Tile * kC3DeltaLd;
-	constexpr int DGROUPS = kC3Tile * kC3Stage / 4;     // 4-float groups of delta per stage
+	constexpr int DGROUPS = kC3Tile * kC3Stage / 4;                     // 4-float groups of delta per stage
 	constexpr int DE = (DGROUPS + T - 1) / T;
-	constexpr int XE = (kC3DwCin * WIN_MAX + T - 1) / T;
+	constexpr int XE = (kC3DwCin * CELLS_MAX + T - 1) / T;
 	static_assert(T % (kC3Stage / 4) == 0, "a thread keeps its column group in every round");
+	static_assert(MAXB == 16 || MAXB == 32, "row-pad bound: taken at B = MAXB it covers 2 <= B <= 16 resp. 1 <= B <= 32");
 	__shared__ float Ds[2][D_DUMMY + 4];
 	__shared__ float Xs[2][X_DUMMY + 1];
-	__shared__ uint32_t Ms[2][kC3Stage];
+	__shared__ int Pk[2][kC3Stage];          // padded word of position k of the stage
+	__shared__ uint32_t Mk[2][3][kC3Stage];  // per tap row: all ones where the tap row is inside the image
 
 	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 	const int khalf = lane >> 5, l32 = lane & 31;
@@ -299,69 +343,92 @@ conv3x3_dw_kernel(const Conv3x3Params p, const float *delta, uint32_t deltaBytes
 	const int halo = p.B + 1;
 	const int win = kC3Stage + 2 * halo;
 	const int plane = p.J;
-	const int stagesTotal = (p.J + kC3Stage - 1) / kC3Stage;
+	const int stagesTotal = p.J / kC3Stage;
 	const int stBeg = blockIdx.z * p.perSplit;
 	const int stEnd = (stBeg + p.perSplit < stagesTotal) ? stBeg + p.perSplit : stagesTotal;
+	const bool movingRows = (kC3Stage % p.B) != 0; // else every stage window starts in the same column
 
-	const __amdgpu_buffer_rsrc_t srcRs = make_rsrc(p.src, p.srcBytes);
-	const __amdgpu_buffer_rsrc_t dRs = make_rsrc(delta, deltaBytes);
+	// the row pads must read as zero: with fixed rows they are never written after this
+	for (int i = tid; i < 2 * (X_DUMMY + 1); i += T) (&Xs[0][0])[i] = 0.f;
 
-	// what this thread stages, fixed for all stages
+	// ---- what this thread stages ------------------------------------------------------------
 	const int dCol = 4 * (tid % (kC3Stage / 4)); // first position of its delta groups inside the stage
-	int dRowOff[DE];                             // (o0 + row) * plane, or -1 for no group / row past the tensor
+	uint32_t dOff[DE];                           // byte offset of the group at stage 0
 	int dLds[DE];
 #pragma unroll
 	for (int e = 0; e < DE; e++) {
 		const int idx = tid + T * e;
 		const int row = idx / (kC3Stage / 4);
 		const bool has = idx < DGROUPS;
-		dRowOff[e] = (has & ((o0 + row) < p.I)) ? (o0 + row) * plane : -1;
+		const bool inside = has & ((o0 + row) < p.I);
+		// rows past the tensor feed accumulator rows that are never stored
+		const uint32_t off = 4u * (uint32_t)((o0 + row) * plane + dCol);
+		dOff[e] = VECD ? (inside ? off : 4u * (uint32_t)dCol) : (inside ? off : kGroupOutOfRange);
 		dLds[e] = has ? row * kC3DeltaLd + dCol : D_DUMMY;
 	}
 	int xChanOff[XE]; // (c0 + c) * plane, or -1
-	int xRel[XE];     // cell position relative to the first position of the stage
-	int xLds[XE];
+	int xMeta[XE];    // (c * XP_LD) << 8 | r with r the flat cell of the window (first cell = stage start - halo);
+	                  // -1 when the thread has no cell in this round
 #pragma unroll
 	for (int e = 0; e < XE; e++) {
 		const int idx = tid + T * e;
-		const int c = idx / win, x = idx - c * win;
+		const int c = idx / win, r = idx - c * win;
 		const bool has = c < kC3DwCin;
 		xChanOff[e] = (has & ((c0 + c) < p.cred)) ? (c0 + c) * plane : -1;
-		xRel[e] = x - halo;
-		xLds[e] = has ? c * SRC_LD + x : X_DUMMY;
+		xMeta[e] = has ? ((c * XP_LD) << 8) | r : -1;
 	}
 
 	float dreg[DE * 4];
 	float xreg[XE];
-	uint32_t mreg = 0;
+	int xLds[XE]; // LDS word of the cell; bit 31: the cell ends an image row (the next word is a row pad)
+	int pkReg = 0;
+	uint32_t mkReg0 = 0, mkReg2 = 0;
 
+// global -> registers for stage ST, and where its cells go in LDS
 #define C3_LOAD_STAGE(ST)                                                                                             \
 	{                                                                                                                 \
 		const int m0_ = (ST) * kC3Stage;                                                                              \
-		_Pragma("unroll") for (int e = 0; e < DE; e++)                                                                \
-		{                                                                                                             \
-			const int m = m0_ + dCol;                                                                                 \
-			if constexpr (VECD) { /* plane % 4 == 0: a group is inside the row or past its end as a whole */          \
-				const bool ok = (dRowOff[e] >= 0) & (m < plane);                                                      \
-				const float4 v4 = *reinterpret_cast<const float4 *>(delta + (ok ? dRowOff[e] + m : 0));               \
-				dreg[4 * e + 0] = ok ? v4.x : 0.f, dreg[4 * e + 1] = ok ? v4.y : 0.f;                                 \
-				dreg[4 * e + 2] = ok ? v4.z : 0.f, dreg[4 * e + 3] = ok ? v4.w : 0.f;                                 \
-			} else {                                                                                                  \
-				const bool rowOk = dRowOff[e] >= 0;                                                                   \
-				const uint32_t off = 4u * (uint32_t)(dRowOff[e] + m);                                                 \
-				dreg[4 * e + 0] = buffer_load(dRs, (rowOk & (m + 0 < plane)) ? off : kOutOfRange);                    \
-				dreg[4 * e + 1] = buffer_load(dRs, (rowOk & (m + 1 < plane)) ? off + 4u : kOutOfRange);               \
-				dreg[4 * e + 2] = buffer_load(dRs, (rowOk & (m + 2 < plane)) ? off + 8u : kOutOfRange);               \
-				dreg[4 * e + 3] = buffer_load(dRs, (rowOk & (m + 3 < plane)) ? off + 12u : kOutOfRange);              \
+		if constexpr (VECD) {                                                                                         \
+			const char *dBlk = reinterpret_cast<const char *>(delta + m0_);                                           \
+			_Pragma("unroll") for (int e = 0; e < DE; e++)                                                            \
+			{                                                                                                         \
+				const float4 v4 = *reinterpret_cast<const float4 *>(dBlk + dOff[e]);                                  \
+				dreg[4 * e + 0] = v4.x, dreg[4 * e + 1] = v4.y, dreg[4 * e + 2] = v4.z, dreg[4 * e + 3] = v4.w;       \
+			}                                                                                                         \
+		} else {                                                                                                      \
+			const __amdgpu_buffer_rsrc_t dRs = make_rsrc(delta + m0_, deltaBytes - 4u * (uint32_t)m0_);               \
+			_Pragma("unroll") for (int e = 0; e < DE; e++)                                                            \
+			{                                                                                                         \
+				dreg[4 * e + 0] = buffer_load(dRs, dOff[e]);                                                          \
+				dreg[4 * e + 1] = buffer_load(dRs, dOff[e] + 4u);                                                     \
+				dreg[4 * e + 2] = buffer_load(dRs, dOff[e] + 8u);                                                     \
+				dreg[4 * e + 3] = buffer_load(dRs, dOff[e] + 12u);                                                    \
 			}                                                                                                         \
 		}                                                                                                             \
+		/* column of the window's first cell; the bias keeps the dividend non-negative */                             \
+		const uint32_t bs_ = (uint32_t)(m0_ + halo * (p.B - 1)) - p.divB.quot((uint32_t)(m0_ + halo * (p.B - 1))) * (uint32_t)p.B; \
 		_Pragma("unroll") for (int e = 0; e < XE; e++)                                                                \
 		{                                                                                                             \
-			const int m = m0_ + xRel[e];                                                                              \
-			const bool ok = (xChanOff[e] >= 0) & (m >= 0) & (m < plane);                                              \
+			const int r_ = xMeta[e] & 255;                                                                            \
+			const int m = m0_ - halo + r_;                                                                            \
+			const bool ok = (xChanOff[e] >= 0) & ((unsigned)m < (unsigned)plane);                                     \
 			xreg[e] = buffer_load(srcRs, ok ? 4u * (uint32_t)(xChanOff[e] + m) : kOutOfRange);                        \
+			if (movingRows | ((ST) == stBeg)) {                                                                       \
+				uint32_t q_, b_;                                                                                      \
+				p.divB.divmod(bs_ + (uint32_t)r_, q_, b_);                                                            \
+				const int word = (xMeta[e] >> 8) + r_ + (int)q_;                                                      \
+				const int end = (b_ == (uint32_t)(p.B - 1)) ? (int)0x80000000 : 0;                                    \
+				xLds[e] = (xMeta[e] >= 0) ? (word | end) : X_DUMMY;                                                   \
+			}                                                                                                         \
 		}                                                                                                             \
-		if (tid < kC3Stage) mreg = border_bits(p, (uint32_t)(m0_ + tid));                                             \
+		if (tid < kC3Stage) {                                                                                         \
+			uint32_t q_, b_, n_, a_;                                                                                  \
+			p.divB.divmod((uint32_t)(m0_ + tid), q_, b_);                                                             \
+			p.divA.divmod(q_, n_, a_);                                                                                \
+			pkReg = halo + tid + (int)p.divB.quot(bs_ + (uint32_t)(halo + tid));                                      \
+			mkReg0 = (a_ != 0u) ? 0xFFFFFFFFu : 0u;                                                                   \
+			mkReg2 = (a_ != (uint32_t)(p.A - 1)) ? 0xFFFFFFFFu : 0u;                                                  \
+		}                                                                                                             \
 	}
 
 #define C3_STORE_STAGE(BUF)                                                                                           \
@@ -371,9 +438,20 @@ conv3x3_dw_kernel(const Conv3x3Params p, const float *delta, uint32_t deltaBytes
 			float *dst = Ds[BUF] + dLds[e];                                                                           \
 			dst[0] = dreg[4 * e], dst[1] = dreg[4 * e + 1], dst[2] = dreg[4 * e + 2], dst[3] = dreg[4 * e + 3];       \
 		}                                                                                                             \
-		_Pragma("unroll") for (int e = 0; e < XE; e++) Xs[BUF][xLds[e]] = xreg[e];                                    \
-		if (tid < kC3Stage) Ms[BUF][tid] = mreg;                                                                      \
+		_Pragma("unroll") for (int e = 0; e < XE; e++) Xs[BUF][xLds[e] & 0x7FFFFFFF] = xreg[e];                       \
+		if (movingRows) { /* the row pads move with the stage: rewrite them */                                        \
+			_Pragma("unroll") for (int e = 0; e < XE; e++)                                                            \
+			    Xs[BUF][(xLds[e] < 0) ? (xLds[e] & 0x7FFFFFFF) + 1 : X_DUMMY] = 0.f;                                  \
+		}                                                                                                             \
+		if (tid < kC3Stage) {                                                                                         \
+			Pk[BUF][tid] = pkReg;                                                                                     \
+			Mk[BUF][0][tid] = mkReg0;                                                                                 \
+			Mk[BUF][1][tid] = 0xFFFFFFFFu;                                                                            \
+			Mk[BUF][2][tid] = mkReg2;                                                                                 \
+		}                                                                                                             \
 	}
+
+	const __amdgpu_buffer_rsrc_t srcRs = make_rsrc(p.src, p.srcBytes);
 
 	v16f acc[3];
 #pragma unroll
@@ -382,9 +460,9 @@ conv3x3_dw_kernel(const Conv3x3Params p, const float *delta, uint32_t deltaBytes
 		for (int v = 0; v < 16; v++) acc[t][v] = 0.f;
 
 	const int aOff = (ob * 32 + l32) * kC3DeltaLd + khalf;
-	const int bOff = l32 * SRC_LD + halo + khalf + (ta - 1) * p.B - 1; // tap (ta, 0); +1, +2 for the other two
-	const int tap0 = ta * 3;
+	const int bOff = l32 * XP_LD + (ta - 1) * (p.B + 1) - 1; // tap (ta, 0) relative to the position's word; +1, +2 for the other two
 
+	__syncthreads(); // the zero fill above
 	if (stBeg < stEnd) {
 		C3_LOAD_STAGE(stBeg);
 		C3_STORE_STAGE(0);
@@ -392,39 +470,45 @@ conv3x3_dw_kernel(const Conv3x3Params p, const float *delta, uint32_t deltaBytes
 	__syncthreads();
 	for (int st = stBeg; st < stEnd; st++) {
 		const int buf = (st - stBeg) & 1;
-		if (st + 1 < stEnd) C3_LOAD_STAGE(st + 1);
+		const bool more = st + 1 < stEnd;
+		if (more) C3_LOAD_STAGE(st + 1);
 
-		// 32 MFMA steps of two positions; per step one delta fragment, the border bits of the two
-		// positions and three shifted source fragments, read one step ahead
+		// 32 MFMA steps of two positions.  Tables are read two steps ahead, fragments one step ahead.
 		const float *aBase = Ds[buf] + aOff;
 		const float *bBase = Xs[buf] + bOff;
-		const uint32_t *mBase = Ms[buf] + khalf;
+		const int *pBase = Pk[buf] + khalf;
+		const uint32_t *mBase = Mk[buf][ta] + khalf;
+		constexpr int STEPS = kC3Stage / 2;
+		int tp[3];
+		uint32_t tm[3];
 		float fa[2], fb[2][3];
-		uint32_t fbits[2];
+		tp[0] = pBase[0], tm[0] = mBase[0];
+		tp[1] = pBase[2], tm[1] = mBase[2];
 		fa[0] = aBase[0];
-		fbits[0] = mBase[0];
 #pragma unroll
-		for (int tb = 0; tb < 3; tb++) fb[0][tb] = bBase[tb];
+		for (int tb = 0; tb < 3; tb++) fb[0][tb] = bBase[tp[0] + tb];
 #pragma unroll
-		for (int s = 0; s < kC3Stage / 2; s++) {
+		for (int s = 0; s < STEPS; s++) {
 			const int cur = s & 1, nxt = cur ^ 1;
-			float bm[3];
-#pragma unroll
-			for (int tb = 0; tb < 3; tb++) bm[tb] = keep_if(fb[cur][tb], fbits[cur], tap0 + tb);
-			if (s + 1 < kC3Stage / 2) {
-				fa[nxt] = aBase[2 * (s + 1)];
-				fbits[nxt] = mBase[2 * (s + 1)];
-#pragma unroll
-				for (int tb = 0; tb < 3; tb++) fb[nxt][tb] = bBase[2 * (s + 1) + tb];
+			if (s + 2 < STEPS) {
+				tp[(s + 2) % 3] = pBase[2 * (s + 2)];
+				tm[(s + 2) % 3] = mBase[2 * (s + 2)];
 			}
+			if (s + 1 < STEPS) {
+				const float *q = bBase + tp[(s + 1) % 3];
+				fa[nxt] = aBase[2 * (s + 1)];
 #pragma unroll
-			for (int tb = 0; tb < 3; tb++) acc[tb] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[cur], bm[tb], acc[tb], 0, 0, 0);
-			__builtin_amdgcn_sched_group_barrier(0x002, 6, 0); // border masking of this step
+				for (int tb = 0; tb < 3; tb++) fb[nxt][tb] = q[tb];
+			}
+			const float am = __int_as_float(__float_as_int(fa[cur]) & (int)tm[s % 3]);
+#pragma unroll
+			for (int tb = 0; tb < 3; tb++) acc[tb] = __builtin_amdgcn_mfma_f32_32x32x2f32(am, fb[cur][tb], acc[tb], 0, 0, 0);
+			__builtin_amdgcn_sched_group_barrier(0x002, 2, 0); // the mask and the next address
 			__builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-			__builtin_amdgcn_sched_group_barrier(0x100, 5, 0); // LDS reads of the next step
+			__builtin_amdgcn_sched_group_barrier(0x100, 6, 0); // LDS reads for the next two steps
 			__builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+			if (s == STEPS / 2 && more) C3_STORE_STAGE(buf ^ 1); // the other buffer was released by the last barrier
 		}
-		if (st + 1 < stEnd) C3_STORE_STAGE(buf ^ 1);
 		__syncthreads();
 	}
 #undef C3_LOAD_STAGE
@@ -438,7 +522,7 @@ conv3x3_dw_kernel(const Conv3x3Params p, const float *delta, uint32_t deltaBytes
 		for (int v = 0; v < 16; v++) {
 			const int o = o0 + ob * 32 + 8 * (v / 4) + 4 * khalf + (v % 4);
 			if (o >= p.I) continue;
-			float *dst = C + (size_t)o * out.ldc + c * 9 + tap0;
+			float *dst = C + (size_t)o * out.ldc + c * 9 + ta * 3;
 #pragma unroll
 			for (int tb = 0; tb < 3; tb++) dst[tb] = acc[tb][v];
 		}

@@ -16,7 +16,7 @@ static inline int check_conv(const char *fn, const fitre_conv_shape *s)
 	              "%s: output extent %dx%d does not follow from input %dx%d, k=%d s=%d p=%d", fn, s->outA, s->outB, s->inA,
 	              s->inB, s->ksize, s->stride, s->padding);
 	FITRE_REQUIRE(s->ksize < 256, "%s: window %d too large", fn, s->ksize);
-	double lim = 1073741823.0; /* operands are read through 32-bit byte offsets */
+	double lim = 1073741800.0; /* operands are read through 32-bit byte offsets, the last 16 bytes of the range mark invalid groups */
 	FITRE_REQUIRE((double)s->samples * s->inA * s->inB * s->inChannels < lim &&
 	                  (double)s->samples * s->outA * s->outB * s->outChannels < lim &&
 	                  (double)s->inChannels * s->ksize * s->ksize * s->outChannels < lim,

@@ -86,9 +86,13 @@ static bool c3_geometry(const fitre_conv_shape *s)
 static bool c3_pos_eligible(const fitre_conv_shape *s, bool dx)
 {
 	int cred = dx ? s->outChannels : s->inChannels;
-	return c3_geometry(s) && cred % kC3CB == 0;
+	return c3_geometry(s) && cred % kC3CB == 0 && c3_pad_window(s->inA, s->inB) <= (s->inB <= 32 ? 384 : 512);
 }
-static bool c3_dw_eligible(const fitre_conv_shape *s) { return c3_geometry(s) && s->inChannels >= 16 && s->outChannels >= 32; }
+static bool c3_dw_eligible(const fitre_conv_shape *s)
+{
+	return c3_geometry(s) && s->inChannels >= 16 && s->outChannels >= 32 && s->inB <= 32 &&
+	       ((long)s->samples * s->inA * s->inB) % kC3Stage == 0;
+}
 
 static BlockPlan c3_pos_plan(const fitre_conv_shape *s, bool dx)
 {
@@ -191,15 +195,15 @@ static int launch_c3_dw(const fitre_conv_shape *s, const float *x, const float *
 	if (grid.y > 65535 || grid.z > 65535) return fail(FITRE_E_UNSUPPORTED, "conv3x3 grid too large");
 	{
 		LaunchScope scope(FITRE_KC_CONV_DW, conv_flops(s), 4);
-		const bool narrow = s->inB <= 32;
+		const bool narrow = s->inB >= 2 && s->inB <= 16;
 		if (vecd && narrow)
-			conv3x3_dw_kernel<true, 32><<<grid, kC3DwThreads, 0, stream()>>>(p, delta, deltaBytes, part);
+			conv3x3_dw_kernel<true, 16><<<grid, kC3DwThreads, 0, stream()>>>(p, delta, deltaBytes, part);
 		else if (vecd)
-			conv3x3_dw_kernel<true, 64><<<grid, kC3DwThreads, 0, stream()>>>(p, delta, deltaBytes, part);
+			conv3x3_dw_kernel<true, 32><<<grid, kC3DwThreads, 0, stream()>>>(p, delta, deltaBytes, part);
 		else if (narrow)
-			conv3x3_dw_kernel<false, 32><<<grid, kC3DwThreads, 0, stream()>>>(p, delta, deltaBytes, part);
+			conv3x3_dw_kernel<false, 16><<<grid, kC3DwThreads, 0, stream()>>>(p, delta, deltaBytes, part);
 		else
-			conv3x3_dw_kernel<false, 64><<<grid, kC3DwThreads, 0, stream()>>>(p, delta, deltaBytes, part);
+			conv3x3_dw_kernel<false, 32><<<grid, kC3DwThreads, 0, stream()>>>(p, delta, deltaBytes, part);
 	}
 	if (plan.splits > 1) launch_splitk_reduce((const float *)ws, plan.splits, I, K, out);
 	return check_launch("conv3x3_dw_kernel");

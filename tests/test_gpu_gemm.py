@@ -36,6 +36,13 @@ CONV_CASES = [
     (1, 8, 8, 66, 66, 3, 1, 1),      # one wider: general engine
     (7, 48, 64, 3, 5, 3, 1, 1),      # odd extents, 105 positions
     (64, 64, 64, 2, 2, 3, 1, 1),     # 2x2 maps
+    # weight-gradient stages whose window starts in a different column every stage (64 % B != 0)
+    (64, 16, 32, 3, 5, 3, 1, 1),     # B = 5, 960 positions
+    (16, 24, 40, 4, 6, 3, 1, 1),     # B = 6, partial channel tiles
+    (8, 16, 32, 2, 24, 3, 1, 1),     # B = 24: the wide-row instantiation
+    (128, 16, 32, 1, 1, 3, 1, 1),    # 1x1 maps: only the centre tap sees data
+    (32, 16, 32, 2, 1, 3, 1, 1),     # single-column maps
+    (4, 16, 32, 1, 16, 3, 1, 1),     # single-row maps
 ]
 
 
