@@ -60,6 +60,8 @@ def gpu_leg(args):
 
     batch = 256
     dev = Device(0)
+    if args.serial:
+        L.check(L.hip.fitre_hip_lanes_enable(0))
     name = C.create_string_buffer(128)
     cus = C.c_int()
     L.check(L.hip.fitre_hip_device_info(C.byref(cus), None, None, None, None, name, 128))
@@ -227,6 +229,8 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
+    ap.add_argument("--serial", action="store_true",
+                    help="run every kernel on one stream (for kernel tracers: durations do not overlap)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (the reference path is single-device and every "

@@ -514,17 +514,29 @@ conv3x3_dw_kernel(const Conv3x3Params p, const float *delta, uint32_t deltaBytes
 #undef C3_LOAD_STAGE
 #undef C3_STORE_STAGE
 
-	// ---- store: dW[o][c][tap]; this wave holds taps (ta, 0..2) of 32 output x 32 input channels ----
+	// ---- store: dW[o][c][tap].  A wave holds taps (ta, 0..2) of 32 output x 32 input channels, i.e.
+	// runs of three words; the three waves of an output-channel block go through LDS together so that
+	// global memory sees whole rows of 32*9 consecutive words. --------------------------------------
 	float *C = out.C + (size_t)blockIdx.z * out.splitStride;
-	const int c = c0 + l32;
-	if (c < p.cred) {
+	float *stage = &Ds[0][0];
+	constexpr int ROW = kC3DwCin * 9, ROW_LD = ROW + 1;
+	static_assert(32 * ROW_LD <= 2 * (D_DUMMY + 4), "the output stage must fit the delta buffers");
+	const int validCols = ((p.cred - c0 < kC3DwCin) ? (p.cred - c0) : kC3DwCin) * 9;
+	for (int r = 0; r < 4; r++) {
+		if (r > 0) __syncthreads(); // the copy of the previous block is done
+		if (ob == r) {
 #pragma unroll
-		for (int v = 0; v < 16; v++) {
-			const int o = o0 + ob * 32 + 8 * (v / 4) + 4 * khalf + (v % 4);
-			if (o >= p.I) continue;
-			float *dst = C + (size_t)o * out.ldc + c * 9 + ta * 3;
+			for (int v = 0; v < 16; v++) {
+				float *dst = stage + (8 * (v / 4) + 4 * khalf + (v % 4)) * ROW_LD + l32 * 9 + ta * 3;
 #pragma unroll
-			for (int tb = 0; tb < 3; tb++) dst[tb] = acc[tb][v];
+				for (int tb = 0; tb < 3; tb++) dst[tb] = acc[tb][v];
+			}
+		}
+		__syncthreads();
+		for (int i = tid; i < 32 * ROW; i += T) {
+			const int row = i / ROW, col = i - row * ROW;
+			const int o = o0 + r * 32 + row;
+			if ((o < p.I) & (col < validCols)) C[(size_t)o * out.ldc + c0 * 9 + col] = stage[row * ROW_LD + col];
 		}
 	}
 }

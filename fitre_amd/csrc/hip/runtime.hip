@@ -15,6 +15,7 @@ constexpr int kLanes = 2;
 static hipStream_t g_lanes[kLanes] = { nullptr, nullptr };
 static hipStream_t g_stream = nullptr; // the selected lane
 static int g_lane = 0;
+static bool g_lanes_on = true;
 constexpr int kJoinEvents = 64;
 static hipEvent_t g_join[kJoinEvents];
 static int g_join_next = 0;
@@ -180,8 +181,18 @@ int fitre_hip_lane_select(int laneIndex)
 	FITRE_NEED_INIT();
 	FITRE_REQUIRE(laneIndex >= 0 && laneIndex < kLanes, "fitre_hip_lane_select: lane %d out of range", laneIndex);
 	// with per-launch accounting on, everything runs on lane 0 so that durations are not shared
-	g_lane = g_profile ? 0 : laneIndex;
+	g_lane = (g_profile || !g_lanes_on) ? 0 : laneIndex;
 	g_stream = g_lanes[g_lane];
+	return FITRE_OK;
+}
+
+int fitre_hip_lanes_enable(int on)
+{
+	FITRE_NEED_INIT();
+	for (int i = 0; i < kLanes; i++) FITRE_HIP_TRY(hipStreamSynchronize(g_lanes[i]));
+	g_lanes_on = (on != 0);
+	g_lane = 0;
+	g_stream = g_lanes[0];
 	return FITRE_OK;
 }
 

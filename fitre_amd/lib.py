@@ -87,6 +87,7 @@ HIP_API = {
     "fitre_hip_gemm": (i32, [i32, i32, i32, i32, i32, f32, vp, i32, vp, i32, f32, vp, i32, vp, vp, sz]),
     "fitre_hip_lane_select": (i32, [i32]),
     "fitre_hip_lane_wait": (i32, [i32, i32]),
+    "fitre_hip_lanes_enable": (i32, [i32]),
     "fitre_hip_kfac_conv_input_factor_workspace": (sz, [vp, i32]),
     "fitre_hip_kfac_conv_input_factor": (i32, [vp, vp, i32, vp, vp, sz]),
     "fitre_hip_kfac_gram_workspace": (sz, [i32, C.c_long]),

@@ -51,6 +51,9 @@ void *fitre_hip_stream(void);
  * lane selection is ignored and everything runs on lane 0, so that launch durations are unshared.
  * No counterpart in the reference, which runs on the null stream and synchronises after every launch. */
 int fitre_hip_lane_select(int lane);
+/* on = 0: every later fitre_hip_lane_select() picks lane 0 (strictly serial execution, e.g. under a
+ * kernel tracer whose per-kernel durations should not overlap); on = 1 (the default) restores lanes. */
+int fitre_hip_lanes_enable(int on);
 int fitre_hip_lane_wait(int waiter, int signaller);
 
 /* ---------------- memory (device/cuda_utils.c; device/cuda_utils.h:15-26) ---------------- */
