@@ -42,6 +42,18 @@ MFMA_CLASSES = ("conv_dw", "conv_dx", "conv_fwd", "fc_gemm", "kfac_factor")
 TILES = {0: "", 1: "64x64", 2: "64x128", 3: "128x64", 4: "128x128"}
 
 
+def measured_traffic(kernel):
+    """HBM bytes per launch of `kernel` as measured with hardware counters in a separate profiler run;
+    the figures and the commands behind them are kept as text under profiles/.  None if not on record."""
+    import glob
+    for path in sorted(glob.glob(os.path.join(ROOT, "profiles", "*hbm_traffic.txt"))):
+        for line in open(path):
+            f = line.split()
+            if len(f) == 3 and f[0] == "traffic_bytes_per_launch" and f[1] == kernel:
+                return int(f[2])
+    return None
+
+
 def read_profile(L):
     rows = []
     for name, cls in KC.items():
@@ -130,7 +142,7 @@ def gpu_leg(args):
     dk = kernels[dom["kernel"]]
     roofline = dict(kernel=dom["kernel"], bound=dk["bound"], achieved=dk["achieved"],
                     peak=PEAK_MFMA_F32_TFLOPS if dk["bound"] == "mfma" else PEAK_HBM_GBS, unit=dk["unit"],
-                    frac=dk["frac"], traffic=None, avg_launch_us=dk["avg_us"],
+                    frac=dk["frac"], traffic=measured_traffic(dom["kernel"]), avg_launch_us=dk["avg_us"],
                     launches_per_step=dk["launches_per_step"])
     conv_rows = [r for r in rows if r["cls"] in ("conv_dw", "conv_dx")]
     conv_ms, conv_work = sum(r["ms"] for r in conv_rows), sum(r["work"] for r in conv_rows)
