@@ -99,9 +99,11 @@ def test_libraries_export_every_declared_symbol():
     for n in hip_names:
         assert hasattr(L.hip, n), n
         assert n in L.HIP_API, "ctypes table lacks %s" % n
-    cnn_names = _declared("fitre_cnn.h", r"\b([A-Za-z_]\w*)\s*\(") + _declared("fitre_shim.h", r"\b([A-Za-z_]\w*)\s*\(")
+    cnn_names = (_declared("fitre_cnn.h", r"\b([A-Za-z_]\w*)\s*\(") + _declared("fitre_shim.h", r"\b([A-Za-z_]\w*)\s*\(") +
+                 _declared("fitre_kfac.h", r"\b([A-Za-z_]\w*)\s*\("))
     cnn_names = [n for n in cnn_names if n not in ("defined",)]
     assert "cnnBackward" in cnn_names and "computeCNNGradient" in cnn_names and "copy_host_device" in cnn_names
+    assert "computeOmegaZFactors" in cnn_names and "computeKFACStorageIndices" in cnn_names
     for n in cnn_names:
         assert hasattr(L.cnn, n), n
     for g in ("BLOCK_SIZE", "WARP_SIZE", "DEVICE_NUM_BLOCKS"):
@@ -115,6 +117,27 @@ def test_struct_sizes_match_the_c_side():
     assert m.batchSize == 2 and m.bias == 1 and m.cLayers == 8
     assert m.convLayer[7].outChannels == 512 and m.poolLayer[7].outHeight == 1
     assert C.sizeof(CNN_MODEL) == 20 * 22 * 4 + 20 * 4 + 20 * 8 * 4 + 8 + 20 * 5 * 4 + 7 * 4 + 3 * 80 + 4 + 2 * 80
+
+
+def test_kfac_storage_indices_follow_the_reference_formula():
+    # solvers/kfac_utils.cu:17-45: input-side slots (K+1)^2 whatever the bias setting, output-side Cout^2
+    from fitre_amd.structs import KFAC_CURVATURE_INFO
+    for m in (build_vgg11(4), build_lenet(4, bias=0)):
+        info = KFAC_CURVATURE_INFO()
+        L.cnn.computeKFACStorageIndices(C.byref(m), C.byref(info))
+        o = l = 0
+        for i in range(m.cLayers):
+            c = m.convLayer[i]
+            assert (info.OmegaZOffsets[i], info.LambdaGOffsets[i]) == (o, l)
+            o += (c.inChannels * c.kSize ** 2 + 1) ** 2
+            l += c.outChannels ** 2
+        for i in range(m.lLayers):
+            f = m.fcLayer[i]
+            assert (info.OmegaZOffsets[m.cLayers + i], info.LambdaGOffsets[m.cLayers + i]) == (o, l)
+            o += (f.in_ + 1) ** 2
+            l += f.out ** 2
+        assert (info.OmegaZOffsets[m.cLayers + m.lLayers], info.LambdaGOffsets[m.cLayers + m.lLayers]) == (o, l)
+        assert L.cnn.kfacFactorsMemRequired(C.byref(m), 4) > 0
 
 
 def test_workspace_requirements_are_positive_and_modest():
