@@ -299,26 +299,29 @@ __device__ __forceinline__ void segment_range(long perChannel, long &lo, long &h
 	if (lo > perChannel) lo = perChannel;
 }
 
-// NOUT sums per (channel, segment): MODE 0: sum x; 1: sum x, sum x*y; 2: sum x, sum x^2
+// sums per (channel, segment): MODE 0: sum x; 1: sum x, sum x*y; 2: sum x, sum x^2;
+// 3: sum x, sum x*y, sum y (slots of four doubles instead of two)
 template <int MODE, bool VEC>
 __global__ void __launch_bounds__(kRedBlock)
 channel_partial_kernel(const float *x, const float *y, long perChannel, double *partial)
 {
 	__shared__ double lds[kRedBlock / kWave];
+	constexpr bool PAIR = (MODE == 1 || MODE == 3);
 	const int c = blockIdx.y;
 	const float *px = x + (size_t)c * perChannel;
-	const float *py = (MODE == 1) ? y + (size_t)c * perChannel : nullptr;
+	const float *py = PAIR ? y + (size_t)c * perChannel : nullptr;
 	long lo, hi;
 	segment_range(perChannel, lo, hi);
-	double s0 = 0.0, s1 = 0.0;
+	double s0 = 0.0, s1 = 0.0, s2 = 0.0;
 	if constexpr (VEC) {
 		for (long i = lo + 4 * (long)threadIdx.x; i + 3 < hi; i += 4 * kRedBlock) {
 			float4 a = *reinterpret_cast<const float4 *>(px + i);
 			float t0 = (a.x + a.y) + (a.z + a.w);
 			s0 += (double)t0;
-			if constexpr (MODE == 1) {
+			if constexpr (PAIR) {
 				float4 b = *reinterpret_cast<const float4 *>(py + i);
 				s1 += (double)(a.x * b.x) + (double)(a.y * b.y) + (double)(a.z * b.z) + (double)(a.w * b.w);
+				if constexpr (MODE == 3) s2 += (double)((b.x + b.y) + (b.z + b.w));
 			}
 			if constexpr (MODE == 2)
 				s1 += (double)a.x * a.x + (double)a.y * a.y + (double)a.z * a.z + (double)a.w * a.w;
@@ -327,24 +330,29 @@ channel_partial_kernel(const float *x, const float *y, long perChannel, double *
 		for (long i = tail + threadIdx.x; i < hi; i += kRedBlock) {
 			float a = px[i];
 			s0 += (double)a;
-			if constexpr (MODE == 1) s1 += (double)(a * py[i]);
+			if constexpr (PAIR) s1 += (double)(a * py[i]);
+			if constexpr (MODE == 3) s2 += (double)py[i];
 			if constexpr (MODE == 2) s1 += (double)a * a;
 		}
 	} else {
 		for (long i = lo + threadIdx.x; i < hi; i += kRedBlock) {
 			float a = px[i];
 			s0 += (double)a;
-			if constexpr (MODE == 1) s1 += (double)(a * py[i]);
+			if constexpr (PAIR) s1 += (double)(a * py[i]);
+			if constexpr (MODE == 3) s2 += (double)py[i];
 			if constexpr (MODE == 2) s1 += (double)a * a;
 		}
 	}
 	double t0 = block_sum<kRedBlock>(s0, lds);
-	double t1 = 0.0;
+	double t1 = 0.0, t2 = 0.0;
 	if constexpr (MODE != 0) t1 = block_sum<kRedBlock>(s1, lds);
+	if constexpr (MODE == 3) t2 = block_sum<kRedBlock>(s2, lds);
 	if (threadIdx.x == 0) {
-		size_t slot = ((size_t)c * gridDim.x + blockIdx.x) * 2;
+		constexpr int SLOT = (MODE == 3) ? 4 : 2;
+		size_t slot = ((size_t)c * gridDim.x + blockIdx.x) * SLOT;
 		partial[slot] = t0;
 		partial[slot + 1] = t1;
+		if constexpr (MODE == 3) partial[slot + 2] = t2;
 	}
 }
 
@@ -405,57 +413,100 @@ bn_normalize_kernel(const float *x, const float *mean, const float *variance, fl
 	}
 }
 
-// batch-norm backward, elementwise part; also leaves the per-segment sum of the
-// result in partialOut (for the bias gradient).
+// dx_i = (m*delta_i - sum(delta) - zhat_i * sum(delta*zhat)) / (m * sqrt(var + eps)), and its channel sum
+// (the bias gradient) in closed form: -sum(delta*zhat) * sum(zhat) / (m * sqrt(var + eps)).
+__device__ __forceinline__ float bn_backward_value(float m, float d, float z, float sum1, float sum2, float scale)
+{
+	return (m * d - sum1 - sum2 * z) * scale;
+}
+
+// batch-norm backward, elementwise part, from the per-segment sums of channel_partial_kernel<3>
 template <bool VEC>
 __global__ void __launch_bounds__(kRedBlock)
 bn_backward_apply_kernel(const float *delta, const float *zhat, const float *variance, const double *partial,
-                         int segmentsIn, float epsilon, long perChannel, float *out, double *partialOut)
+                         int segmentsIn, float epsilon, long perChannel, float *out, float *biasGrad)
 {
-	__shared__ double lds[kRedBlock / kWave];
 	const int c = blockIdx.y;
-	double d1 = 0.0, d2 = 0.0;
+	double d1 = 0.0, d2 = 0.0, d3 = 0.0;
 	for (int k = 0; k < segmentsIn; k++) {
-		d1 += partial[((size_t)c * segmentsIn + k) * 2];
-		d2 += partial[((size_t)c * segmentsIn + k) * 2 + 1];
+		const double *slot = partial + ((size_t)c * segmentsIn + k) * 4;
+		d1 += slot[0], d2 += slot[1], d3 += slot[2];
 	}
 	const float m = (float)perChannel;
 	const float sum1 = (float)d1, sum2 = (float)d2;
 	const float scale = 1.f / (m * sqrtf(epsilon + variance[c]));
+	if (biasGrad && blockIdx.x == 0 && threadIdx.x == 0) biasGrad[c] = (float)(-d2 * d3 * (double)scale);
 	const float *pd = delta + (size_t)c * perChannel;
 	const float *pz = zhat + (size_t)c * perChannel;
 	float *po = out + (size_t)c * perChannel;
 	long lo, hi;
 	segment_range(perChannel, lo, hi);
-	double acc = 0.0;
 	if constexpr (VEC) {
 		for (long i = lo + 4 * (long)threadIdx.x; i + 3 < hi; i += 4 * kRedBlock) {
 			float4 d = *reinterpret_cast<const float4 *>(pd + i);
 			float4 z = *reinterpret_cast<const float4 *>(pz + i);
 			float4 r;
-			r.x = (m * d.x - sum1 - sum2 * z.x) * scale;
-			r.y = (m * d.y - sum1 - sum2 * z.y) * scale;
-			r.z = (m * d.z - sum1 - sum2 * z.z) * scale;
-			r.w = (m * d.w - sum1 - sum2 * z.w) * scale;
+			r.x = bn_backward_value(m, d.x, z.x, sum1, sum2, scale);
+			r.y = bn_backward_value(m, d.y, z.y, sum1, sum2, scale);
+			r.z = bn_backward_value(m, d.z, z.z, sum1, sum2, scale);
+			r.w = bn_backward_value(m, d.w, z.w, sum1, sum2, scale);
 			*reinterpret_cast<float4 *>(po + i) = r;
-			acc += (double)((r.x + r.y) + (r.z + r.w));
 		}
 		long tail = lo + ((hi - lo) / 4) * 4;
-		for (long i = tail + threadIdx.x; i < hi; i += kRedBlock) {
-			float r = (m * pd[i] - sum1 - sum2 * pz[i]) * scale;
-			po[i] = r;
-			acc += (double)r;
+		for (long i = tail + threadIdx.x; i < hi; i += kRedBlock) po[i] = bn_backward_value(m, pd[i], pz[i], sum1, sum2, scale);
+	} else {
+		for (long i = lo + threadIdx.x; i < hi; i += kRedBlock) po[i] = bn_backward_value(m, pd[i], pz[i], sum1, sum2, scale);
+	}
+}
+
+// The same for short channels: one workgroup per channel sums, then applies (the second read of
+// delta and zhat comes from the cache), one launch instead of two.
+constexpr long kBnSmallChannel = 4096;
+template <bool VEC>
+__global__ void __launch_bounds__(kRedBlock)
+bn_backward_small_kernel(const float *delta, const float *zhat, const float *variance, float epsilon, long perChannel,
+                         float *out, float *biasGrad)
+{
+	__shared__ double lds[kRedBlock / kWave];
+	const int c = blockIdx.x;
+	const float *pd = delta + (size_t)c * perChannel;
+	const float *pz = zhat + (size_t)c * perChannel;
+	float *po = out + (size_t)c * perChannel;
+	double s1 = 0.0, s2 = 0.0, s3 = 0.0;
+	if constexpr (VEC) {
+		for (long i = 4 * (long)threadIdx.x; i < perChannel; i += 4 * kRedBlock) {
+			float4 d = *reinterpret_cast<const float4 *>(pd + i);
+			float4 z = *reinterpret_cast<const float4 *>(pz + i);
+			s1 += (double)((d.x + d.y) + (d.z + d.w));
+			s2 += (double)(d.x * z.x) + (double)(d.y * z.y) + (double)(d.z * z.z) + (double)(d.w * z.w);
+			s3 += (double)((z.x + z.y) + (z.z + z.w));
 		}
 	} else {
-		for (long i = lo + threadIdx.x; i < hi; i += kRedBlock) {
-			float r = (m * pd[i] - sum1 - sum2 * pz[i]) * scale;
-			po[i] = r;
-			acc += (double)r;
+		for (long i = threadIdx.x; i < perChannel; i += kRedBlock) {
+			float d = pd[i], z = pz[i];
+			s1 += (double)d, s2 += (double)(d * z), s3 += (double)z;
 		}
 	}
-	if (partialOut) {
-		double t = block_sum<kRedBlock>(acc, lds);
-		if (threadIdx.x == 0) partialOut[((size_t)c * gridDim.x + blockIdx.x) * 2] = t;
+	const double d1 = block_sum<kRedBlock>(s1, lds);
+	const double d2 = block_sum<kRedBlock>(s2, lds);
+	const double d3 = block_sum<kRedBlock>(s3, lds);
+	const float m = (float)perChannel;
+	const float sum1 = (float)d1, sum2 = (float)d2;
+	const float scale = 1.f / (m * sqrtf(epsilon + variance[c]));
+	if (biasGrad && threadIdx.x == 0) biasGrad[c] = (float)(-d2 * d3 * (double)scale);
+	if constexpr (VEC) {
+		for (long i = 4 * (long)threadIdx.x; i < perChannel; i += 4 * kRedBlock) {
+			float4 d = *reinterpret_cast<const float4 *>(pd + i);
+			float4 z = *reinterpret_cast<const float4 *>(pz + i);
+			float4 r;
+			r.x = bn_backward_value(m, d.x, z.x, sum1, sum2, scale);
+			r.y = bn_backward_value(m, d.y, z.y, sum1, sum2, scale);
+			r.z = bn_backward_value(m, d.z, z.z, sum1, sum2, scale);
+			r.w = bn_backward_value(m, d.w, z.w, sum1, sum2, scale);
+			*reinterpret_cast<float4 *>(po + i) = r;
+		}
+	} else {
+		for (long i = threadIdx.x; i < perChannel; i += kRedBlock) po[i] = bn_backward_value(m, pd[i], pz[i], sum1, sum2, scale);
 	}
 }
 
@@ -748,20 +799,23 @@ int fitre_hip_batch_norm_backward(const float *delta, const float *zhat, const f
 	if (rc) return rc;
 	int S = segments_for(channels, perChannel);
 	double *partial = (double *)ws;
-	double *partialOut = partial + (size_t)channels * S * 2;
 	LaunchScope scope(FITRE_KC_BN_BWD, 12.0 * (double)channels * (double)perChannel + 8.0 * channels);
 	dim3 grid(S, channels);
 	bool vec = aligned16(delta) && aligned16(zhat) && aligned16(out) && (perChannel % 4 == 0);
-	if (vec) {
-		channel_partial_kernel<1, true><<<grid, kRedBlock, 0, stream()>>>(delta, zhat, perChannel, partial);
+	if (perChannel <= kBnSmallChannel && channels >= 128) {
+		if (vec)
+			bn_backward_small_kernel<true><<<channels, kRedBlock, 0, stream()>>>(delta, zhat, variance, epsilon, perChannel, out, biasGrad);
+		else
+			bn_backward_small_kernel<false><<<channels, kRedBlock, 0, stream()>>>(delta, zhat, variance, epsilon, perChannel, out, biasGrad);
+	} else if (vec) {
+		channel_partial_kernel<3, true><<<grid, kRedBlock, 0, stream()>>>(delta, zhat, perChannel, partial);
 		bn_backward_apply_kernel<true><<<grid, kRedBlock, 0, stream()>>>(delta, zhat, variance, partial, S, epsilon, perChannel,
-		                                                                 out, biasGrad ? partialOut : nullptr);
+		                                                                 out, biasGrad);
 	} else {
-		channel_partial_kernel<1, false><<<grid, kRedBlock, 0, stream()>>>(delta, zhat, perChannel, partial);
+		channel_partial_kernel<3, false><<<grid, kRedBlock, 0, stream()>>>(delta, zhat, perChannel, partial);
 		bn_backward_apply_kernel<false><<<grid, kRedBlock, 0, stream()>>>(delta, zhat, variance, partial, S, epsilon, perChannel,
-		                                                                  out, biasGrad ? partialOut : nullptr);
+		                                                                  out, biasGrad);
 	}
-	if (biasGrad) channel_finish_kernel<<<blocks_for(channels, 64), 64, 0, stream()>>>(partialOut, S, 0, channels, biasGrad);
 	return check_launch("batch_norm_backward");
 }
 

@@ -237,7 +237,8 @@ def test_bn_backward_reference_known_answer(dev):
     np.testing.assert_allclose(dev.download(out, 4), g["expected"], rtol=2e-5)
 
 
-@pytest.mark.parametrize("Cn,N,A,B,mis", [(3, 5, 4, 6, 0), (64, 8, 32, 32, 0), (6, 37, 28, 28, 0), (5, 3, 3, 3, 1), (16, 1024, 28, 28, 0)])
+@pytest.mark.parametrize("Cn,N,A,B,mis", [(3, 5, 4, 6, 0), (64, 8, 32, 32, 0), (6, 37, 28, 28, 0), (5, 3, 3, 3, 1), (16, 1024, 28, 28, 0),
+                                          (128, 4, 8, 8, 0), (130, 3, 5, 7, 1), (512, 256, 4, 4, 0)])  # one-workgroup-per-channel backward
 def test_batch_norm_forward_backward(dev, oracle64, Cn, N, A, B, mis):
     per = N * A * B
     rng = np.random.default_rng(per % 1000)
