@@ -37,8 +37,9 @@ PEAK_MFMA_F32_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
 
 KC = dict(conv_dw=0, conv_dx=1, conv_fwd=2, fc_gemm=3, splitk_reduce=4, bn_bwd=5, bn_fwd=6, pool_bwd=7, pool_fwd=8,
-          act_bwd=9, act_fwd=10, bias_grad=11, softmax=12, permute=13, blas1=14, pool_act_bwd=15, kfac_factor=16)
-MFMA_CLASSES = ("conv_dw", "conv_dx", "conv_fwd", "fc_gemm", "kfac_factor")
+          act_bwd=9, act_fwd=10, bias_grad=11, softmax=12, permute=13, blas1=14, pool_act_bwd=15, kfac_factor=16,
+          spd_inverse=17)
+MFMA_CLASSES = ("conv_dw", "conv_dx", "conv_fwd", "fc_gemm", "kfac_factor", "spd_inverse")
 TILES = {0: "", 1: "64x64", 2: "64x128", 3: "128x64", 4: "128x128"}
 
 

@@ -14,6 +14,14 @@ constexpr int kWave = 64;
 void set_error(const char *fmt, ...);
 int fail(int code, const char *fmt, ...);
 hipStream_t stream(); // the selected lane
+// Column-major product C(MxN) = alpha*op(A)*op(B) + beta*C on the tile engine (defined with
+// fitre_hip_gemm).  flags: kGemmMirror = the product is symmetric (M == N, same operand on
+// both sides): compute the tiles on and above the diagonal and mirror them; kGemmTriK = both
+// operands are zero where the reduction index is below their row / column index.
+constexpr int kGemmMirror = 1, kGemmTriK = 2;
+int gemm_ex(int transA, int transB, int M, int N, int K, float alpha, const float *A, int lda, const float *B, int ldb,
+            float beta, float *C, int ldc, const float *bias, int flags, int kernelClass, void *ws, size_t wsBytes);
+size_t gemm_ex_workspace(int M, int N, int K, int flags);
 int lane();           // its index (0 or 1)
 bool ready();
 

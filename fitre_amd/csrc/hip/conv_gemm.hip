@@ -209,6 +209,39 @@ static int launch_c3_dw(const fitre_conv_shape *s, const float *x, const float *
 	return check_launch("conv3x3_dw_kernel");
 }
 
+size_t gemm_ex_workspace(int M, int N, int K, int flags)
+{
+	if (M <= 0 || N <= 0 || K <= 0) return 0;
+	return plan_gemm(N, M, K, (flags & kGemmMirror) != 0).wsBytes;
+}
+
+int gemm_ex(int transA, int transB, int M, int N, int K, float alpha, const float *A, int lda, const float *B, int ldb,
+            float beta, float *C, int ldc, const float *bias, int flags, int kernelClass, void *ws, size_t wsBytes)
+{
+	FITRE_REQUIRE(A && B && C, "fitre_hip_gemm: null pointer");
+	FITRE_REQUIRE(M > 0 && N > 0 && K > 0, "fitre_hip_gemm: non-positive shape %d x %d x %d", M, N, K);
+	FITRE_REQUIRE((transA == 0 || transA == 1) && (transB == 0 || transB == 1), "fitre_hip_gemm: bad transpose flags");
+	FITRE_REQUIRE(lda >= (transA ? K : M) && ldb >= (transB ? N : K) && ldc >= M, "fitre_hip_gemm: leading dimension too small");
+	const size_t aElems = (size_t)lda * (transA ? M : K), bElems = (size_t)ldb * (transB ? K : N);
+	FITRE_REQUIRE(aElems < ((size_t)1 << 30) && bElems < ((size_t)1 << 30), "fitre_hip_gemm: an operand exceeds 2^30 elements");
+	const int I = N, J = M, R = K;
+	GemmPlan plan = plan_gemm(I, J, R, (flags & kGemmMirror) != 0);
+	OutParams out{ C, (long)ldc, 0, nullptr, bias, alpha, beta, (flags & kGemmMirror) ? 1 : 0, (flags & kGemmTriK) ? 1 : 0 };
+	FITRE_REQUIRE(!(flags & kGemmMirror) || M == N, "gemm: a mirrored product must be square");
+	const double flops = 2.0 * (double)M * N * K;
+	// engine A(i = n, k): op(B)(k, n).  transB == 0: B[n*ldb + k] (contiguous along k); else B[k*ldb + n]
+	// engine B(j = m, k): op(A)(m, k).  transA == 0: A[k*lda + m] (contiguous along m); else A[m*lda + k]
+	PlainParams bk{ B, (uint32_t)(bElems * sizeof(float)), ldb, I };
+	PlainParams br = bk;
+	PlainParams ar{ A, (uint32_t)(aElems * sizeof(float)), lda, J };
+	PlainParams ak = ar;
+	if (!transB && !transA) return launch_gemm<PlainKContig, PlainRowContig>(bk, ar, out, I, J, R, plan, ws, wsBytes, kernelClass, flops);
+	if (!transB && transA) return launch_gemm<PlainKContig, PlainKContig>(bk, ak, out, I, J, R, plan, ws, wsBytes, kernelClass, flops);
+	if (transB && !transA) return launch_gemm<PlainRowContig, PlainRowContig>(br, ar, out, I, J, R, plan, ws, wsBytes, kernelClass, flops);
+	return launch_gemm<PlainRowContig, PlainKContig>(br, ak, out, I, J, R, plan, ws, wsBytes, kernelClass, flops);
+}
+
+
 } // namespace fitre
 
 using namespace fitre;
@@ -303,36 +336,13 @@ int fitre_hip_conv_input_grad(const fitre_conv_shape *s, const float *delta, con
 // ---- general column-major GEMM ---------------------------------------------------
 // C(MxN) column-major is C[n*ldc + m]: engine i = n (column), j = m (row, contiguous).
 // A operand of the engine (rows i = n) is op(B)^T, B operand (rows j = m) is op(A).
-size_t fitre_hip_gemm_workspace(int M, int N, int K)
-{
-	if (M <= 0 || N <= 0 || K <= 0) return 0;
-	return plan_gemm(N, M, K).wsBytes;
-}
+size_t fitre_hip_gemm_workspace(int M, int N, int K) { return gemm_ex_workspace(M, N, K, 0); }
 
 int fitre_hip_gemm(int transA, int transB, int M, int N, int K, float alpha, const float *A, int lda, const float *B, int ldb,
                    float beta, float *C, int ldc, const float *bias, void *ws, size_t wsBytes)
 {
 	FITRE_NEED_INIT();
-	FITRE_REQUIRE(A && B && C, "fitre_hip_gemm: null pointer");
-	FITRE_REQUIRE(M > 0 && N > 0 && K > 0, "fitre_hip_gemm: non-positive shape %d x %d x %d", M, N, K);
-	FITRE_REQUIRE((transA == 0 || transA == 1) && (transB == 0 || transB == 1), "fitre_hip_gemm: bad transpose flags");
-	FITRE_REQUIRE(lda >= (transA ? K : M) && ldb >= (transB ? N : K) && ldc >= M, "fitre_hip_gemm: leading dimension too small");
-	const size_t aElems = (size_t)lda * (transA ? M : K), bElems = (size_t)ldb * (transB ? K : N);
-	FITRE_REQUIRE(aElems < ((size_t)1 << 30) && bElems < ((size_t)1 << 30), "fitre_hip_gemm: an operand exceeds 2^30 elements");
-	const int I = N, J = M, R = K;
-	GemmPlan plan = plan_gemm(I, J, R);
-	OutParams out{ C, (long)ldc, 0, nullptr, bias, alpha, beta };
-	const double flops = 2.0 * (double)M * N * K;
-	// engine A(i = n, k): op(B)(k, n).  transB == 0: B[n*ldb + k] (contiguous along k); else B[k*ldb + n]
-	// engine B(j = m, k): op(A)(m, k).  transA == 0: A[k*lda + m] (contiguous along m); else A[m*lda + k]
-	PlainParams bk{ B, (uint32_t)(bElems * sizeof(float)), ldb, I };
-	PlainParams br = bk;
-	PlainParams ar{ A, (uint32_t)(aElems * sizeof(float)), lda, J };
-	PlainParams ak = ar;
-	if (!transB && !transA) return launch_gemm<PlainKContig, PlainRowContig>(bk, ar, out, I, J, R, plan, ws, wsBytes, FITRE_KC_FC_GEMM, flops);
-	if (!transB && transA) return launch_gemm<PlainKContig, PlainKContig>(bk, ak, out, I, J, R, plan, ws, wsBytes, FITRE_KC_FC_GEMM, flops);
-	if (transB && !transA) return launch_gemm<PlainRowContig, PlainRowContig>(br, ar, out, I, J, R, plan, ws, wsBytes, FITRE_KC_FC_GEMM, flops);
-	return launch_gemm<PlainRowContig, PlainKContig>(br, ak, out, I, J, R, plan, ws, wsBytes, FITRE_KC_FC_GEMM, flops);
+	return gemm_ex(transA, transB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, bias, 0, FITRE_KC_FC_GEMM, ws, wsBytes);
 }
 
 } // extern "C"

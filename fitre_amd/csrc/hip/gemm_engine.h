@@ -366,6 +366,9 @@ struct OutParams {
 	// diagonal are skipped, elements with j < i are not stored and every stored element with
 	// j > i is also written to C[j][i].  With split-K the mirroring happens in the reduction.
 	int mirror;
+	// Both operands are lower triangular in the reduction index (element (row, k) is zero for
+	// k < row): the reduction of a tile starts at the larger of its two first rows.
+	int triK;
 };
 
 // ---------------------------------------------------------------------------
@@ -386,9 +389,13 @@ mfma_gemm_kernel(const typename OpA::Params pa, const typename OpB::Params pb, c
 	const int lane = tid & 63;
 	const int wave = tid >> 6;
 	const int i0 = blockIdx.y * BM, j0 = blockIdx.x * BN;
-	const int kbeg = blockIdx.z * kChunk;
+	int kbeg = blockIdx.z * kChunk;
 	const int kend = (kbeg + kChunk < R) ? kbeg + kChunk : R;
 	if (out.mirror && j0 + BN <= i0) return; // the mirror tile produces these elements
+	if (out.triK) {
+		const int first = ((i0 > j0) ? i0 : j0) & ~(BK - 1);
+		kbeg = (kbeg > first) ? kbeg : first;
+	}
 
 	OpA opA;
 	OpB opB;

@@ -94,7 +94,8 @@ enum fitre_kernel_class {
 	FITRE_KC_BLAS1 = 14,
 	FITRE_KC_POOL_ACT_BWD = 15,
 	FITRE_KC_KFAC_FACTOR = 16,
-	FITRE_KC_COUNT = 17
+	FITRE_KC_SPD_INVERSE = 17,
+	FITRE_KC_COUNT = 18
 };
 int fitre_hip_profile_enable(int on); /* on=1 clears the counters and starts; on=0 stops */
 /* launches, summed milliseconds and summed algorithmic work of one class (syncs first) */
@@ -259,6 +260,18 @@ int fitre_hip_kfac_fc_input_factor(const float *z, int in, int samples, int with
  * out x samples; order out. */
 int fitre_hip_kfac_fc_output_factor(const float *delta, int out, int samples, float *factor, void *ws,
                                     size_t wsBytes);
+
+/* inverse = (matrix + shift*I)^-1 for a symmetric positive definite matrix of order n (column-major ==
+ * row-major, full storage in and out): blocked Cholesky, inverse of the factor, symmetric product.
+ * Replaces computeMatrixInverseCusolver (solvers/kfac_inverses.cu:133-186: identity right-hand side,
+ * ker_add_regularization with lambda + dampGamma, cusolverDnDpotrf, cusolverDnDpotrs).
+ * ws: 256-byte aligned, at least fitre_hip_spd_inverse_workspace(n) bytes.  info (host pointer, may be
+ * NULL): receives 0, or the 1-based index of the first non-positive pivot -- the call then also fails
+ * with FITRE_E_ARGUMENT, as the reference exits on devInfo != 0; with info == NULL the call does not wait
+ * for the device and a failed factorization shows as NaNs in the result. */
+size_t fitre_hip_spd_inverse_workspace(int n);
+int fitre_hip_spd_inverse(const float *matrix, int n, float shift, float *inverse, void *ws, size_t wsBytes,
+                          int *info);
 
 #ifdef __cplusplus
 }

@@ -690,6 +690,49 @@ void oracle_kfac_fc_output_factor(const real *delta, int out, int samples, real 
 	for (size_t i = 0; i < (size_t)out * out; i++) factor[i] *= (real)samples;
 }
 
+/* solvers/kfac_inverses.cu:133-186 (computeMatrixInverseCusolver): identity right-hand side, copy of
+ * the matrix with lambda + dampGamma added to the diagonal, Cholesky factorization of the lower
+ * triangle (what cusolverDnDpotrf computes: A = L L^T, column by column) and the two triangular
+ * solves of cusolverDnDpotrs for every column of the identity.  matrix and inverse are n x n
+ * column-major; devScratch holds n*n reals.  Returns 0, or the 1-based index of the first
+ * non-positive pivot (cusolver's devInfo), in which case inverse is not meaningful. */
+int oracle_matrix_inverse(const real *matrix, real *inverse, int n, real lambda, real dampGamma, real *devScratch)
+{
+	real *L = devScratch;
+	for (size_t i = 0; i < (size_t)n * n; i++) inverse[i] = 0;
+	for (int i = 0; i < n; i++) inverse[(size_t)i * n + i] = 1;
+	memcpy(L, matrix, sizeof(real) * (size_t)n * n);
+	for (int i = 0; i < n; i++) L[(size_t)i * n + i] += lambda + dampGamma;
+	for (int j = 0; j < n; j++) {
+		real d = L[(size_t)j * n + j];
+		for (int k = 0; k < j; k++) d -= L[(size_t)k * n + j] * L[(size_t)k * n + j];
+		if (!(d > 0)) return j + 1;
+		d = (real)sqrt((double)d);
+		L[(size_t)j * n + j] = d;
+#pragma omp parallel for schedule(static)
+		for (int i = j + 1; i < n; i++) {
+			real v = L[(size_t)j * n + i];
+			for (int k = 0; k < j; k++) v -= L[(size_t)k * n + i] * L[(size_t)k * n + j];
+			L[(size_t)j * n + i] = v / d;
+		}
+	}
+#pragma omp parallel for schedule(static)
+	for (int c = 0; c < n; c++) {
+		real *x = inverse + (size_t)c * n;
+		for (int i = 0; i < n; i++) { /* L y = e_c */
+			real v = x[i];
+			for (int k = 0; k < i; k++) v -= L[(size_t)k * n + i] * x[k];
+			x[i] = v / L[(size_t)i * n + i];
+		}
+		for (int i = n - 1; i >= 0; i--) { /* L^T x = y */
+			real v = x[i];
+			for (int k = i + 1; k < n; k++) v -= L[(size_t)i * n + k] * x[k];
+			x[i] = v / L[(size_t)i * n + i];
+		}
+	}
+	return 0;
+}
+
 /* ------------------------------------------------------------------ */
 /* whole model                                                         */
 /* ------------------------------------------------------------------ */

@@ -159,6 +159,13 @@ class Oracle:
         self.lib.oracle_kfac_fc_output_factor(self.p(delta), n_out, samples, self.p(factor))
         return factor.reshape(n_out, n_out)
 
+    def matrix_inverse(self, matrix, n, lam, gamma):
+        """(info, inverse) of matrix + (lam + gamma) I."""
+        matrix = self.arr(matrix)
+        inverse, scratch = self.zeros(n * n), self.zeros(n * n)
+        info = self.lib.oracle_matrix_inverse(self.p(matrix), self.p(inverse), n, self.r(lam), self.r(gamma), self.p(scratch))
+        return info, inverse.reshape(n, n)
+
     def activation_forward(self, act, x):
         x = self.arr(x).copy()
         rc = self.lib.oracle_activation_forward(act, self.p(x), C.c_size_t(x.size))

@@ -175,3 +175,49 @@ def test_model_factor_passes(dev, oracle64, name):
     for q in (omega, lam, ws):
         dev.free(q)
     gm.release()
+
+
+# ---------------------------------------------------------------------------- inverse of a factor
+def _spd(n, rng, cond):
+    q, _ = np.linalg.qr(rng.standard_normal((n, n)))
+    ev = np.geomspace(1.0, 1.0 / cond, n)
+    return ((q * ev) @ q.T).astype(np.float32)
+
+
+@pytest.mark.parametrize("n", [1, 3, 28, 64, 65, 129, 400, 577, 1153])
+def test_spd_inverse(dev, oracle64, n):
+    """(A + shift I)^-1 against the oracle's Cholesky inverse.  The error of an inverse computed in float32
+    grows with the condition number; the matrices here have condition ~50 after the shift and the
+    tolerance is the path's 1e-4."""
+    rng = np.random.default_rng(n)
+    a = _spd(n, rng, 1000.0)
+    a = ((a + a.T) / 2).astype(np.float32)
+    shift = 0.02
+    pa = dev.upload(a.reshape(-1))
+    out = dev.upload(np.full(n * n, np.nan, dtype=np.float32))
+    nb = hip.fitre_hip_spd_inverse_workspace(n)
+    ws = dev.alloc(nb)
+    info = C.c_int(-1)
+    L.check(hip.fitre_hip_spd_inverse(pa, n, shift, out, ws, nb, C.byref(info)))
+    assert info.value == 0
+    got = dev.download(out, n * n).reshape(n, n)
+    oinfo, want = oracle64.matrix_inverse(a.astype(np.float64), n, shift, 0.0)
+    assert oinfo == 0
+    assert rel_err(got, want) < TOL
+    assert np.array_equal(got, got.T)
+    resid = (a.astype(np.float64) + shift * np.eye(n)) @ got.astype(np.float64) - np.eye(n)
+    assert np.abs(resid).max() < 1e-4
+    for q in (pa, out, ws):
+        dev.free(q)
+
+
+def test_spd_inverse_reports_indefinite_matrix(dev):
+    a = np.array([[1.0, 2.0], [2.0, 1.0]], dtype=np.float32)
+    pa, out = dev.upload(a.reshape(-1)), dev.zeros(4)
+    nb = hip.fitre_hip_spd_inverse_workspace(2)
+    ws = dev.alloc(nb)
+    info = C.c_int(0)
+    assert hip.fitre_hip_spd_inverse(pa, 2, 0.0, out, ws, nb, C.byref(info)) == 2
+    assert info.value == 2
+    assert b"positive definite" in hip.fitre_hip_last_error()
+    assert hip.fitre_hip_spd_inverse(pa, 2, 0.0, out, ws, 16, C.byref(info)) == 4

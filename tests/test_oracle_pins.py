@@ -351,3 +351,39 @@ def test_kfac_output_and_fc_factors_against_numpy(oracle64):
     dl = rng.standard_normal((N, n_out))
     got = oracle64.kfac_fc_output_factor(dl.reshape(-1), n_out, N)
     np.testing.assert_allclose(got, dl.T @ dl * N, atol=1e-12)
+
+
+# ------------------------------------------------------------------ matrix inverse
+def spd_matrix(n, rng, cond=50.0):
+    q, _ = np.linalg.qr(rng.standard_normal((n, n)))
+    ev = np.geomspace(1.0, 1.0 / cond, n)
+    return (q * ev) @ q.T
+
+
+@pytest.mark.parametrize("n", [1, 2, 7, 64, 65, 200])
+def test_matrix_inverse_against_scipy_cholesky(oracle64, n):
+    import scipy.linalg
+    rng = np.random.default_rng(n)
+    a = spd_matrix(n, rng)
+    lam, gamma = 1e-3, 2e-2
+    info, inv = oracle64.matrix_inverse(a, n, lam, gamma)
+    assert info == 0
+    shifted = a + (lam + gamma) * np.eye(n)
+    want = scipy.linalg.cho_solve(scipy.linalg.cho_factor(shifted, lower=True), np.eye(n))
+    np.testing.assert_allclose(inv, want, rtol=0, atol=1e-11 * np.abs(want).max())
+    np.testing.assert_allclose(shifted @ inv, np.eye(n), atol=1e-11)
+    np.testing.assert_allclose(inv, inv.T, atol=1e-12 * np.abs(inv).max())
+
+
+def test_matrix_inverse_closed_form_and_failure(oracle64):
+    # diagonal matrix: the damping enters every pivot
+    d = np.array([4.0, 1.0, 0.25])
+    info, inv = oracle64.matrix_inverse(np.diag(d), 3, 0.5, 0.25)
+    assert info == 0
+    np.testing.assert_allclose(inv, np.diag(1.0 / (d + 0.75)), atol=1e-15)
+    # 2x2 with a known inverse
+    info, inv = oracle64.matrix_inverse(np.array([[2.0, 1.0], [1.0, 2.0]]), 2, 0.0, 0.0)
+    np.testing.assert_allclose(inv, np.array([[2.0, -1.0], [-1.0, 2.0]]) / 3.0, atol=1e-15)
+    # indefinite: the second pivot is 1 - 4 < 0, reported 1-based like cusolver's devInfo
+    info, _ = oracle64.matrix_inverse(np.array([[1.0, 2.0], [2.0, 1.0]]), 2, 0.0, 0.0)
+    assert info == 2
