@@ -187,13 +187,45 @@ def kfac_leg(L, dev, gm, model, batch, passes):
     L.check(L.hip.fitre_hip_profile_enable(0))
     rows = [r for r in read_profile(L) if r["cls"] == "kfac_factor"]
     ms, work = sum(r["ms"] for r in rows), sum(r["work"] for r in rows)
-    for q in (omega, lam, ws):
-        dev.free(q)
     rate = work / (ms * 1e-3) / 1e12 if ms else 0.0
-    return dict(ms_per_pass=round(wall_ms, 4), kernel_ms_per_pass=round(ms / passes, 4),
-                gflop_per_pass=round(work / passes / 1e9, 2), achieved=round(rate, 2), unit="TFLOP/s",
-                frac=round(rate / PEAK_MFMA_F32_TFLOPS, 4),
-                note="upper-triangle flops n(n+1)*positions; all %d layers, both sides" % last)
+    out = dict(ms_per_pass=round(wall_ms, 4), kernel_ms_per_pass=round(ms / passes, 4),
+               gflop_per_pass=round(work / passes / 1e9, 2), achieved=round(rate, 2), unit="TFLOP/s",
+               frac=round(rate / PEAK_MFMA_F32_TFLOPS, 4),
+               note="upper-triangle flops n(n+1)*positions; all %d layers, both sides" % last)
+
+    # factors + damped inverses of every layer, then the natural gradient of the gradient in HBM
+    oinv, linv = omega, lam  # the factor storage is free again: the full passes build factors in scratch
+    ngrad = dev.zeros(model.pSize)
+    info.regLambda, info.dampGamma = 1e-3, 1e-1
+    info.OmegaZInv, info.LambdaGInv = oinv.value, linv.value
+    info.gradient, info.nGradient = gm.grad.value, ngrad.value
+    need = max(L.cnn.kfacInverseMemRequired(C.byref(model), batch), L.cnn.kfacNaturalGradientMemRequired(C.byref(model)))
+    ws2 = dev.alloc(4 * need + 512)
+
+    def inverses():
+        L.cnn.computeOmegaZ(C.byref(info), C.byref(model), C.byref(gm.data), batch, None, gm.z, oinv, model.zOffsets,
+                            model.zztOffsets, ws2, None)
+        L.cnn.computeLambdaDelta(C.byref(info), C.byref(model), batch, gm.dx, None, linv, model.zOffsets, model.zztOffsets,
+                                 ws2, None)
+
+    inverses()
+    dev.sync()
+    t0 = time.perf_counter()
+    inverses()
+    dev.sync()
+    out["factors_and_inverses_ms"] = round(1e3 * (time.perf_counter() - t0), 3)
+    L.cnn.computeNaturalGradient(C.byref(model), C.byref(info), ws2, None)
+    dev.sync()
+    t0 = time.perf_counter()
+    for _ in range(passes):
+        L.cnn.computeNaturalGradient(C.byref(model), C.byref(info), ws2, None)
+    dev.sync()
+    out["natural_gradient_ms"] = round(1e3 * (time.perf_counter() - t0) / passes, 4)
+    out["natural_gradient_finite"] = bool(np.isfinite(dev.download(ngrad, model.pSize)).all())
+    out["damping"] = 1e-3 + 1e-1
+    for q in (omega, lam, ws, ws2, ngrad):
+        dev.free(q)
+    return out
 
 
 def cpu_leg(batch=64, repeats=10):

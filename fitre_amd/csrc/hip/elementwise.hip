@@ -229,6 +229,17 @@ __global__ void __launch_bounds__(256) row_sum_kernel(const float *mat, int rows
 	}
 }
 
+// dst[c*ldd + r] = src[c*lds + r] for r < rows, c < cols
+__global__ void __launch_bounds__(256) copy_2d_kernel(const float *src, long lds_, float *dst, long ldd, int rows, int cols)
+{
+	const long total = (long)rows * cols;
+	const long stride = (long)gridDim.x * blockDim.x;
+	for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
+		const long c = idx / rows, r = idx - c * rows;
+		dst[c * ldd + r] = src[c * lds_ + r];
+	}
+}
+
 } // namespace fitre
 
 using namespace fitre;
@@ -322,6 +333,15 @@ int fitre_hip_add_channel_bias(float *x, int channels, long perChannel, const fl
 	add_channel_bias_kernel<<<grid, 256, 0, stream()>>>(x, perChannel, bias);
 	return check_launch("add_channel_bias_kernel");
 }
+int fitre_hip_copy_2d(float *dst, long ldd, const float *src, long lds_, int rows, int cols)
+{
+	EW_CHECK("fitre_hip_copy_2d", dst && src && rows > 0 && cols > 0);
+	FITRE_REQUIRE(ldd >= 1 && lds_ >= 1, "fitre_hip_copy_2d: non-positive leading dimension");
+	LaunchScope scope(FITRE_KC_BLAS1, 8.0 * (double)rows * cols);
+	copy_2d_kernel<<<blocks_for((long)rows * cols, 512, 8192), 256, 0, stream()>>>(src, lds_, dst, ldd, rows, cols);
+	return check_launch("copy_2d_kernel");
+}
+
 int fitre_hip_row_sum(const float *mat, int rows, int cols, float *out)
 {
 	EW_CHECK("fitre_hip_row_sum", mat && out && rows > 0 && cols > 0);

@@ -137,3 +137,201 @@ void computeLambdaDeltaFactors(KFAC_CURVATURE_INFO *kfac_info, CNN_MODEL *model,
 	}
 	HIP_CALL(fitre_hip_sync());
 }
+
+/* ---- inverses ------------------------------------------------------------------------------ */
+
+void computeMatrixInverse(real *matrix, real *inverse, int n, real *devPtr, real lambda, real dampGamma)
+{
+	int info = -1;
+	int rc = fitre_hip_spd_inverse(matrix, n, lambda + dampGamma, inverse, devPtr, fitre_hip_spd_inverse_workspace(n), &info);
+	if (rc != FITRE_OK) {
+		if (info > 0)
+			fprintf(stderr, "We have a problem with the LU factorization ... %d\n", info);
+		else
+			fprintf(stderr, "computeMatrixInverse: error %d: %s\n", rc, fitre_hip_last_error());
+		exit(-1);
+	}
+}
+
+static size_t round_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+/* layout of the scratch of the two inverse passes: [factor | workspace of its product or inverse] */
+static size_t inverse_scratch_bytes(const CNN_MODEL *model, int samples, size_t *factorBytes)
+{
+	size_t order = 1, ws = factor_ws_bytes(model, samples);
+	for (int l = 0; l < model->cLayers; l++) {
+		const CONV_LAYER *c = &model->convLayer[l];
+		size_t k = (size_t)c->inChannels * c->kSize * c->kSize + 1;
+		order = max_sz(order, max_sz(k, (size_t)c->outChannels));
+	}
+	for (int l = 0; l < model->lLayers; l++)
+		order = max_sz(order, max_sz((size_t)model->fcLayer[l].in + 1, (size_t)model->fcLayer[l].out));
+	ws = max_sz(ws, fitre_hip_spd_inverse_workspace((int)order));
+	*factorBytes = round_up(order * order * sizeof(real), 256);
+	return *factorBytes + round_up(ws, 256) + 256;
+}
+
+long kfacInverseMemRequired(CNN_MODEL *model, int samples)
+{
+	size_t factorBytes;
+	return (long)(inverse_scratch_bytes(model, samples, &factorBytes) / sizeof(real)) + 64;
+}
+
+static char *aligned_base(real *devPtr) { return (char *)(((size_t)devPtr + 255) & ~(size_t)255); }
+
+void computeOmegaZ(KFAC_CURVATURE_INFO *kfac_info, CNN_MODEL *model, DEVICE_DATASET *data, int samples,
+                   real *dampedInput, real *dampedZ, real *omegaZInv, int *zOffsets, int *zztOffsets, real *devPtr,
+                   real *pageLckPtr)
+{
+	(void)pageLckPtr;
+	const int *omega = kfac_info->OmegaZOffsets;
+	const int withBias = model->bias != 0;
+	const int nc = model->cLayers;
+	size_t factorBytes;
+	const size_t total = inverse_scratch_bytes(model, samples, &factorBytes);
+	char *base = aligned_base(devPtr);
+	real *zzt = (real *)base;
+	real *ws = (real *)(base + factorBytes);
+	const size_t wsBytes = total - factorBytes - 256;
+
+	for (int l = 0; l < nc; l++) {
+		const CONV_LAYER *c = &model->convLayer[l];
+		const real *input;
+		if (dampedInput != NULL)
+			input = (l == 0) ? dampedInput : dampedZ + zztOffsets[l];
+		else
+			input = (l == 0) ? data->currentBatch : dampedZ + zOffsets[l] + model->convLayer[l - 1].outputOffset;
+		const int zCols = c->inChannels * c->kSize * c->kSize + (withBias ? 1 : 0);
+		fitre_conv_shape s = conv_shape(c, samples);
+		HIP_CALL(fitre_hip_kfac_conv_input_factor(&s, input, withBias, zzt, ws, wsBytes));
+		computeMatrixInverse(zzt, omegaZInv + omega[l], zCols, ws, kfac_info->regLambda, kfac_info->dampGamma);
+	}
+	for (int l = 0; l < model->lLayers; l++) {
+		const FC_LAYER *f = &model->fcLayer[l];
+		const real *input;
+		if (dampedInput != NULL)
+			input = dampedZ + zztOffsets[nc + l];
+		else if (l == 0)
+			input = dampedZ + zOffsets[nc] + model->convLayer[nc - 1].outputOffset;
+		else
+			input = dampedZ + zOffsets[nc + l];
+		const int zRows = f->in + (withBias ? 1 : 0);
+		HIP_CALL(fitre_hip_kfac_fc_input_factor(input, f->in, samples, withBias, zzt, ws, wsBytes));
+		computeMatrixInverse(zzt, omegaZInv + omega[nc + l], zRows, ws, kfac_info->regLambda, kfac_info->dampGamma);
+	}
+	HIP_CALL(fitre_hip_sync());
+}
+
+void computeLambdaDelta(KFAC_CURVATURE_INFO *kfac_info, CNN_MODEL *model, int samples, real *dx, real *dampedLambda,
+                        real *lambdaGInv, int *zOffsets, int *zztOffsets, real *devPtr, real *pageLckPtr)
+{
+	(void)pageLckPtr;
+	const int *lambda = kfac_info->LambdaGOffsets;
+	const int nc = model->cLayers;
+	size_t factorBytes;
+	const size_t total = inverse_scratch_bytes(model, samples, &factorBytes);
+	char *base = aligned_base(devPtr);
+	real *ggt = (real *)base;
+	real *ws = (real *)(base + factorBytes);
+	const size_t wsBytes = total - factorBytes - 256;
+
+	for (int l = 0; l < nc; l++) {
+		const CONV_LAYER *c = &model->convLayer[l];
+		const real *delta;
+		if (dampedLambda != NULL)
+			delta = dampedLambda + zztOffsets[l + 1];
+		else if (c->batchNorm == PERFORM_NO_BATCH_NORM)
+			delta = dx + zOffsets[l + 1] + c->activationOffset;
+		else
+			delta = dx + zOffsets[l + 1] + c->batchNormOffset;
+		fitre_conv_shape s = conv_shape(c, samples);
+		HIP_CALL(fitre_hip_kfac_conv_output_factor(&s, delta, ggt, ws, wsBytes));
+		computeMatrixInverse(ggt, lambdaGInv + lambda[l], c->outChannels, ws, kfac_info->regLambda, kfac_info->dampGamma);
+	}
+	for (int l = 0; l < model->lLayers; l++) {
+		const FC_LAYER *f = &model->fcLayer[l];
+		const real *delta = (dampedLambda != NULL) ? dampedLambda + zztOffsets[nc + l + 1] : dx + zOffsets[nc + l + 1];
+		HIP_CALL(fitre_hip_kfac_fc_output_factor(delta, f->out, samples, ggt, ws, wsBytes));
+		computeMatrixInverse(ggt, lambdaGInv + lambda[nc + l], f->out, ws, kfac_info->regLambda, kfac_info->dampGamma);
+	}
+	HIP_CALL(fitre_hip_sync());
+}
+
+/* ---- natural gradient ---------------------------------------------------------------------- */
+
+static size_t natural_gradient_bytes(const CNN_MODEL *model, size_t *matBytes)
+{
+	size_t mat = 256, ws = 256;
+	const int b = model->bias != 0 ? 1 : 0;
+	for (int l = 0; l < model->cLayers; l++) {
+		const CONV_LAYER *c = &model->convLayer[l];
+		int k = c->inChannels * c->kSize * c->kSize + b, o = c->outChannels;
+		mat = max_sz(mat, (size_t)k * o * sizeof(real));
+		ws = max_sz(ws, max_sz(fitre_hip_gemm_workspace(k, o, o), fitre_hip_gemm_workspace(k, o, k)));
+	}
+	for (int l = 0; l < model->lLayers; l++) {
+		const FC_LAYER *f = &model->fcLayer[l];
+		int k = f->in + b, o = f->out;
+		mat = max_sz(mat, (size_t)k * o * sizeof(real));
+		ws = max_sz(ws, max_sz(fitre_hip_gemm_workspace(o, k, o), fitre_hip_gemm_workspace(o, k, k)));
+	}
+	*matBytes = round_up(mat, 256);
+	return 3 * *matBytes + round_up(ws, 256) + 256;
+}
+
+long kfacNaturalGradientMemRequired(CNN_MODEL *model)
+{
+	size_t matBytes;
+	return (long)(natural_gradient_bytes(model, &matBytes) / sizeof(real)) + 64;
+}
+
+void computeNaturalGradient(CNN_MODEL *model, KFAC_CURVATURE_INFO *kfacInfo, real *devPtr, real *hostPtr)
+{
+	(void)hostPtr;
+	const int *wOffsets = model->wOffsets, *bOffsets = model->bOffsets;
+	const int *omegaOff = kfacInfo->OmegaZOffsets, *lambdaOff = kfacInfo->LambdaGOffsets;
+	const real *vec = kfacInfo->gradient;
+	real *nGradient = kfacInfo->nGradient;
+	const int bias = model->bias != 0, nc = model->cLayers;
+	size_t matBytes;
+	const size_t total = natural_gradient_bytes(model, &matBytes);
+	char *base = aligned_base(devPtr);
+	real *wb = (real *)base, *u = (real *)(base + matBytes), *zt = (real *)(base + 2 * matBytes);
+	void *ws = base + 3 * matBytes;
+	const size_t wsBytes = total - 3 * matBytes - 256;
+
+	/* Convolution layers.  The reference forms Lambda * wb' * Omega (Cout x (K+1)) and transposes the
+	 * weight part back; Lambda and Omega are symmetric, so the transposed product Omega * (wb * Lambda)
+	 * is the same matrix already in the parameter layout ((K+1) x Cout, one column per filter). */
+	for (int c = 0; c < nc; c++) {
+		const CONV_LAYER *l = &model->convLayer[c];
+		const int K = l->inChannels * l->kSize * l->kSize, O = l->outChannels, R = K + bias;
+		const real *omega = kfacInfo->OmegaZInv + omegaOff[c], *lambda = kfacInfo->LambdaGInv + lambdaOff[c];
+		const real *v = vec + wOffsets[c];
+		real *ng = nGradient + wOffsets[c];
+		const real *mat = v;
+		if (bias) { /* wb = [filter ; bias] per column, solvers/kfac_natural_gradient.cu:107-119 */
+			HIP_CALL(fitre_hip_copy_2d(wb, R, v, K, K, O));
+			HIP_CALL(fitre_hip_copy_2d(wb + K, R, vec + bOffsets[c], 1, 1, O));
+			mat = wb;
+		}
+		HIP_CALL(fitre_hip_gemm(0, 0, R, O, O, 1.f, mat, R, lambda, O, 0.f, u, R, NULL, ws, wsBytes));
+		if (bias) {
+			HIP_CALL(fitre_hip_gemm(0, 0, R, O, R, 1.f, omega, R, u, R, 0.f, zt, R, NULL, ws, wsBytes));
+			HIP_CALL(fitre_hip_copy_2d(ng, K, zt, R, K, O));
+			HIP_CALL(fitre_hip_copy_2d(nGradient + bOffsets[c], 1, zt + K, R, 1, O));
+		} else {
+			HIP_CALL(fitre_hip_gemm(0, 0, R, O, R, 1.f, omega, R, u, R, 0.f, ng, R, NULL, ws, wsBytes));
+		}
+	}
+	/* Linear layers: the gradient block [W | b] already is the out x (in + 1) matrix
+	 * (solvers/kfac_natural_gradient.cu:196-229). */
+	for (int f = 0; f < model->lLayers; f++) {
+		const FC_LAYER *l = &model->fcLayer[f];
+		const int R = l->in + bias, O = l->out;
+		const real *omega = kfacInfo->OmegaZInv + omegaOff[nc + f], *lambda = kfacInfo->LambdaGInv + lambdaOff[nc + f];
+		HIP_CALL(fitre_hip_gemm(0, 0, O, R, O, 1.f, lambda, O, vec + wOffsets[nc + f], O, 0.f, u, O, NULL, ws, wsBytes));
+		HIP_CALL(fitre_hip_gemm(0, 0, O, R, R, 1.f, u, O, omega, R, 0.f, nGradient + wOffsets[nc + f], O, NULL, ws, wsBytes));
+	}
+	HIP_CALL(fitre_hip_sync());
+}

@@ -110,6 +110,10 @@ int fitre_hip_profile_read_tile(int kernelClass, int tile, long *launches, doubl
 int fitre_hip_axpy(int n, float alpha, const float *x, float *y);         /* y += alpha x */
 int fitre_hip_scal(int n, float alpha, float *x);                         /* x *= alpha */
 int fitre_hip_copy(int n, const float *x, float *y);                      /* y = x */
+/* dst[c*ldd + r] = src[c*lds + r], r < rows, c < cols: cudaMemcpy2D device-to-device as the reference
+ * uses it (solvers/kfac_inverses.cu:596-600, kfac_natural_gradient.cu:107-111), widths in elements.
+ * Leading dimensions below `rows` are allowed (ld 1 with rows 1 walks a strided vector). */
+int fitre_hip_copy_2d(float *dst, long ldd, const float *src, long lds, int rows, int cols);
 int fitre_hip_dot(int n, const float *x, const float *y, float *result);  /* host result, complete on return */
 int fitre_hip_nrm2(int n, const float *x, float *result);                 /* host result */
 int fitre_hip_asum(int n, const float *x, float *result);                 /* host result */

@@ -66,6 +66,34 @@ void computeOmegaZFactors(KFAC_CURVATURE_INFO *kfac_info, CNN_MODEL *model, DEVI
 void computeLambdaDeltaFactors(KFAC_CURVATURE_INFO *kfac_info, CNN_MODEL *model, int samples, real *dx,
                                real *dampedLambda, real *lambdaGGT, int *zOffsets, int *zztOffsets, real *devPtr);
 
+/* inverse = (matrix + (lambda + dampGamma) I)^-1, order n, both dense n x n
+ * (solvers/kfac_inverses.cu:133-186, computeMatrixInverseCusolver without the cuSOLVER handles).
+ * devPtr: fitre_hip_spd_inverse_workspace(n) bytes of scratch, 256-byte aligned.  Exits with the
+ * reference's message when the matrix is not positive definite. */
+void computeMatrixInverse(real *matrix, real *inverse, int n, real *devPtr, real lambda, real dampGamma);
+
+/* Scratch (in reals) computeOmegaZ / computeLambdaDelta may carve from devPtr: the largest factor
+ * plus the workspaces of its product and of its inverse. */
+long kfacInverseMemRequired(CNN_MODEL *model, int samples);
+
+/* solvers/kfac_inverses.cu:450-630 and :759-857 in full: every layer's factor (built in scratch, as in
+ * the reference) and its damped inverse, stored at omegaZInv + OmegaZOffsets[l] resp.
+ * lambdaGInv + LambdaGOffsets[l].  Damping: kfac_info->regLambda + kfac_info->dampGamma on the diagonal.
+ * pageLckPtr is unused (the reference reads cuSOLVER's devInfo through it). */
+void computeOmegaZ(KFAC_CURVATURE_INFO *kfac_info, CNN_MODEL *model, DEVICE_DATASET *data, int samples,
+                   real *dampedInput, real *dampedZ, real *omegaZInv, int *zOffsets, int *zztOffsets, real *devPtr,
+                   real *pageLckPtr);
+void computeLambdaDelta(KFAC_CURVATURE_INFO *kfac_info, CNN_MODEL *model, int samples, real *dx, real *dampedLambda,
+                        real *lambdaGInv, int *zOffsets, int *zztOffsets, real *devPtr, real *pageLckPtr);
+
+/* Scratch (in reals) of computeNaturalGradient. */
+long kfacNaturalGradientMemRequired(CNN_MODEL *model);
+/* solvers/kfac_natural_gradient.cu:36-241: per layer nGradient = Lambda^-1 * gradient * Omega^-1 with the
+ * layer's gradient seen as a Cout x (K + bias) matrix (convolution) resp. out x (in + bias) (linear);
+ * reads kfacInfo->gradient, OmegaZInv, LambdaGInv, writes kfacInfo->nGradient in the flat parameter
+ * layout.  hostPtr is unused. */
+void computeNaturalGradient(CNN_MODEL *model, KFAC_CURVATURE_INFO *kfacInfo, real *devPtr, real *hostPtr);
+
 #ifdef __cplusplus
 }
 #endif

@@ -733,6 +733,49 @@ int oracle_matrix_inverse(const real *matrix, real *inverse, int n, real lambda,
 	return 0;
 }
 
+/* solvers/kfac_natural_gradient.cu:36-241 (computeNaturalGradient): per convolution layer wb = the
+ * (K+1) x Cout matrix [filter ; bias], result = Lambda * wb', nGrad = result * Omega (Cout x (K+1),
+ * leading dimension Cout), then the weight part transposed back with the bias column left where the
+ * flat layout keeps the bias; per linear layer Lambda * [W | b] * Omega in place.  devScratch holds
+ * three of the largest (K+1) x Cout matrices. */
+void oracle_natural_gradient(const CNN_MODEL *model, const int *omegaZOffsets, const int *lambdaGOffsets,
+                             const real *omegaPtr, const real *lambdaPtr, const real *vec, real *nGradient,
+                             real *devScratch)
+{
+	const int *wOffsets = model->wOffsets, *bOffsets = model->bOffsets;
+	for (int c = 0; c < model->cLayers; c++) {
+		const CONV_LAYER *convLayer = &model->convLayer[c];
+		int outChannels = convLayer->outChannels, K = convLayer->inChannels * convLayer->kSize * convLayer->kSize;
+		int cols = K + ((model->bias == 0) ? 0 : 1);
+		const real *omegaZ = omegaPtr + omegaZOffsets[c], *lambdaG = lambdaPtr + lambdaGOffsets[c];
+		const real *vComponent = vec + wOffsets[c];
+		real *nGradComponent = nGradient + wOffsets[c];
+		real *wb = devScratch, *nextDevPtr = wb + (size_t)outChannels * cols;
+		for (int o = 0; o < outChannels; o++) {
+			for (int k = 0; k < K; k++) wb[(size_t)o * cols + k] = vComponent[(size_t)o * K + k];
+			if (model->bias != 0) wb[(size_t)o * cols + cols - 1] = vec[bOffsets[c] + o];
+		}
+		oracle_gemm(OP_N, OP_T, outChannels, cols, outChannels, 1, lambdaG, outChannels, wb, cols, 0, nextDevPtr,
+		            outChannels);
+		oracle_gemm(OP_N, OP_N, outChannels, cols, cols, 1, nextDevPtr, outChannels, omegaZ, cols, 0, nGradComponent,
+		            outChannels);
+		/* cublasDgeam(OP_T): K x Cout <- (Cout x K)' of the weight part, then copied back */
+		for (int o = 0; o < outChannels; o++)
+			for (int k = 0; k < K; k++) nextDevPtr[(size_t)o * K + k] = nGradComponent[(size_t)k * outChannels + o];
+		memcpy(nGradComponent, nextDevPtr, sizeof(real) * (size_t)outChannels * K);
+	}
+	for (int l = 0; l < model->lLayers; l++) {
+		const FC_LAYER *ll = &model->fcLayer[l];
+		int at = model->cLayers + l, cols = ll->in + ((model->bias == 0) ? 0 : 1);
+		const real *omegaZ = omegaPtr + omegaZOffsets[at], *lambdaG = lambdaPtr + lambdaGOffsets[at];
+		real *nextDevPtr = devScratch;
+		oracle_gemm(OP_N, OP_N, ll->out, cols, ll->out, 1, lambdaG, ll->out, vec + wOffsets[at], ll->out, 0, nextDevPtr,
+		            ll->out);
+		oracle_gemm(OP_N, OP_N, ll->out, cols, cols, 1, nextDevPtr, ll->out, omegaZ, cols, 0, nGradient + wOffsets[at],
+		            ll->out);
+	}
+}
+
 /* ------------------------------------------------------------------ */
 /* whole model                                                         */
 /* ------------------------------------------------------------------ */

@@ -166,6 +166,23 @@ class Oracle:
         info = self.lib.oracle_matrix_inverse(self.p(matrix), self.p(inverse), n, self.r(lam), self.r(gamma), self.p(scratch))
         return info, inverse.reshape(n, n)
 
+    def natural_gradient(self, model, omega_offsets, lambda_offsets, omega_inv, lambda_inv, vec):
+        omega_inv, lambda_inv, vec = self.arr(omega_inv), self.arr(lambda_inv), self.arr(vec)
+        oo = (C.c_int * len(omega_offsets))(*omega_offsets)
+        lo = (C.c_int * len(lambda_offsets))(*lambda_offsets)
+        out = self.zeros(model.pSize)
+        big = 1
+        for i in range(model.cLayers):
+            c = model.convLayer[i]
+            big = max(big, (c.inChannels * c.kSize ** 2 + 1) * c.outChannels)
+        for i in range(model.lLayers):
+            f = model.fcLayer[i]
+            big = max(big, (f.in_ + 1) * f.out)
+        scratch = self.zeros(3 * big)
+        self.lib.oracle_natural_gradient(C.byref(model), oo, lo, self.p(omega_inv), self.p(lambda_inv), self.p(vec),
+                                         self.p(out), self.p(scratch))
+        return out
+
     def activation_forward(self, act, x):
         x = self.arr(x).copy()
         rc = self.lib.oracle_activation_forward(act, self.p(x), C.c_size_t(x.size))

@@ -221,3 +221,78 @@ def test_spd_inverse_reports_indefinite_matrix(dev):
     assert info.value == 2
     assert b"positive definite" in hip.fitre_hip_last_error()
     assert hip.fitre_hip_spd_inverse(pa, 2, 0.0, out, ws, 16, C.byref(info)) == 4
+
+
+@pytest.mark.parametrize("name", ["lenet_bias", "small_vgg_bn", "no_bias"])
+def test_model_inverses_and_natural_gradient(dev, oracle64, name):
+    """computeOmegaZ + computeLambdaDelta (factor and damped inverse per layer) and computeNaturalGradient after a
+    forward and a backward pass.  The factors themselves are checked in test_model_factor_passes; here every
+    inverse is compared with the oracle's inverse of the factor the device produced (computeOmegaZFactors on
+    the same z / dx), and the natural gradient with the oracle's on the inverses the device produced.
+    Tolerance of an inverse: the path's 1e-4 for condition numbers up to 50, growing linearly with the
+    condition number beyond that (a float32 Cholesky cannot do better)."""
+    from fitre_amd.structs import KFAC_CURVATURE_INFO
+    from helpers import GpuModel, batch_inputs, he_weights
+    model, batch = next((m, b) for n, m, b in _model_cases() if n == name)
+    rng = np.random.default_rng(sum(map(ord, name)) + 1)
+    w = he_weights(model, rng).astype(np.float32)
+    x, y = batch_inputs(model, batch, rng)
+    x = x.astype(np.float32)
+    gm = GpuModel(dev, model, w, x, y, batch)
+    gm.forward()
+    gm.backward()
+    grad = gm.get("grad")
+    info = KFAC_CURVATURE_INFO()
+    L.cnn.computeKFACStorageIndices(C.byref(model), C.byref(info))
+    lam, gamma = 0.05, 0.15
+    info.regLambda, info.dampGamma = lam, gamma
+    nc, nl = model.cLayers, model.lLayers
+    tot_o, tot_l = info.OmegaZOffsets[nc + nl], info.LambdaGOffsets[nc + nl]
+    ofac, lfac = dev.zeros(tot_o), dev.zeros(tot_l)
+    oinv, linv = dev.zeros(tot_o), dev.zeros(tot_l)
+    need = max(L.cnn.kfacInverseMemRequired(C.byref(model), batch), L.cnn.kfacNaturalGradientMemRequired(C.byref(model)),
+               L.cnn.kfacFactorsMemRequired(C.byref(model), batch))
+    ws = dev.alloc(4 * need + 512)
+    L.cnn.computeOmegaZFactors(C.byref(info), C.byref(model), C.byref(gm.data), batch, None, gm.z, ofac, model.zOffsets,
+                               model.zztOffsets, ws)
+    L.cnn.computeLambdaDeltaFactors(C.byref(info), C.byref(model), batch, gm.dx, None, lfac, model.zOffsets, model.zztOffsets, ws)
+    L.cnn.computeOmegaZ(C.byref(info), C.byref(model), C.byref(gm.data), batch, None, gm.z, oinv, model.zOffsets,
+                        model.zztOffsets, ws, None)
+    L.cnn.computeLambdaDelta(C.byref(info), C.byref(model), batch, gm.dx, None, linv, model.zOffsets, model.zztOffsets, ws, None)
+    fac_o, fac_l = dev.download(ofac, tot_o), dev.download(lfac, tot_l)
+    got_o, got_l = dev.download(oinv, tot_o), dev.download(linv, tot_l)
+    bias = model.bias != 0
+
+    def check(got, factor, what):
+        n = int(round(np.sqrt(factor.size)))
+        factor = factor.reshape(n, n).astype(np.float64)
+        oi, want = oracle64.matrix_inverse(factor, n, lam, gamma)
+        assert oi == 0
+        ev = np.linalg.eigvalsh(factor + (lam + gamma) * np.eye(n))
+        tol = TOL * max(1.0, (ev[-1] / ev[0]) / 50.0)
+        assert rel_err(got.reshape(n, n), want) < tol, (what, ev[-1] / ev[0])
+        assert np.abs((factor + (lam + gamma) * np.eye(n)) @ got.reshape(n, n) - np.eye(n)).max() < tol, what
+
+    for l in range(nc + nl):
+        if l < nc:
+            c = model.convLayer[l]
+            n_in, n_out = c.inChannels * c.kSize ** 2 + (1 if bias else 0), c.outChannels
+        else:
+            f = model.fcLayer[l - nc]
+            n_in, n_out = f.in_ + (1 if bias else 0), f.out
+        o0, l0 = info.OmegaZOffsets[l], info.LambdaGOffsets[l]
+        check(got_o[o0:o0 + n_in * n_in], fac_o[o0:o0 + n_in * n_in], ("omega", l))
+        check(got_l[l0:l0 + n_out * n_out], fac_l[l0:l0 + n_out * n_out], ("lambda", l))
+
+    # natural gradient of the gradient the backward pass produced
+    ngrad = dev.upload(np.full(model.pSize, np.nan, dtype=np.float32))
+    info.OmegaZInv, info.LambdaGInv = oinv.value, linv.value
+    info.gradient, info.nGradient = gm.grad.value, ngrad.value
+    L.cnn.computeNaturalGradient(C.byref(model), C.byref(info), ws, None)
+    got = dev.download(ngrad, model.pSize)
+    want = oracle64.natural_gradient(model, list(info.OmegaZOffsets), list(info.LambdaGOffsets), got_o, got_l, grad)
+    assert np.isfinite(got).all()
+    assert rel_err(got, want) < TOL
+    for q in (ofac, lfac, oinv, linv, ws, ngrad):
+        dev.free(q)
+    gm.release()

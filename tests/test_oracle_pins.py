@@ -387,3 +387,38 @@ def test_matrix_inverse_closed_form_and_failure(oracle64):
     # indefinite: the second pivot is 1 - 4 < 0, reported 1-based like cusolver's devInfo
     info, _ = oracle64.matrix_inverse(np.array([[1.0, 2.0], [2.0, 1.0]]), 2, 0.0, 0.0)
     assert info == 2
+
+
+def test_natural_gradient_against_kron_solve(oracle64):
+    """Per layer the natural gradient is Lambda^-1 G Omega^-1 with G the layer's gradient as a Cout x (K+1)
+    matrix; vec(A G B) = (B' kron A) vec(G), so it must equal the solution of the Kronecker-factored system."""
+    from fitre_amd.structs import CNN_ACT_NONE, CNN_ACT_SWISH, MAX_POOL
+    from helpers import build_custom
+    model = build_custom(3, 6, 6, 2, [dict(cout=3, k=3, pad=1, pool=(MAX_POOL, 2, 2, 0), bn=False, act=CNN_ACT_SWISH)],
+                         [(4, CNN_ACT_NONE)], bias=1)
+    rng = np.random.default_rng(5)
+    g = rng.standard_normal(model.pSize)
+    dims = [(2 * 9 + 1, 3), (3 * 3 * 3 + 1, 4)]          # (K+1, Cout) of the conv layer, (in+1, out) of the FC layer
+    oo, lo, om, la = [0], [0], [], []
+    for k1, o in dims:
+        a, b = rng.standard_normal((k1, k1)), rng.standard_normal((o, o))
+        om.append(a @ a.T + np.eye(k1))
+        la.append(b @ b.T + np.eye(o))
+        oo.append(oo[-1] + k1 * k1)
+        lo.append(lo[-1] + o * o)
+    got = oracle64.natural_gradient(model, oo, lo, np.concatenate([m.reshape(-1) for m in om]),
+                                    np.concatenate([m.reshape(-1) for m in la]), g)
+    # conv layer: flat layout [W (Cout x K, K fastest) | b (Cout)]
+    K, O = 18, 3
+    G = np.concatenate([g[:O * K].reshape(O, K), g[O * K:O * K + O, None]], axis=1)        # Cout x (K+1)
+    want = la[0] @ G @ om[0]
+    np.testing.assert_allclose(got[:O * K].reshape(O, K), want[:, :K], atol=1e-11)
+    np.testing.assert_allclose(got[O * K:O * K + O], want[:, K], atol=1e-11)
+    # FC layer: [W | b] column-major out x (in+1)
+    off, n_in, n_out = model.wOffsets[1], 27, 4
+    Gf = g[off:off + n_out * (n_in + 1)].reshape(n_in + 1, n_out).T
+    wantf = la[1] @ Gf @ om[1]
+    np.testing.assert_allclose(got[off:off + n_out * (n_in + 1)].reshape(n_in + 1, n_out).T, wantf, atol=1e-11)
+    # the Kronecker identity on the conv block
+    vecG = G.reshape(-1, order="F")
+    np.testing.assert_allclose(np.kron(om[0].T, la[0]) @ vecG, want.reshape(-1, order="F"), atol=1e-10)
