@@ -18,13 +18,19 @@ namespace fitre {
 
 constexpr int kNb = 64; // block order of the factorization
 
-// One wave factors the nb x nb (nb <= 64) diagonal block in place (lower triangle; lane i holds
-// row i) and writes the inverse of the factor, 64 x 64 column-major, padded with the identity.
+// value of v in lane `lane` (a compile-time lane index), as a wave-uniform scalar
+__device__ __forceinline__ float lane_value(float v, int lane)
+{
+	return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
+}
+
+// One wave factors the nb x nb (nb <= 64) diagonal block in place (lower triangle) and writes the
+// inverse of the factor, 64 x 64 column-major, padded with the identity.  Lane i holds row i in
+// registers; what a step needs from another lane's row comes through v_readlane as a scalar, so
+// there is no LDS traffic and no barrier in the 2 x 2016 multiply-adds.
 // info: set to the 1-based global index of the first non-positive pivot.
 __global__ void __launch_bounds__(64) chol_diag_kernel(float *W, int ld, int k0, int nb, float *Linv, int *info)
 {
-	__shared__ float col[kNb];
-	__shared__ float Ls[kNb][kNb + 1];
 	const int i = threadIdx.x;
 	float a[kNb];
 	float *blk = W + (size_t)k0 * ld + k0;
@@ -33,37 +39,34 @@ __global__ void __launch_bounds__(64) chol_diag_kernel(float *W, int ld, int k0,
 		const bool inside = (i < nb) & (j < nb);
 		a[j] = inside ? blk[(size_t)j * ld + i] : ((i == j) ? 1.f : 0.f);
 	}
+	float rdiag[kNb]; // 1 / L[j][j], wave-uniform
+	int bad = 0;
 #pragma unroll
 	for (int j = 0; j < kNb; j++) {
-		const float ajj = __shfl(a[j], j, 64);
-		if (!(ajj > 0.f)) {
-			if (i == 0) atomicCAS(info, 0, k0 + j + 1);
-		}
+		const float ajj = lane_value(a[j], j);
+		if (!(ajj > 0.f) && bad == 0) bad = k0 + j + 1;
 		const float d = rsqrtf(ajj);
-		const float lij = (i == j) ? ajj * d : a[j] * d; // sqrt(ajj) on the diagonal
-		a[j] = lij;
-		__syncthreads();
-		col[i] = lij;
-		__syncthreads();
+		rdiag[j] = d;
+		a[j] = (i == j) ? ajj * d : a[j] * d; // column j of L; sqrt(ajj) on the diagonal
 #pragma unroll
-		for (int k = j + 1; k < kNb; k++) a[k] -= lij * col[k]; // entries above the diagonal (k > i) are never used
+		for (int k = j + 1; k < kNb; k++) a[k] -= a[j] * lane_value(a[j], k); // entries above the diagonal are never used
 	}
-	// L back to the matrix and into LDS
+	if (bad != 0 && i == 0) atomicCAS(info, 0, bad);
 #pragma unroll
-	for (int j = 0; j < kNb; j++) {
-		const float v = (j <= i) ? a[j] : 0.f;
-		Ls[i][j] = v;
-		if ((i < nb) & (j < nb) & (j <= i)) blk[(size_t)j * ld + i] = v;
-	}
-	__syncthreads();
-	// lane c solves L x = e_c
+	for (int j = 0; j < kNb; j++)
+		if ((i < nb) & (j < nb) & (j <= i)) blk[(size_t)j * ld + i] = a[j];
+	// lane c solves L x = e_c by forward substitution; L[r][k] is lane r's a[k]
 	float x[kNb];
 #pragma unroll
 	for (int r = 0; r < kNb; r++) {
-		float acc = (r == i) ? 1.f : 0.f;
+		float acc0 = (r == i) ? 1.f : 0.f, acc1 = 0.f;
 #pragma unroll
-		for (int k = 0; k < r; k++) acc -= Ls[r][k] * x[k];
-		x[r] = acc / Ls[r][r];
+		for (int k = 0; k < r; k++) {
+			const float l = lane_value(a[k], r);
+			if (k & 1) acc1 -= l * x[k];
+			else acc0 -= l * x[k];
+		}
+		x[r] = (acc0 + acc1) * rdiag[r];
 	}
 #pragma unroll
 	for (int r = 0; r < kNb; r++) Linv[(size_t)i * kNb + r] = x[r];
