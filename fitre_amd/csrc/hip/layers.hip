@@ -542,6 +542,23 @@ softmax_ce_kernel(const float *logits, const float *target, int rows, int classe
 	if (lane == 0 && (label < 1 || label > classes)) nll[row] = 0.f;
 }
 
+// hits[r] = 1 when the first class with the largest probability (> 0) is the 1-based target, else 0
+__global__ void __launch_bounds__(256) accuracy_hits_kernel(const float *probs, const float *target, int rows, int classes, float *hits)
+{
+	const int r = blockIdx.x * blockDim.x + threadIdx.x;
+	if (r >= rows) return;
+	float best = 0.f;
+	int arg = 0;
+	for (int c = 0; c < classes; c++) {
+		const float p = probs[(size_t)r * classes + c];
+		if (best < p) {
+			best = p;
+			arg = c;
+		}
+	}
+	hits[r] = ((float)(arg + 1) == target[r]) ? 1.f : 0.f;
+}
+
 __global__ void cross_entropy_error_kernel(const float *probs, const float *target, int rows, int classes, float *errors)
 {
 	long total = (long)rows * classes;
@@ -846,6 +863,16 @@ int fitre_hip_softmax_cross_entropy(const float *logits, const float *target, in
 	FITRE_HIP_TRY(hipStreamSynchronize(stream()));
 	*lossHost = *g_loss_host;
 	return FITRE_OK;
+}
+
+int fitre_hip_accuracy_hits(const float *probs, const float *target, int rows, int classes, float *hits)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(probs && target && hits, "fitre_hip_accuracy_hits: null pointer");
+	FITRE_REQUIRE(rows > 0 && classes > 0, "fitre_hip_accuracy_hits: non-positive shape %d x %d", rows, classes);
+	LaunchScope scope(FITRE_KC_SOFTMAX, 4.0 * (double)rows * (classes + 2));
+	accuracy_hits_kernel<<<blocks_for(rows, 256), 256, 0, stream()>>>(probs, target, rows, classes, hits);
+	return check_launch("accuracy_hits_kernel");
 }
 
 int fitre_hip_cross_entropy_error(const float *probs, const float *target, int rows, int classes, float *errors)

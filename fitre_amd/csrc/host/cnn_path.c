@@ -335,3 +335,10 @@ real computeCNNGradient(CNN_MODEL *model, DEVICE_DATASET *data, SCRATCH_AREA *sc
 	scratch->nextPageLckPtr = oldPagePtr;
 	return lossVal;
 }
+
+real computeAccuracy(real *probs, real *target, int rows, int numClasses, real *devPtr, real *pageLckPtr)
+{
+	HIP_CALL(fitre_hip_accuracy_hits(probs, target, rows, numClasses, devPtr));
+	HIP_CALL(fitre_hip_dot(rows, devPtr, devPtr, pageLckPtr)); /* complete on return */
+	return (real)((*pageLckPtr * 100.) / (real)rows);
+}

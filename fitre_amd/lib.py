@@ -75,6 +75,7 @@ HIP_API = {
     "fitre_hip_row_sum": (i32, [vp, i32, i32, vp]),
     "fitre_hip_softmax_cross_entropy": (i32, [vp, vp, i32, i32, vp, vp, pf32]),
     "fitre_hip_cross_entropy_error": (i32, [vp, vp, i32, i32, vp]),
+    "fitre_hip_accuracy_hits": (i32, [vp, vp, i32, i32, vp]),
     "fitre_hip_reshape": (i32, [vp, i32, i32, i32, vp]),
     "fitre_hip_conv_to_fc": (i32, [vp, i32, i32, i32, i32, vp]),
     "fitre_hip_fc_to_conv": (i32, [vp, i32, i32, i32, i32, vp]),
@@ -120,6 +121,7 @@ CNN_API = {
     "cnnBackward": (None, [pmodel, pdata, vp, vp, vp, vp, vp, vp, i32, i32, vp]),
     "evaluateCNNModel": (f32, [pmodel, pdata, pscratch, vp, vp, vp, i32, i32]),
     "computeCNNGradient": (f32, [pmodel, pdata, pscratch, vp, vp, vp, vp, vp, i32, i32, f32]),
+    "computeAccuracy": (f32, [vp, vp, i32, i32, vp, pf32]),
     # include/fitre_kfac.h
     "computeKFACStorageIndices": (None, [pmodel, pkfac]),
     "kfacFactorsMemRequired": (lng, [pmodel, i32]),

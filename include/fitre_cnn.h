@@ -82,6 +82,11 @@ real computeCNNGradient(CNN_MODEL *model, DEVICE_DATASET *data, SCRATCH_AREA *sc
                         real *probs, real *lossFuncErrors, real *gradient, int offset, int curBatchSize,
                         real weightDecay);
 
+/* Percentage of rows whose most probable class (first maximum) is the label; *pageLckPtr receives the
+ * number of hits, as callers read it (functions/cnn_accuracy.cu:39-59, :89-91).  devPtr: rows reals
+ * of device scratch; pageLckPtr: a host pointer. */
+real computeAccuracy(real *probs, real *target, int rows, int numClasses, real *devPtr, real *pageLckPtr);
+
 #ifdef __cplusplus
 }
 #endif

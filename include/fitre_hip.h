@@ -194,6 +194,9 @@ int fitre_hip_softmax_cross_entropy(const float *logits, const float *target, in
 /* errors = (probs - onehot)/rows only (computeCrossEntropyError, :231-245) */
 int fitre_hip_cross_entropy_error(const float *probs, const float *target, int rows, int classes,
                                   float *errors);
+/* hits[r] = 1 if the first class of largest probability equals the 1-based label target[r], else 0
+ * (ker_compute_accuracy, functions/cnn_accuracy.cu:15-37: strict '<' scan starting from probability 0). */
+int fitre_hip_accuracy_hits(const float *probs, const float *target, int rows, int classes, float *hits);
 
 /* ---------------- layout changes at the conv <-> FC boundary ---------------- */
 /* [right][left][chunk] -> [left][right][chunk]   (dev_backprop_convolution.cu:140-168) */

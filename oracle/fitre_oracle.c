@@ -776,6 +776,26 @@ void oracle_natural_gradient(const CNN_MODEL *model, const int *omegaZOffsets, c
 	}
 }
 
+/* functions/cnn_accuracy.cu:15-59 (ker_compute_accuracy + computeAccuracy): hits counted with the
+ * strict '<' scan from probability 0; returns the percentage, *hitsOut the count. */
+real oracle_compute_accuracy(const real *probs, const real *target, int rows, int numClasses, real *hitsOut)
+{
+	real hits = 0;
+	for (int idx = 0; idx < rows; idx++) {
+		real maxProb = 0;
+		int myClass = 0;
+		for (int c = 0; c < numClasses; c++) {
+			if (maxProb < probs[(size_t)idx * numClasses + c]) {
+				maxProb = probs[(size_t)idx * numClasses + c];
+				myClass = c;
+			}
+		}
+		if ((real)(myClass + 1) == target[idx]) hits += 1;
+	}
+	if (hitsOut) *hitsOut = hits;
+	return (hits * 100) / (real)rows;
+}
+
 /* ------------------------------------------------------------------ */
 /* whole model                                                         */
 /* ------------------------------------------------------------------ */

@@ -183,6 +183,13 @@ class Oracle:
                                          self.p(out), self.p(scratch))
         return out
 
+    def compute_accuracy(self, probs, target, rows, classes):
+        probs, target = self.arr(probs), self.arr(target)
+        hits = self.creal(0)
+        self.lib.oracle_compute_accuracy.restype = self.creal
+        pct = self.lib.oracle_compute_accuracy(self.p(probs), self.p(target), rows, classes, C.byref(hits))
+        return float(pct), float(hits.value)
+
     def activation_forward(self, act, x):
         x = self.arr(x).copy()
         rc = self.lib.oracle_activation_forward(act, self.p(x), C.c_size_t(x.size))

@@ -327,3 +327,17 @@ def test_boundary_permutes(dev, oracle64):
     ok(hip.fitre_hip_reshape(px, Cn, N, A * B, out))
     np.testing.assert_array_equal(dev.download(out, x.size), oracle64.reshape(x, Cn, N, A * B))
     assert hip.fitre_hip_conv_to_fc(px, Cn, N, A, B, px) == 2  # in place is refused
+
+
+@pytest.mark.parametrize("rows,classes", [(4, 3), (256, 10), (1000, 1000), (1, 1)])
+def test_compute_accuracy(dev, oracle64, rows, classes):
+    rng = np.random.default_rng(rows + classes)
+    p = rng.random((rows, classes)).astype(np.float32)
+    p[0, :] = 0.25 if classes > 1 else 1.0       # a tie: the first class wins
+    t = rng.integers(1, classes + 1, rows).astype(np.float32)
+    pp, pt, scratch = dev.upload(p.reshape(-1)), dev.upload(t), dev.zeros(rows)
+    hits = C.c_float(-1)
+    pct = L.cnn.computeAccuracy(pp, pt, rows, classes, scratch, C.byref(hits))
+    wpct, whits = oracle64.compute_accuracy(p.reshape(-1), t, rows, classes)
+    assert hits.value == whits
+    assert abs(pct - wpct) < 1e-4

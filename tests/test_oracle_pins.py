@@ -422,3 +422,18 @@ def test_natural_gradient_against_kron_solve(oracle64):
     # the Kronecker identity on the conv block
     vecG = G.reshape(-1, order="F")
     np.testing.assert_allclose(np.kron(om[0].T, la[0]) @ vecG, want.reshape(-1, order="F"), atol=1e-10)
+
+
+def test_compute_accuracy_counts_first_maximum(oracle64):
+    probs = np.array([[0.1, 0.7, 0.2],     # class 2
+                      [0.4, 0.4, 0.2],     # tie: first maximum, class 1
+                      [0.0, 0.0, 0.0],     # nothing exceeds 0: class 1 by default
+                      [0.2, 0.3, 0.5]])    # class 3
+    target = np.array([2.0, 2.0, 1.0, 1.0])
+    pct, hits = oracle64.compute_accuracy(probs.reshape(-1), target, 4, 3)
+    assert hits == 2 and pct == 50.0
+    rng = np.random.default_rng(0)
+    p = rng.random((100, 10))
+    t = rng.integers(1, 11, 100).astype(np.float64)
+    pct, hits = oracle64.compute_accuracy(p.reshape(-1), t, 100, 10)
+    assert hits == float(np.sum(p.argmax(1) + 1 == t)) and abs(pct - hits) < 1e-12
