@@ -229,6 +229,39 @@ __global__ void __launch_bounds__(256) row_sum_kernel(const float *mat, int rows
 	}
 }
 
+// Counter-based generator: element g of the stream is a splitmix64 hash of seed and g, so the
+// same (seed, position) gives the same number whatever the launch shape.  24 random bits make
+// a float in (0, 1].
+__host__ __device__ inline unsigned long long splitmix64(unsigned long long seed, unsigned long long g)
+{
+	unsigned long long z = seed + (g + 1ull) * 0x9E3779B97F4A7C15ull;
+	z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+	z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+	return z ^ (z >> 31);
+}
+__device__ __forceinline__ float uniform_from(unsigned long long z) { return (float)((z >> 40) + 1ull) * (1.0f / 16777216.0f); }
+
+__global__ void __launch_bounds__(256) random_uniform_kernel(float *out, long n, unsigned long long seed, unsigned long long first)
+{
+	const long stride = (long)gridDim.x * blockDim.x;
+	for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) out[i] = uniform_from(splitmix64(seed, first + i));
+}
+// Box-Muller on consecutive pairs of the uniform stream
+__global__ void __launch_bounds__(256) random_normal_kernel(float *out, long n, unsigned long long seed, unsigned long long first)
+{
+	const long pairs = (n + 1) / 2;
+	const long stride = (long)gridDim.x * blockDim.x;
+	for (long j = (long)blockIdx.x * blockDim.x + threadIdx.x; j < pairs; j += stride) {
+		const float u1 = uniform_from(splitmix64(seed, first + 2 * j)), u2 = uniform_from(splitmix64(seed, first + 2 * j + 1));
+		const float r = sqrtf(-2.f * logf(u1));
+		float sn, cs;
+		sincosf(6.28318530717958647692f * u2, &sn, &cs);
+		out[2 * j] = r * cs;
+		if (2 * j + 1 < n) out[2 * j + 1] = r * sn;
+	}
+}
+static unsigned long long g_rng_seed = 1234ull, g_rng_next = 0ull;
+
 // dst[c*ldd + r] = src[c*lds + r] for r < rows, c < cols
 __global__ void __launch_bounds__(256) copy_2d_kernel(const float *src, long lds_, float *dst, long ldd, int rows, int cols)
 {
@@ -333,6 +366,33 @@ int fitre_hip_add_channel_bias(float *x, int channels, long perChannel, const fl
 	add_channel_bias_kernel<<<grid, 256, 0, stream()>>>(x, perChannel, bias);
 	return check_launch("add_channel_bias_kernel");
 }
+int fitre_hip_random_seed(unsigned long long seed)
+{
+	g_rng_seed = seed;
+	g_rng_next = 0ull;
+	return FITRE_OK;
+}
+
+int fitre_hip_random_uniform(float *out, long n)
+{
+	EW_CHECK("fitre_hip_random_uniform", out && n >= 0);
+	if (n == 0) return FITRE_OK;
+	LaunchScope scope(FITRE_KC_BLAS1, 4.0 * (double)n);
+	random_uniform_kernel<<<blocks_for(n, 1024, 4096), 256, 0, stream()>>>(out, n, g_rng_seed, g_rng_next);
+	g_rng_next += (unsigned long long)n;
+	return check_launch("random_uniform_kernel");
+}
+
+int fitre_hip_random_normal(float *out, long n)
+{
+	EW_CHECK("fitre_hip_random_normal", out && n >= 0);
+	if (n == 0) return FITRE_OK;
+	LaunchScope scope(FITRE_KC_BLAS1, 4.0 * (double)n);
+	random_normal_kernel<<<blocks_for((n + 1) / 2, 1024, 4096), 256, 0, stream()>>>(out, n, g_rng_seed, g_rng_next);
+	g_rng_next += (unsigned long long)(2 * ((n + 1) / 2));
+	return check_launch("random_normal_kernel");
+}
+
 int fitre_hip_copy_2d(float *dst, long ldd, const float *src, long lds_, int rows, int cols)
 {
 	EW_CHECK("fitre_hip_copy_2d", dst && src && rows > 0 && cols > 0);

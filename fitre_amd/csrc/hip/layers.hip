@@ -542,6 +542,26 @@ softmax_ce_kernel(const float *logits, const float *target, int rows, int classe
 	if (lane == 0 && (label < 1 || label > classes)) nll[row] = 0.f;
 }
 
+// classes[r] = 1-based index of the first class whose cumulative probability reaches uniforms[r];
+// classes + 1 if rounding keeps the total below it
+__global__ void __launch_bounds__(256) multinomial_classes_kernel(const float *probs, const float *uniforms, int samples, int classes,
+                                                                   float *out)
+{
+	const int r = blockIdx.x * blockDim.x + threadIdx.x;
+	if (r >= samples) return;
+	const float u = uniforms[r];
+	float c = 0.f;
+	int pick = classes + 1;
+	for (int i = 0; i < classes; i++) {
+		c += probs[(size_t)r * classes + i];
+		if (c >= u) {
+			pick = i + 1;
+			break;
+		}
+	}
+	out[r] = (float)pick;
+}
+
 // hits[r] = 1 when the first class with the largest probability (> 0) is the 1-based target, else 0
 __global__ void __launch_bounds__(256) accuracy_hits_kernel(const float *probs, const float *target, int rows, int classes, float *hits)
 {
@@ -863,6 +883,16 @@ int fitre_hip_softmax_cross_entropy(const float *logits, const float *target, in
 	FITRE_HIP_TRY(hipStreamSynchronize(stream()));
 	*lossHost = *g_loss_host;
 	return FITRE_OK;
+}
+
+int fitre_hip_multinomial_classes(const float *probs, const float *uniforms, int samples, int classes, float *out)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(probs && uniforms && out, "fitre_hip_multinomial_classes: null pointer");
+	FITRE_REQUIRE(samples > 0 && classes > 0, "fitre_hip_multinomial_classes: non-positive shape %d x %d", samples, classes);
+	LaunchScope scope(FITRE_KC_SOFTMAX, 4.0 * (double)samples * (classes + 2));
+	multinomial_classes_kernel<<<blocks_for(samples, 256), 256, 0, stream()>>>(probs, uniforms, samples, classes, out);
+	return check_launch("multinomial_classes_kernel");
 }
 
 int fitre_hip_accuracy_hits(const float *probs, const float *target, int rows, int classes, float *hits)

@@ -342,3 +342,24 @@ real computeAccuracy(real *probs, real *target, int rows, int numClasses, real *
 	HIP_CALL(fitre_hip_dot(rows, devPtr, devPtr, pageLckPtr)); /* complete on return */
 	return (real)((*pageLckPtr * 100.) / (real)rows);
 }
+
+void computeCrossEntropyError(real *probs, int rows, int num_classes, real *target, real *errors)
+{
+	HIP_CALL(fitre_hip_cross_entropy_error(probs, target, rows, num_classes, errors));
+	HIP_CALL(fitre_hip_sync());
+}
+
+void getMultinomialDistSample(real *probs, int samples, int numClasses, real *distClasses, real *devPtr)
+{
+	HIP_CALL(fitre_hip_random_uniform(devPtr, samples));
+	HIP_CALL(fitre_hip_multinomial_classes(probs, devPtr, samples, numClasses, distClasses));
+	HIP_CALL(fitre_hip_sync());
+}
+
+void computeDistributionErrors(real *probs, real *distTarget, real *distError, int rows, int num_classes, real *devPtr,
+                               real *hostPtr)
+{
+	(void)hostPtr;
+	getMultinomialDistSample(probs, rows, num_classes, distTarget, devPtr);
+	computeCrossEntropyError(probs, rows, num_classes, distTarget, distError);
+}

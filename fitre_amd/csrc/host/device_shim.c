@@ -138,3 +138,11 @@ void print_device_mem_usage(void)
 	fprintf(stderr, "device memory: used %zu MB, free %zu MB, total %zu MB\n", (total - freeb) >> 20, freeb >> 20,
 	        total >> 20);
 }
+
+void getRandomVector(int n, real *hostPtr, real *devPtr, RAND_GENERATOR r)
+{
+	int rc = (r == RAND_NORMAL) ? fitre_hip_random_normal(devPtr, n) : fitre_hip_random_uniform(devPtr, n);
+	if (rc) die("getRandomVector", -1);
+	if (hostPtr != NULL && fitre_hip_copy_d2h(hostPtr, devPtr, sizeof(real) * (size_t)n)) die("getRandomVector: copy", -1);
+	if (hostPtr == NULL && fitre_hip_sync()) die("getRandomVector: sync", -1);
+}

@@ -76,6 +76,10 @@ HIP_API = {
     "fitre_hip_softmax_cross_entropy": (i32, [vp, vp, i32, i32, vp, vp, pf32]),
     "fitre_hip_cross_entropy_error": (i32, [vp, vp, i32, i32, vp]),
     "fitre_hip_accuracy_hits": (i32, [vp, vp, i32, i32, vp]),
+    "fitre_hip_multinomial_classes": (i32, [vp, vp, i32, i32, vp]),
+    "fitre_hip_random_seed": (i32, [C.c_ulonglong]),
+    "fitre_hip_random_uniform": (i32, [vp, lng]),
+    "fitre_hip_random_normal": (i32, [vp, lng]),
     "fitre_hip_reshape": (i32, [vp, i32, i32, i32, vp]),
     "fitre_hip_conv_to_fc": (i32, [vp, i32, i32, i32, i32, vp]),
     "fitre_hip_fc_to_conv": (i32, [vp, i32, i32, i32, i32, vp]),
@@ -122,6 +126,10 @@ CNN_API = {
     "evaluateCNNModel": (f32, [pmodel, pdata, pscratch, vp, vp, vp, i32, i32]),
     "computeCNNGradient": (f32, [pmodel, pdata, pscratch, vp, vp, vp, vp, vp, i32, i32, f32]),
     "computeAccuracy": (f32, [vp, vp, i32, i32, vp, pf32]),
+    "computeCrossEntropyError": (None, [vp, i32, i32, vp, vp]),
+    "getMultinomialDistSample": (None, [vp, i32, i32, vp, vp]),
+    "computeDistributionErrors": (None, [vp, vp, vp, i32, i32, vp, vp]),
+    "getRandomVector": (None, [i32, vp, vp, i32]),
     # include/fitre_kfac.h
     "computeKFACStorageIndices": (None, [pmodel, pkfac]),
     "kfacFactorsMemRequired": (lng, [pmodel, i32]),

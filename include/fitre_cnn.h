@@ -82,6 +82,16 @@ real computeCNNGradient(CNN_MODEL *model, DEVICE_DATASET *data, SCRATCH_AREA *sc
                         real *probs, real *lossFuncErrors, real *gradient, int offset, int curBatchSize,
                         real weightDecay);
 
+/* errors = (probs - onehot(target)) / rows (functions/softmax_loss.cu:141-175 as called from :131). */
+void computeCrossEntropyError(real *probs, int rows, int num_classes, real *target, real *errors);
+/* One class per sample drawn from the model's own predictive distribution
+ * (functions/dev_dist_errors.cu:39-53); devPtr: samples (+1) reals of scratch for the uniform draws. */
+void getMultinomialDistSample(real *probs, int samples, int numClasses, real *distClasses, real *devPtr);
+/* Sampled targets and the loss errors against them -- the input of the backward pass that builds the
+ * Fisher (KFAC) statistics (functions/softmax_loss.cu:104-136).  hostPtr is unused. */
+void computeDistributionErrors(real *probs, real *distTarget, real *distError, int rows, int num_classes,
+                               real *devPtr, real *hostPtr);
+
 /* Percentage of rows whose most probable class (first maximum) is the label; *pageLckPtr receives the
  * number of hits, as callers read it (functions/cnn_accuracy.cu:39-59, :89-91).  devPtr: rows reals
  * of device scratch; pageLckPtr: a host pointer. */

@@ -121,6 +121,13 @@ int fitre_hip_norm_inf(int n, const float *x, float *result);             /* dev
 int fitre_hip_sum(int n, const float *x, float *result);                  /* utilities/reduce.cu:32-84 */
 
 /* ---------------- elementwise helpers ---------------- */
+/* Seeded generator replacing the cuRAND handle of device/gen_random.cu:25-52: a counter-based
+ * stream (splitmix64 of seed and position; restated in the test oracle), uniform in (0, 1] resp.
+ * standard normal (Box-Muller on consecutive pairs).  Each call continues the stream;
+ * fitre_hip_random_seed() restarts it.  Default seed 1234 (gen_random.cu:36). */
+int fitre_hip_random_seed(unsigned long long seed);
+int fitre_hip_random_uniform(float *out, long n);
+int fitre_hip_random_normal(float *out, long n);
 int fitre_hip_fill(float *x, long n, float value);                        /* dev_initializations.cu:7-14, dev_activations.cu:89-95 */
 int fitre_hip_hadamard(const float *x, float *y, long n);                 /* y *= x                  dev_hadamard.cu:4-10 */
 int fitre_hip_hadamard2(const float *m1, const float *m2, const float *m3, const float *m4, long n,
@@ -197,6 +204,10 @@ int fitre_hip_cross_entropy_error(const float *probs, const float *target, int r
 /* hits[r] = 1 if the first class of largest probability equals the 1-based label target[r], else 0
  * (ker_compute_accuracy, functions/cnn_accuracy.cu:15-37: strict '<' scan starting from probability 0). */
 int fitre_hip_accuracy_hits(const float *probs, const float *target, int rows, int classes, float *hits);
+/* out[r] = 1-based class drawn from row r of probs by inverting the cumulative sum at uniforms[r]
+ * (ker_compute_dist_classes, functions/dev_dist_errors.cu:12-35; classes + 1 when rounding keeps the
+ * cumulative sum below the draw). */
+int fitre_hip_multinomial_classes(const float *probs, const float *uniforms, int samples, int classes, float *out);
 
 /* ---------------- layout changes at the conv <-> FC boundary ---------------- */
 /* [right][left][chunk] -> [left][right][chunk]   (dev_backprop_convolution.cu:140-168) */

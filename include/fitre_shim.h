@@ -46,6 +46,11 @@ void copy_host_device(void *host, void *dev, size_t size, enum cudaMemcpyKind di
 void copy_device(void *dst, void *src, size_t size, int err_code);
 void print_device_mem_usage(void);
 
+/* device/gen_random.h:6-13: n standard-normal or uniform (0, 1] reals into devPtr, copied to hostPtr
+ * when it is not NULL.  The stream is seeded with fitre_hip_random_seed(). */
+typedef enum random_generator { RAND_NORMAL = 1, RAND_UNIFORM } RAND_GENERATOR;
+void getRandomVector(int n, real *hostPtr, real *devPtr, RAND_GENERATOR r);
+
 #ifdef __cplusplus
 }
 #endif

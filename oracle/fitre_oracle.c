@@ -796,6 +796,38 @@ real oracle_compute_accuracy(const real *probs, const real *target, int rows, in
 	return (hits * 100) / (real)rows;
 }
 
+/* functions/dev_dist_errors.cu:12-35 (ker_compute_dist_classes): inverse-CDF draw of one 1-based
+ * class per sample from the uniform numbers distProbs. */
+void oracle_multinomial_classes(const real *probs, int samples, int numClasses, const real *distProbs, real *distClasses)
+{
+	for (int idx = 0; idx < samples; idx++) {
+		real c = 0;
+		distClasses[idx] = -1;
+		for (int i = 0; i < numClasses; i++) {
+			c += probs[(size_t)idx * numClasses + i];
+			if (c >= distProbs[idx]) {
+				distClasses[idx] = i + 1;
+				i += (numClasses + 1);
+			}
+		}
+		if (distClasses[idx] == -1) distClasses[idx] = numClasses + 1;
+	}
+}
+
+/* The seeded stream that stands in for cuRAND (device/gen_random.cu:25-52): element g is the
+ * splitmix64 hash of seed + (g+1)*golden, its top 24 bits + 1 scaled to (0, 1].  Integer arithmetic:
+ * every implementation of it must agree bit for bit. */
+void oracle_uniform_stream(unsigned long long seed, unsigned long long first, long n, float *out)
+{
+	for (long i = 0; i < n; i++) {
+		unsigned long long z = seed + (first + (unsigned long long)i + 1ull) * 0x9E3779B97F4A7C15ull;
+		z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+		z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+		z = z ^ (z >> 31);
+		out[i] = (float)((z >> 40) + 1ull) * (1.0f / 16777216.0f);
+	}
+}
+
 /* ------------------------------------------------------------------ */
 /* whole model                                                         */
 /* ------------------------------------------------------------------ */

@@ -190,6 +190,17 @@ class Oracle:
         pct = self.lib.oracle_compute_accuracy(self.p(probs), self.p(target), rows, classes, C.byref(hits))
         return float(pct), float(hits.value)
 
+    def multinomial_classes(self, probs, uniforms, samples, classes):
+        probs, uniforms = self.arr(probs), self.arr(uniforms)
+        out = self.zeros(samples)
+        self.lib.oracle_multinomial_classes(self.p(probs), samples, classes, self.p(uniforms), self.p(out))
+        return out
+
+    def uniform_stream(self, seed, first, n):
+        out = np.zeros(int(n), dtype=np.float32)
+        self.lib.oracle_uniform_stream(C.c_ulonglong(seed), C.c_ulonglong(first), C.c_long(n), self.p(out))
+        return out
+
     def activation_forward(self, act, x):
         x = self.arr(x).copy()
         rc = self.lib.oracle_activation_forward(act, self.p(x), C.c_size_t(x.size))

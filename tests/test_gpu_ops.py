@@ -341,3 +341,50 @@ def test_compute_accuracy(dev, oracle64, rows, classes):
     wpct, whits = oracle64.compute_accuracy(p.reshape(-1), t, rows, classes)
     assert hits.value == whits
     assert abs(pct - wpct) < 1e-4
+
+
+def test_random_streams(dev, oracle64):
+    ok(hip.fitre_hip_random_seed(4321))
+    a, b = dev.zeros(1001), dev.zeros(64)
+    ok(hip.fitre_hip_random_uniform(a, 1001))
+    ok(hip.fitre_hip_random_uniform(b, 64))          # continues the stream
+    np.testing.assert_array_equal(dev.download(a, 1001), oracle64.uniform_stream(4321, 0, 1001))
+    np.testing.assert_array_equal(dev.download(b, 64), oracle64.uniform_stream(4321, 1001, 64))
+    ok(hip.fitre_hip_random_seed(4321))
+    ok(hip.fitre_hip_random_uniform(b, 64))          # re-seeding restarts it
+    np.testing.assert_array_equal(dev.download(b, 64), oracle64.uniform_stream(4321, 0, 64))
+    # normal: Box-Muller of consecutive pairs of the same stream
+    n = 200001
+    c = dev.zeros(n)
+    ok(hip.fitre_hip_random_seed(7))
+    ok(hip.fitre_hip_random_normal(c, n))
+    got = dev.download(c, n)
+    u = oracle64.uniform_stream(7, 0, n + 1).astype(np.float64)
+    r = np.sqrt(-2 * np.log(u[0::2]))
+    want = np.stack([r * np.cos(2 * np.pi * u[1::2]), r * np.sin(2 * np.pi * u[1::2])], axis=1).reshape(-1)[:n]
+    assert np.abs(got - want).max() < 5e-5
+    assert abs(got.mean()) < 1e-2 and abs(got.std() - 1) < 1e-2
+
+
+@pytest.mark.parametrize("rows,classes", [(5, 3), (256, 10), (4096, 1000)])
+def test_distribution_errors(dev, oracle64, rows, classes):
+    """computeDistributionErrors: targets drawn from the predictive distribution with the seeded stream, and the
+    cross-entropy errors against them; bit-exact classes given the same uniform numbers."""
+    rng = np.random.default_rng(rows)
+    p = rng.random((rows, classes)).astype(np.float32)
+    p = (p / p.sum(1, keepdims=True)).astype(np.float32)
+    pp = dev.upload(p.reshape(-1))
+    tgt, err, scratch = dev.zeros(rows), dev.zeros(rows * classes), dev.zeros(rows + 1)
+    ok(hip.fitre_hip_random_seed(99))
+    L.cnn.computeDistributionErrors(pp, tgt, err, rows, classes, scratch, None)
+    u = oracle64.uniform_stream(99, 0, rows)
+    # the oracle in float32 arithmetic: the running sum must round as on the device
+    import oracle.oracle as O
+    want_t = O.Oracle(double=False).multinomial_classes(p.reshape(-1), u, rows, classes)
+    got_t = dev.download(tgt, rows)
+    np.testing.assert_array_equal(got_t, want_t)
+    want_e = oracle64.cross_entropy_error(p.reshape(-1), got_t, rows, classes)
+    assert rel_err(dev.download(err, rows * classes), want_e) < 1e-6
+    # the empirical class frequencies follow the probabilities
+    if rows >= 4096:
+        assert abs(np.mean(got_t) - np.mean((p * np.arange(1, classes + 1)).sum(1))) < 0.05 * classes

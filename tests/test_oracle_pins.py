@@ -437,3 +437,36 @@ def test_compute_accuracy_counts_first_maximum(oracle64):
     t = rng.integers(1, 11, 100).astype(np.float64)
     pct, hits = oracle64.compute_accuracy(p.reshape(-1), t, 100, 10)
     assert hits == float(np.sum(p.argmax(1) + 1 == t)) and abs(pct - hits) < 1e-12
+
+
+def test_multinomial_classes_inverse_cdf(oracle64):
+    probs = np.array([[0.2, 0.5, 0.3], [0.2, 0.5, 0.3], [0.2, 0.5, 0.3], [0.2, 0.5, 0.3], [0.25, 0.25, 0.25]])
+    u = np.array([0.1, 0.2, 0.2000001, 0.95, 0.9])      # boundary included in the lower class (c >= u)
+    got = oracle64.multinomial_classes(probs.reshape(-1), u, 5, 3)
+    np.testing.assert_array_equal(got, [1, 1, 2, 3, 4])  # last row: the total stays below the draw -> classes + 1
+    rng = np.random.default_rng(3)
+    p = rng.random((2000, 7))
+    p /= p.sum(1, keepdims=True)
+    uu = rng.random(2000)
+    want = 1 + (np.cumsum(p, axis=1) >= uu[:, None]).argmax(1)
+    np.testing.assert_array_equal(oracle64.multinomial_classes(p.reshape(-1), uu, 2000, 7), want)
+
+
+def test_uniform_stream_known_values_and_statistics(oracle64):
+    # splitmix64 with seed 0 produces the published first outputs when hashed position by position
+    def splitmix(seed, g):
+        m = (1 << 64) - 1
+        z = (seed + (g + 1) * 0x9E3779B97F4A7C15) & m
+        z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & m
+        z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & m
+        return z ^ (z >> 31)
+    assert splitmix(0, 0) == 0xE220A8397B1DCDAF and splitmix(0, 1) == 0x6E789E6AA1B965F4  # reference vectors of SplitMix64
+    got = oracle64.uniform_stream(1234, 5, 1000)
+    want = np.array([((splitmix(1234, 5 + i) >> 40) + 1) / 16777216.0 for i in range(1000)], dtype=np.float32)
+    np.testing.assert_array_equal(got, want)
+    big = oracle64.uniform_stream(99, 0, 200000)
+    assert big.min() > 0 and big.max() <= 1
+    assert abs(big.mean() - 0.5) < 3e-3 and abs(big.var() - 1 / 12) < 2e-3
+    # continuing the stream equals one long draw
+    np.testing.assert_array_equal(np.concatenate([oracle64.uniform_stream(7, 0, 10), oracle64.uniform_stream(7, 10, 6)]),
+                                  oracle64.uniform_stream(7, 0, 16))
