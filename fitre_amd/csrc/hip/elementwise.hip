@@ -79,6 +79,35 @@ struct FSqrDecay { float decay; __device__ float operator()(float x, float y, fl
 
 __device__ __forceinline__ float sigmoidf(float x) { return 1.f / (1.f + expf(-x)); }
 
+// terms of the fully connected models' output heads (a = target y, b = network output or logit)
+struct FScaledDiff { float scale; __device__ float operator()(float y, float z, float, float) const { return scale * (y - z); } };
+struct FSquaredDiff { __device__ float operator()(float y, float z, float, float) const { return (y - z) * (y - z); } };
+struct FLogisticLl { // y*x - log(1 + exp(x)), written as the reference does to stay finite for large |x|
+	__device__ float operator()(float y, float x, float, float) const
+	{
+		const float ind = (x >= 0.f) ? 1.f : 0.f;
+		return x * (y - ind) - logf(1.f + expf(x - 2.f * x * ind));
+	}
+};
+struct FSoftmaxLl { __device__ float operator()(float y, float z, float, float) const { return y * logf(z); } };
+
+// x[:, c] = exp(x[:, c]) / sum(exp(x[:, c])) for a column-major rows x cols matrix; one wave per column
+__global__ void __launch_bounds__(256) column_softmax_kernel(float *x, int rows, int cols)
+{
+	const int lane = threadIdx.x & 63;
+	const int c = blockIdx.x * 4 + (threadIdx.x >> 6);
+	if (c >= cols) return;
+	float *p = x + (size_t)c * rows;
+	float sum = 0.f;
+	for (int r = lane; r < rows; r += 64) {
+		const float e = expf(p[r]);
+		p[r] = e;
+		sum += e;
+	}
+	sum = wave_sum(sum);
+	for (int r = lane; r < rows; r += 64) p[r] = p[r] / sum;
+}
+
 struct ActRelu { __device__ float operator()(float x, float, float, float) const { return x < 0.f ? 0.f : x; } };
 struct ActSoftplus { __device__ float operator()(float x, float, float, float) const { return x < 20.f ? logf(1.f + expf(x)) : x; } };
 struct ActElu { __device__ float operator()(float x, float, float, float) const { return x < 0.f ? (expf(x) - 1.f) : x; } };
@@ -366,6 +395,26 @@ int fitre_hip_add_channel_bias(float *x, int channels, long perChannel, const fl
 	add_channel_bias_kernel<<<grid, 256, 0, stream()>>>(x, perChannel, bias);
 	return check_launch("add_channel_bias_kernel");
 }
+int fitre_hip_column_softmax(float *x, int rows, int cols)
+{
+	EW_CHECK("fitre_hip_column_softmax", x && rows > 0 && cols > 0);
+	LaunchScope scope(FITRE_KC_SOFTMAX, 8.0 * (double)rows * cols);
+	column_softmax_kernel<<<(cols + 3) / 4, 256, 0, stream()>>>(x, rows, cols);
+	return check_launch("column_softmax_kernel");
+}
+
+int fitre_hip_output_terms(int kind, const float *y, const float *z, long n, float scale, float *out)
+{
+	EW_CHECK("fitre_hip_output_terms", y && z && out && n >= 0);
+	switch (kind) {
+	case FITRE_TERM_SCALED_DIFFERENCE: return launch_map<2>("scaled_difference", FITRE_KC_SOFTMAX, y, z, nullptr, nullptr, out, n, FScaledDiff{ scale });
+	case FITRE_TERM_SQUARED_DIFFERENCE: return launch_map<2>("squared_difference", FITRE_KC_SOFTMAX, y, z, nullptr, nullptr, out, n, FSquaredDiff{});
+	case FITRE_TERM_LOGISTIC_LL: return launch_map<2>("logistic_ll", FITRE_KC_SOFTMAX, y, z, nullptr, nullptr, out, n, FLogisticLl{});
+	case FITRE_TERM_SOFTMAX_LL: return launch_map<2>("softmax_ll", FITRE_KC_SOFTMAX, y, z, nullptr, nullptr, out, n, FSoftmaxLl{});
+	default: return fail(FITRE_E_UNSUPPORTED, "fitre_hip_output_terms: unknown kind %d", kind);
+	}
+}
+
 int fitre_hip_random_seed(unsigned long long seed)
 {
 	g_rng_seed = seed;

@@ -6,7 +6,7 @@ import fails with the reason.  Build with ``python -m fitre_amd.build``.
 import ctypes as C
 import os
 
-from .structs import (CNN_MODEL, CONV_LAYER, DEVICE_DATASET, KFAC_CURVATURE_INFO, POOL_LAYER, SCRATCH_AREA,
+from .structs import (CNN_MODEL, CONV_LAYER, DEVICE_DATASET, KFAC_CURVATURE_INFO, NN_MODEL, POOL_LAYER, SCRATCH_AREA,
                       fitre_conv_shape)
 
 _PKG = os.path.dirname(os.path.abspath(__file__))
@@ -18,6 +18,7 @@ pvp, pi32, pf32 = C.POINTER(C.c_void_p), C.POINTER(C.c_int), C.POINTER(C.c_float
 pshape = C.POINTER(fitre_conv_shape)
 pmodel, pdata, pscratch = C.POINTER(CNN_MODEL), C.POINTER(DEVICE_DATASET), C.POINTER(SCRATCH_AREA)
 pkfac = C.POINTER(KFAC_CURVATURE_INFO)
+pnn = C.POINTER(NN_MODEL)
 
 # name -> (restype, argtypes); mirrors include/fitre_hip.h
 HIP_API = {
@@ -77,6 +78,8 @@ HIP_API = {
     "fitre_hip_cross_entropy_error": (i32, [vp, vp, i32, i32, vp]),
     "fitre_hip_accuracy_hits": (i32, [vp, vp, i32, i32, vp]),
     "fitre_hip_multinomial_classes": (i32, [vp, vp, i32, i32, vp]),
+    "fitre_hip_column_softmax": (i32, [vp, i32, i32]),
+    "fitre_hip_output_terms": (i32, [i32, vp, vp, lng, f32, vp]),
     "fitre_hip_random_seed": (i32, [C.c_ulonglong]),
     "fitre_hip_random_uniform": (i32, [vp, lng]),
     "fitre_hip_random_normal": (i32, [vp, lng]),
@@ -141,6 +144,17 @@ CNN_API = {
     "computeLambdaDelta": (None, [pkfac, pmodel, i32, vp, vp, vp, pi32, pi32, vp, vp]),
     "kfacNaturalGradientMemRequired": (lng, [pmodel]),
     "computeNaturalGradient": (None, [pmodel, pkfac, vp, vp]),
+    # include/fitre_fc.h
+    "fitre_build_nn": (None, [pnn, pi32, pi32, i32, i32, i32]),
+    "initSampledZOffsets": (None, [pnn, i32]),
+    "initRZOffsets": (None, [pnn, i32]),
+    "initSampledROffsets": (None, [pnn, i32]),
+    "nnForwardMemRequired": (lng, [pnn, i32]),
+    "nnGradientMemRequired": (lng, [pnn, i32]),
+    "applyLayerActivation": (None, [i32, vp, i32, i32, vp, i32, vp, i32, i32, vp, vp, vp]),
+    "nnForwardPass": (None, [pnn, pdata, vp, vp, vp, pf32, pf32, vp, vp, i32, i32]),
+    "evaluateModel": (None, [pnn, pdata, pscratch, vp, pf32, pf32, i32, i32]),
+    "computeGradient": (None, [pnn, pdata, pscratch, vp, vp, vp, vp, pf32, pf32, i32]),
     "getDeviceParameters": (None, []),
     "fitre_env_init": (None, [pscratch, i32, sz]),
     "cuda_env_init": (None, [pscratch, i32]),

@@ -60,6 +60,19 @@ class CNN_MODEL(C.Structure):
     ]
 
 
+class NN_MODEL(C.Structure):
+    """include/fitre_nn.h (nn/nn_decl.h:157-183 of the reference)."""
+    _fields_ = ([("layerSizes", C.c_int * MAX_LAYERS), ("actFuns", C.c_int * MAX_LAYERS)] +
+                [(n, C.c_int) for n in ("numLayers", "type", "pSize", "zSize", "sampledZSize", "sampledRSize", "rFullSize")] +
+                [(n, C.c_int * MAX_LAYERS) for n in ("wOffsets", "bOffsets", "zOffsets", "sZOffsets", "rZOffsets",
+                                                     "sRZOffsets")])
+
+
+MODEL_TYPE_MSE, MODEL_TYPE_CLASSIFICATION = 0, 1
+TEST_DATA, TRAIN_DATA = 0, 1
+FULL_DATASET, SAMPLED_DATASET = 0, 1
+
+
 class SCRATCH_AREA(C.Structure):
     _fields_ = [(n, C.c_void_p) for n in (
         "hostWorkspace", "devWorkspace", "pageLckWorkspace", "nextDevPtr", "nextHostPtr", "nextPageLckPtr")]

@@ -121,6 +121,21 @@ int fitre_hip_norm_inf(int n, const float *x, float *result);             /* dev
 int fitre_hip_sum(int n, const float *x, float *result);                  /* utilities/reduce.cu:32-84 */
 
 /* ---------------- elementwise helpers ---------------- */
+/* Output heads of the fully connected models (functions/eval_gradient.cu:231-555).
+ * column_softmax: x[:, c] = exp(x[:, c]) / sum_r exp(x[r, c]) in place, column-major rows x cols, no
+ * maximum shift (kerNNApplyExp + Dgemv column sums + kerNNComputeSoftmax, eval_gradient.cu:162-193).
+ * output_terms: out[i] = f(y[i], z[i]) with
+ *   SCALED_DIFFERENCE   scale*(y - z)                     kerNNComputeLayerError, dev_layer_error.cu:4-11
+ *   SQUARED_DIFFERENCE  (y - z)^2                         kerNNComputeLogLikelihoodLinear / kerNNComputeModelError
+ *   LOGISTIC_LL         z*(y - [z>=0]) - log(1 + exp(z - 2 z [z>=0]))   (z = logit) dev_loglikelihood.cu:22-41
+ *   SOFTMAX_LL          y*log(z)                          dev_loglikelihood.cu:4-11 */
+#define FITRE_TERM_SCALED_DIFFERENCE  0
+#define FITRE_TERM_SQUARED_DIFFERENCE 1
+#define FITRE_TERM_LOGISTIC_LL        2
+#define FITRE_TERM_SOFTMAX_LL         3
+int fitre_hip_column_softmax(float *x, int rows, int cols);
+int fitre_hip_output_terms(int kind, const float *y, const float *z, long n, float scale, float *out);
+
 /* Seeded generator replacing the cuRAND handle of device/gen_random.cu:25-52: a counter-based
  * stream (splitmix64 of seed and position; restated in the test oracle), uniform in (0, 1] resp.
  * standard normal (Box-Muller on consecutive pairs).  Each call continues the stream;

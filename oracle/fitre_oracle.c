@@ -829,6 +829,124 @@ void oracle_uniform_stream(unsigned long long seed, unsigned long long first, lo
 }
 
 /* ------------------------------------------------------------------ */
+/* fully connected model family (functions/eval_gradient.cu)           */
+/* ------------------------------------------------------------------ */
+
+/* functions/eval_gradient.cu:29-229 (applyLayerActivation) without the copy of W z + b behind the
+ * output (that copy belongs to the CNN path; for the last layer of an NN_MODEL it lies past zSize).
+ * ACT_SOFTMAX: exp, column sums, division -- no maximum shift (:162-193). */
+static int oracle_nn_layer(int actFunction, const real *W, int wRows, int wCols, const real *b, const real *z,
+                           int zCols, real *output)
+{
+	oracle_gemm(OP_N, OP_N, wRows, zCols, wCols, 1, W, wRows, z, wCols, 0, output, wRows);
+	if (b != NULL)
+		for (int n = 0; n < zCols; n++)
+			for (int r = 0; r < wRows; r++) output[(size_t)n * wRows + r] += b[r];
+	if (actFunction == ACT_SOFTMAX) {
+		for (int n = 0; n < zCols; n++) {
+			real sum = 0;
+			for (int r = 0; r < wRows; r++) {
+				output[(size_t)n * wRows + r] = exp(output[(size_t)n * wRows + r]);
+				sum += output[(size_t)n * wRows + r];
+			}
+			for (int r = 0; r < wRows; r++) output[(size_t)n * wRows + r] /= sum;
+		}
+		return 0;
+	}
+	if (actFunction == ACT_NONE) return 0;
+	return oracle_activation_forward(actFunction, output, (size_t)wRows * zCols);
+}
+
+/* functions/eval_gradient.cu:275-555 (nnForwardPass) on explicit data: dataset is features x numCols,
+ * target outSize x numColsTarget.  Fills z (at zOffsets) and errTerm, returns the log-likelihood
+ * figure (-(1/numColsTarget) * sum of the head's terms, dev_loglikelihood.cu:4-41) and *modelError. */
+real oracle_nn_forward(const NN_MODEL *model, const real *weights, const real *dataset, const real *target,
+                       int numCols, int numColsTarget, const int *zOffsets, real *z, real *errTerm,
+                       real *modelError, real *devScratch)
+{
+	const int numLayers = model->numLayers;
+	const int *layerSizes = model->layerSizes;
+	for (int i = 0; i < numLayers; i++) {
+		const real *in = (i == 0) ? dataset : z + zOffsets[i];
+		if (oracle_nn_layer(model->actFuns[i], weights + model->wOffsets[i], layerSizes[i + 1], layerSizes[i],
+		                    weights + model->bOffsets[i], in, numCols, z + zOffsets[i + 1]) != 0)
+			return (real)NAN;
+	}
+	const real *out = z + zOffsets[numLayers];
+	size_t numElements = (size_t)layerSizes[numLayers] * numColsTarget;
+	real logLikelihood = 0;
+	int head = model->actFuns[numLayers - 1];
+	if (head == ACT_LINEAR) {
+		for (size_t i = 0; i < numElements; i++) logLikelihood += pow(target[i] - out[i], 2.0);
+		for (size_t i = 0; i < numElements; i++) errTerm[i] = 2.0 * (target[i] - out[i]);
+	} else if (head == ACT_LOGISTIC) {
+		real *xi = devScratch;
+		const real *in = (numLayers == 1) ? dataset : z + zOffsets[numLayers - 1];
+		oracle_nn_layer(ACT_LINEAR, weights + model->wOffsets[numLayers - 1], layerSizes[numLayers],
+		                layerSizes[numLayers - 1], weights + model->bOffsets[numLayers - 1], in, numCols, xi);
+		for (size_t i = 0; i < numElements; i++) {
+			real lx = xi[i], lxx = (lx >= 0) ? 1 : 0;
+			logLikelihood += lx * (target[i] - lxx) - log(1 + exp(lx - 2.0 * lx * lxx));
+		}
+		for (size_t i = 0; i < numElements; i++) errTerm[i] = 1.0 * (target[i] - out[i]);
+	} else if (head == ACT_SOFTMAX) {
+		for (size_t i = 0; i < numElements; i++) logLikelihood += target[i] * log(out[i]);
+		for (size_t i = 0; i < numElements; i++) errTerm[i] = 1.0 * (target[i] - out[i]);
+	}
+	logLikelihood *= -1.0 / (real)numColsTarget;
+	*modelError = 0;
+	if (model->type == MODEL_TYPE_MSE) {
+		real e = 0;
+		for (size_t i = 0; i < numElements; i++) e += pow(target[i] - out[i], 2.0);
+		*modelError = e / (real)numColsTarget;
+	}
+	return logLikelihood;
+}
+
+/* functions/eval_gradient.cu:561-914 (computeGradient): forward pass, then per layer from the top
+ * db = sum(err, 2), dW = err * z_i', dx_i = err, err = W_i' * err with the logistic / tanh derivative
+ * of the layer below (dev_layer_error.cu:13-29), and the final scale -1/n.  The first layer's weight
+ * gradient reads the data set (:704).  errScratch holds max layer size x n reals. */
+real oracle_nn_gradient(const NN_MODEL *model, const real *weights, const real *dataset, const real *target, int n,
+                        const int *zOffsets, const int *rZOffsets, real *z, real *dx, real *gradient,
+                        real *modelError, real *errScratch, real *devScratch)
+{
+	const int numLayers = model->numLayers;
+	const int *layerSizes = model->layerSizes;
+	real *errorTerm = errScratch;
+	real ll = oracle_nn_forward(model, weights, dataset, target, n, n, zOffsets, z, errorTerm, modelError, devScratch);
+	real *next = devScratch;
+	for (int i = numLayers - 1; i >= 0; i--) {
+		int out = layerSizes[i + 1], in = layerSizes[i];
+		size_t count = (size_t)out * n;
+		if (i < numLayers - 1) {
+			const real *xi = z + zOffsets[i + 1];
+			if (model->actFuns[i] == ACT_LOGISTIC) {
+				for (size_t k = 0; k < count; k++) errorTerm[k] = errorTerm[k] * xi[k] * (1.0 - xi[k]);
+			} else if (model->actFuns[i] == ACT_TANH) {
+				for (size_t k = 0; k < count; k++) errorTerm[k] *= (1.0 + xi[k]) * (1.0 - xi[k]);
+			} else if (model->actFuns[i] != ACT_LINEAR) {
+				return (real)NAN;
+			}
+		}
+		for (int r = 0; r < out; r++) {
+			real sum = 0;
+			for (int c = 0; c < n; c++) sum += errorTerm[(size_t)c * out + r];
+			gradient[model->bOffsets[i] + r] = sum;
+		}
+		const real *zin = (i == 0) ? dataset : z + zOffsets[i];
+		oracle_gemm(OP_N, OP_T, out, in, n, 1, errorTerm, out, zin, in, 0, gradient + model->wOffsets[i], out);
+		memcpy(dx + rZOffsets[i], errorTerm, sizeof(real) * count);
+		if (i > 0) {
+			oracle_gemm(OP_T, OP_N, in, n, out, 1, weights + model->wOffsets[i], out, dx + rZOffsets[i], out, 0, next, in);
+			memcpy(errorTerm, next, sizeof(real) * (size_t)in * n);
+		}
+	}
+	for (int i = 0; i < model->pSize; i++) gradient[i] *= -(1.0 / (real)n);
+	return ll;
+}
+
+/* ------------------------------------------------------------------ */
 /* whole model                                                         */
 /* ------------------------------------------------------------------ */
 

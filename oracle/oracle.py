@@ -201,6 +201,30 @@ class Oracle:
         self.lib.oracle_uniform_stream(C.c_ulonglong(seed), C.c_ulonglong(first), C.c_long(n), self.p(out))
         return out
 
+    # ---- fully connected model family -----------------------------------
+    def nn_gradient(self, model, weights, dataset, target, n):
+        """(ll, model_error, gradient, z, dx) for an NN_MODEL whose z / rZ offsets were built for n points."""
+        weights, dataset, target = self.arr(weights), self.arr(dataset), self.arr(target)
+        big = max(model.layerSizes[i] for i in range(model.numLayers + 1)) * n
+        z, dx, grad = self.zeros(model.zSize + big), self.zeros(model.rFullSize + big), self.zeros(model.pSize)
+        err, scratch = self.zeros(big), self.zeros(big)
+        merr = self.creal(0)
+        self.lib.oracle_nn_gradient.restype = self.creal
+        ll = self.lib.oracle_nn_gradient(C.byref(model), self.p(weights), self.p(dataset), self.p(target), n, model.zOffsets,
+                                         model.rZOffsets, self.p(z), self.p(dx), self.p(grad), C.byref(merr), self.p(err),
+                                         self.p(scratch))
+        return float(ll), float(merr.value), grad, z[:model.zSize], dx[:model.rFullSize]
+
+    def nn_forward(self, model, weights, dataset, target, n_cols, n_cols_target):
+        weights, dataset, target = self.arr(weights), self.arr(dataset), self.arr(target)
+        big = max(model.layerSizes[i] for i in range(model.numLayers + 1)) * max(n_cols, n_cols_target)
+        z, err, scratch = self.zeros(model.zSize + big), self.zeros(big), self.zeros(big)
+        merr = self.creal(0)
+        self.lib.oracle_nn_forward.restype = self.creal
+        ll = self.lib.oracle_nn_forward(C.byref(model), self.p(weights), self.p(dataset), self.p(target), n_cols,
+                                        n_cols_target, model.zOffsets, self.p(z), self.p(err), C.byref(merr), self.p(scratch))
+        return float(ll), float(merr.value), z[:model.zSize], err[:model.layerSizes[model.numLayers] * n_cols_target]
+
     def activation_forward(self, act, x):
         x = self.arr(x).copy()
         rc = self.lib.oracle_activation_forward(act, self.p(x), C.c_size_t(x.size))
