@@ -146,3 +146,37 @@ void getRandomVector(int n, real *hostPtr, real *devPtr, RAND_GENERATOR r)
 	if (hostPtr != NULL && fitre_hip_copy_d2h(hostPtr, devPtr, sizeof(real) * (size_t)n)) die("getRandomVector: copy", -1);
 	if (hostPtr == NULL && fitre_hip_sync()) die("getRandomVector: sync", -1);
 }
+
+void writeVector(real *mat, int rows, char *file, int hostData, real *dscratch)
+{
+	FILE *f = fopen(file, "w");
+	real *t = dscratch;
+	if (f == NULL) {
+		fprintf(stderr, "Error opening the path .... !\n");
+		exit(-1);
+	}
+	if (hostData == 1)
+		t = mat;
+	else if (fitre_hip_copy_d2h(t, mat, sizeof(real) * (size_t)rows))
+		die("writeVector: copy", -1);
+	for (int i = 0; i < rows; i++) fprintf(f, "%6.10f\n", t[i]);
+	fclose(f);
+}
+
+int readVector(real *vec, int rows, char *file, int offset, real *dscratch)
+{
+	(void)dscratch;
+	FILE *handle = fopen(file, "r");
+	char line[1024];
+	int index = 0;
+	if (handle == NULL) {
+		fprintf(stderr, "Error opening the path... \n");
+		exit(-1);
+	}
+	while (index < rows && fgets(line, sizeof(line), handle) != NULL) {
+		if (line[0] == 0 || line[0] == '\n') break;
+		vec[index++] = (real)atof(line) + (real)offset;
+	}
+	fclose(handle);
+	return index;
+}

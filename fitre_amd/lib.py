@@ -133,6 +133,8 @@ CNN_API = {
     "getMultinomialDistSample": (None, [vp, i32, i32, vp, vp]),
     "computeDistributionErrors": (None, [vp, vp, vp, i32, i32, vp, vp]),
     "getRandomVector": (None, [i32, vp, vp, i32]),
+    "writeVector": (None, [vp, i32, C.c_char_p, i32, vp]),
+    "readVector": (i32, [vp, i32, C.c_char_p, i32, vp]),
     # include/fitre_kfac.h
     "computeKFACStorageIndices": (None, [pmodel, pkfac]),
     "kfacFactorsMemRequired": (lng, [pmodel, i32]),

@@ -46,6 +46,13 @@ void copy_host_device(void *host, void *dev, size_t size, enum cudaMemcpyKind di
 void copy_device(void *dst, void *src, size_t size, int err_code);
 void print_device_mem_usage(void);
 
+/* utilities/print_utils.c:136-186: one value per line, "%6.10f".  writeVector: hostData == 1 writes the
+ * host vector mat; otherwise mat is a device vector and dscratch a host buffer of at least rows reals.
+ * readVector: reads up to rows values into the HOST vector vec, adds offset to each, returns the count
+ * (the format of the <net>_<init>.params files, e.g. pytorch/kfac/lenet_xavier.txt). */
+void writeVector(real *mat, int rows, char *file, int hostData, real *dscratch);
+int readVector(real *vec, int rows, char *file, int offset, real *dscratch);
+
 /* device/gen_random.h:6-13: n standard-normal or uniform (0, 1] reals into devPtr, copied to hostPtr
  * when it is not NULL.  The stream is seeded with fitre_hip_random_seed(). */
 typedef enum random_generator { RAND_NORMAL = 1, RAND_UNIFORM } RAND_GENERATOR;

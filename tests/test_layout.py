@@ -145,3 +145,26 @@ def test_workspace_requirements_are_positive_and_modest():
     m = build_vgg11(256)
     fwd, bwd = L.cnn.cnnForwardMemRequired(C.byref(m)), L.cnn.cnnBackwardMemRequired(C.byref(m))
     assert 0 < fwd * 4 < 512e6 and 0 < bwd * 4 < 512e6
+
+
+def test_vector_text_io_round_trip(tmp_path):
+    """readVector / writeVector (utilities/print_utils.c:136-186): the first lines of the reference's LeNet weight
+    file parse to the values numpy reads, and a written vector reads back to the printed precision."""
+    here = os.path.dirname(os.path.abspath(__file__))
+    path = os.path.join(here, "golden", "lenet_xavier_head.txt")
+    want = np.loadtxt(path)
+    vec = np.zeros(100, dtype=np.float32)
+    got = L.cnn.readVector(vec.ctypes.data_as(C.c_void_p), 100, path.encode(), 0, None)
+    assert got == want.size == 64
+    np.testing.assert_array_equal(vec[:64], want.astype(np.float32))
+    # fewer rows than lines, and the additive offset (used for 1-based labels)
+    got = L.cnn.readVector(vec.ctypes.data_as(C.c_void_p), 10, path.encode(), 1, None)
+    assert got == 10
+    np.testing.assert_allclose(vec[:10], want[:10] + 1, atol=1e-6)
+    out = str(tmp_path / "v.txt").encode()
+    src = np.array([0.5, -1.25, 3.0000000001, 1e-11], dtype=np.float32)
+    L.cnn.writeVector(src.ctypes.data_as(C.c_void_p), 4, out, 1, None)
+    assert open(out).read().splitlines() == ["0.5000000000", "-1.2500000000", "3.0000000000", "0.0000000000"]
+    back = np.zeros(4, dtype=np.float32)
+    assert L.cnn.readVector(back.ctypes.data_as(C.c_void_p), 4, out, 0, None) == 4
+    np.testing.assert_allclose(back, src, atol=1e-10)
