@@ -1162,4 +1162,376 @@ real oracle_cnn_gradient(const CNN_MODEL *model, const real *weights, const real
 	return loss;
 }
 
+
+/* ------------------------------------------------------------------ */
+/* Hessian-vector product (R-operator forward and backward passes)     */
+/* ------------------------------------------------------------------ */
+/*
+ * Restatement of functions/cnn_hessian_vec.cu:18-122 (cnnHv), cnn_hv_forward.cu:53-222
+ * (cnnROpForward), cnn_hv_backward.cu:70-912 (cnnROpBackward), rop_fc_layer.cu:34-133
+ * (applyROpLayerActivation), eval_convolution.cu:285-... (applyROpConvolutionLayer),
+ * dev_pool.cu:123-221 (applyROpPoolLayer), dev_batch_norm.cu:637-960 (batch-norm R-op) and
+ * softmax_loss.cu:251-300 (computeROpCrossEntropyError_simple): R{.} is the directional derivative
+ * along `vector` in weight space; the forward pass carries R{z} through every layer, the backward
+ * pass carries R{delta} and emits R{gradient} = H * vector.
+ * Departures from the reference code, all of them defects there: every layer uses its own
+ * activation (the reference passes actFuns[0] for all, cnn_hv_forward.cu:125), the batch-norm R-op
+ * indexes variances by channel (dev_batch_norm.cu:181 indexes by element), the swish second
+ * derivative is evaluated per element (swish.cu:47 multiplies the index), and D1-D6 of the
+ * gradient path apply unchanged.
+ */
+
+/* out = rdelta * f'(.) + delta * f''(.) * rz_in: the R-operator of delta * f'(.)
+ * (first derivatives as in oracle_activation_backward; second derivatives: logistic a(1-a)(1-2a),
+ * tanh -2a(1-a^2), softplus s(1-s), swish s(1-s)(2 + x(1-2s)), ELU e^x below zero, ReLU 0). */
+int oracle_activation_rop_backward(int actFun, const real *rdelta, const real *delta, const real *z_in,
+                                   const real *z_out, const real *rz_in, real *out, size_t n)
+{
+	for (size_t i = 0; i < n; i++) {
+		real f1, f2;
+		switch (actFun) {
+		case ACT_LOGISTIC: {
+			real a = z_out[i];
+			f1 = a * (1.0 - a), f2 = a * (1.0 - a) * (1.0 - 2.0 * a);
+			break;
+		}
+		case ACT_TANH: {
+			real a = z_out[i];
+			f1 = (1.0 + a) * (1.0 - a), f2 = -2.0 * a * (1.0 + a) * (1.0 - a);
+			break;
+		}
+		case CNN_ACT_SOFTPLUS: {
+			real s = 1. / (1. + exp(-z_in[i]));
+			f1 = s, f2 = s * (1. - s);
+			break;
+		}
+		case CNN_ACT_SWISH: {
+			real x = z_in[i], s = 1. / (1. + exp(-x));
+			f1 = z_out[i] + s * (1. - z_out[i]);
+			f2 = s * (1. - s) * (2. + x * (1. - 2. * s));
+			break;
+		}
+		case CNN_ACT_RELU:
+			f1 = (z_out[i] > 0) ? 1 : 0, f2 = 0;
+			break;
+		case CNN_ACT_ELU:
+			f1 = (z_out[i] < 0) ? z_out[i] + 1.0 : 1, f2 = (z_out[i] < 0) ? z_out[i] + 1.0 : 0;
+			break;
+		case ACT_LINEAR:
+		case CNN_ACT_NONE:
+			f1 = 1, f2 = 0;
+			break;
+		default:
+			return -1;
+		}
+		out[i] = rdelta[i] * f1 + delta[i] * f2 * rz_in[i];
+	}
+	return 0;
+}
+
+/* dev_pool.cu:123-174 (ker_rop_max_pool_layer): R{max pool} picks R{z} where z has its maximum
+ * (first maximum in memory order, as the pooling itself). */
+void oracle_max_pool_forward_routed(const real *values, const real *z_act, int samples, int channels, int height,
+                                    int width, int ksize, int stride, int padding, int p_height, int p_width,
+                                    real *output)
+{
+	size_t maps = (size_t)samples * channels;
+	for (size_t m = 0; m < maps; m++) {
+		const real *in = z_act + m * height * width, *val = values + m * height * width;
+		real *out = output + m * p_height * p_width;
+		for (int pw = 0; pw < p_width; pw++)
+			for (int ph = 0; ph < p_height; ph++) {
+				int idx = argmax_in_window(in, height, width, ksize, ph * stride - padding, pw * stride - padding);
+				out[ph + pw * p_height] = (idx == INT_MAX) ? 0 : val[idx];
+			}
+	}
+}
+
+/* R-operator of the batch-norm backward formula (dev_batch_norm.cu:787-960), per channel with
+ * s = sqrt(var + eps), m elements, <.> the mean over the channel:
+ *   R{dc} = ( R{dx} - <R{dx}> - R{zhat} <dx zhat> - zhat ( <R{dx} zhat> + <dx R{zhat}> ) ) / s
+ *           - dc <zhat R{x}> / s
+ * dx = gradient at the batch-norm output, dc = at its input, x the input itself. */
+void oracle_batch_norm_rop_backward(const real *rdelta_x, const real *delta_x, const real *zhat, const real *rzhat,
+                                    const real *rx, const real *delta_c, const real *variance, int height, int width,
+                                    int channels, int samples, real epsilon, real *output)
+{
+	size_t rows = (size_t)height * width * samples;
+#pragma omp parallel for schedule(static)
+	for (int c = 0; c < channels; c++) {
+		size_t o = (size_t)c * rows;
+		real a = 0, b = 0, cc = 0, d = 0, e = 0;
+		for (size_t i = 0; i < rows; i++) {
+			a += rdelta_x[o + i];
+			b += delta_x[o + i] * zhat[o + i];
+			cc += rdelta_x[o + i] * zhat[o + i];
+			d += delta_x[o + i] * rzhat[o + i];
+			e += zhat[o + i] * rx[o + i];
+		}
+		real m = (real)rows, s = sqrt(variance[c] + epsilon);
+		a /= m, b /= m, cc /= m, d /= m, e /= m;
+		for (size_t i = 0; i < rows; i++)
+			output[o + i] = (rdelta_x[o + i] - a - rzhat[o + i] * b - zhat[o + i] * (cc + d)) / s - delta_c[o + i] * e / s;
+	}
+}
+
+/* softmax_loss.cu:251-300: R{(p - y)/rows} = p_i (R{z_i} - sum_j p_j R{z_j}) / rows. */
+void oracle_cross_entropy_rop_error(const real *rz, const real *probs, int rows, int numclasses, real *rError)
+{
+	for (int idx = 0; idx < rows; idx++) {
+		real s = 0;
+		for (int j = 0; j < numclasses; j++) s += probs[(size_t)idx * numclasses + j] * rz[(size_t)idx * numclasses + j];
+		for (int i = 0; i < numclasses; i++)
+			rError[(size_t)idx * numclasses + i] =
+			    probs[(size_t)idx * numclasses + i] * (rz[(size_t)idx * numclasses + i] - s) / (real)rows;
+	}
+}
+
+static void feature_dims(const CNN_MODEL *model, int *fh, int *fw)
+{
+	const CONV_LAYER *c = &model->convLayer[model->cLayers - 1];
+	const POOL_LAYER *p = &model->poolLayer[model->cLayers - 1];
+	*fh = (p->type != NO_POOL) ? p->outHeight : c->outHeight;
+	*fw = (p->type != NO_POOL) ? p->outWidth : c->outWidth;
+}
+
+/* activation output of conv layer l in the convolution layout (departure D6: the last layer's
+ * unpooled output was permuted in place by the forward pass and is rebuilt into tmp) */
+static const real *conv_act_out(const CNN_MODEL *model, int l, const real *z, int n, real *tmp)
+{
+	const CONV_LAYER *c = &model->convLayer[l];
+	const real *slab = z + model->zOffsets[l + 1];
+	if (l == model->cLayers - 1 && model->poolLayer[l].type == NO_POOL) {
+		size_t count = (size_t)n * c->activationVolumn;
+		const real *actIn = (c->batchNorm != PERFORM_NO_BATCH_NORM) ? slab + c->batchNormOffset : slab;
+		memcpy(tmp, actIn, sizeof(real) * count);
+		oracle_activation_forward(model->actFuns[l], tmp, count);
+		return tmp;
+	}
+	return slab + c->activationOffset;
+}
+
+/* cnn_hv_forward.cu:53-222.  rz has the layout of z. */
+int oracle_cnn_rop_forward(const CNN_MODEL *model, const real *weights, const real *vector, const real *x,
+                           const real *z, real *rz, int n)
+{
+	const int *wOffsets = model->wOffsets, *bOffsets = model->bOffsets, *zOffsets = model->zOffsets;
+	int nc = model->cLayers;
+	size_t big = max_patch_reals(model, n) + (size_t)model->maxDeltaSize;
+	real *scratch = (real *)malloc(sizeof(real) * big), *tmp = (real *)malloc(sizeof(real) * (size_t)model->maxDeltaSize);
+	if (!scratch || !tmp) return -1;
+	for (int l = 0; l < nc; l++) {
+		const CONV_LAYER *c = &model->convLayer[l];
+		const POOL_LAYER *p = &model->poolLayer[l];
+		const real *slab = z + zOffsets[l + 1];
+		real *rslab = rz + zOffsets[l + 1];
+		size_t M = (size_t)n * c->outHeight * c->outWidth, count = M * c->outChannels;
+		int K = c->kSize * c->kSize * c->inChannels;
+		const real *in = (l == 0) ? x : z + zOffsets[l] + model->convLayer[l - 1].outputOffset;
+		/* R{conv} = im2col(z_in) * V + im2col(R{z_in}) * W + Vb */
+		oracle_im2col(in, n, c->inChannels, c->height, c->width, c->kSize, c->padding, c->stride, scratch);
+		oracle_gemm(OP_N, OP_N, (int)M, c->outChannels, K, 1, scratch, (int)M, vector + wOffsets[l], K, 0, rslab, (int)M);
+		if (l > 0) {
+			const real *rin = rz + zOffsets[l] + model->convLayer[l - 1].outputOffset;
+			oracle_im2col(rin, n, c->inChannels, c->height, c->width, c->kSize, c->padding, c->stride, scratch);
+			oracle_gemm(OP_N, OP_N, (int)M, c->outChannels, K, 1, scratch, (int)M, weights + wOffsets[l], K, 1, rslab, (int)M);
+		}
+		if (model->bias != 0)
+			for (int o = 0; o < c->outChannels; o++)
+				for (size_t i = 0; i < M; i++) rslab[(size_t)o * M + i] += vector[bOffsets[l] + o];
+		const real *rpre = rslab, *actIn = slab;
+		if (c->batchNorm != PERFORM_NO_BATCH_NORM) {
+			/* R{zhat} = (R{x} - <R{x}> - zhat <zhat R{x}>) / s: the backward formula applied to R{x} */
+			oracle_batch_norm_backward(rslab, c->outHeight, c->outWidth, c->outChannels, n,
+			                           slab + c->batchNormOffset + c->variancesOffset, rslab + c->batchNormOffset,
+			                           slab + c->batchNormOffset, BATCH_NORM_EPSILON);
+			rpre = rslab + c->batchNormOffset;
+			actIn = slab + c->batchNormOffset;
+		}
+		const real *actOut = conv_act_out(model, l, z, n, tmp);
+		real *ract = rslab + c->activationOffset;
+		memcpy(ract, rpre, sizeof(real) * count);
+		if (oracle_activation_backward(model->actFuns[l], ract, actIn, actOut, count)) return -1;
+		if (p->type == MAX_POOL)
+			oracle_max_pool_forward_routed(ract, actOut, n, c->outChannels, c->outHeight, c->outWidth, p->pSize, p->stride,
+			                               p->padding, p->outHeight, p->outWidth, rslab + c->poolOffset);
+		else if (p->type == AVG_POOL)
+			oracle_avg_pool_forward(ract, n, c->outChannels, c->outHeight, c->outWidth, p->pSize, p->stride, p->padding,
+			                        p->outHeight, p->outWidth, rslab + c->poolOffset);
+		else if (p->type != NO_POOL)
+			return -1;
+	}
+	/* feature permute of R{z}, as the forward pass did for z (cnn_hv_forward.cu:178-195) */
+	const CONV_LAYER *c = &model->convLayer[nc - 1];
+	int fh, fw;
+	feature_dims(model, &fh, &fw);
+	real *rfeat = rz + zOffsets[nc] + c->outputOffset;
+	oracle_reshape(rfeat, c->outChannels, n, fh * fw, scratch);
+	oracle_transpose(scratch, c->outChannels * n, fh, fw, rfeat);
+
+	for (int f = 0; f < model->lLayers; f++) {
+		const FC_LAYER *fc = &model->fcLayer[f];
+		int at = nc + f;
+		int off = (f == 0) ? c->outputOffset : 0;
+		const real *zin = z + zOffsets[at] + off, *rzin = rz + zOffsets[at] + off;
+		const real *zl = z + zOffsets[at + 1];
+		real *rzl = rz + zOffsets[at + 1];
+		size_t count = (size_t)fc->out * n;
+		real *rpre = rzl + fc->offset;
+		/* R{W z + b} = V z + W R{z} + Vb (rop_fc_layer.cu:34-133) */
+		oracle_gemm(OP_N, OP_N, fc->out, n, fc->in, 1, vector + wOffsets[at], fc->out, zin, fc->in, 0, rpre, fc->out);
+		oracle_gemm(OP_N, OP_N, fc->out, n, fc->in, 1, weights + wOffsets[at], fc->out, rzin, fc->in, 1, rpre, fc->out);
+		if (model->bias != 0)
+			for (int i = 0; i < n; i++)
+				for (int r = 0; r < fc->out; r++) rpre[(size_t)i * fc->out + r] += vector[bOffsets[at] + r];
+		memcpy(rzl, rpre, sizeof(real) * count);
+		if (oracle_activation_backward(fc->actFun, rzl, zl + fc->offset, zl, count)) return -1;
+	}
+	free(scratch);
+	free(tmp);
+	return 0;
+}
+
+/* cnn_hv_backward.cu:70-912.  rError = R{loss errors}; hv receives R{gradient}. */
+int oracle_cnn_rop_backward(const CNN_MODEL *model, const real *weights, const real *vector, const real *x,
+                            const real *z, const real *rz, const real *dx, const real *lossFuncErrors,
+                            const real *rError, real *hv, int n, int numClasses)
+{
+	const int *wOffsets = model->wOffsets, *bOffsets = model->bOffsets, *zOffsets = model->zOffsets;
+	int nc = model->cLayers;
+	size_t dsz = (size_t)model->maxDeltaSize;
+	real *scratch = (real *)malloc(sizeof(real) * (max_patch_reals(model, n) + dsz));
+	real *rdelta = (real *)calloc(dsz, sizeof(real)), *rnext = (real *)calloc(dsz, sizeof(real));
+	real *dout = (real *)calloc(dsz, sizeof(real)), *tmp = (real *)calloc(dsz, sizeof(real));
+	real *wtmp = (real *)calloc((size_t)model->pSize, sizeof(real));
+	if (!scratch || !rdelta || !rnext || !dout || !tmp || !wtmp) return -1;
+	const CONV_LAYER *last = &model->convLayer[nc - 1];
+	memcpy(rdelta, rError, sizeof(real) * (size_t)numClasses * n);
+	memcpy(dout, lossFuncErrors, sizeof(real) * (size_t)numClasses * n);
+
+	for (int f = model->lLayers - 1; f >= 0; f--) {
+		const FC_LAYER *fc = &model->fcLayer[f];
+		int at = nc + f;
+		int off = (f == 0) ? last->outputOffset : 0;
+		const real *zl = z + zOffsets[at + 1], *rzl = rz + zOffsets[at + 1];
+		const real *zin = z + zOffsets[at] + off, *rzin = rz + zOffsets[at] + off;
+		const real *dpre = dx + zOffsets[at + 1];
+		size_t count = (size_t)fc->out * n;
+		/* R{delta f'(x)} */
+		if (oracle_activation_rop_backward(fc->actFun, rdelta, dout, zl + fc->offset, zl, rzl + fc->offset, tmp, count))
+			return -1;
+		/* R{dW} = R{d} z' + d R{z}' ; R{db} = R{d} 1 */
+		oracle_gemm(OP_N, OP_T, fc->out, fc->in, n, 1, tmp, fc->out, zin, fc->in, 0, hv + wOffsets[at], fc->out);
+		oracle_gemm(OP_N, OP_T, fc->out, fc->in, n, 1, dpre, fc->out, rzin, fc->in, 1, hv + wOffsets[at], fc->out);
+		if (model->bias != 0)
+			for (int r = 0; r < fc->out; r++) {
+				real s = 0;
+				for (int i = 0; i < n; i++) s += tmp[(size_t)i * fc->out + r];
+				hv[bOffsets[at] + r] = s;
+			}
+		/* R{W' d} = V' d + W' R{d};  and the gradient at the output of the layer below, W' d */
+		oracle_gemm(OP_T, OP_N, fc->in, n, fc->out, 1, vector + wOffsets[at], fc->out, dpre, fc->out, 0, rnext, fc->in);
+		oracle_gemm(OP_T, OP_N, fc->in, n, fc->out, 1, weights + wOffsets[at], fc->out, tmp, fc->out, 1, rnext, fc->in);
+		oracle_gemm(OP_T, OP_N, fc->in, n, fc->out, 1, weights + wOffsets[at], fc->out, dpre, fc->out, 0, dout, fc->in);
+		real *t = rdelta;
+		rdelta = rnext;
+		rnext = t;
+	}
+	{
+		int fh, fw;
+		feature_dims(model, &fh, &fw);
+		oracle_reshape(rdelta, n, last->outChannels, fh * fw, scratch);
+		oracle_transpose_rc(scratch, last->outChannels * n, fh, fw, rdelta);
+	}
+	for (int c = nc - 1; c >= 0; c--) {
+		const CONV_LAYER *l = &model->convLayer[c];
+		const POOL_LAYER *p = &model->poolLayer[c];
+		const real *slab = z + zOffsets[c + 1], *rslab = rz + zOffsets[c + 1], *dslab = dx + zOffsets[c + 1];
+		size_t count = (size_t)n * l->activationVolumn;
+		int bn = l->batchNorm != PERFORM_NO_BATCH_NORM;
+		const real *actIn = bn ? slab + l->batchNormOffset : slab;
+		const real *ractIn = bn ? rslab + l->batchNormOffset : rslab;
+		const real *actOut = conv_act_out(model, c, z, n, tmp);
+		/* R through the pooling: the same routing as the gradient (dev_pool.cu:346-398) */
+		if (p->type == MAX_POOL)
+			oracle_max_pool_backward(rdelta, actOut, l->outChannels, p->height, p->width, p->pSize, p->stride, p->padding,
+			                         p->outHeight, p->outWidth, n, rnext);
+		else if (p->type == AVG_POOL)
+			oracle_avg_pool_backward(rdelta, l->outChannels, p->height, p->width, p->pSize, p->stride, p->padding,
+			                         p->outHeight, p->outWidth, n, rnext);
+		else if (p->type == NO_POOL)
+			memcpy(rnext, rdelta, sizeof(real) * count);
+		else
+			return -1;
+		/* R{delta f'(x)}: delta at the activation output is the dx snapshot at +0 */
+		if (oracle_activation_rop_backward(model->actFuns[c], rnext, dslab, actIn, actOut, ractIn, rdelta, count)) return -1;
+		const real *dc = dslab + l->activationOffset; /* gradient at the convolution output */
+		real *rdc = rdelta;
+		if (bn) {
+			oracle_batch_norm_rop_backward(rdelta, dslab + l->activationOffset, slab + l->batchNormOffset,
+			                               rslab + l->batchNormOffset, rslab, dslab + l->batchNormOffset,
+			                               slab + l->batchNormOffset + l->variancesOffset, l->outHeight, l->outWidth,
+			                               l->outChannels, n, BATCH_NORM_EPSILON, rnext);
+			dc = dslab + l->batchNormOffset;
+			rdc = rnext;
+		}
+		size_t M = (size_t)p->height * p->width * n;
+		if (model->bias != 0)
+			for (int o = 0; o < l->outChannels; o++) {
+				real s = 0;
+				for (size_t i = 0; i < M; i++) s += rdc[(size_t)o * M + i];
+				hv[bOffsets[c] + o] = s;
+			}
+		const real *in = (c == 0) ? x : z + zOffsets[c] + model->convLayer[c - 1].outputOffset;
+		size_t wcount = (size_t)l->outChannels * l->inChannels * l->kSize * l->kSize;
+		/* R{dW} = im2col(z_in)' R{dc} + im2col(R{z_in})' dc */
+		oracle_conv_weight_gradient(in, rdc, n, l->inChannels, l->height, l->width, l->kSize, l->padding, l->stride,
+		                            l->outChannels, hv + wOffsets[c], scratch);
+		if (c != 0) {
+			const real *rin = rz + zOffsets[c] + model->convLayer[c - 1].outputOffset;
+			oracle_conv_weight_gradient(rin, dc, n, l->inChannels, l->height, l->width, l->kSize, l->padding, l->stride,
+			                            l->outChannels, wtmp, scratch);
+			for (size_t i = 0; i < wcount; i++) hv[wOffsets[c] + i] += wtmp[i];
+			/* R{dX} = dX(R{dc}, W) + dX(dc, V) */
+			real *other = (rdc == rdelta) ? rnext : rdelta;
+			size_t inCount = (size_t)n * l->height * l->width * l->inChannels;
+			oracle_conv_input_gradient(rdc, p->height, p->width, l->outChannels, weights + wOffsets[c], l->kSize, l->kSize,
+			                           l->height, l->width, l->padding, l->inChannels, n, other, scratch);
+			oracle_conv_input_gradient(dc, p->height, p->width, l->outChannels, vector + wOffsets[c], l->kSize, l->kSize,
+			                           l->height, l->width, l->padding, l->inChannels, n, tmp, scratch);
+			for (size_t i = 0; i < inCount; i++) other[i] += tmp[i];
+			if (other != rdelta) {
+				real *t = rdelta;
+				rdelta = rnext;
+				rnext = t;
+			}
+		}
+	}
+	free(scratch), free(rdelta), free(rnext), free(dout), free(tmp), free(wtmp);
+	return 0;
+}
+
+/* cnn_hessian_vec.cu:18-122 (cnnHv): R forward, R of the loss errors, R backward.  z, probs,
+ * lossFuncErrors and dx come from oracle_cnn_gradient on the same batch.  No weight-decay term
+ * (the reference leaves that to computeQuadraticModel). */
+int oracle_cnn_hv(const CNN_MODEL *model, const real *weights, const real *x, const real *z, const real *probs,
+                  const real *lossFuncErrors, const real *dx, const real *vector, real *hv, int n, int numClasses)
+{
+	int nc = model->cLayers;
+	real *rz = (real *)calloc((size_t)model->zSize, sizeof(real));
+	real *rError = (real *)calloc((size_t)numClasses * n, sizeof(real));
+	if (!rz || !rError) return -1;
+	int rc = oracle_cnn_rop_forward(model, weights, vector, x, z, rz, n);
+	if (rc == 0) {
+		const real *rlogits = (model->lLayers == 0)
+		                          ? rz + model->zOffsets[nc] + model->convLayer[nc - 1].outputOffset
+		                          : rz + model->zOffsets[nc + model->lLayers];
+		oracle_cross_entropy_rop_error(rlogits, probs, n, numClasses, rError);
+		rc = oracle_cnn_rop_backward(model, weights, vector, x, z, rz, dx, lossFuncErrors, rError, hv, n, numClasses);
+	}
+	free(rz);
+	free(rError);
+	return rc;
+}
+
 int oracle_sizeof_real(void) { return (int)sizeof(real); }

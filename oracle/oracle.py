@@ -85,6 +85,17 @@ class Oracle:
                                             batch, self.r(weight_decay))
         return dict(loss=float(loss), gradient=grad, z=z, dx=dx, probs=probs, errors=errors)
 
+    def hessian_vector(self, model: CNN_MODEL, weights, x, z, probs, errors, dx, vector, classes, batch):
+        """H * vector of the mean loss at `weights` (no weight-decay term), from the z / probs / errors / dx of a
+        gradient call on the same batch."""
+        arrs = [self.arr(a) for a in (weights, x, z, probs, errors, dx, vector)]
+        hv = self.zeros(model.pSize)
+        rc = self.lib.oracle_cnn_hv(C.byref(model), self.p(arrs[0]), self.p(arrs[1]), self.p(arrs[2]), self.p(arrs[3]),
+                                    self.p(arrs[4]), self.p(arrs[5]), self.p(arrs[6]), self.p(hv), batch, classes)
+        if rc != 0:
+            raise ValueError("oracle_cnn_hv failed (unknown activation or pool code)")
+        return hv
+
     # ---- single operations ------------------------------------------------
     def gemm(self, ta, tb, M, N, K, alpha, A, lda, B, ldb, beta, Cm, ldc):
         A, B, Cm = self.arr(A), self.arr(B), self.arr(Cm).copy()

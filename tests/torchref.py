@@ -132,3 +132,43 @@ def run(model, wflat, x_flat, y, batch, dtype=torch.float64, want_intermediates=
     loss.backward()
     return dict(loss=loss.item(), gradient=pack_grads(model, convs, fcs), stages=stages, fc_stages=fc_stages,
                 logits=h.detach().numpy())
+
+
+def forward_loss(model, convs, fcs, x_flat, y, batch, dtype=torch.float64):
+    c0 = model.convLayer[0]
+    h = to_nchw(x_flat, c0.inChannels, batch, c0.width, c0.height, dtype)
+    for l in range(model.cLayers):
+        c, p = model.convLayer[l], model.poolLayer[l]
+        W, b = convs[l]
+        pre = F.conv2d(h, W, b, stride=c.stride, padding=c.padding)
+        if c.batchNorm != PERFORM_NO_BATCH_NORM:
+            pre = F.batch_norm(pre, None, None, training=True, eps=1e-5)
+        h = act_torch(model.actFuns[l], pre)
+        if p.type == MAX_POOL:
+            h = F.max_pool2d(h, p.pSize, p.stride, p.padding)
+        elif p.type == AVG_POOL:
+            h = F.avg_pool2d(h, p.pSize, p.stride, p.padding, count_include_pad=True)
+    h = h.reshape(batch, -1)
+    for f in range(model.lLayers):
+        W, b = fcs[f]
+        h = act_torch(model.fcLayer[f].actFun, F.linear(h, W, b))
+    return F.cross_entropy(h, torch.tensor(np.asarray(y, dtype=np.int64) - 1))
+
+
+def hessian_vector(model, wflat, x_flat, y, batch, vflat):
+    """H * v of the mean cross-entropy loss by double backward, in the flat parameter layout."""
+    convs, fcs = unpack(model, wflat)
+    vconvs, vfcs = unpack(model, vflat)
+    params = [t for pair in convs + fcs for t in pair if t is not None]
+    vs = [t.detach() for pair in vconvs + vfcs for t in pair if t is not None]
+    loss = forward_loss(model, convs, fcs, x_flat, y, batch)
+    grads = torch.autograd.grad(loss, params, create_graph=True)
+    dot = sum((g * v).sum() for g, v in zip(grads, vs))
+    hv = torch.autograd.grad(dot, params, allow_unused=True)
+    it = iter(hv)
+    for pair in convs + fcs:
+        for t in pair:
+            if t is not None:
+                g = next(it)
+                t.grad = torch.zeros_like(t) if g is None else g
+    return pack_grads(model, convs, fcs)
