@@ -122,6 +122,7 @@ def gpu_leg(args):
     grad = gm.get("grad")
     finite = bool(np.isfinite(grad).all() and np.isfinite(loss))
     kfac = kfac_leg(L, dev, gm, model, batch, max(2, args.steps // 4))
+    kfac["hessian_vector_ms"] = hv_leg(L, dev, gm, model, batch, max(2, args.steps // 4))
     gm.release()
     dev.close()
 
@@ -226,6 +227,27 @@ def kfac_leg(L, dev, gm, model, batch, passes):
     for q in (omega, lam, ws, ws2, ngrad):
         dev.free(q)
     return out
+
+
+def hv_leg(L, dev, gm, model, batch, passes):
+    """cnnHv (R-operator forward and backward passes) along a random direction, on the z / dx in HBM."""
+    v = dev.upload(np.random.default_rng(5).standard_normal(model.pSize).astype(np.float32))
+    hv = dev.zeros(model.pSize)
+    ws = dev.alloc(4 * L.cnn.cnnHvMemRequired(C.byref(model)) + 512)
+
+    def run():
+        L.cnn.cnnHv(C.byref(model), C.byref(gm.data), gm.z, gm.probs, gm.errors, gm.dx, v, hv, 0, batch, ws, None, 0.0)
+
+    run()
+    dev.sync()
+    t0 = time.perf_counter()
+    for _ in range(passes):
+        run()
+    dev.sync()
+    ms = 1e3 * (time.perf_counter() - t0) / passes
+    for q in (v, hv, ws):
+        dev.free(q)
+    return round(ms, 4)
 
 
 def cpu_leg(batch=64, repeats=10):

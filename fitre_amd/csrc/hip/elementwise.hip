@@ -291,6 +291,39 @@ __global__ void __launch_bounds__(256) random_normal_kernel(float *out, long n, 
 }
 static unsigned long long g_rng_seed = 1234ull, g_rng_next = 0ull;
 
+// out = rdelta * f'(.) + delta * f''(.) * rz_in: the directional derivative of delta * f'(.)
+__device__ __forceinline__ void act_derivatives(int actFun, float zi, float zo, float &f1, float &f2)
+{
+	switch (actFun) {
+	case ACT_LOGISTIC: f1 = zo * (1.f - zo), f2 = f1 * (1.f - 2.f * zo); break;
+	case ACT_TANH: f1 = (1.f + zo) * (1.f - zo), f2 = -2.f * zo * f1; break;
+	case CNN_ACT_SOFTPLUS: {
+		const float s = sigmoidf(zi);
+		f1 = s, f2 = s * (1.f - s);
+		break;
+	}
+	case CNN_ACT_SWISH: {
+		const float s = sigmoidf(zi);
+		f1 = zo + s * (1.f - zo), f2 = s * (1.f - s) * (2.f + zi * (1.f - 2.f * s));
+		break;
+	}
+	case CNN_ACT_RELU: f1 = zo > 0.f ? 1.f : 0.f, f2 = 0.f; break;
+	case CNN_ACT_ELU: f1 = zo < 0.f ? zo + 1.f : 1.f, f2 = zo < 0.f ? zo + 1.f : 0.f; break;
+	default: f1 = 1.f, f2 = 0.f; break;
+	}
+}
+__global__ void __launch_bounds__(256) activation_rop_backward_kernel(int actFun, const float *rdelta, const float *delta,
+                                                                       const float *z_in, const float *z_out, const float *rz_in,
+                                                                       float *out, long n)
+{
+	const long stride = (long)gridDim.x * blockDim.x;
+	for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+		float f1, f2;
+		act_derivatives(actFun, z_in ? z_in[i] : 0.f, z_out ? z_out[i] : 0.f, f1, f2);
+		out[i] = rdelta[i] * f1 + delta[i] * f2 * rz_in[i];
+	}
+}
+
 // dst[c*ldd + r] = src[c*lds + r] for r < rows, c < cols
 __global__ void __launch_bounds__(256) copy_2d_kernel(const float *src, long lds_, float *dst, long ldd, int rows, int cols)
 {
@@ -395,6 +428,29 @@ int fitre_hip_add_channel_bias(float *x, int channels, long perChannel, const fl
 	add_channel_bias_kernel<<<grid, 256, 0, stream()>>>(x, perChannel, bias);
 	return check_launch("add_channel_bias_kernel");
 }
+int fitre_hip_activation_rop_backward(int actFun, const float *rdelta, const float *delta, const float *z_in,
+                                      const float *z_out, const float *rz_in, float *out, long n)
+{
+	EW_CHECK("fitre_hip_activation_rop_backward", rdelta && delta && rz_in && out && n >= 0);
+	switch (actFun) {
+	case ACT_LOGISTIC: case ACT_TANH: case CNN_ACT_RELU: case CNN_ACT_ELU:
+		FITRE_REQUIRE(z_out, "fitre_hip_activation_rop_backward: activation %d needs z_out", actFun);
+		break;
+	case CNN_ACT_SOFTPLUS:
+		FITRE_REQUIRE(z_in, "fitre_hip_activation_rop_backward: softplus needs z_in");
+		break;
+	case CNN_ACT_SWISH:
+		FITRE_REQUIRE(z_in && z_out, "fitre_hip_activation_rop_backward: swish needs z_in and z_out");
+		break;
+	case ACT_LINEAR: case CNN_ACT_NONE: break;
+	default: return fail(FITRE_E_UNSUPPORTED, "fitre_hip_activation_rop_backward: unknown activation code %d", actFun);
+	}
+	if (n == 0) return FITRE_OK;
+	LaunchScope scope(FITRE_KC_ACT_BWD, 24.0 * (double)n);
+	activation_rop_backward_kernel<<<blocks_for(n, 1024, 8192), 256, 0, stream()>>>(actFun, rdelta, delta, z_in, z_out, rz_in, out, n);
+	return check_launch("activation_rop_backward_kernel");
+}
+
 int fitre_hip_column_softmax(float *x, int rows, int cols)
 {
 	EW_CHECK("fitre_hip_column_softmax", x && rows > 0 && cols > 0);

@@ -90,6 +90,22 @@ __global__ void __launch_bounds__(256) pool_forward_kernel(const float *in, Pool
 	}
 }
 
+// out[pooled cell] = values[argmax of z over the cell's window]: what a max pool passes on of a
+// second tensor that rides along (the directional derivative of its input)
+__global__ void __launch_bounds__(256) pool_routed_kernel(const float *values, const float *z, PoolGeom g, long maps, float *out)
+{
+	long total = maps * g.outA * g.outB;
+	long stride = (long)gridDim.x * blockDim.x;
+	for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+		uint32_t q, ob, oa, map;
+		g.divOutB.divmod((uint32_t)i, q, ob);
+		g.divOutA.divmod(q, map, oa);
+		float best;
+		int arg = window_argmax(z + (size_t)map * g.inA * g.inB, g, (int)oa, (int)ob, best);
+		out[i] = (arg < 0) ? 0.f : values[(size_t)map * g.inA * g.inB + arg];
+	}
+}
+
 // Gradient reaching input cell (a, b) of one map: sum over the windows that
 // contain the cell.  No atomics: every input cell is owned by one thread.
 template <int POOL> // 0 max, 1 average
@@ -510,6 +526,57 @@ bn_backward_small_kernel(const float *delta, const float *zhat, const float *var
 	}
 }
 
+// Directional derivative of the batch-norm backward formula.  Per channel, with s = sqrt(var + eps)
+// and <.> the mean over the channel:
+//   out = ( rdx - <rdx> - rzhat <dx zhat> - zhat ( <rdx zhat> + <dx rzhat> ) ) / s  -  dc <zhat rx> / s
+// Pass 1: five sums per (channel, segment), slots of eight doubles.
+__global__ void __launch_bounds__(kRedBlock)
+bn_rop_partial_kernel(const float *rdx, const float *dx, const float *zhat, const float *rzhat, const float *rx, long perChannel,
+                      double *partial)
+{
+	__shared__ double lds[kRedBlock / kWave];
+	const size_t base = (size_t)blockIdx.y * perChannel;
+	long lo, hi;
+	segment_range(perChannel, lo, hi);
+	double s[5] = { 0.0, 0.0, 0.0, 0.0, 0.0 };
+	for (long i = lo + threadIdx.x; i < hi; i += kRedBlock) {
+		const float a = rdx[base + i], d = dx[base + i], z = zhat[base + i], rz = rzhat[base + i], x = rx[base + i];
+		s[0] += (double)a;
+		s[1] += (double)(d * z);
+		s[2] += (double)(a * z);
+		s[3] += (double)(d * rz);
+		s[4] += (double)(z * x);
+	}
+	double t[5];
+#pragma unroll
+	for (int k = 0; k < 5; k++) t[k] = block_sum<kRedBlock>(s[k], lds);
+	if (threadIdx.x == 0) {
+		double *slot = partial + ((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 8;
+#pragma unroll
+		for (int k = 0; k < 5; k++) slot[k] = t[k];
+	}
+}
+__global__ void __launch_bounds__(kRedBlock)
+bn_rop_apply_kernel(const float *rdx, const float *zhat, const float *rzhat, const float *dc, const float *variance,
+                    const double *partial, int segments, float epsilon, long perChannel, float *out)
+{
+	const int c = blockIdx.y;
+	double t[5] = { 0.0, 0.0, 0.0, 0.0, 0.0 };
+	for (int k = 0; k < segments; k++) {
+		const double *slot = partial + ((size_t)c * segments + k) * 8;
+#pragma unroll
+		for (int j = 0; j < 5; j++) t[j] += slot[j];
+	}
+	const double m = (double)perChannel;
+	const float inv = 1.f / sqrtf(variance[c] + epsilon);
+	const float a = (float)(t[0] / m), b = (float)(t[1] / m), cd = (float)((t[2] + t[3]) / m), e = (float)(t[4] / m);
+	const size_t base = (size_t)c * perChannel;
+	long lo, hi;
+	segment_range(perChannel, lo, hi);
+	for (long i = lo + threadIdx.x; i < hi; i += kRedBlock)
+		out[base + i] = (rdx[base + i] - a - rzhat[base + i] * b - zhat[base + i] * cd) * inv - dc[base + i] * e * inv;
+}
+
 static inline bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
 // =====================================================================
@@ -577,6 +644,19 @@ __global__ void __launch_bounds__(256) accuracy_hits_kernel(const float *probs, 
 		}
 	}
 	hits[r] = ((float)(arg + 1) == target[r]) ? 1.f : 0.f;
+}
+
+// rError[r][i] = p_i (rz_i - sum_j p_j rz_j) / rows
+__global__ void __launch_bounds__(256) cross_entropy_rop_error_kernel(const float *rz, const float *probs, int rows, int classes,
+                                                                       float *rError)
+{
+	const int r = blockIdx.x * blockDim.x + threadIdx.x;
+	if (r >= rows) return;
+	const float *p = probs + (size_t)r * classes, *z = rz + (size_t)r * classes;
+	float s = 0.f;
+	for (int j = 0; j < classes; j++) s += p[j] * z[j];
+	const float inv = 1.f / (float)rows;
+	for (int i = 0; i < classes; i++) rError[(size_t)r * classes + i] = p[i] * (z[i] - s) * inv;
 }
 
 __global__ void cross_entropy_error_kernel(const float *probs, const float *target, int rows, int classes, float *errors)
@@ -759,7 +839,7 @@ int fitre_hip_pool_backward(int poolType, const float *delta, const float *z_in,
 size_t fitre_hip_batch_norm_workspace(int channels, long perChannel)
 {
 	if (channels <= 0 || perChannel <= 0) return 0;
-	return (size_t)channels * segments_for(channels, perChannel) * 2 * sizeof(double) * 2 + 64;
+	return (size_t)channels * segments_for(channels, perChannel) * 8 * sizeof(double) + 64; // slots of up to eight sums
 }
 
 size_t fitre_hip_channel_sum_workspace(int channels, long perChannel)
@@ -883,6 +963,54 @@ int fitre_hip_softmax_cross_entropy(const float *logits, const float *target, in
 	FITRE_HIP_TRY(hipStreamSynchronize(stream()));
 	*lossHost = *g_loss_host;
 	return FITRE_OK;
+}
+
+int fitre_hip_cross_entropy_rop_error(const float *rz, const float *probs, int rows, int classes, float *rError)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(rz && probs && rError, "fitre_hip_cross_entropy_rop_error: null pointer");
+	FITRE_REQUIRE(rows > 0 && classes > 0, "fitre_hip_cross_entropy_rop_error: non-positive shape %d x %d", rows, classes);
+	LaunchScope scope(FITRE_KC_SOFTMAX, 12.0 * (double)rows * classes);
+	cross_entropy_rop_error_kernel<<<blocks_for(rows, 256), 256, 0, stream()>>>(rz, probs, rows, classes, rError);
+	return check_launch("cross_entropy_rop_error_kernel");
+}
+
+int fitre_hip_batch_norm_rop_backward(const float *rdelta_x, const float *delta_x, const float *zhat, const float *rzhat,
+                                      const float *rx, const float *delta_c, const float *variance, int channels,
+                                      long perChannel, float epsilon, float *out, void *ws, size_t wsBytes)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(rdelta_x && delta_x && zhat && rzhat && rx && delta_c && variance && out,
+	              "fitre_hip_batch_norm_rop_backward: null pointer");
+	int rc = check_channels("fitre_hip_batch_norm_rop_backward", channels, perChannel, ws, wsBytes);
+	if (rc) return rc;
+	const int S = segments_for(channels, perChannel);
+	if (wsBytes < (size_t)channels * S * 8 * sizeof(double))
+		return fail(FITRE_E_WORKSPACE, "fitre_hip_batch_norm_rop_backward: workspace of %zu bytes is smaller than the %zu required",
+		            wsBytes, (size_t)channels * S * 8 * sizeof(double));
+	double *partial = (double *)ws;
+	LaunchScope scope(FITRE_KC_BN_BWD, 28.0 * (double)channels * (double)perChannel);
+	dim3 grid(S, channels);
+	bn_rop_partial_kernel<<<grid, kRedBlock, 0, stream()>>>(rdelta_x, delta_x, zhat, rzhat, rx, perChannel, partial);
+	bn_rop_apply_kernel<<<grid, kRedBlock, 0, stream()>>>(rdelta_x, zhat, rzhat, delta_c, variance, partial, S, epsilon, perChannel, out);
+	return check_launch("batch_norm_rop_backward");
+}
+
+int fitre_hip_pool_forward_routed(int poolType, const float *values, const float *z_act, int channels, int samples, int inA,
+                                  int inB, int ksize, int stride, int padding, int outA, int outB, float *out)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(values && out, "fitre_hip_pool_forward_routed: null pointer");
+	if (poolType == AVG_POOL) return fitre_hip_pool_forward(AVG_POOL, values, channels, samples, inA, inB, ksize, stride, padding, outA, outB, out);
+	if (poolType != MAX_POOL) return fail(FITRE_E_UNSUPPORTED, "fitre_hip_pool_forward_routed: unknown pool type %d", poolType);
+	FITRE_REQUIRE(z_act, "fitre_hip_pool_forward_routed: z_act is required for max pooling");
+	int rc = check_pool_shape("fitre_hip_pool_forward_routed", channels, samples, inA, inB, ksize, stride, padding, outA, outB);
+	if (rc) return rc;
+	PoolGeom g = make_geom(inA, inB, ksize, stride, padding, outA, outB);
+	const long maps = (long)channels * samples;
+	LaunchScope scope(FITRE_KC_POOL_FWD, 4.0 * (double)maps * ((double)inA * inB + 2.0 * outA * outB));
+	pool_routed_kernel<<<blocks_for(maps * outA * outB, 256, 16384), 256, 0, stream()>>>(values, z_act, g, maps, out);
+	return check_launch("pool_routed_kernel");
 }
 
 int fitre_hip_multinomial_classes(const float *probs, const float *uniforms, int samples, int classes, float *out)

@@ -97,6 +97,10 @@ HIP_API = {
     "fitre_hip_lane_select": (i32, [i32]),
     "fitre_hip_lane_wait": (i32, [i32, i32]),
     "fitre_hip_lanes_enable": (i32, [i32]),
+    "fitre_hip_activation_rop_backward": (i32, [i32, vp, vp, vp, vp, vp, vp, lng]),
+    "fitre_hip_pool_forward_routed": (i32, [i32, vp, vp] + [i32] * 9 + [vp]),
+    "fitre_hip_batch_norm_rop_backward": (i32, [vp, vp, vp, vp, vp, vp, vp, i32, lng, f32, vp, vp, sz]),
+    "fitre_hip_cross_entropy_rop_error": (i32, [vp, vp, i32, i32, vp]),
     "fitre_hip_spd_inverse_workspace": (sz, [i32]),
     "fitre_hip_spd_inverse": (i32, [vp, i32, f32, vp, vp, sz, pi32]),
     "fitre_hip_kfac_conv_input_factor_workspace": (sz, [vp, i32]),
@@ -146,6 +150,10 @@ CNN_API = {
     "computeLambdaDelta": (None, [pkfac, pmodel, i32, vp, vp, vp, pi32, pi32, vp, vp]),
     "kfacNaturalGradientMemRequired": (lng, [pmodel]),
     "computeNaturalGradient": (None, [pmodel, pkfac, vp, vp]),
+    # include/fitre_hv.h
+    "cnnHvMemRequired": (lng, [pmodel]),
+    "cnnHv": (None, [pmodel, pdata, vp, vp, vp, vp, vp, vp, i32, i32, vp, vp, f32]),
+    "computeQuadraticModel": (f32, [pmodel, pdata, vp, vp, vp, vp, vp, vp, f32, i32, i32, f32, vp, vp, pf32]),
     # include/fitre_fc.h
     "fitre_build_nn": (None, [pnn, pi32, pi32, i32, i32, i32]),
     "initSampledZOffsets": (None, [pnn, i32]),

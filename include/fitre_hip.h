@@ -294,6 +294,28 @@ int fitre_hip_kfac_fc_input_factor(const float *z, int in, int samples, int with
 int fitre_hip_kfac_fc_output_factor(const float *delta, int out, int samples, float *factor, void *ws,
                                     size_t wsBytes);
 
+/* ---- R-operator (Hessian-vector product) pieces --------------------------------------------------
+ * out = rdelta * f'(.) + delta * f''(.) * rz_in, the directional derivative of delta * f'(.) when
+ * delta moves by rdelta and the activation's input by rz_in (second derivatives of
+ * functions/swish.cu:45-56, dev_activations.cu; z_in / z_out as in fitre_hip_activation_backward). */
+int fitre_hip_activation_rop_backward(int actFun, const float *rdelta, const float *delta, const float *z_in,
+                                      const float *z_out, const float *rz_in, float *out, long n);
+/* Max pool: out = values at the arg-max positions of z_act (ker_rop_max_pool_layer, functions/dev_pool.cu:123-174);
+ * average pool: the average of values (z_act unused). */
+int fitre_hip_pool_forward_routed(int poolType, const float *values, const float *z_act, int channels, int samples,
+                                  int inA, int inB, int ksize, int stride, int padding, int outA, int outB, float *out);
+/* Directional derivative of batch-norm backward (computeROpBatchNormBackward, functions/dev_batch_norm.cu:787-960):
+ * with s = sqrt(var + eps) and <.> the per-channel mean,
+ *   out = (rdelta_x - <rdelta_x> - rzhat <delta_x zhat> - zhat (<rdelta_x zhat> + <delta_x rzhat>)) / s - delta_c <zhat rx> / s
+ * delta_x / delta_c: gradient at the batch-norm output / input, rx / rzhat: R{.} of its input / output.
+ * The directional derivative of batch-norm FORWARD is fitre_hip_batch_norm_backward applied to rx.
+ * Workspace: fitre_hip_batch_norm_workspace(channels, perChannel). */
+int fitre_hip_batch_norm_rop_backward(const float *rdelta_x, const float *delta_x, const float *zhat, const float *rzhat,
+                                      const float *rx, const float *delta_c, const float *variance, int channels,
+                                      long perChannel, float epsilon, float *out, void *ws, size_t wsBytes);
+/* rError = p_i (rz_i - sum_j p_j rz_j) / rows (computeROpCrossEntropyError_simple, functions/softmax_loss.cu:251-300) */
+int fitre_hip_cross_entropy_rop_error(const float *rz, const float *probs, int rows, int classes, float *rError);
+
 /* inverse = (matrix + shift*I)^-1 for a symmetric positive definite matrix of order n (column-major ==
  * row-major, full storage in and out): blocked Cholesky, inverse of the factor, symmetric product.
  * Replaces computeMatrixInverseCusolver (solvers/kfac_inverses.cu:133-186: identity right-hand side,

@@ -69,3 +69,115 @@ def test_oracle_hv_symmetry_and_taylor(oracle64, name):
             ft = oracle64.gradient(model, w + t * d, x, y, k, batch)["loss"]
             rem.append(abs(ft - f0 - t * (g @ d) - 0.5 * t * t * (d @ hd)))
         assert rem[0] / rem[1] > 6 and rem[1] / rem[2] > 6, rem   # 8 for an exact Hessian, 4 for a wrong one
+
+
+# ------------------------------------------------------------------------------------------ GPU
+from fitre_amd import lib as L  # noqa: E402
+
+TOL = 1e-4
+
+
+def gpu_hv(dev, gm, model, batch, v32):
+    pv = dev.upload(v32)
+    hv = dev.upload(np.full(model.pSize, np.nan, dtype=np.float32))
+    ws = dev.alloc(4 * L.cnn.cnnHvMemRequired(C.byref(model)) + 512)
+    L.cnn.cnnHv(C.byref(model), C.byref(gm.data), gm.z, gm.probs, gm.errors, gm.dx, pv, hv, 0, batch, ws, None, 0.0)
+    out = dev.download(hv, model.pSize)
+    for q in (pv, hv, ws):
+        dev.free(q)
+    return out
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", list(MODELS))
+def test_gpu_hv_against_oracle_on_the_same_inputs(dev, oracle64, name):
+    """cnnHv against the oracle's R passes run on the z / probs / errors / dx the device produced (the ReLU masks
+    and pooling selections are functions of z; see the gradient tests)."""
+    from helpers import GpuModel
+    rng = np.random.default_rng(sum(map(ord, name)) + 3)
+    model, batch, w, x, y, v = setup(name, rng)
+    w32, x32, v32 = w.astype(np.float32), x.astype(np.float32), v.astype(np.float32)
+    gm = GpuModel(dev, model, w32, x32, y, batch)
+    gm.gradient()
+    got = gpu_hv(dev, gm, model, batch, v32)
+    k = classes_of(model)
+    want = oracle64.hessian_vector(model, w32, x32, gm.get("z"), gm.get("probs"), gm.get("errors"), gm.get("dx"), v32, k, batch)
+    assert np.isfinite(got).all()
+    assert rel_err(got, want) < TOL
+    # and end to end against double backward (small smooth-enough models: a looser bound)
+    assert rel_err(got, torchref.hessian_vector(model, w32, x32, y, batch, v32)) < 5e-4
+    gm.release()
+
+
+@pytest.mark.gpu
+def test_gpu_quadratic_model_step(dev, oracle64):
+    from helpers import GpuModel
+    name = "swish_maxpool_fc"
+    rng = np.random.default_rng(11)
+    model, batch, w, x, y, v = setup(name, rng)
+    w32, x32, v32 = w.astype(np.float32), x.astype(np.float32), v.astype(np.float32)
+    gm = GpuModel(dev, model, w32, x32, y, batch)
+    gm.gradient()
+    g = gm.get("grad")
+    hv = gpu_hv(dev, gm, model, batch, v32).astype(np.float64)
+    decay = 1e-3
+    hv_d = hv + decay * w32                      # the reference adds weightDecay * weights
+    vhv, gv, nrm = hv_d @ v32, g.astype(np.float64) @ v32, np.linalg.norm(v32.astype(np.float64))
+    for delta in (1e-3, 1e3):
+        pv = dev.upload(v32)
+        ws = dev.alloc(4 * (L.cnn.cnnHvMemRequired(C.byref(model)) + model.pSize) + 512)
+        host = (C.c_float * 3)()
+        m = L.cnn.computeQuadraticModel(C.byref(model), C.byref(gm.data), gm.z, gm.probs, gm.errors, gm.dx, gm.grad, pv,
+                                        delta, 0, batch, decay, ws, None, host)
+        if vhv < 0:
+            step = delta / nrm
+        else:
+            step = min(gv / (vhv + 1e-6), delta / (nrm + 1e-16))
+        want = 0.5 * vhv * step * step - gv * step
+        assert abs(host[1] - vhv) < 1e-3 * max(1, abs(vhv)) and abs(host[0] - gv) < 1e-3 * max(1, abs(gv))
+        assert abs(m - want) < 1e-3 * max(1e-6, abs(want))
+        assert rel_err(dev.download(pv, model.pSize), step * v32) < 1e-3
+        dev.free(pv)
+        dev.free(ws)
+    gm.release()
+
+
+@pytest.mark.gpu
+def test_gpu_hv_full_size_vgg_symmetry_and_finite_difference(dev):
+    """A network of VGG-11's shape (eight 3x3 convolutions 64..512 with batch norm and swish, FC 512->10), batch 64,
+    with average instead of max pooling so that the loss is smooth: u'Hv = v'Hu, and Hv against the central
+    difference of the gradient along v (across a max-pool arg-max flip the gradient jumps, which a difference
+    quotient sees and a Hessian does not)."""
+    from helpers import GpuModel
+    batch = 64
+    widths, pooled = [64, 128, 256, 256, 512, 512, 512, 512], {0, 1, 3, 5, 7}
+    convs = [dict(cout=c, k=3, pad=1, pool=(AVG_POOL, 2, 2, 0) if i in pooled else None, bn=True, act=CNN_ACT_SWISH)
+             for i, c in enumerate(widths)]
+    model = build_custom(batch, 32, 32, 3, convs, [(10, CNN_ACT_NONE)])
+    rng = np.random.default_rng(2024)
+    w = he_weights(model, rng).astype(np.float32)
+    x, y = batch_inputs(model, batch, rng)
+    x = x.astype(np.float32)
+    u = rng.standard_normal(model.pSize).astype(np.float32)
+    # a direction that perturbs every weight by a fraction of its own size, so that a float32 gradient
+    # difference stays far above the rounding noise of the gradients
+    v = (w * rng.standard_normal(model.pSize)).astype(np.float32)
+    gm = GpuModel(dev, model, w, x, y, batch)
+    gm.gradient()
+    hv, hu = gpu_hv(dev, gm, model, batch, v), gpu_hv(dev, gm, model, batch, u)
+    assert np.isfinite(hv).all() and np.isfinite(hu).all()
+    a, b = float(u.astype(np.float64) @ hv), float(v.astype(np.float64) @ hu)
+    assert abs(a - b) < 2e-3 * max(abs(a), abs(b)), (a, b)
+    # central difference of the gradient, projected on a few random directions to average the float32 noise
+    eps = 5e-3
+    grads = []
+    for sign in (1.0, -1.0):
+        gm2 = GpuModel(dev, model, (w + sign * eps * v).astype(np.float32), x, y, batch)
+        gm2.gradient()
+        grads.append(gm2.get("grad").astype(np.float64))
+        gm2.release()
+    fd = (grads[0] - grads[1]) / (2 * eps)
+    for r in (u, v):
+        p, q = float(r.astype(np.float64) @ fd), float(r.astype(np.float64) @ hv)
+        assert abs(p - q) < 5e-2 * max(abs(p), abs(q)), (p, q)
+    gm.release()
