@@ -43,7 +43,7 @@ struct BlockPlan {
 
 // Splits a reduction of nBlocks equal blocks (blockUs microseconds of matrix-pipe time each) over
 // workgroups so that the compute units are evenly loaded; same cost model as plan_gemm.
-static BlockPlan plan_blocks(long tiles, long nBlocks, double blockUs, int residentPerCu, long I, long J)
+static BlockPlan plan_blocks_search(long tiles, long nBlocks, double blockUs, int residentPerCu, long I, long J)
 {
 	BlockPlan best{ 1, (int)nBlocks, 0 };
 	double bestT = 1e30;
@@ -63,6 +63,30 @@ static BlockPlan plan_blocks(long tiles, long nBlocks, double blockUs, int resid
 		}
 	}
 	return best;
+}
+
+// memo of the search (a layer asks for the same plan on every call)
+static BlockPlan plan_blocks(long tiles, long nBlocks, double blockUs, int residentPerCu, long I, long J)
+{
+	struct Entry {
+		long tiles, nBlocks, I, J;
+		double blockUs;
+		int resident;
+		BlockPlan plan;
+	};
+	constexpr int kEntries = 64;
+	static Entry table[kEntries];
+	static int used = 0, next = 0;
+	for (int i = 0; i < used; i++) {
+		const Entry &e = table[i];
+		if (e.tiles == tiles && e.nBlocks == nBlocks && e.I == I && e.J == J && e.blockUs == blockUs && e.resident == residentPerCu)
+			return e.plan;
+	}
+	Entry e{ tiles, nBlocks, I, J, blockUs, residentPerCu, plan_blocks_search(tiles, nBlocks, blockUs, residentPerCu, I, J) };
+	table[next] = e;
+	next = (next + 1) % kEntries;
+	if (used < kEntries) used++;
+	return e.plan;
 }
 
 static BlockPlan fit_blocks(BlockPlan p, long nBlocks, long I, long J, const void *ws, size_t wsBytes)

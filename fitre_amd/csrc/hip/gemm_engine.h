@@ -643,7 +643,7 @@ inline double estimate_us(long tiles, int bm, int bn, long I, long J, long R, lo
 }
 
 // mirror: a symmetric product (I == J) that only computes the tiles on and above the diagonal
-inline GemmPlan plan_gemm(long I, long J, long R, bool mirror = false)
+inline GemmPlan plan_gemm_search(long I, long J, long R, bool mirror)
 {
 	GemmPlan p;
 	p.bm = (I <= 64) ? 64 : 128;
@@ -671,6 +671,27 @@ inline GemmPlan plan_gemm(long I, long J, long R, bool mirror = false)
 	p.kChunk = (int)bestChunk;
 	p.wsBytes = (bestSplits > 1) ? (size_t)bestSplits * I * J * sizeof(float) : 0;
 	return p;
+}
+
+// The search above walks up to 1024 split counts; a layer asks for the same plan on every call
+// (and once more per workspace query), so the results are kept in a small table.
+inline GemmPlan plan_gemm(long I, long J, long R, bool mirror = false)
+{
+	struct Entry {
+		long I, J, R;
+		bool mirror;
+		GemmPlan plan;
+	};
+	constexpr int kEntries = 128;
+	static Entry table[kEntries];
+	static int used = 0, next = 0;
+	for (int i = 0; i < used; i++)
+		if (table[i].I == I && table[i].J == J && table[i].R == R && table[i].mirror == mirror) return table[i].plan;
+	Entry e{ I, J, R, mirror, plan_gemm_search(I, J, R, mirror) };
+	table[next] = e;
+	next = (next + 1) % kEntries;
+	if (used < kEntries) used++;
+	return e.plan;
 }
 
 // Shrinks the number of splits until the partial tiles fit the workspace the
