@@ -23,6 +23,9 @@ int gemm_ex(int transA, int transB, int M, int N, int K, float alpha, const floa
             float beta, float *C, int ldc, const float *bias, int flags, int kernelClass, void *ws, size_t wsBytes);
 size_t gemm_ex_workspace(int M, int N, int K, int flags);
 int lane();           // its index (0 or 1)
+int lane_compute_units();     // compute units a kernel launched on the selected lane can occupy
+int lane_compute_units_min(); // the smallest such count over the lanes
+int device_compute_units();
 bool ready();
 
 #define FITRE_HIP_TRY(expr)                                                                          \

@@ -43,7 +43,7 @@ struct BlockPlan {
 
 // Splits a reduction of nBlocks equal blocks (blockUs microseconds of matrix-pipe time each) over
 // workgroups so that the compute units are evenly loaded; same cost model as plan_gemm.
-static BlockPlan plan_blocks_search(long tiles, long nBlocks, double blockUs, int residentPerCu, long I, long J)
+static BlockPlan plan_blocks_search(long tiles, long nBlocks, double blockUs, int residentPerCu, long I, long J, long cus)
 {
 	BlockPlan best{ 1, (int)nBlocks, 0 };
 	double bestT = 1e30;
@@ -51,7 +51,7 @@ static BlockPlan plan_blocks_search(long tiles, long nBlocks, double blockUs, in
 		long per = (nBlocks + s - 1) / s;
 		long eff = (nBlocks + per - 1) / per;
 		long groups = tiles * eff;
-		long perCu = (groups + kComputeUnits - 1) / kComputeUnits;
+		long perCu = (groups + cus - 1) / cus;
 		double e = perCu >= residentPerCu ? 0.85 : (perCu * 2 >= residentPerCu + 1 ? 0.72 : 0.55);
 		double t = (double)perCu * (double)per * blockUs / e + 3.0;
 		if (eff > 1) t += 4.0 + (double)(eff + 1) * (double)I * (double)J * 4.0 / 3.0e6;
@@ -66,12 +66,12 @@ static BlockPlan plan_blocks_search(long tiles, long nBlocks, double blockUs, in
 }
 
 // memo of the search (a layer asks for the same plan on every call)
-static BlockPlan plan_blocks(long tiles, long nBlocks, double blockUs, int residentPerCu, long I, long J)
+static BlockPlan plan_blocks(long tiles, long nBlocks, double blockUs, int residentPerCu, long I, long J, int cus)
 {
 	struct Entry {
 		long tiles, nBlocks, I, J;
 		double blockUs;
-		int resident;
+		int resident, cus;
 		BlockPlan plan;
 	};
 	constexpr int kEntries = 64;
@@ -79,10 +79,12 @@ static BlockPlan plan_blocks(long tiles, long nBlocks, double blockUs, int resid
 	static int used = 0, next = 0;
 	for (int i = 0; i < used; i++) {
 		const Entry &e = table[i];
-		if (e.tiles == tiles && e.nBlocks == nBlocks && e.I == I && e.J == J && e.blockUs == blockUs && e.resident == residentPerCu)
+		if (e.tiles == tiles && e.nBlocks == nBlocks && e.I == I && e.J == J && e.blockUs == blockUs && e.resident == residentPerCu &&
+		    e.cus == cus)
 			return e.plan;
 	}
-	Entry e{ tiles, nBlocks, I, J, blockUs, residentPerCu, plan_blocks_search(tiles, nBlocks, blockUs, residentPerCu, I, J) };
+	Entry e{ tiles,         nBlocks, I, J, blockUs, residentPerCu,
+		     cus,           plan_blocks_search(tiles, nBlocks, blockUs, residentPerCu, I, J, cus) };
 	table[next] = e;
 	next = (next + 1) % kEntries;
 	if (used < kEntries) used++;
@@ -118,21 +120,34 @@ static bool c3_dw_eligible(const fitre_conv_shape *s)
 	       ((long)s->samples * s->inA * s->inB) % kC3Stage == 0;
 }
 
-static BlockPlan c3_pos_plan(const fitre_conv_shape *s, bool dx)
+// cus: compute units of the lane the kernel is launched on (0 = the selected lane)
+static BlockPlan c3_pos_plan(const fitre_conv_shape *s, bool dx, int cus = 0)
 {
+	if (cus <= 0) cus = lane_compute_units();
 	long I = dx ? s->inChannels : s->outChannels, J = (long)s->samples * s->inA * s->inB;
 	long cred = dx ? s->outChannels : s->inChannels;
 	long it = I <= 64 ? 64 : kC3Tile;
 	long tiles = ((I + it - 1) / it) * ((J + kC3Tile - 1) / kC3Tile);
 	double blockUs = (9.0 * kC3CB / 2.0) * (it / 32.0) * 64.0 / 2400.0; // MFMA steps x blocks per wave x 64 cycles
-	return plan_blocks(tiles, cred / kC3CB, blockUs, it == 64 ? 3 : 2, I, J);
+	return plan_blocks(tiles, cred / kC3CB, blockUs, it == 64 ? 3 : 2, I, J, cus);
 }
-static BlockPlan c3_dw_plan(const fitre_conv_shape *s)
+static BlockPlan c3_dw_plan(const fitre_conv_shape *s, int cus = 0)
 {
+	if (cus <= 0) cus = lane_compute_units();
 	long J = (long)s->samples * s->inA * s->inB;
 	long tiles = ((s->inChannels + kC3DwCin - 1) / kC3DwCin) * ((s->outChannels + kC3Tile - 1) / kC3Tile);
 	double stageUs = (kC3Stage / 2.0) * 9.0 * 64.0 / 2400.0; // three waves per SIMD, three MFMAs per step each
-	return plan_blocks(tiles, (J + kC3Stage - 1) / kC3Stage, stageUs, 1, s->outChannels, (long)s->inChannels * 9);
+	return plan_blocks(tiles, (J + kC3Stage - 1) / kC3Stage, stageUs, 1, s->outChannels, (long)s->inChannels * 9, cus);
+}
+static size_t c3_pos_workspace(const fitre_conv_shape *s, bool dx)
+{
+	size_t a = c3_pos_plan(s, dx, device_compute_units()).wsBytes, b = c3_pos_plan(s, dx, lane_compute_units_min()).wsBytes;
+	return a > b ? a : b;
+}
+static size_t c3_dw_workspace(const fitre_conv_shape *s)
+{
+	size_t a = c3_dw_plan(s, device_compute_units()).wsBytes, b = c3_dw_plan(s, lane_compute_units_min()).wsBytes;
+	return a > b ? a : b;
 }
 
 template <bool DX>
@@ -236,7 +251,7 @@ static int launch_c3_dw(const fitre_conv_shape *s, const float *x, const float *
 size_t gemm_ex_workspace(int M, int N, int K, int flags)
 {
 	if (M <= 0 || N <= 0 || K <= 0) return 0;
-	return plan_gemm(N, M, K, (flags & kGemmMirror) != 0).wsBytes;
+	return plan_gemm_workspace(N, M, K, (flags & kGemmMirror) != 0);
 }
 
 int gemm_ex(int transA, int transB, int M, int N, int K, float alpha, const float *A, int lda, const float *B, int ldb,
@@ -276,8 +291,8 @@ extern "C" {
 size_t fitre_hip_conv_forward_workspace(const fitre_conv_shape *s)
 {
 	if (!s) return 0;
-	if (c3_pos_eligible(s, false)) return c3_pos_plan(s, false).wsBytes;
-	return plan_gemm(s->outChannels, (long)s->samples * s->outA * s->outB, (long)s->inChannels * s->ksize * s->ksize).wsBytes;
+	if (c3_pos_eligible(s, false)) return c3_pos_workspace(s, false);
+	return plan_gemm_workspace(s->outChannels, (long)s->samples * s->outA * s->outB, (long)s->inChannels * s->ksize * s->ksize);
 }
 
 int fitre_hip_conv_forward(const fitre_conv_shape *s, const float *x, const float *w, const float *bias, float *y, void *ws,
@@ -302,8 +317,8 @@ int fitre_hip_conv_forward(const fitre_conv_shape *s, const float *x, const floa
 size_t fitre_hip_conv_weight_grad_workspace(const fitre_conv_shape *s)
 {
 	if (!s) return 0;
-	if (c3_dw_eligible(s)) return c3_dw_plan(s).wsBytes;
-	return plan_gemm(s->outChannels, (long)s->inChannels * s->ksize * s->ksize, (long)s->samples * s->outA * s->outB).wsBytes;
+	if (c3_dw_eligible(s)) return c3_dw_workspace(s);
+	return plan_gemm_workspace(s->outChannels, (long)s->inChannels * s->ksize * s->ksize, (long)s->samples * s->outA * s->outB);
 }
 
 int fitre_hip_conv_weight_grad(const fitre_conv_shape *s, const float *x, const float *delta, float *dW, void *ws, size_t wsBytes)
@@ -325,8 +340,8 @@ int fitre_hip_conv_weight_grad(const fitre_conv_shape *s, const float *x, const 
 size_t fitre_hip_conv_input_grad_workspace(const fitre_conv_shape *s)
 {
 	if (!s) return 0;
-	if (c3_pos_eligible(s, true)) return c3_pos_plan(s, true).wsBytes;
-	return plan_gemm(s->inChannels, (long)s->samples * s->inA * s->inB, (long)s->outChannels * s->ksize * s->ksize).wsBytes;
+	if (c3_pos_eligible(s, true)) return c3_pos_workspace(s, true);
+	return plan_gemm_workspace(s->inChannels, (long)s->samples * s->inA * s->inB, (long)s->outChannels * s->ksize * s->ksize);
 }
 
 int fitre_hip_conv_input_grad(const fitre_conv_shape *s, const float *delta, const float *w, float *dx, void *ws, size_t wsBytes)

@@ -619,19 +619,19 @@ struct GemmPlan {
 };
 
 constexpr int kGemmBK = 16;
-constexpr int kComputeUnits = 256; // MI355X
 
 // Estimated duration (microseconds) of a product cut into `splits` reduction ranges.
 // Workgroups are spread evenly over the compute units; a compute unit runs up to three of
 // them at once, and the more it holds the better the matrix pipes stay fed.  A split
 // product pays for writing and re-reading its partial tiles.
-inline double estimate_us(long tiles, int bm, int bn, long I, long J, long R, long splits, long *chunkOut, long *splitsOut)
+inline double estimate_us(long tiles, int bm, int bn, long I, long J, long R, long splits, long cus, long *chunkOut,
+                          long *splitsOut)
 {
 	long chunk = (R + splits - 1) / splits;
 	chunk = ((chunk + kGemmBK - 1) / kGemmBK) * kGemmBK;
 	long s = (R + chunk - 1) / chunk;
 	long groups = tiles * s;
-	long perCu = (groups + kComputeUnits - 1) / kComputeUnits;
+	long perCu = (groups + cus - 1) / cus;
 	// one k-step of a bm x bn tile keeps the four matrix pipes of a compute unit busy for this long
 	double stepUs = (double)(bm / 32) * (bn / 32) * (kGemmBK / 2) * 64.0 / 4.0 / 2400.0;
 	double eff = perCu >= 3 ? 0.80 : (perCu == 2 ? 0.68 : 0.52);
@@ -643,7 +643,7 @@ inline double estimate_us(long tiles, int bm, int bn, long I, long J, long R, lo
 }
 
 // mirror: a symmetric product (I == J) that only computes the tiles on and above the diagonal
-inline GemmPlan plan_gemm_search(long I, long J, long R, bool mirror)
+inline GemmPlan plan_gemm_search(long I, long J, long R, bool mirror, long cus)
 {
 	GemmPlan p;
 	p.bm = (I <= 64) ? 64 : 128;
@@ -660,7 +660,7 @@ inline GemmPlan plan_gemm_search(long I, long J, long R, bool mirror)
 	long bestChunk = ((R + kGemmBK - 1) / kGemmBK) * kGemmBK, bestSplits = 1;
 	for (long s = 1; s <= maxSplits; s++) {
 		long chunk, eff;
-		double t = estimate_us(tiles, p.bm, p.bn, I, J, R, s, &chunk, &eff);
+		double t = estimate_us(tiles, p.bm, p.bn, I, J, R, s, cus, &chunk, &eff);
 		if (t < best) {
 			best = t;
 			bestChunk = chunk;
@@ -674,24 +674,36 @@ inline GemmPlan plan_gemm_search(long I, long J, long R, bool mirror)
 }
 
 // The search above walks up to 1024 split counts; a layer asks for the same plan on every call
-// (and once more per workspace query), so the results are kept in a small table.
-inline GemmPlan plan_gemm(long I, long J, long R, bool mirror = false)
+// (and once more per workspace query), so the results are kept in a small table.  The plan is
+// made for the compute units of the lane the product will be launched on.
+inline GemmPlan plan_gemm(long I, long J, long R, bool mirror = false, int cus = 0)
 {
 	struct Entry {
 		long I, J, R;
 		bool mirror;
+		int cus;
 		GemmPlan plan;
 	};
+	if (cus <= 0) cus = lane_compute_units();
 	constexpr int kEntries = 128;
 	static Entry table[kEntries];
 	static int used = 0, next = 0;
 	for (int i = 0; i < used; i++)
-		if (table[i].I == I && table[i].J == J && table[i].R == R && table[i].mirror == mirror) return table[i].plan;
-	Entry e{ I, J, R, mirror, plan_gemm_search(I, J, R, mirror) };
+		if (table[i].I == I && table[i].J == J && table[i].R == R && table[i].mirror == mirror && table[i].cus == cus)
+			return table[i].plan;
+	Entry e{ I, J, R, mirror, cus, plan_gemm_search(I, J, R, mirror, cus) };
 	table[next] = e;
 	next = (next + 1) % kEntries;
 	if (used < kEntries) used++;
 	return e.plan;
+}
+
+// Workspace that covers the plan of every lane (a size query does not know the lane of the launch).
+inline size_t plan_gemm_workspace(long I, long J, long R, bool mirror = false)
+{
+	size_t a = plan_gemm(I, J, R, mirror, device_compute_units()).wsBytes;
+	size_t b = plan_gemm(I, J, R, mirror, lane_compute_units_min()).wsBytes;
+	return a > b ? a : b;
 }
 
 // Shrinks the number of splits until the partial tiles fit the workspace the

@@ -37,7 +37,7 @@ size_t fitre_hip_kfac_conv_input_factor_workspace(const fitre_conv_shape *s, int
 {
 	if (!s) return 0;
 	const long n = (long)s->inChannels * s->ksize * s->ksize + (withBias ? 1 : 0);
-	return plan_gemm(n, n, (long)s->samples * s->outA * s->outB, true).wsBytes;
+	return plan_gemm_workspace(n, n, (long)s->samples * s->outA * s->outB, true);
 }
 
 int fitre_hip_kfac_conv_input_factor(const fitre_conv_shape *s, const float *x, int withBias, float *factor, void *ws,
@@ -66,7 +66,7 @@ int fitre_hip_kfac_conv_input_factor(const fitre_conv_shape *s, const float *x, 
 size_t fitre_hip_kfac_gram_workspace(int order, long reduce)
 {
 	if (order <= 0 || reduce <= 0) return 0;
-	return plan_gemm(order, order, reduce, true).wsBytes;
+	return plan_gemm_workspace(order, order, reduce, true);
 }
 
 int fitre_hip_kfac_conv_output_factor(const fitre_conv_shape *s, const float *delta, float *factor, void *ws, size_t wsBytes)

@@ -4,6 +4,7 @@
 // everything is queued on the selected lane, lane 0 unless a caller overlaps
 // independent work on lane 1).
 #include <stdarg.h>
+#include <stdlib.h>
 #include <string.h>
 #include <vector>
 #include "common.h"
@@ -16,6 +17,12 @@ static hipStream_t g_lanes[kLanes] = { nullptr, nullptr };
 static hipStream_t g_stream = nullptr; // the selected lane
 static int g_lane = 0;
 static bool g_lanes_on = true;
+// Compute units a kernel launched on each lane can occupy.  Lane 1 can be created with a
+// compute-unit mask that leaves a share of every XCD free (FITRE_LANE1_CUS), so that work on
+// lane 0 always finds idle compute units while a chip-filling kernel runs on lane 1; the
+// planners size their grids for the lane's share.  Off unless asked for: on the gradient path
+// it measured within noise of two unmasked lanes.
+static int g_lane_cus[kLanes] = { 256, 256 };
 constexpr int kJoinEvents = 64;
 static hipEvent_t g_join[kJoinEvents];
 static int g_join_next = 0;
@@ -56,6 +63,14 @@ int fail(int code, const char *fmt, ...)
 
 hipStream_t stream() { return g_stream; }
 int lane() { return g_lane; }
+int lane_compute_units() { return g_lane_cus[g_lane]; }
+int lane_compute_units_min()
+{
+	int m = g_lane_cus[0];
+	for (int i = 1; i < kLanes; i++) m = g_lane_cus[i] < m ? g_lane_cus[i] : m;
+	return m;
+}
+int device_compute_units() { return g_lane_cus[0]; }
 bool ready() { return g_ready; }
 
 int check_launch(const char *what)
@@ -140,7 +155,26 @@ int fitre_hip_init(int device)
 	FITRE_HIP_TRY(hipSetDevice(device));
 	if (g_ready && g_device == device) return FITRE_OK;
 	if (g_ready) fitre_hip_shutdown();
-	for (int i = 0; i < kLanes; i++) FITRE_HIP_TRY(hipStreamCreate(&g_lanes[i])); // default priority
+	int cus = 0;
+	FITRE_HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device));
+	if (cus <= 0 || cus > 1024) return fail(FITRE_E_DEVICE, "fitre_hip_init: device reports %d compute units", cus);
+	FITRE_HIP_TRY(hipStreamCreate(&g_lanes[0])); // default priority
+	g_lane_cus[0] = cus;
+	// Lane 1 masked: the first `share` bits of the mask; the driver deals mask bits round-robin to
+	// the XCDs, so every XCD keeps the same number of compute units.
+	int share = cus;
+	if (const char *env = getenv("FITRE_LANE1_CUS")) share = atoi(env);
+	share -= share % 8;
+	if (share >= 8 && share < cus) {
+		uint32_t mask[32];
+		memset(mask, 0, sizeof(mask));
+		for (int b = 0; b < share; b++) mask[b / 32] |= 1u << (b % 32);
+		FITRE_HIP_TRY(hipExtStreamCreateWithCUMask(&g_lanes[1], (uint32_t)((cus + 31) / 32), mask));
+		g_lane_cus[1] = share;
+	} else {
+		FITRE_HIP_TRY(hipStreamCreate(&g_lanes[1]));
+		g_lane_cus[1] = cus;
+	}
 	for (int i = 0; i < kJoinEvents; i++) FITRE_HIP_TRY(hipEventCreateWithFlags(&g_join[i], hipEventDisableTiming));
 	g_join_next = 0;
 	g_stream = g_lanes[0];

@@ -90,7 +90,6 @@ static size_t backward_chain_ws_bytes(const CNN_MODEL *model, int batch)
 	}
 	for (int i = 0; i < model->lLayers; i++) {
 		const FC_LAYER *f = &model->fcLayer[i];
-		need = max_sz(need, fitre_hip_gemm_workspace(f->out, f->in, batch));
 		need = max_sz(need, fitre_hip_gemm_workspace(f->in, batch, f->out));
 	}
 	return (need + 255) & ~(size_t)255;
@@ -102,6 +101,10 @@ static size_t backward_side_ws_bytes(const CNN_MODEL *model, int batch)
 	for (int i = 0; i < model->cLayers; i++) {
 		fitre_conv_shape s = conv_shape(&model->convLayer[i], batch);
 		need = max_sz(need, fitre_hip_conv_weight_grad_workspace(&s));
+	}
+	for (int i = 0; i < model->lLayers; i++) {
+		const FC_LAYER *f = &model->fcLayer[i];
+		need = max_sz(need, fitre_hip_gemm_workspace(f->out, f->in, batch));
 	}
 	return (need + 255) & ~(size_t)255;
 }
@@ -228,16 +231,22 @@ void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, 
 
 		/* delta *= f'(.) */
 		HIP_CALL(fitre_hip_activation_backward(l->actFun, delta, zl + l->offset, zl, delta, count));
+		/* The chain (lane 0) goes straight on to delta = W' * delta.  It writes the buffer that the
+		 * layer above handed to lane 1, so lane 0 first waits for what lane 1 still reads there. */
+		HIP_CALL(fitre_hip_lane_wait(1, 0));
+		HIP_CALL(fitre_hip_lane_wait(0, 1));
+		HIP_CALL(fitre_hip_gemm(1, 0, l->in, n, l->out, 1.f, weights + wOffsets[f + nc], l->out, delta, l->out, 0.f,
+		                        delta_new, l->in, NULL, ws, wsBytes));
+		/* Beside it, on lane 1, what nothing later in this pass reads: */
+		HIP_CALL(fitre_hip_lane_select(1));
 		/* dW = delta * z' */
 		HIP_CALL(fitre_hip_gemm(0, 1, l->out, l->in, n, 1.f, delta, l->out, zin, l->in, 0.f,
-		                        gradient + wOffsets[f + nc], l->out, NULL, ws, wsBytes));
+		                        gradient + wOffsets[f + nc], l->out, NULL, sideWs, sideBytes));
 		/* db = delta * 1 */
 		if (model->bias != 0) HIP_CALL(fitre_hip_row_sum(delta, l->out, n, gradient + bOffsets[f + nc]));
 		/* snapshot kept for the Hessian-vector product and the KFAC factors */
 		HIP_CALL(fitre_hip_copy_d2d(dx + zOffsets[f + nc + 1], delta, sizeof(real) * (size_t)count));
-		/* delta = W' * delta */
-		HIP_CALL(fitre_hip_gemm(1, 0, l->in, n, l->out, 1.f, weights + wOffsets[f + nc], l->out, delta, l->out, 0.f,
-		                        delta_new, l->in, NULL, ws, wsBytes));
+		HIP_CALL(fitre_hip_lane_select(0));
 		temp = delta_new;
 		delta_new = delta;
 		delta = temp;
@@ -247,6 +256,7 @@ void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, 
 	{
 		int extA, extB;
 		feature_extent(model, &extA, &extB);
+		HIP_CALL(fitre_hip_lane_wait(0, 1)); /* lane 1 may still read delta_new (the first FC layer's delta) */
 		HIP_CALL(fitre_hip_fc_to_conv(delta, last->outChannels, n, extA, extB, delta_new));
 		temp = delta_new;
 		delta_new = delta;
@@ -293,13 +303,15 @@ void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, 
 
 		const real *input = (c == 0) ? data->currentBatch : z + zOffsets[c] + model->convLayer[c - 1].outputOffset;
 		fitre_conv_shape shape = conv_shape(l, n);
-		/* The weight gradient needs this layer's delta and input, both final by now, and nothing
-		 * later reads its result: it runs on lane 1 beside the chain that goes on to the layers below. */
+		/* The input gradient fills the chip first.  The weight gradient, whose result nothing later
+		 * reads, is queued behind it on lane 1, whose kernels leave a share of the compute units
+		 * free: the bandwidth-bound kernels of the layer below (split reduction, pooling, batch
+		 * norm) run on those while the weight gradient keeps the matrix pipes busy. */
+		if (c != 0) HIP_CALL(fitre_hip_conv_input_grad(&shape, cur, weights + wOffsets[c], delta, ws, wsBytes));
 		HIP_CALL(fitre_hip_lane_wait(1, 0));
 		HIP_CALL(fitre_hip_lane_select(1));
 		HIP_CALL(fitre_hip_conv_weight_grad(&shape, input, cur, gradient + wOffsets[c], sideWs, sideBytes));
 		HIP_CALL(fitre_hip_lane_select(0));
-		if (c != 0) HIP_CALL(fitre_hip_conv_input_grad(&shape, cur, weights + wOffsets[c], delta, ws, wsBytes));
 	}
 	HIP_CALL(fitre_hip_sync());
 }
