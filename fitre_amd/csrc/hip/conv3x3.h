@@ -342,12 +342,29 @@ conv3x3_dw_kernel(const Conv3x3Params p, const float *delta, uint32_t deltaBytes
 	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 	const int khalf = lane >> 5, l32 = lane & 31;
 	const int ob = wave & 3, ta = wave >> 2; // output-channel block, tap row
-	const int c0 = blockIdx.x * kC3DwCin, o0 = blockIdx.y * kC3Tile;
+	// Workgroups are dealt to the eight XCDs (each with its own L2) round-robin by launch index.
+	// Renumber them so that an XCD holds consecutive indices, input-channel tile fastest and split
+	// slowest: the workgroups that read the same range of positions -- the same delta rows and the
+	// same input rows -- then share an L2 instead of fetching them once per XCD.
+	int bx = blockIdx.x, by = blockIdx.y, bz = blockIdx.z;
+	{
+		const unsigned groups = gridDim.x * gridDim.y * gridDim.z;
+		if ((groups & 7u) == 0) {
+			const unsigned lin = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+			const unsigned logical = (lin & 7u) * (groups >> 3) + (lin >> 3);
+			const unsigned tiles = gridDim.x * gridDim.y;
+			bz = (int)(logical / tiles);
+			const unsigned rem = logical - (unsigned)bz * tiles;
+			by = (int)(rem / gridDim.x);
+			bx = (int)(rem - (unsigned)by * gridDim.x);
+		}
+	}
+	const int c0 = bx * kC3DwCin, o0 = by * kC3Tile;
 	const int halo = p.B + 1;
 	const int win = kC3Stage + 2 * halo;
 	const int plane = p.J;
 	const int stagesTotal = p.J / kC3Stage;
-	const int stBeg = blockIdx.z * p.perSplit;
+	const int stBeg = bz * p.perSplit;
 	const int stEnd = (stBeg + p.perSplit < stagesTotal) ? stBeg + p.perSplit : stagesTotal;
 	const bool movingRows = (kC3Stage % p.B) != 0; // else every stage window starts in the same column
 
@@ -520,7 +537,7 @@ conv3x3_dw_kernel(const Conv3x3Params p, const float *delta, uint32_t deltaBytes
 	// ---- store: dW[o][c][tap].  A wave holds taps (ta, 0..2) of 32 output x 32 input channels, i.e.
 	// runs of three words; the three waves of an output-channel block go through LDS together so that
 	// global memory sees whole rows of 32*9 consecutive words. --------------------------------------
-	float *C = out.C + (size_t)blockIdx.z * out.splitStride;
+	float *C = out.C + (size_t)bz * out.splitStride;
 	float *stage = &Ds[0][0];
 	constexpr int ROW = kC3DwCin * 9, ROW_LD = ROW + 1;
 	static_assert(32 * ROW_LD <= 2 * (D_DUMMY + 4), "the output stage must fit the delta buffers");
