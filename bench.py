@@ -16,6 +16,8 @@ Prints ONE JSON line: backward images/sec, plus
                 same K steps (the first, timed pass runs without per-launch events), against the
                 157.3 TFLOP/s fp32-MFMA peak;
   kernels       the same accounting for every kernel class of the backward pass;
+  bandwidth_kernels  pool+activation and batch-norm backward run alone at the two largest layers'
+                shapes, against the 8 TB/s HBM peak;
   cpu_baseline  the C restatement of the reference's algorithm (float32, OpenMP) timed on the host
                 cores on a bounded sample (same network, smaller batch);
   torch_cpu     torch autograd of the same network on the host cores (float32), for orientation.
@@ -124,6 +126,7 @@ def gpu_leg(args):
     kfac = kfac_leg(L, dev, gm, model, batch, max(2, args.steps // 4))
     kfac["hessian_vector_ms"] = hv_leg(L, dev, gm, model, batch, max(2, args.steps // 4))
     gm.release()
+    bandwidth = bandwidth_leg(L, dev, batch)
     dev.close()
 
     kernels = {}
@@ -153,7 +156,61 @@ def gpu_leg(args):
     conv["frac"] = round(conv["achieved"] / PEAK_MFMA_F32_TFLOPS, 4)
     return dict(wall=wall, ms_events=ms_events.value, batch=batch, loss=loss, finite=finite,
                 device=name.value.decode(), compute_units=cus.value, roofline=roofline, kernels=kernels,
-                conv_backward_gemms=conv, kfac_factors=kfac)
+                conv_backward_gemms=conv, kfac_factors=kfac, bandwidth_kernels=bandwidth)
+
+
+def bandwidth_leg(L, dev, batch, reps=20):
+    """The bandwidth-bound backward kernels run alone at the shapes of the two largest layers
+    (64 x 32x32 and 128 x 16x16 maps per image, max-pool 2, ReLU, batch norm): algorithmic bytes / time
+    against the 8 TB/s HBM peak, with a plain copy of the same tensor beside them.  Inside the backward
+    pass the per-class averages of `kernels` are dominated by the small layers' launches; the tensors here
+    are the ones that carry the bytes.  The same buffers are used by every repeat, so part of the traffic
+    is served by the memory-side cache, as it is in the pass itself (a layer's delta is read right after
+    it is written)."""
+    hip = L.hip
+    ev0, ev1 = C.c_void_p(), C.c_void_p()
+    L.check(hip.fitre_hip_event_create(C.byref(ev0)))
+    L.check(hip.fitre_hip_event_create(C.byref(ev1)))
+
+    def timed(fn):
+        L.check(fn())
+        L.check(fn())
+        dev.sync()
+        L.check(hip.fitre_hip_event_record(ev0))
+        for _ in range(reps):
+            L.check(fn())
+        L.check(hip.fitre_hip_event_record(ev1))
+        dev.sync()
+        ms = C.c_float()
+        L.check(hip.fitre_hip_event_elapsed_ms(ev0, ev1, C.byref(ms)))
+        return ms.value / reps * 1e-3
+
+    rng = np.random.default_rng(0xF17E0004)
+    relu = 13  # CNN_ACT_RELU
+    out = {}
+    for name, channels, hw in (("layer0_64x32x32", 64, 32), ("layer1_128x16x16", 128, 16)):
+        per = batch * hw * hw
+        n = channels * per
+        zhat = dev.upload(rng.standard_normal(n).astype(np.float32))
+        zact = dev.zeros(n)
+        L.check(hip.fitre_hip_activation_forward(relu, zhat, zact, n))
+        var = dev.upload(np.ones(channels, np.float32))
+        dpool, dact, dbn, bias = dev.zeros(n), dev.zeros(n), dev.zeros(n), dev.zeros(channels)
+        delta = dev.upload(rng.standard_normal(n // 4).astype(np.float32))
+        nb = hip.fitre_hip_batch_norm_workspace(channels, per)
+        ws = dev.alloc(nb)
+        t_copy = timed(lambda: hip.fitre_hip_copy(n, zhat, dbn))
+        t_pool = timed(lambda: hip.fitre_hip_pool_act_backward(0, relu, delta, zhat, zact, channels, batch, hw, hw, 2, 2,
+                                                               0, hw // 2, hw // 2, dpool, dact))
+        t_bn = timed(lambda: hip.fitre_hip_batch_norm_backward(dact, zhat, var, channels, per, 1e-5, dbn, bias, ws, nb))
+        rows = dict(copy=(8.0 * n, t_copy),                 # read + write
+                    pool_act_bwd=(4.0 * (n / 4 + 3 * n), t_pool),  # delta (pooled), z_act read; two gradients written
+                    bn_bwd=(12.0 * n, t_bn))                # delta, zhat read once; dx written (the kernel pair moves 20 B)
+        out[name] = {k: dict(us=round(t * 1e6, 2), achieved=round(b / t / 1e9, 1), unit="GB/s",
+                             frac=round(b / t / 1e9 / PEAK_HBM_GBS, 4)) for k, (b, t) in rows.items()}
+        for p in (zhat, zact, var, dpool, dact, dbn, bias, delta, ws):
+            dev.free(p)
+    return out
 
 
 def kfac_leg(L, dev, gm, model, batch, passes):
@@ -324,6 +381,7 @@ def main():
         "roofline": g["roofline"],
         "conv_backward_gemms": g["conv_backward_gemms"],
         "kfac_factors": g["kfac_factors"],
+        "bandwidth_kernels": g["bandwidth_kernels"],
         "kernels": g["kernels"],
         "wall_ms_per_step": round(1e3 * g["wall"] / args.steps, 4),
         "loss": round(g["loss"], 6),

@@ -526,6 +526,216 @@ bn_backward_small_kernel(const float *delta, const float *zhat, const float *var
 	}
 }
 
+// ---------------------------------------------------------------------
+// pool + activation + batch-norm backward in two launches (one for short channels)
+// ---------------------------------------------------------------------
+// The batch-norm backward sums are sums over the gradient this pass writes, so it leaves them behind
+// and the batch-norm step is the elementwise pass alone: 12 bytes per element instead of 20.
+
+// the four cells of a 16-byte group: gradient after the activation, and the sums' terms
+__device__ __forceinline__ float4 act_backward4(int actFun, float4 g, float4 zi, float4 zo)
+{
+	g.x *= act_derivative(actFun, zi.x, zo.x);
+	g.y *= act_derivative(actFun, zi.y, zo.y);
+	g.z *= act_derivative(actFun, zi.z, zo.z);
+	g.w *= act_derivative(actFun, zi.w, zo.w);
+	return g;
+}
+__device__ __forceinline__ float4 relu4(float4 v)
+{
+	return make_float4(v.x > 0.f ? v.x : 0.f, v.y > 0.f ? v.y : 0.f, v.z > 0.f ? v.z : 0.f, v.w > 0.f ? v.w : 0.f);
+}
+__device__ __forceinline__ void bn_sums4(float4 g, float4 z, double &s1, double &s2, double &s3)
+{
+	s1 += (double)((g.x + g.y) + (g.z + g.w));
+	s2 += (double)(g.x * z.x) + (double)(g.y * z.y) + (double)(g.z * z.z) + (double)(g.w * z.w);
+	s3 += (double)((z.x + z.y) + (z.z + z.w));
+}
+// routes the two pooled gradients d of a 2 x 4 patch (rows r0, r1 of the pool input) to the window maxima
+__device__ __forceinline__ void route2x4(float4 r0, float4 r1, float2 d, float4 &g0, float4 &g1)
+{
+	g0 = make_float4(0.f, 0.f, 0.f, 0.f);
+	g1 = g0;
+	int arg = scan2x2(r0.x, r0.y, r1.x, r1.y);
+	if (arg == 0) g0.x = d.x;
+	else if (arg == 1) g0.y = d.x;
+	else if (arg == 2) g1.x = d.x;
+	else if (arg == 3) g1.y = d.x;
+	arg = scan2x2(r0.z, r0.w, r1.z, r1.w);
+	if (arg == 0) g0.z = d.y;
+	else if (arg == 1) g0.w = d.y;
+	else if (arg == 2) g1.z = d.y;
+	else if (arg == 3) g1.w = d.y;
+}
+
+// B == 2: a window is the 16-byte group (a, 0), (a, 1), (a + 1, 0), (a + 1, 1)
+__device__ __forceinline__ float4 route2x2(float4 r, float d)
+{
+	float4 g = make_float4(0.f, 0.f, 0.f, 0.f);
+	const int arg = scan2x2(r.x, r.y, r.z, r.w);
+	if (arg == 0) g.x = d;
+	else if (arg == 1) g.y = d;
+	else if (arg == 2) g.z = d;
+	else if (arg == 3) g.w = d;
+	return g;
+}
+
+// One (channel, segment) per workgroup.  POOL 0: 2x2 / stride 2 max pool (B % 4 == 0, A even), the
+// unit of work is a 2 x 4 patch; POOL 2: no pooling, the unit is a 16-byte group; POOL 3: 2x2 / stride 2
+// max pool of maps with B == 2, where pooled cell q of a channel is its 16-byte group q.  z_act == nullptr:
+// the activation is ReLU and its output is max(zhat, 0).  partial: slots of four doubles
+// (sum g, sum g*zhat, sum zhat) per (channel, segment).
+template <int POOL>
+__global__ void __launch_bounds__(kRedBlock)
+pool_act_sums_kernel(const float *delta, const float *zhat, const float *z_act, int inA, int inB, int samples, int actFun,
+                     float *dxPool, float *dxAct, double *partial)
+{
+	__shared__ double lds[kRedBlock / kWave];
+	const int c = blockIdx.y;
+	const long perChannel = (long)samples * inA * inB;
+	const size_t base = (size_t)c * perChannel;
+	double s1 = 0.0, s2 = 0.0, s3 = 0.0;
+	if constexpr (POOL == 2 || POOL == 3) {
+		long lo, hi;
+		segment_range(perChannel, lo, hi);
+		for (long i = lo + 4 * (long)threadIdx.x; i + 3 < hi; i += 4 * kRedBlock) {
+			const float4 zi = *reinterpret_cast<const float4 *>(zhat + base + i);
+			const float4 zo = z_act ? *reinterpret_cast<const float4 *>(z_act + base + i) : relu4(zi);
+			float4 g;
+			if constexpr (POOL == 2) g = *reinterpret_cast<const float4 *>(delta + base + i);
+			else g = route2x2(zo, delta[(base + i) / 4]);
+			if (dxPool) *reinterpret_cast<float4 *>(dxPool + base + i) = g;
+			g = act_backward4(actFun, g, zi, zo);
+			*reinterpret_cast<float4 *>(dxAct + base + i) = g;
+			bn_sums4(g, zi, s1, s2, s3);
+		}
+	} else {
+		const int outB2 = inB / 4, outA = inA / 2;
+		const int perMap = outA * outB2;
+		const long patches = (long)samples * perMap;
+		const long per = (patches + gridDim.x - 1) / gridDim.x;
+		const long lo = (long)blockIdx.x * per;
+		const long hi = (lo + per < patches) ? lo + per : patches;
+		const size_t dBase = (size_t)c * samples * outA * (inB / 2);
+		for (long i = lo + threadIdx.x; i < hi; i += kRedBlock) {
+			const long map = i / perMap;
+			const int rem = (int)(i - map * perMap);
+			const int oa = rem / outB2, pb = rem - oa * outB2;
+			const size_t inOff = base + (size_t)map * inA * inB + (size_t)(2 * oa) * inB + 4 * pb;
+			const size_t dOff = dBase + (size_t)map * outA * (inB / 2) + (size_t)oa * (inB / 2) + 2 * pb;
+			const float4 i0 = *reinterpret_cast<const float4 *>(zhat + inOff);
+			const float4 i1 = *reinterpret_cast<const float4 *>(zhat + inOff + inB);
+			const float4 r0 = z_act ? *reinterpret_cast<const float4 *>(z_act + inOff) : relu4(i0);
+			const float4 r1 = z_act ? *reinterpret_cast<const float4 *>(z_act + inOff + inB) : relu4(i1);
+			const float2 d = *reinterpret_cast<const float2 *>(delta + dOff);
+			float4 g0, g1;
+			route2x4(r0, r1, d, g0, g1);
+			if (dxPool) {
+				*reinterpret_cast<float4 *>(dxPool + inOff) = g0;
+				*reinterpret_cast<float4 *>(dxPool + inOff + inB) = g1;
+			}
+			g0 = act_backward4(actFun, g0, i0, r0);
+			g1 = act_backward4(actFun, g1, i1, r1);
+			*reinterpret_cast<float4 *>(dxAct + inOff) = g0;
+			*reinterpret_cast<float4 *>(dxAct + inOff + inB) = g1;
+			bn_sums4(g0, i0, s1, s2, s3);
+			bn_sums4(g1, i1, s1, s2, s3);
+		}
+	}
+	const double t1 = block_sum<kRedBlock>(s1, lds);
+	const double t2 = block_sum<kRedBlock>(s2, lds);
+	const double t3 = block_sum<kRedBlock>(s3, lds);
+	if (threadIdx.x == 0) {
+		double *slot = partial + ((size_t)c * gridDim.x + blockIdx.x) * 4;
+		slot[0] = t1, slot[1] = t2, slot[2] = t3;
+	}
+}
+
+// Short channels (at most kBnSmallChannel cells): one workgroup per channel keeps the gradient and zhat
+// in registers between the sums and the batch-norm formula; one launch for the three steps.
+template <int POOL>
+__global__ void __launch_bounds__(kRedBlock)
+pool_act_bn_small_kernel(const float *delta, const float *zhat, const float *z_act, const float *variance, int inA, int inB,
+                         int samples, int actFun, float epsilon, float *dxPool, float *dxAct, float *dxBn, float *biasGrad)
+{
+	__shared__ double lds[kRedBlock / kWave];
+	constexpr int G = (int)(kBnSmallChannel / (4 * kRedBlock)); // 16-byte groups per thread
+	static_assert(G >= 2 && G % 2 == 0, "a 2 x 4 patch is two groups");
+	const int c = blockIdx.x;
+	const long perChannel = (long)samples * inA * inB;
+	const size_t base = (size_t)c * perChannel;
+	float4 g[G], z[G];
+	long off[G]; // offset of the group inside the channel, -1: none
+	double s1 = 0.0, s2 = 0.0, s3 = 0.0;
+	if constexpr (POOL == 2 || POOL == 3) {
+#pragma unroll
+		for (int k = 0; k < G; k++) {
+			const long i = 4 * ((long)threadIdx.x + (long)k * kRedBlock);
+			off[k] = (i + 3 < perChannel) ? i : -1;
+			if (off[k] < 0) continue;
+			z[k] = *reinterpret_cast<const float4 *>(zhat + base + i);
+			const float4 zo = z_act ? *reinterpret_cast<const float4 *>(z_act + base + i) : relu4(z[k]);
+			if constexpr (POOL == 2) g[k] = *reinterpret_cast<const float4 *>(delta + base + i);
+			else g[k] = route2x2(zo, delta[(base + i) / 4]);
+			if (dxPool) *reinterpret_cast<float4 *>(dxPool + base + i) = g[k];
+			g[k] = act_backward4(actFun, g[k], z[k], zo);
+			*reinterpret_cast<float4 *>(dxAct + base + i) = g[k];
+			bn_sums4(g[k], z[k], s1, s2, s3);
+		}
+	} else {
+		const int outB2 = inB / 4, outA = inA / 2;
+		const int perMap = outA * outB2;
+		const long patches = (long)samples * perMap;
+		const size_t dBase = (size_t)c * samples * outA * (inB / 2);
+#pragma unroll
+		for (int k = 0; k < G / 2; k++) {
+			const long i = (long)threadIdx.x + (long)k * kRedBlock;
+			off[2 * k] = off[2 * k + 1] = -1;
+			if (i >= patches) continue;
+			const long map = i / perMap;
+			const int rem = (int)(i - map * perMap);
+			const int oa = rem / outB2, pb = rem - oa * outB2;
+			const long in = map * inA * inB + (long)(2 * oa) * inB + 4 * pb;
+			const size_t dOff = dBase + (size_t)map * outA * (inB / 2) + (size_t)oa * (inB / 2) + 2 * pb;
+			off[2 * k] = in;
+			off[2 * k + 1] = in + inB;
+			z[2 * k] = *reinterpret_cast<const float4 *>(zhat + base + in);
+			z[2 * k + 1] = *reinterpret_cast<const float4 *>(zhat + base + in + inB);
+			const float4 r0 = z_act ? *reinterpret_cast<const float4 *>(z_act + base + in) : relu4(z[2 * k]);
+			const float4 r1 = z_act ? *reinterpret_cast<const float4 *>(z_act + base + in + inB) : relu4(z[2 * k + 1]);
+			const float2 d = *reinterpret_cast<const float2 *>(delta + dOff);
+			route2x4(r0, r1, d, g[2 * k], g[2 * k + 1]);
+			if (dxPool) {
+				*reinterpret_cast<float4 *>(dxPool + base + in) = g[2 * k];
+				*reinterpret_cast<float4 *>(dxPool + base + in + inB) = g[2 * k + 1];
+			}
+			g[2 * k] = act_backward4(actFun, g[2 * k], z[2 * k], r0);
+			g[2 * k + 1] = act_backward4(actFun, g[2 * k + 1], z[2 * k + 1], r1);
+			*reinterpret_cast<float4 *>(dxAct + base + in) = g[2 * k];
+			*reinterpret_cast<float4 *>(dxAct + base + in + inB) = g[2 * k + 1];
+			bn_sums4(g[2 * k], z[2 * k], s1, s2, s3);
+			bn_sums4(g[2 * k + 1], z[2 * k + 1], s1, s2, s3);
+		}
+	}
+	const double d1 = block_sum<kRedBlock>(s1, lds);
+	const double d2 = block_sum<kRedBlock>(s2, lds);
+	const double d3 = block_sum<kRedBlock>(s3, lds);
+	const float m = (float)perChannel;
+	const float sum1 = (float)d1, sum2 = (float)d2;
+	const float scale = 1.f / (m * sqrtf(epsilon + variance[c]));
+	if (biasGrad && threadIdx.x == 0) biasGrad[c] = (float)(-d2 * d3 * (double)scale);
+#pragma unroll
+	for (int k = 0; k < G; k++) {
+		if (off[k] < 0) continue;
+		float4 r;
+		r.x = bn_backward_value(m, g[k].x, z[k].x, sum1, sum2, scale);
+		r.y = bn_backward_value(m, g[k].y, z[k].y, sum1, sum2, scale);
+		r.z = bn_backward_value(m, g[k].z, z[k].z, sum1, sum2, scale);
+		r.w = bn_backward_value(m, g[k].w, z[k].w, sum1, sum2, scale);
+		*reinterpret_cast<float4 *>(dxBn + base + off[k]) = r;
+	}
+}
+
 // Directional derivative of the batch-norm backward formula.  Per channel, with s = sqrt(var + eps)
 // and <.> the mean over the channel:
 //   out = ( rdx - <rdx> - rzhat <dx zhat> - zhat ( <rdx zhat> + <dx rzhat> ) ) / s  -  dc <zhat rx> / s
@@ -934,6 +1144,79 @@ int fitre_hip_batch_norm_backward(const float *delta, const float *zhat, const f
 		                                                                  out, biasGrad);
 	}
 	return check_launch("batch_norm_backward");
+}
+
+int fitre_hip_pool_act_bn_backward(int poolType, int actFun, const float *delta, const float *zhat, const float *z_act,
+                                   const float *variance, int channels, int samples, int inA, int inB, int ksize, int stride,
+                                   int padding, int outA, int outB, float epsilon, float *dxPool, float *dxAct, float *dxBn,
+                                   float *biasGrad, void *ws, size_t wsBytes)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(delta && zhat && variance && dxAct && dxBn, "fitre_hip_pool_act_bn_backward: null pointer");
+	FITRE_REQUIRE(z_act || actFun == CNN_ACT_RELU,
+	              "fitre_hip_pool_act_bn_backward: z_act may be left out for ReLU only (activation %d)", actFun);
+	FITRE_REQUIRE(act_known(actFun), "fitre_hip_pool_act_bn_backward: unknown activation code %d", actFun);
+	FITRE_REQUIRE(channels > 0 && samples > 0 && inA > 0 && inB > 0, "fitre_hip_pool_act_bn_backward: non-positive shape");
+	const long perChannel = (long)samples * inA * inB;
+	int rc = check_channels("fitre_hip_pool_act_bn_backward", channels, perChannel, ws, wsBytes);
+	if (rc) return rc;
+	FITRE_REQUIRE((double)channels * (double)perChannel < 2147483647.0, "fitre_hip_pool_act_bn_backward: tensor exceeds 2^31 elements");
+	const bool aligned = aligned16(zhat) && aligned16(dxAct) && aligned16(dxBn) && (!z_act || aligned16(z_act)) &&
+	                     (!dxPool || aligned16(dxPool));
+	bool fused = false;
+	if (poolType == NO_POOL)
+		fused = aligned && aligned16(delta) && perChannel % 4 == 0;
+	else if (poolType == MAX_POOL)
+		fused = aligned && ksize == 2 && stride == 2 && padding == 0 && (inB % 4 == 0 || inB == 2) && inA % 2 == 0 &&
+		        outA == inA / 2 && outB == inB / 2 && (((uintptr_t)delta & 7) == 0);
+	const int variant = (poolType == NO_POOL) ? 2 : (inB == 2 ? 3 : 0);
+	if (!fused) {
+		// other windows / layouts: the separate passes (z_act rebuilt for the ReLU shortcut)
+		const float *zo = z_act;
+		if (!zo) {
+			rc = fitre_hip_activation_forward(actFun, zhat, dxBn, (long)channels * perChannel);
+			if (rc) return rc;
+			zo = dxBn; // free until the batch-norm step writes it
+		}
+		rc = fitre_hip_pool_act_backward(poolType, actFun, delta, zhat, zo, channels, samples, inA, inB, ksize, stride, padding,
+		                                 outA, outB, dxPool, dxAct);
+		if (rc) return rc;
+		return fitre_hip_batch_norm_backward(dxAct, zhat, variance, channels, perChannel, epsilon, dxBn, biasGrad, ws, wsBytes);
+	}
+	const double total = (double)channels * (double)perChannel;
+	const double poolBytes = 4.0 * total * (2 + (dxPool ? 1 : 0) + (z_act ? 1 : 0)) +
+	                         4.0 * (poolType == NO_POOL ? total : total / 4);
+	if (perChannel <= kBnSmallChannel && channels >= 128) {
+		LaunchScope scope(FITRE_KC_POOL_ACT_BWD, poolBytes + 4.0 * total);
+		if (variant == 2)
+			pool_act_bn_small_kernel<2><<<channels, kRedBlock, 0, stream()>>>(delta, zhat, z_act, variance, inA, inB, samples, actFun,
+			                                                                 epsilon, dxPool, dxAct, dxBn, biasGrad);
+		else if (variant == 3)
+			pool_act_bn_small_kernel<3><<<channels, kRedBlock, 0, stream()>>>(delta, zhat, z_act, variance, inA, inB, samples, actFun,
+			                                                                 epsilon, dxPool, dxAct, dxBn, biasGrad);
+		else
+			pool_act_bn_small_kernel<0><<<channels, kRedBlock, 0, stream()>>>(delta, zhat, z_act, variance, inA, inB, samples, actFun,
+			                                                                 epsilon, dxPool, dxAct, dxBn, biasGrad);
+		return check_launch("pool_act_bn_small_kernel");
+	}
+	const int S = segments_for(channels, perChannel);
+	double *partial = (double *)ws;
+	dim3 grid(S, channels);
+	{
+		LaunchScope scope(FITRE_KC_POOL_ACT_BWD, poolBytes);
+		if (variant == 2)
+			pool_act_sums_kernel<2><<<grid, kRedBlock, 0, stream()>>>(delta, zhat, z_act, inA, inB, samples, actFun, dxPool, dxAct, partial);
+		else if (variant == 3)
+			pool_act_sums_kernel<3><<<grid, kRedBlock, 0, stream()>>>(delta, zhat, z_act, inA, inB, samples, actFun, dxPool, dxAct, partial);
+		else
+			pool_act_sums_kernel<0><<<grid, kRedBlock, 0, stream()>>>(delta, zhat, z_act, inA, inB, samples, actFun, dxPool, dxAct, partial);
+		rc = check_launch("pool_act_sums_kernel");
+		if (rc) return rc;
+	}
+	LaunchScope scope(FITRE_KC_BN_BWD, 12.0 * total + 8.0 * channels);
+	bn_backward_apply_kernel<true><<<grid, kRedBlock, 0, stream()>>>(dxAct, zhat, variance, partial, S, epsilon, perChannel, dxBn,
+	                                                                 biasGrad);
+	return check_launch("bn_backward_apply_kernel");
 }
 
 int fitre_hip_softmax_cross_entropy(const float *logits, const float *target, int rows, int classes, float *probs,

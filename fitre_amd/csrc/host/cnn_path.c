@@ -277,28 +277,34 @@ void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, 
 		}
 		const real *actIn = has_bn(l) ? slab + l->batchNormOffset : slab;
 		const real *actOut = slab + l->activationOffset;
+		/* With batch norm and ReLU the fused pass derives the activation output from its input. */
+		const int fusedRelu = has_bn(l) && act == CNN_ACT_RELU;
 		if (c == nc - 1 && p->type == NO_POOL) {
 			/* The forward pass rewrote this layer's activation output into the FC layout in place;
 			 * rebuild it from the activation input (the reference reads the permuted buffer,
 			 * functions/cnn_backward.cu:574-580). */
-			HIP_CALL(fitre_hip_activation_forward(act, actIn, delta_new, perChannel * l->outChannels));
+			if (!fusedRelu) HIP_CALL(fitre_hip_activation_forward(act, actIn, delta_new, perChannel * l->outChannels));
 			actOut = delta_new;
 		}
-		/* pool backward -> dx slab + 0; times f'(.) -> dx slab + activationOffset */
-		HIP_CALL(fitre_hip_pool_act_backward(p->type, act, delta, actIn, actOut, l->outChannels, n, p->width, p->height,
-		                                     p->pSize, p->stride, p->padding, p->outWidth, p->outHeight, dslab,
-		                                     dslab + l->activationOffset));
-		const real *cur = dslab + l->activationOffset;
-
+		const real *cur;
 		if (has_bn(l)) {
-			/* batch-norm backward -> dx slab + batchNormOffset; its column sums are the bias gradient */
-			HIP_CALL(fitre_hip_batch_norm_backward(cur, slab + l->batchNormOffset,
-			                                       slab + l->batchNormOffset + l->variancesOffset, l->outChannels,
-			                                       perChannel, (real)BATCH_NORM_EPSILON, dslab + l->batchNormOffset,
-			                                       (model->bias != 0) ? gradient + bOffsets[c] : NULL, ws, wsBytes));
+			/* pool backward -> dx slab + 0; times f'(.) -> dx slab + activationOffset; batch-norm backward ->
+			 * dx slab + batchNormOffset, its column sums being the bias gradient */
+			HIP_CALL(fitre_hip_pool_act_bn_backward(p->type, act, delta, actIn, fusedRelu ? NULL : actOut,
+			                                        slab + l->batchNormOffset + l->variancesOffset, l->outChannels, n, p->width,
+			                                        p->height, p->pSize, p->stride, p->padding, p->outWidth, p->outHeight,
+			                                        (real)BATCH_NORM_EPSILON, dslab, dslab + l->activationOffset,
+			                                        dslab + l->batchNormOffset,
+			                                        (model->bias != 0) ? gradient + bOffsets[c] : NULL, ws, wsBytes));
 			cur = dslab + l->batchNormOffset;
-		} else if (model->bias != 0) {
-			HIP_CALL(fitre_hip_channel_sum(cur, l->outChannels, perChannel, gradient + bOffsets[c], ws, wsBytes));
+		} else {
+			/* pool backward -> dx slab + 0; times f'(.) -> dx slab + activationOffset */
+			HIP_CALL(fitre_hip_pool_act_backward(p->type, act, delta, actIn, actOut, l->outChannels, n, p->width, p->height,
+			                                     p->pSize, p->stride, p->padding, p->outWidth, p->outHeight, dslab,
+			                                     dslab + l->activationOffset));
+			cur = dslab + l->activationOffset;
+			if (model->bias != 0)
+				HIP_CALL(fitre_hip_channel_sum(cur, l->outChannels, perChannel, gradient + bOffsets[c], ws, wsBytes));
 		}
 
 		const real *input = (c == 0) ? data->currentBatch : z + zOffsets[c] + model->convLayer[c - 1].outputOffset;

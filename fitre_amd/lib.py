@@ -68,6 +68,7 @@ HIP_API = {
     "fitre_hip_pool_backward": (i32, [i32, vp, vp] + [i32] * 9 + [vp]),
     "fitre_hip_max_pool_argmax": (i32, [vp] + [i32] * 9 + [vp]),
     "fitre_hip_pool_act_backward": (i32, [i32, i32, vp, vp, vp] + [i32] * 9 + [vp, vp]),
+    "fitre_hip_pool_act_bn_backward": (i32, [i32, i32, vp, vp, vp, vp] + [i32] * 9 + [f32, vp, vp, vp, vp, vp, sz]),
     "fitre_hip_batch_norm_workspace": (sz, [i32, lng]),
     "fitre_hip_batch_norm_forward": (i32, [vp, i32, lng, vp, vp, vp, vp, vp, f32, f32, i32, vp, sz]),
     "fitre_hip_batch_norm_backward": (i32, [vp, vp, vp, i32, lng, f32, vp, vp, vp, sz]),

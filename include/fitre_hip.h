@@ -198,6 +198,19 @@ int fitre_hip_batch_norm_backward(const float *delta, const float *zhat, const f
                                   int channels, long perChannel, float epsilon, float *out,
                                   float *biasGrad, void *ws, size_t wsBytes);
 
+/* fitre_hip_pool_act_backward followed by fitre_hip_batch_norm_backward of its dxAct, as the backward pass
+ * runs them for a layer with batch norm (functions/cnn_backward.cu:586-660): the pool/activation pass leaves the
+ * batch-norm sums behind, so the batch-norm step moves 12 bytes per element instead of 20.  zhat is the
+ * activation input (the batch-norm output).  z_act may be NULL when actFun is ReLU: the activation output is
+ * then taken as max(zhat, 0), bit-identical to what the forward pass stored.  Fused for no pooling and for
+ * 2x2 / stride 2 max pooling on 16-byte-aligned tensors; every other case runs the two separate passes.
+ * Workspace: fitre_hip_batch_norm_workspace(channels, samples * inA * inB). */
+int fitre_hip_pool_act_bn_backward(int poolType, int actFun, const float *delta, const float *zhat,
+                                   const float *z_act, const float *variance, int channels, int samples,
+                                   int inA, int inB, int ksize, int stride, int padding, int outA, int outB,
+                                   float epsilon, float *dxPool, float *dxAct, float *dxBn, float *biasGrad,
+                                   void *ws, size_t wsBytes);
+
 /* ---------------- reductions ---------------- */
 /* out[c] = sum of the perChannel contiguous values of channel c (conv bias gradient,
  * functions/cnn_backward.cu:662-689). */

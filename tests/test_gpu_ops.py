@@ -277,6 +277,66 @@ def test_batch_norm_forward_backward(dev, oracle64, Cn, N, A, B, mis):
         dev.free(b)
 
 
+# C, N, A, B, k, s, p: fused sums (large channels), one-workgroup-per-channel (short channels, >= 128
+# of them), and shapes that fall back to the separate passes
+FUSED_BN_GEOMS = [
+    (3, 40, 16, 16, 2, 2, 0),    # two-launch fused path, several segments
+    (64, 8, 32, 32, 2, 2, 0),
+    (5, 9, 6, 12, 2, 2, 0),
+    (128, 16, 4, 4, 2, 2, 0),    # short channels: one launch
+    (160, 7, 8, 8, 2, 2, 0),
+    (130, 2, 2, 4, 2, 2, 0),
+    (512, 64, 2, 2, 2, 2, 0),    # maps with B == 2: a window is one 16-byte group
+    (5, 2100, 6, 2, 2, 2, 0),    # the same on long channels
+    (2, 3, 6, 10, 2, 2, 0),      # B % 4 != 0: separate passes
+    (2, 2, 7, 5, 3, 2, 1),       # 3/2/1 window: separate passes
+]
+
+
+@pytest.mark.parametrize("geom", FUSED_BN_GEOMS)
+@pytest.mark.parametrize("act,derive", [(CNN_ACT_RELU, True), (CNN_ACT_RELU, False), (CNN_ACT_SWISH, False)])
+@pytest.mark.parametrize("kind", [MAX_POOL, NO_POOL, AVG_POOL])
+def test_fused_pool_activation_batch_norm_backward(dev, oracle64, geom, act, derive, kind):
+    """fitre_hip_pool_act_bn_backward against the oracle's three steps (functions/cnn_backward.cu:586-660)."""
+    Cn, N, A, B, k, s, p = geom
+    oA, oB = ((A + 2 * p - k) // s + 1, (B + 2 * p - k) // s + 1) if kind != NO_POOL else (A, B)
+    per = N * A * B
+    rng = np.random.default_rng(Cn * 7 + A + act + kind)
+    zhat = rng.standard_normal(Cn * per).astype(np.float32)
+    zact = oracle64.activation_forward(act, zhat.astype(np.float64)).astype(np.float32)
+    var = (0.5 + rng.random(Cn)).astype(np.float32)
+    d = rng.standard_normal(Cn * N * oA * oB).astype(np.float32)
+    pz, pa, pd, pv = dev.upload(zhat), dev.upload(zact), dev.upload(d), dev.upload(var)
+    dxp, dxa, dxb, bias = dev.zeros(zhat.size), dev.zeros(zhat.size), dev.zeros(zhat.size), dev.zeros(Cn)
+    ws, nb = bn_ws(dev, Cn, per)
+    ok(hip.fitre_hip_pool_act_bn_backward(kind, act, pd, pz, None if derive else pa, pv, Cn, N, A, B, k, s, p, oA, oB, 1e-5,
+                                          dxp, dxa, dxb, bias, ws, nb))
+    if kind == NO_POOL:
+        wantp = d.astype(np.float64)
+    else:
+        wantp = oracle64.pool_backward(kind, d, zact, N, Cn, B, A, k, s, p)
+    wanta = oracle64.activation_backward(act, wantp, zhat.astype(np.float64), zact.astype(np.float64))
+    gotp, gota, gotb = (dev.download(b, zhat.size) for b in (dxp, dxa, dxb))
+    assert rel_err(gotp, wantp) < 1e-6
+    if kind == MAX_POOL:
+        np.testing.assert_array_equal(gotp != 0, wantp != 0)  # the routing is exact
+    assert rel_err(gota, wanta) < 1e-5
+    # batch-norm step on the gradient the device itself wrote (isolates it from rounding of the first two)
+    wantb = oracle64.batch_norm_backward(gota, zhat, var, B, A, Cn, N)
+    assert rel_err(gotb, wantb) < TOL
+    np.testing.assert_allclose(dev.download(bias, Cn), gotb.astype(np.float64).reshape(Cn, per).sum(1),
+                               atol=1e-5 * np.abs(gotb).max() * np.sqrt(per) + 1e-7)
+    for b in (pz, pa, pd, pv, dxp, dxa, dxb, bias, ws):
+        dev.free(b)
+
+
+def test_fused_backward_rejects_missing_activation_output(dev):
+    p = dev.zeros(256)
+    ws, nb = bn_ws(dev, 1, 64)
+    assert hip.fitre_hip_pool_act_bn_backward(NO_POOL, CNN_ACT_SWISH, p, p, None, p, 1, 1, 8, 8, 1, 1, 0, 8, 8, 1e-5, p, p, p, None, ws, nb) == 2
+    assert b"ReLU only" in hip.fitre_hip_last_error()
+
+
 def test_workspace_too_small_is_reported(dev):
     p = dev.zeros(4096)
     assert hip.fitre_hip_batch_norm_backward(p, p, p, 4, 1024, 1e-5, p, None, p, 8) == 4
