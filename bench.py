@@ -160,55 +160,52 @@ def gpu_leg(args):
 
 
 def bandwidth_leg(L, dev, batch, reps=20):
-    """The bandwidth-bound backward kernels run alone at the shapes of the two largest layers
-    (64 x 32x32 and 128 x 16x16 maps per image, max-pool 2, ReLU, batch norm): algorithmic bytes / time
-    against the 8 TB/s HBM peak, with a plain copy of the same tensor beside them.  Inside the backward
-    pass the per-class averages of `kernels` are dominated by the small layers' launches; the tensors here
-    are the ones that carry the bytes.  The same buffers are used by every repeat, so part of the traffic
-    is served by the memory-side cache, as it is in the pass itself (a layer's delta is read right after
-    it is written)."""
+    """The bandwidth-bound backward step of a layer (max-pool 2 + ReLU + batch norm, the entry point
+    cnnBackward calls) run alone at the shapes of the two largest layers, 64 x 32x32 and 128 x 16x16 maps
+    per image: algorithmic bytes / kernel time against the 8 TB/s HBM peak, per-launch events as in
+    `kernels`, with a plain copy of the same tensor beside it.  Inside the backward pass the per-class
+    averages of `kernels` are dominated by the small layers' launches; the tensors here are the ones
+    that carry the bytes.  The same buffers are used by every repeat, so part of the traffic is served
+    by the memory-side cache, as it is in the pass itself (a layer's delta is read right after it is
+    written)."""
     hip = L.hip
-    ev0, ev1 = C.c_void_p(), C.c_void_p()
-    L.check(hip.fitre_hip_event_create(C.byref(ev0)))
-    L.check(hip.fitre_hip_event_create(C.byref(ev1)))
-
-    def timed(fn):
-        L.check(fn())
-        L.check(fn())
-        dev.sync()
-        L.check(hip.fitre_hip_event_record(ev0))
-        for _ in range(reps):
-            L.check(fn())
-        L.check(hip.fitre_hip_event_record(ev1))
-        dev.sync()
-        ms = C.c_float()
-        L.check(hip.fitre_hip_event_elapsed_ms(ev0, ev1, C.byref(ms)))
-        return ms.value / reps * 1e-3
-
     rng = np.random.default_rng(0xF17E0004)
-    relu = 13  # CNN_ACT_RELU
+    relu, max_pool = 13, 0  # CNN_ACT_RELU, MAX_POOL
     out = {}
     for name, channels, hw in (("layer0_64x32x32", 64, 32), ("layer1_128x16x16", 128, 16)):
         per = batch * hw * hw
         n = channels * per
         zhat = dev.upload(rng.standard_normal(n).astype(np.float32))
-        zact = dev.zeros(n)
-        L.check(hip.fitre_hip_activation_forward(relu, zhat, zact, n))
         var = dev.upload(np.ones(channels, np.float32))
         dpool, dact, dbn, bias = dev.zeros(n), dev.zeros(n), dev.zeros(n), dev.zeros(channels)
         delta = dev.upload(rng.standard_normal(n // 4).astype(np.float32))
         nb = hip.fitre_hip_batch_norm_workspace(channels, per)
         ws = dev.alloc(nb)
-        t_copy = timed(lambda: hip.fitre_hip_copy(n, zhat, dbn))
-        t_pool = timed(lambda: hip.fitre_hip_pool_act_backward(0, relu, delta, zhat, zact, channels, batch, hw, hw, 2, 2,
-                                                               0, hw // 2, hw // 2, dpool, dact))
-        t_bn = timed(lambda: hip.fitre_hip_batch_norm_backward(dact, zhat, var, channels, per, 1e-5, dbn, bias, ws, nb))
-        rows = dict(copy=(8.0 * n, t_copy),                 # read + write
-                    pool_act_bwd=(4.0 * (n / 4 + 3 * n), t_pool),  # delta (pooled), z_act read; two gradients written
-                    bn_bwd=(12.0 * n, t_bn))                # delta, zhat read once; dx written (the kernel pair moves 20 B)
-        out[name] = {k: dict(us=round(t * 1e6, 2), achieved=round(b / t / 1e9, 1), unit="GB/s",
-                             frac=round(b / t / 1e9 / PEAK_HBM_GBS, 4)) for k, (b, t) in rows.items()}
-        for p in (zhat, zact, var, dpool, dact, dbn, bias, delta, ws):
+
+        def step():
+            L.check(hip.fitre_hip_pool_act_bn_backward(max_pool, relu, delta, zhat, None, var, channels, batch, hw, hw, 2, 2, 0,
+                                                       hw // 2, hw // 2, 1e-5, dpool, dact, dbn, bias, ws, nb))
+            L.check(hip.fitre_hip_copy(n, zhat, dbn))
+
+        step()
+        dev.sync()
+        L.check(hip.fitre_hip_profile_enable(1))
+        for _ in range(reps):
+            step()
+        dev.sync()
+        L.check(hip.fitre_hip_profile_enable(0))
+        rows = {r["cls"]: r for r in read_profile(L)}
+        # pool_act_bwd: delta (pooled) and zhat read, two gradients written; bn_bwd: gradient and zhat read,
+        # result written; blas1: the copy, read + write
+        want = dict(pool_act_bwd=4.0 * (n / 4 + 3 * n), bn_bwd=12.0 * n + 8.0 * channels, blas1=8.0 * n)
+        entry = {}
+        for cls, nbytes in want.items():
+            r = rows[cls]
+            t = r["ms"] * 1e-3 / r["launches"]
+            entry["copy" if cls == "blas1" else cls] = dict(us=round(t * 1e6, 2), achieved=round(nbytes / t / 1e9, 1), unit="GB/s",
+                                                            frac=round(nbytes / t / 1e9 / PEAK_HBM_GBS, 4))
+        out[name] = entry
+        for p in (zhat, var, dpool, dact, dbn, bias, delta, ws):
             dev.free(p)
     return out
 

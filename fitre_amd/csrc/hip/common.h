@@ -158,6 +158,33 @@ __device__ __forceinline__ T block_sum(T v, T *lds)
 	return total;
 }
 
+// Three sums at once (two barriers instead of six); every thread gets the totals.
+// lds must hold 3 * BLOCK/64 values of T.
+template <int BLOCK, typename T>
+__device__ __forceinline__ void block_sum3(T &a, T &b, T &c, T *lds)
+{
+	constexpr int WAVES = BLOCK / kWave;
+	a = wave_sum(a);
+	b = wave_sum(b);
+	c = wave_sum(c);
+	if constexpr (WAVES == 1) return;
+	const int wave = threadIdx.x / kWave;
+	__syncthreads();
+	if ((threadIdx.x % kWave) == 0) {
+		lds[3 * wave] = a;
+		lds[3 * wave + 1] = b;
+		lds[3 * wave + 2] = c;
+	}
+	__syncthreads();
+	a = lds[0], b = lds[1], c = lds[2];
+#pragma unroll
+	for (int w = 1; w < WAVES; w++) {
+		a += lds[3 * w];
+		b += lds[3 * w + 1];
+		c += lds[3 * w + 2];
+	}
+}
+
 inline unsigned blocks_for(long n, int perBlock, unsigned cap = 1u << 20)
 {
 	long b = (n + perBlock - 1) / perBlock;

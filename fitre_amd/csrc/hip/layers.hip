@@ -442,36 +442,53 @@ __global__ void __launch_bounds__(kRedBlock)
 bn_backward_apply_kernel(const float *delta, const float *zhat, const float *variance, const double *partial,
                          int segmentsIn, float epsilon, long perChannel, float *out, float *biasGrad)
 {
+	__shared__ double lds[3 * kRedBlock / kWave];
 	const int c = blockIdx.y;
-	double d1 = 0.0, d2 = 0.0, d3 = 0.0;
-	for (int k = 0; k < segmentsIn; k++) {
-		const double *slot = partial + ((size_t)c * segmentsIn + k) * 4;
-		d1 += slot[0], d2 += slot[1], d3 += slot[2];
-	}
-	const float m = (float)perChannel;
-	const float sum1 = (float)d1, sum2 = (float)d2;
-	const float scale = 1.f / (m * sqrtf(epsilon + variance[c]));
-	if (biasGrad && blockIdx.x == 0 && threadIdx.x == 0) biasGrad[c] = (float)(-d2 * d3 * (double)scale);
 	const float *pd = delta + (size_t)c * perChannel;
 	const float *pz = zhat + (size_t)c * perChannel;
 	float *po = out + (size_t)c * perChannel;
 	long lo, hi;
 	segment_range(perChannel, lo, hi);
+	// the first group's loads are in flight while the segment sums are combined
+	long i = lo + 4 * (long)threadIdx.x;
+	float4 d = make_float4(0.f, 0.f, 0.f, 0.f), z = d;
 	if constexpr (VEC) {
-		for (long i = lo + 4 * (long)threadIdx.x; i + 3 < hi; i += 4 * kRedBlock) {
-			float4 d = *reinterpret_cast<const float4 *>(pd + i);
-			float4 z = *reinterpret_cast<const float4 *>(pz + i);
+		if (i + 3 < hi) {
+			d = *reinterpret_cast<const float4 *>(pd + i);
+			z = *reinterpret_cast<const float4 *>(pz + i);
+		}
+	}
+	double a1 = 0.0, a2 = 0.0, a3 = 0.0;
+	for (int k = threadIdx.x; k < segmentsIn; k += kRedBlock) {
+		const double *slot = partial + ((size_t)c * segmentsIn + k) * 4;
+		a1 += slot[0], a2 += slot[1], a3 += slot[2];
+	}
+	block_sum3<kRedBlock>(a1, a2, a3, lds);
+	const double d1 = a1, d2 = a2, d3 = a3;
+	const float m = (float)perChannel;
+	const float sum1 = (float)d1, sum2 = (float)d2;
+	const float scale = 1.f / (m * sqrtf(epsilon + variance[c]));
+	if (biasGrad && blockIdx.x == 0 && threadIdx.x == 0) biasGrad[c] = (float)(-d2 * d3 * (double)scale);
+	if constexpr (VEC) {
+		while (i + 3 < hi) {
+			const long next = i + 4 * kRedBlock;
+			float4 dn = d, zn = z;
+			if (next + 3 < hi) {
+				dn = *reinterpret_cast<const float4 *>(pd + next);
+				zn = *reinterpret_cast<const float4 *>(pz + next);
+			}
 			float4 r;
 			r.x = bn_backward_value(m, d.x, z.x, sum1, sum2, scale);
 			r.y = bn_backward_value(m, d.y, z.y, sum1, sum2, scale);
 			r.z = bn_backward_value(m, d.z, z.z, sum1, sum2, scale);
 			r.w = bn_backward_value(m, d.w, z.w, sum1, sum2, scale);
 			*reinterpret_cast<float4 *>(po + i) = r;
+			d = dn, z = zn, i = next;
 		}
 		long tail = lo + ((hi - lo) / 4) * 4;
-		for (long i = tail + threadIdx.x; i < hi; i += kRedBlock) po[i] = bn_backward_value(m, pd[i], pz[i], sum1, sum2, scale);
+		for (long t = tail + threadIdx.x; t < hi; t += kRedBlock) po[t] = bn_backward_value(m, pd[t], pz[t], sum1, sum2, scale);
 	} else {
-		for (long i = lo + threadIdx.x; i < hi; i += kRedBlock) po[i] = bn_backward_value(m, pd[i], pz[i], sum1, sum2, scale);
+		for (long t = lo + threadIdx.x; t < hi; t += kRedBlock) po[t] = bn_backward_value(m, pd[t], pz[t], sum1, sum2, scale);
 	}
 }
 
@@ -547,8 +564,9 @@ __device__ __forceinline__ float4 relu4(float4 v)
 }
 __device__ __forceinline__ void bn_sums4(float4 g, float4 z, double &s1, double &s2, double &s3)
 {
+	// four terms in float, the running sums in double
 	s1 += (double)((g.x + g.y) + (g.z + g.w));
-	s2 += (double)(g.x * z.x) + (double)(g.y * z.y) + (double)(g.z * z.z) + (double)(g.w * z.w);
+	s2 += (double)((g.x * z.x + g.y * z.y) + (g.z * z.z + g.w * z.w));
 	s3 += (double)((z.x + z.y) + (z.z + z.w));
 }
 // routes the two pooled gradients d of a 2 x 4 patch (rows r0, r1 of the pool input) to the window maxima
@@ -590,7 +608,7 @@ __global__ void __launch_bounds__(kRedBlock)
 pool_act_sums_kernel(const float *delta, const float *zhat, const float *z_act, int inA, int inB, int samples, int actFun,
                      float *dxPool, float *dxAct, double *partial)
 {
-	__shared__ double lds[kRedBlock / kWave];
+	__shared__ double lds[3 * kRedBlock / kWave];
 	const int c = blockIdx.y;
 	const long perChannel = (long)samples * inA * inB;
 	const size_t base = (size_t)c * perChannel;
@@ -642,12 +660,10 @@ pool_act_sums_kernel(const float *delta, const float *zhat, const float *z_act, 
 			bn_sums4(g1, i1, s1, s2, s3);
 		}
 	}
-	const double t1 = block_sum<kRedBlock>(s1, lds);
-	const double t2 = block_sum<kRedBlock>(s2, lds);
-	const double t3 = block_sum<kRedBlock>(s3, lds);
+	block_sum3<kRedBlock>(s1, s2, s3, lds);
 	if (threadIdx.x == 0) {
 		double *slot = partial + ((size_t)c * gridDim.x + blockIdx.x) * 4;
-		slot[0] = t1, slot[1] = t2, slot[2] = t3;
+		slot[0] = s1, slot[1] = s2, slot[2] = s3;
 	}
 }
 
@@ -658,7 +674,7 @@ __global__ void __launch_bounds__(kRedBlock)
 pool_act_bn_small_kernel(const float *delta, const float *zhat, const float *z_act, const float *variance, int inA, int inB,
                          int samples, int actFun, float epsilon, float *dxPool, float *dxAct, float *dxBn, float *biasGrad)
 {
-	__shared__ double lds[kRedBlock / kWave];
+	__shared__ double lds[3 * kRedBlock / kWave];
 	constexpr int G = (int)(kBnSmallChannel / (4 * kRedBlock)); // 16-byte groups per thread
 	static_assert(G >= 2 && G % 2 == 0, "a 2 x 4 patch is two groups");
 	const int c = blockIdx.x;
@@ -717,9 +733,8 @@ pool_act_bn_small_kernel(const float *delta, const float *zhat, const float *z_a
 			bn_sums4(g[2 * k + 1], z[2 * k + 1], s1, s2, s3);
 		}
 	}
-	const double d1 = block_sum<kRedBlock>(s1, lds);
-	const double d2 = block_sum<kRedBlock>(s2, lds);
-	const double d3 = block_sum<kRedBlock>(s3, lds);
+	block_sum3<kRedBlock>(s1, s2, s3, lds);
+	const double d1 = s1, d2 = s2, d3 = s3;
 	const float m = (float)perChannel;
 	const float sum1 = (float)d1, sum2 = (float)d2;
 	const float scale = 1.f / (m * sqrtf(epsilon + variance[c]));
