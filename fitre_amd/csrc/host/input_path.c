@@ -1,0 +1,106 @@
+/* Mini-batch selection and augmentation with the reference's names (utilities/sample_matrix.cu,
+ * solvers/kfac_da.cu, augmentation/dev_crop.cu, dev_flip.cu, dev_normalize.cu) over the device layer. */
+#include <stdio.h>
+#include <stdlib.h>
+
+#include "fitre_hip.h"
+#include "fitre_input.h"
+#include "fitre_shim.h"
+
+#define HIP_CALL(expr)                                                                       \
+	do {                                                                                     \
+		int rc_ = (expr);                                                                    \
+		if (rc_ != 0) {                                                                      \
+			fprintf(stderr, "%s:%d: %s\n  %s\n", __FILE__, __LINE__, #expr, fitre_hip_last_error()); \
+			exit(-1);                                                                        \
+		}                                                                                    \
+	} while (0)
+
+/* augmentation/dev_normalize.cu:55-62 */
+static void dataset_statistics(DATASET_TYPE datasetType, const real **mean, const real **std)
+{
+	static const real mean_cifar10[3] = { 0.4914f, 0.4822f, 0.4465f }, std_cifar10[3] = { 0.2470f, 0.2435f, 0.2616f };
+	static const real mean_cifar100[3] = { 0.5071f, 0.4865f, 0.4409f }, std_cifar100[3] = { 0.2673f, 0.2564f, 0.2762f };
+	static const real mean_imagenet[3] = { 0.4799f, 0.4478f, 0.3972f }, std_imagenet[3] = { 0.2769f, 0.2690f, 0.2820f };
+	switch (datasetType) {
+	case CIFAR10: *mean = mean_cifar10, *std = std_cifar10; break;
+	case CIFAR100: *mean = mean_cifar100, *std = std_cifar100; break;
+	case IMAGENET: *mean = mean_imagenet, *std = std_imagenet; break;
+	default: fprintf(stderr, "Unknown DatasetType here... \n\n"); exit(-1);
+	}
+}
+
+static void need_three_channels(const char *fn, int channels)
+{
+	if (channels != 3) {
+		fprintf(stderr, "%s: the data-set statistics cover 3 channels, the images have %d\n", fn, channels);
+		exit(-1);
+	}
+}
+
+void selectColumnMatrix(DEVICE_DATASET *data, int sampleSize, int *indices, int offset)
+{
+	HIP_CALL(fitre_hip_extract_columns(data->sampledTrainX, data->trainSetX, indices + offset, data->features, sampleSize));
+	HIP_CALL(fitre_hip_extract_columns(data->sampledTrainY, data->trainSetY, indices + offset, 1, sampleSize));
+	HIP_CALL(fitre_hip_sync());
+}
+
+void randomCrop(real *input, int samples, int height, int width, int channels, int padding, real *output, real *devPtr,
+                real *hostPtr, real defaultValue, real *probs)
+{
+	(void)hostPtr;
+	(void)probs;
+	getRandomVector(2 * samples, NULL, devPtr, RAND_UNIFORM);
+	HIP_CALL(fitre_hip_augment_batch(input, 0, samples, channels, height, width, devPtr, padding, defaultValue, NULL, NULL, NULL,
+	                                 1.f, output));
+	HIP_CALL(fitre_hip_sync());
+}
+
+void flipData(real *input, real *output, int samples, int channels, int height, int width, real *probs, real *devPtr,
+              real *hostPtr)
+{
+	(void)devPtr;
+	(void)hostPtr;
+	HIP_CALL(fitre_hip_augment_batch(input, 0, samples, channels, height, width, NULL, 0, 0.f, probs, NULL, NULL, 1.f, output));
+	HIP_CALL(fitre_hip_sync());
+}
+
+void normalizeCIFAR10(real *input, int samples, int channels, int height, int width, real *devPtr, real *hostPtr,
+                      DATASET_TYPE datasetType)
+{
+	(void)devPtr;
+	(void)hostPtr;
+	const real *mean, *std;
+	dataset_statistics(datasetType, &mean, &std);
+	need_three_channels("normalizeCIFAR10", channels);
+	HIP_CALL(fitre_hip_augment_batch(input, 0, samples, channels, height, width, NULL, 0, 0.f, NULL, mean, std, 255.f, input));
+	HIP_CALL(fitre_hip_sync());
+}
+
+void augmentData(CNN_MODEL *model, DEVICE_DATASET *data, int offset, int currentBatchSize, real *devPtr, real *hostPtr,
+                 int enableDA, DATASET_TYPE datasetType)
+{
+	(void)offset;
+	(void)hostPtr;
+	const CONV_LAYER *c = &model->convLayer[0];
+	const int channels = c->inChannels, height = c->height, width = c->width, samples = currentBatchSize;
+	real *first = data->sampledTrainX;
+	real *second = first + (size_t)samples * channels * height * width;
+	const real *mean, *std;
+	dataset_statistics(datasetType, &mean, &std);
+	need_three_channels("augmentData", channels);
+
+	const real *cropUniforms = NULL, *flipUniforms = NULL;
+	if (enableDA >= 1) {
+		/* the draws of the reference, in its order: one vector it never reads, the crop offsets, the flips */
+		getRandomVector(samples, NULL, devPtr, RAND_UNIFORM);
+		getRandomVector(2 * samples, NULL, devPtr + samples, RAND_UNIFORM);
+		getRandomVector(samples, NULL, devPtr, RAND_UNIFORM);
+		cropUniforms = devPtr + samples;
+		flipUniforms = devPtr;
+	}
+	HIP_CALL(fitre_hip_augment_batch(first, 1, samples, channels, height, width, cropUniforms, 4, 0.f, flipUniforms, mean, std,
+	                                 255.f, second));
+	HIP_CALL(fitre_hip_sync());
+	data->currentBatch = second;
+}

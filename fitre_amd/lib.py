@@ -69,6 +69,10 @@ HIP_API = {
     "fitre_hip_max_pool_argmax": (i32, [vp] + [i32] * 9 + [vp]),
     "fitre_hip_pool_act_backward": (i32, [i32, i32, vp, vp, vp] + [i32] * 9 + [vp, vp]),
     "fitre_hip_pool_act_bn_backward": (i32, [i32, i32, vp, vp, vp, vp] + [i32] * 9 + [f32, vp, vp, vp, vp, vp, sz]),
+    "fitre_hip_extract_columns": (i32, [vp, vp, vp, i32, i32]),
+    "fitre_hip_augment_batch": (i32, [vp, i32, i32, i32, i32, i32, vp, i32, f32, vp, vp, vp, f32, vp]),
+    "fitre_hip_crop_shifts": (i32, [vp, i32, i32, vp]),
+    "fitre_hip_shift_images": (i32, [vp, i32, i32, i32, i32, vp, vp, f32, vp]),
     "fitre_hip_batch_norm_workspace": (sz, [i32, lng]),
     "fitre_hip_batch_norm_forward": (i32, [vp, i32, lng, vp, vp, vp, vp, vp, f32, f32, i32, vp, sz]),
     "fitre_hip_batch_norm_backward": (i32, [vp, vp, vp, i32, lng, f32, vp, vp, vp, sz]),
@@ -140,6 +144,12 @@ CNN_API = {
     "getRandomVector": (None, [i32, vp, vp, i32]),
     "writeVector": (None, [vp, i32, C.c_char_p, i32, vp]),
     "readVector": (i32, [vp, i32, C.c_char_p, i32, vp]),
+    # include/fitre_input.h
+    "selectColumnMatrix": (None, [pdata, i32, vp, i32]),
+    "randomCrop": (None, [vp, i32, i32, i32, i32, i32, vp, vp, vp, f32, vp]),
+    "flipData": (None, [vp, vp, i32, i32, i32, i32, vp, vp, vp]),
+    "normalizeCIFAR10": (None, [vp, i32, i32, i32, i32, vp, vp, i32]),
+    "augmentData": (None, [pmodel, pdata, i32, i32, vp, vp, i32, i32]),
     # include/fitre_kfac.h
     "computeKFACStorageIndices": (None, [pmodel, pkfac]),
     "kfacFactorsMemRequired": (lng, [pmodel, i32]),

@@ -211,6 +211,27 @@ int fitre_hip_pool_act_bn_backward(int poolType, int actFun, const float *delta,
                                    float epsilon, float *dxPool, float *dxAct, float *dxBn, float *biasGrad,
                                    void *ws, size_t wsBytes);
 
+/* ---------------- mini-batch selection and augmentation ---------------- */
+/* tgt column j = src column indices[j], columns of `rows` values (kerExtractColumns,
+ * device/extract_columns.cu:8-20).  indices is a device array. */
+int fitre_hip_extract_columns(float *tgt, const float *src, const int *indices, int rows, int columns);
+/* The layer-0 input in one pass: out[c][n][col][row] (height = rows, fastest) gathered from `sampled`,
+ * which is [samples][channels][cells] when sampleMajor (reshapeMatrix of solvers/kfac_da.cu:37) or already
+ * channel-major; cropUniforms (2*samples device values in (0, 1], row shifts then column shifts, or NULL):
+ * shift by trunc(100 u) mod (2 padding + 1) - padding, cells from outside read `fill`
+ * (augmentation/dev_crop.cu:10-58); flipUniforms (samples values or NULL): below 0.5 the image is mirrored
+ * along the width axis (dev_flip.cu:68-104; the crop applies to the unflipped image, as in the reference's
+ * order); mean/stdv (HOST arrays of `channels` values, or NULL): x = (x / scale - mean[c]) / stdv[c]
+ * (dev_normalize.cu:12-36), applied to filled cells too.  In place only for the normalisation alone. */
+int fitre_hip_augment_batch(const float *sampled, int sampleMajor, int samples, int channels, int height,
+                            int width, const float *cropUniforms, int padding, float fill,
+                            const float *flipUniforms, const float *mean, const float *stdv, float scale,
+                            float *out);
+/* the two kernels of randomCrop on their own (dev_crop.cu:52-58 and 10-50, channel-major images) */
+int fitre_hip_crop_shifts(const float *uniforms, int count, int padding, int *shifts);
+int fitre_hip_shift_images(const float *in, int samples, int channels, int height, int width,
+                           const int *shiftRow, const int *shiftCol, float fill, float *out);
+
 /* ---------------- reductions ---------------- */
 /* out[c] = sum of the perChannel contiguous values of channel c (conv bias gradient,
  * functions/cnn_backward.cu:662-689). */

@@ -1534,4 +1534,91 @@ int oracle_cnn_hv(const CNN_MODEL *model, const real *weights, const real *x, co
 	return rc;
 }
 
+/* ------------------------------------------------------------------ */
+/* Input pipeline: batch selection and augmentation                    */
+/* ------------------------------------------------------------------ */
+
+/* device/extract_columns.cu:8-20 (kerExtractColumns): column j of tgt is column indices[j] of src,
+ * columns of `rows` values. */
+void oracle_extract_columns(real *tgt, const real *src, const int *indices, int rows, long numElements)
+{
+	for (long j = 0; j < numElements; j++) {
+		long colId = j / rows, rowId = j % rows;
+		tgt[j] = src[(size_t)indices[colId] * rows + rowId];
+	}
+}
+
+/* augmentation/dev_crop.cu:52-58 (ker_convert): uniform in [0, 1) -> shift in [-padding, padding].
+ * The first `samples` values are the row shifts, the next `samples` the column shifts. */
+void oracle_crop_shifts(const real *uniforms, int samples, int padding, int *shifts)
+{
+	for (int i = 0; i < 2 * samples; i++) shifts[i] = (int)((double)uniforms[i] * 100.) % (2 * padding + 1) - padding;
+}
+
+/* augmentation/dev_crop.cu:10-50 (ker_random_crop) on [channels][samples][width][height] (height fastest):
+ * every image is shifted by (shiftRow, shiftCol); cells that leave the image read defaultVal. */
+void oracle_random_crop(const real *input, int samples, int height, int width, int channels, const int *shiftRow,
+                        const int *shiftCol, real defaultVal, real *output)
+{
+	for (int imgIdx = 0; imgIdx < samples; imgIdx++)
+		for (int idx = 0; idx < height * width * channels; idx++) {
+			int chId = idx / (height * width), chIdx = idx % (height * width);
+			int row = chIdx % height, col = chIdx / height;
+			int cRow = shiftRow[imgIdx], cCol = shiftCol[imgIdx];
+			real val;
+			if (cRow + row < 0 || cCol + col < 0 || cRow + row >= height || cCol + col >= width) val = defaultVal;
+			else val = input[(size_t)chId * samples * height * width + (size_t)imgIdx * height * width +
+				             (size_t)(col + cCol) * height + (row + cRow)];
+			output[(size_t)chId * samples * height * width + (size_t)imgIdx * height * width + (size_t)col * height + row] = val;
+		}
+}
+
+/* augmentation/dev_flip.cu:68-104 (ker_random_flip): images with probs < 0.5 are mirrored along the
+ * width (column) axis, the others copied.  (The reference splits the cell index by `width` where the
+ * layout needs `height`; the two agree on the square images it is used on, and the layout's own split
+ * is restated here.) */
+void oracle_random_flip(const real *input, int samples, int channels, int height, int width, const real *probs, real *output)
+{
+	for (int imgIdx = 0; imgIdx < samples; imgIdx++)
+		for (int idx = 0; idx < height * width * channels; idx++) {
+			int chId = idx / (height * width), chIdx = idx % (height * width);
+			int row = chIdx % height, col = chIdx / height;
+			size_t base = (size_t)chId * samples * height * width + (size_t)imgIdx * height * width;
+			size_t src = base + (size_t)col * height + row, tgt = src;
+			if (probs[imgIdx] < 0.5) tgt = base + (size_t)(width - 1 - col) * height + row;
+			output[tgt] = input[src];
+		}
+}
+
+/* augmentation/dev_normalize.cu:12-36 (ker_normalize): x = (x / nrConstant - mean[c]) / std[c], in place. */
+void oracle_normalize(real *input, int samples, int height, int width, int channels, const real *means, const real *std,
+                      real nrConstant)
+{
+	for (int c = 0; c < channels; c++)
+		for (size_t i = 0; i < (size_t)samples * height * width; i++) {
+			real *x = input + (size_t)c * samples * height * width + i;
+			*x /= nrConstant;
+			*x = (*x - means[c]) / std[c];
+		}
+}
+
+/* solvers/kfac_da.cu:22-89 (augmentData) given the uniforms it would draw: [samples][channels][cells] ->
+ * [channels][samples][cells] (reshapeMatrix), then with enableDA crop by at most 4 cells (fill 0) and
+ * flip, then the data set's normalisation with the pixel scale 255.  cropUniforms: 2*samples values,
+ * flipUniforms: samples values.  scratch holds one batch. */
+void oracle_augment_data(const real *sampled, int samples, int channels, int height, int width, int enableDA,
+                         const real *cropUniforms, const real *flipUniforms, const real *means, const real *std,
+                         real *scratch, real *output)
+{
+	oracle_reshape(sampled, samples, channels, height * width, output);
+	if (enableDA >= 1) {
+		int *shifts = (int *)malloc(sizeof(int) * 2 * (size_t)samples);
+		oracle_crop_shifts(cropUniforms, samples, 4, shifts);
+		oracle_random_crop(output, samples, height, width, channels, shifts, shifts + samples, 0, scratch);
+		oracle_random_flip(scratch, samples, channels, height, width, flipUniforms, output);
+		free(shifts);
+	}
+	oracle_normalize(output, samples, height, width, channels, means, std, 255.);
+}
+
 int oracle_sizeof_real(void) { return (int)sizeof(real); }

@@ -325,3 +325,46 @@ class Oracle:
         out = self.zeros(x.size)
         (self.lib.oracle_transpose_rc if rc else self.lib.oracle_transpose)(self.p(x), maps, height, width, self.p(out))
         return out
+
+    # ---- input pipeline
+    def extract_columns(self, src, indices, rows):
+        src = self.arr(src)
+        idx = np.ascontiguousarray(indices, dtype=np.int32)
+        out = self.zeros(rows * idx.size)
+        self.lib.oracle_extract_columns(self.p(out), self.p(src), idx.ctypes.data_as(C.c_void_p), rows, C.c_long(rows * idx.size))
+        return out
+
+    def crop_shifts(self, uniforms, samples, padding):
+        u = self.arr(uniforms)
+        out = np.zeros(2 * samples, dtype=np.int32)
+        self.lib.oracle_crop_shifts(self.p(u), samples, padding, out.ctypes.data_as(C.c_void_p))
+        return out
+
+    def random_crop(self, x, samples, height, width, channels, shift_row, shift_col, default=0.0):
+        x = self.arr(x)
+        sr = np.ascontiguousarray(shift_row, dtype=np.int32)
+        sc = np.ascontiguousarray(shift_col, dtype=np.int32)
+        out = self.zeros(x.size)
+        self.lib.oracle_random_crop(self.p(x), samples, height, width, channels, sr.ctypes.data_as(C.c_void_p),
+                                    sc.ctypes.data_as(C.c_void_p), self.r(default), self.p(out))
+        return out
+
+    def random_flip(self, x, samples, channels, height, width, probs):
+        x, probs = self.arr(x), self.arr(probs)
+        out = self.zeros(x.size)
+        self.lib.oracle_random_flip(self.p(x), samples, channels, height, width, self.p(probs), self.p(out))
+        return out
+
+    def normalize(self, x, samples, height, width, channels, means, std, scale=255.0):
+        x = self.arr(x).copy()
+        means, std = self.arr(means), self.arr(std)
+        self.lib.oracle_normalize(self.p(x), samples, height, width, channels, self.p(means), self.p(std), self.r(scale))
+        return x
+
+    def augment_data(self, sampled, samples, channels, height, width, enable, crop_uniforms, flip_uniforms, means, std):
+        sampled = self.arr(sampled)
+        cu, fu, means, std = self.arr(crop_uniforms), self.arr(flip_uniforms), self.arr(means), self.arr(std)
+        scratch, out = self.zeros(sampled.size), self.zeros(sampled.size)
+        self.lib.oracle_augment_data(self.p(sampled), samples, channels, height, width, int(enable), self.p(cu), self.p(fu),
+                                     self.p(means), self.p(std), self.p(scratch), self.p(out))
+        return out

@@ -470,3 +470,94 @@ def test_uniform_stream_known_values_and_statistics(oracle64):
     # continuing the stream equals one long draw
     np.testing.assert_array_equal(np.concatenate([oracle64.uniform_stream(7, 0, 10), oracle64.uniform_stream(7, 10, 6)]),
                                   oracle64.uniform_stream(7, 0, 16))
+
+
+# ------------------------------------------------------------------ input pipeline
+def _images(rng, C, N, W, H):
+    """[C][N][W][H] flat (H fastest) and the same data as an array indexed [c][n][col][row]."""
+    x = rng.integers(0, 256, size=C * N * W * H).astype(np.float64)
+    return x, x.reshape(C, N, W, H)
+
+
+def test_extract_columns_is_fancy_indexing(oracle64):
+    rng = np.random.default_rng(3)
+    rows, cols = 7, 20
+    src = rng.standard_normal(rows * cols)
+    idx = rng.integers(0, cols, size=9)
+    want = src.reshape(cols, rows)[idx].reshape(-1)   # column-major features x columns: column j is a contiguous run
+    np.testing.assert_array_equal(oracle64.extract_columns(src, idx, rows), want)
+
+
+def test_crop_shifts_known_values(oracle64):
+    # trunc(u * 100) mod 9 - 4 for padding 4 (augmentation/dev_crop.cu:57)
+    u = [0.0, 0.004, 0.01, 0.37, 0.44, 0.45, 0.99, 0.089999]
+    want = [-4, -4, -3, 37 % 9 - 4, 44 % 9 - 4, 45 % 9 - 4, 99 % 9 - 4, 8 % 9 - 4]
+    np.testing.assert_array_equal(oracle64.crop_shifts(u, 4, 4), want)
+    rng = np.random.default_rng(0)
+    s = oracle64.crop_shifts(rng.random(2000), 1000, 4)
+    assert s.min() == -4 and s.max() == 4
+    # padding 2: values in [-2, 2]
+    s2 = oracle64.crop_shifts(rng.random(2000), 1000, 2)
+    assert s2.min() == -2 and s2.max() == 2
+
+
+def test_random_crop_is_a_zero_filled_shift(oracle64):
+    rng = np.random.default_rng(5)
+    C, N, W, H = 3, 6, 5, 7   # rectangular: a swapped axis would show
+    x, img = _images(rng, C, N, W, H)
+    sr = np.array([0, 2, -3, 4, -1, 6])
+    sc = np.array([0, -1, 2, 0, 4, -4])
+    got = oracle64.random_crop(x, N, H, W, C, sr, sc, default=-9.0).reshape(C, N, W, H)
+    for n in range(N):
+        # out[col][row] = in[col + sc][row + sr]: pad by the largest shift, then slice
+        P = 8
+        padded = np.pad(img[:, n], ((0, 0), (P, P), (P, P)), constant_values=-9.0)
+        want = padded[:, P + sc[n]:P + sc[n] + W, P + sr[n]:P + sr[n] + H]
+        np.testing.assert_array_equal(got[:, n], want)
+    # zero shift is the identity
+    np.testing.assert_array_equal(oracle64.random_crop(x, N, H, W, C, np.zeros(N), np.zeros(N)), x)
+
+
+def test_random_flip_mirrors_the_column_axis(oracle64):
+    rng = np.random.default_rng(6)
+    C, N, W, H = 2, 5, 6, 4
+    x, img = _images(rng, C, N, W, H)
+    probs = np.array([0.1, 0.5, 0.49999, 0.9, 0.0])
+    got = oracle64.random_flip(x, N, C, H, W, probs).reshape(C, N, W, H)
+    for n in range(N):
+        want = np.flip(img[:, n], axis=1) if probs[n] < 0.5 else img[:, n]
+        np.testing.assert_array_equal(got[:, n], want)
+    # an involution
+    np.testing.assert_array_equal(oracle64.random_flip(got.reshape(-1), N, C, H, W, probs), x)
+
+
+def test_normalize_closed_form(oracle64):
+    rng = np.random.default_rng(7)
+    C, N, W, H = 3, 4, 3, 5
+    x, img = _images(rng, C, N, W, H)
+    mean, std = np.array([0.4914, 0.4822, 0.4465]), np.array([0.2470, 0.2435, 0.2616])
+    want = (img / 255.0 - mean[:, None, None, None]) / std[:, None, None, None]
+    np.testing.assert_allclose(oracle64.normalize(x, N, H, W, C, mean, std).reshape(C, N, W, H), want, rtol=1e-15)
+
+
+def test_augment_data_composition(oracle64):
+    """solvers/kfac_da.cu:22-89: sample-major -> channel-major, crop, flip, normalise."""
+    rng = np.random.default_rng(8)
+    C, N, W, H = 3, 7, 8, 8
+    sampled = rng.integers(0, 256, size=N * C * W * H).astype(np.float64)      # [N][C][W][H]
+    cu, fu = rng.random(2 * N), rng.random(N)
+    mean, std = np.array([0.5071, 0.4865, 0.4409]), np.array([0.2673, 0.2564, 0.2762])
+    img = sampled.reshape(N, C, W, H).transpose(1, 0, 2, 3)                     # [C][N][W][H]
+    shifts = (np.trunc(cu * 100).astype(int) % 9) - 4
+    out = np.empty_like(img)
+    for n in range(N):
+        padded = np.pad(img[:, n], ((0, 0), (4, 4), (4, 4)))
+        sr, sc = shifts[n], shifts[N + n]
+        v = padded[:, 4 + sc:4 + sc + W, 4 + sr:4 + sr + H]
+        out[:, n] = np.flip(v, axis=1) if fu[n] < 0.5 else v
+    want = (out / 255.0 - mean[:, None, None, None]) / std[:, None, None, None]
+    got = oracle64.augment_data(sampled, N, C, H, W, 1, cu, fu, mean, std).reshape(C, N, W, H)
+    np.testing.assert_allclose(got, want, rtol=1e-15)
+    # without augmentation: layout change and normalisation only
+    plain = oracle64.augment_data(sampled, N, C, H, W, 0, cu, fu, mean, std).reshape(C, N, W, H)
+    np.testing.assert_allclose(plain, (img / 255.0 - mean[:, None, None, None]) / std[:, None, None, None], rtol=1e-15)
