@@ -183,7 +183,7 @@ def bandwidth_leg(L, dev, batch, reps=20):
         ws = dev.alloc(nb)
 
         def step():
-            L.check(hip.fitre_hip_pool_act_bn_backward(max_pool, relu, delta, zhat, None, var, channels, batch, hw, hw, 2, 2, 0,
+            L.check(hip.fitre_hip_pool_act_bn_backward(max_pool, relu, delta, 1, 0, zhat, None, var, channels, batch, hw, hw, 2, 2, 0,
                                                        hw // 2, hw // 2, 1e-5, dpool, dact, dbn, bias, ws, nb))
             L.check(hip.fitre_hip_copy(n, zhat, dbn))
 

@@ -150,9 +150,11 @@ static size_t c3_dw_workspace(const fitre_conv_shape *s)
 	return a > b ? a : b;
 }
 
+// leftSplits (may be null): when the product is split, skip the reduction launch, leave the partial
+// results in ws and report their number there (the caller's consumer sums them)
 template <bool DX>
 static int launch_c3_pos(const fitre_conv_shape *s, const float *src, const float *w, const float *bias, float *outPtr, void *ws,
-                         size_t wsBytes)
+                         size_t wsBytes, int *leftSplits = nullptr)
 {
 	const int I = DX ? s->inChannels : s->outChannels, cred = DX ? s->outChannels : s->inChannels;
 	const int J = s->samples * s->inA * s->inB;
@@ -198,7 +200,8 @@ static int launch_c3_pos(const fitre_conv_shape *s, const float *src, const floa
 		}
 #undef C3_LAUNCH
 	}
-	if (plan.splits > 1) launch_splitk_reduce((const float *)ws, plan.splits, I, J, out);
+	if (leftSplits) *leftSplits = plan.splits;
+	if (plan.splits > 1 && !leftSplits) launch_splitk_reduce((const float *)ws, plan.splits, I, J, out);
 	return check_launch("conv3x3_pos_kernel");
 }
 
@@ -370,6 +373,31 @@ int fitre_hip_conv_input_grad(const fitre_conv_shape *s, const float *delta, con
 	rc = attach_patch_table(pb, plan.bn);
 	if (rc) return rc;
 	return launch_gemm<FlipWeightKContig, PatchRowContig>(pa, pb, out, I, J, R, plan, ws, wsBytes, FITRE_KC_CONV_DX, conv_flops(s));
+}
+
+int fitre_hip_conv_input_grad_split(const fitre_conv_shape *s, const float *delta, const float *w, float *dx, void *ws,
+                                    size_t wsBytes, fitre_split_view *view)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(view != nullptr, "fitre_hip_conv_input_grad_split: null view");
+	view->base = dx;
+	view->splits = 1;
+	view->stride = 0;
+	int rc = check_conv("fitre_hip_conv_input_grad_split", s);
+	if (rc) return rc;
+	FITRE_REQUIRE(delta && w && dx, "fitre_hip_conv_input_grad_split: null pointer");
+	if (s->stride == 1 && s->padding < s->ksize && c3_pos_eligible(s, true)) {
+		int splits = 1;
+		rc = launch_c3_pos<true>(s, delta, w, nullptr, dx, ws, wsBytes, &splits);
+		if (rc) return rc;
+		if (splits > 1) {
+			view->base = (float *)ws;
+			view->splits = splits;
+			view->stride = (long)s->inChannels * s->samples * s->inA * s->inB;
+		}
+		return FITRE_OK;
+	}
+	return fitre_hip_conv_input_grad(s, delta, w, dx, ws, wsBytes);
 }
 
 // ---- general column-major GEMM ---------------------------------------------------

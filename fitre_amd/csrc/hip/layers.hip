@@ -598,6 +598,44 @@ __device__ __forceinline__ float4 route2x2(float4 r, float d)
 	return g;
 }
 
+// delta given as `splits` slabs `stride` floats apart: their sum in slab order, accumulated in double
+// (what the split-K reduction kernel would have written)
+__device__ __forceinline__ float4 load_sum4(const float *p, int splits, long stride)
+{
+	float4 t = *reinterpret_cast<const float4 *>(p);
+	if (splits == 1) return t;
+	double a0 = t.x, a1 = t.y, a2 = t.z, a3 = t.w;
+	for (int s = 1; s < splits; s++) {
+		t = *reinterpret_cast<const float4 *>(p + (size_t)s * stride);
+		a0 += (double)t.x, a1 += (double)t.y, a2 += (double)t.z, a3 += (double)t.w;
+	}
+	return make_float4((float)a0, (float)a1, (float)a2, (float)a3);
+}
+__device__ __forceinline__ float2 load_sum2(const float *p, int splits, long stride)
+{
+	float2 t = *reinterpret_cast<const float2 *>(p);
+	if (splits == 1) return t;
+	double a0 = t.x, a1 = t.y;
+	for (int s = 1; s < splits; s++) {
+		t = *reinterpret_cast<const float2 *>(p + (size_t)s * stride);
+		a0 += (double)t.x, a1 += (double)t.y;
+	}
+	return make_float2((float)a0, (float)a1);
+}
+__device__ __forceinline__ float load_sum1(const float *p, int splits, long stride)
+{
+	if (splits == 1) return *p;
+	double a = 0.0;
+	for (int s = 0; s < splits; s++) a += (double)p[(size_t)s * stride];
+	return (float)a;
+}
+// slab 0 += the other slabs (same order and precision)
+__global__ void __launch_bounds__(256) sum_slabs_kernel(float *base, int splits, long stride, long n)
+{
+	const long step = (long)gridDim.x * blockDim.x;
+	for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += step) base[i] = load_sum1(base + i, splits, stride);
+}
+
 // One (channel, segment) per workgroup.  POOL 0: 2x2 / stride 2 max pool (B % 4 == 0, A even), the
 // unit of work is a 2 x 4 patch; POOL 2: no pooling, the unit is a 16-byte group; POOL 3: 2x2 / stride 2
 // max pool of maps with B == 2, where pooled cell q of a channel is its 16-byte group q.  z_act == nullptr:
@@ -605,8 +643,8 @@ __device__ __forceinline__ float4 route2x2(float4 r, float d)
 // (sum g, sum g*zhat, sum zhat) per (channel, segment).
 template <int POOL>
 __global__ void __launch_bounds__(kRedBlock)
-pool_act_sums_kernel(const float *delta, const float *zhat, const float *z_act, int inA, int inB, int samples, int actFun,
-                     float *dxPool, float *dxAct, double *partial)
+pool_act_sums_kernel(const float *delta, int dSplits, long dStride, const float *zhat, const float *z_act, int inA, int inB,
+                     int samples, int actFun, float *dxPool, float *dxAct, double *partial)
 {
 	__shared__ double lds[3 * kRedBlock / kWave];
 	const int c = blockIdx.y;
@@ -620,8 +658,8 @@ pool_act_sums_kernel(const float *delta, const float *zhat, const float *z_act, 
 			const float4 zi = *reinterpret_cast<const float4 *>(zhat + base + i);
 			const float4 zo = z_act ? *reinterpret_cast<const float4 *>(z_act + base + i) : relu4(zi);
 			float4 g;
-			if constexpr (POOL == 2) g = *reinterpret_cast<const float4 *>(delta + base + i);
-			else g = route2x2(zo, delta[(base + i) / 4]);
+			if constexpr (POOL == 2) g = load_sum4(delta + base + i, dSplits, dStride);
+			else g = route2x2(zo, load_sum1(delta + (base + i) / 4, dSplits, dStride));
 			if (dxPool) *reinterpret_cast<float4 *>(dxPool + base + i) = g;
 			g = act_backward4(actFun, g, zi, zo);
 			*reinterpret_cast<float4 *>(dxAct + base + i) = g;
@@ -645,7 +683,7 @@ pool_act_sums_kernel(const float *delta, const float *zhat, const float *z_act, 
 			const float4 i1 = *reinterpret_cast<const float4 *>(zhat + inOff + inB);
 			const float4 r0 = z_act ? *reinterpret_cast<const float4 *>(z_act + inOff) : relu4(i0);
 			const float4 r1 = z_act ? *reinterpret_cast<const float4 *>(z_act + inOff + inB) : relu4(i1);
-			const float2 d = *reinterpret_cast<const float2 *>(delta + dOff);
+			const float2 d = load_sum2(delta + dOff, dSplits, dStride);
 			float4 g0, g1;
 			route2x4(r0, r1, d, g0, g1);
 			if (dxPool) {
@@ -671,8 +709,9 @@ pool_act_sums_kernel(const float *delta, const float *zhat, const float *z_act, 
 // in registers between the sums and the batch-norm formula; one launch for the three steps.
 template <int POOL>
 __global__ void __launch_bounds__(kRedBlock)
-pool_act_bn_small_kernel(const float *delta, const float *zhat, const float *z_act, const float *variance, int inA, int inB,
-                         int samples, int actFun, float epsilon, float *dxPool, float *dxAct, float *dxBn, float *biasGrad)
+pool_act_bn_small_kernel(const float *delta, int dSplits, long dStride, const float *zhat, const float *z_act,
+                         const float *variance, int inA, int inB, int samples, int actFun, float epsilon, float *dxPool,
+                         float *dxAct, float *dxBn, float *biasGrad)
 {
 	__shared__ double lds[3 * kRedBlock / kWave];
 	constexpr int G = (int)(kBnSmallChannel / (4 * kRedBlock)); // 16-byte groups per thread
@@ -691,8 +730,8 @@ pool_act_bn_small_kernel(const float *delta, const float *zhat, const float *z_a
 			if (off[k] < 0) continue;
 			z[k] = *reinterpret_cast<const float4 *>(zhat + base + i);
 			const float4 zo = z_act ? *reinterpret_cast<const float4 *>(z_act + base + i) : relu4(z[k]);
-			if constexpr (POOL == 2) g[k] = *reinterpret_cast<const float4 *>(delta + base + i);
-			else g[k] = route2x2(zo, delta[(base + i) / 4]);
+			if constexpr (POOL == 2) g[k] = load_sum4(delta + base + i, dSplits, dStride);
+			else g[k] = route2x2(zo, load_sum1(delta + (base + i) / 4, dSplits, dStride));
 			if (dxPool) *reinterpret_cast<float4 *>(dxPool + base + i) = g[k];
 			g[k] = act_backward4(actFun, g[k], z[k], zo);
 			*reinterpret_cast<float4 *>(dxAct + base + i) = g[k];
@@ -719,7 +758,7 @@ pool_act_bn_small_kernel(const float *delta, const float *zhat, const float *z_a
 			z[2 * k + 1] = *reinterpret_cast<const float4 *>(zhat + base + in + inB);
 			const float4 r0 = z_act ? *reinterpret_cast<const float4 *>(z_act + base + in) : relu4(z[2 * k]);
 			const float4 r1 = z_act ? *reinterpret_cast<const float4 *>(z_act + base + in + inB) : relu4(z[2 * k + 1]);
-			const float2 d = *reinterpret_cast<const float2 *>(delta + dOff);
+			const float2 d = load_sum2(delta + dOff, dSplits, dStride);
 			route2x4(r0, r1, d, g[2 * k], g[2 * k + 1]);
 			if (dxPool) {
 				*reinterpret_cast<float4 *>(dxPool + base + in) = g[2 * k];
@@ -1161,12 +1200,14 @@ int fitre_hip_batch_norm_backward(const float *delta, const float *zhat, const f
 	return check_launch("batch_norm_backward");
 }
 
-int fitre_hip_pool_act_bn_backward(int poolType, int actFun, const float *delta, const float *zhat, const float *z_act,
-                                   const float *variance, int channels, int samples, int inA, int inB, int ksize, int stride,
-                                   int padding, int outA, int outB, float epsilon, float *dxPool, float *dxAct, float *dxBn,
-                                   float *biasGrad, void *ws, size_t wsBytes)
+int fitre_hip_pool_act_bn_backward(int poolType, int actFun, float *delta, int deltaSplits, long deltaStride, const float *zhat,
+                                   const float *z_act, const float *variance, int channels, int samples, int inA, int inB,
+                                   int ksize, int stride, int padding, int outA, int outB, float epsilon, float *dxPool,
+                                   float *dxAct, float *dxBn, float *biasGrad, void *ws, size_t wsBytes)
 {
 	FITRE_NEED_INIT();
+	FITRE_REQUIRE(deltaSplits >= 1 && (deltaSplits == 1 || deltaStride > 0),
+	              "fitre_hip_pool_act_bn_backward: bad split view (%d slabs, stride %ld)", deltaSplits, deltaStride);
 	FITRE_REQUIRE(delta && zhat && variance && dxAct && dxBn, "fitre_hip_pool_act_bn_backward: null pointer");
 	FITRE_REQUIRE(z_act || actFun == CNN_ACT_RELU,
 	              "fitre_hip_pool_act_bn_backward: z_act may be left out for ReLU only (activation %d)", actFun);
@@ -1180,13 +1221,19 @@ int fitre_hip_pool_act_bn_backward(int poolType, int actFun, const float *delta,
 	                     (!dxPool || aligned16(dxPool));
 	bool fused = false;
 	if (poolType == NO_POOL)
-		fused = aligned && aligned16(delta) && perChannel % 4 == 0;
+		fused = aligned && aligned16(delta) && perChannel % 4 == 0 && (deltaSplits == 1 || deltaStride % 4 == 0);
 	else if (poolType == MAX_POOL)
 		fused = aligned && ksize == 2 && stride == 2 && padding == 0 && (inB % 4 == 0 || inB == 2) && inA % 2 == 0 &&
-		        outA == inA / 2 && outB == inB / 2 && (((uintptr_t)delta & 7) == 0);
+		        outA == inA / 2 && outB == inB / 2 && (((uintptr_t)delta & 7) == 0) && (deltaSplits == 1 || deltaStride % 2 == 0);
 	const int variant = (poolType == NO_POOL) ? 2 : (inB == 2 ? 3 : 0);
 	if (!fused) {
-		// other windows / layouts: the separate passes (z_act rebuilt for the ReLU shortcut)
+		// other windows / layouts: the separate passes (slabs summed, z_act rebuilt for the ReLU shortcut)
+		if (deltaSplits > 1) {
+			const long nd = (poolType == NO_POOL) ? (long)channels * perChannel : (long)channels * samples * outA * outB;
+			sum_slabs_kernel<<<blocks_for(nd, 256, 8192), 256, 0, stream()>>>(delta, deltaSplits, deltaStride, nd);
+			rc = check_launch("sum_slabs_kernel");
+			if (rc) return rc;
+		}
 		const float *zo = z_act;
 		if (!zo) {
 			rc = fitre_hip_activation_forward(actFun, zhat, dxBn, (long)channels * perChannel);
@@ -1200,17 +1247,17 @@ int fitre_hip_pool_act_bn_backward(int poolType, int actFun, const float *delta,
 	}
 	const double total = (double)channels * (double)perChannel;
 	const double poolBytes = 4.0 * total * (2 + (dxPool ? 1 : 0) + (z_act ? 1 : 0)) +
-	                         4.0 * (poolType == NO_POOL ? total : total / 4);
+	                         4.0 * deltaSplits * (poolType == NO_POOL ? total : total / 4);
 	if (perChannel <= kBnSmallChannel && channels >= 128) {
 		LaunchScope scope(FITRE_KC_POOL_ACT_BWD, poolBytes + 4.0 * total);
 		if (variant == 2)
-			pool_act_bn_small_kernel<2><<<channels, kRedBlock, 0, stream()>>>(delta, zhat, z_act, variance, inA, inB, samples, actFun,
+			pool_act_bn_small_kernel<2><<<channels, kRedBlock, 0, stream()>>>(delta, deltaSplits, deltaStride, zhat, z_act, variance, inA, inB, samples, actFun,
 			                                                                 epsilon, dxPool, dxAct, dxBn, biasGrad);
 		else if (variant == 3)
-			pool_act_bn_small_kernel<3><<<channels, kRedBlock, 0, stream()>>>(delta, zhat, z_act, variance, inA, inB, samples, actFun,
+			pool_act_bn_small_kernel<3><<<channels, kRedBlock, 0, stream()>>>(delta, deltaSplits, deltaStride, zhat, z_act, variance, inA, inB, samples, actFun,
 			                                                                 epsilon, dxPool, dxAct, dxBn, biasGrad);
 		else
-			pool_act_bn_small_kernel<0><<<channels, kRedBlock, 0, stream()>>>(delta, zhat, z_act, variance, inA, inB, samples, actFun,
+			pool_act_bn_small_kernel<0><<<channels, kRedBlock, 0, stream()>>>(delta, deltaSplits, deltaStride, zhat, z_act, variance, inA, inB, samples, actFun,
 			                                                                 epsilon, dxPool, dxAct, dxBn, biasGrad);
 		return check_launch("pool_act_bn_small_kernel");
 	}
@@ -1220,11 +1267,11 @@ int fitre_hip_pool_act_bn_backward(int poolType, int actFun, const float *delta,
 	{
 		LaunchScope scope(FITRE_KC_POOL_ACT_BWD, poolBytes);
 		if (variant == 2)
-			pool_act_sums_kernel<2><<<grid, kRedBlock, 0, stream()>>>(delta, zhat, z_act, inA, inB, samples, actFun, dxPool, dxAct, partial);
+			pool_act_sums_kernel<2><<<grid, kRedBlock, 0, stream()>>>(delta, deltaSplits, deltaStride, zhat, z_act, inA, inB, samples, actFun, dxPool, dxAct, partial);
 		else if (variant == 3)
-			pool_act_sums_kernel<3><<<grid, kRedBlock, 0, stream()>>>(delta, zhat, z_act, inA, inB, samples, actFun, dxPool, dxAct, partial);
+			pool_act_sums_kernel<3><<<grid, kRedBlock, 0, stream()>>>(delta, deltaSplits, deltaStride, zhat, z_act, inA, inB, samples, actFun, dxPool, dxAct, partial);
 		else
-			pool_act_sums_kernel<0><<<grid, kRedBlock, 0, stream()>>>(delta, zhat, z_act, inA, inB, samples, actFun, dxPool, dxAct, partial);
+			pool_act_sums_kernel<0><<<grid, kRedBlock, 0, stream()>>>(delta, deltaSplits, deltaStride, zhat, z_act, inA, inB, samples, actFun, dxPool, dxAct, partial);
 		rc = check_launch("pool_act_sums_kernel");
 		if (rc) return rc;
 	}

@@ -79,20 +79,36 @@ static size_t forward_ws_bytes(const CNN_MODEL *model, int batch)
 /* cnnBackward carves two workspaces from devPtr: one for the chain that produces each layer's
  * delta (pool / activation / batch norm / input gradient, lane 0) and one for the weight gradients,
  * which run beside that chain on lane 1. */
-static size_t backward_chain_ws_bytes(const CNN_MODEL *model, int batch)
+/* The chain workspace has two parts that are live at the same time: the input gradient's split partials,
+ * which the pool / activation pass of the layer below sums while it reads them, and that pass's
+ * batch-norm sums. */
+static size_t backward_dx_ws_bytes(const CNN_MODEL *model, int batch)
 {
 	size_t need = 256;
-	for (int i = 0; i < model->cLayers; i++) {
-		const CONV_LAYER *c = &model->convLayer[i];
-		fitre_conv_shape s = conv_shape(c, batch);
-		if (i != 0) need = max_sz(need, fitre_hip_conv_input_grad_workspace(&s));
-		need = max_sz(need, fitre_hip_batch_norm_workspace(c->outChannels, (long)batch * c->outWidth * c->outHeight));
+	for (int i = 1; i < model->cLayers; i++) {
+		fitre_conv_shape s = conv_shape(&model->convLayer[i], batch);
+		need = max_sz(need, fitre_hip_conv_input_grad_workspace(&s));
 	}
 	for (int i = 0; i < model->lLayers; i++) {
 		const FC_LAYER *f = &model->fcLayer[i];
 		need = max_sz(need, fitre_hip_gemm_workspace(f->in, batch, f->out));
 	}
 	return (need + 255) & ~(size_t)255;
+}
+
+static size_t backward_bn_ws_bytes(const CNN_MODEL *model, int batch)
+{
+	size_t need = 256;
+	for (int i = 0; i < model->cLayers; i++) {
+		const CONV_LAYER *c = &model->convLayer[i];
+		need = max_sz(need, fitre_hip_batch_norm_workspace(c->outChannels, (long)batch * c->outWidth * c->outHeight));
+	}
+	return (need + 255) & ~(size_t)255;
+}
+
+static size_t backward_chain_ws_bytes(const CNN_MODEL *model, int batch)
+{
+	return backward_dx_ws_bytes(model, batch) + backward_bn_ws_bytes(model, batch);
 }
 
 static size_t backward_side_ws_bytes(const CNN_MODEL *model, int batch)
@@ -210,9 +226,11 @@ void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, 
 	const int *wOffsets = model->wOffsets, *bOffsets = model->bOffsets, *zOffsets = model->zOffsets;
 	const real *weights = data->weights;
 	const int n = batchSize, nc = model->cLayers;
-	void *ws = (void *)devPtr;
-	const size_t wsBytes = backward_chain_ws_bytes(model, model->batchSize);
-	void *sideWs = (void *)((char *)devPtr + wsBytes);
+	void *ws = (void *)devPtr; /* input-gradient partials (and the FC products' splits) */
+	const size_t wsBytes = backward_dx_ws_bytes(model, model->batchSize);
+	void *bnWs = (void *)((char *)devPtr + wsBytes);
+	const size_t bnBytes = backward_bn_ws_bytes(model, model->batchSize);
+	void *sideWs = (void *)((char *)bnWs + bnBytes);
 	const size_t sideBytes = backward_side_ws_bytes(model, model->batchSize);
 	real *temp;
 
@@ -263,6 +281,9 @@ void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, 
 		delta = temp;
 	}
 
+	/* delta as the layer above left it: a plain tensor, or the unsummed split partials of its input
+	 * gradient (summed by the pool / activation pass below while it reads them) */
+	fitre_split_view dview = { delta, 1, 0 };
 	for (int c = nc - 1; c >= 0; c--) {
 		const CONV_LAYER *l = &model->convLayer[c];
 		const POOL_LAYER *p = &model->poolLayer[c];
@@ -290,12 +311,13 @@ void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, 
 		if (has_bn(l)) {
 			/* pool backward -> dx slab + 0; times f'(.) -> dx slab + activationOffset; batch-norm backward ->
 			 * dx slab + batchNormOffset, its column sums being the bias gradient */
-			HIP_CALL(fitre_hip_pool_act_bn_backward(p->type, act, delta, actIn, fusedRelu ? NULL : actOut,
+			HIP_CALL(fitre_hip_pool_act_bn_backward(p->type, act, dview.base, dview.splits, dview.stride, actIn,
+			                                        fusedRelu ? NULL : actOut,
 			                                        slab + l->batchNormOffset + l->variancesOffset, l->outChannels, n, p->width,
 			                                        p->height, p->pSize, p->stride, p->padding, p->outWidth, p->outHeight,
 			                                        (real)BATCH_NORM_EPSILON, dslab, dslab + l->activationOffset,
 			                                        dslab + l->batchNormOffset,
-			                                        (model->bias != 0) ? gradient + bOffsets[c] : NULL, ws, wsBytes));
+			                                        (model->bias != 0) ? gradient + bOffsets[c] : NULL, bnWs, bnBytes));
 			cur = dslab + l->batchNormOffset;
 		} else {
 			/* pool backward -> dx slab + 0; times f'(.) -> dx slab + activationOffset */
@@ -304,7 +326,7 @@ void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, 
 			                                     dslab + l->activationOffset));
 			cur = dslab + l->activationOffset;
 			if (model->bias != 0)
-				HIP_CALL(fitre_hip_channel_sum(cur, l->outChannels, perChannel, gradient + bOffsets[c], ws, wsBytes));
+				HIP_CALL(fitre_hip_channel_sum(cur, l->outChannels, perChannel, gradient + bOffsets[c], bnWs, bnBytes));
 		}
 
 		const real *input = (c == 0) ? data->currentBatch : z + zOffsets[c] + model->convLayer[c - 1].outputOffset;
@@ -313,7 +335,14 @@ void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, 
 		 * reads, is queued behind it on lane 1, whose kernels leave a share of the compute units
 		 * free: the bandwidth-bound kernels of the layer below (split reduction, pooling, batch
 		 * norm) run on those while the weight gradient keeps the matrix pipes busy. */
-		if (c != 0) HIP_CALL(fitre_hip_conv_input_grad(&shape, cur, weights + wOffsets[c], delta, ws, wsBytes));
+		if (c != 0) {
+			if (has_bn(&model->convLayer[c - 1])) {
+				HIP_CALL(fitre_hip_conv_input_grad_split(&shape, cur, weights + wOffsets[c], delta, ws, wsBytes, &dview));
+			} else {
+				HIP_CALL(fitre_hip_conv_input_grad(&shape, cur, weights + wOffsets[c], delta, ws, wsBytes));
+				dview.base = delta, dview.splits = 1, dview.stride = 0;
+			}
+		}
 		HIP_CALL(fitre_hip_lane_wait(1, 0));
 		HIP_CALL(fitre_hip_lane_select(1));
 		HIP_CALL(fitre_hip_conv_weight_grad(&shape, input, cur, gradient + wOffsets[c], sideWs, sideBytes));

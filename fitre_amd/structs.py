@@ -106,6 +106,11 @@ class KFAC_CURVATURE_INFO(C.Structure):
                 [("inverseFreq", C.c_int)])
 
 
+class fitre_split_view(C.Structure):
+    """include/fitre_hip.h: unsummed split partials of an input gradient."""
+    _fields_ = [("base", C.c_void_p), ("splits", C.c_int), ("stride", C.c_long)]
+
+
 class fitre_conv_shape(C.Structure):
     _fields_ = [(n, C.c_int) for n in (
         "samples", "inChannels", "outChannels", "inA", "inB", "outA", "outB", "ksize", "stride", "padding")]

@@ -204,12 +204,15 @@ int fitre_hip_batch_norm_backward(const float *delta, const float *zhat, const f
  * activation input (the batch-norm output).  z_act may be NULL when actFun is ReLU: the activation output is
  * then taken as max(zhat, 0), bit-identical to what the forward pass stored.  Fused for no pooling and for
  * 2x2 / stride 2 max pooling on 16-byte-aligned tensors; every other case runs the two separate passes.
+ * delta may be given as deltaSplits > 1 slabs deltaStride floats apart whose sum, in slab order, is the
+ * gradient (the view fitre_hip_conv_input_grad_split leaves; the unfused fallback sums them into the first
+ * slab); deltaSplits = 1 for a plain tensor.
  * Workspace: fitre_hip_batch_norm_workspace(channels, samples * inA * inB). */
-int fitre_hip_pool_act_bn_backward(int poolType, int actFun, const float *delta, const float *zhat,
-                                   const float *z_act, const float *variance, int channels, int samples,
-                                   int inA, int inB, int ksize, int stride, int padding, int outA, int outB,
-                                   float epsilon, float *dxPool, float *dxAct, float *dxBn, float *biasGrad,
-                                   void *ws, size_t wsBytes);
+int fitre_hip_pool_act_bn_backward(int poolType, int actFun, float *delta, int deltaSplits, long deltaStride,
+                                   const float *zhat, const float *z_act, const float *variance, int channels,
+                                   int samples, int inA, int inB, int ksize, int stride, int padding, int outA,
+                                   int outB, float epsilon, float *dxPool, float *dxAct, float *dxBn,
+                                   float *biasGrad, void *ws, size_t wsBytes);
 
 /* ---------------- mini-batch selection and augmentation ---------------- */
 /* tgt column j = src column indices[j], columns of `rows` values (kerExtractColumns,
@@ -292,6 +295,19 @@ int fitre_hip_conv_weight_grad(const fitre_conv_shape *s, const float *x, const 
 size_t fitre_hip_conv_input_grad_workspace(const fitre_conv_shape *s);
 int fitre_hip_conv_input_grad(const fitre_conv_shape *s, const float *delta, const float *w, float *dx,
                               void *ws, size_t wsBytes);
+/* The same product, but when its reduction is split over workgroups the partial results are left unsummed
+ * for the consumer to add up while it reads them (fitre_hip_pool_act_bn_backward takes such a view): one
+ * launch and one pass over dx less.  view->base points at view->splits slabs of Cin*N*inA*inB floats,
+ * view->stride floats apart, inside ws (which must then stay untouched until the consumer has run); the
+ * gradient is their sum in slab order.  An unsplit product writes dx as usual and reports splits = 1,
+ * base = dx. */
+typedef struct fitre_split_view {
+	float *base;
+	int splits;
+	long stride;
+} fitre_split_view;
+int fitre_hip_conv_input_grad_split(const fitre_conv_shape *s, const float *delta, const float *w, float *dx,
+                                    void *ws, size_t wsBytes, fitre_split_view *view);
 
 /* Column-major GEMM C(MxN) = alpha*op(A)*op(B) + beta*C with the argument meaning of cublasDgemm
  * (transA/transB: 0 = N, 1 = T).  Used for the FC layers (eval_gradient.cu:63-67,

@@ -159,6 +159,38 @@ def test_split_k_is_deterministic_and_workspace_independent(dev, oracle64):
     assert rel_err(dev.download(out, Cout * Cin * k * k), want) < TOL
 
 
+@pytest.mark.parametrize("case", [(256, 256, 512, 4, 4), (64, 512, 512, 2, 2), (96, 200, 520, 4, 4), (4, 16, 32, 8, 8), (2, 4, 6, 9, 9)])
+def test_input_gradient_left_as_split_partials(dev, case):
+    """fitre_hip_conv_input_grad_split: the slabs of the view, summed in order in double, are what
+    fitre_hip_conv_input_grad writes -- bit for bit; an unsplit product reports one slab at dx."""
+    from fitre_amd.structs import fitre_split_view
+    N, Cin, Cout, A, B = case
+    shape = conv_shape(N, Cin, Cout, A, B, 3, 1, 1)
+    rng = np.random.default_rng(Cin + A)
+    w = (rng.standard_normal(Cout * Cin * 9) / np.sqrt(Cin * 9)).astype(np.float32)
+    d = rng.standard_normal(Cout * N * A * B).astype(np.float32)
+    n = Cin * N * A * B
+    pw, pd = dev.upload(w), dev.upload(d)
+    nb = hip.fitre_hip_conv_input_grad_workspace(C.byref(shape))
+    ws, ref, out = dev.alloc(nb), dev.zeros(n), dev.upload(np.full(n, 7.0, np.float32))
+    L.check(hip.fitre_hip_conv_input_grad(C.byref(shape), pd, pw, ref, ws, nb))
+    want = dev.download(ref, n)
+    view = fitre_split_view()
+    L.check(hip.fitre_hip_conv_input_grad_split(C.byref(shape), pd, pw, out, ws, nb, C.byref(view)))
+    if view.splits == 1:
+        assert view.base == out.value
+        np.testing.assert_array_equal(dev.download(out, n), want)
+    else:
+        assert view.base == ws.value and view.stride == n and nb >= 4 * n * view.splits
+        acc = np.zeros(n)
+        for q in range(view.splits):
+            acc += dev.download(ws, n, offset=q * view.stride).astype(np.float64)
+        np.testing.assert_array_equal(acc.astype(np.float32), want)
+        np.testing.assert_array_equal(dev.download(out, n), np.full(n, 7.0, np.float32))   # dx itself is left alone
+    for q in (pw, pd, ws, ref, out):
+        dev.free(q)
+
+
 GEMM_CASES = [  # M, N, K
     (10, 256, 512), (512, 256, 10), (120, 7, 400), (84, 128, 120), (1, 1, 1), (129, 65, 33), (300, 200, 64), (64, 64, 4096),
 ]

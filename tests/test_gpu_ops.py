@@ -294,10 +294,13 @@ FUSED_BN_GEOMS = [
 
 
 @pytest.mark.parametrize("geom", FUSED_BN_GEOMS)
-@pytest.mark.parametrize("act,derive", [(CNN_ACT_RELU, True), (CNN_ACT_RELU, False), (CNN_ACT_SWISH, False)])
+@pytest.mark.parametrize("act,derive,slabs", [(CNN_ACT_RELU, True, 1), (CNN_ACT_RELU, False, 1), (CNN_ACT_SWISH, False, 1),
+                                              (CNN_ACT_RELU, True, 3), (CNN_ACT_SWISH, False, 8)])
 @pytest.mark.parametrize("kind", [MAX_POOL, NO_POOL, AVG_POOL])
-def test_fused_pool_activation_batch_norm_backward(dev, oracle64, geom, act, derive, kind):
-    """fitre_hip_pool_act_bn_backward against the oracle's three steps (functions/cnn_backward.cu:586-660)."""
+def test_fused_pool_activation_batch_norm_backward(dev, oracle64, geom, act, derive, slabs, kind):
+    """fitre_hip_pool_act_bn_backward against the oracle's three steps (functions/cnn_backward.cu:586-660).
+    slabs > 1: delta arrives as unsummed split partials (the view of fitre_hip_conv_input_grad_split); the
+    gradient is their sum in slab order, accumulated in double and rounded once."""
     Cn, N, A, B, k, s, p = geom
     oA, oB = ((A + 2 * p - k) // s + 1, (B + 2 * p - k) // s + 1) if kind != NO_POOL else (A, B)
     per = N * A * B
@@ -305,12 +308,20 @@ def test_fused_pool_activation_batch_norm_backward(dev, oracle64, geom, act, der
     zhat = rng.standard_normal(Cn * per).astype(np.float32)
     zact = oracle64.activation_forward(act, zhat.astype(np.float64)).astype(np.float32)
     var = (0.5 + rng.random(Cn)).astype(np.float32)
-    d = rng.standard_normal(Cn * N * oA * oB).astype(np.float32)
-    pz, pa, pd, pv = dev.upload(zhat), dev.upload(zact), dev.upload(d), dev.upload(var)
+    nd = Cn * N * oA * oB
+    stride = nd + (8 - nd % 8) % 8 + 8           # slabs 16-byte aligned, with a gap
+    parts = rng.standard_normal((slabs, stride)).astype(np.float32)
+    d = parts[:, :nd].astype(np.float64).sum(axis=0).astype(np.float32) if slabs > 1 else parts[0, :nd].copy()
+    if slabs > 1:   # sequential double accumulation, as on the device
+        acc = np.zeros(nd)
+        for q in range(slabs):
+            acc += parts[q, :nd].astype(np.float64)
+        d = acc.astype(np.float32)
+    pz, pa, pd, pv = dev.upload(zhat), dev.upload(zact), dev.upload(parts.reshape(-1)), dev.upload(var)
     dxp, dxa, dxb, bias = dev.zeros(zhat.size), dev.zeros(zhat.size), dev.zeros(zhat.size), dev.zeros(Cn)
     ws, nb = bn_ws(dev, Cn, per)
-    ok(hip.fitre_hip_pool_act_bn_backward(kind, act, pd, pz, None if derive else pa, pv, Cn, N, A, B, k, s, p, oA, oB, 1e-5,
-                                          dxp, dxa, dxb, bias, ws, nb))
+    ok(hip.fitre_hip_pool_act_bn_backward(kind, act, pd, slabs, stride, pz, None if derive else pa, pv, Cn, N, A, B, k, s, p, oA,
+                                          oB, 1e-5, dxp, dxa, dxb, bias, ws, nb))
     if kind == NO_POOL:
         wantp = d.astype(np.float64)
     else:
@@ -333,8 +344,10 @@ def test_fused_pool_activation_batch_norm_backward(dev, oracle64, geom, act, der
 def test_fused_backward_rejects_missing_activation_output(dev):
     p = dev.zeros(256)
     ws, nb = bn_ws(dev, 1, 64)
-    assert hip.fitre_hip_pool_act_bn_backward(NO_POOL, CNN_ACT_SWISH, p, p, None, p, 1, 1, 8, 8, 1, 1, 0, 8, 8, 1e-5, p, p, p, None, ws, nb) == 2
+    assert hip.fitre_hip_pool_act_bn_backward(NO_POOL, CNN_ACT_SWISH, p, 1, 0, p, None, p, 1, 1, 8, 8, 1, 1, 0, 8, 8, 1e-5, p, p, p, None, ws, nb) == 2
     assert b"ReLU only" in hip.fitre_hip_last_error()
+    assert hip.fitre_hip_pool_act_bn_backward(NO_POOL, CNN_ACT_RELU, p, 2, 0, p, None, p, 1, 1, 8, 8, 1, 1, 0, 8, 8, 1e-5, p, p, p, None, ws, nb) == 2
+    assert b"split view" in hip.fitre_hip_last_error()
 
 
 def test_workspace_too_small_is_reported(dev):
