@@ -217,3 +217,75 @@ def test_vgg11_full_size_directional_derivative(vgg_full, dev):
     L.check(L.hip.fitre_hip_copy_h2d(gm.w, w.ctypes.data_as(C.c_void_p), 4 * w.size))
     fd = (losses[0] - losses[1]) / (2 * h)
     assert abs(fd - np.dot(g, d)) < 0.05 * abs(np.dot(g, d)) + 1e-3
+
+
+# ------------------------------------------------------------------ AlexNet at its full size: properties
+@pytest.fixture(scope="module")
+def alexnet_full(dev):
+    """3 x 224 x 224, batch 64, 1000 classes: 11x11/s4, 5x5, 3x3 convolutions, max-pool 3/2, FC 9216-4096-4096-1000
+    (62 M parameters).  Too large for the CPU oracle in a test; checked through what holds at any size."""
+    batch = 64
+    model = build_alexnet(batch)
+    rng = np.random.default_rng(4242)
+    w = he_weights(model, rng).astype(np.float32)
+    # He-normal weights on N(0,1) pixels give logits in the hundreds; the loss then sits on the floor the
+    # reference puts under the probabilities (p + 1e-10, functions/softmax_loss.cu) and stops following the
+    # gradient.  A small last layer keeps the softmax in its smooth range.
+    last = model.cLayers + model.lLayers - 1
+    w[model.wOffsets[last]:model.bOffsets[last]] *= np.float32(0.02)
+    x, y = batch_inputs(model, batch, rng)
+    gm = GpuModel(dev, model, w, x.astype(np.float32), y, batch)
+    yield gm, w
+    gm.release()
+
+
+def test_alexnet_full_size_properties(alexnet_full, dev):
+    gm, w = alexnet_full
+    model, batch = gm.model, gm.batch
+    assert model.cLayers == 5 and model.lLayers == 3 and model.fcLayer[0].in_ == 9216
+    loss = gm.forward()
+    assert np.isfinite(loss) and 5.0 < loss < 12.0        # log(1000) = 6.9 for uninformed predictions
+    probs = gm.get("probs").reshape(batch, 1000)
+    np.testing.assert_allclose(probs.sum(1), 1.0, atol=1e-5)
+    err = gm.get("errors").reshape(batch, 1000)
+    gm.backward()
+    g1 = gm.get("grad")
+    assert np.isfinite(g1).all()
+    for l in range(8):                                      # every layer receives a gradient
+        n = model.bOffsets[l] - model.wOffsets[l]
+        assert np.abs(g1[model.wOffsets[l]:model.wOffsets[l] + n]).max() > 0, l
+    gm.backward()
+    np.testing.assert_array_equal(g1, gm.get("grad"))       # bitwise run-to-run determinism
+    # last FC layer in closed form: bias gradient = column sums of the loss errors, weight gradient = errors x input
+    z = gm.get("z")
+    last = model.cLayers + model.lLayers - 1
+    f = model.fcLayer[model.lLayers - 1]
+    zin = z[model.zOffsets[last]:][:f.in_ * batch].reshape(batch, f.in_).astype(np.float64)
+    want = zin.T @ err.astype(np.float64)
+    got = g1[model.wOffsets[last]:model.wOffsets[last] + f.in_ * f.out].reshape(f.in_, f.out)
+    assert rel_err(got, want) < TOL
+    np.testing.assert_allclose(g1[model.bOffsets[last]:model.bOffsets[last] + f.out], err.astype(np.float64).sum(0), atol=1e-6)
+    # linear in the incoming errors, exactly for a power of two
+    L.check(L.hip.fitre_hip_scal(1000 * batch, 2.0, gm.errors))
+    gm.backward()
+    np.testing.assert_array_equal(gm.get("grad"), 2 * g1)
+
+
+def test_alexnet_full_size_directional_derivative(alexnet_full, dev):
+    """g'd against a central difference of the loss along a random direction d (fp32 forward)."""
+    gm, w = alexnet_full
+    gm.forward()
+    gm.backward()
+    g = gm.get("grad").astype(np.float64)
+    rng = np.random.default_rng(98)
+    d = rng.standard_normal(w.size).astype(np.float32)
+    d *= np.float32(1.0 / np.linalg.norm(d.astype(np.float64)))
+    h = 5e-2
+    losses = []
+    for sgn in (+1, -1):
+        L.check(L.hip.fitre_hip_copy_h2d(gm.w, (w + np.float32(sgn * h) * d).ctypes.data_as(C.c_void_p), 4 * w.size))
+        losses.append(gm.forward())
+    L.check(L.hip.fitre_hip_copy_h2d(gm.w, w.ctypes.data_as(C.c_void_p), 4 * w.size))
+    fd = (losses[0] - losses[1]) / (2 * h)
+    gd = float(np.dot(g, d.astype(np.float64)))
+    assert abs(fd - gd) < 0.05 * abs(gd) + 1e-3, (fd, gd)
