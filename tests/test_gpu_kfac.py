@@ -296,3 +296,66 @@ def test_model_inverses_and_natural_gradient(dev, oracle64, name):
     for q in (ofac, lfac, oinv, linv, ws, ngrad):
         dev.free(q)
     gm.release()
+
+
+def test_vgg11_full_size_factor_inverses_with_the_benchmark_damping(dev):
+    """The KFAC configuration of the benchmark at its real size: VGG-11, batch 256, damping lambda = 1e-3 and nothing
+    else.  Input factors reach order 4609 with 1024 patches behind them (rank deficient: the damping alone keeps them
+    positive definite) and condition numbers up to 1e6, which float32 can only invert to about cond * 2^-24.  Checked:
+    every Cholesky succeeds (a non-positive pivot ends the process, as in the reference), every inverse is finite and
+    exactly symmetric, and (F + lambda I) X v = v for random v within 1e-7 * cond."""
+    from fitre_amd.structs import KFAC_CURVATURE_INFO
+    from helpers import GpuModel, batch_inputs, build_vgg11, he_weights
+    batch, lam = 256, 1e-3
+    model = build_vgg11(batch, bn=True)
+    rng = np.random.default_rng(7)
+    w = he_weights(model, rng).astype(np.float32)
+    x, y = batch_inputs(model, batch, rng)
+    gm = GpuModel(dev, model, w, x.astype(np.float32), y, batch)
+    gm.forward()
+    gm.backward()
+    info = KFAC_CURVATURE_INFO()
+    L.cnn.computeKFACStorageIndices(C.byref(model), C.byref(info))
+    layers = model.cLayers + model.lLayers
+    tot_o, tot_l = info.OmegaZOffsets[layers], info.LambdaGOffsets[layers]
+    ofac, lfac, oinv, linv = dev.zeros(tot_o), dev.zeros(tot_l), dev.zeros(tot_o), dev.zeros(tot_l)
+    need = max(L.cnn.kfacInverseMemRequired(C.byref(model), batch), L.cnn.kfacFactorsMemRequired(C.byref(model), batch),
+               L.cnn.kfacNaturalGradientMemRequired(C.byref(model)))
+    ws = dev.alloc(4 * need + 512)
+    info.regLambda, info.dampGamma = lam, 0.0
+    L.cnn.computeOmegaZFactors(C.byref(info), C.byref(model), C.byref(gm.data), batch, None, gm.z, ofac, model.zOffsets,
+                               model.zztOffsets, ws)
+    L.cnn.computeLambdaDeltaFactors(C.byref(info), C.byref(model), batch, gm.dx, None, lfac, model.zOffsets, model.zztOffsets, ws)
+    L.cnn.computeOmegaZ(C.byref(info), C.byref(model), C.byref(gm.data), batch, None, gm.z, oinv, model.zOffsets,
+                        model.zztOffsets, ws, None)
+    L.cnn.computeLambdaDelta(C.byref(info), C.byref(model), batch, gm.dx, None, linv, model.zOffsets, model.zztOffsets, ws, None)
+    assert info.OmegaZOffsets[6] - info.OmegaZOffsets[5] == 4609 * 4609
+    for F, X, offs, what in ((dev.download(ofac, tot_o), dev.download(oinv, tot_o), info.OmegaZOffsets, "omega"),
+                             (dev.download(lfac, tot_l), dev.download(linv, tot_l), info.LambdaGOffsets, "lambda")):
+        for l in range(layers):
+            n = int(round(np.sqrt(offs[l + 1] - offs[l])))
+            A = F[offs[l]:offs[l] + n * n].reshape(n, n).astype(np.float64)
+            Xi = X[offs[l]:offs[l] + n * n].reshape(n, n)
+            assert np.isfinite(Xi).all(), (what, l)
+            np.testing.assert_array_equal(Xi, Xi.T)
+            v = np.random.default_rng(l).standard_normal((n, 4))
+            u = v[:, 0].copy()
+            for _ in range(30):                      # largest eigenvalue by power iteration
+                u = A @ u
+                top = np.linalg.norm(u)
+                u /= top
+            cond = (top + lam) / lam                 # the smallest eigenvalue of F + lambda I is at least lambda
+            resid = np.linalg.norm(A @ (Xi.astype(np.float64) @ v) + lam * (Xi.astype(np.float64) @ v) - v, axis=0).max()
+            assert resid < 1e-7 * cond * np.linalg.norm(v, axis=0).min(), (what, l, n, resid, cond)
+    # the natural gradient built from them is finite
+    ngrad = dev.zeros(model.pSize)
+    info.OmegaZInv, info.LambdaGInv = oinv.value, linv.value
+    info.gradient, info.nGradient = gm.grad.value, ngrad.value
+    L.cnn.computeNaturalGradient(C.byref(model), C.byref(info), ws, None)
+    ng = dev.download(ngrad, model.pSize)
+    assert np.isfinite(ng).all() and np.abs(ng).max() > 0
+    # a descent direction: g' (F^-1 g) > 0 for a positive definite Fisher approximation
+    assert float(np.dot(ng.astype(np.float64), gm.get("grad").astype(np.float64))) > 0
+    for q in (ofac, lfac, oinv, linv, ws, ngrad):
+        dev.free(q)
+    gm.release()
