@@ -251,7 +251,7 @@ def kfac_leg(L, dev, gm, model, batch, passes):
     # factors + damped inverses of every layer, then the natural gradient of the gradient in HBM
     oinv, linv = omega, lam  # the factor storage is free again: the full passes build factors in scratch
     ngrad = dev.zeros(model.pSize)
-    info.regLambda, info.dampGamma = 1e-3, 1e-1
+    info.regLambda, info.dampGamma = 1e-3, 0.0  # the damping of the KFAC configuration
     info.OmegaZInv, info.LambdaGInv = oinv.value, linv.value
     info.gradient, info.nGradient = gm.grad.value, ngrad.value
     need = max(L.cnn.kfacInverseMemRequired(C.byref(model), batch), L.cnn.kfacNaturalGradientMemRequired(C.byref(model)))
@@ -277,7 +277,7 @@ def kfac_leg(L, dev, gm, model, batch, passes):
     dev.sync()
     out["natural_gradient_ms"] = round(1e3 * (time.perf_counter() - t0) / passes, 4)
     out["natural_gradient_finite"] = bool(np.isfinite(dev.download(ngrad, model.pSize)).all())
-    out["damping"] = 1e-3 + 1e-1
+    out["damping"] = 1e-3
     for q in (omega, lam, ws, ws2, ngrad):
         dev.free(q)
     return out

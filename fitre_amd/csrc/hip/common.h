@@ -22,7 +22,8 @@ constexpr int kGemmMirror = 1, kGemmTriK = 2;
 int gemm_ex(int transA, int transB, int M, int N, int K, float alpha, const float *A, int lda, const float *B, int ldb,
             float beta, float *C, int ldc, const float *bias, int flags, int kernelClass, void *ws, size_t wsBytes);
 size_t gemm_ex_workspace(int M, int N, int K, int flags);
-int lane();           // its index (0 or 1)
+constexpr int kMaxLanes = 4; // one hardware queue each
+int lane();           // its index (0 .. kMaxLanes - 1)
 int lane_compute_units();     // compute units a kernel launched on the selected lane can occupy
 int lane_compute_units_min(); // the smallest such count over the lanes
 int device_compute_units();

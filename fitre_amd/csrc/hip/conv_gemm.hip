@@ -7,8 +7,8 @@ namespace fitre {
 
 // Device table of the patch decode, owned by the layer and grown on demand; every use is
 // ordered on the layer's stream.
-static unsigned long long *g_ktables[2] = { nullptr, nullptr }; // one per lane
-static int g_ktable_caps[2] = { 0, 0 };
+static unsigned long long *g_ktables[kMaxLanes] = {}; // one per lane
+static int g_ktable_caps[kMaxLanes] = {};
 
 // bn = tile extent along the positions, which fixes how the waves stride through a slice
 static int attach_patch_table(PatchGeom &g, int bn)

@@ -1,8 +1,8 @@
 // Environment, memory and timing entry points of the device layer.
 // Replaces device/cuda_environment.c, device/cuda_utils.c and device/query.c
-// of the reference (handles become two streams -- "lanes" -- owned by this file:
+// of the reference (handles become four streams -- "lanes" -- owned by this file:
 // everything is queued on the selected lane, lane 0 unless a caller overlaps
-// independent work on lane 1).
+// independent work on the others).
 #include <stdarg.h>
 #include <stdlib.h>
 #include <string.h>
@@ -12,8 +12,8 @@
 namespace fitre {
 
 static thread_local char g_error[512] = "";
-constexpr int kLanes = 2;
-static hipStream_t g_lanes[kLanes] = { nullptr, nullptr };
+constexpr int kLanes = kMaxLanes;
+static hipStream_t g_lanes[kLanes] = {};
 static hipStream_t g_stream = nullptr; // the selected lane
 static int g_lane = 0;
 static bool g_lanes_on = true;
@@ -22,7 +22,7 @@ static bool g_lanes_on = true;
 // lane 0 always finds idle compute units while a chip-filling kernel runs on lane 1; the
 // planners size their grids for the lane's share.  Off unless asked for: on the gradient path
 // it measured within noise of two unmasked lanes.
-static int g_lane_cus[kLanes] = { 256, 256 };
+static int g_lane_cus[kLanes] = { 256, 256, 256, 256 };
 constexpr int kJoinEvents = 64;
 static hipEvent_t g_join[kJoinEvents];
 static int g_join_next = 0;
@@ -174,6 +174,10 @@ int fitre_hip_init(int device)
 	} else {
 		FITRE_HIP_TRY(hipStreamCreate(&g_lanes[1]));
 		g_lane_cus[1] = cus;
+	}
+	for (int i = 2; i < kLanes; i++) {
+		FITRE_HIP_TRY(hipStreamCreate(&g_lanes[i]));
+		g_lane_cus[i] = cus;
 	}
 	for (int i = 0; i < kJoinEvents; i++) FITRE_HIP_TRY(hipEventCreateWithFlags(&g_join[i], hipEventDisableTiming));
 	g_join_next = 0;

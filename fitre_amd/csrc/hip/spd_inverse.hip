@@ -146,9 +146,11 @@ size_t fitre_hip_spd_inverse_workspace(int n)
 	return inverse_layout(n).total;
 }
 
-int fitre_hip_spd_inverse(const float *matrix, int n, float shift, float *inverse, void *ws, size_t wsBytes, int *info)
+// queues the whole inverse on the selected lane; pivotInfo: device int that receives the 1-based index of the
+// first non-positive pivot, or stays zero (null: a slot of the workspace)
+static int spd_inverse_run(const float *matrix, int n, float shift, float *inverse, void *ws, size_t wsBytes, int *pivotInfo,
+                           int **infoSlot)
 {
-	FITRE_NEED_INIT();
 	FITRE_REQUIRE(matrix && inverse && ws, "fitre_hip_spd_inverse: null pointer");
 	FITRE_REQUIRE(n > 0 && n <= 23000, "fitre_hip_spd_inverse: order %d out of range", n);
 	FITRE_REQUIRE((((uintptr_t)ws) & 255) == 0, "fitre_hip_spd_inverse: workspace must be 256-byte aligned");
@@ -159,7 +161,8 @@ int fitre_hip_spd_inverse(const float *matrix, int n, float shift, float *invers
 	char *base = (char *)ws;
 	float *W = (float *)(base + lay.w), *X = (float *)(base + lay.x), *Linv = (float *)(base + lay.linv);
 	float *P = (float *)(base + lay.panel);
-	int *dInfo = (int *)(base + lay.info);
+	int *dInfo = pivotInfo ? pivotInfo : (int *)(base + lay.info);
+	if (infoSlot) *infoSlot = dInfo;
 	void *gws = base + lay.gemm;
 	const size_t gBytes = lay.gemmBytes;
 	float *T = inverse; // free until the last product
@@ -216,6 +219,15 @@ int fitre_hip_spd_inverse(const float *matrix, int n, float shift, float *invers
 	// ---- 3. A^-1 = X^T X ------------------------------------------------------------------------
 	rc = gemm_ex(1, 0, n, n, n, 1.f, X, n, X, n, 0.f, inverse, n, nullptr, kGemmMirror | kGemmTriK, KC, gws, gBytes);
 	if (rc) return rc;
+	return check_launch("fitre_hip_spd_inverse");
+}
+
+int fitre_hip_spd_inverse(const float *matrix, int n, float shift, float *inverse, void *ws, size_t wsBytes, int *info)
+{
+	FITRE_NEED_INIT();
+	int *dInfo = nullptr;
+	int rc = spd_inverse_run(matrix, n, shift, inverse, ws, wsBytes, nullptr, &dInfo);
+	if (rc) return rc;
 	if (info) {
 		int h = 0;
 		FITRE_HIP_TRY(hipMemcpyAsync(&h, dInfo, sizeof(int), hipMemcpyDeviceToHost, stream()));
@@ -223,7 +235,14 @@ int fitre_hip_spd_inverse(const float *matrix, int n, float shift, float *invers
 		*info = h;
 		if (h != 0) return fail(FITRE_E_ARGUMENT, "fitre_hip_spd_inverse: the matrix is not positive definite (pivot %d)", h);
 	}
-	return check_launch("fitre_hip_spd_inverse");
+	return FITRE_OK;
+}
+
+int fitre_hip_spd_inverse_queued(const float *matrix, int n, float shift, float *inverse, void *ws, size_t wsBytes, int *pivotInfo)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(pivotInfo != nullptr, "fitre_hip_spd_inverse_queued: null pivot slot");
+	return spd_inverse_run(matrix, n, shift, inverse, ws, wsBytes, pivotInfo, nullptr);
 }
 
 } // extern "C"

@@ -171,13 +171,71 @@ static size_t inverse_scratch_bytes(const CNN_MODEL *model, int samples, size_t 
 	return *factorBytes + round_up(ws, 256) + 256;
 }
 
+static char *aligned_base(real *devPtr) { return (char *)(((size_t)devPtr + 255) & ~(size_t)255); }
+
+/* The inverses of a pass are independent of each other: they are dealt to the four lanes, each lane with a
+ * [factor | workspace] region of its own, and the pivot reports are read once at the end. */
+#define KFAC_LANES 4
+#define KFAC_INFO_BYTES 1024 /* one int per layer, MAX_LAYERS of them */
+
 long kfacInverseMemRequired(CNN_MODEL *model, int samples)
 {
 	size_t factorBytes;
-	return (long)(inverse_scratch_bytes(model, samples, &factorBytes) / sizeof(real)) + 64;
+	return (long)((KFAC_LANES * inverse_scratch_bytes(model, samples, &factorBytes) + KFAC_INFO_BYTES) / sizeof(real)) + 64;
 }
 
-static char *aligned_base(real *devPtr) { return (char *)(((size_t)devPtr + 255) & ~(size_t)255); }
+typedef struct inverse_pass {
+	char *region[KFAC_LANES]; /* [factor | workspace] of each lane */
+	size_t factorBytes, wsBytes;
+	int *pivots;              /* device, one per layer */
+	double load[KFAC_LANES];  /* work dealt to each lane so far */
+	int layers;
+} INVERSE_PASS;
+
+static void inverse_pass_begin(INVERSE_PASS *p, const CNN_MODEL *model, int samples, real *devPtr)
+{
+	const size_t total = inverse_scratch_bytes(model, samples, &p->factorBytes);
+	char *base = aligned_base(devPtr);
+	p->pivots = (int *)base;
+	for (int k = 0; k < KFAC_LANES; k++) {
+		p->region[k] = base + KFAC_INFO_BYTES + (size_t)k * total;
+		p->load[k] = 0;
+	}
+	p->wsBytes = total - p->factorBytes - 256;
+	p->layers = model->cLayers + model->lLayers;
+	for (int k = 1; k < KFAC_LANES; k++) HIP_CALL(fitre_hip_lane_wait(k, 0)); /* after what lane 0 has queued so far (z, dx) */
+}
+
+/* the lane with the least work so far takes the next matrix of order n; returns its factor buffer */
+static real *inverse_pass_pick(INVERSE_PASS *p, int n, real **ws)
+{
+	int lane = 0;
+	for (int k = 1; k < KFAC_LANES; k++)
+		if (p->load[k] < p->load[lane]) lane = k;
+	p->load[lane] += (double)n * n; /* measured: the time of an inverse grows a little slower than n^2 */
+	HIP_CALL(fitre_hip_lane_select(lane));
+	*ws = (real *)(p->region[lane] + p->factorBytes);
+	return (real *)p->region[lane];
+}
+
+static void inverse_pass_queue(INVERSE_PASS *p, int layer, real *factor, real *inverse, int n, real *ws, real shift)
+{
+	HIP_CALL(fitre_hip_spd_inverse_queued(factor, n, shift, inverse, ws, p->wsBytes, p->pivots + layer));
+}
+
+static void inverse_pass_end(INVERSE_PASS *p)
+{
+	int host[MAX_LAYERS];
+	HIP_CALL(fitre_hip_lane_select(0));
+	HIP_CALL(fitre_hip_sync());
+	HIP_CALL(fitre_hip_copy_d2h(host, p->pivots, sizeof(int) * (size_t)p->layers));
+	for (int l = 0; l < p->layers; l++)
+		if (host[l] != 0) {
+			fprintf(stderr, "We have a problem with the LU factorization ... %d (layer %d)\n", host[l], l);
+			exit(-1);
+		}
+}
+
 
 void computeOmegaZ(KFAC_CURVATURE_INFO *kfac_info, CNN_MODEL *model, DEVICE_DATASET *data, int samples,
                    real *dampedInput, real *dampedZ, real *omegaZInv, int *zOffsets, int *zztOffsets, real *devPtr,
@@ -187,14 +245,12 @@ void computeOmegaZ(KFAC_CURVATURE_INFO *kfac_info, CNN_MODEL *model, DEVICE_DATA
 	const int *omega = kfac_info->OmegaZOffsets;
 	const int withBias = model->bias != 0;
 	const int nc = model->cLayers;
-	size_t factorBytes;
-	const size_t total = inverse_scratch_bytes(model, samples, &factorBytes);
-	char *base = aligned_base(devPtr);
-	real *zzt = (real *)base;
-	real *ws = (real *)(base + factorBytes);
-	const size_t wsBytes = total - factorBytes - 256;
+	const real shift = kfac_info->regLambda + kfac_info->dampGamma;
+	INVERSE_PASS pass;
+	inverse_pass_begin(&pass, model, samples, devPtr);
 
-	for (int l = 0; l < nc; l++) {
+	/* largest orders first, so that the two lanes end at about the same time */
+	for (int l = nc - 1; l >= 0; l--) {
 		const CONV_LAYER *c = &model->convLayer[l];
 		const real *input;
 		if (dampedInput != NULL)
@@ -203,8 +259,9 @@ void computeOmegaZ(KFAC_CURVATURE_INFO *kfac_info, CNN_MODEL *model, DEVICE_DATA
 			input = (l == 0) ? data->currentBatch : dampedZ + zOffsets[l] + model->convLayer[l - 1].outputOffset;
 		const int zCols = c->inChannels * c->kSize * c->kSize + (withBias ? 1 : 0);
 		fitre_conv_shape s = conv_shape(c, samples);
-		HIP_CALL(fitre_hip_kfac_conv_input_factor(&s, input, withBias, zzt, ws, wsBytes));
-		computeMatrixInverse(zzt, omegaZInv + omega[l], zCols, ws, kfac_info->regLambda, kfac_info->dampGamma);
+		real *ws, *zzt = inverse_pass_pick(&pass, zCols, &ws);
+		HIP_CALL(fitre_hip_kfac_conv_input_factor(&s, input, withBias, zzt, ws, pass.wsBytes));
+		inverse_pass_queue(&pass, l, zzt, omegaZInv + omega[l], zCols, ws, shift);
 	}
 	for (int l = 0; l < model->lLayers; l++) {
 		const FC_LAYER *f = &model->fcLayer[l];
@@ -216,10 +273,11 @@ void computeOmegaZ(KFAC_CURVATURE_INFO *kfac_info, CNN_MODEL *model, DEVICE_DATA
 		else
 			input = dampedZ + zOffsets[nc + l];
 		const int zRows = f->in + (withBias ? 1 : 0);
-		HIP_CALL(fitre_hip_kfac_fc_input_factor(input, f->in, samples, withBias, zzt, ws, wsBytes));
-		computeMatrixInverse(zzt, omegaZInv + omega[nc + l], zRows, ws, kfac_info->regLambda, kfac_info->dampGamma);
+		real *ws, *zzt = inverse_pass_pick(&pass, zRows, &ws);
+		HIP_CALL(fitre_hip_kfac_fc_input_factor(input, f->in, samples, withBias, zzt, ws, pass.wsBytes));
+		inverse_pass_queue(&pass, nc + l, zzt, omegaZInv + omega[nc + l], zRows, ws, shift);
 	}
-	HIP_CALL(fitre_hip_sync());
+	inverse_pass_end(&pass);
 }
 
 void computeLambdaDelta(KFAC_CURVATURE_INFO *kfac_info, CNN_MODEL *model, int samples, real *dx, real *dampedLambda,
@@ -228,14 +286,11 @@ void computeLambdaDelta(KFAC_CURVATURE_INFO *kfac_info, CNN_MODEL *model, int sa
 	(void)pageLckPtr;
 	const int *lambda = kfac_info->LambdaGOffsets;
 	const int nc = model->cLayers;
-	size_t factorBytes;
-	const size_t total = inverse_scratch_bytes(model, samples, &factorBytes);
-	char *base = aligned_base(devPtr);
-	real *ggt = (real *)base;
-	real *ws = (real *)(base + factorBytes);
-	const size_t wsBytes = total - factorBytes - 256;
+	const real shift = kfac_info->regLambda + kfac_info->dampGamma;
+	INVERSE_PASS pass;
+	inverse_pass_begin(&pass, model, samples, devPtr);
 
-	for (int l = 0; l < nc; l++) {
+	for (int l = nc - 1; l >= 0; l--) {
 		const CONV_LAYER *c = &model->convLayer[l];
 		const real *delta;
 		if (dampedLambda != NULL)
@@ -245,16 +300,18 @@ void computeLambdaDelta(KFAC_CURVATURE_INFO *kfac_info, CNN_MODEL *model, int sa
 		else
 			delta = dx + zOffsets[l + 1] + c->batchNormOffset;
 		fitre_conv_shape s = conv_shape(c, samples);
-		HIP_CALL(fitre_hip_kfac_conv_output_factor(&s, delta, ggt, ws, wsBytes));
-		computeMatrixInverse(ggt, lambdaGInv + lambda[l], c->outChannels, ws, kfac_info->regLambda, kfac_info->dampGamma);
+		real *ws, *ggt = inverse_pass_pick(&pass, c->outChannels, &ws);
+		HIP_CALL(fitre_hip_kfac_conv_output_factor(&s, delta, ggt, ws, pass.wsBytes));
+		inverse_pass_queue(&pass, l, ggt, lambdaGInv + lambda[l], c->outChannels, ws, shift);
 	}
 	for (int l = 0; l < model->lLayers; l++) {
 		const FC_LAYER *f = &model->fcLayer[l];
 		const real *delta = (dampedLambda != NULL) ? dampedLambda + zztOffsets[nc + l + 1] : dx + zOffsets[nc + l + 1];
-		HIP_CALL(fitre_hip_kfac_fc_output_factor(delta, f->out, samples, ggt, ws, wsBytes));
-		computeMatrixInverse(ggt, lambdaGInv + lambda[nc + l], f->out, ws, kfac_info->regLambda, kfac_info->dampGamma);
+		real *ws, *ggt = inverse_pass_pick(&pass, f->out, &ws);
+		HIP_CALL(fitre_hip_kfac_fc_output_factor(delta, f->out, samples, ggt, ws, pass.wsBytes));
+		inverse_pass_queue(&pass, nc + l, ggt, lambdaGInv + lambda[nc + l], f->out, ws, shift);
 	}
-	HIP_CALL(fitre_hip_sync());
+	inverse_pass_end(&pass);
 }
 
 /* ---- natural gradient ---------------------------------------------------------------------- */

@@ -43,11 +43,11 @@ int fitre_hip_device_info(int *computeUnits, int *waveSize, int *maxThreadsPerBl
                           size_t *freeBytes, char *name, int nameLen);
 /* the hipStream_t of the selected lane, as an opaque pointer */
 void *fitre_hip_stream(void);
-/* The layer owns two streams ("lanes", both at default priority).  Every call queues its work on the
- * selected lane (0 after init).  A caller that has two independent chains of work may put one on
- * lane 1 and order the chains with fitre_hip_lane_wait(waiter, signaller): work queued on `waiter`
- * after the call starts only when everything queued on `signaller` before the call has finished.
- * fitre_hip_sync() waits for both lanes.  While per-launch accounting is on (fitre_hip_profile_enable)
+/* The layer owns four streams ("lanes" 0..3, all at default priority).  Every call queues its work on the
+ * selected lane (0 after init).  A caller that has independent chains of work may put them on different
+ * lanes and order them with fitre_hip_lane_wait(waiter, signaller): work queued on `waiter` after the
+ * call starts only when everything queued on `signaller` before the call has finished.  The backward
+ * pass uses lanes 0 and 1, the KFAC inverse passes all four.  fitre_hip_sync() waits for every lane.  While per-launch accounting is on (fitre_hip_profile_enable)
  * lane selection is ignored and everything runs on lane 0, so that launch durations are unshared.
  * No counterpart in the reference, which runs on the null stream and synchronises after every launch. */
 int fitre_hip_lane_select(int lane);
@@ -377,6 +377,11 @@ int fitre_hip_cross_entropy_rop_error(const float *rz, const float *probs, int r
 size_t fitre_hip_spd_inverse_workspace(int n);
 int fitre_hip_spd_inverse(const float *matrix, int n, float shift, float *inverse, void *ws, size_t wsBytes,
                           int *info);
+/* The same inverse queued on the selected lane without waiting for it: pivotInfo is a DEVICE int that holds
+ * 0 or the index of the first non-positive pivot once the lane has drained.  Lets independent inverses run
+ * side by side on different lanes (each with its own matrix, result and workspace). */
+int fitre_hip_spd_inverse_queued(const float *matrix, int n, float shift, float *inverse, void *ws,
+                                 size_t wsBytes, int *pivotInfo);
 
 #ifdef __cplusplus
 }
