@@ -294,9 +294,6 @@ conv3x3_pos_kernel(const Conv3x3Params p, const OutParams out)
 // ---------------------------------------------------------------------------------
 // weight gradient
 // ---------------------------------------------------------------------------------
-#ifndef C3_DW_ATTR
-#define C3_DW_ATTR
-#endif
 constexpr int kC3DwThreads = 768;          // 12 waves: (output-channel block 0..3) x (tap row 0..2)
 constexpr int kC3Stage = 64;               // positions per LDS stage
 constexpr int kC3DwCin = 32;               // input channels per workgroup
@@ -320,7 +317,7 @@ constexpr int kC3DeltaLd = kC3Stage + 1;   // odd row stride of the delta stage
 // Requires positions % 64 == 0 (no partial stage).
 // MAXB: widest image row this instantiation's source window holds: 16 (for 2 <= B <= 16) or 32
 template <bool VECD, int MAXB>
-__global__ void __launch_bounds__(kC3DwThreads) C3_DW_ATTR
+__global__ void __launch_bounds__(kC3DwThreads)
 conv3x3_dw_kernel(const Conv3x3Params p, const float *delta, uint32_t deltaBytes, const OutParams out)
 {
 	constexpr int T = kC3DwThreads;

@@ -341,6 +341,32 @@ def test_fused_pool_activation_batch_norm_backward(dev, oracle64, geom, act, der
         dev.free(b)
 
 
+@pytest.mark.parametrize("kind", [MAX_POOL, NO_POOL])
+def test_fused_backward_on_a_tensor_larger_than_the_caches(dev, oracle64, kind):
+    """52 MB per tensor: the pool gradient is then written with streaming stores."""
+    Cn, N, A, B = 64, 200, 32, 32
+    oA, oB = (A // 2, B // 2) if kind == MAX_POOL else (A, B)
+    per = N * A * B
+    rng = np.random.default_rng(kind + 5)
+    zhat = rng.standard_normal(Cn * per).astype(np.float32)
+    zact = np.maximum(zhat, 0)
+    var = (0.5 + rng.random(Cn)).astype(np.float32)
+    d = rng.standard_normal(Cn * N * oA * oB).astype(np.float32)
+    pz, pd, pv = dev.upload(zhat), dev.upload(d), dev.upload(var)
+    dxp, dxa, dxb, bias = dev.zeros(zhat.size), dev.zeros(zhat.size), dev.zeros(zhat.size), dev.zeros(Cn)
+    ws, nb = bn_ws(dev, Cn, per)
+    ok(hip.fitre_hip_pool_act_bn_backward(kind, CNN_ACT_RELU, pd, 1, 0, pz, None, pv, Cn, N, A, B, 2, 2, 0, oA, oB, 1e-5, dxp, dxa,
+                                          dxb, bias, ws, nb))
+    wantp = oracle64.pool_backward(kind, d, zact, N, Cn, B, A, 2, 2, 0) if kind == MAX_POOL else d.astype(np.float64)
+    gotp, gota, gotb = (dev.download(b, zhat.size) for b in (dxp, dxa, dxb))
+    np.testing.assert_array_equal(gotp, wantp.astype(np.float32))
+    np.testing.assert_array_equal(gota, np.where(zhat > 0, gotp, np.float32(0)))
+    wantb = oracle64.batch_norm_backward(gota, zhat, var, B, A, Cn, N)
+    assert rel_err(gotb, wantb) < TOL
+    for b in (pz, pd, pv, dxp, dxa, dxb, bias, ws):
+        dev.free(b)
+
+
 def test_fused_backward_rejects_missing_activation_output(dev):
     p = dev.zeros(256)
     ws, nb = bn_ws(dev, 1, 64)
