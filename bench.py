@@ -121,6 +121,15 @@ def gpu_leg(args):
     dev.sync()
     L.check(L.hip.fitre_hip_profile_enable(0))
     rows = read_profile(L)
+    # the forward pass that produces z (not part of the metric), for orientation
+    gm.forward()
+    dev.sync()
+    t0f = time.perf_counter()
+    for _ in range(10):
+        gm.forward()
+    dev.sync()
+    forward_ms = 1e3 * (time.perf_counter() - t0f) / 10
+    gm.backward()  # dx of the last forward pass, for the legs below
     grad = gm.get("grad")
     finite = bool(np.isfinite(grad).all() and np.isfinite(loss))
     kfac = kfac_leg(L, dev, gm, model, batch, max(2, args.steps // 4))
@@ -156,7 +165,7 @@ def gpu_leg(args):
     conv["frac"] = round(conv["achieved"] / PEAK_MFMA_F32_TFLOPS, 4)
     return dict(wall=wall, ms_events=ms_events.value, batch=batch, loss=loss, finite=finite,
                 device=name.value.decode(), compute_units=cus.value, roofline=roofline, kernels=kernels,
-                conv_backward_gemms=conv, kfac_factors=kfac, bandwidth_kernels=bandwidth)
+                conv_backward_gemms=conv, kfac_factors=kfac, bandwidth_kernels=bandwidth, forward_ms=round(forward_ms, 4))
 
 
 def bandwidth_leg(L, dev, batch, reps=20):
@@ -379,6 +388,7 @@ def main():
         "conv_backward_gemms": g["conv_backward_gemms"],
         "kfac_factors": g["kfac_factors"],
         "bandwidth_kernels": g["bandwidth_kernels"],
+        "forward_ms_per_pass": g["forward_ms"],
         "kernels": g["kernels"],
         "wall_ms_per_step": round(1e3 * g["wall"] / args.steps, 4),
         "loss": round(g["loss"], 6),
