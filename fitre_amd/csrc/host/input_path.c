@@ -3,6 +3,7 @@
 #include <stdio.h>
 #include <stdlib.h>
 
+#include "fitre_cnn.h"
 #include "fitre_hip.h"
 #include "fitre_input.h"
 #include "fitre_shim.h"
@@ -103,4 +104,58 @@ void augmentData(CNN_MODEL *model, DEVICE_DATASET *data, int offset, int current
 	                                 255.f, second));
 	HIP_CALL(fitre_hip_sync());
 	data->currentBatch = second;
+}
+
+/* One evaluation sweep in batches of model->batchSize (the last one shorter): copy the batch's columns
+ * and labels, layout change + normalisation (no augmentation), forward pass, accuracy.
+ * functions/cnn_accuracy.cu:61-110 (test set) and :112-174 (training set; the reference's sweep stops
+ * before a final short batch yet divides by the full size, and so does this one). */
+static void generalization_sweep(CNN_MODEL *model, DEVICE_DATASET *data, SCRATCH_AREA *scratch, real *z, real *probs,
+                                 real *errors, const real *setX, const real *setY, int setSize, EVAL_TYPE mode,
+                                 int dropShortTail, real *likelihood, real *accuracy)
+{
+	real hits = 0;
+	int curIdx = 0, curBatchSize = model->batchSize;
+	real *nextDevPtr = scratch->nextDevPtr, *nextHostPtr = scratch->nextHostPtr, *nextPageLckPtr = scratch->nextPageLckPtr;
+	*likelihood = 0;
+	*accuracy = 0;
+	if (curBatchSize > setSize) curBatchSize = setSize;
+	while (curIdx < setSize && curBatchSize > 0) {
+		HIP_CALL(fitre_hip_copy_d2d(data->sampledTrainX, setX + (size_t)data->features * curIdx,
+		                            sizeof(real) * (size_t)data->features * curBatchSize));
+		HIP_CALL(fitre_hip_copy_d2d(data->sampledTrainY, setY + curIdx, sizeof(real) * (size_t)curBatchSize));
+		augmentData(model, data, curIdx, curBatchSize, nextDevPtr, nextHostPtr, 0, data->datasetType);
+		real batchLikelihood = cnnForward(model, data, scratch, z, probs, errors, curIdx, curBatchSize, mode);
+		*likelihood += batchLikelihood * curBatchSize;
+		computeAccuracy(probs, (real *)(setY + curIdx), curBatchSize, data->numClasses, nextDevPtr, nextPageLckPtr);
+		hits += *nextPageLckPtr;
+		curIdx += curBatchSize;
+		if (curIdx + model->batchSize < setSize) {
+			curBatchSize = model->batchSize;
+		} else {
+			curBatchSize = setSize - curIdx;
+			if (dropShortTail) break;
+		}
+	}
+	*accuracy = hits * (real)100. / (real)setSize;
+	*likelihood /= (real)setSize;
+}
+
+void computeTestGeneralizationErrors(CNN_MODEL *model, DEVICE_DATASET *data, SCRATCH_AREA *scratch, real *z, real *probs,
+                                     real *errors, real *likelihood, real *accuracy)
+{
+	generalization_sweep(model, data, scratch, z, probs, errors, data->testSetX, data->testSetY, data->testSizeX,
+	                     MODEL_TEST_ACCURACY, 0, likelihood, accuracy);
+}
+
+void computeTrainGeneralizationErrors(CNN_MODEL *model, DEVICE_DATASET *data, HOST_DATASET *host, SCRATCH_AREA *scratch, real *z,
+                                      real *probs, real *errors, real *likelihood, real *accuracy)
+{
+	(void)host; /* the reference reads it for data sets kept in host memory only */
+	if (data->datasetType == IMAGENET) {
+		fprintf(stderr, "computeTrainGeneralizationErrors: data sets kept in host memory are not supported\n");
+		exit(-1);
+	}
+	generalization_sweep(model, data, scratch, z, probs, errors, data->trainSetX, data->trainSetY, data->trainSizeX,
+	                     MODEL_TRAIN_ACCURACY, 1, likelihood, accuracy);
 }

@@ -152,6 +152,8 @@ CNN_API = {
     "flipData": (None, [vp, vp, i32, i32, i32, i32, vp, vp, vp]),
     "normalizeCIFAR10": (None, [vp, i32, i32, i32, i32, vp, vp, i32]),
     "augmentData": (None, [pmodel, pdata, i32, i32, vp, vp, i32, i32]),
+    "computeTestGeneralizationErrors": (None, [pmodel, pdata, pscratch, vp, vp, vp, pf32, pf32]),
+    "computeTrainGeneralizationErrors": (None, [pmodel, pdata, vp, pscratch, vp, vp, vp, pf32, pf32]),
     # include/fitre_kfac.h
     "computeKFACStorageIndices": (None, [pmodel, pkfac]),
     "kfacFactorsMemRequired": (lng, [pmodel, i32]),

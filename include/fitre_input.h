@@ -40,6 +40,16 @@ void normalizeCIFAR10(real *input, int samples, int channels, int height, int wi
 void augmentData(CNN_MODEL *model, DEVICE_DATASET *data, int offset, int currentBatchSize, real *devPtr, real *hostPtr,
                  int enableDA, DATASET_TYPE datasetType);
 
+/* functions/cnn_accuracy.cu:61-174: mean negative log-likelihood and accuracy (percent) over the whole test
+ * resp. training set, in batches of model->batchSize through augmentData (no augmentation) and cnnForward.
+ * The sets are device-resident, features x size column-major; pixel values 0..255; data->sampledTrainX must
+ * hold two batches (augmentData writes the second), scratch->nextDevPtr cnnForwardMemRequired reals,
+ * scratch->nextPageLckPtr one real of host memory.  Batch-norm layers use their running statistics. */
+void computeTestGeneralizationErrors(CNN_MODEL *model, DEVICE_DATASET *data, SCRATCH_AREA *scratch, real *z, real *probs,
+                                     real *errors, real *likelihood, real *accuracy);
+void computeTrainGeneralizationErrors(CNN_MODEL *model, DEVICE_DATASET *data, HOST_DATASET *host, SCRATCH_AREA *scratch,
+                                      real *z, real *probs, real *errors, real *likelihood, real *accuracy);
+
 #ifdef __cplusplus
 }
 #endif

@@ -140,3 +140,55 @@ def test_select_and_augment_with_the_reference_names(dev, oracle64, enable, data
     if enable:
         plain = oracle64.augment_data(X.reshape(train, feats)[picked].reshape(-1), N, C_, H, W, 0, cu, fu, np.float32(mean), np.float32(std))
         assert rel_err(got, plain) > 1e-3   # the augmentation did move pixels
+
+
+def test_generalization_error_sweeps(dev, oracle64):
+    """computeTestGeneralizationErrors / computeTrainGeneralizationErrors (functions/cnn_accuracy.cu:61-174): whole-set
+    loss and accuracy in batches, against the oracle's forward pass on the oracle's normalised batches.  20 images in
+    batches of 8: the test sweep ends with a batch of 4, the training sweep stops before it (as the reference does)
+    and still divides by 20."""
+    from helpers import GpuModel, he_weights
+    rng = np.random.default_rng(31)
+    batch, size, classes = 8, 20, 10
+    model = build_lenet(batch)
+    feats = 3 * 32 * 32
+    X = rng.integers(0, 256, size=(size, feats)).astype(np.float32)
+    Y = rng.integers(1, classes + 1, size=size).astype(np.float32)
+    w = he_weights(model, rng).astype(np.float32) * np.float32(0.3)
+    gm = GpuModel(dev, model, w, np.zeros(batch * feats, np.float32), np.ones(batch, np.float32), batch)
+    data = gm.data
+    setX, setY = dev.upload(X.reshape(-1)), dev.upload(Y)
+    sampledX, sampledY = dev.zeros(2 * batch * feats), dev.zeros(batch)
+    data.trainSetX, data.trainSetY, data.testSetX, data.testSetY = setX.value, setY.value, setX.value, setY.value
+    data.trainSizeX, data.testSizeX, data.features, data.datasetType = size, size, feats, CIFAR10
+    data.sampledTrainX, data.sampledTrainY = sampledX.value, sampledY.value
+    pinned = (C.c_float * 4)()
+    gm.scratch.nextPageLckPtr = C.cast(pinned, C.c_void_p).value
+    mean, std = STATS[CIFAR10]
+
+    def reference(limit_full_batches):
+        nll, hits, idx = 0.0, 0, 0
+        while idx < size:
+            n = min(batch, size - idx)
+            if limit_full_batches and n < batch:
+                break
+            xb = oracle64.augment_data(X[idx:idx + n].reshape(-1), n, 3, 32, 32, 0, np.zeros(2 * n), np.zeros(n),
+                                       np.float32(mean), np.float32(std))
+            loss, _, probs, _ = oracle64.forward(model, w, xb, Y[idx:idx + n], classes, n, mode=30)
+            nll += loss * n
+            hits += int((np.argmax(probs.reshape(n, classes), axis=1) + 1 == Y[idx:idx + n]).sum())
+            idx += n
+        return nll / size, 100.0 * hits / size
+
+    like, acc = C.c_float(), C.c_float()
+    L.cnn.computeTestGeneralizationErrors(C.byref(model), C.byref(data), C.byref(gm.scratch), gm.z, gm.probs, gm.errors,
+                                          C.byref(like), C.byref(acc))
+    want_l, want_a = reference(False)
+    assert abs(like.value - want_l) < 1e-4 * abs(want_l) and abs(acc.value - want_a) < 1e-4
+    L.cnn.computeTrainGeneralizationErrors(C.byref(model), C.byref(data), None, C.byref(gm.scratch), gm.z, gm.probs, gm.errors,
+                                           C.byref(like), C.byref(acc))
+    want_l, want_a = reference(True)
+    assert abs(like.value - want_l) < 1e-4 * abs(want_l) and abs(acc.value - want_a) < 1e-4
+    for q in (setX, setY, sampledX, sampledY):
+        dev.free(q)
+    gm.release()
