@@ -136,6 +136,7 @@ def gpu_leg(args):
     kfac["hessian_vector_ms"] = hv_leg(L, dev, gm, model, batch, max(2, args.steps // 4))
     gm.release()
     bandwidth = bandwidth_leg(L, dev, batch)
+    others = other_configs_leg(L, dev)
     dev.close()
 
     kernels = {}
@@ -165,7 +166,36 @@ def gpu_leg(args):
     conv["frac"] = round(conv["achieved"] / PEAK_MFMA_F32_TFLOPS, 4)
     return dict(wall=wall, ms_events=ms_events.value, batch=batch, loss=loss, finite=finite,
                 device=name.value.decode(), compute_units=cus.value, roofline=roofline, kernels=kernels,
-                conv_backward_gemms=conv, kfac_factors=kfac, bandwidth_kernels=bandwidth, forward_ms=round(forward_ms, 4))
+                conv_backward_gemms=conv, kfac_factors=kfac, bandwidth_kernels=bandwidth, forward_ms=round(forward_ms, 4),
+                other_configs=others)
+
+
+def other_configs_leg(L, dev, steps=10):
+    """Backward images/sec of the other benchmark networks (the same step: copy of the loss errors + one
+    cnnBackward), for orientation: LeNet-style b128, the same with batch norm b1024, AlexNet-style
+    3x224x224 b64 with 1000 classes."""
+    from helpers import GpuModel, batch_inputs, build_alexnet, build_lenet, he_weights
+    out = {}
+    for name, build, batch in (("lenet_b128", lambda: build_lenet(128), 128),
+                               ("lenet_bn_b1024", lambda: build_lenet(1024, bn=True), 1024),
+                               ("alexnet_224_b64", lambda: build_alexnet(64), 64)):
+        model = build()
+        rng = np.random.default_rng(0xF17E0005 + batch)
+        w = he_weights(model, rng).astype(np.float32)
+        x, y = batch_inputs(model, batch, rng)
+        gm = GpuModel(dev, model, w, x.astype(np.float32), y, batch)
+        gm.forward()
+        gm.backward()
+        dev.sync()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            gm.backward()
+        dev.sync()
+        dt = time.perf_counter() - t0
+        out[name] = dict(images_per_s=round(batch * steps / dt, 1), ms_per_step=round(1e3 * dt / steps, 4),
+                         finite=bool(np.isfinite(gm.get("grad")).all()))
+        gm.release()
+    return out
 
 
 def bandwidth_leg(L, dev, batch, reps=20):
@@ -389,6 +419,7 @@ def main():
         "kfac_factors": g["kfac_factors"],
         "bandwidth_kernels": g["bandwidth_kernels"],
         "forward_ms_per_pass": g["forward_ms"],
+        "other_configs": g["other_configs"],
         "kernels": g["kernels"],
         "wall_ms_per_step": round(1e3 * g["wall"] / args.steps, 4),
         "loss": round(g["loss"], 6),
