@@ -180,6 +180,52 @@ pool_backward_kernel(const float *delta, const float *z_in, const float *z_act, 
 	}
 }
 
+// Overlapping max-pool windows (e.g. 3x3 / stride 2): one workgroup per map keeps the map and the
+// arg-max of every window in LDS, so a window is scanned once instead of once per cell it contains
+// (up to four times for 3/2), and each cell then looks up the windows it belongs to.  Same scan and
+// the same order of additions as pool_backward_kernel<0>: identical results.  Maps of up to
+// kPoolMapCells cells and kPoolMapWindows windows.
+constexpr int kPoolMapCells = 4096, kPoolMapWindows = 1280;
+template <bool FUSE_ACT>
+__global__ void __launch_bounds__(256)
+maxpool_map_backward_kernel(const float *delta, const float *z_in, const float *z_act, PoolGeom g, int actFun, float *dxPool,
+                            float *dxAct)
+{
+	__shared__ float zmap[kPoolMapCells];
+	__shared__ int arg[kPoolMapWindows];
+	const int cells = g.inA * g.inB, windows = g.outA * g.outB;
+	const size_t mapOff = (size_t)blockIdx.x * cells;
+	const float *dmap = delta + (size_t)blockIdx.x * windows;
+	for (int i = threadIdx.x; i < cells; i += blockDim.x) zmap[i] = z_act[mapOff + i];
+	__syncthreads();
+	for (int w = threadIdx.x; w < windows; w += blockDim.x) {
+		uint32_t oa, ob;
+		g.divOutB.divmod((uint32_t)w, oa, ob);
+		float best;
+		arg[w] = window_argmax(zmap, g, (int)oa, (int)ob, best);
+	}
+	__syncthreads();
+	for (int i = threadIdx.x; i < cells; i += blockDim.x) {
+		uint32_t a, b;
+		g.divInB.divmod((uint32_t)i, a, b);
+		int oaHi = ((int)a + g.padding) / g.stride, obHi = ((int)b + g.padding) / g.stride;
+		int oaLo = ((int)a + g.padding - g.ksize + g.stride) / g.stride, obLo = ((int)b + g.padding - g.ksize + g.stride) / g.stride;
+		if ((int)a + g.padding - g.ksize + 1 <= 0) oaLo = 0;
+		if ((int)b + g.padding - g.ksize + 1 <= 0) obLo = 0;
+		if (oaHi >= g.outA) oaHi = g.outA - 1;
+		if (obHi >= g.outB) obHi = g.outB - 1;
+		float acc = 0.f;
+		for (int oa = oaLo; oa <= oaHi; oa++)
+			for (int ob = obLo; ob <= obHi; ob++)
+				if (arg[oa * g.outB + ob] == i) acc += dmap[oa * g.outB + ob];
+		if (dxPool) dxPool[mapOff + i] = acc;
+		if constexpr (FUSE_ACT) {
+			const float zi = z_in ? z_in[mapOff + i] : 0.f;
+			dxAct[mapOff + i] = acc * act_derivative(actFun, zi, zmap[i]);
+		}
+	}
+}
+
 // strict-> scan of four values in order, starting below every finite float
 __device__ __forceinline__ int scan2x2(float v0, float v1, float v2, float v3)
 {
@@ -1070,9 +1116,14 @@ int fitre_hip_pool_act_backward(int poolType, int actFun, const float *delta, co
 		bool fast = ksize == 2 && stride == 2 && padding == 0 && (inB % 4 == 0) && (inA % 2 == 0) && aligned16(z_act) &&
 		            aligned16(dxAct) && (!dxPool || aligned16(dxPool)) && (!z_in || aligned16(z_in)) &&
 		            (((uintptr_t)delta & 7) == 0);
+		const bool perMap = !fast && inA * inB <= kPoolMapCells && outA * outB <= kPoolMapWindows && inA * inB >= 64 &&
+		                    maps <= 0x7fffffffL;
 		if (fast)
 			maxpool2_backward_kernel<true><<<blocks_for(total / 8, 256, 16384), 256, 0, stream()>>>(
 			    delta, act_needs_zin(actFun) ? z_in : nullptr, z_act, inA, inB, maps, actFun, dxPool, dxAct);
+		else if (perMap)
+			maxpool_map_backward_kernel<true><<<(unsigned)maps, 256, 0, stream()>>>(delta, act_needs_zin(actFun) ? z_in : nullptr, z_act, g,
+			                                                                      actFun, dxPool, dxAct);
 		else
 			pool_backward_kernel<0, true><<<blocks, 256, 0, stream()>>>(delta, z_in, z_act, g, maps, actFun, dxPool, dxAct);
 	} else if (poolType == AVG_POOL) {
@@ -1101,9 +1152,13 @@ int fitre_hip_pool_backward(int poolType, const float *delta, const float *z_in,
 	if (poolType == MAX_POOL) {
 		bool fast = ksize == 2 && stride == 2 && padding == 0 && (inB % 4 == 0) && (inA % 2 == 0) && aligned16(z_in) &&
 		            aligned16(out) && (((uintptr_t)delta & 7) == 0);
+		const bool perMap = !fast && inA * inB <= kPoolMapCells && outA * outB <= kPoolMapWindows && inA * inB >= 64 &&
+		                    maps <= 0x7fffffffL;
 		if (fast)
 			maxpool2_backward_kernel<false><<<blocks_for(total / 8, 256, 16384), 256, 0, stream()>>>(
 			    delta, nullptr, z_in, inA, inB, maps, CNN_ACT_NONE, out, nullptr);
+		else if (perMap)
+			maxpool_map_backward_kernel<false><<<(unsigned)maps, 256, 0, stream()>>>(delta, nullptr, z_in, g, CNN_ACT_NONE, out, nullptr);
 		else
 			pool_backward_kernel<0, false><<<blocks, 256, 0, stream()>>>(delta, nullptr, z_in, g, maps, CNN_ACT_NONE, out, nullptr);
 	} else if (poolType == AVG_POOL) {

@@ -148,6 +148,11 @@ POOL_GEOMS = [  # C, N, A(width), B(height), k, s, p
     (2, 2, 6, 6, 3, 1, 0),      # heavily overlapping
     (8, 1, 2, 2, 3, 2, 1),      # drivers/pool_driver.cu
     (2, 2, 5, 5, 2, 2, 0),      # odd extent: last row/column unpooled
+    # maps of 64 cells and more with overlapping windows: the one-workgroup-per-map kernel
+    (2, 3, 9, 11, 3, 2, 1),     # 3/2/1 on a rectangular map
+    (4, 2, 55, 55, 3, 2, 0),    # AlexNet's first pool
+    (2, 2, 12, 12, 3, 1, 1),    # stride 1: every cell in up to nine windows
+    (3, 2, 16, 16, 2, 2, 1),    # 2x2 with padding (not the 16-byte fast path)
 ]
 
 
@@ -180,7 +185,7 @@ def test_pool_forward_backward(dev, oracle64, geom, kind):
 
 def test_max_pool_ties_are_bit_exact(dev, oracle64):
     # all-equal windows (post-ReLU zeros), two-way ties, negative ties; 2x2 fast path and generic path
-    for (A, B, k, s, p) in [(4, 4, 2, 2, 0), (4, 8, 2, 2, 0), (5, 5, 3, 2, 1), (6, 6, 3, 1, 0)]:
+    for (A, B, k, s, p) in [(4, 4, 2, 2, 0), (4, 8, 2, 2, 0), (5, 5, 3, 2, 1), (6, 6, 3, 1, 0), (13, 13, 3, 2, 0), (10, 9, 3, 1, 1)]:
         rng = np.random.default_rng(A * B)
         x = rng.integers(-1, 2, size=3 * 2 * A * B).astype(np.float32)  # values in {-1, 0, 1}: ties everywhere
         oA, oB = (A + 2 * p - k) // s + 1, (B + 2 * p - k) // s + 1
@@ -194,7 +199,7 @@ def test_max_pool_ties_are_bit_exact(dev, oracle64):
         np.testing.assert_array_equal(dev.download(back, x.size), oracle64.pool_backward(0, d, x, 2, 3, B, A, k, s, p).astype(np.float32))
 
 
-@pytest.mark.parametrize("geom", POOL_GEOMS[:4])
+@pytest.mark.parametrize("geom", POOL_GEOMS[:4] + POOL_GEOMS[7:])
 @pytest.mark.parametrize("act", [CNN_ACT_RELU, CNN_ACT_SWISH, CNN_ACT_SOFTPLUS, CNN_ACT_NONE])
 @pytest.mark.parametrize("kind", [MAX_POOL, AVG_POOL, NO_POOL])
 def test_fused_pool_activation_backward(dev, oracle64, geom, act, kind):
