@@ -42,7 +42,14 @@
  * pytorch/testing/my.out:9; brute-force direct convolution and its adjoint
  * identities; float64 autograd of the textbook layers; a Taylor remainder
  * test of the whole gradient (utilities/cnn_derivative_test.cu:197-199);
- * the logged LeNet parameter offsets.  No function here is "parity unpinned".
+ * the logged LeNet parameter offsets; the Kronecker factors against unfold
+ * patches and numpy Gram products; the inverse against scipy's Cholesky
+ * solver; the natural gradient against a Kronecker-product solve; the fully
+ * connected model family against autograd of each head's loss; the
+ * Hessian-vector product against float64 double backward, its symmetry and
+ * the second-order Taylor remainder; the input pipeline against numpy
+ * pad/slice, flip, transposes and the closed-form normalisation.
+ * No function here is "parity unpinned".
  */
 #include <float.h>
 #include <limits.h>
