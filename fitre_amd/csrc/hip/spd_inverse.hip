@@ -2,13 +2,13 @@
 // reference obtains from cusolverDnDpotrf + cusolverDnDpotrs with an identity right-hand side
 // (solvers/kfac_inverses.cu:133-186), for the KFAC factors (order up to Cin*k*k + 1 = 4609).
 //
-//   1. W = A + shift*I = L L^T      blocked right-looking Cholesky, 64-wide block columns:
-//                                   a one-wave kernel factors the diagonal block and inverts its
-//                                   factor, the panel and the symmetric trailing update are
-//                                   products on the MFMA tile engine;
-//   2. X = L^-1                     pairwise block recursion  [X11 0; -X22 L21 X11, X22]  bottom-up,
-//                                   two engine products per pair;
-//   3. A^-1 = X^T X                 one symmetric engine product whose reduction skips the zero
+//   1. W = A + shift*I = L L^T and X = L^-1 together, by halving: for W = [A11 .; A21 A22]
+//        (L11, X11) of A11;  L21 = A21 X11^T;  A22 -= L21 L21^T;  (L22, X22) of that;
+//        X21 = -X22 (L21 X11).
+//      Every product is as large as the halves it joins (rank n/2, n/4, ... updates on the MFMA
+//      tile engine instead of n/64 rank-64 ones), and a 64 x 64 leaf is one one-wave kernel that
+//      factors the block and inverts its factor;
+//   2. A^-1 = X^T X                 one symmetric engine product whose reduction skips the zero
 //                                   part of the triangular operand.
 // All matrices are column-major with leading dimension n; only lower triangles are meaningful
 // in W and X (X's upper triangle is kept at zero).
@@ -106,32 +106,84 @@ struct InverseLayout {
 
 static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
+// largest split-K workspace the products of a node of `blocks` 64-wide block columns (order nn) ask for
+static size_t node_gemm_workspace(int blocks, int nn)
+{
+	if (blocks <= 1) return 0;
+	const int b1 = blocks / 2, n1 = b1 * kNb, m = nn - n1;
+	size_t g = gemm_ex_workspace(m, n1, n1, 0);
+	size_t a = gemm_ex_workspace(m, m, n1, kGemmMirror);
+	g = a > g ? a : g;
+	a = gemm_ex_workspace(m, n1, m, 0);
+	g = a > g ? a : g;
+	a = node_gemm_workspace(b1, n1);
+	g = a > g ? a : g;
+	a = node_gemm_workspace(blocks - b1, m);
+	return a > g ? a : g;
+}
+
 static InverseLayout inverse_layout(int n)
 {
 	InverseLayout l;
 	const size_t nn = (size_t)n * n * sizeof(float);
 	const int blocks = (n + kNb - 1) / kNb;
-	size_t g = 0;
-	// the largest split workspaces the products below can ask for
-	g = gemm_ex_workspace(n, n, kNb, kGemmMirror) > g ? gemm_ex_workspace(n, n, kNb, kGemmMirror) : g;
-	g = gemm_ex_workspace(n, kNb, kNb, 0) > g ? gemm_ex_workspace(n, kNb, kNb, 0) : g;
-	for (int s = kNb; s < n; s *= 2) {
-		int m = (s < n - s) ? s : n - s; // rows of the lower block can be up to s
-		size_t a = gemm_ex_workspace(s, s, s, 0);
-		g = a > g ? a : g;
-		(void)m;
-	}
+	size_t g = node_gemm_workspace(blocks, n);
 	size_t c = gemm_ex_workspace(n, n, n, kGemmMirror);
 	g = c > g ? c : g;
 	l.w = 0;
 	l.x = align256(l.w + nn);
 	l.linv = align256(l.x + nn);
-	l.panel = align256(l.linv + (size_t)blocks * kNb * kNb * sizeof(float));
-	l.info = align256(l.panel + (size_t)n * kNb * sizeof(float));
+	l.panel = align256(l.linv + (size_t)kNb * kNb * sizeof(float));
+	l.info = l.panel; // no panel buffer: the products' temporaries live in the result matrix
 	l.gemm = align256(l.info + 256);
 	l.gemmBytes = align256(g + 256);
 	l.total = l.gemm + l.gemmBytes;
 	return l;
+}
+
+// state of one inverse while its launches are queued
+struct InverseRun {
+	float *W, *X, *Linv, *T, *T2; // T, T2: temporaries of up to (n/2 + 64) x n/2 each, inside the result matrix
+	int n;
+	int *dInfo;
+	void *gws;
+	size_t gBytes;
+};
+
+// L and X = L^-1 of the diagonal block of `blocks` block columns that starts at row/column r0 (order nn)
+static int chol_and_inverse(const InverseRun &r, int r0, int blocks, int nn)
+{
+	const int KC = FITRE_KC_SPD_INVERSE;
+	const int n = r.n;
+	if (blocks == 1) {
+		{
+			LaunchScope scope(KC, 2.0 * kNb * kNb * kNb / 3.0);
+			chol_diag_kernel<<<1, 64, 0, stream()>>>(r.W, n, r0, nn, r.Linv, r.dInfo);
+		}
+		block_copy_kernel<<<blocks_for((long)nn * nn, 256, 64), 256, 0, stream()>>>(r.Linv, kNb, r.X + (size_t)r0 * n + r0, n, nn, nn);
+		return check_launch("chol_diag_kernel");
+	}
+	const int b1 = blocks / 2, n1 = b1 * kNb, m = nn - n1, r1 = r0 + n1;
+	int rc = chol_and_inverse(r, r0, b1, n1);
+	if (rc) return rc;
+	float *A21 = r.W + (size_t)r0 * n + r1;
+	float *A22 = r.W + (size_t)r1 * n + r1;
+	const float *X11 = r.X + (size_t)r0 * n + r0;
+	// L21 = A21 * X11^T (m x n1), through T, then back into W
+	rc = gemm_ex(0, 1, m, n1, n1, 1.f, A21, n, X11, n, 0.f, r.T, m, nullptr, 0, KC, r.gws, r.gBytes);
+	if (rc) return rc;
+	block_copy_kernel<<<blocks_for((long)m * n1, 256, 8192), 256, 0, stream()>>>(r.T, m, A21, n, m, n1);
+	// A22 -= L21 L21^T
+	rc = gemm_ex(0, 1, m, m, n1, -1.f, r.T, m, r.T, m, 1.f, A22, n, nullptr, kGemmMirror, KC, r.gws, r.gBytes);
+	if (rc) return rc;
+	rc = chol_and_inverse(r, r1, blocks - b1, m);
+	if (rc) return rc;
+	// X21 = -X22 * (L21 * X11)
+	const float *X22 = r.X + (size_t)r1 * n + r1;
+	float *X21 = r.X + (size_t)r0 * n + r1;
+	rc = gemm_ex(0, 0, m, n1, n1, 1.f, A21, n, X11, n, 0.f, r.T2, m, nullptr, 0, KC, r.gws, r.gBytes);
+	if (rc) return rc;
+	return gemm_ex(0, 0, m, n1, m, -1.f, X22, n, r.T2, m, 0.f, X21, n, nullptr, 0, KC, r.gws, r.gBytes);
 }
 
 } // namespace fitre
@@ -160,12 +212,10 @@ static int spd_inverse_run(const float *matrix, int n, float shift, float *inver
 		            lay.total);
 	char *base = (char *)ws;
 	float *W = (float *)(base + lay.w), *X = (float *)(base + lay.x), *Linv = (float *)(base + lay.linv);
-	float *P = (float *)(base + lay.panel);
 	int *dInfo = pivotInfo ? pivotInfo : (int *)(base + lay.info);
 	if (infoSlot) *infoSlot = dInfo;
 	void *gws = base + lay.gemm;
 	const size_t gBytes = lay.gemmBytes;
-	float *T = inverse; // free until the last product
 	const int blocks = (n + kNb - 1) / kNb;
 	const int KC = FITRE_KC_SPD_INVERSE;
 	int rc;
@@ -176,47 +226,14 @@ static int spd_inverse_run(const float *matrix, int n, float shift, float *inver
 		fill_zero_kernel<<<blocks_for((long)n * n, 256, 8192), 256, 0, stream()>>>(X, (long)n * n);
 		fill_zero_kernel<<<1, 64, 0, stream()>>>((float *)dInfo, 1);
 	}
-	// ---- 1. Cholesky ----------------------------------------------------------------------------
-	for (int b = 0; b < blocks; b++) {
-		const int k0 = b * kNb, nb = (n - k0 < kNb) ? n - k0 : kNb, m = n - k0 - nb;
-		{
-			LaunchScope scope(KC, 2.0 * kNb * kNb * kNb / 3.0);
-			chol_diag_kernel<<<1, 64, 0, stream()>>>(W, n, k0, nb, Linv + (size_t)b * kNb * kNb, dInfo);
-		}
-		if (m <= 0) break;
-		float *A21 = W + (size_t)k0 * n + k0 + nb;
-		// L21 = A21 * L11^-T  (m x nb) through the panel buffer, then back into W
-		rc = gemm_ex(0, 1, m, nb, nb, 1.f, A21, n, Linv + (size_t)b * kNb * kNb, kNb, 0.f, P, m, nullptr, 0, KC, gws, gBytes);
-		if (rc) return rc;
-		block_copy_kernel<<<blocks_for((long)m * nb, 256, 4096), 256, 0, stream()>>>(P, m, A21, n, m, nb);
-		// A22 -= L21 L21^T
-		float *A22 = W + (size_t)(k0 + nb) * n + k0 + nb;
-		rc = gemm_ex(0, 1, m, m, nb, -1.f, P, m, P, m, 1.f, A22, n, nullptr, kGemmMirror, KC, gws, gBytes);
-		if (rc) return rc;
-	}
-	// ---- 2. X = L^-1 ----------------------------------------------------------------------------
-	for (int b = 0; b < blocks; b++) {
-		const int k0 = b * kNb, nb = (n - k0 < kNb) ? n - k0 : kNb;
-		block_copy_kernel<<<blocks_for((long)nb * nb, 256, 64), 256, 0, stream()>>>(Linv + (size_t)b * kNb * kNb, kNb,
-		                                                                           X + (size_t)k0 * n + k0, n, nb, nb);
-	}
-	for (int s = 1; s < blocks; s *= 2) {
-		for (int lo = 0; lo + s < blocks; lo += 2 * s) {
-			const int mid = lo + s, hi = (lo + 2 * s < blocks) ? lo + 2 * s : blocks;
-			const int r1 = lo * kNb, m1 = s * kNb;
-			const int r2 = mid * kNb, m2 = ((hi * kNb < n) ? hi * kNb : n) - r2;
-			const float *L21 = W + (size_t)r1 * n + r2;
-			const float *X11 = X + (size_t)r1 * n + r1;
-			const float *X22 = X + (size_t)r2 * n + r2;
-			float *X21 = X + (size_t)r1 * n + r2;
-			// T = L21 * X11 (m2 x m1), X21 = -X22 * T
-			rc = gemm_ex(0, 0, m2, m1, m1, 1.f, L21, n, X11, n, 0.f, T, m2, nullptr, 0, KC, gws, gBytes);
-			if (rc) return rc;
-			rc = gemm_ex(0, 0, m2, m1, m2, -1.f, X22, n, T, m2, 0.f, X21, n, nullptr, 0, KC, gws, gBytes);
-			if (rc) return rc;
-		}
-	}
-	// ---- 3. A^-1 = X^T X ------------------------------------------------------------------------
+	// ---- 1. Cholesky factor and its inverse ---------------------------------------------------
+	InverseRun run;
+	run.W = W, run.X = X, run.Linv = Linv, run.n = n, run.dInfo = dInfo, run.gws = gws, run.gBytes = gBytes;
+	run.T = inverse;                              // the result matrix is free until the last product
+	run.T2 = inverse + ((size_t)n * n + 1) / 2;   // each temporary is at most (n/2 + 32) x n/2 <= n*n/2 floats
+	rc = chol_and_inverse(run, 0, blocks, n);
+	if (rc) return rc;
+	// ---- 2. A^-1 = X^T X ------------------------------------------------------------------------
 	rc = gemm_ex(1, 0, n, n, n, 1.f, X, n, X, n, 0.f, inverse, n, nullptr, kGemmMirror | kGemmTriK, KC, gws, gBytes);
 	if (rc) return rc;
 	return check_launch("fitre_hip_spd_inverse");
