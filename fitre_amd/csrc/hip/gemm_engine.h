@@ -636,7 +636,7 @@ inline double estimate_us(long tiles, int bm, int bn, long I, long J, long R, lo
 	double stepUs = (double)(bm / 32) * (bn / 32) * (kGemmBK / 2) * 64.0 / 4.0 / 2400.0;
 	double eff = perCu >= 3 ? 0.80 : (perCu == 2 ? 0.68 : 0.52);
 	double t = (double)perCu * (double)(chunk / kGemmBK) * stepUs / eff + 3.0;
-	if (s > 1) t += 4.0 + (double)(s + 1) * (double)I * (double)J * 4.0 / 3.0e6; // ~3 TB/s, bytes -> us
+	if (s > 1) t += 8.0 + (double)(s + 1) * (double)I * (double)J * 4.0 / 3.0e6; // second launch; ~3 TB/s, bytes -> us
 	*chunkOut = chunk;
 	*splitsOut = s;
 	return t;

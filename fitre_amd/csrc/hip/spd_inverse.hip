@@ -25,11 +25,11 @@ __device__ __forceinline__ float lane_value(float v, int lane)
 }
 
 // One wave factors the nb x nb (nb <= 64) diagonal block in place (lower triangle) and writes the
-// inverse of the factor, 64 x 64 column-major, padded with the identity.  Lane i holds row i in
+// inverse of the factor into the same block of Xout (lower triangle, leading dimension ld).  Lane i holds row i in
 // registers; what a step needs from another lane's row comes through v_readlane as a scalar, so
 // there is no LDS traffic and no barrier in the 2 x 2016 multiply-adds.
 // info: set to the 1-based global index of the first non-positive pivot.
-__global__ void __launch_bounds__(64) chol_diag_kernel(float *W, int ld, int k0, int nb, float *Linv, int *info)
+__global__ void __launch_bounds__(64) chol_diag_kernel(float *W, int ld, int k0, int nb, float *Xout, int *info)
 {
 	const int i = threadIdx.x;
 	float a[kNb];
@@ -68,8 +68,15 @@ __global__ void __launch_bounds__(64) chol_diag_kernel(float *W, int ld, int k0,
 		}
 		x[r] = (acc0 + acc1) * rdiag[r];
 	}
+	// x[r] is element (r, i) of the inverse, i.e. this lane holds column i.  Columns are contiguous in
+	// memory: turn the block through LDS so that a store instruction writes 64 consecutive rows of one column.
+	__shared__ float turn[kNb][kNb + 1];
 #pragma unroll
-	for (int r = 0; r < kNb; r++) Linv[(size_t)i * kNb + r] = x[r];
+	for (int r = 0; r < kNb; r++) turn[i][r] = x[r];
+	__syncthreads();
+	float *xblk = Xout + (size_t)k0 * ld + k0;
+	for (int c = 0; c < nb; c++)
+		if ((i < nb) & (i >= c)) xblk[(size_t)c * ld + i] = turn[c][i];
 }
 
 __global__ void __launch_bounds__(256) shifted_copy_kernel(const float *A, float *W, int n, float shift)
@@ -142,46 +149,58 @@ static InverseLayout inverse_layout(int n)
 }
 
 // state of one inverse while its launches are queued
+constexpr int kMaxDepth = 16;
 struct InverseRun {
-	float *W, *X, *Linv, *T, *T2; // T, T2: temporaries of up to (n/2 + 64) x n/2 each, inside the result matrix
+	float *W, *X;
+	float *L21[kMaxDepth]; // per recursion depth: the off-diagonal block of the factor (a node's children work one level down)
+	float *T2;             // temporary of the last product of a node
 	int n;
 	int *dInfo;
 	void *gws;
 	size_t gBytes;
 };
 
+// floats of the largest L21 block at every recursion depth
+static void l21_sizes(int blocks, int nn, int depth, size_t *need)
+{
+	if (blocks <= 1 || depth >= kMaxDepth) return;
+	const int b1 = blocks / 2, n1 = b1 * kNb, m = nn - n1;
+	const size_t sz = (size_t)m * n1;
+	if (sz > need[depth]) need[depth] = sz;
+	l21_sizes(b1, n1, depth + 1, need);
+	l21_sizes(blocks - b1, m, depth + 1, need);
+}
+
 // L and X = L^-1 of the diagonal block of `blocks` block columns that starts at row/column r0 (order nn)
-static int chol_and_inverse(const InverseRun &r, int r0, int blocks, int nn)
+static int chol_and_inverse(const InverseRun &r, int r0, int blocks, int nn, int depth = 0)
 {
 	const int KC = FITRE_KC_SPD_INVERSE;
 	const int n = r.n;
 	if (blocks == 1) {
-		{
-			LaunchScope scope(KC, 2.0 * kNb * kNb * kNb / 3.0);
-			chol_diag_kernel<<<1, 64, 0, stream()>>>(r.W, n, r0, nn, r.Linv, r.dInfo);
-		}
-		block_copy_kernel<<<blocks_for((long)nn * nn, 256, 64), 256, 0, stream()>>>(r.Linv, kNb, r.X + (size_t)r0 * n + r0, n, nn, nn);
+		LaunchScope scope(KC, 2.0 * kNb * kNb * kNb / 3.0);
+		chol_diag_kernel<<<1, 64, 0, stream()>>>(r.W, n, r0, nn, r.X, r.dInfo);
 		return check_launch("chol_diag_kernel");
 	}
 	const int b1 = blocks / 2, n1 = b1 * kNb, m = nn - n1, r1 = r0 + n1;
-	int rc = chol_and_inverse(r, r0, b1, n1);
+	FITRE_REQUIRE(depth < kMaxDepth, "fitre_hip_spd_inverse: recursion deeper than %d", kMaxDepth);
+	int rc = chol_and_inverse(r, r0, b1, n1, depth + 1);
 	if (rc) return rc;
-	float *A21 = r.W + (size_t)r0 * n + r1;
+	const float *A21 = r.W + (size_t)r0 * n + r1;
 	float *A22 = r.W + (size_t)r1 * n + r1;
 	const float *X11 = r.X + (size_t)r0 * n + r0;
-	// L21 = A21 * X11^T (m x n1), through T, then back into W
-	rc = gemm_ex(0, 1, m, n1, n1, 1.f, A21, n, X11, n, 0.f, r.T, m, nullptr, 0, KC, r.gws, r.gBytes);
+	float *L21 = r.L21[depth];
+	// L21 = A21 * X11^T (m x n1); W keeps A21: only X is needed in the end
+	rc = gemm_ex(0, 1, m, n1, n1, 1.f, A21, n, X11, n, 0.f, L21, m, nullptr, 0, KC, r.gws, r.gBytes);
 	if (rc) return rc;
-	block_copy_kernel<<<blocks_for((long)m * n1, 256, 8192), 256, 0, stream()>>>(r.T, m, A21, n, m, n1);
 	// A22 -= L21 L21^T
-	rc = gemm_ex(0, 1, m, m, n1, -1.f, r.T, m, r.T, m, 1.f, A22, n, nullptr, kGemmMirror, KC, r.gws, r.gBytes);
+	rc = gemm_ex(0, 1, m, m, n1, -1.f, L21, m, L21, m, 1.f, A22, n, nullptr, kGemmMirror, KC, r.gws, r.gBytes);
 	if (rc) return rc;
-	rc = chol_and_inverse(r, r1, blocks - b1, m);
+	rc = chol_and_inverse(r, r1, blocks - b1, m, depth + 1);
 	if (rc) return rc;
 	// X21 = -X22 * (L21 * X11)
 	const float *X22 = r.X + (size_t)r1 * n + r1;
 	float *X21 = r.X + (size_t)r0 * n + r1;
-	rc = gemm_ex(0, 0, m, n1, n1, 1.f, A21, n, X11, n, 0.f, r.T2, m, nullptr, 0, KC, r.gws, r.gBytes);
+	rc = gemm_ex(0, 0, m, n1, n1, 1.f, L21, m, X11, n, 0.f, r.T2, m, nullptr, 0, KC, r.gws, r.gBytes);
 	if (rc) return rc;
 	return gemm_ex(0, 0, m, n1, m, -1.f, X22, n, r.T2, m, 0.f, X21, n, nullptr, 0, KC, r.gws, r.gBytes);
 }
@@ -211,7 +230,7 @@ static int spd_inverse_run(const float *matrix, int n, float shift, float *inver
 		return fail(FITRE_E_WORKSPACE, "fitre_hip_spd_inverse: workspace of %zu bytes is smaller than the %zu required", wsBytes,
 		            lay.total);
 	char *base = (char *)ws;
-	float *W = (float *)(base + lay.w), *X = (float *)(base + lay.x), *Linv = (float *)(base + lay.linv);
+	float *W = (float *)(base + lay.w), *X = (float *)(base + lay.x);
 	int *dInfo = pivotInfo ? pivotInfo : (int *)(base + lay.info);
 	if (infoSlot) *infoSlot = dInfo;
 	void *gws = base + lay.gemm;
@@ -227,10 +246,22 @@ static int spd_inverse_run(const float *matrix, int n, float shift, float *inver
 		fill_zero_kernel<<<1, 64, 0, stream()>>>((float *)dInfo, 1);
 	}
 	// ---- 1. Cholesky factor and its inverse ---------------------------------------------------
+	// The result matrix is free until the last product and holds the temporaries: T2 (at most a
+	// quarter of the matrix) in its second half, the per-depth L21 blocks (a quarter, a sixteenth,
+	// ... of it) in the first.
 	InverseRun run;
-	run.W = W, run.X = X, run.Linv = Linv, run.n = n, run.dInfo = dInfo, run.gws = gws, run.gBytes = gBytes;
-	run.T = inverse;                              // the result matrix is free until the last product
-	run.T2 = inverse + ((size_t)n * n + 1) / 2;   // each temporary is at most (n/2 + 32) x n/2 <= n*n/2 floats
+	run.W = W, run.X = X, run.n = n, run.dInfo = dInfo, run.gws = gws, run.gBytes = gBytes;
+	run.T2 = inverse + ((size_t)n * n + 1) / 2;
+	{
+		size_t need[kMaxDepth] = {};
+		l21_sizes(blocks, n, 0, need);
+		size_t off = 0;
+		for (int d = 0; d < kMaxDepth; d++) {
+			run.L21[d] = inverse + off;
+			off += (need[d] + 63) & ~(size_t)63;
+		}
+		FITRE_REQUIRE(off <= ((size_t)n * n + 1) / 2, "fitre_hip_spd_inverse: temporaries do not fit (order %d)", n);
+	}
 	rc = chol_and_inverse(run, 0, blocks, n);
 	if (rc) return rc;
 	// ---- 2. A^-1 = X^T X ------------------------------------------------------------------------
