@@ -289,3 +289,15 @@ def test_alexnet_full_size_directional_derivative(alexnet_full, dev):
     fd = (losses[0] - losses[1]) / (2 * h)
     gd = float(np.dot(g, d.astype(np.float64)))
     assert abs(fd - gd) < 0.05 * abs(gd) + 1e-3, (fd, gd)
+
+
+def test_vgg11_full_size_against_the_oracle(dev, oracle64):
+    """The benchmark network at the benchmark batch (256): every z and dx slot and the flat gradient against the
+    float64 oracle (tens of seconds of host time on the GPU box's cores)."""
+    compare_with_oracle(dev, oracle64, build_vgg11(256, bn=True), 256, seed=21)
+
+
+def test_alexnet_full_size_against_the_oracle(dev, oracle64):
+    """AlexNet at 3 x 224 x 224, batch 64, 1000 classes against the float64 oracle: 11x11 / stride 4 and 5x5
+    convolutions, 3/2 max pooling, FC 9216-4096-4096-1000."""
+    compare_with_oracle(dev, oracle64, build_alexnet(64), 64, seed=22)
