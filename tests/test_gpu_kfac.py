@@ -112,11 +112,13 @@ def _model_cases():
                                                       dict(cout=9, k=3, pad=1, pool=None, bn=True, act=CNN_ACT_SWISH),
                                                       dict(cout=5, k=3, pad=1, pool=(MAX_POOL, 2, 2, 0), bn=False, act=CNN_ACT_RELU)],
                                        [(7, CNN_ACT_NONE)], bias=1), 12
+    from helpers import build_vgg11
+    yield "vgg11_b256", build_vgg11(256, bn=True), 256   # the benchmark's KFAC configuration at its full size
     yield "no_bias", build_custom(5, 6, 6, 2, [dict(cout=4, k=3, pad=0, pool=(AVG_POOL, 2, 2, 0), bn=False, act=CNN_ACT_SWISH)],
                                   [(6, CNN_ACT_SWISH), (3, CNN_ACT_NONE)], bias=0), 5
 
 
-@pytest.mark.parametrize("name", ["lenet_bias", "small_vgg_bn", "no_bias"])
+@pytest.mark.parametrize("name", ["lenet_bias", "small_vgg_bn", "no_bias", "vgg11_b256"])
 def test_model_factor_passes(dev, oracle64, name):
     """computeOmegaZFactors / computeLambdaDeltaFactors after a forward and a backward pass: every layer's
     factor against the oracle's factor of the same z / dx contents, at the offsets of computeKFACStorageIndices."""
