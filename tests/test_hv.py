@@ -181,3 +181,29 @@ def test_gpu_hv_full_size_vgg_symmetry_and_finite_difference(dev):
         p, q = float(r.astype(np.float64) @ fd), float(r.astype(np.float64) @ hv)
         assert abs(p - q) < 5e-2 * max(abs(p), abs(q)), (p, q)
     gm.release()
+
+
+@pytest.mark.gpu
+def test_gpu_hv_full_size_vgg_against_oracle(dev, oracle64):
+    """The benchmark's Hessian-vector configuration at its full size: VGG-11 (batch norm, ReLU, max pooling), batch
+    256, a seeded N(0,1) direction; cnnHv against the oracle's R passes on the z / probs / errors / dx the device
+    produced.  Per-layer blocks are compared separately so that a small layer cannot hide behind a large one."""
+    from helpers import GpuModel, batch_inputs, build_vgg11, he_weights
+    batch = 256
+    model = build_vgg11(batch, bn=True)
+    rng = np.random.default_rng(0xF17E)
+    w32 = he_weights(model, rng).astype(np.float32)
+    x, y = batch_inputs(model, batch, rng)
+    x32 = x.astype(np.float32)
+    v32 = rng.standard_normal(model.pSize).astype(np.float32)
+    gm = GpuModel(dev, model, w32, x32, y, batch)
+    gm.gradient()
+    got = gpu_hv(dev, gm, model, batch, v32)
+    want = oracle64.hessian_vector(model, w32, x32, gm.get("z"), gm.get("probs"), gm.get("errors"), gm.get("dx"), v32, 10, batch)
+    gm.release()
+    assert np.isfinite(got).all()
+    assert rel_err(got, want) < TOL
+    nl = model.cLayers + model.lLayers
+    for l in range(nl):
+        a, b = model.wOffsets[l], model.bOffsets[l]
+        assert rel_err(got[a:b], want[a:b]) < TOL, "weights of layer %d" % l
