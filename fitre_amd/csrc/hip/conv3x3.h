@@ -558,4 +558,142 @@ conv3x3_dw_kernel(const Conv3x3Params p, const float *delta, uint32_t deltaBytes
 	}
 }
 
+// ---------------------------------------------------------------------------------
+// weight gradient of a layer with very few input channels (the first layer: Cin = 3)
+// ---------------------------------------------------------------------------------
+// With Cin*9 <= 32 the whole patch index (c, ta, tb) fits the 32 columns of ONE accumulator block,
+// so the product is a plain  dW[64 x 27] = delta[64 x M] * patch[M x 27]  whose cost is reading
+// delta once (HBM-bound, not MFMA-bound).  A workgroup walks chunks of 128 positions = whole image
+// rows: delta goes through LDS as [channel][position]; the layer input as a window of R + 2 rows
+// with a zero column on either side and zero rows above / below the image, so that the patch
+// element of lane k = (c, ta, tb) at position (row r, column b) of the chunk is the word
+// c*plane + (r + ta)*(B + 2) + b + tb: no border test.  Four waves take 32 positions each and are
+// summed through LDS at the end; every workgroup leaves one partial 64 x 27 block (split layout
+// of the general engine: combined by splitk_reduce_kernel).
+// Requires B a power of two, 2 <= B <= 128, (A*B) % 128 == 0 or 128 % (A*B) == 0 -- here:
+// A % (128 / B) == 0 --, Cin <= 3, Cout <= 64.
+constexpr int kThinChunk = 128;
+constexpr int kThinDeltaLd = kThinChunk + 1;
+constexpr int kThinXPlane = 400; // words per input channel of the window: (R + 2) * (B + 2) <= 396
+
+struct ThinDwParams {
+	const float *x;     // [Cin][N][A][B]
+	const float *delta; // [Cout][N][A][B]
+	int cin, cout;
+	int A, B, logB;
+	int plane;          // N*A*B
+	int chunks;         // plane / 128
+	int perGroup;       // chunks per workgroup
+};
+
+__global__ void __launch_bounds__(kGemmThreads)
+conv3x3_dw_thin_kernel(const ThinDwParams p, float *partial)
+{
+	__shared__ float Ds[2][64 * kThinDeltaLd];
+	__shared__ float Xs[2][3 * kThinXPlane];
+	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+	const int khalf = lane >> 5, l32 = lane & 31;
+	const int R = kThinChunk >> p.logB;  // image rows per chunk
+	const int rowLd = p.B + 2;
+	const int imageCells = p.A * p.B;
+	const int qBeg = blockIdx.x * p.perGroup;
+	const int qEnd = (qBeg + p.perGroup < p.chunks) ? qBeg + p.perGroup : p.chunks;
+
+	// this lane's patch column k = (c, ta, tb); columns past Cin*9 repeat the last one and are never stored
+	const int K = p.cin * 9;
+	const int k = (l32 < K) ? l32 : K - 1;
+	const int kc = k / 9, kt = k - kc * 9, kta = kt / 3, ktb = kt - kta * 3;
+	const int xBase = kc * kThinXPlane + kta * rowLd + ktb;
+
+	// staging: delta 64 x 128 as 2048 groups of four, eight per thread; the window cell by cell
+	constexpr int DE = 64 * kThinChunk / 4 / kGemmThreads;
+	float4 dreg[DE];
+	constexpr int XE = (3 * kThinXPlane + kGemmThreads - 1) / kGemmThreads;
+	float xreg[XE];
+	const int winCells = (R + 2) * rowLd;
+
+	auto load_chunk = [&](int q) {
+		const int m0 = q * kThinChunk;
+#pragma unroll
+		for (int e = 0; e < DE; e++) {
+			const int g = tid + kGemmThreads * e;
+			const int o = g / (kThinChunk / 4), c4 = g - o * (kThinChunk / 4);
+			dreg[e] = (o < p.cout) ? *reinterpret_cast<const float4 *>(p.delta + (size_t)o * p.plane + m0 + 4 * c4)
+			                       : make_float4(0.f, 0.f, 0.f, 0.f);
+		}
+		const int n = m0 / imageCells;
+		const int a0 = (m0 - n * imageCells) >> p.logB; // first image row of the chunk
+#pragma unroll
+		for (int e = 0; e < XE; e++) {
+			const int w = tid + kGemmThreads * e;
+			const int c = w / winCells, cell = w - c * winCells;
+			float v = 0.f;
+			if (c < p.cin) {
+				const int r = cell / rowLd, col = cell - r * rowLd;
+				const int a = a0 - 1 + r, b = col - 1;
+				if (a >= 0 && a < p.A && b >= 0 && b < p.B) v = p.x[(size_t)c * p.plane + (size_t)n * imageCells + a * p.B + b];
+			}
+			xreg[e] = v;
+		}
+	};
+	auto store_chunk = [&](int buf) {
+#pragma unroll
+		for (int e = 0; e < DE; e++) {
+			const int g = tid + kGemmThreads * e;
+			const int o = g / (kThinChunk / 4), c4 = g - o * (kThinChunk / 4);
+			float *dst = Ds[buf] + o * kThinDeltaLd + 4 * c4;
+			dst[0] = dreg[e].x, dst[1] = dreg[e].y, dst[2] = dreg[e].z, dst[3] = dreg[e].w;
+		}
+#pragma unroll
+		for (int e = 0; e < XE; e++) {
+			const int w = tid + kGemmThreads * e;
+			const int c = w / winCells, cell = w - c * winCells;
+			if (c < 3) Xs[buf][c * kThinXPlane + cell] = xreg[e];
+		}
+	};
+
+	v16f acc0, acc1;
+#pragma unroll
+	for (int v = 0; v < 16; v++) acc0[v] = 0.f, acc1[v] = 0.f;
+
+	if (qBeg < qEnd) {
+		load_chunk(qBeg);
+		store_chunk(0);
+	}
+	__syncthreads();
+	for (int q = qBeg; q < qEnd; q++) {
+		const int buf = (q - qBeg) & 1;
+		const bool more = q + 1 < qEnd;
+		if (more) load_chunk(q + 1);
+		const float *dA = Ds[buf] + l32 * kThinDeltaLd + wave * 32 + khalf;
+		const float *dB = dA + 32 * kThinDeltaLd;
+#pragma unroll
+		for (int st = 0; st < 16; st++) {
+			const int pos = wave * 32 + 2 * st + khalf; // position inside the chunk
+			const int r = pos >> p.logB, b = pos & (p.B - 1);
+			const float bv = Xs[buf][xBase + r * rowLd + b];
+			acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(dA[2 * st], bv, acc0, 0, 0, 0);
+			acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(dB[2 * st], bv, acc1, 0, 0, 0);
+		}
+		if (more) store_chunk(buf ^ 1);
+		__syncthreads();
+	}
+
+	// sum the four waves through LDS (the delta buffers are free now), then one coalesced store
+	float *red = &Ds[0][0]; // [wave][64][33]
+	static_assert(4 * 64 * 33 <= 2 * 64 * kThinDeltaLd, "the wave partials fit the delta buffers");
+#pragma unroll
+	for (int v = 0; v < 16; v++) {
+		const int row = 8 * (v / 4) + 4 * khalf + (v % 4);
+		red[(wave * 64 + row) * 33 + l32] = acc0[v];
+		red[(wave * 64 + 32 + row) * 33 + l32] = acc1[v];
+	}
+	__syncthreads();
+	float *out = partial + (size_t)blockIdx.x * p.cout * K;
+	for (int i = tid; i < p.cout * K; i += kGemmThreads) {
+		const int o = i / K, kk = i - o * K;
+		out[i] = (red[(0 * 64 + o) * 33 + kk] + red[(1 * 64 + o) * 33 + kk]) + (red[(2 * 64 + o) * 33 + kk] + red[(3 * 64 + o) * 33 + kk]);
+	}
+}
+
 } // namespace fitre

@@ -43,6 +43,14 @@ CONV_CASES = [
     (128, 16, 32, 1, 1, 3, 1, 1),    # 1x1 maps: only the centre tap sees data
     (32, 16, 32, 2, 1, 3, 1, 1),     # single-column maps
     (4, 16, 32, 1, 16, 3, 1, 1),     # single-row maps
+    # weight gradient with at most three input channels (the first layer's kernel): chunks of whole image rows
+    (6, 3, 64, 32, 32, 3, 1, 1),     # the benchmark's first layer at a small batch
+    (5, 3, 64, 8, 16, 3, 1, 1),      # eight rows per chunk
+    (3, 2, 40, 32, 4, 3, 1, 1),      # 32 rows per chunk, partial output-channel block
+    (2, 1, 7, 2, 64, 3, 1, 1),       # one input channel, two rows per chunk
+    (3, 3, 64, 1, 128, 3, 1, 1),     # one row per chunk: nothing above or below
+    (2, 3, 16, 12, 32, 3, 1, 1),     # A not a multiple of the rows per chunk... 12 % 4 == 0: eligible
+    (2, 3, 16, 6, 32, 3, 1, 1),      # 6 % 4 != 0: general engine
 ]
 
 
