@@ -492,3 +492,38 @@ def test_distribution_errors(dev, oracle64, rows, classes):
     # the empirical class frequencies follow the probabilities
     if rows >= 4096:
         assert abs(np.mean(got_t) - np.mean((p * np.arange(1, classes + 1)).sum(1))) < 0.05 * classes
+
+
+def test_empty_inputs(dev):
+    """Zero-length vectors are no-ops (reductions give 0), zero-sized tensors of the layer kernels are argument
+    errors, negative sizes always are; nothing is launched with an empty grid."""
+    p = dev.upload(np.arange(8, dtype=np.float32))
+    q = dev.upload(np.full(8, 3.0, np.float32))
+    res = (C.c_float * 1)(7.0)
+    ok(hip.fitre_hip_axpy(0, 2.0, p, q))
+    ok(hip.fitre_hip_scal(0, 2.0, q))
+    ok(hip.fitre_hip_copy(0, p, q))
+    ok(hip.fitre_hip_fill(q, 0, 9.0))
+    ok(hip.fitre_hip_hadamard(p, q, 0))
+    ok(hip.fitre_hip_activation_forward(CNN_ACT_RELU, p, q, 0))
+    ok(hip.fitre_hip_activation_backward(CNN_ACT_RELU, p, p, p, q, 0))
+    np.testing.assert_array_equal(dev.download(q, 8), np.full(8, 3.0, np.float32))
+    for fn in (hip.fitre_hip_nrm2, hip.fitre_hip_asum, hip.fitre_hip_sum):
+        res[0] = 7.0
+        ok(fn(0, p, res))
+        assert res[0] == 0.0
+    ok(hip.fitre_hip_dot(0, p, q, res))
+    assert res[0] == 0.0
+    assert hip.fitre_hip_axpy(-1, 2.0, p, q) == 2
+    assert hip.fitre_hip_activation_forward(CNN_ACT_RELU, p, q, -5) == 2
+    assert hip.fitre_hip_pool_forward(MAX_POOL, p, 0, 1, 2, 2, 2, 2, 0, 1, 1, q) == 2
+    assert hip.fitre_hip_pool_backward(MAX_POOL, p, p, 1, 0, 2, 2, 2, 2, 0, 1, 1, q) == 2
+    ws, nb = bn_ws(dev, 1, 8)
+    assert hip.fitre_hip_batch_norm_backward(p, p, p, 0, 8, 1e-5, q, None, ws, nb) == 2
+    assert hip.fitre_hip_batch_norm_backward(p, p, p, 1, 0, 1e-5, q, None, ws, nb) == 2
+    assert hip.fitre_hip_channel_sum(p, 0, 8, q, ws, nb) == 2
+    assert hip.fitre_hip_softmax_cross_entropy(p, p, 0, 4, q, q, res) == 2
+    from helpers import conv_shape
+    s = conv_shape(0, 2, 2, 2, 2, 3, 1, 1)
+    assert hip.fitre_hip_conv_weight_grad(C.byref(s), p, p, q, None, 0) == 2
+    assert hip.fitre_hip_conv_input_grad(C.byref(s), p, p, q, None, 0) == 2
