@@ -328,7 +328,13 @@ conv3x3_dw_kernel(const Conv3x3Params p, const float *delta, uint32_t deltaBytes
 	constexpr int D_DUMMY = kC3Tile * kC3DeltaLd;
 	constexpr int DGROUPS = kC3Tile * kC3Stage / 4;                     // 4-float groups of delta per stage
 	constexpr int DE = (DGROUPS + T - 1) / T;
-	constexpr int XE = (kC3DwCin * CELLS_MAX + T - 1) / T;
+	// source window staging: a thread keeps ONE cell of the window and takes it from XCP channels apart
+	// in every pass, so where a cell comes from and where it goes differ between passes by constants
+	// only (few live registers: this kernel leaves room for a bandwidth kernel's waves beside its own)
+	constexpr int XG = (MAXB == 16) ? 128 : 192; // threads per channel in a pass (>= cells of the window)
+	constexpr int XCP = T / XG;                  // channels per pass
+	constexpr int XE = (kC3DwCin + XCP - 1) / XCP;
+	static_assert(XG >= CELLS_MAX && T % XG == 0, "one thread per window cell");
 	static_assert(T % (kC3Stage / 4) == 0, "a thread keeps its column group in every round");
 	static_assert(MAXB == 16 || MAXB == 32, "row-pad bound: taken at B = MAXB it covers 2 <= B <= 16 resp. 1 <= B <= 32");
 	__shared__ float Ds[2][D_DUMMY + 4];
@@ -383,21 +389,11 @@ conv3x3_dw_kernel(const Conv3x3Params p, const float *delta, uint32_t deltaBytes
 		dOff[e] = VECD ? (inside ? off : 4u * (uint32_t)dCol) : (inside ? off : kGroupOutOfRange);
 		dLds[e] = has ? row * kC3DeltaLd + dCol : D_DUMMY;
 	}
-	int xChanOff[XE]; // (c0 + c) * plane, or -1
-	int xMeta[XE];    // (c * XP_LD) << 8 | r with r the flat cell of the window (first cell = stage start - halo);
-	                  // -1 when the thread has no cell in this round
-#pragma unroll
-	for (int e = 0; e < XE; e++) {
-		const int idx = tid + T * e;
-		const int c = idx / win, r = idx - c * win;
-		const bool has = c < kC3DwCin;
-		xChanOff[e] = (has & ((c0 + c) < p.cred)) ? (c0 + c) * plane : -1;
-		xMeta[e] = has ? ((c * XP_LD) << 8) | r : -1;
-	}
-
+	const int xr = tid % XG, xcg = tid / XG; // the thread's window cell (first cell = stage start - halo) and first channel
+	const bool xHas = xr < win;
 	float dreg[DE * 4];
 	float xreg[XE];
-	int xLds[XE]; // LDS word of the cell; bit 31: the cell ends an image row (the next word is a row pad)
+	int xWord = X_DUMMY; // LDS word of the cell in channel xcg; bit 31: the cell ends an image row (the next word is a row pad)
 	int pkReg = 0;
 	uint32_t mkReg0 = 0, mkReg2 = 0;
 
@@ -424,18 +420,21 @@ conv3x3_dw_kernel(const Conv3x3Params p, const float *delta, uint32_t deltaBytes
 		}                                                                                                             \
 		/* column of the window's first cell; the bias keeps the dividend non-negative */                             \
 		const uint32_t bs_ = (uint32_t)(m0_ + halo * (p.B - 1)) - p.divB.quot((uint32_t)(m0_ + halo * (p.B - 1))) * (uint32_t)p.B; \
-		_Pragma("unroll") for (int e = 0; e < XE; e++)                                                                \
 		{                                                                                                             \
-			const int r_ = xMeta[e] & 255;                                                                            \
-			const int m = m0_ - halo + r_;                                                                            \
-			const bool ok = (xChanOff[e] >= 0) & ((unsigned)m < (unsigned)plane);                                     \
-			xreg[e] = buffer_load(srcRs, ok ? 4u * (uint32_t)(xChanOff[e] + m) : kOutOfRange);                        \
+			const int m = m0_ - halo + xr;                                                                            \
+			const bool okm = xHas & ((unsigned)m < (unsigned)plane);                                                  \
+			_Pragma("unroll") for (int e = 0; e < XE; e++)                                                            \
+			{                                                                                                         \
+				const int c = xcg + XCP * e;                                                                          \
+				const bool ok = okm & (c < kC3DwCin) & ((c0 + c) < p.cred);                                           \
+				xreg[e] = buffer_load(srcRs, ok ? 4u * (uint32_t)((c0 + c) * plane + m) : kOutOfRange);               \
+			}                                                                                                         \
 			if (movingRows | ((ST) == stBeg)) {                                                                       \
 				uint32_t q_, b_;                                                                                      \
-				p.divB.divmod(bs_ + (uint32_t)r_, q_, b_);                                                            \
-				const int word = (xMeta[e] >> 8) + r_ + (int)q_;                                                      \
+				p.divB.divmod(bs_ + (uint32_t)xr, q_, b_);                                                            \
+				const int word = xcg * XP_LD + xr + (int)q_;                                                          \
 				const int end = (b_ == (uint32_t)(p.B - 1)) ? (int)0x80000000 : 0;                                    \
-				xLds[e] = (xMeta[e] >= 0) ? (word | end) : X_DUMMY;                                                   \
+				xWord = xHas ? (word | end) : X_DUMMY;                                                                \
 			}                                                                                                         \
 		}                                                                                                             \
 		if (tid < kC3Stage) {                                                                                         \
@@ -455,10 +454,17 @@ conv3x3_dw_kernel(const Conv3x3Params p, const float *delta, uint32_t deltaBytes
 			float *dst = Ds[BUF] + dLds[e];                                                                           \
 			dst[0] = dreg[4 * e], dst[1] = dreg[4 * e + 1], dst[2] = dreg[4 * e + 2], dst[3] = dreg[4 * e + 3];       \
 		}                                                                                                             \
-		_Pragma("unroll") for (int e = 0; e < XE; e++) Xs[BUF][xLds[e] & 0x7FFFFFFF] = xreg[e];                       \
+		_Pragma("unroll") for (int e = 0; e < XE; e++)                                                                \
+		{                                                                                                             \
+			const bool has = xHas & ((xcg + XCP * e) < kC3DwCin);                                                     \
+			Xs[BUF][has ? (xWord & 0x7FFFFFFF) + e * XCP * XP_LD : X_DUMMY] = xreg[e];                                \
+		}                                                                                                             \
 		if (movingRows) { /* the row pads move with the stage: rewrite them */                                        \
 			_Pragma("unroll") for (int e = 0; e < XE; e++)                                                            \
-			    Xs[BUF][(xLds[e] < 0) ? (xLds[e] & 0x7FFFFFFF) + 1 : X_DUMMY] = 0.f;                                  \
+			{                                                                                                         \
+				const bool has = (xWord < 0) & ((xcg + XCP * e) < kC3DwCin);                                          \
+				Xs[BUF][has ? (xWord & 0x7FFFFFFF) + e * XCP * XP_LD + 1 : X_DUMMY] = 0.f;                            \
+			}                                                                                                         \
 		}                                                                                                             \
 		if (tid < kC3Stage) {                                                                                         \
 			Pk[BUF][tid] = pkReg;                                                                                     \
