@@ -352,15 +352,15 @@ conv3x3_dw_kernel(const Conv3x3Params p, const float *delta, uint32_t deltaBytes
 	int bx = blockIdx.x, by = blockIdx.y, bz = blockIdx.z;
 	{
 		const unsigned groups = gridDim.x * gridDim.y * gridDim.z;
-		if ((groups & 7u) == 0) {
-			const unsigned lin = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
-			const unsigned logical = (lin & 7u) * (groups >> 3) + (lin >> 3);
-			const unsigned tiles = gridDim.x * gridDim.y;
-			bz = (int)(logical / tiles);
-			const unsigned rem = logical - (unsigned)bz * tiles;
-			by = (int)(rem / gridDim.x);
-			bx = (int)(rem - (unsigned)by * gridDim.x);
-		}
+		const unsigned lin = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+		// XCD x receives launch indices x, x + 8, ...: groups / 8 of them, one more on the first groups % 8
+		const unsigned xcd = lin & 7u, each = groups >> 3, extra = groups & 7u;
+		const unsigned logical = xcd * each + (xcd < extra ? xcd : extra) + (lin >> 3);
+		const unsigned tiles = gridDim.x * gridDim.y;
+		bz = (int)(logical / tiles);
+		const unsigned rem = logical - (unsigned)bz * tiles;
+		by = (int)(rem / gridDim.x);
+		bx = (int)(rem - (unsigned)by * gridDim.x);
 	}
 	const int c0 = bx * kC3DwCin, o0 = by * kC3Tile;
 	const int halo = p.B + 1;

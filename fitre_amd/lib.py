@@ -165,6 +165,17 @@ CNN_API = {
     "computeLambdaDelta": (None, [pkfac, pmodel, i32, vp, vp, vp, pi32, pi32, vp, vp]),
     "kfacNaturalGradientMemRequired": (lng, [pmodel]),
     "computeNaturalGradient": (None, [pmodel, pkfac, vp, vp]),
+    # include/fitre_solver.h
+    "genRandomVector": (None, [pi32, i32, i32]),
+    "allocSampledDataset": (None, [pdata, i32]),
+    "initBatchNormData": (None, [pmodel, vp, pi32]),
+    "updateRunningStats": (None, [vp, vp, i32, f32]),
+    "computeSpeedUpOmegaZ": (None, [pkfac, pmodel, pdata, i32, vp, pi32, vp, vp, pi32, i32]),
+    "computeSpeedUpLambdaDelta": (None, [pkfac, pmodel, i32, vp, vp, pi32, pi32, i32]),
+    "kfacTrustRegionMemRequired": (lng, [pmodel, pdata, pkfac]),
+    "kfacTrustRegionHostMemRequired": (lng, [pdata]),
+    "kfacTrustRegionReports": (i32, [vp, i32]),
+    "subsampledTrustRegionKFAC": (None, [pmodel, pdata, vp, pkfac, vp, pscratch, i32, i32]),
     # include/fitre_hv.h
     "cnnHvMemRequired": (lng, [pmodel]),
     "cnnHv": (None, [pmodel, pdata, vp, vp, vp, vp, vp, vp, i32, i32, vp, vp, f32]),

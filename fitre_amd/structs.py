@@ -106,6 +106,21 @@ class KFAC_CURVATURE_INFO(C.Structure):
                 [("inverseFreq", C.c_int)])
 
 
+class TRUST_REGION_PARAMS(C.Structure):
+    """include/fitre_solver.h (solvers/params.h:12-35 of the reference)."""
+    _fields_ = ([(n, C.c_float) for n in ("delta", "minDelta", "maxDelta", "eta1", "eta2", "gamma1", "gamma2")] +
+                [("maxProps", C.c_ulong), ("maxMatVecs", C.c_int), ("maxEpochs", C.c_int), ("maxIters", C.c_int),
+                 ("hessianType", C.c_int), ("alpha", C.c_float), ("curIteration", C.c_int), ("hs", C.c_float),
+                 ("lambda_", C.c_float)])
+
+
+class KFAC_TR_EPOCH_REPORT(C.Structure):
+    """include/fitre_solver.h: what one pass over the training set left behind."""
+    _fields_ = ([("iteration", C.c_int), ("miniBatches", C.c_int), ("rejectedSteps", C.c_int)] +
+                [(n, C.c_float) for n in ("trainLikelihood", "trainAccuracy", "testLikelihood", "testAccuracy",
+                                          "weightNorm", "delta", "seconds")])
+
+
 class fitre_split_view(C.Structure):
     """include/fitre_hip.h: unsummed split partials of an input gradient."""
     _fields_ = [("base", C.c_void_p), ("splits", C.c_int), ("stride", C.c_long)]
