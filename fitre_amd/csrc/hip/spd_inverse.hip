@@ -6,8 +6,8 @@
 //        (L11, X11) of A11;  L21 = A21 X11^T;  A22 -= L21 L21^T;  (L22, X22) of that;
 //        X21 = -X22 (L21 X11).
 //      Every product is as large as the halves it joins (rank n/2, n/4, ... updates on the MFMA
-//      tile engine instead of n/64 rank-64 ones), and a 64 x 64 leaf is one one-wave kernel that
-//      factors the block and inverts its factor;
+//      tile engine instead of n/64 rank-64 ones), and a leaf of order <= 128 is one workgroup that
+//      factors the block and inverts its factor without leaving LDS;
 //   2. A^-1 = X^T X                 one symmetric engine product whose reduction skips the zero
 //                                   part of the triangular operand.
 // All matrices are column-major with leading dimension n; only lower triangles are meaningful
@@ -17,6 +17,7 @@
 namespace fitre {
 
 constexpr int kNb = 64; // block order of the factorization
+typedef float v16f __attribute__((ext_vector_type(16)));
 
 // value of v in lane `lane` (a compile-time lane index), as a wave-uniform scalar
 __device__ __forceinline__ float lane_value(float v, int lane)
@@ -24,59 +25,231 @@ __device__ __forceinline__ float lane_value(float v, int lane)
 	return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
 }
 
-// One wave factors the nb x nb (nb <= 64) diagonal block in place (lower triangle) and writes the
-// inverse of the factor into the same block of Xout (lower triangle, leading dimension ld).  Lane i holds row i in
-// registers; what a step needs from another lane's row comes through v_readlane as a scalar, so
-// there is no LDS traffic and no barrier in the 2 x 2016 multiply-adds.
-// info: set to the 1-based global index of the first non-positive pivot.
-__global__ void __launch_bounds__(64) chol_diag_kernel(float *W, int ld, int k0, int nb, float *Xout, int *info)
+// ---- leaf of the recursion: a diagonal block of order <= 128, one workgroup, everything in LDS --------
+//
+// The block is cut into 32 x 32 sub-blocks.  A sub-block on the diagonal is factored, and its factor
+// inverted, by one wave with a row per lane (what a step needs from another lane's row comes through
+// v_readlane as a scalar: no LDS traffic, no barrier inside the 2 x 496 multiply-adds); everything off
+// the diagonal is 32 x 32 x 32 products on the matrix pipes, one tile per wave, operands read from LDS:
+//     for kb:  (L[kb][kb], X[kb][kb]) of W[kb][kb];   L[ib][kb] = W[ib][kb] X[kb][kb]^T  (ib > kb);
+//              W[ib][jb] -= L[ib][kb] L[jb][kb]^T  (ib >= jb > kb)
+//     for ib:  X[ib][jb] = -X[ib][ib] * sum_{jb <= k < ib} L[ib][k] X[k][jb]  (jb < ib)
+// Both matrices are column-major in LDS with a leading dimension of 129 words, which makes the
+// stride-129 accesses of the transposed operands and of the accumulator layout conflict-free.
+constexpr int kSub = 32;                 // order of a sub-block
+constexpr int kLeafBlocks = 2;           // 64-wide block columns a leaf covers
+constexpr int kLeaf = kLeafBlocks * kNb; // largest leaf order
+constexpr int kLeafLd = kLeaf + 1;
+
+// One wave: factor sub-block kb of Ws in registers, write its factor back (lower triangle) and the inverse
+// of the factor into the same sub-block of Xs (zeros above the diagonal).  Returns the 1-based index inside the
+// leaf of the first non-positive pivot of this sub-block, or 0.
+//
+// Lane i holds row i of the block (a[]) and column i of the inverse in the making (y[], which starts as the unit
+// vector e_i and is forward-substituted column by column).  Step j scales column j, and then every later column k
+// takes a[k] -= a[j] * L[k][j] and y[k] -= y[j] * L[k][j]: the same scalar L[k][j] (lane k's a[j], through
+// v_readlane) serves the factorization and the inversion.  The scalars are fetched eight at a time ahead of their
+// sixteen multiply-adds: with one wave on the SIMD a multiply-add right behind its own v_readlane waits for it.
+// columns K0 .. K0+7 (those below kSub) of step J
+template <int J, int K0>
+__device__ __forceinline__ void factor_update_group(float (&a)[kSub], float (&y)[kSub])
 {
-	const int i = threadIdx.x;
-	float a[kNb];
-	float *blk = W + (size_t)k0 * ld + k0;
+	constexpr int N = (kSub - K0 < 8) ? (kSub - K0) : 8;
+	int s[N];
 #pragma unroll
-	for (int j = 0; j < kNb; j++) {
-		const bool inside = (i < nb) & (j < nb);
-		a[j] = inside ? blk[(size_t)j * ld + i] : ((i == j) ? 1.f : 0.f);
+	for (int q = 0; q < N; q++) s[q] = __builtin_amdgcn_readlane(__float_as_int(a[J]), K0 + q);
+	// all lane reads of the group before its first multiply-add
+	if constexpr (N == 8)
+		asm volatile("" : "+s"(s[0]), "+s"(s[1]), "+s"(s[2]), "+s"(s[3]), "+s"(s[4]), "+s"(s[5]), "+s"(s[6]), "+s"(s[7]));
+#pragma unroll
+	for (int q = 0; q < N; q++) {
+		a[K0 + q] -= a[J] * __int_as_float(s[q]); // entries above the diagonal are never used
+		y[K0 + q] -= y[J] * __int_as_float(s[q]);
 	}
-	float rdiag[kNb]; // 1 / L[j][j], wave-uniform
+	// the updates stay in this step: left to itself the compiler postpones each until column k is needed and keeps
+	// the 496 scalars alive (spilled) until then
+	if constexpr (N == 8) {
+		asm volatile("" : "+v"(a[K0]), "+v"(a[K0 + 1]), "+v"(a[K0 + 2]), "+v"(a[K0 + 3]), "+v"(a[K0 + 4]), "+v"(a[K0 + 5]),
+		             "+v"(a[K0 + 6]), "+v"(a[K0 + 7]));
+		asm volatile("" : "+v"(y[K0]), "+v"(y[K0 + 1]), "+v"(y[K0 + 2]), "+v"(y[K0 + 3]), "+v"(y[K0 + 4]), "+v"(y[K0 + 5]),
+		             "+v"(y[K0 + 6]), "+v"(y[K0 + 7]));
+	} else {
+#pragma unroll
+		for (int q = 0; q < N; q++) asm volatile("" : "+v"(a[K0 + q]), "+v"(y[K0 + q]));
+	}
+	if constexpr (K0 + 8 < kSub) factor_update_group<J, K0 + 8>(a, y);
+}
+
+// steps J .. kSub-1; first: base of the 1-based pivot numbering
+template <int J>
+__device__ __forceinline__ void factor_steps(float (&a)[kSub], float (&y)[kSub], int first, int &bad)
+{
+	const float ajj = lane_value(a[J], J);
+	if (!(ajj > 0.f) && bad == 0) bad = first + J + 1;
+	const float d = rsqrtf(ajj);
+	a[J] *= d; // column J of L; lane J's own entry becomes ajj / sqrt(ajj), the diagonal
+	y[J] *= d; // row J of the inverse is complete
+	if constexpr (J + 1 < kSub) {
+		factor_update_group<J, J + 1>(a, y);
+		factor_steps<J + 1>(a, y, first, bad);
+	}
+}
+
+__device__ __forceinline__ int factor_sub_block(float *Ws, float *Xs, int kb, int lane)
+{
+	const int i = lane & (kSub - 1);
+	float *wb = Ws + (kb * kSub) * kLeafLd + kb * kSub;
+	float *xb = Xs + (kb * kSub) * kLeafLd + kb * kSub;
+	float a[kSub], y[kSub];
+#pragma unroll
+	for (int j = 0; j < kSub; j++) {
+		a[j] = wb[j * kLeafLd + i];
+		y[j] = (i == j) ? 1.f : 0.f;
+	}
 	int bad = 0;
+	factor_steps<0>(a, y, kb * kSub, bad);
+	// y[r] is element (r, i) of the inverse: this lane holds column i
+	if (lane < kSub) {
 #pragma unroll
-	for (int j = 0; j < kNb; j++) {
-		const float ajj = lane_value(a[j], j);
-		if (!(ajj > 0.f) && bad == 0) bad = k0 + j + 1;
-		const float d = rsqrtf(ajj);
-		rdiag[j] = d;
-		a[j] = (i == j) ? ajj * d : a[j] * d; // column j of L; sqrt(ajj) on the diagonal
-#pragma unroll
-		for (int k = j + 1; k < kNb; k++) a[k] -= a[j] * lane_value(a[j], k); // entries above the diagonal are never used
-	}
-	if (bad != 0 && i == 0) atomicCAS(info, 0, bad);
-#pragma unroll
-	for (int j = 0; j < kNb; j++)
-		if ((i < nb) & (j < nb) & (j <= i)) blk[(size_t)j * ld + i] = a[j];
-	// lane c solves L x = e_c by forward substitution; L[r][k] is lane r's a[k]
-	float x[kNb];
-#pragma unroll
-	for (int r = 0; r < kNb; r++) {
-		float acc0 = (r == i) ? 1.f : 0.f, acc1 = 0.f;
-#pragma unroll
-		for (int k = 0; k < r; k++) {
-			const float l = lane_value(a[k], r);
-			if (k & 1) acc1 -= l * x[k];
-			else acc0 -= l * x[k];
+		for (int j = 0; j < kSub; j++) {
+			wb[j * kLeafLd + i] = a[j];
+			xb[i * kLeafLd + j] = y[j];
 		}
-		x[r] = (acc0 + acc1) * rdiag[r];
 	}
-	// x[r] is element (r, i) of the inverse, i.e. this lane holds column i.  Columns are contiguous in
-	// memory: turn the block through LDS so that a store instruction writes 64 consecutive rows of one column.
-	__shared__ float turn[kNb][kNb + 1];
+	return bad;
+}
+
+// acc += A * B for 32 x 32 operands in LDS.  element (r, k) of A is at A[k * aK + r * aR], element
+// (k, c) of B at B[k * bK + c * bC].
+__device__ __forceinline__ void sub_block_product(const float *A, int aR, int aK, const float *B, int bK, int bC, int lane,
+                                                  v16f &acc)
+{
+	const int l32 = lane & 31, khalf = lane >> 5;
+	const float *ap = A + l32 * aR + khalf * aK;
+	const float *bp = B + l32 * bC + khalf * bK;
 #pragma unroll
-	for (int r = 0; r < kNb; r++) turn[i][r] = x[r];
+	for (int s = 0; s < kSub / 2; s++)
+		acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ap[2 * s * aK], bp[2 * s * bK], acc, 0, 0, 0);
+}
+
+// register v of lane l holds row 8*(v/4) + 4*(l/32) + v%4, column l%32 of a 32 x 32 accumulator
+__device__ __forceinline__ void store_sub_block(float *M, int lane, const v16f &acc, float scale)
+{
+	float *col = M + (lane & 31) * kLeafLd + 4 * (lane >> 5);
+#pragma unroll
+	for (int v = 0; v < 16; v++) col[8 * (v / 4) + (v % 4)] = acc[v] * scale;
+}
+
+__device__ __forceinline__ void load_sub_block(const float *M, int lane, v16f &acc)
+{
+	const float *col = M + (lane & 31) * kLeafLd + 4 * (lane >> 5);
+#pragma unroll
+	for (int v = 0; v < 16; v++) acc[v] = col[8 * (v / 4) + (v % 4)];
+}
+
+// sub-block (rb, cb) of a matrix held column-major in LDS
+__device__ __forceinline__ float *sub_block(float *M, int rb, int cb) { return M + (cb * kSub) * kLeafLd + rb * kSub; }
+
+// The diagonal block of order nn (1..128) that starts at row/column k0 of W (column-major, leading dimension
+// ld, lower triangle read): X = L^-1 of its Cholesky factor into the same block of Xout (lower triangle written).
+// info: set to the 1-based global index of the first non-positive pivot.
+__global__ void __launch_bounds__(256) chol_leaf_kernel(const float *W, int ld, int k0, int nn, float *Xout, int *info)
+{
+	__shared__ float Ws[kLeaf * kLeafLd];
+	__shared__ float Xs[kLeaf * kLeafLd];
+	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+	const int nb = (nn + kSub - 1) / kSub, order = nb * kSub;
+	const float *blk = W + (size_t)k0 * ld + k0;
+	// Thread (r, h) moves row r, columns of parity h: the sub-blocks on and below the diagonal only (the rest of Ws is
+	// scratch, and Xs is written before it is read), a sub-block column of sixteen loads in flight at a time.
+	const int row = tid & (kLeaf - 1), half = tid >> 7, rowBlock = row >> 5;
+	if (row < order) {
+#pragma unroll
+		for (int b = 0; b < kLeaf / kSub; b++) {
+			if (b > rowBlock) break;
+			float v[kSub / 2];
+#pragma unroll
+			for (int q = 0; q < kSub / 2; q++) {
+				const int c = b * kSub + half + 2 * q;
+				// rows and columns beyond the block: identity, which factors to itself
+				v[q] = ((row < nn) & (c < nn)) ? blk[(size_t)c * ld + row] : ((row == c) ? 1.f : 0.f);
+			}
+#pragma unroll
+			for (int q = 0; q < kSub / 2; q++) Ws[(b * kSub + half + 2 * q) * kLeafLd + row] = v[q];
+		}
+	}
 	__syncthreads();
+
+	for (int kb = 0; kb < nb; kb++) {
+		if (wave == 0) {
+			const int bad = factor_sub_block(Ws, Xs, kb, lane);
+			if (bad != 0 && lane == 0) atomicCAS(info, 0, k0 + bad);
+		}
+		__syncthreads();
+		// column kb of the factor below the diagonal: one sub-block per wave
+		{
+			const int ib = kb + 1 + wave;
+			v16f acc = {};
+			if (ib < nb) {
+				// A = W[ib][kb]; B[k][c] = X[kb][kb][c][k]
+				sub_block_product(sub_block(Ws, ib, kb), 1, kLeafLd, sub_block(Xs, kb, kb), kLeafLd, 1, lane, acc);
+				store_sub_block(sub_block(Ws, ib, kb), lane, acc, 1.f);
+			}
+		}
+		__syncthreads();
+		// what is left of the lower triangle: W[ib][jb] -= L[ib][kb] L[jb][kb]^T
+		{
+			const int left = nb - kb - 1, tiles = left * (left + 1) / 2;
+			for (int t = wave; t < tiles; t += 4) {
+				int ib = 0, first = 0; // tile t of the triangle, row by row
+				while (first + ib + 1 <= t) first += ++ib;
+				const int jb = t - first;
+				float *C = sub_block(Ws, kb + 1 + ib, kb + 1 + jb);
+				v16f acc = {};
+				// A = L[ib][kb]; B[k][c] = L[jb][kb][c][k]
+				sub_block_product(sub_block(Ws, kb + 1 + ib, kb), 1, kLeafLd, sub_block(Ws, kb + 1 + jb, kb), kLeafLd, 1, lane, acc);
+				v16f old;
+				load_sub_block(C, lane, old);
+#pragma unroll
+				for (int v = 0; v < 16; v++) acc[v] = old[v] - acc[v];
+				store_sub_block(C, lane, acc, 1.f);
+			}
+		}
+		__syncthreads();
+	}
+
+	// the inverse of the factor below its diagonal sub-blocks, one row of sub-blocks after the other; the sums go
+	// through the unused upper triangle of Ws on their way from accumulator to operand layout
+	for (int ib = 1; ib < nb; ib++) {
+		const int jb = wave;
+		if (jb < ib) {
+			v16f acc = {};
+			for (int k = jb; k < ib; k++) // A = L[ib][k]; B = X[k][jb]
+				sub_block_product(sub_block(Ws, ib, k), 1, kLeafLd, sub_block(Xs, k, jb), 1, kLeafLd, lane, acc);
+			store_sub_block(sub_block(Ws, jb, ib), lane, acc, 1.f);
+		}
+		__syncthreads();
+		if (jb < ib) {
+			v16f acc = {};
+			// A = X[ib][ib]; B = the sum above
+			sub_block_product(sub_block(Xs, ib, ib), 1, kLeafLd, sub_block(Ws, jb, ib), 1, kLeafLd, lane, acc);
+			store_sub_block(sub_block(Xs, ib, jb), lane, acc, -1.f);
+		}
+		__syncthreads();
+	}
+
 	float *xblk = Xout + (size_t)k0 * ld + k0;
-	for (int c = 0; c < nb; c++)
-		if ((i < nb) & (i >= c)) xblk[(size_t)c * ld + i] = turn[c][i];
+	if (row < nn) {
+#pragma unroll
+		for (int b = 0; b < kLeaf / kSub; b++) {
+			if (b > rowBlock) break;
+#pragma unroll
+			for (int q = 0; q < kSub / 2; q++) {
+				const int c = b * kSub + half + 2 * q;
+				if (c <= row) xblk[(size_t)c * ld + row] = Xs[c * kLeafLd + row];
+			}
+		}
+	}
 }
 
 __global__ void __launch_bounds__(256) shifted_copy_kernel(const float *A, float *W, int n, float shift)
@@ -116,7 +289,7 @@ static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 // largest split-K workspace the products of a node of `blocks` 64-wide block columns (order nn) ask for
 static size_t node_gemm_workspace(int blocks, int nn)
 {
-	if (blocks <= 1) return 0;
+	if (blocks <= kLeafBlocks) return 0;
 	const int b1 = blocks / 2, n1 = b1 * kNb, m = nn - n1;
 	size_t g = gemm_ex_workspace(m, n1, n1, 0);
 	size_t a = gemm_ex_workspace(m, m, n1, kGemmMirror);
@@ -163,7 +336,7 @@ struct InverseRun {
 // floats of the largest L21 block at every recursion depth
 static void l21_sizes(int blocks, int nn, int depth, size_t *need)
 {
-	if (blocks <= 1 || depth >= kMaxDepth) return;
+	if (blocks <= kLeafBlocks || depth >= kMaxDepth) return;
 	const int b1 = blocks / 2, n1 = b1 * kNb, m = nn - n1;
 	const size_t sz = (size_t)m * n1;
 	if (sz > need[depth]) need[depth] = sz;
@@ -176,10 +349,10 @@ static int chol_and_inverse(const InverseRun &r, int r0, int blocks, int nn, int
 {
 	const int KC = FITRE_KC_SPD_INVERSE;
 	const int n = r.n;
-	if (blocks == 1) {
-		LaunchScope scope(KC, 2.0 * kNb * kNb * kNb / 3.0);
-		chol_diag_kernel<<<1, 64, 0, stream()>>>(r.W, n, r0, nn, r.X, r.dInfo);
-		return check_launch("chol_diag_kernel");
+	if (blocks <= kLeafBlocks) {
+		LaunchScope scope(KC, 2.0 * nn * (double)nn * nn / 3.0);
+		chol_leaf_kernel<<<1, 256, 0, stream()>>>(r.W, n, r0, nn, r.X, r.dInfo);
+		return check_launch("chol_leaf_kernel");
 	}
 	const int b1 = blocks / 2, n1 = b1 * kNb, m = nn - n1, r1 = r0 + n1;
 	FITRE_REQUIRE(depth < kMaxDepth, "fitre_hip_spd_inverse: recursion deeper than %d", kMaxDepth);
