@@ -18,10 +18,18 @@ hipStream_t stream(); // the selected lane
 // fitre_hip_gemm).  flags: kGemmMirror = the product is symmetric (M == N, same operand on
 // both sides): compute the tiles on and above the diagonal and mirror them; kGemmTriK = both
 // operands are zero where the reduction index is below their row / column index.
-constexpr int kGemmMirror = 1, kGemmTriK = 2;
+// kGemmBLowerTri / kGemmBUpperTri: op(B) (K x N) is zero above / below its diagonal; kGemmALowerTri: op(A) (M x K) is zero
+// above its diagonal -- the reduction skips the zero part (batched products only).
+constexpr int kGemmMirror = 1, kGemmTriK = 2, kGemmBLowerTri = 4, kGemmBUpperTri = 8, kGemmALowerTri = 16;
 int gemm_ex(int transA, int transB, int M, int N, int K, float alpha, const float *A, int lda, const float *B, int ldb,
             float beta, float *C, int ldc, const float *bias, int flags, int kernelClass, void *ws, size_t wsBytes);
 size_t gemm_ex_workspace(int M, int N, int K, int flags);
+// `batch` such products of one shape in one launch (plus one reduction launch when split).  Problem b reads
+// A + b*strideA, B + b*strideB, writes C + b*strideC and keeps its split-K partials in (char *)ws + b*wsStrideBytes;
+// wsBytes is the workspace of ONE problem (gemm_ex_workspace).
+int gemm_ex_batched(int batch, int transA, int transB, int M, int N, int K, float alpha, const float *A, int lda, long strideA,
+                    const float *B, int ldb, long strideB, float beta, float *C, int ldc, long strideC, int flags, int kernelClass,
+                    void *ws, size_t wsBytes, long wsStrideBytes);
 constexpr int kMaxLanes = 4; // one hardware queue each
 int lane();           // its index (0 .. kMaxLanes - 1)
 int lane_compute_units();     // compute units a kernel launched on the selected lane can occupy

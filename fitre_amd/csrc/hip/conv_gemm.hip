@@ -328,6 +328,39 @@ int gemm_ex(int transA, int transB, int M, int N, int K, float alpha, const floa
 }
 
 
+int gemm_ex_batched(int batch, int transA, int transB, int M, int N, int K, float alpha, const float *A, int lda, long strideA,
+                    const float *B, int ldb, long strideB, float beta, float *C, int ldc, long strideC, int flags, int kernelClass,
+                    void *ws, size_t wsBytes, long wsStrideBytes)
+{
+	FITRE_REQUIRE(A && B && C, "gemm_ex_batched: null pointer");
+	FITRE_REQUIRE(batch >= 1 && batch <= 64, "gemm_ex_batched: batch of %d", batch);
+	FITRE_REQUIRE(M > 0 && N > 0 && K > 0, "gemm_ex_batched: non-positive shape %d x %d x %d", M, N, K);
+	FITRE_REQUIRE((transA == 0 || transA == 1) && (transB == 0 || transB == 1), "gemm_ex_batched: bad transpose flags");
+	FITRE_REQUIRE(lda >= (transA ? K : M) && ldb >= (transB ? N : K) && ldc >= M, "gemm_ex_batched: leading dimension too small");
+	FITRE_REQUIRE(wsStrideBytes % 4 == 0, "gemm_ex_batched: workspace stride must be a multiple of 4 bytes");
+	const size_t aElems = (size_t)lda * (transA ? M : K), bElems = (size_t)ldb * (transB ? K : N);
+	FITRE_REQUIRE(aElems < ((size_t)1 << 30) && bElems < ((size_t)1 << 30), "gemm_ex_batched: an operand exceeds 2^30 elements");
+	FITRE_REQUIRE(!(flags & kGemmMirror) || M == N, "gemm: a mirrored product must be square");
+	const int I = N, J = M, R = K;
+	// every problem of the batch gets its share of the compute units
+	int cus = lane_compute_units() / batch;
+	if (cus < 1) cus = 1;
+	GemmPlan plan = plan_gemm(I, J, R, (flags & kGemmMirror) != 0, cus);
+	// engine operand A is op(B), engine operand B is op(A) (see gemm_ex)
+	const int tri = ((flags & kGemmTriK) ? kTriBoth : 0) | ((flags & kGemmBLowerTri) ? kTriAFromRow : 0) |
+	                ((flags & kGemmBUpperTri) ? kTriAToRow : 0) | ((flags & kGemmALowerTri) ? kTriBToRow : 0);
+	OutParams out{ C, (long)ldc, 0, nullptr, nullptr, alpha, beta, (flags & kGemmMirror) ? 1 : 0, tri };
+	const double flops = 2.0 * (double)M * N * K;
+	PlainParams bk{ B, (uint32_t)(bElems * sizeof(float)), ldb, I };
+	PlainParams ar{ A, (uint32_t)(aElems * sizeof(float)), lda, J };
+	const BatchStrides bs{ batch, strideB, strideA, strideC, wsStrideBytes / 4 };
+	if (!transB && !transA) return launch_gemm_batched<PlainKContig, PlainRowContig>(bk, ar, out, I, J, R, plan, ws, wsBytes, kernelClass, flops, bs);
+	if (!transB && transA) return launch_gemm_batched<PlainKContig, PlainKContig>(bk, ar, out, I, J, R, plan, ws, wsBytes, kernelClass, flops, bs);
+	if (transB && !transA) return launch_gemm_batched<PlainRowContig, PlainRowContig>(bk, ar, out, I, J, R, plan, ws, wsBytes, kernelClass, flops, bs);
+	return launch_gemm_batched<PlainRowContig, PlainKContig>(bk, ar, out, I, J, R, plan, ws, wsBytes, kernelClass, flops, bs);
+}
+
+
 } // namespace fitre
 
 using namespace fitre;

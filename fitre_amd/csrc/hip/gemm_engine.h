@@ -366,18 +366,22 @@ struct OutParams {
 	// diagonal are skipped, elements with j < i are not stored and every stored element with
 	// j > i is also written to C[j][i].  With split-K the mirroring happens in the reduction.
 	int mirror;
-	// Both operands are lower triangular in the reduction index (element (row, k) is zero for
-	// k < row): the reduction of a tile starts at the larger of its two first rows.
+	// Bit mask of kTri*: operands that are zero on one side of the diagonal in the reduction index.
 	int triK;
 };
+// both operands: element (row, k) is zero for k < row, so the reduction of a tile starts at the larger of its first rows
+constexpr int kTriBoth = 1;
+constexpr int kTriAFromRow = 2; // operand A: element (i, k) is zero for k < i
+constexpr int kTriAToRow = 4;   // operand A: element (i, k) is zero for k > i
+constexpr int kTriBToRow = 8;   // operand B: element (j, k) is zero for k > j
 
 // ---------------------------------------------------------------------------
 // the kernel
 // ---------------------------------------------------------------------------
+// One workgroup's tile of reduction range `split` (the body of both kernels below).
 template <class Cfg, class OpA, class OpB>
-__global__ void __launch_bounds__(kGemmThreads)
-mfma_gemm_kernel(const typename OpA::Params pa, const typename OpB::Params pb, const OutParams out, int I, int J, int R,
-                 int kChunk)
+__device__ __forceinline__ void gemm_tile(const typename OpA::Params &pa, const typename OpB::Params &pb, const OutParams &out,
+                                          int I, int J, int R, int kChunk, int splitIndex)
 {
 	constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK;
 	constexpr int TM = Cfg::TM, TN = Cfg::TN;
@@ -389,13 +393,21 @@ mfma_gemm_kernel(const typename OpA::Params pa, const typename OpB::Params pb, c
 	const int lane = tid & 63;
 	const int wave = tid >> 6;
 	const int i0 = blockIdx.y * BM, j0 = blockIdx.x * BN;
-	int kbeg = blockIdx.z * kChunk;
-	const int kend = (kbeg + kChunk < R) ? kbeg + kChunk : R;
+	int kbeg = splitIndex * kChunk;
+	int kend = (kbeg + kChunk < R) ? kbeg + kChunk : R;
 	if (out.mirror && j0 + BN <= i0) return; // the mirror tile produces these elements
-	if (out.triK) {
+	// triangular operands: the part of the reduction range in which an operand of this tile is all zero is skipped
+	// (a split whose whole range falls there writes a zero partial tile)
+	if (out.triK & kTriBoth) {
 		const int first = ((i0 > j0) ? i0 : j0) & ~(BK - 1);
 		kbeg = (kbeg > first) ? kbeg : first;
 	}
+	if (out.triK & kTriAFromRow) {
+		const int first = i0 & ~(BK - 1);
+		kbeg = (kbeg > first) ? kbeg : first;
+	}
+	if (out.triK & kTriAToRow) kend = (kend < i0 + BM) ? kend : i0 + BM;
+	if (out.triK & kTriBToRow) kend = (kend < j0 + BN) ? kend : j0 + BN;
 
 	OpA opA;
 	OpB opB;
@@ -460,7 +472,7 @@ mfma_gemm_kernel(const typename OpA::Params pa, const typename OpB::Params pb, c
 	// accumulator layout of the 32x32 block: register v of lane l holds
 	// row 8*(v/4) + 4*(l/32) + v%4, column l%32.
 	const bool split = out.splitStride != 0;
-	float *C = out.C + (size_t)blockIdx.z * out.splitStride;
+	float *C = out.C + (size_t)splitIndex * out.splitStride;
 #pragma unroll
 	for (int tm = 0; tm < TM; tm++) {
 #pragma unroll
@@ -487,12 +499,36 @@ mfma_gemm_kernel(const typename OpA::Params pa, const typename OpB::Params pb, c
 	}
 }
 
+template <class Cfg, class OpA, class OpB>
+__global__ void __launch_bounds__(kGemmThreads)
+mfma_gemm_kernel(const typename OpA::Params pa, const typename OpB::Params pb, const OutParams out, int I, int J, int R,
+                 int kChunk)
+{
+	gemm_tile<Cfg, OpA, OpB>(pa, pb, out, I, J, R, kChunk, blockIdx.z);
+}
+
+// `batch` independent products of one shape in one launch: grid.z = batch * splits; problem b reads its operands
+// aStride / bStride elements behind problem b-1's and writes cStride elements behind (plain operands only).
+template <class Cfg, class OpA, class OpB>
+__global__ void __launch_bounds__(kGemmThreads)
+mfma_gemm_batched_kernel(typename OpA::Params pa, typename OpB::Params pb, OutParams out, int I, int J, int R, int kChunk,
+                         int splits, long aStride, long bStride, long cStride)
+{
+	const int batch = blockIdx.z / splits, split = blockIdx.z - batch * splits;
+	pa.p += (size_t)batch * aStride;
+	pb.p += (size_t)batch * bStride;
+	out.C += (size_t)batch * cStride;
+	gemm_tile<Cfg, OpA, OpB>(pa, pb, out, I, J, R, kChunk, split);
+}
+
 // C[i*ldc + j] = alpha * sum_s ws[s][i][j] (+bias) + beta*C, partials summed in split order.
 // VEC = 4: four consecutive j per thread with 16-byte reads (J % 4 == 0, aligned workspace).
 template <int VEC>
 __global__ void __launch_bounds__(256)
-splitk_reduce_kernel(const float *ws, int splits, int I, int J, OutParams out)
+splitk_reduce_kernel(const float *ws, int splits, int I, int J, OutParams out, long wsBatchStride = 0, long cBatchStride = 0)
 {
+	ws += (size_t)blockIdx.y * wsBatchStride; // blockIdx.y: problem of a batch (0 otherwise)
+	out.C += (size_t)blockIdx.y * cBatchStride;
 	const long total = (long)I * J;
 	const long groups = total / VEC;
 	const long stride = (long)gridDim.x * blockDim.x;
@@ -547,8 +583,10 @@ splitk_reduce_kernel(const float *ws, int splits, int I, int J, OutParams out)
 // combined in a fixed order -- the parallelism comes from the partials, not from the output.
 template <int VEC>
 __global__ void __launch_bounds__(256)
-splitk_reduce_wide_kernel(const float *ws, int splits, int I, int J, OutParams out)
+splitk_reduce_wide_kernel(const float *ws, int splits, int I, int J, OutParams out, long wsBatchStride = 0, long cBatchStride = 0)
 {
+	ws += (size_t)blockIdx.y * wsBatchStride;
+	out.C += (size_t)blockIdx.y * cBatchStride;
 	__shared__ double part[16][16 * VEC + 1];
 	const long total = (long)I * J;
 	const long groups = total / VEC;
@@ -592,19 +630,21 @@ splitk_reduce_wide_kernel(const float *ws, int splits, int I, int J, OutParams o
 }
 
 // Sums `splits` partial I x J matrices from ws into fin (alpha, beta and biases applied once).
-static inline void launch_splitk_reduce(const float *ws, int splits, int I, int J, const OutParams &fin)
+static inline void launch_splitk_reduce(const float *ws, int splits, int I, int J, const OutParams &fin, int batch = 1,
+                                        long wsBatchStride = 0, long cBatchStride = 0)
 {
-	LaunchScope scope(FITRE_KC_SPLITK_REDUCE, 4.0 * (double)I * J * (splits + 1));
-	const bool vec = (J % 4 == 0) && ((((uintptr_t)ws) & 15) == 0);
+	LaunchScope scope(FITRE_KC_SPLITK_REDUCE, 4.0 * (double)I * J * (splits + 1) * batch);
+	const bool vec = (J % 4 == 0) && ((((uintptr_t)ws) & 15) == 0) && (wsBatchStride % 4 == 0);
 	const long groups = (long)I * J / (vec ? 4 : 1);
 	const bool wide = splits >= 32 && groups <= 64 * 1024; // too few outputs to fill the chip one thread each
 	if (wide) {
-		const unsigned blocks = (unsigned)((groups + 15) / 16);
-		if (vec) splitk_reduce_wide_kernel<4><<<blocks, 256, 0, stream()>>>(ws, splits, I, J, fin);
-		else splitk_reduce_wide_kernel<1><<<blocks, 256, 0, stream()>>>(ws, splits, I, J, fin);
+		const dim3 blocks((unsigned)((groups + 15) / 16), (unsigned)batch);
+		if (vec) splitk_reduce_wide_kernel<4><<<blocks, 256, 0, stream()>>>(ws, splits, I, J, fin, wsBatchStride, cBatchStride);
+		else splitk_reduce_wide_kernel<1><<<blocks, 256, 0, stream()>>>(ws, splits, I, J, fin, wsBatchStride, cBatchStride);
 	} else {
-		if (vec) splitk_reduce_kernel<4><<<blocks_for(groups, 256, 8192), 256, 0, stream()>>>(ws, splits, I, J, fin);
-		else splitk_reduce_kernel<1><<<blocks_for(groups, 256, 8192), 256, 0, stream()>>>(ws, splits, I, J, fin);
+		const dim3 blocks(blocks_for(groups, 256, 8192), (unsigned)batch);
+		if (vec) splitk_reduce_kernel<4><<<blocks, 256, 0, stream()>>>(ws, splits, I, J, fin, wsBatchStride, cBatchStride);
+		else splitk_reduce_kernel<1><<<blocks, 256, 0, stream()>>>(ws, splits, I, J, fin, wsBatchStride, cBatchStride);
 	}
 }
 
@@ -770,6 +810,63 @@ static int launch_gemm(const PA &pa, const PB &pb, const OutParams &out, int I, 
 	if (plan.bm == 64 && plan.bn == 128) return launch_tile<OpA, OpB, 64, 128>(pa, pb, out, I, J, R, plan, ws, kernelClass, flops);
 	if (plan.bm == 128 && plan.bn == 64) return launch_tile<OpA, OpB, 128, 64>(pa, pb, out, I, J, R, plan, ws, kernelClass, flops);
 	return launch_tile<OpA, OpB, 64, 64>(pa, pb, out, I, J, R, plan, ws, kernelClass, flops);
+}
+
+// ---- batched products of plain operands ------------------------------------------------------------------------
+struct BatchStrides {
+	int batch;
+	long a, b, c; // elements between the operands / results of consecutive problems
+	long ws;      // floats between their split-K workspaces
+};
+
+template <template <int, int> class OpA, template <int, int> class OpB, int BM, int BN>
+static int launch_tile_batched(const PlainParams &pa, const PlainParams &pb, const OutParams &out, int I, int J, int R,
+                               const GemmPlan &plan, void *ws, int kernelClass, double flops, const BatchStrides &bs)
+{
+	typedef TileCfg<BM, BN, kGemmBK> Cfg;
+	constexpr int tileId = (BM == 64 ? (BN == 64 ? 1 : 2) : (BN == 64 ? 3 : 4));
+	typedef OpA<BM, kGemmBK> A;
+	typedef OpB<BN, kGemmBK> B;
+	dim3 grid((J + BN - 1) / BN, (I + BM - 1) / BM, plan.splits * bs.batch);
+	if (grid.y > 65535 || grid.z > 65535) return fail(FITRE_E_UNSUPPORTED, "gemm grid %u x %u x %u too large", grid.x, grid.y, grid.z);
+	if (plan.splits > 1) {
+		OutParams part = out;
+		part.C = (float *)ws;
+		part.ldc = J;
+		part.splitStride = (long)I * J;
+		{
+			LaunchScope scope(kernelClass, flops * bs.batch, tileId);
+			mfma_gemm_batched_kernel<Cfg, A, B><<<grid, kGemmThreads, 0, stream()>>>(pa, pb, part, I, J, R, plan.kChunk, plan.splits, bs.a,
+			                                                                        bs.b, bs.ws);
+		}
+		OutParams fin = out;
+		fin.splitStride = 0;
+		launch_splitk_reduce((const float *)ws, plan.splits, I, J, fin, bs.batch, bs.ws, bs.c);
+	} else {
+		OutParams direct = out;
+		direct.splitStride = 0;
+		LaunchScope scope(kernelClass, flops * bs.batch, tileId);
+		mfma_gemm_batched_kernel<Cfg, A, B><<<grid, kGemmThreads, 0, stream()>>>(pa, pb, direct, I, J, R, plan.kChunk, 1, bs.a, bs.b, bs.c);
+	}
+	return check_launch("mfma_gemm_batched_kernel");
+}
+
+// wsBytes: the workspace of ONE problem (problem b's starts bs.ws floats behind problem b-1's)
+template <template <int, int> class OpA, template <int, int> class OpB>
+static int launch_gemm_batched(const PlainParams &pa, const PlainParams &pb, const OutParams &out, int I, int J, int R,
+                               const GemmPlan &ideal, void *ws, size_t wsBytes, int kernelClass, double flops, const BatchStrides &bs)
+{
+	const GemmPlan plan = fit_plan(ideal, I, J, R, ws, wsBytes);
+	if (plan.wsBytes > 0) {
+		if (!ws || (((uintptr_t)ws) & 3)) return fail(FITRE_E_WORKSPACE, "split-K workspace is null or misaligned");
+		if (wsBytes < plan.wsBytes)
+			return fail(FITRE_E_WORKSPACE, "split-K workspace of %zu bytes is smaller than the %zu required", wsBytes, plan.wsBytes);
+	}
+	if (plan.bm == 128 && plan.bn == 128)
+		return launch_tile_batched<OpA, OpB, 128, 128>(pa, pb, out, I, J, R, plan, ws, kernelClass, flops, bs);
+	if (plan.bm == 64 && plan.bn == 128) return launch_tile_batched<OpA, OpB, 64, 128>(pa, pb, out, I, J, R, plan, ws, kernelClass, flops, bs);
+	if (plan.bm == 128 && plan.bn == 64) return launch_tile_batched<OpA, OpB, 128, 64>(pa, pb, out, I, J, R, plan, ws, kernelClass, flops, bs);
+	return launch_tile_batched<OpA, OpB, 64, 64>(pa, pb, out, I, J, R, plan, ws, kernelClass, flops, bs);
 }
 
 } // namespace fitre

@@ -153,8 +153,13 @@ __device__ __forceinline__ float *sub_block(float *M, int rb, int cb) { return M
 // The diagonal block of order nn (1..128) that starts at row/column k0 of W (column-major, leading dimension
 // ld, lower triangle read): X = L^-1 of its Cholesky factor into the same block of Xout (lower triangle written).
 // info: set to the 1-based global index of the first non-positive pivot.
-__global__ void __launch_bounds__(256) chol_leaf_kernel(const float *W, int ld, int k0, int nn, float *Xout, int *info)
+// Workgroup b of the launch works on the b-th matrix of a batch (wStride / xStride floats behind the one before).
+__global__ void __launch_bounds__(256) chol_leaf_kernel(const float *W, int ld, int k0, int nn, float *Xout, int *info, long wStride,
+                                                        long xStride)
 {
+	W += (size_t)blockIdx.x * wStride;
+	Xout += (size_t)blockIdx.x * xStride;
+	info += blockIdx.x;
 	__shared__ float Ws[kLeaf * kLeafLd];
 	__shared__ float Xs[kLeaf * kLeafLd];
 	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -252,8 +257,11 @@ __global__ void __launch_bounds__(256) chol_leaf_kernel(const float *W, int ld, 
 	}
 }
 
-__global__ void __launch_bounds__(256) shifted_copy_kernel(const float *A, float *W, int n, float shift)
+// blockIdx.y: matrix of a batch
+__global__ void __launch_bounds__(256) shifted_copy_kernel(const float *A, float *W, int n, float shift, long aStride, long wStride)
 {
+	A += (size_t)blockIdx.y * aStride;
+	W += (size_t)blockIdx.y * wStride;
 	const long total = (long)n * n;
 	const long stride = (long)gridDim.x * blockDim.x;
 	for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
@@ -273,8 +281,9 @@ __global__ void __launch_bounds__(256) block_copy_kernel(const float *src, int l
 	}
 }
 
-__global__ void __launch_bounds__(256) fill_zero_kernel(float *p, long n)
+__global__ void __launch_bounds__(256) fill_zero_kernel(float *p, long n, long batchStride)
 {
+	p += (size_t)blockIdx.y * batchStride;
 	const long stride = (long)gridDim.x * blockDim.x;
 	for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < n; idx += stride) p[idx] = 0.f;
 }
@@ -324,6 +333,9 @@ static InverseLayout inverse_layout(int n)
 // state of one inverse while its launches are queued
 constexpr int kMaxDepth = 16;
 struct InverseRun {
+	int batch;       // matrices worked on side by side, every launch covers all of them
+	long sWs, sInv;  // floats between the workspaces (W, X, product workspace) resp. the result matrices of two of them
+	long wsStrideBytes;
 	float *W, *X;
 	float *L21[kMaxDepth]; // per recursion depth: the off-diagonal block of the factor (a node's children work one level down)
 	float *T2;             // temporary of the last product of a node
@@ -350,8 +362,8 @@ static int chol_and_inverse(const InverseRun &r, int r0, int blocks, int nn, int
 	const int KC = FITRE_KC_SPD_INVERSE;
 	const int n = r.n;
 	if (blocks <= kLeafBlocks) {
-		LaunchScope scope(KC, 2.0 * nn * (double)nn * nn / 3.0);
-		chol_leaf_kernel<<<1, 256, 0, stream()>>>(r.W, n, r0, nn, r.X, r.dInfo);
+		LaunchScope scope(KC, 2.0 * nn * (double)nn * nn / 3.0 * r.batch);
+		chol_leaf_kernel<<<r.batch, 256, 0, stream()>>>(r.W, n, r0, nn, r.X, r.dInfo, r.sWs, r.sWs);
 		return check_launch("chol_leaf_kernel");
 	}
 	const int b1 = blocks / 2, n1 = b1 * kNb, m = nn - n1, r1 = r0 + n1;
@@ -363,19 +375,23 @@ static int chol_and_inverse(const InverseRun &r, int r0, int blocks, int nn, int
 	const float *X11 = r.X + (size_t)r0 * n + r0;
 	float *L21 = r.L21[depth];
 	// L21 = A21 * X11^T (m x n1); W keeps A21: only X is needed in the end
-	rc = gemm_ex(0, 1, m, n1, n1, 1.f, A21, n, X11, n, 0.f, L21, m, nullptr, 0, KC, r.gws, r.gBytes);
+	rc = gemm_ex_batched(r.batch, 0, 1, m, n1, n1, 1.f, A21, n, r.sWs, X11, n, r.sWs, 0.f, L21, m, r.sInv, kGemmBUpperTri, KC, r.gws, r.gBytes,
+	                     r.wsStrideBytes);
 	if (rc) return rc;
 	// A22 -= L21 L21^T
-	rc = gemm_ex(0, 1, m, m, n1, -1.f, L21, m, L21, m, 1.f, A22, n, nullptr, kGemmMirror, KC, r.gws, r.gBytes);
+	rc = gemm_ex_batched(r.batch, 0, 1, m, m, n1, -1.f, L21, m, r.sInv, L21, m, r.sInv, 1.f, A22, n, r.sWs, kGemmMirror, KC, r.gws,
+	                     r.gBytes, r.wsStrideBytes);
 	if (rc) return rc;
 	rc = chol_and_inverse(r, r1, blocks - b1, m, depth + 1);
 	if (rc) return rc;
 	// X21 = -X22 * (L21 * X11)
 	const float *X22 = r.X + (size_t)r1 * n + r1;
 	float *X21 = r.X + (size_t)r0 * n + r1;
-	rc = gemm_ex(0, 0, m, n1, n1, 1.f, L21, m, X11, n, 0.f, r.T2, m, nullptr, 0, KC, r.gws, r.gBytes);
+	rc = gemm_ex_batched(r.batch, 0, 0, m, n1, n1, 1.f, L21, m, r.sInv, X11, n, r.sWs, 0.f, r.T2, m, r.sInv, kGemmBLowerTri, KC, r.gws, r.gBytes,
+	                     r.wsStrideBytes);
 	if (rc) return rc;
-	return gemm_ex(0, 0, m, n1, m, -1.f, X22, n, r.T2, m, 0.f, X21, n, nullptr, 0, KC, r.gws, r.gBytes);
+	return gemm_ex_batched(r.batch, 0, 0, m, n1, m, -1.f, X22, n, r.sWs, r.T2, m, r.sInv, 0.f, X21, n, r.sWs, kGemmALowerTri, KC, r.gws, r.gBytes,
+	                       r.wsStrideBytes);
 }
 
 } // namespace fitre
@@ -390,18 +406,33 @@ size_t fitre_hip_spd_inverse_workspace(int n)
 	return inverse_layout(n).total;
 }
 
-// queues the whole inverse on the selected lane; pivotInfo: device int that receives the 1-based index of the
-// first non-positive pivot, or stays zero (null: a slot of the workspace)
+// Everything one call needs to know about the matrices it inverts side by side: problem b reads
+// matrix + b*matrixStride, writes inverse + b*inverseStride (floats), works in (char *)ws + b*wsStrideBytes and
+// reports its pivot in pivotInfo[b].
+struct InverseBatch {
+	int batch;
+	long matrixStride, inverseStride, wsStrideBytes;
+};
+
+// queues the whole inverse on the selected lane; pivotInfo: device ints (one per matrix) that receive the 1-based
+// index of the first non-positive pivot, or stay zero (null: a slot of the workspace, single matrices only)
 static int spd_inverse_run(const float *matrix, int n, float shift, float *inverse, void *ws, size_t wsBytes, int *pivotInfo,
-                           int **infoSlot)
+                           int **infoSlot, const InverseBatch &ib)
 {
 	FITRE_REQUIRE(matrix && inverse && ws, "fitre_hip_spd_inverse: null pointer");
 	FITRE_REQUIRE(n > 0 && n <= 23000, "fitre_hip_spd_inverse: order %d out of range", n);
 	FITRE_REQUIRE((((uintptr_t)ws) & 255) == 0, "fitre_hip_spd_inverse: workspace must be 256-byte aligned");
+	FITRE_REQUIRE(ib.batch >= 1 && ib.batch <= 16, "fitre_hip_spd_inverse: batch of %d", ib.batch);
 	const InverseLayout lay = inverse_layout(n);
 	if (wsBytes < lay.total)
 		return fail(FITRE_E_WORKSPACE, "fitre_hip_spd_inverse: workspace of %zu bytes is smaller than the %zu required", wsBytes,
 		            lay.total);
+	if (ib.batch > 1) {
+		FITRE_REQUIRE(pivotInfo != nullptr, "fitre_hip_spd_inverse: a batch needs pivot slots");
+		FITRE_REQUIRE(ib.wsStrideBytes % 256 == 0 && (size_t)ib.wsStrideBytes >= lay.total,
+		              "fitre_hip_spd_inverse: workspaces of a batch overlap or are misaligned");
+		FITRE_REQUIRE(ib.inverseStride >= (long)n * n && ib.matrixStride >= (long)n * n, "fitre_hip_spd_inverse: matrices of a batch overlap");
+	}
 	char *base = (char *)ws;
 	float *W = (float *)(base + lay.w), *X = (float *)(base + lay.x);
 	int *dInfo = pivotInfo ? pivotInfo : (int *)(base + lay.info);
@@ -410,19 +441,22 @@ static int spd_inverse_run(const float *matrix, int n, float shift, float *inver
 	const size_t gBytes = lay.gemmBytes;
 	const int blocks = (n + kNb - 1) / kNb;
 	const int KC = FITRE_KC_SPD_INVERSE;
+	const long sWs = ib.wsStrideBytes / 4;
 	int rc;
 
 	{
-		LaunchScope scope(FITRE_KC_BLAS1, 8.0 * (double)n * n);
-		shifted_copy_kernel<<<blocks_for((long)n * n, 256, 8192), 256, 0, stream()>>>(matrix, W, n, shift);
-		fill_zero_kernel<<<blocks_for((long)n * n, 256, 8192), 256, 0, stream()>>>(X, (long)n * n);
-		fill_zero_kernel<<<1, 64, 0, stream()>>>((float *)dInfo, 1);
+		LaunchScope scope(FITRE_KC_BLAS1, 8.0 * (double)n * n * ib.batch);
+		const dim3 grid(blocks_for((long)n * n, 256, 8192), (unsigned)ib.batch);
+		shifted_copy_kernel<<<grid, 256, 0, stream()>>>(matrix, W, n, shift, ib.matrixStride, sWs);
+		fill_zero_kernel<<<grid, 256, 0, stream()>>>(X, (long)n * n, sWs);
+		fill_zero_kernel<<<1, 64, 0, stream()>>>((float *)dInfo, ib.batch, 0);
 	}
 	// ---- 1. Cholesky factor and its inverse ---------------------------------------------------
 	// The result matrix is free until the last product and holds the temporaries: T2 (at most a
 	// quarter of the matrix) in its second half, the per-depth L21 blocks (a quarter, a sixteenth,
 	// ... of it) in the first.
 	InverseRun run;
+	run.batch = ib.batch, run.sWs = sWs, run.sInv = ib.inverseStride, run.wsStrideBytes = ib.wsStrideBytes;
 	run.W = W, run.X = X, run.n = n, run.dInfo = dInfo, run.gws = gws, run.gBytes = gBytes;
 	run.T2 = inverse + ((size_t)n * n + 1) / 2;
 	{
@@ -438,7 +472,8 @@ static int spd_inverse_run(const float *matrix, int n, float shift, float *inver
 	rc = chol_and_inverse(run, 0, blocks, n);
 	if (rc) return rc;
 	// ---- 2. A^-1 = X^T X ------------------------------------------------------------------------
-	rc = gemm_ex(1, 0, n, n, n, 1.f, X, n, X, n, 0.f, inverse, n, nullptr, kGemmMirror | kGemmTriK, KC, gws, gBytes);
+	rc = gemm_ex_batched(ib.batch, 1, 0, n, n, n, 1.f, X, n, sWs, X, n, sWs, 0.f, inverse, n, ib.inverseStride, kGemmMirror | kGemmTriK,
+	                     KC, gws, gBytes, ib.wsStrideBytes);
 	if (rc) return rc;
 	return check_launch("fitre_hip_spd_inverse");
 }
@@ -447,7 +482,7 @@ int fitre_hip_spd_inverse(const float *matrix, int n, float shift, float *invers
 {
 	FITRE_NEED_INIT();
 	int *dInfo = nullptr;
-	int rc = spd_inverse_run(matrix, n, shift, inverse, ws, wsBytes, nullptr, &dInfo);
+	int rc = spd_inverse_run(matrix, n, shift, inverse, ws, wsBytes, nullptr, &dInfo, InverseBatch{ 1, 0, 0, 0 });
 	if (rc) return rc;
 	if (info) {
 		int h = 0;
@@ -463,7 +498,16 @@ int fitre_hip_spd_inverse_queued(const float *matrix, int n, float shift, float 
 {
 	FITRE_NEED_INIT();
 	FITRE_REQUIRE(pivotInfo != nullptr, "fitre_hip_spd_inverse_queued: null pivot slot");
-	return spd_inverse_run(matrix, n, shift, inverse, ws, wsBytes, pivotInfo, nullptr);
+	return spd_inverse_run(matrix, n, shift, inverse, ws, wsBytes, pivotInfo, nullptr, InverseBatch{ 1, 0, 0, 0 });
+}
+
+int fitre_hip_spd_inverse_batched_queued(int batch, const float *matrix, long matrixStride, int n, float shift, float *inverse,
+                                         long inverseStride, void *ws, size_t wsBytes, long wsStrideBytes, int *pivotInfo)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(pivotInfo != nullptr, "fitre_hip_spd_inverse_batched_queued: null pivot slots");
+	return spd_inverse_run(matrix, n, shift, inverse, ws, wsBytes, pivotInfo, nullptr,
+	                       InverseBatch{ batch, matrixStride, inverseStride, wsStrideBytes });
 }
 
 } // extern "C"

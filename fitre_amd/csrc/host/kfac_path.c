@@ -173,145 +173,218 @@ static size_t inverse_scratch_bytes(const CNN_MODEL *model, int samples, size_t 
 
 static char *aligned_base(real *devPtr) { return (char *)(((size_t)devPtr + 255) & ~(size_t)255); }
 
-/* The inverses of a pass are independent of each other: they are dealt to the four lanes, each lane with a
- * [factor | workspace] region of its own, and the pivot reports are read once at the end. */
+/* The inverses of a pass are independent of each other.  Consecutive layers whose factors have the same order
+ * (the wide layers at the end of a VGG) are inverted as ONE batch -- one chain of launches, each covering all
+ * matrices of the batch -- and the batches are dealt, costliest first, to the four lanes.  Every lane owns as
+ * many [factor | workspace] slots as the largest batch it accepts; the pivot reports are read once at the end. */
 #define KFAC_LANES 4
+#define KFAC_SLOTS 7
+#define KFAC_MAX_BATCH 3
+#define KFAC_MIN_BATCH_ORDER 1024
 #define KFAC_INFO_BYTES 1024 /* one int per layer, MAX_LAYERS of them */
+static const int kLaneSlots[KFAC_LANES] = { 3, 2, 1, 1 };
+static const int kLaneFirstSlot[KFAC_LANES] = { 0, 3, 5, 6 };
 
 long kfacInverseMemRequired(CNN_MODEL *model, int samples)
 {
 	size_t factorBytes;
-	return (long)((KFAC_LANES * inverse_scratch_bytes(model, samples, &factorBytes) + KFAC_INFO_BYTES) / sizeof(real)) + 64;
+	return (long)((KFAC_SLOTS * inverse_scratch_bytes(model, samples, &factorBytes) + KFAC_INFO_BYTES) / sizeof(real)) + 64;
 }
 
-typedef struct inverse_pass {
-	char *region[KFAC_LANES]; /* [factor | workspace] of each lane */
-	size_t factorBytes, wsBytes;
-	int *pivots;              /* device, one per layer */
-	double load[KFAC_LANES];  /* work dealt to each lane so far */
-	int layers;
-} INVERSE_PASS;
+/* writes the factor of `layer` (pass numbering: convolution layers, then linear ones) into `factor` */
+typedef void (*FACTOR_FN)(void *ctx, int layer, real *factor, real *ws, size_t wsBytes);
 
-static void inverse_pass_begin(INVERSE_PASS *p, const CNN_MODEL *model, int samples, real *devPtr)
+typedef struct inverse_job {
+	int first, count; /* layers first .. first+count-1 */
+	int order;
+	double cost;
+	int lane;
+} INVERSE_JOB;
+
+static int job_by_cost(const void *a, const void *b)
 {
-	const size_t total = inverse_scratch_bytes(model, samples, &p->factorBytes);
+	const INVERSE_JOB *x = (const INVERSE_JOB *)a, *y = (const INVERSE_JOB *)b;
+	if (x->cost != y->cost) return x->cost < y->cost ? 1 : -1;
+	return x->first - y->first;
+}
+
+/* order[l]: order of layer l's factor; offset[l]: where its inverse goes in inverseBase (offset[l+1] - offset[l] is
+ * at least order[l]^2); group[l]: layers may share a batch only inside one group (convolution / linear) */
+static void inverse_pass_run(const CNN_MODEL *model, int samples, real *devPtr, int layers, const int *order, const int *offset,
+                             const int *group, real *inverseBase, real shift, FACTOR_FN make, void *ctx)
+{
+	size_t factorBytes;
+	const size_t slotBytes = inverse_scratch_bytes(model, samples, &factorBytes);
+	const size_t wsBytes = slotBytes - factorBytes - 256;
 	char *base = aligned_base(devPtr);
-	p->pivots = (int *)base;
-	for (int k = 0; k < KFAC_LANES; k++) {
-		p->region[k] = base + KFAC_INFO_BYTES + (size_t)k * total;
-		p->load[k] = 0;
+	int *pivots = (int *)base;
+	char *slots = base + KFAC_INFO_BYTES;
+
+	/* batches: runs of consecutive layers of one order, at most KFAC_MAX_BATCH long */
+	INVERSE_JOB jobs[MAX_LAYERS];
+	int nJobs = 0;
+	for (int l = 0; l < layers;) {
+		int count = 1;
+		/* small matrices gain nothing from a shared chain (measured: the output-side pass, orders up to 512, is
+		 * faster with one lane per matrix) */
+		while (order[l] >= KFAC_MIN_BATCH_ORDER && l + count < layers && count < KFAC_MAX_BATCH && order[l + count] == order[l] && group[l + count] == group[l] &&
+		       offset[l + count + 1] - offset[l + count] == offset[l + 1] - offset[l])
+			count++;
+		INVERSE_JOB *j = &jobs[nJobs++];
+		j->first = l;
+		j->count = count;
+		j->order = order[l];
+		/* measured: the time of an inverse grows a little slower than n^2, and a batch pays for the chain once */
+		j->cost = (double)order[l] * order[l] * (0.6 + 0.4 * count);
+		l += count;
 	}
-	p->wsBytes = total - p->factorBytes - 256;
-	p->layers = model->cLayers + model->lLayers;
+	qsort(jobs, (size_t)nJobs, sizeof(INVERSE_JOB), job_by_cost);
+	double load[KFAC_LANES] = { 0, 0, 0, 0 };
+	for (int i = 0; i < nJobs; i++) {
+		int lane = -1;
+		for (int k = 0; k < KFAC_LANES; k++)
+			if (kLaneSlots[k] >= jobs[i].count && (lane < 0 || load[k] < load[lane])) lane = k;
+		jobs[i].lane = lane;
+		load[lane] += jobs[i].cost;
+	}
+
 	for (int k = 1; k < KFAC_LANES; k++) HIP_CALL(fitre_hip_lane_wait(k, 0)); /* after what lane 0 has queued so far (z, dx) */
-}
-
-/* the lane with the least work so far takes the next matrix of order n; returns its factor buffer */
-static real *inverse_pass_pick(INVERSE_PASS *p, int n, real **ws)
-{
-	int lane = 0;
-	for (int k = 1; k < KFAC_LANES; k++)
-		if (p->load[k] < p->load[lane]) lane = k;
-	p->load[lane] += (double)n * n; /* measured: the time of an inverse grows a little slower than n^2 */
-	HIP_CALL(fitre_hip_lane_select(lane));
-	*ws = (real *)(p->region[lane] + p->factorBytes);
-	return (real *)p->region[lane];
-}
-
-static void inverse_pass_queue(INVERSE_PASS *p, int layer, real *factor, real *inverse, int n, real *ws, real shift)
-{
-	HIP_CALL(fitre_hip_spd_inverse_queued(factor, n, shift, inverse, ws, p->wsBytes, p->pivots + layer));
-}
-
-static void inverse_pass_end(INVERSE_PASS *p)
-{
+	for (int i = 0; i < nJobs; i++) {
+		const INVERSE_JOB *j = &jobs[i];
+		char *slot0 = slots + (size_t)kLaneFirstSlot[j->lane] * slotBytes;
+		HIP_CALL(fitre_hip_lane_select(j->lane));
+		for (int b = 0; b < j->count; b++) {
+			char *slot = slot0 + (size_t)b * slotBytes;
+			make(ctx, j->first + b, (real *)slot, (real *)(slot + factorBytes), wsBytes);
+		}
+		const int l = j->first;
+		if (j->count == 1)
+			HIP_CALL(fitre_hip_spd_inverse_queued((real *)slot0, j->order, shift, inverseBase + offset[l], slot0 + factorBytes, wsBytes,
+			                                      pivots + l));
+		else
+			HIP_CALL(fitre_hip_spd_inverse_batched_queued(j->count, (real *)slot0, (long)(slotBytes / sizeof(real)), j->order, shift,
+			                                              inverseBase + offset[l], (long)(offset[l + 1] - offset[l]),
+			                                              slot0 + factorBytes, wsBytes, (long)slotBytes, pivots + l));
+	}
 	int host[MAX_LAYERS];
 	HIP_CALL(fitre_hip_lane_select(0));
 	HIP_CALL(fitre_hip_sync());
-	HIP_CALL(fitre_hip_copy_d2h(host, p->pivots, sizeof(int) * (size_t)p->layers));
-	for (int l = 0; l < p->layers; l++)
+	HIP_CALL(fitre_hip_copy_d2h(host, pivots, sizeof(int) * (size_t)layers));
+	for (int l = 0; l < layers; l++)
 		if (host[l] != 0) {
 			fprintf(stderr, "We have a problem with the LU factorization ... %d (layer %d)\n", host[l], l);
 			exit(-1);
 		}
 }
 
+typedef struct omega_ctx {
+	const CNN_MODEL *model;
+	const DEVICE_DATASET *data;
+	int samples, withBias;
+	const real *dampedInput, *dampedZ;
+	const int *zOffsets, *zztOffsets;
+} OMEGA_CTX;
+
+static void omega_factor(void *ctx, int layer, real *factor, real *ws, size_t wsBytes)
+{
+	const OMEGA_CTX *o = (const OMEGA_CTX *)ctx;
+	const CNN_MODEL *model = o->model;
+	const int nc = model->cLayers;
+	if (layer < nc) {
+		const int l = layer;
+		const CONV_LAYER *c = &model->convLayer[l];
+		const real *input;
+		if (o->dampedInput != NULL)
+			input = (l == 0) ? o->dampedInput : o->dampedZ + o->zztOffsets[l];
+		else
+			input = (l == 0) ? o->data->currentBatch : o->dampedZ + o->zOffsets[l] + model->convLayer[l - 1].outputOffset;
+		fitre_conv_shape s = conv_shape(c, o->samples);
+		HIP_CALL(fitre_hip_kfac_conv_input_factor(&s, input, o->withBias, factor, ws, wsBytes));
+	} else {
+		const int l = layer - nc;
+		const FC_LAYER *f = &model->fcLayer[l];
+		const real *input;
+		if (o->dampedInput != NULL)
+			input = o->dampedZ + o->zztOffsets[nc + l];
+		else if (l == 0)
+			input = o->dampedZ + o->zOffsets[nc] + model->convLayer[nc - 1].outputOffset;
+		else
+			input = o->dampedZ + o->zOffsets[nc + l];
+		HIP_CALL(fitre_hip_kfac_fc_input_factor(input, f->in, o->samples, o->withBias, factor, ws, wsBytes));
+	}
+}
 
 void computeOmegaZ(KFAC_CURVATURE_INFO *kfac_info, CNN_MODEL *model, DEVICE_DATASET *data, int samples,
                    real *dampedInput, real *dampedZ, real *omegaZInv, int *zOffsets, int *zztOffsets, real *devPtr,
                    real *pageLckPtr)
 {
 	(void)pageLckPtr;
-	const int *omega = kfac_info->OmegaZOffsets;
 	const int withBias = model->bias != 0;
-	const int nc = model->cLayers;
-	const real shift = kfac_info->regLambda + kfac_info->dampGamma;
-	INVERSE_PASS pass;
-	inverse_pass_begin(&pass, model, samples, devPtr);
-
-	/* largest orders first, so that the two lanes end at about the same time */
-	for (int l = nc - 1; l >= 0; l--) {
+	const int nc = model->cLayers, layers = nc + model->lLayers;
+	int order[MAX_LAYERS], group[MAX_LAYERS];
+	for (int l = 0; l < nc; l++) {
 		const CONV_LAYER *c = &model->convLayer[l];
-		const real *input;
-		if (dampedInput != NULL)
-			input = (l == 0) ? dampedInput : dampedZ + zztOffsets[l];
-		else
-			input = (l == 0) ? data->currentBatch : dampedZ + zOffsets[l] + model->convLayer[l - 1].outputOffset;
-		const int zCols = c->inChannels * c->kSize * c->kSize + (withBias ? 1 : 0);
-		fitre_conv_shape s = conv_shape(c, samples);
-		real *ws, *zzt = inverse_pass_pick(&pass, zCols, &ws);
-		HIP_CALL(fitre_hip_kfac_conv_input_factor(&s, input, withBias, zzt, ws, pass.wsBytes));
-		inverse_pass_queue(&pass, l, zzt, omegaZInv + omega[l], zCols, ws, shift);
+		order[l] = c->inChannels * c->kSize * c->kSize + (withBias ? 1 : 0);
+		group[l] = 0;
 	}
 	for (int l = 0; l < model->lLayers; l++) {
-		const FC_LAYER *f = &model->fcLayer[l];
-		const real *input;
-		if (dampedInput != NULL)
-			input = dampedZ + zztOffsets[nc + l];
-		else if (l == 0)
-			input = dampedZ + zOffsets[nc] + model->convLayer[nc - 1].outputOffset;
-		else
-			input = dampedZ + zOffsets[nc + l];
-		const int zRows = f->in + (withBias ? 1 : 0);
-		real *ws, *zzt = inverse_pass_pick(&pass, zRows, &ws);
-		HIP_CALL(fitre_hip_kfac_fc_input_factor(input, f->in, samples, withBias, zzt, ws, pass.wsBytes));
-		inverse_pass_queue(&pass, nc + l, zzt, omegaZInv + omega[nc + l], zRows, ws, shift);
+		order[nc + l] = model->fcLayer[l].in + (withBias ? 1 : 0);
+		group[nc + l] = 1;
 	}
-	inverse_pass_end(&pass);
+	OMEGA_CTX ctx = { model, data, samples, withBias, dampedInput, dampedZ, zOffsets, zztOffsets };
+	inverse_pass_run(model, samples, devPtr, layers, order, kfac_info->OmegaZOffsets, group, omegaZInv,
+	                 kfac_info->regLambda + kfac_info->dampGamma, omega_factor, &ctx);
+}
+
+typedef struct lambda_ctx {
+	const CNN_MODEL *model;
+	int samples;
+	const real *dx, *dampedLambda;
+	const int *zOffsets, *zztOffsets;
+} LAMBDA_CTX;
+
+static void lambda_factor(void *ctx, int layer, real *factor, real *ws, size_t wsBytes)
+{
+	const LAMBDA_CTX *o = (const LAMBDA_CTX *)ctx;
+	const CNN_MODEL *model = o->model;
+	const int nc = model->cLayers;
+	if (layer < nc) {
+		const int l = layer;
+		const CONV_LAYER *c = &model->convLayer[l];
+		const real *delta;
+		if (o->dampedLambda != NULL)
+			delta = o->dampedLambda + o->zztOffsets[l + 1];
+		else if (c->batchNorm == PERFORM_NO_BATCH_NORM)
+			delta = o->dx + o->zOffsets[l + 1] + c->activationOffset;
+		else
+			delta = o->dx + o->zOffsets[l + 1] + c->batchNormOffset;
+		fitre_conv_shape s = conv_shape(c, o->samples);
+		HIP_CALL(fitre_hip_kfac_conv_output_factor(&s, delta, factor, ws, wsBytes));
+	} else {
+		const int l = layer - nc;
+		const FC_LAYER *f = &model->fcLayer[l];
+		const real *delta = (o->dampedLambda != NULL) ? o->dampedLambda + o->zztOffsets[nc + l + 1] : o->dx + o->zOffsets[nc + l + 1];
+		HIP_CALL(fitre_hip_kfac_fc_output_factor(delta, f->out, o->samples, factor, ws, wsBytes));
+	}
 }
 
 void computeLambdaDelta(KFAC_CURVATURE_INFO *kfac_info, CNN_MODEL *model, int samples, real *dx, real *dampedLambda,
                         real *lambdaGInv, int *zOffsets, int *zztOffsets, real *devPtr, real *pageLckPtr)
 {
 	(void)pageLckPtr;
-	const int *lambda = kfac_info->LambdaGOffsets;
-	const int nc = model->cLayers;
-	const real shift = kfac_info->regLambda + kfac_info->dampGamma;
-	INVERSE_PASS pass;
-	inverse_pass_begin(&pass, model, samples, devPtr);
-
-	for (int l = nc - 1; l >= 0; l--) {
-		const CONV_LAYER *c = &model->convLayer[l];
-		const real *delta;
-		if (dampedLambda != NULL)
-			delta = dampedLambda + zztOffsets[l + 1];
-		else if (c->batchNorm == PERFORM_NO_BATCH_NORM)
-			delta = dx + zOffsets[l + 1] + c->activationOffset;
-		else
-			delta = dx + zOffsets[l + 1] + c->batchNormOffset;
-		fitre_conv_shape s = conv_shape(c, samples);
-		real *ws, *ggt = inverse_pass_pick(&pass, c->outChannels, &ws);
-		HIP_CALL(fitre_hip_kfac_conv_output_factor(&s, delta, ggt, ws, pass.wsBytes));
-		inverse_pass_queue(&pass, l, ggt, lambdaGInv + lambda[l], c->outChannels, ws, shift);
+	const int nc = model->cLayers, layers = nc + model->lLayers;
+	int order[MAX_LAYERS], group[MAX_LAYERS];
+	for (int l = 0; l < nc; l++) {
+		order[l] = model->convLayer[l].outChannels;
+		group[l] = 0;
 	}
 	for (int l = 0; l < model->lLayers; l++) {
-		const FC_LAYER *f = &model->fcLayer[l];
-		const real *delta = (dampedLambda != NULL) ? dampedLambda + zztOffsets[nc + l + 1] : dx + zOffsets[nc + l + 1];
-		real *ws, *ggt = inverse_pass_pick(&pass, f->out, &ws);
-		HIP_CALL(fitre_hip_kfac_fc_output_factor(delta, f->out, samples, ggt, ws, pass.wsBytes));
-		inverse_pass_queue(&pass, nc + l, ggt, lambdaGInv + lambda[nc + l], f->out, ws, shift);
+		order[nc + l] = model->fcLayer[l].out;
+		group[nc + l] = 1;
 	}
-	inverse_pass_end(&pass);
+	LAMBDA_CTX ctx = { model, samples, dx, dampedLambda, zOffsets, zztOffsets };
+	inverse_pass_run(model, samples, devPtr, layers, order, kfac_info->LambdaGOffsets, group, lambdaGInv,
+	                 kfac_info->regLambda + kfac_info->dampGamma, lambda_factor, &ctx);
 }
 
 /* ---- natural gradient ---------------------------------------------------------------------- */

@@ -110,6 +110,7 @@ HIP_API = {
     "fitre_hip_spd_inverse_workspace": (sz, [i32]),
     "fitre_hip_spd_inverse": (i32, [vp, i32, f32, vp, vp, sz, pi32]),
     "fitre_hip_spd_inverse_queued": (i32, [vp, i32, f32, vp, vp, sz, vp]),
+    "fitre_hip_spd_inverse_batched_queued": (i32, [i32, vp, lng, i32, f32, vp, lng, vp, sz, lng, vp]),
     "fitre_hip_kfac_conv_input_factor_workspace": (sz, [vp, i32]),
     "fitre_hip_kfac_conv_input_factor": (i32, [vp, vp, i32, vp, vp, sz]),
     "fitre_hip_kfac_gram_workspace": (sz, [i32, C.c_long]),

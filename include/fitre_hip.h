@@ -382,6 +382,15 @@ int fitre_hip_spd_inverse(const float *matrix, int n, float shift, float *invers
  * side by side on different lanes (each with its own matrix, result and workspace). */
 int fitre_hip_spd_inverse_queued(const float *matrix, int n, float shift, float *inverse, void *ws,
                                  size_t wsBytes, int *pivotInfo);
+/* `batch` (1..16) matrices of ONE order inverted side by side by one chain of launches, every launch covering
+ * all of them (the KFAC factors of consecutive layers of equal width): matrix b is at
+ * matrix + b*matrixStride, its inverse goes to inverse + b*inverseStride (strides in floats, at least n*n), its
+ * workspace is (char *)ws + b*wsStrideBytes (a multiple of 256, at least fitre_hip_spd_inverse_workspace(n) =
+ * wsBytes), its pivot report pivotInfo[b] (device ints).  An inverse is a chain of several hundred small dependent
+ * launches; a batch pays for the chain once. */
+int fitre_hip_spd_inverse_batched_queued(int batch, const float *matrix, long matrixStride, int n, float shift,
+                                         float *inverse, long inverseStride, void *ws, size_t wsBytes,
+                                         long wsStrideBytes, int *pivotInfo);
 
 #ifdef __cplusplus
 }

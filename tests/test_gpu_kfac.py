@@ -213,6 +213,49 @@ def test_spd_inverse(dev, oracle64, n):
         dev.free(q)
 
 
+@pytest.mark.parametrize("n,batch", [(1, 2), (33, 3), (129, 4), (200, 3), (577, 2)])
+def test_spd_inverse_batched(dev, oracle64, n, batch):
+    """Several matrices of one order through one chain of launches: each result against the oracle's inverse of
+    its own matrix, with strides larger than the matrices, and the pivot report of the one indefinite matrix of
+    a second batch in its own slot."""
+    rng = np.random.default_rng(100 * n + batch)
+    shift = 0.02
+    mats = [((lambda a: (a + a.T) / 2)(_spd(n, rng, 1000.0))).astype(np.float32) for _ in range(batch)]
+    m_stride, i_stride = n * n + 24, n * n + 64
+    packed = np.zeros(batch * m_stride, np.float32)
+    for b, a in enumerate(mats):
+        packed[b * m_stride:b * m_stride + n * n] = a.reshape(-1)
+    pa = dev.upload(packed)
+    out = dev.upload(np.full(batch * i_stride, np.nan, dtype=np.float32))
+    one = hip.fitre_hip_spd_inverse_workspace(n)
+    ws_stride = (one + 255) // 256 * 256 + 512
+    ws = dev.alloc(batch * ws_stride)
+    piv = dev.upload(np.full(batch, -1, np.int32), np.int32)
+    L.check(hip.fitre_hip_spd_inverse_batched_queued(batch, pa, m_stride, n, shift, out, i_stride, ws, one, ws_stride, piv))
+    dev.sync()
+    assert not dev.download(piv, batch, np.int32).any()
+    got_all = dev.download(out, batch * i_stride)
+    for b, a in enumerate(mats):
+        got = got_all[b * i_stride:b * i_stride + n * n].reshape(n, n)
+        _, want = oracle64.matrix_inverse(a.astype(np.float64), n, shift, 0.0)
+        assert rel_err(got, want) < TOL, b
+        assert np.array_equal(got, got.T)
+        assert np.isnan(got_all[b * i_stride + n * n:(b + 1) * i_stride]).all()    # nothing written between the results
+    if n >= 33:
+        bad = 1 if batch > 1 else 0
+        packed[bad * m_stride + 5 * n + 5] = -7.0                                    # a negative diagonal entry
+        L.check(hip.fitre_hip_copy_h2d(pa, packed.ctypes.data_as(C.c_void_p), packed.nbytes))
+        L.check(hip.fitre_hip_spd_inverse_batched_queued(batch, pa, m_stride, n, shift, out, i_stride, ws, one, ws_stride, piv))
+        dev.sync()
+        report = dev.download(piv, batch, np.int32)
+        assert report[bad] == 6 and not np.delete(report, bad).any(), report
+    # argument checks: overlapping workspaces, overlapping results
+    assert hip.fitre_hip_spd_inverse_batched_queued(2, pa, m_stride, n, shift, out, i_stride, ws, one, 256 if one > 256 else 0, piv) != 0
+    assert hip.fitre_hip_spd_inverse_batched_queued(2, pa, m_stride, n, shift, out, n * n - 1, ws, one, ws_stride, piv) != 0
+    for q in (pa, out, ws, piv):
+        dev.free(q)
+
+
 def test_spd_inverse_reports_indefinite_matrix(dev):
     a = np.array([[1.0, 2.0], [2.0, 1.0]], dtype=np.float32)
     pa, out = dev.upload(a.reshape(-1)), dev.zeros(4)
