@@ -361,6 +361,34 @@ int gemm_ex_batched(int batch, int transA, int transB, int M, int N, int K, floa
 }
 
 
+// C(MxN) = alpha*op(A)*op(B) + beta*C (+ bias per row), column-major, for products far below one engine tile: sixteen
+// lanes share an output element, each takes every sixteenth reduction index, and their sums are combined by shuffles.
+constexpr double kSmallProductWork = 4.0e6; // multiply-adds
+__global__ void __launch_bounds__(256) small_product_kernel(int transA, int transB, int M, int N, int K, float alpha, const float *A,
+                                                            int lda, const float *B, int ldb, float beta, float *C, int ldc,
+                                                            const float *bias)
+{
+	const int part = threadIdx.x & 15;
+	const long o = (long)blockIdx.x * 16 + (threadIdx.x >> 4);
+	const bool live = o < (long)M * N;
+	const int n = live ? (int)(o / M) : 0, m = live ? (int)(o - (long)n * M) : 0;
+	const float *a = transA ? A + (size_t)m * lda : A + m;
+	const float *b = transB ? B + n : B + (size_t)n * ldb;
+	const long aStep = transA ? 1 : lda, bStep = transB ? ldb : 1;
+	float acc = 0.f;
+	for (int k = part; k < K; k += 16) acc = fmaf(a[k * aStep], b[k * bStep], acc);
+#pragma unroll
+	for (int off = 8; off >= 1; off >>= 1) acc += __shfl_xor(acc, off, 16);
+	if (live && part == 0) {
+		float v = alpha * acc;
+		if (bias) v += bias[m];
+		float *dst = C + (size_t)n * ldc + m;
+		if (beta != 0.f) v += beta * *dst;
+		*dst = v;
+	}
+}
+
+
 } // namespace fitre
 
 using namespace fitre;
@@ -490,6 +518,17 @@ int fitre_hip_gemm(int transA, int transB, int M, int N, int K, float alpha, con
                    float beta, float *C, int ldc, const float *bias, void *ws, size_t wsBytes)
 {
 	FITRE_NEED_INIT();
+	if (M > 0 && N > 0 && K > 0 && (double)M * N * K <= kSmallProductWork) {
+		// a product this small (the output layer of a network: ten classes) does not fill one tile of the engine
+		FITRE_REQUIRE(A && B && C, "fitre_hip_gemm: null pointer");
+		FITRE_REQUIRE((transA == 0 || transA == 1) && (transB == 0 || transB == 1), "fitre_hip_gemm: bad transpose flags");
+		FITRE_REQUIRE(lda >= (transA ? K : M) && ldb >= (transB ? N : K) && ldc >= M, "fitre_hip_gemm: leading dimension too small");
+		const long outputs = (long)M * N;
+		LaunchScope scope(FITRE_KC_FC_GEMM, 2.0 * (double)M * N * K, 0);
+		small_product_kernel<<<(unsigned)((outputs + 15) / 16), 256, 0, stream()>>>(transA, transB, M, N, K, alpha, A, lda, B, ldb, beta, C,
+		                                                                         ldc, bias);
+		return check_launch("small_product_kernel");
+	}
 	return gemm_ex(transA, transB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, bias, 0, FITRE_KC_FC_GEMM, ws, wsBytes);
 }
 

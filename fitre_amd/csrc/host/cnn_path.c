@@ -93,6 +93,12 @@ static size_t backward_dx_ws_bytes(const CNN_MODEL *model, int batch)
 		const FC_LAYER *f = &model->fcLayer[i];
 		need = max_sz(need, fitre_hip_gemm_workspace(f->in, batch, f->out));
 	}
+	if (model->cLayers > 0) {
+		/* the first linear layer's delta in the convolution layout, until the last convolution layer has read it */
+		int extA, extB;
+		feature_extent(model, &extA, &extB);
+		need = max_sz(need, sizeof(real) * (size_t)extA * extB * batch * model->convLayer[model->cLayers - 1].outChannels);
+	}
 	return (need + 255) & ~(size_t)255;
 }
 
@@ -270,20 +276,19 @@ void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, 
 		delta = temp;
 	}
 
-	/* [N][C][b*A+a] -> [C][N][a*B+b] */
+	/* [N][C][b*A+a] -> [C][N][a*B+b], into the chain workspace: lane 1 may still read delta_new (the first linear
+	 * layer's delta), and the chain does not wait for it.  The workspace is free until the last convolution layer's
+	 * input gradient, which is queued behind the pass that reads this tensor. */
+	real *features = (real *)ws;
 	{
 		int extA, extB;
 		feature_extent(model, &extA, &extB);
-		HIP_CALL(fitre_hip_lane_wait(0, 1)); /* lane 1 may still read delta_new (the first FC layer's delta) */
-		HIP_CALL(fitre_hip_fc_to_conv(delta, last->outChannels, n, extA, extB, delta_new));
-		temp = delta_new;
-		delta_new = delta;
-		delta = temp;
+		HIP_CALL(fitre_hip_fc_to_conv(delta, last->outChannels, n, extA, extB, features));
 	}
 
 	/* delta as the layer above left it: a plain tensor, or the unsummed split partials of its input
 	 * gradient (summed by the pool / activation pass below while it reads them) */
-	fitre_split_view dview = { delta, 1, 0 };
+	fitre_split_view dview = { features, 1, 0 };
 	for (int c = nc - 1; c >= 0; c--) {
 		const CONV_LAYER *l = &model->convLayer[c];
 		const POOL_LAYER *p = &model->poolLayer[c];
@@ -304,7 +309,10 @@ void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, 
 			/* The forward pass rewrote this layer's activation output into the FC layout in place;
 			 * rebuild it from the activation input (the reference reads the permuted buffer,
 			 * functions/cnn_backward.cu:574-580). */
-			if (!fusedRelu) HIP_CALL(fitre_hip_activation_forward(act, actIn, delta_new, perChannel * l->outChannels));
+			if (!fusedRelu) {
+				HIP_CALL(fitre_hip_lane_wait(0, 1)); /* lane 1 may still read delta_new */
+				HIP_CALL(fitre_hip_activation_forward(act, actIn, delta_new, perChannel * l->outChannels));
+			}
 			actOut = delta_new;
 		}
 		const real *cur;
@@ -321,7 +329,7 @@ void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, 
 			cur = dslab + l->batchNormOffset;
 		} else {
 			/* pool backward -> dx slab + 0; times f'(.) -> dx slab + activationOffset */
-			HIP_CALL(fitre_hip_pool_act_backward(p->type, act, delta, actIn, actOut, l->outChannels, n, p->width, p->height,
+			HIP_CALL(fitre_hip_pool_act_backward(p->type, act, dview.base, actIn, actOut, l->outChannels, n, p->width, p->height,
 			                                     p->pSize, p->stride, p->padding, p->outWidth, p->outHeight, dslab,
 			                                     dslab + l->activationOffset));
 			cur = dslab + l->activationOffset;
