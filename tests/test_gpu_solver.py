@@ -30,7 +30,7 @@ def synthetic_sets(rng, classes, per_class, test_per_class, features):
     return draw(per_class), draw(test_per_class)
 
 
-def run_solver(dev, inverse_freq, epochs, seed):
+def run_solver(dev, inverse_freq, epochs, seed, check_grad=0, momentum=0.0, reg_lambda=0.0):
     rng = np.random.default_rng(seed)
     batch, classes, feats = 64, 10, 3 * 32 * 32
     model = build_lenet(batch, bn=True)
@@ -46,8 +46,8 @@ def run_solver(dev, inverse_freq, epochs, seed):
     data.features, data.height, data.width = feats, 32, 32
 
     info = KFAC_CURVATURE_INFO()
-    info.regLambda, info.dampGamma, info.momentum, info.stats_decay = 0.0, 0.1, 0.0, 0.9
-    info.checkGrad, info.inverseFreq = 0, inverse_freq
+    info.regLambda, info.dampGamma, info.momentum, info.stats_decay = reg_lambda, 0.1, momentum, 0.9
+    info.checkGrad, info.inverseFreq = check_grad, inverse_freq
     tr = TRUST_REGION_PARAMS()
     tr.delta, tr.minDelta, tr.maxDelta, tr.maxIters = 0.5, 1e-3, 4.0, epochs
 
@@ -90,6 +90,16 @@ def test_solver_trains_a_separable_set(dev, inverse_freq, epochs):
     assert reports[-1].trainAccuracy > 70.0 and reports[-1].testAccuracy > 70.0, [(r.trainAccuracy, r.testAccuracy) for r in reports]
     assert sum(r.rejectedSteps for r in reports) <= 7, [r.rejectedSteps for r in reports]
     assert all(r.weightNorm > 0 and r.seconds > 0 for r in reports)
+
+
+def test_solver_with_gradient_check_momentum_and_weight_decay(dev):
+    """The branch that compares the natural-gradient step with the plain gradient step (checkGrad), a momentum
+    term on the step and L2 regularisation in gradient and curvature: the loop still trains."""
+    reports, weights, delta = run_solver(dev, 1, 3, seed=5, check_grad=1, momentum=0.2, reg_lambda=1e-4)
+    assert np.isfinite(weights).all()
+    losses = [r.trainLikelihood for r in reports]
+    assert np.isfinite(losses).all() and losses[-1] < 1.5 and losses[-1] < losses[0], losses
+    assert reports[-1].trainAccuracy > 60.0, [r.trainAccuracy for r in reports]
 
 
 def test_solver_is_reproducible(dev):
