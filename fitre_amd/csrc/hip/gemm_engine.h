@@ -671,11 +671,18 @@ inline double estimate_us(long tiles, int bm, int bn, long I, long J, long R, lo
 	chunk = ((chunk + kGemmBK - 1) / kGemmBK) * kGemmBK;
 	long s = (R + chunk - 1) / chunk;
 	long groups = tiles * s;
-	long perCu = (groups + cus - 1) / cus;
 	// one k-step of a bm x bn tile keeps the four matrix pipes of a compute unit busy for this long
 	double stepUs = (double)(bm / 32) * (bn / 32) * (kGemmBK / 2) * 64.0 / 4.0 / 2400.0;
-	double eff = perCu >= 3 ? 0.80 : (perCu == 2 ? 0.68 : 0.52);
-	double t = (double)perCu * (double)(chunk / kGemmBK) * stepUs / eff + 3.0;
+	// Workgroups run in rounds of three per compute unit; a round that is not full leaves the pipes less well fed,
+	// and one behind full rounds worse still (measured on symmetric products of order 1152 and 2304: 684 workgroups
+	// beat 1197, which beat 855).
+	const double perGroup = (double)(chunk / kGemmBK) * stepUs;
+	const long full = groups / (3 * cus), rest = groups - full * 3 * cus;
+	const long perCu = (rest + cus - 1) / cus;
+	double t = (double)full * 3.0 * perGroup / 0.80 + 3.0;
+	if (perCu >= 3) t += 3.0 * perGroup / 0.80;
+	else if (perCu == 2) t += 2.0 * perGroup / 0.62;
+	else if (perCu == 1) t += perGroup / (full > 0 ? 0.40 : 0.52);
 	if (s > 1) t += 8.0 + (double)(s + 1) * (double)I * (double)J * 4.0 / 3.0e6; // second launch; ~3 TB/s, bytes -> us
 	*chunkOut = chunk;
 	*splitsOut = s;

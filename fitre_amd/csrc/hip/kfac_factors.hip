@@ -6,25 +6,68 @@
 //   fully connected, input    A = Z Z^T / samples,  Z = [ z ; 1 ]   (z is in x samples)
 //   fully connected, output   G = D D^T * samples,  D = delta (out x samples)
 //
-// The patch matrix P is never materialised: both operands of P^T P gather their elements
-// from the image, and the column of ones is a constant row of the operand.
+// The input-side factor of a convolution first writes P^T (one row per patch index, positions
+// contiguous, the row of ones last) into its workspace and then runs the plain symmetric product
+// on it: 150 MB at most for VGG-11 at batch 256, written and read at HBM speed, against operand
+// fetches that decode every element's patch coordinates (measured: 100-124 TFLOP/s on the rows
+// against 63 with the gather).  With a workspace too small for the rows both operands gather their
+// elements from the image and the column of ones is a constant row of the operand.
 #include "conv_common.h"
 
 namespace fitre {
 
-// last row and column of the fully connected input factor: A[n][j] = A[j][n] = mean_s z[j][s], A[n][n] = 1.
-// `sums` holds the row sums of z and may alias the factor's last row.
-__global__ void __launch_bounds__(256) fc_factor_border_kernel(float *factor, const float *sums, int in, float invSamples)
+// last row and column of an input factor of order in + 1 (the bias): A[n][j] = A[j][n] = sums[j] * scale, A[n][n] = corner.
+// `sums` holds the row sums of the operand and may alias the factor's last row.
+__global__ void __launch_bounds__(256) fc_factor_border_kernel(float *factor, const float *sums, int in, float scale, float corner)
 {
 	const int n = in + 1;
 	const int j = blockIdx.x * blockDim.x + threadIdx.x;
 	if (j < in) {
-		float v = sums[j] * invSamples;
+		float v = sums[j] * scale;
 		factor[(size_t)in * n + j] = v;
 		factor[(size_t)j * n + in] = v;
 	} else if (j == in) {
-		factor[(size_t)in * n + in] = 1.f;
+		factor[(size_t)in * n + in] = corner;
 	}
+}
+
+// rows[row][m] = src[c][n][oa*stride - pad + ta][ob*stride - pad + tb] for row = (c, ta, tb) and position m = (n, oa, ob),
+// zero outside the image.  blockIdx.y: row.
+__global__ void __launch_bounds__(256) patch_rows_kernel(PatchGeom g, float *rows)
+{
+	const uint32_t row = blockIdx.y;
+	float *dst = rows + (size_t)row * g.positions;
+	const long stride = (long)gridDim.x * blockDim.x;
+	uint32_t c, tap, ta, tb;
+	g.divTaps.divmod(row, c, tap);
+	g.divK.divmod(tap, ta, tb);
+	const float *src = g.src + (size_t)c * g.chanStride;
+	for (long m = (long)blockIdx.x * blockDim.x + threadIdx.x; m < g.positions; m += stride) {
+		uint32_t q, ob, n, oa;
+		g.divOutB.divmod((uint32_t)m, q, ob);
+		g.divOutA.divmod(q, n, oa);
+		const int a = (int)oa * g.stride - g.pad + (int)ta, b = (int)ob * g.stride - g.pad + (int)tb;
+		const bool ok = ((unsigned)a < (unsigned)g.srcA) & ((unsigned)b < (unsigned)g.srcB);
+		dst[m] = ok ? src[(size_t)n * g.srcA * g.srcB + (size_t)a * g.srcB + b] : 0.f;
+	}
+}
+
+static size_t patch_rows_bytes(const fitre_conv_shape *s)
+{
+	const size_t bytes = (size_t)s->inChannels * s->ksize * s->ksize * (size_t)s->samples * s->outA * s->outB * sizeof(float);
+	return (bytes + 255) & ~(size_t)255;
+}
+
+// workspace behind the rows: the product's split partials, then (the product queued) the partial sums of the rows
+static size_t patch_rows_tail_bytes(const fitre_conv_shape *s, int withBias)
+{
+	const long K = (long)s->inChannels * s->ksize * s->ksize, R = (long)s->samples * s->outA * s->outB;
+	size_t tail = plan_gemm_workspace(K, K, R, true);
+	if (withBias) {
+		const size_t sums = fitre_hip_channel_sum_workspace((int)K, R);
+		tail = sums > tail ? sums : tail;
+	}
+	return (tail + 255) & ~(size_t)255;
 }
 
 } // namespace fitre
@@ -37,7 +80,12 @@ size_t fitre_hip_kfac_conv_input_factor_workspace(const fitre_conv_shape *s, int
 {
 	if (!s) return 0;
 	const long n = (long)s->inChannels * s->ksize * s->ksize + (withBias ? 1 : 0);
-	return plan_gemm_workspace(n, n, (long)s->samples * s->outA * s->outB, true);
+	const size_t product = plan_gemm_workspace(n, n, (long)s->samples * s->outA * s->outB, true);
+	const size_t rows = patch_rows_bytes(s);
+	// the rows of P^T in front of the product's own workspace, when an operand of that size can be addressed
+	if (rows / sizeof(float) >= ((size_t)1 << 30)) return product;
+	const size_t withRows = rows + patch_rows_tail_bytes(s, withBias);
+	return withRows > product ? withRows : product;
 }
 
 int fitre_hip_kfac_conv_input_factor(const fitre_conv_shape *s, const float *x, int withBias, float *factor, void *ws,
@@ -58,6 +106,29 @@ int fitre_hip_kfac_conv_input_factor(const fitre_conv_shape *s, const float *x, 
 	GemmPlan plan = plan_gemm(n, n, R, true);
 	OutParams out{ factor, (long)n, 0, nullptr, nullptr, 1.f / (cells * cells * (float)s->samples), 0.f, 1 };
 	const double flops = (double)n * (n + 1) * (double)R; // 2 flops per element of the upper triangle and position
+	// Rows of P^T in the workspace, the plain symmetric product on them (order K: whole tiles for the usual channel
+	// counts), and the bias row and column from the row sums: A[n][j] = sum_m P[m][j] / samples.
+	const size_t rowBytes = patch_rows_bytes(s);
+	if (ws && (((uintptr_t)ws) & 255) == 0 && rowBytes / sizeof(float) < ((size_t)1 << 30) &&
+	    wsBytes >= rowBytes + patch_rows_tail_bytes(s, withBias)) {
+		float *rows = (float *)ws;
+		void *tail = (char *)ws + rowBytes;
+		const size_t tailBytes = wsBytes - rowBytes;
+		{
+			LaunchScope scope(FITRE_KC_BLAS1, 2.0 * (double)rowBytes);
+			const dim3 grid(blocks_for(R, 256, 64), (unsigned)K);
+			patch_rows_kernel<<<grid, 256, 0, stream()>>>(g, rows);
+		}
+		PlainParams pr{ rows, (uint32_t)rowBytes, R, K };
+		rc = launch_gemm<PlainKContig, PlainKContig>(pr, pr, out, K, K, R, plan_gemm(K, K, R, true), tail, tailBytes,
+		                                             FITRE_KC_KFAC_FACTOR, flops);
+		if (rc || !withBias) return rc;
+		float *last = factor + (size_t)K * n;
+		rc = fitre_hip_channel_sum(rows, K, R, last, tail, tailBytes);
+		if (rc) return rc;
+		fc_factor_border_kernel<<<blocks_for(n, 256), 256, 0, stream()>>>(factor, last, K, 1.f / (cells * (float)s->samples), cells);
+		return check_launch("fc_factor_border_kernel");
+	}
 	if (withBias)
 		return launch_gemm<PatchKContigOnes, PatchKContigOnes>(g, g, out, n, n, R, plan, ws, wsBytes, FITRE_KC_KFAC_FACTOR, flops);
 	return launch_gemm<PatchKContig, PatchKContig>(g, g, out, n, n, R, plan, ws, wsBytes, FITRE_KC_KFAC_FACTOR, flops);
@@ -100,7 +171,7 @@ int fitre_hip_kfac_fc_input_factor(const float *z, int in, int samples, int with
 	float *last = factor + (size_t)in * n;
 	rc = fitre_hip_row_sum(z, in, samples, last);
 	if (rc) return rc;
-	fc_factor_border_kernel<<<blocks_for(n, 256), 256, 0, stream()>>>(factor, last, in, 1.f / (float)samples);
+	fc_factor_border_kernel<<<blocks_for(n, 256), 256, 0, stream()>>>(factor, last, in, 1.f / (float)samples, 1.f);
 	return check_launch("fc_factor_border_kernel");
 }
 

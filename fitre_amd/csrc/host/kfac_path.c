@@ -2,7 +2,7 @@
  * Kronecker-factor stage of the KFAC curvature approximation as C host code over the
  * C-ABI device layer: layer walk and data sources of solvers/kfac_inverses.cu:450-630
  * (computeOmegaZ) and :759-857 (computeLambdaDelta), storage offsets of
- * solvers/kfac_utils.cu:6-54.  No patch matrix, no scaled copies: each factor is one
+ * solvers/kfac_utils.cu:6-54.  No scaled copies: each factor is one
  * symmetric product on the device.
  */
 #include <stdio.h>

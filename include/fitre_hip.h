@@ -324,7 +324,10 @@ int fitre_hip_gemm(int transA, int transB, int M, int N, int K, float alpha, con
  *
  * Convolution, input side (solvers/kfac_inverses.cu:489-540): A = P^T P / samples with
  * P = [ im2col(x) / (outA*outB) , 1 ], order Cin*k*k (+1 with bias); patch column order
- * (c, ta, tb) as in the weight layout.  The patch matrix is not materialised. */
+ * (c, ta, tb) as in the weight layout.  With the workspace the _workspace call asks for, the transposed
+ * patch matrix (Cin*k*k rows of samples*outA*outB values) is written there first and the product runs on
+ * it; with a 256-byte aligned workspace that only covers the split-K partials, or a smaller one, both
+ * operands gather their elements from x instead (slower, no extra memory). */
 size_t fitre_hip_kfac_conv_input_factor_workspace(const fitre_conv_shape *s, int withBias);
 int fitre_hip_kfac_conv_input_factor(const fitre_conv_shape *s, const float *x, int withBias, float *factor,
                                      void *ws, size_t wsBytes);
