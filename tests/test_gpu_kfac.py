@@ -49,6 +49,36 @@ def test_conv_input_factor(dev, oracle64, case, bias):
     assert np.array_equal(got, got.T)  # the lower triangle is a copy of the upper one
 
 
+@pytest.mark.parametrize("bias", [True, False])
+@pytest.mark.parametrize("case", FACTOR_CASES[:4])
+def test_conv_input_factor_without_room_for_the_patch_rows(dev, oracle64, case, bias):
+    """A workspace that only covers the product's split partials (or none at all): both operands gather their
+    elements from the image; same result as with the rows written out."""
+    N, Cin, Cout, A, B, k, s, p = case
+    shape = conv_shape(N, Cin, Cout, A, B, k, s, p)
+    n = Cin * k * k + (1 if bias else 0)
+    rng = np.random.default_rng(sum(case) + 7)
+    x = (rng.standard_normal(Cin * N * A * B) + 0.3).astype(np.float32)
+    px = dev.upload(x)
+    full = hip.fitre_hip_kfac_conv_input_factor_workspace(C.byref(shape), int(bias))
+    small = hip.fitre_hip_kfac_gram_workspace(n, N * shape.outA * shape.outB)
+    assert small < full
+    ws = dev.alloc(full)
+    want = oracle64.kfac_conv_input_factor(x, N, Cin, B, A, k, p, s, bias)
+    results = []
+    for nb in (full, small, 0):
+        out = dev.upload(np.full(n * n, np.nan, dtype=np.float32))
+        L.check(hip.fitre_hip_kfac_conv_input_factor(C.byref(shape), px, int(bias), out, ws if nb else None, nb))
+        got = dev.download(out, n * n).reshape(n, n)
+        assert rel_err(got, want) < TOL, nb
+        assert np.array_equal(got, got.T)
+        results.append(got)
+        dev.free(out)
+    assert rel_err(results[1], results[0]) < 1e-5 and rel_err(results[2], results[0]) < 1e-5
+    for q in (px, ws):
+        dev.free(q)
+
+
 @pytest.mark.parametrize("case", [(4, 3, 64, 32, 32, 3, 1, 1), (2, 64, 130, 16, 16, 3, 1, 1), (16, 8, 300, 2, 2, 3, 1, 1),
                                   (2, 3, 6, 32, 32, 5, 1, 0)])
 def test_conv_output_factor(dev, oracle64, case):
