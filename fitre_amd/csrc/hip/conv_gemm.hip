@@ -346,6 +346,8 @@ int gemm_ex_batched(int batch, int transA, int transB, int M, int N, int K, floa
 	int cus = lane_compute_units() / batch;
 	if (cus < 1) cus = 1;
 	GemmPlan plan = plan_gemm(I, J, R, (flags & kGemmMirror) != 0, cus);
+	GemmPlan deep;
+	if (deep_slice_plan(I, J, R, (flags & kGemmMirror) != 0, batch, lane_compute_units(), plan, &deep)) plan = deep;
 	// engine operand A is op(B), engine operand B is op(A) (see gemm_ex)
 	const int tri = ((flags & kGemmTriK) ? kTriBoth : 0) | ((flags & kGemmBLowerTri) ? kTriAFromRow : 0) |
 	                ((flags & kGemmBUpperTri) ? kTriAToRow : 0) | ((flags & kGemmALowerTri) ? kTriBToRow : 0);

@@ -656,9 +656,12 @@ struct GemmPlan {
 	int splits;     // grid.z
 	int kChunk;     // reduction indices per split (multiple of BK)
 	size_t wsBytes; // workspace needed (0 when unsplit)
+	int bk;         // depth of a reduction slice (kGemmBK; kGemmDeepBK for small batched products)
+	double estimateUs;
 };
 
 constexpr int kGemmBK = 16;
+constexpr int kGemmDeepBK = 64;
 
 // Estimated duration (microseconds) of a product cut into `splits` reduction ranges.
 // Workgroups are spread evenly over the compute units; a compute unit runs up to three of
@@ -717,6 +720,8 @@ inline GemmPlan plan_gemm_search(long I, long J, long R, bool mirror, long cus)
 	p.splits = (int)bestSplits;
 	p.kChunk = (int)bestChunk;
 	p.wsBytes = (bestSplits > 1) ? (size_t)bestSplits * I * J * sizeof(float) : 0;
+	p.bk = kGemmBK;
+	p.estimateUs = best;
 	return p;
 }
 
@@ -819,6 +824,28 @@ static int launch_gemm(const PA &pa, const PB &pb, const OutParams &out, int I, 
 	return launch_tile<OpA, OpB, 64, 64>(pa, pb, out, I, J, R, plan, ws, kernelClass, flops);
 }
 
+// A product whose output is a handful of tiles and whose reduction is short spends its time waiting for one global
+// load per reduction slice: with slices of sixteen a 128 x 128 x 128 product lasts 8-12 us, split or not.  Such
+// products run unsplit on 64 x 64 tiles with slices of sixty-four (four times fewer dependent loads, sixteen elements
+// per thread and operand in flight).  `groups`: tiles of all problems of the launch.
+inline bool deep_slice_plan(long I, long J, long R, bool mirror, int batch, long cus, const GemmPlan &standard, GemmPlan *deep)
+{
+	if (I > 384 || J > 384 || R > 1024) return false;
+	long ti = (I + 63) / 64, tj = (J + 63) / 64;
+	long tiles = mirror ? ti * (ti + 1) / 2 : ti * tj;
+	long rounds = (tiles * batch + 3 * cus - 1) / (3 * cus);
+	long steps = (R + kGemmDeepBK - 1) / kGemmDeepBK;
+	double estimate = (double)rounds * (double)steps * 1.6 + 3.0;
+	if (estimate >= standard.estimateUs) return false;
+	deep->bm = deep->bn = 64;
+	deep->splits = 1;
+	deep->kChunk = (int)(steps * kGemmDeepBK);
+	deep->wsBytes = 0;
+	deep->bk = kGemmDeepBK;
+	deep->estimateUs = estimate;
+	return true;
+}
+
 // ---- batched products of plain operands ------------------------------------------------------------------------
 struct BatchStrides {
 	int batch;
@@ -826,14 +853,14 @@ struct BatchStrides {
 	long ws;      // floats between their split-K workspaces
 };
 
-template <template <int, int> class OpA, template <int, int> class OpB, int BM, int BN>
+template <template <int, int> class OpA, template <int, int> class OpB, int BM, int BN, int BK = kGemmBK>
 static int launch_tile_batched(const PlainParams &pa, const PlainParams &pb, const OutParams &out, int I, int J, int R,
                                const GemmPlan &plan, void *ws, int kernelClass, double flops, const BatchStrides &bs)
 {
-	typedef TileCfg<BM, BN, kGemmBK> Cfg;
+	typedef TileCfg<BM, BN, BK> Cfg;
 	constexpr int tileId = (BM == 64 ? (BN == 64 ? 1 : 2) : (BN == 64 ? 3 : 4));
-	typedef OpA<BM, kGemmBK> A;
-	typedef OpB<BN, kGemmBK> B;
+	typedef OpA<BM, BK> A;
+	typedef OpB<BN, BK> B;
 	dim3 grid((J + BN - 1) / BN, (I + BM - 1) / BM, plan.splits * bs.batch);
 	if (grid.y > 65535 || grid.z > 65535) return fail(FITRE_E_UNSUPPORTED, "gemm grid %u x %u x %u too large", grid.x, grid.y, grid.z);
 	if (plan.splits > 1) {
@@ -869,6 +896,7 @@ static int launch_gemm_batched(const PlainParams &pa, const PlainParams &pb, con
 		if (wsBytes < plan.wsBytes)
 			return fail(FITRE_E_WORKSPACE, "split-K workspace of %zu bytes is smaller than the %zu required", wsBytes, plan.wsBytes);
 	}
+	if (plan.bk == kGemmDeepBK) return launch_tile_batched<OpA, OpB, 64, 64, kGemmDeepBK>(pa, pb, out, I, J, R, plan, ws, kernelClass, flops, bs);
 	if (plan.bm == 128 && plan.bn == 128)
 		return launch_tile_batched<OpA, OpB, 128, 128>(pa, pb, out, I, J, R, plan, ws, kernelClass, flops, bs);
 	if (plan.bm == 64 && plan.bn == 128) return launch_tile_batched<OpA, OpB, 64, 128>(pa, pb, out, I, J, R, plan, ws, kernelClass, flops, bs);
