@@ -270,17 +270,6 @@ __global__ void __launch_bounds__(256) shifted_copy_kernel(const float *A, float
 	}
 }
 
-// dst (rows x cols, ld ldd) = src (ld lds)
-__global__ void __launch_bounds__(256) block_copy_kernel(const float *src, int lds_, float *dst, int ldd, int rows, int cols)
-{
-	const long total = (long)rows * cols;
-	const long stride = (long)gridDim.x * blockDim.x;
-	for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
-		const int c = (int)(idx / rows), r = (int)(idx - (long)c * rows);
-		dst[(size_t)c * ldd + r] = src[(size_t)c * lds_ + r];
-	}
-}
-
 __global__ void __launch_bounds__(256) fill_zero_kernel(float *p, long n, long batchStride)
 {
 	p += (size_t)blockIdx.y * batchStride;
