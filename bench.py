@@ -134,6 +134,7 @@ def gpu_leg(args):
     finite = bool(np.isfinite(grad).all() and np.isfinite(loss))
     kfac = kfac_leg(L, dev, gm, model, batch, max(2, args.steps // 4))
     kfac["hessian_vector_ms"] = hv_leg(L, dev, gm, model, batch, max(2, args.steps // 4))
+    kfac["trust_region_step_ms"] = kfac_step_leg(L, dev, gm, model, batch, 3)
     gm.release()
     bandwidth = bandwidth_leg(L, dev, batch)
     others = other_configs_leg(L, dev)
@@ -341,6 +342,44 @@ def hv_leg(L, dev, gm, model, batch, passes):
     for q in (v, hv, ws):
         dev.free(q)
     return round(ms, 4)
+
+
+def kfac_step_leg(L, dev, gm, model, batch, repeats):
+    """The pieces above as ONE timed sequence, the way a KFAC trust-region step strings them together: full
+    backward, both factor + damped-inverse passes, the natural gradient, one Hessian-vector product."""
+    from fitre_amd.structs import KFAC_CURVATURE_INFO
+
+    info = KFAC_CURVATURE_INFO()
+    L.cnn.computeKFACStorageIndices(C.byref(model), C.byref(info))
+    last = model.cLayers + model.lLayers
+    oinv, linv = dev.zeros(info.OmegaZOffsets[last]), dev.zeros(info.LambdaGOffsets[last])
+    ngrad, hv = dev.zeros(model.pSize), dev.zeros(model.pSize)
+    info.regLambda, info.dampGamma = 1e-3, 0.0
+    info.OmegaZInv, info.LambdaGInv = oinv.value, linv.value
+    info.gradient, info.nGradient = gm.grad.value, ngrad.value
+    need = max(L.cnn.kfacInverseMemRequired(C.byref(model), batch), L.cnn.kfacNaturalGradientMemRequired(C.byref(model)),
+               L.cnn.cnnHvMemRequired(C.byref(model)))
+    ws = dev.alloc(4 * need + 512)
+
+    def step():
+        gm.backward()
+        L.cnn.computeOmegaZ(C.byref(info), C.byref(model), C.byref(gm.data), batch, None, gm.z, oinv, model.zOffsets,
+                            model.zztOffsets, ws, None)
+        L.cnn.computeLambdaDelta(C.byref(info), C.byref(model), batch, gm.dx, None, linv, model.zOffsets, model.zztOffsets,
+                                 ws, None)
+        L.cnn.computeNaturalGradient(C.byref(model), C.byref(info), ws, None)
+        L.cnn.cnnHv(C.byref(model), C.byref(gm.data), gm.z, gm.probs, gm.errors, gm.dx, ngrad, hv, 0, batch, ws, None, 0.0)
+
+    step()
+    dev.sync()
+    t0 = time.perf_counter()
+    for _ in range(repeats):
+        step()
+    dev.sync()
+    ms = 1e3 * (time.perf_counter() - t0) / repeats
+    for q in (oinv, linv, ngrad, hv, ws):
+        dev.free(q)
+    return round(ms, 3)
 
 
 def cpu_leg(batch=64, repeats=10):
