@@ -346,7 +346,7 @@ def hv_leg(L, dev, gm, model, batch, passes):
 
 def kfac_step_leg(L, dev, gm, model, batch, repeats):
     """The pieces above as ONE timed sequence, the way a KFAC trust-region step strings them together: full
-    backward, both factor + damped-inverse passes, the natural gradient, one Hessian-vector product."""
+    backward, the factors and damped inverses of both sides (one pass), the natural gradient, one Hessian-vector product."""
     from fitre_amd.structs import KFAC_CURVATURE_INFO
 
     info = KFAC_CURVATURE_INFO()
@@ -363,10 +363,8 @@ def kfac_step_leg(L, dev, gm, model, batch, repeats):
 
     def step():
         gm.backward()
-        L.cnn.computeOmegaZ(C.byref(info), C.byref(model), C.byref(gm.data), batch, None, gm.z, oinv, model.zOffsets,
-                            model.zztOffsets, ws, None)
-        L.cnn.computeLambdaDelta(C.byref(info), C.byref(model), batch, gm.dx, None, linv, model.zOffsets, model.zztOffsets,
-                                 ws, None)
+        L.cnn.computeOmegaZAndLambdaDelta(C.byref(info), C.byref(model), C.byref(gm.data), batch, None, gm.z, gm.dx, None,
+                                          model.zOffsets, model.zztOffsets, ws)
         L.cnn.computeNaturalGradient(C.byref(model), C.byref(info), ws, None)
         L.cnn.cnnHv(C.byref(model), C.byref(gm.data), gm.z, gm.probs, gm.errors, gm.dx, ngrad, hv, 0, batch, ws, None, 0.0)
 

@@ -191,12 +191,23 @@ long kfacInverseMemRequired(CNN_MODEL *model, int samples)
 	return (long)((KFAC_SLOTS * inverse_scratch_bytes(model, samples, &factorBytes) + KFAC_INFO_BYTES) / sizeof(real)) + 64;
 }
 
-/* writes the factor of `layer` (pass numbering: convolution layers, then linear ones) into `factor` */
+/* writes the factor of `layer` (convolution layers, then linear ones) into `factor` */
 typedef void (*FACTOR_FN)(void *ctx, int layer, real *factor, real *ws, size_t wsBytes);
 
-typedef struct inverse_job {
-	int first, count; /* layers first .. first+count-1 */
+/* one matrix of a pass: how to make its factor, its order, where its inverse goes.  Consecutive items may share a
+ * batch when they have the same order and group and their inverses are `stride` reals apart. */
+typedef struct inverse_item {
+	FACTOR_FN make;
+	void *ctx;
+	int layer;
 	int order;
+	int group;
+	real *inverse;
+	long stride; /* room behind `inverse` up to the next layer's slot */
+} INVERSE_ITEM;
+
+typedef struct inverse_job {
+	int first, count; /* items first .. first+count-1 */
 	double cost;
 	int lane;
 } INVERSE_JOB;
@@ -208,10 +219,9 @@ static int job_by_cost(const void *a, const void *b)
 	return x->first - y->first;
 }
 
-/* order[l]: order of layer l's factor; offset[l]: where its inverse goes in inverseBase (offset[l+1] - offset[l] is
- * at least order[l]^2); group[l]: layers may share a batch only inside one group (convolution / linear) */
-static void inverse_pass_run(const CNN_MODEL *model, int samples, real *devPtr, int layers, const int *order, const int *offset,
-                             const int *group, real *inverseBase, real shift, FACTOR_FN make, void *ctx)
+#define KFAC_MAX_ITEMS (2 * MAX_LAYERS)
+
+static void inverse_pass_run(const CNN_MODEL *model, int samples, real *devPtr, const INVERSE_ITEM *items, int count, real shift)
 {
 	size_t factorBytes;
 	const size_t slotBytes = inverse_scratch_bytes(model, samples, &factorBytes);
@@ -220,23 +230,23 @@ static void inverse_pass_run(const CNN_MODEL *model, int samples, real *devPtr, 
 	int *pivots = (int *)base;
 	char *slots = base + KFAC_INFO_BYTES;
 
-	/* batches: runs of consecutive layers of one order, at most KFAC_MAX_BATCH long */
-	INVERSE_JOB jobs[MAX_LAYERS];
+	/* batches: runs of consecutive items of one order, at most KFAC_MAX_BATCH long */
+	INVERSE_JOB jobs[KFAC_MAX_ITEMS];
 	int nJobs = 0;
-	for (int l = 0; l < layers;) {
-		int count = 1;
-		/* small matrices gain nothing from a shared chain (measured: the output-side pass, orders up to 512, is
+	for (int i = 0; i < count;) {
+		int n = 1;
+		/* small matrices gain nothing from a shared chain (measured: the output-side factors, orders up to 512, are
 		 * faster with one lane per matrix) */
-		while (order[l] >= KFAC_MIN_BATCH_ORDER && l + count < layers && count < KFAC_MAX_BATCH && order[l + count] == order[l] && group[l + count] == group[l] &&
-		       offset[l + count + 1] - offset[l + count] == offset[l + 1] - offset[l])
-			count++;
+		while (items[i].order >= KFAC_MIN_BATCH_ORDER && i + n < count && n < KFAC_MAX_BATCH && items[i + n].order == items[i].order &&
+		       items[i + n].group == items[i].group && items[i + n].stride == items[i].stride &&
+		       items[i + n].inverse == items[i + n - 1].inverse + items[i].stride)
+			n++;
 		INVERSE_JOB *j = &jobs[nJobs++];
-		j->first = l;
-		j->count = count;
-		j->order = order[l];
+		j->first = i;
+		j->count = n;
 		/* measured: the time of an inverse grows a little slower than n^2, and a batch pays for the chain once */
-		j->cost = (double)order[l] * order[l] * (0.6 + 0.4 * count);
-		l += count;
+		j->cost = (double)items[i].order * items[i].order * (0.6 + 0.4 * n);
+		i += n;
 	}
 	qsort(jobs, (size_t)nJobs, sizeof(INVERSE_JOB), job_by_cost);
 	double load[KFAC_LANES] = { 0, 0, 0, 0 };
@@ -251,28 +261,29 @@ static void inverse_pass_run(const CNN_MODEL *model, int samples, real *devPtr, 
 	for (int k = 1; k < KFAC_LANES; k++) HIP_CALL(fitre_hip_lane_wait(k, 0)); /* after what lane 0 has queued so far (z, dx) */
 	for (int i = 0; i < nJobs; i++) {
 		const INVERSE_JOB *j = &jobs[i];
+		const INVERSE_ITEM *it = &items[j->first];
 		char *slot0 = slots + (size_t)kLaneFirstSlot[j->lane] * slotBytes;
 		HIP_CALL(fitre_hip_lane_select(j->lane));
 		for (int b = 0; b < j->count; b++) {
 			char *slot = slot0 + (size_t)b * slotBytes;
-			make(ctx, j->first + b, (real *)slot, (real *)(slot + factorBytes), wsBytes);
+			it[b].make(it[b].ctx, it[b].layer, (real *)slot, (real *)(slot + factorBytes), wsBytes);
 		}
-		const int l = j->first;
 		if (j->count == 1)
-			HIP_CALL(fitre_hip_spd_inverse_queued((real *)slot0, j->order, shift, inverseBase + offset[l], slot0 + factorBytes, wsBytes,
-			                                      pivots + l));
+			HIP_CALL(fitre_hip_spd_inverse_queued((real *)slot0, it->order, shift, it->inverse, slot0 + factorBytes, wsBytes,
+			                                      pivots + j->first));
 		else
-			HIP_CALL(fitre_hip_spd_inverse_batched_queued(j->count, (real *)slot0, (long)(slotBytes / sizeof(real)), j->order, shift,
-			                                              inverseBase + offset[l], (long)(offset[l + 1] - offset[l]),
-			                                              slot0 + factorBytes, wsBytes, (long)slotBytes, pivots + l));
+			HIP_CALL(fitre_hip_spd_inverse_batched_queued(j->count, (real *)slot0, (long)(slotBytes / sizeof(real)), it->order, shift,
+			                                              it->inverse, it->stride, slot0 + factorBytes, wsBytes, (long)slotBytes,
+			                                              pivots + j->first));
 	}
-	int host[MAX_LAYERS];
+	int host[KFAC_MAX_ITEMS];
 	HIP_CALL(fitre_hip_lane_select(0));
 	HIP_CALL(fitre_hip_sync());
-	HIP_CALL(fitre_hip_copy_d2h(host, pivots, sizeof(int) * (size_t)layers));
-	for (int l = 0; l < layers; l++)
-		if (host[l] != 0) {
-			fprintf(stderr, "We have a problem with the LU factorization ... %d (layer %d)\n", host[l], l);
+	HIP_CALL(fitre_hip_copy_d2h(host, pivots, sizeof(int) * (size_t)count));
+	for (int i = 0; i < count; i++)
+		if (host[i] != 0) {
+			fprintf(stderr, "We have a problem with the LU factorization ... %d (%s factor of layer %d)\n", host[i],
+			        items[i].group < 2 ? "input" : "output", items[i].layer);
 			exit(-1);
 		}
 }
@@ -314,26 +325,40 @@ static void omega_factor(void *ctx, int layer, real *factor, real *ws, size_t ws
 	}
 }
 
+/* items of the input-side factors; returns their number */
+static int omega_items(INVERSE_ITEM *items, const KFAC_CURVATURE_INFO *kfac_info, const CNN_MODEL *model, OMEGA_CTX *ctx,
+                       real *omegaZInv)
+{
+	const int nc = model->cLayers, layers = nc + model->lLayers;
+	const int *omega = kfac_info->OmegaZOffsets;
+	for (int l = 0; l < layers; l++) {
+		INVERSE_ITEM *it = &items[l];
+		it->make = omega_factor;
+		it->ctx = ctx;
+		it->layer = l;
+		if (l < nc) {
+			const CONV_LAYER *c = &model->convLayer[l];
+			it->order = c->inChannels * c->kSize * c->kSize + (ctx->withBias ? 1 : 0);
+			it->group = 0;
+		} else {
+			it->order = model->fcLayer[l - nc].in + (ctx->withBias ? 1 : 0);
+			it->group = 1;
+		}
+		it->inverse = omegaZInv + omega[l];
+		it->stride = (long)omega[l + 1] - omega[l];
+	}
+	return layers;
+}
+
 void computeOmegaZ(KFAC_CURVATURE_INFO *kfac_info, CNN_MODEL *model, DEVICE_DATASET *data, int samples,
                    real *dampedInput, real *dampedZ, real *omegaZInv, int *zOffsets, int *zztOffsets, real *devPtr,
                    real *pageLckPtr)
 {
 	(void)pageLckPtr;
-	const int withBias = model->bias != 0;
-	const int nc = model->cLayers, layers = nc + model->lLayers;
-	int order[MAX_LAYERS], group[MAX_LAYERS];
-	for (int l = 0; l < nc; l++) {
-		const CONV_LAYER *c = &model->convLayer[l];
-		order[l] = c->inChannels * c->kSize * c->kSize + (withBias ? 1 : 0);
-		group[l] = 0;
-	}
-	for (int l = 0; l < model->lLayers; l++) {
-		order[nc + l] = model->fcLayer[l].in + (withBias ? 1 : 0);
-		group[nc + l] = 1;
-	}
-	OMEGA_CTX ctx = { model, data, samples, withBias, dampedInput, dampedZ, zOffsets, zztOffsets };
-	inverse_pass_run(model, samples, devPtr, layers, order, kfac_info->OmegaZOffsets, group, omegaZInv,
-	                 kfac_info->regLambda + kfac_info->dampGamma, omega_factor, &ctx);
+	OMEGA_CTX ctx = { model, data, samples, model->bias != 0, dampedInput, dampedZ, zOffsets, zztOffsets };
+	INVERSE_ITEM items[KFAC_MAX_ITEMS];
+	const int count = omega_items(items, kfac_info, model, &ctx, omegaZInv);
+	inverse_pass_run(model, samples, devPtr, items, count, kfac_info->regLambda + kfac_info->dampGamma);
 }
 
 typedef struct lambda_ctx {
@@ -368,23 +393,44 @@ static void lambda_factor(void *ctx, int layer, real *factor, real *ws, size_t w
 	}
 }
 
+static int lambda_items(INVERSE_ITEM *items, const KFAC_CURVATURE_INFO *kfac_info, const CNN_MODEL *model, LAMBDA_CTX *ctx,
+                        real *lambdaGInv)
+{
+	const int nc = model->cLayers, layers = nc + model->lLayers;
+	const int *lambda = kfac_info->LambdaGOffsets;
+	for (int l = 0; l < layers; l++) {
+		INVERSE_ITEM *it = &items[l];
+		it->make = lambda_factor;
+		it->ctx = ctx;
+		it->layer = l;
+		it->order = l < nc ? model->convLayer[l].outChannels : model->fcLayer[l - nc].out;
+		it->group = l < nc ? 2 : 3;
+		it->inverse = lambdaGInv + lambda[l];
+		it->stride = (long)lambda[l + 1] - lambda[l];
+	}
+	return layers;
+}
+
 void computeLambdaDelta(KFAC_CURVATURE_INFO *kfac_info, CNN_MODEL *model, int samples, real *dx, real *dampedLambda,
                         real *lambdaGInv, int *zOffsets, int *zztOffsets, real *devPtr, real *pageLckPtr)
 {
 	(void)pageLckPtr;
-	const int nc = model->cLayers, layers = nc + model->lLayers;
-	int order[MAX_LAYERS], group[MAX_LAYERS];
-	for (int l = 0; l < nc; l++) {
-		order[l] = model->convLayer[l].outChannels;
-		group[l] = 0;
-	}
-	for (int l = 0; l < model->lLayers; l++) {
-		order[nc + l] = model->fcLayer[l].out;
-		group[nc + l] = 1;
-	}
 	LAMBDA_CTX ctx = { model, samples, dx, dampedLambda, zOffsets, zztOffsets };
-	inverse_pass_run(model, samples, devPtr, layers, order, kfac_info->LambdaGOffsets, group, lambdaGInv,
-	                 kfac_info->regLambda + kfac_info->dampGamma, lambda_factor, &ctx);
+	INVERSE_ITEM items[KFAC_MAX_ITEMS];
+	const int count = lambda_items(items, kfac_info, model, &ctx, lambdaGInv);
+	inverse_pass_run(model, samples, devPtr, items, count, kfac_info->regLambda + kfac_info->dampGamma);
+}
+
+void computeOmegaZAndLambdaDelta(KFAC_CURVATURE_INFO *kfac_info, CNN_MODEL *model, DEVICE_DATASET *data, int samples,
+                                 real *dampedInput, real *dampedZ, real *dx, real *dampedLambda, int *zOffsets, int *zztOffsets,
+                                 real *devPtr)
+{
+	OMEGA_CTX octx = { model, data, samples, model->bias != 0, dampedInput, dampedZ, zOffsets, zztOffsets };
+	LAMBDA_CTX lctx = { model, samples, dx, dampedLambda, zOffsets, zztOffsets };
+	INVERSE_ITEM items[KFAC_MAX_ITEMS];
+	int count = omega_items(items, kfac_info, model, &octx, kfac_info->OmegaZInv);
+	count += lambda_items(items + count, kfac_info, model, &lctx, kfac_info->LambdaGInv);
+	inverse_pass_run(model, samples, devPtr, items, count, kfac_info->regLambda + kfac_info->dampGamma);
 }
 
 /* ---- natural gradient ---------------------------------------------------------------------- */

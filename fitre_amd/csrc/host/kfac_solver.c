@@ -331,17 +331,13 @@ void subsampledTrustRegionKFAC(CNN_MODEL *model, DEVICE_DATASET *data, HOST_DATA
 				computeSpeedUpLambdaDelta(kfacInfo, model, (int)curBatchSize, distributionDX, dampedLambda, model->zOffsets,
 				                          model->zztOffsets, iter + (int)offset);
 			}
-			if (kfacInfo->inverseFreq == 1 || (iter == 0 && miniBatchNo == 0)) {
-				computeOmegaZ(kfacInfo, model, data, (int)curBatchSize, NULL, z, kfacInfo->OmegaZInv, model->zOffsets, model->zztOffsets,
-				              nextDevPtr, nextPageLckPtr);
-				computeLambdaDelta(kfacInfo, model, (int)curBatchSize, distributionDX, NULL, kfacInfo->LambdaGInv, model->zOffsets,
-				                   model->zztOffsets, nextDevPtr, nextPageLckPtr);
-			} else if (miniBatchNo % (unsigned int)kfacInfo->inverseFreq == 0) {
-				computeOmegaZ(kfacInfo, model, NULL, (int)curBatchSize, dampedInput, dampedZ, kfacInfo->OmegaZInv, model->zOffsets,
-				              model->zztOffsets, nextDevPtr, nextPageLckPtr);
-				computeLambdaDelta(kfacInfo, model, (int)curBatchSize, NULL, dampedLambda, kfacInfo->LambdaGInv, model->zOffsets,
-				                   model->zztOffsets, nextDevPtr, nextPageLckPtr);
-			}
+			/* the reference's computeOmegaZ followed by computeLambdaDelta, here as one pass over both sides */
+			if (kfacInfo->inverseFreq == 1 || (iter == 0 && miniBatchNo == 0))
+				computeOmegaZAndLambdaDelta(kfacInfo, model, data, (int)curBatchSize, NULL, z, distributionDX, NULL, model->zOffsets,
+				                            model->zztOffsets, nextDevPtr);
+			else if (miniBatchNo % (unsigned int)kfacInfo->inverseFreq == 0)
+				computeOmegaZAndLambdaDelta(kfacInfo, model, NULL, (int)curBatchSize, dampedInput, dampedZ, NULL, dampedLambda,
+				                            model->zOffsets, model->zztOffsets, nextDevPtr);
 			sumInverses += now_seconds() - t0;
 
 			t0 = now_seconds();

@@ -164,6 +164,7 @@ CNN_API = {
     "computeMatrixInverse": (None, [vp, vp, i32, vp, f32, f32]),
     "computeOmegaZ": (None, [pkfac, pmodel, pdata, i32, vp, vp, vp, pi32, pi32, vp, vp]),
     "computeLambdaDelta": (None, [pkfac, pmodel, i32, vp, vp, vp, pi32, pi32, vp, vp]),
+    "computeOmegaZAndLambdaDelta": (None, [pkfac, pmodel, pdata, i32, vp, vp, vp, vp, pi32, pi32, vp]),
     "kfacNaturalGradientMemRequired": (lng, [pmodel]),
     "computeNaturalGradient": (None, [pmodel, pkfac, vp, vp]),
     # include/fitre_solver.h

@@ -86,6 +86,13 @@ void computeOmegaZ(KFAC_CURVATURE_INFO *kfac_info, CNN_MODEL *model, DEVICE_DATA
 void computeLambdaDelta(KFAC_CURVATURE_INFO *kfac_info, CNN_MODEL *model, int samples, real *dx, real *dampedLambda,
                         real *lambdaGInv, int *zOffsets, int *zztOffsets, real *devPtr, real *pageLckPtr);
 
+/* Both passes as one (no counterpart in the reference, whose solver calls them one after the other): the small
+ * output-side inverses run on the lanes that the large input-side ones leave idle.  Same results, written to
+ * kfac_info->OmegaZInv and kfac_info->LambdaGInv; devPtr as for the single passes. */
+void computeOmegaZAndLambdaDelta(KFAC_CURVATURE_INFO *kfac_info, CNN_MODEL *model, DEVICE_DATASET *data, int samples,
+                                 real *dampedInput, real *dampedZ, real *dx, real *dampedLambda, int *zOffsets,
+                                 int *zztOffsets, real *devPtr);
+
 /* Scratch (in reals) of computeNaturalGradient. */
 long kfacNaturalGradientMemRequired(CNN_MODEL *model);
 /* solvers/kfac_natural_gradient.cu:36-241: per layer nGradient = Lambda^-1 * gradient * Omega^-1 with the

@@ -373,6 +373,41 @@ def test_model_inverses_and_natural_gradient(dev, oracle64, name):
     gm.release()
 
 
+@pytest.mark.parametrize("name", ["lenet_bias", "small_vgg_bn", "vgg11_b256"])
+def test_both_inverse_passes_as_one(dev, name):
+    """computeOmegaZAndLambdaDelta against computeOmegaZ followed by computeLambdaDelta on the same z / dx: the same
+    matrices, whatever lanes and batches they were dealt to."""
+    from fitre_amd.structs import KFAC_CURVATURE_INFO
+    from helpers import GpuModel, batch_inputs, he_weights
+    model, batch = next((m, b) for n, m, b in _model_cases() if n == name)
+    rng = np.random.default_rng(sum(map(ord, name)) + 5)
+    w = he_weights(model, rng).astype(np.float32)
+    x, y = batch_inputs(model, batch, rng)
+    gm = GpuModel(dev, model, w, x.astype(np.float32), y, batch)
+    gm.forward()
+    gm.backward()
+    info = KFAC_CURVATURE_INFO()
+    L.cnn.computeKFACStorageIndices(C.byref(model), C.byref(info))
+    info.regLambda, info.dampGamma = (1e-3, 0.0) if name == "vgg11_b256" else (0.05, 0.15)
+    last = model.cLayers + model.lLayers
+    tot_o, tot_l = info.OmegaZOffsets[last], info.LambdaGOffsets[last]
+    o1, l1, o2, l2 = dev.zeros(tot_o), dev.zeros(tot_l), dev.zeros(tot_o), dev.zeros(tot_l)
+    ws = dev.alloc(4 * L.cnn.kfacInverseMemRequired(C.byref(model), batch) + 512)
+    L.cnn.computeOmegaZ(C.byref(info), C.byref(model), C.byref(gm.data), batch, None, gm.z, o1, model.zOffsets, model.zztOffsets,
+                        ws, None)
+    L.cnn.computeLambdaDelta(C.byref(info), C.byref(model), batch, gm.dx, None, l1, model.zOffsets, model.zztOffsets, ws, None)
+    info.OmegaZInv, info.LambdaGInv = o2.value, l2.value
+    L.cnn.computeOmegaZAndLambdaDelta(C.byref(info), C.byref(model), C.byref(gm.data), batch, None, gm.z, gm.dx, None,
+                                      model.zOffsets, model.zztOffsets, ws)
+    a, b = dev.download(o1, tot_o), dev.download(o2, tot_o)
+    assert np.isfinite(a).all() and rel_err(b, a) < 1e-6
+    a, b = dev.download(l1, tot_l), dev.download(l2, tot_l)
+    assert np.isfinite(a).all() and rel_err(b, a) < 1e-6
+    for q in (o1, l1, o2, l2, ws):
+        dev.free(q)
+    gm.release()
+
+
 def test_vgg11_full_size_factor_inverses_with_the_benchmark_damping(dev):
     """The KFAC configuration of the benchmark at its real size: VGG-11, batch 256, damping lambda = 1e-3 and nothing
     else.  Input factors reach order 4609 with 1024 patches behind them (rank deficient: the damping alone keeps them

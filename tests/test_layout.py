@@ -107,6 +107,7 @@ def test_libraries_export_every_declared_symbol():
     assert "computeOmegaZFactors" in cnn_names and "computeKFACStorageIndices" in cnn_names
     assert "cnnHv" in cnn_names and "computeQuadraticModel" in cnn_names
     assert "augmentData" in cnn_names and "selectColumnMatrix" in cnn_names and "computeTestGeneralizationErrors" in cnn_names
+    assert "computeOmegaZAndLambdaDelta" in cnn_names
     assert "subsampledTrustRegionKFAC" in cnn_names and "genRandomVector" in cnn_names
     assert "computeGradient" in cnn_names and "nnForwardPass" in cnn_names and "computeNaturalGradient" in cnn_names
     for n in cnn_names:
