@@ -34,16 +34,16 @@ __device__ __forceinline__ float lane_value(float v, int lane)
 //     for kb:  (L[kb][kb], X[kb][kb]) of W[kb][kb];   L[ib][kb] = W[ib][kb] X[kb][kb]^T  (ib > kb);
 //              W[ib][jb] -= L[ib][kb] L[jb][kb]^T  (ib >= jb > kb)
 //     for ib:  X[ib][jb] = -X[ib][ib] * sum_{jb <= k < ib} L[ib][k] X[k][jb]  (jb < ib)
-// Both matrices are column-major in LDS with a leading dimension of 129 words, which makes the
+// The matrix is column-major in LDS with a leading dimension of 129 words, which makes the
 // stride-129 accesses of the transposed operands and of the accumulator layout conflict-free.
 constexpr int kSub = 32;                 // order of a sub-block
 constexpr int kLeafBlocks = 2;           // 64-wide block columns a leaf covers
 constexpr int kLeaf = kLeafBlocks * kNb; // largest leaf order
 constexpr int kLeafLd = kLeaf + 1;
 
-// One wave: factor sub-block kb of Ws in registers, write its factor back (lower triangle) and the inverse
-// of the factor into the same sub-block of Xs (zeros above the diagonal).  Returns the 1-based index inside the
-// leaf of the first non-positive pivot of this sub-block, or 0.
+// One wave: factor diagonal sub-block kb of Ms in registers and put the inverse of its factor in its place (zeros
+// above the diagonal).  Returns the 1-based index inside the leaf of the first non-positive pivot of this sub-block,
+// or 0.
 //
 // Lane i holds row i of the block (a[]) and column i of the inverse in the making (y[], which starts as the unit
 // vector e_i and is forward-substituted column by column).  Step j scales column j, and then every later column k
@@ -95,11 +95,10 @@ __device__ __forceinline__ void factor_steps(float (&a)[kSub], float (&y)[kSub],
 	}
 }
 
-__device__ __forceinline__ int factor_sub_block(float *Ws, float *Xs, int kb, int lane)
+__device__ __forceinline__ int factor_sub_block(float *Ms, int kb, int lane)
 {
 	const int i = lane & (kSub - 1);
-	float *wb = Ws + (kb * kSub) * kLeafLd + kb * kSub;
-	float *xb = Xs + (kb * kSub) * kLeafLd + kb * kSub;
+	float *wb = Ms + (kb * kSub) * kLeafLd + kb * kSub;
 	float a[kSub], y[kSub];
 #pragma unroll
 	for (int j = 0; j < kSub; j++) {
@@ -108,13 +107,11 @@ __device__ __forceinline__ int factor_sub_block(float *Ws, float *Xs, int kb, in
 	}
 	int bad = 0;
 	factor_steps<0>(a, y, kb * kSub, bad);
-	// y[r] is element (r, i) of the inverse: this lane holds column i
+	// y[r] is element (r, i) of the inverse: this lane holds column i.  The inverse replaces the block: nothing reads
+	// a diagonal sub-block of the factor itself again.
 	if (lane < kSub) {
 #pragma unroll
-		for (int j = 0; j < kSub; j++) {
-			wb[j * kLeafLd + i] = a[j];
-			xb[i * kLeafLd + j] = y[j];
-		}
+		for (int j = 0; j < kSub; j++) wb[i * kLeafLd + j] = y[j];
 	}
 	return bad;
 }
@@ -160,13 +157,15 @@ __global__ void __launch_bounds__(256) chol_leaf_kernel(const float *W, int ld, 
 	W += (size_t)blockIdx.x * wStride;
 	Xout += (size_t)blockIdx.x * xStride;
 	info += blockIdx.x;
+	// ONE matrix in LDS (66 KB), turned from W into L and then into X in place: with both kept side by side (132 KB) the
+	// workgroup only fits on a compute unit that runs next to nothing else, and beside another lane's chip-filling
+	// product every leaf of the chain waited for that product's tail.
 	__shared__ float Ws[kLeaf * kLeafLd];
-	__shared__ float Xs[kLeaf * kLeafLd];
 	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 	const int nb = (nn + kSub - 1) / kSub, order = nb * kSub;
 	const float *blk = W + (size_t)k0 * ld + k0;
 	// Thread (r, h) moves row r, columns of parity h: the sub-blocks on and below the diagonal only (the rest of Ws is
-	// scratch, and Xs is written before it is read), a sub-block column of sixteen loads in flight at a time.
+	// scratch), a sub-block column of sixteen loads in flight at a time.
 	const int row = tid & (kLeaf - 1), half = tid >> 7, rowBlock = row >> 5;
 	if (row < order) {
 #pragma unroll
@@ -187,7 +186,7 @@ __global__ void __launch_bounds__(256) chol_leaf_kernel(const float *W, int ld, 
 
 	for (int kb = 0; kb < nb; kb++) {
 		if (wave == 0) {
-			const int bad = factor_sub_block(Ws, Xs, kb, lane);
+			const int bad = factor_sub_block(Ws, kb, lane);
 			if (bad != 0 && lane == 0) atomicCAS(info, 0, k0 + bad);
 		}
 		__syncthreads();
@@ -197,7 +196,7 @@ __global__ void __launch_bounds__(256) chol_leaf_kernel(const float *W, int ld, 
 			v16f acc = {};
 			if (ib < nb) {
 				// A = W[ib][kb]; B[k][c] = X[kb][kb][c][k]
-				sub_block_product(sub_block(Ws, ib, kb), 1, kLeafLd, sub_block(Xs, kb, kb), kLeafLd, 1, lane, acc);
+				sub_block_product(sub_block(Ws, ib, kb), 1, kLeafLd, sub_block(Ws, kb, kb), kLeafLd, 1, lane, acc);
 				store_sub_block(sub_block(Ws, ib, kb), lane, acc, 1.f);
 			}
 		}
@@ -223,22 +222,23 @@ __global__ void __launch_bounds__(256) chol_leaf_kernel(const float *W, int ld, 
 		__syncthreads();
 	}
 
-	// the inverse of the factor below its diagonal sub-blocks, one row of sub-blocks after the other; the sums go
-	// through the unused upper triangle of Ws on their way from accumulator to operand layout
+	// The inverse of the factor below its diagonal sub-blocks, one row of sub-blocks after the other, each row of X
+	// taking the place of that row of L once every wave has read it; the sums go through the unused upper triangle of
+	// Ws on their way from accumulator to operand layout.
 	for (int ib = 1; ib < nb; ib++) {
 		const int jb = wave;
 		if (jb < ib) {
 			v16f acc = {};
 			for (int k = jb; k < ib; k++) // A = L[ib][k]; B = X[k][jb]
-				sub_block_product(sub_block(Ws, ib, k), 1, kLeafLd, sub_block(Xs, k, jb), 1, kLeafLd, lane, acc);
+				sub_block_product(sub_block(Ws, ib, k), 1, kLeafLd, sub_block(Ws, k, jb), 1, kLeafLd, lane, acc);
 			store_sub_block(sub_block(Ws, jb, ib), lane, acc, 1.f);
 		}
 		__syncthreads();
 		if (jb < ib) {
 			v16f acc = {};
 			// A = X[ib][ib]; B = the sum above
-			sub_block_product(sub_block(Xs, ib, ib), 1, kLeafLd, sub_block(Ws, jb, ib), 1, kLeafLd, lane, acc);
-			store_sub_block(sub_block(Xs, ib, jb), lane, acc, -1.f);
+			sub_block_product(sub_block(Ws, ib, ib), 1, kLeafLd, sub_block(Ws, jb, ib), 1, kLeafLd, lane, acc);
+			store_sub_block(sub_block(Ws, ib, jb), lane, acc, -1.f);
 		}
 		__syncthreads();
 	}
@@ -251,7 +251,7 @@ __global__ void __launch_bounds__(256) chol_leaf_kernel(const float *W, int ld, 
 #pragma unroll
 			for (int q = 0; q < kSub / 2; q++) {
 				const int c = b * kSub + half + 2 * q;
-				if (c <= row) xblk[(size_t)c * ld + row] = Xs[c * kLeafLd + row];
+				if (c <= row) xblk[(size_t)c * ld + row] = Ws[c * kLeafLd + row];
 			}
 		}
 	}
