@@ -36,9 +36,13 @@ constexpr int kC3Tile = 128; // positions (and output channels) per workgroup ti
 struct Conv3x3Params {
 	const float *src;   // [Cred][N][A][B]
 	const float *w;     // [Cout][Cin][3][3]
+	// A sum of two products of one shape in one launch (the R operator's conv(z, V) + conv(R{z}, W) and its like): the
+	// reduction runs over the first pair (src, w) and then over the second; for the weight gradient `w2` is the second
+	// delta.  Null for a single product.
+	const float *src2, *w2;
 	uint32_t srcBytes, wBytes;
 	int I;              // output channels of this product
-	int cred;           // reduction channels
+	int cred;           // reduction channels of ONE pair
 	int J;              // positions N*A*B
 	int A, B;
 	int perSplit;       // channel blocks (position-contiguous) or position stages (weight gradient) per split
@@ -123,7 +127,8 @@ conv3x3_pos_kernel(const Conv3x3Params p, const OutParams out)
 	const int halo = p.B + 1;
 	const int win = kC3Tile + 2 * halo;
 	const int plane = p.J; // floats per channel of src
-	const int cbTotal = p.cred / CB;
+	const int cbHalf = p.cred / CB;                      // channel blocks of one (src, w) pair
+	const int cbTotal = p.src2 ? 2 * cbHalf : cbHalf;
 	const int cbBeg = blockIdx.z * p.perSplit;
 	const int cbEnd = (cbBeg + p.perSplit < cbTotal) ? cbBeg + p.perSplit : cbTotal;
 	const int rowLen = DX ? p.I * 9 : p.cred * 9;
@@ -197,17 +202,19 @@ conv3x3_pos_kernel(const Conv3x3Params p, const OutParams out)
 // global -> registers for channel block CBI (a macro: the register arrays must stay registers)
 #define C3_LOAD_BLOCK(CBI)                                                                                            \
 	{                                                                                                                 \
-		const int c0_ = (CBI) * CB;                                                                                   \
+		const bool second_ = (CBI) >= cbHalf; /* uniform: the block belongs to the second pair */                    \
+		const int c0_ = ((CBI) - (second_ ? cbHalf : 0)) * CB;                                                        \
+		const float *wSel = second_ ? p.w2 : p.w, *sSel = second_ ? p.src2 : p.src;                                   \
 		const size_t wShift = DX ? (size_t)c0_ * rowLen : (size_t)c0_ * 9; /* floats, uniform */                      \
 		if constexpr (VECW) {                                                                                         \
-			const char *wBlk = reinterpret_cast<const char *>(p.w + wShift);                                          \
+			const char *wBlk = reinterpret_cast<const char *>(wSel + wShift);                                         \
 			_Pragma("unroll") for (int e = 0; e < K::WE; e++)                                                         \
 			{                                                                                                         \
 				const float4 v4 = *reinterpret_cast<const float4 *>(wBlk + wOff[e]);                                  \
 				wreg[4 * e + 0] = v4.x, wreg[4 * e + 1] = v4.y, wreg[4 * e + 2] = v4.z, wreg[4 * e + 3] = v4.w;       \
 			}                                                                                                         \
 		} else {                                                                                                      \
-			const __amdgpu_buffer_rsrc_t wRs = make_rsrc(p.w + wShift, p.wBytes - (uint32_t)(4 * wShift));            \
+			const __amdgpu_buffer_rsrc_t wRs = make_rsrc(wSel + wShift, p.wBytes - (uint32_t)(4 * wShift));           \
 			_Pragma("unroll") for (int e = 0; e < K::WE; e++)                                                         \
 			{                                                                                                         \
 				wreg[4 * e + 0] = buffer_load(wRs, wOff[e]);                                                          \
@@ -217,7 +224,7 @@ conv3x3_pos_kernel(const Conv3x3Params p, const OutParams out)
 			}                                                                                                         \
 		}                                                                                                             \
 		const size_t sShift = (size_t)c0_ * plane;                                                                    \
-		const __amdgpu_buffer_rsrc_t sRs = make_rsrc(p.src + sShift, p.srcBytes - (uint32_t)(4 * sShift));            \
+		const __amdgpu_buffer_rsrc_t sRs = make_rsrc(sSel + sShift, p.srcBytes - (uint32_t)(4 * sShift));            \
 		_Pragma("unroll") for (int e = 0; e < K::SE; e++) sreg[e] = buffer_load(sRs, sOff[e]);                        \
 	}
 
@@ -366,7 +373,8 @@ conv3x3_dw_kernel(const Conv3x3Params p, const float *delta, uint32_t deltaBytes
 	const int halo = p.B + 1;
 	const int win = kC3Stage + 2 * halo;
 	const int plane = p.J;
-	const int stagesTotal = p.J / kC3Stage;
+	const int stagesHalf = p.J / kC3Stage;                       // stages of one (src, delta) pair
+	const int stagesTotal = p.src2 ? 2 * stagesHalf : stagesHalf; // a second pair continues the reduction
 	const int stBeg = bz * p.perSplit;
 	const int stEnd = (stBeg + p.perSplit < stagesTotal) ? stBeg + p.perSplit : stagesTotal;
 	const bool movingRows = (kC3Stage % p.B) != 0; // else every stage window starts in the same column
@@ -400,16 +408,19 @@ conv3x3_dw_kernel(const Conv3x3Params p, const float *delta, uint32_t deltaBytes
 // global -> registers for stage ST, and where its cells go in LDS
 #define C3_LOAD_STAGE(ST)                                                                                             \
 	{                                                                                                                 \
-		const int m0_ = (ST) * kC3Stage;                                                                              \
+		const bool second_ = (ST) >= stagesHalf; /* uniform: the stage belongs to the second pair */                 \
+		const int m0_ = ((ST) - (second_ ? stagesHalf : 0)) * kC3Stage;                                               \
+		const float *dSel = second_ ? p.w2 : delta;                                                                   \
+		const __amdgpu_buffer_rsrc_t xRs = second_ ? srcRs2 : srcRs;                                                  \
 		if constexpr (VECD) {                                                                                         \
-			const char *dBlk = reinterpret_cast<const char *>(delta + m0_);                                           \
+			const char *dBlk = reinterpret_cast<const char *>(dSel + m0_);                                            \
 			_Pragma("unroll") for (int e = 0; e < DE; e++)                                                            \
 			{                                                                                                         \
 				const float4 v4 = *reinterpret_cast<const float4 *>(dBlk + dOff[e]);                                  \
 				dreg[4 * e + 0] = v4.x, dreg[4 * e + 1] = v4.y, dreg[4 * e + 2] = v4.z, dreg[4 * e + 3] = v4.w;       \
 			}                                                                                                         \
 		} else {                                                                                                      \
-			const __amdgpu_buffer_rsrc_t dRs = make_rsrc(delta + m0_, deltaBytes - 4u * (uint32_t)m0_);               \
+			const __amdgpu_buffer_rsrc_t dRs = make_rsrc(dSel + m0_, deltaBytes - 4u * (uint32_t)m0_);                \
 			_Pragma("unroll") for (int e = 0; e < DE; e++)                                                            \
 			{                                                                                                         \
 				dreg[4 * e + 0] = buffer_load(dRs, dOff[e]);                                                          \
@@ -427,7 +438,7 @@ conv3x3_dw_kernel(const Conv3x3Params p, const float *delta, uint32_t deltaBytes
 			{                                                                                                         \
 				const int c = xcg + XCP * e;                                                                          \
 				const bool ok = okm & (c < kC3DwCin) & ((c0 + c) < p.cred);                                           \
-				xreg[e] = buffer_load(srcRs, ok ? 4u * (uint32_t)((c0 + c) * plane + m) : kOutOfRange);               \
+				xreg[e] = buffer_load(xRs, ok ? 4u * (uint32_t)((c0 + c) * plane + m) : kOutOfRange);                 \
 			}                                                                                                         \
 			if (movingRows | ((ST) == stBeg)) {                                                                       \
 				uint32_t q_, b_;                                                                                      \
@@ -475,6 +486,7 @@ conv3x3_dw_kernel(const Conv3x3Params p, const float *delta, uint32_t deltaBytes
 	}
 
 	const __amdgpu_buffer_rsrc_t srcRs = make_rsrc(p.src, p.srcBytes);
+	const __amdgpu_buffer_rsrc_t srcRs2 = make_rsrc(p.src2 ? p.src2 : p.src, p.srcBytes);
 
 	v16f acc[3];
 #pragma unroll

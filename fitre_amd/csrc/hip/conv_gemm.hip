@@ -121,7 +121,8 @@ static bool c3_dw_eligible(const fitre_conv_shape *s)
 }
 
 // cus: compute units of the lane the kernel is launched on (0 = the selected lane)
-static BlockPlan c3_pos_plan(const fitre_conv_shape *s, bool dx, int cus = 0)
+// pairs = 2: a sum of two products of this shape in one launch (twice the reduction)
+static BlockPlan c3_pos_plan(const fitre_conv_shape *s, bool dx, int cus = 0, int pairs = 1)
 {
 	if (cus <= 0) cus = lane_compute_units();
 	long I = dx ? s->inChannels : s->outChannels, J = (long)s->samples * s->inA * s->inB;
@@ -129,24 +130,24 @@ static BlockPlan c3_pos_plan(const fitre_conv_shape *s, bool dx, int cus = 0)
 	long it = I <= 64 ? 64 : kC3Tile;
 	long tiles = ((I + it - 1) / it) * ((J + kC3Tile - 1) / kC3Tile);
 	double blockUs = (9.0 * kC3CB / 2.0) * (it / 32.0) * 64.0 / 2400.0; // MFMA steps x blocks per wave x 64 cycles
-	return plan_blocks(tiles, cred / kC3CB, blockUs, it == 64 ? 3 : 2, I, J, cus);
+	return plan_blocks(tiles, pairs * cred / kC3CB, blockUs, it == 64 ? 3 : 2, I, J, cus);
 }
-static BlockPlan c3_dw_plan(const fitre_conv_shape *s, int cus = 0)
+static BlockPlan c3_dw_plan(const fitre_conv_shape *s, int cus = 0, int pairs = 1)
 {
 	if (cus <= 0) cus = lane_compute_units();
 	long J = (long)s->samples * s->inA * s->inB;
 	long tiles = ((s->inChannels + kC3DwCin - 1) / kC3DwCin) * ((s->outChannels + kC3Tile - 1) / kC3Tile);
 	double stageUs = (kC3Stage / 2.0) * 9.0 * 64.0 / 2400.0; // three waves per SIMD, three MFMAs per step each
-	return plan_blocks(tiles, (J + kC3Stage - 1) / kC3Stage, stageUs, 1, s->outChannels, (long)s->inChannels * 9, cus);
+	return plan_blocks(tiles, pairs * ((J + kC3Stage - 1) / kC3Stage), stageUs, 1, s->outChannels, (long)s->inChannels * 9, cus);
 }
-static size_t c3_pos_workspace(const fitre_conv_shape *s, bool dx)
+static size_t c3_pos_workspace(const fitre_conv_shape *s, bool dx, int pairs = 1)
 {
-	size_t a = c3_pos_plan(s, dx, device_compute_units()).wsBytes, b = c3_pos_plan(s, dx, lane_compute_units_min()).wsBytes;
+	size_t a = c3_pos_plan(s, dx, device_compute_units(), pairs).wsBytes, b = c3_pos_plan(s, dx, lane_compute_units_min(), pairs).wsBytes;
 	return a > b ? a : b;
 }
-static size_t c3_dw_workspace(const fitre_conv_shape *s)
+static size_t c3_dw_workspace(const fitre_conv_shape *s, int pairs = 1)
 {
-	size_t a = c3_dw_plan(s, device_compute_units()).wsBytes, b = c3_dw_plan(s, lane_compute_units_min()).wsBytes;
+	size_t a = c3_dw_plan(s, device_compute_units(), pairs).wsBytes, b = c3_dw_plan(s, lane_compute_units_min(), pairs).wsBytes;
 	return a > b ? a : b;
 }
 
@@ -154,15 +155,18 @@ static size_t c3_dw_workspace(const fitre_conv_shape *s)
 // results in ws and report their number there (the caller's consumer sums them)
 template <bool DX>
 static int launch_c3_pos(const fitre_conv_shape *s, const float *src, const float *w, const float *bias, float *outPtr, void *ws,
-                         size_t wsBytes, int *leftSplits = nullptr)
+                         size_t wsBytes, int *leftSplits = nullptr, const float *src2 = nullptr, const float *w2 = nullptr)
 {
 	const int I = DX ? s->inChannels : s->outChannels, cred = DX ? s->outChannels : s->inChannels;
 	const int J = s->samples * s->inA * s->inB;
-	BlockPlan plan = fit_blocks(c3_pos_plan(s, DX), cred / kC3CB, I, J, ws, wsBytes);
+	const int pairs = src2 ? 2 : 1;
+	BlockPlan plan = fit_blocks(c3_pos_plan(s, DX, 0, pairs), pairs * cred / kC3CB, I, J, ws, wsBytes);
 	if (plan.wsBytes > 0 && (((uintptr_t)ws) & 3)) return fail(FITRE_E_WORKSPACE, "split workspace is misaligned");
 	Conv3x3Params p;
 	p.src = src;
 	p.w = w;
+	p.src2 = src2;
+	p.w2 = w2;
 	p.srcBytes = (uint32_t)((size_t)cred * J * sizeof(float));
 	p.wBytes = (uint32_t)((size_t)s->outChannels * s->inChannels * 9 * sizeof(float));
 	p.I = I;
@@ -179,12 +183,12 @@ static int launch_c3_pos(const fitre_conv_shape *s, const float *src, const floa
 		part.C = (float *)ws;
 		part.splitStride = (long)I * J;
 	}
-	const bool vecw = ((((uintptr_t)w) & 15) == 0) && (DX ? (I % 4 == 0) : true);
+	const bool vecw = ((((uintptr_t)w) & 15) == 0) && (!w2 || (((uintptr_t)w2) & 15) == 0) && (DX ? (I % 4 == 0) : true);
 	const int it = I <= 64 ? 64 : kC3Tile;
 	dim3 grid((J + kC3Tile - 1) / kC3Tile, (I + it - 1) / it, plan.splits);
 	if (grid.y > 65535 || grid.z > 65535) return fail(FITRE_E_UNSUPPORTED, "conv3x3 grid too large");
 	{
-		LaunchScope scope(DX ? FITRE_KC_CONV_DX : FITRE_KC_CONV_FWD, conv_flops(s), it == 64 ? 2 : 4);
+		LaunchScope scope(DX ? FITRE_KC_CONV_DX : FITRE_KC_CONV_FWD, pairs * conv_flops(s), it == 64 ? 2 : 4);
 		const bool narrow = s->inB <= 32;
 #define C3_LAUNCH(V, MB, IT_) conv3x3_pos_kernel<kC3CB, DX, V, MB, IT_><<<grid, kGemmThreads, 0, stream()>>>(p, part)
 		if (it == 64) {
@@ -205,14 +209,19 @@ static int launch_c3_pos(const fitre_conv_shape *s, const float *src, const floa
 	return check_launch("conv3x3_pos_kernel");
 }
 
-static int launch_c3_dw(const fitre_conv_shape *s, const float *x, const float *delta, float *dW, void *ws, size_t wsBytes)
+// x2 / delta2 (may be null): a second (input, delta) pair whose product is added to the first one's
+static int launch_c3_dw(const fitre_conv_shape *s, const float *x, const float *delta, float *dW, void *ws, size_t wsBytes,
+                        const float *x2 = nullptr, const float *delta2 = nullptr)
 {
 	const int I = s->outChannels, cin = s->inChannels, K = cin * 9;
 	const int J = s->samples * s->inA * s->inB;
-	const int stages = (J + kC3Stage - 1) / kC3Stage;
-	BlockPlan plan = fit_blocks(c3_dw_plan(s), stages, I, K, ws, wsBytes);
+	const int pairs = x2 ? 2 : 1;
+	const int stages = pairs * ((J + kC3Stage - 1) / kC3Stage);
+	BlockPlan plan = fit_blocks(c3_dw_plan(s, 0, pairs), stages, I, K, ws, wsBytes);
 	if (plan.wsBytes > 0 && (((uintptr_t)ws) & 3)) return fail(FITRE_E_WORKSPACE, "split workspace is misaligned");
 	Conv3x3Params p;
+	p.src2 = x2;
+	p.w2 = delta2;
 	p.src = x;
 	p.w = nullptr;
 	p.srcBytes = (uint32_t)((size_t)cin * J * sizeof(float));
@@ -232,11 +241,11 @@ static int launch_c3_dw(const fitre_conv_shape *s, const float *x, const float *
 		part.splitStride = (long)I * K;
 	}
 	const uint32_t deltaBytes = (uint32_t)((size_t)I * J * sizeof(float));
-	const bool vecd = ((((uintptr_t)delta) & 15) == 0) && (J % 4 == 0);
+	const bool vecd = ((((uintptr_t)delta) & 15) == 0) && (!delta2 || (((uintptr_t)delta2) & 15) == 0) && (J % 4 == 0);
 	dim3 grid((cin + kC3DwCin - 1) / kC3DwCin, (I + kC3Tile - 1) / kC3Tile, plan.splits);
 	if (grid.y > 65535 || grid.z > 65535) return fail(FITRE_E_UNSUPPORTED, "conv3x3 grid too large");
 	{
-		LaunchScope scope(FITRE_KC_CONV_DW, conv_flops(s), 4);
+		LaunchScope scope(FITRE_KC_CONV_DW, pairs * conv_flops(s), 4);
 		const bool narrow = s->inB >= 2 && s->inB <= 16;
 		if (vecd && narrow)
 			conv3x3_dw_kernel<true, 16><<<grid, kC3DwThreads, 0, stream()>>>(p, delta, deltaBytes, part);
@@ -484,6 +493,57 @@ int fitre_hip_conv_input_grad(const fitre_conv_shape *s, const float *delta, con
 	rc = attach_patch_table(pb, plan.bn);
 	if (rc) return rc;
 	return launch_gemm<FlipWeightKContig, PatchRowContig>(pa, pb, out, I, J, R, plan, ws, wsBytes, FITRE_KC_CONV_DX, conv_flops(s));
+}
+
+// ---- sums of two products of one shape (the R operator's pairs) ---------------------------------------------------
+int fitre_hip_conv_pair_supported(const fitre_conv_shape *s, int kind)
+{
+	if (!s) return 0;
+	if (kind == 0) return c3_pos_eligible(s, false) ? 1 : 0;
+	if (kind == 1) return (s->stride == 1 && c3_pos_eligible(s, true)) ? 1 : 0;
+	if (kind == 2) return c3_dw_eligible(s) ? 1 : 0;
+	return 0;
+}
+
+size_t fitre_hip_conv_pair_workspace(const fitre_conv_shape *s, int kind)
+{
+	if (!fitre_hip_conv_pair_supported(s, kind)) return 0;
+	if (kind == 2) return c3_dw_workspace(s, 2);
+	return c3_pos_workspace(s, kind == 1, 2);
+}
+
+int fitre_hip_conv_forward_pair(const fitre_conv_shape *s, const float *x1, const float *w1, const float *x2, const float *w2,
+                                const float *bias, float *y, void *ws, size_t wsBytes)
+{
+	FITRE_NEED_INIT();
+	int rc = check_conv("fitre_hip_conv_forward_pair", s);
+	if (rc) return rc;
+	FITRE_REQUIRE(x1 && w1 && x2 && w2 && y, "fitre_hip_conv_forward_pair: null pointer");
+	if (!c3_pos_eligible(s, false)) return fail(FITRE_E_UNSUPPORTED, "fitre_hip_conv_forward_pair: only 3x3 windows with stride 1 and padding 1");
+	return launch_c3_pos<false>(s, x1, w1, bias, y, ws, wsBytes, nullptr, x2, w2);
+}
+
+int fitre_hip_conv_input_grad_pair(const fitre_conv_shape *s, const float *delta1, const float *w1, const float *delta2,
+                                   const float *w2, float *dx, void *ws, size_t wsBytes)
+{
+	FITRE_NEED_INIT();
+	int rc = check_conv("fitre_hip_conv_input_grad_pair", s);
+	if (rc) return rc;
+	FITRE_REQUIRE(delta1 && w1 && delta2 && w2 && dx, "fitre_hip_conv_input_grad_pair: null pointer");
+	if (s->stride != 1 || !c3_pos_eligible(s, true))
+		return fail(FITRE_E_UNSUPPORTED, "fitre_hip_conv_input_grad_pair: only 3x3 windows with stride 1 and padding 1");
+	return launch_c3_pos<true>(s, delta1, w1, nullptr, dx, ws, wsBytes, nullptr, delta2, w2);
+}
+
+int fitre_hip_conv_weight_grad_pair(const fitre_conv_shape *s, const float *x1, const float *delta1, const float *x2,
+                                    const float *delta2, float *dW, void *ws, size_t wsBytes)
+{
+	FITRE_NEED_INIT();
+	int rc = check_conv("fitre_hip_conv_weight_grad_pair", s);
+	if (rc) return rc;
+	FITRE_REQUIRE(x1 && delta1 && x2 && delta2 && dW, "fitre_hip_conv_weight_grad_pair: null pointer");
+	if (!c3_dw_eligible(s)) return fail(FITRE_E_UNSUPPORTED, "fitre_hip_conv_weight_grad_pair: shape outside the 3x3 weight-gradient kernel");
+	return launch_c3_dw(s, x1, delta1, dW, ws, wsBytes, x2, delta2);
 }
 
 int fitre_hip_conv_input_grad_split(const fitre_conv_shape *s, const float *delta, const float *w, float *dx, void *ws,

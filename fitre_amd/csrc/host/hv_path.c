@@ -75,6 +75,7 @@ static size_t hv_ws_bytes(const CNN_MODEL *model, int batch)
 		need = max_sz(need, fitre_hip_conv_forward_workspace(&s));
 		need = max_sz(need, fitre_hip_conv_weight_grad_workspace(&s));
 		if (i != 0) need = max_sz(need, fitre_hip_conv_input_grad_workspace(&s));
+		for (int kind = 0; kind < 3; kind++) need = max_sz(need, fitre_hip_conv_pair_workspace(&s, kind));
 		need = max_sz(need, fitre_hip_batch_norm_workspace(c->outChannels, (long)batch * c->outWidth * c->outHeight));
 	}
 	if (model->cLayers > 0) {
@@ -126,12 +127,19 @@ static void rop_forward(CNN_MODEL *model, const real *weights, const real *vecto
 		const long perChannel = (long)n * c->outWidth * c->outHeight, count = perChannel * c->outChannels;
 		const real *in = (l == 0) ? x : z + zOffsets[l] + model->convLayer[l - 1].outputOffset;
 		fitre_conv_shape shape = conv_shape(c, n);
-		/* R{conv} = conv(z_in, V) + Vb + conv(R{z_in}, W) */
-		HIP_CALL(fitre_hip_conv_forward(&shape, in, vector + wOffsets[l], bias ? vector + bOffsets[l] : NULL, rslab, ws, wsBytes));
-		if (l > 0) {
+		/* R{conv} = conv(z_in, V) + Vb + conv(R{z_in}, W): one launch whose reduction runs over both products where the
+		 * shape allows, else two products and an addition */
+		const real *vb = bias ? vector + bOffsets[l] : NULL;
+		if (l > 0 && fitre_hip_conv_pair_supported(&shape, 0)) {
 			const real *rin = rz + zOffsets[l] + model->convLayer[l - 1].outputOffset;
-			HIP_CALL(fitre_hip_conv_forward(&shape, rin, weights + wOffsets[l], NULL, tmp, ws, wsBytes));
-			HIP_CALL(fitre_hip_axpy((int)count, 1.f, tmp, rslab));
+			HIP_CALL(fitre_hip_conv_forward_pair(&shape, in, vector + wOffsets[l], rin, weights + wOffsets[l], vb, rslab, ws, wsBytes));
+		} else {
+			HIP_CALL(fitre_hip_conv_forward(&shape, in, vector + wOffsets[l], vb, rslab, ws, wsBytes));
+			if (l > 0) {
+				const real *rin = rz + zOffsets[l] + model->convLayer[l - 1].outputOffset;
+				HIP_CALL(fitre_hip_conv_forward(&shape, rin, weights + wOffsets[l], NULL, tmp, ws, wsBytes));
+				HIP_CALL(fitre_hip_axpy((int)count, 1.f, tmp, rslab));
+			}
 		}
 		const real *rpre = rslab, *actIn = slab;
 		if (has_bn(c)) {
@@ -251,18 +259,28 @@ static void rop_backward(CNN_MODEL *model, const real *weights, const real *vect
 		const real *in = (c == 0) ? x : z + zOffsets[c] + model->convLayer[c - 1].outputOffset;
 		const long wcount = (long)l->outChannels * l->inChannels * l->kSize * l->kSize;
 		fitre_conv_shape shape = conv_shape(l, n);
-		/* R{dW} = dW(z_in, R{dc}) + dW(R{z_in}, dc) */
-		HIP_CALL(fitre_hip_conv_weight_grad(&shape, in, rdc, hv + wOffsets[c], ws, wsBytes));
-		if (c != 0) {
+		/* R{dW} = dW(z_in, R{dc}) + dW(R{z_in}, dc); the input of the first layer carries no R term */
+		if (c == 0) {
+			HIP_CALL(fitre_hip_conv_weight_grad(&shape, in, rdc, hv + wOffsets[c], ws, wsBytes));
+		} else {
 			const real *rin = rz + zOffsets[c] + model->convLayer[c - 1].outputOffset;
-			HIP_CALL(fitre_hip_conv_weight_grad(&shape, rin, dc, wtmp, ws, wsBytes));
-			HIP_CALL(fitre_hip_axpy((int)wcount, 1.f, wtmp, hv + wOffsets[c]));
+			if (fitre_hip_conv_pair_supported(&shape, 2)) {
+				HIP_CALL(fitre_hip_conv_weight_grad_pair(&shape, in, rdc, rin, dc, hv + wOffsets[c], ws, wsBytes));
+			} else {
+				HIP_CALL(fitre_hip_conv_weight_grad(&shape, in, rdc, hv + wOffsets[c], ws, wsBytes));
+				HIP_CALL(fitre_hip_conv_weight_grad(&shape, rin, dc, wtmp, ws, wsBytes));
+				HIP_CALL(fitre_hip_axpy((int)wcount, 1.f, wtmp, hv + wOffsets[c]));
+			}
 			/* R{dX} = dX(R{dc}, W) + dX(dc, V) */
 			real *other = (rdc == rdelta) ? rnext : rdelta;
 			const long inCount = (long)n * l->height * l->width * l->inChannels;
-			HIP_CALL(fitre_hip_conv_input_grad(&shape, rdc, weights + wOffsets[c], other, ws, wsBytes));
-			HIP_CALL(fitre_hip_conv_input_grad(&shape, dc, vector + wOffsets[c], tmp, ws, wsBytes));
-			HIP_CALL(fitre_hip_axpy((int)inCount, 1.f, tmp, other));
+			if (fitre_hip_conv_pair_supported(&shape, 1)) {
+				HIP_CALL(fitre_hip_conv_input_grad_pair(&shape, rdc, weights + wOffsets[c], dc, vector + wOffsets[c], other, ws, wsBytes));
+			} else {
+				HIP_CALL(fitre_hip_conv_input_grad(&shape, rdc, weights + wOffsets[c], other, ws, wsBytes));
+				HIP_CALL(fitre_hip_conv_input_grad(&shape, dc, vector + wOffsets[c], tmp, ws, wsBytes));
+				HIP_CALL(fitre_hip_axpy((int)inCount, 1.f, tmp, other));
+			}
 			if (other != rdelta) t = rdelta, rdelta = rnext, rnext = t;
 		}
 	}

@@ -69,6 +69,11 @@ HIP_API = {
     "fitre_hip_max_pool_argmax": (i32, [vp] + [i32] * 9 + [vp]),
     "fitre_hip_pool_act_backward": (i32, [i32, i32, vp, vp, vp] + [i32] * 9 + [vp, vp]),
     "fitre_hip_pool_act_bn_backward": (i32, [i32, i32, vp, i32, lng, vp, vp, vp] + [i32] * 9 + [f32, vp, vp, vp, vp, vp, sz]),
+    "fitre_hip_conv_pair_supported": (i32, [pshape, i32]),
+    "fitre_hip_conv_pair_workspace": (sz, [pshape, i32]),
+    "fitre_hip_conv_forward_pair": (i32, [pshape, vp, vp, vp, vp, vp, vp, vp, sz]),
+    "fitre_hip_conv_input_grad_pair": (i32, [pshape, vp, vp, vp, vp, vp, vp, sz]),
+    "fitre_hip_conv_weight_grad_pair": (i32, [pshape, vp, vp, vp, vp, vp, vp, sz]),
     "fitre_hip_conv_input_grad_split": (i32, [pshape, vp, vp, vp, vp, sz, vp]),
     "fitre_hip_extract_columns": (i32, [vp, vp, vp, i32, i32]),
     "fitre_hip_augment_batch": (i32, [vp, i32, i32, i32, i32, i32, vp, i32, f32, vp, vp, vp, f32, vp]),

@@ -295,6 +295,23 @@ int fitre_hip_conv_weight_grad(const fitre_conv_shape *s, const float *x, const 
 size_t fitre_hip_conv_input_grad_workspace(const fitre_conv_shape *s);
 int fitre_hip_conv_input_grad(const fitre_conv_shape *s, const float *delta, const float *w, float *dx,
                               void *ws, size_t wsBytes);
+/* Sums of two products of one shape in one launch, for the R operator of the Hessian-vector product
+ * (functions/cnn_hv_forward.cu, cnn_hv_backward.cu: every convolution there is a sum of two):
+ *   forward_pair:      y  = conv(x1, w1) + conv(x2, w2) + bias
+ *   input_grad_pair:   dx = dX(delta1, w1) + dX(delta2, w2)
+ *   weight_grad_pair:  dW = dW(x1, delta1) + dW(x2, delta2)
+ * The reduction simply runs over the first pair and then over the second: one set of accumulators, one epilogue, one
+ * reduction of split partials, no temporary and no addition pass.  3x3 / stride 1 / padding 1 shapes that the
+ * specialised kernels take only (kind 0 forward, 1 input gradient, 2 weight gradient): ask _pair_supported first;
+ * the _pair_workspace of an unsupported shape is 0. */
+int fitre_hip_conv_pair_supported(const fitre_conv_shape *s, int kind);
+size_t fitre_hip_conv_pair_workspace(const fitre_conv_shape *s, int kind);
+int fitre_hip_conv_forward_pair(const fitre_conv_shape *s, const float *x1, const float *w1, const float *x2,
+                                const float *w2, const float *bias, float *y, void *ws, size_t wsBytes);
+int fitre_hip_conv_input_grad_pair(const fitre_conv_shape *s, const float *delta1, const float *w1,
+                                   const float *delta2, const float *w2, float *dx, void *ws, size_t wsBytes);
+int fitre_hip_conv_weight_grad_pair(const fitre_conv_shape *s, const float *x1, const float *delta1, const float *x2,
+                                    const float *delta2, float *dW, void *ws, size_t wsBytes);
 /* The same product, but when its reduction is split over workgroups the partial results are left unsummed
  * for the consumer to add up while it reads them (fitre_hip_pool_act_bn_backward takes such a view): one
  * launch and one pass over dx less.  view->base points at view->splits slabs of Cin*N*inA*inB floats,

@@ -103,6 +103,70 @@ def test_conv_input_gradient(dev, oracle64, case):
     assert rel_err(got, want) < TOL
 
 
+PAIR_CASES = [c for c in CONV_CASES if c[5] == 3 and c[6] == 1 and c[7] == 1] + [(256, 64, 128, 16, 16, 3, 1, 1),
+                                                                                 (64, 512, 512, 2, 2, 3, 1, 1)]
+
+
+@pytest.mark.parametrize("case", PAIR_CASES)
+def test_sums_of_two_products_in_one_launch(dev, oracle64, case):
+    """conv(x1,w1) + conv(x2,w2) + bias, dX(d1,w1) + dX(d2,w2) and dW(x1,d1) + dW(x2,d2) through the pair entry points,
+    for every shape the specialised 3x3 kernels take, against the oracle's two products added in float64 (and, at the
+    two benchmark-sized shapes, against the device's own two products added)."""
+    N, Cin, Cout, A, B, k, s, p = case
+    shape = conv_shape(N, Cin, Cout, A, B, k, s, p)
+    rng = np.random.default_rng(sum(case) + 11)
+    big = N * A * B * max(Cin, Cout) > 2_000_000
+    xs = [rng.standard_normal(Cin * N * A * B).astype(np.float32) for _ in range(2)]
+    ws_ = [(rng.standard_normal(Cout * Cin * 9) / np.sqrt(Cin * 9)).astype(np.float32) for _ in range(2)]
+    ds = [rng.standard_normal(Cout * N * A * B).astype(np.float32) for _ in range(2)]
+    b = rng.standard_normal(Cout).astype(np.float32)
+    px, pw, pd, pb = [dev.upload(v) for v in xs], [dev.upload(v) for v in ws_], [dev.upload(v) for v in ds], dev.upload(b)
+
+    def single(which, i):
+        """the device's single product (reference when the oracle would take too long)"""
+        if which == 0:
+            nb = hip.fitre_hip_conv_forward_workspace(C.byref(shape)); w_ = dev.alloc(nb); out = dev.zeros(ds[0].size)
+            L.check(hip.fitre_hip_conv_forward(C.byref(shape), px[i], pw[i], pb if i == 0 else None, out, w_, nb)); n = ds[0].size
+        elif which == 1:
+            nb = hip.fitre_hip_conv_input_grad_workspace(C.byref(shape)); w_ = dev.alloc(nb); out = dev.zeros(xs[0].size)
+            L.check(hip.fitre_hip_conv_input_grad(C.byref(shape), pd[i], pw[i], out, w_, nb)); n = xs[0].size
+        else:
+            nb = hip.fitre_hip_conv_weight_grad_workspace(C.byref(shape)); w_ = dev.alloc(nb); out = dev.zeros(ws_[0].size)
+            L.check(hip.fitre_hip_conv_weight_grad(C.byref(shape), px[i], pd[i], out, w_, nb)); n = ws_[0].size
+        got = dev.download(out, n).astype(np.float64)
+        dev.free(w_), dev.free(out)
+        return got
+
+    for kind in (0, 1, 2):
+        if not hip.fitre_hip_conv_pair_supported(C.byref(shape), kind):
+            assert hip.fitre_hip_conv_pair_workspace(C.byref(shape), kind) == 0
+            continue
+        nb = hip.fitre_hip_conv_pair_workspace(C.byref(shape), kind)
+        wsp = dev.alloc(nb)
+        if kind == 0:
+            out = dev.upload(np.full(ds[0].size, np.nan, np.float32))
+            L.check(hip.fitre_hip_conv_forward_pair(C.byref(shape), px[0], pw[0], px[1], pw[1], pb, out, wsp, nb))
+            got = dev.download(out, ds[0].size)
+            want = single(0, 0) + single(0, 1) if big else (oracle64.conv_forward(xs[0], ws_[0], b, N, Cin, B, A, 3, 1, 1, Cout) +
+                                                           oracle64.conv_forward(xs[1], ws_[1], 0 * b, N, Cin, B, A, 3, 1, 1, Cout))
+        elif kind == 1:
+            out = dev.upload(np.full(xs[0].size, np.nan, np.float32))
+            L.check(hip.fitre_hip_conv_input_grad_pair(C.byref(shape), pd[0], pw[0], pd[1], pw[1], out, wsp, nb))
+            got = dev.download(out, xs[0].size)
+            want = single(1, 0) + single(1, 1) if big else (oracle64.conv_input_grad(ds[0], ws_[0], N, Cin, B, A, 3, 1, Cout) +
+                                                           oracle64.conv_input_grad(ds[1], ws_[1], N, Cin, B, A, 3, 1, Cout))
+        else:
+            out = dev.upload(np.full(ws_[0].size, np.nan, np.float32))
+            L.check(hip.fitre_hip_conv_weight_grad_pair(C.byref(shape), px[0], pd[0], px[1], pd[1], out, wsp, nb))
+            got = dev.download(out, ws_[0].size)
+            want = single(2, 0) + single(2, 1) if big else (oracle64.conv_weight_grad(xs[0], ds[0], N, Cin, B, A, 3, 1, 1, Cout) +
+                                                           oracle64.conv_weight_grad(xs[1], ds[1], N, Cin, B, A, 3, 1, 1, Cout))
+        assert rel_err(got, want) < TOL, kind
+        dev.free(wsp), dev.free(out)
+    for q in px + pw + pd + [pb]:
+        dev.free(q)
+
+
 def test_conv3x3_with_unaligned_weight_and_delta_pointers(dev, oracle64):
     """Flat parameter vectors put weight blocks at arbitrary offsets: the fast paths must fall back to
     4-byte accesses when a pointer is not 16-byte aligned."""
