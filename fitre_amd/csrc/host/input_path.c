@@ -1,6 +1,7 @@
 /* Mini-batch selection and augmentation with the reference's names (utilities/sample_matrix.cu,
  * solvers/kfac_da.cu, augmentation/dev_crop.cu, dev_flip.cu, dev_normalize.cu) over the device layer. */
 #include <stdio.h>
+#include <string.h>
 #include <stdlib.h>
 
 #include "fitre_cnn.h"
@@ -106,13 +107,45 @@ void augmentData(CNN_MODEL *model, DEVICE_DATASET *data, int offset, int current
 	data->currentBatch = second;
 }
 
+/* rows indices[offset + i] (indices == NULL: offset + i) of the host set, gathered in a staging buffer and sent
+ * as one copy each for images and labels */
+static void select_host_rows(HOST_DATASET *host, real *trainX, real *trainY, int numSamples, const int *indices, int offset,
+                             real *labelsOut)
+{
+	const size_t features = (size_t)host->features;
+	real *stage = (real *)malloc((size_t)(numSamples > 0 ? numSamples : 1) * (features + 1) * sizeof(real));
+	if (stage == NULL) {
+		fprintf(stderr, "selectHostMatrix: no host memory for %d images of %zu values\n", numSamples, features);
+		exit(-1);
+	}
+	real *labels = stage + (size_t)numSamples * features;
+	for (int i = 0; i < numSamples; i++) {
+		const int row = indices != NULL ? indices[offset + i] : offset + i;
+		if (row < 0 || row >= host->trainSizeX) {
+			fprintf(stderr, "selectHostMatrix: index %d outside the training set of %d images\n", row, host->trainSizeX);
+			exit(-1);
+		}
+		memcpy(stage + (size_t)i * features, host->trainSetX + (size_t)row * features, features * sizeof(real));
+		labels[i] = host->trainSetY[row];
+		if (labelsOut != NULL) labelsOut[i] = labels[i];
+	}
+	HIP_CALL(fitre_hip_copy_h2d(trainX, stage, (size_t)numSamples * features * sizeof(real)));
+	HIP_CALL(fitre_hip_copy_h2d(trainY, labels, (size_t)numSamples * sizeof(real)));
+	free(stage);
+}
+
+void selectHostMatrix(HOST_DATASET *host, real *trainX, real *trainY, int numSamples, int *indices, int offset, real *hostPtr)
+{
+	select_host_rows(host, trainX, trainY, numSamples, indices, offset, hostPtr);
+}
+
 /* One evaluation sweep in batches of model->batchSize (the last one shorter): copy the batch's columns
  * and labels, layout change + normalisation (no augmentation), forward pass, accuracy.
  * functions/cnn_accuracy.cu:61-110 (test set) and :112-174 (training set; the reference's sweep stops
  * before a final short batch yet divides by the full size, and so does this one). */
 static void generalization_sweep(CNN_MODEL *model, DEVICE_DATASET *data, SCRATCH_AREA *scratch, real *z, real *probs,
-                                 real *errors, const real *setX, const real *setY, int setSize, EVAL_TYPE mode,
-                                 int dropShortTail, real *likelihood, real *accuracy)
+                                 real *errors, const real *setX, const real *setY, HOST_DATASET *hostSet, int setSize,
+                                 EVAL_TYPE mode, int dropShortTail, real *likelihood, real *accuracy)
 {
 	real hits = 0;
 	int curIdx = 0, curBatchSize = model->batchSize;
@@ -121,13 +154,18 @@ static void generalization_sweep(CNN_MODEL *model, DEVICE_DATASET *data, SCRATCH
 	*accuracy = 0;
 	if (curBatchSize > setSize) curBatchSize = setSize;
 	while (curIdx < setSize && curBatchSize > 0) {
-		HIP_CALL(fitre_hip_copy_d2d(data->sampledTrainX, setX + (size_t)data->features * curIdx,
-		                            sizeof(real) * (size_t)data->features * curBatchSize));
-		HIP_CALL(fitre_hip_copy_d2d(data->sampledTrainY, setY + curIdx, sizeof(real) * (size_t)curBatchSize));
+		if (hostSet != NULL) {
+			select_host_rows(hostSet, data->sampledTrainX, data->sampledTrainY, curBatchSize, NULL, curIdx, NULL);
+		} else {
+			HIP_CALL(fitre_hip_copy_d2d(data->sampledTrainX, setX + (size_t)data->features * curIdx,
+			                            sizeof(real) * (size_t)data->features * curBatchSize));
+			HIP_CALL(fitre_hip_copy_d2d(data->sampledTrainY, setY + curIdx, sizeof(real) * (size_t)curBatchSize));
+		}
 		augmentData(model, data, curIdx, curBatchSize, nextDevPtr, nextHostPtr, 0, data->datasetType);
 		real batchLikelihood = cnnForward(model, data, scratch, z, probs, errors, curIdx, curBatchSize, mode);
 		*likelihood += batchLikelihood * curBatchSize;
-		computeAccuracy(probs, (real *)(setY + curIdx), curBatchSize, data->numClasses, nextDevPtr, nextPageLckPtr);
+		computeAccuracy(probs, hostSet != NULL ? data->sampledTrainY : (real *)(setY + curIdx), curBatchSize, data->numClasses,
+		                nextDevPtr, nextPageLckPtr);
 		hits += *nextPageLckPtr;
 		curIdx += curBatchSize;
 		if (curIdx + model->batchSize < setSize) {
@@ -144,18 +182,23 @@ static void generalization_sweep(CNN_MODEL *model, DEVICE_DATASET *data, SCRATCH
 void computeTestGeneralizationErrors(CNN_MODEL *model, DEVICE_DATASET *data, SCRATCH_AREA *scratch, real *z, real *probs,
                                      real *errors, real *likelihood, real *accuracy)
 {
-	generalization_sweep(model, data, scratch, z, probs, errors, data->testSetX, data->testSetY, data->testSizeX,
+	generalization_sweep(model, data, scratch, z, probs, errors, data->testSetX, data->testSetY, NULL, data->testSizeX,
 	                     MODEL_TEST_ACCURACY, 0, likelihood, accuracy);
 }
 
 void computeTrainGeneralizationErrors(CNN_MODEL *model, DEVICE_DATASET *data, HOST_DATASET *host, SCRATCH_AREA *scratch, real *z,
                                       real *probs, real *errors, real *likelihood, real *accuracy)
 {
-	(void)host; /* the reference reads it for data sets kept in host memory only */
+	/* a training set kept in host memory (the reference's IMAGENET case, functions/cnn_accuracy.cu:136-143)
+	 * is read through the host struct, batch by batch */
+	HOST_DATASET *hostSet = NULL;
 	if (data->datasetType == IMAGENET) {
-		fprintf(stderr, "computeTrainGeneralizationErrors: data sets kept in host memory are not supported\n");
-		exit(-1);
+		if (host == NULL || host->trainSetX == NULL || host->trainSetY == NULL) {
+			fprintf(stderr, "computeTrainGeneralizationErrors: the training set is neither on the device nor on the host\n");
+			exit(-1);
+		}
+		hostSet = host;
 	}
-	generalization_sweep(model, data, scratch, z, probs, errors, data->trainSetX, data->trainSetY, data->trainSizeX,
+	generalization_sweep(model, data, scratch, z, probs, errors, data->trainSetX, data->trainSetY, hostSet, data->trainSizeX,
 	                     MODEL_TRAIN_ACCURACY, 1, likelihood, accuracy);
 }

@@ -210,15 +210,25 @@ void subsampledTrustRegionKFAC(CNN_MODEL *model, DEVICE_DATASET *data, HOST_DATA
 	(void)master;
 	(void)slave;
 	const DATASET_TYPE datasetType = host != NULL ? host->datasetType : data->datasetType;
-	if (datasetType != CIFAR10 && datasetType != CIFAR100) {
-		/* the reference's third case reads mini-batches from host memory (selectHostMatrix) */
+	/* the third case keeps the training set in host memory and reads mini-batches from there
+	 * (selectHostMatrix, solvers/kfac_trust_region.cu:322-337) */
+	const int hostResident = datasetType == IMAGENET;
+	if (datasetType != CIFAR10 && datasetType != CIFAR100 && datasetType != IMAGENET) {
 		fprintf(stderr, "Problem with the dataset initialization.... \n\n");
+		exit(-1);
+	}
+	if (hostResident && (host == NULL || host->trainSetX == NULL || host->trainSetY == NULL)) {
+		fprintf(stderr, "subsampledTrustRegionKFAC: a host-resident data set needs the host struct's training arrays\n");
 		exit(-1);
 	}
 	const int layers = model->cLayers + model->lLayers;
 	const int components = model->pSize;
 	const long batch = model->batchSize, classes = data->numClasses;
 	real *pageLckPtr = scratch->nextPageLckPtr;
+	/* what the loop carves from the arenas is released when it returns: a second call with the same struct
+	 * starts from the same addresses (the reference leaves the pointers advanced) */
+	real *const entryDevPtr = scratch->nextDevPtr, *const entryHostPtr = scratch->nextHostPtr;
+	real *const entryPageLckPtr = scratch->nextPageLckPtr;
 	int *hostIndices = (int *)scratch->nextHostPtr;
 	real *nextHostPtr = scratch->nextHostPtr + round_up(data->trainSizeX);
 
@@ -297,7 +307,10 @@ void subsampledTrustRegionKFAC(CNN_MODEL *model, DEVICE_DATASET *data, HOST_DATA
 				break;
 
 			t0 = now_seconds();
-			selectColumnMatrix(data, (int)curBatchSize, shuffleIndices, (int)offset);
+			if (hostResident)
+				selectHostMatrix(host, data->sampledTrainX, data->sampledTrainY, (int)curBatchSize, hostIndices, (int)offset, NULL);
+			else
+				selectColumnMatrix(data, (int)curBatchSize, shuffleIndices, (int)offset);
 			augmentData(model, data, (int)offset, (int)curBatchSize, scratchBegin, nextHostPtr, 1, datasetType);
 			sumAugment += now_seconds() - t0;
 
@@ -427,4 +440,7 @@ void subsampledTrustRegionKFAC(CNN_MODEL *model, DEVICE_DATASET *data, HOST_DATA
 		g_report_count++;
 	}
 	if (g_report_count > MAX_REPORTS) g_report_count = MAX_REPORTS;
+	scratch->nextDevPtr = entryDevPtr;
+	scratch->nextHostPtr = entryHostPtr;
+	scratch->nextPageLckPtr = entryPageLckPtr;
 }

@@ -154,6 +154,7 @@ CNN_API = {
     "readVector": (i32, [vp, i32, C.c_char_p, i32, vp]),
     # include/fitre_input.h
     "selectColumnMatrix": (None, [pdata, i32, vp, i32]),
+    "selectHostMatrix": (None, [vp, vp, vp, i32, vp, i32, vp]),
     "randomCrop": (None, [vp, i32, i32, i32, i32, i32, vp, vp, vp, f32, vp]),
     "flipData": (None, [vp, vp, i32, i32, i32, i32, vp, vp, vp]),
     "normalizeCIFAR10": (None, [vp, i32, i32, i32, i32, vp, vp, i32]),
@@ -183,6 +184,24 @@ CNN_API = {
     "kfacTrustRegionHostMemRequired": (lng, [pdata]),
     "kfacTrustRegionReports": (i32, [vp, i32]),
     "subsampledTrustRegionKFAC": (None, [pmodel, pdata, vp, pkfac, vp, pscratch, i32, i32]),
+    # include/fitre_dataset.h
+    "convertToColumnMajor": (None, [vp, i32, i32, vp]),
+    "convertCIFARToColumnMajor": (None, [vp, vp, i32, i32, i32, i32]),
+    "imageNormalization": (None, [vp, i32, i32, i32, i32, f32, i32]),
+    "readCIFARDataset": (None, [C.c_char_p, C.c_char_p, i32, C.c_char_p, vp, vp, i32, i32, i32, i32, i32]),
+    "initialize_device_data": (None, [vp, pdata]),
+    "initialize_device_image": (None, [vp, pdata]),
+    "cleanup_dataset": (None, [vp, pdata]),
+    "fitreSetDatasetFolder": (None, [i32, C.c_char_p]),
+    "fitreSetWeightsFolder": (None, [C.c_char_p]),
+    "getCIFAR10": (i32, [pmodel, vp, pdata, pscratch]),
+    "getCIFAR100": (i32, [pmodel, vp, pdata, pscratch]),
+    "getTinyImageNet": (i32, [pmodel, vp, pdata, pscratch]),
+    "cnnInitializations": (None, [pmodel, pdata]),
+    "initKFACTrustRegionParams": (None, [vp, i32]),
+    "initKFACInfo": (None, [pkfac]),
+    "kfacParamsFileName": (i32, [pmodel, i32, i32, C.c_char_p, i32]),
+    "testKFACTrustRegion": (None, [pmodel, pdata, vp, pscratch, f32, f32, i32, i32, i32, i32, i32, i32, f32, i32]),
     # include/fitre_hv.h
     "cnnHvMemRequired": (lng, [pmodel]),
     "cnnHv": (None, [pmodel, pdata, vp, vp, vp, vp, vp, vp, i32, i32, vp, vp, f32]),

@@ -78,6 +78,13 @@ class SCRATCH_AREA(C.Structure):
         "hostWorkspace", "devWorkspace", "pageLckWorkspace", "nextDevPtr", "nextHostPtr", "nextPageLckPtr")]
 
 
+class HOST_DATASET(C.Structure):
+    """include/fitre_types.h (core/structdefs.h of the reference): the data set in host memory."""
+    _fields_ = ([(n, C.POINTER(C.c_float)) for n in ("trainSetX", "trainSetY", "testSetX", "testSetY")] +
+                [(n, C.c_int) for n in ("trainSizeX", "trainSizeY", "testSizeX", "testSizeY", "features", "height", "width",
+                                        "numClasses", "datasetType")])
+
+
 class SparseDataset(C.Structure):
     _fields_ = [("rowPtr", C.c_void_p), ("colPtr", C.c_void_p), ("rowCsrPtr", C.c_void_p),
                 ("valPtr", C.c_void_p), ("nnz", C.c_int), ("sortedVals", C.c_void_p), ("P", C.c_void_p),

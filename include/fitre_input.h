@@ -20,6 +20,12 @@ extern "C" {
  * values each) and of trainSetY into sampledTrainX / sampledTrainY.  indices is a DEVICE array. */
 void selectColumnMatrix(DEVICE_DATASET *data, int sampleSize, int *indices, int offset);
 
+/* utilities/dataset_utils.c:10-25: the same selection from a training set kept in HOST memory: images
+ * indices[offset .. offset+numSamples) of host->trainSetX and their labels into the device buffers trainX,
+ * trainY.  indices is a HOST array.  The rows are gathered in a host staging buffer and
+ * sent as one copy (the reference sends one copy per image); hostPtr, if not NULL, receives the labels too. */
+void selectHostMatrix(HOST_DATASET *host, real *trainX, real *trainY, int numSamples, int *indices, int offset, real *hostPtr);
+
 /* augmentation/dev_crop.cu:60-94: every image shifted by a random (row, column) offset in
  * [-padding, padding], cells from outside read defaultValue.  devPtr: 2*samples reals and as many ints
  * of device scratch; probs and hostPtr are unused, as in the reference. */
@@ -42,7 +48,7 @@ void augmentData(CNN_MODEL *model, DEVICE_DATASET *data, int offset, int current
 
 /* functions/cnn_accuracy.cu:61-174: mean negative log-likelihood and accuracy (percent) over the whole test
  * resp. training set, in batches of model->batchSize through augmentData (no augmentation) and cnnForward.
- * The sets are device-resident, features x size column-major; pixel values 0..255; data->sampledTrainX must
+ * The sets are device-resident (datasetType IMAGENET: the training set is read from `host`), features x size column-major; pixel values 0..255; data->sampledTrainX must
  * hold two batches (augmentData writes the second), scratch->nextDevPtr cnnForwardMemRequired reals,
  * scratch->nextPageLckPtr one real of host memory.  Batch-norm layers use their running statistics. */
 void computeTestGeneralizationErrors(CNN_MODEL *model, DEVICE_DATASET *data, SCRATCH_AREA *scratch, real *z, real *probs,

@@ -95,7 +95,9 @@ int kfacTrustRegionReports(KFAC_TR_EPOCH_REPORT *out, int capacity);
  * place), datasetType CIFAR10 or CIFAR100.  kfacInfo: regLambda, dampGamma, momentum, stats_decay,
  * checkGrad, inverseFreq (1: factors and inverses from every mini-batch; k > 1: from running averages,
  * every k-th mini-batch).  trParams: delta (updated), minDelta, maxDelta, maxIters = passes over the
- * training set.  The sampled-batch buffers are allocated here (allocSampledDataset) and stay with data. */
+ * training set.  The sampled-batch buffers are allocated here (allocSampledDataset) and stay with data.
+ * scratch->nextDevPtr / nextHostPtr / nextPageLckPtr move while the loop runs and are back at their entry values on
+ * return. */
 void subsampledTrustRegionKFAC(CNN_MODEL *model, DEVICE_DATASET *data, HOST_DATASET *host, KFAC_CURVATURE_INFO *kfacInfo,
                                TRUST_REGION_PARAMS *trParams, SCRATCH_AREA *scratch, int master, int slave);
 

@@ -101,7 +101,8 @@ def test_libraries_export_every_declared_symbol():
         assert n in L.HIP_API, "ctypes table lacks %s" % n
     cnn_names = (_declared("fitre_cnn.h", r"\b([A-Za-z_]\w*)\s*\(") + _declared("fitre_shim.h", r"\b([A-Za-z_]\w*)\s*\(") +
                  _declared("fitre_kfac.h", r"\b([A-Za-z_]\w*)\s*\(") + _declared("fitre_fc.h", r"\b([A-Za-z_]\w*)\s*\(") +
-                 _declared("fitre_hv.h", r"\b([A-Za-z_]\w*)\s*\(") + _declared("fitre_input.h", r"\b([A-Za-z_]\w*)\s*\(") + _declared("fitre_solver.h", r"\b([A-Za-z_]\w*)\s*\("))
+                 _declared("fitre_hv.h", r"\b([A-Za-z_]\w*)\s*\(") + _declared("fitre_input.h", r"\b([A-Za-z_]\w*)\s*\(") + _declared("fitre_solver.h", r"\b([A-Za-z_]\w*)\s*\(") +
+                 _declared("fitre_dataset.h", r"\b([A-Za-z_]\w*)\s*\("))
     cnn_names = [n for n in cnn_names if n not in ("defined",)]
     assert "cnnBackward" in cnn_names and "computeCNNGradient" in cnn_names and "copy_host_device" in cnn_names
     assert "computeOmegaZFactors" in cnn_names and "computeKFACStorageIndices" in cnn_names
@@ -109,6 +110,7 @@ def test_libraries_export_every_declared_symbol():
     assert "augmentData" in cnn_names and "selectColumnMatrix" in cnn_names and "computeTestGeneralizationErrors" in cnn_names
     assert "computeOmegaZAndLambdaDelta" in cnn_names
     assert "subsampledTrustRegionKFAC" in cnn_names and "genRandomVector" in cnn_names
+    assert "readCIFARDataset" in cnn_names and "testKFACTrustRegion" in cnn_names and "selectHostMatrix" in cnn_names
     assert "computeGradient" in cnn_names and "nnForwardPass" in cnn_names and "computeNaturalGradient" in cnn_names
     for n in cnn_names:
         assert hasattr(L.cnn, n), n
