@@ -4,6 +4,7 @@
  * drivers/kfac_trust_region_driver.cu).  Records are transposed into the column-major image layout while
  * they are read, so no second host copy of the set is needed.
  */
+#define _GNU_SOURCE
 #include <limits.h>
 #include <math.h>
 #include <stdio.h>
@@ -83,6 +84,54 @@ void imageNormalization(real *src, int numImages, int channels, int height, int 
 		const real m = mean[datasetType - 1][c % 3], s = std[datasetType - 1][c % 3];
 		for (size_t i = 0; i < perChannel; i++) p[i] = (p[i] / constant - m) / s;
 	}
+}
+
+/* ---- delimited text ---------------------------------------------------------------------------- */
+
+static int count_tokens(const char *line)
+{
+	int n = 0, inToken = 0;
+	for (const char *c = line; *c; c++) {
+		const int sep = *c == ',' || *c == ' ' || *c == '\n' || *c == '\r' || *c == '\t';
+		if (!sep && !inToken) n++;
+		inToken = !sep;
+	}
+	return n;
+}
+
+void readDelimitedMatrix(char *fileName, real **data, int *rows, int *cols)
+{
+	FILE *f = fopen(fileName, "r");
+	fprintf(stderr, "Reading file: %s \n", fileName);
+	if (f == NULL) {
+		fprintf(stderr, "Error opening the dataset.... !\n");
+		exit(-1);
+	}
+	char *line = NULL;
+	size_t cap = 0;
+	*rows = *cols = 0;
+	while (getline(&line, &cap, f) > 0) { /* first pass: the shape; an empty line ends the matrix */
+		const int n = count_tokens(line);
+		if (n == 0) break;
+		*cols = n;
+		(*rows)++;
+	}
+	fprintf(stderr, "Rows : %d, Columns : %d \n", *rows, *cols);
+	const size_t total = (size_t)*rows * (size_t)*cols;
+	*data = (real *)calloc(total > 0 ? total : 1, sizeof(real));
+	if (*data == NULL) {
+		fprintf(stderr, "readDelimitedMatrix: no host memory for %d x %d values\n", *rows, *cols);
+		exit(-1);
+	}
+	rewind(f);
+	for (int r = 0; r < *rows && getline(&line, &cap, f) > 0; r++) {
+		int c = 0;
+		for (char *word = strtok(line, ", \n\r\t"); word != NULL && c < *cols; word = strtok(NULL, ", \n\r\t"))
+			(*data)[(size_t)r * *cols + c++] = (real)atof(word);
+	}
+	free(line);
+	fclose(f);
+	fprintf(stderr, "Done reading: %s \n", fileName);
 }
 
 /* ---- record files ---------------------------------------------------------------------------- */

@@ -188,6 +188,7 @@ CNN_API = {
     "convertToColumnMajor": (None, [vp, i32, i32, vp]),
     "convertCIFARToColumnMajor": (None, [vp, vp, i32, i32, i32, i32]),
     "imageNormalization": (None, [vp, i32, i32, i32, i32, f32, i32]),
+    "readDelimitedMatrix": (None, [C.c_char_p, C.POINTER(C.POINTER(C.c_float)), pi32, pi32]),
     "readCIFARDataset": (None, [C.c_char_p, C.c_char_p, i32, C.c_char_p, vp, vp, i32, i32, i32, i32, i32]),
     "initialize_device_data": (None, [vp, pdata]),
     "initialize_device_image": (None, [vp, pdata]),

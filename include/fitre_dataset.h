@@ -36,6 +36,11 @@ void convertCIFARToColumnMajor(real *src, real *tgt, int datasetSize, int channe
  * datasetType 1, 2, 3 selects the CIFAR-10, CIFAR-100 or ImageNet statistics; anything else exits(-1). */
 void imageNormalization(real *src, int numImages, int channels, int height, int width, real constant, int datasetType);
 
+/* utilities/dataset.c:198-240: a text matrix, one row per line, values separated by commas or blanks, into a
+ * malloc'ed row-major array; the last line's token count is the column count (as there), an empty line ends the
+ * matrix, short rows are padded with zeros.  Lines of any length (the reference stops at 4 MiB). */
+void readDelimitedMatrix(char *fileName, real **data, int *rows, int *cols);
+
 /* utilities/dataset.c:373-571.  Reads dir + train + "1.bin" .. dir + train + "<numFiles>.bin" and the test file
  * dir + test (dataset 3: dir + test + "1.bin" and "2.bin") into malloc'ed host arrays of `data`, sets
  * trainSizeX/Y, testSizeX/Y, features and numClasses (10, 100, 200).  A trailing partial record counts as a

@@ -172,3 +172,22 @@ def test_driver_defaults():
     assert (info.stats_decay, info.momentum, info.regLambda, info.dampGamma, info.checkGrad) == (
         np.float32(0.8), 0.0, np.float32(1e-3), 100.0, 1)
     assert info.OmegaZInv is None and list(info.OmegaZOffsets) == [0] * 20
+
+
+def test_delimited_text_matrix(tmp_path):
+    rng = np.random.default_rng(6)
+    m = rng.standard_normal((7, 5)).astype(np.float32)
+    lines = [", ".join("%.9g" % v for v in row) for row in m[:4]] + [" ".join("%.9g" % v for v in row) for row in m[4:]]
+    path = tmp_path / "m.csv"
+    path.write_text("\n".join(lines) + "\n\n9, 9, 9, 9, 9\n")          # the empty line ends the matrix
+    data, rows, cols = C.POINTER(C.c_float)(), C.c_int(), C.c_int()
+    cnn.readDelimitedMatrix(str(path).encode(), C.byref(data), C.byref(rows), C.byref(cols))
+    assert (rows.value, cols.value) == (7, 5)
+    np.testing.assert_array_equal(as_array(data, 35).reshape(7, 5), m)
+    C.CDLL(None).free(C.cast(data, C.c_void_p))
+    wide = tmp_path / "wide.csv"                                           # one line far beyond any fixed buffer
+    row = np.arange(300000, dtype=np.float32)
+    wide.write_text(",".join("%d" % v for v in row) + "\n")
+    cnn.readDelimitedMatrix(str(wide).encode(), C.byref(data), C.byref(rows), C.byref(cols))
+    assert (rows.value, cols.value) == (1, 300000)
+    np.testing.assert_array_equal(as_array(data, 300000), row)
