@@ -132,12 +132,15 @@ def gpu_leg(args):
     gm.backward()  # dx of the last forward pass, for the legs below
     grad = gm.get("grad")
     finite = bool(np.isfinite(grad).all() and np.isfinite(loss))
-    kfac = kfac_leg(L, dev, gm, model, batch, max(2, args.steps // 4))
-    kfac["hessian_vector_ms"] = hv_leg(L, dev, gm, model, batch, max(2, args.steps // 4))
-    kfac["trust_region_step_ms"] = kfac_step_leg(L, dev, gm, model, batch, 3)
+    kfac, bandwidth, others = None, None, None
+    if not args.headline_only:
+        kfac = kfac_leg(L, dev, gm, model, batch, max(2, args.steps // 4))
+        kfac["hessian_vector_ms"] = hv_leg(L, dev, gm, model, batch, max(2, args.steps // 4))
+        kfac["trust_region_step_ms"] = kfac_step_leg(L, dev, gm, model, batch, 3)
     gm.release()
-    bandwidth = bandwidth_leg(L, dev, batch)
-    others = other_configs_leg(L, dev)
+    if not args.headline_only:
+        bandwidth = bandwidth_leg(L, dev, batch)
+        others = other_configs_leg(L, dev)
     dev.close()
 
     kernels = {}
@@ -428,6 +431,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--serial", action="store_true",
                     help="run every kernel on one stream (for kernel tracers: durations do not overlap)")
+    ap.add_argument("--headline-only", action="store_true",
+                    help="only the headline workload (no factor / inverse / Hessian-vector / bandwidth / other-network legs): "
+                         "under a kernel tracer every launch then belongs to the VGG-11 batch-256 passes")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (the reference path is single-device and every "
