@@ -324,6 +324,23 @@ __global__ void __launch_bounds__(256) activation_rop_backward_kernel(int actFun
 	}
 }
 
+// out = f'(z) rdz + rx g(z) dx with dx the delta BELOW the activation (dx = f'(z) dz, so f''(z) dz = g(z) dx):
+// logistic f' = z (1 - z), g = 1 - 2 z; tanh f' = (1 + z)(1 - z), g = -2 z; linear f' = 1, g = 0.  rx == nullptr: first term only.
+__global__ void __launch_bounds__(256) fc_rop_backward_kernel(int actFun, const float *z, const float *rdz, const float *rx,
+                                                               const float *dx, float *out, long n)
+{
+	const long stride = (long)gridDim.x * blockDim.x;
+	for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+		const float zi = z ? z[i] : 0.f;
+		float f1 = 1.f, g = 0.f;
+		if (actFun == ACT_LOGISTIC) f1 = (1.f - zi) * zi, g = 1.f - 2.f * zi;
+		else if (actFun == ACT_TANH) f1 = (1.f + zi) * (1.f - zi), g = -2.f * zi;
+		float v = f1 * rdz[i];
+		if (rx) v += rx[i] * g * dx[i];
+		out[i] = v;
+	}
+}
+
 // dst[c*ldd + r] = src[c*lds + r] for r < rows, c < cols
 __global__ void __launch_bounds__(256) copy_2d_kernel(const float *src, long lds_, float *dst, long ldd, int rows, int cols)
 {
@@ -449,6 +466,18 @@ int fitre_hip_activation_rop_backward(int actFun, const float *rdelta, const flo
 	LaunchScope scope(FITRE_KC_ACT_BWD, 24.0 * (double)n);
 	activation_rop_backward_kernel<<<blocks_for(n, 1024, 8192), 256, 0, stream()>>>(actFun, rdelta, delta, z_in, z_out, rz_in, out, n);
 	return check_launch("activation_rop_backward_kernel");
+}
+
+int fitre_hip_fc_rop_backward(int actFun, const float *z, const float *rdz, const float *rx, const float *dx, float *out, long n)
+{
+	EW_CHECK("fitre_hip_fc_rop_backward", rdz && out && n >= 0 && (rx == nullptr || dx != nullptr));
+	if (actFun != ACT_LOGISTIC && actFun != ACT_TANH && actFun != ACT_LINEAR)
+		return fail(FITRE_E_UNSUPPORTED, "fitre_hip_fc_rop_backward: activation code %d (logistic, tanh and linear only)", actFun);
+	FITRE_REQUIRE(z || actFun == ACT_LINEAR, "fitre_hip_fc_rop_backward: activation %d needs z", actFun);
+	if (n == 0) return FITRE_OK;
+	LaunchScope scope(FITRE_KC_ACT_BWD, 20.0 * (double)n);
+	fc_rop_backward_kernel<<<blocks_for(n, 1024, 8192), 256, 0, stream()>>>(actFun, z, rdz, rx, dx, out, n);
+	return check_launch("fc_rop_backward_kernel");
 }
 
 int fitre_hip_column_softmax(float *x, int rows, int cols)

@@ -970,17 +970,16 @@ __global__ void __launch_bounds__(256) accuracy_hits_kernel(const float *probs, 
 	hits[r] = ((float)(arg + 1) == target[r]) ? 1.f : 0.f;
 }
 
-// rError[r][i] = p_i (rz_i - sum_j p_j rz_j) / rows
+// rError[r][i] = p_i (rz_i - sum_j p_j rz_j) * scale
 __global__ void __launch_bounds__(256) cross_entropy_rop_error_kernel(const float *rz, const float *probs, int rows, int classes,
-                                                                       float *rError)
+                                                                       float scale, float *rError)
 {
 	const int r = blockIdx.x * blockDim.x + threadIdx.x;
 	if (r >= rows) return;
 	const float *p = probs + (size_t)r * classes, *z = rz + (size_t)r * classes;
 	float s = 0.f;
 	for (int j = 0; j < classes; j++) s += p[j] * z[j];
-	const float inv = 1.f / (float)rows;
-	for (int i = 0; i < classes; i++) rError[(size_t)r * classes + i] = p[i] * (z[i] - s) * inv;
+	for (int i = 0; i < classes; i++) rError[(size_t)r * classes + i] = p[i] * (z[i] - s) * scale;
 }
 
 __global__ void cross_entropy_error_kernel(const float *probs, const float *target, int rows, int classes, float *errors)
@@ -1386,7 +1385,17 @@ int fitre_hip_cross_entropy_rop_error(const float *rz, const float *probs, int r
 	FITRE_REQUIRE(rz && probs && rError, "fitre_hip_cross_entropy_rop_error: null pointer");
 	FITRE_REQUIRE(rows > 0 && classes > 0, "fitre_hip_cross_entropy_rop_error: non-positive shape %d x %d", rows, classes);
 	LaunchScope scope(FITRE_KC_SOFTMAX, 12.0 * (double)rows * classes);
-	cross_entropy_rop_error_kernel<<<blocks_for(rows, 256), 256, 0, stream()>>>(rz, probs, rows, classes, rError);
+	cross_entropy_rop_error_kernel<<<blocks_for(rows, 256), 256, 0, stream()>>>(rz, probs, rows, classes, 1.f / (float)rows, rError);
+	return check_launch("cross_entropy_rop_error_kernel");
+}
+
+int fitre_hip_column_softmax_rop(const float *probs, const float *rx, int rows, int cols, float *out)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(probs && rx && out, "fitre_hip_column_softmax_rop: null pointer");
+	FITRE_REQUIRE(rows > 0 && cols > 0, "fitre_hip_column_softmax_rop: non-positive shape %d x %d", rows, cols);
+	LaunchScope scope(FITRE_KC_SOFTMAX, 12.0 * (double)rows * cols);
+	cross_entropy_rop_error_kernel<<<blocks_for(cols, 256), 256, 0, stream()>>>(rx, probs, cols, rows, 1.f, out);
 	return check_launch("cross_entropy_rop_error_kernel");
 }
 

@@ -283,3 +283,138 @@ void computeGradient(NN_MODEL *model, DEVICE_DATASET *data, SCRATCH_AREA *scratc
 	HIP_CALL(fitre_hip_scal(model->pSize, (real)(-1.0 / (double)n), dW));
 	HIP_CALL(fitre_hip_sync());
 }
+
+/* ---- Hessian-vector products (functions/eval_hessian_vec.cu, eval_gauss_newton_hessian_vec.cu) ---- */
+
+typedef struct hv_layout {
+	long n, zReals, rReals;
+	size_t wsBytes;
+} HV_LAYOUT;
+
+static HV_LAYOUT hv_layout(const NN_MODEL *model, const DEVICE_DATASET *data, DATASET_SIZE allData)
+{
+	HV_LAYOUT l;
+	l.n = (allData == FULL_DATASET) ? data->trainSizeX : data->sampleSize;
+	l.zReals = (allData == FULL_DATASET) ? model->zSize : model->sampledZSize;
+	l.rReals = (allData == FULL_DATASET) ? model->rFullSize : model->sampledRSize;
+	l.wsBytes = product_ws_bytes(model, (int)l.n, 1);
+	return l;
+}
+
+/* [RdW | Rdz | Rdx | Rz | Rx | 2 x features (the reference's vector of ones) | one layer-sized temporary | products] */
+long nnHessianVecMemRequired(NN_MODEL *model, DEVICE_DATASET *data, DATASET_SIZE allData)
+{
+	const HV_LAYOUT l = hv_layout(model, data, allData);
+	return (long)model->pSize + 3 * l.zReals + l.rReals + 2L * data->features + (long)largest_layer(model) * l.n +
+	       (long)(l.wsBytes / sizeof(real)) + 256;
+}
+
+static void nn_rop(NN_MODEL *model, DEVICE_DATASET *data, real *z, real *dx, real *vec, real *weights, SCRATCH_AREA *scratch,
+                   DATASET_SIZE allData, int gaussNewton)
+{
+	const int *layerSizes = model->layerSizes;
+	const int *zOffsets = (allData == FULL_DATASET) ? model->zOffsets : model->sZOffsets;
+	const int *rZOffsets = (allData == FULL_DATASET) ? model->rZOffsets : model->sRZOffsets;
+	const int *bOffsets = model->bOffsets, *wOffsets = model->wOffsets;
+	const int numLayers = model->numLayers;
+	const HV_LAYOUT l = hv_layout(model, data, allData);
+	const int n = (int)l.n;
+	const real *trainX = (allData == FULL_DATASET) ? data->trainSetX : data->sampledTrainX;
+	const char *who = gaussNewton ? "gaussNewtonHessianVec" : "hessianVec";
+
+	const int head = model->actFuns[numLayers - 1];
+	if (head != ACT_LOGISTIC && head != ACT_SOFTMAX) { /* eval_hessian_vec.cu:300-303: the linear head is not derived */
+		fprintf(stderr, "%s: output layer %d is neither logistic nor softmax\n", who, head);
+		exit(-1);
+	}
+
+	real *RdW = scratch->nextDevPtr;
+	real *Rdz = RdW + model->pSize;
+	real *Rdx = Rdz + l.zReals;
+	real *Rz = Rdx + l.rReals;
+	real *Rx = Rz + l.zReals;
+	real *oneVector = Rx + l.zReals; /* kept for the layout; row sums need no ones */
+	real *tmp = oneVector + 2L * data->features;
+	void *ws = align_reals(tmp + (long)largest_layer(model) * n);
+	const real *VW = vec;
+
+	HIP_CALL(fitre_hip_memset(RdW, 0, sizeof(real) * (size_t)model->pSize));
+
+	/* forward: Rx_{i+1} = VW_i z_i + Vb_i + W_i Rz_i;  Rz_{i+1} = f'(.) Rx_{i+1} */
+	for (int i = 0; i < numLayers; i++) {
+		const int out = layerSizes[i + 1], in = layerSizes[i];
+		const long count = (long)out * n;
+		real *rxi = Rx + zOffsets[i + 1], *rzi = Rz + zOffsets[i + 1];
+		const real *zin = (i == 0) ? trainX : z + zOffsets[i];
+		const real *zout = z + zOffsets[i + 1];
+		HIP_CALL(fitre_hip_gemm(0, 0, out, n, in, 1.f, VW + wOffsets[i], out, zin, in, 0.f, rxi, out, VW + bOffsets[i], ws, l.wsBytes));
+		if (i > 0)
+			HIP_CALL(fitre_hip_gemm(0, 0, out, n, in, 1.f, weights + wOffsets[i], out, Rz + zOffsets[i], in, 1.f, rxi, out, NULL, ws,
+			                        l.wsBytes));
+		switch (model->actFuns[i]) {
+		case ACT_LOGISTIC:
+		case ACT_TANH:
+			HIP_CALL(fitre_hip_activation_backward(model->actFuns[i], rxi, NULL, zout, rzi, count));
+			break;
+		case ACT_LINEAR:
+			HIP_CALL(fitre_hip_copy_d2d(rzi, rxi, sizeof(real) * (size_t)count));
+			break;
+		case ACT_SOFTMAX:
+			HIP_CALL(fitre_hip_column_softmax_rop(zout, rxi, out, n, rzi));
+			break;
+		default:
+			fprintf(stderr, "hessianVec: unknown activation function at Layer: %d \n", i);
+			exit(-1);
+		}
+	}
+
+	/* backward, from the head: Rdx_L = -Rz_{L+1} */
+	for (int i = numLayers - 1; i >= 0; i--) {
+		const int out = layerSizes[i + 1], in = layerSizes[i];
+		const long count = (long)out * n;
+		real *rdxi = Rdx + rZOffsets[i];
+		const real *dxi = dx + rZOffsets[i];
+		const real *zin = (i == 0) ? trainX : z + zOffsets[i];
+		if (i == numLayers - 1) {
+			HIP_CALL(fitre_hip_copy_d2d(rdxi, Rz + zOffsets[numLayers], sizeof(real) * (size_t)count));
+			HIP_CALL(fitre_hip_scal((int)count, -1.f, rdxi));
+		} else {
+			const int act = model->actFuns[i];
+			if (act != ACT_LOGISTIC && act != ACT_TANH && act != ACT_LINEAR) {
+				fprintf(stderr, "%s: unknown activation function at Layer: %d \n", who, i);
+				exit(-1);
+			}
+			/* the reference's sweep leaves Rdx of a tanh layer unset (eval_hessian_vec.cu:418-420); its derivative is used here */
+			HIP_CALL(fitre_hip_fc_rop_backward(act, z + zOffsets[i + 1], Rdz + zOffsets[i + 1], gaussNewton ? NULL : Rx + zOffsets[i + 1],
+			                                   gaussNewton ? NULL : dxi, rdxi, count));
+		}
+		/* RdW_i = Rdx_i z_i' (+ dx_i Rz_i', zero for the first layer);  Rdb_i = sum(Rdx_i, 2) */
+		HIP_CALL(fitre_hip_gemm(0, 1, out, in, n, 1.f, rdxi, out, zin, in, 0.f, RdW + wOffsets[i], out, NULL, ws, l.wsBytes));
+		if (!gaussNewton && i > 0)
+			HIP_CALL(fitre_hip_gemm(0, 1, out, in, n, 1.f, dxi, out, Rz + zOffsets[i], in, 1.f, RdW + wOffsets[i], out, NULL, ws,
+			                        l.wsBytes));
+		HIP_CALL(fitre_hip_row_sum(rdxi, out, n, RdW + bOffsets[i]));
+		/* Rdz_i = W_i' Rdx_i (+ VW_i' dx_i; the Gauss-Newton variant keeps that term for the top layer only,
+		 * eval_gauss_newton_hessian_vec.cu:262-275) */
+		if (i > 0) {
+			real *rdzi = Rdz + zOffsets[i];
+			HIP_CALL(fitre_hip_gemm(1, 0, in, n, out, 1.f, weights + wOffsets[i], out, rdxi, out, 0.f, rdzi, in, NULL, ws, l.wsBytes));
+			if (!gaussNewton || i == numLayers - 1)
+				HIP_CALL(fitre_hip_gemm(1, 0, in, n, out, 1.f, VW + wOffsets[i], out, dxi, out, 1.f, rdzi, in, NULL, ws, l.wsBytes));
+		}
+	}
+	HIP_CALL(fitre_hip_scal(model->pSize, (real)(-1.0 / (double)n), RdW));
+	HIP_CALL(fitre_hip_sync());
+}
+
+void hessianVec(NN_MODEL *model, DEVICE_DATASET *data, real *z, real *dx, real *vec, real *weights, SCRATCH_AREA *scratch,
+                DATASET_SIZE allData)
+{
+	nn_rop(model, data, z, dx, vec, weights, scratch, allData, 0);
+}
+
+void gaussNewtonHessianVec(NN_MODEL *model, DEVICE_DATASET *data, real *z, real *dx, real *vec, real *weights,
+                           SCRATCH_AREA *scratch, DATASET_SIZE allData)
+{
+	nn_rop(model, data, z, dx, vec, weights, scratch, allData, 1);
+}

@@ -112,6 +112,8 @@ HIP_API = {
     "fitre_hip_pool_forward_routed": (i32, [i32, vp, vp] + [i32] * 9 + [vp]),
     "fitre_hip_batch_norm_rop_backward": (i32, [vp, vp, vp, vp, vp, vp, vp, i32, lng, f32, vp, vp, sz]),
     "fitre_hip_cross_entropy_rop_error": (i32, [vp, vp, i32, i32, vp]),
+    "fitre_hip_fc_rop_backward": (i32, [i32, vp, vp, vp, vp, vp, lng]),
+    "fitre_hip_column_softmax_rop": (i32, [vp, vp, i32, i32, vp]),
     "fitre_hip_spd_inverse_workspace": (sz, [i32]),
     "fitre_hip_spd_inverse": (i32, [vp, i32, f32, vp, vp, sz, pi32]),
     "fitre_hip_spd_inverse_queued": (i32, [vp, i32, f32, vp, vp, sz, vp]),
@@ -218,6 +220,9 @@ CNN_API = {
     "nnForwardPass": (None, [pnn, pdata, vp, vp, vp, pf32, pf32, vp, vp, i32, i32]),
     "evaluateModel": (None, [pnn, pdata, pscratch, vp, pf32, pf32, i32, i32]),
     "computeGradient": (None, [pnn, pdata, pscratch, vp, vp, vp, vp, pf32, pf32, i32]),
+    "nnHessianVecMemRequired": (lng, [pnn, pdata, i32]),
+    "hessianVec": (None, [pnn, pdata, vp, vp, vp, vp, pscratch, i32]),
+    "gaussNewtonHessianVec": (None, [pnn, pdata, vp, vp, vp, vp, pscratch, i32]),
     "getDeviceParameters": (None, []),
     "fitre_env_init": (None, [pscratch, i32, sz]),
     "cuda_env_init": (None, [pscratch, i32]),

@@ -64,6 +64,21 @@ void evaluateModel(NN_MODEL *model, DEVICE_DATASET *data, SCRATCH_AREA *scratch,
 void computeGradient(NN_MODEL *model, DEVICE_DATASET *data, SCRATCH_AREA *scratch, real *weights, real *z, real *dx,
                      real *gradient, real *ll, real *err, DATASET_SIZE dSize);
 
+/* functions/eval_hessian_vec.h:9-11 and functions/eval_gauss_newton_hessian_vec.h:9-11: the Hessian resp. the
+ * Gauss-Newton matrix of the loss computeGradient differentiates, times vec, by the R-operator; z and dx are the
+ * ones computeGradient left at the same weights and data (allData selects the full or the sampled set and its
+ * offsets).  The product, scaled by -1/n like the gradient, is left in the first pSize reals behind
+ * scratch->nextDevPtr, as in the reference; nnHessianVecMemRequired (no counterpart there) is how many reals it
+ * uses from that pointer.  Heads: logistic and softmax (the linear head exits, eval_hessian_vec.cu:300-303).
+ * Hidden layers: logistic, linear, and tanh -- for tanh the reference's backward sweep leaves the layer's term unset
+ * (:418-420) and the derivative is used here.  The Gauss-Newton variant keeps the reference's VW' dx term of the top
+ * layer (eval_gauss_newton_hessian_vec.cu:262-275). */
+long nnHessianVecMemRequired(NN_MODEL *model, DEVICE_DATASET *data, DATASET_SIZE allData);
+void hessianVec(NN_MODEL *model, DEVICE_DATASET *data, real *z, real *dx, real *vec, real *weights, SCRATCH_AREA *scratch,
+                DATASET_SIZE allData);
+void gaussNewtonHessianVec(NN_MODEL *model, DEVICE_DATASET *data, real *z, real *dx, real *vec, real *weights,
+                           SCRATCH_AREA *scratch, DATASET_SIZE allData);
+
 #ifdef __cplusplus
 }
 #endif

@@ -383,6 +383,14 @@ int fitre_hip_pool_forward_routed(int poolType, const float *values, const float
 int fitre_hip_batch_norm_rop_backward(const float *rdelta_x, const float *delta_x, const float *zhat, const float *rzhat,
                                       const float *rx, const float *delta_c, const float *variance, int channels,
                                       long perChannel, float epsilon, float *out, void *ws, size_t wsBytes);
+/* The R-operator over a fully connected model (functions/eval_hessian_vec.cu):
+ * fc_rop_backward: out = f'(z) rdz + rx g(z) dx, the directional derivative of dx = f'(z) dz written with dx
+ *   itself (eval_backprop_hessian, functions/dev_hessian_helpers.cu:7-15: logistic, g = 1 - 2 z; tanh here too,
+ *   g = -2 z; linear: out = rdz); rx == NULL leaves the second term out (eval_gauss_newton_backprop, :17-26).
+ * column_softmax_rop: out = p . rx - p sum(p . rx) per column of the rows x cols matrices
+ *   (functions/eval_hessian_vec.cu:219-262). */
+int fitre_hip_fc_rop_backward(int actFun, const float *z, const float *rdz, const float *rx, const float *dx, float *out, long n);
+int fitre_hip_column_softmax_rop(const float *probs, const float *rx, int rows, int cols, float *out);
 /* rError = p_i (rz_i - sum_j p_j rz_j) / rows (computeROpCrossEntropyError_simple, functions/softmax_loss.cu:251-300) */
 int fitre_hip_cross_entropy_rop_error(const float *rz, const float *probs, int rows, int classes, float *rError);
 

@@ -45,7 +45,9 @@
  * the logged LeNet parameter offsets; the Kronecker factors against unfold
  * patches and numpy Gram products; the inverse against scipy's Cholesky
  * solver; the natural gradient against a Kronecker-product solve; the fully
- * connected model family against autograd of each head's loss; the
+ * connected model family against autograd of each head's loss, its Hessian
+ * and Gauss-Newton products against float64 double backward resp. autograd's
+ * jvp / vjp around the head's Hessian (tests/test_fc_model.py); the CNN
  * Hessian-vector product against float64 double backward, its symmetry and
  * the second-order Taylor remainder; the input pipeline against numpy
  * pad/slice, flip, transposes and the closed-form normalisation.
@@ -951,6 +953,116 @@ real oracle_nn_gradient(const NN_MODEL *model, const real *weights, const real *
 	}
 	for (int i = 0; i < model->pSize; i++) gradient[i] *= -(1.0 / (real)n);
 	return ll;
+}
+
+/* functions/eval_hessian_vec.cu:20-545 (hessianVec, gaussNewton == 0) and
+ * functions/eval_gauss_newton_hessian_vec.cu:21-361 (gaussNewtonHessianVec, gaussNewton == 1): the R-operator
+ * over an NN_MODEL, given z and dx of oracle_nn_gradient at the same weights and data.
+ *   forward   Rx_{i+1} = VW_i z_i + Vb_i + W_i Rz_i,  Rz_{i+1} = f'(.) Rx_{i+1}; softmax: z.rx - z sum(z.rx)
+ *   head      Rdx_L = -Rz_{L+1}   (logistic and softmax heads; the linear head is refused there, NAN here)
+ *   backward  RdW_i = Rdx_i z_i' [+ dx_i Rz_i'],  Rdb_i = sum(Rdx_i, 2),  Rdz_i = [VW_i' dx_i +] W_i' Rdx_i,
+ *             Rdx_{i-1} = f'(z_i) Rdz_i [+ Rx_i (1 - 2 z_i) dx_{i-1}]   (dev_hessian_helpers.cu:7-26)
+ *   result    -(1/n) [RdW, Rdb]
+ * The bracketed terms are the second-order ones; the Gauss-Newton variant drops them EXCEPT VW' dx of the
+ * top layer (eval_gauss_newton_hessian_vec.cu:262-275 keeps it); topLayerTerm = 0 drops that one too, which
+ * is the textbook Gauss-Newton product and exists here so that tests can pin both.  Hidden tanh layers: the
+ * reference leaves Rdx unset in the backward sweep (:418-420); the derivative is restated here
+ * (f' = 1 - z^2, f'' dz = -2 z dx). */
+int oracle_nn_hessian_vec(const NN_MODEL *model, const real *weights, const real *vec, const real *dataset, int n,
+                          const int *zOffsets, const int *rZOffsets, const real *z, const real *dx, int gaussNewton,
+                          int topLayerTerm, real *result)
+{
+	const int L = model->numLayers;
+	const int *ls = model->layerSizes, *wOff = model->wOffsets, *bOff = model->bOffsets;
+	const int head = model->actFuns[L - 1];
+	if (head != ACT_LOGISTIC && head != ACT_SOFTMAX) return -1;
+	size_t zTotal = 0, widest = 0;
+	for (int i = 0; i <= L; i++) {
+		size_t end = (size_t)zOffsets[i] + (size_t)ls[i] * n;
+		if (end > zTotal) zTotal = end;
+		if ((size_t)ls[i] > widest) widest = ls[i];
+	}
+	real *Rz = (real *)calloc(zTotal, sizeof(real)), *Rx = (real *)calloc(zTotal, sizeof(real));
+	real *Rdz = (real *)calloc(zTotal, sizeof(real));
+	real *Rdx = (real *)calloc(widest * n, sizeof(real));
+	int rc = 0;
+	for (int i = 0; i < L && rc == 0; i++) {
+		const int out = ls[i + 1], in = ls[i];
+		const real *zin = (i == 0) ? dataset : z + zOffsets[i];
+		real *rxi = Rx + zOffsets[i + 1], *rzi = Rz + zOffsets[i + 1];
+		const real *zo = z + zOffsets[i + 1];
+		oracle_gemm(OP_N, OP_N, out, n, in, 1, vec + wOff[i], out, zin, in, 0, rxi, out);
+		for (int c = 0; c < n; c++)
+			for (int r = 0; r < out; r++) rxi[(size_t)c * out + r] += vec[bOff[i] + r];
+		if (i > 0) oracle_gemm(OP_N, OP_N, out, n, in, 1, weights + wOff[i], out, Rz + zOffsets[i], in, 1, rxi, out);
+		const size_t count = (size_t)out * n;
+		switch (model->actFuns[i]) {
+		case ACT_LOGISTIC:
+			for (size_t k = 0; k < count; k++) rzi[k] = rxi[k] * zo[k] * (1.0 - zo[k]);
+			break;
+		case ACT_TANH:
+			for (size_t k = 0; k < count; k++) rzi[k] = rxi[k] * (1.0 + zo[k]) * (1.0 - zo[k]);
+			break;
+		case ACT_LINEAR:
+			memcpy(rzi, rxi, sizeof(real) * count);
+			break;
+		case ACT_SOFTMAX:
+			for (int c = 0; c < n; c++) {
+				real sum = 0;
+				for (int r = 0; r < out; r++) sum += zo[(size_t)c * out + r] * rxi[(size_t)c * out + r];
+				for (int r = 0; r < out; r++) {
+					const size_t k = (size_t)c * out + r;
+					rzi[k] = zo[k] * rxi[k] - zo[k] * sum;
+				}
+			}
+			break;
+		default: rc = -1;
+		}
+	}
+	for (int i = L - 1; i >= 0 && rc == 0; i--) {
+		const int out = ls[i + 1], in = ls[i];
+		const size_t count = (size_t)out * n;
+		const real *dxi = dx + rZOffsets[i];
+		const real *zin = (i == 0) ? dataset : z + zOffsets[i];
+		if (i == L - 1) {
+			for (size_t k = 0; k < count; k++) Rdx[k] = -Rz[zOffsets[L] + k];
+		} else {
+			const real *zo = z + zOffsets[i + 1], *rdz = Rdz + zOffsets[i + 1], *rx = Rx + zOffsets[i + 1];
+			const int second = !gaussNewton;
+			switch (model->actFuns[i]) {
+			case ACT_LOGISTIC:
+				for (size_t k = 0; k < count; k++)
+					Rdx[k] = (1.0 - zo[k]) * zo[k] * rdz[k] + (second ? rx[k] * (1.0 - 2 * zo[k]) * dxi[k] : 0);
+				break;
+			case ACT_TANH:
+				for (size_t k = 0; k < count; k++)
+					Rdx[k] = (1.0 + zo[k]) * (1.0 - zo[k]) * rdz[k] + (second ? rx[k] * (-2.0 * zo[k]) * dxi[k] : 0);
+				break;
+			case ACT_LINEAR:
+				memcpy(Rdx, rdz, sizeof(real) * count);
+				break;
+			default: rc = -1;
+			}
+			if (rc) break;
+		}
+		oracle_gemm(OP_N, OP_T, out, in, n, 1, Rdx, out, zin, in, 0, result + wOff[i], out);
+		if (!gaussNewton && i > 0)
+			oracle_gemm(OP_N, OP_T, out, in, n, 1, dxi, out, Rz + zOffsets[i], in, 1, result + wOff[i], out);
+		for (int r = 0; r < out; r++) {
+			real sum = 0;
+			for (int c = 0; c < n; c++) sum += Rdx[(size_t)c * out + r];
+			result[bOff[i] + r] = sum;
+		}
+		if (i > 0) {
+			real *rdzi = Rdz + zOffsets[i];
+			oracle_gemm(OP_T, OP_N, in, n, out, 1, weights + wOff[i], out, Rdx, out, 0, rdzi, in);
+			const int vwTerm = !gaussNewton || (i == L - 1 && topLayerTerm);
+			if (vwTerm) oracle_gemm(OP_T, OP_N, in, n, out, 1, vec + wOff[i], out, dxi, out, 1, rdzi, in);
+		}
+	}
+	for (int k = 0; k < model->pSize && rc == 0; k++) result[k] *= -(1.0 / (real)n);
+	free(Rz), free(Rx), free(Rdz), free(Rdx);
+	return rc;
 }
 
 /* ------------------------------------------------------------------ */

@@ -226,6 +226,17 @@ class Oracle:
                                          self.p(scratch))
         return float(ll), float(merr.value), grad, z[:model.zSize], dx[:model.rFullSize]
 
+    def nn_hessian_vec(self, model, weights, vec, dataset, n, z, dx, gauss_newton=False, top_layer_term=True):
+        """Hessian (or Gauss-Newton) times vec for an NN_MODEL, from z and dx of nn_gradient at the same point."""
+        weights, vec, dataset, z, dx = (self.arr(a) for a in (weights, vec, dataset, z, dx))
+        out = self.zeros(model.pSize)
+        rc = self.lib.oracle_nn_hessian_vec(C.byref(model), self.p(weights), self.p(vec), self.p(dataset), n, model.zOffsets,
+                                            model.rZOffsets, self.p(z), self.p(dx), int(gauss_newton), int(top_layer_term),
+                                            self.p(out))
+        if rc:
+            raise ValueError("unsupported head or activation")
+        return out
+
     def nn_forward(self, model, weights, dataset, target, n_cols, n_cols_target):
         weights, dataset, target = self.arr(weights), self.arr(dataset), self.arr(target)
         big = max(model.layerSizes[i] for i in range(model.numLayers + 1)) * max(n_cols, n_cols_target)

@@ -95,6 +95,94 @@ def test_oracle_gradient_against_autograd(oracle64, name):
         assert merr == 0
 
 
+def torch_net(m, wt, x, upto=None):
+    """(last pre-activation, last output) of the first `upto` layers (all by default) at the flat parameters wt."""
+    h = torch.tensor(x, dtype=torch.float64)
+    a = None
+    for i in range(m.numLayers if upto is None else upto):
+        out, inn = m.layerSizes[i + 1], m.layerSizes[i]
+        W = wt[m.wOffsets[i]:m.wOffsets[i] + out * inn].reshape(inn, out).t()
+        a = h @ W.t() + wt[m.bOffsets[i]:m.bOffsets[i] + out]
+        h = {ACT_LOGISTIC: torch.sigmoid, ACT_TANH: torch.tanh, ACT_LINEAR: lambda t: t,
+             ACT_SOFTMAX: lambda t: torch.softmax(t, dim=1)}[m.actFuns[i]](a)
+    return a, h
+
+
+def torch_nll(m, wt, x, y):
+    logits, h = torch_net(m, wt, x)
+    yt = torch.tensor(y, dtype=torch.float64)
+    if m.actFuns[m.numLayers - 1] == ACT_LOGISTIC:
+        return -(yt * logits - torch.nn.functional.softplus(logits)).sum() / x.shape[0]
+    return -(yt * torch.log(h)).sum() / x.shape[0]
+
+
+HV_CASES = ["autoencoder_logistic", "classifier_softmax", "one_layer_logistic"]
+
+
+@pytest.mark.parametrize("name", HV_CASES)
+def test_oracle_hessian_vector_product_against_double_backward(oracle64, name):
+    """hessianVec (functions/eval_hessian_vec.cu) is the Hessian of the loss whose gradient computeGradient
+    returns, times the vector: pinned by differentiating autograd's gradient once more."""
+    rng = np.random.default_rng(sum(map(ord, name)) + 1)
+    n = 9
+    m, w, x, y = make_data(name, n, rng)
+    v = rng.standard_normal(m.pSize)
+    _, _, grad, z, dx = oracle64.nn_gradient(m, w, x.reshape(-1), y.reshape(-1), n)
+    got = oracle64.nn_hessian_vec(m, w, v, x.reshape(-1), n, z, dx)
+    wt = torch.tensor(w, dtype=torch.float64, requires_grad=True)
+    g, = torch.autograd.grad(torch_nll(m, wt, x, y), wt, create_graph=True)
+    np.testing.assert_allclose(g.detach().numpy(), grad, atol=1e-12)
+    want, = torch.autograd.grad(g @ torch.tensor(v), wt)
+    np.testing.assert_allclose(got, want.numpy(), atol=1e-11 * max(1, np.abs(want.numpy()).max()))
+    # symmetry of the Hessian: u' H v == v' H u
+    u = rng.standard_normal(m.pSize)
+    hu = oracle64.nn_hessian_vec(m, w, u, x.reshape(-1), n, z, dx)
+    assert abs(u @ got - v @ hu) < 1e-10 * max(1, abs(u @ got))
+
+
+@pytest.mark.parametrize("name", HV_CASES)
+def test_oracle_gauss_newton_product(oracle64, name):
+    """Without the top layer's VW' dx term the product is J' H_L J v (J: logits by parameters, H_L: the head's
+    Hessian in the logits); with it (as eval_gauss_newton_hessian_vec.cu:262-275 has it) the difference is that
+    term back-propagated through the layers below, -(1/n) vjp(z_{L-1}; VW_L' (y - out))."""
+    rng = np.random.default_rng(sum(map(ord, name)) + 2)
+    n = 8
+    m, w, x, y = make_data(name, n, rng)
+    v = rng.standard_normal(m.pSize)
+    _, _, _, z, dx = oracle64.nn_gradient(m, w, x.reshape(-1), y.reshape(-1), n)
+    plain = oracle64.nn_hessian_vec(m, w, v, x.reshape(-1), n, z, dx, gauss_newton=True, top_layer_term=False)
+    as_reference = oracle64.nn_hessian_vec(m, w, v, x.reshape(-1), n, z, dx, gauss_newton=True, top_layer_term=True)
+    wt = torch.tensor(w, dtype=torch.float64, requires_grad=True)
+    logits_of = lambda p: torch_net(m, p, x)[0]
+    logits, ju = torch.autograd.functional.jvp(logits_of, wt, torch.tensor(v))
+    out = torch.sigmoid(logits) if m.actFuns[m.numLayers - 1] == ACT_LOGISTIC else torch.softmax(logits, dim=1)
+    if m.actFuns[m.numLayers - 1] == ACT_LOGISTIC:
+        hju = out * (1 - out) * ju
+    else:
+        hju = out * ju - out * (out * ju).sum(dim=1, keepdim=True)
+    _, want = torch.autograd.functional.vjp(logits_of, wt, hju / n)
+    np.testing.assert_allclose(plain, want.numpy(), atol=1e-11 * max(1, np.abs(want.numpy()).max()))
+    # positive semi-definite
+    assert v @ plain > -1e-12
+    nl = m.numLayers
+    if nl == 1:
+        np.testing.assert_array_equal(as_reference, plain)
+        return
+    o, i = m.layerSizes[nl], m.layerSizes[nl - 1]
+    VW = torch.tensor(v[m.wOffsets[nl - 1]:m.wOffsets[nl - 1] + o * i]).reshape(i, o).t()
+    cot = (torch.tensor(y) - out) @ VW                               # n x in: (VW' dx)' per point
+    _, extra = torch.autograd.functional.vjp(lambda p: torch_net(m, p, x, upto=nl - 1)[1], wt, cot)
+    np.testing.assert_allclose(as_reference - plain, -extra.numpy() / n, atol=1e-11 * max(1, np.abs(extra.numpy()).max()))
+    assert np.abs(as_reference - plain).max() > 1e-6                 # the term is there
+
+
+def test_oracle_hessian_vector_refuses_the_linear_head(oracle64):
+    m, w, x, y = make_data("regression_linear", 5, np.random.default_rng(0))
+    _, _, _, z, dx = oracle64.nn_gradient(m, w, x.reshape(-1), y.reshape(-1), 5)
+    with pytest.raises(ValueError):
+        oracle64.nn_hessian_vec(m, w, w, x.reshape(-1), 5, z, dx)
+
+
 def test_oracle_offsets_follow_the_reference_arithmetic(oracle64):
     m = build_nn([5, 4, 3], [ACT_LOGISTIC, ACT_LINEAR], MODEL_TYPE_MSE, 10)
     assert (m.wOffsets[0], m.bOffsets[0], m.wOffsets[1], m.bOffsets[1], m.pSize) == (0, 20, 24, 36, 39)
@@ -180,3 +268,84 @@ def test_gpu_apply_layer_activation_keeps_the_pre_activation_copy(dev, oracle64)
     want = np.exp(pre) / np.exp(pre).sum(1, keepdims=True)
     assert rel_err(got[:rows * n].reshape(n, rows), want) < 1e-5
     assert rel_err(got[rows * n:].reshape(n, rows), pre) < 1e-5
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", HV_CASES)
+@pytest.mark.parametrize("n", [11, 300])
+def test_gpu_hessian_vector_products_against_oracle(dev, oracle64, name, n):
+    """hessianVec and gaussNewtonHessianVec after computeGradient at the same point, result at the head of the arena."""
+    rng = np.random.default_rng(sum(map(ord, name)) + 7 * n)
+    m, w, x, y = make_data(name, n, rng)
+    w32, x32, y32 = w.astype(np.float32), x.astype(np.float32), y.astype(np.float32)
+    v32 = rng.standard_normal(m.pSize).astype(np.float32)
+    data, scratch, pw = device_setup(dev, m, w32, x32, y32, n)
+    z, dx, grad, pv = dev.zeros(m.zSize), dev.zeros(m.rFullSize), dev.zeros(m.pSize), dev.upload(v32)
+    ll, merr = C.c_float(), C.c_float()
+    L.cnn.computeGradient(C.byref(m), C.byref(data), C.byref(scratch), pw, z, dx, grad, C.byref(ll), C.byref(merr), FULL_DATASET)
+    need = L.cnn.nnHessianVecMemRequired(C.byref(m), C.byref(data), FULL_DATASET)
+    arena = dev.upload(np.full(need, np.nan, np.float32))          # nothing may rely on a cleared arena
+    hv_scratch = SCRATCH_AREA()
+    hv_scratch.devWorkspace = hv_scratch.nextDevPtr = arena.value
+    _, _, _, oz, odx = oracle64.nn_gradient(m, w32, x32.reshape(-1), y32.reshape(-1), n)
+    L.cnn.hessianVec(C.byref(m), C.byref(data), z, dx, pv, pw, C.byref(hv_scratch), FULL_DATASET)
+    want = oracle64.nn_hessian_vec(m, w32, v32, x32.reshape(-1), n, oz, odx)
+    assert rel_err(dev.download(arena, m.pSize), want) < TOL
+    L.cnn.gaussNewtonHessianVec(C.byref(m), C.byref(data), z, dx, pv, pw, C.byref(hv_scratch), FULL_DATASET)
+    want = oracle64.nn_hessian_vec(m, w32, v32, x32.reshape(-1), n, oz, odx, gauss_newton=True)
+    assert rel_err(dev.download(arena, m.pSize), want) < TOL
+    for q in (z, dx, grad, pv, arena):
+        dev.free(q)
+
+
+@pytest.mark.gpu
+def test_gpu_hessian_vector_product_on_the_sampled_set(dev, oracle64):
+    name, n = "autoencoder_logistic", 64
+    rng = np.random.default_rng(13)
+    m, w, _, _ = make_data(name, n, rng)
+    x = rng.random((n, m.layerSizes[0]))
+    w32, x32 = w.astype(np.float32), x.astype(np.float32)
+    v32 = rng.standard_normal(m.pSize).astype(np.float32)
+    data, scratch, pw = device_setup(dev, m, w32, x32, x32, n, sampled=True)
+    z, dx, grad, pv = dev.zeros(m.sampledZSize), dev.zeros(m.sampledRSize), dev.zeros(m.pSize), dev.upload(v32)
+    ll, merr = C.c_float(), C.c_float()
+    L.cnn.computeGradient(C.byref(m), C.byref(data), C.byref(scratch), pw, z, dx, grad, C.byref(ll), C.byref(merr), SAMPLED_DATASET)
+    need = L.cnn.nnHessianVecMemRequired(C.byref(m), C.byref(data), SAMPLED_DATASET)
+    arena = dev.upload(np.full(need, np.nan, np.float32))
+    hv_scratch = SCRATCH_AREA()
+    hv_scratch.devWorkspace = hv_scratch.nextDevPtr = arena.value
+    L.cnn.hessianVec(C.byref(m), C.byref(data), z, dx, pv, pw, C.byref(hv_scratch), SAMPLED_DATASET)
+    _, _, _, oz, odx = oracle64.nn_gradient(m, w32, x32.reshape(-1), x32.reshape(-1), n)
+    want = oracle64.nn_hessian_vec(m, w32, v32, x32.reshape(-1), n, oz, odx)
+    assert rel_err(dev.download(arena, m.pSize), want) < TOL
+    for q in (z, dx, grad, pv, arena):
+        dev.free(q)
+
+
+@pytest.mark.gpu
+def test_gpu_rop_pieces_against_their_formulas(dev):
+    rng = np.random.default_rng(21)
+    n = 5000
+    z = rng.random(n).astype(np.float32) * 1.8 - 0.9
+    rdz, rx, dxv = (rng.standard_normal(n).astype(np.float32) for _ in range(3))
+    pz, prdz, prx, pdx, out = dev.upload(z), dev.upload(rdz), dev.upload(rx), dev.upload(dxv), dev.zeros(n)
+    z64, rdz64, rx64, dx64 = (a.astype(np.float64) for a in (z, rdz, rx, dxv))
+    forms = {ACT_LOGISTIC: ((1 - z64) * z64, 1 - 2 * z64), ACT_TANH: ((1 + z64) * (1 - z64), -2 * z64),
+             ACT_LINEAR: (np.ones(n), np.zeros(n))}
+    for act, (f1, g) in forms.items():
+        L.check(L.hip.fitre_hip_fc_rop_backward(act, pz, prdz, prx, pdx, out, n))
+        np.testing.assert_allclose(dev.download(out, n), f1 * rdz64 + rx64 * g * dx64, rtol=0, atol=2e-6)
+        L.check(L.hip.fitre_hip_fc_rop_backward(act, pz, prdz, None, None, out, n))
+        np.testing.assert_allclose(dev.download(out, n), f1 * rdz64, rtol=0, atol=1e-6)
+    assert L.hip.fitre_hip_fc_rop_backward(ACT_SOFTMAX, pz, prdz, prx, pdx, out, n) != 0      # not an element-wise activation
+    rows, cols = 7, 300
+    logits = rng.standard_normal((cols, rows))
+    p = np.exp(logits) / np.exp(logits).sum(axis=1, keepdims=True)
+    r = rng.standard_normal((cols, rows))
+    pp, pr, po = dev.upload(p.reshape(-1)), dev.upload(r.reshape(-1)), dev.zeros(rows * cols)
+    L.check(L.hip.fitre_hip_column_softmax_rop(pp, pr, rows, cols, po))
+    want = p * r - p * (p * r).sum(axis=1, keepdims=True)
+    np.testing.assert_allclose(dev.download(po, rows * cols).reshape(cols, rows), want, rtol=0, atol=1e-6)
+    assert abs(dev.download(po, rows * cols).reshape(cols, rows).sum(axis=1)).max() < 1e-6    # the directions sum to zero
+    for q in (pz, prdz, prx, pdx, out, pp, pr, po):
+        dev.free(q)
