@@ -176,6 +176,25 @@ def test_oracle_gauss_newton_product(oracle64, name):
     assert np.abs(as_reference - plain).max() > 1e-6                 # the term is there
 
 
+@pytest.mark.parametrize("name", HV_CASES)
+def test_oracle_second_order_taylor_remainder(oracle64, name):
+    """utilities/derivative_test.cu:150-199 for this family: f(w + e v) - f(w) - e g'v - e^2/2 v'Hv shrinks like e^3."""
+    rng = np.random.default_rng(sum(map(ord, name)) + 3)
+    n = 10
+    m, w, x, y = make_data(name, n, rng)
+    v = rng.standard_normal(m.pSize)
+    v /= np.linalg.norm(v)
+    f0, _, g, z, dx = oracle64.nn_gradient(m, w, x.reshape(-1), y.reshape(-1), n)
+    hv = oracle64.nn_hessian_vec(m, w, v, x.reshape(-1), n, z, dx)
+    rem = []
+    for e in (1e-1, 5e-2, 2.5e-2):
+        f1 = oracle64.nn_forward(m, w + e * v, x.reshape(-1), y.reshape(-1), n, n)[0]
+        rem.append(abs(f1 - f0 - e * (g @ v) - 0.5 * e * e * (v @ hv)))
+    assert rem[0] > 1e-9                                # not trivially zero
+    for a, b in zip(rem, rem[1:]):
+        assert 6.0 < a / b < 10.5, rem                  # halving e divides the remainder by about 8
+
+
 def test_oracle_hessian_vector_refuses_the_linear_head(oracle64):
     m, w, x, y = make_data("regression_linear", 5, np.random.default_rng(0))
     _, _, _, z, dx = oracle64.nn_gradient(m, w, x.reshape(-1), y.reshape(-1), 5)
