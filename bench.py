@@ -134,8 +134,8 @@ def gpu_leg(args):
     finite = bool(np.isfinite(grad).all() and np.isfinite(loss))
     kfac, bandwidth, others = None, None, None
     if not args.headline_only:
-        kfac = kfac_leg(L, dev, gm, model, batch, max(2, args.steps // 4))
-        kfac["hessian_vector_ms"] = hv_leg(L, dev, gm, model, batch, max(2, args.steps // 4))
+        kfac = kfac_leg(L, dev, gm, model, batch, min(10, max(2, args.steps // 4)))
+        kfac["hessian_vector_ms"] = hv_leg(L, dev, gm, model, batch, min(10, max(2, args.steps // 4)))
         kfac["trust_region_step_ms"] = kfac_step_leg(L, dev, gm, model, batch, 3)
     gm.release()
     if not args.headline_only:
@@ -426,8 +426,8 @@ def torch_leg(batch=32, repeats=3):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--serial", action="store_true",
                     help="run every kernel on one stream (for kernel tracers: durations do not overlap)")
