@@ -212,28 +212,37 @@ static void set_fc(CNN_MODEL *model, int l, int in, int out, int act, int batchS
 	model->fcLayer[l].offset = batchSize * out;
 }
 
-void fitre_build_vgg11(CNN_MODEL *model, int batchSize, int height, int width, int inChannels,
-                       int numClasses, int bias, int enableBatchNorm, int convAct)
+/* The VGG family of nn/read_vgg.c: 3x3 / pad 1 convolutions of the given widths, max pool 2 after the marked
+ * ones, one linear layer on the flattened features. */
+static void build_vgg(CNN_MODEL *model, int name, const int *channels, const int *pooled, int count, int batchSize,
+                      int height, int width, int inChannels, int numClasses, int bias, int enableBatchNorm, int convAct)
 {
-	static const int channels[8] = { 64, 128, 256, 256, 512, 512, 512, 512 };
-	static const int pooled[8] = { 1, 1, 0, 1, 0, 1, 0, 1 };
 	BATCH_NORM_TYPES bn = enableBatchNorm ? PERFORM_BATCH_NORM : PERFORM_NO_BATCH_NORM;
 
 	memset(model, 0, sizeof(*model));
 	model->enableBatchNorm = enableBatchNorm;
 	int h = height, w = width, cin = inChannels;
-	for (int l = 0; l < 8; l++) {
+	for (int l = 0; l < count; l++) {
 		model->actFuns[l] = convAct;
-		makeLayer(&model->convLayer[l], &model->poolLayer[l], pooled[l] ? MAX_POOL : NO_POOL, cin,
-		          channels[l], h, w, &h, &w, batchSize, bn);
+		makeLayer(&model->convLayer[l], &model->poolLayer[l], pooled[l] ? MAX_POOL : NO_POOL, cin, channels[l], h, w, &h, &w,
+		          batchSize, bn);
 		cin = channels[l];
 	}
-	model->cLayers = 8;
+	model->cLayers = count;
 	set_fc(model, 0, cin * h * w, numClasses, CNN_ACT_NONE, batchSize);
 	model->lLayers = 1;
 	model->bias = bias;
-	model->name = CNN_VGG11NET;
+	model->name = name;
 	fitre_finalize_model(model, height, width, batchSize);
+}
+
+void fitre_build_vgg11(CNN_MODEL *model, int batchSize, int height, int width, int inChannels,
+                       int numClasses, int bias, int enableBatchNorm, int convAct)
+{
+	static const int channels[8] = { 64, 128, 256, 256, 512, 512, 512, 512 };
+	static const int pooled[8] = { 1, 1, 0, 1, 0, 1, 0, 1 };
+	build_vgg(model, CNN_VGG11NET, channels, pooled, 8, batchSize, height, width, inChannels, numClasses, bias, enableBatchNorm,
+	          convAct);
 }
 
 void readVGG11(CNN_MODEL *model, int batchSize, int height, int width, int numClasses, int inChannels,
@@ -242,6 +251,37 @@ void readVGG11(CNN_MODEL *model, int batchSize, int height, int width, int numCl
 	(void)datasetType; /* FC fan-in follows from the image size: 512 at 32x32, 2048 at 64x64 */
 	fitre_build_vgg11(model, batchSize, height, width, inChannels, numClasses, bias, enableBatchNorm,
 	                  CNN_ACT_SWISH);
+}
+
+/* nn/read_vgg.c:345-424, :486-579, :642-750: the deeper members, swish after every convolution as there */
+void readVGG13(CNN_MODEL *model, int batchSize, int height, int width, int numClasses, int inChannels, int bias,
+               int enableBatchNorm, DATASET_TYPE datasetType)
+{
+	static const int channels[10] = { 64, 64, 128, 128, 256, 256, 512, 512, 512, 512 };
+	static const int pooled[10] = { 0, 1, 0, 1, 0, 1, 0, 1, 0, 1 };
+	(void)datasetType;
+	build_vgg(model, CNN_VGG13NET, channels, pooled, 10, batchSize, height, width, inChannels, numClasses, bias, enableBatchNorm,
+	          CNN_ACT_SWISH);
+}
+
+void readVGG16(CNN_MODEL *model, int batchSize, int height, int width, int numClasses, int inChannels, int bias,
+               int enableBatchNorm, DATASET_TYPE datasetType)
+{
+	static const int channels[13] = { 64, 64, 128, 128, 256, 256, 256, 512, 512, 512, 512, 512, 512 };
+	static const int pooled[13] = { 0, 1, 0, 1, 0, 0, 1, 0, 0, 1, 0, 0, 1 };
+	(void)datasetType;
+	build_vgg(model, CNN_VGG16NET, channels, pooled, 13, batchSize, height, width, inChannels, numClasses, bias, enableBatchNorm,
+	          CNN_ACT_SWISH);
+}
+
+void readVGG19(CNN_MODEL *model, int batchSize, int height, int width, int numClasses, int inChannels, int bias,
+               int enableBatchNorm, DATASET_TYPE datasetType)
+{
+	static const int channels[16] = { 64, 64, 128, 128, 256, 256, 256, 256, 512, 512, 512, 512, 512, 512, 512, 512 };
+	static const int pooled[16] = { 0, 1, 0, 1, 0, 0, 0, 1, 0, 0, 0, 1, 0, 0, 0, 1 };
+	(void)datasetType;
+	build_vgg(model, CNN_VGG19NET, channels, pooled, 16, batchSize, height, width, inChannels, numClasses, bias, enableBatchNorm,
+	          CNN_ACT_SWISH);
 }
 
 void fitre_build_lenet(CNN_MODEL *model, int batchSize, int height, int width, int inChannels,

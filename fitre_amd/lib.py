@@ -136,6 +136,9 @@ CNN_API = {
     "computeZOffsets": (None, [pmodel, i32, i32, i32]),
     "makeLayer": (None, [pconv, ppool, i32, i32, i32, i32, i32, pi32, pi32, i32, i32]),
     "readVGG11": (None, [pmodel, i32, i32, i32, i32, i32, i32, i32, i32]),
+    "readVGG13": (None, [pmodel, i32, i32, i32, i32, i32, i32, i32, i32]),
+    "readVGG16": (None, [pmodel, i32, i32, i32, i32, i32, i32, i32, i32]),
+    "readVGG19": (None, [pmodel, i32, i32, i32, i32, i32, i32, i32, i32]),
     "fitre_make_conv_layer": (None, [pconv, ppool] + [i32] * 13 + [pi32, pi32]),
     "fitre_finalize_model": (None, [pmodel, i32, i32, i32]),
     "fitre_build_lenet": (None, [pmodel] + [i32] * 9),

@@ -40,6 +40,13 @@ void makeLayer(CONV_LAYER *conv, POOL_LAYER *pool, POOL_TYPE poolFun, int inChan
 /* VGG-11 as the reference builds it (swish; nn/read_vgg.c:216-300). */
 void readVGG11(CNN_MODEL *model, int batchSize, int height, int width, int numClasses, int inChannels,
                int bias, int enableBatchNorm, DATASET_TYPE datasetType);
+/* nn/read_vgg.h:10-12: 10, 13 and 16 convolutions (64,64,M,128,128,M,256,256[,256[,256]],M,512,...), same arguments */
+void readVGG13(CNN_MODEL *model, int batchSize, int height, int width, int numClasses, int inChannels, int bias,
+               int enableBatchNorm, DATASET_TYPE datasetType);
+void readVGG16(CNN_MODEL *model, int batchSize, int height, int width, int numClasses, int inChannels, int bias,
+               int enableBatchNorm, DATASET_TYPE datasetType);
+void readVGG19(CNN_MODEL *model, int batchSize, int height, int width, int numClasses, int inChannels, int bias,
+               int enableBatchNorm, DATASET_TYPE datasetType);
 
 /* ---- builders that have no counterpart in the reference: the same slab
  * scheme as makeLayer for arbitrary kernel / stride / padding / pooling ---- */

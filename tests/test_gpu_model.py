@@ -108,6 +108,18 @@ def test_vgg11_swish_reference_network(dev, oracle64):
     compare_with_oracle(dev, oracle64, build_vgg11(8, bn=True, act=CNN_ACT_SWISH, bias=0), 8, seed=14)
 
 
+@pytest.mark.parametrize("reader,convs", [("readVGG13", 10), ("readVGG16", 13), ("readVGG19", 16)])
+def test_deeper_vgg_members_as_the_reference_builds_them(dev, oracle64, reader, convs):
+    """nn/read_vgg.c:345-750: swish after every convolution, batch norm, bias; forward, loss and gradient against the oracle."""
+    import ctypes as C
+    from fitre_amd import lib as L
+    from fitre_amd.structs import CNN_MODEL
+    model = CNN_MODEL()
+    getattr(L.cnn, reader)(C.byref(model), 6, 32, 32, 10, 3, 1, 1, 10)
+    assert model.cLayers == convs and model.lLayers == 1 and model.fcLayer[0].in_ == 512
+    compare_with_oracle(dev, oracle64, model, 6, seed=30 + convs)
+
+
 def test_alexnet_reduced(dev, oracle64):
     # AlexNet layer types at a reduced image (67 -> 16 -> 7 -> 3 -> 1): 11x11/s4/p2, 5x5/p2, 3x3, maxpool 3/2
     compare_with_oracle(dev, oracle64, build_alexnet(4, classes=50, size=67), 4, seed=15)

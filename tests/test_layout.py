@@ -175,3 +175,22 @@ def test_vector_text_io_round_trip(tmp_path):
     back = np.zeros(4, dtype=np.float32)
     assert L.cnn.readVector(back.ctypes.data_as(C.c_void_p), 4, out, 0, None) == 4
     np.testing.assert_allclose(back, src, atol=1e-10)
+
+
+def test_vgg_family_parameter_counts():
+    """readVGG11/13/16/19 (nn/read_vgg.c): the convolution stacks are the standard ones, whose parameter counts are
+    known (9 220 480, 9 404 992, 14 714 688 and 20 024 384 with biases), plus the 512 -> 10 linear layer."""
+    from fitre_amd.structs import CNN_MODEL
+    known = {"readVGG11": (8, 9220480, 2), "readVGG13": (10, 9404992, 3), "readVGG16": (13, 14714688, 4),
+             "readVGG19": (16, 20024384, 5)}
+    for reader, (convs, conv_params, name) in known.items():
+        m = CNN_MODEL()
+        getattr(L.cnn, reader)(C.byref(m), 32, 32, 32, 10, 3, 1, 1, 10)
+        assert (m.cLayers, m.lLayers, m.name, m.bias, m.enableBatchNorm) == (convs, 1, name, 1, 1)
+        assert m.pSize == conv_params + 512 * 10 + 10
+        assert all(m.actFuns[i] == 14 for i in range(convs))                      # swish
+        assert sum(1 for i in range(convs) if m.poolLayer[i].type != 2) == 5      # five max pools: 32 -> 1
+        assert m.poolLayer[convs - 1].outHeight == 1 and m.fcLayer[0].in_ == 512
+        m64 = CNN_MODEL()
+        getattr(L.cnn, reader)(C.byref(m64), 8, 64, 64, 200, 3, 0, 0, 30)
+        assert m64.fcLayer[0].in_ == 2048 and m64.bias == 0                       # 64 x 64 images: 512 * 4 features
