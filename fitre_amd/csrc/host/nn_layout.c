@@ -334,3 +334,52 @@ void fitre_build_alexnet(CNN_MODEL *model, int batchSize, int height, int width,
 	model->name = CNN_ALEXNET;
 	fitre_finalize_model(model, height, width, batchSize);
 }
+
+/* nn/read_nn.c:500-700: the reference's LeNet -- 5x5 convolutions of 6 and 16 channels, each with swish and a
+ * 2 / 2 AVERAGE pool, linear layers 120, 84 (swish) and 10.  (width before height, as there.)  With batch norm on,
+ * the slab of a layer is laid out as makeLayer does for the VGG family; the reference's own offsets for this
+ * network place the normalisation behind the pool, which its forward pass does not follow. */
+void readLenetCNN(CNN_MODEL *model, int channels, int width, int height, int batchSize, int enableBias, int enableBatchNorm)
+{
+	BATCH_NORM_TYPES bn = enableBatchNorm ? PERFORM_BATCH_NORM : PERFORM_NO_BATCH_NORM;
+	memset(model, 0, sizeof(*model));
+	model->enableBatchNorm = enableBatchNorm;
+	int h = height, w = width;
+	model->actFuns[0] = CNN_ACT_SWISH;
+	fitre_make_conv_layer(&model->convLayer[0], &model->poolLayer[0], channels, 6, h, w, 5, 1, 0, AVG_POOL, 2, 2, 0, batchSize, bn,
+	                      &h, &w);
+	model->actFuns[1] = CNN_ACT_SWISH;
+	fitre_make_conv_layer(&model->convLayer[1], &model->poolLayer[1], 6, 16, h, w, 5, 1, 0, AVG_POOL, 2, 2, 0, batchSize, bn, &h, &w);
+	model->cLayers = 2;
+	set_fc(model, 0, 16 * h * w, 120, CNN_ACT_SWISH, batchSize);
+	set_fc(model, 1, 120, 84, CNN_ACT_SWISH, batchSize);
+	set_fc(model, 2, 84, 10, CNN_ACT_NONE, batchSize);
+	model->lLayers = 3;
+	model->bias = enableBias;
+	model->name = CNN_LENET;
+	fitre_finalize_model(model, height, width, batchSize);
+}
+
+/* nn/read_alexnet.c:14-215: the reference's CIFAR-sized "AlexNet" -- two 5x5 / pad 2 convolutions of 64 channels,
+ * each with swish and a 3 / 2 / 1 max pool, linear layers 384, 192 (swish) and numClasses. */
+void readAlexNetCNN(CNN_MODEL *model, int batchSize, int height, int width, int numClasses, int enableBias, int enableBatchNorm)
+{
+	BATCH_NORM_TYPES bn = enableBatchNorm ? PERFORM_BATCH_NORM : PERFORM_NO_BATCH_NORM;
+	memset(model, 0, sizeof(*model));
+	model->enableBatchNorm = enableBatchNorm;
+	int h = height, w = width, cin = 3;
+	for (int l = 0; l < 2; l++) {
+		model->actFuns[l] = CNN_ACT_SWISH;
+		fitre_make_conv_layer(&model->convLayer[l], &model->poolLayer[l], cin, 64, h, w, 5, 1, 2, MAX_POOL, 3, 2, 1, batchSize, bn,
+		                      &h, &w);
+		cin = 64;
+	}
+	model->cLayers = 2;
+	set_fc(model, 0, 64 * h * w, 384, CNN_ACT_SWISH, batchSize);
+	set_fc(model, 1, 384, 192, CNN_ACT_SWISH, batchSize);
+	set_fc(model, 2, 192, numClasses, CNN_ACT_NONE, batchSize);
+	model->lLayers = 3;
+	model->bias = enableBias;
+	model->name = CNN_ALEXNET;
+	fitre_finalize_model(model, height, width, batchSize);
+}

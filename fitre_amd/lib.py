@@ -136,6 +136,8 @@ CNN_API = {
     "computeZOffsets": (None, [pmodel, i32, i32, i32]),
     "makeLayer": (None, [pconv, ppool, i32, i32, i32, i32, i32, pi32, pi32, i32, i32]),
     "readVGG11": (None, [pmodel, i32, i32, i32, i32, i32, i32, i32, i32]),
+    "readLenetCNN": (None, [pmodel, i32, i32, i32, i32, i32, i32]),
+    "readAlexNetCNN": (None, [pmodel, i32, i32, i32, i32, i32, i32]),
     "readVGG13": (None, [pmodel, i32, i32, i32, i32, i32, i32, i32, i32]),
     "readVGG16": (None, [pmodel, i32, i32, i32, i32, i32, i32, i32, i32]),
     "readVGG19": (None, [pmodel, i32, i32, i32, i32, i32, i32, i32, i32]),

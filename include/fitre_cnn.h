@@ -40,6 +40,12 @@ void makeLayer(CONV_LAYER *conv, POOL_LAYER *pool, POOL_TYPE poolFun, int inChan
 /* VGG-11 as the reference builds it (swish; nn/read_vgg.c:216-300). */
 void readVGG11(CNN_MODEL *model, int batchSize, int height, int width, int numClasses, int inChannels,
                int bias, int enableBatchNorm, DATASET_TYPE datasetType);
+/* nn/read_nn.h:18-19 and nn/read_alexnet.h:7-8: the reference's two small networks as it builds them -- LeNet with
+ * swish and 2 / 2 average pools (6 and 16 channels; linear 120, 84, 10), and its CIFAR-sized "AlexNet" (two 5x5 / pad 2
+ * convolutions of 64 channels with 3 / 2 / 1 max pools; linear 384, 192, numClasses).  fitre_build_lenet /
+ * fitre_build_alexnet below take activations and pooling as arguments (the latter is the five-convolution network). */
+void readLenetCNN(CNN_MODEL *model, int channels, int width, int height, int batchSize, int enableBias, int enableBatchNorm);
+void readAlexNetCNN(CNN_MODEL *model, int batchSize, int height, int width, int numClasses, int enableBias, int enableBatchNorm);
 /* nn/read_vgg.h:10-12: 10, 13 and 16 convolutions (64,64,M,128,128,M,256,256[,256[,256]],M,512,...), same arguments */
 void readVGG13(CNN_MODEL *model, int batchSize, int height, int width, int numClasses, int inChannels, int bias,
                int enableBatchNorm, DATASET_TYPE datasetType);

@@ -4,7 +4,7 @@
  * departure: the device arena is sized with kfacTrustRegionMemRequired instead of taking all free memory
  * (cuda_allocate_workspace, which is there too).
  *
- *   kfac_driver <dataset 1|2|3> <network 1|3> <epochs> <dampGamma> <maxRadius> <inverseFreq> <regLambda>
+ *   kfac_driver <dataset 1|2|3> <network 1|2|3> <epochs> <dampGamma> <maxRadius> <inverseFreq> <regLambda>
  *               <initialization 0|1|2> <dataset folder> <weights folder>
  *
  * Without arguments it prints this usage and exits with status 2 before anything touches a device.
@@ -50,7 +50,8 @@ int main(int argc, char **argv)
 	default: fprintf(stderr, " Unknown dataset parameter: %d \n", dataset); return 1;
 	}
 	switch (network) {
-	case 1: fitre_build_lenet(&model, batch, deviceData.height, deviceData.width, 3, deviceData.numClasses, 1, 1, CNN_ACT_SWISH, CNN_ACT_SWISH); break;
+	case 1: readLenetCNN(&model, 3, deviceData.width, deviceData.height, batch, 1, 1); break;
+	case 2: readAlexNetCNN(&model, batch, deviceData.height, deviceData.width, deviceData.numClasses, 1, 1); break;
 	case 3: readVGG11(&model, batch, deviceData.height, deviceData.width, deviceData.numClasses, 3, 1, 1, hostData.datasetType); break;
 	default: fprintf(stderr, "Unknown NETWORK Name: %d \n", network); return 1;
 	}

@@ -120,6 +120,21 @@ def test_deeper_vgg_members_as_the_reference_builds_them(dev, oracle64, reader, 
     compare_with_oracle(dev, oracle64, model, 6, seed=30 + convs)
 
 
+@pytest.mark.parametrize("which,bn", [("lenet", 0), ("lenet", 1), ("alexnet", 0), ("alexnet", 1)])
+def test_small_reference_networks_as_the_reference_builds_them(dev, oracle64, which, bn):
+    """readLenetCNN (swish, average pools) and readAlexNetCNN (5x5 / pad 2, 3 / 2 / 1 max pools), nn/read_nn.c:500-700,
+    nn/read_alexnet.c:14-215."""
+    import ctypes as C
+    from fitre_amd import lib as L
+    from fitre_amd.structs import CNN_MODEL
+    model = CNN_MODEL()
+    if which == "lenet":
+        L.cnn.readLenetCNN(C.byref(model), 3, 32, 32, 12, 1, bn)
+    else:
+        L.cnn.readAlexNetCNN(C.byref(model), 12, 32, 32, 10, 1, bn)
+    compare_with_oracle(dev, oracle64, model, 12, seed=40 + bn)
+
+
 def test_alexnet_reduced(dev, oracle64):
     # AlexNet layer types at a reduced image (67 -> 16 -> 7 -> 3 -> 1): 11x11/s4/p2, 5x5/p2, 3x3, maxpool 3/2
     compare_with_oracle(dev, oracle64, build_alexnet(4, classes=50, size=67), 4, seed=15)

@@ -194,3 +194,21 @@ def test_vgg_family_parameter_counts():
         m64 = CNN_MODEL()
         getattr(L.cnn, reader)(C.byref(m64), 8, 64, 64, 200, 3, 0, 0, 30)
         assert m64.fcLayer[0].in_ == 2048 and m64.bias == 0                       # 64 x 64 images: 512 * 4 features
+
+
+def test_small_reference_networks():
+    """readLenetCNN (nn/read_nn.c:500-700) and readAlexNetCNN (nn/read_alexnet.c:14-215): layer shapes as written there."""
+    from fitre_amd.structs import CNN_MODEL
+    m = CNN_MODEL()
+    L.cnn.readLenetCNN(C.byref(m), 3, 32, 32, 64, 1, 0)
+    assert (m.cLayers, m.lLayers, m.name, m.pSize) == (2, 3, 0, 62006)
+    assert [m.poolLayer[i].type for i in range(2)] == [1, 1] and [m.actFuns[i] for i in range(2)] == [14, 14]   # average pool, swish
+    assert (m.fcLayer[0].in_, m.fcLayer[0].out, m.fcLayer[1].out, m.fcLayer[2].out) == (400, 120, 84, 10)
+    assert (m.fcLayer[0].actFun, m.fcLayer[1].actFun, m.fcLayer[2].actFun) == (14, 14, 10)          # swish, swish, none
+    a = CNN_MODEL()
+    L.cnn.readAlexNetCNN(C.byref(a), 32, 32, 32, 10, 1, 1)
+    assert (a.cLayers, a.lLayers, a.name) == (2, 3, 1)
+    assert [(a.convLayer[i].kSize, a.convLayer[i].padding, a.convLayer[i].outChannels) for i in range(2)] == [(5, 2, 64)] * 2
+    assert [(a.poolLayer[i].pSize, a.poolLayer[i].stride, a.poolLayer[i].padding, a.poolLayer[i].type) for i in range(2)] == [(3, 2, 1, 0)] * 2
+    assert (a.poolLayer[0].outHeight, a.poolLayer[1].outHeight, a.fcLayer[0].in_) == (16, 8, 64 * 8 * 8)
+    assert a.pSize == 4864 + 102464 + 1573248 + 73920 + 1930
