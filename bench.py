@@ -1,7 +1,9 @@
 #!/usr/bin/env python3
 """Benchmark of the CNN backward pass on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--serial] [--headline-only]
+
+Defaults: 20 warm-up and 100 timed passes (a shorter region ends while the clocks are still ramping).
 
 Workload: VGG-11-style network, fp32, batch 256, 3x32x32 N(0,1) inputs, 10 uniform classes, eight
 3x3/pad-1 convolutions (64,128,256,256,512,512,512,512) each with non-affine batch norm and ReLU,
