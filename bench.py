@@ -35,7 +35,6 @@ import numpy as np
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
-sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 PEAK_MFMA_F32_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
@@ -73,7 +72,7 @@ def read_profile(L):
 
 def gpu_leg(args):
     from fitre_amd import lib as L
-    from helpers import Device, GpuModel, at, batch_inputs, build_vgg11, he_weights
+    from fitre_amd.harness import Device, GpuModel, at, batch_inputs, build_vgg11, he_weights
 
     batch = 256
     dev = Device(0)
@@ -180,7 +179,7 @@ def other_configs_leg(L, dev, steps=10):
     """Backward images/sec of the other benchmark networks (the same step: copy of the loss errors + one
     cnnBackward), for orientation: LeNet-style b128, the same with batch norm b1024, AlexNet-style
     3x224x224 b64 with 1000 classes."""
-    from helpers import GpuModel, batch_inputs, build_alexnet, build_lenet, he_weights
+    from fitre_amd.harness import GpuModel, batch_inputs, build_alexnet, build_lenet, he_weights
     out = {}
     for name, build, batch in (("lenet_b128", lambda: build_lenet(128), 128),
                                ("lenet_bn_b1024", lambda: build_lenet(1024, bn=True), 1024),
@@ -388,7 +387,7 @@ def kfac_step_leg(L, dev, gm, model, batch, repeats):
 def cpu_leg(batch=64, repeats=10):
     """float32 build of the oracle (the reference's algorithm restated in C, OpenMP over the host
     cores): one forward, then `repeats` backward passes on the same network at a smaller batch."""
-    from helpers import batch_inputs, build_vgg11, he_weights
+    from fitre_amd.harness import batch_inputs, build_vgg11, he_weights
     from oracle.oracle import Oracle
 
     o = Oracle(double=False)
@@ -409,8 +408,8 @@ def cpu_leg(batch=64, repeats=10):
 
 def torch_leg(batch=32, repeats=3):
     import torch
-    import torchref
-    from helpers import batch_inputs, build_vgg11, he_weights
+    from oracle import torchref
+    from fitre_amd.harness import batch_inputs, build_vgg11, he_weights
 
     model = build_vgg11(batch, bn=True)
     rng = np.random.default_rng(1)

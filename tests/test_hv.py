@@ -5,7 +5,7 @@ import ctypes as C
 import numpy as np
 import pytest
 
-import torchref
+from oracle import torchref
 from fitre_amd.structs import (ACT_TANH, AVG_POOL, CNN_ACT_NONE, CNN_ACT_RELU, CNN_ACT_SOFTPLUS, CNN_ACT_SWISH, MAX_POOL)
 from helpers import batch_inputs, build_custom, he_weights, rel_err
 

@@ -3,7 +3,7 @@ flat gradient) and the reference's own Taylor-remainder test (utilities/cnn_deri
 import numpy as np
 import pytest
 
-import torchref
+from oracle import torchref
 from fitre_amd.structs import (ACT_LOGISTIC, ACT_TANH, AVG_POOL, CNN_ACT_ELU, CNN_ACT_NONE, CNN_ACT_RELU,
                                CNN_ACT_SOFTPLUS, CNN_ACT_SWISH, MAX_POOL, NO_POOL, PERFORM_NO_BATCH_NORM)
 from helpers import batch_inputs, build_custom, build_lenet, he_weights, num_classes, rel_err

@@ -10,7 +10,7 @@ import torch
 import torch.nn.functional as F
 
 from fitre_amd.structs import (ACT_LOGISTIC, ACT_TANH, CNN_ACT_ELU, CNN_ACT_RELU, CNN_ACT_SOFTPLUS, CNN_ACT_SWISH)
-from torchref import from_nchw, to_nchw
+from oracle.torchref import from_nchw, to_nchw
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 
@@ -234,7 +234,7 @@ def test_max_pool_tie_break_is_first_maximum_in_memory_order(oracle64):
 # ------------------------------------------------------------------ activations
 @pytest.mark.parametrize("code", [CNN_ACT_RELU, CNN_ACT_SWISH, CNN_ACT_SOFTPLUS, CNN_ACT_ELU, ACT_LOGISTIC, ACT_TANH])
 def test_activation_forward_backward_against_autograd(oracle64, code):
-    from torchref import act_torch
+    from oracle.torchref import act_torch
     rng = np.random.default_rng(13)
     x = rng.standard_normal(257) * 3
     x[:3] = [25.0, -25.0, 0.5]
