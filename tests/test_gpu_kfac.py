@@ -216,6 +216,84 @@ def _spd(n, rng, cond):
     return ((q * ev) @ q.T).astype(np.float32)
 
 
+def _spd_reflected(n, rng, cond):
+    """A dense symmetric matrix with the eigenvalues geomspace(1, 1/cond, n), in O(n^2 log n): the diagonal matrix of
+    the (shuffled) eigenvalues conjugated by an orthonormal cosine transform, random signs and two random Householder
+    reflections — exactly known spectrum, for orders where a QR factorisation of a random matrix would dominate the
+    test."""
+    from scipy.fft import dct
+    a = np.diag(rng.permutation(np.geomspace(1.0, 1.0 / cond, n)))
+    a = dct(dct(a, axis=0, norm="ortho"), axis=1, norm="ortho")
+    sign = rng.choice([-1.0, 1.0], n)
+    a = sign[:, None] * a * sign[None, :]
+    for _ in range(2):
+        u = rng.standard_normal(n)
+        u /= np.linalg.norm(u)
+        au = a @ u
+        a = a - 2.0 * np.outer(u, au) - 2.0 * np.outer(au, u) + 4.0 * (u @ au) * np.outer(u, u)
+    return ((a + a.T) / 2).astype(np.float32)
+
+
+@pytest.mark.parametrize("n", [2305, 4609])
+def test_spd_inverse_at_the_largest_factor_orders(dev, n):
+    """The orders of VGG-11's input-side factors (9*256+1, 9*512+1), which are the only ones that reach the upper
+    levels of the halving recursion, the triangular-operand range skipping and the deep-slice products: against a
+    float64 LAPACK inverse.  Spectrum geomspace(1, 1e-3) + 0.02: condition 49 after the shift; tolerance the path's
+    1e-4 (max-abs error over the largest magnitude of the float64 inverse), result exactly symmetric."""
+    rng = np.random.default_rng(n)
+    a = _spd_reflected(n, rng, 1000.0)
+    shift = 0.02
+    pa = dev.upload(a.reshape(-1))
+    out = dev.upload(np.full(n * n, np.nan, dtype=np.float32))
+    nb = hip.fitre_hip_spd_inverse_workspace(n)
+    ws = dev.alloc(nb)
+    info = C.c_int(-1)
+    L.check(hip.fitre_hip_spd_inverse(pa, n, shift, out, ws, nb, C.byref(info)))
+    assert info.value == 0
+    got = dev.download(out, n * n).reshape(n, n)
+    a64 = a.astype(np.float64) + shift * np.eye(n)
+    ev = np.linalg.eigvalsh(a64)
+    assert 40 < ev[-1] / ev[0] < 60
+    want = np.linalg.inv(a64)
+    assert rel_err(got, want) < TOL
+    assert np.array_equal(got, got.T)
+    assert np.abs(a64 @ got.astype(np.float64) - np.eye(n)).max() < 1e-4
+    for q in (pa, out, ws):
+        dev.free(q)
+
+
+@pytest.mark.parametrize("n", [2305, 4609])
+def test_spd_inverse_batched_at_the_largest_factor_orders(dev, n):
+    """Three matrices of one order through one chain of launches, as computeOmegaZ batches VGG-11's last three
+    input-side factors: each against the float64 LAPACK inverse of its own matrix at 1e-4, exactly symmetric,
+    strides larger than the matrices and nothing written between the results."""
+    batch, shift = 3, 0.02
+    rng = np.random.default_rng(7 * n)
+    mats = [_spd_reflected(n, rng, 1000.0) for _ in range(batch)]
+    m_stride, i_stride = n * n + 24, n * n + 64
+    packed = np.zeros(batch * m_stride, np.float32)
+    for b, a in enumerate(mats):
+        packed[b * m_stride:b * m_stride + n * n] = a.reshape(-1)
+    pa = dev.upload(packed)
+    out = dev.upload(np.full(batch * i_stride, np.nan, dtype=np.float32))
+    one = hip.fitre_hip_spd_inverse_workspace(n)
+    ws_stride = (one + 255) // 256 * 256 + 512
+    ws = dev.alloc(batch * ws_stride)
+    piv = dev.upload(np.full(batch, -1, np.int32), np.int32)
+    L.check(hip.fitre_hip_spd_inverse_batched_queued(batch, pa, m_stride, n, shift, out, i_stride, ws, one, ws_stride, piv))
+    dev.sync()
+    assert not dev.download(piv, batch, np.int32).any()
+    got_all = dev.download(out, batch * i_stride)
+    for b, a in enumerate(mats):
+        got = got_all[b * i_stride:b * i_stride + n * n].reshape(n, n)
+        want = np.linalg.inv(a.astype(np.float64) + shift * np.eye(n))
+        assert rel_err(got, want) < TOL, b
+        assert np.array_equal(got, got.T)
+        assert np.isnan(got_all[b * i_stride + n * n:(b + 1) * i_stride]).all()
+    for q in (pa, out, ws, piv):
+        dev.free(q)
+
+
 @pytest.mark.parametrize("n", [1, 3, 28, 64, 65, 129, 400, 577, 1153])
 def test_spd_inverse(dev, oracle64, n):
     """(A + shift I)^-1 against the oracle's Cholesky inverse.  The error of an inverse computed in float32
@@ -464,6 +542,33 @@ def test_vgg11_full_size_factor_inverses_with_the_benchmark_damping(dev):
     L.cnn.computeNaturalGradient(C.byref(model), C.byref(info), ws, None)
     ng = dev.download(ngrad, model.pSize)
     assert np.isfinite(ng).all() and np.abs(ng).max() > 0
+    # against the oracle's natural gradient fed the inverses the device produced, layer block by layer block (weights
+    # and bias of a layer are adjacent in the flat layout).  With damping 1e-3 on rank-deficient factors the inverses
+    # have entries near 1000 that cancel in the product (the gradient lies in the factor's range, where the inverse is
+    # small): a float32 product cannot be more accurate than a few rounding units of |inverse| |gradient| |inverse|,
+    # whatever the kernel.  The tolerance is the path's 1e-4 of the block's largest magnitude for cancellation ratios
+    # kappa = max(|Omega^-1| |wb| |Lambda^-1|) / max|result| up to 1000 and grows linearly beyond, i.e. 1e-7 * kappa:
+    # 1.7 float32 rounding units of the product of magnitudes (measured: 0.13 units; kappa = 3e4 for the 4609-order
+    # layers, 1e6 for the ten-class output layer, below 500 for the first six layers).
+    from oracle.oracle import Oracle
+    inv_o, inv_l, g_host = dev.download(oinv, tot_o), dev.download(linv, tot_l), gm.get("grad")
+    want = Oracle(double=True).natural_gradient(model, list(info.OmegaZOffsets), list(info.LambdaGOffsets), inv_o, inv_l, g_host)
+    for l in range(layers):
+        lo = model.wOffsets[l]
+        hi = model.wOffsets[l + 1] if l + 1 < layers else model.pSize
+        n_out = int(round(np.sqrt(info.LambdaGOffsets[l + 1] - info.LambdaGOffsets[l])))
+        n_in = int(round(np.sqrt(info.OmegaZOffsets[l + 1] - info.OmegaZOffsets[l])))
+        om = np.abs(inv_o[info.OmegaZOffsets[l]:info.OmegaZOffsets[l] + n_in * n_in].astype(np.float64)).reshape(n_in, n_in)
+        la = np.abs(inv_l[info.LambdaGOffsets[l]:info.LambdaGOffsets[l] + n_out * n_out].astype(np.float64)).reshape(n_out, n_out)
+        gl = np.abs(g_host[lo:hi].astype(np.float64))
+        if l < model.cLayers:       # [Cout][K] weights then Cout biases -> Cout x (K+1)
+            wb = np.concatenate([gl[:n_out * (n_in - 1)].reshape(n_out, n_in - 1), gl[n_out * (n_in - 1):].reshape(n_out, 1)], axis=1)
+        else:                       # column-major out x in, then out biases
+            wb = np.concatenate([gl[:n_out * (n_in - 1)].reshape(n_in - 1, n_out).T, gl[n_out * (n_in - 1):].reshape(n_out, 1)], axis=1)
+        kappa = float((la @ wb @ om).max() / np.abs(want[lo:hi]).max())
+        err = rel_err(ng[lo:hi], want[lo:hi])
+        print("natural gradient layer %d: error %.2e, cancellation ratio %.0f" % (l, err, kappa))
+        assert err < TOL * max(1.0, kappa / 1000.0), ("natural gradient", l, err, kappa)
     # a descent direction: g' (F^-1 g) > 0 for a positive definite Fisher approximation
     assert float(np.dot(ng.astype(np.float64), gm.get("grad").astype(np.float64))) > 0
     for q in (ofac, lfac, oinv, linv, ws, ngrad):
