@@ -36,6 +36,10 @@ int lane_compute_units();     // compute units a kernel launched on the selected
 int lane_compute_units_min(); // the smallest such count over the lanes
 int device_compute_units();
 bool ready();
+int current_device();            // the device fitre_hip_init selected, -1 before
+// Per-device set-up of the file that holds the batch-norm kernels (address of its static scratch
+// array on the current device); called by fitre_hip_init with the device current.
+int layers_device_setup(int device);
 
 #define FITRE_HIP_TRY(expr)                                                                          \
 	do {                                                                                             \

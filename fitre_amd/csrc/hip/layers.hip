@@ -1046,6 +1046,27 @@ __global__ void boundary_permute_kernel(const float *in, int C, int N, int A, in
 	}
 }
 
+// ---- the entry point that allocates nothing ---------------------------------------------------
+// The per-(channel, segment) sums of the batch-norm backward step live in a file-scope device
+// array instead of a caller's workspace.  Every GPU holds its own copy of the array at its own
+// address; the address is looked up once per device, with that device current, by
+// layers_device_setup() (called from fitre_hip_init) and host code only ever uses that pointer.
+static __device__ __align__(256) unsigned char scratch[FITRE_HIP_STATIC_SCRATCH_BYTES];
+constexpr int kMaxDevices = 64;
+static void *g_scratch_ptr[kMaxDevices] = {};
+
+int layers_device_setup(int device)
+{
+	if (device < 0 || device >= kMaxDevices)
+		return fail(FITRE_E_ARGUMENT, "device index %d beyond the %d this layer keeps a scratch address for", device, kMaxDevices);
+	if (g_scratch_ptr[device]) return FITRE_OK;
+	void *ptr = nullptr;
+	FITRE_HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+	if (!ptr) return fail(FITRE_E_DEVICE, "hipGetSymbolAddress returned a null address for the static scratch array");
+	g_scratch_ptr[device] = ptr;
+	return FITRE_OK;
+}
+
 } // namespace fitre
 
 using namespace fitre;
@@ -1239,15 +1260,11 @@ int fitre_hip_batch_norm_forward(const float *in, int channels, long perChannel,
 	return check_launch("batch_norm_forward");
 }
 
-int fitre_hip_batch_norm_backward(const float *delta, const float *zhat, const float *variance, int channels,
-                                  long perChannel, float epsilon, float *out, float *biasGrad, void *ws, size_t wsBytes)
+// The launches of the stand-alone batch-norm backward step; `partial` holds the per-(channel, segment) sums.
+static int bn_backward_launch(const float *delta, const float *zhat, const float *variance, int channels, long perChannel,
+                              float epsilon, float *out, float *biasGrad, double *partial)
 {
-	FITRE_NEED_INIT();
-	FITRE_REQUIRE(delta && zhat && variance && out, "fitre_hip_batch_norm_backward: null pointer");
-	int rc = check_channels("fitre_hip_batch_norm_backward", channels, perChannel, ws, wsBytes);
-	if (rc) return rc;
 	int S = segments_for(channels, perChannel);
-	double *partial = (double *)ws;
 	LaunchScope scope(FITRE_KC_BN_BWD, 12.0 * (double)channels * (double)perChannel + 8.0 * channels);
 	dim3 grid(S, channels);
 	bool vec = aligned16(delta) && aligned16(zhat) && aligned16(out) && (perChannel % 4 == 0);
@@ -1266,6 +1283,38 @@ int fitre_hip_batch_norm_backward(const float *delta, const float *zhat, const f
 		                                                                  out, biasGrad);
 	}
 	return check_launch("batch_norm_backward");
+}
+
+int fitre_hip_batch_norm_backward(const float *delta, const float *zhat, const float *variance, int channels,
+                                  long perChannel, float epsilon, float *out, float *biasGrad, void *ws, size_t wsBytes)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(delta && zhat && variance && out, "fitre_hip_batch_norm_backward: null pointer");
+	int rc = check_channels("fitre_hip_batch_norm_backward", channels, perChannel, ws, wsBytes);
+	if (rc) return rc;
+	return bn_backward_launch(delta, zhat, variance, channels, perChannel, epsilon, out, biasGrad, (double *)ws);
+}
+
+int fitre_hip_batch_norm_backward_static(const float *delta, const float *zhat, const float *variance, int channels,
+                                         long perChannel, float epsilon, float *out, float *biasGrad)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(delta && zhat && variance && out, "fitre_hip_batch_norm_backward_static: null pointer");
+	FITRE_REQUIRE(channels > 0 && perChannel > 0, "fitre_hip_batch_norm_backward_static: non-positive shape (channels=%d, perChannel=%ld)",
+	              channels, perChannel);
+	FITRE_REQUIRE(channels <= 65535, "fitre_hip_batch_norm_backward_static: %d channels exceed the grid limit", channels);
+	const size_t need = fitre_hip_batch_norm_workspace(channels, perChannel);
+	if (need > (size_t)FITRE_HIP_STATIC_SCRATCH_BYTES)
+		return fail(FITRE_E_WORKSPACE,
+		            "fitre_hip_batch_norm_backward_static: %d channels of %ld elements need %zu bytes of partial sums, the static "
+		            "scratch array holds %d; use fitre_hip_batch_norm_backward with a workspace",
+		            channels, perChannel, need, FITRE_HIP_STATIC_SCRATCH_BYTES);
+	const int device = current_device();
+	void *ptr = (device >= 0 && device < kMaxDevices) ? g_scratch_ptr[device] : nullptr;
+	if (!ptr) return fail(FITRE_E_DEVICE, "fitre_hip_batch_norm_backward_static: no scratch address for device %d", device);
+	// every (channel, segment) slot the apply pass reads is written by the partial-sum pass of the
+	// same call, so nothing of an earlier call's contents has to be cleared
+	return bn_backward_launch(delta, zhat, variance, channels, perChannel, epsilon, out, biasGrad, (double *)ptr);
 }
 
 int fitre_hip_pool_act_bn_backward(int poolType, int actFun, float *delta, int deltaSplits, long deltaStride, const float *zhat,

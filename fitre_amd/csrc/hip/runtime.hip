@@ -72,6 +72,7 @@ int lane_compute_units_min()
 }
 int device_compute_units() { return g_lane_cus[0]; }
 bool ready() { return g_ready; }
+int current_device() { return g_ready ? g_device : -1; }
 
 int check_launch(const char *what)
 {
@@ -155,6 +156,7 @@ int fitre_hip_init(int device)
 	FITRE_HIP_TRY(hipSetDevice(device));
 	if (g_ready && g_device == device) return FITRE_OK;
 	if (g_ready) fitre_hip_shutdown();
+	if (int rc = layers_device_setup(device)) return rc;
 	int cus = 0;
 	FITRE_HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device));
 	if (cus <= 0 || cus > 1024) return fail(FITRE_E_DEVICE, "fitre_hip_init: device reports %d compute units", cus);

@@ -82,6 +82,7 @@ HIP_API = {
     "fitre_hip_batch_norm_workspace": (sz, [i32, lng]),
     "fitre_hip_batch_norm_forward": (i32, [vp, i32, lng, vp, vp, vp, vp, vp, f32, f32, i32, vp, sz]),
     "fitre_hip_batch_norm_backward": (i32, [vp, vp, vp, i32, lng, f32, vp, vp, vp, sz]),
+    "fitre_hip_batch_norm_backward_static": (i32, [vp, vp, vp, i32, lng, f32, vp, vp]),
     "fitre_hip_channel_sum_workspace": (sz, [i32, lng]),
     "fitre_hip_channel_sum": (i32, [vp, i32, lng, vp, vp, sz]),
     "fitre_hip_row_sum": (i32, [vp, i32, i32, vp]),

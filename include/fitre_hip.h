@@ -197,6 +197,18 @@ int fitre_hip_batch_norm_forward(const float *in, int channels, long perChannel,
 int fitre_hip_batch_norm_backward(const float *delta, const float *zhat, const float *variance,
                                   int channels, long perChannel, float epsilon, float *out,
                                   float *biasGrad, void *ws, size_t wsBytes);
+/* The same step for callers that cannot allocate device memory or hand over a workspace (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  The
+ * per-(channel, segment) partial sums live in a file-scope device array of FITRE_HIP_STATIC_SCRATCH_BYTES that
+ * every GPU the library runs on holds until the process ends; the call makes no hipMalloc / hipFree and no
+ * allocating library call.  Shapes whose partial sums (fitre_hip_batch_norm_workspace) exceed the array are
+ * rejected with FITRE_E_WORKSPACE.  All calls on one GPU share that GPU's array: calls that overlap on one GPU
+ * (two lanes, two host threads) race; calls queued on one lane do not.  Results are bit-identical to
+ * fitre_hip_batch_norm_backward on the same inputs. */
+#define FITRE_HIP_STATIC_SCRATCH_BYTES (1 << 20)
+int fitre_hip_batch_norm_backward_static(const float *delta, const float *zhat, const float *variance,
+                                         int channels, long perChannel, float epsilon, float *out,
+                                         float *biasGrad);
 
 /* fitre_hip_pool_act_backward followed by fitre_hip_batch_norm_backward of its dxAct, as the backward pass
  * runs them for a layer with batch norm (functions/cnn_backward.cu:586-660): the pool/activation pass leaves the
