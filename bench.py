@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the CNN backward pass on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--serial] [--headline-only]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--serial] [--headline-only] [--config NAME]
 
 Defaults: 20 warm-up and 100 timed passes (a shorter region ends while the clocks are still ramping).
 
@@ -20,9 +20,10 @@ Prints ONE JSON line: backward images/sec, plus
   kernels       the same accounting for every kernel class of the backward pass;
   bandwidth_kernels  pool+activation and batch-norm backward run alone at the two largest layers'
                 shapes, against the 8 TB/s HBM peak;
-  cpu_baseline  the C restatement of the reference's algorithm (float32, OpenMP) timed on the host
-                cores on a bounded sample (same network, smaller batch);
-  torch_cpu     torch autograd of the same network on the host cores (float32), for orientation.
+  cpu_baseline  the gradient path the reference checks itself against (torch autograd of the same network,
+                float32, batch 256) on the host cores: median of 10 passes after 3 warm-ups, backward only
+                (`value`) and forward + backward; `c_port` beside it is the C restatement of the reference's
+                algorithm (float32, OpenMP) on a smaller batch.
 """
 import argparse
 import ctypes as C
@@ -47,15 +48,46 @@ TILES = {0: "", 1: "64x64", 2: "64x128", 3: "128x64", 4: "128x128"}
 
 
 def measured_traffic(kernel):
-    """HBM bytes per launch of `kernel` as measured with hardware counters in a separate profiler run;
-    the figures and the commands behind them are kept as text under profiles/.  None if not on record."""
+    """HBM bytes per launch of `kernel` as measured with hardware counters (FETCH_SIZE, WRITE_SIZE) in separate
+    profiler runs of this program; the figures and the commands behind them are kept as text under profiles/.
+    Returns (bytes, file name, commit of the tree the counters were taken at) or (None, None, None)."""
     import glob
     for path in sorted(glob.glob(os.path.join(ROOT, "profiles", "*hbm_traffic.txt"))):
+        found, tree = None, None
         for line in open(path):
             f = line.split()
             if len(f) == 3 and f[0] == "traffic_bytes_per_launch" and f[1] == kernel:
-                return int(f[2])
-    return None
+                found = int(f[2])
+            if len(f) == 2 and f[0] == "tree":
+                tree = f[1]
+        if found is not None:
+            return found, os.path.relpath(path, ROOT), tree
+    return None, None, None
+
+
+def tree_commit():
+    import subprocess
+    try:
+        return subprocess.run(["git", "-C", ROOT, "rev-parse", "--short", "HEAD"], stdout=subprocess.PIPE,
+                              stderr=subprocess.DEVNULL, text=True, timeout=10).stdout.strip() or None
+    except (OSError, subprocess.SubprocessError):
+        return None
+
+
+def kernel_table(rows, steps):
+    """Per kernel class (and tile variant): launches per step, average launch duration, achieved rate against the
+    bound of its class (fp32 MFMA for the contraction kernels, HBM for the others)."""
+    kernels = {}
+    for r in rows:
+        avg_us = 1e3 * r["ms"] / r["launches"]
+        mfma = r["cls"] in MFMA_CLASSES
+        rate = r["work"] / (r["ms"] * 1e-3) / (1e12 if mfma else 1e9) if r["ms"] > 0 else 0.0
+        peak = PEAK_MFMA_F32_TFLOPS if mfma else PEAK_HBM_GBS
+        kernels[r["kernel"]] = dict(bound="mfma" if mfma else "hbm", launches_per_step=r["launches"] / steps,
+                                    avg_us=round(avg_us, 2), ms_per_step=round(r["ms"] / steps, 4),
+                                    achieved=round(rate, 2 if mfma else 1), unit="TFLOP/s" if mfma else "GB/s",
+                                    frac=round(rate / peak, 4))
+    return kernels
 
 
 def read_profile(L):
@@ -144,26 +176,18 @@ def gpu_leg(args):
         others = other_configs_leg(L, dev)
     dev.close()
 
-    kernels = {}
-    for r in rows:
-        avg_us = 1e3 * r["ms"] / r["launches"]
-        per_step = r["launches"] / args.steps
-        if r["cls"] in MFMA_CLASSES:
-            rate = r["work"] / (r["ms"] * 1e-3) / 1e12 if r["ms"] > 0 else 0.0
-            kernels[r["kernel"]] = dict(bound="mfma", launches_per_step=per_step, avg_us=round(avg_us, 2),
-                                        ms_per_step=round(r["ms"] / args.steps, 4), achieved=round(rate, 2),
-                                        unit="TFLOP/s", frac=round(rate / PEAK_MFMA_F32_TFLOPS, 4))
-        else:
-            rate = r["work"] / (r["ms"] * 1e-3) / 1e9 if r["ms"] > 0 else 0.0
-            kernels[r["kernel"]] = dict(bound="hbm", launches_per_step=per_step, avg_us=round(avg_us, 2),
-                                        ms_per_step=round(r["ms"] / args.steps, 4), achieved=round(rate, 1),
-                                        unit="GB/s", frac=round(rate / PEAK_HBM_GBS, 4))
+    kernels = kernel_table(rows, args.steps)
     dom = max(rows, key=lambda r: r["ms"])
     dk = kernels[dom["kernel"]]
     roofline = dict(kernel=dom["kernel"], bound=dk["bound"], achieved=dk["achieved"],
                     peak=PEAK_MFMA_F32_TFLOPS if dk["bound"] == "mfma" else PEAK_HBM_GBS, unit=dk["unit"],
-                    frac=dk["frac"], traffic=measured_traffic(dom["kernel"]), avg_launch_us=dk["avg_us"],
+                    frac=dk["frac"], traffic=None, avg_launch_us=dk["avg_us"],
                     launches_per_step=dk["launches_per_step"])
+    traffic, source, taken_at = measured_traffic(dom["kernel"])
+    roofline["traffic"] = traffic
+    roofline["traffic_source"] = dict(file=source, counters_taken_at_commit=taken_at, this_tree=tree_commit(),
+                                      note="FETCH_SIZE / WRITE_SIZE of separate rocprofv3 --pmc runs of this program, "
+                                           "scaled by the calibration copy; not re-measured in this run")
     conv_rows = [r for r in rows if r["cls"] in ("conv_dw", "conv_dx")]
     conv_ms, conv_work = sum(r["ms"] for r in conv_rows), sum(r["work"] for r in conv_rows)
     conv = dict(ms_per_step=round(conv_ms / args.steps, 4), gflop_per_step=round(conv_work / args.steps / 1e9, 2),
@@ -175,30 +199,53 @@ def gpu_leg(args):
                 other_configs=others)
 
 
-def other_configs_leg(L, dev, steps=10):
+OTHER_CONFIGS = ("lenet_b128", "lenet_bn_b1024", "alexnet_224_b64")
+
+
+def other_configs_leg(L, dev, steps=10, only=None):
     """Backward images/sec of the other benchmark networks (the same step: copy of the loss errors + one
-    cnnBackward), for orientation: LeNet-style b128, the same with batch norm b1024, AlexNet-style
-    3x224x224 b64 with 1000 classes."""
+    cnnBackward): LeNet-style b128, the same with batch norm b1024, AlexNet-style 3x224x224 b64 with 1000 classes.
+    Each with the per-launch accounting of a second pass of the same steps: every kernel class against its
+    bound, and `roofline` = the class with the largest summed time."""
     from fitre_amd.harness import GpuModel, batch_inputs, build_alexnet, build_lenet, he_weights
     out = {}
     for name, build, batch in (("lenet_b128", lambda: build_lenet(128), 128),
                                ("lenet_bn_b1024", lambda: build_lenet(1024, bn=True), 1024),
                                ("alexnet_224_b64", lambda: build_alexnet(64), 64)):
+        if only and name != only:
+            continue
         model = build()
         rng = np.random.default_rng(0xF17E0005 + batch)
         w = he_weights(model, rng).astype(np.float32)
         x, y = batch_inputs(model, batch, rng)
         gm = GpuModel(dev, model, w, x.astype(np.float32), y, batch)
         gm.forward()
-        gm.backward()
+        for _ in range(3):
+            gm.backward()
         dev.sync()
         t0 = time.perf_counter()
         for _ in range(steps):
             gm.backward()
         dev.sync()
         dt = time.perf_counter() - t0
+        L.check(L.hip.fitre_hip_profile_enable(1))
+        for _ in range(steps):
+            gm.backward()
+        dev.sync()
+        L.check(L.hip.fitre_hip_profile_enable(0))
+        rows = read_profile(L)
+        kernels = kernel_table(rows, steps)
+        dom = max(rows, key=lambda r: r["ms"])
+        dk = kernels[dom["kernel"]]
         out[name] = dict(images_per_s=round(batch * steps / dt, 1), ms_per_step=round(1e3 * dt / steps, 4),
-                         finite=bool(np.isfinite(gm.get("grad")).all()))
+                         finite=bool(np.isfinite(gm.get("grad")).all()),
+                         launches_per_step=sum(r["launches"] for r in rows) / steps,
+                         kernel_ms_per_step=round(sum(r["ms"] for r in rows) / steps, 4),
+                         roofline=dict(kernel=dom["kernel"], bound=dk["bound"], achieved=dk["achieved"],
+                                       peak=PEAK_MFMA_F32_TFLOPS if dk["bound"] == "mfma" else PEAK_HBM_GBS,
+                                       unit=dk["unit"], frac=dk["frac"], avg_launch_us=dk["avg_us"],
+                                       launches_per_step=dk["launches_per_step"]),
+                         kernels=kernels)
         gm.release()
     return out
 
@@ -384,7 +431,17 @@ def kfac_step_leg(L, dev, gm, model, batch, repeats):
     return round(ms, 3)
 
 
-def cpu_leg(batch=64, repeats=10):
+def cpu_model_name():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def c_port_leg(batch=64, repeats=5):
     """float32 build of the oracle (the reference's algorithm restated in C, OpenMP over the host
     cores): one forward, then `repeats` backward passes on the same network at a smaller batch."""
     from fitre_amd.harness import batch_inputs, build_vgg11, he_weights
@@ -402,26 +459,32 @@ def cpu_leg(batch=64, repeats=10):
         o.backward(model, w, x, z, errors, batch)
     dt = time.perf_counter() - t0
     cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
-    return dict(value=round(batch * repeats / dt, 2), unit="images/s", cores=cores, kind="port",
-                sample="VGG-11 backward, float32, batch %d x %d passes, C restatement with OpenMP" % (batch, repeats))
+    return dict(value=round(batch * repeats / dt, 2), unit="images/s (backward only)", cores=cores,
+                sample="VGG-11 backward, float32, batch %d x %d passes, C restatement of the reference's algorithm with OpenMP"
+                       % (batch, repeats))
 
 
-def torch_leg(batch=32, repeats=3):
+def cpu_leg(batch=256, warmup=3, repeats=10):
+    """The CPU gradient path the reference checks itself against (pytorch/gradtest: torch autograd through conv2d /
+    batch_norm / relu / max_pool2d / linear / cross_entropy), as the oracle's torch model, float32, on the host
+    cores, at the benchmark's own network and batch: `warmup` untimed passes, `repeats` timed, medians.  `value` is
+    the backward-only rate (the GPU metric is backward-only); forward + backward is given beside it."""
     import torch
     from oracle import torchref
     from fitre_amd.harness import batch_inputs, build_vgg11, he_weights
 
     model = build_vgg11(batch, bn=True)
-    rng = np.random.default_rng(1)
+    rng = np.random.default_rng(0xF17E0003)
     w = he_weights(model, rng)
     x, y = batch_inputs(model, batch, rng)
-    torchref.run(model, w, x, y, batch, dtype=torch.float32, want_intermediates=False)
-    t0 = time.perf_counter()
-    for _ in range(repeats):
-        torchref.run(model, w, x, y, batch, dtype=torch.float32, want_intermediates=False)
-    dt = time.perf_counter() - t0
-    return dict(value=round(batch * repeats / dt, 2), unit="images/s (forward+backward)", threads=torch.get_num_threads(),
-                sample="torch %s autograd, float32, batch %d x %d" % (torch.__version__, batch, repeats))
+    both, back = torchref.time_gradient(model, w, x, y, batch, dtype=torch.float32, warmup=warmup, repeats=repeats)
+    return dict(value=round(batch / back, 2), unit="images/s", cores=os.cpu_count(), threads=torch.get_num_threads(),
+                kind="port", cpu=cpu_model_name(),
+                forward_backward_images_per_s=round(batch / both, 2),
+                backward_ms=round(1e3 * back, 2), forward_backward_ms=round(1e3 * both, 2),
+                sample="torch %s autograd, float32, VGG-11 + batch norm, batch %d, 3x32x32: median of %d passes after %d "
+                       "warm-ups; value = backward only (loss.backward() with the forward pass done), "
+                       "forward_backward_images_per_s = both" % (torch.__version__, batch, repeats, warmup))
 
 
 def main():
@@ -435,11 +498,23 @@ def main():
     ap.add_argument("--headline-only", action="store_true",
                     help="only the headline workload (no factor / inverse / Hessian-vector / bandwidth / other-network legs): "
                          "under a kernel tracer every launch then belongs to the VGG-11 batch-256 passes")
+    ap.add_argument("--config", choices=OTHER_CONFIGS, default=None,
+                    help="run ONLY this other benchmark network (its forward pass once, 3 + steps + steps backward passes) and "
+                         "print its entry of other_configs: under a kernel tracer every launch then belongs to it")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (the reference path is single-device and every "
                  "box here has one GPU); --gpus %d is not supported" % args.gpus)
 
+    if args.config:
+        from fitre_amd import lib as L
+        from fitre_amd.harness import Device
+        dev = Device(0)
+        if args.serial:
+            L.check(L.hip.fitre_hip_lanes_enable(0))
+        print(json.dumps({args.config: other_configs_leg(L, dev, steps=args.steps, only=args.config)[args.config]}))
+        dev.close()
+        return
     g = gpu_leg(args)
     seconds = g["ms_events"] * 1e-3
     value = g["batch"] * args.steps / seconds
@@ -470,11 +545,11 @@ def main():
         "finite": g["finite"],
     }
     if not args.no_cpu:
-        line["cpu_baseline"] = cpu_leg()
         try:
-            line["torch_cpu"] = torch_leg()
-        except Exception as exc:  # torch is optional on the box
-            line["torch_cpu"] = {"error": str(exc)}
+            line["cpu_baseline"] = cpu_leg()
+            line["cpu_baseline"]["c_port"] = c_port_leg()
+        except ImportError as exc:  # no torch on the box: the C restatement alone
+            line["cpu_baseline"] = dict(c_port_leg(), kind="port", note="torch not importable: %s" % exc)
     print(json.dumps(line))
 
 

@@ -155,6 +155,30 @@ def forward_loss(model, convs, fcs, x_flat, y, batch, dtype=torch.float64):
     return F.cross_entropy(h, torch.tensor(np.asarray(y, dtype=np.int64) - 1))
 
 
+def time_gradient(model, wflat, x_flat, y, batch, dtype=torch.float32, warmup=3, repeats=10):
+    """Wall time of the autograd gradient on the host cores, the way pytorch/gradtest times its models
+    (alexnet_cifar.py:48-62 forward, :88-101 loss.backward()): `warmup` untimed passes, then `repeats` timed
+    ones; returns the medians in seconds of forward + backward and of backward alone (loss.backward() with the
+    forward pass done beforehand)."""
+    import time
+    convs, fcs = unpack(model, wflat, dtype)
+    params = [t for pair in convs + fcs for t in pair if t is not None]
+    x_flat = np.asarray(x_flat, dtype=np.float64)
+    both, back = [], []
+    for i in range(warmup + repeats):
+        for t in params:
+            t.grad = None
+        t0 = time.perf_counter()
+        loss = forward_loss(model, convs, fcs, x_flat, y, batch, dtype)
+        t1 = time.perf_counter()
+        loss.backward()
+        t2 = time.perf_counter()
+        if i >= warmup:
+            both.append(t2 - t0)
+            back.append(t2 - t1)
+    return float(np.median(both)), float(np.median(back))
+
+
 def hessian_vector(model, wflat, x_flat, y, batch, vflat):
     """H * v of the mean cross-entropy loss by double backward, in the flat parameter layout."""
     convs, fcs = unpack(model, wflat)
