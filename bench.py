@@ -74,10 +74,12 @@ def tree_commit():
         return None
 
 
-def kernel_table(rows, steps):
+def kernel_table(rows, steps, launches=None):
     """Per kernel class (and tile variant): launches per step, average launch duration, achieved rate against the
-    bound of its class (fp32 MFMA for the contraction kernels, HBM for the others)."""
+    bound of its class (fp32 MFMA for the contraction kernels, HBM for the others); with `launches`, also the
+    four largest shapes of each kernel on their own (`largest`: work in FLOP resp. bytes)."""
     kernels = {}
+    big = largest_launches(launches) if launches else {}
     for r in rows:
         avg_us = 1e3 * r["ms"] / r["launches"]
         mfma = r["cls"] in MFMA_CLASSES
@@ -87,7 +89,46 @@ def kernel_table(rows, steps):
                                     avg_us=round(avg_us, 2), ms_per_step=round(r["ms"] / steps, 4),
                                     achieved=round(rate, 2 if mfma else 1), unit="TFLOP/s" if mfma else "GB/s",
                                     frac=round(rate / peak, 4))
+        if r["kernel"] in big:
+            kernels[r["kernel"]]["largest"] = big[r["kernel"]]
+        if r["kernel"] in ("conv_dw", "conv_dx"):
+            # the untiled variants of these classes are the dense per-image form of 3x3 convolutions on 2x2 maps
+            kernels[r["kernel"]]["note"] = ("3x3 windows on 2x2 maps as dense products: the work counted is the nine-tap "
+                                            "2*M*K*Cout, of which the kernel executes 16/36 (the rest multiplies padding)")
     return kernels
+
+
+def read_launches(L):
+    """Every accounted launch of the last accounting period: (kernel name, class, work, ms)."""
+    n = C.c_long()
+    L.check(L.hip.fitre_hip_profile_launch_count(C.byref(n)))
+    names = {v: k for k, v in KC.items()}
+    out = []
+    cls, tile, ms, work = C.c_int(), C.c_int(), C.c_double(), C.c_double()
+    for i in range(n.value):
+        L.check(L.hip.fitre_hip_profile_read_launch(i, C.byref(cls), C.byref(tile), C.byref(ms), C.byref(work)))
+        name = names[cls.value]
+        out.append((name + ("/" + TILES[tile.value] if tile.value else ""), name, work.value, ms.value))
+    return out
+
+
+def largest_launches(launches, keep=4):
+    """Per kernel, the `keep` shapes that carry the most algorithmic work (launches of equal work are one shape:
+    the same layer in every step), each with its own average duration and fraction of its bound — class averages
+    are dominated by the many launches that last a few microseconds."""
+    shapes = {}
+    for kernel, cls, work, ms in launches:
+        e = shapes.setdefault((kernel, cls, work), [0, 0.0])
+        e[0] += 1
+        e[1] += ms
+    out = {}
+    for (kernel, cls, work), (n, ms) in shapes.items():
+        mfma = cls in MFMA_CLASSES
+        t = ms * 1e-3 / n
+        rate = work / t / (1e12 if mfma else 1e9) if t > 0 else 0.0
+        out.setdefault(kernel, []).append(dict(work=work, launches=n, avg_us=round(t * 1e6, 2), achieved=round(rate, 2 if mfma else 1),
+                                               frac=round(rate / (PEAK_MFMA_F32_TFLOPS if mfma else PEAK_HBM_GBS), 4)))
+    return {k: sorted(v, key=lambda e: -e["work"])[:keep] for k, v in out.items()}
 
 
 def read_profile(L):
@@ -154,6 +195,7 @@ def gpu_leg(args):
     dev.sync()
     L.check(L.hip.fitre_hip_profile_enable(0))
     rows = read_profile(L)
+    launches = read_launches(L)
     # the forward pass that produces z (not part of the metric), for orientation
     gm.forward()
     dev.sync()
@@ -176,7 +218,7 @@ def gpu_leg(args):
         others = other_configs_leg(L, dev)
     dev.close()
 
-    kernels = kernel_table(rows, args.steps)
+    kernels = kernel_table(rows, args.steps, launches)
     dom = max(rows, key=lambda r: r["ms"])
     dk = kernels[dom["kernel"]]
     roofline = dict(kernel=dom["kernel"], bound=dk["bound"], achieved=dk["achieved"],
@@ -234,7 +276,7 @@ def other_configs_leg(L, dev, steps=10, only=None):
         dev.sync()
         L.check(L.hip.fitre_hip_profile_enable(0))
         rows = read_profile(L)
-        kernels = kernel_table(rows, steps)
+        kernels = kernel_table(rows, steps, read_launches(L))
         dom = max(rows, key=lambda r: r["ms"])
         dk = kernels[dom["kernel"]]
         out[name] = dict(images_per_s=round(batch * steps / dt, 1), ms_per_step=round(1e3 * dt / steps, 4),

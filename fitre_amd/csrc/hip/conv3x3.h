@@ -116,6 +116,7 @@ template <int CB, bool DX, bool VECW, int MAXB, int IT>
 __global__ void __launch_bounds__(kGemmThreads)
 conv3x3_pos_kernel(const Conv3x3Params p, const OutParams out)
 {
+	FITRE_RAISE_MATRIX_WAVE_PRIORITY();
 	typedef C3Pos<CB, DX, MAXB, IT> K;
 	constexpr int TM = K::TM, TN = K::TN;
 	__shared__ __attribute__((aligned(16))) float As[K::A_FLOATS + 4];
@@ -327,6 +328,7 @@ template <bool VECD, int MAXB>
 __global__ void __launch_bounds__(kC3DwThreads)
 conv3x3_dw_kernel(const Conv3x3Params p, const float *delta, uint32_t deltaBytes, const OutParams out)
 {
+	FITRE_RAISE_MATRIX_WAVE_PRIORITY();
 	constexpr int T = kC3DwThreads;
 	constexpr int CELLS_MAX = kC3Stage + 2 * (MAXB + 1);               // flat window cells per channel
 	constexpr int XP_MAX = CELLS_MAX + (CELLS_MAX + MAXB - 2) / MAXB + 1; // with row pads (largest at B = MAXB)

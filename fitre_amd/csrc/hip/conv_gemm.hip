@@ -2,6 +2,7 @@
 // column-major GEMM, all on the fp32-MFMA tile engine.
 #include "conv3x3.h"
 #include "conv_common.h"
+#include "conv_quad.h"
 
 namespace fitre {
 
@@ -304,6 +305,13 @@ static int launch_thin_dw(const fitre_conv_shape *s, const float *x, const float
 	return check_launch("conv3x3_dw_thin_kernel");
 }
 
+// the dense form of a 3x3 convolution on 2 x 2 maps, when the caller's workspace holds what it needs
+// (the full size the *_workspace() query reports; with less the nine-tap kernels run)
+static bool quad_usable(const fitre_conv_shape *s, const void *ws, size_t wsBytes, size_t need)
+{
+	return quad_eligible(s) && ws && ((((uintptr_t)ws) & 15) == 0) && wsBytes >= need;
+}
+
 size_t gemm_ex_workspace(int M, int N, int K, int flags)
 {
 	if (M <= 0 || N <= 0 || K <= 0) return 0;
@@ -436,6 +444,10 @@ int fitre_hip_conv_forward(const fitre_conv_shape *s, const float *x, const floa
 size_t fitre_hip_conv_weight_grad_workspace(const fitre_conv_shape *s)
 {
 	if (!s) return 0;
+	if (quad_eligible(s)) {
+		const size_t q = quad_weight_grad_workspace(s), c = c3_dw_eligible(s) ? c3_dw_workspace(s) : 0;
+		return q > c ? q : c;
+	}
 	if (c3_dw_eligible(s)) return c3_dw_workspace(s);
 	size_t general = plan_gemm_workspace(s->outChannels, (long)s->inChannels * s->ksize * s->ksize, (long)s->samples * s->outA * s->outB);
 	if (thin_dw_eligible(s) && thin_dw_workspace(s) > general) return thin_dw_workspace(s);
@@ -448,6 +460,8 @@ int fitre_hip_conv_weight_grad(const fitre_conv_shape *s, const float *x, const 
 	int rc = check_conv("fitre_hip_conv_weight_grad", s);
 	if (rc) return rc;
 	FITRE_REQUIRE(x && delta && dW, "fitre_hip_conv_weight_grad: null pointer");
+	if (quad_usable(s, ws, wsBytes, quad_weight_grad_workspace(s)) && (((((uintptr_t)x) | ((uintptr_t)delta)) & 15) == 0))
+		return quad_weight_grad(s, x, delta, dW, ws, wsBytes);
 	if (c3_dw_eligible(s)) return launch_c3_dw(s, x, delta, dW, ws, wsBytes);
 	if (thin_dw_eligible(s) && ws && wsBytes >= thin_dw_workspace(s) && ((((uintptr_t)delta) | ((uintptr_t)ws)) & 15) == 0)
 		return launch_thin_dw(s, x, delta, dW, ws);
@@ -463,6 +477,10 @@ int fitre_hip_conv_weight_grad(const fitre_conv_shape *s, const float *x, const 
 size_t fitre_hip_conv_input_grad_workspace(const fitre_conv_shape *s)
 {
 	if (!s) return 0;
+	if (quad_eligible(s)) {
+		const size_t q = quad_input_grad_workspace(s), c = c3_pos_eligible(s, true) ? c3_pos_workspace(s, true) : 0;
+		return q > c ? q : c;
+	}
 	if (c3_pos_eligible(s, true)) return c3_pos_workspace(s, true);
 	return plan_gemm_workspace(s->inChannels, (long)s->samples * s->inA * s->inB, (long)s->outChannels * s->ksize * s->ksize);
 }
@@ -476,6 +494,8 @@ int fitre_hip_conv_input_grad(const fitre_conv_shape *s, const float *delta, con
 	if (s->stride != 1)
 		return fail(FITRE_E_UNSUPPORTED, "fitre_hip_conv_input_grad: stride %d (only stride 1 is back-propagated through)", s->stride);
 	FITRE_REQUIRE(s->padding < s->ksize, "fitre_hip_conv_input_grad: padding %d >= window %d", s->padding, s->ksize);
+	if (quad_usable(s, ws, wsBytes, quad_input_grad_workspace(s)) && (((((uintptr_t)dx) | ((uintptr_t)delta) | ((uintptr_t)w)) & 15) == 0))
+		return quad_input_grad(s, delta, w, nullptr, dx, ws, wsBytes, nullptr, nullptr);
 	if (c3_pos_eligible(s, true)) return launch_c3_pos<true>(s, delta, w, nullptr, dx, ws, wsBytes);
 	const int I = s->inChannels, J = s->samples * s->inA * s->inB, R = s->outChannels * s->ksize * s->ksize;
 	GemmPlan plan = plan_gemm(I, J, R);
@@ -546,8 +566,26 @@ int fitre_hip_conv_weight_grad_pair(const fitre_conv_shape *s, const float *x1, 
 	return launch_c3_dw(s, x1, delta1, dW, ws, wsBytes, x2, delta2);
 }
 
-int fitre_hip_conv_input_grad_split(const fitre_conv_shape *s, const float *delta, const float *w, float *dx, void *ws,
-                                    size_t wsBytes, fitre_split_view *view)
+size_t fitre_hip_conv_input_grad_prepared_bytes(const fitre_conv_shape *s)
+{
+	return (s && quad_eligible(s)) ? quad_weff_bytes(s) : 0;
+}
+
+int fitre_hip_conv_input_grad_prepare(const fitre_conv_shape *s, const float *w, void *prepared, size_t preparedBytes)
+{
+	FITRE_NEED_INIT();
+	int rc = check_conv("fitre_hip_conv_input_grad_prepare", s);
+	if (rc) return rc;
+	FITRE_REQUIRE(w && prepared, "fitre_hip_conv_input_grad_prepare: null pointer");
+	if (!quad_eligible(s)) return fail(FITRE_E_UNSUPPORTED, "fitre_hip_conv_input_grad_prepare: nothing to prepare for this shape");
+	if (preparedBytes < quad_weff_bytes(s) || (((uintptr_t)prepared) & 15))
+		return fail(FITRE_E_WORKSPACE, "fitre_hip_conv_input_grad_prepare: buffer of %zu bytes is misaligned or smaller than the %zu required",
+		            preparedBytes, quad_weff_bytes(s));
+	return quad_prepare_weights(s, w, (float *)prepared);
+}
+
+int fitre_hip_conv_input_grad_split_prepared(const fitre_conv_shape *s, const float *delta, const float *w, const void *prepared,
+                                             float *dx, void *ws, size_t wsBytes, fitre_split_view *view)
 {
 	FITRE_NEED_INIT();
 	FITRE_REQUIRE(view != nullptr, "fitre_hip_conv_input_grad_split: null view");
@@ -557,6 +595,20 @@ int fitre_hip_conv_input_grad_split(const fitre_conv_shape *s, const float *delt
 	int rc = check_conv("fitre_hip_conv_input_grad_split", s);
 	if (rc) return rc;
 	FITRE_REQUIRE(delta && w && dx, "fitre_hip_conv_input_grad_split: null pointer");
+	const bool aligned = (((((uintptr_t)dx) | ((uintptr_t)delta) | ((uintptr_t)w) | ((uintptr_t)ws) | ((uintptr_t)prepared)) & 15) == 0);
+	if (quad_eligible(s) && aligned && ws &&
+	    wsBytes >= (prepared ? quad_input_grad_workspace(s) - quad_weff_bytes(s) : quad_input_grad_workspace(s))) {
+		int splits = 1;
+		float *partials = nullptr;
+		rc = quad_input_grad(s, delta, w, (const float *)prepared, dx, ws, wsBytes, &splits, &partials);
+		if (rc) return rc;
+		if (splits > 1) {
+			view->base = partials;
+			view->splits = splits;
+			view->stride = (long)s->inChannels * s->samples * 4;
+		}
+		return FITRE_OK;
+	}
 	if (s->stride == 1 && s->padding < s->ksize && c3_pos_eligible(s, true)) {
 		int splits = 1;
 		rc = launch_c3_pos<true>(s, delta, w, nullptr, dx, ws, wsBytes, &splits);
@@ -569,6 +621,12 @@ int fitre_hip_conv_input_grad_split(const fitre_conv_shape *s, const float *delt
 		return FITRE_OK;
 	}
 	return fitre_hip_conv_input_grad(s, delta, w, dx, ws, wsBytes);
+}
+
+int fitre_hip_conv_input_grad_split(const fitre_conv_shape *s, const float *delta, const float *w, float *dx, void *ws,
+                                    size_t wsBytes, fitre_split_view *view)
+{
+	return fitre_hip_conv_input_grad_split_prepared(s, delta, w, nullptr, dx, ws, wsBytes, view);
 }
 
 // ---- general column-major GEMM ---------------------------------------------------

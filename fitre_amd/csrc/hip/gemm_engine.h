@@ -368,6 +368,11 @@ struct OutParams {
 	int mirror;
 	// Bit mask of kTri*: operands that are zero on one side of the diagonal in the reduction index.
 	int triK;
+	// Non-zero: rows come in groups of four that are interleaved with the columns in memory -- element (i, j)
+	// lives at C[(i / 4) * quadLd + 4 * j + i % 4] (a [C][N][2][2] tensor with i = (c, cell), j = n; quadLd = 4 J).
+	// A lane's four consecutive rows then form one 16-byte group.  Applies to split partials as well (each a
+	// permutation of I x J elements, I % 4 == 0); bias, beta and mirror are not used with it.
+	long quadLd;
 };
 // both operands: element (row, k) is zero for k < row, so the reduction of a tile starts at the larger of its first rows
 constexpr int kTriBoth = 1;
@@ -485,7 +490,7 @@ __device__ __forceinline__ void gemm_tile(const typename OpA::Params &pa, const 
 				if (i >= I) continue;
 				if (out.mirror && j < i) continue;
 				float val = acc[tm][tn][v];
-				float *dst = C + (size_t)i * out.ldc + j;
+				float *dst = out.quadLd ? C + (size_t)(i >> 2) * out.quadLd + 4 * (size_t)j + (i & 3) : C + (size_t)i * out.ldc + j;
 				if (!split) {
 					val *= out.alpha;
 					if (out.biasI) val += out.biasI[i];
@@ -527,6 +532,7 @@ template <int VEC>
 __global__ void __launch_bounds__(256)
 splitk_reduce_kernel(const float *ws, int splits, int I, int J, OutParams out, long wsBatchStride = 0, long cBatchStride = 0)
 {
+	FITRE_RAISE_WAVE_PRIORITY();
 	ws += (size_t)blockIdx.y * wsBatchStride; // blockIdx.y: problem of a batch (0 otherwise)
 	out.C += (size_t)blockIdx.y * cBatchStride;
 	const long total = (long)I * J;
@@ -585,6 +591,7 @@ template <int VEC>
 __global__ void __launch_bounds__(256)
 splitk_reduce_wide_kernel(const float *ws, int splits, int I, int J, OutParams out, long wsBatchStride = 0, long cBatchStride = 0)
 {
+	FITRE_RAISE_WAVE_PRIORITY();
 	ws += (size_t)blockIdx.y * wsBatchStride;
 	out.C += (size_t)blockIdx.y * cBatchStride;
 	__shared__ double part[16][16 * VEC + 1];

@@ -180,6 +180,26 @@ pool_backward_kernel(const float *delta, const float *z_in, const float *z_act, 
 	}
 }
 
+// No pooling, 16-byte accesses: dxPool = delta (a snapshot, may be null), dxAct = delta * f'(.).
+__global__ void __launch_bounds__(256)
+nopool_act_backward_vec_kernel(const float4 *delta, const float4 *z_in, const float4 *z_act, long groups, int actFun, float4 *dxPool,
+                               float4 *dxAct)
+{
+	const long stride = (long)gridDim.x * blockDim.x;
+	for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < groups; i += stride) {
+		const float4 d = delta[i];
+		const float4 zo = z_act ? z_act[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+		const float4 zi = z_in ? z_in[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+		if (dxPool) dxPool[i] = d;
+		float4 r;
+		r.x = d.x * act_derivative(actFun, zi.x, zo.x);
+		r.y = d.y * act_derivative(actFun, zi.y, zo.y);
+		r.z = d.z * act_derivative(actFun, zi.z, zo.z);
+		r.w = d.w * act_derivative(actFun, zi.w, zo.w);
+		dxAct[i] = r;
+	}
+}
+
 // Overlapping max-pool windows (e.g. 3x3 / stride 2): one workgroup per map keeps the map and the
 // arg-max of every window in LDS, so a window is scanned once instead of once per cell it contains
 // (up to four times for 3/2), and each cell then looks up the windows it belongs to.  Same scan and
@@ -224,6 +244,181 @@ maxpool_map_backward_kernel(const float *delta, const float *z_in, const float *
 			dxAct[mapOff + i] = acc * act_derivative(actFun, zi, zmap[i]);
 		}
 	}
+}
+
+// The same for windows of compile-time extent and stride (3 / 2: AlexNet-style pools), moved with 16-byte
+// accesses: a workgroup owns `mapsPerGroup` consecutive maps, i.e. one contiguous range of the tensor, and
+// walks it in 16-byte groups aligned in global memory (the range may start anywhere: the first and last group
+// are handled cell by cell).  The maps and the pooled gradient go to LDS first, every thread with all its loads
+// in flight at once; then one scan per window; then every cell looks up the (at most ceil(KS/ST)^2) windows
+// that contain it, in the same order as pool_backward_kernel<0>, so the results are identical.
+template <bool FUSE_ACT, int KS, int ST>
+__global__ void __launch_bounds__(256)
+maxpool_maps_backward_kernel(const float *delta, const float *z_in, const float *z_act, PoolGeom g, int mapsPerGroup, long maps,
+                             FastDiv divCells, FastDiv divWindows, int actFun, float *dxPool, float *dxAct)
+{
+	// LDS sized by the launch for the group it processes: [maps | pooled gradient | window arg-max]
+	extern __shared__ __align__(16) unsigned char pool_lds[];
+	float *zs = reinterpret_cast<float *>(pool_lds);
+	float *dl = zs + ((mapsPerGroup * g.inA * g.inB + 8 + 3) & ~3);
+	int *arg = reinterpret_cast<int *>(dl + mapsPerGroup * g.outA * g.outB);
+	constexpr int kVecPerThread = (kPoolMapCells + 8) / 4 / 256 + 1; // 5
+	constexpr int kWinPerThread = kPoolMapWindows / 256;             // 5
+	const int cells = g.inA * g.inB, windows = g.outA * g.outB;
+	const long firstMap = (long)blockIdx.x * mapsPerGroup;
+	const int nMaps = (int)((maps - firstMap < (long)mapsPerGroup) ? (maps - firstMap) : (long)mapsPerGroup);
+	const int nCells = nMaps * cells, nWin = nMaps * windows;
+	const size_t g0 = (size_t)firstMap * cells;
+	const int lead = (int)(g0 & 3);
+	const int nVec = (lead + nCells + 3) >> 2;
+	const size_t vbase = g0 - lead; // multiple of four floats
+	const int tid = threadIdx.x;
+
+	// ---- stage the maps and the pooled gradient
+	{
+		float4 t[kVecPerThread];
+#pragma unroll
+		for (int k = 0; k < kVecPerThread; k++) {
+			const int v = tid + 256 * k;
+			const int e0 = 4 * v - lead;
+			t[k] = make_float4(0.f, 0.f, 0.f, 0.f);
+			if (v < nVec) {
+				if (e0 >= 0 && e0 + 3 < nCells) {
+					t[k] = *reinterpret_cast<const float4 *>(z_act + vbase + 4 * (size_t)v);
+				} else {
+					if (e0 >= 0 && e0 < nCells) t[k].x = z_act[vbase + 4 * (size_t)v];
+					if (e0 + 1 >= 0 && e0 + 1 < nCells) t[k].y = z_act[vbase + 4 * (size_t)v + 1];
+					if (e0 + 2 >= 0 && e0 + 2 < nCells) t[k].z = z_act[vbase + 4 * (size_t)v + 2];
+					if (e0 + 3 >= 0 && e0 + 3 < nCells) t[k].w = z_act[vbase + 4 * (size_t)v + 3];
+				}
+			}
+		}
+		float d[kWinPerThread];
+#pragma unroll
+		for (int k = 0; k < kWinPerThread; k++) {
+			const int w = tid + 256 * k;
+			d[k] = (w < nWin) ? delta[(size_t)firstMap * windows + w] : 0.f;
+		}
+#pragma unroll
+		for (int k = 0; k < kVecPerThread; k++) {
+			const int v = tid + 256 * k;
+			if (v < nVec) *reinterpret_cast<float4 *>(zs + 4 * v) = t[k];
+		}
+#pragma unroll
+		for (int k = 0; k < kWinPerThread; k++) {
+			const int w = tid + 256 * k;
+			if (w < nWin) dl[w] = d[k];
+		}
+	}
+	__syncthreads();
+
+	// ---- one scan per window: first maximum in memory order (strict >), offset inside its map
+	for (int w = tid; w < nWin; w += 256) {
+		uint32_t m, r, oa, ob;
+		divWindows.divmod((uint32_t)w, m, r);
+		g.divOutB.divmod(r, oa, ob);
+		const float *zmap = zs + lead + (int)m * cells;
+		const int a0 = (int)oa * ST - g.padding, b0 = (int)ob * ST - g.padding;
+		float best = -FLT_MAX;
+		int at = -1;
+#pragma unroll
+		for (int da = 0; da < KS; da++) {
+			const int a = a0 + da;
+			if (a < 0 || a >= g.inA) continue;
+#pragma unroll
+			for (int db = 0; db < KS; db++) {
+				const int b = b0 + db;
+				if (b < 0 || b >= g.inB) continue;
+				const float t = zmap[a * g.inB + b];
+				if (t > best) {
+					best = t;
+					at = a * g.inB + b;
+				}
+			}
+		}
+		arg[w] = at;
+	}
+	__syncthreads();
+
+	// ---- every cell gathers from the windows that contain it
+	for (int v = tid; v < nVec; v += 256) {
+		const int e0 = 4 * v - lead;
+		float acc[4], zo[4];
+#pragma unroll
+		for (int e = 0; e < 4; e++) {
+			const int i = e0 + e;
+			acc[e] = 0.f;
+			zo[e] = zs[4 * v + e];
+			if (i < 0 || i >= nCells) continue;
+			uint32_t m, r, a, b;
+			divCells.divmod((uint32_t)i, m, r);
+			g.divInB.divmod(r, a, b);
+			int oaHi = ((int)a + g.padding) / ST, obHi = ((int)b + g.padding) / ST;
+			int oaLo = ((int)a + g.padding - KS + ST) / ST, obLo = ((int)b + g.padding - KS + ST) / ST;
+			if ((int)a + g.padding - KS + 1 <= 0) oaLo = 0;
+			if ((int)b + g.padding - KS + 1 <= 0) obLo = 0;
+			if (oaHi >= g.outA) oaHi = g.outA - 1;
+			if (obHi >= g.outB) obHi = g.outB - 1;
+			const int wbase = (int)m * windows;
+			for (int oa = oaLo; oa <= oaHi; oa++)
+				for (int ob = obLo; ob <= obHi; ob++) {
+					const int w = wbase + oa * g.outB + ob;
+					if (arg[w] == (int)r) acc[e] += dl[w];
+				}
+		}
+		const size_t at = vbase + 4 * (size_t)v;
+		const bool whole = e0 >= 0 && e0 + 3 < nCells;
+		if (dxPool) {
+			if (whole) {
+				*reinterpret_cast<float4 *>(dxPool + at) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+			} else {
+#pragma unroll
+				for (int e = 0; e < 4; e++)
+					if (e0 + e >= 0 && e0 + e < nCells) dxPool[at + e] = acc[e];
+			}
+		}
+		if constexpr (FUSE_ACT) {
+			float zi[4] = { 0.f, 0.f, 0.f, 0.f };
+			if (z_in) {
+				if (whole) {
+					const float4 q = *reinterpret_cast<const float4 *>(z_in + at);
+					zi[0] = q.x, zi[1] = q.y, zi[2] = q.z, zi[3] = q.w;
+				} else {
+#pragma unroll
+					for (int e = 0; e < 4; e++)
+						if (e0 + e >= 0 && e0 + e < nCells) zi[e] = z_in[at + e];
+				}
+			}
+			float r4[4];
+#pragma unroll
+			for (int e = 0; e < 4; e++) r4[e] = acc[e] * act_derivative(actFun, zi[e], zo[e]);
+			if (whole) {
+				*reinterpret_cast<float4 *>(dxAct + at) = make_float4(r4[0], r4[1], r4[2], r4[3]);
+			} else {
+#pragma unroll
+				for (int e = 0; e < 4; e++)
+					if (e0 + e >= 0 && e0 + e < nCells) dxAct[at + e] = r4[e];
+			}
+		}
+	}
+}
+
+// LDS bytes of maxpool_maps_backward_kernel for groups of `per` maps
+static size_t maps_group_lds(int cells, int windows, int per)
+{
+	return sizeof(float) * (size_t)((per * cells + 8 + 3) & ~3) + 2 * sizeof(float) * (size_t)per * windows;
+}
+
+// How many consecutive maps one workgroup of maxpool_maps_backward_kernel takes: as many as fit its LDS arrays,
+// but no more than leaves about six workgroups per compute unit.
+static int maps_per_group(int cells, int windows, long maps)
+{
+	long fit = kPoolMapCells / cells;
+	if (kPoolMapWindows / windows < fit) fit = kPoolMapWindows / windows;
+	long spread = maps / 1536;
+	if (spread < 1) spread = 1;
+	if (fit > spread) fit = spread;
+	return (int)(fit < 1 ? 1 : fit);
 }
 
 // strict-> scan of four values in order, starting below every finite float
@@ -488,6 +683,7 @@ __global__ void __launch_bounds__(kRedBlock)
 bn_backward_apply_kernel(const float *delta, const float *zhat, const float *variance, const double *partial,
                          int segmentsIn, float epsilon, long perChannel, float *out, float *biasGrad)
 {
+	FITRE_RAISE_WAVE_PRIORITY();
 	__shared__ double lds[3 * kRedBlock / kWave];
 	const int c = blockIdx.y;
 	const float *pd = delta + (size_t)c * perChannel;
@@ -546,6 +742,7 @@ __global__ void __launch_bounds__(kRedBlock)
 bn_backward_small_kernel(const float *delta, const float *zhat, const float *variance, float epsilon, long perChannel,
                          float *out, float *biasGrad)
 {
+	FITRE_RAISE_WAVE_PRIORITY();
 	__shared__ double lds[kRedBlock / kWave];
 	const int c = blockIdx.x;
 	const float *pd = delta + (size_t)c * perChannel;
@@ -706,6 +903,7 @@ __global__ void __launch_bounds__(kRedBlock)
 pool_act_sums_kernel(const float *delta, int dSplits, long dStride, const float *zhat, const float *z_act, int inA, int inB,
                      int samples, int actFun, float *dxPool, bool streamPool, float *dxAct, double *partial)
 {
+	FITRE_RAISE_WAVE_PRIORITY();
 	__shared__ double lds[3 * kRedBlock / kWave];
 	const int c = blockIdx.y;
 	const long perChannel = (long)samples * inA * inB;
@@ -773,6 +971,7 @@ pool_act_bn_small_kernel(const float *delta, int dSplits, long dStride, const fl
                          const float *variance, int inA, int inB, int samples, int actFun, float epsilon, float *dxPool,
                          float *dxAct, float *dxBn, float *biasGrad)
 {
+	FITRE_RAISE_WAVE_PRIORITY();
 	__shared__ double lds[3 * kRedBlock / kWave];
 	constexpr int G = (int)(kBnSmallChannel / (4 * kRedBlock)); // 16-byte groups per thread
 	static_assert(G >= 2 && G % 2 == 0, "a 2 x 4 patch is two groups");
@@ -1138,10 +1337,17 @@ int fitre_hip_pool_act_backward(int poolType, int actFun, const float *delta, co
 		            (((uintptr_t)delta & 7) == 0);
 		const bool perMap = !fast && inA * inB <= kPoolMapCells && outA * outB <= kPoolMapWindows && inA * inB >= 64 &&
 		                    maps <= 0x7fffffffL;
+		const bool grouped = perMap && ksize == 3 && stride == 2 && aligned16(z_act) && aligned16(dxAct) &&
+		                     (!dxPool || aligned16(dxPool)) && (!z_in || aligned16(z_in));
 		if (fast)
 			maxpool2_backward_kernel<true><<<blocks_for(total / 8, 256, 16384), 256, 0, stream()>>>(
 			    delta, act_needs_zin(actFun) ? z_in : nullptr, z_act, inA, inB, maps, actFun, dxPool, dxAct);
-		else if (perMap)
+		else if (grouped) {
+			const int per = maps_per_group(inA * inB, outA * outB, maps);
+			maxpool_maps_backward_kernel<true, 3, 2><<<(unsigned)((maps + per - 1) / per), 256, maps_group_lds(inA * inB, outA * outB, per), stream()>>>(
+			    delta, act_needs_zin(actFun) ? z_in : nullptr, z_act, g, per, maps, FastDiv((uint32_t)(inA * inB)),
+			    FastDiv((uint32_t)(outA * outB)), actFun, dxPool, dxAct);
+		} else if (perMap)
 			maxpool_map_backward_kernel<true><<<(unsigned)maps, 256, 0, stream()>>>(delta, act_needs_zin(actFun) ? z_in : nullptr, z_act, g,
 			                                                                      actFun, dxPool, dxAct);
 		else
@@ -1149,7 +1355,14 @@ int fitre_hip_pool_act_backward(int poolType, int actFun, const float *delta, co
 	} else if (poolType == AVG_POOL) {
 		pool_backward_kernel<1, true><<<blocks, 256, 0, stream()>>>(delta, z_in, z_act, g, maps, actFun, dxPool, dxAct);
 	} else if (poolType == NO_POOL) {
-		pool_backward_kernel<2, true><<<blocks, 256, 0, stream()>>>(delta, z_in, z_act, g, maps, actFun, dxPool, dxAct);
+		if (total % 4 == 0 && aligned16(delta) && aligned16(dxAct) && (!dxPool || aligned16(dxPool)) && (!z_in || aligned16(z_in)) &&
+		    (!z_act || aligned16(z_act)))
+			nopool_act_backward_vec_kernel<<<blocks_for(total / 4, 256, 16384), 256, 0, stream()>>>(
+			    reinterpret_cast<const float4 *>(delta), reinterpret_cast<const float4 *>(act_needs_zin(actFun) ? z_in : nullptr),
+			    reinterpret_cast<const float4 *>(z_act), total / 4, actFun, reinterpret_cast<float4 *>(dxPool),
+			    reinterpret_cast<float4 *>(dxAct));
+		else
+			pool_backward_kernel<2, true><<<blocks, 256, 0, stream()>>>(delta, z_in, z_act, g, maps, actFun, dxPool, dxAct);
 	} else {
 		return fail(FITRE_E_UNSUPPORTED, "fitre_hip_pool_act_backward: unknown pool type %d", poolType);
 	}
@@ -1177,7 +1390,12 @@ int fitre_hip_pool_backward(int poolType, const float *delta, const float *z_in,
 		if (fast)
 			maxpool2_backward_kernel<false><<<blocks_for(total / 8, 256, 16384), 256, 0, stream()>>>(
 			    delta, nullptr, z_in, inA, inB, maps, CNN_ACT_NONE, out, nullptr);
-		else if (perMap)
+		else if (perMap && ksize == 3 && stride == 2 && aligned16(z_in) && aligned16(out)) {
+			const int per = maps_per_group(inA * inB, outA * outB, maps);
+			maxpool_maps_backward_kernel<false, 3, 2><<<(unsigned)((maps + per - 1) / per), 256, maps_group_lds(inA * inB, outA * outB, per), stream()>>>(
+			    delta, nullptr, z_in, g, per, maps, FastDiv((uint32_t)(inA * inB)), FastDiv((uint32_t)(outA * outB)), CNN_ACT_NONE, out,
+			    nullptr);
+		} else if (perMap)
 			maxpool_map_backward_kernel<false><<<(unsigned)maps, 256, 0, stream()>>>(delta, nullptr, z_in, g, CNN_ACT_NONE, out, nullptr);
 		else
 			pool_backward_kernel<0, false><<<blocks, 256, 0, stream()>>>(delta, nullptr, z_in, g, maps, CNN_ACT_NONE, out, nullptr);

@@ -40,7 +40,15 @@ static ClassTotals g_totals[FITRE_KC_COUNT][FITRE_TILE_VARIANTS];
 struct Pending {
 	hipEvent_t start, stop;
 	int cls, tile;
+	double work;
 };
+// every accounted launch in issue order, for per-launch figures (bounded: the oldest are kept)
+struct LaunchRecord {
+	int cls, tile;
+	double work, ms;
+};
+constexpr size_t kMaxLaunchRecords = 1 << 16;
+static std::vector<LaunchRecord> g_records;
 static std::vector<Pending> g_pending;
 static std::vector<hipEvent_t> g_event_pool;
 
@@ -97,8 +105,10 @@ static void drain_pending()
 {
 	for (Pending &p : g_pending) {
 		float ms = 0.f;
-		if (hipEventSynchronize(p.stop) == hipSuccess && hipEventElapsedTime(&ms, p.start, p.stop) == hipSuccess)
+		if (hipEventSynchronize(p.stop) == hipSuccess && hipEventElapsedTime(&ms, p.start, p.stop) == hipSuccess) {
 			g_totals[p.cls][p.tile].ms += ms;
+			if (g_records.size() < kMaxLaunchRecords) g_records.push_back({ p.cls, p.tile, p.work, (double)ms });
+		}
 		g_event_pool.push_back(p.start);
 		g_event_pool.push_back(p.stop);
 	}
@@ -113,6 +123,7 @@ LaunchScope::LaunchScope(int kernelClass, double work, int tile) : slot(-1)
 	p.stop = take_event();
 	p.cls = kernelClass;
 	p.tile = tile;
+	p.work = work;
 	if (!p.start || !p.stop) return;
 	g_totals[kernelClass][tile].launches += 1;
 	g_totals[kernelClass][tile].work += work;
@@ -398,7 +409,10 @@ int fitre_hip_profile_enable(int on)
 	FITRE_NEED_INIT();
 	for (int i = 0; i < kLanes; i++) FITRE_HIP_TRY(hipStreamSynchronize(g_lanes[i]));
 	drain_pending();
-	if (on) memset(g_totals, 0, sizeof(g_totals));
+	if (on) {
+		memset(g_totals, 0, sizeof(g_totals));
+		g_records.clear();
+	}
 	g_profile = (on != 0);
 	if (g_profile) {
 		g_lane = 0;
@@ -436,6 +450,31 @@ int fitre_hip_profile_read_tile(int kernelClass, int tile, long *launches, doubl
 	if (launches) *launches = g_totals[kernelClass][tile].launches;
 	if (milliseconds) *milliseconds = g_totals[kernelClass][tile].ms;
 	if (work) *work = g_totals[kernelClass][tile].work;
+	return FITRE_OK;
+}
+
+int fitre_hip_profile_launch_count(long *count)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(count != nullptr, "fitre_hip_profile_launch_count: null result pointer");
+	FITRE_HIP_TRY(hipStreamSynchronize(g_stream));
+	drain_pending();
+	*count = (long)g_records.size();
+	return FITRE_OK;
+}
+
+int fitre_hip_profile_read_launch(long index, int *kernelClass, int *tile, double *milliseconds, double *work)
+{
+	FITRE_NEED_INIT();
+	FITRE_HIP_TRY(hipStreamSynchronize(g_stream));
+	drain_pending();
+	FITRE_REQUIRE(index >= 0 && (size_t)index < g_records.size(), "fitre_hip_profile_read_launch: index %ld of %zu records", index,
+	              g_records.size());
+	const LaunchRecord &r = g_records[(size_t)index];
+	if (kernelClass) *kernelClass = r.cls;
+	if (tile) *tile = r.tile;
+	if (milliseconds) *milliseconds = r.ms;
+	if (work) *work = r.work;
 	return FITRE_OK;
 }
 

@@ -131,9 +131,21 @@ static size_t backward_side_ws_bytes(const CNN_MODEL *model, int batch)
 	return (need + 255) & ~(size_t)255;
 }
 
+/* Rearranged weight copies that some input gradients multiply by (fitre_hip_conv_input_grad_prepare): made at the
+ * start of the pass on a lane of their own, one buffer per layer that has one. */
+static size_t backward_prepared_bytes(const CNN_MODEL *model, int batch)
+{
+	size_t need = 0;
+	for (int i = 1; i < model->cLayers; i++) {
+		fitre_conv_shape s = conv_shape(&model->convLayer[i], batch);
+		need += (fitre_hip_conv_input_grad_prepared_bytes(&s) + 255) & ~(size_t)255;
+	}
+	return need;
+}
+
 static size_t backward_ws_bytes(const CNN_MODEL *model, int batch)
 {
-	return backward_chain_ws_bytes(model, batch) + backward_side_ws_bytes(model, batch);
+	return backward_chain_ws_bytes(model, batch) + backward_side_ws_bytes(model, batch) + backward_prepared_bytes(model, batch);
 }
 
 long cnnForwardMemRequired(CNN_MODEL *model)
@@ -238,6 +250,9 @@ void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, 
 	const size_t bnBytes = backward_bn_ws_bytes(model, model->batchSize);
 	void *sideWs = (void *)((char *)bnWs + bnBytes);
 	const size_t sideBytes = backward_side_ws_bytes(model, model->batchSize);
+	char *preparedWs = (char *)sideWs + sideBytes;
+	const void *prepared[MAX_LAYERS] = { NULL };
+	int preparedPending = 0;
 	real *temp;
 
 	if (nc < 1 || n < 1 || n > model->batchSize) {
@@ -246,6 +261,26 @@ void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, 
 		exit(-1);
 	}
 	const CONV_LAYER *last = &model->convLayer[nc - 1];
+
+	/* Weight copies of the layers whose input gradient reads one: they depend on the weights only, so lane 2 makes
+	 * them while the chain works through the linear layers. */
+	{
+		int any = 0;
+		for (int c = 1; c < nc; c++) {
+			fitre_conv_shape shape = conv_shape(&model->convLayer[c], n);
+			/* the buffers are laid out for the model's batch size; a shape's need does not depend on the batch */
+			const size_t bytes = fitre_hip_conv_input_grad_prepared_bytes(&shape);
+			prepared[c] = NULL;
+			if (bytes == 0 || !has_bn(&model->convLayer[c - 1])) continue;
+			if (!any) HIP_CALL(fitre_hip_lane_select(2));
+			any = 1;
+			HIP_CALL(fitre_hip_conv_input_grad_prepare(&shape, weights + wOffsets[c], preparedWs, bytes));
+			prepared[c] = preparedWs;
+			preparedWs += (bytes + 255) & ~(size_t)255;
+		}
+		if (any) HIP_CALL(fitre_hip_lane_select(0));
+		preparedPending = any;
+	}
 
 	for (int f = model->lLayers - 1; f >= 0; f--) {
 		const FC_LAYER *l = &model->fcLayer[f];
@@ -345,7 +380,12 @@ void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, 
 		 * norm) run on those while the weight gradient keeps the matrix pipes busy. */
 		if (c != 0) {
 			if (has_bn(&model->convLayer[c - 1])) {
-				HIP_CALL(fitre_hip_conv_input_grad_split(&shape, cur, weights + wOffsets[c], delta, ws, wsBytes, &dview));
+				if (prepared[c] && preparedPending) { /* the chain's first use of a copy lane 2 made */
+					HIP_CALL(fitre_hip_lane_wait(0, 2));
+					preparedPending = 0;
+				}
+				HIP_CALL(fitre_hip_conv_input_grad_split_prepared(&shape, cur, weights + wOffsets[c], prepared[c], delta, ws, wsBytes,
+				                                                  &dview));
 			} else {
 				HIP_CALL(fitre_hip_conv_input_grad(&shape, cur, weights + wOffsets[c], delta, ws, wsBytes));
 				dview.base = delta, dview.splits = 1, dview.stride = 0;

@@ -43,6 +43,8 @@ HIP_API = {
     "fitre_hip_profile_enable": (i32, [i32]),
     "fitre_hip_profile_read": (i32, [i32, C.POINTER(lng), C.POINTER(C.c_double), C.POINTER(C.c_double)]),
     "fitre_hip_profile_read_tile": (i32, [i32, i32, C.POINTER(lng), C.POINTER(C.c_double), C.POINTER(C.c_double)]),
+    "fitre_hip_profile_launch_count": (i32, [C.POINTER(lng)]),
+    "fitre_hip_profile_read_launch": (i32, [lng, pi32, pi32, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
     "fitre_hip_axpy": (i32, [i32, f32, vp, vp]),
     "fitre_hip_scal": (i32, [i32, f32, vp]),
     "fitre_hip_copy": (i32, [i32, vp, vp]),
@@ -75,6 +77,9 @@ HIP_API = {
     "fitre_hip_conv_input_grad_pair": (i32, [pshape, vp, vp, vp, vp, vp, vp, sz]),
     "fitre_hip_conv_weight_grad_pair": (i32, [pshape, vp, vp, vp, vp, vp, vp, sz]),
     "fitre_hip_conv_input_grad_split": (i32, [pshape, vp, vp, vp, vp, sz, vp]),
+    "fitre_hip_conv_input_grad_prepared_bytes": (sz, [pshape]),
+    "fitre_hip_conv_input_grad_prepare": (i32, [pshape, vp, vp, sz]),
+    "fitre_hip_conv_input_grad_split_prepared": (i32, [pshape, vp, vp, vp, vp, vp, sz, vp]),
     "fitre_hip_extract_columns": (i32, [vp, vp, vp, i32, i32]),
     "fitre_hip_augment_batch": (i32, [vp, i32, i32, i32, i32, i32, vp, i32, f32, vp, vp, vp, f32, vp]),
     "fitre_hip_crop_shifts": (i32, [vp, i32, i32, vp]),

@@ -104,6 +104,10 @@ int fitre_hip_profile_read(int kernelClass, long *launches, double *milliseconds
  * one: 0 = not tiled, 1 = 64x64, 2 = 64x128, 3 = 128x64, 4 = 128x128 (channel rows x contiguous columns). */
 #define FITRE_TILE_VARIANTS 5
 int fitre_hip_profile_read_tile(int kernelClass, int tile, long *launches, double *milliseconds, double *work);
+/* The accounted launches one by one, in issue order since the last fitre_hip_profile_enable(1) (at most 65 536
+ * are kept): class, tile variant, duration and algorithmic work of launch `index` < *count. */
+int fitre_hip_profile_launch_count(long *count);
+int fitre_hip_profile_read_launch(long index, int *kernelClass, int *tile, double *milliseconds, double *work);
 
 /* ---------------- level-1 helpers (the cublasD* calls of the solvers and of
  * functions/cnn_gradient.cu:54-56, functions/softmax_loss.cu:243) ---------------- */
@@ -337,6 +341,18 @@ typedef struct fitre_split_view {
 } fitre_split_view;
 int fitre_hip_conv_input_grad_split(const fitre_conv_shape *s, const float *delta, const float *w, float *dx,
                                     void *ws, size_t wsBytes, fitre_split_view *view);
+/* Some shapes multiply by a rearranged copy of the weights (3x3 windows on 2 x 2 maps: the dense per-image form
+ * of the convolution, 16/36 of the multiply-adds of the nine-tap form).  The copy depends on the weights only, so
+ * a caller can have it made ahead of the chain that needs it, on another lane:
+ *   _prepared_bytes  size of the copy, 0 when the shape has none;
+ *   _prepare         builds it (stream-ordered);
+ *   _split_prepared  fitre_hip_conv_input_grad_split reading it (prepared == NULL: built inside, in ws).
+ * No counterpart in the reference, whose weights are reordered per call (dev_backprop_convolution.cu:140-156). */
+size_t fitre_hip_conv_input_grad_prepared_bytes(const fitre_conv_shape *s);
+int fitre_hip_conv_input_grad_prepare(const fitre_conv_shape *s, const float *w, void *prepared, size_t preparedBytes);
+int fitre_hip_conv_input_grad_split_prepared(const fitre_conv_shape *s, const float *delta, const float *w,
+                                             const void *prepared, float *dx, void *ws, size_t wsBytes,
+                                             fitre_split_view *view);
 
 /* Column-major GEMM C(MxN) = alpha*op(A)*op(B) + beta*C with the argument meaning of cublasDgemm
  * (transA/transB: 0 = N, 1 = T).  Used for the FC layers (eval_gradient.cu:63-67,

@@ -153,6 +153,11 @@ POOL_GEOMS = [  # C, N, A(width), B(height), k, s, p
     (4, 2, 55, 55, 3, 2, 0),    # AlexNet's first pool
     (2, 2, 12, 12, 3, 1, 1),    # stride 1: every cell in up to nine windows
     (3, 2, 16, 16, 2, 2, 1),    # 2x2 with padding (not the 16-byte fast path)
+    # 3/2 windows through the kernel that gives a workgroup several consecutive maps and moves them in 16-byte groups
+    (7, 3, 13, 13, 3, 2, 0),    # 21 maps of 169 cells: ranges that start at every alignment
+    (257, 13, 13, 13, 3, 2, 0), # 3341 maps: two maps per workgroup, the last workgroup with one
+    (5, 3, 27, 27, 3, 2, 0),    # AlexNet's second pool
+    (3, 5, 15, 9, 3, 2, 1),     # padding 1, rectangular, odd cell count
 ]
 
 
