@@ -180,6 +180,20 @@ pool_backward_kernel(const float *delta, const float *z_in, const float *z_act, 
 	}
 }
 
+// 16-byte store; stream: nothing reads the value again soon and the tensor is larger than the caches
+// can usefully hold, so it is written past them (measured on a 67 MB tensor: the pass 44 -> 36.5 us; on
+// a 34 MB one the plain store is the faster)
+__device__ __forceinline__ void store4(float *p, float4 v, bool stream)
+{
+	if (stream) {
+		typedef float v4f __attribute__((ext_vector_type(4)));
+		v4f t = { v.x, v.y, v.z, v.w };
+		__builtin_nontemporal_store(t, reinterpret_cast<v4f *>(p));
+	} else {
+		*reinterpret_cast<float4 *>(p) = v;
+	}
+}
+
 // No pooling, 16-byte accesses: dxPool = delta (a snapshot, may be null), dxAct = delta * f'(.).
 __global__ void __launch_bounds__(256)
 nopool_act_backward_vec_kernel(const float4 *delta, const float4 *z_in, const float4 *z_act, long groups, int actFun, float4 *dxPool,
@@ -247,157 +261,199 @@ maxpool_map_backward_kernel(const float *delta, const float *z_in, const float *
 }
 
 // The same for windows of compile-time extent and stride (3 / 2: AlexNet-style pools), moved with 16-byte
-// accesses: a workgroup owns `mapsPerGroup` consecutive maps, i.e. one contiguous range of the tensor, and
-// walks it in 16-byte groups aligned in global memory (the range may start anywhere: the first and last group
-// are handled cell by cell).  The maps and the pooled gradient go to LDS first, every thread with all its loads
-// in flight at once; then one scan per window; then every cell looks up the (at most ceil(KS/ST)^2) windows
-// that contain it, in the same order as pool_backward_kernel<0>, so the results are identical.
+// accesses: a "group" is `mapsPerGroup` consecutive maps, i.e. one contiguous range of the tensor, walked in
+// 16-byte groups aligned in global memory (the range may start anywhere: its first and last 16 bytes are
+// handled cell by cell).  One group per workgroup: maps and
+// pooled gradient to LDS (every load of a thread in flight at once), one scan per window, then every cell looks
+// up the (at most ceil(KS/ST)^2) windows that contain it, in the same order as pool_backward_kernel<0>, so the
+// results are identical.
+struct PoolGroup {
+	int nCells, nWin, lead, nVec;
+	size_t vbase, dbase;
+};
+constexpr int kPoolVecPerThread = (kPoolMapCells + 8) / 4 / 256 + 1; // 5
+constexpr int kPoolWinPerThread = kPoolMapWindows / 256;             // 5
+
+__device__ __forceinline__ PoolGroup pool_group(long group, int mapsPerGroup, long maps, int cells, int windows)
+{
+	PoolGroup q;
+	const long firstMap = group * mapsPerGroup;
+	long n = maps - firstMap;
+	if (n > mapsPerGroup) n = mapsPerGroup;
+	if (n < 0) n = 0;
+	q.nCells = (int)n * cells;
+	q.nWin = (int)n * windows;
+	const size_t g0 = (size_t)firstMap * cells;
+	q.lead = (int)(g0 & 3);
+	q.nVec = q.nCells ? (q.lead + q.nCells + 3) >> 2 : 0;
+	q.vbase = g0 - q.lead; // multiple of four floats
+	q.dbase = (size_t)firstMap * windows;
+	return q;
+}
+
+__device__ __forceinline__ void pool_group_load(const PoolGroup &q, const float *z_act, const float *delta, int tid,
+                                                float4 (&t)[kPoolVecPerThread], float (&d)[kPoolWinPerThread])
+{
+#pragma unroll
+	for (int k = 0; k < kPoolVecPerThread; k++) {
+		const int v = tid + 256 * k;
+		const int e0 = 4 * v - q.lead;
+		t[k] = make_float4(0.f, 0.f, 0.f, 0.f);
+		if (v < q.nVec) {
+			const float *src = z_act + q.vbase + 4 * (size_t)v;
+			if (e0 >= 0 && e0 + 3 < q.nCells) {
+				t[k] = *reinterpret_cast<const float4 *>(src);
+			} else {
+				if (e0 >= 0 && e0 < q.nCells) t[k].x = src[0];
+				if (e0 + 1 >= 0 && e0 + 1 < q.nCells) t[k].y = src[1];
+				if (e0 + 2 >= 0 && e0 + 2 < q.nCells) t[k].z = src[2];
+				if (e0 + 3 >= 0 && e0 + 3 < q.nCells) t[k].w = src[3];
+			}
+		}
+	}
+#pragma unroll
+	for (int k = 0; k < kPoolWinPerThread; k++) {
+		const int w = tid + 256 * k;
+		d[k] = (w < q.nWin) ? delta[q.dbase + w] : 0.f;
+	}
+}
+
 template <bool FUSE_ACT, int KS, int ST>
 __global__ void __launch_bounds__(256)
-maxpool_maps_backward_kernel(const float *delta, const float *z_in, const float *z_act, PoolGeom g, int mapsPerGroup, long maps,
-                             FastDiv divCells, FastDiv divWindows, int actFun, float *dxPool, float *dxAct)
+maxpool_maps_backward_kernel(const float *delta, const float *z_in, const float *z_act, PoolGeom g, int mapsPerGroup,
+                             long maps, FastDiv divCells, FastDiv divWindows, int actFun, float *dxPool, float *dxAct, bool streamPool)
 {
-	// LDS sized by the launch for the group it processes: [maps | pooled gradient | window arg-max]
+	// LDS sized by the launch for one group: [maps | pooled gradient | window arg-max]
 	extern __shared__ __align__(16) unsigned char pool_lds[];
 	float *zs = reinterpret_cast<float *>(pool_lds);
 	float *dl = zs + ((mapsPerGroup * g.inA * g.inB + 8 + 3) & ~3);
 	int *arg = reinterpret_cast<int *>(dl + mapsPerGroup * g.outA * g.outB);
-	constexpr int kVecPerThread = (kPoolMapCells + 8) / 4 / 256 + 1; // 5
-	constexpr int kWinPerThread = kPoolMapWindows / 256;             // 5
 	const int cells = g.inA * g.inB, windows = g.outA * g.outB;
-	const long firstMap = (long)blockIdx.x * mapsPerGroup;
-	const int nMaps = (int)((maps - firstMap < (long)mapsPerGroup) ? (maps - firstMap) : (long)mapsPerGroup);
-	const int nCells = nMaps * cells, nWin = nMaps * windows;
-	const size_t g0 = (size_t)firstMap * cells;
-	const int lead = (int)(g0 & 3);
-	const int nVec = (lead + nCells + 3) >> 2;
-	const size_t vbase = g0 - lead; // multiple of four floats
 	const int tid = threadIdx.x;
+	constexpr int NC = (KS + ST - 1) / ST;
 
-	// ---- stage the maps and the pooled gradient
 	{
-		float4 t[kVecPerThread];
+		const PoolGroup cur = pool_group((long)blockIdx.x, mapsPerGroup, maps, cells, windows);
+		// ---- global -> registers (every load of the thread in flight at once) -> LDS.  One group per workgroup:
+		// a workgroup that walks several groups, with or without the next group's loads held in registers across
+		// the work on the current one, was measured and is slower (86 resp. 110 registers instead of 56: the
+		// kernel is bound by latency, i.e. by how many workgroups a compute unit holds).
+		{
+			float4 t[kPoolVecPerThread];
+			float d[kPoolWinPerThread];
+			pool_group_load(cur, z_act, delta, tid, t, d);
 #pragma unroll
-		for (int k = 0; k < kVecPerThread; k++) {
-			const int v = tid + 256 * k;
-			const int e0 = 4 * v - lead;
-			t[k] = make_float4(0.f, 0.f, 0.f, 0.f);
-			if (v < nVec) {
-				if (e0 >= 0 && e0 + 3 < nCells) {
-					t[k] = *reinterpret_cast<const float4 *>(z_act + vbase + 4 * (size_t)v);
-				} else {
-					if (e0 >= 0 && e0 < nCells) t[k].x = z_act[vbase + 4 * (size_t)v];
-					if (e0 + 1 >= 0 && e0 + 1 < nCells) t[k].y = z_act[vbase + 4 * (size_t)v + 1];
-					if (e0 + 2 >= 0 && e0 + 2 < nCells) t[k].z = z_act[vbase + 4 * (size_t)v + 2];
-					if (e0 + 3 >= 0 && e0 + 3 < nCells) t[k].w = z_act[vbase + 4 * (size_t)v + 3];
-				}
+			for (int k = 0; k < kPoolVecPerThread; k++) {
+				const int v = tid + 256 * k;
+				if (v < cur.nVec) *reinterpret_cast<float4 *>(zs + 4 * v) = t[k];
+			}
+#pragma unroll
+			for (int k = 0; k < kPoolWinPerThread; k++) {
+				const int w = tid + 256 * k;
+				if (w < cur.nWin) dl[w] = d[k];
 			}
 		}
-		float d[kWinPerThread];
-#pragma unroll
-		for (int k = 0; k < kWinPerThread; k++) {
-			const int w = tid + 256 * k;
-			d[k] = (w < nWin) ? delta[(size_t)firstMap * windows + w] : 0.f;
-		}
-#pragma unroll
-		for (int k = 0; k < kVecPerThread; k++) {
-			const int v = tid + 256 * k;
-			if (v < nVec) *reinterpret_cast<float4 *>(zs + 4 * v) = t[k];
-		}
-#pragma unroll
-		for (int k = 0; k < kWinPerThread; k++) {
-			const int w = tid + 256 * k;
-			if (w < nWin) dl[w] = d[k];
-		}
-	}
-	__syncthreads();
+		__syncthreads();
 
-	// ---- one scan per window: first maximum in memory order (strict >), offset inside its map
-	for (int w = tid; w < nWin; w += 256) {
-		uint32_t m, r, oa, ob;
-		divWindows.divmod((uint32_t)w, m, r);
-		g.divOutB.divmod(r, oa, ob);
-		const float *zmap = zs + lead + (int)m * cells;
-		const int a0 = (int)oa * ST - g.padding, b0 = (int)ob * ST - g.padding;
-		float best = -FLT_MAX;
-		int at = -1;
+		// ---- one scan per window: first maximum in memory order (strict >), offset inside its map
+		for (int w = tid; w < cur.nWin; w += 256) {
+			uint32_t m, r, oa, ob;
+			divWindows.divmod((uint32_t)w, m, r);
+			g.divOutB.divmod(r, oa, ob);
+			const float *zmap = zs + cur.lead + (int)m * cells;
+			const int a0 = (int)oa * ST - g.padding, b0 = (int)ob * ST - g.padding;
+			float best = -FLT_MAX;
+			int at = -1;
 #pragma unroll
-		for (int da = 0; da < KS; da++) {
-			const int a = a0 + da;
-			if (a < 0 || a >= g.inA) continue;
+			for (int da = 0; da < KS; da++) {
+				const int a = a0 + da;
+				if (a < 0 || a >= g.inA) continue;
 #pragma unroll
-			for (int db = 0; db < KS; db++) {
-				const int b = b0 + db;
-				if (b < 0 || b >= g.inB) continue;
-				const float t = zmap[a * g.inB + b];
-				if (t > best) {
-					best = t;
-					at = a * g.inB + b;
+				for (int db = 0; db < KS; db++) {
+					const int b = b0 + db;
+					if (b < 0 || b >= g.inB) continue;
+					const float zv = zmap[a * g.inB + b];
+					if (zv > best) {
+						best = zv;
+						at = a * g.inB + b;
+					}
 				}
 			}
+			arg[w] = at;
 		}
-		arg[w] = at;
-	}
-	__syncthreads();
+		__syncthreads();
 
-	// ---- every cell gathers from the windows that contain it
-	for (int v = tid; v < nVec; v += 256) {
-		const int e0 = 4 * v - lead;
-		float acc[4], zo[4];
+		// ---- every cell gathers from the windows that contain it: at most NC = ceil(KS / ST) along each axis, the
+		// last of them (a + padding) / ST; all candidates are read at once and added in ascending window order
+		for (int v = tid; v < cur.nVec; v += 256) {
+			const int e0 = 4 * v - cur.lead;
+			float acc[4], zo[4];
 #pragma unroll
-		for (int e = 0; e < 4; e++) {
-			const int i = e0 + e;
-			acc[e] = 0.f;
-			zo[e] = zs[4 * v + e];
-			if (i < 0 || i >= nCells) continue;
-			uint32_t m, r, a, b;
-			divCells.divmod((uint32_t)i, m, r);
-			g.divInB.divmod(r, a, b);
-			int oaHi = ((int)a + g.padding) / ST, obHi = ((int)b + g.padding) / ST;
-			int oaLo = ((int)a + g.padding - KS + ST) / ST, obLo = ((int)b + g.padding - KS + ST) / ST;
-			if ((int)a + g.padding - KS + 1 <= 0) oaLo = 0;
-			if ((int)b + g.padding - KS + 1 <= 0) obLo = 0;
-			if (oaHi >= g.outA) oaHi = g.outA - 1;
-			if (obHi >= g.outB) obHi = g.outB - 1;
-			const int wbase = (int)m * windows;
-			for (int oa = oaLo; oa <= oaHi; oa++)
-				for (int ob = obLo; ob <= obHi; ob++) {
-					const int w = wbase + oa * g.outB + ob;
-					if (arg[w] == (int)r) acc[e] += dl[w];
+			for (int e = 0; e < 4; e++) {
+				const int i = e0 + e;
+				acc[e] = 0.f;
+				zo[e] = zs[4 * v + e];
+				const bool live = i >= 0 && i < cur.nCells;
+				uint32_t m, r, a, b;
+				divCells.divmod((uint32_t)(live ? i : 0), m, r);
+				g.divInB.divmod(r, a, b);
+				const int ta = (int)a + g.padding, tb = (int)b + g.padding;
+				const int oaHi = ta / ST, obHi = tb / ST;
+				const int wbase = (int)m * windows;
+				int hit[NC][NC];
+				float dv[NC][NC];
+#pragma unroll
+				for (int da = NC - 1; da >= 0; da--) {
+					const int oa = oaHi - da;
+					const bool okA = live && oa >= 0 && oa < g.outA && ta - oa * ST < KS;
+#pragma unroll
+					for (int db = NC - 1; db >= 0; db--) {
+						const int ob = obHi - db;
+						const bool ok = okA && ob >= 0 && ob < g.outB && tb - ob * ST < KS;
+						const int w = ok ? wbase + oa * g.outB + ob : 0;
+						hit[da][db] = ok ? arg[w] : -2;
+						dv[da][db] = dl[w];
+					}
 				}
-		}
-		const size_t at = vbase + 4 * (size_t)v;
-		const bool whole = e0 >= 0 && e0 + 3 < nCells;
-		if (dxPool) {
-			if (whole) {
-				*reinterpret_cast<float4 *>(dxPool + at) = make_float4(acc[0], acc[1], acc[2], acc[3]);
-			} else {
 #pragma unroll
-				for (int e = 0; e < 4; e++)
-					if (e0 + e >= 0 && e0 + e < nCells) dxPool[at + e] = acc[e];
+				for (int da = NC - 1; da >= 0; da--)
+#pragma unroll
+					for (int db = NC - 1; db >= 0; db--)
+						if (hit[da][db] == (int)r) acc[e] += dv[da][db];
 			}
-		}
-		if constexpr (FUSE_ACT) {
-			float zi[4] = { 0.f, 0.f, 0.f, 0.f };
-			if (z_in) {
+			const size_t at = cur.vbase + 4 * (size_t)v;
+			const bool whole = e0 >= 0 && e0 + 3 < cur.nCells;
+			if (dxPool) {
 				if (whole) {
-					const float4 q = *reinterpret_cast<const float4 *>(z_in + at);
-					zi[0] = q.x, zi[1] = q.y, zi[2] = q.z, zi[3] = q.w;
+					store4(dxPool + at, make_float4(acc[0], acc[1], acc[2], acc[3]), streamPool);
 				} else {
 #pragma unroll
 					for (int e = 0; e < 4; e++)
-						if (e0 + e >= 0 && e0 + e < nCells) zi[e] = z_in[at + e];
+						if (e0 + e >= 0 && e0 + e < cur.nCells) dxPool[at + e] = acc[e];
 				}
 			}
-			float r4[4];
+			if constexpr (FUSE_ACT) {
+				float zi[4] = { 0.f, 0.f, 0.f, 0.f };
+				if (z_in) {
+					if (whole) {
+						const float4 zq = *reinterpret_cast<const float4 *>(z_in + at);
+						zi[0] = zq.x, zi[1] = zq.y, zi[2] = zq.z, zi[3] = zq.w;
+					} else {
 #pragma unroll
-			for (int e = 0; e < 4; e++) r4[e] = acc[e] * act_derivative(actFun, zi[e], zo[e]);
-			if (whole) {
-				*reinterpret_cast<float4 *>(dxAct + at) = make_float4(r4[0], r4[1], r4[2], r4[3]);
-			} else {
+						for (int e = 0; e < 4; e++)
+							if (e0 + e >= 0 && e0 + e < cur.nCells) zi[e] = z_in[at + e];
+					}
+				}
+				float r4[4];
 #pragma unroll
-				for (int e = 0; e < 4; e++)
-					if (e0 + e >= 0 && e0 + e < nCells) dxAct[at + e] = r4[e];
+				for (int e = 0; e < 4; e++) r4[e] = acc[e] * act_derivative(actFun, zi[e], zo[e]);
+				if (whole) {
+					*reinterpret_cast<float4 *>(dxAct + at) = make_float4(r4[0], r4[1], r4[2], r4[3]);
+				} else {
+#pragma unroll
+					for (int e = 0; e < 4; e++)
+						if (e0 + e >= 0 && e0 + e < cur.nCells) dxAct[at + e] = r4[e];
+				}
 			}
 		}
 	}
@@ -879,20 +935,6 @@ __global__ void __launch_bounds__(256) sum_slabs_kernel(float *base, int splits,
 	for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += step) base[i] = load_sum1(base + i, splits, stride);
 }
 
-// 16-byte store; stream: nothing reads the value again soon and the tensor is larger than the caches
-// can usefully hold, so it is written past them (measured on a 67 MB tensor: the pass 44 -> 36.5 us; on
-// a 34 MB one the plain store is the faster)
-__device__ __forceinline__ void store4(float *p, float4 v, bool stream)
-{
-	if (stream) {
-		typedef float v4f __attribute__((ext_vector_type(4)));
-		v4f t = { v.x, v.y, v.z, v.w };
-		__builtin_nontemporal_store(t, reinterpret_cast<v4f *>(p));
-	} else {
-		*reinterpret_cast<float4 *>(p) = v;
-	}
-}
-
 // One (channel, segment) per workgroup.  POOL 0: 2x2 / stride 2 max pool (B % 4 == 0, A even), the
 // unit of work is a 2 x 4 patch; POOL 2: no pooling, the unit is a 16-byte group; POOL 3: 2x2 / stride 2
 // max pool of maps with B == 2, where pooled cell q of a channel is its 16-byte group q.  z_act == nullptr:
@@ -1344,9 +1386,10 @@ int fitre_hip_pool_act_backward(int poolType, int actFun, const float *delta, co
 			    delta, act_needs_zin(actFun) ? z_in : nullptr, z_act, inA, inB, maps, actFun, dxPool, dxAct);
 		else if (grouped) {
 			const int per = maps_per_group(inA * inB, outA * outB, maps);
-			maxpool_maps_backward_kernel<true, 3, 2><<<(unsigned)((maps + per - 1) / per), 256, maps_group_lds(inA * inB, outA * outB, per), stream()>>>(
+			const long groups = (maps + per - 1) / per;
+			maxpool_maps_backward_kernel<true, 3, 2><<<(unsigned)groups, 256, maps_group_lds(inA * inB, outA * outB, per), stream()>>>(
 			    delta, act_needs_zin(actFun) ? z_in : nullptr, z_act, g, per, maps, FastDiv((uint32_t)(inA * inB)),
-			    FastDiv((uint32_t)(outA * outB)), actFun, dxPool, dxAct);
+			    FastDiv((uint32_t)(outA * outB)), actFun, dxPool, dxAct, 4.0 * (double)total >= 48.0 * 1024 * 1024);
 		} else if (perMap)
 			maxpool_map_backward_kernel<true><<<(unsigned)maps, 256, 0, stream()>>>(delta, act_needs_zin(actFun) ? z_in : nullptr, z_act, g,
 			                                                                      actFun, dxPool, dxAct);
@@ -1392,9 +1435,10 @@ int fitre_hip_pool_backward(int poolType, const float *delta, const float *z_in,
 			    delta, nullptr, z_in, inA, inB, maps, CNN_ACT_NONE, out, nullptr);
 		else if (perMap && ksize == 3 && stride == 2 && aligned16(z_in) && aligned16(out)) {
 			const int per = maps_per_group(inA * inB, outA * outB, maps);
-			maxpool_maps_backward_kernel<false, 3, 2><<<(unsigned)((maps + per - 1) / per), 256, maps_group_lds(inA * inB, outA * outB, per), stream()>>>(
+			const long groups = (maps + per - 1) / per;
+			maxpool_maps_backward_kernel<false, 3, 2><<<(unsigned)groups, 256, maps_group_lds(inA * inB, outA * outB, per), stream()>>>(
 			    delta, nullptr, z_in, g, per, maps, FastDiv((uint32_t)(inA * inB)), FastDiv((uint32_t)(outA * outB)), CNN_ACT_NONE, out,
-			    nullptr);
+			    nullptr, false);
 		} else if (perMap)
 			maxpool_map_backward_kernel<false><<<(unsigned)maps, 256, 0, stream()>>>(delta, nullptr, z_in, g, CNN_ACT_NONE, out, nullptr);
 		else

@@ -123,6 +123,9 @@ static size_t backward_side_ws_bytes(const CNN_MODEL *model, int batch)
 	for (int i = 0; i < model->cLayers; i++) {
 		fitre_conv_shape s = conv_shape(&model->convLayer[i], batch);
 		need = max_sz(need, fitre_hip_conv_weight_grad_workspace(&s));
+		if (!has_bn(&model->convLayer[i]))
+			need = max_sz(need, fitre_hip_channel_sum_workspace(model->convLayer[i].outChannels,
+			                                                    (long)batch * model->convLayer[i].outWidth * model->convLayer[i].outHeight));
 	}
 	for (int i = 0; i < model->lLayers; i++) {
 		const FC_LAYER *f = &model->fcLayer[i];
@@ -367,9 +370,7 @@ void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, 
 			HIP_CALL(fitre_hip_pool_act_backward(p->type, act, dview.base, actIn, actOut, l->outChannels, n, p->width, p->height,
 			                                     p->pSize, p->stride, p->padding, p->outWidth, p->outHeight, dslab,
 			                                     dslab + l->activationOffset));
-			cur = dslab + l->activationOffset;
-			if (model->bias != 0)
-				HIP_CALL(fitre_hip_channel_sum(cur, l->outChannels, perChannel, gradient + bOffsets[c], bnWs, bnBytes));
+			cur = dslab + l->activationOffset; /* its channel sums (the bias gradient) are taken on lane 1, below */
 		}
 
 		const real *input = (c == 0) ? data->currentBatch : z + zOffsets[c] + model->convLayer[c - 1].outputOffset;
@@ -393,6 +394,9 @@ void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, 
 		}
 		HIP_CALL(fitre_hip_lane_wait(1, 0));
 		HIP_CALL(fitre_hip_lane_select(1));
+		/* without batch norm the bias gradient is a pass of its own over delta; nothing in the chain reads it */
+		if (!has_bn(l) && model->bias != 0)
+			HIP_CALL(fitre_hip_channel_sum(cur, l->outChannels, perChannel, gradient + bOffsets[c], sideWs, sideBytes));
 		HIP_CALL(fitre_hip_conv_weight_grad(&shape, input, cur, gradient + wOffsets[c], sideWs, sideBytes));
 		HIP_CALL(fitre_hip_lane_select(0));
 	}

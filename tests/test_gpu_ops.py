@@ -158,6 +158,8 @@ POOL_GEOMS = [  # C, N, A(width), B(height), k, s, p
     (257, 13, 13, 13, 3, 2, 0), # 3341 maps: two maps per workgroup, the last workgroup with one
     (5, 3, 27, 27, 3, 2, 0),    # AlexNet's second pool
     (3, 5, 15, 9, 3, 2, 1),     # padding 1, rectangular, odd cell count
+    (3, 1367, 47, 47, 3, 2, 0), # 4101 large maps: two groups per workgroup (the second loaded while the first is
+                                # worked on), the last workgroup with one
 ]
 
 
