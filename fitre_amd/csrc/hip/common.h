@@ -40,6 +40,12 @@ int current_device();            // the device fitre_hip_init selected, -1 befor
 // Per-device set-up of the file that holds the batch-norm kernels (address of its static scratch
 // array on the current device); called by fitre_hip_init with the device current.
 int layers_device_setup(int device);
+// Shutdown hooks of the files that keep device buffers between calls (loss scratch, reduction partials, patch
+// decode tables): free them and forget their sizes, so that a later fitre_hip_init -- possibly on another device --
+// starts clean.  Called by fitre_hip_shutdown after every lane has drained.
+void layers_release();
+void elementwise_release();
+void conv_gemm_release();
 
 #define FITRE_HIP_TRY(expr)                                                                          \
 	do {                                                                                             \

@@ -11,6 +11,14 @@ namespace fitre {
 static unsigned long long *g_ktables[kMaxLanes] = {}; // one per lane
 static int g_ktable_caps[kMaxLanes] = {};
 
+void conv_gemm_release()
+{
+	for (int i = 0; i < kMaxLanes; i++) {
+		if (g_ktables[i]) (void)hipFree(g_ktables[i]);
+		g_ktables[i] = nullptr, g_ktable_caps[i] = 0;
+	}
+}
+
 // bn = tile extent along the positions, which fixes how the waves stride through a slice
 static int attach_patch_table(PatchGeom &g, int bn)
 {

@@ -177,6 +177,13 @@ constexpr int kRedBlocks = 1024;
 static double *g_partials = nullptr; // kRedBlocks doubles + 1 float result slot
 static float *g_host_result = nullptr;
 
+void elementwise_release()
+{
+	if (g_partials) (void)hipFree(g_partials);
+	if (g_host_result) (void)hipHostFree(g_host_result);
+	g_partials = nullptr, g_host_result = nullptr;
+}
+
 static int ensure_reduce_buffers()
 {
 	if (g_partials) return FITRE_OK;

@@ -1248,6 +1248,13 @@ static float *g_nll = nullptr;
 static int g_nll_rows = 0;
 static float *g_loss_host = nullptr;
 
+void layers_release()
+{
+	if (g_nll) (void)hipFree(g_nll);
+	if (g_loss_host) (void)hipHostFree(g_loss_host);
+	g_nll = nullptr, g_loss_host = nullptr, g_nll_rows = 0;
+}
+
 // =====================================================================
 // layout changes
 // =====================================================================
@@ -1668,7 +1675,7 @@ int fitre_hip_softmax_cross_entropy(const float *logits, const float *target, in
 	FITRE_REQUIRE(logits && target && probs && lossHost, "fitre_hip_softmax_cross_entropy: null pointer");
 	FITRE_REQUIRE(rows > 0 && classes > 0, "fitre_hip_softmax_cross_entropy: non-positive shape (%d x %d)", rows, classes);
 	if (rows > g_nll_rows) {
-		FITRE_HIP_TRY(hipStreamSynchronize(stream()));
+		FITRE_HIP_TRY(hipDeviceSynchronize()); // the buffer is shared by every lane
 		if (g_nll) FITRE_HIP_TRY(hipFree(g_nll));
 		g_nll = nullptr;
 		g_nll_rows = 0;

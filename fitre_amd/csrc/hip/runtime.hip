@@ -207,6 +207,9 @@ int fitre_hip_shutdown(void)
 	if (!g_ready) return FITRE_OK;
 	for (int i = 0; i < kLanes; i++) (void)hipStreamSynchronize(g_lanes[i]);
 	drain_pending();
+	layers_release();
+	elementwise_release();
+	conv_gemm_release();
 	for (hipEvent_t e : g_event_pool) (void)hipEventDestroy(e);
 	g_event_pool.clear();
 	for (int i = 0; i < kJoinEvents; i++) (void)hipEventDestroy(g_join[i]);

@@ -151,6 +151,13 @@ static size_t backward_ws_bytes(const CNN_MODEL *model, int batch)
 	return backward_chain_ws_bytes(model, batch) + backward_side_ws_bytes(model, batch) + backward_prepared_bytes(model, batch);
 }
 
+int fitreBackwardUnsupportedLayer(const CNN_MODEL *model)
+{
+	for (int c = 1; c < model->cLayers; c++)
+		if (model->convLayer[c].stride != 1) return c + 1;
+	return 0;
+}
+
 long cnnForwardMemRequired(CNN_MODEL *model)
 {
 	return (long)((forward_ws_bytes(model, model->batchSize) + sizeof(real) - 1) / sizeof(real));
@@ -261,6 +268,12 @@ void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, 
 	if (nc < 1 || n < 1 || n > model->batchSize) {
 		fprintf(stderr, "cnnBackward: needs at least one convolution layer and 1 <= batch (%d) <= model batch (%d)\n", n,
 		        model->batchSize);
+		exit(-1);
+	}
+	if (fitreBackwardUnsupportedLayer(model)) {
+		fprintf(stderr, "cnnBackward: convolution layer %d has stride %d; only the first layer may be strided (the input "
+		                "gradient is implemented for stride 1)\n",
+		        fitreBackwardUnsupportedLayer(model), model->convLayer[fitreBackwardUnsupportedLayer(model) - 1].stride);
 		exit(-1);
 	}
 	const CONV_LAYER *last = &model->convLayer[nc - 1];

@@ -295,6 +295,11 @@ void cnnHv(CNN_MODEL *model, DEVICE_DATASET *data, real *z, real *probs, real *l
 		fprintf(stderr, "cnnHv: needs convolution and linear layers and 1 <= batch (%d) <= model batch (%d)\n", n, model->batchSize);
 		exit(-1);
 	}
+	if (fitreBackwardUnsupportedLayer(model)) {
+		fprintf(stderr, "cnnHv: convolution layer %d has stride %d; only the first layer may be strided\n",
+		        fitreBackwardUnsupportedLayer(model), model->convLayer[fitreBackwardUnsupportedLayer(model) - 1].stride);
+		exit(-1);
+	}
 	const size_t dBytes = up256(sizeof(real) * (size_t)model->maxDeltaSize);
 	char *base = (char *)(((size_t)devPtr + 255) & ~(size_t)255);
 	real *rz = (real *)base;

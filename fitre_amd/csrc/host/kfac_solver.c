@@ -210,6 +210,12 @@ void subsampledTrustRegionKFAC(CNN_MODEL *model, DEVICE_DATASET *data, HOST_DATA
 	(void)master;
 	(void)slave;
 	const DATASET_TYPE datasetType = host != NULL ? host->datasetType : data->datasetType;
+	if (host != NULL && host->datasetType != data->datasetType) {
+		/* the training loop reads the host set's type, the per-pass sweeps the device set's: they must agree */
+		fprintf(stderr, "subsampledTrustRegionKFAC: data set type of the host set (%d) and of the device set (%d) differ\n",
+		        (int)host->datasetType, (int)data->datasetType);
+		exit(-1);
+	}
 	/* the third case keeps the training set in host memory and reads mini-batches from there
 	 * (selectHostMatrix, solvers/kfac_trust_region.cu:322-337) */
 	const int hostResident = datasetType == IMAGENET;
@@ -272,8 +278,13 @@ void subsampledTrustRegionKFAC(CNN_MODEL *model, DEVICE_DATASET *data, HOST_DATA
 	kfacInfo->dampedLambda = dampedLambda;
 
 	generateParamReport(model, kfacInfo, trParams);
-	fprintf(stderr, "Allocating Sampling Dataset... %d\n", model->batchSize);
-	allocSampledDataset(data, 2 * model->batchSize);
+	/* the sampling buffers stay with the data set: a second call of the solver reuses them (the reference allocates
+	 * them again on every call and never frees them) */
+	if (data->sampledTrainX == NULL || data->sampledTrainY == NULL || data->sampleSize < 2 * model->batchSize) {
+		fprintf(stderr, "Allocating Sampling Dataset... %d\n", model->batchSize);
+		/* buffers that are too small are left to their owner, which may be the caller */
+		allocSampledDataset(data, 2 * model->batchSize);
+	}
 
 	scratch->nextDevPtr = scratchBegin;
 	scratch->nextHostPtr = nextHostPtr;

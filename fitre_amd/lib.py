@@ -156,6 +156,7 @@ CNN_API = {
     "cnnForward": (f32, [pmodel, pdata, pscratch, vp, vp, vp, i32, i32, i32]),
     "cnnBackwardMemRequired": (lng, [pmodel]),
     "cnnBackward": (None, [pmodel, pdata, vp, vp, vp, vp, vp, vp, i32, i32, vp]),
+    "fitreBackwardUnsupportedLayer": (i32, [pmodel]),
     "evaluateCNNModel": (f32, [pmodel, pdata, pscratch, vp, vp, vp, i32, i32]),
     "computeCNNGradient": (f32, [pmodel, pdata, pscratch, vp, vp, vp, vp, vp, i32, i32, f32]),
     "computeAccuracy": (f32, [vp, vp, i32, i32, vp, pf32]),

@@ -88,6 +88,13 @@ long cnnBackwardMemRequired(CNN_MODEL *model);
  * delta and delta_new (each >= maxDeltaSize reals) are clobbered. */
 void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, real *gradient, real *dx,
                  real *delta, real *delta_new, int offset, int batchSize, real *hostPtr);
+/* Back-propagation goes through stride-1 convolutions only: every convolution layer above the first must have
+ * stride 1 (the first layer's input gradient is never taken, so its stride is free -- AlexNet's 11x11 / 4).  The
+ * reference's backpropConvolution (functions/dev_backprop_convolution.cu:173-247) has the same limit (its patch
+ * gather is written for stride 1).  Returns 0 when `model` can be back-propagated through, else the 1-based index of
+ * the first offending layer; cnnBackward and cnnHv call it before their first launch and exit(-1) with a message. */
+int fitreBackwardUnsupportedLayer(const CNN_MODEL *model);
+
 real evaluateCNNModel(CNN_MODEL *model, DEVICE_DATASET *data, SCRATCH_AREA *scratch, real *z,
                       real *probs, real *lossFuncErrors, int offset, int curBatchSize);
 /* forward + backward + gradient += weightDecay * weights; returns the loss. */

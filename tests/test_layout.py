@@ -212,3 +212,27 @@ def test_small_reference_networks():
     assert [(a.poolLayer[i].pSize, a.poolLayer[i].stride, a.poolLayer[i].padding, a.poolLayer[i].type) for i in range(2)] == [(3, 2, 1, 0)] * 2
     assert (a.poolLayer[0].outHeight, a.poolLayer[1].outHeight, a.fcLayer[0].in_) == (16, 8, 64 * 8 * 8)
     assert a.pSize == 4864 + 102464 + 1573248 + 73920 + 1930
+
+
+def test_strided_convolution_above_the_first_layer_is_rejected_before_any_launch():
+    """Back-propagation is implemented for stride-1 convolutions; a model with a strided layer above the first is
+    reported by fitreBackwardUnsupportedLayer, and cnnBackward exits with a message before it touches the device (run
+    in a child process: the reference's error convention is exit(-1))."""
+    import subprocess
+    import sys
+    ok = build_custom(2, 16, 16, 3, [dict(cout=4, k=5, stride=2, pad=2), dict(cout=4, k=3, pad=1)], [(3, 0)])
+    assert L.cnn.fitreBackwardUnsupportedLayer(C.byref(ok)) == 0           # a strided FIRST layer is fine (AlexNet)
+    bad = build_custom(2, 16, 16, 3, [dict(cout=4, k=3, pad=1), dict(cout=4, k=3, stride=2, pad=1)], [(3, 0)])
+    assert L.cnn.fitreBackwardUnsupportedLayer(C.byref(bad)) == 2
+    code = (
+        "import ctypes as C, sys\n"
+        "sys.path.insert(0, %r)\n"
+        "from fitre_amd import lib as L\n"
+        "from fitre_amd.harness import build_custom\n"
+        "from fitre_amd.structs import DEVICE_DATASET\n"
+        "m = build_custom(2, 16, 16, 3, [dict(cout=4, k=3, pad=1), dict(cout=4, k=3, stride=2, pad=1)], [(3, 0)])\n"
+        "L.cnn.cnnBackward(C.byref(m), C.byref(DEVICE_DATASET()), None, None, None, None, None, None, 0, 2, None)\n"
+        "print('returned')\n" % ROOT)
+    proc = subprocess.run([sys.executable, "-c", code], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=120)
+    assert proc.returncode != 0 and "returned" not in proc.stdout
+    assert "stride 2" in proc.stderr and "layer 2" in proc.stderr
