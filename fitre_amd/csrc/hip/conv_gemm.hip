@@ -3,6 +3,7 @@
 #include "conv3x3.h"
 #include "conv_common.h"
 #include "conv_quad.h"
+#include "conv_thin.h"
 
 namespace fitre {
 
@@ -390,7 +391,7 @@ int gemm_ex_batched(int batch, int transA, int transB, int M, int N, int K, floa
 
 // C(MxN) = alpha*op(A)*op(B) + beta*C (+ bias per row), column-major, for products far below one engine tile: sixteen
 // lanes share an output element, each takes every sixteenth reduction index, and their sums are combined by shuffles.
-constexpr double kSmallProductWork = 4.0e6; // multiply-adds
+constexpr double kSmallProductWork = 8.0e6; // multiply-adds (LeNet's first linear layer at batch 128: 6.1e6, 20 -> 8 us)
 __global__ void __launch_bounds__(256) small_product_kernel(int transA, int transB, int M, int N, int K, float alpha, const float *A,
                                                             int lda, const float *B, int ldb, float beta, float *C, int ldc,
                                                             const float *bias)
@@ -458,7 +459,8 @@ size_t fitre_hip_conv_weight_grad_workspace(const fitre_conv_shape *s)
 	}
 	if (c3_dw_eligible(s)) return c3_dw_workspace(s);
 	size_t general = plan_gemm_workspace(s->outChannels, (long)s->inChannels * s->ksize * s->ksize, (long)s->samples * s->outA * s->outB);
-	if (thin_dw_eligible(s) && thin_dw_workspace(s) > general) return thin_dw_workspace(s);
+	if (thin_dw_eligible(s) && thin_dw_workspace(s) > general) general = thin_dw_workspace(s);
+	if (thin_dw_general_eligible(s) && thin_dw_general_workspace(s) > general) general = thin_dw_general_workspace(s);
 	return general;
 }
 
@@ -473,6 +475,8 @@ int fitre_hip_conv_weight_grad(const fitre_conv_shape *s, const float *x, const 
 	if (c3_dw_eligible(s)) return launch_c3_dw(s, x, delta, dW, ws, wsBytes);
 	if (thin_dw_eligible(s) && ws && wsBytes >= thin_dw_workspace(s) && ((((uintptr_t)delta) | ((uintptr_t)ws)) & 15) == 0)
 		return launch_thin_dw(s, x, delta, dW, ws);
+	if (thin_dw_general_eligible(s) && ws && wsBytes >= thin_dw_general_workspace(s) && ((((uintptr_t)ws) & 15) == 0))
+		return launch_thin_dw_general(s, x, delta, dW, ws);
 	const int I = s->outChannels, J = s->inChannels * s->ksize * s->ksize, R = s->samples * s->outA * s->outB;
 	GemmPlan plan = plan_gemm(I, J, R);
 	PlainParams pa{ delta, (uint32_t)((size_t)I * R * sizeof(float)), R, I };
@@ -505,6 +509,7 @@ int fitre_hip_conv_input_grad(const fitre_conv_shape *s, const float *delta, con
 	if (quad_usable(s, ws, wsBytes, quad_input_grad_workspace(s)) && (((((uintptr_t)dx) | ((uintptr_t)delta) | ((uintptr_t)w)) & 15) == 0))
 		return quad_input_grad(s, delta, w, nullptr, dx, ws, wsBytes, nullptr, nullptr);
 	if (c3_pos_eligible(s, true)) return launch_c3_pos<true>(s, delta, w, nullptr, dx, ws, wsBytes);
+	if (thin_dx_eligible(s) && s->inChannels <= 8) return launch_thin_dx(s, delta, w, dx);
 	const int I = s->inChannels, J = s->samples * s->inA * s->inB, R = s->outChannels * s->ksize * s->ksize;
 	GemmPlan plan = plan_gemm(I, J, R);
 	FlipWeightParams pa;

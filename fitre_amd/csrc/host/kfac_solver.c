@@ -278,13 +278,11 @@ void subsampledTrustRegionKFAC(CNN_MODEL *model, DEVICE_DATASET *data, HOST_DATA
 	kfacInfo->dampedLambda = dampedLambda;
 
 	generateParamReport(model, kfacInfo, trParams);
-	/* the sampling buffers stay with the data set: a second call of the solver reuses them (the reference allocates
-	 * them again on every call and never frees them) */
-	if (data->sampledTrainX == NULL || data->sampledTrainY == NULL || data->sampleSize < 2 * model->batchSize) {
-		fprintf(stderr, "Allocating Sampling Dataset... %d\n", model->batchSize);
-		/* buffers that are too small are left to their owner, which may be the caller */
-		allocSampledDataset(data, 2 * model->batchSize);
-	}
+	/* As in the reference, every call allocates its sampling buffers and leaves them to the caller, who frees
+	 * data->sampledTrainX / sampledTrainY with cuda_free when done with the data set (a caller that runs the solver
+	 * again on the same struct frees them in between). */
+	fprintf(stderr, "Allocating Sampling Dataset... %d\n", model->batchSize);
+	allocSampledDataset(data, 2 * model->batchSize);
 
 	scratch->nextDevPtr = scratchBegin;
 	scratch->nextHostPtr = nextHostPtr;
