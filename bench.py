@@ -392,9 +392,9 @@ def kfac_leg(L, dev, gm, model, batch, passes):
 
     def inverses():
         L.cnn.computeOmegaZ(C.byref(info), C.byref(model), C.byref(gm.data), batch, None, gm.z, oinv, model.zOffsets,
-                            model.zztOffsets, ws2, None)
+                            model.zztOffsets, ws2, None, None, None, None)
         L.cnn.computeLambdaDelta(C.byref(info), C.byref(model), batch, gm.dx, None, linv, model.zOffsets, model.zztOffsets,
-                                 ws2, None)
+                                 ws2, None, None, None, None)
 
     inverses()
     dev.sync()

@@ -359,6 +359,31 @@ __global__ void __launch_bounds__(256) copy_2d_kernel(const float *src, long lds
 	}
 }
 
+// C(m x n) = alpha * op(A) + beta * op(B), column-major; one workgroup per 32 x 32 tile of C.  A transposed
+// operand's tile is read along ITS contiguous index and turned in LDS (33-word rows: conflict-free), so every
+// global access is coalesced.
+__global__ void __launch_bounds__(256) geam_kernel(int transA, int transB, int m, int n, float alpha, const float *A, int lda, float beta,
+                                                   const float *B, int ldb, float *C, int ldc)
+{
+	__shared__ float ta[32][33], tb[32][33];
+	const int r0 = blockIdx.x * 32, c0 = blockIdx.y * 32;
+	const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5; // ty = 0..7
+	// transposed operands: element (r, c) of op(X) is X[r * ld + c]: read with c contiguous
+	if (A && transA)
+		for (int q = ty; q < 32; q += 8) ta[q][tx] = (r0 + q < m && c0 + tx < n) ? A[(size_t)(r0 + q) * lda + c0 + tx] : 0.f;
+	if (B && transB)
+		for (int q = ty; q < 32; q += 8) tb[q][tx] = (r0 + q < m && c0 + tx < n) ? B[(size_t)(r0 + q) * ldb + c0 + tx] : 0.f;
+	__syncthreads();
+	for (int q = ty; q < 32; q += 8) {
+		const int r = r0 + tx, c = c0 + q;
+		if (r >= m || c >= n) continue;
+		float v = 0.f;
+		if (A) v += alpha * (transA ? ta[tx][q] : A[(size_t)c * lda + r]);
+		if (B) v += beta * (transB ? tb[tx][q] : B[(size_t)c * ldb + r]);
+		C[(size_t)c * ldc + r] = v;
+	}
+}
+
 } // namespace fitre
 
 using namespace fitre;
@@ -532,6 +557,25 @@ int fitre_hip_random_normal(float *out, long n)
 	random_normal_kernel<<<blocks_for((n + 1) / 2, 1024, 4096), 256, 0, stream()>>>(out, n, g_rng_seed, g_rng_next);
 	g_rng_next += (unsigned long long)(2 * ((n + 1) / 2));
 	return check_launch("random_normal_kernel");
+}
+
+int fitre_hip_geam(int transA, int transB, int m, int n, float alpha, const float *A, int lda, float beta, const float *B, int ldb,
+                   float *C, int ldc)
+{
+	EW_CHECK("fitre_hip_geam", C && m > 0 && n > 0);
+	FITRE_REQUIRE((transA == 0 || transA == 1) && (transB == 0 || transB == 1), "fitre_hip_geam: bad transpose flags");
+	FITRE_REQUIRE(A || alpha == 0.f, "fitre_hip_geam: A is null with alpha != 0");
+	FITRE_REQUIRE(B || beta == 0.f, "fitre_hip_geam: B is null with beta != 0");
+	FITRE_REQUIRE(ldc >= m && (!A || lda >= (transA ? n : m)) && (!B || ldb >= (transB ? n : m)),
+	              "fitre_hip_geam: leading dimension too small");
+	// in-place use as cuBLAS allows it: C may be A (resp. B) only when that operand is not transposed and shares ldc
+	FITRE_REQUIRE(!(C == A && (transA || lda != ldc)) && !(C == B && (transB || ldb != ldc)),
+	              "fitre_hip_geam: in-place only for an untransposed operand with the same leading dimension");
+	LaunchScope scope(FITRE_KC_BLAS1, 4.0 * (double)m * n * (1 + (A && alpha != 0.f ? 1 : 0) + (B && beta != 0.f ? 1 : 0)));
+	dim3 grid((m + 31) / 32, (n + 31) / 32);
+	geam_kernel<<<grid, 256, 0, stream()>>>(transA, transB, m, n, alpha, (alpha != 0.f) ? A : nullptr, lda, beta,
+	                                        (beta != 0.f) ? B : nullptr, ldb, C, ldc);
+	return check_launch("geam_kernel");
 }
 
 int fitre_hip_copy_2d(float *dst, long ldd, const float *src, long lds_, int rows, int cols)

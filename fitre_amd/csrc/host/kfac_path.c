@@ -352,9 +352,9 @@ static int omega_items(INVERSE_ITEM *items, const KFAC_CURVATURE_INFO *kfac_info
 
 void computeOmegaZ(KFAC_CURVATURE_INFO *kfac_info, CNN_MODEL *model, DEVICE_DATASET *data, int samples,
                    real *dampedInput, real *dampedZ, real *omegaZInv, int *zOffsets, int *zztOffsets, real *devPtr,
-                   real *pageLckPtr)
+                   real *pageLckPtr, cublasHandle_t blasHandle, cudaStream_t curStream, cusolverDnHandle_t curHandle)
 {
-	(void)pageLckPtr;
+	(void)pageLckPtr, (void)blasHandle, (void)curStream, (void)curHandle;
 	OMEGA_CTX ctx = { model, data, samples, model->bias != 0, dampedInput, dampedZ, zOffsets, zztOffsets };
 	INVERSE_ITEM items[KFAC_MAX_ITEMS];
 	const int count = omega_items(items, kfac_info, model, &ctx, omegaZInv);
@@ -412,9 +412,10 @@ static int lambda_items(INVERSE_ITEM *items, const KFAC_CURVATURE_INFO *kfac_inf
 }
 
 void computeLambdaDelta(KFAC_CURVATURE_INFO *kfac_info, CNN_MODEL *model, int samples, real *dx, real *dampedLambda,
-                        real *lambdaGInv, int *zOffsets, int *zztOffsets, real *devPtr, real *pageLckPtr)
+                        real *lambdaGInv, int *zOffsets, int *zztOffsets, real *devPtr, real *pageLckPtr,
+                        cublasHandle_t blasHandle, cudaStream_t curStream, cusolverDnHandle_t curHandle)
 {
-	(void)pageLckPtr;
+	(void)pageLckPtr, (void)blasHandle, (void)curStream, (void)curHandle;
 	LAMBDA_CTX ctx = { model, samples, dx, dampedLambda, zOffsets, zztOffsets };
 	INVERSE_ITEM items[KFAC_MAX_ITEMS];
 	const int count = lambda_items(items, kfac_info, model, &ctx, lambdaGInv);

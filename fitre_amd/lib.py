@@ -49,6 +49,7 @@ HIP_API = {
     "fitre_hip_scal": (i32, [i32, f32, vp]),
     "fitre_hip_copy": (i32, [i32, vp, vp]),
     "fitre_hip_copy_2d": (i32, [vp, lng, vp, lng, i32, i32]),
+    "fitre_hip_geam": (i32, [i32, i32, i32, i32, f32, vp, i32, f32, vp, i32, vp, i32]),
     "fitre_hip_dot": (i32, [i32, vp, vp, pf32]),
     "fitre_hip_nrm2": (i32, [i32, vp, pf32]),
     "fitre_hip_asum": (i32, [i32, vp, pf32]),
@@ -182,8 +183,8 @@ CNN_API = {
     "computeLambdaDeltaFactors": (None, [pkfac, pmodel, i32, vp, vp, vp, pi32, pi32, vp]),
     "kfacInverseMemRequired": (lng, [pmodel, i32]),
     "computeMatrixInverse": (None, [vp, vp, i32, vp, f32, f32]),
-    "computeOmegaZ": (None, [pkfac, pmodel, pdata, i32, vp, vp, vp, pi32, pi32, vp, vp]),
-    "computeLambdaDelta": (None, [pkfac, pmodel, i32, vp, vp, vp, pi32, pi32, vp, vp]),
+    "computeOmegaZ": (None, [pkfac, pmodel, pdata, i32, vp, vp, vp, pi32, pi32, vp, vp, vp, vp, vp]),
+    "computeLambdaDelta": (None, [pkfac, pmodel, i32, vp, vp, vp, pi32, pi32, vp, vp, vp, vp, vp]),
     "computeOmegaZAndLambdaDelta": (None, [pkfac, pmodel, pdata, i32, vp, vp, vp, vp, pi32, pi32, vp]),
     "kfacNaturalGradientMemRequired": (lng, [pmodel]),
     "computeNaturalGradient": (None, [pmodel, pkfac, vp, vp]),

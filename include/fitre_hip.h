@@ -118,6 +118,12 @@ int fitre_hip_copy(int n, const float *x, float *y);                      /* y =
  * uses it (solvers/kfac_inverses.cu:596-600, kfac_natural_gradient.cu:107-111), widths in elements.
  * Leading dimensions below `rows` are allowed (ld 1 with rows 1 walks a strided vector). */
 int fitre_hip_copy_2d(float *dst, long ldd, const float *src, long lds, int rows, int cols);
+/* C(m x n) = alpha * op(A) + beta * op(B), column-major, with the argument meaning of cublasDgeam as the
+ * reference's solvers use it to transpose (solvers/kfac_natural_gradient.cu:166-170: OP_T, OP_N, beta = 0, B = NULL).
+ * transA / transB: 0 = N, 1 = T.  A null operand needs a zero coefficient; C may alias an untransposed operand
+ * that has the same leading dimension. */
+int fitre_hip_geam(int transA, int transB, int m, int n, float alpha, const float *A, int lda, float beta, const float *B,
+                   int ldb, float *C, int ldc);
 int fitre_hip_dot(int n, const float *x, const float *y, float *result);  /* host result, complete on return */
 int fitre_hip_nrm2(int n, const float *x, float *result);                 /* host result */
 int fitre_hip_asum(int n, const float *x, float *result);                 /* host result */

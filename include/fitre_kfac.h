@@ -80,11 +80,18 @@ long kfacInverseMemRequired(CNN_MODEL *model, int samples);
  * the reference) and its damped inverse, stored at omegaZInv + OmegaZOffsets[l] resp.
  * lambdaGInv + LambdaGOffsets[l].  Damping: kfac_info->regLambda + kfac_info->dampGamma on the diagonal.
  * pageLckPtr is unused (the reference reads cuSOLVER's devInfo through it). */
+/* The three trailing arguments are the reference's vendor handles (cublasHandle_t, cudaStream_t,
+ * cusolverDnHandle_t, solvers/kfac_inverses.h:28-34), kept so that its solver source compiles against this
+ * header unchanged; they are opaque pointers and are ignored (the device layer owns its streams). */
+typedef void *cublasHandle_t;
+typedef void *cudaStream_t;
+typedef void *cusolverDnHandle_t;
 void computeOmegaZ(KFAC_CURVATURE_INFO *kfac_info, CNN_MODEL *model, DEVICE_DATASET *data, int samples,
                    real *dampedInput, real *dampedZ, real *omegaZInv, int *zOffsets, int *zztOffsets, real *devPtr,
-                   real *pageLckPtr);
+                   real *pageLckPtr, cublasHandle_t blasHandle, cudaStream_t curStream, cusolverDnHandle_t curHandle);
 void computeLambdaDelta(KFAC_CURVATURE_INFO *kfac_info, CNN_MODEL *model, int samples, real *dx, real *dampedLambda,
-                        real *lambdaGInv, int *zOffsets, int *zztOffsets, real *devPtr, real *pageLckPtr);
+                        real *lambdaGInv, int *zOffsets, int *zztOffsets, real *devPtr, real *pageLckPtr,
+                        cublasHandle_t blasHandle, cudaStream_t curStream, cusolverDnHandle_t curHandle);
 
 /* Both passes as one (no counterpart in the reference, whose solver calls them one after the other): the small
  * output-side inverses run on the lanes that the large input-side ones leave idle.  Same results, written to

@@ -410,8 +410,8 @@ def test_model_inverses_and_natural_gradient(dev, oracle64, name):
                                model.zztOffsets, ws)
     L.cnn.computeLambdaDeltaFactors(C.byref(info), C.byref(model), batch, gm.dx, None, lfac, model.zOffsets, model.zztOffsets, ws)
     L.cnn.computeOmegaZ(C.byref(info), C.byref(model), C.byref(gm.data), batch, None, gm.z, oinv, model.zOffsets,
-                        model.zztOffsets, ws, None)
-    L.cnn.computeLambdaDelta(C.byref(info), C.byref(model), batch, gm.dx, None, linv, model.zOffsets, model.zztOffsets, ws, None)
+                        model.zztOffsets, ws, None, None, None, None)
+    L.cnn.computeLambdaDelta(C.byref(info), C.byref(model), batch, gm.dx, None, linv, model.zOffsets, model.zztOffsets, ws, None, None, None, None)
     fac_o, fac_l = dev.download(ofac, tot_o), dev.download(lfac, tot_l)
     got_o, got_l = dev.download(oinv, tot_o), dev.download(linv, tot_l)
     bias = model.bias != 0
@@ -472,8 +472,8 @@ def test_both_inverse_passes_as_one(dev, name):
     o1, l1, o2, l2 = dev.zeros(tot_o), dev.zeros(tot_l), dev.zeros(tot_o), dev.zeros(tot_l)
     ws = dev.alloc(4 * L.cnn.kfacInverseMemRequired(C.byref(model), batch) + 512)
     L.cnn.computeOmegaZ(C.byref(info), C.byref(model), C.byref(gm.data), batch, None, gm.z, o1, model.zOffsets, model.zztOffsets,
-                        ws, None)
-    L.cnn.computeLambdaDelta(C.byref(info), C.byref(model), batch, gm.dx, None, l1, model.zOffsets, model.zztOffsets, ws, None)
+                        ws, None, None, None, None)
+    L.cnn.computeLambdaDelta(C.byref(info), C.byref(model), batch, gm.dx, None, l1, model.zOffsets, model.zztOffsets, ws, None, None, None, None)
     info.OmegaZInv, info.LambdaGInv = o2.value, l2.value
     L.cnn.computeOmegaZAndLambdaDelta(C.byref(info), C.byref(model), C.byref(gm.data), batch, None, gm.z, gm.dx, None,
                                       model.zOffsets, model.zztOffsets, ws)
@@ -515,8 +515,8 @@ def test_vgg11_full_size_factor_inverses_with_the_benchmark_damping(dev):
                                model.zztOffsets, ws)
     L.cnn.computeLambdaDeltaFactors(C.byref(info), C.byref(model), batch, gm.dx, None, lfac, model.zOffsets, model.zztOffsets, ws)
     L.cnn.computeOmegaZ(C.byref(info), C.byref(model), C.byref(gm.data), batch, None, gm.z, oinv, model.zOffsets,
-                        model.zztOffsets, ws, None)
-    L.cnn.computeLambdaDelta(C.byref(info), C.byref(model), batch, gm.dx, None, linv, model.zOffsets, model.zztOffsets, ws, None)
+                        model.zztOffsets, ws, None, None, None, None)
+    L.cnn.computeLambdaDelta(C.byref(info), C.byref(model), batch, gm.dx, None, linv, model.zOffsets, model.zztOffsets, ws, None, None, None, None)
     assert info.OmegaZOffsets[6] - info.OmegaZOffsets[5] == 4609 * 4609
     for F, X, offs, what in ((dev.download(ofac, tot_o), dev.download(oinv, tot_o), info.OmegaZOffsets, "omega"),
                              (dev.download(lfac, tot_l), dev.download(linv, tot_l), info.LambdaGOffsets, "lambda")):

@@ -77,9 +77,9 @@ def test_kfac_trust_region_minibatches(dev):
             L.cnn.cnnBackward(C.byref(model), C.byref(data), at(ws, 2 * model.maxDeltaSize), gm.z, dist_grad, dist_dx, dist_err,
                               ws, offset, batch, None)
             L.cnn.computeOmegaZ(C.byref(info), C.byref(model), C.byref(data), batch, None, gm.z, oinv, model.zOffsets,
-                                model.zztOffsets, ws, None)
+                                model.zztOffsets, ws, None, None, None, None)
             L.cnn.computeLambdaDelta(C.byref(info), C.byref(model), batch, dist_dx, None, linv, model.zOffsets, model.zztOffsets,
-                                     ws, None)
+                                     ws, None, None, None, None)
             L.cnn.computeNaturalGradient(C.byref(model), C.byref(info), ws, None)
             # quadratic model along the natural gradient; scales ngrad to the step
             m_err = L.cnn.computeQuadraticModel(C.byref(model), C.byref(data), gm.z, gm.probs, gm.errors, gm.dx, gm.grad, ngrad,

@@ -534,3 +534,30 @@ def test_empty_inputs(dev):
     s = conv_shape(0, 2, 2, 2, 2, 3, 1, 1)
     assert hip.fitre_hip_conv_weight_grad(C.byref(s), p, p, q, None, 0) == 2
     assert hip.fitre_hip_conv_input_grad(C.byref(s), p, p, q, None, 0) == 2
+
+
+@pytest.mark.parametrize("m,n", [(1, 1), (5, 7), (32, 32), (33, 65), (513, 4609), (300, 10)])
+@pytest.mark.parametrize("ta,tb", [(0, 0), (1, 0), (0, 1), (1, 1)])
+def test_geam(dev, m, n, ta, tb):
+    """C = alpha op(A) + beta op(B) (the reference's cublasDgeam, solvers/kfac_natural_gradient.cu:166-170) against
+    numpy on column-major operands with padded leading dimensions; the reference's own use (transpose: beta = 0, B null)
+    bit for bit."""
+    rng = np.random.default_rng(m * 7 + n + 2 * ta + tb)
+    lda, ldb, ldc = (n if ta else m) + 3, (n if tb else m) + 1, m + 2
+    a = rng.standard_normal(lda * (m if ta else n)).astype(np.float32)
+    b = rng.standard_normal(ldb * (m if tb else n)).astype(np.float32)
+    A = a.reshape((m if ta else n), lda).T[: (n if ta else m)]          # column-major view: A[r, c] = a[c * lda + r]
+    B = b.reshape((m if tb else n), ldb).T[: (n if tb else m)]
+    opA, opB = (A.T if ta else A), (B.T if tb else B)
+    pa, pb = dev.upload(a), dev.upload(b)
+    pc = dev.upload(np.full(ldc * n, 9.0, np.float32))
+    ok(hip.fitre_hip_geam(ta, tb, m, n, 0.75, pa, lda, -1.5, pb, ldb, pc, ldc))
+    got = dev.download(pc, ldc * n).reshape(n, ldc)
+    want = (np.float32(0.75) * opA + np.float32(-1.5) * opB).T                  # [c][r]
+    np.testing.assert_allclose(got[:, :m], want, rtol=1e-6, atol=1e-6)
+    assert (got[:, m:] == 9.0).all()                                          # the padding of C is left alone
+    ok(hip.fitre_hip_geam(ta, 0, m, n, 1.0, pa, lda, 0.0, None, m, pc, ldc))    # the transpose / copy use
+    np.testing.assert_array_equal(dev.download(pc, ldc * n).reshape(n, ldc)[:, :m], opA.T)
+    assert hip.fitre_hip_geam(ta, tb, m, n, 1.0, pa, lda, 1.0, None, ldb, pc, ldc) == 2
+    for q in (pa, pb, pc):
+        dev.free(q)
