@@ -78,29 +78,31 @@ __global__ void __launch_bounds__(256) thin_input_grad_kernel(const ThinConvPara
 #pragma unroll
 		for (int ci = 0; ci < CIN; ci++) acc[ci] = 0.f;
 		const float *dimg = dl + (int)img * p.cout * ocells;
-		const int ks = KS ? KS : p.ksize;
 		for (int co = 0; co < p.cout; co++) {
 			const float *wco = wl + co * taps * CIN;
 			const float *dco = dimg + co * ocells;
+			auto tap = [&](int ta, int tb, int ks) {
+				const int oa = (int)a - ta + p.pad, ob = (int)b - tb + p.pad;
+				const bool ok = ((unsigned)oa < (unsigned)p.outA) & ((unsigned)ob < (unsigned)p.outB);
+				const float d = dco[ok ? oa * p.outB + ob : 0] * (ok ? 1.f : 0.f);
+				const float4 *wq = reinterpret_cast<const float4 *>(wco + (ta * ks + tb) * CIN); // the same for every lane
 #pragma unroll
-			for (int ta = 0; ta < ks; ta++) {
-				const int oa = (int)a - ta + p.pad;
-				const bool okA = (unsigned)oa < (unsigned)p.outA;
-#pragma unroll
-				for (int tb = 0; tb < ks; tb++) {
-					const int ob = (int)b - tb + p.pad;
-					const bool ok = okA & ((unsigned)ob < (unsigned)p.outB);
-					const float d = dco[ok ? oa * p.outB + ob : 0] * (ok ? 1.f : 0.f);
-					const float4 *wq = reinterpret_cast<const float4 *>(wco + (ta * ks + tb) * CIN); // the same for every lane
-#pragma unroll
-					for (int g = 0; g < CIN / 4; g++) {
-						const float4 wv = wq[g];
-						acc[4 * g] = fmaf(wv.x, d, acc[4 * g]);
-						acc[4 * g + 1] = fmaf(wv.y, d, acc[4 * g + 1]);
-						acc[4 * g + 2] = fmaf(wv.z, d, acc[4 * g + 2]);
-						acc[4 * g + 3] = fmaf(wv.w, d, acc[4 * g + 3]);
-					}
+				for (int g = 0; g < CIN / 4; g++) {
+					const float4 wv = wq[g];
+					acc[4 * g] = fmaf(wv.x, d, acc[4 * g]);
+					acc[4 * g + 1] = fmaf(wv.y, d, acc[4 * g + 1]);
+					acc[4 * g + 2] = fmaf(wv.z, d, acc[4 * g + 2]);
+					acc[4 * g + 3] = fmaf(wv.w, d, acc[4 * g + 3]);
 				}
+			};
+			if constexpr (KS > 0) {
+#pragma unroll
+				for (int ta = 0; ta < KS; ta++)
+#pragma unroll
+					for (int tb = 0; tb < KS; tb++) tap(ta, tb, KS);
+			} else {
+				for (int ta = 0; ta < p.ksize; ta++)
+					for (int tb = 0; tb < p.ksize; tb++) tap(ta, tb, p.ksize);
 			}
 		}
 #pragma unroll
@@ -166,7 +168,6 @@ __global__ void __launch_bounds__(512) thin_weight_grad_kernel(const ThinConvPar
 		__syncthreads();
 		if (live) {
 			const float *xc = xs + ci * cells;
-#pragma unroll 4
 			for (int q = slice; q < ocells; q += slices) {
 				uint32_t oa, ob;
 				p.divOutB.divmod((uint32_t)q, oa, ob);
