@@ -44,7 +44,7 @@ KC = dict(conv_dw=0, conv_dx=1, conv_fwd=2, fc_gemm=3, splitk_reduce=4, bn_bwd=5
           act_bwd=9, act_fwd=10, bias_grad=11, softmax=12, permute=13, blas1=14, pool_act_bwd=15, kfac_factor=16,
           spd_inverse=17)
 MFMA_CLASSES = ("conv_dw", "conv_dx", "conv_fwd", "fc_gemm", "kfac_factor", "spd_inverse")
-TILES = {0: "", 1: "64x64", 2: "64x128", 3: "128x64", 4: "128x128"}
+TILES = {0: "", 1: "64x64", 2: "64x128", 3: "128x64", 4: "128x128", 5: "96x128"}
 
 
 def measured_traffic(kernel):
@@ -134,7 +134,7 @@ def largest_launches(launches, keep=4):
 def read_profile(L):
     rows = []
     for name, cls in KC.items():
-        for tile in range(5):
+        for tile in range(6):
             n, ms, work = C.c_long(), C.c_double(), C.c_double()
             L.check(L.hip.fitre_hip_profile_read_tile(cls, tile, C.byref(n), C.byref(ms), C.byref(work)))
             if n.value:

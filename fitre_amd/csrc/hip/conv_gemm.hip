@@ -428,7 +428,7 @@ size_t fitre_hip_conv_forward_workspace(const fitre_conv_shape *s)
 {
 	if (!s) return 0;
 	if (c3_pos_eligible(s, false)) return c3_pos_workspace(s, false);
-	return plan_gemm_workspace(s->outChannels, (long)s->samples * s->outA * s->outB, (long)s->inChannels * s->ksize * s->ksize);
+	return plan_gemm_workspace(s->outChannels, (long)s->samples * s->outA * s->outB, (long)s->inChannels * s->ksize * s->ksize, false, true);
 }
 
 int fitre_hip_conv_forward(const fitre_conv_shape *s, const float *x, const float *w, const float *bias, float *y, void *ws,
@@ -440,7 +440,7 @@ int fitre_hip_conv_forward(const fitre_conv_shape *s, const float *x, const floa
 	FITRE_REQUIRE(x && w && y, "fitre_hip_conv_forward: null pointer");
 	if (c3_pos_eligible(s, false)) return launch_c3_pos<false>(s, x, w, bias, y, ws, wsBytes);
 	const int I = s->outChannels, J = s->samples * s->outA * s->outB, R = s->inChannels * s->ksize * s->ksize;
-	GemmPlan plan = plan_gemm(I, J, R);
+	GemmPlan plan = plan_gemm(I, J, R, false, 0, true);
 	PlainParams pa{ w, (uint32_t)((size_t)I * R * sizeof(float)), R, I };
 	PatchGeom pb = make_patch_geom(x, s->inChannels, s->samples, s->inA, s->inB, s->outA, s->outB, s->ksize, s->stride, s->padding);
 	OutParams out{ y, (long)J, 0, bias, nullptr, 1.f, 0.f };
@@ -458,10 +458,16 @@ size_t fitre_hip_conv_weight_grad_workspace(const fitre_conv_shape *s)
 		return q > c ? q : c;
 	}
 	if (c3_dw_eligible(s)) return c3_dw_workspace(s);
-	size_t general = plan_gemm_workspace(s->outChannels, (long)s->inChannels * s->ksize * s->ksize, (long)s->samples * s->outA * s->outB);
+	size_t general = plan_gemm_workspace(s->outChannels, (long)s->inChannels * s->ksize * s->ksize, (long)s->samples * s->outA * s->outB, false, true);
 	if (thin_dw_eligible(s) && thin_dw_workspace(s) > general) general = thin_dw_workspace(s);
 	if (thin_dw_general_eligible(s) && thin_dw_general_workspace(s) > general) general = thin_dw_general_workspace(s);
 	return general;
+}
+
+int fitre_hip_conv_weight_grad_runs_beside(const fitre_conv_shape *s)
+{
+	if (!s) return 0;
+	return (quad_eligible(s) || c3_dw_eligible(s) || thin_dw_eligible(s) || thin_dw_general_eligible(s)) ? 1 : 0;
 }
 
 int fitre_hip_conv_weight_grad(const fitre_conv_shape *s, const float *x, const float *delta, float *dW, void *ws, size_t wsBytes)
@@ -478,7 +484,7 @@ int fitre_hip_conv_weight_grad(const fitre_conv_shape *s, const float *x, const 
 	if (thin_dw_general_eligible(s) && ws && wsBytes >= thin_dw_general_workspace(s) && ((((uintptr_t)ws) & 15) == 0))
 		return launch_thin_dw_general(s, x, delta, dW, ws);
 	const int I = s->outChannels, J = s->inChannels * s->ksize * s->ksize, R = s->samples * s->outA * s->outB;
-	GemmPlan plan = plan_gemm(I, J, R);
+	GemmPlan plan = plan_gemm(I, J, R, false, 0, true);
 	PlainParams pa{ delta, (uint32_t)((size_t)I * R * sizeof(float)), R, I };
 	PatchGeom pb = make_patch_geom(x, s->inChannels, s->samples, s->inA, s->inB, s->outA, s->outB, s->ksize, s->stride, s->padding);
 	OutParams out{ dW, (long)J, 0, nullptr, nullptr, 1.f, 0.f };
@@ -494,7 +500,7 @@ size_t fitre_hip_conv_input_grad_workspace(const fitre_conv_shape *s)
 		return q > c ? q : c;
 	}
 	if (c3_pos_eligible(s, true)) return c3_pos_workspace(s, true);
-	return plan_gemm_workspace(s->inChannels, (long)s->samples * s->inA * s->inB, (long)s->outChannels * s->ksize * s->ksize);
+	return plan_gemm_workspace(s->inChannels, (long)s->samples * s->inA * s->inB, (long)s->outChannels * s->ksize * s->ksize, false, true);
 }
 
 int fitre_hip_conv_input_grad(const fitre_conv_shape *s, const float *delta, const float *w, float *dx, void *ws, size_t wsBytes)
@@ -511,7 +517,7 @@ int fitre_hip_conv_input_grad(const fitre_conv_shape *s, const float *delta, con
 	if (c3_pos_eligible(s, true)) return launch_c3_pos<true>(s, delta, w, nullptr, dx, ws, wsBytes);
 	if (thin_dx_eligible(s) && s->inChannels <= 8) return launch_thin_dx(s, delta, w, dx);
 	const int I = s->inChannels, J = s->samples * s->inA * s->inB, R = s->outChannels * s->ksize * s->ksize;
-	GemmPlan plan = plan_gemm(I, J, R);
+	GemmPlan plan = plan_gemm(I, J, R, false, 0, true);
 	FlipWeightParams pa;
 	pa.w = w;
 	pa.bytes = (uint32_t)((size_t)s->outChannels * s->inChannels * s->ksize * s->ksize * sizeof(float));

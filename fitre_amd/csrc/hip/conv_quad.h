@@ -18,7 +18,6 @@
 // consecutive rows or reduction indices are the four cells of one map), and the input gradient's
 // tile stores put a lane's four rows -- the four cells of a map -- into one 16-byte group.
 #pragma once
-#include <stdlib.h>
 #include "conv_common.h"
 
 namespace fitre {
@@ -255,36 +254,14 @@ static int quad_launch(const PA &pa, const PB &pb, const OutParams &out, int I, 
 	// measured sweep (512 x 512 channels, 256 images): 64 x 64 tiles with about four workgroups per compute unit,
 	// deep reduction slices: weight gradient 46 -> 36 us (unsplit, slices of 64), input gradient 43 -> 40 us
 	// (eight splits, slices of 32).
-	GemmPlan ideal = quad_plan(I, J, R);
-	if (const char *env = getenv("FITRE_QUAD_TILE")) { // experiment: tile, split and slice override "bm,bn,splits,bk"
-		int bm = 0, bn = 0, sp = 0, bk = 16;
-		if (sscanf(env, "%d,%d,%d,%d", &bm, &bn, &sp, &bk) >= 3) {
-			ideal.bm = bm, ideal.bn = bn, ideal.bk = bk;
-			long chunk = (R + sp - 1) / sp;
-			chunk = ((chunk + bk - 1) / bk) * bk;
-			ideal.splits = (int)((R + chunk - 1) / chunk);
-			ideal.kChunk = (int)chunk;
-			ideal.wsBytes = ideal.splits > 1 ? (size_t)ideal.splits * I * J * sizeof(float) : 0;
-		}
-	}
+	const GemmPlan ideal = quad_plan(I, J, R);
 	GemmPlan plan = ideal;
 	if (plan.splits > 1 && (!ws || wsBytes < plan.wsBytes)) plan = quad_plan(I, J, R, 1); // no room for partials: unsplit
 	if (plan.wsBytes > 0 && (!ws || (((uintptr_t)ws) & 15) || wsBytes < plan.wsBytes))
 		return fail(FITRE_E_WORKSPACE, "split-K workspace of %zu bytes is null, misaligned or smaller than the %zu required", wsBytes,
 		            plan.wsBytes);
-#define QUAD_TILE(BM_, BN_, BK_)                                                                                                   \
-	if (plan.bm == BM_ && plan.bn == BN_ && plan.bk == BK_)                                                                        \
-	return quad_launch_tile<OpA, OpB, BM_, BN_, BK_>(pa, pb, out, I, J, R, plan, ws, kernelClass, flops, leftSplits)
-	QUAD_TILE(128, 128, 16);
-	QUAD_TILE(64, 128, 16);
-	QUAD_TILE(128, 64, 16);
-	QUAD_TILE(64, 64, 16);
-	QUAD_TILE(128, 128, 32);
-	QUAD_TILE(64, 128, 32);
-	QUAD_TILE(128, 64, 32);
-	QUAD_TILE(64, 64, 32);
-	QUAD_TILE(64, 64, 64);
-#undef QUAD_TILE
+	if (plan.bk == 64) return quad_launch_tile<OpA, OpB, 64, 64, 64>(pa, pb, out, I, J, R, plan, ws, kernelClass, flops, leftSplits);
+	if (plan.bk == 32) return quad_launch_tile<OpA, OpB, 64, 64, 32>(pa, pb, out, I, J, R, plan, ws, kernelClass, flops, leftSplits);
 	return fail(FITRE_E_UNSUPPORTED, "no tile %d x %d x %d", plan.bm, plan.bn, plan.bk);
 }
 

@@ -25,15 +25,27 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 
 constexpr int kGemmThreads = 256;
 
-template <int BM_, int BN_, int BK_>
+// WAVES_M x WAVES_N: how the four waves are arranged over the tile.  2 x 2 for the square tiles; 1 x 4 for
+// the 96-row tile (three 32-row blocks per wave, no padding for 96-channel layers such as AlexNet's).
+template <int BM_, int BN_, int BK_, int WAVES_M_ = 2, int WAVES_N_ = 2>
 struct TileCfg {
 	static constexpr int BM = BM_, BN = BN_, BK = BK_;
-	static constexpr int WM = BM / 2, WN = BN / 2; // wave tile
+	static constexpr int WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
+	static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N; // wave tile
 	static constexpr int TM = WM / 32, TN = WN / 32; // 32x32 blocks per wave
-	static_assert(BM % 64 == 0 && BN % 64 == 0 && BK % 2 == 0, "tile shape");
+	static_assert(WAVES_M * WAVES_N == 4, "four waves per workgroup");
+	static_assert(WM % 32 == 0 && WN % 32 == 0 && BK % 2 == 0, "tile shape");
 	static_assert((BM * BK) % kGemmThreads == 0 && (BN * BK) % kGemmThreads == 0, "tile shape");
 	static_assert(kGemmThreads % BK == 0, "BK must divide the workgroup");
 };
+
+// Operands whose threads walk the rows in steps of 256 / BK (the reduction-contiguous ones) work for any row
+// count that gives whole elements per thread, 96 included; they say so with `kAnyRows`.  The row-contiguous
+// operands need 256 % ROWS == 0.
+template <class T, class = void>
+struct operand_any_rows { static constexpr bool value = false; };
+template <class T>
+struct operand_any_rows<T, decltype((void)T::kAnyRows)> { static constexpr bool value = T::kAnyRows; };
 
 // ---------------------------------------------------------------------------
 // operands.  ROWS is BM or BN.  Every operand provides
@@ -113,6 +125,7 @@ struct PlainRowContig {
 // element(row, k) = p[row * ld + k]   (contiguous along the reduction index)
 template <int ROWS, int BK>
 struct PlainKContig {
+	static constexpr bool kAnyRows = true;
 	static constexpr int E = ROWS * BK / kGemmThreads;
 	static constexpr int RSTEP = kGemmThreads / BK;
 	static constexpr int LD = LdsStride<ROWS, BK>::value;
@@ -314,6 +327,7 @@ struct FlipWeightParams {
 };
 template <int ROWS, int BK>
 struct FlipWeightKContig {
+	static constexpr bool kAnyRows = true;
 	static constexpr int E = ROWS * BK / kGemmThreads;
 	static constexpr int RSTEP = kGemmThreads / BK;
 	static constexpr int LD = LdsStride<ROWS, BK>::value;
@@ -432,8 +446,9 @@ __device__ __forceinline__ void gemm_tile(const typename OpA::Params &pa, const 
 	opB.load(kbeg, kend, rb);
 
 	const int khalf = lane >> 5;
-	const float *aRd = As + khalf * LDA + (wave >> 1) * Cfg::WM + (lane & 31);
-	const float *bRd = Bs + khalf * LDB + (wave & 1) * Cfg::WN + (lane & 31);
+	const int waveM = wave / Cfg::WAVES_N, waveN = wave % Cfg::WAVES_N;
+	const float *aRd = As + khalf * LDA + waveM * Cfg::WM + (lane & 31);
+	const float *bRd = Bs + khalf * LDB + waveN * Cfg::WN + (lane & 31);
 
 	for (int k0 = kbeg; k0 < kend; k0 += BK) {
 		__syncthreads(); // everyone is done reading the previous slice
@@ -482,11 +497,11 @@ __device__ __forceinline__ void gemm_tile(const typename OpA::Params &pa, const 
 	for (int tm = 0; tm < TM; tm++) {
 #pragma unroll
 		for (int tn = 0; tn < TN; tn++) {
-			const int j = j0 + (wave & 1) * Cfg::WN + tn * 32 + (lane & 31);
+			const int j = j0 + waveN * Cfg::WN + tn * 32 + (lane & 31);
 			if (j >= J) continue;
 #pragma unroll
 			for (int v = 0; v < 16; v++) {
-				const int i = i0 + (wave >> 1) * Cfg::WM + tm * 32 + 8 * (v / 4) + 4 * khalf + (v % 4);
+				const int i = i0 + waveM * Cfg::WM + tm * 32 + 8 * (v / 4) + 4 * khalf + (v % 4);
 				if (i >= I) continue;
 				if (out.mirror && j < i) continue;
 				float val = acc[tm][tn][v];
@@ -700,11 +715,13 @@ inline double estimate_us(long tiles, int bm, int bn, long I, long J, long R, lo
 }
 
 // mirror: a symmetric product (I == J) that only computes the tiles on and above the diagonal
-inline GemmPlan plan_gemm_search(long I, long J, long R, bool mirror, long cus)
+// rows96: the row operand can feed a 96-row tile (operand_any_rows): used when it saves a quarter of a 128-row tile
+inline GemmPlan plan_gemm_search(long I, long J, long R, bool mirror, long cus, bool rows96 = false)
 {
 	GemmPlan p;
 	p.bm = (I <= 64) ? 64 : 128;
 	p.bn = (J <= 64) ? 64 : 128;
+	if (rows96 && !mirror && I > 64 && I <= 96 && p.bn == 128) p.bm = 96;
 	long tiles = ((I + p.bm - 1) / p.bm) * ((J + p.bn - 1) / p.bn);
 	if (mirror) {
 		long t = (I + p.bm - 1) / p.bm;
@@ -735,12 +752,13 @@ inline GemmPlan plan_gemm_search(long I, long J, long R, bool mirror, long cus)
 // The search above walks up to 1024 split counts; a layer asks for the same plan on every call
 // (and once more per workspace query), so the results are kept in a small table.  The plan is
 // made for the compute units of the lane the product will be launched on.
-inline GemmPlan plan_gemm(long I, long J, long R, bool mirror = false, int cus = 0)
+inline GemmPlan plan_gemm(long I, long J, long R, bool mirror = false, int cus = 0, bool rows96 = false)
 {
 	struct Entry {
 		long I, J, R;
 		bool mirror;
 		int cus;
+		bool rows96;
 		GemmPlan plan;
 	};
 	if (cus <= 0) cus = lane_compute_units();
@@ -748,9 +766,10 @@ inline GemmPlan plan_gemm(long I, long J, long R, bool mirror = false, int cus =
 	static Entry table[kEntries];
 	static int used = 0, next = 0;
 	for (int i = 0; i < used; i++)
-		if (table[i].I == I && table[i].J == J && table[i].R == R && table[i].mirror == mirror && table[i].cus == cus)
+		if (table[i].I == I && table[i].J == J && table[i].R == R && table[i].mirror == mirror && table[i].cus == cus &&
+		    table[i].rows96 == rows96)
 			return table[i].plan;
-	Entry e{ I, J, R, mirror, cus, plan_gemm_search(I, J, R, mirror, cus) };
+	Entry e{ I, J, R, mirror, cus, rows96, plan_gemm_search(I, J, R, mirror, cus, rows96) };
 	table[next] = e;
 	next = (next + 1) % kEntries;
 	if (used < kEntries) used++;
@@ -758,10 +777,10 @@ inline GemmPlan plan_gemm(long I, long J, long R, bool mirror = false, int cus =
 }
 
 // Workspace that covers the plan of every lane (a size query does not know the lane of the launch).
-inline size_t plan_gemm_workspace(long I, long J, long R, bool mirror = false)
+inline size_t plan_gemm_workspace(long I, long J, long R, bool mirror = false, bool rows96 = false)
 {
-	size_t a = plan_gemm(I, J, R, mirror, device_compute_units()).wsBytes;
-	size_t b = plan_gemm(I, J, R, mirror, lane_compute_units_min()).wsBytes;
+	size_t a = plan_gemm(I, J, R, mirror, device_compute_units(), rows96).wsBytes;
+	size_t b = plan_gemm(I, J, R, mirror, lane_compute_units_min(), rows96).wsBytes;
 	return a > b ? a : b;
 }
 
@@ -787,8 +806,8 @@ template <template <int, int> class OpA, template <int, int> class OpB, int BM, 
 static int launch_tile(const typename OpA<BM, kGemmBK>::Params &pa, const typename OpB<BN, kGemmBK>::Params &pb,
                        const OutParams &out, int I, int J, int R, const GemmPlan &plan, void *ws, int kernelClass, double flops)
 {
-	typedef TileCfg<BM, BN, kGemmBK> Cfg;
-	constexpr int tileId = (BM == 64 ? (BN == 64 ? 1 : 2) : (BN == 64 ? 3 : 4));
+	typedef TileCfg<BM, BN, kGemmBK, (BM == 96 ? 1 : 2), (BM == 96 ? 4 : 2)> Cfg;
+	constexpr int tileId = (BM == 96 ? 5 : (BM == 64 ? (BN == 64 ? 1 : 2) : (BN == 64 ? 3 : 4)));
 	typedef OpA<BM, kGemmBK> A;
 	typedef OpB<BN, kGemmBK> B;
 	dim3 grid((J + BN - 1) / BN, (I + BM - 1) / BM, plan.splits);
@@ -824,6 +843,12 @@ static int launch_gemm(const PA &pa, const PB &pb, const OutParams &out, int I, 
 		if (!ws || (((uintptr_t)ws) & 3)) return fail(FITRE_E_WORKSPACE, "split-K workspace is null or misaligned");
 		if (wsBytes < plan.wsBytes)
 			return fail(FITRE_E_WORKSPACE, "split-K workspace of %zu bytes is smaller than the %zu required", wsBytes, plan.wsBytes);
+	}
+	if (plan.bm == 96) {
+		if constexpr (operand_any_rows<OpA<96, kGemmBK>>::value)
+			return launch_tile<OpA, OpB, 96, 128>(pa, pb, out, I, J, R, plan, ws, kernelClass, flops);
+		else
+			return fail(FITRE_E_UNSUPPORTED, "a 96-row tile needs a reduction-contiguous row operand");
 	}
 	if (plan.bm == 128 && plan.bn == 128) return launch_tile<OpA, OpB, 128, 128>(pa, pb, out, I, J, R, plan, ws, kernelClass, flops);
 	if (plan.bm == 64 && plan.bn == 128) return launch_tile<OpA, OpB, 64, 128>(pa, pb, out, I, J, R, plan, ws, kernelClass, flops);

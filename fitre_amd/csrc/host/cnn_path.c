@@ -405,13 +405,20 @@ void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, 
 				dview.base = delta, dview.splits = 1, dview.stride = 0;
 			}
 		}
+		/* A weight gradient on the general tile engine stays in line: beside the next layer's matrix kernels both would
+		 * lose more than the overlap gains.  Its workspace is lane 1's, so the lanes are ordered around it. */
+		const int beside = fitre_hip_conv_weight_grad_runs_beside(&shape);
 		HIP_CALL(fitre_hip_lane_wait(1, 0));
-		HIP_CALL(fitre_hip_lane_select(1));
+		if (beside) {
+			HIP_CALL(fitre_hip_lane_select(1));
+		} else {
+			HIP_CALL(fitre_hip_lane_wait(0, 1));
+		}
 		/* without batch norm the bias gradient is a pass of its own over delta; nothing in the chain reads it */
 		if (!has_bn(l) && model->bias != 0)
 			HIP_CALL(fitre_hip_channel_sum(cur, l->outChannels, perChannel, gradient + bOffsets[c], sideWs, sideBytes));
 		HIP_CALL(fitre_hip_conv_weight_grad(&shape, input, cur, gradient + wOffsets[c], sideWs, sideBytes));
-		HIP_CALL(fitre_hip_lane_select(0));
+		if (beside) HIP_CALL(fitre_hip_lane_select(0));
 	}
 	HIP_CALL(fitre_hip_sync());
 }

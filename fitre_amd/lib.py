@@ -107,6 +107,7 @@ HIP_API = {
     "fitre_hip_conv_forward_workspace": (sz, [pshape]),
     "fitre_hip_conv_forward": (i32, [pshape, vp, vp, vp, vp, vp, sz]),
     "fitre_hip_conv_weight_grad_workspace": (sz, [pshape]),
+    "fitre_hip_conv_weight_grad_runs_beside": (i32, [pshape]),
     "fitre_hip_conv_weight_grad": (i32, [pshape, vp, vp, vp, vp, sz]),
     "fitre_hip_conv_input_grad_workspace": (sz, [pshape]),
     "fitre_hip_conv_input_grad": (i32, [pshape, vp, vp, vp, vp, sz]),

@@ -101,8 +101,8 @@ int fitre_hip_profile_enable(int on); /* on=1 clears the counters and starts; on
 /* launches, summed milliseconds and summed algorithmic work of one class (syncs first) */
 int fitre_hip_profile_read(int kernelClass, long *launches, double *milliseconds, double *work);
 /* The MFMA classes run one of several tile instantiations of the same kernel template; tile selects
- * one: 0 = not tiled, 1 = 64x64, 2 = 64x128, 3 = 128x64, 4 = 128x128 (channel rows x contiguous columns). */
-#define FITRE_TILE_VARIANTS 5
+ * one: 0 = not tiled, 1 = 64x64, 2 = 64x128, 3 = 128x64, 4 = 128x128, 5 = 96x128 (channel rows x contiguous columns). */
+#define FITRE_TILE_VARIANTS 6
 int fitre_hip_profile_read_tile(int kernelClass, int tile, long *launches, double *milliseconds, double *work);
 /* The accounted launches one by one, in issue order since the last fitre_hip_profile_enable(1) (at most 65 536
  * are kept): class, tile variant, duration and algorithmic work of launch `index` < *count. */
@@ -310,6 +310,13 @@ int fitre_hip_conv_forward(const fitre_conv_shape *s, const float *x, const floa
 /* dW[Cout][Cin*k*k] = sum over (n,a,b) of patch(x) * delta.  Replaces im2col + GEMM of
  * functions/cnn_backward.cu:771-783. */
 size_t fitre_hip_conv_weight_grad_workspace(const fitre_conv_shape *s);
+/* 1 when this shape's weight gradient runs on a kernel built to share the compute units with other work (the 3x3
+ * kernel: one workgroup per compute unit with register room left; the dense and direct forms), 0 when it runs on the
+ * general tile engine, whose workgroups want the compute units to themselves: beside another matrix kernel both
+ * lose more than the overlap gains (AlexNet batch 64: 3.27 ms per pass with every weight gradient on a second lane,
+ * 3.08 ms with the general-engine ones in line).  cnnBackward puts a weight gradient on its second lane only when
+ * this says 1. */
+int fitre_hip_conv_weight_grad_runs_beside(const fitre_conv_shape *s);
 int fitre_hip_conv_weight_grad(const fitre_conv_shape *s, const float *x, const float *delta, float *dW,
                                void *ws, size_t wsBytes);
 /* dx[Cin][N][inA][inB] = transposed convolution of delta with w; stride must be 1.  Replaces

@@ -27,6 +27,10 @@ CONV_CASES = [
     (1, 1, 1, 5, 5, 3, 1, 0),        # degenerate
     (2, 4, 5, 7, 7, 1, 1, 0),        # 1x1 window
     (2, 4, 6, 9, 9, 3, 2, 1),        # stride 2
+    # 65..96 channel rows on the general engine: the 96-row tile (AlexNet's 96-channel layers)
+    (2, 96, 40, 13, 13, 5, 1, 2),    # input gradient with 96 rows
+    (2, 20, 96, 13, 13, 5, 1, 2),    # forward and weight gradient with 96 rows
+    (2, 80, 72, 9, 9, 5, 1, 2),      # 80 and 72 rows: partial 96-row tiles
     # 3x3 / stride 1 / pad 1 fast paths: tile edges in every dimension
     (3, 8, 16, 8, 8, 3, 1, 1),       # 192 positions: not a multiple of the 128-position tile
     (2, 16, 40, 6, 10, 3, 1, 1),     # rectangular maps, 40 output channels
