@@ -4,6 +4,7 @@
 #include "conv_common.h"
 #include "conv_quad.h"
 #include "conv_thin.h"
+#include "linear_small.h"
 
 namespace fitre {
 
@@ -657,6 +658,18 @@ int fitre_hip_gemm(int transA, int transB, int M, int N, int K, float alpha, con
                    float beta, float *C, int ldc, const float *bias, void *ws, size_t wsBytes)
 {
 	FITRE_NEED_INIT();
+	if (small_gemm_fits(M, N, K) && (long)M * N >= 256) {
+		FITRE_REQUIRE(A && B && C, "fitre_hip_gemm: null pointer");
+		FITRE_REQUIRE((transA == 0 || transA == 1) && (transB == 0 || transB == 1), "fitre_hip_gemm: bad transpose flags");
+		FITRE_REQUIRE(lda >= (transA ? K : M) && ldb >= (transB ? N : K) && ldc >= M, "fitre_hip_gemm: leading dimension too small");
+		SmallGemmParams p{};
+		p.M = M, p.N = N, p.K = K;
+		p.A = A, p.sAm = transA ? lda : 1, p.sAk = transA ? 1 : lda;
+		p.B = B, p.sBk = transB ? ldb : 1, p.sBn = transB ? 1 : ldb;
+		p.C = C, p.ldc = ldc, p.alpha = alpha, p.beta = beta, p.bias = bias;
+		p.act = -1;
+		return launch_small_gemm(p, FITRE_KC_FC_GEMM);
+	}
 	if (M > 0 && N > 0 && K > 0 && (double)M * N * K <= kSmallProductWork) {
 		// a product this small (the output layer of a network: ten classes) does not fill one tile of the engine
 		FITRE_REQUIRE(A && B && C, "fitre_hip_gemm: null pointer");
@@ -669,6 +682,63 @@ int fitre_hip_gemm(int transA, int transB, int M, int N, int K, float alpha, con
 		return check_launch("small_product_kernel");
 	}
 	return gemm_ex(transA, transB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, bias, 0, FITRE_KC_FC_GEMM, ws, wsBytes);
+}
+
+// ---- backward products of a fully connected layer --------------------------------------------
+int fitre_hip_linear_is_small(int in, int out, int n) { return small_gemm_fits(in, n, out) && small_gemm_fits(out, in, n); }
+
+int fitre_hip_linear_input_grad(int in, int out, int n, const float *W, const float *delta, int actBelow, const float *zPre,
+                                const float *zPost, int extA, int extB, float *result, float *staging, void *ws, size_t wsBytes)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(in > 0 && out > 0 && n > 0, "fitre_hip_linear_input_grad: non-positive shape %d x %d, %d samples", out, in, n);
+	FITRE_REQUIRE(W && delta && result && result != delta, "fitre_hip_linear_input_grad: null or aliased pointer");
+	const bool permute = extA > 0 || extB > 0;
+	FITRE_REQUIRE(!permute || (extA > 0 && extB > 0 && in % (extA * extB) == 0),
+	              "fitre_hip_linear_input_grad: %d inputs are not whole %d x %d maps", in, extA, extB);
+	const bool derivative = actBelow != CNN_ACT_NONE && actBelow != ACT_LINEAR && actBelow >= 0;
+	if (small_gemm_fits(in, n, out)) {
+		SmallGemmParams p{};
+		p.M = in, p.N = n, p.K = out;
+		p.A = W, p.sAm = out, p.sAk = 1;
+		p.B = delta, p.sBk = 1, p.sBn = out;
+		p.C = result, p.ldc = in, p.alpha = 1.f, p.beta = 0.f;
+		p.act = derivative ? actBelow : -1, p.zPre = zPre, p.zPost = zPost;
+		p.extA = permute ? extA : 0, p.extB = permute ? extB : 0;
+		return launch_small_gemm(p, FITRE_KC_FC_GEMM);
+	}
+	// the engine, then the steps of the epilogue one by one
+	float *plain = permute ? staging : result;
+	FITRE_REQUIRE(plain != nullptr && plain != delta, "fitre_hip_linear_input_grad: a product of this size needs the staging buffer");
+	int rc = gemm_ex(1, 0, in, n, out, 1.f, W, out, delta, out, 0.f, plain, in, nullptr, 0, FITRE_KC_FC_GEMM, ws, wsBytes);
+	if (rc) return rc;
+	if (derivative) {
+		rc = fitre_hip_activation_backward(actBelow, plain, zPre, zPost, plain, (long)in * n);
+		if (rc) return rc;
+	}
+	if (permute) return fitre_hip_fc_to_conv(plain, in / (extA * extB), n, extA, extB, result);
+	return FITRE_OK;
+}
+
+int fitre_hip_linear_weight_grad(int in, int out, int n, const float *delta, const float *zin, float *dW, float *db, void *ws,
+                                 size_t wsBytes)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(in > 0 && out > 0 && n > 0, "fitre_hip_linear_weight_grad: non-positive shape %d x %d, %d samples", out, in, n);
+	FITRE_REQUIRE(delta && zin && dW, "fitre_hip_linear_weight_grad: null pointer");
+	if (small_gemm_fits(out, in, n)) {
+		SmallGemmParams p{};
+		p.M = out, p.N = in, p.K = n;
+		p.A = delta, p.sAm = 1, p.sAk = out;
+		p.B = zin, p.sBk = in, p.sBn = 1;
+		p.C = dW, p.ldc = out, p.alpha = 1.f, p.beta = 0.f;
+		p.act = -1;
+		p.rowSums = db;
+		return launch_small_gemm(p, FITRE_KC_FC_GEMM);
+	}
+	int rc = gemm_ex(0, 1, out, in, n, 1.f, delta, out, zin, in, 0.f, dW, out, nullptr, 0, FITRE_KC_FC_GEMM, ws, wsBytes);
+	if (rc || !db) return rc;
+	return fitre_hip_row_sum(delta, out, n, db);
 }
 
 } // extern "C"

@@ -1,0 +1,138 @@
+// Products of a fully connected layer that are far below one tile of the MFMA engine (LeNet's 400-120-84-10
+// tail at batch 128: 0.1 to 6 million multiply-adds).  At that size a pass is bound by the number of launches,
+// so the kernel here takes what the reference queues as separate steps into its epilogue:
+//
+//   input gradient   delta_below = f'(z_below) .* (W' * delta)        functions/cnn_backward.cu:250-254, then the
+//                    activation step of the next loop iteration (:100-172), optionally stored in the
+//                    convolution layout (the permutation at the boundary, :330-348)
+//   weight gradient  dW = delta * z', db = delta * 1                  functions/cnn_backward.cu:189-197, :216-224
+//
+// One workgroup owns a 32 x 32 block of the result and walks the reduction in blocks of 32 through LDS; a thread
+// holds 2 x 2 results.  The order of the additions is fixed by the shape alone.
+#pragma once
+#include "common.h"
+#include "fitre_nn.h"
+
+namespace fitre {
+
+constexpr int kSmallTile = 32;
+
+struct SmallGemmParams {
+	int M, N, K;
+	const float *A; // op(A)(m, k) = A[m * sAm + k * sAk]
+	long sAm, sAk;
+	const float *B; // op(B)(k, n) = B[k * sBk + n * sBn]
+	long sBk, sBn;
+	float *C; // C(m, n) = C[n * ldc + m], or the convolution layout when extA > 0
+	long ldc;
+	float alpha, beta;
+	const float *bias; // added per row m, or null
+	int act;           // >= 0: the result is multiplied by f'(.) taken from zPre / zPost (laid out like C, leading dimension M)
+	const float *zPre, *zPost;
+	int extA, extB;  // > 0: row m = (c * extB + b) * extA + a goes to [c][n][a][b]
+	float *rowSums;  // sum over k of op(A)(m, k) for every m, or null
+};
+
+__device__ __forceinline__ float act_backward_value(int actFun, float d, float zi, float zo)
+{
+	switch (actFun) {
+	case ACT_LOGISTIC: return d * zo * (1.f - zo);
+	case ACT_TANH: return d * ((1.f + zo) * (1.f - zo));
+	case CNN_ACT_SOFTPLUS: return d * (1.f / (1.f + expf(-zi)));
+	case CNN_ACT_SWISH: {
+		float t = 1.f / (1.f + expf(-zi));
+		return d * (zo + t * (1.f - zo));
+	}
+	case CNN_ACT_RELU: return zo > 0.f ? d : 0.f;
+	case CNN_ACT_ELU: return zo < 0.f ? d * (zo + 1.f) : d;
+	default: return d;
+	}
+}
+
+__global__ void __launch_bounds__(256) small_gemm_kernel(const SmallGemmParams p)
+{
+	__shared__ float As[kSmallTile][kSmallTile + 1]; // [k][m]
+	__shared__ float Bs[kSmallTile][kSmallTile + 1]; // [k][n]
+	const int tid = threadIdx.x;
+	const int m0 = blockIdx.x * kSmallTile, n0 = blockIdx.y * kSmallTile;
+	const int tm = tid & 15, tn = tid >> 4;
+	// loads run along whichever index is contiguous in memory
+	const bool aAlongM = p.sAm == 1, bAlongN = p.sBn == 1;
+	const int lo = tid & 31, hi = tid >> 5; // hi: 0..7
+	float acc00 = 0.f, acc01 = 0.f, acc10 = 0.f, acc11 = 0.f, rs0 = 0.f, rs1 = 0.f;
+	const bool sums = p.rowSums != nullptr && blockIdx.y == 0 && tn == 0;
+	for (int k0 = 0; k0 < p.K; k0 += kSmallTile) {
+		float av[4], bv[4];
+#pragma unroll
+		for (int i = 0; i < 4; i++) {
+			const int am = aAlongM ? lo : hi + 8 * i, ak = aAlongM ? hi + 8 * i : lo;
+			const int bn = bAlongN ? lo : hi + 8 * i, bk = bAlongN ? hi + 8 * i : lo;
+			const bool aok = (m0 + am < p.M) & (k0 + ak < p.K), bok = (n0 + bn < p.N) & (k0 + bk < p.K);
+			av[i] = aok ? p.A[(long)(m0 + am) * p.sAm + (long)(k0 + ak) * p.sAk] : 0.f;
+			bv[i] = bok ? p.B[(long)(k0 + bk) * p.sBk + (long)(n0 + bn) * p.sBn] : 0.f;
+		}
+		__syncthreads(); // the previous block's readers are done
+#pragma unroll
+		for (int i = 0; i < 4; i++) {
+			const int am = aAlongM ? lo : hi + 8 * i, ak = aAlongM ? hi + 8 * i : lo;
+			const int bn = bAlongN ? lo : hi + 8 * i, bk = bAlongN ? hi + 8 * i : lo;
+			As[ak][am] = av[i];
+			Bs[bk][bn] = bv[i];
+		}
+		__syncthreads();
+#pragma unroll
+		for (int k = 0; k < kSmallTile; k++) {
+			const float a0 = As[k][tm], a1 = As[k][tm + 16], b0 = Bs[k][tn], b1 = Bs[k][tn + 16];
+			acc00 = fmaf(a0, b0, acc00);
+			acc10 = fmaf(a1, b0, acc10);
+			acc01 = fmaf(a0, b1, acc01);
+			acc11 = fmaf(a1, b1, acc11);
+			if (sums) rs0 += a0, rs1 += a1;
+		}
+	}
+	if (sums) {
+		if (m0 + tm < p.M) p.rowSums[m0 + tm] = rs0;
+		if (m0 + tm + 16 < p.M) p.rowSums[m0 + tm + 16] = rs1;
+	}
+	const int planeAB = p.extA * p.extB;
+	auto store = [&](int m, int n, float acc) {
+		if (m >= p.M || n >= p.N) return;
+		float v = p.alpha * acc;
+		if (p.bias) v += p.bias[m];
+		if (p.act >= 0) {
+			const long zi = (long)n * p.M + m;
+			v = act_backward_value(p.act, v, p.zPre ? p.zPre[zi] : 0.f, p.zPost ? p.zPost[zi] : 0.f);
+		}
+		long dst = (long)n * p.ldc + m;
+		if (p.extA > 0) {
+			const int c = m / planeAB, r = m - c * planeAB;
+			const int b = r / p.extA, a = r - b * p.extA;
+			dst = (((long)c * p.N + n) * p.extA + a) * p.extB + b;
+		}
+		if (p.beta != 0.f) v += p.beta * p.C[dst];
+		p.C[dst] = v;
+	};
+	store(m0 + tm, n0 + tn, acc00);
+	store(m0 + tm + 16, n0 + tn, acc10);
+	store(m0 + tm, n0 + tn + 16, acc01);
+	store(m0 + tm + 16, n0 + tn + 16, acc11);
+}
+
+// A product is "small" when it is below one wave of engine tiles and its reduction is short enough for one
+// workgroup per result block to walk it alone.
+constexpr double kSmallGemmWork = 3.2e7; // multiply-adds
+constexpr int kSmallGemmMaxK = 512;
+static inline bool small_gemm_fits(int M, int N, int K)
+{
+	return M > 0 && N > 0 && K > 0 && K <= kSmallGemmMaxK && (double)M * N * K <= kSmallGemmWork;
+}
+
+static inline int launch_small_gemm(const SmallGemmParams &p, int kernelClass)
+{
+	dim3 grid((unsigned)((p.M + kSmallTile - 1) / kSmallTile), (unsigned)((p.N + kSmallTile - 1) / kSmallTile));
+	LaunchScope scope(kernelClass, 2.0 * (double)p.M * p.N * p.K, 0);
+	small_gemm_kernel<<<grid, 256, 0, stream()>>>(p);
+	return check_launch("small_gemm_kernel");
+}
+
+} // namespace fitre

@@ -139,6 +139,23 @@ LaunchScope::~LaunchScope()
 	if (g_pending.size() >= 2048) drain_pending();
 }
 
+// Plain device-to-device copy as a kernel: cheaper to queue than a runtime copy for the small
+// tensors of a pass.
+__global__ void copy_bytes_kernel(unsigned char *dst, const unsigned char *src, size_t n, int wide)
+{
+	const size_t stride = (size_t)gridDim.x * blockDim.x;
+	const size_t first = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+	size_t done = 0;
+	if (wide) {
+		const size_t words = n / 16;
+		const uint4 *s16 = reinterpret_cast<const uint4 *>(src);
+		uint4 *d16 = reinterpret_cast<uint4 *>(dst);
+		for (size_t i = first; i < words; i += stride) d16[i] = s16[i];
+		done = words * 16;
+	}
+	for (size_t i = done + first; i < n; i += stride) dst[i] = src[i];
+}
+
 // Byte fill as a kernel: a memset node recorded into a captured graph is not
 // reliable on this platform, a kernel node is.
 __global__ void fill_bytes_kernel(unsigned char *p, unsigned char v, size_t n)
@@ -368,6 +385,12 @@ int fitre_hip_copy_d2d(void *dst, const void *src, size_t bytes)
 	FITRE_NEED_INIT();
 	FITRE_REQUIRE(dst && src, "fitre_hip_copy_d2d: null pointer");
 	if (bytes == 0 || dst == src) return FITRE_OK;
+	if (bytes <= ((size_t)4 << 20)) {
+		const int wide = (((uintptr_t)dst | (uintptr_t)src) & 15) == 0;
+		unsigned blocks = blocks_for((long)(bytes / 16 + 1), 256, 4096);
+		copy_bytes_kernel<<<blocks, 256, 0, g_stream>>>((unsigned char *)dst, (const unsigned char *)src, bytes, wide);
+		return check_launch("copy_bytes_kernel");
+	}
 	FITRE_HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, g_stream));
 	return FITRE_OK;
 }

@@ -263,7 +263,6 @@ void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, 
 	char *preparedWs = (char *)sideWs + sideBytes;
 	const void *prepared[MAX_LAYERS] = { NULL };
 	int preparedPending = 0;
-	real *temp;
 
 	if (nc < 1 || n < 1 || n > model->batchSize) {
 		fprintf(stderr, "cnnBackward: needs at least one convolution layer and 1 <= batch (%d) <= model batch (%d)\n", n,
@@ -298,44 +297,44 @@ void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, 
 		preparedPending = any;
 	}
 
+	/* Linear layers, top down.  The delta of a layer (after its activation derivative) is written once, into the
+	 * layer's dx slot -- the snapshot the Hessian-vector product and the KFAC factors read -- and everything that
+	 * follows reads it there: the chain (lane 0) never writes a buffer that lane 1 still reads, so it never waits
+	 * for lane 1.  The last product leaves the first convolution-side delta in the chain workspace, already in
+	 * the convolution layout [C][N][a*B+b] (the reference permutes it separately, functions/cnn_backward.cu:330-348);
+	 * the workspace is free until the last convolution layer's input gradient, which is queued behind the pass
+	 * that reads this tensor. */
+	real *features = (real *)ws;
+	int extA, extB;
+	feature_extent(model, &extA, &extB);
 	for (int f = model->lLayers - 1; f >= 0; f--) {
 		const FC_LAYER *l = &model->fcLayer[f];
 		real *zl = z + zOffsets[f + nc + 1];
-		const long count = (long)l->out * n;
+		real *slot = dx + zOffsets[f + nc + 1];
 		const real *zin = z + zOffsets[f + nc] + ((f == 0) ? last->outputOffset : 0);
 
-		/* delta *= f'(.) */
-		HIP_CALL(fitre_hip_activation_backward(l->actFun, delta, zl + l->offset, zl, delta, count));
-		/* The chain (lane 0) goes straight on to delta = W' * delta.  It writes the buffer that the
-		 * layer above handed to lane 1, so lane 0 first waits for what lane 1 still reads there. */
+		/* delta .* f'(.) of the output layer (a plain copy when it has no activation); the layers below get theirs
+		 * from the epilogue of the product above them */
+		if (f == model->lLayers - 1)
+			HIP_CALL(fitre_hip_activation_backward(l->actFun, delta, zl + l->offset, zl, slot, (long)l->out * n));
 		HIP_CALL(fitre_hip_lane_wait(1, 0));
-		HIP_CALL(fitre_hip_lane_wait(0, 1));
-		HIP_CALL(fitre_hip_gemm(1, 0, l->in, n, l->out, 1.f, weights + wOffsets[f + nc], l->out, delta, l->out, 0.f,
-		                        delta_new, l->in, NULL, ws, wsBytes));
-		/* Beside it, on lane 1, what nothing later in this pass reads: */
+		/* the chain goes straight on: delta of the layer below = f'(.) .* (W' * delta) */
+		if (f > 0) {
+			const FC_LAYER *below = &model->fcLayer[f - 1];
+			real *zb = z + zOffsets[f + nc];
+			HIP_CALL(fitre_hip_linear_input_grad(l->in, l->out, n, weights + wOffsets[f + nc], slot, below->actFun,
+			                                     zb + below->offset, zb, 0, 0, dx + zOffsets[f + nc], NULL, ws, wsBytes));
+		} else {
+			HIP_CALL(fitre_hip_linear_input_grad(l->in, l->out, n, weights + wOffsets[f + nc], slot, -1, NULL, NULL, extA, extB,
+			                                     features, delta_new, ws, wsBytes));
+		}
+		/* beside it, on lane 1, what nothing later in this pass reads: dW = delta * z', db = delta * 1 */
 		HIP_CALL(fitre_hip_lane_select(1));
-		/* dW = delta * z' */
-		HIP_CALL(fitre_hip_gemm(0, 1, l->out, l->in, n, 1.f, delta, l->out, zin, l->in, 0.f,
-		                        gradient + wOffsets[f + nc], l->out, NULL, sideWs, sideBytes));
-		/* db = delta * 1 */
-		if (model->bias != 0) HIP_CALL(fitre_hip_row_sum(delta, l->out, n, gradient + bOffsets[f + nc]));
-		/* snapshot kept for the Hessian-vector product and the KFAC factors */
-		HIP_CALL(fitre_hip_copy_d2d(dx + zOffsets[f + nc + 1], delta, sizeof(real) * (size_t)count));
+		HIP_CALL(fitre_hip_linear_weight_grad(l->in, l->out, n, slot, zin, gradient + wOffsets[f + nc],
+		                                      (model->bias != 0) ? gradient + bOffsets[f + nc] : NULL, sideWs, sideBytes));
 		HIP_CALL(fitre_hip_lane_select(0));
-		temp = delta_new;
-		delta_new = delta;
-		delta = temp;
 	}
-
-	/* [N][C][b*A+a] -> [C][N][a*B+b], into the chain workspace: lane 1 may still read delta_new (the first linear
-	 * layer's delta), and the chain does not wait for it.  The workspace is free until the last convolution layer's
-	 * input gradient, which is queued behind the pass that reads this tensor. */
-	real *features = (real *)ws;
-	{
-		int extA, extB;
-		feature_extent(model, &extA, &extB);
-		HIP_CALL(fitre_hip_fc_to_conv(delta, last->outChannels, n, extA, extB, features));
-	}
+	if (model->lLayers == 0) HIP_CALL(fitre_hip_fc_to_conv(delta, last->outChannels, n, extA, extB, features));
 
 	/* delta as the layer above left it: a plain tensor, or the unsummed split partials of its input
 	 * gradient (summed by the pool / activation pass below while it reads them) */
@@ -360,10 +359,7 @@ void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, 
 			/* The forward pass rewrote this layer's activation output into the FC layout in place;
 			 * rebuild it from the activation input (the reference reads the permuted buffer,
 			 * functions/cnn_backward.cu:574-580). */
-			if (!fusedRelu) {
-				HIP_CALL(fitre_hip_lane_wait(0, 1)); /* lane 1 may still read delta_new */
-				HIP_CALL(fitre_hip_activation_forward(act, actIn, delta_new, perChannel * l->outChannels));
-			}
+			if (!fusedRelu) HIP_CALL(fitre_hip_activation_forward(act, actIn, delta_new, perChannel * l->outChannels));
 			actOut = delta_new;
 		}
 		const real *cur;

@@ -1,0 +1,144 @@
+"""Backward products of one fully connected layer (fitre_hip_linear_input_grad / _weight_grad) against float64
+numpy on the same float32 operands: the fused single-launch kernel for small layers and the sequence of plain
+steps for large ones must both give W' * delta times the activation derivative of the layer below (optionally in
+the convolution layout), dW = delta * z' and db = delta * 1."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from fitre_amd import lib as L
+from fitre_amd.structs import CNN_ACT_ELU, CNN_ACT_NONE, CNN_ACT_RELU, CNN_ACT_SOFTPLUS, CNN_ACT_SWISH
+from helpers import rel_err
+
+pytestmark = pytest.mark.gpu
+hip = L.hip
+TOL = 1e-5  # float32 products of at most 4096 terms against float64
+
+
+def ok(rc):
+    assert rc == 0, hip.fitre_hip_last_error().decode()
+
+
+def derivative(act, zi, zo):
+    """f'(.) as functions/cnn_backward.cu:100-172 applies it (ReLU and ELU decide on the activation output)."""
+    sig = 1.0 / (1.0 + np.exp(-zi))
+    return {CNN_ACT_RELU: (zo > 0).astype(np.float64), CNN_ACT_ELU: np.where(zo < 0, zo + 1.0, 1.0),
+            CNN_ACT_SOFTPLUS: sig, CNN_ACT_SWISH: zo + sig * (1.0 - zo), CNN_ACT_NONE: np.ones_like(zi), -1: np.ones_like(zi)}[act]
+
+
+def forward_act(act, zi):
+    sig = 1.0 / (1.0 + np.exp(-zi))
+    return {CNN_ACT_RELU: np.maximum(zi, 0), CNN_ACT_ELU: np.where(zi < 0, np.exp(zi) - 1.0, zi),
+            CNN_ACT_SOFTPLUS: np.log1p(np.exp(zi)), CNN_ACT_SWISH: zi * sig, CNN_ACT_NONE: zi, -1: zi}[act]
+
+
+# (in, out, samples): LeNet's tail at batch 128 and ragged sizes around the 32-wide blocks (small kernel); AlexNet-like
+# and long-reduction layers (the engine path)
+SMALL = [(84, 10, 128), (120, 84, 128), (400, 120, 128), (33, 31, 65), (1, 1, 1), (64, 32, 32), (100, 7, 500)]
+LARGE = [(1024, 512, 64), (400, 120, 1024), (4096, 100, 96)]
+
+
+@pytest.mark.parametrize("act", [CNN_ACT_RELU, CNN_ACT_SWISH, CNN_ACT_SOFTPLUS, CNN_ACT_ELU, CNN_ACT_NONE, -1])
+@pytest.mark.parametrize("n_in,n_out,n", SMALL + LARGE)
+def test_input_gradient_with_the_derivative_below(dev, n_in, n_out, n, act):
+    assert bool(hip.fitre_hip_linear_is_small(n_in, n_out, n)) == ((n_in, n_out, n) in SMALL)
+    rng = np.random.default_rng(n_in * 31 + n_out * 7 + n + (act if act > 0 else 0))
+    w = rng.standard_normal(n_out * n_in).astype(np.float32)        # out x in, column-major
+    d = rng.standard_normal(n_out * n).astype(np.float32)           # out x n
+    zpre = rng.standard_normal(n_in * n).astype(np.float32)         # in x n
+    zpost = forward_act(act, zpre.astype(np.float64)).astype(np.float32)
+    W = w.reshape(n_in, n_out).T.astype(np.float64)                 # W[o, i]
+    D = d.reshape(n, n_out).T.astype(np.float64)                    # D[o, s]
+    want = (W.T @ D) * derivative(act, zpre.reshape(n, n_in).T.astype(np.float64), zpost.reshape(n, n_in).T.astype(np.float64))
+    pw, pd, pzi, pzo = dev.upload(w), dev.upload(d), dev.upload(zpre), dev.upload(zpost)
+    out = dev.upload(np.full(n_in * n, 7.0, np.float32))
+    ws_bytes = hip.fitre_hip_gemm_workspace(n_in, n, n_out)
+    ws = dev.alloc(ws_bytes)
+    ok(hip.fitre_hip_linear_input_grad(n_in, n_out, n, pw, pd, act, pzi, pzo, 0, 0, out, None, ws, ws_bytes))
+    got = dev.download(out, n_in * n).reshape(n, n_in).T
+    assert rel_err(got, want) < TOL
+    for p in (pw, pd, pzi, pzo, out, ws):
+        dev.free(p)
+
+
+@pytest.mark.parametrize("channels,ext_a,ext_b,n_out,n", [(16, 5, 5, 120, 128), (3, 2, 7, 33, 40), (1, 1, 1, 5, 9),
+                                                           (256, 6, 6, 512, 64), (64, 3, 2, 100, 1200)])
+def test_input_gradient_in_the_convolution_layout(dev, channels, ext_a, ext_b, n_out, n):
+    """Row m = (c * B + b) * A + a of the product lands at [c][sample][a][b] (fitre_hip_fc_to_conv's permutation)."""
+    n_in = channels * ext_a * ext_b
+    rng = np.random.default_rng(n_in + n_out + n)
+    w = rng.standard_normal(n_out * n_in).astype(np.float32)
+    d = rng.standard_normal(n_out * n).astype(np.float32)
+    W = w.reshape(n_in, n_out).T.astype(np.float64)
+    D = d.reshape(n, n_out).T.astype(np.float64)
+    plain = W.T @ D                                                  # [m][s]
+    want = plain.reshape(channels, ext_b, ext_a, n).transpose(0, 3, 2, 1)   # [c][s][a][b]
+    pw, pd = dev.upload(w), dev.upload(d)
+    out = dev.zeros(n_in * n)
+    staging = dev.zeros(n_in * n)
+    ws_bytes = hip.fitre_hip_gemm_workspace(n_in, n, n_out)
+    ws = dev.alloc(ws_bytes)
+    ok(hip.fitre_hip_linear_input_grad(n_in, n_out, n, pw, pd, -1, None, None, ext_a, ext_b, out, staging, ws, ws_bytes))
+    got = dev.download(out, n_in * n).reshape(channels, n, ext_a, ext_b)
+    assert rel_err(got, want) < TOL
+    if not hip.fitre_hip_linear_is_small(n_in, n_out, n):
+        # a large layer without the staging buffer is refused before anything is queued
+        assert hip.fitre_hip_linear_input_grad(n_in, n_out, n, pw, pd, -1, None, None, ext_a, ext_b, out, None, ws, ws_bytes) == 2
+    assert hip.fitre_hip_linear_input_grad(n_in, n_out, n, pw, pd, -1, None, None, ext_a + 1, ext_b, out, staging, ws, ws_bytes) == 2 \
+        or n_in % ((ext_a + 1) * ext_b) == 0
+    for p in (pw, pd, out, staging, ws):
+        dev.free(p)
+
+
+@pytest.mark.parametrize("bias", [True, False])
+@pytest.mark.parametrize("n_in,n_out,n", SMALL + LARGE)
+def test_weight_and_bias_gradient(dev, n_in, n_out, n, bias):
+    rng = np.random.default_rng(n_in * 3 + n_out * 5 + n)
+    d = rng.standard_normal(n_out * n).astype(np.float32)
+    zin = rng.standard_normal(n_in * n).astype(np.float32)
+    D = d.reshape(n, n_out).T.astype(np.float64)
+    Z = zin.reshape(n, n_in).T.astype(np.float64)
+    pd, pz = dev.upload(d), dev.upload(zin)
+    dw = dev.upload(np.full(n_out * n_in, 3.0, np.float32))
+    db = dev.upload(np.full(n_out + 4, 5.0, np.float32))
+    ws_bytes = hip.fitre_hip_gemm_workspace(n_out, n_in, n)
+    ws = dev.alloc(ws_bytes)
+    ok(hip.fitre_hip_linear_weight_grad(n_in, n_out, n, pd, pz, dw, db if bias else None, ws, ws_bytes))
+    got = dev.download(dw, n_out * n_in).reshape(n_in, n_out).T
+    assert rel_err(got, D @ Z.T) < TOL
+    got_b = dev.download(db, n_out + 4)
+    if bias:
+        assert rel_err(got_b[:n_out], D.sum(axis=1)) < TOL
+        assert (got_b[n_out:] == 5.0).all()
+    else:
+        assert (got_b == 5.0).all()
+    for p in (pd, pz, dw, db, ws):
+        dev.free(p)
+
+
+def test_small_layers_are_deterministic(dev):
+    """Two runs of the fused kernels give the same bits."""
+    n_in, n_out, n = 400, 120, 128
+    rng = np.random.default_rng(0)
+    d = rng.standard_normal(n_out * n).astype(np.float32)
+    zin = rng.standard_normal(n_in * n).astype(np.float32)
+    pd, pz = dev.upload(d), dev.upload(zin)
+    runs = []
+    for _ in range(2):
+        dw, db = dev.zeros(n_out * n_in), dev.zeros(n_out)
+        ok(hip.fitre_hip_linear_weight_grad(n_in, n_out, n, pd, pz, dw, db, None, 0))
+        runs.append((dev.download(dw, n_out * n_in), dev.download(db, n_out)))
+        dev.free(dw), dev.free(db)
+    assert np.array_equal(runs[0][0], runs[1][0]) and np.array_equal(runs[0][1], runs[1][1])
+    dev.free(pd), dev.free(pz)
+
+
+def test_linear_arguments_are_checked(dev):
+    p = dev.zeros(64)
+    assert hip.fitre_hip_linear_input_grad(0, 4, 4, p, p, -1, None, None, 0, 0, p, None, None, 0) == 2
+    assert hip.fitre_hip_linear_input_grad(4, 4, 4, p, p, -1, None, None, 0, 0, p, None, None, 0) == 2  # result aliases delta
+    assert hip.fitre_hip_linear_input_grad(4, 4, 4, None, p, -1, None, None, 0, 0, p, None, None, 0) == 2
+    assert hip.fitre_hip_linear_weight_grad(4, 4, 0, p, p, p, None, None, 0) == 2
+    assert hip.fitre_hip_linear_weight_grad(4, 4, 4, p, None, p, None, None, 0) == 2
+    dev.free(p)
