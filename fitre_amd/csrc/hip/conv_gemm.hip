@@ -483,13 +483,38 @@ int fitre_hip_conv_weight_grad(const fitre_conv_shape *s, const float *x, const 
 	if (thin_dw_eligible(s) && ws && wsBytes >= thin_dw_workspace(s) && ((((uintptr_t)delta) | ((uintptr_t)ws)) & 15) == 0)
 		return launch_thin_dw(s, x, delta, dW, ws);
 	if (thin_dw_general_eligible(s) && ws && wsBytes >= thin_dw_general_workspace(s) && ((((uintptr_t)ws) & 15) == 0))
-		return launch_thin_dw_general(s, x, delta, dW, ws);
+		return launch_thin_dw_general(s, x, delta, dW, nullptr, ws);
 	const int I = s->outChannels, J = s->inChannels * s->ksize * s->ksize, R = s->samples * s->outA * s->outB;
 	GemmPlan plan = plan_gemm(I, J, R, false, 0, true);
 	PlainParams pa{ delta, (uint32_t)((size_t)I * R * sizeof(float)), R, I };
 	PatchGeom pb = make_patch_geom(x, s->inChannels, s->samples, s->inA, s->inB, s->outA, s->outB, s->ksize, s->stride, s->padding);
 	OutParams out{ dW, (long)J, 0, nullptr, nullptr, 1.f, 0.f };
 	return launch_gemm<PlainKContig, PatchKContig>(pa, pb, out, I, J, R, plan, ws, wsBytes, FITRE_KC_CONV_DW, conv_flops(s));
+}
+
+// weight and bias gradient of a layer without batch norm: one pass over delta where the thin kernel applies
+size_t fitre_hip_conv_weight_bias_grad_workspace(const fitre_conv_shape *s)
+{
+	if (!s) return 0;
+	const size_t w = fitre_hip_conv_weight_grad_workspace(s);
+	const size_t b = fitre_hip_channel_sum_workspace(s->outChannels, (long)s->samples * s->outA * s->outB);
+	return w > b ? w : b;
+}
+
+int fitre_hip_conv_weight_bias_grad(const fitre_conv_shape *s, const float *x, const float *delta, float *dW, float *db, void *ws,
+                                    size_t wsBytes)
+{
+	FITRE_NEED_INIT();
+	if (!db) return fitre_hip_conv_weight_grad(s, x, delta, dW, ws, wsBytes);
+	int rc = check_conv("fitre_hip_conv_weight_bias_grad", s);
+	if (rc) return rc;
+	FITRE_REQUIRE(x && delta && dW, "fitre_hip_conv_weight_bias_grad: null pointer");
+	if (thin_dw_general_eligible(s) && ws && wsBytes >= thin_dw_general_workspace(s) && ((((uintptr_t)ws) & 15) == 0))
+		return launch_thin_dw_general(s, x, delta, dW, db, ws);
+	// the bias gradient first: it is done with the workspace before the weight gradient takes it
+	rc = fitre_hip_channel_sum(delta, s->outChannels, (long)s->samples * s->outA * s->outB, db, ws, wsBytes);
+	if (rc) return rc;
+	return fitre_hip_conv_weight_grad(s, x, delta, dW, ws, wsBytes);
 }
 
 // ---- input gradient: I = Cin, J = input positions, R = Cout*k*k ----------------
@@ -516,7 +541,7 @@ int fitre_hip_conv_input_grad(const fitre_conv_shape *s, const float *delta, con
 	if (quad_usable(s, ws, wsBytes, quad_input_grad_workspace(s)) && (((((uintptr_t)dx) | ((uintptr_t)delta) | ((uintptr_t)w)) & 15) == 0))
 		return quad_input_grad(s, delta, w, nullptr, dx, ws, wsBytes, nullptr, nullptr);
 	if (c3_pos_eligible(s, true)) return launch_c3_pos<true>(s, delta, w, nullptr, dx, ws, wsBytes);
-	if (thin_dx_eligible(s) && s->inChannels <= 8) return launch_thin_dx(s, delta, w, dx);
+	if (thin_dx_eligible(s)) return launch_thin_dx(s, delta, w, dx);
 	const int I = s->inChannels, J = s->samples * s->inA * s->inB, R = s->outChannels * s->ksize * s->ksize;
 	GemmPlan plan = plan_gemm(I, J, R, false, 0, true);
 	FlipWeightParams pa;

@@ -5,14 +5,14 @@
 // GFLOP per pass at batch 1024).  Here both gradients are computed with ordinary vector multiply-adds by
 // workgroups that keep one image at a time in LDS:
 //
-//   input gradient   one thread per input cell (n, a, b), Cin accumulators in registers; the image's delta
-//                    (all output channels) and the weights ([co][tap][ci]: the channels of a tap are one or two
-//                    broadcast 16-byte reads) in LDS;
+//   input gradient   one thread per (input channel, input cell) with the channel uniform over a wave: the image's
+//                    delta (all output channels, zero border) in LDS, the weights through scalar loads;
 //   weight gradient  one thread per (patch index k = (ci, ta, tb), position slice), Cout accumulators in
 //                    registers; per position one LDS read of the input cell and Cout / 4 broadcast 16-byte
-//                    reads of delta (stored [position][channel]); slices are added in a fixed order, every
-//                    workgroup leaves one partial Cout x K block and splitk_reduce sums the blocks in
-//                    workgroup order -- the result does not depend on scheduling.
+//                    reads of delta (stored [position][channel]); a patch index of constant one yields the bias
+//                    gradient in the same loop; slices are added in a fixed order, every workgroup leaves one
+//                    partial Cout x (K + 1) block and a reduction sums the blocks in workgroup order -- the
+//                    result does not depend on scheduling.
 #pragma once
 #include "conv_common.h"
 
@@ -27,126 +27,139 @@ struct ThinConvParams {
 	const float *w;     // [Cout][Cin][k][k]     (input gradient)
 	int cin, cout, samples, inA, inB, outA, outB, ksize, stride, pad;
 	int imagesPerGroup;
+	int ciPerGroup; // input gradient: input channels per workgroup
+	int parts, rowsPerUnit, unitsPerGroup; // weight gradient: bands of output rows per image, rows per band, units per workgroup
 	FastDiv divInB, divOutB, divK, divKK, divCells, divOcells;
+	FastDiv divPlane, divPB; // input gradient: bordered delta plane and its row length
+	FastDiv divPBx;          // weight gradient: row length of the bordered input
+	FastDiv divXPlane[2], divDPos[2]; // weight gradient: bordered input plane / positions of a full band [0] and of an image's last band [1]
 };
 
 // ---- input gradient (stride 1): dx[ci][n][a][b] = sum_co sum_taps W[co][ci][ta][tb] * delta[co][n][a - ta + p][b - tb + p]
-// LDS: [weights as [co][tap][CIN] | delta of the group's images as [image][co][outA * outB]]
-// KS: window extent known at compile time (the tap loops are unrolled: all of a channel's delta reads in flight), 0: any
-template <int CIN, int KS>
-__global__ void __launch_bounds__(256) thin_input_grad_kernel(const ThinConvParams p, float *dx)
+// One workgroup per (image, group of input channels).  The image's delta (all output channels) sits in LDS with a
+// zero border of k - 1 - p cells, so that no tap needs a bounds check; a wave takes 64 cells of one input channel
+// at a time: the channel is the same for the whole wave, so the weights W[co][ci][.] come through scalar loads
+// and every tap is one LDS read and one multiply-add.
+// KS: window extent known at compile time (the tap loops are unrolled), 0: any
+template <int KS>
+__global__ void __launch_bounds__(256)
+thin_input_grad_kernel(const ThinConvParams p, const float *__restrict__ w, const float *__restrict__ delta, float *__restrict__ dx)
 {
 	extern __shared__ __align__(16) float thin_lds[];
 	const int tid = threadIdx.x;
-	const int cells = p.inA * p.inB, ocells = p.outA * p.outB, taps = p.ksize * p.ksize;
-	const int n0 = blockIdx.x * p.imagesPerGroup;
-	const int imgs = (p.samples - n0 < p.imagesPerGroup) ? p.samples - n0 : p.imagesPerGroup;
+	const int ks = KS > 0 ? KS : p.ksize;
+	const int cells = p.inA * p.inB, ocells = p.outA * p.outB, taps = ks * ks;
+	const int border = ks - 1 - p.pad;
+	const int PB = p.inB + ks - 1, plane = (p.inA + ks - 1) * PB;
+	const int n = blockIdx.x;
 	const size_t oplane = (size_t)p.samples * ocells, iplane = (size_t)p.samples * cells;
-	float *wl = thin_lds;
-	float *dl = thin_lds + p.cout * taps * CIN;
-	// weights: W[co][ci][tap] -> wl[(co * taps + tap) * CIN + ci], zero for ci >= cin
-	for (int i = tid; i < p.cout * taps * CIN; i += 256) {
-		const int ci = i % CIN, r = i / CIN;
-		uint32_t co, tap;
-		p.divKK.divmod((uint32_t)r, co, tap);
-		wl[i] = (ci < p.cin) ? p.w[((size_t)co * p.cin + ci) * taps + tap] : 0.f;
-	}
-	// delta, eight loads of a thread in flight at a time
-	const int total = imgs * p.cout * ocells;
+	// delta with its border, eight loads of a thread in flight at a time
+	const int total = p.cout * plane;
 	for (int base = tid; base < total; base += 256 * 8) {
 		float v[8];
 #pragma unroll
 		for (int u = 0; u < 8; u++) {
 			const int i = base + 256 * u;
-			uint32_t t, q, img, co;
-			p.divOcells.divmod((uint32_t)(i < total ? i : 0), t, q);
-			img = t / (uint32_t)p.cout, co = t - img * (uint32_t)p.cout;
-			v[u] = (i < total) ? p.delta[(size_t)co * oplane + (size_t)(n0 + (int)img) * ocells + q] : 0.f;
+			uint32_t co, q, r, c;
+			p.divPlane.divmod((uint32_t)(i < total ? i : 0), co, q);
+			p.divPB.divmod(q, r, c);
+			const int oa = (int)r - border, ob = (int)c - border;
+			const bool ok = (i < total) & ((unsigned)oa < (unsigned)p.outA) & ((unsigned)ob < (unsigned)p.outB);
+			v[u] = ok ? delta[(size_t)co * oplane + (size_t)n * ocells + oa * p.outB + ob] : 0.f;
 		}
 #pragma unroll
 		for (int u = 0; u < 8; u++) {
 			const int i = base + 256 * u;
-			if (i < total) dl[i] = v[u];
+			if (i < total) thin_lds[i] = v[u];
 		}
 	}
 	__syncthreads();
-	for (int pos = tid; pos < imgs * cells; pos += 256) {
-		uint32_t img, cell, a, b;
-		p.divCells.divmod((uint32_t)pos, img, cell);
-		p.divInB.divmod(cell, a, b);
-		float acc[CIN];
-#pragma unroll
-		for (int ci = 0; ci < CIN; ci++) acc[ci] = 0.f;
-		const float *dimg = dl + (int)img * p.cout * ocells;
+	const int lane = tid & 63, wave = tid >> 6;
+	const int chunks = (cells + 63) / 64, chunk = (cells + chunks - 1) / chunks; // cells per wave, evenly
+	const int ci0 = blockIdx.y * p.ciPerGroup;
+	const int ciN = (p.cin - ci0 < p.ciPerGroup) ? p.cin - ci0 : p.ciPerGroup;
+	for (int task = wave; task < ciN * chunks; task += 4) {
+		const int ci = __builtin_amdgcn_readfirstlane(ci0 + task / chunks);
+		const int part = task % chunks;
+		const int cell = part * chunk + lane;
+		const bool live = lane < chunk && cell < cells;
+		uint32_t a, b;
+		p.divInB.divmod((uint32_t)(live ? cell : 0), a, b);
+		// delta[a - ta + p][b - tb + p] is the bordered cell [a + (k - 1 - ta)][b + (k - 1 - tb)]
+		const float *d0 = thin_lds + (int)a * PB + (int)b;
+		const float *wci = w + (size_t)ci * taps;
+		float acc = 0.f;
 		for (int co = 0; co < p.cout; co++) {
-			const float *wco = wl + co * taps * CIN;
-			const float *dco = dimg + co * ocells;
-			auto tap = [&](int ta, int tb, int ks) {
-				const int oa = (int)a - ta + p.pad, ob = (int)b - tb + p.pad;
-				const bool ok = ((unsigned)oa < (unsigned)p.outA) & ((unsigned)ob < (unsigned)p.outB);
-				const float d = dco[ok ? oa * p.outB + ob : 0] * (ok ? 1.f : 0.f);
-				const float4 *wq = reinterpret_cast<const float4 *>(wco + (ta * ks + tb) * CIN); // the same for every lane
-#pragma unroll
-				for (int g = 0; g < CIN / 4; g++) {
-					const float4 wv = wq[g];
-					acc[4 * g] = fmaf(wv.x, d, acc[4 * g]);
-					acc[4 * g + 1] = fmaf(wv.y, d, acc[4 * g + 1]);
-					acc[4 * g + 2] = fmaf(wv.z, d, acc[4 * g + 2]);
-					acc[4 * g + 3] = fmaf(wv.w, d, acc[4 * g + 3]);
-				}
-			};
+			const float *wk = wci + (size_t)co * p.cin * taps;
+			const float *dco = d0 + co * plane;
 			if constexpr (KS > 0) {
 #pragma unroll
-				for (int ta = 0; ta < KS; ta++)
+				for (int ta = 0; ta < KS; ta++) {
+					const float *drow = dco + (KS - 1 - ta) * PB;
 #pragma unroll
-					for (int tb = 0; tb < KS; tb++) tap(ta, tb, KS);
+					for (int tb = 0; tb < KS; tb++) acc = fmaf(wk[ta * KS + tb], drow[KS - 1 - tb], acc);
+				}
 			} else {
-				for (int ta = 0; ta < p.ksize; ta++)
-					for (int tb = 0; tb < p.ksize; tb++) tap(ta, tb, p.ksize);
+				for (int ta = 0; ta < ks; ta++)
+					for (int tb = 0; tb < ks; tb++) acc = fmaf(wk[ta * ks + tb], dco[(ks - 1 - ta) * PB + (ks - 1 - tb)], acc);
 			}
 		}
-#pragma unroll
-		for (int ci = 0; ci < CIN; ci++)
-			if (ci < p.cin) dx[(size_t)ci * iplane + (size_t)n0 * cells + pos] = acc[ci];
+		if (live) dx[(size_t)ci * iplane + (size_t)n * cells + cell] = acc;
 	}
 }
 
-// ---- weight gradient: dW[co][k] = sum over positions of delta[co][position] * patch[position][k]
-// blockDim = 512.  LDS: [x of one image | delta of one image as [position][COUT] | slice sums]
+// ---- weight gradient: dW[co][k] = sum over positions of delta[co][position] * patch[position][k], and with the
+// patch extended by a constant one (index k = K) the bias gradient db[co] = sum of delta[co][.] comes out of the
+// same loop (functions/cnn_backward.cu:662-689 takes it with a ones-vector product of its own).
+// blockDim = 512: thread (k, slice), slices = 512 / (K + 1).  A workgroup walks its units (image, band of output
+// rows) one at a time.  LDS: [x rows of the band, zero border of `pad` cells | delta of the band as
+// [position][COUT]]; afterwards the slice sums.
 template <int COUT>
-__global__ void __launch_bounds__(512) thin_weight_grad_kernel(const ThinConvParams p, float *partial)
+__global__ void __launch_bounds__(512)
+thin_weight_grad_kernel(const ThinConvParams p, const float *__restrict__ x, const float *__restrict__ delta, float *__restrict__ partial)
 {
 	extern __shared__ __align__(16) float thin_lds[];
 	const int tid = threadIdx.x;
-	const int K = p.cin * p.ksize * p.ksize;
+	const int K = p.cin * p.ksize * p.ksize, K1 = K + 1;
 	const int cells = p.inA * p.inB, ocells = p.outA * p.outB;
-	const int slices = 512 / K; // >= 1 (host checks K <= 512)
+	const int slices = 512 / K1; // >= 1 (host checks K + 1 <= 512)
+	const int PBx = p.inB + 2 * p.pad;
+	const int xRowsMax = (p.rowsPerUnit - 1) * p.stride + p.ksize;
 	float *xs = thin_lds;
-	float *ds = thin_lds + ((cells * p.cin + 3) & ~3);
-	const int k = tid % K, slice = tid / K;
-	const bool live = slice < slices;
+	float *ds = thin_lds + ((p.cin * xRowsMax * PBx + 3) & ~3);
+	const int k = tid % K1, slice = tid / K1;
+	const bool live = slice < slices, ones = k == K;
 	uint32_t ci, tap, ta, tb;
-	p.divKK.divmod((uint32_t)k, ci, tap);
+	p.divKK.divmod((uint32_t)(ones ? 0 : k), ci, tap);
 	p.divK.divmod(tap, ta, tb);
 	float acc[COUT];
 #pragma unroll
 	for (int c = 0; c < COUT; c++) acc[c] = 0.f;
 	const size_t oplane = (size_t)p.samples * ocells, iplane = (size_t)p.samples * cells;
-	const int n0 = blockIdx.x * p.imagesPerGroup;
-	const int imgs = (p.samples - n0 < p.imagesPerGroup) ? p.samples - n0 : p.imagesPerGroup;
-	for (int img = 0; img < imgs; img++) {
-		const int n = n0 + img;
-		__syncthreads(); // the previous image's readers are done
+	const int units = p.samples * p.parts;
+	const int u0 = blockIdx.x * p.unitsPerGroup;
+	const int u1 = (u0 + p.unitsPerGroup < units) ? u0 + p.unitsPerGroup : units;
+	for (int unit = u0; unit < u1; unit++) {
+		const int n = unit / p.parts, part = unit - n * p.parts;
+		const int oa0 = part * p.rowsPerUnit;
+		const int rows = (p.outA - oa0 < p.rowsPerUnit) ? p.outA - oa0 : p.rowsPerUnit;
+		const int xRows = (rows - 1) * p.stride + p.ksize;
+		const int a0 = oa0 * p.stride - p.pad; // input row of the band's first bordered row
+		__syncthreads(); // the previous unit's readers are done
 		// eight loads of a thread in flight at a time
-		const int xTotal = p.cin * cells, dTotal = COUT * ocells;
+		const int xPlane = xRows * PBx, xTotal = p.cin * xPlane, dPos = rows * p.outB, dTotal = COUT * dPos;
+		const FastDiv divXPlane = p.divXPlane[rows == p.rowsPerUnit ? 0 : 1], divDPos = p.divDPos[rows == p.rowsPerUnit ? 0 : 1];
 		for (int base = tid; base < xTotal; base += 512 * 8) {
 			float v[8];
 #pragma unroll
 			for (int u = 0; u < 8; u++) {
 				const int i = base + 512 * u;
-				uint32_t c, q;
-				p.divCells.divmod((uint32_t)(i < xTotal ? i : 0), c, q);
-				v[u] = (i < xTotal) ? p.x[(size_t)c * iplane + (size_t)n * cells + q] : 0.f;
+				uint32_t c, q, r, col;
+				divXPlane.divmod((uint32_t)(i < xTotal ? i : 0), c, q);
+				p.divPBx.divmod(q, r, col);
+				const int a = a0 + (int)r, b = (int)col - p.pad;
+				const bool ok = (i < xTotal) & ((unsigned)a < (unsigned)p.inA) & ((unsigned)b < (unsigned)p.inB);
+				v[u] = ok ? x[(size_t)c * iplane + (size_t)n * cells + a * p.inB + b] : 0.f;
 			}
 #pragma unroll
 			for (int u = 0; u < 8; u++)
@@ -158,8 +171,8 @@ __global__ void __launch_bounds__(512) thin_weight_grad_kernel(const ThinConvPar
 #pragma unroll
 			for (int u = 0; u < 8; u++) {
 				const int i = base + 512 * u; // reads contiguous along the positions of a channel
-				p.divOcells.divmod((uint32_t)(i < dTotal ? i : 0), c[u], q[u]);
-				v[u] = (i < dTotal && (int)c[u] < p.cout) ? p.delta[(size_t)c[u] * oplane + (size_t)n * ocells + q[u]] : 0.f;
+				divDPos.divmod((uint32_t)(i < dTotal ? i : 0), c[u], q[u]);
+				v[u] = (i < dTotal && (int)c[u] < p.cout) ? delta[(size_t)c[u] * oplane + (size_t)n * ocells + oa0 * p.outB + q[u]] : 0.f;
 			}
 #pragma unroll
 			for (int u = 0; u < 8; u++)
@@ -167,13 +180,12 @@ __global__ void __launch_bounds__(512) thin_weight_grad_kernel(const ThinConvPar
 		}
 		__syncthreads();
 		if (live) {
-			const float *xc = xs + ci * cells;
-			for (int q = slice; q < ocells; q += slices) {
-				uint32_t oa, ob;
-				p.divOutB.divmod((uint32_t)q, oa, ob);
-				const int a = (int)oa * p.stride + (int)ta - p.pad, b = (int)ob * p.stride + (int)tb - p.pad;
-				const bool ok = ((unsigned)a < (unsigned)p.inA) & ((unsigned)b < (unsigned)p.inB);
-				const float xv = ok ? xc[a * p.inB + b] : 0.f;
+			// position q = (r, ob) of the band reads the bordered cell [r * stride + ta][ob * stride + tb]
+			const float *xc = xs + ((int)ci * xRows + (int)ta) * PBx + (int)tb;
+			uint32_t r, ob;
+			p.divOutB.divmod((uint32_t)slice, r, ob);
+			for (int q = slice; q < dPos; q += slices) {
+				const float xv = ones ? 1.f : xc[((int)r * PBx + (int)ob) * p.stride];
 				const float4 *dq = reinterpret_cast<const float4 *>(ds + q * COUT);
 #pragma unroll
 				for (int g = 0; g < COUT / 4; g++) {
@@ -183,23 +195,48 @@ __global__ void __launch_bounds__(512) thin_weight_grad_kernel(const ThinConvPar
 					acc[4 * g + 2] = fmaf(d.z, xv, acc[4 * g + 2]);
 					acc[4 * g + 3] = fmaf(d.w, xv, acc[4 * g + 3]);
 				}
+				ob += (uint32_t)slices;
+				while (ob >= (uint32_t)p.outB) ob -= (uint32_t)p.outB, r++;
 			}
 		}
 	}
-	// slices of one k are added in slice order; the sums go out as one Cout x K block per workgroup
+	// slices of one k are added in slice order; the sums go out as one Cout x (K + 1) block per workgroup
 	__syncthreads();
 	float *red = thin_lds; // [slice][k][COUT]
 	if (live) {
 #pragma unroll
-		for (int c = 0; c < COUT; c++) red[(slice * K + k) * COUT + c] = acc[c];
+		for (int c = 0; c < COUT; c++) red[(slice * K1 + k) * COUT + c] = acc[c];
 	}
 	__syncthreads();
-	float *out = partial + (size_t)blockIdx.x * p.cout * K;
-	for (int i = tid; i < p.cout * K; i += 512) {
-		const int c = i / K, kk = i - c * K;
+	float *out = partial + (size_t)blockIdx.x * p.cout * K1;
+	for (int i = tid; i < p.cout * K1; i += 512) {
+		const int c = i / K1, kk = i - c * K1;
 		float s = 0.f;
-		for (int sl = 0; sl < slices; sl++) s += red[(sl * K + kk) * COUT + c];
+		for (int sl = 0; sl < slices; sl++) s += red[(sl * K1 + kk) * COUT + c];
 		out[i] = s;
+	}
+}
+
+// dW[c][k] (k < K) and db[c] (k = K) = sum over the workgroups' blocks, in workgroup order: sixteen phases each add
+// every sixteenth block in double precision and are combined in phase order.
+__global__ void __launch_bounds__(256) thin_dw_reduce_kernel(const float *partial, int groups, int cout, int K, float *dW, float *db)
+{
+	__shared__ double part[16][17];
+	const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+	const int total = cout * (K + 1);
+	const int idx = blockIdx.x * 16 + tx;
+	double acc = 0.0;
+	if (idx < total)
+		for (int s = ty; s < groups; s += 16) acc += (double)partial[(size_t)s * total + idx];
+	part[ty][tx] = acc;
+	__syncthreads();
+	if (ty == 0 && idx < total) {
+		double sum = 0.0;
+#pragma unroll
+		for (int q = 0; q < 16; q++) sum += part[q][tx];
+		const int c = idx / (K + 1), kk = idx - c * (K + 1);
+		if (kk < K) dW[(size_t)c * K + kk] = (float)sum;
+		else if (db) db[c] = (float)sum;
 	}
 }
 
@@ -211,6 +248,11 @@ static inline ThinConvParams thin_params(const fitre_conv_shape *s)
 	p.inA = s->inA, p.inB = s->inB, p.outA = s->outA, p.outB = s->outB;
 	p.ksize = s->ksize, p.stride = s->stride, p.pad = s->padding;
 	p.imagesPerGroup = 1;
+	p.ciPerGroup = 1;
+	p.parts = 1, p.rowsPerUnit = s->outA, p.unitsPerGroup = 1;
+	p.divPBx = FastDiv((uint32_t)(s->inB + 2 * s->padding));
+	p.divPB = FastDiv((uint32_t)(s->inB + s->ksize - 1));
+	p.divPlane = FastDiv((uint32_t)((s->inA + s->ksize - 1) * (s->inB + s->ksize - 1)));
 	p.divInB = FastDiv((uint32_t)s->inB);
 	p.divOutB = FastDiv((uint32_t)s->outB);
 	p.divK = FastDiv((uint32_t)s->ksize);
@@ -221,89 +263,100 @@ static inline ThinConvParams thin_params(const fitre_conv_shape *s)
 }
 
 // ---- input gradient --------------------------------------------------------------------------------------------
-constexpr int kThinDxLdsFloats = 15360; // 60 KB: weights + delta of the group's images
-static inline int thin_dx_cin_pad(const fitre_conv_shape *s) { return s->inChannels <= 4 ? 4 : (s->inChannels <= 8 ? 8 : 16); }
-static inline int thin_dx_weight_floats(const fitre_conv_shape *s) { return s->outChannels * s->ksize * s->ksize * thin_dx_cin_pad(s); }
-static inline int thin_dx_images(const fitre_conv_shape *s)
+constexpr int kThinDxLdsFloats = 15360; // 60 KB: the bordered delta of one image
+static inline int thin_dx_lds_floats(const fitre_conv_shape *s)
 {
-	const int perImage = s->outChannels * s->outA * s->outB, cells = s->inA * s->inB;
-	const int room = kThinDxLdsFloats - thin_dx_weight_floats(s);
-	int imgs = (256 + cells - 1) / cells;
-	if (imgs * perImage > room) imgs = room / perImage;
-	if (s->samples / (imgs > 0 ? imgs : 1) < 2 * device_compute_units()) imgs = 1; // few images: spread them over the chip
-	return imgs < 1 ? 1 : imgs;
+	return s->outChannels * (s->inA + s->ksize - 1) * (s->inB + s->ksize - 1);
 }
 static inline bool thin_dx_eligible(const fitre_conv_shape *s)
 {
-	return s->stride == 1 && s->inChannels <= kThinMaxChannels && s->outChannels <= 32 && s->ksize <= 7 &&
-	       s->inChannels * s->outChannels <= 256 &&
-	       thin_dx_weight_floats(s) + s->outChannels * s->outA * s->outB <= kThinDxLdsFloats;
+	return s->stride == 1 && s->padding <= s->ksize - 1 && s->inChannels <= kThinMaxChannels && s->outChannels <= 32 &&
+	       s->ksize <= 7 && s->inChannels * s->outChannels <= 256 && thin_dx_lds_floats(s) <= kThinDxLdsFloats;
 }
 static int launch_thin_dx(const fitre_conv_shape *s, const float *delta, const float *w, float *dx)
 {
 	ThinConvParams p = thin_params(s);
-	p.delta = delta, p.w = w;
-	p.imagesPerGroup = thin_dx_images(s);
-	const int groups = (s->samples + p.imagesPerGroup - 1) / p.imagesPerGroup;
-	const size_t lds = sizeof(float) * ((size_t)p.imagesPerGroup * s->outChannels * s->outA * s->outB + (size_t)thin_dx_weight_floats(s));
+	// enough workgroups for two per compute unit where the batch alone does not give them
+	int groupsY = (2 * device_compute_units() + s->samples - 1) / s->samples;
+	if (groupsY > s->inChannels) groupsY = s->inChannels;
+	if (groupsY < 1) groupsY = 1;
+	p.ciPerGroup = (s->inChannels + groupsY - 1) / groupsY;
+	groupsY = (s->inChannels + p.ciPerGroup - 1) / p.ciPerGroup;
+	const dim3 grid((unsigned)s->samples, (unsigned)groupsY);
+	const size_t lds = sizeof(float) * (size_t)thin_dx_lds_floats(s);
 	LaunchScope scope(FITRE_KC_CONV_DX, conv_flops(s), 0);
-#define THIN_DX(CIN_, KS_) thin_input_grad_kernel<CIN_, KS_><<<groups, 256, lds, stream()>>>(p, dx)
-	if (s->inChannels <= 4) {
-		if (s->ksize == 5) THIN_DX(4, 5);
-		else if (s->ksize == 3) THIN_DX(4, 3);
-		else THIN_DX(4, 0);
-	} else if (s->inChannels <= 8) {
-		if (s->ksize == 5) THIN_DX(8, 5);
-		else if (s->ksize == 3) THIN_DX(8, 3);
-		else THIN_DX(8, 0);
-	} else {
-		THIN_DX(16, 0);
-	}
-#undef THIN_DX
+	if (s->ksize == 5) thin_input_grad_kernel<5><<<grid, 256, lds, stream()>>>(p, w, delta, dx);
+	else if (s->ksize == 3) thin_input_grad_kernel<3><<<grid, 256, lds, stream()>>>(p, w, delta, dx);
+	else thin_input_grad_kernel<0><<<grid, 256, lds, stream()>>>(p, w, delta, dx);
 	return check_launch("thin_input_grad_kernel");
 }
 
 // ---- weight gradient -------------------------------------------------------------------------------------------
 static inline int thin_dw_pad(int cout) { return cout <= 8 ? 8 : 16; }
+struct ThinDwPlan {
+	int parts, rowsPerUnit, unitsPerGroup, groups;
+};
+// One workgroup per compute unit where the batch gives that many images; below that the images are cut into bands
+// of output rows (at least four rows each).
+static inline ThinDwPlan thin_dw_plan(const fitre_conv_shape *s)
+{
+	const int target = device_compute_units();
+	ThinDwPlan pl;
+	pl.parts = (target + s->samples - 1) / s->samples;
+	if (pl.parts > s->outA / 4) pl.parts = s->outA / 4;
+	if (pl.parts < 1) pl.parts = 1;
+	pl.rowsPerUnit = (s->outA + pl.parts - 1) / pl.parts;
+	pl.parts = (s->outA + pl.rowsPerUnit - 1) / pl.rowsPerUnit;
+	const long units = (long)s->samples * pl.parts;
+	long groups = 2L * target < units ? 2L * target : units;
+	pl.unitsPerGroup = (int)((units + groups - 1) / groups);
+	pl.groups = (int)((units + pl.unitsPerGroup - 1) / pl.unitsPerGroup);
+	return pl;
+}
 static inline size_t thin_dw_lds_floats(const fitre_conv_shape *s)
 {
-	const int K = s->inChannels * s->ksize * s->ksize, cp = thin_dw_pad(s->outChannels);
-	const size_t stage = (size_t)((s->inA * s->inB * s->inChannels + 3) & ~3) + (size_t)s->outA * s->outB * cp;
-	const size_t red = (size_t)(512 / K) * K * cp;
+	const ThinDwPlan pl = thin_dw_plan(s);
+	const int K1 = s->inChannels * s->ksize * s->ksize + 1, cp = thin_dw_pad(s->outChannels);
+	const int xRows = (pl.rowsPerUnit - 1) * s->stride + s->ksize;
+	const size_t stage = (size_t)((s->inChannels * xRows * (s->inB + 2 * s->padding) + 3) & ~3) + (size_t)pl.rowsPerUnit * s->outB * cp;
+	const size_t red = (size_t)(512 / K1) * K1 * cp;
 	return stage > red ? stage : red;
 }
 static inline bool thin_dw_general_eligible(const fitre_conv_shape *s)
 {
 	const int K = s->inChannels * s->ksize * s->ksize;
-	return s->outChannels <= kThinMaxChannels && K <= 512 && K >= 16 && thin_dw_lds_floats(s) <= (size_t)kThinLdsFloats;
+	return s->outChannels <= kThinMaxChannels && K < 512 && K >= 16 && thin_dw_lds_floats(s) <= (size_t)kThinLdsFloats;
 }
-static inline int thin_dw_general_groups(const fitre_conv_shape *s, int *imagesPerGroup)
-{
-	int groups = 2 * device_compute_units();
-	if (groups > s->samples) groups = s->samples;
-	const int per = (s->samples + groups - 1) / groups;
-	*imagesPerGroup = per;
-	return (s->samples + per - 1) / per;
-}
+// sized for the largest number of workgroups any batch size gets, so that a buffer laid out for a model's full
+// batch also serves its partial batches
 static inline size_t thin_dw_general_workspace(const fitre_conv_shape *s)
 {
-	int per;
-	return sizeof(float) * (size_t)thin_dw_general_groups(s, &per) * s->outChannels * s->inChannels * s->ksize * s->ksize;
+	return sizeof(float) * 2 * (size_t)device_compute_units() * s->outChannels * (s->inChannels * s->ksize * s->ksize + 1);
 }
-static int launch_thin_dw_general(const fitre_conv_shape *s, const float *x, const float *delta, float *dW, void *ws)
+// db may be null
+static int launch_thin_dw_general(const fitre_conv_shape *s, const float *x, const float *delta, float *dW, float *db, void *ws)
 {
 	ThinConvParams p = thin_params(s);
-	p.x = x, p.delta = delta;
-	const int groups = thin_dw_general_groups(s, &p.imagesPerGroup);
+	const ThinDwPlan pl = thin_dw_plan(s);
+	p.parts = pl.parts, p.rowsPerUnit = pl.rowsPerUnit, p.unitsPerGroup = pl.unitsPerGroup;
+	const int lastRows = s->outA - (pl.parts - 1) * pl.rowsPerUnit;
+	const int bandRows[2] = { pl.rowsPerUnit, lastRows };
+	for (int i = 0; i < 2; i++) {
+		p.divXPlane[i] = FastDiv((uint32_t)(((bandRows[i] - 1) * s->stride + s->ksize) * (s->inB + 2 * s->padding)));
+		p.divDPos[i] = FastDiv((uint32_t)(bandRows[i] * s->outB));
+	}
 	const int K = s->inChannels * s->ksize * s->ksize;
 	const size_t lds = sizeof(float) * thin_dw_lds_floats(s);
 	{
 		LaunchScope scope(FITRE_KC_CONV_DW, conv_flops(s), 0);
-		if (thin_dw_pad(s->outChannels) == 8) thin_weight_grad_kernel<8><<<groups, 512, lds, stream()>>>(p, (float *)ws);
-		else thin_weight_grad_kernel<16><<<groups, 512, lds, stream()>>>(p, (float *)ws);
+		if (thin_dw_pad(s->outChannels) == 8) thin_weight_grad_kernel<8><<<pl.groups, 512, lds, stream()>>>(p, x, delta, (float *)ws);
+		else thin_weight_grad_kernel<16><<<pl.groups, 512, lds, stream()>>>(p, x, delta, (float *)ws);
 	}
-	OutParams out{ dW, (long)K, 0, nullptr, nullptr, 1.f, 0.f };
-	launch_splitk_reduce((const float *)ws, groups, s->outChannels, K, out);
+	{
+		const int total = s->outChannels * (K + 1);
+		LaunchScope scope(FITRE_KC_SPLITK_REDUCE, 4.0 * (double)total * (pl.groups + 1));
+		thin_dw_reduce_kernel<<<(total + 15) / 16, 256, 0, stream()>>>((const float *)ws, pl.groups, s->outChannels, K, dW, db);
+	}
 	return check_launch("thin_weight_grad_kernel");
 }
 

@@ -7,7 +7,7 @@
 //                    convolution layout (the permutation at the boundary, :330-348)
 //   weight gradient  dW = delta * z', db = delta * 1                  functions/cnn_backward.cu:189-197, :216-224
 //
-// One workgroup owns a 32 x 32 block of the result and walks the reduction in blocks of 32 through LDS; a thread
+// One workgroup owns a 32 x 32 block of the result and walks the reduction in blocks of 64 through LDS; a thread
 // holds 2 x 2 results.  The order of the additions is fixed by the shape alone.
 #pragma once
 #include "common.h"
@@ -16,6 +16,7 @@
 namespace fitre {
 
 constexpr int kSmallTile = 32;
+constexpr int kSmallDepth = 64; // reduction indices per block
 
 struct SmallGemmParams {
 	int M, N, K;
@@ -51,37 +52,39 @@ __device__ __forceinline__ float act_backward_value(int actFun, float d, float z
 
 __global__ void __launch_bounds__(256) small_gemm_kernel(const SmallGemmParams p)
 {
-	__shared__ float As[kSmallTile][kSmallTile + 1]; // [k][m]
-	__shared__ float Bs[kSmallTile][kSmallTile + 1]; // [k][n]
+	__shared__ float As[kSmallDepth][kSmallTile + 1]; // [k][m]
+	__shared__ float Bs[kSmallDepth][kSmallTile + 1]; // [k][n]
 	const int tid = threadIdx.x;
 	const int m0 = blockIdx.x * kSmallTile, n0 = blockIdx.y * kSmallTile;
 	const int tm = tid & 15, tn = tid >> 4;
-	// loads run along whichever index is contiguous in memory
+	// loads run along whichever index is contiguous in memory; all of a block's loads are in flight together
 	const bool aAlongM = p.sAm == 1, bAlongN = p.sBn == 1;
-	const int lo = tid & 31, hi = tid >> 5; // hi: 0..7
+	constexpr int kPer = kSmallDepth * kSmallTile / 256; // elements of each operand a thread loads per block
 	float acc00 = 0.f, acc01 = 0.f, acc10 = 0.f, acc11 = 0.f, rs0 = 0.f, rs1 = 0.f;
 	const bool sums = p.rowSums != nullptr && blockIdx.y == 0 && tn == 0;
-	for (int k0 = 0; k0 < p.K; k0 += kSmallTile) {
-		float av[4], bv[4];
+	for (int k0 = 0; k0 < p.K; k0 += kSmallDepth) {
+		float av[kPer], bv[kPer];
 #pragma unroll
-		for (int i = 0; i < 4; i++) {
-			const int am = aAlongM ? lo : hi + 8 * i, ak = aAlongM ? hi + 8 * i : lo;
-			const int bn = bAlongN ? lo : hi + 8 * i, bk = bAlongN ? hi + 8 * i : lo;
+		for (int i = 0; i < kPer; i++) {
+			const int e = tid + 256 * i; // along the tile: e % 32; along the depth: e / 32 -- or the other way round
+			const int am = aAlongM ? (e & 31) : e / kSmallDepth, ak = aAlongM ? (e >> 5) : e % kSmallDepth;
+			const int bn = bAlongN ? (e & 31) : e / kSmallDepth, bk = bAlongN ? (e >> 5) : e % kSmallDepth;
 			const bool aok = (m0 + am < p.M) & (k0 + ak < p.K), bok = (n0 + bn < p.N) & (k0 + bk < p.K);
 			av[i] = aok ? p.A[(long)(m0 + am) * p.sAm + (long)(k0 + ak) * p.sAk] : 0.f;
 			bv[i] = bok ? p.B[(long)(k0 + bk) * p.sBk + (long)(n0 + bn) * p.sBn] : 0.f;
 		}
 		__syncthreads(); // the previous block's readers are done
 #pragma unroll
-		for (int i = 0; i < 4; i++) {
-			const int am = aAlongM ? lo : hi + 8 * i, ak = aAlongM ? hi + 8 * i : lo;
-			const int bn = bAlongN ? lo : hi + 8 * i, bk = bAlongN ? hi + 8 * i : lo;
+		for (int i = 0; i < kPer; i++) {
+			const int e = tid + 256 * i;
+			const int am = aAlongM ? (e & 31) : e / kSmallDepth, ak = aAlongM ? (e >> 5) : e % kSmallDepth;
+			const int bn = bAlongN ? (e & 31) : e / kSmallDepth, bk = bAlongN ? (e >> 5) : e % kSmallDepth;
 			As[ak][am] = av[i];
 			Bs[bk][bn] = bv[i];
 		}
 		__syncthreads();
-#pragma unroll
-		for (int k = 0; k < kSmallTile; k++) {
+		const int depth = (p.K - k0 < kSmallDepth) ? p.K - k0 : kSmallDepth;
+		for (int k = 0; k < depth; k++) {
 			const float a0 = As[k][tm], a1 = As[k][tm + 16], b0 = Bs[k][tn], b1 = Bs[k][tn + 16];
 			acc00 = fmaf(a0, b0, acc00);
 			acc10 = fmaf(a1, b0, acc10);

@@ -273,6 +273,7 @@ int fitre_hip_lane_wait(int waiter, int signaller)
 	FITRE_REQUIRE(waiter >= 0 && waiter < kLanes && signaller >= 0 && signaller < kLanes,
 	              "fitre_hip_lane_wait: lane out of range (%d waits for %d)", waiter, signaller);
 	if (waiter == signaller) return FITRE_OK;
+	if (g_profile || !g_lanes_on) return FITRE_OK; // everything is queued on lane 0: already in order
 	hipEvent_t e = g_join[g_join_next];
 	g_join_next = (g_join_next + 1) % kJoinEvents;
 	FITRE_HIP_TRY(hipEventRecord(e, g_lanes[signaller]));

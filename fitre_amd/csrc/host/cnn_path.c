@@ -246,6 +246,23 @@ real cnnForward(CNN_MODEL *model, DEVICE_DATASET *data, SCRATCH_AREA *scratch, r
 	return loss;
 }
 
+/* Multiply-adds of the convolution layers' two gradient products: what decides whether a pass is long enough for
+ * the lanes to pay.  Ordering two lanes costs the host two runtime calls per dependency, about as long as a
+ * kernel of LeNet at batch 128 runs, so a pass of such kernels is faster queued on one lane (measured: 0.136 ms
+ * against 0.167 ms); from about LeNet at batch 1024 on the overlap wins. */
+static double backward_conv_work(const CNN_MODEL *model, int n)
+{
+	double macs = 0;
+	for (int c = 0; c < model->cLayers; c++) {
+		const CONV_LAYER *l = &model->convLayer[c];
+		macs += 2.0 * n * l->outHeight * l->outWidth * (double)l->outChannels * l->inChannels * l->kSize * l->kSize;
+	}
+	return macs;
+}
+#define LANE_WORK_THRESHOLD 2.0e9
+#define LANE_SELECT(lane_) do { if (lanes) HIP_CALL(fitre_hip_lane_select(lane_)); } while (0)
+#define LANE_WAIT(waiter_, signaller_) do { if (lanes) HIP_CALL(fitre_hip_lane_wait(waiter_, signaller_)); } while (0)
+
 void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, real *gradient, real *dx, real *delta,
                  real *delta_new, int offset, int batchSize, real *hostPtr)
 {
@@ -254,6 +271,7 @@ void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, 
 	const int *wOffsets = model->wOffsets, *bOffsets = model->bOffsets, *zOffsets = model->zOffsets;
 	const real *weights = data->weights;
 	const int n = batchSize, nc = model->cLayers;
+	const int lanes = backward_conv_work(model, n) >= LANE_WORK_THRESHOLD;
 	void *ws = (void *)devPtr; /* input-gradient partials (and the FC products' splits) */
 	const size_t wsBytes = backward_dx_ws_bytes(model, model->batchSize);
 	void *bnWs = (void *)((char *)devPtr + wsBytes);
@@ -287,13 +305,13 @@ void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, 
 			const size_t bytes = fitre_hip_conv_input_grad_prepared_bytes(&shape);
 			prepared[c] = NULL;
 			if (bytes == 0 || !has_bn(&model->convLayer[c - 1])) continue;
-			if (!any) HIP_CALL(fitre_hip_lane_select(2));
+			if (!any) LANE_SELECT(2);
 			any = 1;
 			HIP_CALL(fitre_hip_conv_input_grad_prepare(&shape, weights + wOffsets[c], preparedWs, bytes));
 			prepared[c] = preparedWs;
 			preparedWs += (bytes + 255) & ~(size_t)255;
 		}
-		if (any) HIP_CALL(fitre_hip_lane_select(0));
+		if (any) LANE_SELECT(0);
 		preparedPending = any;
 	}
 
@@ -317,7 +335,7 @@ void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, 
 		 * from the epilogue of the product above them */
 		if (f == model->lLayers - 1)
 			HIP_CALL(fitre_hip_activation_backward(l->actFun, delta, zl + l->offset, zl, slot, (long)l->out * n));
-		HIP_CALL(fitre_hip_lane_wait(1, 0));
+		LANE_WAIT(1, 0);
 		/* the chain goes straight on: delta of the layer below = f'(.) .* (W' * delta) */
 		if (f > 0) {
 			const FC_LAYER *below = &model->fcLayer[f - 1];
@@ -329,10 +347,10 @@ void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, 
 			                                     features, delta_new, ws, wsBytes));
 		}
 		/* beside it, on lane 1, what nothing later in this pass reads: dW = delta * z', db = delta * 1 */
-		HIP_CALL(fitre_hip_lane_select(1));
+		LANE_SELECT(1);
 		HIP_CALL(fitre_hip_linear_weight_grad(l->in, l->out, n, slot, zin, gradient + wOffsets[f + nc],
 		                                      (model->bias != 0) ? gradient + bOffsets[f + nc] : NULL, sideWs, sideBytes));
-		HIP_CALL(fitre_hip_lane_select(0));
+		LANE_SELECT(0);
 	}
 	if (model->lLayers == 0) HIP_CALL(fitre_hip_fc_to_conv(delta, last->outChannels, n, extA, extB, features));
 
@@ -391,7 +409,7 @@ void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, 
 		if (c != 0) {
 			if (has_bn(&model->convLayer[c - 1])) {
 				if (prepared[c] && preparedPending) { /* the chain's first use of a copy lane 2 made */
-					HIP_CALL(fitre_hip_lane_wait(0, 2));
+					LANE_WAIT(0, 2);
 					preparedPending = 0;
 				}
 				HIP_CALL(fitre_hip_conv_input_grad_split_prepared(&shape, cur, weights + wOffsets[c], prepared[c], delta, ws, wsBytes,
@@ -404,17 +422,18 @@ void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, 
 		/* A weight gradient on the general tile engine stays in line: beside the next layer's matrix kernels both would
 		 * lose more than the overlap gains.  Its workspace is lane 1's, so the lanes are ordered around it. */
 		const int beside = fitre_hip_conv_weight_grad_runs_beside(&shape);
-		HIP_CALL(fitre_hip_lane_wait(1, 0));
+		LANE_WAIT(1, 0);
 		if (beside) {
-			HIP_CALL(fitre_hip_lane_select(1));
+			LANE_SELECT(1);
 		} else {
-			HIP_CALL(fitre_hip_lane_wait(0, 1));
+			LANE_WAIT(0, 1);
 		}
-		/* without batch norm the bias gradient is a pass of its own over delta; nothing in the chain reads it */
-		if (!has_bn(l) && model->bias != 0)
-			HIP_CALL(fitre_hip_channel_sum(cur, l->outChannels, perChannel, gradient + bOffsets[c], sideWs, sideBytes));
-		HIP_CALL(fitre_hip_conv_weight_grad(&shape, input, cur, gradient + wOffsets[c], sideWs, sideBytes));
-		if (beside) HIP_CALL(fitre_hip_lane_select(0));
+		/* without batch norm the bias gradient is taken here as well (with batch norm it is a by-product of its
+		 * backward pass above); nothing in the chain reads either */
+		HIP_CALL(fitre_hip_conv_weight_bias_grad(&shape, input, cur, gradient + wOffsets[c],
+		                                         (!has_bn(l) && model->bias != 0) ? gradient + bOffsets[c] : NULL, sideWs,
+		                                         sideBytes));
+		if (beside) LANE_SELECT(0);
 	}
 	HIP_CALL(fitre_hip_sync());
 }

@@ -109,6 +109,8 @@ HIP_API = {
     "fitre_hip_conv_weight_grad_workspace": (sz, [pshape]),
     "fitre_hip_conv_weight_grad_runs_beside": (i32, [pshape]),
     "fitre_hip_conv_weight_grad": (i32, [pshape, vp, vp, vp, vp, sz]),
+    "fitre_hip_conv_weight_bias_grad_workspace": (sz, [pshape]),
+    "fitre_hip_conv_weight_bias_grad": (i32, [pshape, vp, vp, vp, vp, vp, sz]),
     "fitre_hip_conv_input_grad_workspace": (sz, [pshape]),
     "fitre_hip_conv_input_grad": (i32, [pshape, vp, vp, vp, vp, sz]),
     "fitre_hip_gemm_workspace": (sz, [i32, i32, i32]),

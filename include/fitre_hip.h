@@ -319,6 +319,13 @@ size_t fitre_hip_conv_weight_grad_workspace(const fitre_conv_shape *s);
 int fitre_hip_conv_weight_grad_runs_beside(const fitre_conv_shape *s);
 int fitre_hip_conv_weight_grad(const fitre_conv_shape *s, const float *x, const float *delta, float *dW,
                                void *ws, size_t wsBytes);
+/* The same with the bias gradient db[Cout] = sum of delta over samples and positions (functions/cnn_backward.cu:
+ * 662-689), for layers without batch norm: one pass over delta where the layer has few channels, else
+ * fitre_hip_channel_sum followed by fitre_hip_conv_weight_grad.  db may be NULL (then this is
+ * fitre_hip_conv_weight_grad). */
+size_t fitre_hip_conv_weight_bias_grad_workspace(const fitre_conv_shape *s);
+int fitre_hip_conv_weight_bias_grad(const fitre_conv_shape *s, const float *x, const float *delta, float *dW,
+                                    float *db, void *ws, size_t wsBytes);
 /* dx[Cin][N][inA][inB] = transposed convolution of delta with w; stride must be 1.  Replaces
  * functions/dev_backprop_convolution.cu:173-247. */
 size_t fitre_hip_conv_input_grad_workspace(const fitre_conv_shape *s);

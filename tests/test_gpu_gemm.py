@@ -58,6 +58,15 @@ CONV_CASES = [
     (3, 3, 64, 1, 128, 3, 1, 1),     # one row per chunk: nothing above or below
     (2, 3, 16, 12, 32, 3, 1, 1),     # A not a multiple of the rows per chunk... 12 % 4 == 0: eligible
     (2, 3, 16, 6, 32, 3, 1, 1),      # 6 % 4 != 0: general engine
+    # few channels, the vector kernels: bands of output rows, several images per workgroup, borders, strides
+    (128, 3, 6, 32, 32, 5, 1, 0),    # LeNet conv1 at batch 128: two bands per image
+    (128, 6, 16, 14, 14, 5, 1, 0),   # LeNet conv2 at batch 128
+    (600, 6, 16, 14, 14, 5, 1, 0),   # more images than workgroups: two units per workgroup, a ragged last one
+    (5, 6, 16, 14, 14, 5, 1, 2),     # padded: the zero border of both kernels
+    (3, 4, 12, 11, 9, 3, 1, 1),      # rectangular, 3x3 window, bands of uneven height
+    (7, 2, 5, 13, 13, 4, 1, 3),      # even window, border of the full window minus one
+    (9, 5, 10, 15, 15, 5, 2, 1),     # strided weight gradient
+    (2, 16, 16, 9, 9, 5, 1, 0),      # sixteen channels each side
 ]
 
 
@@ -108,6 +117,35 @@ def test_conv_weight_gradient(dev, oracle64, case):
 def test_conv_input_gradient(dev, oracle64, case):
     got, want = run_conv(dev, oracle64, case, "dx")
     assert rel_err(got, want) < TOL
+
+
+@pytest.mark.parametrize("case", [c for c in CONV_CASES if c[1] <= 16 and c[2] <= 16 or c in CONV_CASES[2:5]])
+def test_conv_weight_and_bias_gradient(dev, oracle64, case):
+    """dW and db = sum of delta per output channel in one call: the fused kernel of thin layers and the two-step path of
+    the others, against the float64 oracle and numpy; the bias slot's neighbours stay untouched."""
+    N, Cin, Cout, A, B, k, s, p = case
+    shape = conv_shape(N, Cin, Cout, A, B, k, s, p)
+    oA, oB = shape.outA, shape.outB
+    rng = np.random.default_rng(sum(case) + 5)
+    x = rng.standard_normal(Cin * N * A * B).astype(np.float32)
+    d = rng.standard_normal(Cout * N * oA * oB).astype(np.float32)
+    px, pd = dev.upload(x), dev.upload(d)
+    nb = hip.fitre_hip_conv_weight_bias_grad_workspace(C.byref(shape))
+    assert nb >= hip.fitre_hip_conv_weight_grad_workspace(C.byref(shape))
+    ws = dev.alloc(nb)
+    dw = dev.upload(np.full(Cout * Cin * k * k + 2, 3.0, np.float32))
+    db = dev.upload(np.full(Cout + 2, 5.0, np.float32))
+    L.check(hip.fitre_hip_conv_weight_bias_grad(C.byref(shape), px, pd, dw, db, ws, nb))
+    got_w, got_b = dev.download(dw, Cout * Cin * k * k + 2), dev.download(db, Cout + 2)
+    assert rel_err(got_w[:-2], oracle64.conv_weight_grad(x, d, N, Cin, B, A, k, p, s, Cout)) < TOL
+    assert rel_err(got_b[:Cout], d.astype(np.float64).reshape(Cout, -1).sum(axis=1)) < TOL
+    assert (got_w[-2:] == 3.0).all() and (got_b[Cout:] == 5.0).all()
+    # without a bias slot: the plain weight gradient
+    L.check(hip.fitre_hip_memset(dw, 0, 4 * Cout * Cin * k * k))
+    L.check(hip.fitre_hip_conv_weight_bias_grad(C.byref(shape), px, pd, dw, None, ws, nb))
+    assert rel_err(dev.download(dw, Cout * Cin * k * k), oracle64.conv_weight_grad(x, d, N, Cin, B, A, k, p, s, Cout)) < TOL
+    for q in (px, pd, ws, dw, db):
+        dev.free(q)
 
 
 PAIR_CASES = [c for c in CONV_CASES if c[5] == 3 and c[6] == 1 and c[7] == 1] + [(256, 64, 128, 16, 16, 3, 1, 1),
