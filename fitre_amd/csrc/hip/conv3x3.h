@@ -631,6 +631,18 @@ conv3x3_dw_thin_kernel(const ThinDwParams p, float *partial)
 	constexpr int XE = (3 * kThinXPlane + kGemmThreads - 1) / kGemmThreads;
 	float xreg[XE];
 	const int winCells = (R + 2) * rowLd;
+	// which window cell each of this thread's XE words is does not depend on the chunk: worked out once
+	// (three divisions by run-time values per word)
+	int xRow[XE], xSrc[XE], xDst[XE]; // window row, channel and column offset in x (< 0: a border cell), word in Xs (< 0: none)
+#pragma unroll
+	for (int e = 0; e < XE; e++) {
+		const int w = tid + kGemmThreads * e;
+		const int c = w / winCells, cell = w - c * winCells;
+		const int r = cell / rowLd, col = cell - r * rowLd;
+		xRow[e] = r;
+		xSrc[e] = (c < p.cin && col >= 1 && col <= p.B) ? c * p.plane + col - 1 : -1; // -1: a border column or no channel
+		xDst[e] = (c < 3) ? c * kThinXPlane + cell : -1;
+	}
 
 	auto load_chunk = [&](int q) {
 		const int m0 = q * kThinChunk;
@@ -643,17 +655,12 @@ conv3x3_dw_thin_kernel(const ThinDwParams p, float *partial)
 		}
 		const int n = m0 / imageCells;
 		const int a0 = (m0 - n * imageCells) >> p.logB; // first image row of the chunk
+		const int imageBase = n * imageCells;
 #pragma unroll
 		for (int e = 0; e < XE; e++) {
-			const int w = tid + kGemmThreads * e;
-			const int c = w / winCells, cell = w - c * winCells;
-			float v = 0.f;
-			if (c < p.cin) {
-				const int r = cell / rowLd, col = cell - r * rowLd;
-				const int a = a0 - 1 + r, b = col - 1;
-				if (a >= 0 && a < p.A && b >= 0 && b < p.B) v = p.x[(size_t)c * p.plane + (size_t)n * imageCells + a * p.B + b];
-			}
-			xreg[e] = v;
+			const int a = a0 - 1 + xRow[e];
+			const bool ok = (xSrc[e] >= 0) & ((unsigned)a < (unsigned)p.A);
+			xreg[e] = ok ? p.x[(size_t)xSrc[e] + (size_t)imageBase + a * p.B] : 0.f;
 		}
 	};
 	auto store_chunk = [&](int buf) {
@@ -665,11 +672,8 @@ conv3x3_dw_thin_kernel(const ThinDwParams p, float *partial)
 			dst[0] = dreg[e].x, dst[1] = dreg[e].y, dst[2] = dreg[e].z, dst[3] = dreg[e].w;
 		}
 #pragma unroll
-		for (int e = 0; e < XE; e++) {
-			const int w = tid + kGemmThreads * e;
-			const int c = w / winCells, cell = w - c * winCells;
-			if (c < 3) Xs[buf][c * kThinXPlane + cell] = xreg[e];
-		}
+		for (int e = 0; e < XE; e++)
+			if (xDst[e] >= 0) Xs[buf][xDst[e]] = xreg[e];
 	};
 
 	v16f acc0, acc1;

@@ -1,0 +1,218 @@
+// 3x3 / stride 1 / pad 1 convolution gradients on 4 x 4 maps without the padding's share of the arithmetic.
+//
+// On a 4 x 4 map 44 of the 16 x 9 = 144 (cell, tap) pairs of an image reach outside it.  The nine-tap kernels
+// of conv3x3.h multiply those with zeros: their MFMA blocks hold consecutive flat positions, i.e. two whole
+// images, so every block has live cells for every tap.  Here a block's 32 columns (input gradient) or its
+// reduction pairs (weight gradient) are the SAME cell of different images: a (cell, tap) pair is then live or
+// dead for the whole block, the dead ones are left out at compile time, and the matrix pipes do 100 / 144 of
+// the work (the layers of VGG-11 with 4 x 4 maps hold 40 % of a backward pass's matrix time).  No border
+// masks, pads or halo are needed: a tap that is issued always reads a cell of the same image.
+#pragma once
+#include "conv3x3.h"
+
+namespace fitre {
+
+constexpr int kCellMap = 4;                   // map extent
+constexpr int kCells = kCellMap * kCellMap;   // cells per image
+constexpr int kCellStageImages = kC3Stage / kCells; // images per weight-gradient stage (64 positions)
+
+__host__ __device__ constexpr bool cell_tap_live(int cell, int tap)
+{
+	const int a = cell / kCellMap + tap / 3 - 1, b = cell % kCellMap + tap % 3 - 1;
+	return a >= 0 && a < kCellMap && b >= 0 && b < kCellMap;
+}
+__host__ __device__ constexpr int cell_tap_source(int cell, int tap) { return cell + (tap / 3 - 1) * kCellMap + (tap % 3 - 1); }
+
+// ---------------------------------------------------------------------------------
+// weight gradient: dW[o][c][tap] = sum over images and live cells of delta[o][n][cell] * src[c][n][cell + tap shift]
+// ---------------------------------------------------------------------------------
+// Geometry of conv3x3_dw_kernel: twelve waves own 128 output channels x 32 input channels x nine taps, a stage
+// is 64 positions = four images.  A reduction pair of an MFMA step is one cell of two neighbouring images, so
+// delta and source sit in LDS as they sit in memory, [channel][image][cell] with an odd row stride.  The nine
+// taps have 9 (corner taps), 12 (edge taps) and 16 (centre) live cells; the three waves of an output-channel
+// block take tap groups of equal weight -- {centre, two opposite corners} = 34, {two edges, a corner} = 33 twice.
+__device__ constexpr int kCellTapGroups[3][3] = { { 4, 0, 8 }, { 1, 3, 2 }, { 5, 7, 6 } };
+
+template <int TG>
+__device__ __forceinline__ void cell_dw_steps(const float *aBase, const float *bBase, v16f (&acc)[3])
+{
+#pragma unroll
+	for (int ip = 0; ip < kCellStageImages / 2; ip++) {
+#pragma unroll
+		for (int cell = 0; cell < kCells; cell++) {
+			const bool any = cell_tap_live(cell, kCellTapGroups[TG][0]) || cell_tap_live(cell, kCellTapGroups[TG][1]) ||
+			                 cell_tap_live(cell, kCellTapGroups[TG][2]);
+			if (!any) continue;
+			const float fa = aBase[ip * 2 * kCells + cell];
+#pragma unroll
+			for (int j = 0; j < 3; j++) {
+				const int tap = kCellTapGroups[TG][j];
+				if (cell_tap_live(cell, tap)) {
+					const float fb = bBase[ip * 2 * kCells + cell_tap_source(cell, tap)];
+					acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa, fb, acc[j], 0, 0, 0);
+				}
+			}
+		}
+	}
+}
+
+template <bool VEC>
+__global__ void __launch_bounds__(kC3DwThreads)
+conv3x3_dw_cell_kernel(const Conv3x3Params p, const float *delta, uint32_t deltaBytes, const OutParams out)
+{
+	FITRE_RAISE_MATRIX_WAVE_PRIORITY();
+	constexpr int T = kC3DwThreads;
+	constexpr int LD = kC3Stage + 1; // odd row stride of both stages
+	constexpr int D_DUMMY = kC3Tile * LD, X_DUMMY = kC3DwCin * LD;
+	constexpr int DGROUPS = kC3Tile * kC3Stage / 4; // 4-float groups of delta per stage
+	constexpr int DE = (DGROUPS + T - 1) / T;
+	constexpr int XGROUPS = kC3DwCin * kC3Stage / 4; // 512: one per thread of the first eight waves
+	static_assert(XGROUPS <= T, "one source group per thread");
+	__shared__ float Ds[2][D_DUMMY + 4];
+	__shared__ float Xs[2][X_DUMMY + 4];
+
+	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+	const int khalf = lane >> 5, l32 = lane & 31;
+	const int ob = wave & 3, tg = wave >> 2; // output-channel block, tap group
+	// workgroups renumbered so that an XCD (its own L2) holds consecutive indices, as in conv3x3_dw_kernel
+	int bx, by, bz;
+	{
+		const unsigned groups = gridDim.x * gridDim.y * gridDim.z;
+		const unsigned lin = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+		const unsigned xcd = lin & 7u, each = groups >> 3, extra = groups & 7u;
+		const unsigned logical = xcd * each + (xcd < extra ? xcd : extra) + (lin >> 3);
+		const unsigned tiles = gridDim.x * gridDim.y;
+		bz = (int)(logical / tiles);
+		const unsigned rem = logical - (unsigned)bz * tiles;
+		by = (int)(rem / gridDim.x);
+		bx = (int)(rem - (unsigned)by * gridDim.x);
+	}
+	const int c0 = bx * kC3DwCin, o0 = by * kC3Tile;
+	const int plane = p.J;
+	const int stagesHalf = p.J / kC3Stage;
+	const int stagesTotal = p.src2 ? 2 * stagesHalf : stagesHalf; // a second (source, delta) pair continues the reduction
+	const int stBeg = bz * p.perSplit;
+	const int stEnd = (stBeg + p.perSplit < stagesTotal) ? stBeg + p.perSplit : stagesTotal;
+
+	// ---- what this thread stages ------------------------------------------------------------
+	const int dCol = 4 * (tid % (kC3Stage / 4));
+	uint32_t dOff[DE];
+	int dLds[DE];
+#pragma unroll
+	for (int e = 0; e < DE; e++) {
+		const int idx = tid + T * e;
+		const int row = idx / (kC3Stage / 4);
+		const bool has = idx < DGROUPS;
+		const bool inside = has & ((o0 + row) < p.I);
+		// rows past the tensor feed accumulator rows that are never stored
+		const uint32_t off = 4u * (uint32_t)((o0 + row) * plane + dCol);
+		dOff[e] = VEC ? (inside ? off : 4u * (uint32_t)dCol) : (inside ? off : kGroupOutOfRange);
+		dLds[e] = has ? row * LD + dCol : D_DUMMY;
+	}
+	const int xRow = tid / (kC3Stage / 4);
+	const bool xHas = tid < XGROUPS;
+	const bool xInside = xHas & ((c0 + xRow) < p.cred);
+	const uint32_t xOff = VEC ? (xInside ? 4u * (uint32_t)((c0 + xRow) * plane + dCol) : 4u * (uint32_t)dCol)
+	                          : (xInside ? 4u * (uint32_t)((c0 + xRow) * plane + dCol) : kGroupOutOfRange);
+	const int xLds = xHas ? xRow * LD + dCol : X_DUMMY;
+	float dreg[DE * 4];
+	float xreg[4];
+
+#define CELL_LOAD_STAGE(ST)                                                                                           \
+	{                                                                                                                 \
+		const bool second_ = (ST) >= stagesHalf; /* uniform */                                                        \
+		const int m0_ = ((ST) - (second_ ? stagesHalf : 0)) * kC3Stage;                                               \
+		const float *dSel = second_ ? p.w2 : delta;                                                                   \
+		const float *xSel = second_ ? p.src2 : p.src;                                                                 \
+		if constexpr (VEC) {                                                                                          \
+			const char *dBlk = reinterpret_cast<const char *>(dSel + m0_);                                            \
+			_Pragma("unroll") for (int e = 0; e < DE; e++)                                                            \
+			{                                                                                                         \
+				const float4 v4 = *reinterpret_cast<const float4 *>(dBlk + dOff[e]);                                  \
+				dreg[4 * e + 0] = v4.x, dreg[4 * e + 1] = v4.y, dreg[4 * e + 2] = v4.z, dreg[4 * e + 3] = v4.w;       \
+			}                                                                                                         \
+			const float4 x4 = *reinterpret_cast<const float4 *>(reinterpret_cast<const char *>(xSel + m0_) + xOff);   \
+			xreg[0] = xInside ? x4.x : 0.f, xreg[1] = xInside ? x4.y : 0.f;                                           \
+			xreg[2] = xInside ? x4.z : 0.f, xreg[3] = xInside ? x4.w : 0.f;                                           \
+		} else {                                                                                                      \
+			const __amdgpu_buffer_rsrc_t dRs = make_rsrc(dSel + m0_, deltaBytes - 4u * (uint32_t)m0_);                \
+			_Pragma("unroll") for (int e = 0; e < DE; e++)                                                            \
+			{                                                                                                         \
+				dreg[4 * e + 0] = buffer_load(dRs, dOff[e]);                                                          \
+				dreg[4 * e + 1] = buffer_load(dRs, dOff[e] + 4u);                                                     \
+				dreg[4 * e + 2] = buffer_load(dRs, dOff[e] + 8u);                                                     \
+				dreg[4 * e + 3] = buffer_load(dRs, dOff[e] + 12u);                                                    \
+			}                                                                                                         \
+			const __amdgpu_buffer_rsrc_t xRs = make_rsrc(xSel + m0_, p.srcBytes - 4u * (uint32_t)m0_);                \
+			xreg[0] = buffer_load(xRs, xOff), xreg[1] = buffer_load(xRs, xOff + 4u);                                  \
+			xreg[2] = buffer_load(xRs, xOff + 8u), xreg[3] = buffer_load(xRs, xOff + 12u);                            \
+		}                                                                                                             \
+	}
+
+#define CELL_STORE_STAGE(BUF)                                                                                         \
+	{                                                                                                                 \
+		_Pragma("unroll") for (int e = 0; e < DE; e++)                                                                \
+		{                                                                                                             \
+			float *dst = Ds[BUF] + dLds[e];                                                                           \
+			dst[0] = dreg[4 * e], dst[1] = dreg[4 * e + 1], dst[2] = dreg[4 * e + 2], dst[3] = dreg[4 * e + 3];       \
+		}                                                                                                             \
+		float *xd = Xs[BUF] + xLds;                                                                                   \
+		xd[0] = xreg[0], xd[1] = xreg[1], xd[2] = xreg[2], xd[3] = xreg[3];                                           \
+	}
+
+	v16f acc[3];
+#pragma unroll
+	for (int t = 0; t < 3; t++)
+#pragma unroll
+		for (int v = 0; v < 16; v++) acc[t][v] = 0.f;
+
+	// fragment of lane (l32, khalf) for cell q of image pair ip: row l32, word (2 * ip + khalf) * 16 + q
+	const int aOff = (ob * 32 + l32) * LD + khalf * kCells;
+	const int bOff = l32 * LD + khalf * kCells;
+
+	if (stBeg < stEnd) {
+		CELL_LOAD_STAGE(stBeg);
+		CELL_STORE_STAGE(0);
+	}
+	__syncthreads();
+	for (int st = stBeg; st < stEnd; st++) {
+		const int buf = (st - stBeg) & 1;
+		const bool more = st + 1 < stEnd;
+		if (more) CELL_LOAD_STAGE(st + 1);
+		const float *aBase = Ds[buf] + aOff;
+		const float *bBase = Xs[buf] + bOff;
+		if (tg == 0) cell_dw_steps<0>(aBase, bBase, acc);
+		else if (tg == 1) cell_dw_steps<1>(aBase, bBase, acc);
+		else cell_dw_steps<2>(aBase, bBase, acc);
+		if (more) CELL_STORE_STAGE(buf ^ 1); // the other buffer was released by the last barrier
+		__syncthreads();
+	}
+#undef CELL_LOAD_STAGE
+#undef CELL_STORE_STAGE
+
+	// ---- store: dW[o][c][tap], through LDS so that global memory sees whole rows of 32 * 9 consecutive words ----
+	float *C = out.C + (size_t)bz * out.splitStride;
+	float *stage = &Ds[0][0];
+	constexpr int ROW = kC3DwCin * 9, ROW_LD = ROW + 1;
+	static_assert(32 * ROW_LD <= 2 * (D_DUMMY + 4), "the output stage must fit the delta buffers");
+	const int validCols = ((p.cred - c0 < kC3DwCin) ? (p.cred - c0) : kC3DwCin) * 9;
+	const int tap0 = kCellTapGroups[tg][0], tap1 = kCellTapGroups[tg][1], tap2 = kCellTapGroups[tg][2];
+	for (int r = 0; r < 4; r++) {
+		if (r > 0) __syncthreads(); // the copy of the previous block is done
+		if (ob == r) {
+#pragma unroll
+			for (int v = 0; v < 16; v++) {
+				float *dst = stage + (8 * (v / 4) + 4 * khalf + (v % 4)) * ROW_LD + l32 * 9;
+				dst[tap0] = acc[0][v], dst[tap1] = acc[1][v], dst[tap2] = acc[2][v];
+			}
+		}
+		__syncthreads();
+		for (int i = tid; i < 32 * ROW; i += T) {
+			const int row = i / ROW, col = i - row * ROW;
+			const int o = o0 + r * 32 + row;
+			if ((o < p.I) & (col < validCols)) C[(size_t)o * out.ldc + c0 * 9 + col] = stage[row * ROW_LD + col];
+		}
+	}
+}
+
+} // namespace fitre

@@ -1,6 +1,8 @@
 // Convolution forward / weight gradient / input gradient and the general
 // column-major GEMM, all on the fp32-MFMA tile engine.
+#include <stdlib.h>
 #include "conv3x3.h"
+#include "conv_cell.h"
 #include "conv_common.h"
 #include "conv_quad.h"
 #include "conv_thin.h"
@@ -143,12 +145,21 @@ static BlockPlan c3_pos_plan(const fitre_conv_shape *s, bool dx, int cus = 0, in
 	double blockUs = (9.0 * kC3CB / 2.0) * (it / 32.0) * 64.0 / 2400.0; // MFMA steps x blocks per wave x 64 cycles
 	return plan_blocks(tiles, pairs * cred / kC3CB, blockUs, it == 64 ? 3 : 2, I, J, cus);
 }
+// 4 x 4 maps: the kernels of conv_cell.h, which leave out the taps that fall outside the image
+static bool cell_geometry(const fitre_conv_shape *s) { return c3_geometry(s) && s->inA == kCellMap && s->inB == kCellMap; }
+static bool cell_kernels_on() // EXPERIMENT toggle
+{
+	static int on = -1;
+	if (on < 0) on = getenv("FITRE_NO_CELL") == nullptr;
+	return on != 0;
+}
 static BlockPlan c3_dw_plan(const fitre_conv_shape *s, int cus = 0, int pairs = 1)
 {
 	if (cus <= 0) cus = lane_compute_units();
 	long J = (long)s->samples * s->inA * s->inB;
 	long tiles = ((s->inChannels + kC3DwCin - 1) / kC3DwCin) * ((s->outChannels + kC3Tile - 1) / kC3Tile);
 	double stageUs = (kC3Stage / 2.0) * 9.0 * 64.0 / 2400.0; // three waves per SIMD, three MFMAs per step each
+	if (cell_geometry(s) && cell_kernels_on()) stageUs *= 100.0 / 144.0;
 	return plan_blocks(tiles, pairs * ((J + kC3Stage - 1) / kC3Stage), stageUs, 1, s->outChannels, (long)s->inChannels * 9, cus);
 }
 static size_t c3_pos_workspace(const fitre_conv_shape *s, bool dx, int pairs = 1)
@@ -258,7 +269,11 @@ static int launch_c3_dw(const fitre_conv_shape *s, const float *x, const float *
 	{
 		LaunchScope scope(FITRE_KC_CONV_DW, pairs * conv_flops(s), 4);
 		const bool narrow = s->inB >= 2 && s->inB <= 16;
-		if (vecd && narrow)
+		const bool vecx = vecd && ((((uintptr_t)x) & 15) == 0) && (!x2 || (((uintptr_t)x2) & 15) == 0);
+		if (cell_geometry(s) && cell_kernels_on()) { // J is a multiple of 64 (eligibility): whole stages of four images
+			if (vecx) conv3x3_dw_cell_kernel<true><<<grid, kC3DwThreads, 0, stream()>>>(p, delta, deltaBytes, part);
+			else conv3x3_dw_cell_kernel<false><<<grid, kC3DwThreads, 0, stream()>>>(p, delta, deltaBytes, part);
+		} else if (vecd && narrow)
 			conv3x3_dw_kernel<true, 16><<<grid, kC3DwThreads, 0, stream()>>>(p, delta, deltaBytes, part);
 		else if (vecd)
 			conv3x3_dw_kernel<true, 32><<<grid, kC3DwThreads, 0, stream()>>>(p, delta, deltaBytes, part);

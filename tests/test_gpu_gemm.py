@@ -43,6 +43,11 @@ CONV_CASES = [
     (40, 68, 200, 2, 2, 3, 1, 1),    # the same with partial tiles in every dimension (272 x 800 x 40)
     (96, 128, 192, 2, 2, 3, 1, 1),   # split reduction of the input gradient
     (24, 64, 64, 2, 2, 3, 1, 1),     # too few images for the dense form: nine-tap kernels
+    # 4x4 maps: the kernels that leave out the taps outside the image (whole stages of four images)
+    (32, 32, 128, 4, 4, 3, 1, 1),    # one tile each way
+    (36, 40, 72, 4, 4, 3, 1, 1),     # partial channel tiles, nine stages
+    (64, 96, 160, 4, 4, 3, 1, 1),    # split reduction
+    (6, 16, 32, 4, 4, 3, 1, 1),      # six images: not whole stages, nine-tap kernels
     # weight-gradient stages whose window starts in a different column every stage (64 % B != 0)
     (64, 16, 32, 3, 5, 3, 1, 1),     # B = 5, 960 positions
     (16, 24, 40, 4, 6, 3, 1, 1),     # B = 6, partial channel tiles
