@@ -22,6 +22,13 @@ __host__ __device__ constexpr bool cell_tap_live(int cell, int tap)
 	return a >= 0 && a < kCellMap && b >= 0 && b < kCellMap;
 }
 __host__ __device__ constexpr int cell_tap_source(int cell, int tap) { return cell + (tap / 3 - 1) * kCellMap + (tap % 3 - 1); }
+// the k-th live tap of a cell, or -1
+__host__ __device__ constexpr int cell_nth_live_tap(int cell, int k)
+{
+	for (int tap = 0; tap < 9; tap++)
+		if (cell_tap_live(cell, tap) && k-- == 0) return tap;
+	return -1;
+}
 
 // ---------------------------------------------------------------------------------
 // weight gradient: dW[o][c][tap] = sum over images and live cells of delta[o][n][cell] * src[c][n][cell + tap shift]
@@ -211,6 +218,212 @@ conv3x3_dw_cell_kernel(const Conv3x3Params p, const float *delta, uint32_t delta
 			const int row = i / ROW, col = i - row * ROW;
 			const int o = o0 + r * 32 + row;
 			if ((o < p.I) & (col < validCols)) C[(size_t)o * out.ldc + c0 * 9 + col] = stage[row * ROW_LD + col];
+		}
+	}
+}
+
+// ---------------------------------------------------------------------------------
+// input gradient (and any position-contiguous product with the DX weight layout):
+//     out[i][n][cell] = sum over c and live taps of W[c][i][8 - tap] * src[c][n][cell + tap shift]
+// ---------------------------------------------------------------------------------
+// A workgroup owns 32 channels x 32 images x the 16 cells; an MFMA block is 32 channels x 32 images of ONE cell.
+// Each of the four waves owns a quadrant of the map -- a corner, two edge cells and a centre cell: 25 live taps,
+// the same for every quadrant -- i.e. four accumulator blocks, and per reduction pair reads the nine taps'
+// weight fragments and the nine source cells around its quadrant for 25 MFMAs.  The source block sits in LDS as
+// [channel][cell][image] (images contiguous: a fragment is 32 consecutive words), the weights as in
+// conv3x3_pos_kernel's input-gradient form: CB rows (reduction channel) of the tile's IT * 9 weights.  The result
+// leaves through LDS as whole 64-byte images ([row][image][cell]).  Requires samples % 32 == 0, cred % CB == 0.
+constexpr int kCellImages = 32; // images per workgroup tile
+constexpr int kCellIT = 32;     // channel rows per workgroup tile
+constexpr int kCellCB = 8;      // reduction channels per LDS block
+
+// the MFMAs of one reduction block for the wave that owns quadrant (QA, QB)
+template <int QA, int QB, int A_LD, int B_LD>
+__device__ __forceinline__ void cell_dx_block(const float *aBase, const float *bBase, v16f (&acc)[2][2])
+{
+	constexpr int CELL_LD = kCellImages + 1;
+#pragma unroll
+	for (int cp = 0; cp < kCellCB / 2; cp++) {
+		const float *aPair = aBase + cp * 2 * A_LD, *bPair = bBase + cp * 2 * B_LD;
+		float a[9], b[kCells];
+#pragma unroll
+		for (int tap = 0; tap < 9; tap++) a[tap] = aPair[8 - tap];
+#pragma unroll
+		for (int q = 0; q < kCells; q++) {
+			const int qa = q / kCellMap, qb = q % kCellMap;
+			const bool used = qa >= 2 * QA - 1 && qa <= 2 * QA + 2 && qb >= 2 * QB - 1 && qb <= 2 * QB + 2;
+			b[q] = used ? bPair[q * CELL_LD] : 0.f;
+		}
+		// the four cells take turns, so that consecutive MFMAs do not wait for each other's accumulator
+#pragma unroll
+		for (int k = 0; k < 9; k++)
+#pragma unroll
+			for (int da = 0; da < 2; da++)
+#pragma unroll
+				for (int db = 0; db < 2; db++) {
+					const int cell = (2 * QA + da) * kCellMap + 2 * QB + db;
+					const int tap = cell_nth_live_tap(cell, k);
+					if (tap < 0) continue;
+					acc[da][db] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[tap], b[cell_tap_source(cell, tap)], acc[da][db], 0, 0, 0);
+				}
+	}
+}
+
+template <bool VECW>
+__global__ void __launch_bounds__(kGemmThreads, 2)
+conv3x3_cell_dx_kernel(const Conv3x3Params p, const OutParams out)
+{
+	FITRE_RAISE_MATRIX_WAVE_PRIORITY();
+	constexpr int IT = kCellIT, CB = kCellCB;
+	constexpr int A_LD = IT * 9 + 4;                     // a multiple of four: 16-byte stores
+	constexpr int A_FLOATS = CB * A_LD, A_DUMMY = A_FLOATS;
+	constexpr int WQ = IT * 9 / 4, WGROUPS = CB * WQ;    // 16-byte groups of weights per block
+	constexpr int WE = (WGROUPS + kGemmThreads - 1) / kGemmThreads;
+	constexpr int CELL_LD = kCellImages + 1;             // images of one cell, odd stride
+	constexpr int B_LD = kCells * CELL_LD + 1;           // per reduction channel
+	constexpr int B_FLOATS = CB * B_LD;
+	constexpr int SGROUPS = CB * kCellImages * kCells / 4; // 16-byte groups of the source block
+	constexpr int SE = SGROUPS / kGemmThreads;
+	static_assert(SGROUPS % kGemmThreads == 0, "whole rounds of source groups");
+	constexpr int IMG_LD = kCells + 1, ROW_LD = kCellImages * IMG_LD; // the output stage: [row][image][cell]
+	constexpr int OUT_ROWS = 8;                                       // rows per round of the output stage
+	constexpr int LDS_FLOATS = (A_FLOATS + 4 + B_FLOATS) > OUT_ROWS * ROW_LD ? (A_FLOATS + 4 + B_FLOATS) : OUT_ROWS * ROW_LD;
+	__shared__ __attribute__((aligned(16))) float lds[LDS_FLOATS];
+	float *As = lds, *Bs = lds + A_FLOATS + 4;
+
+	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+	const int khalf = lane >> 5, l32 = lane & 31;
+	const int i0 = blockIdx.y * IT, n0 = blockIdx.x * kCellImages;
+	const int plane = p.J;
+	const int cbTotal = p.cred / CB;
+	const int cbBeg = blockIdx.z * p.perSplit;
+	const int cbEnd = (cbBeg + p.perSplit < cbTotal) ? cbBeg + p.perSplit : cbTotal;
+	const int rowLen = p.I * 9;
+
+	// ---- what this thread stages, the same for every channel block -------------------------
+	uint32_t wOff[WE];
+	int wLds[WE];
+#pragma unroll
+	for (int e = 0; e < WE; e++) {
+		const int idx = tid + kGemmThreads * e;
+		const int row = idx / WQ, qd = idx - row * WQ;
+		const bool has = idx < WGROUPS;
+		const int colG = i0 * 9 + 4 * qd;
+		const bool inside = has & (colG + 3 < rowLen);
+		const uint32_t off = 4u * (uint32_t)(row * rowLen + colG);
+		// columns past the tensor only feed accumulator rows that are never stored
+		wOff[e] = VECW ? (inside ? off : 0u) : (has ? off : kGroupOutOfRange);
+		wLds[e] = has ? row * A_LD + 4 * qd : A_DUMMY;
+	}
+	// source: group g = tid + 256 * e of the block's CB x (32 images x 16 cells) floats; a group is four cells of an image
+	uint32_t sOff[SE];
+	int sLds[SE];
+#pragma unroll
+	for (int e = 0; e < SE; e++) {
+		const int g = tid + kGemmThreads * e;
+		const int c = g / (kCellImages * kCells / 4), r = g - c * (kCellImages * kCells / 4);
+		const int img = r / (kCells / 4), q0 = 4 * (r - img * (kCells / 4));
+		sOff[e] = 4u * (uint32_t)(c * plane + (n0 + img) * kCells + q0);
+		sLds[e] = c * B_LD + q0 * CELL_LD + img;
+	}
+	float wreg[WE * 4];
+	float sreg[SE * 4];
+
+	v16f acc[2][2];
+#pragma unroll
+	for (int x = 0; x < 4; x++)
+#pragma unroll
+		for (int v = 0; v < 16; v++) acc[x >> 1][x & 1][v] = 0.f;
+
+	const float *aBase = As + khalf * A_LD + l32 * 9;
+	const float *bBase = Bs + khalf * B_LD + l32;
+
+#define CELL_LOAD_BLOCK(CBI)                                                                                          \
+	{                                                                                                                 \
+		const int c0_ = (CBI) * CB;                                                                                   \
+		const size_t wShift = (size_t)c0_ * rowLen; /* floats, uniform */                                             \
+		if constexpr (VECW) {                                                                                         \
+			const char *wBlk = reinterpret_cast<const char *>(p.w + wShift);                                          \
+			_Pragma("unroll") for (int e = 0; e < WE; e++)                                                            \
+			{                                                                                                         \
+				const float4 v4 = *reinterpret_cast<const float4 *>(wBlk + wOff[e]);                                  \
+				wreg[4 * e + 0] = v4.x, wreg[4 * e + 1] = v4.y, wreg[4 * e + 2] = v4.z, wreg[4 * e + 3] = v4.w;       \
+			}                                                                                                         \
+		} else {                                                                                                      \
+			const __amdgpu_buffer_rsrc_t wRs = make_rsrc(p.w + wShift, p.wBytes - (uint32_t)(4 * wShift));            \
+			_Pragma("unroll") for (int e = 0; e < WE; e++)                                                            \
+			{                                                                                                         \
+				wreg[4 * e + 0] = buffer_load(wRs, wOff[e]);                                                          \
+				wreg[4 * e + 1] = buffer_load(wRs, wOff[e] + 4u);                                                     \
+				wreg[4 * e + 2] = buffer_load(wRs, wOff[e] + 8u);                                                     \
+				wreg[4 * e + 3] = buffer_load(wRs, wOff[e] + 12u);                                                    \
+			}                                                                                                         \
+		}                                                                                                             \
+		const size_t sShift = (size_t)c0_ * plane;                                                                    \
+		const __amdgpu_buffer_rsrc_t sRs = make_rsrc(p.src + sShift, p.srcBytes - (uint32_t)(4 * sShift));           \
+		_Pragma("unroll") for (int e = 0; e < SE; e++)                                                                \
+		{                                                                                                             \
+			sreg[4 * e + 0] = buffer_load(sRs, sOff[e]);                                                              \
+			sreg[4 * e + 1] = buffer_load(sRs, sOff[e] + 4u);                                                         \
+			sreg[4 * e + 2] = buffer_load(sRs, sOff[e] + 8u);                                                         \
+			sreg[4 * e + 3] = buffer_load(sRs, sOff[e] + 12u);                                                        \
+		}                                                                                                             \
+	}
+
+	if (cbBeg < cbEnd) CELL_LOAD_BLOCK(cbBeg);
+	for (int cb = cbBeg; cb < cbEnd; cb++) {
+		__syncthreads();
+#pragma unroll
+		for (int e = 0; e < WE; e++)
+			*reinterpret_cast<float4 *>(As + wLds[e]) = make_float4(wreg[4 * e], wreg[4 * e + 1], wreg[4 * e + 2], wreg[4 * e + 3]);
+#pragma unroll
+		for (int e = 0; e < SE; e++) {
+			float *dst = Bs + sLds[e];
+			dst[0] = sreg[4 * e], dst[CELL_LD] = sreg[4 * e + 1], dst[2 * CELL_LD] = sreg[4 * e + 2], dst[3 * CELL_LD] = sreg[4 * e + 3];
+		}
+		__syncthreads();
+		if (cb + 1 < cbEnd) CELL_LOAD_BLOCK(cb + 1);
+		if (wave == 0) cell_dx_block<0, 0, A_LD, B_LD>(aBase, bBase, acc);
+		else if (wave == 1) cell_dx_block<0, 1, A_LD, B_LD>(aBase, bBase, acc);
+		else if (wave == 2) cell_dx_block<1, 0, A_LD, B_LD>(aBase, bBase, acc);
+		else cell_dx_block<1, 1, A_LD, B_LD>(aBase, bBase, acc);
+	}
+#undef CELL_LOAD_BLOCK
+
+	// ---- store: out[i][(n0 + image) * 16 + cell].  A row of the tile is 32 images x 16 cells = 2 KB of consecutive
+	// words, but a lane holds one cell of one image: eight rows at a time go through LDS and leave as 16-byte
+	// groups of whole rows. ------------------------------------------------------------------------------------
+	float *C = out.C + (size_t)blockIdx.z * out.splitStride;
+	const bool split = out.splitStride != 0;
+	const int QA = wave >> 1, QB = wave & 1;
+	float *stage = lds;
+#pragma unroll
+	for (int vg = 0; vg < 4; vg++) {
+		__syncthreads(); // the previous round has left (first round: the last block's fragments are read)
+#pragma unroll
+		for (int da = 0; da < 2; da++)
+#pragma unroll
+			for (int db = 0; db < 2; db++) {
+				const int cell = (2 * QA + da) * kCellMap + 2 * QB + db;
+#pragma unroll
+				for (int vv = 0; vv < 4; vv++) stage[(4 * khalf + vv) * ROW_LD + l32 * IMG_LD + cell] = acc[da][db][4 * vg + vv];
+			}
+		__syncthreads();
+#pragma unroll
+		for (int k = 0; k < OUT_ROWS * kCellImages * kCells / 4 / kGemmThreads; k++) {
+			const int f = tid + kGemmThreads * k; // 16-byte group of the round
+			const int row = f / (kCellImages * kCells / 4), g = f - row * (kCellImages * kCells / 4);
+			const int img = g / (kCells / 4), cell0 = 4 * (g - img * (kCells / 4));
+			const int i = i0 + 8 * vg + row;
+			const float *src = stage + row * ROW_LD + img * IMG_LD + cell0;
+			float4 val = make_float4(src[0], src[1], src[2], src[3]);
+			if (i < p.I) {
+				if (!split && out.biasI) {
+					const float bi = out.biasI[i];
+					val.x += bi, val.y += bi, val.z += bi, val.w += bi;
+				}
+				*reinterpret_cast<float4 *>(C + (size_t)i * out.ldc + (size_t)(n0 + img) * kCells + cell0) = val;
+			}
 		}
 	}
 }

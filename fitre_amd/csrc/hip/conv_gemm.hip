@@ -135,16 +135,6 @@ static bool c3_dw_eligible(const fitre_conv_shape *s)
 
 // cus: compute units of the lane the kernel is launched on (0 = the selected lane)
 // pairs = 2: a sum of two products of this shape in one launch (twice the reduction)
-static BlockPlan c3_pos_plan(const fitre_conv_shape *s, bool dx, int cus = 0, int pairs = 1)
-{
-	if (cus <= 0) cus = lane_compute_units();
-	long I = dx ? s->inChannels : s->outChannels, J = (long)s->samples * s->inA * s->inB;
-	long cred = dx ? s->outChannels : s->inChannels;
-	long it = I <= 64 ? 64 : kC3Tile;
-	long tiles = ((I + it - 1) / it) * ((J + kC3Tile - 1) / kC3Tile);
-	double blockUs = (9.0 * kC3CB / 2.0) * (it / 32.0) * 64.0 / 2400.0; // MFMA steps x blocks per wave x 64 cycles
-	return plan_blocks(tiles, pairs * cred / kC3CB, blockUs, it == 64 ? 3 : 2, I, J, cus);
-}
 // 4 x 4 maps: the kernels of conv_cell.h, which leave out the taps that fall outside the image
 static bool cell_geometry(const fitre_conv_shape *s) { return c3_geometry(s) && s->inA == kCellMap && s->inB == kCellMap; }
 static bool cell_kernels_on() // EXPERIMENT toggle
@@ -152,6 +142,26 @@ static bool cell_kernels_on() // EXPERIMENT toggle
 	static int on = -1;
 	if (on < 0) on = getenv("FITRE_NO_CELL") == nullptr;
 	return on != 0;
+}
+// the input gradient on 4 x 4 maps in the cell form: whole tiles of 32 images, one product
+static bool cell_dx_eligible(const fitre_conv_shape *s, int pairs)
+{
+	return cell_geometry(s) && cell_kernels_on() && pairs == 1 && s->samples % kCellImages == 0 && s->outChannels % kCellCB == 0;
+}
+static BlockPlan c3_pos_plan(const fitre_conv_shape *s, bool dx, int cus = 0, int pairs = 1)
+{
+	if (cus <= 0) cus = lane_compute_units();
+	long I = dx ? s->inChannels : s->outChannels, J = (long)s->samples * s->inA * s->inB;
+	long cred = dx ? s->outChannels : s->inChannels;
+	if (dx && cell_dx_eligible(s, pairs)) {
+		const long tiles = ((I + kCellIT - 1) / kCellIT) * (s->samples / kCellImages);
+		const double blockUs = (kCellCB / 2.0) * 25.0 * 64.0 / 2400.0; // reduction pairs x MFMAs per wave and pair x 64 cycles
+		return plan_blocks(tiles, cred / kCellCB, blockUs, 2, I, J, cus);
+	}
+	long it = I <= 64 ? 64 : kC3Tile;
+	long tiles = ((I + it - 1) / it) * ((J + kC3Tile - 1) / kC3Tile);
+	double blockUs = (9.0 * kC3CB / 2.0) * (it / 32.0) * 64.0 / 2400.0; // MFMA steps x blocks per wave x 64 cycles
+	return plan_blocks(tiles, pairs * cred / kC3CB, blockUs, it == 64 ? 3 : 2, I, J, cus);
 }
 static BlockPlan c3_dw_plan(const fitre_conv_shape *s, int cus = 0, int pairs = 1)
 {
@@ -206,6 +216,19 @@ static int launch_c3_pos(const fitre_conv_shape *s, const float *src, const floa
 		part.splitStride = (long)I * J;
 	}
 	const bool vecw = ((((uintptr_t)w) & 15) == 0) && (!w2 || (((uintptr_t)w2) & 15) == 0) && (DX ? (I % 4 == 0) : true);
+	// (the cell kernel stores 16-byte groups; a plan made for it also fits the nine-tap kernel: same block size)
+	if (DX && cell_dx_eligible(s, pairs) && (((uintptr_t)part.C) & 15) == 0) {
+		dim3 grid((unsigned)(s->samples / kCellImages), (unsigned)((I + kCellIT - 1) / kCellIT), (unsigned)plan.splits);
+		if (grid.y > 65535 || grid.z > 65535) return fail(FITRE_E_UNSUPPORTED, "conv3x3 grid too large");
+		{
+			LaunchScope scope(FITRE_KC_CONV_DX, conv_flops(s), 4);
+			if (vecw) conv3x3_cell_dx_kernel<true><<<grid, kGemmThreads, 0, stream()>>>(p, part);
+			else conv3x3_cell_dx_kernel<false><<<grid, kGemmThreads, 0, stream()>>>(p, part);
+		}
+		if (leftSplits) *leftSplits = plan.splits;
+		if (plan.splits > 1 && !leftSplits) launch_splitk_reduce((const float *)ws, plan.splits, I, J, out);
+		return check_launch("conv3x3_cell_dx_kernel");
+	}
 	const int it = I <= 64 ? 64 : kC3Tile;
 	dim3 grid((J + kC3Tile - 1) / kC3Tile, (I + it - 1) / it, plan.splits);
 	if (grid.y > 65535 || grid.z > 65535) return fail(FITRE_E_UNSUPPORTED, "conv3x3 grid too large");
