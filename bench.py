@@ -44,7 +44,7 @@ KC = dict(conv_dw=0, conv_dx=1, conv_fwd=2, fc_gemm=3, splitk_reduce=4, bn_bwd=5
           act_bwd=9, act_fwd=10, bias_grad=11, softmax=12, permute=13, blas1=14, pool_act_bwd=15, kfac_factor=16,
           spd_inverse=17)
 MFMA_CLASSES = ("conv_dw", "conv_dx", "conv_fwd", "fc_gemm", "kfac_factor", "spd_inverse")
-TILES = {0: "", 1: "64x64", 2: "64x128", 3: "128x64", 4: "128x128", 5: "96x128"}
+TILES = {0: "", 1: "64x64", 2: "64x128", 3: "128x64", 4: "128x128", 5: "96x128", 6: "dense2x2", 7: "cell4x4", 8: "cell8x8"}
 
 
 def measured_traffic(kernel):
@@ -91,10 +91,17 @@ def kernel_table(rows, steps, launches=None):
                                     frac=round(rate / peak, 4))
         if r["kernel"] in big:
             kernels[r["kernel"]]["largest"] = big[r["kernel"]]
-        if r["kernel"] in ("conv_dw", "conv_dx"):
-            # the untiled variants of these classes are the dense per-image form of 3x3 convolutions on 2x2 maps
+        if r["kernel"].endswith("/dense2x2"):
             kernels[r["kernel"]]["note"] = ("3x3 windows on 2x2 maps as dense products: the work counted is the nine-tap "
                                             "2*M*K*Cout, of which the kernel executes 16/36 (the rest multiplies padding)")
+        if r["kernel"].endswith("/cell8x8"):
+            kernels[r["kernel"]]["note"] = ("weight gradient of 3x3 windows on 8x8 maps, a reduction pair being one cell of two "
+                                            "images: the work counted is the nine-tap 2*M*K*Cout, of which the kernel executes "
+                                            "484/576 (the rest multiplies padding)")
+        if r["kernel"].endswith("/cell4x4"):
+            kernels[r["kernel"]]["note"] = ("3x3 windows on 4x4 maps, an MFMA block being one cell of 32 images: the work "
+                                            "counted is the nine-tap 2*M*K*Cout, of which the kernel executes 100/144 (the "
+                                            "rest multiplies padding)")
     return kernels
 
 
@@ -134,7 +141,7 @@ def largest_launches(launches, keep=4):
 def read_profile(L):
     rows = []
     for name, cls in KC.items():
-        for tile in range(6):
+        for tile in range(len(TILES)):
             n, ms, work = C.c_long(), C.c_double(), C.c_double()
             L.check(L.hip.fitre_hip_profile_read_tile(cls, tile, C.byref(n), C.byref(ms), C.byref(work)))
             if n.value:

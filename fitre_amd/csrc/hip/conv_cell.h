@@ -223,6 +223,216 @@ conv3x3_dw_cell_kernel(const Conv3x3Params p, const float *delta, uint32_t delta
 }
 
 // ---------------------------------------------------------------------------------
+// weight gradient on 8 x 8 maps: the same idea with a stage of 64 positions = the upper or the lower half (four
+// rows) of TWO neighbouring images.  92 of the 576 (cell, tap) pairs of an image are dead (16 %); a stage has 242
+// live ones of 288.  The source stage holds the half's four rows and the row above / below it that lies inside
+// the image (five rows of eight cells per image), so no tap that is issued leaves it.  Tap groups {centre, two
+// opposite corners}, {down, up, up-right}, {left, right, down-left}: 81 / 77 / 84 live pairs on an upper half,
+// 81 / 84 / 77 on a lower one, against 96 steps of the nine-tap kernel.
+// ---------------------------------------------------------------------------------
+constexpr int kCell8Map = 8;
+constexpr int kCell8Half = 32;                 // cells of half a map
+constexpr int kCell8SrcCells = 5 * kCell8Map;  // source cells per image and half
+__device__ constexpr int kCell8TapGroups[3][3] = { { 4, 0, 8 }, { 7, 1, 2 }, { 3, 5, 6 } };
+
+// LOWER: the stage is the lower half (rows 4..7; the source rows are 3..7), else the upper (rows 0..3; source 0..4)
+template <int TG, bool LOWER>
+__device__ __forceinline__ void cell8_dw_steps(const float *aBase, const float *bBase, v16f (&acc)[3])
+{
+#pragma unroll
+	for (int cell = 0; cell < kCell8Half; cell++) {
+		const int a = cell / kCell8Map + (LOWER ? 4 : 0), b = cell % kCell8Map; // row and column in the image
+		bool live[3] = { false, false, false };
+		int src[3] = { 0, 0, 0 };
+#pragma unroll
+		for (int j = 0; j < 3; j++) {
+			const int tap = kCell8TapGroups[TG][j];
+			const int sa = a + tap / 3 - 1, sb = b + tap % 3 - 1;
+			live[j] = sa >= 0 && sa < kCell8Map && sb >= 0 && sb < kCell8Map;
+			src[j] = (sa - (LOWER ? 3 : 0)) * kCell8Map + sb; // word inside the image's five source rows
+		}
+		if (!(live[0] || live[1] || live[2])) continue;
+		const float fa = aBase[cell];
+#pragma unroll
+		for (int j = 0; j < 3; j++)
+			if (live[j]) acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa, bBase[src[j]], acc[j], 0, 0, 0);
+	}
+}
+
+template <bool VEC>
+__global__ void __launch_bounds__(kC3DwThreads)
+conv3x3_dw_cell8_kernel(const Conv3x3Params p, const float *delta, uint32_t deltaBytes, const OutParams out)
+{
+	FITRE_RAISE_MATRIX_WAVE_PRIORITY();
+	constexpr int T = kC3DwThreads;
+	constexpr int D_LD = kC3Stage + 1;              // delta: [row][image of the pair][32 cells], odd stride
+	constexpr int X_LD = 2 * kCell8SrcCells + 1;    // source: [row][image of the pair][40 cells], odd stride
+	constexpr int D_DUMMY = kC3Tile * D_LD, X_DUMMY = kC3DwCin * X_LD;
+	constexpr int DGROUPS = kC3Tile * kC3Stage / 4; // 16-byte groups of delta per stage
+	constexpr int DE = (DGROUPS + T - 1) / T;
+	constexpr int XGROUPS = kC3DwCin * 2 * kCell8SrcCells / 4; // 640: one per thread of the first ten waves
+	static_assert(XGROUPS <= T, "one source group per thread");
+	constexpr int IMG = kCell8Map * kCell8Map;
+	__shared__ float Ds[2][D_DUMMY + 4];
+	__shared__ float Xs[2][X_DUMMY + 4];
+
+	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+	const int khalf = lane >> 5, l32 = lane & 31;
+	const int ob = wave & 3, tg = wave >> 2; // output-channel block, tap group
+	// workgroups renumbered so that an XCD (its own L2) holds consecutive indices, as in conv3x3_dw_kernel
+	int bx, by, bz;
+	{
+		const unsigned groups = gridDim.x * gridDim.y * gridDim.z;
+		const unsigned lin = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+		const unsigned xcd = lin & 7u, each = groups >> 3, extra = groups & 7u;
+		const unsigned logical = xcd * each + (xcd < extra ? xcd : extra) + (lin >> 3);
+		const unsigned tiles = gridDim.x * gridDim.y;
+		bz = (int)(logical / tiles);
+		const unsigned rem = logical - (unsigned)bz * tiles;
+		by = (int)(rem / gridDim.x);
+		bx = (int)(rem - (unsigned)by * gridDim.x);
+	}
+	const int c0 = bx * kC3DwCin, o0 = by * kC3Tile;
+	const int plane = p.J;
+	const int stagesHalf = p.J / kC3Stage; // stage st: image pair st / 2, half st % 2
+	const int stagesTotal = p.src2 ? 2 * stagesHalf : stagesHalf;
+	const int stBeg = bz * p.perSplit;
+	const int stEnd = (stBeg + p.perSplit < stagesTotal) ? stBeg + p.perSplit : stagesTotal;
+
+	// ---- what this thread stages: offsets relative to the first cell of the stage's image pair -----------------
+	uint32_t dOff[DE]; // without the half's 32 cells
+	int dLds[DE];
+#pragma unroll
+	for (int e = 0; e < DE; e++) {
+		const int idx = tid + T * e;
+		const int row = idx / (kC3Stage / 4), g = idx - row * (kC3Stage / 4); // g: 0..15 = image of the pair x 8 groups
+		const int img = g / 8, cg = 4 * (g - img * 8);
+		const bool has = idx < DGROUPS;
+		const bool inside = has & ((o0 + row) < p.I);
+		const uint32_t off = 4u * (uint32_t)((o0 + row) * plane + img * IMG + cg);
+		// rows past the tensor feed accumulator rows that are never stored
+		dOff[e] = VEC ? (inside ? off : 4u * (uint32_t)(img * IMG + cg)) : (inside ? off : kGroupOutOfRange);
+		dLds[e] = has ? row * D_LD + img * kCell8Half + cg : D_DUMMY;
+	}
+	// source: group tid of [32 rows][2 images][10 groups of four cells = five image rows]
+	const int xRow = tid / (2 * kCell8SrcCells / 4), xg = tid - xRow * (2 * kCell8SrcCells / 4);
+	const int xImg = xg / (kCell8SrcCells / 4), xCg = 4 * (xg - xImg * (kCell8SrcCells / 4));
+	const bool xHas = tid < XGROUPS;
+	const bool xInside = xHas & ((c0 + xRow) < p.cred);
+	const uint32_t xOffRaw = 4u * (uint32_t)((c0 + xRow) * plane + xImg * IMG + xCg); // plus the first source row of the half
+	const uint32_t xOff = VEC ? (xInside ? xOffRaw : 4u * (uint32_t)(xImg * IMG + xCg)) : (xInside ? xOffRaw : kGroupOutOfRange);
+	const int xLds = xHas ? xRow * X_LD + xImg * kCell8SrcCells + xCg : X_DUMMY;
+	float dreg[DE * 4];
+	float xreg[4];
+
+#define CELL8_LOAD_STAGE(ST)                                                                                          \
+	{                                                                                                                 \
+		const bool second_ = (ST) >= stagesHalf; /* uniform */                                                        \
+		const int s_ = (ST) - (second_ ? stagesHalf : 0);                                                             \
+		const int pair0_ = (s_ >> 1) * 2 * IMG;            /* first cell of the image pair */                         \
+		const int dBase_ = pair0_ + (s_ & 1) * kCell8Half;  /* the half's first cell */                               \
+		const int xBase_ = pair0_ + (s_ & 1) * 3 * kCell8Map; /* its first source row: 0 or 3 */                      \
+		const float *dSel = second_ ? p.w2 : delta;                                                                   \
+		const float *xSel = second_ ? p.src2 : p.src;                                                                 \
+		if constexpr (VEC) {                                                                                          \
+			const char *dBlk = reinterpret_cast<const char *>(dSel + dBase_);                                         \
+			_Pragma("unroll") for (int e = 0; e < DE; e++)                                                            \
+			{                                                                                                         \
+				const float4 v4 = *reinterpret_cast<const float4 *>(dBlk + dOff[e]);                                  \
+				dreg[4 * e + 0] = v4.x, dreg[4 * e + 1] = v4.y, dreg[4 * e + 2] = v4.z, dreg[4 * e + 3] = v4.w;       \
+			}                                                                                                         \
+			const float4 x4 = *reinterpret_cast<const float4 *>(reinterpret_cast<const char *>(xSel + xBase_) + xOff); \
+			xreg[0] = xInside ? x4.x : 0.f, xreg[1] = xInside ? x4.y : 0.f;                                           \
+			xreg[2] = xInside ? x4.z : 0.f, xreg[3] = xInside ? x4.w : 0.f;                                           \
+		} else {                                                                                                      \
+			const __amdgpu_buffer_rsrc_t dRs = make_rsrc(dSel + dBase_, deltaBytes - 4u * (uint32_t)dBase_);          \
+			_Pragma("unroll") for (int e = 0; e < DE; e++)                                                            \
+			{                                                                                                         \
+				dreg[4 * e + 0] = buffer_load(dRs, dOff[e]);                                                          \
+				dreg[4 * e + 1] = buffer_load(dRs, dOff[e] + 4u);                                                     \
+				dreg[4 * e + 2] = buffer_load(dRs, dOff[e] + 8u);                                                     \
+				dreg[4 * e + 3] = buffer_load(dRs, dOff[e] + 12u);                                                    \
+			}                                                                                                         \
+			const __amdgpu_buffer_rsrc_t xRs = make_rsrc(xSel + xBase_, p.srcBytes - 4u * (uint32_t)xBase_);          \
+			xreg[0] = buffer_load(xRs, xOff), xreg[1] = buffer_load(xRs, xOff + 4u);                                  \
+			xreg[2] = buffer_load(xRs, xOff + 8u), xreg[3] = buffer_load(xRs, xOff + 12u);                            \
+		}                                                                                                             \
+	}
+
+#define CELL8_STORE_STAGE(BUF)                                                                                        \
+	{                                                                                                                 \
+		_Pragma("unroll") for (int e = 0; e < DE; e++)                                                                \
+		{                                                                                                             \
+			float *dst = Ds[BUF] + dLds[e];                                                                           \
+			dst[0] = dreg[4 * e], dst[1] = dreg[4 * e + 1], dst[2] = dreg[4 * e + 2], dst[3] = dreg[4 * e + 3];       \
+		}                                                                                                             \
+		float *xd = Xs[BUF] + xLds;                                                                                   \
+		xd[0] = xreg[0], xd[1] = xreg[1], xd[2] = xreg[2], xd[3] = xreg[3];                                           \
+	}
+
+	v16f acc[3];
+#pragma unroll
+	for (int t = 0; t < 3; t++)
+#pragma unroll
+		for (int v = 0; v < 16; v++) acc[t][v] = 0.f;
+
+	// fragment of lane (l32, khalf): row l32, image khalf of the pair
+	const int aOff = (ob * 32 + l32) * D_LD + khalf * kCell8Half;
+	const int bOff = l32 * X_LD + khalf * kCell8SrcCells;
+
+	if (stBeg < stEnd) {
+		CELL8_LOAD_STAGE(stBeg);
+		CELL8_STORE_STAGE(0);
+	}
+	__syncthreads();
+	for (int st = stBeg; st < stEnd; st++) {
+		const int buf = (st - stBeg) & 1;
+		const bool more = st + 1 < stEnd;
+		if (more) CELL8_LOAD_STAGE(st + 1);
+		const float *aBase = Ds[buf] + aOff;
+		const float *bBase = Xs[buf] + bOff;
+		const bool lower = (st & 1) != 0; // stagesHalf is even, so this holds for the second pair as well
+		if (!lower) {
+			if (tg == 0) cell8_dw_steps<0, false>(aBase, bBase, acc);
+			else if (tg == 1) cell8_dw_steps<1, false>(aBase, bBase, acc);
+			else cell8_dw_steps<2, false>(aBase, bBase, acc);
+		} else {
+			if (tg == 0) cell8_dw_steps<0, true>(aBase, bBase, acc);
+			else if (tg == 1) cell8_dw_steps<1, true>(aBase, bBase, acc);
+			else cell8_dw_steps<2, true>(aBase, bBase, acc);
+		}
+		if (more) CELL8_STORE_STAGE(buf ^ 1); // the other buffer was released by the last barrier
+		__syncthreads();
+	}
+#undef CELL8_LOAD_STAGE
+#undef CELL8_STORE_STAGE
+
+	// ---- store: dW[o][c][tap], through LDS so that global memory sees whole rows of 32 * 9 consecutive words ----
+	float *C = out.C + (size_t)bz * out.splitStride;
+	float *stage = &Ds[0][0];
+	constexpr int ROW = kC3DwCin * 9, ROW_LD = ROW + 1;
+	static_assert(32 * ROW_LD <= 2 * (D_DUMMY + 4), "the output stage must fit the delta buffers");
+	const int validCols = ((p.cred - c0 < kC3DwCin) ? (p.cred - c0) : kC3DwCin) * 9;
+	const int tap0 = kCell8TapGroups[tg][0], tap1 = kCell8TapGroups[tg][1], tap2 = kCell8TapGroups[tg][2];
+	for (int r = 0; r < 4; r++) {
+		if (r > 0) __syncthreads(); // the copy of the previous block is done
+		if (ob == r) {
+#pragma unroll
+			for (int v = 0; v < 16; v++) {
+				float *dst = stage + (8 * (v / 4) + 4 * khalf + (v % 4)) * ROW_LD + l32 * 9;
+				dst[tap0] = acc[0][v], dst[tap1] = acc[1][v], dst[tap2] = acc[2][v];
+			}
+		}
+		__syncthreads();
+		for (int i = tid; i < 32 * ROW; i += T) {
+			const int row = i / ROW, col = i - row * ROW;
+			const int o = o0 + r * 32 + row;
+			if ((o < p.I) & (col < validCols)) C[(size_t)o * out.ldc + c0 * 9 + col] = stage[row * ROW_LD + col];
+		}
+	}
+}
+
+// ---------------------------------------------------------------------------------
 // input gradient (and any position-contiguous product with the DX weight layout):
 //     out[i][n][cell] = sum over c and live taps of W[c][i][8 - tap] * src[c][n][cell + tap shift]
 // ---------------------------------------------------------------------------------
@@ -295,7 +505,8 @@ conv3x3_cell_dx_kernel(const Conv3x3Params p, const OutParams out)
 	const int khalf = lane >> 5, l32 = lane & 31;
 	const int i0 = blockIdx.y * IT, n0 = blockIdx.x * kCellImages;
 	const int plane = p.J;
-	const int cbTotal = p.cred / CB;
+	const int cbHalf = p.cred / CB;                    // channel blocks of one (src, w) pair
+	const int cbTotal = p.src2 ? 2 * cbHalf : cbHalf; // a second pair continues the reduction
 	const int cbBeg = blockIdx.z * p.perSplit;
 	const int cbEnd = (cbBeg + p.perSplit < cbTotal) ? cbBeg + p.perSplit : cbTotal;
 	const int rowLen = p.I * 9;
@@ -340,17 +551,19 @@ conv3x3_cell_dx_kernel(const Conv3x3Params p, const OutParams out)
 
 #define CELL_LOAD_BLOCK(CBI)                                                                                          \
 	{                                                                                                                 \
-		const int c0_ = (CBI) * CB;                                                                                   \
+		const bool second_ = (CBI) >= cbHalf; /* uniform: the block belongs to the second pair */                    \
+		const int c0_ = ((CBI) - (second_ ? cbHalf : 0)) * CB;                                                        \
+		const float *wSel = second_ ? p.w2 : p.w, *sSel = second_ ? p.src2 : p.src;                                   \
 		const size_t wShift = (size_t)c0_ * rowLen; /* floats, uniform */                                             \
 		if constexpr (VECW) {                                                                                         \
-			const char *wBlk = reinterpret_cast<const char *>(p.w + wShift);                                          \
+			const char *wBlk = reinterpret_cast<const char *>(wSel + wShift);                                         \
 			_Pragma("unroll") for (int e = 0; e < WE; e++)                                                            \
 			{                                                                                                         \
 				const float4 v4 = *reinterpret_cast<const float4 *>(wBlk + wOff[e]);                                  \
 				wreg[4 * e + 0] = v4.x, wreg[4 * e + 1] = v4.y, wreg[4 * e + 2] = v4.z, wreg[4 * e + 3] = v4.w;       \
 			}                                                                                                         \
 		} else {                                                                                                      \
-			const __amdgpu_buffer_rsrc_t wRs = make_rsrc(p.w + wShift, p.wBytes - (uint32_t)(4 * wShift));            \
+			const __amdgpu_buffer_rsrc_t wRs = make_rsrc(wSel + wShift, p.wBytes - (uint32_t)(4 * wShift));            \
 			_Pragma("unroll") for (int e = 0; e < WE; e++)                                                            \
 			{                                                                                                         \
 				wreg[4 * e + 0] = buffer_load(wRs, wOff[e]);                                                          \
@@ -360,7 +573,7 @@ conv3x3_cell_dx_kernel(const Conv3x3Params p, const OutParams out)
 			}                                                                                                         \
 		}                                                                                                             \
 		const size_t sShift = (size_t)c0_ * plane;                                                                    \
-		const __amdgpu_buffer_rsrc_t sRs = make_rsrc(p.src + sShift, p.srcBytes - (uint32_t)(4 * sShift));           \
+		const __amdgpu_buffer_rsrc_t sRs = make_rsrc(sSel + sShift, p.srcBytes - (uint32_t)(4 * sShift));           \
 		_Pragma("unroll") for (int e = 0; e < SE; e++)                                                                \
 		{                                                                                                             \
 			sreg[4 * e + 0] = buffer_load(sRs, sOff[e]);                                                              \

@@ -137,6 +137,8 @@ static bool c3_dw_eligible(const fitre_conv_shape *s)
 // pairs = 2: a sum of two products of this shape in one launch (twice the reduction)
 // 4 x 4 maps: the kernels of conv_cell.h, which leave out the taps that fall outside the image
 static bool cell_geometry(const fitre_conv_shape *s) { return c3_geometry(s) && s->inA == kCellMap && s->inB == kCellMap; }
+// 8 x 8 maps: the weight gradient's stage is half a map of two images
+static bool cell8_geometry(const fitre_conv_shape *s) { return c3_geometry(s) && s->inA == kCell8Map && s->inB == kCell8Map && s->samples % 2 == 0; }
 static bool cell_kernels_on() // EXPERIMENT toggle
 {
 	static int on = -1;
@@ -146,7 +148,8 @@ static bool cell_kernels_on() // EXPERIMENT toggle
 // the input gradient on 4 x 4 maps in the cell form: whole tiles of 32 images, one product
 static bool cell_dx_eligible(const fitre_conv_shape *s, int pairs)
 {
-	return cell_geometry(s) && cell_kernels_on() && pairs == 1 && s->samples % kCellImages == 0 && s->outChannels % kCellCB == 0;
+	(void)pairs; // a second (delta, weights) pair continues the reduction
+	return cell_geometry(s) && cell_kernels_on() && s->samples % kCellImages == 0 && s->outChannels % kCellCB == 0;
 }
 static BlockPlan c3_pos_plan(const fitre_conv_shape *s, bool dx, int cus = 0, int pairs = 1)
 {
@@ -156,7 +159,7 @@ static BlockPlan c3_pos_plan(const fitre_conv_shape *s, bool dx, int cus = 0, in
 	if (dx && cell_dx_eligible(s, pairs)) {
 		const long tiles = ((I + kCellIT - 1) / kCellIT) * (s->samples / kCellImages);
 		const double blockUs = (kCellCB / 2.0) * 25.0 * 64.0 / 2400.0; // reduction pairs x MFMAs per wave and pair x 64 cycles
-		return plan_blocks(tiles, cred / kCellCB, blockUs, 2, I, J, cus);
+		return plan_blocks(tiles, pairs * cred / kCellCB, blockUs, 2, I, J, cus);
 	}
 	long it = I <= 64 ? 64 : kC3Tile;
 	long tiles = ((I + it - 1) / it) * ((J + kC3Tile - 1) / kC3Tile);
@@ -170,6 +173,7 @@ static BlockPlan c3_dw_plan(const fitre_conv_shape *s, int cus = 0, int pairs = 
 	long tiles = ((s->inChannels + kC3DwCin - 1) / kC3DwCin) * ((s->outChannels + kC3Tile - 1) / kC3Tile);
 	double stageUs = (kC3Stage / 2.0) * 9.0 * 64.0 / 2400.0; // three waves per SIMD, three MFMAs per step each
 	if (cell_geometry(s) && cell_kernels_on()) stageUs *= 100.0 / 144.0;
+	if (cell8_geometry(s) && cell_kernels_on()) stageUs *= 84.0 / 96.0;
 	return plan_blocks(tiles, pairs * ((J + kC3Stage - 1) / kC3Stage), stageUs, 1, s->outChannels, (long)s->inChannels * 9, cus);
 }
 static size_t c3_pos_workspace(const fitre_conv_shape *s, bool dx, int pairs = 1)
@@ -221,7 +225,7 @@ static int launch_c3_pos(const fitre_conv_shape *s, const float *src, const floa
 		dim3 grid((unsigned)(s->samples / kCellImages), (unsigned)((I + kCellIT - 1) / kCellIT), (unsigned)plan.splits);
 		if (grid.y > 65535 || grid.z > 65535) return fail(FITRE_E_UNSUPPORTED, "conv3x3 grid too large");
 		{
-			LaunchScope scope(FITRE_KC_CONV_DX, conv_flops(s), 4);
+			LaunchScope scope(FITRE_KC_CONV_DX, pairs * conv_flops(s), 7);
 			if (vecw) conv3x3_cell_dx_kernel<true><<<grid, kGemmThreads, 0, stream()>>>(p, part);
 			else conv3x3_cell_dx_kernel<false><<<grid, kGemmThreads, 0, stream()>>>(p, part);
 		}
@@ -290,10 +294,14 @@ static int launch_c3_dw(const fitre_conv_shape *s, const float *x, const float *
 	dim3 grid((cin + kC3DwCin - 1) / kC3DwCin, (I + kC3Tile - 1) / kC3Tile, plan.splits);
 	if (grid.y > 65535 || grid.z > 65535) return fail(FITRE_E_UNSUPPORTED, "conv3x3 grid too large");
 	{
-		LaunchScope scope(FITRE_KC_CONV_DW, pairs * conv_flops(s), 4);
+		LaunchScope scope(FITRE_KC_CONV_DW, pairs * conv_flops(s),
+		                  !cell_kernels_on() ? 4 : (cell_geometry(s) ? 7 : (cell8_geometry(s) ? 8 : 4)));
 		const bool narrow = s->inB >= 2 && s->inB <= 16;
 		const bool vecx = vecd && ((((uintptr_t)x) & 15) == 0) && (!x2 || (((uintptr_t)x2) & 15) == 0);
-		if (cell_geometry(s) && cell_kernels_on()) { // J is a multiple of 64 (eligibility): whole stages of four images
+		if (cell8_geometry(s) && cell_kernels_on()) { // whole pairs of images (eligibility)
+			if (vecx) conv3x3_dw_cell8_kernel<true><<<grid, kC3DwThreads, 0, stream()>>>(p, delta, deltaBytes, part);
+			else conv3x3_dw_cell8_kernel<false><<<grid, kC3DwThreads, 0, stream()>>>(p, delta, deltaBytes, part);
+		} else if (cell_geometry(s) && cell_kernels_on()) { // J is a multiple of 64 (eligibility): whole stages of four images
 			if (vecx) conv3x3_dw_cell_kernel<true><<<grid, kC3DwThreads, 0, stream()>>>(p, delta, deltaBytes, part);
 			else conv3x3_dw_cell_kernel<false><<<grid, kC3DwThreads, 0, stream()>>>(p, delta, deltaBytes, part);
 		} else if (vecd && narrow)

@@ -227,7 +227,7 @@ static int quad_launch_tile(const PA &pa, const PB &pb, const OutParams &out, in
 		if (!out.quadLd) part.ldc = J;
 	}
 	{
-		LaunchScope scope(kernelClass, flops, 0);
+		LaunchScope scope(kernelClass, flops, 6);
 		mfma_gemm_kernel<Cfg, OpA<BM, BK>, OpB<BN, BK>><<<grid, kGemmThreads, 0, stream()>>>(pa, pb, part, I, J, R, plan.kChunk);
 	}
 	if (leftSplits) *leftSplits = plan.splits;

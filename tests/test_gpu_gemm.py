@@ -48,6 +48,10 @@ CONV_CASES = [
     (36, 40, 72, 4, 4, 3, 1, 1),     # partial channel tiles, nine stages
     (64, 96, 160, 4, 4, 3, 1, 1),    # split reduction
     (6, 16, 32, 4, 4, 3, 1, 1),      # six images: not whole stages, nine-tap kernels
+    # 8x8 maps: the weight gradient's stages are half maps of two images
+    (6, 32, 128, 8, 8, 3, 1, 1),     # one tile, six stages
+    (18, 48, 160, 8, 8, 3, 1, 1),    # partial tiles, split reduction
+    (3, 16, 32, 8, 8, 3, 1, 1),      # an odd number of images: nine-tap kernel
     # weight-gradient stages whose window starts in a different column every stage (64 % B != 0)
     (64, 16, 32, 3, 5, 3, 1, 1),     # B = 5, 960 positions
     (16, 24, 40, 4, 6, 3, 1, 1),     # B = 6, partial channel tiles
