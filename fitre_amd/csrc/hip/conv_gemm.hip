@@ -139,17 +139,11 @@ static bool c3_dw_eligible(const fitre_conv_shape *s)
 static bool cell_geometry(const fitre_conv_shape *s) { return c3_geometry(s) && s->inA == kCellMap && s->inB == kCellMap; }
 // 8 x 8 maps: the weight gradient's stage is half a map of two images
 static bool cell8_geometry(const fitre_conv_shape *s) { return c3_geometry(s) && s->inA == kCell8Map && s->inB == kCell8Map && s->samples % 2 == 0; }
-static bool cell_kernels_on() // EXPERIMENT toggle
-{
-	static int on = -1;
-	if (on < 0) on = getenv("FITRE_NO_CELL") == nullptr;
-	return on != 0;
-}
 // the input gradient on 4 x 4 maps in the cell form: whole tiles of 32 images, one product
 static bool cell_dx_eligible(const fitre_conv_shape *s, int pairs)
 {
 	(void)pairs; // a second (delta, weights) pair continues the reduction
-	return cell_geometry(s) && cell_kernels_on() && s->samples % kCellImages == 0 && s->outChannels % kCellCB == 0;
+	return cell_geometry(s) && s->samples % kCellImages == 0 && s->outChannels % kCellCB == 0;
 }
 static BlockPlan c3_pos_plan(const fitre_conv_shape *s, bool dx, int cus = 0, int pairs = 1)
 {
@@ -172,8 +166,8 @@ static BlockPlan c3_dw_plan(const fitre_conv_shape *s, int cus = 0, int pairs = 
 	long J = (long)s->samples * s->inA * s->inB;
 	long tiles = ((s->inChannels + kC3DwCin - 1) / kC3DwCin) * ((s->outChannels + kC3Tile - 1) / kC3Tile);
 	double stageUs = (kC3Stage / 2.0) * 9.0 * 64.0 / 2400.0; // three waves per SIMD, three MFMAs per step each
-	if (cell_geometry(s) && cell_kernels_on()) stageUs *= 100.0 / 144.0;
-	if (cell8_geometry(s) && cell_kernels_on()) stageUs *= 84.0 / 96.0;
+	if (cell_geometry(s)) stageUs *= 100.0 / 144.0;
+	if (cell8_geometry(s)) stageUs *= 84.0 / 96.0;
 	return plan_blocks(tiles, pairs * ((J + kC3Stage - 1) / kC3Stage), stageUs, 1, s->outChannels, (long)s->inChannels * 9, cus);
 }
 static size_t c3_pos_workspace(const fitre_conv_shape *s, bool dx, int pairs = 1)
@@ -295,13 +289,13 @@ static int launch_c3_dw(const fitre_conv_shape *s, const float *x, const float *
 	if (grid.y > 65535 || grid.z > 65535) return fail(FITRE_E_UNSUPPORTED, "conv3x3 grid too large");
 	{
 		LaunchScope scope(FITRE_KC_CONV_DW, pairs * conv_flops(s),
-		                  !cell_kernels_on() ? 4 : (cell_geometry(s) ? 7 : (cell8_geometry(s) ? 8 : 4)));
+		                  cell_geometry(s) ? 7 : (cell8_geometry(s) ? 8 : 4));
 		const bool narrow = s->inB >= 2 && s->inB <= 16;
 		const bool vecx = vecd && ((((uintptr_t)x) & 15) == 0) && (!x2 || (((uintptr_t)x2) & 15) == 0);
-		if (cell8_geometry(s) && cell_kernels_on()) { // whole pairs of images (eligibility)
+		if (cell8_geometry(s)) { // whole pairs of images (eligibility)
 			if (vecx) conv3x3_dw_cell8_kernel<true><<<grid, kC3DwThreads, 0, stream()>>>(p, delta, deltaBytes, part);
 			else conv3x3_dw_cell8_kernel<false><<<grid, kC3DwThreads, 0, stream()>>>(p, delta, deltaBytes, part);
-		} else if (cell_geometry(s) && cell_kernels_on()) { // J is a multiple of 64 (eligibility): whole stages of four images
+		} else if (cell_geometry(s)) { // J is a multiple of 64 (eligibility): whole stages of four images
 			if (vecx) conv3x3_dw_cell_kernel<true><<<grid, kC3DwThreads, 0, stream()>>>(p, delta, deltaBytes, part);
 			else conv3x3_dw_cell_kernel<false><<<grid, kC3DwThreads, 0, stream()>>>(p, delta, deltaBytes, part);
 		} else if (vecd && narrow)
