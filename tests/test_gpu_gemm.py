@@ -47,6 +47,7 @@ CONV_CASES = [
     (32, 32, 128, 4, 4, 3, 1, 1),    # one tile each way
     (36, 40, 72, 4, 4, 3, 1, 1),     # partial channel tiles, nine stages
     (64, 96, 160, 4, 4, 3, 1, 1),    # split reduction
+    (32, 40, 72, 4, 4, 3, 1, 1),     # whole image tiles with partial channel tiles in the input gradient's cell form
     (6, 16, 32, 4, 4, 3, 1, 1),      # six images: not whole stages, nine-tap kernels
     # 8x8 maps: the weight gradient's stages are half maps of two images
     (6, 32, 128, 8, 8, 3, 1, 1),     # one tile, six stages
