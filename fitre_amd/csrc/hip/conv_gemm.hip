@@ -753,11 +753,12 @@ int fitre_hip_gemm(int transA, int transB, int M, int N, int K, float alpha, con
 int fitre_hip_linear_is_small(int in, int out, int n) { return small_gemm_fits(in, n, out) && small_gemm_fits(out, in, n); }
 
 int fitre_hip_linear_input_grad(int in, int out, int n, const float *W, const float *delta, int actBelow, const float *zPre,
-                                const float *zPost, int extA, int extB, float *result, float *staging, void *ws, size_t wsBytes)
+                                const float *zPost, int extA, int extB, float *result, float *staging, void *ws, size_t wsBytes,
+                                float *deltaCopy)
 {
 	FITRE_NEED_INIT();
 	FITRE_REQUIRE(in > 0 && out > 0 && n > 0, "fitre_hip_linear_input_grad: non-positive shape %d x %d, %d samples", out, in, n);
-	FITRE_REQUIRE(W && delta && result && result != delta, "fitre_hip_linear_input_grad: null or aliased pointer");
+	FITRE_REQUIRE(W && delta && result && result != delta && result != deltaCopy, "fitre_hip_linear_input_grad: null or aliased pointer");
 	const bool permute = extA > 0 || extB > 0;
 	FITRE_REQUIRE(!permute || (extA > 0 && extB > 0 && in % (extA * extB) == 0),
 	              "fitre_hip_linear_input_grad: %d inputs are not whole %d x %d maps", in, extA, extB);
@@ -770,9 +771,14 @@ int fitre_hip_linear_input_grad(int in, int out, int n, const float *W, const fl
 		p.C = result, p.ldc = in, p.alpha = 1.f, p.beta = 0.f;
 		p.act = derivative ? actBelow : -1, p.zPre = zPre, p.zPost = zPost;
 		p.extA = permute ? extA : 0, p.extB = permute ? extB : 0;
+		p.copyB = (deltaCopy && deltaCopy != delta) ? deltaCopy : nullptr;
 		return launch_small_gemm(p, FITRE_KC_FC_GEMM);
 	}
 	// the engine, then the steps of the epilogue one by one
+	if (deltaCopy && deltaCopy != delta) {
+		int rcCopy = fitre_hip_copy_d2d(deltaCopy, delta, sizeof(float) * (size_t)out * n);
+		if (rcCopy) return rcCopy;
+	}
 	float *plain = permute ? staging : result;
 	FITRE_REQUIRE(plain != nullptr && plain != delta, "fitre_hip_linear_input_grad: a product of this size needs the staging buffer");
 	int rc = gemm_ex(1, 0, in, n, out, 1.f, W, out, delta, out, 0.f, plain, in, nullptr, 0, FITRE_KC_FC_GEMM, ws, wsBytes);

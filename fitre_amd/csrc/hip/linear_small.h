@@ -32,6 +32,7 @@ struct SmallGemmParams {
 	const float *zPre, *zPost;
 	int extA, extB;  // > 0: row m = (c * extB + b) * extA + a goes to [c][n][a][b]
 	float *rowSums;  // sum over k of op(A)(m, k) for every m, or null
+	float *copyB;    // op(B) is also written here, in B's own layout, or null (the workgroups of the first block row do it)
 };
 
 __device__ __forceinline__ float act_backward_value(int actFun, float d, float zi, float zo)
@@ -72,6 +73,7 @@ __global__ void __launch_bounds__(256) small_gemm_kernel(const SmallGemmParams p
 			const bool aok = (m0 + am < p.M) & (k0 + ak < p.K), bok = (n0 + bn < p.N) & (k0 + bk < p.K);
 			av[i] = aok ? p.A[(long)(m0 + am) * p.sAm + (long)(k0 + ak) * p.sAk] : 0.f;
 			bv[i] = bok ? p.B[(long)(k0 + bk) * p.sBk + (long)(n0 + bn) * p.sBn] : 0.f;
+			if (p.copyB != nullptr && blockIdx.x == 0 && bok) p.copyB[(long)(k0 + bk) * p.sBk + (long)(n0 + bn) * p.sBn] = bv[i];
 		}
 		__syncthreads(); // the previous block's readers are done
 #pragma unroll

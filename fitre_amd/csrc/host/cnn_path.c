@@ -331,21 +331,31 @@ void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, 
 		real *slot = dx + zOffsets[f + nc + 1];
 		const real *zin = z + zOffsets[f + nc] + ((f == 0) ? last->outputOffset : 0);
 
-		/* delta .* f'(.) of the output layer (a plain copy when it has no activation); the layers below get theirs
-		 * from the epilogue of the product above them */
-		if (f == model->lLayers - 1)
-			HIP_CALL(fitre_hip_activation_backward(l->actFun, delta, zl + l->offset, zl, slot, (long)l->out * n));
-		LANE_WAIT(1, 0);
+		/* delta .* f'(.) of the output layer; the layers below get theirs from the epilogue of the product above them.
+		 * Without an activation it is the caller's delta as it stands: the product reads it there and leaves the copy in
+		 * the slot on its way. */
+		const real *cur_delta = slot;
+		real *snapshot = NULL;
+		if (f == model->lLayers - 1) {
+			if (l->actFun == CNN_ACT_NONE || l->actFun == ACT_LINEAR) {
+				cur_delta = delta;
+				snapshot = slot;
+			} else {
+				HIP_CALL(fitre_hip_activation_backward(l->actFun, delta, zl + l->offset, zl, slot, (long)l->out * n));
+			}
+		}
+		if (!snapshot) LANE_WAIT(1, 0);
 		/* the chain goes straight on: delta of the layer below = f'(.) .* (W' * delta) */
 		if (f > 0) {
 			const FC_LAYER *below = &model->fcLayer[f - 1];
 			real *zb = z + zOffsets[f + nc];
-			HIP_CALL(fitre_hip_linear_input_grad(l->in, l->out, n, weights + wOffsets[f + nc], slot, below->actFun,
-			                                     zb + below->offset, zb, 0, 0, dx + zOffsets[f + nc], NULL, ws, wsBytes));
+			HIP_CALL(fitre_hip_linear_input_grad(l->in, l->out, n, weights + wOffsets[f + nc], cur_delta, below->actFun,
+			                                     zb + below->offset, zb, 0, 0, dx + zOffsets[f + nc], NULL, ws, wsBytes, snapshot));
 		} else {
-			HIP_CALL(fitre_hip_linear_input_grad(l->in, l->out, n, weights + wOffsets[f + nc], slot, -1, NULL, NULL, extA, extB,
-			                                     features, delta_new, ws, wsBytes));
+			HIP_CALL(fitre_hip_linear_input_grad(l->in, l->out, n, weights + wOffsets[f + nc], cur_delta, -1, NULL, NULL, extA, extB,
+			                                     features, delta_new, ws, wsBytes, snapshot));
 		}
+		if (snapshot) LANE_WAIT(1, 0); /* lane 1 reads the slot the product has just filled */
 		/* beside it, on lane 1, what nothing later in this pass reads: dW = delta * z', db = delta * 1 */
 		LANE_SELECT(1);
 		HIP_CALL(fitre_hip_linear_weight_grad(l->in, l->out, n, slot, zin, gradient + wOffsets[f + nc],

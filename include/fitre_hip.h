@@ -393,14 +393,16 @@ int fitre_hip_gemm(int transA, int transB, int M, int N, int K, float alpha, con
  *   pointers a call of fitre_hip_activation_backward would take), no derivative for CNN_ACT_NONE / ACT_LINEAR / a
  *   negative code.  extA, extB > 0: the rows are whole extA x extB maps of a convolution layer and the result is
  *   stored in its layout [channel][sample][a][b] (the permutation of fitre_hip_fc_to_conv); `staging` (in x n
- *   floats, may be NULL for a small layer) then holds the unpermuted product of a large layer.
+ *   floats, may be NULL for a small layer) then holds the unpermuted product of a large layer.  deltaCopy (may be
+ *   NULL): delta is also copied there (the snapshot of functions/cnn_backward.cu:238-240, for a layer whose delta the
+ *   caller did not produce itself).
  *   weight gradient (:189-197 and the bias gradient :216-224): dW(out x in) = delta * zin', db(out) = delta * 1
  *   (db may be NULL).
  * ws / wsBytes: fitre_hip_gemm_workspace of the respective product (unused for small layers). */
 int fitre_hip_linear_is_small(int in, int out, int n);
 int fitre_hip_linear_input_grad(int in, int out, int n, const float *W, const float *delta, int actBelow,
                                 const float *zPre, const float *zPost, int extA, int extB, float *result,
-                                float *staging, void *ws, size_t wsBytes);
+                                float *staging, void *ws, size_t wsBytes, float *deltaCopy);
 int fitre_hip_linear_weight_grad(int in, int out, int n, const float *delta, const float *zin, float *dW, float *db,
                                  void *ws, size_t wsBytes);
 

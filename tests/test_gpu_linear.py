@@ -55,10 +55,13 @@ def test_input_gradient_with_the_derivative_below(dev, n_in, n_out, n, act):
     out = dev.upload(np.full(n_in * n, 7.0, np.float32))
     ws_bytes = hip.fitre_hip_gemm_workspace(n_in, n, n_out)
     ws = dev.alloc(ws_bytes)
-    ok(hip.fitre_hip_linear_input_grad(n_in, n_out, n, pw, pd, act, pzi, pzo, 0, 0, out, None, ws, ws_bytes))
+    snap = dev.upload(np.full(n_out * n + 3, 9.0, np.float32))   # the copy of delta the call leaves on its way
+    ok(hip.fitre_hip_linear_input_grad(n_in, n_out, n, pw, pd, act, pzi, pzo, 0, 0, out, None, ws, ws_bytes, snap))
     got = dev.download(out, n_in * n).reshape(n, n_in).T
     assert rel_err(got, want) < TOL
-    for p in (pw, pd, pzi, pzo, out, ws):
+    copied = dev.download(snap, n_out * n + 3)
+    assert np.array_equal(copied[:-3], d) and (copied[-3:] == 9.0).all()
+    for p in (pw, pd, pzi, pzo, out, ws, snap):
         dev.free(p)
 
 
@@ -79,13 +82,13 @@ def test_input_gradient_in_the_convolution_layout(dev, channels, ext_a, ext_b, n
     staging = dev.zeros(n_in * n)
     ws_bytes = hip.fitre_hip_gemm_workspace(n_in, n, n_out)
     ws = dev.alloc(ws_bytes)
-    ok(hip.fitre_hip_linear_input_grad(n_in, n_out, n, pw, pd, -1, None, None, ext_a, ext_b, out, staging, ws, ws_bytes))
+    ok(hip.fitre_hip_linear_input_grad(n_in, n_out, n, pw, pd, -1, None, None, ext_a, ext_b, out, staging, ws, ws_bytes, None))
     got = dev.download(out, n_in * n).reshape(channels, n, ext_a, ext_b)
     assert rel_err(got, want) < TOL
     if not hip.fitre_hip_linear_is_small(n_in, n_out, n):
         # a large layer without the staging buffer is refused before anything is queued
-        assert hip.fitre_hip_linear_input_grad(n_in, n_out, n, pw, pd, -1, None, None, ext_a, ext_b, out, None, ws, ws_bytes) == 2
-    assert hip.fitre_hip_linear_input_grad(n_in, n_out, n, pw, pd, -1, None, None, ext_a + 1, ext_b, out, staging, ws, ws_bytes) == 2 \
+        assert hip.fitre_hip_linear_input_grad(n_in, n_out, n, pw, pd, -1, None, None, ext_a, ext_b, out, None, ws, ws_bytes, None) == 2
+    assert hip.fitre_hip_linear_input_grad(n_in, n_out, n, pw, pd, -1, None, None, ext_a + 1, ext_b, out, staging, ws, ws_bytes, None) == 2 \
         or n_in % ((ext_a + 1) * ext_b) == 0
     for p in (pw, pd, out, staging, ws):
         dev.free(p)
@@ -136,9 +139,9 @@ def test_small_layers_are_deterministic(dev):
 
 def test_linear_arguments_are_checked(dev):
     p = dev.zeros(64)
-    assert hip.fitre_hip_linear_input_grad(0, 4, 4, p, p, -1, None, None, 0, 0, p, None, None, 0) == 2
-    assert hip.fitre_hip_linear_input_grad(4, 4, 4, p, p, -1, None, None, 0, 0, p, None, None, 0) == 2  # result aliases delta
-    assert hip.fitre_hip_linear_input_grad(4, 4, 4, None, p, -1, None, None, 0, 0, p, None, None, 0) == 2
+    assert hip.fitre_hip_linear_input_grad(0, 4, 4, p, p, -1, None, None, 0, 0, p, None, None, 0, None) == 2
+    assert hip.fitre_hip_linear_input_grad(4, 4, 4, p, p, -1, None, None, 0, 0, p, None, None, 0, None) == 2  # result aliases delta
+    assert hip.fitre_hip_linear_input_grad(4, 4, 4, None, p, -1, None, None, 0, 0, p, None, None, 0, None) == 2
     assert hip.fitre_hip_linear_weight_grad(4, 4, 0, p, p, p, None, None, 0) == 2
     assert hip.fitre_hip_linear_weight_grad(4, 4, 4, p, None, p, None, None, 0) == 2
     dev.free(p)
