@@ -5,8 +5,9 @@
 // GFLOP per pass at batch 1024).  Here both gradients are computed with ordinary vector multiply-adds by
 // workgroups that keep one image at a time in LDS:
 //
-//   input gradient   one thread per (input channel, input cell) with the channel uniform over a wave: the image's
-//                    delta (all output channels, zero border) in LDS, the weights through scalar loads;
+//   input gradient   one thread per (input channel, four neighbouring cells of a row) with the channel uniform over
+//                    a wave: the image's delta (all output channels, zero border) in LDS, read in 16-byte groups,
+//                    the weights through scalar loads;
 //   weight gradient  one thread per (patch index k = (ci, ta, tb), position slice), Cout accumulators in
 //                    registers; per position one LDS read of the input cell and Cout / 4 broadcast 16-byte
 //                    reads of delta (stored [position][channel]); a patch index of constant one yields the bias
@@ -31,16 +32,22 @@ struct ThinConvParams {
 	int parts, rowsPerUnit, unitsPerGroup; // weight gradient: bands of output rows per image, rows per band, units per workgroup
 	FastDiv divInB, divOutB, divK, divKK, divCells, divOcells;
 	FastDiv divPlane, divPB; // input gradient: bordered delta plane and its row length
+	FastDiv divGroups;       // input gradient: groups of four cells per image row
 	FastDiv divPBx;          // weight gradient: row length of the bordered input
 	FastDiv divXPlane[2], divDPos[2]; // weight gradient: bordered input plane / positions of a full band [0] and of an image's last band [1]
 };
 
 // ---- input gradient (stride 1): dx[ci][n][a][b] = sum_co sum_taps W[co][ci][ta][tb] * delta[co][n][a - ta + p][b - tb + p]
 // One workgroup per (image, group of input channels).  The image's delta (all output channels) sits in LDS with a
-// zero border of k - 1 - p cells, so that no tap needs a bounds check; a wave takes 64 cells of one input channel
-// at a time: the channel is the same for the whole wave, so the weights W[co][ci][.] come through scalar loads
-// and every tap is one LDS read and one multiply-add.
+// zero border of k - 1 - p cells, so that no tap needs a bounds check, in rows padded to a multiple of four words.
+// A thread owns FOUR neighbouring cells of a row (columns 4g .. 4g + 3): the k + 3 delta words a window row needs
+// for them are two aligned 16-byte reads (k = 5) that feed 4 k multiply-adds -- a quarter of the LDS traffic of a
+// thread per cell, which is what bounds this kernel.  A wave works on ONE input channel at a time, so the weights
+// W[co][ci][.] come through scalar loads and a multiply-add takes a scalar operand.
 // KS: window extent known at compile time (the tap loops are unrolled), 0: any
+constexpr int kThinDxCells = 4; // cells of a row per thread
+__host__ __device__ inline int thin_dx_row_words(int inB, int ks) { return (((inB + 3) & ~3) + ks - 1 + 3) & ~3; }
+
 template <int KS>
 __global__ void __launch_bounds__(256)
 thin_input_grad_kernel(const ThinConvParams p, const float *__restrict__ w, const float *__restrict__ delta, float *__restrict__ dx)
@@ -50,7 +57,7 @@ thin_input_grad_kernel(const ThinConvParams p, const float *__restrict__ w, cons
 	const int ks = KS > 0 ? KS : p.ksize;
 	const int cells = p.inA * p.inB, ocells = p.outA * p.outB, taps = ks * ks;
 	const int border = ks - 1 - p.pad;
-	const int PB = p.inB + ks - 1, plane = (p.inA + ks - 1) * PB;
+	const int PB = thin_dx_row_words(p.inB, ks), plane = (p.inA + ks - 1) * PB;
 	const int n = blockIdx.x;
 	const size_t oplane = (size_t)p.samples * ocells, iplane = (size_t)p.samples * cells;
 	// delta with its border, eight loads of a thread in flight at a time
@@ -75,36 +82,60 @@ thin_input_grad_kernel(const ThinConvParams p, const float *__restrict__ w, cons
 	}
 	__syncthreads();
 	const int lane = tid & 63, wave = tid >> 6;
-	const int chunks = (cells + 63) / 64, chunk = (cells + chunks - 1) / chunks; // cells per wave, evenly
+	const int groups = (p.inB + kThinDxCells - 1) / kThinDxCells; // column groups of a row
+	const int items = p.inA * groups;                              // threads' worth of work per input channel
+	const int chunks = (items + 63) / 64, chunk = (items + chunks - 1) / chunks; // items per wave, evenly
 	const int ci0 = blockIdx.y * p.ciPerGroup;
 	const int ciN = (p.cin - ci0 < p.ciPerGroup) ? p.cin - ci0 : p.ciPerGroup;
 	for (int task = wave; task < ciN * chunks; task += 4) {
 		const int ci = __builtin_amdgcn_readfirstlane(ci0 + task / chunks);
 		const int part = task % chunks;
-		const int cell = part * chunk + lane;
-		const bool live = lane < chunk && cell < cells;
-		uint32_t a, b;
-		p.divInB.divmod((uint32_t)(live ? cell : 0), a, b);
+		const int item = part * chunk + lane;
+		const bool live = lane < chunk && item < items;
+		uint32_t a, g;
+		p.divGroups.divmod((uint32_t)(live ? item : 0), a, g);
+		const int b0 = kThinDxCells * (int)g;
 		// delta[a - ta + p][b - tb + p] is the bordered cell [a + (k - 1 - ta)][b + (k - 1 - tb)]
-		const float *d0 = thin_lds + (int)a * PB + (int)b;
+		const float *d0 = thin_lds + (int)a * PB + b0;
 		const float *wci = w + (size_t)ci * taps;
-		float acc = 0.f;
+		float acc[kThinDxCells] = { 0.f, 0.f, 0.f, 0.f };
 		for (int co = 0; co < p.cout; co++) {
 			const float *wk = wci + (size_t)co * p.cin * taps;
 			const float *dco = d0 + co * plane;
 			if constexpr (KS > 0) {
+				constexpr int WORDS = (KS + kThinDxCells - 1 + 3) & ~3; // delta words of a window row, in whole 16-byte groups
 #pragma unroll
 				for (int ta = 0; ta < KS; ta++) {
-					const float *drow = dco + (KS - 1 - ta) * PB;
+					const float4 *drow = reinterpret_cast<const float4 *>(dco + (KS - 1 - ta) * PB);
+					float d[WORDS];
 #pragma unroll
-					for (int tb = 0; tb < KS; tb++) acc = fmaf(wk[ta * KS + tb], drow[KS - 1 - tb], acc);
+					for (int q = 0; q < WORDS / 4; q++) {
+						const float4 v4 = drow[q];
+						d[4 * q] = v4.x, d[4 * q + 1] = v4.y, d[4 * q + 2] = v4.z, d[4 * q + 3] = v4.w;
+					}
+#pragma unroll
+					for (int tb = 0; tb < KS; tb++) {
+						const float wv = wk[ta * KS + tb];
+#pragma unroll
+						for (int jj = 0; jj < kThinDxCells; jj++) acc[jj] = fmaf(wv, d[jj + KS - 1 - tb], acc[jj]);
+					}
 				}
 			} else {
 				for (int ta = 0; ta < ks; ta++)
-					for (int tb = 0; tb < ks; tb++) acc = fmaf(wk[ta * ks + tb], dco[(ks - 1 - ta) * PB + (ks - 1 - tb)], acc);
+					for (int tb = 0; tb < ks; tb++) {
+						const float wv = wk[ta * ks + tb];
+						const float *dd = dco + (ks - 1 - ta) * PB + (ks - 1 - tb);
+#pragma unroll
+						for (int jj = 0; jj < kThinDxCells; jj++) acc[jj] = fmaf(wv, dd[jj], acc[jj]);
+					}
 			}
 		}
-		if (live) dx[(size_t)ci * iplane + (size_t)n * cells + cell] = acc;
+		if (live) {
+			float *out = dx + (size_t)ci * iplane + (size_t)n * cells + (int)a * p.inB + b0;
+#pragma unroll
+			for (int jj = 0; jj < kThinDxCells; jj++)
+				if (b0 + jj < p.inB) out[jj] = acc[jj];
+		}
 	}
 }
 
@@ -251,8 +282,9 @@ static inline ThinConvParams thin_params(const fitre_conv_shape *s)
 	p.ciPerGroup = 1;
 	p.parts = 1, p.rowsPerUnit = s->outA, p.unitsPerGroup = 1;
 	p.divPBx = FastDiv((uint32_t)(s->inB + 2 * s->padding));
-	p.divPB = FastDiv((uint32_t)(s->inB + s->ksize - 1));
-	p.divPlane = FastDiv((uint32_t)((s->inA + s->ksize - 1) * (s->inB + s->ksize - 1)));
+	p.divPB = FastDiv((uint32_t)thin_dx_row_words(s->inB, s->ksize));
+	p.divPlane = FastDiv((uint32_t)((s->inA + s->ksize - 1) * thin_dx_row_words(s->inB, s->ksize)));
+	p.divGroups = FastDiv((uint32_t)((s->inB + 3) / 4));
 	p.divInB = FastDiv((uint32_t)s->inB);
 	p.divOutB = FastDiv((uint32_t)s->outB);
 	p.divK = FastDiv((uint32_t)s->ksize);
@@ -266,7 +298,7 @@ static inline ThinConvParams thin_params(const fitre_conv_shape *s)
 constexpr int kThinDxLdsFloats = 15360; // 60 KB: the bordered delta of one image
 static inline int thin_dx_lds_floats(const fitre_conv_shape *s)
 {
-	return s->outChannels * (s->inA + s->ksize - 1) * (s->inB + s->ksize - 1);
+	return s->outChannels * (s->inA + s->ksize - 1) * thin_dx_row_words(s->inB, s->ksize);
 }
 static inline bool thin_dx_eligible(const fitre_conv_shape *s)
 {
