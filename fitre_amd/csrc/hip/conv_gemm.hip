@@ -752,6 +752,13 @@ int fitre_hip_gemm(int transA, int transB, int M, int N, int K, float alpha, con
 // ---- backward products of a fully connected layer --------------------------------------------
 int fitre_hip_linear_is_small(int in, int out, int n) { return small_gemm_fits(in, n, out) && small_gemm_fits(out, in, n); }
 
+size_t fitre_hip_linear_weight_grad_workspace(int in, int out, int n)
+{
+	const size_t g = gemm_ex_workspace(out, in, n, 0);
+	const size_t r = small_gemm_ranges_fit(out, in, n) ? small_gemm_ranges_workspace(out, in, n) : 0;
+	return g > r ? g : r;
+}
+
 int fitre_hip_linear_input_grad(int in, int out, int n, const float *W, const float *delta, int actBelow, const float *zPre,
                                 const float *zPost, int extA, int extB, float *result, float *staging, void *ws, size_t wsBytes,
                                 float *deltaCopy)
@@ -806,6 +813,16 @@ int fitre_hip_linear_weight_grad(int in, int out, int n, const float *delta, con
 		p.act = -1;
 		p.rowSums = db;
 		return launch_small_gemm(p, FITRE_KC_FC_GEMM);
+	}
+	if (small_gemm_ranges_fit(out, in, n) && ws && wsBytes >= small_gemm_ranges_workspace(out, in, n) && ((((uintptr_t)ws) & 3) == 0)) {
+		SmallGemmParams p{};
+		p.M = out, p.N = in, p.K = n;
+		p.A = delta, p.sAm = 1, p.sAk = out;
+		p.B = zin, p.sBk = in, p.sBn = 1;
+		p.C = dW, p.ldc = out, p.alpha = 1.f, p.beta = 0.f;
+		p.act = -1;
+		p.rowSums = db;
+		return launch_small_gemm_ranges(p, FITRE_KC_FC_GEMM, ws);
 	}
 	int rc = gemm_ex(0, 1, out, in, n, 1.f, delta, out, zin, in, 0.f, dW, out, nullptr, 0, FITRE_KC_FC_GEMM, ws, wsBytes);
 	if (rc || !db) return rc;

@@ -936,7 +936,8 @@ __global__ void __launch_bounds__(256) sum_slabs_kernel(float *base, int splits,
 }
 
 // One (channel, segment) per workgroup.  POOL 0: 2x2 / stride 2 max pool (B % 4 == 0, A even), the
-// unit of work is a 2 x 4 patch; POOL 2: no pooling, the unit is a 16-byte group; POOL 3: 2x2 / stride 2
+// unit of work is a 2 x 4 patch; POOL 1: the same for any even B, the unit is one 2 x 2 window moved as two 8-byte
+// rows; POOL 2: no pooling, the unit is a 16-byte group; POOL 3: 2x2 / stride 2
 // max pool of maps with B == 2, where pooled cell q of a channel is its 16-byte group q.  z_act == nullptr:
 // the activation is ReLU and its output is max(zhat, 0).  partial: slots of four doubles
 // (sum g, sum g*zhat, sum zhat) per (channel, segment).
@@ -963,6 +964,40 @@ pool_act_sums_kernel(const float *delta, int dSplits, long dStride, const float 
 			if (dxPool) store4(dxPool + base + i, g, streamPool);
 			g = act_backward4(actFun, g, zi, zo);
 			*reinterpret_cast<float4 *>(dxAct + base + i) = g;
+			bn_sums4(g, zi, s1, s2, s3);
+		}
+	} else if constexpr (POOL == 1) {
+		const int outB = inB / 2, outA = inA / 2;
+		const int perMap = outA * outB;
+		const long patches = (long)samples * perMap;
+		const long per = (patches + gridDim.x - 1) / gridDim.x;
+		const long lo = (long)blockIdx.x * per;
+		const long hi = (lo + per < patches) ? lo + per : patches;
+		const size_t dBase = (size_t)c * samples * perMap;
+		for (long i = lo + threadIdx.x; i < hi; i += kRedBlock) {
+			const long map = i / perMap;
+			const int rem = (int)(i - map * perMap);
+			const int oa = rem / outB, pb = rem - oa * outB;
+			const size_t inOff = base + (size_t)map * inA * inB + (size_t)(2 * oa) * inB + 2 * pb;
+			const float2 a0 = *reinterpret_cast<const float2 *>(zhat + inOff);
+			const float2 a1 = *reinterpret_cast<const float2 *>(zhat + inOff + inB);
+			const float4 zi = make_float4(a0.x, a0.y, a1.x, a1.y);
+			float4 zo;
+			if (z_act) {
+				const float2 q0 = *reinterpret_cast<const float2 *>(z_act + inOff);
+				const float2 q1 = *reinterpret_cast<const float2 *>(z_act + inOff + inB);
+				zo = make_float4(q0.x, q0.y, q1.x, q1.y);
+			} else {
+				zo = relu4(zi);
+			}
+			float4 g = route2x2(zo, load_sum1(delta + dBase + i, dSplits, dStride));
+			if (dxPool) {
+				*reinterpret_cast<float2 *>(dxPool + inOff) = make_float2(g.x, g.y);
+				*reinterpret_cast<float2 *>(dxPool + inOff + inB) = make_float2(g.z, g.w);
+			}
+			g = act_backward4(actFun, g, zi, zo);
+			*reinterpret_cast<float2 *>(dxAct + inOff) = make_float2(g.x, g.y);
+			*reinterpret_cast<float2 *>(dxAct + inOff + inB) = make_float2(g.z, g.w);
 			bn_sums4(g, zi, s1, s2, s3);
 		}
 	} else {
@@ -1609,9 +1644,9 @@ int fitre_hip_pool_act_bn_backward(int poolType, int actFun, float *delta, int d
 	if (poolType == NO_POOL)
 		fused = aligned && aligned16(delta) && perChannel % 4 == 0 && (deltaSplits == 1 || deltaStride % 4 == 0);
 	else if (poolType == MAX_POOL)
-		fused = aligned && ksize == 2 && stride == 2 && padding == 0 && (inB % 4 == 0 || inB == 2) && inA % 2 == 0 &&
+		fused = aligned && ksize == 2 && stride == 2 && padding == 0 && inB % 2 == 0 && inA % 2 == 0 && perChannel % 4 == 0 &&
 		        outA == inA / 2 && outB == inB / 2 && (((uintptr_t)delta & 7) == 0) && (deltaSplits == 1 || deltaStride % 2 == 0);
-	const int variant = (poolType == NO_POOL) ? 2 : (inB == 2 ? 3 : 0);
+	const int variant = (poolType == NO_POOL) ? 2 : (inB == 2 ? 3 : (inB % 4 == 0 ? 0 : 1));
 	if (!fused) {
 		// other windows / layouts: the separate passes (slabs summed, z_act rebuilt for the ReLU shortcut)
 		if (deltaSplits > 1) {
@@ -1634,7 +1669,7 @@ int fitre_hip_pool_act_bn_backward(int poolType, int actFun, float *delta, int d
 	const double total = (double)channels * (double)perChannel;
 	const double poolBytes = 4.0 * total * (2 + (dxPool ? 1 : 0) + (z_act ? 1 : 0)) +
 	                         4.0 * deltaSplits * (poolType == NO_POOL ? total : total / 4);
-	if (perChannel <= kBnSmallChannel && channels >= 128) {
+	if (perChannel <= kBnSmallChannel && channels >= 128 && variant != 1) {
 		LaunchScope scope(FITRE_KC_POOL_ACT_BWD, poolBytes + 4.0 * total);
 		if (variant == 2)
 			pool_act_bn_small_kernel<2><<<channels, kRedBlock, 0, stream()>>>(delta, deltaSplits, deltaStride, zhat, z_act, variance, inA, inB, samples, actFun,
@@ -1653,7 +1688,9 @@ int fitre_hip_pool_act_bn_backward(int poolType, int actFun, float *delta, int d
 	const bool streamPool = 4.0 * total >= 48.0 * 1024 * 1024; // the pool gradient is a snapshot nothing reads in this pass
 	{
 		LaunchScope scope(FITRE_KC_POOL_ACT_BWD, poolBytes);
-		if (variant == 2)
+		if (variant == 1)
+			pool_act_sums_kernel<1><<<grid, kRedBlock, 0, stream()>>>(delta, deltaSplits, deltaStride, zhat, z_act, inA, inB, samples, actFun, dxPool, streamPool, dxAct, partial);
+		else if (variant == 2)
 			pool_act_sums_kernel<2><<<grid, kRedBlock, 0, stream()>>>(delta, deltaSplits, deltaStride, zhat, z_act, inA, inB, samples, actFun, dxPool, streamPool, dxAct, partial);
 		else if (variant == 3)
 			pool_act_sums_kernel<3><<<grid, kRedBlock, 0, stream()>>>(delta, deltaSplits, deltaStride, zhat, z_act, inA, inB, samples, actFun, dxPool, streamPool, dxAct, partial);

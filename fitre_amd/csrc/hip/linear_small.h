@@ -33,6 +33,8 @@ struct SmallGemmParams {
 	int extA, extB;  // > 0: row m = (c * extB + b) * extA + a goes to [c][n][a][b]
 	float *rowSums;  // sum over k of op(A)(m, k) for every m, or null
 	float *copyB;    // op(B) is also written here, in B's own layout, or null (the workgroups of the first block row do it)
+	int kChunk;      // > 0: the reduction is cut into ranges of kChunk, one per blockIdx.z, whose raw sums go to `partial`
+	float *partial;  // [range][N * M results, then M row sums] (no epilogue: small_gemm_reduce_kernel applies alpha and stores)
 };
 
 __device__ __forceinline__ float act_backward_value(int actFun, float d, float zi, float zo)
@@ -63,14 +65,16 @@ __global__ void __launch_bounds__(256) small_gemm_kernel(const SmallGemmParams p
 	constexpr int kPer = kSmallDepth * kSmallTile / 256; // elements of each operand a thread loads per block
 	float acc00 = 0.f, acc01 = 0.f, acc10 = 0.f, acc11 = 0.f, rs0 = 0.f, rs1 = 0.f;
 	const bool sums = p.rowSums != nullptr && blockIdx.y == 0 && tn == 0;
-	for (int k0 = 0; k0 < p.K; k0 += kSmallDepth) {
+	const int kBeg = p.kChunk > 0 ? (int)blockIdx.z * p.kChunk : 0;
+	const int kEnd = (p.kChunk > 0 && kBeg + p.kChunk < p.K) ? kBeg + p.kChunk : p.K;
+	for (int k0 = kBeg; k0 < kEnd; k0 += kSmallDepth) {
 		float av[kPer], bv[kPer];
 #pragma unroll
 		for (int i = 0; i < kPer; i++) {
 			const int e = tid + 256 * i; // along the tile: e % 32; along the depth: e / 32 -- or the other way round
 			const int am = aAlongM ? (e & 31) : e / kSmallDepth, ak = aAlongM ? (e >> 5) : e % kSmallDepth;
 			const int bn = bAlongN ? (e & 31) : e / kSmallDepth, bk = bAlongN ? (e >> 5) : e % kSmallDepth;
-			const bool aok = (m0 + am < p.M) & (k0 + ak < p.K), bok = (n0 + bn < p.N) & (k0 + bk < p.K);
+			const bool aok = (m0 + am < p.M) & (k0 + ak < kEnd), bok = (n0 + bn < p.N) & (k0 + bk < kEnd);
 			av[i] = aok ? p.A[(long)(m0 + am) * p.sAm + (long)(k0 + ak) * p.sAk] : 0.f;
 			bv[i] = bok ? p.B[(long)(k0 + bk) * p.sBk + (long)(n0 + bn) * p.sBn] : 0.f;
 			if (p.copyB != nullptr && blockIdx.x == 0 && bok) p.copyB[(long)(k0 + bk) * p.sBk + (long)(n0 + bn) * p.sBn] = bv[i];
@@ -85,7 +89,7 @@ __global__ void __launch_bounds__(256) small_gemm_kernel(const SmallGemmParams p
 			Bs[bk][bn] = bv[i];
 		}
 		__syncthreads();
-		const int depth = (p.K - k0 < kSmallDepth) ? p.K - k0 : kSmallDepth;
+		const int depth = (kEnd - k0 < kSmallDepth) ? kEnd - k0 : kSmallDepth;
 		for (int k = 0; k < depth; k++) {
 			const float a0 = As[k][tm], a1 = As[k][tm + 16], b0 = Bs[k][tn], b1 = Bs[k][tn + 16];
 			acc00 = fmaf(a0, b0, acc00);
@@ -94,6 +98,21 @@ __global__ void __launch_bounds__(256) small_gemm_kernel(const SmallGemmParams p
 			acc11 = fmaf(a1, b1, acc11);
 			if (sums) rs0 += a0, rs1 += a1;
 		}
+	}
+	if (p.kChunk > 0) { // raw sums of this reduction range
+		float *part = p.partial + (size_t)blockIdx.z * ((size_t)p.M * p.N + p.M);
+		if (sums) {
+			if (m0 + tm < p.M) part[(size_t)p.M * p.N + m0 + tm] = rs0;
+			if (m0 + tm + 16 < p.M) part[(size_t)p.M * p.N + m0 + tm + 16] = rs1;
+		}
+		auto put = [&](int m, int n, float acc) {
+			if (m < p.M && n < p.N) part[(size_t)n * p.M + m] = acc;
+		};
+		put(m0 + tm, n0 + tn, acc00);
+		put(m0 + tm + 16, n0 + tn, acc10);
+		put(m0 + tm, n0 + tn + 16, acc01);
+		put(m0 + tm + 16, n0 + tn + 16, acc11);
+		return;
 	}
 	if (sums) {
 		if (m0 + tm < p.M) p.rowSums[m0 + tm] = rs0;
@@ -123,13 +142,64 @@ __global__ void __launch_bounds__(256) small_gemm_kernel(const SmallGemmParams p
 	store(m0 + tm + 16, n0 + tn + 16, acc11);
 }
 
+// C = alpha * (sum of the ranges' partial results, in range order, in double) and the row sums likewise
+__global__ void __launch_bounds__(256) small_gemm_reduce_kernel(const float *partial, int ranges, int M, int N, float alpha, float *C,
+                                                                long ldc, float *rowSums)
+{
+	const long per = (long)M * N + M;
+	const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+	if (i >= per) return;
+	double acc = 0.0;
+	for (int r = 0; r < ranges; r++) acc += (double)partial[(size_t)r * per + i];
+	if (i < (long)M * N) {
+		const long n = i / M, m = i - n * M;
+		C[n * ldc + m] = alpha * (float)acc;
+	} else if (rowSums) {
+		rowSums[i - (long)M * N] = (float)acc;
+	}
+}
+
 // A product is "small" when it is below one wave of engine tiles and its reduction is short enough for one
 // workgroup per result block to walk it alone.
 constexpr double kSmallGemmWork = 3.2e7; // multiply-adds
 constexpr int kSmallGemmMaxK = 512;
+constexpr double kSmallGemmShortWork = 1.3e8; // the bound for reductions of at most two blocks (a wide, shallow product)
 static inline bool small_gemm_fits(int M, int N, int K)
 {
-	return M > 0 && N > 0 && K > 0 && K <= kSmallGemmMaxK && (double)M * N * K <= kSmallGemmWork;
+	if (M <= 0 || N <= 0 || K <= 0 || K > kSmallGemmMaxK) return false;
+	return (double)M * N * K <= (K <= 2 * kSmallDepth ? kSmallGemmShortWork : kSmallGemmWork);
+}
+
+// A long reduction over a small result (the weight gradient of a small linear layer at a large batch): ranges of
+// kSmallRange reduction indices go to different workgroups and a second launch adds their partial results.
+constexpr int kSmallRange = 128;
+constexpr int kSmallMaxRanges = 64;
+static inline bool small_gemm_ranges_fit(int M, int N, int K)
+{
+	return M > 0 && N > 0 && K > kSmallGemmMaxK && K <= kSmallRange * kSmallMaxRanges && (long)M * N <= 65536 &&
+	       (double)M * N * K <= 4.0e8;
+}
+static inline size_t small_gemm_ranges_workspace(int M, int N, int K)
+{
+	return sizeof(float) * (size_t)((K + kSmallRange - 1) / kSmallRange) * ((size_t)M * N + M);
+}
+// plain product + row sums only (no bias, activation, permutation, beta)
+static inline int launch_small_gemm_ranges(SmallGemmParams p, int kernelClass, void *ws)
+{
+	const int ranges = (p.K + kSmallRange - 1) / kSmallRange;
+	float *C = p.C, *rowSums = p.rowSums;
+	const float alpha = p.alpha;
+	p.kChunk = kSmallRange, p.partial = (float *)ws;
+	p.rowSums = rowSums ? (float *)ws : nullptr; // only its being non-null matters to the kernel in this mode
+	dim3 grid((unsigned)((p.M + kSmallTile - 1) / kSmallTile), (unsigned)((p.N + kSmallTile - 1) / kSmallTile), (unsigned)ranges);
+	{
+		LaunchScope scope(kernelClass, 2.0 * (double)p.M * p.N * p.K, 0);
+		small_gemm_kernel<<<grid, 256, 0, stream()>>>(p);
+	}
+	const long per = (long)p.M * p.N + p.M;
+	LaunchScope scope(FITRE_KC_SPLITK_REDUCE, 4.0 * (double)per * (ranges + 1));
+	small_gemm_reduce_kernel<<<(unsigned)((per + 255) / 256), 256, 0, stream()>>>((const float *)ws, ranges, p.M, p.N, alpha, C, p.ldc, rowSums);
+	return check_launch("small_gemm_kernel");
 }
 
 static inline int launch_small_gemm(const SmallGemmParams &p, int kernelClass)

@@ -129,7 +129,7 @@ static size_t backward_side_ws_bytes(const CNN_MODEL *model, int batch)
 	}
 	for (int i = 0; i < model->lLayers; i++) {
 		const FC_LAYER *f = &model->fcLayer[i];
-		need = max_sz(need, fitre_hip_gemm_workspace(f->out, f->in, batch));
+		need = max_sz(need, fitre_hip_linear_weight_grad_workspace(f->in, f->out, batch));
 	}
 	return (need + 255) & ~(size_t)255;
 }
@@ -259,7 +259,22 @@ static double backward_conv_work(const CNN_MODEL *model, int n)
 	}
 	return macs;
 }
+/* What the lanes can hide is the chain's bandwidth-bound steps (pooling, activation, batch norm: about 28 bytes per
+ * activation with batch norm, 16 without) behind the weight gradients' matrix work.  Where a pass has little of
+ * them per multiply-add, two matrix kernels side by side only get in each other's way: AlexNet at batch 64 (about
+ * 400 FLOP per such byte) takes 2.94 ms on one lane and 3.04 ms on two, VGG-11 with batch norm at batch 256 (about
+ * 140) 1.52 ms against 1.39 ms. */
+static double backward_flop_per_elementwise_byte(const CNN_MODEL *model, int n)
+{
+	double bytes = 0;
+	for (int c = 0; c < model->cLayers; c++) {
+		const CONV_LAYER *l = &model->convLayer[c];
+		bytes += (double)n * l->outHeight * l->outWidth * l->outChannels * (has_bn(l) ? 28.0 : 16.0);
+	}
+	return bytes > 0 ? 2.0 * backward_conv_work(model, n) / bytes : 0.0;
+}
 #define LANE_WORK_THRESHOLD 2.0e9
+#define LANE_INTENSITY_LIMIT 250.0
 #define LANE_SELECT(lane_) do { if (lanes) HIP_CALL(fitre_hip_lane_select(lane_)); } while (0)
 #define LANE_WAIT(waiter_, signaller_) do { if (lanes) HIP_CALL(fitre_hip_lane_wait(waiter_, signaller_)); } while (0)
 
@@ -271,7 +286,7 @@ void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, 
 	const int *wOffsets = model->wOffsets, *bOffsets = model->bOffsets, *zOffsets = model->zOffsets;
 	const real *weights = data->weights;
 	const int n = batchSize, nc = model->cLayers;
-	const int lanes = backward_conv_work(model, n) >= LANE_WORK_THRESHOLD;
+	const int lanes = backward_conv_work(model, n) >= LANE_WORK_THRESHOLD && backward_flop_per_elementwise_byte(model, n) < LANE_INTENSITY_LIMIT;
 	void *ws = (void *)devPtr; /* input-gradient partials (and the FC products' splits) */
 	const size_t wsBytes = backward_dx_ws_bytes(model, model->batchSize);
 	void *bnWs = (void *)((char *)devPtr + wsBytes);

@@ -116,6 +116,7 @@ HIP_API = {
     "fitre_hip_gemm_workspace": (sz, [i32, i32, i32]),
     "fitre_hip_gemm": (i32, [i32, i32, i32, i32, i32, f32, vp, i32, vp, i32, f32, vp, i32, vp, vp, sz]),
     "fitre_hip_linear_is_small": (i32, [i32, i32, i32]),
+    "fitre_hip_linear_weight_grad_workspace": (sz, [i32, i32, i32]),
     "fitre_hip_linear_input_grad": (i32, [i32, i32, i32, vp, vp, i32, vp, vp, i32, i32, vp, vp, vp, sz, vp]),
     "fitre_hip_linear_weight_grad": (i32, [i32, i32, i32, vp, vp, vp, vp, vp, sz]),
     "fitre_hip_lane_select": (i32, [i32]),

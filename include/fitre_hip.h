@@ -398,8 +398,11 @@ int fitre_hip_gemm(int transA, int transB, int M, int N, int K, float alpha, con
  *   caller did not produce itself).
  *   weight gradient (:189-197 and the bias gradient :216-224): dW(out x in) = delta * zin', db(out) = delta * 1
  *   (db may be NULL).
- * ws / wsBytes: fitre_hip_gemm_workspace of the respective product (unused for small layers). */
+ * ws / wsBytes: fitre_hip_gemm_workspace(in, n, out) for the input gradient, fitre_hip_linear_weight_grad_workspace for
+ * the weight gradient (a small layer at a large batch cuts the batch into ranges and adds their partial results in a
+ * second launch); unused for small layers. */
 int fitre_hip_linear_is_small(int in, int out, int n);
+size_t fitre_hip_linear_weight_grad_workspace(int in, int out, int n);
 int fitre_hip_linear_input_grad(int in, int out, int n, const float *W, const float *delta, int actBelow,
                                 const float *zPre, const float *zPost, int extA, int extB, float *result,
                                 float *staging, void *ws, size_t wsBytes, float *deltaCopy);

@@ -33,10 +33,10 @@ def forward_act(act, zi):
             CNN_ACT_SOFTPLUS: np.log1p(np.exp(zi)), CNN_ACT_SWISH: zi * sig, CNN_ACT_NONE: zi, -1: zi}[act]
 
 
-# (in, out, samples): LeNet's tail at batch 128 and ragged sizes around the 32-wide blocks (small kernel); AlexNet-like
-# and long-reduction layers (the engine path)
-SMALL = [(84, 10, 128), (120, 84, 128), (400, 120, 128), (33, 31, 65), (1, 1, 1), (64, 32, 32), (100, 7, 500)]
-LARGE = [(1024, 512, 64), (400, 120, 1024), (4096, 100, 96)]
+# (in, out, samples): LeNet's tail at batch 128, ragged sizes around the 32-wide blocks and a wide, shallow product (small
+# kernel); AlexNet-like layers (the engine) and long reductions over small results (ranges of the batch + a second launch)
+SMALL = [(84, 10, 128), (120, 84, 128), (400, 120, 128), (33, 31, 65), (1, 1, 1), (64, 32, 32), (100, 7, 500), (4096, 100, 96)]
+LARGE = [(1024, 512, 64), (400, 120, 1024), (4096, 1000, 64), (84, 10, 1024), (120, 84, 3000), (33, 7, 8192)]
 
 
 @pytest.mark.parametrize("act", [CNN_ACT_RELU, CNN_ACT_SWISH, CNN_ACT_SOFTPLUS, CNN_ACT_ELU, CNN_ACT_NONE, -1])
@@ -66,7 +66,7 @@ def test_input_gradient_with_the_derivative_below(dev, n_in, n_out, n, act):
 
 
 @pytest.mark.parametrize("channels,ext_a,ext_b,n_out,n", [(16, 5, 5, 120, 128), (3, 2, 7, 33, 40), (1, 1, 1, 5, 9),
-                                                           (256, 6, 6, 512, 64), (64, 3, 2, 100, 1200)])
+                                                           (256, 6, 6, 512, 64), (64, 3, 2, 600, 1200)])
 def test_input_gradient_in_the_convolution_layout(dev, channels, ext_a, ext_b, n_out, n):
     """Row m = (c * B + b) * A + a of the product lands at [c][sample][a][b] (fitre_hip_fc_to_conv's permutation)."""
     n_in = channels * ext_a * ext_b
@@ -105,7 +105,7 @@ def test_weight_and_bias_gradient(dev, n_in, n_out, n, bias):
     pd, pz = dev.upload(d), dev.upload(zin)
     dw = dev.upload(np.full(n_out * n_in, 3.0, np.float32))
     db = dev.upload(np.full(n_out + 4, 5.0, np.float32))
-    ws_bytes = hip.fitre_hip_gemm_workspace(n_out, n_in, n)
+    ws_bytes = hip.fitre_hip_linear_weight_grad_workspace(n_in, n_out, n)
     ws = dev.alloc(ws_bytes)
     ok(hip.fitre_hip_linear_weight_grad(n_in, n_out, n, pd, pz, dw, db if bias else None, ws, ws_bytes))
     got = dev.download(dw, n_out * n_in).reshape(n_in, n_out).T

@@ -300,7 +300,11 @@ FUSED_BN_GEOMS = [
     (130, 2, 2, 4, 2, 2, 0),
     (512, 64, 2, 2, 2, 2, 0),    # maps with B == 2: a window is one 16-byte group
     (5, 2100, 6, 2, 2, 2, 0),    # the same on long channels
-    (2, 3, 6, 10, 2, 2, 0),      # B % 4 != 0: separate passes
+    (2, 4, 6, 10, 2, 2, 0),      # B % 4 == 2: windows moved as 8-byte rows (LeNet's 10 x 10 maps)
+    (16, 32, 10, 10, 2, 2, 0),   # the same, several segments
+    (130, 2, 2, 6, 2, 2, 0),     # the same on short channels (two launches)
+    (2, 3, 6, 10, 2, 2, 0),      # channel length not a multiple of four: separate passes
+    (3, 4, 6, 5, 2, 2, 0),       # odd B: separate passes
     (2, 2, 7, 5, 3, 2, 1),       # 3/2/1 window: separate passes
 ]
 
