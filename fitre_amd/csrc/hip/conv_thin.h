@@ -30,6 +30,7 @@ struct ThinConvParams {
 	int imagesPerGroup;
 	int ciPerGroup; // input gradient: input channels per workgroup
 	int parts, rowsPerUnit, unitsPerGroup; // weight gradient: bands of output rows per image, rows per band, units per workgroup
+	int xRowWords;                         // weight gradient: words per row of the bordered input in LDS
 	FastDiv divInB, divOutB, divK, divKK, divCells, divOcells;
 	FastDiv divPlane, divPB; // input gradient: bordered delta plane and its row length
 	FastDiv divGroups;       // input gradient: groups of four cells per image row
@@ -154,7 +155,7 @@ thin_weight_grad_kernel(const ThinConvParams p, const float *__restrict__ x, con
 	const int K = p.cin * p.ksize * p.ksize, K1 = K + 1;
 	const int cells = p.inA * p.inB, ocells = p.outA * p.outB;
 	const int slices = 512 / K1; // >= 1 (host checks K + 1 <= 512)
-	const int PBx = p.inB + 2 * p.pad;
+	const int PBx = p.xRowWords; // >= inB + 2 * pad, chosen so that the lanes' patch offsets spread over the LDS banks
 	const int xRowsMax = (p.rowsPerUnit - 1) * p.stride + p.ksize;
 	float *xs = thin_lds;
 	float *ds = thin_lds + ((p.cin * xRowsMax * PBx + 3) & ~3);
@@ -211,23 +212,35 @@ thin_weight_grad_kernel(const ThinConvParams p, const float *__restrict__ x, con
 		}
 		__syncthreads();
 		if (live) {
-			// position q = (r, ob) of the band reads the bordered cell [r * stride + ta][ob * stride + tb]
-			const float *xc = xs + ((int)ci * xRows + (int)ta) * PBx + (int)tb;
-			uint32_t r, ob;
-			p.divOutB.divmod((uint32_t)slice, r, ob);
-			for (int q = slice; q < dPos; q += slices) {
-				const float xv = ones ? 1.f : xc[((int)r * PBx + (int)ob) * p.stride];
+			// A slice takes a run of consecutive positions, row segment by row segment: position (r, ob) of the band
+			// reads the bordered cell [r * stride + ta][ob * stride + tb], so inside a segment both operands advance
+			// by constants.
+			const int run = (dPos + slices - 1) / slices;
+			int q = slice * run;
+			const int qEnd = (q + run < dPos) ? q + run : dPos;
+			uint32_t r = 0, ob = 0;
+			p.divOutB.divmod((uint32_t)(q < dPos ? q : 0), r, ob);
+			const float *xrow = xs + ((int)ci * xRows + (int)ta + (int)r * p.stride) * PBx + (int)tb;
+			while (q < qEnd) {
+				int segEnd = q + (p.outB - (int)ob);
+				segEnd = segEnd < qEnd ? segEnd : qEnd;
+				const float *xp = xrow + (int)ob * p.stride;
 				const float4 *dq = reinterpret_cast<const float4 *>(ds + q * COUT);
+				for (; q < segEnd; q++) {
+					const float xv = ones ? 1.f : *xp;
+					xp += p.stride;
 #pragma unroll
-				for (int g = 0; g < COUT / 4; g++) {
-					const float4 d = dq[g];
-					acc[4 * g] = fmaf(d.x, xv, acc[4 * g]);
-					acc[4 * g + 1] = fmaf(d.y, xv, acc[4 * g + 1]);
-					acc[4 * g + 2] = fmaf(d.z, xv, acc[4 * g + 2]);
-					acc[4 * g + 3] = fmaf(d.w, xv, acc[4 * g + 3]);
+					for (int g = 0; g < COUT / 4; g++) {
+						const float4 d = dq[g];
+						acc[4 * g] = fmaf(d.x, xv, acc[4 * g]);
+						acc[4 * g + 1] = fmaf(d.y, xv, acc[4 * g + 1]);
+						acc[4 * g + 2] = fmaf(d.z, xv, acc[4 * g + 2]);
+						acc[4 * g + 3] = fmaf(d.w, xv, acc[4 * g + 3]);
+					}
+					dq += COUT / 4;
 				}
-				ob += (uint32_t)slices;
-				while (ob >= (uint32_t)p.outB) ob -= (uint32_t)p.outB, r++;
+				ob = 0;
+				xrow += p.stride * PBx;
 			}
 		}
 	}
@@ -271,6 +284,25 @@ __global__ void __launch_bounds__(256) thin_dw_reduce_kernel(const float *partia
 	}
 }
 
+// Words per row of the weight gradient's bordered input in LDS.  The lanes of a wave are consecutive patch indices
+// (tb fastest, then ta): they read words tb + ta * row apart, so a row length that is a multiple of 32 puts all of
+// a window's rows on the same banks (LeNet's first layer: 32-wide images, 15 lanes per bank).  The row is padded
+// until the window's k * k offsets cover as many different banks as they can.
+static inline int thin_dw_row_words(const fitre_conv_shape *s)
+{
+	const int base = s->inB + 2 * s->padding, k = s->ksize;
+	int best = base, bestBanks = -1;
+	for (int row = base; row < base + 32; row++) {
+		unsigned used = 0;
+		for (int ta = 0; ta < k; ta++)
+			for (int tb = 0; tb < k; tb++) used |= 1u << ((tb + ta * row) & 31);
+		const int banks = __builtin_popcount(used);
+		if (banks > bestBanks) bestBanks = banks, best = row;
+		if (banks == (k * k < 32 ? k * k : 32)) break;
+	}
+	return best;
+}
+
 static inline ThinConvParams thin_params(const fitre_conv_shape *s)
 {
 	ThinConvParams p;
@@ -281,7 +313,8 @@ static inline ThinConvParams thin_params(const fitre_conv_shape *s)
 	p.imagesPerGroup = 1;
 	p.ciPerGroup = 1;
 	p.parts = 1, p.rowsPerUnit = s->outA, p.unitsPerGroup = 1;
-	p.divPBx = FastDiv((uint32_t)(s->inB + 2 * s->padding));
+	p.xRowWords = thin_dw_row_words(s);
+	p.divPBx = FastDiv((uint32_t)p.xRowWords);
 	p.divPB = FastDiv((uint32_t)thin_dx_row_words(s->inB, s->ksize));
 	p.divPlane = FastDiv((uint32_t)((s->inA + s->ksize - 1) * thin_dx_row_words(s->inB, s->ksize)));
 	p.divGroups = FastDiv((uint32_t)((s->inB + 3) / 4));
@@ -350,7 +383,7 @@ static inline size_t thin_dw_lds_floats(const fitre_conv_shape *s)
 	const ThinDwPlan pl = thin_dw_plan(s);
 	const int K1 = s->inChannels * s->ksize * s->ksize + 1, cp = thin_dw_pad(s->outChannels);
 	const int xRows = (pl.rowsPerUnit - 1) * s->stride + s->ksize;
-	const size_t stage = (size_t)((s->inChannels * xRows * (s->inB + 2 * s->padding) + 3) & ~3) + (size_t)pl.rowsPerUnit * s->outB * cp;
+	const size_t stage = (size_t)((s->inChannels * xRows * thin_dw_row_words(s) + 3) & ~3) + (size_t)pl.rowsPerUnit * s->outB * cp;
 	const size_t red = (size_t)(512 / K1) * K1 * cp;
 	return stage > red ? stage : red;
 }
@@ -374,7 +407,7 @@ static int launch_thin_dw_general(const fitre_conv_shape *s, const float *x, con
 	const int lastRows = s->outA - (pl.parts - 1) * pl.rowsPerUnit;
 	const int bandRows[2] = { pl.rowsPerUnit, lastRows };
 	for (int i = 0; i < 2; i++) {
-		p.divXPlane[i] = FastDiv((uint32_t)(((bandRows[i] - 1) * s->stride + s->ksize) * (s->inB + 2 * s->padding)));
+		p.divXPlane[i] = FastDiv((uint32_t)(((bandRows[i] - 1) * s->stride + s->ksize) * p.xRowWords));
 		p.divDPos[i] = FastDiv((uint32_t)(bandRows[i] * s->outB));
 	}
 	const int K = s->inChannels * s->ksize * s->ksize;
