@@ -227,6 +227,23 @@ def test_vgg11_full_size_backward_is_linear_in_delta(vgg_full, dev):
     np.testing.assert_array_equal(g2, 2 * g1)
 
 
+def test_vgg11_full_size_one_lane_gives_the_same_bits(vgg_full, dev):
+    """At this size cnnBackward spreads its launches over the lanes; with the lanes switched off everything is queued
+    on one stream.  The kernels and the order of every sum are the same, so gradient and dx must be too, bit for bit."""
+    gm, w = vgg_full
+    gm.forward()
+    gm.backward()
+    grad, dx = gm.get("grad"), gm.get("dx")
+    L.check(L.hip.fitre_hip_lanes_enable(0))
+    try:
+        L.check(L.hip.fitre_hip_memset(gm.grad, 0xFF, 4 * gm.model.pSize))
+        gm.backward()
+        np.testing.assert_array_equal(gm.get("grad").view(np.uint32), grad.view(np.uint32))
+        np.testing.assert_array_equal(gm.get("dx").view(np.uint32), dx.view(np.uint32))
+    finally:
+        L.check(L.hip.fitre_hip_lanes_enable(1))
+
+
 def test_vgg11_full_size_directional_derivative(vgg_full, dev):
     """g'd against a central difference of the loss along a random direction d (fp32 forward)."""
     gm, w = vgg_full
