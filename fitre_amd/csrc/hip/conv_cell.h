@@ -448,16 +448,17 @@ constexpr int kCellIT = 32;     // channel rows per workgroup tile
 constexpr int kCellCB = 8;      // reduction channels per LDS block
 
 // the MFMAs of one reduction block for the wave that owns quadrant (QA, QB)
-template <int QA, int QB, int A_LD, int B_LD>
+// A_PAIR: words between the weight fragments of two reduction pairs; FLIP: the weight of tap t is stored at 8 - t
+template <int QA, int QB, int A_PAIR, bool FLIP, int B_LD>
 __device__ __forceinline__ void cell_dx_block(const float *aBase, const float *bBase, v16f (&acc)[2][2])
 {
 	constexpr int CELL_LD = kCellImages + 1;
 #pragma unroll
 	for (int cp = 0; cp < kCellCB / 2; cp++) {
-		const float *aPair = aBase + cp * 2 * A_LD, *bPair = bBase + cp * 2 * B_LD;
+		const float *aPair = aBase + cp * A_PAIR, *bPair = bBase + cp * 2 * B_LD;
 		float a[9], b[kCells];
 #pragma unroll
-		for (int tap = 0; tap < 9; tap++) a[tap] = aPair[8 - tap];
+		for (int tap = 0; tap < 9; tap++) a[tap] = aPair[FLIP ? 8 - tap : tap];
 #pragma unroll
 		for (int q = 0; q < kCells; q++) {
 			const int qa = q / kCellMap, qb = q % kCellMap;
@@ -479,15 +480,18 @@ __device__ __forceinline__ void cell_dx_block(const float *aBase, const float *b
 	}
 }
 
-template <bool VECW>
+// DX = false: the forward product, out[i][n][cell] = bias[i] + sum over c and live taps of W[i][c][tap] * src[c][n][cell + tap
+// shift]; its weights sit in LDS as IT rows (output channel) of the block's CB * 9 weights, odd row stride.
+template <bool DX, bool VECW>
 __global__ void __launch_bounds__(kGemmThreads, 2)
 conv3x3_cell_dx_kernel(const Conv3x3Params p, const OutParams out)
 {
 	FITRE_RAISE_MATRIX_WAVE_PRIORITY();
 	constexpr int IT = kCellIT, CB = kCellCB;
-	constexpr int A_LD = IT * 9 + 4;                     // a multiple of four: 16-byte stores
-	constexpr int A_FLOATS = CB * A_LD, A_DUMMY = A_FLOATS;
-	constexpr int WQ = IT * 9 / 4, WGROUPS = CB * WQ;    // 16-byte groups of weights per block
+	constexpr int A_LD = DX ? (IT * 9 + 4) : (CB * 9 + 1); // input gradient: a multiple of four (16-byte stores)
+	constexpr int A_FLOATS = DX ? CB * A_LD : IT * A_LD, A_DUMMY = A_FLOATS;
+	constexpr int WQ = DX ? (IT * 9 / 4) : (CB * 9 / 4);   // 16-byte groups per LDS row
+	constexpr int WGROUPS = (DX ? CB : IT) * WQ;           // 16-byte groups of weights per block
 	constexpr int WE = (WGROUPS + kGemmThreads - 1) / kGemmThreads;
 	constexpr int CELL_LD = kCellImages + 1;             // images of one cell, odd stride
 	constexpr int B_LD = kCells * CELL_LD + 1;           // per reduction channel
@@ -509,7 +513,7 @@ conv3x3_cell_dx_kernel(const Conv3x3Params p, const OutParams out)
 	const int cbTotal = p.src2 ? 2 * cbHalf : cbHalf; // a second pair continues the reduction
 	const int cbBeg = blockIdx.z * p.perSplit;
 	const int cbEnd = (cbBeg + p.perSplit < cbTotal) ? cbBeg + p.perSplit : cbTotal;
-	const int rowLen = p.I * 9;
+	const int rowLen = DX ? p.I * 9 : p.cred * 9;
 
 	// ---- what this thread stages, the same for every channel block -------------------------
 	uint32_t wOff[WE];
@@ -519,11 +523,14 @@ conv3x3_cell_dx_kernel(const Conv3x3Params p, const OutParams out)
 		const int idx = tid + kGemmThreads * e;
 		const int row = idx / WQ, qd = idx - row * WQ;
 		const bool has = idx < WGROUPS;
-		const int colG = i0 * 9 + 4 * qd;
-		const bool inside = has & (colG + 3 < rowLen);
-		const uint32_t off = 4u * (uint32_t)(row * rowLen + colG);
-		// columns past the tensor only feed accumulator rows that are never stored
-		wOff[e] = VECW ? (inside ? off : 0u) : (has ? off : kGroupOutOfRange);
+		// input gradient: row = reduction channel, w[(c0 + row) * I * 9 + i0 * 9 + 4 * qd ..]
+		// forward:        row = output channel,    w[(i0 + row) * cred * 9 + c0 * 9 + 4 * qd ..]
+		const int rowG = DX ? row : (i0 + row);
+		const int colG = DX ? (i0 * 9 + 4 * qd) : (4 * qd);
+		const bool inside = has & (DX ? (colG + 3 < rowLen) : (rowG < p.I));
+		const uint32_t off = 4u * (uint32_t)(rowG * rowLen + colG);
+		// rows or columns past the tensor only feed accumulator rows that are never stored
+		wOff[e] = VECW ? (inside ? off : 0u) : (inside ? off : kGroupOutOfRange);
 		wLds[e] = has ? row * A_LD + 4 * qd : A_DUMMY;
 	}
 	// source: group g = tid + 256 * e of the block's CB x (32 images x 16 cells) floats; a group is four cells of an image
@@ -546,7 +553,8 @@ conv3x3_cell_dx_kernel(const Conv3x3Params p, const OutParams out)
 #pragma unroll
 		for (int v = 0; v < 16; v++) acc[x >> 1][x & 1][v] = 0.f;
 
-	const float *aBase = As + khalf * A_LD + l32 * 9;
+	const float *aBase = DX ? (As + khalf * A_LD + l32 * 9) : (As + l32 * A_LD + khalf * 9);
+	constexpr int A_PAIR = DX ? 2 * A_LD : 18;
 	const float *bBase = Bs + khalf * B_LD + l32;
 
 #define CELL_LOAD_BLOCK(CBI)                                                                                          \
@@ -554,7 +562,7 @@ conv3x3_cell_dx_kernel(const Conv3x3Params p, const OutParams out)
 		const bool second_ = (CBI) >= cbHalf; /* uniform: the block belongs to the second pair */                    \
 		const int c0_ = ((CBI) - (second_ ? cbHalf : 0)) * CB;                                                        \
 		const float *wSel = second_ ? p.w2 : p.w, *sSel = second_ ? p.src2 : p.src;                                   \
-		const size_t wShift = (size_t)c0_ * rowLen; /* floats, uniform */                                             \
+		const size_t wShift = DX ? (size_t)c0_ * rowLen : (size_t)c0_ * 9; /* floats, uniform */                      \
 		if constexpr (VECW) {                                                                                         \
 			const char *wBlk = reinterpret_cast<const char *>(wSel + wShift);                                         \
 			_Pragma("unroll") for (int e = 0; e < WE; e++)                                                            \
@@ -587,8 +595,14 @@ conv3x3_cell_dx_kernel(const Conv3x3Params p, const OutParams out)
 	for (int cb = cbBeg; cb < cbEnd; cb++) {
 		__syncthreads();
 #pragma unroll
-		for (int e = 0; e < WE; e++)
-			*reinterpret_cast<float4 *>(As + wLds[e]) = make_float4(wreg[4 * e], wreg[4 * e + 1], wreg[4 * e + 2], wreg[4 * e + 3]);
+		for (int e = 0; e < WE; e++) {
+			float *dst = As + wLds[e];
+			if constexpr (DX) {
+				*reinterpret_cast<float4 *>(dst) = make_float4(wreg[4 * e], wreg[4 * e + 1], wreg[4 * e + 2], wreg[4 * e + 3]);
+			} else {
+				dst[0] = wreg[4 * e], dst[1] = wreg[4 * e + 1], dst[2] = wreg[4 * e + 2], dst[3] = wreg[4 * e + 3];
+			}
+		}
 #pragma unroll
 		for (int e = 0; e < SE; e++) {
 			float *dst = Bs + sLds[e];
@@ -596,10 +610,10 @@ conv3x3_cell_dx_kernel(const Conv3x3Params p, const OutParams out)
 		}
 		__syncthreads();
 		if (cb + 1 < cbEnd) CELL_LOAD_BLOCK(cb + 1);
-		if (wave == 0) cell_dx_block<0, 0, A_LD, B_LD>(aBase, bBase, acc);
-		else if (wave == 1) cell_dx_block<0, 1, A_LD, B_LD>(aBase, bBase, acc);
-		else if (wave == 2) cell_dx_block<1, 0, A_LD, B_LD>(aBase, bBase, acc);
-		else cell_dx_block<1, 1, A_LD, B_LD>(aBase, bBase, acc);
+		if (wave == 0) cell_dx_block<0, 0, A_PAIR, DX, B_LD>(aBase, bBase, acc);
+		else if (wave == 1) cell_dx_block<0, 1, A_PAIR, DX, B_LD>(aBase, bBase, acc);
+		else if (wave == 2) cell_dx_block<1, 0, A_PAIR, DX, B_LD>(aBase, bBase, acc);
+		else cell_dx_block<1, 1, A_PAIR, DX, B_LD>(aBase, bBase, acc);
 	}
 #undef CELL_LOAD_BLOCK
 

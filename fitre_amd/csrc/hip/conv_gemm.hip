@@ -139,18 +139,18 @@ static bool c3_dw_eligible(const fitre_conv_shape *s)
 static bool cell_geometry(const fitre_conv_shape *s) { return c3_geometry(s) && s->inA == kCellMap && s->inB == kCellMap; }
 // 8 x 8 maps: the weight gradient's stage is half a map of two images
 static bool cell8_geometry(const fitre_conv_shape *s) { return c3_geometry(s) && s->inA == kCell8Map && s->inB == kCell8Map && s->samples % 2 == 0; }
-// the input gradient on 4 x 4 maps in the cell form: whole tiles of 32 images, one product
-static bool cell_dx_eligible(const fitre_conv_shape *s, int pairs)
+// the position-contiguous products on 4 x 4 maps in the cell form: whole tiles of 32 images (a second (source,
+// weights) pair continues the reduction)
+static bool cell_pos_eligible(const fitre_conv_shape *s, bool dx)
 {
-	(void)pairs; // a second (delta, weights) pair continues the reduction
-	return cell_geometry(s) && s->samples % kCellImages == 0 && s->outChannels % kCellCB == 0;
+	return cell_geometry(s) && s->samples % kCellImages == 0 && (dx ? s->outChannels : s->inChannels) % kCellCB == 0;
 }
 static BlockPlan c3_pos_plan(const fitre_conv_shape *s, bool dx, int cus = 0, int pairs = 1)
 {
 	if (cus <= 0) cus = lane_compute_units();
 	long I = dx ? s->inChannels : s->outChannels, J = (long)s->samples * s->inA * s->inB;
 	long cred = dx ? s->outChannels : s->inChannels;
-	if (dx && cell_dx_eligible(s, pairs)) {
+	if (cell_pos_eligible(s, dx)) {
 		const long tiles = ((I + kCellIT - 1) / kCellIT) * (s->samples / kCellImages);
 		const double blockUs = (kCellCB / 2.0) * 25.0 * 64.0 / 2400.0; // reduction pairs x MFMAs per wave and pair x 64 cycles
 		return plan_blocks(tiles, pairs * cred / kCellCB, blockUs, 2, I, J, cus);
@@ -215,13 +215,13 @@ static int launch_c3_pos(const fitre_conv_shape *s, const float *src, const floa
 	}
 	const bool vecw = ((((uintptr_t)w) & 15) == 0) && (!w2 || (((uintptr_t)w2) & 15) == 0) && (DX ? (I % 4 == 0) : true);
 	// (the cell kernel stores 16-byte groups; a plan made for it also fits the nine-tap kernel: same block size)
-	if (DX && cell_dx_eligible(s, pairs) && (((uintptr_t)part.C) & 15) == 0) {
+	if (cell_pos_eligible(s, DX) && (((uintptr_t)part.C) & 15) == 0) {
 		dim3 grid((unsigned)(s->samples / kCellImages), (unsigned)((I + kCellIT - 1) / kCellIT), (unsigned)plan.splits);
 		if (grid.y > 65535 || grid.z > 65535) return fail(FITRE_E_UNSUPPORTED, "conv3x3 grid too large");
 		{
-			LaunchScope scope(FITRE_KC_CONV_DX, pairs * conv_flops(s), 7);
-			if (vecw) conv3x3_cell_dx_kernel<true><<<grid, kGemmThreads, 0, stream()>>>(p, part);
-			else conv3x3_cell_dx_kernel<false><<<grid, kGemmThreads, 0, stream()>>>(p, part);
+			LaunchScope scope(DX ? FITRE_KC_CONV_DX : FITRE_KC_CONV_FWD, pairs * conv_flops(s), 7);
+			if (vecw) conv3x3_cell_dx_kernel<DX, true><<<grid, kGemmThreads, 0, stream()>>>(p, part);
+			else conv3x3_cell_dx_kernel<DX, false><<<grid, kGemmThreads, 0, stream()>>>(p, part);
 		}
 		if (leftSplits) *leftSplits = plan.splits;
 		if (plan.splits > 1 && !leftSplits) launch_splitk_reduce((const float *)ws, plan.splits, I, J, out);
