@@ -110,12 +110,25 @@ void readDelimitedMatrix(char *fileName, real **data, int *rows, int *cols)
 	char *line = NULL;
 	size_t cap = 0;
 	*rows = *cols = 0;
+	int ragged = 0, first = 0;
 	while (getline(&line, &cap, f) > 0) { /* first pass: the shape; an empty line ends the matrix */
 		const int n = count_tokens(line);
 		if (n == 0) break;
+		if (*rows == 0) first = n;
+		if (n != first) ragged++;
 		*cols = n;
 		(*rows)++;
 	}
+	/* an empty line in the middle of a file, or rows of different lengths, give a matrix that is not what the file
+	 * holds: say so (the shape is still taken as before: rows up to the empty line, columns of the last row) */
+	while (getline(&line, &cap, f) > 0)
+		if (count_tokens(line) > 0) {
+			fprintf(stderr, "readDelimitedMatrix: %s: stopped at the empty line after row %d, but more rows follow\n", fileName, *rows);
+			break;
+		}
+	if (ragged)
+		fprintf(stderr, "readDelimitedMatrix: %s: %d of %d rows do not have the %d values of the first row; missing values read as 0\n",
+		        fileName, ragged, *rows, first);
 	fprintf(stderr, "Rows : %d, Columns : %d \n", *rows, *cols);
 	const size_t total = (size_t)*rows * (size_t)*cols;
 	*data = (real *)calloc(total > 0 ? total : 1, sizeof(real));

@@ -191,3 +191,27 @@ def test_delimited_text_matrix(tmp_path):
     cnn.readDelimitedMatrix(str(wide).encode(), C.byref(data), C.byref(rows), C.byref(cols))
     assert (rows.value, cols.value) == (1, 300000)
     np.testing.assert_array_equal(as_array(data, 300000), row)
+
+
+def test_delimited_text_matrix_reports_what_it_drops(tmp_path, capfd):
+    """Rows after an empty line and rows of uneven length are named on stderr; a clean file draws neither message."""
+    data, rows, cols = C.POINTER(C.c_float)(), C.c_int(), C.c_int()
+    clean = tmp_path / "clean.csv"
+    clean.write_text("1,2,3\n4,5,6\n\n")                                  # a trailing empty line drops nothing
+    cnn.readDelimitedMatrix(str(clean).encode(), C.byref(data), C.byref(rows), C.byref(cols))
+    err = capfd.readouterr().err
+    assert (rows.value, cols.value) == (2, 3) and "readDelimitedMatrix" not in err
+    C.CDLL(None).free(C.cast(data, C.c_void_p))
+    cut = tmp_path / "cut.csv"
+    cut.write_text("1,2,3\n4,5,6\n\n7,8,9\n")
+    cnn.readDelimitedMatrix(str(cut).encode(), C.byref(data), C.byref(rows), C.byref(cols))
+    err = capfd.readouterr().err
+    assert (rows.value, cols.value) == (2, 3) and "stopped at the empty line after row 2" in err
+    C.CDLL(None).free(C.cast(data, C.c_void_p))
+    ragged = tmp_path / "ragged.csv"
+    ragged.write_text("1,2,3\n4,5\n7,8,9\n")
+    cnn.readDelimitedMatrix(str(ragged).encode(), C.byref(data), C.byref(rows), C.byref(cols))
+    err = capfd.readouterr().err
+    assert (rows.value, cols.value) == (3, 3) and "1 of 3 rows do not have the 3 values" in err
+    np.testing.assert_array_equal(as_array(data, 9), [1, 2, 3, 4, 5, 0, 7, 8, 9])
+    C.CDLL(None).free(C.cast(data, C.c_void_p))
