@@ -30,6 +30,26 @@ size_t gemm_ex_workspace(int M, int N, int K, int flags);
 int gemm_ex_batched(int batch, int transA, int transB, int M, int N, int K, float alpha, const float *A, int lda, long strideA,
                     const float *B, int ldb, long strideB, float beta, float *C, int ldc, long strideC, int flags, int kernelClass,
                     void *ws, size_t wsBytes, long wsStrideBytes);
+// One argument set of gemm_ex_batched; gemm_pair_batched queues two such products that do not depend on each other --
+// as ONE launch when both run unsplit on the same tile (the chip then sees the tiles of both at once, and a chain of
+// dependent launches is one launch shorter), as two launches otherwise.
+struct BatchedProduct {
+	int transA, transB, M, N, K;
+	float alpha;
+	const float *A;
+	int lda;
+	long strideA;
+	const float *B;
+	int ldb;
+	long strideB;
+	float beta;
+	float *C;
+	int ldc;
+	long strideC;
+	int flags;
+};
+int gemm_pair_batched(int batch, const BatchedProduct &first, const BatchedProduct &second, int kernelClass, void *ws, size_t wsBytes,
+                      long wsStrideBytes);
 constexpr int kMaxLanes = 4; // one hardware queue each
 int lane();           // its index (0 .. kMaxLanes - 1)
 int lane_compute_units();     // compute units a kernel launched on the selected lane can occupy

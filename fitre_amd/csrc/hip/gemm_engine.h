@@ -387,7 +387,32 @@ struct OutParams {
 	// A lane's four consecutive rows then form one 16-byte group.  Applies to split partials as well (each a
 	// permutation of I x J elements, I % 4 == 0); bias, beta and mirror are not used with it.
 	long quadLd;
+	// Non-zero tapRows: both operands are patch rows in tap-major order (rows t * tapRows .. of tap t = (ta, tb) of a
+	// tapKs x tapKs window, stride 1, padding tapPad) over the reduction index (cell of the tapOutA x tapOutB output map,
+	// image), cells row by row, tapImages images per cell.  Row (t, c) is zero at the cells whose tap falls outside the
+	// tapSrcA x tapSrcB image, so the reduction of a tile (one tap on each side: tapRows is a multiple of the tile) runs
+	// from the first to the last cell at which both taps are inside; a pair of taps that never are gives a zero tile.
+	int tapRows, tapImages, tapKs, tapPad, tapOutA, tapOutB, tapSrcA, tapSrcB;
 };
+
+// first and one-past-last reduction index of the cells at which taps t1 and t2 both fall inside the image (lo >= hi: none)
+__host__ __device__ inline void tap_pair_range(const OutParams &o, int t1, int t2, int &lo, int &hi)
+{
+	const int a1 = t1 / o.tapKs - o.tapPad, b1 = t1 % o.tapKs - o.tapPad; // source cell = output cell + (a, b)
+	const int a2 = t2 / o.tapKs - o.tapPad, b2 = t2 % o.tapKs - o.tapPad;
+	const int amin = a1 < a2 ? a1 : a2, amax = a1 > a2 ? a1 : a2;
+	const int bmin = b1 < b2 ? b1 : b2, bmax = b1 > b2 ? b1 : b2;
+	int alo = -amin > 0 ? -amin : 0, ahi = o.tapSrcA - 1 - amax;
+	int blo = -bmin > 0 ? -bmin : 0, bhi = o.tapSrcB - 1 - bmax;
+	if (ahi > o.tapOutA - 1) ahi = o.tapOutA - 1;
+	if (bhi > o.tapOutB - 1) bhi = o.tapOutB - 1;
+	if (alo > ahi || blo > bhi) {
+		lo = hi = 0;
+		return;
+	}
+	lo = (alo * o.tapOutB + blo) * o.tapImages;
+	hi = (ahi * o.tapOutB + bhi + 1) * o.tapImages;
+}
 // both operands: element (row, k) is zero for k < row, so the reduction of a tile starts at the larger of its first rows
 constexpr int kTriBoth = 1;
 constexpr int kTriAFromRow = 2; // operand A: element (i, k) is zero for k < i
@@ -398,15 +423,14 @@ constexpr int kTriBToRow = 8;   // operand B: element (j, k) is zero for k > j
 // the kernel
 // ---------------------------------------------------------------------------
 // One workgroup's tile of reduction range `split` (the body of both kernels below).
+// As, Bs: the workgroup's LDS for one reduction slice of each operand (BK * OpA::LD resp. BK * OpB::LD floats)
 template <class Cfg, class OpA, class OpB>
 __device__ __forceinline__ void gemm_tile(const typename OpA::Params &pa, const typename OpB::Params &pb, const OutParams &out,
-                                          int I, int J, int R, int kChunk, int splitIndex)
+                                          int I, int J, int R, int kChunk, int splitIndex, float *As, float *Bs)
 {
 	constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK;
 	constexpr int TM = Cfg::TM, TN = Cfg::TN;
 	constexpr int LDA = OpA::LD, LDB = OpB::LD;
-	__shared__ float As[BK * LDA];
-	__shared__ float Bs[BK * LDB];
 
 	const int tid = threadIdx.x;
 	const int lane = tid & 63;
@@ -427,6 +451,13 @@ __device__ __forceinline__ void gemm_tile(const typename OpA::Params &pa, const 
 	}
 	if (out.triK & kTriAToRow) kend = (kend < i0 + BM) ? kend : i0 + BM;
 	if (out.triK & kTriBToRow) kend = (kend < j0 + BN) ? kend : j0 + BN;
+	if (out.tapRows) {
+		int lo, hi;
+		tap_pair_range(out, i0 / out.tapRows, j0 / out.tapRows, lo, hi);
+		lo &= ~(BK - 1);
+		kbeg = (kbeg > lo) ? kbeg : lo;
+		kend = (kend < hi) ? kend : hi;
+	}
 
 	OpA opA;
 	OpB opB;
@@ -524,7 +555,9 @@ __global__ void __launch_bounds__(kGemmThreads)
 mfma_gemm_kernel(const typename OpA::Params pa, const typename OpB::Params pb, const OutParams out, int I, int J, int R,
                  int kChunk)
 {
-	gemm_tile<Cfg, OpA, OpB>(pa, pb, out, I, J, R, kChunk, blockIdx.z);
+	__shared__ float As[Cfg::BK * OpA::LD];
+	__shared__ float Bs[Cfg::BK * OpB::LD];
+	gemm_tile<Cfg, OpA, OpB>(pa, pb, out, I, J, R, kChunk, blockIdx.z, As, Bs);
 }
 
 // `batch` independent products of one shape in one launch: grid.z = batch * splits; problem b reads its operands
@@ -538,7 +571,47 @@ mfma_gemm_batched_kernel(typename OpA::Params pa, typename OpB::Params pb, OutPa
 	pa.p += (size_t)batch * aStride;
 	pb.p += (size_t)batch * bStride;
 	out.C += (size_t)batch * cStride;
-	gemm_tile<Cfg, OpA, OpB>(pa, pb, out, I, J, R, kChunk, split);
+	__shared__ float As[Cfg::BK * OpA::LD];
+	__shared__ float Bs[Cfg::BK * OpB::LD];
+	gemm_tile<Cfg, OpA, OpB>(pa, pb, out, I, J, R, kChunk, split, As, Bs);
+}
+
+// Two unsplit batched products of different operand kinds in one launch (products that do not depend on each other
+// and would each leave most of the chip idle, or its last round of workgroups): blockIdx.z = which * batch + problem.
+// The grid covers the larger tile count of the two; a workgroup outside its product's tiles leaves at once.
+struct PairSide {
+	PlainParams pa, pb;
+	OutParams out;
+	int I, J, R;
+	int tilesI, tilesJ;
+	long aStride, bStride, cStride;
+};
+
+template <class Cfg, class OpA1, class OpB1, class OpA2, class OpB2>
+__global__ void __launch_bounds__(kGemmThreads)
+mfma_gemm_pair_kernel(PairSide first, PairSide second, int batch)
+{
+	constexpr int LA = OpA1::LD > OpA2::LD ? OpA1::LD : OpA2::LD;
+	constexpr int LB = OpB1::LD > OpB2::LD ? OpB1::LD : OpB2::LD;
+	__shared__ float As[Cfg::BK * LA];
+	__shared__ float Bs[Cfg::BK * LB];
+	const bool isSecond = (int)blockIdx.z >= batch; // uniform over the workgroup
+	const int problem = isSecond ? blockIdx.z - batch : blockIdx.z;
+	if (!isSecond) {
+		if ((int)blockIdx.y >= first.tilesI || (int)blockIdx.x >= first.tilesJ) return;
+		first.pa.p += (size_t)problem * first.aStride;
+		first.pb.p += (size_t)problem * first.bStride;
+		first.out.C += (size_t)problem * first.cStride;
+		const int kChunk = (first.R + Cfg::BK - 1) / Cfg::BK * Cfg::BK;
+		gemm_tile<Cfg, OpA1, OpB1>(first.pa, first.pb, first.out, first.I, first.J, first.R, kChunk, 0, As, Bs);
+	} else {
+		if ((int)blockIdx.y >= second.tilesI || (int)blockIdx.x >= second.tilesJ) return;
+		second.pa.p += (size_t)problem * second.aStride;
+		second.pb.p += (size_t)problem * second.bStride;
+		second.out.C += (size_t)problem * second.cStride;
+		const int kChunk = (second.R + Cfg::BK - 1) / Cfg::BK * Cfg::BK;
+		gemm_tile<Cfg, OpA2, OpB2>(second.pa, second.pb, second.out, second.I, second.J, second.R, kChunk, 0, As, Bs);
+	}
 }
 
 // C[i*ldc + j] = alpha * sum_s ws[s][i][j] (+bias) + beta*C, partials summed in split order.
@@ -862,7 +935,11 @@ static int launch_gemm(const PA &pa, const PB &pb, const OutParams &out, int I, 
 // per thread and operand in flight).  `groups`: tiles of all problems of the launch.
 inline bool deep_slice_plan(long I, long J, long R, bool mirror, int batch, long cus, const GemmPlan &standard, GemmPlan *deep)
 {
-	if (I > 384 || J > 384 || R > 1024) return false;
+	// one problem: up to 384 x 384 results; side by side, two or more problems bring enough 64 x 64 tiles for the chip up
+	// to order 1280 (measured on halves of order 576 and 1152 of three matrices: 36 -> 22 us and 106 -> 85 us per product
+	// with its reduction)
+	const long limit = batch >= 2 ? 1280 : 384;
+	if (I > limit || J > limit || R > (batch >= 2 ? 1280 : 1024)) return false;
 	long ti = (I + 63) / 64, tj = (J + 63) / 64;
 	long tiles = mirror ? ti * (ti + 1) / 2 : ti * tj;
 	long rounds = (tiles * batch + 3 * cus - 1) / (3 * cus);

@@ -327,7 +327,7 @@ struct InverseRun {
 	long wsStrideBytes;
 	float *W, *X;
 	float *L21[kMaxDepth]; // per recursion depth: the off-diagonal block of the factor (a node's children work one level down)
-	float *T2;             // temporary of the last product of a node
+	float *T2[kMaxDepth];  // per recursion depth: L21 * X11, the inner product of X21 (same sizes as L21)
 	int n;
 	int *dInfo;
 	void *gws;
@@ -367,19 +367,19 @@ static int chol_and_inverse(const InverseRun &r, int r0, int blocks, int nn, int
 	rc = gemm_ex_batched(r.batch, 0, 1, m, n1, n1, 1.f, A21, n, r.sWs, X11, n, r.sWs, 0.f, L21, m, r.sInv, kGemmBUpperTri, KC, r.gws, r.gBytes,
 	                     r.wsStrideBytes);
 	if (rc) return rc;
-	// A22 -= L21 L21^T
-	rc = gemm_ex_batched(r.batch, 0, 1, m, m, n1, -1.f, L21, m, r.sInv, L21, m, r.sInv, 1.f, A22, n, r.sWs, kGemmMirror, KC, r.gws,
-	                     r.gBytes, r.wsStrideBytes);
+	// A22 -= L21 L21^T and, side by side with it, T2 = L21 * X11, the inner product of X21 = -X22 * (L21 * X11): nothing
+	// needs it before the right half is done, and nothing it reads changes until then.
+	float *T2 = r.T2[depth];
+	const BatchedProduct update{ 0, 1, m, m, n1, -1.f, L21, m, r.sInv, L21, m, r.sInv, 1.f, A22, n, r.sWs, kGemmMirror };
+	const BatchedProduct inner{ 0, 0, m, n1, n1, 1.f, L21, m, r.sInv, X11, n, r.sWs, 0.f, T2, m, r.sInv, kGemmBLowerTri };
+	rc = gemm_pair_batched(r.batch, update, inner, KC, r.gws, r.gBytes, r.wsStrideBytes);
 	if (rc) return rc;
 	rc = chol_and_inverse(r, r1, blocks - b1, m, depth + 1);
 	if (rc) return rc;
 	// X21 = -X22 * (L21 * X11)
 	const float *X22 = r.X + (size_t)r1 * n + r1;
 	float *X21 = r.X + (size_t)r0 * n + r1;
-	rc = gemm_ex_batched(r.batch, 0, 0, m, n1, n1, 1.f, L21, m, r.sInv, X11, n, r.sWs, 0.f, r.T2, m, r.sInv, kGemmBLowerTri, KC, r.gws, r.gBytes,
-	                     r.wsStrideBytes);
-	if (rc) return rc;
-	return gemm_ex_batched(r.batch, 0, 0, m, n1, m, -1.f, X22, n, r.sWs, r.T2, m, r.sInv, 0.f, X21, n, r.sWs, kGemmALowerTri, KC, r.gws, r.gBytes,
+	return gemm_ex_batched(r.batch, 0, 0, m, n1, m, -1.f, X22, n, r.sWs, T2, m, r.sInv, 0.f, X21, n, r.sWs, kGemmALowerTri, KC, r.gws, r.gBytes,
 	                       r.wsStrideBytes);
 }
 
@@ -441,22 +441,21 @@ static int spd_inverse_run(const float *matrix, int n, float shift, float *inver
 		fill_zero_kernel<<<1, 64, 0, stream()>>>((float *)dInfo, ib.batch, 0);
 	}
 	// ---- 1. Cholesky factor and its inverse ---------------------------------------------------
-	// The result matrix is free until the last product and holds the temporaries: T2 (at most a
-	// quarter of the matrix) in its second half, the per-depth L21 blocks (a quarter, a sixteenth,
-	// ... of it) in the first.
+	// The result matrix is free until the last product and holds the temporaries: the per-depth L21 blocks (a quarter, a
+	// sixteenth, ... of it) in its first half, the per-depth T2 blocks, of the same sizes, in the second.
 	InverseRun run;
 	run.batch = ib.batch, run.sWs = sWs, run.sInv = ib.inverseStride, run.wsStrideBytes = ib.wsStrideBytes;
 	run.W = W, run.X = X, run.n = n, run.dInfo = dInfo, run.gws = gws, run.gBytes = gBytes;
-	run.T2 = inverse + ((size_t)n * n + 1) / 2;
 	{
 		size_t need[kMaxDepth] = {};
 		l21_sizes(blocks, n, 0, need);
 		size_t off = 0;
 		for (int d = 0; d < kMaxDepth; d++) {
 			run.L21[d] = inverse + off;
+			run.T2[d] = inverse + ((size_t)n * n + 1) / 2 + off;
 			off += (need[d] + 63) & ~(size_t)63;
 		}
-		FITRE_REQUIRE(off <= ((size_t)n * n + 1) / 2, "fitre_hip_spd_inverse: temporaries do not fit (order %d)", n);
+		FITRE_REQUIRE(off <= (size_t)n * n / 2, "fitre_hip_spd_inverse: temporaries do not fit (order %d)", n);
 	}
 	rc = chol_and_inverse(run, 0, blocks, n);
 	if (rc) return rc;

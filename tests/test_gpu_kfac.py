@@ -24,6 +24,15 @@ FACTOR_CASES = [
     (3, 5, 7, 9, 6, 3, 1, 1),       # rectangular
     (1, 1, 1, 5, 5, 3, 1, 0),       # degenerate
     (2, 7, 5, 7, 7, 1, 1, 0),       # 1x1 window: order 8
+    # small maps, channels in whole tiles: rows by tap over cell-major positions, reduction cut to the cells both taps see
+    (16, 128, 8, 4, 4, 3, 1, 1),    # order 1153
+    (16, 128, 8, 2, 2, 3, 1, 1),    # 2 x 2 map: opposite taps share no cell (zero tiles)
+    (32, 128, 8, 8, 8, 3, 1, 1),    # 8 x 8 map, split reduction
+    (16, 256, 8, 4, 4, 3, 1, 1),    # order 2305
+    (16, 128, 8, 4, 2, 3, 1, 1),    # rectangular map
+    (16, 128, 4, 4, 4, 5, 1, 2),    # 5 x 5 window: order 3201
+    (16, 128, 4, 6, 6, 3, 1, 0),    # no padding: every tap inside at every cell
+    (8, 128, 8, 4, 4, 3, 1, 1),     # eight images: not whole reduction slices per cell, plain rows
 ]
 
 
