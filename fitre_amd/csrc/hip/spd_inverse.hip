@@ -45,73 +45,70 @@ constexpr int kLeafLd = kLeaf + 1;
 // above the diagonal).  Returns the 1-based index inside the leaf of the first non-positive pivot of this sub-block,
 // or 0.
 //
-// Lane i holds row i of the block (a[]) and column i of the inverse in the making (y[], which starts as the unit
-// vector e_i and is forward-substituted column by column).  Step j scales column j, and then every later column k
-// takes a[k] -= a[j] * L[k][j] and y[k] -= y[j] * L[k][j]: the same scalar L[k][j] (lane k's a[j], through
-// v_readlane) serves the factorization and the inversion.  The scalars are fetched eight at a time ahead of their
-// sixteen multiply-adds: with one wave on the SIMD a multiply-add right behind its own v_readlane waits for it.
+// The lower half of the wave holds the block, lane i its row i; the upper half holds the inverse in the making, lane
+// 32 + i its column i, which starts as the unit vector e_i and is forward-substituted column by column.  Both live in the
+// SAME registers v[0..31] (one column each), because both take the same steps: step j scales column j, and then every
+// later column k takes v[k] -= v[j] * L[k][j] -- the factorization in the lower half, the substitution in the upper,
+// one multiply-add for the two -- with the scalar L[k][j] = lane k's v[j] fetched through v_readlane.  The scalars are
+// fetched eight at a time ahead of their eight multiply-adds: with one wave on the SIMD a multiply-add right behind its
+// own v_readlane waits for it.
 // columns K0 .. K0+7 (those below kSub) of step J
 template <int J, int K0>
-__device__ __forceinline__ void factor_update_group(float (&a)[kSub], float (&y)[kSub])
+__device__ __forceinline__ void factor_update_group(float (&v)[kSub])
 {
 	constexpr int N = (kSub - K0 < 8) ? (kSub - K0) : 8;
 	int s[N];
 #pragma unroll
-	for (int q = 0; q < N; q++) s[q] = __builtin_amdgcn_readlane(__float_as_int(a[J]), K0 + q);
+	for (int q = 0; q < N; q++) s[q] = __builtin_amdgcn_readlane(__float_as_int(v[J]), K0 + q);
 	// all lane reads of the group before its first multiply-add
 	if constexpr (N == 8)
 		asm volatile("" : "+s"(s[0]), "+s"(s[1]), "+s"(s[2]), "+s"(s[3]), "+s"(s[4]), "+s"(s[5]), "+s"(s[6]), "+s"(s[7]));
 #pragma unroll
-	for (int q = 0; q < N; q++) {
-		a[K0 + q] -= a[J] * __int_as_float(s[q]); // entries above the diagonal are never used
-		y[K0 + q] -= y[J] * __int_as_float(s[q]);
-	}
+	for (int q = 0; q < N; q++) v[K0 + q] -= v[J] * __int_as_float(s[q]); // entries above the diagonal are never used
 	// the updates stay in this step: left to itself the compiler postpones each until column k is needed and keeps
 	// the 496 scalars alive (spilled) until then
 	if constexpr (N == 8) {
-		asm volatile("" : "+v"(a[K0]), "+v"(a[K0 + 1]), "+v"(a[K0 + 2]), "+v"(a[K0 + 3]), "+v"(a[K0 + 4]), "+v"(a[K0 + 5]),
-		             "+v"(a[K0 + 6]), "+v"(a[K0 + 7]));
-		asm volatile("" : "+v"(y[K0]), "+v"(y[K0 + 1]), "+v"(y[K0 + 2]), "+v"(y[K0 + 3]), "+v"(y[K0 + 4]), "+v"(y[K0 + 5]),
-		             "+v"(y[K0 + 6]), "+v"(y[K0 + 7]));
+		asm volatile("" : "+v"(v[K0]), "+v"(v[K0 + 1]), "+v"(v[K0 + 2]), "+v"(v[K0 + 3]), "+v"(v[K0 + 4]), "+v"(v[K0 + 5]),
+		             "+v"(v[K0 + 6]), "+v"(v[K0 + 7]));
 	} else {
 #pragma unroll
-		for (int q = 0; q < N; q++) asm volatile("" : "+v"(a[K0 + q]), "+v"(y[K0 + q]));
+		for (int q = 0; q < N; q++) asm volatile("" : "+v"(v[K0 + q]));
 	}
-	if constexpr (K0 + 8 < kSub) factor_update_group<J, K0 + 8>(a, y);
+	if constexpr (K0 + 8 < kSub) factor_update_group<J, K0 + 8>(v);
 }
 
 // steps J .. kSub-1; first: base of the 1-based pivot numbering
 template <int J>
-__device__ __forceinline__ void factor_steps(float (&a)[kSub], float (&y)[kSub], int first, int &bad)
+__device__ __forceinline__ void factor_steps(float (&v)[kSub], int first, int &bad)
 {
-	const float ajj = lane_value(a[J], J);
+	const float ajj = lane_value(v[J], J);
 	if (!(ajj > 0.f) && bad == 0) bad = first + J + 1;
 	const float d = rsqrtf(ajj);
-	a[J] *= d; // column J of L; lane J's own entry becomes ajj / sqrt(ajj), the diagonal
-	y[J] *= d; // row J of the inverse is complete
+	v[J] *= d; // column J of L (lane J's own entry becomes ajj / sqrt(ajj), the diagonal); row J of the inverse is complete
 	if constexpr (J + 1 < kSub) {
-		factor_update_group<J, J + 1>(a, y);
-		factor_steps<J + 1>(a, y, first, bad);
+		factor_update_group<J, J + 1>(v);
+		factor_steps<J + 1>(v, first, bad);
 	}
 }
 
 __device__ __forceinline__ int factor_sub_block(float *Ms, int kb, int lane)
 {
 	const int i = lane & (kSub - 1);
+	const bool inverseHalf = lane >= kSub;
 	float *wb = Ms + (kb * kSub) * kLeafLd + kb * kSub;
-	float a[kSub], y[kSub];
+	float v[kSub];
 #pragma unroll
 	for (int j = 0; j < kSub; j++) {
-		a[j] = wb[j * kLeafLd + i];
-		y[j] = (i == j) ? 1.f : 0.f;
+		const float a = wb[j * kLeafLd + i];
+		v[j] = inverseHalf ? ((i == j) ? 1.f : 0.f) : a;
 	}
 	int bad = 0;
-	factor_steps<0>(a, y, kb * kSub, bad);
-	// y[r] is element (r, i) of the inverse: this lane holds column i.  The inverse replaces the block: nothing reads
-	// a diagonal sub-block of the factor itself again.
-	if (lane < kSub) {
+	factor_steps<0>(v, kb * kSub, bad);
+	// in the upper half v[r] is element (r, i) of the inverse: the lane holds column i.  The inverse replaces the block:
+	// nothing reads a diagonal sub-block of the factor itself again.
+	if (inverseHalf) {
 #pragma unroll
-		for (int j = 0; j < kSub; j++) wb[i * kLeafLd + j] = y[j];
+		for (int j = 0; j < kSub; j++) wb[i * kLeafLd + j] = v[j];
 	}
 	return bad;
 }
