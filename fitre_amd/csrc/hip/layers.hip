@@ -899,35 +899,49 @@ __device__ __forceinline__ float4 route2x2(float4 r, float d)
 
 // delta given as `splits` slabs `stride` floats apart: their sum in slab order, accumulated in double
 // (what the split-K reduction kernel would have written)
-__device__ __forceinline__ float4 load_sum4(const float *p, int splits, long stride)
+// (four slabs are read before the first of them is added: a loop that adds each slab as it arrives pays one memory
+// latency per slab)
+template <class T>
+__device__ __forceinline__ void add_in_double(double (&a)[sizeof(T) / sizeof(float)], const T &t)
 {
-	float4 t = *reinterpret_cast<const float4 *>(p);
-	if (splits == 1) return t;
-	double a0 = t.x, a1 = t.y, a2 = t.z, a3 = t.w;
-	for (int s = 1; s < splits; s++) {
-		t = *reinterpret_cast<const float4 *>(p + (size_t)s * stride);
-		a0 += (double)t.x, a1 += (double)t.y, a2 += (double)t.z, a3 += (double)t.w;
+	const float *f = reinterpret_cast<const float *>(&t);
+#pragma unroll
+	for (int v = 0; v < (int)(sizeof(T) / sizeof(float)); v++) a[v] += (double)f[v];
+}
+template <class T>
+__device__ __forceinline__ T load_sum_groups(const float *p, int splits, long stride)
+{
+	constexpr int V = sizeof(T) / sizeof(float);
+	if (splits == 1) return *reinterpret_cast<const T *>(p);
+	double a[V];
+#pragma unroll
+	for (int v = 0; v < V; v++) a[v] = 0.0;
+	int s = 0;
+	for (; s + 4 <= splits; s += 4) {
+		T t[4];
+#pragma unroll
+		for (int u = 0; u < 4; u++) t[u] = *reinterpret_cast<const T *>(p + (size_t)(s + u) * stride);
+#pragma unroll
+		for (int u = 0; u < 4; u++) add_in_double<T>(a, t[u]);
 	}
-	return make_float4((float)a0, (float)a1, (float)a2, (float)a3);
-}
-__device__ __forceinline__ float2 load_sum2(const float *p, int splits, long stride)
-{
-	float2 t = *reinterpret_cast<const float2 *>(p);
-	if (splits == 1) return t;
-	double a0 = t.x, a1 = t.y;
-	for (int s = 1; s < splits; s++) {
-		t = *reinterpret_cast<const float2 *>(p + (size_t)s * stride);
-		a0 += (double)t.x, a1 += (double)t.y;
+	if (s + 2 <= splits) {
+		T t[2];
+#pragma unroll
+		for (int u = 0; u < 2; u++) t[u] = *reinterpret_cast<const T *>(p + (size_t)(s + u) * stride);
+#pragma unroll
+		for (int u = 0; u < 2; u++) add_in_double<T>(a, t[u]);
+		s += 2;
 	}
-	return make_float2((float)a0, (float)a1);
+	if (s < splits) add_in_double<T>(a, *reinterpret_cast<const T *>(p + (size_t)s * stride));
+	T r;
+	float *f = reinterpret_cast<float *>(&r);
+#pragma unroll
+	for (int v = 0; v < V; v++) f[v] = (float)a[v];
+	return r;
 }
-__device__ __forceinline__ float load_sum1(const float *p, int splits, long stride)
-{
-	if (splits == 1) return *p;
-	double a = 0.0;
-	for (int s = 0; s < splits; s++) a += (double)p[(size_t)s * stride];
-	return (float)a;
-}
+__device__ __forceinline__ float4 load_sum4(const float *p, int splits, long stride) { return load_sum_groups<float4>(p, splits, stride); }
+__device__ __forceinline__ float2 load_sum2(const float *p, int splits, long stride) { return load_sum_groups<float2>(p, splits, stride); }
+__device__ __forceinline__ float load_sum1(const float *p, int splits, long stride) { return load_sum_groups<float>(p, splits, stride); }
 // slab 0 += the other slabs (same order and precision)
 __global__ void __launch_bounds__(256) sum_slabs_kernel(float *base, int splits, long stride, long n)
 {
