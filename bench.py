@@ -68,9 +68,16 @@ def measured_traffic(kernel):
 def tree_commit():
     import subprocess
     try:
-        return subprocess.run(["git", "-C", ROOT, "rev-parse", "--short", "HEAD"], stdout=subprocess.PIPE,
-                              stderr=subprocess.DEVNULL, text=True, timeout=10).stdout.strip() or None
+        rev = subprocess.run(["git", "-C", ROOT, "rev-parse", "--short", "HEAD"], stdout=subprocess.PIPE,
+                             stderr=subprocess.DEVNULL, text=True, timeout=10).stdout.strip()
     except (OSError, subprocess.SubprocessError):
+        rev = ""
+    if rev:
+        return rev
+    try:  # a copy of the tree without its history: the commit the build step noted
+        with open(os.path.join(ROOT, "fitre_amd", "BUILD_TREE")) as f:
+            return f.read().strip() or None
+    except OSError:
         return None
 
 

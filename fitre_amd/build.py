@@ -76,9 +76,25 @@ def build_host(verbose=True):
     return CNN_LIB
 
 
+def stamp_tree():
+    """Notes the commit the libraries are built from (fitre_amd/BUILD_TREE, a '+' behind it when the tree has changes
+    that are not committed): what bench.py reports where the tree travels without its history."""
+    try:
+        rev = subprocess.run(["git", "-C", ROOT, "rev-parse", "--short", "HEAD"], stdout=subprocess.PIPE, stderr=subprocess.DEVNULL,
+                             text=True, timeout=10).stdout.strip()
+        dirty = subprocess.run(["git", "-C", ROOT, "status", "--porcelain", "--untracked-files=no"], stdout=subprocess.PIPE,
+                               stderr=subprocess.DEVNULL, text=True, timeout=10).stdout.strip()
+    except (OSError, subprocess.SubprocessError):
+        return
+    if rev:
+        with open(os.path.join(PKG, "BUILD_TREE"), "w") as f:
+            f.write(rev + ("+" if dirty else "") + "\n")
+
+
 def build_all(verbose=True):
     build_hip(verbose)
     build_host(verbose)
+    stamp_tree()
     return HIP_LIB, CNN_LIB
 
 
