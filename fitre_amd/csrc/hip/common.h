@@ -31,8 +31,8 @@ int gemm_ex_batched(int batch, int transA, int transB, int M, int N, int K, floa
                     const float *B, int ldb, long strideB, float beta, float *C, int ldc, long strideC, int flags, int kernelClass,
                     void *ws, size_t wsBytes, long wsStrideBytes);
 // One argument set of gemm_ex_batched; gemm_pair_batched queues two such products that do not depend on each other --
-// as ONE launch when both run unsplit on the same tile (the chip then sees the tiles of both at once, and a chain of
-// dependent launches is one launch shorter), as two launches otherwise.
+// as ONE launch when both are small enough to run unsplit on the deep 64 x 64 tile (a chain of dependent launches is then
+// one launch shorter), as two launches otherwise.
 struct BatchedProduct {
 	int transA, transB, M, N, K;
 	float alpha;

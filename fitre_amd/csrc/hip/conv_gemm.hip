@@ -497,9 +497,10 @@ int gemm_pair_batched(int batch, const BatchedProduct &f, const BatchedProduct &
 	rc = batched_check("gemm_pair_batched", batch, g.transA, g.transB, g.M, g.N, g.K, g.A, g.lda, g.B, g.ldb, g.C, g.ldc, g.flags, wsStrideBytes);
 	if (rc) return rc;
 	const GemmPlan pf = batched_plan(batch, f.N, f.M, f.K, f.flags), pg = batched_plan(batch, g.N, g.M, g.K, g.flags);
-	const bool oneLaunch = pf.splits == 1 && pg.splits == 1 && pf.bk == pg.bk && pf.bm == pg.bm && pf.bn == pg.bn && pf.bm == pf.bn &&
-	                       ((pf.bk == kGemmDeepBK && pf.bm == 64) || (pf.bk == kGemmBK && pf.bm == 128)) && !f.transA && f.transB &&
-	                       !g.transA && !g.transB;
+	// one launch where both run unsplit on the deep 64 x 64 tile (every node of the inverse's recursion below order 1280
+	// resp. 384); larger products each fill the chip, or split their reduction, and are queued one after the other
+	const bool oneLaunch = pf.splits == 1 && pg.splits == 1 && pf.bk == kGemmDeepBK && pg.bk == kGemmDeepBK && pf.bm == 64 && pf.bn == 64 &&
+	                       pg.bm == 64 && pg.bn == 64 && !f.transA && f.transB && !g.transA && !g.transB;
 	if (!oneLaunch) {
 		rc = gemm_ex_batched(batch, f.transA, f.transB, f.M, f.N, f.K, f.alpha, f.A, f.lda, f.strideA, f.B, f.ldb, f.strideB, f.beta, f.C, f.ldc,
 		                     f.strideC, f.flags, kernelClass, ws, wsBytes, wsStrideBytes);
@@ -508,9 +509,7 @@ int gemm_pair_batched(int batch, const BatchedProduct &f, const BatchedProduct &
 		                       g.ldc, g.strideC, g.flags, kernelClass, ws, wsBytes, wsStrideBytes);
 	}
 	const double flops = (2.0 * (double)f.M * f.N * f.K + 2.0 * (double)g.M * g.N * g.K) * batch;
-	if (pf.bk == kGemmDeepBK)
-		return launch_pair<TileCfg<64, 64, kGemmDeepBK> >(batch, pair_side(f, 64, 64), pair_side(g, 64, 64), kernelClass, flops, 1);
-	return launch_pair<TileCfg<128, 128, kGemmBK> >(batch, pair_side(f, 128, 128), pair_side(g, 128, 128), kernelClass, flops, 4);
+	return launch_pair<TileCfg<64, 64, kGemmDeepBK> >(batch, pair_side(f, 64, 64), pair_side(g, 64, 64), kernelClass, flops, 1);
 }
 
 
