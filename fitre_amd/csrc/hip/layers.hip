@@ -726,6 +726,120 @@ bn_normalize_kernel(const float *x, const float *mean, const float *variance, fl
 	}
 }
 
+// the activation functions, as fitre_hip_activation_forward evaluates them
+__device__ __forceinline__ float act_forward_value(int actFun, float x)
+{
+	switch (actFun) {
+	case CNN_ACT_RELU: return x < 0.f ? 0.f : x;
+	case CNN_ACT_SOFTPLUS: return x < 20.f ? logf(1.f + expf(x)) : x;
+	case CNN_ACT_ELU: return x < 0.f ? (expf(x) - 1.f) : x;
+	case CNN_ACT_SWISH: return x / (1.f + expf(-x));
+	case ACT_LOGISTIC: return 1.f / (1.f + expf(-x));
+	case ACT_TANH: return tanhf(x);
+	default: return x;
+	}
+}
+__device__ __forceinline__ float4 act_forward4(int actFun, float4 v)
+{
+	return make_float4(act_forward_value(actFun, v.x), act_forward_value(actFun, v.y), act_forward_value(actFun, v.z),
+	                   act_forward_value(actFun, v.w));
+}
+// strict-> scan of a 2 x 2 window in memory order, as the pooling kernels scan it
+__device__ __forceinline__ float max2x2(float v0, float v1, float v2, float v3)
+{
+	float best = -FLT_MAX;
+	if (v0 > best) best = v0;
+	if (v1 > best) best = v1;
+	if (v2 > best) best = v2;
+	if (v3 > best) best = v3;
+	return best;
+}
+
+// Normalisation, activation and 2x2 / stride 2 max pooling of a layer in one pass over its convolution output: x is
+// read once and zhat, the activation output and the pooled output are written (the three separate passes read four
+// tensors for the same three results).  One (channel, segment) per workgroup.  `partial`: the per-segment sums of x and
+// x^2 of channel_partial_kernel<2> (segmentsIn per channel) -- every workgroup of a channel adds them up in the same
+// order, the first one also stores the statistics; null: statMean / statVar hold the statistics to use.  zhat null: no
+// normalisation (x goes into the activation as it is).  POOL 0: the unit of work is a 2 x 4 patch (B % 4 == 0, A even);
+// POOL 2: no pooling, the unit is a 16-byte group.
+template <int POOL>
+__global__ void __launch_bounds__(kRedBlock)
+bn_act_pool_forward_kernel(const float *x, const double *partial, int segmentsIn, float momentum, float *mean, float *variance,
+                           float *runMean, float *runVar, const float *statMean, const float *statVar, float epsilon, int samples,
+                           int inA, int inB, int actFun, float *zhat, float *actOut, float *poolOut)
+{
+	const int c = blockIdx.y;
+	const long perChannel = (long)samples * inA * inB;
+	float mu = 0.f, inv = 1.f;
+	if (zhat) {
+		float var;
+		if (partial) {
+			double s = 0.0, ss = 0.0;
+			for (int k = 0; k < segmentsIn; k++) {
+				s += partial[((size_t)c * segmentsIn + k) * 2];
+				ss += partial[((size_t)c * segmentsIn + k) * 2 + 1];
+			}
+			const double m = s / (double)perChannel;
+			double v = ss / (double)perChannel - m * m;
+			if (v < 0.0) v = 0.0;
+			mu = (float)m;
+			var = (float)v;
+			if (blockIdx.x == 0 && threadIdx.x == 0) {
+				mean[c] = mu;
+				variance[c] = var;
+				runMean[c] = momentum * runMean[c] + (1.f - momentum) * mu;
+				runVar[c] = momentum * runVar[c] + (1.f - momentum) * var;
+			}
+		} else {
+			mu = statMean[c];
+			var = statVar[c];
+		}
+		inv = 1.f / sqrtf(var + epsilon);
+	}
+	const size_t base = (size_t)c * perChannel;
+	if constexpr (POOL == 2) {
+		const long groups = perChannel / 4;
+		const long per = (groups + gridDim.x - 1) / gridDim.x;
+		const long lo = (long)blockIdx.x * per;
+		const long hi = (lo + per < groups) ? lo + per : groups;
+		for (long i = lo + threadIdx.x; i < hi; i += kRedBlock) {
+			float4 a = *reinterpret_cast<const float4 *>(x + base + 4 * i);
+			if (zhat) {
+				a.x = (a.x - mu) * inv, a.y = (a.y - mu) * inv, a.z = (a.z - mu) * inv, a.w = (a.w - mu) * inv;
+				*reinterpret_cast<float4 *>(zhat + base + 4 * i) = a;
+			}
+			*reinterpret_cast<float4 *>(actOut + base + 4 * i) = act_forward4(actFun, a);
+		}
+	} else {
+		const int outB2 = inB / 4, outA = inA / 2, outB = inB / 2;
+		const int perMap = outA * outB2;
+		const long patches = (long)samples * perMap;
+		const long per = (patches + gridDim.x - 1) / gridDim.x;
+		const long lo = (long)blockIdx.x * per;
+		const long hi = (lo + per < patches) ? lo + per : patches;
+		const size_t pBase = (size_t)c * samples * outA * outB;
+		for (long i = lo + threadIdx.x; i < hi; i += kRedBlock) {
+			const long map = i / perMap;
+			const int rem = (int)(i - map * perMap);
+			const int oa = rem / outB2, pb = rem - oa * outB2;
+			const size_t in = base + (size_t)map * inA * inB + (size_t)(2 * oa) * inB + 4 * pb;
+			float4 a0 = *reinterpret_cast<const float4 *>(x + in);
+			float4 a1 = *reinterpret_cast<const float4 *>(x + in + inB);
+			if (zhat) {
+				a0.x = (a0.x - mu) * inv, a0.y = (a0.y - mu) * inv, a0.z = (a0.z - mu) * inv, a0.w = (a0.w - mu) * inv;
+				a1.x = (a1.x - mu) * inv, a1.y = (a1.y - mu) * inv, a1.z = (a1.z - mu) * inv, a1.w = (a1.w - mu) * inv;
+				*reinterpret_cast<float4 *>(zhat + in) = a0;
+				*reinterpret_cast<float4 *>(zhat + in + inB) = a1;
+			}
+			const float4 r0 = act_forward4(actFun, a0), r1 = act_forward4(actFun, a1);
+			*reinterpret_cast<float4 *>(actOut + in) = r0;
+			*reinterpret_cast<float4 *>(actOut + in + inB) = r1;
+			*reinterpret_cast<float2 *>(poolOut + pBase + (size_t)map * outA * outB + (size_t)oa * outB + 2 * pb) =
+			    make_float2(max2x2(r0.x, r0.y, r1.x, r1.y), max2x2(r0.z, r0.w, r1.z, r1.w));
+		}
+	}
+}
+
 // dx_i = (m*delta_i - sum(delta) - zhat_i * sum(delta*zhat)) / (m * sqrt(var + eps)), and its channel sum
 // (the bias gradient) in closed form: -sum(delta*zhat) * sum(zhat) / (m * sqrt(var + eps)).
 __device__ __forceinline__ float bn_backward_value(float m, float d, float z, float sum1, float sum2, float scale)
@@ -1576,6 +1690,60 @@ int fitre_hip_batch_norm_forward(const float *in, int channels, long perChannel,
 	else
 		bn_normalize_kernel<false><<<grid, kRedBlock, 0, stream()>>>(in, mu, var, epsilon, perChannel, zhat);
 	return check_launch("batch_norm_forward");
+}
+
+int fitre_hip_bn_act_pool_forward(const float *in, int channels, int samples, int inA, int inB, float *zhat, float *mean,
+                                  float *variance, float *runningMean, float *runningVariance, float epsilon, float momentum,
+                                  int train, int actFun, float *actOut, int poolType, int ksize, int stride, int padding, int outA,
+                                  int outB, float *poolOut, void *ws, size_t wsBytes)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(in && actOut, "fitre_hip_bn_act_pool_forward: null pointer");
+	FITRE_REQUIRE(!zhat || (mean && variance && runningMean && runningVariance), "fitre_hip_bn_act_pool_forward: null statistics");
+	FITRE_REQUIRE(poolType == NO_POOL || poolOut, "fitre_hip_bn_act_pool_forward: null pooled output");
+	FITRE_REQUIRE(act_known(actFun), "fitre_hip_bn_act_pool_forward: unknown activation code %d", actFun);
+	FITRE_REQUIRE(channels > 0 && samples > 0 && inA > 0 && inB > 0, "fitre_hip_bn_act_pool_forward: non-positive shape");
+	const long perChannel = (long)samples * inA * inB, count = perChannel * channels;
+	int rc;
+	if (zhat) {
+		rc = check_channels("fitre_hip_bn_act_pool_forward", channels, perChannel, ws, wsBytes);
+		if (rc) return rc;
+	}
+	const bool pool2 = poolType == MAX_POOL && ksize == 2 && stride == 2 && padding == 0 && inB % 4 == 0 && inA % 2 == 0 &&
+	                   outA == inA / 2 && outB == inB / 2 && (((uintptr_t)poolOut) & 7) == 0;
+	const bool fused = (poolType == NO_POOL || pool2) && perChannel % 4 == 0 && channels <= 65535 && aligned16(in) && aligned16(actOut) &&
+	                   (!zhat || aligned16(zhat));
+	if (!fused) {
+		const float *actIn = in;
+		if (zhat) {
+			rc = fitre_hip_batch_norm_forward(in, channels, perChannel, zhat, mean, variance, runningMean, runningVariance, epsilon, momentum,
+			                                  train, ws, wsBytes);
+			if (rc) return rc;
+			actIn = zhat;
+		}
+		rc = fitre_hip_activation_forward(actFun, actIn, actOut, count);
+		if (rc || poolType == NO_POOL) return rc;
+		return fitre_hip_pool_forward(poolType, actOut, channels, samples, inA, inB, ksize, stride, padding, outA, outB, poolOut);
+	}
+	const int S = segments_for(channels, perChannel);
+	double *partial = nullptr;
+	const dim3 grid(S, channels);
+	if (zhat && train) {
+		partial = (double *)ws;
+		LaunchScope scope(FITRE_KC_BN_FWD, 4.0 * (double)count);
+		channel_partial_kernel<2, true><<<grid, kRedBlock, 0, stream()>>>(in, nullptr, perChannel, partial);
+	}
+	const double moved = 4.0 * (double)count * (zhat ? 3 : 2) + (poolType == NO_POOL ? 0.0 : (double)count);
+	LaunchScope scope(zhat ? FITRE_KC_BN_FWD : FITRE_KC_ACT_FWD, moved);
+	if (poolType == NO_POOL)
+		bn_act_pool_forward_kernel<2><<<grid, kRedBlock, 0, stream()>>>(in, partial, S, momentum, mean, variance, runningMean, runningVariance,
+		                                                                runningMean, runningVariance, epsilon, samples, inA, inB, actFun,
+		                                                                zhat, actOut, poolOut);
+	else
+		bn_act_pool_forward_kernel<0><<<grid, kRedBlock, 0, stream()>>>(in, partial, S, momentum, mean, variance, runningMean, runningVariance,
+		                                                                runningMean, runningVariance, epsilon, samples, inA, inB, actFun,
+		                                                                zhat, actOut, poolOut);
+	return check_launch("bn_act_pool_forward_kernel");
 }
 
 // The launches of the stand-alone batch-norm backward step; `partial` holds the per-(channel, segment) sums.

@@ -194,26 +194,22 @@ real cnnForward(CNN_MODEL *model, DEVICE_DATASET *data, SCRATCH_AREA *scratch, r
 		const real *in = (l == 0) ? data->currentBatch : z + zOffsets[l] + model->convLayer[l - 1].outputOffset;
 		real *slab = z + zOffsets[l + 1];
 		real *actOut = slab + cv->activationOffset;
-		const long perChannel = (long)n * cv->outWidth * cv->outHeight;
-		const long count = perChannel * cv->outChannels;
 		fitre_conv_shape shape = conv_shape(cv, n);
 
 		HIP_CALL(fitre_hip_conv_forward(&shape, in, weights + wOffsets[l],
 		                                (model->bias == 0) ? NULL : weights + bOffsets[l], slab, ws, wsBytes));
-		if (has_bn(cv)) {
-			real *bnOut = slab + cv->batchNormOffset;
-			HIP_CALL(fitre_hip_batch_norm_forward(slab, cv->outChannels, perChannel, bnOut, bnOut + cv->meansOffset,
-			                                      bnOut + cv->variancesOffset, bnOut + cv->runningMeansOffset,
-			                                      bnOut + cv->runningVariancesOffset, (real)BATCH_NORM_EPSILON,
-			                                      (real)BATCH_NORM_MOMENTUM, forTesting == MODEL_TRAIN, ws, wsBytes));
-			HIP_CALL(fitre_hip_activation_forward(model->actFuns[l], bnOut, actOut, count));
-		} else {
-			HIP_CALL(fitre_hip_activation_forward(model->actFuns[l], slab, actOut, count));
+		/* batch norm (where the layer has it), activation and pooling: one pass over the convolution output where the
+		 * shapes allow, the separate passes otherwise */
+		{
+			real *bnOut = has_bn(cv) ? slab + cv->batchNormOffset : NULL;
+			const int pooled = pl->type != NO_POOL;
+			HIP_CALL(fitre_hip_bn_act_pool_forward(
+			    slab, cv->outChannels, n, pooled ? pl->width : cv->outWidth, pooled ? pl->height : cv->outHeight, bnOut,
+			    bnOut ? bnOut + cv->meansOffset : NULL, bnOut ? bnOut + cv->variancesOffset : NULL,
+			    bnOut ? bnOut + cv->runningMeansOffset : NULL, bnOut ? bnOut + cv->runningVariancesOffset : NULL,
+			    (real)BATCH_NORM_EPSILON, (real)BATCH_NORM_MOMENTUM, forTesting == MODEL_TRAIN, model->actFuns[l], actOut, pl->type,
+			    pl->pSize, pl->stride, pl->padding, pl->outWidth, pl->outHeight, pooled ? slab + cv->poolOffset : NULL, ws, wsBytes));
 		}
-		if (pl->type != NO_POOL)
-			HIP_CALL(fitre_hip_pool_forward(pl->type, actOut, cv->outChannels, n, pl->width, pl->height, pl->pSize,
-			                                pl->stride, pl->padding, pl->outWidth, pl->outHeight,
-			                                slab + cv->poolOffset));
 	}
 
 	/* [C][N][a*B+b] -> [N][C][b*A+a], in place through the workspace */

@@ -87,6 +87,8 @@ HIP_API = {
     "fitre_hip_shift_images": (i32, [vp, i32, i32, i32, i32, vp, vp, f32, vp]),
     "fitre_hip_batch_norm_workspace": (sz, [i32, lng]),
     "fitre_hip_batch_norm_forward": (i32, [vp, i32, lng, vp, vp, vp, vp, vp, f32, f32, i32, vp, sz]),
+    "fitre_hip_bn_act_pool_forward": (i32, [vp, i32, i32, i32, i32, vp, vp, vp, vp, vp, f32, f32, i32, i32, vp, i32, i32, i32, i32, i32,
+                                            i32, vp, vp, sz]),
     "fitre_hip_batch_norm_backward": (i32, [vp, vp, vp, i32, lng, f32, vp, vp, vp, sz]),
     "fitre_hip_batch_norm_backward_static": (i32, [vp, vp, vp, i32, lng, f32, vp, vp]),
     "fitre_hip_channel_sum_workspace": (sz, [i32, lng]),

@@ -205,6 +205,18 @@ size_t fitre_hip_batch_norm_workspace(int channels, long perChannel);
 int fitre_hip_batch_norm_forward(const float *in, int channels, long perChannel, float *zhat, float *mean,
                                  float *variance, float *runningMean, float *runningVariance,
                                  float epsilon, float momentum, int train, void *ws, size_t wsBytes);
+/* fitre_hip_batch_norm_forward, fitre_hip_activation_forward of its zhat and fitre_hip_pool_forward of that, as the
+ * forward pass runs them for a convolution layer (functions/cnn_forward.cu:124-205): after the statistics, ONE pass
+ * reads the convolution output and writes zhat, the activation output and the pooled output (the three passes read
+ * four tensors for the same results; the values are the same bit for bit).  zhat NULL: a layer without batch norm, `in`
+ * goes into the activation as it is (the statistics pointers are not used).  poolType NO_POOL: poolOut and the
+ * window arguments are not used.  Fused for no pooling and for 2x2 / stride 2 max pooling (A even, B a multiple of 4,
+ * 16-byte-aligned tensors); every other case runs the separate passes.  Workspace (with batch norm):
+ * fitre_hip_batch_norm_workspace(channels, samples * inA * inB). */
+int fitre_hip_bn_act_pool_forward(const float *in, int channels, int samples, int inA, int inB, float *zhat, float *mean,
+                                  float *variance, float *runningMean, float *runningVariance, float epsilon,
+                                  float momentum, int train, int actFun, float *actOut, int poolType, int ksize,
+                                  int stride, int padding, int outA, int outB, float *poolOut, void *ws, size_t wsBytes);
 /* out = (m*delta - sum(delta) - zhat*sum(delta*zhat)) / (m*sqrt(eps+var)), m = perChannel.  :550-621.
  * biasGrad (may be NULL) receives the per-channel sum of out. */
 int fitre_hip_batch_norm_backward(const float *delta, const float *zhat, const float *variance,

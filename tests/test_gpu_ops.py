@@ -309,6 +309,60 @@ FUSED_BN_GEOMS = [
 ]
 
 
+@pytest.mark.parametrize("bn,train", [(True, 1), (True, 0), (False, 1)])
+@pytest.mark.parametrize("act", [CNN_ACT_RELU, CNN_ACT_SWISH])
+@pytest.mark.parametrize("kind", [MAX_POOL, NO_POOL])
+@pytest.mark.parametrize("geom", FUSED_BN_GEOMS)
+def test_fused_batch_norm_activation_pool_forward(dev, oracle64, geom, kind, act, bn, train):
+    """One call for the normalisation, activation and pooling of a layer's convolution output against the three
+    separate entry points on the same input: the same bits in every output (fused shapes and the ones that fall back
+    alike), the statistics to rounding, and zhat against the oracle."""
+    Cn, N, A, B, k, s, p = geom
+    oA, oB = (A + 2 * p - k) // s + 1, (B + 2 * p - k) // s + 1
+    per = N * A * B
+    rng = np.random.default_rng(Cn * 7 + N + A * B)
+    x = (rng.standard_normal(Cn * per) * 1.3 + 0.2).astype(np.float32)
+    px = dev.upload(x)
+    ws, nb = bn_ws(dev, Cn, per)
+    running = np.concatenate([np.zeros(2 * Cn), np.full(Cn, 0.25), np.full(Cn, 1.5)]).astype(np.float32)
+    pooled = Cn * N * oA * oB
+
+    def separate():
+        stats = dev.upload(running)
+        mean, var, rmean, rvar = (at(stats, i * Cn) for i in range(4))
+        zh, ao, po = dev.zeros(Cn * per), dev.zeros(Cn * per), dev.zeros(pooled)
+        src = px
+        if bn:
+            ok(hip.fitre_hip_batch_norm_forward(px, Cn, per, zh, mean, var, rmean, rvar, 1e-5, 0.9, train, ws, nb))
+            src = zh
+        ok(hip.fitre_hip_activation_forward(act, src, ao, Cn * per))
+        if kind != NO_POOL:
+            ok(hip.fitre_hip_pool_forward(kind, ao, Cn, N, A, B, k, s, p, oA, oB, po))
+        return [dev.download(b, n) for b, n in ((zh, Cn * per), (ao, Cn * per), (po, pooled), (stats, 4 * Cn))]
+
+    def fused():
+        stats = dev.upload(running)
+        mean, var, rmean, rvar = (at(stats, i * Cn) for i in range(4))
+        zh, ao, po = dev.zeros(Cn * per), dev.zeros(Cn * per), dev.zeros(pooled)
+        ok(hip.fitre_hip_bn_act_pool_forward(px, Cn, N, A, B, zh if bn else None, mean if bn else None, var if bn else None,
+                                             rmean if bn else None, rvar if bn else None, 1e-5, 0.9, train, act, ao, kind, k, s, p,
+                                             oA, oB, po if kind != NO_POOL else None, ws, nb))
+        return [dev.download(b, n) for b, n in ((zh, Cn * per), (ao, Cn * per), (po, pooled), (stats, 4 * Cn))]
+
+    want, got = separate(), fused()
+    np.testing.assert_allclose(got[3], want[3], rtol=1e-6, atol=1e-7)
+    if np.array_equal(got[3], want[3]):            # the same statistics to the bit: so is everything made from them
+        for g, w in zip(got[:3], want[:3]):
+            np.testing.assert_array_equal(g, w)
+    else:
+        for g, w in zip(got[:3], want[:3]):
+            assert rel_err(g, w) < 1e-6
+    if bn and train:
+        zhat, *_ = oracle64.batch_norm_forward(x, B, A, Cn, N, running=(np.full(Cn, 0.25), np.full(Cn, 1.5)))
+        assert rel_err(got[0], zhat) < 1e-5
+    dev.free(ws)
+
+
 @pytest.mark.parametrize("geom", FUSED_BN_GEOMS)
 @pytest.mark.parametrize("act,derive,slabs", [(CNN_ACT_RELU, True, 1), (CNN_ACT_RELU, False, 1), (CNN_ACT_SWISH, False, 1),
                                               (CNN_ACT_RELU, True, 3), (CNN_ACT_SWISH, False, 8)])
