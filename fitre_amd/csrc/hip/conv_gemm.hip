@@ -696,7 +696,10 @@ int fitre_hip_conv_pair_supported(const fitre_conv_shape *s, int kind)
 size_t fitre_hip_conv_pair_workspace(const fitre_conv_shape *s, int kind)
 {
 	if (!fitre_hip_conv_pair_supported(s, kind)) return 0;
-	if (kind == 2) return c3_dw_workspace(s, 2);
+	if (kind == 2) {
+		const size_t nine = c3_dw_workspace(s, 2), dense = quad_eligible(s) ? quad_weight_grad_workspace(s) : 0;
+		return nine > dense ? nine : dense;
+	}
 	return c3_pos_workspace(s, kind == 1, 2);
 }
 
@@ -731,6 +734,10 @@ int fitre_hip_conv_weight_grad_pair(const fitre_conv_shape *s, const float *x1, 
 	if (rc) return rc;
 	FITRE_REQUIRE(x1 && delta1 && x2 && delta2 && dW, "fitre_hip_conv_weight_grad_pair: null pointer");
 	if (!c3_dw_eligible(s)) return fail(FITRE_E_UNSUPPORTED, "fitre_hip_conv_weight_grad_pair: shape outside the 3x3 weight-gradient kernel");
+	// 2 x 2 maps: the two dense products into one buffer, folded once
+	if (quad_usable(s, ws, wsBytes, quad_weight_grad_workspace(s)) &&
+	    (((((uintptr_t)x1) | ((uintptr_t)delta1) | ((uintptr_t)x2) | ((uintptr_t)delta2)) & 15) == 0))
+		return quad_weight_grad(s, x1, delta1, dW, ws, wsBytes, x2, delta2);
 	return launch_c3_dw(s, x1, delta1, dW, ws, wsBytes, x2, delta2);
 }
 

@@ -304,7 +304,9 @@ static int quad_input_grad(const fitre_conv_shape *s, const float *delta, const 
 }
 
 // dW[co][ci][3][3] from x[ci][n][a'b'] and delta[co][n][ab].  ws: [dWeff | split partials].
-static int quad_weight_grad(const fitre_conv_shape *s, const float *x, const float *delta, float *dW, void *ws, size_t wsBytes)
+// x2 / delta2: a second (input, delta) pair whose product is added before the fold (the R operator's sums of two products)
+static int quad_weight_grad(const fitre_conv_shape *s, const float *x, const float *delta, float *dW, void *ws, size_t wsBytes,
+                            const float *x2 = nullptr, const float *delta2 = nullptr)
 {
 	const int cin = s->inChannels, cout = s->outChannels, N = s->samples;
 	const size_t weffBytes = quad_weff_bytes(s);
@@ -319,6 +321,12 @@ static int quad_weight_grad(const fitre_conv_shape *s, const float *x, const flo
 	OutParams out{ dweff, (long)J, 0, nullptr, nullptr, 1.f, 0.f };
 	int rc = quad_launch<QuadRowOp, QuadRowOp>(pa, pb, out, I, J, R, rest, wsBytes - weffBytes, FITRE_KC_CONV_DW, conv_flops(s), nullptr);
 	if (rc) return rc;
+	if (x2) {
+		pa.p = delta2, pb.p = x2;
+		out.beta = 1.f;
+		rc = quad_launch<QuadRowOp, QuadRowOp>(pa, pb, out, I, J, R, rest, wsBytes - weffBytes, FITRE_KC_CONV_DW, conv_flops(s), nullptr);
+		if (rc) return rc;
+	}
 	{
 		LaunchScope scope(FITRE_KC_PERMUTE, 4.0 * 25.0 * (double)cin * cout);
 		quad_fold_kernel<<<dim3((cin + 255) / 256, cout), 256, 0, stream()>>>(dweff, cin, cout, dW);
