@@ -131,6 +131,44 @@ def test_activations(dev, oracle64, act, n, misalign):
         dev.free(b)
 
 
+@pytest.mark.parametrize("act", ACTS)
+@pytest.mark.parametrize("n,misalign", [(4096, 0), (1001, 1), (1000, 1)])
+def test_activation_directional_derivative_backward(dev, act, n, misalign):
+    """R{delta f'(x)} = R{delta} f'(x) + delta f''(x) R{x} against the closed forms of f' and f'' in float64 (16-byte
+    path, which leaves out the tensors an activation does not use, and the element-wise path)."""
+    rng = np.random.default_rng(100 + act)
+    x = (rng.standard_normal(n) * 2).astype(np.float64)
+    sg = 1.0 / (1.0 + np.exp(-x))
+    if act == CNN_ACT_RELU:
+        f, f1, f2 = np.maximum(x, 0), (x > 0) * 1.0, 0 * x
+    elif act == CNN_ACT_SWISH:
+        f, f1, f2 = x * sg, sg + x * sg * (1 - sg), sg * (1 - sg) * (2 + x * (1 - 2 * sg))
+    elif act == CNN_ACT_SOFTPLUS:
+        f, f1, f2 = np.log1p(np.exp(x)), sg, sg * (1 - sg)
+    elif act == CNN_ACT_ELU:
+        f, f1, f2 = np.where(x < 0, np.exp(x) - 1, x), np.where(x < 0, np.exp(x), 1.0), np.where(x < 0, np.exp(x), 0.0)
+    elif act == ACT_LOGISTIC:
+        f, f1, f2 = sg, sg * (1 - sg), sg * (1 - sg) * (1 - 2 * sg)
+    elif act == ACT_TANH:
+        t = np.tanh(x)
+        f, f1, f2 = t, 1 - t * t, -2 * t * (1 - t * t)
+    else:
+        f, f1, f2 = x, 1 + 0 * x, 0 * x
+    rd, d, rz = (rng.standard_normal(n) for _ in range(3))
+    want = rd.astype(np.float32).astype(np.float64) * f1 + d.astype(np.float32).astype(np.float64) * f2 * rz.astype(np.float32)
+
+    def up(v):
+        buf = dev.upload(np.concatenate([np.zeros(misalign, np.float32), v.astype(np.float32)]))
+        return buf, at(buf, misalign)
+    bufs = [up(v) for v in (rd, d, x, f, rz)]
+    out = dev.zeros(n + misalign)
+    ok(hip.fitre_hip_activation_rop_backward(act, bufs[0][1], bufs[1][1], bufs[2][1], bufs[3][1], bufs[4][1], at(out, misalign), n))
+    assert rel_err(dev.download(at(out, misalign), n), want) < 2e-5
+    for b, _ in bufs:
+        dev.free(b)
+    dev.free(out)
+
+
 def test_unknown_activation_code_is_an_error(dev):
     p = dev.zeros(16)
     assert hip.fitre_hip_activation_forward(99, p, p, 16) == 3
