@@ -1258,6 +1258,7 @@ pool_act_bn_small_kernel(const float *delta, int dSplits, long dStride, const fl
 // and <.> the mean over the channel:
 //   out = ( rdx - <rdx> - rzhat <dx zhat> - zhat ( <rdx zhat> + <dx rzhat> ) ) / s  -  dc <zhat rx> / s
 // Pass 1: five sums per (channel, segment), slots of eight doubles.
+template <bool VEC>
 __global__ void __launch_bounds__(kRedBlock)
 bn_rop_partial_kernel(const float *rdx, const float *dx, const float *zhat, const float *rzhat, const float *rx, long perChannel,
                       double *partial)
@@ -1267,13 +1268,26 @@ bn_rop_partial_kernel(const float *rdx, const float *dx, const float *zhat, cons
 	long lo, hi;
 	segment_range(perChannel, lo, hi);
 	double s[5] = { 0.0, 0.0, 0.0, 0.0, 0.0 };
-	for (long i = lo + threadIdx.x; i < hi; i += kRedBlock) {
-		const float a = rdx[base + i], d = dx[base + i], z = zhat[base + i], rz = rzhat[base + i], x = rx[base + i];
-		s[0] += (double)a;
-		s[1] += (double)(d * z);
-		s[2] += (double)(a * z);
-		s[3] += (double)(d * rz);
-		s[4] += (double)(z * x);
+	if constexpr (VEC) { // 16-byte groups (perChannel % 4 == 0, aligned tensors: segments are whole groups)
+		for (long i = lo + 4 * (long)threadIdx.x; i + 3 < hi; i += 4 * kRedBlock) {
+			const float4 a = *reinterpret_cast<const float4 *>(rdx + base + i), d = *reinterpret_cast<const float4 *>(dx + base + i);
+			const float4 z = *reinterpret_cast<const float4 *>(zhat + base + i), rz = *reinterpret_cast<const float4 *>(rzhat + base + i);
+			const float4 x = *reinterpret_cast<const float4 *>(rx + base + i);
+			s[0] += (double)((a.x + a.y) + (a.z + a.w));
+			s[1] += (double)(d.x * z.x) + (double)(d.y * z.y) + (double)(d.z * z.z) + (double)(d.w * z.w);
+			s[2] += (double)(a.x * z.x) + (double)(a.y * z.y) + (double)(a.z * z.z) + (double)(a.w * z.w);
+			s[3] += (double)(d.x * rz.x) + (double)(d.y * rz.y) + (double)(d.z * rz.z) + (double)(d.w * rz.w);
+			s[4] += (double)(z.x * x.x) + (double)(z.y * x.y) + (double)(z.z * x.z) + (double)(z.w * x.w);
+		}
+	} else {
+		for (long i = lo + threadIdx.x; i < hi; i += kRedBlock) {
+			const float a = rdx[base + i], d = dx[base + i], z = zhat[base + i], rz = rzhat[base + i], x = rx[base + i];
+			s[0] += (double)a;
+			s[1] += (double)(d * z);
+			s[2] += (double)(a * z);
+			s[3] += (double)(d * rz);
+			s[4] += (double)(z * x);
+		}
 	}
 	double t[5];
 #pragma unroll
@@ -1284,6 +1298,7 @@ bn_rop_partial_kernel(const float *rdx, const float *dx, const float *zhat, cons
 		for (int k = 0; k < 5; k++) slot[k] = t[k];
 	}
 }
+template <bool VEC>
 __global__ void __launch_bounds__(kRedBlock)
 bn_rop_apply_kernel(const float *rdx, const float *zhat, const float *rzhat, const float *dc, const float *variance,
                     const double *partial, int segments, float epsilon, long perChannel, float *out)
@@ -1301,8 +1316,21 @@ bn_rop_apply_kernel(const float *rdx, const float *zhat, const float *rzhat, con
 	const size_t base = (size_t)c * perChannel;
 	long lo, hi;
 	segment_range(perChannel, lo, hi);
-	for (long i = lo + threadIdx.x; i < hi; i += kRedBlock)
-		out[base + i] = (rdx[base + i] - a - rzhat[base + i] * b - zhat[base + i] * cd) * inv - dc[base + i] * e * inv;
+	if constexpr (VEC) {
+		for (long i = lo + 4 * (long)threadIdx.x; i + 3 < hi; i += 4 * kRedBlock) {
+			const float4 r = *reinterpret_cast<const float4 *>(rdx + base + i), rz = *reinterpret_cast<const float4 *>(rzhat + base + i);
+			const float4 z = *reinterpret_cast<const float4 *>(zhat + base + i), d = *reinterpret_cast<const float4 *>(dc + base + i);
+			float4 o;
+			o.x = (r.x - a - rz.x * b - z.x * cd) * inv - d.x * e * inv;
+			o.y = (r.y - a - rz.y * b - z.y * cd) * inv - d.y * e * inv;
+			o.z = (r.z - a - rz.z * b - z.z * cd) * inv - d.z * e * inv;
+			o.w = (r.w - a - rz.w * b - z.w * cd) * inv - d.w * e * inv;
+			*reinterpret_cast<float4 *>(out + base + i) = o;
+		}
+	} else {
+		for (long i = lo + threadIdx.x; i < hi; i += kRedBlock)
+			out[base + i] = (rdx[base + i] - a - rzhat[base + i] * b - zhat[base + i] * cd) * inv - dc[base + i] * e * inv;
+	}
 }
 
 static inline bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
@@ -1952,8 +1980,15 @@ int fitre_hip_batch_norm_rop_backward(const float *rdelta_x, const float *delta_
 	double *partial = (double *)ws;
 	LaunchScope scope(FITRE_KC_BN_BWD, 28.0 * (double)channels * (double)perChannel);
 	dim3 grid(S, channels);
-	bn_rop_partial_kernel<<<grid, kRedBlock, 0, stream()>>>(rdelta_x, delta_x, zhat, rzhat, rx, perChannel, partial);
-	bn_rop_apply_kernel<<<grid, kRedBlock, 0, stream()>>>(rdelta_x, zhat, rzhat, delta_c, variance, partial, S, epsilon, perChannel, out);
+	const bool vec = perChannel % 4 == 0 && aligned16(rdelta_x) && aligned16(delta_x) && aligned16(zhat) && aligned16(rzhat) && aligned16(rx) &&
+	                 aligned16(delta_c) && aligned16(out);
+	if (vec) {
+		bn_rop_partial_kernel<true><<<grid, kRedBlock, 0, stream()>>>(rdelta_x, delta_x, zhat, rzhat, rx, perChannel, partial);
+		bn_rop_apply_kernel<true><<<grid, kRedBlock, 0, stream()>>>(rdelta_x, zhat, rzhat, delta_c, variance, partial, S, epsilon, perChannel, out);
+	} else {
+		bn_rop_partial_kernel<false><<<grid, kRedBlock, 0, stream()>>>(rdelta_x, delta_x, zhat, rzhat, rx, perChannel, partial);
+		bn_rop_apply_kernel<false><<<grid, kRedBlock, 0, stream()>>>(rdelta_x, zhat, rzhat, delta_c, variance, partial, S, epsilon, perChannel, out);
+	}
 	return check_launch("batch_norm_rop_backward");
 }
 

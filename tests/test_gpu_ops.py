@@ -327,6 +327,32 @@ def test_batch_norm_forward_backward(dev, oracle64, Cn, N, A, B, mis):
         dev.free(b)
 
 
+@pytest.mark.parametrize("Cn,per,mis", [(3, 4096, 0), (64, 32768, 0), (5, 1001, 0), (4, 4096, 1), (130, 64, 0)])
+def test_batch_norm_backward_directional_derivative(dev, Cn, per, mis):
+    """out = (R{dx} - <R{dx}> - R{zhat} <dx zhat> - zhat (<R{dx} zhat> + <dx R{zhat}>)) / s - dc <zhat R{x}> / s per channel
+    (<.> the mean over the channel, s = sqrt(var + eps)) against the same formula in float64: 16-byte path and the
+    element-wise one (odd channel length, misaligned tensors)."""
+    rng = np.random.default_rng(Cn + per)
+    names = ("rdx", "dx", "zhat", "rzhat", "rx", "dc")
+    t = {k: rng.standard_normal((Cn, per)).astype(np.float32) for k in names}
+    var = (rng.random(Cn) + 0.5).astype(np.float32)
+    eps = 1e-5
+    f = {k: v.astype(np.float64) for k, v in t.items()}
+    sdev = np.sqrt(var.astype(np.float64) + eps)[:, None]
+    mean = lambda v: v.mean(axis=1, keepdims=True)
+    want = (f["rdx"] - mean(f["rdx"]) - f["rzhat"] * mean(f["dx"] * f["zhat"]) -
+            f["zhat"] * (mean(f["rdx"] * f["zhat"]) + mean(f["dx"] * f["rzhat"]))) / sdev - f["dc"] * mean(f["zhat"] * f["rx"]) / sdev
+    bufs = {k: dev.upload(np.concatenate([np.zeros(mis, np.float32), v.reshape(-1)])) for k, v in t.items()}
+    p = {k: at(b, mis) for k, b in bufs.items()}
+    out = dev.zeros(Cn * per + mis)
+    ws, nb = bn_ws(dev, Cn, per)
+    ok(hip.fitre_hip_batch_norm_rop_backward(p["rdx"], p["dx"], p["zhat"], p["rzhat"], p["rx"], p["dc"], dev.upload(var), Cn, per, eps,
+                                             at(out, mis), ws, nb))
+    assert rel_err(dev.download(at(out, mis), Cn * per), want.reshape(-1)) < 1e-5
+    for b in list(bufs.values()) + [out, ws]:
+        dev.free(b)
+
+
 # C, N, A, B, k, s, p: fused sums (large channels), one-workgroup-per-channel (short channels, >= 128
 # of them), and shapes that fall back to the separate passes
 FUSED_BN_GEOMS = [
