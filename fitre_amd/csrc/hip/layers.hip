@@ -489,6 +489,28 @@ __device__ __forceinline__ int scan2x2(float v0, float v1, float v2, float v3)
 	return arg;
 }
 
+// pool_routed_kernel for 2x2 / stride 2 / no padding windows on maps with B % 4 == 0 and A even: one thread per pair of
+// pooled cells adjacent along B, i.e. a 2 x 4 patch of z and of the values, moved with 16-byte accesses.
+__global__ void __launch_bounds__(256) pool_routed2_kernel(const float *values, const float *z, int inA, int inB, long maps, float *out)
+{
+	const int outB2 = inB / 4, outA = inA / 2, outB = inB / 2;
+	const long perMap = (long)outA * outB2, total = maps * perMap;
+	const long stride = (long)gridDim.x * blockDim.x;
+	for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+		const long map = i / perMap;
+		const int rem = (int)(i - map * perMap);
+		const int oa = rem / outB2, pb = rem - oa * outB2;
+		const size_t in = (size_t)map * inA * inB + (size_t)(2 * oa) * inB + 4 * pb;
+		const float4 z0 = *reinterpret_cast<const float4 *>(z + in), z1 = *reinterpret_cast<const float4 *>(z + in + inB);
+		const float4 v0 = *reinterpret_cast<const float4 *>(values + in), v1 = *reinterpret_cast<const float4 *>(values + in + inB);
+		const int a = scan2x2(z0.x, z0.y, z1.x, z1.y), b = scan2x2(z0.z, z0.w, z1.z, z1.w);
+		float2 r;
+		r.x = a == 0 ? v0.x : (a == 1 ? v0.y : (a == 2 ? v1.x : (a == 3 ? v1.y : 0.f)));
+		r.y = b == 0 ? v0.z : (b == 1 ? v0.w : (b == 2 ? v1.z : (b == 3 ? v1.w : 0.f)));
+		*reinterpret_cast<float2 *>(out + (size_t)map * outA * outB + (size_t)oa * outB + 2 * pb) = r;
+	}
+}
+
 // Non-overlapping 2x2 / stride 2 / no padding max pool, even extents: one
 // thread per pair of pooled cells adjacent along B, i.e. a 2 x 4 input patch
 // moved with 16-byte accesses.  Fused with the activation derivative.
@@ -2004,7 +2026,12 @@ int fitre_hip_pool_forward_routed(int poolType, const float *values, const float
 	if (rc) return rc;
 	PoolGeom g = make_geom(inA, inB, ksize, stride, padding, outA, outB);
 	const long maps = (long)channels * samples;
-	LaunchScope scope(FITRE_KC_POOL_FWD, 4.0 * (double)maps * ((double)inA * inB + 2.0 * outA * outB));
+	LaunchScope scope(FITRE_KC_POOL_FWD, 4.0 * (double)maps * (2.0 * inA * inB + (double)outA * outB));
+	if (ksize == 2 && stride == 2 && padding == 0 && inB % 4 == 0 && inA % 2 == 0 && outA == inA / 2 && outB == inB / 2 && aligned16(values) &&
+	    aligned16(z_act) && (((uintptr_t)out) & 7) == 0) {
+		pool_routed2_kernel<<<blocks_for(maps * outA * (inB / 4), 256, 16384), 256, 0, stream()>>>(values, z_act, inA, inB, maps, out);
+		return check_launch("pool_routed2_kernel");
+	}
 	pool_routed_kernel<<<blocks_for(maps * outA * outB, 256, 16384), 256, 0, stream()>>>(values, z_act, g, maps, out);
 	return check_launch("pool_routed_kernel");
 }

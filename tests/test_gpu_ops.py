@@ -228,6 +228,27 @@ def test_pool_forward_backward(dev, oracle64, geom, kind):
         np.testing.assert_array_equal(got != 0, wantb != 0)
 
 
+@pytest.mark.parametrize("geom", [(4, 3, 8, 8, 2, 2, 0), (3, 5, 6, 12, 2, 2, 0), (64, 16, 4, 4, 2, 2, 0), (2, 3, 6, 10, 2, 2, 0),
+                                  (3, 2, 9, 11, 3, 2, 1), (2, 2, 5, 5, 2, 2, 0)])
+def test_pool_forward_routed(dev, oracle64, geom):
+    """What a max pool passes on of a second tensor: the value at the arg-max of z in every window (16-byte path for
+    2x2 windows on rows of a multiple of four cells, the general kernel otherwise), exact."""
+    Cn, N, A, B, k, s, p = geom
+    oA, oB = (A + 2 * p - k) // s + 1, (B + 2 * p - k) // s + 1
+    rng = np.random.default_rng(A * 100 + B)
+    z = rng.standard_normal(Cn * N * A * B).astype(np.float32)
+    z[:16] = 0.5                                           # ties: the first cell in memory order wins
+    v = rng.standard_normal(z.size).astype(np.float32)
+    pz, pv, out = dev.upload(z), dev.upload(v), dev.zeros(Cn * N * oA * oB)
+    ok(hip.fitre_hip_pool_forward_routed(MAX_POOL, pv, pz, Cn, N, A, B, k, s, p, oA, oB, out))
+    arg = np.asarray(oracle64.max_pool_argmax(z, N, Cn, B, A, k, s, p)).reshape(Cn * N, oA * oB)
+    want = np.take_along_axis(v.reshape(Cn * N, A * B), arg, axis=1)
+    np.testing.assert_array_equal(dev.download(out, want.size), want.reshape(-1))
+    for b in (pz, pv, out):
+        dev.free(b)
+
+
+
 def test_max_pool_ties_are_bit_exact(dev, oracle64):
     # all-equal windows (post-ReLU zeros), two-way ties, negative ties; 2x2 fast path and generic path
     for (A, B, k, s, p) in [(4, 4, 2, 2, 0), (4, 8, 2, 2, 0), (5, 5, 3, 2, 1), (6, 6, 3, 1, 0), (13, 13, 3, 2, 0), (10, 9, 3, 1, 1)]:
