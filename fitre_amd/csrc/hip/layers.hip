@@ -1276,6 +1276,80 @@ pool_act_bn_small_kernel(const float *delta, int dSplits, long dStride, const fl
 	}
 }
 
+// The directional derivative of a layer's batch norm, activation and 2x2 / stride 2 max pooling in one pass (the R
+// operator's forward sweep): R{bn out} is the batch-norm backward formula applied to R{x} (sums of channel_partial_kernel<3>
+// over (R{x}, zhat)), R{act out} = R{bn out} * f'(.), and the pooled value is the one at the arg-max of the activation
+// output.  z_act null (ReLU only): the activation output is max(zhat, 0), bit for bit what the forward pass stored.
+// POOL 0: units of 2 x 4 patches; POOL 2: no pooling, 16-byte groups.
+template <int POOL>
+__global__ void __launch_bounds__(kRedBlock)
+bn_act_pool_rop_forward_kernel(const float *rx, const float *zhat, const float *z_act, const float *variance, const double *partial,
+                               int segmentsIn, float epsilon, int samples, int inA, int inB, int actFun, float *rbn, float *ract,
+                               float *rpool)
+{
+	__shared__ double lds[3 * kRedBlock / kWave];
+	const int c = blockIdx.y;
+	const long perChannel = (long)samples * inA * inB;
+	double a1 = 0.0, a2 = 0.0, a3 = 0.0;
+	for (int k = threadIdx.x; k < segmentsIn; k += kRedBlock) {
+		const double *slot = partial + ((size_t)c * segmentsIn + k) * 4;
+		a1 += slot[0], a2 += slot[1], a3 += slot[2];
+	}
+	block_sum3<kRedBlock>(a1, a2, a3, lds);
+	const float m = (float)perChannel;
+	const float sum1 = (float)a1, sum2 = (float)a2;
+	const float scale = 1.f / (m * sqrtf(epsilon + variance[c]));
+	const size_t base = (size_t)c * perChannel;
+	auto step = [&](size_t at, float4 &zo) { // R{bn out} and R{act out} of one group; zo: its activation output
+		const float4 d = *reinterpret_cast<const float4 *>(rx + at), z = *reinterpret_cast<const float4 *>(zhat + at);
+		zo = z_act ? *reinterpret_cast<const float4 *>(z_act + at) : relu4(z);
+		float4 r;
+		r.x = bn_backward_value(m, d.x, z.x, sum1, sum2, scale);
+		r.y = bn_backward_value(m, d.y, z.y, sum1, sum2, scale);
+		r.z = bn_backward_value(m, d.z, z.z, sum1, sum2, scale);
+		r.w = bn_backward_value(m, d.w, z.w, sum1, sum2, scale);
+		*reinterpret_cast<float4 *>(rbn + at) = r;
+		// a zero derivative gives +0 whatever the sign of R{bn out}, as the activation's own backward kernel does for ReLU
+		const float fx = act_derivative(actFun, z.x, zo.x), fy = act_derivative(actFun, z.y, zo.y);
+		const float fz = act_derivative(actFun, z.z, zo.z), fw = act_derivative(actFun, z.w, zo.w);
+		r.x = fx == 0.f ? 0.f : r.x * fx, r.y = fy == 0.f ? 0.f : r.y * fy;
+		r.z = fz == 0.f ? 0.f : r.z * fz, r.w = fw == 0.f ? 0.f : r.w * fw;
+		*reinterpret_cast<float4 *>(ract + at) = r;
+		return r;
+	};
+	if constexpr (POOL == 2) {
+		const long groups = perChannel / 4;
+		const long per = (groups + gridDim.x - 1) / gridDim.x;
+		const long lo = (long)blockIdx.x * per;
+		const long hi = (lo + per < groups) ? lo + per : groups;
+		for (long i = lo + threadIdx.x; i < hi; i += kRedBlock) {
+			float4 zo;
+			step(base + 4 * i, zo);
+		}
+	} else {
+		const int outB2 = inB / 4, outA = inA / 2, outB = inB / 2;
+		const int perMap = outA * outB2;
+		const long patches = (long)samples * perMap;
+		const long per = (patches + gridDim.x - 1) / gridDim.x;
+		const long lo = (long)blockIdx.x * per;
+		const long hi = (lo + per < patches) ? lo + per : patches;
+		const size_t pBase = (size_t)c * samples * outA * outB;
+		for (long i = lo + threadIdx.x; i < hi; i += kRedBlock) {
+			const long map = i / perMap;
+			const int rem = (int)(i - map * perMap);
+			const int oa = rem / outB2, pb = rem - oa * outB2;
+			const size_t in = base + (size_t)map * inA * inB + (size_t)(2 * oa) * inB + 4 * pb;
+			float4 z0, z1;
+			const float4 r0 = step(in, z0), r1 = step(in + inB, z1);
+			const int a = scan2x2(z0.x, z0.y, z1.x, z1.y), b = scan2x2(z0.z, z0.w, z1.z, z1.w);
+			float2 r;
+			r.x = a == 0 ? r0.x : (a == 1 ? r0.y : (a == 2 ? r1.x : (a == 3 ? r1.y : 0.f)));
+			r.y = b == 0 ? r0.z : (b == 1 ? r0.w : (b == 2 ? r1.z : (b == 3 ? r1.w : 0.f)));
+			*reinterpret_cast<float2 *>(rpool + pBase + (size_t)map * outA * outB + (size_t)oa * outB + 2 * pb) = r;
+		}
+	}
+}
+
 // Directional derivative of the batch-norm backward formula.  Per channel, with s = sqrt(var + eps)
 // and <.> the mean over the channel:
 //   out = ( rdx - <rdx> - rzhat <dx zhat> - zhat ( <rdx zhat> + <dx rzhat> ) ) / s  -  dc <zhat rx> / s
@@ -2034,6 +2108,45 @@ int fitre_hip_pool_forward_routed(int poolType, const float *values, const float
 	}
 	pool_routed_kernel<<<blocks_for(maps * outA * outB, 256, 16384), 256, 0, stream()>>>(values, z_act, g, maps, out);
 	return check_launch("pool_routed_kernel");
+}
+
+int fitre_hip_bn_act_pool_rop_forward(const float *rx, const float *zhat, const float *z_act, const float *variance, int channels,
+                                      int samples, int inA, int inB, float epsilon, int actFun, float *rbn, float *ract, int poolType,
+                                      int ksize, int stride, int padding, int outA, int outB, float *rpool, void *ws, size_t wsBytes)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(rx && zhat && variance && rbn && ract, "fitre_hip_bn_act_pool_rop_forward: null pointer");
+	FITRE_REQUIRE(poolType == NO_POOL || rpool, "fitre_hip_bn_act_pool_rop_forward: null pooled output");
+	FITRE_REQUIRE(act_known(actFun), "fitre_hip_bn_act_pool_rop_forward: unknown activation code %d", actFun);
+	FITRE_REQUIRE(z_act || actFun == CNN_ACT_RELU, "fitre_hip_bn_act_pool_rop_forward: z_act is required (only ReLU's output can be derived)");
+	FITRE_REQUIRE(channels > 0 && samples > 0 && inA > 0 && inB > 0, "fitre_hip_bn_act_pool_rop_forward: non-positive shape");
+	const long perChannel = (long)samples * inA * inB, count = perChannel * channels;
+	int rc = check_channels("fitre_hip_bn_act_pool_rop_forward", channels, perChannel, ws, wsBytes);
+	if (rc) return rc;
+	const bool pool2 = poolType == MAX_POOL && ksize == 2 && stride == 2 && padding == 0 && inB % 4 == 0 && inA % 2 == 0 &&
+	                   outA == inA / 2 && outB == inB / 2 && (((uintptr_t)rpool) & 7) == 0;
+	const bool fused = (poolType == NO_POOL || pool2) && perChannel % 4 == 0 && aligned16(rx) && aligned16(zhat) && aligned16(rbn) &&
+	                   aligned16(ract) && (!z_act || aligned16(z_act));
+	if (!fused) {
+		FITRE_REQUIRE(z_act, "fitre_hip_bn_act_pool_rop_forward: this shape runs the separate passes, which need z_act");
+		rc = fitre_hip_batch_norm_backward(rx, zhat, variance, channels, perChannel, epsilon, rbn, nullptr, ws, wsBytes);
+		if (rc) return rc;
+		rc = fitre_hip_activation_backward(actFun, rbn, zhat, z_act, ract, count);
+		if (rc || poolType == NO_POOL) return rc;
+		return fitre_hip_pool_forward_routed(poolType, ract, z_act, channels, samples, inA, inB, ksize, stride, padding, outA, outB, rpool);
+	}
+	const int S = segments_for(channels, perChannel);
+	double *partial = (double *)ws;
+	const dim3 grid(S, channels);
+	LaunchScope scope(FITRE_KC_BN_BWD, 4.0 * (double)count * (2 + 2 + 2 + (z_act ? 1 : 0)) + (poolType == NO_POOL ? 0.0 : (double)count));
+	channel_partial_kernel<3, true><<<grid, kRedBlock, 0, stream()>>>(rx, zhat, perChannel, partial);
+	if (poolType == NO_POOL)
+		bn_act_pool_rop_forward_kernel<2><<<grid, kRedBlock, 0, stream()>>>(rx, zhat, z_act, variance, partial, S, epsilon, samples, inA, inB,
+		                                                                    actFun, rbn, ract, rpool);
+	else
+		bn_act_pool_rop_forward_kernel<0><<<grid, kRedBlock, 0, stream()>>>(rx, zhat, z_act, variance, partial, S, epsilon, samples, inA, inB,
+		                                                                    actFun, rbn, ract, rpool);
+	return check_launch("bn_act_pool_rop_forward_kernel");
 }
 
 int fitre_hip_multinomial_classes(const float *probs, const float *uniforms, int samples, int classes, float *out)

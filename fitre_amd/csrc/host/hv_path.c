@@ -141,23 +141,31 @@ static void rop_forward(CNN_MODEL *model, const real *weights, const real *vecto
 				HIP_CALL(fitre_hip_axpy((int)count, 1.f, tmp, rslab));
 			}
 		}
-		const real *rpre = rslab, *actIn = slab;
-		if (has_bn(c)) {
-			HIP_CALL(fitre_hip_batch_norm_backward(rslab, slab + c->batchNormOffset, slab + c->batchNormOffset + c->variancesOffset,
-			                                       c->outChannels, perChannel, (real)BATCH_NORM_EPSILON,
-			                                       rslab + c->batchNormOffset, NULL, ws, wsBytes));
-			rpre = rslab + c->batchNormOffset;
-			actIn = slab + c->batchNormOffset;
-		}
 		const real *actOut = conv_act_out(model, l, z, n, actbuf);
 		real *ract = rslab + c->activationOffset;
-		HIP_CALL(fitre_hip_activation_backward(model->actFuns[l], rpre, actIn, actOut, ract, count));
-		if (p->type == MAX_POOL || p->type == AVG_POOL)
-			HIP_CALL(fitre_hip_pool_forward_routed(p->type, ract, actOut, c->outChannels, n, p->width, p->height, p->pSize,
-			                                       p->stride, p->padding, p->outWidth, p->outHeight, rslab + c->poolOffset));
-		else if (p->type != NO_POOL) {
-			fprintf(stderr, "Unknown Pool Function... \n");
-			exit(-1);
+		if (has_bn(c)) {
+			/* batch norm forward's R-operator is its backward formula on R{x}; with the activation's and the pooling's in one
+			 * pass over R{x} and zhat where the shapes allow */
+			const int pooled = p->type == MAX_POOL || p->type == AVG_POOL;
+			if (p->type != NO_POOL && !pooled) {
+				fprintf(stderr, "Unknown Pool Function... \n");
+				exit(-1);
+			}
+			HIP_CALL(fitre_hip_bn_act_pool_rop_forward(rslab, slab + c->batchNormOffset, actOut,
+			                                           slab + c->batchNormOffset + c->variancesOffset, c->outChannels, n,
+			                                           pooled ? p->width : c->outWidth, pooled ? p->height : c->outHeight,
+			                                           (real)BATCH_NORM_EPSILON, model->actFuns[l], rslab + c->batchNormOffset, ract, p->type,
+			                                           p->pSize, p->stride, p->padding, p->outWidth, p->outHeight,
+			                                           pooled ? rslab + c->poolOffset : NULL, ws, wsBytes));
+		} else {
+			HIP_CALL(fitre_hip_activation_backward(model->actFuns[l], rslab, slab, actOut, ract, count));
+			if (p->type == MAX_POOL || p->type == AVG_POOL)
+				HIP_CALL(fitre_hip_pool_forward_routed(p->type, ract, actOut, c->outChannels, n, p->width, p->height, p->pSize,
+				                                       p->stride, p->padding, p->outWidth, p->outHeight, rslab + c->poolOffset));
+			else if (p->type != NO_POOL) {
+				fprintf(stderr, "Unknown Pool Function... \n");
+				exit(-1);
+			}
 		}
 	}
 	/* the feature permute of the forward pass, on R{z} */

@@ -126,6 +126,8 @@ HIP_API = {
     "fitre_hip_lanes_enable": (i32, [i32]),
     "fitre_hip_activation_rop_backward": (i32, [i32, vp, vp, vp, vp, vp, vp, lng]),
     "fitre_hip_pool_forward_routed": (i32, [i32, vp, vp] + [i32] * 9 + [vp]),
+    "fitre_hip_bn_act_pool_rop_forward": (i32, [vp, vp, vp, vp, i32, i32, i32, i32, f32, i32, vp, vp, i32, i32, i32, i32, i32, i32, vp, vp,
+                                                sz]),
     "fitre_hip_batch_norm_rop_backward": (i32, [vp, vp, vp, vp, vp, vp, vp, i32, lng, f32, vp, vp, sz]),
     "fitre_hip_cross_entropy_rop_error": (i32, [vp, vp, i32, i32, vp]),
     "fitre_hip_fc_rop_backward": (i32, [i32, vp, vp, vp, vp, vp, lng]),

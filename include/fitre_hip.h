@@ -460,6 +460,17 @@ int fitre_hip_activation_rop_backward(int actFun, const float *rdelta, const flo
  * average pool: the average of values (z_act unused). */
 int fitre_hip_pool_forward_routed(int poolType, const float *values, const float *z_act, int channels, int samples,
                                   int inA, int inB, int ksize, int stride, int padding, int outA, int outB, float *out);
+/* The R operator's forward sweep through what follows a convolution with batch norm (functions/cnn_hv_forward.cu:120-222):
+ * R{bn out} = the batch-norm backward formula applied to rx (fitre_hip_batch_norm_backward), R{act out} = R{bn out} * f'(.)
+ * (fitre_hip_activation_backward) and, through a max pool, the value at the arg-max of the activation output
+ * (fitre_hip_pool_forward_routed) -- after the sums, ONE pass that reads rx and zhat and writes all three (the same results as
+ * the three passes).  z_act may be NULL when actFun is ReLU (the activation output is then max(zhat, 0)) and the shape is
+ * fused: no pooling or 2x2 / stride 2 max pooling, A even, B a multiple of 4, 16-byte-aligned tensors; every other case
+ * runs the three passes and needs z_act.  Workspace: fitre_hip_batch_norm_workspace(channels, samples * inA * inB). */
+int fitre_hip_bn_act_pool_rop_forward(const float *rx, const float *zhat, const float *z_act, const float *variance,
+                                      int channels, int samples, int inA, int inB, float epsilon, int actFun, float *rbn,
+                                      float *ract, int poolType, int ksize, int stride, int padding, int outA, int outB,
+                                      float *rpool, void *ws, size_t wsBytes);
 /* Directional derivative of batch-norm backward (computeROpBatchNormBackward, functions/dev_batch_norm.cu:787-960):
  * with s = sqrt(var + eps) and <.> the per-channel mean,
  *   out = (rdelta_x - <rdelta_x> - rzhat <delta_x zhat> - zhat (<rdelta_x zhat> + <delta_x rzhat>)) / s - delta_c <zhat rx> / s

@@ -374,6 +374,54 @@ def test_batch_norm_backward_directional_derivative(dev, Cn, per, mis):
         dev.free(b)
 
 
+@pytest.mark.parametrize("derive", [False, True])
+@pytest.mark.parametrize("act", [CNN_ACT_RELU, CNN_ACT_SWISH])
+@pytest.mark.parametrize("kind", [MAX_POOL, NO_POOL])
+@pytest.mark.parametrize("geom", [(3, 40, 16, 16, 2, 2, 0), (64, 8, 32, 32, 2, 2, 0), (5, 9, 6, 12, 2, 2, 0), (160, 7, 8, 8, 2, 2, 0),
+                                  (2, 4, 6, 10, 2, 2, 0), (2, 2, 7, 5, 3, 2, 1)])
+def test_fused_directional_derivative_forward(dev, geom, kind, act, derive):
+    """R{bn out}, R{act out} and the routed pooled values of a layer in one call against the three separate entry
+    points (fused shapes and those that fall back); `derive`: without the activation output, which only ReLU allows."""
+    Cn, N, A, B, k, s, p = geom
+    if derive and act != CNN_ACT_RELU:
+        pytest.skip("only ReLU's output can be derived from zhat")
+    oA, oB = (A + 2 * p - k) // s + 1, (B + 2 * p - k) // s + 1
+    per = N * A * B
+    fusable = (kind == NO_POOL or (k == 2 and B % 4 == 0 and A % 2 == 0)) and per % 4 == 0
+    rng = np.random.default_rng(Cn * 3 + A * B + act)
+    rx = rng.standard_normal(Cn * per).astype(np.float32)
+    zhat = rng.standard_normal(Cn * per).astype(np.float32)
+    var = (rng.random(Cn) + 0.5).astype(np.float32)
+    prx, pzh, pvar = dev.upload(rx), dev.upload(zhat), dev.upload(var)
+    zact = dev.zeros(Cn * per)
+    ok(hip.fitre_hip_activation_forward(act, pzh, zact, Cn * per))
+    ws, nb = bn_ws(dev, Cn, per)
+    pooled = Cn * N * oA * oB
+
+    def run(fused):
+        rbn, ract, rpool = dev.zeros(Cn * per), dev.zeros(Cn * per), dev.zeros(pooled)
+        if fused:
+            rc = hip.fitre_hip_bn_act_pool_rop_forward(prx, pzh, None if derive else zact, pvar, Cn, N, A, B, 1e-5, act, rbn, ract, kind, k, s,
+                                                       p, oA, oB, rpool if kind != NO_POOL else None, ws, nb)
+            if derive and not fusable:
+                assert rc != 0                       # the separate passes need the activation output
+                return None
+            ok(rc)
+        else:
+            ok(hip.fitre_hip_batch_norm_backward(prx, pzh, pvar, Cn, per, 1e-5, rbn, None, ws, nb))
+            ok(hip.fitre_hip_activation_backward(act, rbn, pzh, zact, ract, Cn * per))
+            if kind != NO_POOL:
+                ok(hip.fitre_hip_pool_forward_routed(kind, ract, zact, Cn, N, A, B, k, s, p, oA, oB, rpool))
+        return [dev.download(b, n) for b, n in ((rbn, Cn * per), (ract, Cn * per), (rpool, pooled))]
+
+    want, got = run(False), run(True)
+    if got is not None:
+        for g, w in zip(got, want):
+            assert rel_err(g, w) < 1e-6
+            np.testing.assert_array_equal(g == 0, w == 0)   # the same routing and the same masks
+    dev.free(ws)
+
+
 # C, N, A, B, k, s, p: fused sums (large channels), one-workgroup-per-channel (short channels, >= 128
 # of them), and shapes that fall back to the separate passes
 FUSED_BN_GEOMS = [
