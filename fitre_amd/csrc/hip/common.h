@@ -5,6 +5,7 @@
 #include <stdint.h>
 #include <stdio.h>
 #include "fitre_hip.h"
+#include "fitre_nn.h"
 
 namespace fitre {
 
@@ -107,6 +108,30 @@ void conv_gemm_release();
 	do {                                                                                             \
 		if (FITRE_MATRIX_WAVE_PRIORITY > 0) __builtin_amdgcn_s_setprio(FITRE_MATRIX_WAVE_PRIORITY);  \
 	} while (0)
+
+// ---- activation functions: first and second derivative ------------------------
+__device__ __forceinline__ float sigmoidf(float x) { return 1.f / (1.f + expf(-x)); }
+// f1 = f'(x), f2 = f''(x) from the activation's input zi and output zo (whichever the function needs)
+__device__ __forceinline__ void act_derivatives(int actFun, float zi, float zo, float &f1, float &f2)
+{
+	switch (actFun) {
+	case ACT_LOGISTIC: f1 = zo * (1.f - zo), f2 = f1 * (1.f - 2.f * zo); break;
+	case ACT_TANH: f1 = (1.f + zo) * (1.f - zo), f2 = -2.f * zo * f1; break;
+	case CNN_ACT_SOFTPLUS: {
+		const float s = sigmoidf(zi);
+		f1 = s, f2 = s * (1.f - s);
+		break;
+	}
+	case CNN_ACT_SWISH: {
+		const float s = sigmoidf(zi);
+		f1 = zo + s * (1.f - zo), f2 = s * (1.f - s) * (2.f + zi * (1.f - 2.f * s));
+		break;
+	}
+	case CNN_ACT_RELU: f1 = zo > 0.f ? 1.f : 0.f, f2 = 0.f; break;
+	case CNN_ACT_ELU: f1 = zo < 0.f ? zo + 1.f : 1.f, f2 = zo < 0.f ? zo + 1.f : 0.f; break;
+	default: f1 = 1.f, f2 = 0.f; break;
+	}
+}
 
 // ---- per-class launch accounting ------------------------------------------
 // A LaunchScope brackets the launches made while it is alive with two events

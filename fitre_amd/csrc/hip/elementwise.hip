@@ -77,7 +77,6 @@ struct FInvScale { float eps; __device__ float operator()(float x, float y, floa
 struct FSqr { __device__ float operator()(float x, float, float, float) const { return x * x; } };
 struct FSqrDecay { float decay; __device__ float operator()(float x, float y, float, float) const { return decay * x + (1.f - decay) * y * y; } };
 
-__device__ __forceinline__ float sigmoidf(float x) { return 1.f / (1.f + expf(-x)); }
 
 // terms of the fully connected models' output heads (a = target y, b = network output or logit)
 struct FScaledDiff { float scale; __device__ float operator()(float y, float z, float, float) const { return scale * (y - z); } };
@@ -299,26 +298,6 @@ __global__ void __launch_bounds__(256) random_normal_kernel(float *out, long n, 
 static unsigned long long g_rng_seed = 1234ull, g_rng_next = 0ull;
 
 // out = rdelta * f'(.) + delta * f''(.) * rz_in: the directional derivative of delta * f'(.)
-__device__ __forceinline__ void act_derivatives(int actFun, float zi, float zo, float &f1, float &f2)
-{
-	switch (actFun) {
-	case ACT_LOGISTIC: f1 = zo * (1.f - zo), f2 = f1 * (1.f - 2.f * zo); break;
-	case ACT_TANH: f1 = (1.f + zo) * (1.f - zo), f2 = -2.f * zo * f1; break;
-	case CNN_ACT_SOFTPLUS: {
-		const float s = sigmoidf(zi);
-		f1 = s, f2 = s * (1.f - s);
-		break;
-	}
-	case CNN_ACT_SWISH: {
-		const float s = sigmoidf(zi);
-		f1 = zo + s * (1.f - zo), f2 = s * (1.f - s) * (2.f + zi * (1.f - 2.f * s));
-		break;
-	}
-	case CNN_ACT_RELU: f1 = zo > 0.f ? 1.f : 0.f, f2 = 0.f; break;
-	case CNN_ACT_ELU: f1 = zo < 0.f ? zo + 1.f : 1.f, f2 = zo < 0.f ? zo + 1.f : 0.f; break;
-	default: f1 = 1.f, f2 = 0.f; break;
-	}
-}
 __global__ void __launch_bounds__(256) activation_rop_backward_kernel(int actFun, const float *rdelta, const float *delta,
                                                                        const float *z_in, const float *z_out, const float *rz_in,
                                                                        float *out, long n)

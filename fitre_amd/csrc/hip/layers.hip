@@ -1429,6 +1429,87 @@ bn_rop_apply_kernel(const float *rdx, const float *zhat, const float *rzhat, con
 	}
 }
 
+// The backward sweep's first three R-steps of a layer with batch norm in one pass: the pooled R{delta} is routed to the
+// arg-max cells (2x2 / stride 2 windows, POOL 0; POOL 2: no pooling), R{delta f'(x)} = R{delta} f'(x) + delta f''(x) R{x}
+// is written to rdOut, and the five sums of bn_rop_partial_kernel over (rdOut, dxAct, zhat, rzhat, rx) are left per
+// (channel, segment) -- what bn_rop_apply_kernel needs.  SECOND false: f'' is zero (ReLU, linear) and `delta` is not
+// read.  z_act null (ReLU only): the activation output is max(zhat, 0).  rzhat is R{x} of the activation: R{bn out}.
+template <int POOL, bool SECOND>
+__global__ void __launch_bounds__(kRedBlock)
+pool_act_bn_rop_sums_kernel(const float *rdeltaPooled, const float *delta, const float *zhat, const float *z_act, const float *rzhat,
+                            const float *dxAct, const float *rx, int inA, int inB, int samples, int actFun, float *rdOut, double *partial)
+{
+	__shared__ double lds[kRedBlock / kWave];
+	const int c = blockIdx.y;
+	const long perChannel = (long)samples * inA * inB;
+	const size_t base = (size_t)c * perChannel;
+	double s[5] = { 0.0, 0.0, 0.0, 0.0, 0.0 };
+	auto step = [&](size_t at, float4 g, float4 z, float4 zo) { // g: R{delta} at the activation output of this group
+		const float4 rz = *reinterpret_cast<const float4 *>(rzhat + at), da = *reinterpret_cast<const float4 *>(dxAct + at);
+		const float4 x = *reinterpret_cast<const float4 *>(rx + at);
+		float4 d = make_float4(0.f, 0.f, 0.f, 0.f);
+		if constexpr (SECOND) d = *reinterpret_cast<const float4 *>(delta + at);
+		float4 r;
+		float f1, f2;
+		act_derivatives(actFun, z.x, zo.x, f1, f2);
+		r.x = SECOND ? g.x * f1 + d.x * f2 * rz.x : g.x * f1;
+		act_derivatives(actFun, z.y, zo.y, f1, f2);
+		r.y = SECOND ? g.y * f1 + d.y * f2 * rz.y : g.y * f1;
+		act_derivatives(actFun, z.z, zo.z, f1, f2);
+		r.z = SECOND ? g.z * f1 + d.z * f2 * rz.z : g.z * f1;
+		act_derivatives(actFun, z.w, zo.w, f1, f2);
+		r.w = SECOND ? g.w * f1 + d.w * f2 * rz.w : g.w * f1;
+		*reinterpret_cast<float4 *>(rdOut + at) = r;
+		s[0] += (double)((r.x + r.y) + (r.z + r.w));
+		s[1] += (double)(da.x * z.x) + (double)(da.y * z.y) + (double)(da.z * z.z) + (double)(da.w * z.w);
+		s[2] += (double)(r.x * z.x) + (double)(r.y * z.y) + (double)(r.z * z.z) + (double)(r.w * z.w);
+		s[3] += (double)(da.x * rz.x) + (double)(da.y * rz.y) + (double)(da.z * rz.z) + (double)(da.w * rz.w);
+		s[4] += (double)(z.x * x.x) + (double)(z.y * x.y) + (double)(z.z * x.z) + (double)(z.w * x.w);
+	};
+	if constexpr (POOL == 2) {
+		const long groups = perChannel / 4;
+		const long per = (groups + gridDim.x - 1) / gridDim.x;
+		const long lo = (long)blockIdx.x * per;
+		const long hi = (lo + per < groups) ? lo + per : groups;
+		for (long i = lo + threadIdx.x; i < hi; i += kRedBlock) {
+			const size_t at = base + 4 * i;
+			const float4 z = *reinterpret_cast<const float4 *>(zhat + at);
+			const float4 zo = z_act ? *reinterpret_cast<const float4 *>(z_act + at) : relu4(z);
+			step(at, *reinterpret_cast<const float4 *>(rdeltaPooled + at), z, zo);
+		}
+	} else {
+		const int outB2 = inB / 4, outA = inA / 2, outB = inB / 2;
+		const int perMap = outA * outB2;
+		const long patches = (long)samples * perMap;
+		const long per = (patches + gridDim.x - 1) / gridDim.x;
+		const long lo = (long)blockIdx.x * per;
+		const long hi = (lo + per < patches) ? lo + per : patches;
+		const size_t pBase = (size_t)c * samples * outA * outB;
+		for (long i = lo + threadIdx.x; i < hi; i += kRedBlock) {
+			const long map = i / perMap;
+			const int rem = (int)(i - map * perMap);
+			const int oa = rem / outB2, pb = rem - oa * outB2;
+			const size_t in = base + (size_t)map * inA * inB + (size_t)(2 * oa) * inB + 4 * pb;
+			const float4 z0 = *reinterpret_cast<const float4 *>(zhat + in), z1 = *reinterpret_cast<const float4 *>(zhat + in + inB);
+			const float4 o0 = z_act ? *reinterpret_cast<const float4 *>(z_act + in) : relu4(z0);
+			const float4 o1 = z_act ? *reinterpret_cast<const float4 *>(z_act + in + inB) : relu4(z1);
+			const float2 d = *reinterpret_cast<const float2 *>(rdeltaPooled + pBase + (size_t)map * outA * outB + (size_t)oa * outB + 2 * pb);
+			float4 g0, g1;
+			route2x4(o0, o1, d, g0, g1);
+			step(in, g0, z0, o0);
+			step(in + inB, g1, z1, o1);
+		}
+	}
+	double t[5];
+#pragma unroll
+	for (int k = 0; k < 5; k++) t[k] = block_sum<kRedBlock>(s[k], lds);
+	if (threadIdx.x == 0) {
+		double *slot = partial + ((size_t)c * gridDim.x + blockIdx.x) * 8;
+#pragma unroll
+		for (int k = 0; k < 5; k++) slot[k] = t[k];
+	}
+}
+
 static inline bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
 // =====================================================================
@@ -2086,6 +2167,66 @@ int fitre_hip_batch_norm_rop_backward(const float *rdelta_x, const float *delta_
 		bn_rop_apply_kernel<false><<<grid, kRedBlock, 0, stream()>>>(rdelta_x, zhat, rzhat, delta_c, variance, partial, S, epsilon, perChannel, out);
 	}
 	return check_launch("batch_norm_rop_backward");
+}
+
+int fitre_hip_pool_act_bn_rop_backward(int poolType, int actFun, const float *rdelta, const float *delta, const float *zhat,
+                                       const float *z_act, const float *rzhat, const float *delta_x, const float *rx,
+                                       const float *delta_c, const float *variance, int channels, int samples, int inA, int inB,
+                                       int ksize, int stride, int padding, int outA, int outB, float epsilon, float *rdeltaAct,
+                                       float *rdeltaX, float *out, void *ws, size_t wsBytes)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(rdelta && delta && zhat && rzhat && delta_x && rx && delta_c && variance && rdeltaX && out,
+	              "fitre_hip_pool_act_bn_rop_backward: null pointer");
+	FITRE_REQUIRE(act_known(actFun), "fitre_hip_pool_act_bn_rop_backward: unknown activation code %d", actFun);
+	FITRE_REQUIRE(channels > 0 && samples > 0 && inA > 0 && inB > 0, "fitre_hip_pool_act_bn_rop_backward: non-positive shape");
+	const long perChannel = (long)samples * inA * inB, count = perChannel * channels;
+	int rc = check_channels("fitre_hip_pool_act_bn_rop_backward", channels, perChannel, ws, wsBytes);
+	if (rc) return rc;
+	const int S = segments_for(channels, perChannel);
+	if (wsBytes < (size_t)channels * S * 8 * sizeof(double))
+		return fail(FITRE_E_WORKSPACE, "fitre_hip_pool_act_bn_rop_backward: workspace of %zu bytes is smaller than the %zu required", wsBytes,
+		            (size_t)channels * S * 8 * sizeof(double));
+	const bool pool2 = poolType == MAX_POOL && ksize == 2 && stride == 2 && padding == 0 && inB % 4 == 0 && inA % 2 == 0 &&
+	                   outA == inA / 2 && outB == inB / 2 && (((uintptr_t)rdelta) & 7) == 0;
+	const bool second = !(actFun == CNN_ACT_RELU || actFun == ACT_LINEAR || actFun == CNN_ACT_NONE);
+	const bool fused = (pool2 || (poolType == NO_POOL && aligned16(rdelta))) && perChannel % 4 == 0 && aligned16(zhat) && aligned16(rzhat) &&
+	                   aligned16(delta_x) && aligned16(rx) && aligned16(delta_c) && aligned16(rdeltaX) && aligned16(out) &&
+	                   (!z_act || aligned16(z_act)) && (!second || aligned16(delta)) && (z_act || actFun == CNN_ACT_RELU);
+	if (!fused) {
+		FITRE_REQUIRE(z_act, "fitre_hip_pool_act_bn_rop_backward: this shape runs the separate passes, which need z_act");
+		const float *atAct = rdelta;
+		if (poolType != NO_POOL) {
+			FITRE_REQUIRE(rdeltaAct, "fitre_hip_pool_act_bn_rop_backward: the separate passes need a buffer for the routed R{delta}");
+			rc = fitre_hip_pool_backward(poolType, rdelta, z_act, channels, samples, inA, inB, ksize, stride, padding, outA, outB, rdeltaAct);
+			if (rc) return rc;
+			atAct = rdeltaAct;
+		}
+		rc = fitre_hip_activation_rop_backward(actFun, atAct, delta, zhat, z_act, rzhat, rdeltaX, count);
+		if (rc) return rc;
+		return fitre_hip_batch_norm_rop_backward(rdeltaX, delta_x, zhat, rzhat, rx, delta_c, variance, channels, perChannel, epsilon, out, ws,
+		                                         wsBytes);
+	}
+	double *partial = (double *)ws;
+	const dim3 grid(S, channels);
+	LaunchScope scope(FITRE_KC_BN_BWD, 4.0 * (double)count * (11.0 + (second ? 1.0 : 0.0) + (z_act ? 1.0 : 0.0)));
+	if (poolType == NO_POOL) {
+		if (second)
+			pool_act_bn_rop_sums_kernel<2, true><<<grid, kRedBlock, 0, stream()>>>(rdelta, delta, zhat, z_act, rzhat, delta_x, rx, inA, inB, samples,
+			                                                                       actFun, rdeltaX, partial);
+		else
+			pool_act_bn_rop_sums_kernel<2, false><<<grid, kRedBlock, 0, stream()>>>(rdelta, delta, zhat, z_act, rzhat, delta_x, rx, inA, inB, samples,
+			                                                                        actFun, rdeltaX, partial);
+	} else {
+		if (second)
+			pool_act_bn_rop_sums_kernel<0, true><<<grid, kRedBlock, 0, stream()>>>(rdelta, delta, zhat, z_act, rzhat, delta_x, rx, inA, inB, samples,
+			                                                                       actFun, rdeltaX, partial);
+		else
+			pool_act_bn_rop_sums_kernel<0, false><<<grid, kRedBlock, 0, stream()>>>(rdelta, delta, zhat, z_act, rzhat, delta_x, rx, inA, inB, samples,
+			                                                                        actFun, rdeltaX, partial);
+	}
+	bn_rop_apply_kernel<true><<<grid, kRedBlock, 0, stream()>>>(rdeltaX, zhat, rzhat, delta_c, variance, partial, S, epsilon, perChannel, out);
+	return check_launch("pool_act_bn_rop_backward");
 }
 
 int fitre_hip_pool_forward_routed(int poolType, const float *values, const float *z_act, int channels, int samples, int inA,

@@ -244,24 +244,31 @@ static void rop_backward(CNN_MODEL *model, const real *weights, const real *vect
 		const real *actIn = bn ? slab + l->batchNormOffset : slab;
 		const real *ractIn = bn ? rslab + l->batchNormOffset : rslab;
 		const real *actOut = conv_act_out(model, c, z, n, dout); /* dout is free once the FC layers are done */
-		/* R through the pooling: the routing of the gradient itself */
-		if (p->type == NO_POOL) {
-			t = rdelta, rdelta = rnext, rnext = t; /* rnext now holds R{delta at the activation output} */
-		} else {
-			HIP_CALL(fitre_hip_pool_backward(p->type, rdelta, actOut, l->outChannels, n, p->width, p->height, p->pSize, p->stride,
-			                                 p->padding, p->outWidth, p->outHeight, rnext));
-		}
-		/* R{delta f'(x)}; delta at the activation output is the dx snapshot at +0 */
-		HIP_CALL(fitre_hip_activation_rop_backward(model->actFuns[c], rnext, dslab, actIn, actOut, ractIn, rdelta, count));
 		const real *dc = dslab + l->activationOffset; /* gradient at the convolution output */
-		real *rdc = rdelta;
+		real *rdc;
 		if (bn) {
-			HIP_CALL(fitre_hip_batch_norm_rop_backward(rdelta, dslab + l->activationOffset, slab + l->batchNormOffset,
-			                                           rslab + l->batchNormOffset, rslab, dslab + l->batchNormOffset,
-			                                           slab + l->batchNormOffset + l->variancesOffset, l->outChannels, perChannel,
-			                                           (real)BATCH_NORM_EPSILON, rnext, ws, wsBytes));
+			/* routing through the pooling, R{delta f'(x)} and the batch-norm R-step: one pass that leaves the sums, one that
+			 * applies the formula (the separate passes where the shape does not allow it).  delta at the activation output is
+			 * the dx snapshot at +0; tmp takes the routed R{delta} when the passes run separately. */
+			const int pooled = p->type != NO_POOL;
+			HIP_CALL(fitre_hip_pool_act_bn_rop_backward(
+			    p->type, model->actFuns[c], rdelta, dslab, slab + l->batchNormOffset, actOut, rslab + l->batchNormOffset,
+			    dslab + l->activationOffset, rslab, dslab + l->batchNormOffset, slab + l->batchNormOffset + l->variancesOffset,
+			    l->outChannels, n, pooled ? p->width : l->outWidth, pooled ? p->height : l->outHeight, p->pSize, p->stride, p->padding,
+			    p->outWidth, p->outHeight, (real)BATCH_NORM_EPSILON, tmp, rnext, rdelta, ws, wsBytes));
 			dc = dslab + l->batchNormOffset;
-			rdc = rnext;
+			rdc = rdelta;
+		} else {
+			/* R through the pooling: the routing of the gradient itself */
+			if (p->type == NO_POOL) {
+				t = rdelta, rdelta = rnext, rnext = t; /* rnext now holds R{delta at the activation output} */
+			} else {
+				HIP_CALL(fitre_hip_pool_backward(p->type, rdelta, actOut, l->outChannels, n, p->width, p->height, p->pSize, p->stride,
+				                                 p->padding, p->outWidth, p->outHeight, rnext));
+			}
+			/* R{delta f'(x)}; delta at the activation output is the dx snapshot at +0 */
+			HIP_CALL(fitre_hip_activation_rop_backward(model->actFuns[c], rnext, dslab, actIn, actOut, ractIn, rdelta, count));
+			rdc = rdelta;
 		}
 		if (bias) HIP_CALL(fitre_hip_channel_sum(rdc, l->outChannels, perChannel, hv + bOffsets[c], ws, wsBytes));
 		const real *in = (c == 0) ? x : z + zOffsets[c] + model->convLayer[c - 1].outputOffset;

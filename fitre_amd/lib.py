@@ -128,6 +128,8 @@ HIP_API = {
     "fitre_hip_pool_forward_routed": (i32, [i32, vp, vp] + [i32] * 9 + [vp]),
     "fitre_hip_bn_act_pool_rop_forward": (i32, [vp, vp, vp, vp, i32, i32, i32, i32, f32, i32, vp, vp, i32, i32, i32, i32, i32, i32, vp, vp,
                                                 sz]),
+    "fitre_hip_pool_act_bn_rop_backward": (i32, [i32, i32, vp, vp, vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, i32, i32,
+                                                 f32, vp, vp, vp, vp, sz]),
     "fitre_hip_batch_norm_rop_backward": (i32, [vp, vp, vp, vp, vp, vp, vp, i32, lng, f32, vp, vp, sz]),
     "fitre_hip_cross_entropy_rop_error": (i32, [vp, vp, i32, i32, vp]),
     "fitre_hip_fc_rop_backward": (i32, [i32, vp, vp, vp, vp, vp, lng]),

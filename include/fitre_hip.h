@@ -480,6 +480,20 @@ int fitre_hip_bn_act_pool_rop_forward(const float *rx, const float *zhat, const 
 int fitre_hip_batch_norm_rop_backward(const float *rdelta_x, const float *delta_x, const float *zhat, const float *rzhat,
                                       const float *rx, const float *delta_c, const float *variance, int channels,
                                       long perChannel, float epsilon, float *out, void *ws, size_t wsBytes);
+/* The backward sweep's R-steps between a layer's pooled R{delta} and R{delta at the convolution output}
+ * (functions/cnn_hv_backward.cu:328-754): fitre_hip_pool_backward of rdelta (routing by the arg-max of z_act),
+ * fitre_hip_activation_rop_backward (delta = the gradient at the activation output, zhat = the activation input, rzhat =
+ * its directional derivative) into rdeltaX, and fitre_hip_batch_norm_rop_backward of that into out -- as TWO launches
+ * where the shape allows: one pass routes, applies the activation's R-step and leaves the five sums, the second applies
+ * the batch-norm formula.  Fused for no pooling and 2x2 / stride 2 max pooling (A even, B a multiple of 4, 16-byte-aligned
+ * tensors); z_act may then be NULL for ReLU, and rdeltaAct (the routed R{delta}, only written by the separate passes) may
+ * be NULL.  Every other case runs the three calls.  Workspace: fitre_hip_batch_norm_workspace(channels, samples * inA * inB),
+ * at least channels * segments * 64 bytes. */
+int fitre_hip_pool_act_bn_rop_backward(int poolType, int actFun, const float *rdelta, const float *delta, const float *zhat,
+                                       const float *z_act, const float *rzhat, const float *delta_x, const float *rx,
+                                       const float *delta_c, const float *variance, int channels, int samples, int inA,
+                                       int inB, int ksize, int stride, int padding, int outA, int outB, float epsilon,
+                                       float *rdeltaAct, float *rdeltaX, float *out, void *ws, size_t wsBytes);
 /* The R-operator over a fully connected model (functions/eval_hessian_vec.cu):
  * fc_rop_backward: out = f'(z) rdz + rx g(z) dx, the directional derivative of dx = f'(z) dz written with dx
  *   itself (eval_backprop_hessian, functions/dev_hessian_helpers.cu:7-15: logistic, g = 1 - 2 z; tanh here too,

@@ -419,6 +419,52 @@ def test_fused_directional_derivative_forward(dev, geom, kind, act, derive):
     dev.free(ws)
 
 
+@pytest.mark.parametrize("act,derive", [(CNN_ACT_RELU, False), (CNN_ACT_RELU, True), (CNN_ACT_SWISH, False)])
+@pytest.mark.parametrize("kind", [MAX_POOL, NO_POOL])
+@pytest.mark.parametrize("geom", [(3, 40, 16, 16, 2, 2, 0), (64, 8, 32, 32, 2, 2, 0), (5, 9, 6, 12, 2, 2, 0), (160, 7, 8, 8, 2, 2, 0),
+                                  (2, 4, 6, 10, 2, 2, 0), (2, 2, 7, 5, 3, 2, 1)])
+def test_fused_directional_derivative_backward(dev, geom, kind, act, derive):
+    """Pooling routing, R{delta f'(x)} and the batch-norm R-step of a layer in one call against the three separate entry
+    points (fused shapes and those that fall back); `derive`: without the activation output, which only ReLU allows."""
+    Cn, N, A, B, k, s, p = geom
+    oA, oB = ((A + 2 * p - k) // s + 1, (B + 2 * p - k) // s + 1) if kind != NO_POOL else (A, B)
+    per = N * A * B
+    fusable = (kind == NO_POOL or (k == 2 and B % 4 == 0 and A % 2 == 0)) and per % 4 == 0
+    rng = np.random.default_rng(Cn * 5 + A * B + act)
+    full = lambda: dev.upload(rng.standard_normal(Cn * per).astype(np.float32))
+    pzh, pdelta, prz, pdx, prx, pdc = (full() for _ in range(6))
+    prd = dev.upload(rng.standard_normal(Cn * N * oA * oB).astype(np.float32))
+    pvar = dev.upload((rng.random(Cn) + 0.5).astype(np.float32))
+    zact = dev.zeros(Cn * per)
+    ok(hip.fitre_hip_activation_forward(act, pzh, zact, Cn * per))
+    ws, nb = bn_ws(dev, Cn, per)
+
+    def run(fused):
+        routed, rdx, out = dev.zeros(Cn * per), dev.zeros(Cn * per), dev.zeros(Cn * per)
+        if fused:
+            rc = hip.fitre_hip_pool_act_bn_rop_backward(kind, act, prd, pdelta, pzh, None if derive else zact, prz, pdx, prx, pdc, pvar, Cn, N,
+                                                        A, B, k, s, p, oA, oB, 1e-5, routed, rdx, out, ws, nb)
+            if derive and not fusable:
+                assert rc != 0                       # the separate passes need the activation output
+                return None
+            ok(rc)
+        else:
+            src = prd
+            if kind != NO_POOL:
+                ok(hip.fitre_hip_pool_backward(kind, prd, zact, Cn, N, A, B, k, s, p, oA, oB, routed))
+                src = routed
+            ok(hip.fitre_hip_activation_rop_backward(act, src, pdelta, pzh, zact, prz, rdx, Cn * per))
+            ok(hip.fitre_hip_batch_norm_rop_backward(rdx, pdx, pzh, prz, prx, pdc, pvar, Cn, per, 1e-5, out, ws, nb))
+        return [dev.download(b, Cn * per) for b in (rdx, out)]
+
+    want, got = run(False), run(True)
+    if got is not None:
+        assert rel_err(got[0], want[0]) < 1e-6
+        np.testing.assert_array_equal(got[0] == 0, want[0] == 0)   # the same routing and the same masks
+        assert rel_err(got[1], want[1]) < 1e-5
+    dev.free(ws)
+
+
 # C, N, A, B, k, s, p: fused sums (large channels), one-workgroup-per-channel (short channels, >= 128
 # of them), and shapes that fall back to the separate passes
 FUSED_BN_GEOMS = [
