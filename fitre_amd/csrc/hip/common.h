@@ -51,6 +51,39 @@ struct BatchedProduct {
 };
 int gemm_pair_batched(int batch, const BatchedProduct &first, const BatchedProduct &second, int kernelClass, void *ws, size_t wsBytes,
                       long wsStrideBytes);
+
+// ---- float64 products (dense_f64.hip) -------------------------------------------------------
+// A matrix operand: element (r, c) of floats or doubles at r * rs + c * cs; kind FITRE_MAT_SYM_PAIR: a symmetric
+// matrix of order rs kept as a pair of floats per element in one dense float matrix with leading dimension cs (the
+// rounded value on and above the diagonal, the remainder below it; see fitre_matrix in fitre_hip.h).
+struct DMat {
+	const void *p;
+	long rs, cs;       // element (r, c) at r * rs + c * cs (pair of floats: order rs, column-major with leading dimension cs)
+	int kind;          // FITRE_MAT_*
+	long onesRow, onesCol; // floats only: a row / column that is not in memory and reads as onesValue (-1: none)
+	double onesValue;
+};
+
+struct DOut {
+	void *p;
+	long rs, cs;
+	int kind;
+};
+inline DMat dmat64(const double *p, long rs, long cs) { return DMat{ p, rs, cs, FITRE_MAT_F64, -1, -1, 0.0 }; }
+inline DMat dmat32(const float *p, long rs, long cs) { return DMat{ p, rs, cs, FITRE_MAT_F32, -1, -1, 0.0 }; }
+// kDgMirror: symmetric product (M == N, C = C^T): only the tiles on and above the diagonal are computed, the others
+// mirrored.  Reduction ranges: A(i, k) is zero for k > i (kDgALower) / k < i (kDgAUpper), B(k, j) is zero for k < j
+// (kDgBLower) / k > j (kDgBUpper).
+constexpr int kDgMirror = 1, kDgALower = 2, kDgAUpper = 4, kDgBLower = 8, kDgBUpper = 16;
+// C(M x N) = alpha * A(M x K) * B(K x N) + beta * C, plus diagAdd on the diagonal, accumulated in float64 on the
+// matrix pipes; queued on the selected lane.  ws: dgemm_workspace bytes, 256-byte aligned (a smaller one costs splits).
+int dgemm(long M, long N, long K, double alpha, DMat A, DMat B, double beta, DOut C, double diagAdd, int flags, int kernelClass,
+          void *ws, size_t wsBytes);
+size_t dgemm_workspace(long M, long N, long K, int flags);
+// result = W^-1 for the symmetric positive definite W (n x n doubles, destroyed), stored dense with leading dimension
+// n as `kind`; pivotInfo (device int): 0, or the 1-based index of the first non-positive pivot.
+int dspd_inverse_run(double *W, int n, void *result, int kind, void *ws, size_t wsBytes, int *pivotInfo);
+size_t dspd_inverse_workspace(int n);
 constexpr int kMaxLanes = 4; // one hardware queue each
 int lane();           // its index (0 .. kMaxLanes - 1)
 int lane_compute_units();     // compute units a kernel launched on the selected lane can occupy

@@ -297,4 +297,80 @@ int fitre_hip_kfac_fc_output_factor(const float *delta, int outDim, int samples,
 	                                                   (double)outDim * (outDim + 1) * (double)samples);
 }
 
+// ---- the same factors accumulated in float64 -----------------------------------------------------------------
+size_t fitre_hip_kfac_conv_input_factor_f64_workspace(const fitre_conv_shape *s, int withBias)
+{
+	if (!s) return 0;
+	const long n = (long)s->inChannels * s->ksize * s->ksize + (withBias ? 1 : 0);
+	return patch_rows_bytes(s) + dgemm_workspace(n, n, (long)s->samples * s->outA * s->outB, kDgMirror);
+}
+
+int fitre_hip_kfac_conv_input_factor_f64(const fitre_conv_shape *s, const float *x, int withBias, double shift, double *factor,
+                                         void *ws, size_t wsBytes)
+{
+	FITRE_NEED_INIT();
+	int rc = check_conv("fitre_hip_kfac_conv_input_factor_f64", s);
+	if (rc) return rc;
+	FITRE_REQUIRE(x && factor && ws, "fitre_hip_kfac_conv_input_factor_f64: null pointer");
+	FITRE_REQUIRE((((uintptr_t)ws) & 255) == 0, "fitre_hip_kfac_conv_input_factor_f64: workspace must be 256-byte aligned");
+	const int K = s->inChannels * s->ksize * s->ksize, n = K + (withBias ? 1 : 0);
+	const long R = (long)s->samples * s->outA * s->outB;
+	const size_t rowBytes = patch_rows_bytes(s);
+	if (wsBytes < rowBytes)
+		return fail(FITRE_E_WORKSPACE, "fitre_hip_kfac_conv_input_factor_f64: workspace of %zu bytes is smaller than the %zu of the patch rows",
+		            wsBytes, rowBytes);
+	const double cells = (double)(s->outA * s->outB);
+	PatchGeom g = make_patch_geom(x, s->inChannels, s->samples, s->inA, s->inB, s->outA, s->outB, s->ksize, s->stride, s->padding);
+	float *rows = (float *)ws;
+	{
+		LaunchScope scope(FITRE_KC_BLAS1, 2.0 * (double)rowBytes);
+		const dim3 grid(blocks_for(R, 256, 64), (unsigned)K);
+		patch_rows_kernel<<<grid, 256, 0, stream()>>>(g, rows);
+	}
+	// rows of P^T unscaled, the row of ones as outA * outB: one factor 1 / (cells^2 * samples) on the product gives P^T P / samples
+	DMat a = dmat32(rows, R, 1);
+	if (withBias) a.onesRow = K, a.onesValue = cells;
+	DMat b = a;
+	b.rs = a.cs, b.cs = a.rs, b.onesRow = -1, b.onesCol = a.onesRow;
+	return dgemm(n, n, R, 1.0 / (cells * cells * (double)s->samples), a, b, 0.0, DOut{ factor, 1, n, FITRE_MAT_F64 }, shift, kDgMirror,
+	             FITRE_KC_KFAC_FACTOR, (char *)ws + rowBytes, wsBytes - rowBytes);
+}
+
+int fitre_hip_kfac_conv_output_factor_f64(const fitre_conv_shape *s, const float *delta, double shift, double *factor, void *ws,
+                                          size_t wsBytes)
+{
+	FITRE_NEED_INIT();
+	int rc = check_conv("fitre_hip_kfac_conv_output_factor_f64", s);
+	if (rc) return rc;
+	FITRE_REQUIRE(delta && factor, "fitre_hip_kfac_conv_output_factor_f64: null pointer");
+	const int n = s->outChannels;
+	const long R = (long)s->samples * s->outA * s->outB;
+	return dgemm(n, n, R, (double)R, dmat32(delta, R, 1), dmat32(delta, 1, R), 0.0, DOut{ factor, 1, n, FITRE_MAT_F64 }, shift, kDgMirror,
+	             FITRE_KC_KFAC_FACTOR, ws, wsBytes);
+}
+
+int fitre_hip_kfac_fc_input_factor_f64(const float *z, int in, int samples, int withBias, double shift, double *factor, void *ws,
+                                       size_t wsBytes)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(z && factor, "fitre_hip_kfac_fc_input_factor_f64: null pointer");
+	FITRE_REQUIRE(in > 0 && samples > 0, "fitre_hip_kfac_fc_input_factor_f64: non-positive shape %d x %d", in, samples);
+	const int n = in + (withBias ? 1 : 0);
+	DMat a = dmat32(z, 1, in);
+	if (withBias) a.onesRow = in, a.onesValue = 1.0;
+	DMat b = a;
+	b.rs = a.cs, b.cs = a.rs, b.onesRow = -1, b.onesCol = a.onesRow;
+	return dgemm(n, n, samples, 1.0 / (double)samples, a, b, 0.0, DOut{ factor, 1, n, FITRE_MAT_F64 }, shift, kDgMirror, FITRE_KC_KFAC_FACTOR, ws,
+	             wsBytes);
+}
+
+int fitre_hip_kfac_fc_output_factor_f64(const float *delta, int outDim, int samples, double shift, double *factor, void *ws, size_t wsBytes)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(delta && factor, "fitre_hip_kfac_fc_output_factor_f64: null pointer");
+	FITRE_REQUIRE(outDim > 0 && samples > 0, "fitre_hip_kfac_fc_output_factor_f64: non-positive shape %d x %d", outDim, samples);
+	return dgemm(outDim, outDim, samples, (double)samples, dmat32(delta, 1, outDim), dmat32(delta, outDim, 1), 0.0,
+	             DOut{ factor, 1, outDim, FITRE_MAT_F64 }, shift, kDgMirror, FITRE_KC_KFAC_FACTOR, ws, wsBytes);
+}
+
 } // extern "C"

@@ -140,25 +140,57 @@ void computeLambdaDeltaFactors(KFAC_CURVATURE_INFO *kfac_info, CNN_MODEL *model,
 
 /* ---- inverses ------------------------------------------------------------------------------ */
 
+static size_t round_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+static char *aligned_base(real *devPtr) { return (char *)(((size_t)devPtr + 255) & ~(size_t)255); }
+
+/* The reference inverts in double (cusolverDnDpotrf / Dpotrs with real = double, solvers/kfac_inverses.cu:133-186);
+ * so does this: the float matrix is widened, inverted in float64 and the inverse rounded to floats. */
 void computeMatrixInverse(real *matrix, real *inverse, int n, real *devPtr, real lambda, real dampGamma)
 {
-	int info = -1;
-	int rc = fitre_hip_spd_inverse(matrix, n, lambda + dampGamma, inverse, devPtr, fitre_hip_spd_inverse_workspace(n), &info);
-	if (rc != FITRE_OK) {
-		if (info > 0)
-			fprintf(stderr, "We have a problem with the LU factorization ... %d\n", info);
-		else
-			fprintf(stderr, "computeMatrixInverse: error %d: %s\n", rc, fitre_hip_last_error());
+	char *base = aligned_base(devPtr);
+	const size_t matBytes = round_up((size_t)n * n * sizeof(double), 256);
+	int *pivot = (int *)(base + matBytes);
+	int host = 0;
+	HIP_CALL(fitre_hip_widen_shift(matrix, n, (double)lambda + (double)dampGamma, (double *)base));
+	HIP_CALL(fitre_hip_spd_inverse_f64_queued((double *)base, n, inverse, FITRE_MAT_F32, base + matBytes + 256,
+	                                          fitre_hip_spd_inverse_f64_workspace(n), pivot));
+	HIP_CALL(fitre_hip_sync());
+	HIP_CALL(fitre_hip_copy_d2h(&host, pivot, sizeof(int)));
+	if (host != 0) {
+		fprintf(stderr, "We have a problem with the LU factorization ... %d\n", host);
 		exit(-1);
 	}
 }
 
-static size_t round_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+long matrixInverseMemRequired(int n)
+{
+	return (long)((round_up((size_t)n * n * sizeof(double), 256) + 512 + fitre_hip_spd_inverse_f64_workspace(n)) / sizeof(real)) + 64;
+}
 
-/* layout of the scratch of the two inverse passes: [factor | workspace of its product or inverse] */
+/* workspace of the float64 factor products of a pass */
+static size_t factor64_ws_bytes(const CNN_MODEL *model, int samples)
+{
+	size_t bytes = 0;
+	int withBias = model->bias != 0;
+	for (int l = 0; l < model->cLayers; l++) {
+		const CONV_LAYER *c = &model->convLayer[l];
+		fitre_conv_shape s = conv_shape(c, samples);
+		bytes = max_sz(bytes, fitre_hip_kfac_conv_input_factor_f64_workspace(&s, withBias));
+		bytes = max_sz(bytes, fitre_hip_gemm_f64_workspace(c->outChannels, c->outChannels, (long)samples * c->outHeight * c->outWidth,
+		                                                   FITRE_GEMM_SYMMETRIC));
+	}
+	for (int l = 0; l < model->lLayers; l++) {
+		const FC_LAYER *f = &model->fcLayer[l];
+		bytes = max_sz(bytes, fitre_hip_gemm_f64_workspace(f->in + 1, f->in + 1, samples, FITRE_GEMM_SYMMETRIC));
+		bytes = max_sz(bytes, fitre_hip_gemm_f64_workspace(f->out, f->out, samples, FITRE_GEMM_SYMMETRIC));
+	}
+	return bytes;
+}
+
+/* layout of one slot of the scratch of the two inverse passes: [factor (doubles) | workspace of its product or inverse] */
 static size_t inverse_scratch_bytes(const CNN_MODEL *model, int samples, size_t *factorBytes)
 {
-	size_t order = 1, ws = factor_ws_bytes(model, samples);
+	size_t order = 1, ws = factor64_ws_bytes(model, samples);
 	for (int l = 0; l < model->cLayers; l++) {
 		const CONV_LAYER *c = &model->convLayer[l];
 		size_t k = (size_t)c->inChannels * c->kSize * c->kSize + 1;
@@ -166,36 +198,26 @@ static size_t inverse_scratch_bytes(const CNN_MODEL *model, int samples, size_t 
 	}
 	for (int l = 0; l < model->lLayers; l++)
 		order = max_sz(order, max_sz((size_t)model->fcLayer[l].in + 1, (size_t)model->fcLayer[l].out));
-	ws = max_sz(ws, fitre_hip_spd_inverse_workspace((int)order));
-	*factorBytes = round_up(order * order * sizeof(real), 256);
+	ws = max_sz(ws, fitre_hip_spd_inverse_f64_workspace((int)order));
+	*factorBytes = round_up(order * order * sizeof(double), 256);
 	return *factorBytes + round_up(ws, 256) + 256;
 }
 
-static char *aligned_base(real *devPtr) { return (char *)(((size_t)devPtr + 255) & ~(size_t)255); }
-
-/* The inverses of a pass are independent of each other.  Consecutive layers whose factors have the same order
- * (the wide layers at the end of a VGG) are inverted as ONE batch -- one chain of launches, each covering all
- * matrices of the batch -- and the batches are dealt, costliest first, to the four lanes.  Every lane owns as
- * many [factor | workspace] slots as the largest batch it accepts; the pivot reports are read once at the end. */
+/* The inverses of a pass are independent of each other: they are dealt, costliest first, to the four lanes, each
+ * of which owns one [factor | workspace] slot; the pivot reports are read once at the end. */
 #define KFAC_LANES 4
-#define KFAC_SLOTS 7
-#define KFAC_MAX_BATCH 3
-#define KFAC_MIN_BATCH_ORDER 1024
-#define KFAC_INFO_BYTES 1024 /* one int per layer, MAX_LAYERS of them */
-static const int kLaneSlots[KFAC_LANES] = { 3, 2, 1, 1 };
-static const int kLaneFirstSlot[KFAC_LANES] = { 0, 3, 5, 6 };
+#define KFAC_INFO_BYTES 1024 /* one int per matrix, 2 * MAX_LAYERS of them */
 
 long kfacInverseMemRequired(CNN_MODEL *model, int samples)
 {
 	size_t factorBytes;
-	return (long)((KFAC_SLOTS * inverse_scratch_bytes(model, samples, &factorBytes) + KFAC_INFO_BYTES) / sizeof(real)) + 64;
+	return (long)((KFAC_LANES * inverse_scratch_bytes(model, samples, &factorBytes) + KFAC_INFO_BYTES) / sizeof(real)) + 64;
 }
 
-/* writes the factor of `layer` (convolution layers, then linear ones) into `factor` */
-typedef void (*FACTOR_FN)(void *ctx, int layer, real *factor, real *ws, size_t wsBytes);
+/* writes the float64 factor of `layer` (convolution layers, then linear ones), damping included, into `factor` */
+typedef void (*FACTOR_FN)(void *ctx, int layer, double shift, double *factor, void *ws, size_t wsBytes);
 
-/* one matrix of a pass: how to make its factor, its order, where its inverse goes.  Consecutive items may share a
- * batch when they have the same order and group and their inverses are `stride` reals apart. */
+/* one matrix of a pass: how to make its factor, its order, where its inverse goes */
 typedef struct inverse_item {
 	FACTOR_FN make;
 	void *ctx;
@@ -203,25 +225,26 @@ typedef struct inverse_item {
 	int order;
 	int group;
 	real *inverse;
-	long stride; /* room behind `inverse` up to the next layer's slot */
 } INVERSE_ITEM;
 
 typedef struct inverse_job {
-	int first, count; /* items first .. first+count-1 */
+	int item;
 	double cost;
-	int lane;
 } INVERSE_JOB;
 
 static int job_by_cost(const void *a, const void *b)
 {
 	const INVERSE_JOB *x = (const INVERSE_JOB *)a, *y = (const INVERSE_JOB *)b;
 	if (x->cost != y->cost) return x->cost < y->cost ? 1 : -1;
-	return x->first - y->first;
+	return x->item - y->item;
 }
 
 #define KFAC_MAX_ITEMS (2 * MAX_LAYERS)
 
-static void inverse_pass_run(const CNN_MODEL *model, int samples, real *devPtr, const INVERSE_ITEM *items, int count, real shift)
+/* Every item: the factor in float64 with the damping on its diagonal, its float64 inverse, and the inverse stored in
+ * the caller's n x n floats as a float pair per element (FITRE_MAT_SYM_PAIR): computeNaturalGradient, the only reader
+ * of these arrays (solvers/kfac_natural_gradient.cu:55-56), takes them in that form. */
+static void inverse_pass_run(const CNN_MODEL *model, int samples, real *devPtr, const INVERSE_ITEM *items, int count, double shift)
 {
 	size_t factorBytes;
 	const size_t slotBytes = inverse_scratch_bytes(model, samples, &factorBytes);
@@ -230,51 +253,26 @@ static void inverse_pass_run(const CNN_MODEL *model, int samples, real *devPtr, 
 	int *pivots = (int *)base;
 	char *slots = base + KFAC_INFO_BYTES;
 
-	/* batches: runs of consecutive items of one order, at most KFAC_MAX_BATCH long */
 	INVERSE_JOB jobs[KFAC_MAX_ITEMS];
-	int nJobs = 0;
-	for (int i = 0; i < count;) {
-		int n = 1;
-		/* small matrices gain nothing from a shared chain (measured: the output-side factors, orders up to 512, are
-		 * faster with one lane per matrix) */
-		while (items[i].order >= KFAC_MIN_BATCH_ORDER && i + n < count && n < KFAC_MAX_BATCH && items[i + n].order == items[i].order &&
-		       items[i + n].group == items[i].group && items[i + n].stride == items[i].stride &&
-		       items[i + n].inverse == items[i + n - 1].inverse + items[i].stride)
-			n++;
-		INVERSE_JOB *j = &jobs[nJobs++];
-		j->first = i;
-		j->count = n;
-		/* measured: the time of an inverse grows a little slower than n^2, and a batch pays for the chain once */
-		j->cost = (double)items[i].order * items[i].order * (0.6 + 0.4 * n);
-		i += n;
+	for (int i = 0; i < count; i++) {
+		jobs[i].item = i;
+		/* a chain of launches whose length grows with the order, plus the arithmetic */
+		jobs[i].cost = (double)items[i].order * (200.0 + (double)items[i].order * items[i].order * 1e-3);
 	}
-	qsort(jobs, (size_t)nJobs, sizeof(INVERSE_JOB), job_by_cost);
+	qsort(jobs, (size_t)count, sizeof(INVERSE_JOB), job_by_cost);
 	double load[KFAC_LANES] = { 0, 0, 0, 0 };
-	for (int i = 0; i < nJobs; i++) {
-		int lane = -1;
-		for (int k = 0; k < KFAC_LANES; k++)
-			if (kLaneSlots[k] >= jobs[i].count && (lane < 0 || load[k] < load[lane])) lane = k;
-		jobs[i].lane = lane;
-		load[lane] += jobs[i].cost;
-	}
-
 	for (int k = 1; k < KFAC_LANES; k++) HIP_CALL(fitre_hip_lane_wait(k, 0)); /* after what lane 0 has queued so far (z, dx) */
-	for (int i = 0; i < nJobs; i++) {
-		const INVERSE_JOB *j = &jobs[i];
-		const INVERSE_ITEM *it = &items[j->first];
-		char *slot0 = slots + (size_t)kLaneFirstSlot[j->lane] * slotBytes;
-		HIP_CALL(fitre_hip_lane_select(j->lane));
-		for (int b = 0; b < j->count; b++) {
-			char *slot = slot0 + (size_t)b * slotBytes;
-			it[b].make(it[b].ctx, it[b].layer, (real *)slot, (real *)(slot + factorBytes), wsBytes);
-		}
-		if (j->count == 1)
-			HIP_CALL(fitre_hip_spd_inverse_queued((real *)slot0, it->order, shift, it->inverse, slot0 + factorBytes, wsBytes,
-			                                      pivots + j->first));
-		else
-			HIP_CALL(fitre_hip_spd_inverse_batched_queued(j->count, (real *)slot0, (long)(slotBytes / sizeof(real)), it->order, shift,
-			                                              it->inverse, it->stride, slot0 + factorBytes, wsBytes, (long)slotBytes,
-			                                              pivots + j->first));
+	for (int i = 0; i < count; i++) {
+		const INVERSE_ITEM *it = &items[jobs[i].item];
+		int lane = 0;
+		for (int k = 1; k < KFAC_LANES; k++)
+			if (load[k] < load[lane]) lane = k;
+		load[lane] += jobs[i].cost;
+		char *slot = slots + (size_t)lane * slotBytes;
+		HIP_CALL(fitre_hip_lane_select(lane));
+		it->make(it->ctx, it->layer, shift, (double *)slot, slot + factorBytes, wsBytes);
+		HIP_CALL(fitre_hip_spd_inverse_f64_queued((double *)slot, it->order, it->inverse, FITRE_MAT_SYM_PAIR, slot + factorBytes, wsBytes,
+		                                          pivots + jobs[i].item));
 	}
 	int host[KFAC_MAX_ITEMS];
 	HIP_CALL(fitre_hip_lane_select(0));
@@ -296,7 +294,7 @@ typedef struct omega_ctx {
 	const int *zOffsets, *zztOffsets;
 } OMEGA_CTX;
 
-static void omega_factor(void *ctx, int layer, real *factor, real *ws, size_t wsBytes)
+static void omega_factor(void *ctx, int layer, double shift, double *factor, void *ws, size_t wsBytes)
 {
 	const OMEGA_CTX *o = (const OMEGA_CTX *)ctx;
 	const CNN_MODEL *model = o->model;
@@ -310,7 +308,7 @@ static void omega_factor(void *ctx, int layer, real *factor, real *ws, size_t ws
 		else
 			input = (l == 0) ? o->data->currentBatch : o->dampedZ + o->zOffsets[l] + model->convLayer[l - 1].outputOffset;
 		fitre_conv_shape s = conv_shape(c, o->samples);
-		HIP_CALL(fitre_hip_kfac_conv_input_factor(&s, input, o->withBias, factor, ws, wsBytes));
+		HIP_CALL(fitre_hip_kfac_conv_input_factor_f64(&s, input, o->withBias, shift, factor, ws, wsBytes));
 	} else {
 		const int l = layer - nc;
 		const FC_LAYER *f = &model->fcLayer[l];
@@ -321,7 +319,7 @@ static void omega_factor(void *ctx, int layer, real *factor, real *ws, size_t ws
 			input = o->dampedZ + o->zOffsets[nc] + model->convLayer[nc - 1].outputOffset;
 		else
 			input = o->dampedZ + o->zOffsets[nc + l];
-		HIP_CALL(fitre_hip_kfac_fc_input_factor(input, f->in, o->samples, o->withBias, factor, ws, wsBytes));
+		HIP_CALL(fitre_hip_kfac_fc_input_factor_f64(input, f->in, o->samples, o->withBias, shift, factor, ws, wsBytes));
 	}
 }
 
@@ -345,7 +343,6 @@ static int omega_items(INVERSE_ITEM *items, const KFAC_CURVATURE_INFO *kfac_info
 			it->group = 1;
 		}
 		it->inverse = omegaZInv + omega[l];
-		it->stride = (long)omega[l + 1] - omega[l];
 	}
 	return layers;
 }
@@ -358,7 +355,7 @@ void computeOmegaZ(KFAC_CURVATURE_INFO *kfac_info, CNN_MODEL *model, DEVICE_DATA
 	OMEGA_CTX ctx = { model, data, samples, model->bias != 0, dampedInput, dampedZ, zOffsets, zztOffsets };
 	INVERSE_ITEM items[KFAC_MAX_ITEMS];
 	const int count = omega_items(items, kfac_info, model, &ctx, omegaZInv);
-	inverse_pass_run(model, samples, devPtr, items, count, kfac_info->regLambda + kfac_info->dampGamma);
+	inverse_pass_run(model, samples, devPtr, items, count, (double)kfac_info->regLambda + (double)kfac_info->dampGamma);
 }
 
 typedef struct lambda_ctx {
@@ -368,7 +365,7 @@ typedef struct lambda_ctx {
 	const int *zOffsets, *zztOffsets;
 } LAMBDA_CTX;
 
-static void lambda_factor(void *ctx, int layer, real *factor, real *ws, size_t wsBytes)
+static void lambda_factor(void *ctx, int layer, double shift, double *factor, void *ws, size_t wsBytes)
 {
 	const LAMBDA_CTX *o = (const LAMBDA_CTX *)ctx;
 	const CNN_MODEL *model = o->model;
@@ -384,12 +381,12 @@ static void lambda_factor(void *ctx, int layer, real *factor, real *ws, size_t w
 		else
 			delta = o->dx + o->zOffsets[l + 1] + c->batchNormOffset;
 		fitre_conv_shape s = conv_shape(c, o->samples);
-		HIP_CALL(fitre_hip_kfac_conv_output_factor(&s, delta, factor, ws, wsBytes));
+		HIP_CALL(fitre_hip_kfac_conv_output_factor_f64(&s, delta, shift, factor, ws, wsBytes));
 	} else {
 		const int l = layer - nc;
 		const FC_LAYER *f = &model->fcLayer[l];
 		const real *delta = (o->dampedLambda != NULL) ? o->dampedLambda + o->zztOffsets[nc + l + 1] : o->dx + o->zOffsets[nc + l + 1];
-		HIP_CALL(fitre_hip_kfac_fc_output_factor(delta, f->out, o->samples, factor, ws, wsBytes));
+		HIP_CALL(fitre_hip_kfac_fc_output_factor_f64(delta, f->out, o->samples, shift, factor, ws, wsBytes));
 	}
 }
 
@@ -406,7 +403,6 @@ static int lambda_items(INVERSE_ITEM *items, const KFAC_CURVATURE_INFO *kfac_inf
 		it->order = l < nc ? model->convLayer[l].outChannels : model->fcLayer[l - nc].out;
 		it->group = l < nc ? 2 : 3;
 		it->inverse = lambdaGInv + lambda[l];
-		it->stride = (long)lambda[l + 1] - lambda[l];
 	}
 	return layers;
 }
@@ -419,7 +415,7 @@ void computeLambdaDelta(KFAC_CURVATURE_INFO *kfac_info, CNN_MODEL *model, int sa
 	LAMBDA_CTX ctx = { model, samples, dx, dampedLambda, zOffsets, zztOffsets };
 	INVERSE_ITEM items[KFAC_MAX_ITEMS];
 	const int count = lambda_items(items, kfac_info, model, &ctx, lambdaGInv);
-	inverse_pass_run(model, samples, devPtr, items, count, kfac_info->regLambda + kfac_info->dampGamma);
+	inverse_pass_run(model, samples, devPtr, items, count, (double)kfac_info->regLambda + (double)kfac_info->dampGamma);
 }
 
 void computeOmegaZAndLambdaDelta(KFAC_CURVATURE_INFO *kfac_info, CNN_MODEL *model, DEVICE_DATASET *data, int samples,
@@ -431,7 +427,7 @@ void computeOmegaZAndLambdaDelta(KFAC_CURVATURE_INFO *kfac_info, CNN_MODEL *mode
 	INVERSE_ITEM items[KFAC_MAX_ITEMS];
 	int count = omega_items(items, kfac_info, model, &octx, kfac_info->OmegaZInv);
 	count += lambda_items(items + count, kfac_info, model, &lctx, kfac_info->LambdaGInv);
-	inverse_pass_run(model, samples, devPtr, items, count, kfac_info->regLambda + kfac_info->dampGamma);
+	inverse_pass_run(model, samples, devPtr, items, count, (double)kfac_info->regLambda + (double)kfac_info->dampGamma);
 }
 
 /* ---- natural gradient ---------------------------------------------------------------------- */
@@ -443,14 +439,14 @@ static size_t natural_gradient_bytes(const CNN_MODEL *model, size_t *matBytes)
 	for (int l = 0; l < model->cLayers; l++) {
 		const CONV_LAYER *c = &model->convLayer[l];
 		int k = c->inChannels * c->kSize * c->kSize + b, o = c->outChannels;
-		mat = max_sz(mat, (size_t)k * o * sizeof(real));
-		ws = max_sz(ws, max_sz(fitre_hip_gemm_workspace(k, o, o), fitre_hip_gemm_workspace(k, o, k)));
+		mat = max_sz(mat, (size_t)k * o * sizeof(double));
+		ws = max_sz(ws, max_sz(fitre_hip_gemm_f64_workspace(k, o, o, 0), fitre_hip_gemm_f64_workspace(k, o, k, 0)));
 	}
 	for (int l = 0; l < model->lLayers; l++) {
 		const FC_LAYER *f = &model->fcLayer[l];
 		int k = f->in + b, o = f->out;
-		mat = max_sz(mat, (size_t)k * o * sizeof(real));
-		ws = max_sz(ws, max_sz(fitre_hip_gemm_workspace(o, k, o), fitre_hip_gemm_workspace(o, k, k)));
+		mat = max_sz(mat, (size_t)k * o * sizeof(double));
+		ws = max_sz(ws, max_sz(fitre_hip_gemm_f64_workspace(o, k, o, 0), fitre_hip_gemm_f64_workspace(o, k, k, 0)));
 	}
 	*matBytes = round_up(mat, 256);
 	return 3 * *matBytes + round_up(ws, 256) + 256;
@@ -460,6 +456,12 @@ long kfacNaturalGradientMemRequired(CNN_MODEL *model)
 {
 	size_t matBytes;
 	return (long)(natural_gradient_bytes(model, &matBytes) / sizeof(real)) + 64;
+}
+
+static fitre_matrix mat_of(const void *data, long rowStride, long colStride, int kind)
+{
+	fitre_matrix m = { data, rowStride, colStride, kind, -1, -1, 0.0 };
+	return m;
 }
 
 void computeNaturalGradient(CNN_MODEL *model, KFAC_CURVATURE_INFO *kfacInfo, real *devPtr, real *hostPtr)
@@ -473,17 +475,21 @@ void computeNaturalGradient(CNN_MODEL *model, KFAC_CURVATURE_INFO *kfacInfo, rea
 	size_t matBytes;
 	const size_t total = natural_gradient_bytes(model, &matBytes);
 	char *base = aligned_base(devPtr);
-	real *wb = (real *)base, *u = (real *)(base + matBytes), *zt = (real *)(base + 2 * matBytes);
+	real *wb = (real *)base, *zt = (real *)(base + 2 * matBytes);
+	double *u = (double *)(base + matBytes);
 	void *ws = base + 3 * matBytes;
 	const size_t wsBytes = total - 3 * matBytes - 256;
 
-	/* Convolution layers.  The reference forms Lambda * wb' * Omega (Cout x (K+1)) and transposes the
+	/* Both inverses are float pairs (inverse_pass_run); the two products of a layer accumulate in float64, the
+	 * first one's result stays in doubles, and only the natural gradient itself is rounded to floats.
+	 * Convolution layers.  The reference forms Lambda * wb' * Omega (Cout x (K+1)) and transposes the
 	 * weight part back; Lambda and Omega are symmetric, so the transposed product Omega * (wb * Lambda)
 	 * is the same matrix already in the parameter layout ((K+1) x Cout, one column per filter). */
 	for (int c = 0; c < nc; c++) {
 		const CONV_LAYER *l = &model->convLayer[c];
 		const int K = l->inChannels * l->kSize * l->kSize, O = l->outChannels, R = K + bias;
-		const real *omega = kfacInfo->OmegaZInv + omegaOff[c], *lambda = kfacInfo->LambdaGInv + lambdaOff[c];
+		const fitre_matrix omega = mat_of(kfacInfo->OmegaZInv + omegaOff[c], R, R, FITRE_MAT_SYM_PAIR);
+		const fitre_matrix lambda = mat_of(kfacInfo->LambdaGInv + lambdaOff[c], O, O, FITRE_MAT_SYM_PAIR);
 		const real *v = vec + wOffsets[c];
 		real *ng = nGradient + wOffsets[c];
 		const real *mat = v;
@@ -492,13 +498,16 @@ void computeNaturalGradient(CNN_MODEL *model, KFAC_CURVATURE_INFO *kfacInfo, rea
 			HIP_CALL(fitre_hip_copy_2d(wb + K, R, vec + bOffsets[c], 1, 1, O));
 			mat = wb;
 		}
-		HIP_CALL(fitre_hip_gemm(0, 0, R, O, O, 1.f, mat, R, lambda, O, 0.f, u, R, NULL, ws, wsBytes));
+		const fitre_matrix g = mat_of(mat, 1, R, FITRE_MAT_F32), um = mat_of(u, 1, R, FITRE_MAT_F64);
+		HIP_CALL(fitre_hip_gemm_f64(R, O, O, 1.0, &g, &lambda, 0.0, &um, 0.0, 0, ws, wsBytes));
 		if (bias) {
-			HIP_CALL(fitre_hip_gemm(0, 0, R, O, R, 1.f, omega, R, u, R, 0.f, zt, R, NULL, ws, wsBytes));
+			const fitre_matrix out = mat_of(zt, 1, R, FITRE_MAT_F32);
+			HIP_CALL(fitre_hip_gemm_f64(R, O, R, 1.0, &omega, &um, 0.0, &out, 0.0, 0, ws, wsBytes));
 			HIP_CALL(fitre_hip_copy_2d(ng, K, zt, R, K, O));
 			HIP_CALL(fitre_hip_copy_2d(nGradient + bOffsets[c], 1, zt + K, R, 1, O));
 		} else {
-			HIP_CALL(fitre_hip_gemm(0, 0, R, O, R, 1.f, omega, R, u, R, 0.f, ng, R, NULL, ws, wsBytes));
+			const fitre_matrix out = mat_of(ng, 1, R, FITRE_MAT_F32);
+			HIP_CALL(fitre_hip_gemm_f64(R, O, R, 1.0, &omega, &um, 0.0, &out, 0.0, 0, ws, wsBytes));
 		}
 	}
 	/* Linear layers: the gradient block [W | b] already is the out x (in + 1) matrix
@@ -506,9 +515,12 @@ void computeNaturalGradient(CNN_MODEL *model, KFAC_CURVATURE_INFO *kfacInfo, rea
 	for (int f = 0; f < model->lLayers; f++) {
 		const FC_LAYER *l = &model->fcLayer[f];
 		const int R = l->in + bias, O = l->out;
-		const real *omega = kfacInfo->OmegaZInv + omegaOff[nc + f], *lambda = kfacInfo->LambdaGInv + lambdaOff[nc + f];
-		HIP_CALL(fitre_hip_gemm(0, 0, O, R, O, 1.f, lambda, O, vec + wOffsets[nc + f], O, 0.f, u, O, NULL, ws, wsBytes));
-		HIP_CALL(fitre_hip_gemm(0, 0, O, R, R, 1.f, u, O, omega, R, 0.f, nGradient + wOffsets[nc + f], O, NULL, ws, wsBytes));
+		const fitre_matrix omega = mat_of(kfacInfo->OmegaZInv + omegaOff[nc + f], R, R, FITRE_MAT_SYM_PAIR);
+		const fitre_matrix lambda = mat_of(kfacInfo->LambdaGInv + lambdaOff[nc + f], O, O, FITRE_MAT_SYM_PAIR);
+		const fitre_matrix g = mat_of(vec + wOffsets[nc + f], 1, O, FITRE_MAT_F32), um = mat_of(u, 1, O, FITRE_MAT_F64);
+		const fitre_matrix out = mat_of(nGradient + wOffsets[nc + f], 1, O, FITRE_MAT_F32);
+		HIP_CALL(fitre_hip_gemm_f64(O, R, O, 1.0, &lambda, &g, 0.0, &um, 0.0, 0, ws, wsBytes));
+		HIP_CALL(fitre_hip_gemm_f64(O, R, R, 1.0, &um, &omega, 0.0, &out, 0.0, 0, ws, wsBytes));
 	}
 	HIP_CALL(fitre_hip_sync());
 }

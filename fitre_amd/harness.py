@@ -105,6 +105,41 @@ def rel_err(a, b):
     return float(np.max(np.abs(a - b)) / (scale if scale > 0 else 1.0))
 
 
+# ---------------------------------------------------------------- float-pair matrices
+def _diagonal_words(n):
+    """Float-pair matrices (FITRE_MAT_SYM_PAIR, include/fitre_hip.h): (row, column) of the word that carries the remainder of diagonal element k in its lower 16 bits."""
+    return [(k + 1, k) if k + 1 < n else (n - 1, 0) for k in range(n)]
+
+
+def pair_decode(a):
+    """The symmetric matrix a float-pair array stands for (a[r][c] = element (r, c) of the device's column-major array)."""
+    n = a.shape[0]
+    bits = np.ascontiguousarray(a, dtype=np.float32).view(np.uint32).copy()
+    diag_lo = np.zeros(n)
+    if n >= 3:
+        for k, (r, c) in enumerate(_diagonal_words(n)):
+            diag_lo[k] = np.uint32((int(bits[r, c]) & 0xFFFF) << 16).view(np.float32)
+            bits[r, c] &= np.uint32(0xFFFF0000)
+    a = bits.view(np.float32).astype(np.float64)
+    full = np.triu(a) + np.tril(a, -1).T
+    full = full + np.triu(full, 1).T
+    full[np.diag_indices(n)] += diag_lo
+    return full
+
+
+def pair_encode(s):
+    n = s.shape[0]
+    hi = s.astype(np.float32)
+    lo = (s - hi.astype(np.float64)).astype(np.float32)
+    out = (np.triu(hi) + np.tril(lo, -1)).astype(np.float32)
+    if n >= 3:
+        bits = out.view(np.uint32)
+        dl = np.diag(lo).copy().view(np.uint32)
+        for k, (r, c) in enumerate(_diagonal_words(n)):
+            bits[r, c] = (int(bits[r, c]) & 0xFFFF0000) | (int(dl[k]) >> 16)
+    return out
+
+
 # ---------------------------------------------------------------- device buffers
 class Device:
     """Owns device buffers through the C-ABI (no torch involved)."""

@@ -7,7 +7,7 @@ import ctypes as C
 import os
 
 from .structs import (CNN_MODEL, CONV_LAYER, DEVICE_DATASET, KFAC_CURVATURE_INFO, NN_MODEL, POOL_LAYER, SCRATCH_AREA,
-                      fitre_conv_shape)
+                      fitre_conv_shape, fitre_matrix)
 
 _PKG = os.path.dirname(os.path.abspath(__file__))
 HIP_LIB_PATH = os.path.join(_PKG, "libfitre_hip.so")
@@ -19,6 +19,7 @@ pshape = C.POINTER(fitre_conv_shape)
 pmodel, pdata, pscratch = C.POINTER(CNN_MODEL), C.POINTER(DEVICE_DATASET), C.POINTER(SCRATCH_AREA)
 pkfac = C.POINTER(KFAC_CURVATURE_INFO)
 pnn = C.POINTER(NN_MODEL)
+f64, pmat = C.c_double, C.POINTER(fitre_matrix)
 
 # name -> (restype, argtypes); mirrors include/fitre_hip.h
 HIP_API = {
@@ -144,6 +145,16 @@ HIP_API = {
     "fitre_hip_kfac_conv_output_factor": (i32, [vp, vp, vp, vp, sz]),
     "fitre_hip_kfac_fc_input_factor": (i32, [vp, i32, i32, i32, vp, vp, sz]),
     "fitre_hip_kfac_fc_output_factor": (i32, [vp, i32, i32, vp, vp, sz]),
+    "fitre_hip_gemm_f64_workspace": (sz, [lng, lng, lng, i32]),
+    "fitre_hip_gemm_f64": (i32, [lng, lng, lng, f64, pmat, pmat, f64, pmat, f64, i32, vp, sz]),
+    "fitre_hip_spd_inverse_f64_workspace": (sz, [i32]),
+    "fitre_hip_spd_inverse_f64_queued": (i32, [vp, i32, vp, i32, vp, sz, vp]),
+    "fitre_hip_widen_shift": (i32, [vp, i32, f64, vp]),
+    "fitre_hip_kfac_conv_input_factor_f64_workspace": (sz, [vp, i32]),
+    "fitre_hip_kfac_conv_input_factor_f64": (i32, [vp, vp, i32, f64, vp, vp, sz]),
+    "fitre_hip_kfac_conv_output_factor_f64": (i32, [vp, vp, f64, vp, vp, sz]),
+    "fitre_hip_kfac_fc_input_factor_f64": (i32, [vp, i32, i32, i32, f64, vp, vp, sz]),
+    "fitre_hip_kfac_fc_output_factor_f64": (i32, [vp, i32, i32, f64, vp, vp, sz]),
 }
 
 pconv, ppool = C.POINTER(CONV_LAYER), C.POINTER(POOL_LAYER)
@@ -196,6 +207,7 @@ CNN_API = {
     "computeLambdaDeltaFactors": (None, [pkfac, pmodel, i32, vp, vp, vp, pi32, pi32, vp]),
     "kfacInverseMemRequired": (lng, [pmodel, i32]),
     "computeMatrixInverse": (None, [vp, vp, i32, vp, f32, f32]),
+    "matrixInverseMemRequired": (lng, [i32]),
     "computeOmegaZ": (None, [pkfac, pmodel, pdata, i32, vp, vp, vp, pi32, pi32, vp, vp, vp, vp, vp]),
     "computeLambdaDelta": (None, [pkfac, pmodel, i32, vp, vp, vp, pi32, pi32, vp, vp, vp, vp, vp]),
     "computeOmegaZAndLambdaDelta": (None, [pkfac, pmodel, pdata, i32, vp, vp, vp, vp, pi32, pi32, vp]),

@@ -136,3 +136,13 @@ class fitre_split_view(C.Structure):
 class fitre_conv_shape(C.Structure):
     _fields_ = [(n, C.c_int) for n in (
         "samples", "inChannels", "outChannels", "inA", "inB", "outA", "outB", "ksize", "stride", "padding")]
+
+
+FITRE_MAT_F32, FITRE_MAT_F64, FITRE_MAT_SYM_PAIR = 0, 1, 2
+FITRE_GEMM_SYMMETRIC, FITRE_GEMM_A_LOWER, FITRE_GEMM_A_UPPER, FITRE_GEMM_B_LOWER, FITRE_GEMM_B_UPPER = 1, 2, 4, 8, 16
+
+
+class fitre_matrix(C.Structure):
+    """Operand of the float64 products (include/fitre_hip.h)."""
+    _fields_ = [("data", C.c_void_p), ("rowStride", C.c_long), ("colStride", C.c_long), ("kind", C.c_int),
+                ("onesRow", C.c_long), ("onesCol", C.c_long), ("onesValue", C.c_double)]

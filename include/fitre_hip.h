@@ -531,6 +531,64 @@ int fitre_hip_spd_inverse_batched_queued(int batch, const float *matrix, long ma
                                          float *inverse, long inverseStride, void *ws, size_t wsBytes,
                                          long wsStrideBytes, int *pivotInfo);
 
+/* ---- float64 products and the float64 inverse -------------------------------------------------------
+ * The reference's KFAC leg is double throughout (real = double, core/datadefs.h:5): cublasDgemm for the factors and the
+ * natural gradient (solvers/kfac_inverses.cu:531-536,808-813, solvers/kfac_natural_gradient.cu:36-241), cusolverDnDpotrf /
+ * Dpotrs for the inverses (solvers/kfac_inverses.cu:133-186).  These entry points do that arithmetic in float64 on the
+ * matrix pipes, on operands that stay in the caller's float arrays.
+ *
+ * fitre_matrix: element (r, c) of a matrix of floats (FITRE_MAT_F32) or doubles (FITRE_MAT_F64) at
+ * data[r * rowStride + c * colStride]; FITRE_MAT_SYM_PAIR is a symmetric matrix of order rowStride kept as a pair of
+ * floats per element in ONE dense float array, column-major with leading dimension colStride: the value rounded to float
+ * on and above the diagonal, value - rounded value below it -- 48 significant bits in the room of a float matrix.  The
+ * diagonal has no word below it for its remainder: the word of element (k + 1, k) ((n - 1, 0) for the last k) keeps
+ * the upper 16 bits of its own remainder and, in its lower 16 bits, the upper 16 bits of the remainder of diagonal element
+ * k, so that both have 32 significant bits (orders below 3: the diagonal stays at float precision).  The upper triangle
+ * alone is the matrix in floats.  onesRow / onesCol (floats only, -1 for none): a row / column that is not in memory and
+ * reads as onesValue (the bias row of a KFAC input factor). */
+enum { FITRE_MAT_F32 = 0, FITRE_MAT_F64 = 1, FITRE_MAT_SYM_PAIR = 2 };
+typedef struct fitre_matrix {
+	const void *data;
+	long rowStride, colStride;
+	int kind;
+	long onesRow, onesCol;
+	double onesValue;
+} fitre_matrix;
+/* flags: the product is symmetric (M == N; only the tiles on and above the diagonal are computed and mirrored);
+ * A(i, k) is zero for k > i (A_LOWER) / for k < i (A_UPPER); B(k, j) is zero for k < j (B_LOWER) / for k > j (B_UPPER):
+ * the reduction skips those ranges. */
+#define FITRE_GEMM_SYMMETRIC 1
+#define FITRE_GEMM_A_LOWER 2
+#define FITRE_GEMM_A_UPPER 4
+#define FITRE_GEMM_B_LOWER 8
+#define FITRE_GEMM_B_UPPER 16
+/* C(M x N) = alpha * A(M x K) * B(K x N) + beta * C, plus diagAdd on the diagonal; C->data is written (any kind; a
+ * float-pair result needs FITRE_GEMM_SYMMETRIC and beta = 0).  ws: 256-byte aligned, fitre_hip_gemm_f64_workspace bytes. */
+size_t fitre_hip_gemm_f64_workspace(long M, long N, long K, int flags);
+int fitre_hip_gemm_f64(long M, long N, long K, double alpha, const fitre_matrix *A, const fitre_matrix *B, double beta,
+                       const fitre_matrix *C, double diagAdd, int flags, void *ws, size_t wsBytes);
+/* inverse = matrix^-1 for a symmetric positive definite matrix of n x n doubles (dense, destroyed): Cholesky factor and
+ * its inverse by halving, then X^T X, all in float64; the result is stored dense with leading dimension n as
+ * inverseKind.  Queued on the selected lane; pivotInfo (device int) holds 0 or the 1-based index of the first
+ * non-positive pivot once the lane has drained.  ws: 256-byte aligned, fitre_hip_spd_inverse_f64_workspace(n) bytes. */
+size_t fitre_hip_spd_inverse_f64_workspace(int n);
+int fitre_hip_spd_inverse_f64_queued(double *matrix, int n, void *inverse, int inverseKind, void *ws, size_t wsBytes,
+                                     int *pivotInfo);
+/* out(n x n doubles) = matrix(n x n floats) + shift * I */
+int fitre_hip_widen_shift(const float *matrix, int n, double shift, double *out);
+/* The four Kronecker factors above accumulated in float64 and written as n x n doubles, with `shift` (the damping) added
+ * on the diagonal.  Workspaces: fitre_hip_kfac_conv_input_factor_f64_workspace (the transposed patch matrix and the
+ * split partials) resp. fitre_hip_gemm_f64_workspace(order, order, reduce, FITRE_GEMM_SYMMETRIC). */
+size_t fitre_hip_kfac_conv_input_factor_f64_workspace(const fitre_conv_shape *s, int withBias);
+int fitre_hip_kfac_conv_input_factor_f64(const fitre_conv_shape *s, const float *x, int withBias, double shift,
+                                         double *factor, void *ws, size_t wsBytes);
+int fitre_hip_kfac_conv_output_factor_f64(const fitre_conv_shape *s, const float *delta, double shift, double *factor,
+                                          void *ws, size_t wsBytes);
+int fitre_hip_kfac_fc_input_factor_f64(const float *z, int in, int samples, int withBias, double shift, double *factor,
+                                       void *ws, size_t wsBytes);
+int fitre_hip_kfac_fc_output_factor_f64(const float *delta, int out, int samples, double shift, double *factor, void *ws,
+                                        size_t wsBytes);
+
 #ifdef __cplusplus
 }
 #endif

@@ -67,19 +67,27 @@ void computeLambdaDeltaFactors(KFAC_CURVATURE_INFO *kfac_info, CNN_MODEL *model,
                                real *dampedLambda, real *lambdaGGT, int *zOffsets, int *zztOffsets, real *devPtr);
 
 /* inverse = (matrix + (lambda + dampGamma) I)^-1, order n, both dense n x n
- * (solvers/kfac_inverses.cu:133-186, computeMatrixInverseCusolver without the cuSOLVER handles).
- * devPtr: fitre_hip_spd_inverse_workspace(n) bytes of scratch, 256-byte aligned.  Exits with the
- * reference's message when the matrix is not positive definite. */
+ * (solvers/kfac_inverses.cu:133-186, computeMatrixInverseCusolver without the cuSOLVER handles).  As in the
+ * reference the arithmetic is double: the matrix is widened, factored and inverted in float64, and the inverse
+ * rounded to reals.  devPtr: matrixInverseMemRequired(n) reals of scratch.  Exits with the reference's message
+ * when the matrix is not positive definite. */
 void computeMatrixInverse(real *matrix, real *inverse, int n, real *devPtr, real lambda, real dampGamma);
+long matrixInverseMemRequired(int n);
 
-/* Scratch (in reals) computeOmegaZ / computeLambdaDelta may carve from devPtr: the largest factor
- * plus the workspaces of its product and of its inverse. */
+/* Scratch (in reals) computeOmegaZ / computeLambdaDelta may carve from devPtr: four lanes, each with the largest
+ * factor in doubles plus the workspaces of its product and of its inverse. */
 long kfacInverseMemRequired(CNN_MODEL *model, int samples);
 
 /* solvers/kfac_inverses.cu:450-630 and :759-857 in full: every layer's factor (built in scratch, as in
  * the reference) and its damped inverse, stored at omegaZInv + OmegaZOffsets[l] resp.
  * lambdaGInv + LambdaGOffsets[l].  Damping: kfac_info->regLambda + kfac_info->dampGamma on the diagonal.
- * pageLckPtr is unused (the reference reads cuSOLVER's devInfo through it). */
+ * pageLckPtr is unused (the reference reads cuSOLVER's devInfo through it).
+ * Precision: the reference does this leg in double.  Here reals are floats, and the factors of a network with a small
+ * damping are too ill-conditioned for float arithmetic (condition 1e4 .. 1e6 at lambda = 1e-3), so every factor is
+ * accumulated, factored and inverted in float64 on the device and the inverse is stored in the caller's n x n reals
+ * as a PAIR of floats per element: the inverse rounded to float on and above the diagonal, the rounding remainder
+ * below it (FITRE_MAT_SYM_PAIR, fitre_hip.h).  The upper triangle alone is the float inverse; computeNaturalGradient,
+ * the only reader of these arrays in the reference (solvers/kfac_natural_gradient.cu:55-56), takes the pairs. */
 /* The three trailing arguments are the reference's vendor handles (cublasHandle_t, cudaStream_t,
  * cusolverDnHandle_t, solvers/kfac_inverses.h:28-34), kept so that its solver source compiles against this
  * header unchanged; they are opaque pointers and are ignored (the device layer owns its streams). */
