@@ -23,11 +23,11 @@ struct DgemmArgs {
 	double alpha, beta, diagAdd;
 	int flags, splits, tilesM, tilesN;
 	double *partials;
+	uint32_t bytesA, bytesB; // extent of the operands in memory
 	float *diagRemainder; // float-pair results: the remainders of the diagonal, folded into the matrix by a pass of its own
 	int aKContig, bKContig;
 };
 
-constexpr int kDgBK = 16;
 static size_t dalign(size_t v) { return (v + 255) & ~(size_t)255; }
 
 __device__ __forceinline__ double dmat_load(const DMat &m, long r, long c)
@@ -85,19 +85,84 @@ __device__ __forceinline__ void dgemm_store(const DgemmArgs &g, long i, long j, 
 	}
 }
 
-// Tile TM x TN, 256 threads = 2 x 2 waves, a wave (TM/2) x (TN/2) = MI x NI blocks of 16 x 16.
-// Lane l of a block holds A(i = l % 16, k = l / 16), B(k = l / 16, j = l % 16) and, in register r of the accumulator,
-// C(i = 4 r + l / 16, j = l % 16).
-// blockIdx.x: tile (row-major over tilesM x tilesN), blockIdx.y: split of the reduction.
-template <int TM, int TN>
+// Global reads go through raw buffer resources: 32-bit byte offsets, no address arithmetic per slice (the slice moves the
+// resource's base, scalar work), and an element outside the matrix gets the offset 0xFFFFFFFF, which the hardware's range
+// check answers with zero.  Every operand must therefore be smaller than 4 GiB.
+constexpr uint32_t kDgOutOfRange = 0xFFFFFFFFu;
+typedef unsigned int v2u __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t dg_rsrc(const void *p, uint32_t bytes)
+{
+	return __builtin_amdgcn_make_buffer_rsrc((void *)p, 0, bytes, 0x00020000);
+}
+
+// What a load leaves in registers until its slice goes to LDS: the bits as they came (a float, a double, or the two
+// words of a float pair).  Converting at once would be a use of the value, and the wave would wait for every load
+// right behind it instead of a slice later.
+template <int KIND>
+struct DgRaw {
+	uint32_t w[KIND == FITRE_MAT_F32 ? 1 : 2];
+};
+
+template <int KIND>
+__device__ __forceinline__ DgRaw<KIND> dg_load(__amdgpu_buffer_rsrc_t r, uint32_t byteOffset)
+{
+	DgRaw<KIND> v;
+	if constexpr (KIND == FITRE_MAT_F64) {
+		const v2u t = __builtin_amdgcn_raw_buffer_load_b64(r, (int)byteOffset, 0, 0);
+		v.w[0] = t.x, v.w[1] = t.y;
+	} else {
+		v.w[0] = __builtin_amdgcn_raw_buffer_load_b32(r, (int)byteOffset, 0, 0);
+	}
+	return v;
+}
+
+// the two words of element (r, c) of a symmetric float pair of order n (see dmat_load); rs covers the whole array
+__device__ __forceinline__ DgRaw<FITRE_MAT_SYM_PAIR> dg_load_pair(__amdgpu_buffer_rsrc_t rs, int n, int ld, int r, int c, bool ok)
+{
+	const int a = r < c ? r : c, b = r < c ? c : r;
+	const int below = (a == b) ? ((a + 1 < n) ? a * ld + a + 1 : n - 1) : a * ld + b;
+	DgRaw<FITRE_MAT_SYM_PAIR> v;
+	v.w[0] = __builtin_amdgcn_raw_buffer_load_b32(rs, ok ? 4 * (b * ld + a) : (int)kDgOutOfRange, 0, 0);
+	v.w[1] = __builtin_amdgcn_raw_buffer_load_b32(rs, ok ? 4 * below : (int)kDgOutOfRange, 0, 0);
+	return v;
+}
+
+template <int KIND>
+__device__ __forceinline__ double dg_value(const DgRaw<KIND> &v, int n, int r, int c)
+{
+	if constexpr (KIND == FITRE_MAT_F64) {
+		return __hiloint2double((int)v.w[1], (int)v.w[0]);
+	} else if constexpr (KIND == FITRE_MAT_F32) {
+		return (double)__uint_as_float(v.w[0]);
+	} else {
+		const int a = r < c ? r : c, b = r < c ? c : r;
+		uint32_t w = v.w[1];
+		if (a == b) w = (n < 3) ? 0u : w << 16;
+		else if (n >= 3 && (b == a + 1 || (a == 0 && b == n - 1))) w &= 0xFFFF0000u;
+		return (double)__uint_as_float(v.w[0]) + (double)__uint_as_float(w);
+	}
+}
+
+// Tile TM x TN, 256 threads = 2 x 2 waves, a wave (TM/2) x (TN/2) = MI x NI blocks of 16 x 16; slices of BK reduction
+// indices, double-buffered in LDS (one barrier per slice; the next slice's global loads are in flight while this one is
+// multiplied).  Lane l of a block holds A(i = l % 16, k = l / 16), B(k = l / 16, j = l % 16) and, in register r of the
+// accumulator, C(i = 4 r + l / 16, j = l % 16).
+// KA / KB: operand kinds (compile-time: the loads of the float and double kinds are one add and one load per element,
+// their offsets computed once per thread).  blockIdx.x: tile (row-major over tilesM x tilesN), blockIdx.y: split.
+template <int TM, int TN, int BK, int KA, int KB>
 __global__ void __launch_bounds__(256) dgemm_kernel(const DgemmArgs g)
 {
-	constexpr int BK = kDgBK;
-	constexpr int LDA = TM + 16, LDB = TN + 16; // row offsets of 16 doubles mod 32: the four k rows of a fragment read hit different banks
+	// An operand's slice sits in LDS as [k][row], rows TM + 16 doubles apart (a row offset of 16 mod 32: the four k rows of a
+	// fragment read hit different banks), when its lanes run along the rows; as [row][k], rows BK + 1 doubles apart, when
+	// they run along k (a k-contiguous operand): the stores of a wave are then contiguous runs of BK doubles, and the
+	// sixteen rows of a fragment read, 2 (BK + 1) words apart, spread over the banks.
+	constexpr int LDA = TM + 16, LDB = TN + 16, LDK = BK + 1;
+	constexpr int BUFA = (BK * LDA > TM * LDK) ? BK * LDA : TM * LDK, BUFB = (BK * LDB > TN * LDK) ? BK * LDB : TN * LDK;
 	constexpr int WTM = TM / 2, WTN = TN / 2, MI = WTM / 16, NI = WTN / 16;
 	constexpr int EA = TM * BK / 256, EB = TN * BK / 256;
-	__shared__ double As[BK * LDA];
-	__shared__ double Bs[BK * LDB];
+	extern __shared__ double lds[];
+	double *As = lds, *Bs = lds + 2 * BUFA; // two buffers each
 	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 	const int wm = wave >> 1, wn = wave & 1;
 	const int tile = blockIdx.x, ti = tile / g.tilesN, tj = tile - ti * g.tilesN;
@@ -123,62 +188,117 @@ __global__ void __launch_bounds__(256) dgemm_kernel(const DgemmArgs g)
 #pragma unroll
 		for (int ni = 0; ni < NI; ni++) acc[mi][ni] = v4d{ 0.0, 0.0, 0.0, 0.0 };
 
-	double ra[EA], rb[EB];
-	auto fetch = [&](int kk) {
+	// Which elements of a slice a thread moves: element q is (row0 + q * rowStep, kq0 + q * kStep) of the tile's slice,
+	// with the lanes along the direction in which the operand is contiguous; its place in LDS and (float / double
+	// operands) its byte offset in memory at reduction index 0 are affine in q as well.
+	constexpr int SA = KA == FITRE_MAT_F64 ? 8 : 4, SB = KB == FITRE_MAT_F64 ? 8 : 4;
+	const int kq0A = g.aKContig ? tid % BK : tid / TM, kStepA = g.aKContig ? 0 : 256 / TM;
+	const int row0A = g.aKContig ? tid / BK : tid % TM, rowStepA = g.aKContig ? 256 / BK : 0;
+	const int kq0B = g.bKContig ? tid % BK : tid / TN, kStepB = g.bKContig ? 0 : 256 / TN;
+	const int row0B = g.bKContig ? tid / BK : tid % TN, rowStepB = g.bKContig ? 256 / BK : 0;
+	const int ldsRowA = g.aKContig ? LDK : 1, ldsKA = g.aKContig ? 1 : LDA; // LDS strides along the rows / along k
+	const int ldsRowB = g.bKContig ? LDK : 1, ldsKB = g.bKContig ? 1 : LDB;
+	const int lds0A = kq0A * ldsKA + row0A * ldsRowA, ldsStepA = kStepA * ldsKA + rowStepA * ldsRowA;
+	const int lds0B = kq0B * ldsKB + row0B * ldsRowB, ldsStepB = kStepB * ldsKB + rowStepB * ldsRowB;
+	const int stepA = (int)g.A.cs, stepB = (int)g.B.rs; // elements per reduction index
+	uint32_t voffA[EA], voffB[EB];
+	uint32_t onesA = 0, onesB = 0; // elements of the constant row / column
 #pragma unroll
-		for (int q = 0; q < EA; q++) {
-			int row, k;
-			if (g.aKContig) k = tid & 15, row = (tid >> 4) + 16 * q;
-			else row = tid % TM, k = tid / TM + (256 / TM) * q;
-			const long gi = i0 + row, gk = kk + k;
-			ra[q] = (gi < g.M && gk < k1) ? dmat_load(g.A, gi, gk) : 0.0;
-		}
+	for (int q = 0; q < EA; q++) {
+		const int gi = i0 + row0A + q * rowStepA;
+		const bool ones = gi == g.A.onesRow;
+		if (ones) onesA |= 1u << q;
+		voffA[q] = (gi < g.M && !ones) ? (uint32_t)SA * (uint32_t)(gi * (int)g.A.rs + (kq0A + q * kStepA) * stepA) : kDgOutOfRange;
+	}
 #pragma unroll
-		for (int q = 0; q < EB; q++) {
-			int col, k;
-			if (g.bKContig) k = tid & 15, col = (tid >> 4) + 16 * q;
-			else col = tid % TN, k = tid / TN + (256 / TN) * q;
-			const long gj = j0 + col, gk = kk + k;
-			rb[q] = (gj < g.N && gk < k1) ? dmat_load(g.B, gk, gj) : 0.0;
-		}
-	};
-	auto stage = [&]() {
-#pragma unroll
-		for (int q = 0; q < EA; q++) {
-			int row, k;
-			if (g.aKContig) k = tid & 15, row = (tid >> 4) + 16 * q;
-			else row = tid % TM, k = tid / TM + (256 / TM) * q;
-			As[k * LDA + row] = ra[q];
-		}
-#pragma unroll
-		for (int q = 0; q < EB; q++) {
-			int col, k;
-			if (g.bKContig) k = tid & 15, col = (tid >> 4) + 16 * q;
-			else col = tid % TN, k = tid / TN + (256 / TN) * q;
-			Bs[k * LDB + col] = rb[q];
-		}
-	};
+	for (int q = 0; q < EB; q++) {
+		const int gj = j0 + row0B + q * rowStepB;
+		const bool ones = gj == g.B.onesCol;
+		if (ones) onesB |= 1u << q;
+		voffB[q] = (gj < g.N && !ones) ? (uint32_t)SB * (uint32_t)(gj * (int)g.B.cs + (kq0B + q * kStepB) * stepB) : kDgOutOfRange;
+	}
 
-	if (k0 < k1) fetch(k0);
-	for (int kk = k0; kk < k1; kk += BK) {
-		__syncthreads(); // the previous slice has been read
-		stage();
-		__syncthreads();
-		if (kk + BK < k1) fetch(kk + BK); // in flight while this slice is multiplied
-		const double *ap = As + (lane >> 4) * LDA + wm * WTM + (lane & 15);
-		const double *bp = Bs + (lane >> 4) * LDB + wn * WTN + (lane & 15);
+	// two slices of loads in flight: slice s + 2 is requested while slice s is multiplied and reaches LDS a slice later
+	DgRaw<KA> ra[2][EA];
+	DgRaw<KB> rb[2][EB];
+	auto fetch = [&](int kk, DgRaw<KA> (&va)[EA], DgRaw<KB> (&vb)[EB]) {
+		const bool whole = kk + BK <= k1;
+		if constexpr (KA == FITRE_MAT_SYM_PAIR) {
+			const __amdgpu_buffer_rsrc_t rs = dg_rsrc(g.A.p, g.bytesA);
+#pragma unroll
+			for (int q = 0; q < EA; q++) {
+				const int gi = i0 + row0A + q * rowStepA, gk = kk + kq0A + q * kStepA;
+				va[q] = dg_load_pair(rs, (int)g.A.rs, (int)g.A.cs, gi, gk, gi < g.M && gk < k1);
+			}
+		} else {
+			const uint32_t adv = (uint32_t)__builtin_amdgcn_readfirstlane(SA * kk * stepA); // wave-uniform: the resource stays in scalar registers
+			const __amdgpu_buffer_rsrc_t rs = dg_rsrc((const char *)g.A.p + adv, g.bytesA - adv);
+#pragma unroll
+			for (int q = 0; q < EA; q++) va[q] = dg_load<KA>(rs, voffA[q] | ((whole | (kk + kq0A + q * kStepA < k1)) ? 0u : kDgOutOfRange));
+		}
+		if constexpr (KB == FITRE_MAT_SYM_PAIR) {
+			const __amdgpu_buffer_rsrc_t rs = dg_rsrc(g.B.p, g.bytesB);
+#pragma unroll
+			for (int q = 0; q < EB; q++) {
+				const int gj = j0 + row0B + q * rowStepB, gk = kk + kq0B + q * kStepB;
+				vb[q] = dg_load_pair(rs, (int)g.B.rs, (int)g.B.cs, gk, gj, gj < g.N && gk < k1);
+			}
+		} else {
+			const uint32_t adv = (uint32_t)__builtin_amdgcn_readfirstlane(SB * kk * stepB);
+			const __amdgpu_buffer_rsrc_t rs = dg_rsrc((const char *)g.B.p + adv, g.bytesB - adv);
+#pragma unroll
+			for (int q = 0; q < EB; q++) vb[q] = dg_load<KB>(rs, voffB[q] | ((whole | (kk + kq0B + q * kStepB < k1)) ? 0u : kDgOutOfRange));
+		}
+	};
+	// slice kk from registers to LDS buffer buf, as doubles, the constant row / column put in
+	auto stage = [&](int buf, int kk, const DgRaw<KA> (&va)[EA], const DgRaw<KB> (&vb)[EB]) {
+#pragma unroll
+		for (int q = 0; q < EA; q++) {
+			const int gk = kk + kq0A + q * kStepA;
+			const double v = dg_value<KA>(va[q], (int)g.A.rs, i0 + row0A + q * rowStepA, gk);
+			As[buf * BUFA + lds0A + q * ldsStepA] = (((onesA >> q) & 1) && gk < k1) ? g.A.onesValue : v;
+		}
+#pragma unroll
+		for (int q = 0; q < EB; q++) {
+			const int gk = kk + kq0B + q * kStepB;
+			const double v = dg_value<KB>(vb[q], (int)g.B.rs, gk, j0 + row0B + q * rowStepB);
+			Bs[buf * BUFB + lds0B + q * ldsStepB] = (((onesB >> q) & 1) && gk < k1) ? g.B.onesValue : v;
+		}
+	};
+	auto multiply = [&](int buf) {
+		const double *ap = As + buf * BUFA + (lane >> 4) * ldsKA + (wm * WTM + (lane & 15)) * ldsRowA;
+		const double *bp = Bs + buf * BUFB + (lane >> 4) * ldsKB + (wn * WTN + (lane & 15)) * ldsRowB;
 #pragma unroll
 		for (int k4 = 0; k4 < BK / 4; k4++) {
 			double a[MI], b[NI];
 #pragma unroll
-			for (int mi = 0; mi < MI; mi++) a[mi] = ap[k4 * 4 * LDA + mi * 16];
+			for (int mi = 0; mi < MI; mi++) a[mi] = ap[k4 * 4 * ldsKA + mi * 16 * ldsRowA];
 #pragma unroll
-			for (int ni = 0; ni < NI; ni++) b[ni] = bp[k4 * 4 * LDB + ni * 16];
+			for (int ni = 0; ni < NI; ni++) b[ni] = bp[k4 * 4 * ldsKB + ni * 16 * ldsRowB];
 #pragma unroll
 			for (int mi = 0; mi < MI; mi++)
 #pragma unroll
 				for (int ni = 0; ni < NI; ni++) acc[mi][ni] = __builtin_amdgcn_mfma_f64_16x16x4f64(a[mi], b[ni], acc[mi][ni], 0, 0, 0);
 		}
+	};
+
+	if (k0 < k1) {
+		fetch(k0, ra[0], rb[0]);
+		stage(0, k0, ra[0], rb[0]);
+		if (k0 + BK < k1) fetch(k0 + BK, ra[1], rb[1]);
+	}
+	__syncthreads();
+	// two slices per round, so that the register sets and LDS buffers have constant indices
+	for (int kk = k0; kk < k1; kk += 2 * BK) {
+		if (kk + 2 * BK < k1) fetch(kk + 2 * BK, ra[0], rb[0]);
+		multiply(0);
+		if (kk + BK < k1) stage(1, kk + BK, ra[1], rb[1]);
+		__syncthreads();
+		if (kk + BK >= k1) break;
+		if (kk + 3 * BK < k1) fetch(kk + 3 * BK, ra[1], rb[1]);
+		multiply(1);
+		if (kk + 2 * BK < k1) stage(0, kk + 2 * BK, ra[0], rb[0]);
+		__syncthreads();
 	}
 
 	if (g.splits > 1) {
@@ -280,6 +400,46 @@ static DMat transposed(const DMat &m)
 	return t;
 }
 
+template <int T, int BK, int KA, int KB>
+static int launch_dgemm_kinds(const DgemmArgs &g, const DgemmPlan &p, dim3 grid)
+{
+	constexpr size_t perOperand = (BK * (T + 16) > T * (BK + 1)) ? BK * (T + 16) : T * (BK + 1);
+	constexpr size_t ldsBytes = (size_t)4 * perOperand * sizeof(double);
+	static bool attributeSet = false; // dynamic LDS above 64 KB has to be allowed once per kernel
+	if (!attributeSet) {
+		FITRE_HIP_TRY(hipFuncSetAttribute((const void *)dgemm_kernel<T, T, BK, KA, KB>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes));
+		attributeSet = true;
+	}
+	dgemm_kernel<T, T, BK, KA, KB><<<grid, 256, ldsBytes, stream()>>>(g);
+	if (p.splits > 1) dgemm_reduce_kernel<T, T><<<grid.x, 256, 0, stream()>>>(g);
+	return FITRE_OK;
+}
+
+template <int KA, int KB>
+static int launch_dgemm_tiles(const DgemmArgs &g, const DgemmPlan &p, dim3 grid)
+{
+	if (p.tile == 128) return launch_dgemm_kinds<128, 16, KA, KB>(g, p, grid);
+	// the small tile takes slices of 32: the products at the bottom of the inverse's recursion (reduction 64) then have all
+	// their loads in flight at once
+	return launch_dgemm_kinds<64, 32, KA, KB>(g, p, grid);
+}
+
+// the operand pairs the library's products have (either order: the kernel may work on the transposed problem)
+static int launch_dgemm(const DgemmArgs &g, const DgemmPlan &p, dim3 grid)
+{
+	constexpr int F32 = FITRE_MAT_F32, F64 = FITRE_MAT_F64, PAIR = FITRE_MAT_SYM_PAIR;
+	const int ka = g.A.kind, kb = g.B.kind;
+	if (ka == F32 && kb == F32) return launch_dgemm_tiles<F32, F32>(g, p, grid);
+	if (ka == F64 && kb == F64) return launch_dgemm_tiles<F64, F64>(g, p, grid);
+	if (ka == F32 && kb == F64) return launch_dgemm_tiles<F32, F64>(g, p, grid);
+	if (ka == F64 && kb == F32) return launch_dgemm_tiles<F64, F32>(g, p, grid);
+	if (ka == F32 && kb == PAIR) return launch_dgemm_tiles<F32, PAIR>(g, p, grid);
+	if (ka == PAIR && kb == F32) return launch_dgemm_tiles<PAIR, F32>(g, p, grid);
+	if (ka == F64 && kb == PAIR) return launch_dgemm_tiles<F64, PAIR>(g, p, grid);
+	if (ka == PAIR && kb == F64) return launch_dgemm_tiles<PAIR, F64>(g, p, grid);
+	return fail(FITRE_E_UNSUPPORTED, "float64 product: no kernel for two float-pair operands");
+}
+
 size_t dgemm_workspace(long M, long N, long K, int flags)
 {
 	// the kernel may work on the transposed problem; the plan is symmetric in M and N
@@ -327,63 +487,113 @@ int dgemm(long M, long N, long K, double alpha, DMat A, DMat B, double beta, DOu
 	g.diagRemainder = diagRemainder;
 	g.aKContig = (A.kind != FITRE_MAT_SYM_PAIR && A.cs == 1 && A.rs != 1);
 	g.bKContig = (B.kind != FITRE_MAT_SYM_PAIR && B.rs == 1 && B.cs != 1);
+	// byte offsets inside an operand are 32-bit
+	auto extent_bytes = [](const DMat &m, long rows, long cols, long ones0, long ones1) {
+		if (m.kind == FITRE_MAT_SYM_PAIR) return ((m.rs - 1) * m.cs + m.rs) * 4;
+		const long r = rows - (ones0 >= 0 ? 1 : 0), c = cols - (ones1 >= 0 ? 1 : 0);
+		return ((r - 1) * m.rs + (c - 1) * m.cs + 1) * (m.kind == FITRE_MAT_F64 ? 8 : 4);
+	};
+	const long bytesA = extent_bytes(A, M, K, A.onesRow, -1), bytesB = extent_bytes(B, K, N, -1, B.onesCol);
+	FITRE_REQUIRE(bytesA > 0 && bytesB > 0 && bytesA < 4294967295l && bytesB < 4294967295l, "float64 product: an operand of 4 GiB or more");
+	FITRE_REQUIRE(A.onesRow < 0 || A.onesRow == M - 1, "float64 product: the constant row must be the last one");
+	FITRE_REQUIRE(B.onesCol < 0 || B.onesCol == N - 1, "float64 product: the constant column must be the last one");
+	g.bytesA = (uint32_t)bytesA, g.bytesB = (uint32_t)bytesB;
+	FITRE_REQUIRE(A.rs >= 0 && A.cs >= 0 && B.rs >= 0 && B.cs >= 0, "float64 product: negative stride");
+	FITRE_REQUIRE(A.onesCol < 0 && B.onesRow < 0, "float64 product: a constant row / column along the reduction is not supported");
 	const dim3 grid((unsigned)(p.tilesM * p.tilesN), (unsigned)p.splits);
 	const double flops = ((flags & kDgMirror) ? 1.0 : 2.0) * (double)M * (double)N * (double)K;
 	LaunchScope scope(kernelClass, flops);
-	if (p.tile == 128) {
-		dgemm_kernel<128, 128><<<grid, 256, 0, stream()>>>(g);
-		if (p.splits > 1) dgemm_reduce_kernel<128, 128><<<grid.x, 256, 0, stream()>>>(g);
-	} else {
-		dgemm_kernel<64, 64><<<grid, 256, 0, stream()>>>(g);
-		if (p.splits > 1) dgemm_reduce_kernel<64, 64><<<grid.x, 256, 0, stream()>>>(g);
-	}
+	int rc = launch_dgemm(g, p, grid);
+	if (rc) return rc;
 	if (diagRemainder) pair_fold_diagonal_kernel<<<blocks_for(M, 256), 256, 0, stream()>>>((float *)C.p, C.cs, (int)M, diagRemainder);
 	return check_launch("float64 product");
 }
 
-// ---- leaf of the inverse: a diagonal block of order <= 64, one workgroup, float64 in LDS ----------------------------
+// ---- leaf of the inverse: a diagonal block of order <= 64, one workgroup, float64 in registers -----------------------
 //
 // One sweep of 64 steps, one barrier each, does the Cholesky factorisation W = L L^T (right-looking) and the inverse of
 // the factor together: the column operations that turn L^T into the identity (scale column j by 1 / l_jj, then column
-// k -= column j * l_kj for k > j) turn the identity into L^-T, and step j of them needs exactly column j of L, which
-// step j of the factorisation has just produced.  Thread (i, q) = (tid % 64, tid / 64) owns row i of the trailing
-// update (columns k = j+1+q, j+5+q, ...) and column i of the inverse in the making (rows q, q+4, ...).  A finished
-// row of X = L^-1 goes to the unused upper triangle of W's copy.
-constexpr int kDLeaf = 64, kDLd = kDLeaf + 1;
+// k -= column j * l_kj for k > j) turn the identity into Y = L^-T, and step j of them needs exactly column j of L, which
+// step j of the factorisation has just produced.  Thread (i, q) = (lane, wave) keeps row i of the trailing matrix --
+// W(i, k) for k = 4 t + q -- and column i of Y -- Y(r, i) for r = 4 t + q -- in registers, 16 doubles each; what a step
+// needs from other threads (column j of W, column j of Y) goes through two small LDS vectors, double-buffered by the
+// parity of the step, and is read back wave-uniformly (broadcasts).  The steps are unrolled by template recursion, so
+// that every register index and every loop bound is a constant.
+constexpr int kDLeaf = 64;
+
+__device__ __forceinline__ double rsqrt_f64(double a)
+{
+	double d = __builtin_amdgcn_rsq(a);
+	d = d * (1.5 - 0.5 * a * d * d);
+	return d * (1.5 - 0.5 * a * d * d);
+}
+
+// Step J.  Entries of a row right of the diagonal (k > i) are never read, so the trailing update runs over them
+// unmasked; what has to be masked is folded into the multiplier (zero where a thread must not update), which keeps
+// the step free of branches and of selects on loaded values.
+template <int J>
+__device__ __forceinline__ void dleaf_steps(double (&w)[16], double (&y)[16], double *Lcol, double *Ycol, int i, int q, int k0, int *info)
+{
+	constexpr int jb = J >> 2, js = J & 3;
+	double *lc = Lcol + (J & 1) * kDLeaf, *yc = Ycol + (J & 1) * kDLeaf;
+	if (q == js) lc[i] = w[jb]; // column J of the trailing matrix (rows >= J are read)
+	if (i == J) {
+#pragma unroll
+		for (int t = 0; t <= jb; t++) yc[4 * t + q] = y[t]; // column J of Y, rows <= J
+	}
+	__syncthreads();
+	const double ajj = lc[J], li = lc[i];
+	double lk[16 - jb], yr[jb + 1];
+#pragma unroll
+	for (int t = jb; t < 16; t++) lk[t - jb] = lc[4 * t + q];
+#pragma unroll
+	for (int t = 0; t <= jb; t++) yr[t] = yc[4 * t + q];
+	if (!(ajj > 0.0) && i == 0 && q == 0) atomicCAS(info, 0, k0 + J + 1);
+	const double d = rsqrt_f64(ajj);
+	const double m = li * (d * d);              // l_iJ / l_JJ
+	const double mw = (i > J) ? m : 0.0;        // rows below the pivot row take the update
+	// trailing matrix: W(i, k) -= l_iJ l_kJ for k > J
+	w[jb] = __builtin_fma((q > js) ? -mw : 0.0, lk[0], w[jb]);
+#pragma unroll
+	for (int t = jb + 1; t < 16; t++) w[t] = __builtin_fma(-mw, lk[t - jb], w[t]);
+	// Y: column i -= column J * l_iJ / l_JJ for i > J, rows r <= J; column J itself is scaled and final (row J of X)
+	const double sc = (i == J) ? d : 1.0;
+#pragma unroll
+	for (int t = 0; t < jb; t++) y[t] = __builtin_fma(-mw, yr[t], y[t]) * sc;
+	y[jb] = __builtin_fma((q <= js) ? -mw : 0.0, yr[jb], y[jb]) * sc;
+	// the updates stay in this step: left to itself the compiler postpones them until a value is needed and keeps
+	// the operands of every postponed step alive
+#pragma unroll
+	for (int t = jb; t < 16; t++) asm volatile("" : "+v"(w[t]));
+#pragma unroll
+	for (int t = 0; t <= jb; t++) asm volatile("" : "+v"(y[t]));
+	if constexpr (J + 1 < kDLeaf) dleaf_steps<J + 1>(w, y, Lcol, Ycol, i, q, k0, info);
+}
 
 __global__ void __launch_bounds__(256) dchol_leaf_kernel(const double *W, long ld, int k0, int nn, double *X, int *info)
 {
-	__shared__ double Ws[kDLeaf * kDLd]; // column-major: (i, k) at k * kDLd + i
-	__shared__ double Ys[kDLeaf * kDLd]; // L^-T in the making, column-major
-	__shared__ double diagX[kDLeaf];
+	__shared__ double Lcol[2 * kDLeaf], Ycol[2 * kDLeaf];
 	const int tid = threadIdx.x, i = tid & 63, q = tid >> 6;
 	const double *blk = W + (size_t)k0 * ld + k0;
-	for (int c = q; c < kDLeaf; c += 4) {
+	double w[16], y[16];
+#pragma unroll
+	for (int t = 0; t < 16; t++) {
+		const int c = 4 * t + q;
 		double v = (i == c) ? 1.0 : 0.0; // beyond the block: identity, which factors to itself
-		if (i < nn && c < nn && i >= c) v = blk[(size_t)c * ld + i];
-		Ws[c * kDLd + i] = v;
-		Ys[c * kDLd + i] = (i == c) ? 1.0 : 0.0;
+		if (i < nn && c <= i) v = blk[(size_t)c * ld + i];
+		w[t] = v;
+		y[t] = (i == c) ? 1.0 : 0.0;
 	}
-	for (int j = 0; j < kDLeaf; j++) {
-		__syncthreads();
-		const double ajj = Ws[j * kDLd + j];
-		if (!(ajj > 0.0) && tid == 0) atomicCAS(info, 0, k0 + j + 1);
-		const double d = 1.0 / sqrt(ajj);
-		if (i > j) {
-			const double lij = Ws[j * kDLd + i] * d;
-			for (int k = j + 1 + q; k <= i; k += 4) Ws[k * kDLd + i] -= lij * (Ws[j * kDLd + k] * d);
-			for (int r = q; r <= j; r += 4) Ys[i * kDLd + r] -= (Ys[j * kDLd + r] * d) * lij;
-		} else if (q == 0) {
-			// row j of X = column j of L^-T, scaled: final
-			if (i == j) diagX[j] = d;
-			else Ws[j * kDLd + i] = Ys[j * kDLd + i] * d; // (i, j) with i < j: above the diagonal, read by nobody
+	dleaf_steps<0>(w, y, Lcol, Ycol, i, q, k0, info);
+	// X(i, r) = Y(r, i) for r <= i
+	double *xblk = X + (size_t)k0 * ld + k0;
+	if (i < nn) {
+#pragma unroll
+		for (int t = 0; t < 16; t++) {
+			const int r = 4 * t + q;
+			if (r <= i) xblk[(size_t)r * ld + i] = y[t];
 		}
 	}
-	__syncthreads();
-	double *xblk = X + (size_t)k0 * ld + k0;
-	// X(j, r), r <= j, from Ws(r, j); thread: row j = i, columns r = q, q + 4, ...
-	if (i < nn)
-		for (int r = q; r <= i; r += 4) xblk[(size_t)r * ld + i] = (r == i) ? diagX[i] : Ws[i * kDLd + r];
 }
 
 __global__ void __launch_bounds__(256) dfill_zero_kernel(double *p, long n)
