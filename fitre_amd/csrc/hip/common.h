@@ -68,6 +68,10 @@ struct DOut {
 	void *p;
 	long rs, cs;
 	int kind;
+	// an optional third term of the result, addScale * add(i, j) (doubles; null: none)
+	const double *add = nullptr;
+	long addRs = 0, addCs = 0;
+	double addScale = 0.0;
 };
 inline DMat dmat64(const double *p, long rs, long cs) { return DMat{ p, rs, cs, FITRE_MAT_F64, -1, -1, 0.0 }; }
 inline DMat dmat32(const float *p, long rs, long cs) { return DMat{ p, rs, cs, FITRE_MAT_F32, -1, -1, 0.0 }; }
@@ -75,7 +79,7 @@ inline DMat dmat32(const float *p, long rs, long cs) { return DMat{ p, rs, cs, F
 // mirrored.  Reduction ranges: A(i, k) is zero for k > i (kDgALower) / k < i (kDgAUpper), B(k, j) is zero for k < j
 // (kDgBLower) / k > j (kDgBUpper).
 constexpr int kDgMirror = 1, kDgALower = 2, kDgAUpper = 4, kDgBLower = 8, kDgBUpper = 16;
-// C(M x N) = alpha * A(M x K) * B(K x N) + beta * C, plus diagAdd on the diagonal, accumulated in float64 on the
+// C(M x N) = alpha * A(M x K) * B(K x N) + beta * C (+ C.addScale * C.add), plus diagAdd on the diagonal, accumulated in float64 on the
 // matrix pipes; queued on the selected lane.  ws: dgemm_workspace bytes, 256-byte aligned (a smaller one costs splits).
 int dgemm(long M, long N, long K, double alpha, DMat A, DMat B, double beta, DOut C, double diagAdd, int flags, int kernelClass,
           void *ws, size_t wsBytes);

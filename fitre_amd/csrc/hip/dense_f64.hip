@@ -58,6 +58,7 @@ __device__ __forceinline__ void dgemm_store(const DgemmArgs &g, long i, long j, 
 {
 	if (i >= g.M || j >= g.N) return;
 	double r = g.alpha * v;
+	if (g.C.add) r += g.C.addScale * g.C.add[i * g.C.addRs + j * g.C.addCs];
 	if (g.C.kind == FITRE_MAT_SYM_PAIR) {
 		if (i > j) return; // diagonal tiles hold both halves
 		float *f = (float *)g.C.p;
@@ -462,6 +463,8 @@ int dgemm(long M, long N, long K, double alpha, DMat A, DMat B, double beta, DOu
 		M = N, N = t;
 		const long s = C.rs;
 		C.rs = C.cs, C.cs = s;
+		const long sa = C.addRs;
+		C.addRs = C.addCs, C.addCs = sa;
 		int f = flags & kDgMirror;
 		if (flags & kDgALower) f |= kDgBUpper;
 		if (flags & kDgAUpper) f |= kDgBLower;
@@ -767,6 +770,21 @@ int fitre_hip_gemm_f64(long M, long N, long K, double alpha, const fitre_matrix 
 	return dgemm(M, N, K, alpha, a, b, beta, c, diagAdd, flags, FITRE_KC_FC_GEMM, ws, wsBytes);
 }
 
+int fitre_hip_gemm_f64_add(long M, long N, long K, double alpha, const fitre_matrix *A, const fitre_matrix *B, double addScale,
+                           const fitre_matrix *add, const fitre_matrix *C, void *ws, size_t wsBytes)
+{
+	FITRE_NEED_INIT();
+	DMat a, b;
+	int rc = to_dmat(A, &a, "fitre_hip_gemm_f64_add");
+	if (rc) return rc;
+	rc = to_dmat(B, &b, "fitre_hip_gemm_f64_add");
+	if (rc) return rc;
+	FITRE_REQUIRE(C && C->data && add && add->data && add->kind == FITRE_MAT_F64, "fitre_hip_gemm_f64_add: null result or addend that is not of doubles");
+	DOut c{ (void *)C->data, C->rowStride, C->colStride, C->kind };
+	c.add = (const double *)add->data, c.addRs = add->rowStride, c.addCs = add->colStride, c.addScale = addScale;
+	return dgemm(M, N, K, alpha, a, b, 0.0, c, 0.0, 0, FITRE_KC_FC_GEMM, ws, wsBytes);
+}
+
 size_t fitre_hip_spd_inverse_f64_workspace(int n) { return dspd_inverse_workspace(n); }
 
 int fitre_hip_spd_inverse_f64_queued(double *matrix, int n, void *inverse, int inverseKind, void *ws, size_t wsBytes, int *pivotInfo)
@@ -776,6 +794,44 @@ int fitre_hip_spd_inverse_f64_queued(double *matrix, int n, void *inverse, int i
 	              "fitre_hip_spd_inverse_f64_queued: unknown result kind %d", inverseKind);
 	FITRE_REQUIRE(pivotInfo != nullptr, "fitre_hip_spd_inverse_f64_queued: null pivot slot");
 	return dspd_inverse_run(matrix, n, inverse, inverseKind, ws, wsBytes, pivotInfo);
+}
+
+// the first words of up to 40 arrays, four each, gathered into one array (what a host needs to tell the forms of stored
+// inverses apart with one copy)
+struct HeaderPointers {
+	const uint32_t *p[40];
+};
+__global__ void gather_headers_kernel(HeaderPointers h, int count, uint32_t *out)
+{
+	const int t = blockIdx.x * blockDim.x + threadIdx.x;
+	if (t < 4 * count) out[t] = h.p[t >> 2][t & 3];
+}
+struct HeaderWords {
+	uint32_t w[16];
+};
+__global__ void write_header_kernel(uint32_t *dst, HeaderWords h, int count)
+{
+	if ((int)threadIdx.x < count) dst[threadIdx.x] = h.w[threadIdx.x];
+}
+
+int fitre_hip_gather_headers(const void *const *arrays, int count, void *out)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(arrays && out && count > 0 && count <= 40, "fitre_hip_gather_headers: bad argument");
+	HeaderPointers h;
+	for (int i = 0; i < count; i++) h.p[i] = (const uint32_t *)arrays[i];
+	gather_headers_kernel<<<1, 256, 0, stream()>>>(h, count, (uint32_t *)out);
+	return check_launch("gather_headers_kernel");
+}
+
+int fitre_hip_write_header(void *dst, const unsigned int *words, int count)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(dst && words && count > 0 && count <= 16, "fitre_hip_write_header: bad argument");
+	HeaderWords h;
+	for (int i = 0; i < count; i++) h.w[i] = words[i];
+	write_header_kernel<<<1, 64, 0, stream()>>>((uint32_t *)dst, h, count);
+	return check_launch("write_header_kernel");
 }
 
 int fitre_hip_widen_shift(const float *matrix, int n, double shift, double *out)

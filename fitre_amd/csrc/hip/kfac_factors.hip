@@ -140,6 +140,28 @@ static size_t patch_rows_tail_bytes(const fitre_conv_shape *s, int withBias)
 	return (tail + 255) & ~(size_t)255;
 }
 
+
+// ---- the operand of an input-side factor itself, for factors kept in low-rank form -----------------------------
+// rows[r][m] (row r contiguous): the patch rows of patch_rows_kernel, and under them (withBias) one row that is outA * outB
+// everywhere: R with P^T P / samples = R R^T / (cells^2 samples).
+__global__ void __launch_bounds__(256) fill_row_kernel(float *row, long n, float v)
+{
+	const long stride = (long)gridDim.x * blockDim.x;
+	for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < n; idx += stride) row[idx] = v;
+}
+
+// out (n x samples, column-major) = [ z ; 1 ] for z (in x samples, column-major)
+__global__ void __launch_bounds__(256) rows_with_ones_kernel(const float *z, int in, int samples, int withBias, float *out)
+{
+	const int n = in + (withBias ? 1 : 0);
+	const long total = (long)n * samples;
+	const long stride = (long)gridDim.x * blockDim.x;
+	for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
+		const int s = (int)(idx / n), r = (int)(idx - (long)s * n);
+		out[idx] = r < in ? z[(size_t)s * in + r] : 1.f;
+	}
+}
+
 } // namespace fitre
 
 using namespace fitre;
@@ -371,6 +393,30 @@ int fitre_hip_kfac_fc_output_factor_f64(const float *delta, int outDim, int samp
 	FITRE_REQUIRE(outDim > 0 && samples > 0, "fitre_hip_kfac_fc_output_factor_f64: non-positive shape %d x %d", outDim, samples);
 	return dgemm(outDim, outDim, samples, (double)samples, dmat32(delta, 1, outDim), dmat32(delta, outDim, 1), 0.0,
 	             DOut{ factor, 1, outDim, FITRE_MAT_F64 }, shift, kDgMirror, FITRE_KC_KFAC_FACTOR, ws, wsBytes);
+}
+
+int fitre_hip_kfac_conv_input_rows(const fitre_conv_shape *s, const float *x, int withBias, float *rows)
+{
+	FITRE_NEED_INIT();
+	int rc = check_conv("fitre_hip_kfac_conv_input_rows", s);
+	if (rc) return rc;
+	FITRE_REQUIRE(x && rows, "fitre_hip_kfac_conv_input_rows: null pointer");
+	const int K = s->inChannels * s->ksize * s->ksize;
+	const long R = (long)s->samples * s->outA * s->outB;
+	PatchGeom g = make_patch_geom(x, s->inChannels, s->samples, s->inA, s->inB, s->outA, s->outB, s->ksize, s->stride, s->padding);
+	LaunchScope scope(FITRE_KC_BLAS1, 4.0 * (double)(K + 1) * (double)R);
+	const dim3 grid(blocks_for(R, 256, 64), (unsigned)K);
+	patch_rows_kernel<<<grid, 256, 0, stream()>>>(g, rows);
+	if (withBias) fill_row_kernel<<<blocks_for(R, 256, 256), 256, 0, stream()>>>(rows + (size_t)K * R, R, (float)(s->outA * s->outB));
+	return check_launch("fitre_hip_kfac_conv_input_rows");
+}
+
+int fitre_hip_kfac_fc_input_rows(const float *z, int in, int samples, int withBias, float *rows)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(z && rows && in > 0 && samples > 0, "fitre_hip_kfac_fc_input_rows: bad argument");
+	rows_with_ones_kernel<<<blocks_for((long)(in + 1) * samples, 256, 4096), 256, 0, stream()>>>(z, in, samples, withBias, rows);
+	return check_launch("rows_with_ones_kernel");
 }
 
 } // extern "C"

@@ -216,10 +216,40 @@ long kfacInverseMemRequired(CNN_MODEL *model, int samples)
 
 /* writes the float64 factor of `layer` (convolution layers, then linear ones), damping included, into `factor` */
 typedef void (*FACTOR_FN)(void *ctx, int layer, double shift, double *factor, void *ws, size_t wsBytes);
+/* writes the operand R of an input-side factor (factor = alpha R R^T, R order x positions) to `rows` and reports its
+ * strides and alpha */
+typedef void (*ROWS_FN)(void *ctx, int layer, real *rows, long *rowStride, long *colStride, double *alpha);
+
+/* An input-side factor with fewer positions behind it than half its order (the last layers of a deep network:
+ * order 9 Cin + 1 from samples * outH * outW patches) is kept in LOW-RANK FORM instead of as a dense inverse:
+ *   (alpha R R^T + s I)^-1 = (I - alpha R S^-1 R^T) / s,   S = s I + alpha R^T R   (positions x positions),
+ * i.e. the slot holds R itself and the inverse of the small matrix S -- an inverse of order positions instead of
+ * order, and three thin products per application instead of one square one.  The slot then starts with a header
+ * whose first word no dense inverse can start with (a negative float on the diagonal of a positive definite
+ * matrix), so that computeNaturalGradient can tell the forms apart:
+ *   word 0 tag, 1 positions, 2 order, 3 / 4 row and column stride of R, 5-6 alpha, 7-8 s (doubles), 9 the word at which
+ *   S^-1 starts;
+ *   R at word KFAC_LOWRANK_HEADER, S^-1 behind it as doubles (at the next 8-byte boundary): applying this form subtracts two
+ *   nearly equal terms, and the 32 bits a float pair has on its diagonal would cost the result three digits. */
+#define KFAC_LOWRANK_TAG 0xF15EED12u
+#define KFAC_LOWRANK_HEADER 64
+static int lowrank_eligible(int order, long positions)
+{
+	return positions >= 1 && 2 * positions <= order && order >= 64 &&
+	       (size_t)KFAC_LOWRANK_HEADER + (size_t)order * positions + 2 * (size_t)positions * positions + 2 <= (size_t)order * order;
+}
+
+/* where S^-1 (doubles) starts in a low-rank slot */
+static double *lowrank_sinv(const real *slot, int order, long positions)
+{
+	return (double *)(((size_t)(slot + KFAC_LOWRANK_HEADER + (size_t)order * positions) + 7) & ~(size_t)7);
+}
 
 /* one matrix of a pass: how to make its factor, its order, where its inverse goes */
 typedef struct inverse_item {
 	FACTOR_FN make;
+	ROWS_FN rows; /* non-NULL: the factor may be kept in low-rank form */
+	long positions;
 	void *ctx;
 	int layer;
 	int order;
@@ -257,7 +287,9 @@ static void inverse_pass_run(const CNN_MODEL *model, int samples, real *devPtr, 
 	for (int i = 0; i < count; i++) {
 		jobs[i].item = i;
 		/* a chain of launches whose length grows with the order, plus the arithmetic */
-		jobs[i].cost = (double)items[i].order * (200.0 + (double)items[i].order * items[i].order * 1e-3);
+		const int lowrank = items[i].rows != NULL && lowrank_eligible(items[i].order, items[i].positions);
+		const double n = lowrank ? (double)items[i].positions : (double)items[i].order;
+		jobs[i].cost = n * (200.0 + n * n * 1e-3) + (lowrank ? 2e-3 * n * n * items[i].order : 0.0);
 	}
 	qsort(jobs, (size_t)count, sizeof(INVERSE_JOB), job_by_cost);
 	double load[KFAC_LANES] = { 0, 0, 0, 0 };
@@ -270,6 +302,25 @@ static void inverse_pass_run(const CNN_MODEL *model, int samples, real *devPtr, 
 		load[lane] += jobs[i].cost;
 		char *slot = slots + (size_t)lane * slotBytes;
 		HIP_CALL(fitre_hip_lane_select(lane));
+		if (it->rows != NULL && lowrank_eligible(it->order, it->positions)) {
+			const long m = it->positions;
+			real *rows = it->inverse + KFAC_LOWRANK_HEADER;
+			long rs, cs;
+			double alpha;
+			it->rows(it->ctx, it->layer, rows, &rs, &cs, &alpha);
+			/* S = shift I + alpha R^T R, in the slot's factor area */
+			fitre_matrix rt = { rows, cs, rs, FITRE_MAT_F32, -1, -1, 0.0 }, r = { rows, rs, cs, FITRE_MAT_F32, -1, -1, 0.0 };
+			fitre_matrix sm = { slot, 1, m, FITRE_MAT_F64, -1, -1, 0.0 };
+			HIP_CALL(fitre_hip_gemm_f64(m, m, it->order, alpha, &rt, &r, 0.0, &sm, shift, FITRE_GEMM_SYMMETRIC, slot + factorBytes, wsBytes));
+			HIP_CALL(fitre_hip_spd_inverse_f64_queued((double *)slot, (int)m, lowrank_sinv(it->inverse, it->order, m), FITRE_MAT_F64,
+			                                          slot + factorBytes, wsBytes, pivots + jobs[i].item));
+			union { double d; unsigned int w[2]; } a = { alpha }, sh = { shift };
+			unsigned int header[10] = { KFAC_LOWRANK_TAG, (unsigned int)m, (unsigned int)it->order, (unsigned int)rs, (unsigned int)cs,
+				                        a.w[0], a.w[1], sh.w[0], sh.w[1],
+				                        (unsigned int)((const real *)lowrank_sinv(it->inverse, it->order, m) - it->inverse) };
+			HIP_CALL(fitre_hip_write_header(it->inverse, header, 10));
+			continue;
+		}
 		it->make(it->ctx, it->layer, shift, (double *)slot, slot + factorBytes, wsBytes);
 		HIP_CALL(fitre_hip_spd_inverse_f64_queued((double *)slot, it->order, it->inverse, FITRE_MAT_SYM_PAIR, slot + factorBytes, wsBytes,
 		                                          pivots + jobs[i].item));
@@ -323,6 +374,40 @@ static void omega_factor(void *ctx, int layer, double shift, double *factor, voi
 	}
 }
 
+static void omega_rows(void *ctx, int layer, real *rows, long *rowStride, long *colStride, double *alpha)
+{
+	const OMEGA_CTX *o = (const OMEGA_CTX *)ctx;
+	const CNN_MODEL *model = o->model;
+	const int nc = model->cLayers;
+	if (layer < nc) {
+		const int l = layer;
+		const CONV_LAYER *c = &model->convLayer[l];
+		const real *input;
+		if (o->dampedInput != NULL)
+			input = (l == 0) ? o->dampedInput : o->dampedZ + o->zztOffsets[l];
+		else
+			input = (l == 0) ? o->data->currentBatch : o->dampedZ + o->zOffsets[l] + model->convLayer[l - 1].outputOffset;
+		fitre_conv_shape s = conv_shape(c, o->samples);
+		HIP_CALL(fitre_hip_kfac_conv_input_rows(&s, input, o->withBias, rows));
+		const double cells = (double)c->outHeight * c->outWidth;
+		*rowStride = (long)o->samples * c->outHeight * c->outWidth, *colStride = 1;
+		*alpha = 1.0 / (cells * cells * (double)o->samples);
+	} else {
+		const int l = layer - nc;
+		const FC_LAYER *f = &model->fcLayer[l];
+		const real *input;
+		if (o->dampedInput != NULL)
+			input = o->dampedZ + o->zztOffsets[nc + l];
+		else if (l == 0)
+			input = o->dampedZ + o->zOffsets[nc] + model->convLayer[nc - 1].outputOffset;
+		else
+			input = o->dampedZ + o->zOffsets[nc + l];
+		HIP_CALL(fitre_hip_kfac_fc_input_rows(input, f->in, o->samples, o->withBias, rows));
+		*rowStride = 1, *colStride = f->in + (o->withBias ? 1 : 0);
+		*alpha = 1.0 / (double)o->samples;
+	}
+}
+
 /* items of the input-side factors; returns their number */
 static int omega_items(INVERSE_ITEM *items, const KFAC_CURVATURE_INFO *kfac_info, const CNN_MODEL *model, OMEGA_CTX *ctx,
                        real *omegaZInv)
@@ -332,14 +417,17 @@ static int omega_items(INVERSE_ITEM *items, const KFAC_CURVATURE_INFO *kfac_info
 	for (int l = 0; l < layers; l++) {
 		INVERSE_ITEM *it = &items[l];
 		it->make = omega_factor;
+		it->rows = omega_rows;
 		it->ctx = ctx;
 		it->layer = l;
 		if (l < nc) {
 			const CONV_LAYER *c = &model->convLayer[l];
 			it->order = c->inChannels * c->kSize * c->kSize + (ctx->withBias ? 1 : 0);
+			it->positions = (long)ctx->samples * c->outHeight * c->outWidth;
 			it->group = 0;
 		} else {
 			it->order = model->fcLayer[l - nc].in + (ctx->withBias ? 1 : 0);
+			it->positions = ctx->samples;
 			it->group = 1;
 		}
 		it->inverse = omegaZInv + omega[l];
@@ -398,6 +486,8 @@ static int lambda_items(INVERSE_ITEM *items, const KFAC_CURVATURE_INFO *kfac_inf
 	for (int l = 0; l < layers; l++) {
 		INVERSE_ITEM *it = &items[l];
 		it->make = lambda_factor;
+		it->rows = NULL;
+		it->positions = 0;
 		it->ctx = ctx;
 		it->layer = l;
 		it->order = l < nc ? model->convLayer[l].outChannels : model->fcLayer[l - nc].out;
@@ -449,7 +539,8 @@ static size_t natural_gradient_bytes(const CNN_MODEL *model, size_t *matBytes)
 		ws = max_sz(ws, max_sz(fitre_hip_gemm_f64_workspace(o, k, o, 0), fitre_hip_gemm_f64_workspace(o, k, k, 0)));
 	}
 	*matBytes = round_up(mat, 256);
-	return 3 * *matBytes + round_up(ws, 256) + 256;
+	/* [wb | u | zt | t1 | t2 | headers | product workspace]; t1, t2 (low-rank form: positions x Cout, positions <= order / 2) */
+	return 5 * *matBytes + KFAC_INFO_BYTES + round_up(ws, 256) + 256;
 }
 
 long kfacNaturalGradientMemRequired(CNN_MODEL *model)
@@ -464,6 +555,46 @@ static fitre_matrix mat_of(const void *data, long rowStride, long colStride, int
 	return m;
 }
 
+/* what the header of an input-side slot says (inverse_pass_run) */
+typedef struct omega_form {
+	int lowrank;
+	long positions, rs, cs;
+	double alpha, shift;
+} OMEGA_FORM;
+
+/* result (rows x cols, `out`) = Omega^-1 applied to u (doubles) from the left (conv: Omega^-1 * u, u order x cols) or
+ * from the right (linear: u * Omega^-1, u rows x order), for either form of the stored inverse */
+static void apply_omega(const OMEGA_FORM *form, const real *slot, int order, int other, int fromLeft, const double *u,
+                        const fitre_matrix *out, double *t1, double *t2, void *ws, size_t wsBytes)
+{
+	const long ldu = fromLeft ? order : other;
+	const fitre_matrix um = mat_of(u, 1, ldu, FITRE_MAT_F64);
+	if (!form->lowrank) {
+		const fitre_matrix omega = mat_of(slot, order, order, FITRE_MAT_SYM_PAIR);
+		if (fromLeft)
+			HIP_CALL(fitre_hip_gemm_f64(order, other, order, 1.0, &omega, &um, 0.0, out, 0.0, 0, ws, wsBytes));
+		else
+			HIP_CALL(fitre_hip_gemm_f64(other, order, order, 1.0, &um, &omega, 0.0, out, 0.0, 0, ws, wsBytes));
+		return;
+	}
+	/* (I - alpha R S^-1 R^T) u / s, resp. u (I - alpha R S^-1 R^T) / s */
+	const long m = form->positions;
+	const real *rows = slot + KFAC_LOWRANK_HEADER;
+	const fitre_matrix r = mat_of(rows, form->rs, form->cs, FITRE_MAT_F32), rt = mat_of(rows, form->cs, form->rs, FITRE_MAT_F32);
+	const fitre_matrix sinv = mat_of(lowrank_sinv(slot, order, m), 1, m, FITRE_MAT_F64);
+	if (fromLeft) {
+		const fitre_matrix a = mat_of(t1, 1, m, FITRE_MAT_F64), b = mat_of(t2, 1, m, FITRE_MAT_F64); /* positions x other */
+		HIP_CALL(fitre_hip_gemm_f64(m, other, order, 1.0, &rt, &um, 0.0, &a, 0.0, 0, ws, wsBytes));
+		HIP_CALL(fitre_hip_gemm_f64(m, other, m, 1.0, &sinv, &a, 0.0, &b, 0.0, 0, ws, wsBytes));
+		HIP_CALL(fitre_hip_gemm_f64_add(order, other, m, -form->alpha / form->shift, &r, &b, 1.0 / form->shift, &um, out, ws, wsBytes));
+	} else {
+		const fitre_matrix a = mat_of(t1, 1, other, FITRE_MAT_F64), b = mat_of(t2, 1, other, FITRE_MAT_F64); /* other x positions */
+		HIP_CALL(fitre_hip_gemm_f64(other, m, order, 1.0, &um, &r, 0.0, &a, 0.0, 0, ws, wsBytes));
+		HIP_CALL(fitre_hip_gemm_f64(other, m, m, 1.0, &a, &sinv, 0.0, &b, 0.0, 0, ws, wsBytes));
+		HIP_CALL(fitre_hip_gemm_f64_add(other, order, m, -form->alpha / form->shift, &b, &rt, 1.0 / form->shift, &um, out, ws, wsBytes));
+	}
+}
+
 void computeNaturalGradient(CNN_MODEL *model, KFAC_CURVATURE_INFO *kfacInfo, real *devPtr, real *hostPtr)
 {
 	(void)hostPtr;
@@ -471,24 +602,46 @@ void computeNaturalGradient(CNN_MODEL *model, KFAC_CURVATURE_INFO *kfacInfo, rea
 	const int *omegaOff = kfacInfo->OmegaZOffsets, *lambdaOff = kfacInfo->LambdaGOffsets;
 	const real *vec = kfacInfo->gradient;
 	real *nGradient = kfacInfo->nGradient;
-	const int bias = model->bias != 0, nc = model->cLayers;
+	const int bias = model->bias != 0, nc = model->cLayers, layers = nc + model->lLayers;
 	size_t matBytes;
 	const size_t total = natural_gradient_bytes(model, &matBytes);
 	char *base = aligned_base(devPtr);
 	real *wb = (real *)base, *zt = (real *)(base + 2 * matBytes);
-	double *u = (double *)(base + matBytes);
-	void *ws = base + 3 * matBytes;
-	const size_t wsBytes = total - 3 * matBytes - 256;
+	double *u = (double *)(base + matBytes), *t1 = (double *)(base + 3 * matBytes), *t2 = (double *)(base + 4 * matBytes);
+	unsigned int *headers = (unsigned int *)(base + 5 * matBytes);
+	void *ws = base + 5 * matBytes + KFAC_INFO_BYTES;
+	const size_t wsBytes = total - 5 * matBytes - KFAC_INFO_BYTES - 256;
 
-	/* Both inverses are float pairs (inverse_pass_run); the two products of a layer accumulate in float64, the
-	 * first one's result stays in doubles, and only the natural gradient itself is rounded to floats.
+	/* which form every input-side inverse is stored in: the heads of the slots, with one copy */
+	OMEGA_FORM forms[MAX_LAYERS];
+	{
+		const void *slots[MAX_LAYERS];
+		unsigned int host[4 * MAX_LAYERS + 8];
+		for (int l = 0; l < layers; l++) slots[l] = kfacInfo->OmegaZInv + omegaOff[l];
+		HIP_CALL(fitre_hip_gather_headers(slots, layers, headers));
+		HIP_CALL(fitre_hip_sync());
+		HIP_CALL(fitre_hip_copy_d2h(host, headers, sizeof(unsigned int) * 4 * (size_t)layers));
+		for (int l = 0; l < layers; l++) {
+			forms[l].lowrank = host[4 * l] == KFAC_LOWRANK_TAG;
+			if (!forms[l].lowrank) continue;
+			unsigned int rest[9];
+			HIP_CALL(fitre_hip_copy_d2h(rest, (const void *)slots[l], sizeof(rest)));
+			union { double d; unsigned int w[2]; } a, sh;
+			a.w[0] = rest[5], a.w[1] = rest[6], sh.w[0] = rest[7], sh.w[1] = rest[8];
+			forms[l].positions = rest[1], forms[l].rs = rest[3], forms[l].cs = rest[4];
+			forms[l].alpha = a.d, forms[l].shift = sh.d;
+		}
+	}
+
+	/* Both inverses are float pairs, or a low-rank form on the input side (inverse_pass_run); the products of a layer
+	 * accumulate in float64, what passes from one to the next stays in doubles, and only the natural gradient itself is
+	 * rounded to floats.
 	 * Convolution layers.  The reference forms Lambda * wb' * Omega (Cout x (K+1)) and transposes the
 	 * weight part back; Lambda and Omega are symmetric, so the transposed product Omega * (wb * Lambda)
 	 * is the same matrix already in the parameter layout ((K+1) x Cout, one column per filter). */
 	for (int c = 0; c < nc; c++) {
 		const CONV_LAYER *l = &model->convLayer[c];
 		const int K = l->inChannels * l->kSize * l->kSize, O = l->outChannels, R = K + bias;
-		const fitre_matrix omega = mat_of(kfacInfo->OmegaZInv + omegaOff[c], R, R, FITRE_MAT_SYM_PAIR);
 		const fitre_matrix lambda = mat_of(kfacInfo->LambdaGInv + lambdaOff[c], O, O, FITRE_MAT_SYM_PAIR);
 		const real *v = vec + wOffsets[c];
 		real *ng = nGradient + wOffsets[c];
@@ -502,12 +655,12 @@ void computeNaturalGradient(CNN_MODEL *model, KFAC_CURVATURE_INFO *kfacInfo, rea
 		HIP_CALL(fitre_hip_gemm_f64(R, O, O, 1.0, &g, &lambda, 0.0, &um, 0.0, 0, ws, wsBytes));
 		if (bias) {
 			const fitre_matrix out = mat_of(zt, 1, R, FITRE_MAT_F32);
-			HIP_CALL(fitre_hip_gemm_f64(R, O, R, 1.0, &omega, &um, 0.0, &out, 0.0, 0, ws, wsBytes));
+			apply_omega(&forms[c], kfacInfo->OmegaZInv + omegaOff[c], R, O, 1, u, &out, t1, t2, ws, wsBytes);
 			HIP_CALL(fitre_hip_copy_2d(ng, K, zt, R, K, O));
 			HIP_CALL(fitre_hip_copy_2d(nGradient + bOffsets[c], 1, zt + K, R, 1, O));
 		} else {
 			const fitre_matrix out = mat_of(ng, 1, R, FITRE_MAT_F32);
-			HIP_CALL(fitre_hip_gemm_f64(R, O, R, 1.0, &omega, &um, 0.0, &out, 0.0, 0, ws, wsBytes));
+			apply_omega(&forms[c], kfacInfo->OmegaZInv + omegaOff[c], R, O, 1, u, &out, t1, t2, ws, wsBytes);
 		}
 	}
 	/* Linear layers: the gradient block [W | b] already is the out x (in + 1) matrix
@@ -515,12 +668,11 @@ void computeNaturalGradient(CNN_MODEL *model, KFAC_CURVATURE_INFO *kfacInfo, rea
 	for (int f = 0; f < model->lLayers; f++) {
 		const FC_LAYER *l = &model->fcLayer[f];
 		const int R = l->in + bias, O = l->out;
-		const fitre_matrix omega = mat_of(kfacInfo->OmegaZInv + omegaOff[nc + f], R, R, FITRE_MAT_SYM_PAIR);
 		const fitre_matrix lambda = mat_of(kfacInfo->LambdaGInv + lambdaOff[nc + f], O, O, FITRE_MAT_SYM_PAIR);
 		const fitre_matrix g = mat_of(vec + wOffsets[nc + f], 1, O, FITRE_MAT_F32), um = mat_of(u, 1, O, FITRE_MAT_F64);
 		const fitre_matrix out = mat_of(nGradient + wOffsets[nc + f], 1, O, FITRE_MAT_F32);
 		HIP_CALL(fitre_hip_gemm_f64(O, R, O, 1.0, &lambda, &g, 0.0, &um, 0.0, 0, ws, wsBytes));
-		HIP_CALL(fitre_hip_gemm_f64(O, R, R, 1.0, &um, &omega, 0.0, &out, 0.0, 0, ws, wsBytes));
+		apply_omega(&forms[nc + f], kfacInfo->OmegaZInv + omegaOff[nc + f], R, O, 0, u, &out, t1, t2, ws, wsBytes);
 	}
 	HIP_CALL(fitre_hip_sync());
 }

@@ -140,6 +140,28 @@ def pair_encode(s):
     return out
 
 
+KFAC_LOWRANK_TAG, KFAC_LOWRANK_HEADER = 0xF15EED12, 64
+
+
+def stored_inverse(words, n):
+    """The dense float64 inverse that the n * n floats of a KFAC slot stand for: a float-pair matrix (column-major), or --
+    input-side factors with few positions behind them -- the low-rank form of kfac_path.c: a header (tag, positions,
+    order, strides of R, alpha and the damping s as doubles, the word at which S^-1 starts), R and S^-1 as doubles, for
+    (alpha R R^T + s I)^-1 = (I - alpha R S^-1 R^T) / s."""
+    words = np.ascontiguousarray(words, dtype=np.float32)
+    head = words[:16].view(np.uint32)
+    if n * n >= 16 and int(head[0]) == KFAC_LOWRANK_TAG:
+        m, order, rs, cs = int(head[1]), int(head[2]), int(head[3]), int(head[4])
+        assert order == n
+        alpha, shift = head[5:9].view(np.float64)
+        body = words[KFAC_LOWRANK_HEADER:]
+        r = np.lib.stride_tricks.as_strided(body, shape=(n, m), strides=(4 * rs, 4 * cs)).astype(np.float64)
+        at = int(head[9])                                    # doubles, at an 8-byte boundary of the device array
+        sinv = words[at:at + 2 * m * m].view(np.float64).reshape(m, m)
+        return (np.eye(n) - alpha * (r @ sinv @ r.T)) / shift
+    return pair_decode(words[:n * n].reshape(n, n).T)
+
+
 # ---------------------------------------------------------------- device buffers
 class Device:
     """Owns device buffers through the C-ABI (no torch involved)."""

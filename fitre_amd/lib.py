@@ -147,6 +147,11 @@ HIP_API = {
     "fitre_hip_kfac_fc_output_factor": (i32, [vp, i32, i32, vp, vp, sz]),
     "fitre_hip_gemm_f64_workspace": (sz, [lng, lng, lng, i32]),
     "fitre_hip_gemm_f64": (i32, [lng, lng, lng, f64, pmat, pmat, f64, pmat, f64, i32, vp, sz]),
+    "fitre_hip_gemm_f64_add": (i32, [lng, lng, lng, f64, pmat, pmat, f64, pmat, pmat, vp, sz]),
+    "fitre_hip_kfac_conv_input_rows": (i32, [vp, vp, i32, vp]),
+    "fitre_hip_kfac_fc_input_rows": (i32, [vp, i32, i32, i32, vp]),
+    "fitre_hip_gather_headers": (i32, [vp, i32, vp]),
+    "fitre_hip_write_header": (i32, [vp, vp, i32]),
     "fitre_hip_spd_inverse_f64_workspace": (sz, [i32]),
     "fitre_hip_spd_inverse_f64_queued": (i32, [vp, i32, vp, i32, vp, sz, vp]),
     "fitre_hip_widen_shift": (i32, [vp, i32, f64, vp]),

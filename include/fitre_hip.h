@@ -567,6 +567,9 @@ typedef struct fitre_matrix {
 size_t fitre_hip_gemm_f64_workspace(long M, long N, long K, int flags);
 int fitre_hip_gemm_f64(long M, long N, long K, double alpha, const fitre_matrix *A, const fitre_matrix *B, double beta,
                        const fitre_matrix *C, double diagAdd, int flags, void *ws, size_t wsBytes);
+/* C = alpha * A * B + addScale * add, add a matrix of doubles (no beta term, no flags). */
+int fitre_hip_gemm_f64_add(long M, long N, long K, double alpha, const fitre_matrix *A, const fitre_matrix *B, double addScale,
+                           const fitre_matrix *add, const fitre_matrix *C, void *ws, size_t wsBytes);
 /* inverse = matrix^-1 for a symmetric positive definite matrix of n x n doubles (dense, destroyed): Cholesky factor and
  * its inverse by halving, then X^T X, all in float64; the result is stored dense with leading dimension n as
  * inverseKind.  Queued on the selected lane; pivotInfo (device int) holds 0 or the 1-based index of the first
@@ -574,6 +577,16 @@ int fitre_hip_gemm_f64(long M, long N, long K, double alpha, const fitre_matrix 
 size_t fitre_hip_spd_inverse_f64_workspace(int n);
 int fitre_hip_spd_inverse_f64_queued(double *matrix, int n, void *inverse, int inverseKind, void *ws, size_t wsBytes,
                                      int *pivotInfo);
+/* The operand of an input-side factor itself, for a factor kept in low-rank form (kfac_path.c): rows[r][m], row r
+ * contiguous over the samples*outA*outB positions, r = the patch index (c, ta, tb), plus (withBias) a last row that is
+ * outA*outB everywhere: A = rows rows^T / ((outA*outB)^2 samples).  Fully connected: rows = [ z ; 1 ], (in + 1) x samples
+ * column-major, A = rows rows^T / samples. */
+int fitre_hip_kfac_conv_input_rows(const fitre_conv_shape *s, const float *x, int withBias, float *rows);
+int fitre_hip_kfac_fc_input_rows(const float *z, int in, int samples, int withBias, float *rows);
+/* The first four 32-bit words of `count` (at most 40) device arrays, gathered into out (device, 4 * count words);
+ * count (at most 16) words written to the head of a device array.  Stream-ordered. */
+int fitre_hip_gather_headers(const void *const *arrays, int count, void *out);
+int fitre_hip_write_header(void *dst, const unsigned int *words, int count);
 /* out(n x n doubles) = matrix(n x n floats) + shift * I */
 int fitre_hip_widen_shift(const float *matrix, int n, double shift, double *out);
 /* The four Kronecker factors above accumulated in float64 and written as n x n doubles, with `shift` (the damping) added

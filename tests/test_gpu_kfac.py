@@ -6,7 +6,7 @@ import numpy as np
 import pytest
 
 from fitre_amd import lib as L
-from helpers import conv_shape, pair_decode, rel_err
+from helpers import conv_shape, stored_inverse, rel_err
 
 pytestmark = pytest.mark.gpu
 TOL = 1e-4
@@ -434,7 +434,7 @@ def test_model_inverses_and_natural_gradient(dev, oracle64, name):
         assert oi == 0
         ev = np.linalg.eigvalsh(factor + (lam + gamma) * np.eye(n))
         tol = TOL * max(1.0, (ev[-1] / ev[0]) / 50.0)
-        got = pair_decode(got.reshape(n, n).T)            # column-major float pairs
+        got = stored_inverse(got, n)                      # float pairs, or the low-rank form
         dec[at:at + n * n] = got.reshape(-1)
         assert rel_err(got, want) < tol, (what, ev[-1] / ev[0])
         assert np.abs((factor + (lam + gamma) * np.eye(n)) @ got - np.eye(n)).max() < tol, what
@@ -467,7 +467,7 @@ def test_model_inverses_and_natural_gradient(dev, oracle64, name):
 @pytest.mark.parametrize("name", ["lenet_bias", "small_vgg_bn", "vgg11_b256"])
 def test_both_inverse_passes_as_one(dev, name):
     """computeOmegaZAndLambdaDelta against computeOmegaZ followed by computeLambdaDelta on the same z / dx: the same
-    matrices, whatever lanes and batches they were dealt to."""
+    matrices, whatever lanes they were dealt to."""
     from fitre_amd.structs import KFAC_CURVATURE_INFO
     from helpers import GpuModel, batch_inputs, he_weights
     model, batch = next((m, b) for n, m, b in _model_cases() if n == name)
@@ -490,10 +490,12 @@ def test_both_inverse_passes_as_one(dev, name):
     info.OmegaZInv, info.LambdaGInv = o2.value, l2.value
     L.cnn.computeOmegaZAndLambdaDelta(C.byref(info), C.byref(model), C.byref(gm.data), batch, None, gm.z, gm.dx, None,
                                       model.zOffsets, model.zztOffsets, ws)
-    a, b = dev.download(o1, tot_o), dev.download(o2, tot_o)
-    assert np.isfinite(a).all() and rel_err(b, a) < 1e-6
-    a, b = dev.download(l1, tot_l), dev.download(l2, tot_l)
-    assert np.isfinite(a).all() and rel_err(b, a) < 1e-6
+    # the stored forms (float pairs, low-rank slots with doubles inside) word for word: a matrix does not depend on the
+    # lane it was dealt to
+    a, b = dev.download(o1, tot_o, dtype=np.uint32), dev.download(o2, tot_o, dtype=np.uint32)
+    assert a.any() and np.array_equal(a, b)
+    a, b = dev.download(l1, tot_l, dtype=np.uint32), dev.download(l2, tot_l, dtype=np.uint32)
+    assert a.any() and np.array_equal(a, b)
     for q in (o1, l1, o2, l2, ws):
         dev.free(q)
     gm.release()
@@ -557,8 +559,9 @@ def test_vgg11_kfac_leg_against_a_float64_pipeline(dev, oracle64):
     256, damping lambda = 1e-3 and nothing else: input-side factors of order up to 4609 with 1024 patches behind them,
     condition numbers up to 7e5) as the solver runs it (computeOmegaZAndLambdaDelta, computeNaturalGradient), against the
     same leg done entirely in float64 on the host from the z / dx / gradient the device holds: the device's own factors
-    and inverses are never fed to the checker.  Bounds: every stored inverse (float pairs) within 1e-7 of the largest
-    element of LAPACK's, every layer block of the natural gradient within 1e-4 of its largest magnitude."""
+    and inverses are never fed to the checker.  Bounds: every stored inverse (float pairs; the low-rank form for the three
+    input-side factors with at most half as many patches as their order) within 1e-7 of the largest element of LAPACK's,
+    every layer block of the natural gradient within 1e-4 of its largest magnitude."""
     from fitre_amd.structs import KFAC_CURVATURE_INFO
     from helpers import GpuModel, batch_inputs, build_vgg11, he_weights
     batch, lam = 256, float(np.float32(1e-3))     # the damping is a real (float) in the reference's struct
@@ -591,9 +594,9 @@ def test_vgg11_kfac_leg_against_a_float64_pipeline(dev, oracle64):
     def compare_inverses(l, omega_inverse, lambda_inverse):
         for want, ptr, offs, what in ((omega_inverse, oinv, info.OmegaZOffsets, "omega"), (lambda_inverse, linv, info.LambdaGOffsets, "lambda")):
             n = want.shape[0]
-            pairs = dev.download(ptr, n * n, offset=offs[l]).reshape(n, n)
-            assert np.isfinite(pairs).all(), (what, l)
-            inverse_errors.append((what, l, rel_err(pair_decode(pairs.T), want)))
+            stored = stored_inverse(dev.download(ptr, n * n, offset=offs[l]), n)
+            assert np.isfinite(stored).all(), (what, l)
+            inverse_errors.append((what, l, rel_err(stored, want)))
 
     want, conds = _float64_natural_gradient(oracle64, model, batch, x, z, dxs, grad, lam, compare_inverses)
     for q in (oinv, linv, ngrad, ws):
