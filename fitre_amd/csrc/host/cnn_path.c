@@ -271,6 +271,14 @@ static double backward_flop_per_elementwise_byte(const CNN_MODEL *model, int n)
 }
 #define LANE_WORK_THRESHOLD 2.0e9
 #define LANE_INTENSITY_LIMIT 250.0
+/* -1: by the two limits above (fitted on LeNet, VGG-11 and AlexNet); 0: one lane; 1: lanes, whatever the network */
+static int g_backward_lanes = -1;
+void fitreSetBackwardLanes(int mode) { g_backward_lanes = mode < 0 ? -1 : (mode ? 1 : 0); }
+int fitreBackwardUsesLanes(CNN_MODEL *model, int batchSize)
+{
+	if (g_backward_lanes >= 0) return g_backward_lanes;
+	return backward_conv_work(model, batchSize) >= LANE_WORK_THRESHOLD && backward_flop_per_elementwise_byte(model, batchSize) < LANE_INTENSITY_LIMIT;
+}
 #define LANE_SELECT(lane_) do { if (lanes) HIP_CALL(fitre_hip_lane_select(lane_)); } while (0)
 #define LANE_WAIT(waiter_, signaller_) do { if (lanes) HIP_CALL(fitre_hip_lane_wait(waiter_, signaller_)); } while (0)
 
@@ -282,7 +290,7 @@ void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, 
 	const int *wOffsets = model->wOffsets, *bOffsets = model->bOffsets, *zOffsets = model->zOffsets;
 	const real *weights = data->weights;
 	const int n = batchSize, nc = model->cLayers;
-	const int lanes = backward_conv_work(model, n) >= LANE_WORK_THRESHOLD && backward_flop_per_elementwise_byte(model, n) < LANE_INTENSITY_LIMIT;
+	const int lanes = fitreBackwardUsesLanes(model, n);
 	void *ws = (void *)devPtr; /* input-gradient partials (and the FC products' splits) */
 	const size_t wsBytes = backward_dx_ws_bytes(model, model->batchSize);
 	void *bnWs = (void *)((char *)devPtr + wsBytes);
@@ -316,7 +324,11 @@ void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, 
 			const size_t bytes = fitre_hip_conv_input_grad_prepared_bytes(&shape);
 			prepared[c] = NULL;
 			if (bytes == 0 || !has_bn(&model->convLayer[c - 1])) continue;
-			if (!any) LANE_SELECT(2);
+			if (!any) {
+				/* behind whatever the caller has queued on lane 0 (a weight update, say): the copies read the weights */
+				LANE_WAIT(2, 0);
+				LANE_SELECT(2);
+			}
 			any = 1;
 			HIP_CALL(fitre_hip_conv_input_grad_prepare(&shape, weights + wOffsets[c], preparedWs, bytes));
 			prepared[c] = preparedWs;

@@ -187,6 +187,8 @@ CNN_API = {
     "cnnBackwardMemRequired": (lng, [pmodel]),
     "cnnBackward": (None, [pmodel, pdata, vp, vp, vp, vp, vp, vp, i32, i32, vp]),
     "fitreBackwardUnsupportedLayer": (i32, [pmodel]),
+    "fitreSetBackwardLanes": (None, [i32]),
+    "fitreBackwardUsesLanes": (i32, [pmodel, i32]),
     "evaluateCNNModel": (f32, [pmodel, pdata, pscratch, vp, vp, vp, i32, i32]),
     "computeCNNGradient": (f32, [pmodel, pdata, pscratch, vp, vp, vp, vp, vp, i32, i32, f32]),
     "computeAccuracy": (f32, [vp, vp, i32, i32, vp, pf32]),

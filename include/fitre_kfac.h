@@ -91,9 +91,12 @@ long kfacInverseMemRequired(CNN_MODEL *model, int samples);
 /* The three trailing arguments are the reference's vendor handles (cublasHandle_t, cudaStream_t,
  * cusolverDnHandle_t, solvers/kfac_inverses.h:28-34), kept so that its solver source compiles against this
  * header unchanged; they are opaque pointers and are ignored (the device layer owns its streams). */
+#ifndef FITRE_VENDOR_HANDLES_DEFINED /* define it before this header where another header already declares the three names */
+#define FITRE_VENDOR_HANDLES_DEFINED
 typedef void *cublasHandle_t;
 typedef void *cudaStream_t;
 typedef void *cusolverDnHandle_t;
+#endif
 void computeOmegaZ(KFAC_CURVATURE_INFO *kfac_info, CNN_MODEL *model, DEVICE_DATASET *data, int samples,
                    real *dampedInput, real *dampedZ, real *omegaZInv, int *zOffsets, int *zztOffsets, real *devPtr,
                    real *pageLckPtr, cublasHandle_t blasHandle, cudaStream_t curStream, cusolverDnHandle_t curHandle);

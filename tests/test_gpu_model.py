@@ -244,6 +244,40 @@ def test_vgg11_full_size_one_lane_gives_the_same_bits(vgg_full, dev):
         L.check(L.hip.fitre_hip_lanes_enable(1))
 
 
+@pytest.mark.parametrize("name", ["lenet_bn_b1024", "alexnet_b64", "vgg11_no_bn_b32"])
+def test_forced_lanes_give_the_same_bits(dev, name):
+    """Networks on the other side of cnnBackward's two lane limits (LeNet + batch norm: too little work; AlexNet: too much
+    arithmetic per elementwise byte; a VGG-11 without batch norm at a small batch in between) and the override
+    fitreSetBackwardLanes: one lane and the lanes give the same gradient and dx, bit for bit."""
+    from helpers import GpuModel, batch_inputs, build_alexnet, build_lenet, build_vgg11, he_weights
+    if name == "lenet_bn_b1024":
+        batch, model = 1024, build_lenet(1024, bn=True)
+    elif name == "alexnet_b64":
+        batch, model = 64, build_alexnet(64)
+    else:
+        batch, model = 32, build_vgg11(32, bn=False)
+    rng = np.random.default_rng(len(name))
+    w = he_weights(model, rng).astype(np.float32)
+    x, y = batch_inputs(model, batch, rng)
+    gm = GpuModel(dev, model, w, x.astype(np.float32), y, batch)
+    gm.forward()
+    results = []
+    try:
+        for mode in (0, 1):
+            L.cnn.fitreSetBackwardLanes(mode)
+            assert L.cnn.fitreBackwardUsesLanes(C.byref(model), batch) == mode
+            L.check(L.hip.fitre_hip_memset(gm.grad, 0xFF, 4 * model.pSize))
+            gm.forward()
+            gm.backward()
+            results.append((gm.get("grad").view(np.uint32), gm.get("dx").view(np.uint32)))
+    finally:
+        L.cnn.fitreSetBackwardLanes(-1)
+    gm.release()
+    assert np.isfinite(results[0][0].view(np.float32)).all()
+    np.testing.assert_array_equal(results[0][0], results[1][0])
+    np.testing.assert_array_equal(results[0][1], results[1][1])
+
+
 def test_vgg11_full_size_directional_derivative(vgg_full, dev):
     """g'd against a central difference of the loss along a random direction d (fp32 forward)."""
     gm, w = vgg_full

@@ -44,6 +44,31 @@ def test_static_scratch_entry_point_matches_the_workspace_one(dev):
     both(dev, 3, 5, seed=4)
 
 
+def _free_bytes():
+    free = C.c_size_t(0)
+    L.check(hip.fitre_hip_device_info(None, None, None, None, C.byref(free), None, 0))
+    return free.value
+
+
+def test_static_scratch_entry_point_allocates_nothing(dev):
+    """The device's free memory is the same before and after calls of the entry point (segmented and single-workgroup
+    shapes), with every buffer of the test allocated beforehand; the workspace entry point's partial sums stay out of it."""
+    channels, per = 64, 65536
+    n = channels * per
+    rng = np.random.default_rng(9)
+    delta, zhat = dev.upload(rng.standard_normal(n).astype(np.float32)), dev.upload(rng.standard_normal(n).astype(np.float32))
+    var, out, bias = dev.upload(rng.uniform(0.5, 2.0, channels).astype(np.float32)), dev.zeros(n), dev.zeros(channels)
+    L.check(hip.fitre_hip_batch_norm_backward_static(delta, zhat, var, channels, per, 1e-5, out, bias))   # first call on the device
+    dev.sync()
+    before = _free_bytes()
+    for c, p in ((channels, per), (16, 4133), (channels, 1024)):
+        L.check(hip.fitre_hip_batch_norm_backward_static(delta, zhat, var, c, p, 1e-5, out, bias))
+    dev.sync()
+    assert _free_bytes() == before
+    for q in (delta, zhat, var, out, bias):
+        dev.free(q)
+
+
 def test_static_scratch_entry_point_rejects_what_does_not_fit(dev):
     channels, per = 20000, 8                           # 20000 slots of 64 bytes > 1 MiB
     assert hip.fitre_hip_batch_norm_workspace(channels, per) > STATIC_BYTES
