@@ -81,34 +81,99 @@ def tree_commit():
         return None
 
 
-def kernel_table(rows, steps, launches=None):
+def live_fraction(layer):
+    """Share of the (output cell, window tap) pairs of a convolution layer whose tap lies inside the image: what is left of
+    the window-count work 2*M*K*Cout when the products with the zero padding are not counted."""
+    def live(size, out, k, stride, pad):
+        return sum(1 for o in range(out) for t in range(k) if 0 <= o * stride - pad + t < size)
+    k = layer.kSize
+    return (live(layer.height, layer.outHeight, k, layer.stride, layer.padding) *
+            live(layer.width, layer.outWidth, k, layer.stride, layer.padding)) / float(k * k * layer.outHeight * layer.outWidth)
+
+
+def conv_live_fractions(model, batch):
+    """Algorithmic work 2*M*K*Cout of every convolution layer's gradient launches -> the live_fraction of the layers with
+    that work (two layers can share it: VGG-11's 256 -> 256 on 8x8 maps and 512 -> 512 on 4x4 maps)."""
+    table = {}
+    for c in range(model.cLayers):
+        l = model.convLayer[c]
+        work = 2.0 * batch * l.outHeight * l.outWidth * l.inChannels * l.kSize ** 2 * l.outChannels
+        table.setdefault(round(work), []).append(live_fraction(l))
+    return table
+
+
+# kernel variants that leave out the products with the padding, and the live fraction of the maps they run on
+SKIPS_PADDING = {"/dense2x2": 16 / 36.0, "/cell4x4": 100 / 144.0, "/cell8x8": 484 / 576.0}
+
+
+def launch_live_fraction(kernel, work, conv_live):
+    """(live fraction of the layer a launch belongs to, whether its kernel leaves the padding's products out).  Layers
+    of equal work: a variant kernel names its map size; the other kernels run the layers the variants do not take, the
+    larger maps."""
+    for suffix, frac in SKIPS_PADDING.items():
+        if kernel.endswith(suffix):
+            return frac, True
+    return max(conv_live.get(round(work), [1.0])), False
+
+
+def kernel_table(rows, steps, launches=None, conv_live=None, fc_batch=None):
     """Per kernel class (and tile variant): launches per step, average launch duration, achieved rate against the
     bound of its class (fp32 MFMA for the contraction kernels, HBM for the others); with `launches`, also the
-    four largest shapes of each kernel on their own (`largest`: work in FLOP resp. bytes)."""
+    four largest shapes of each kernel on their own (`largest`: work in FLOP resp. bytes).
+    Convolution gradients (conv_live given): the library counts the window-count work 2*M*K*Cout per launch; `frac` is
+    by the multiply-adds the kernel EXECUTES (the cell and dense variants leave out the products with the padding, the
+    nine-tap kernels do not), `frac_ninetap` by the window count (can exceed 1 for those variants), `frac_useful` by the
+    work without any product with the padding.  Fully connected products at a batch of at most 128 (fc_batch) move
+    more bytes of weights than they can multiply: they are scored against HBM, bytes = the weight matrix once."""
     kernels = {}
     big = largest_launches(launches) if launches else {}
+    executed, useful = {}, {}
+    if launches and conv_live:
+        for kernel, cls, work, ms in launches:
+            if cls not in ("conv_dw", "conv_dx"):
+                continue
+            live, skips = launch_live_fraction(kernel, work, conv_live)
+            executed[kernel] = executed.get(kernel, 0.0) + work * (live if skips else 1.0)
+            useful[kernel] = useful.get(kernel, 0.0) + work * live
     for r in rows:
         avg_us = 1e3 * r["ms"] / r["launches"]
         mfma = r["cls"] in MFMA_CLASSES
+        if r["cls"] == "fc_gemm" and fc_batch is not None and fc_batch <= 128:
+            nbytes = 2.0 * r["work"] / fc_batch              # work = 2 * batch * in * out FLOP -> 4 * in * out bytes
+            rate = nbytes / (r["ms"] * 1e-3) / 1e9 if r["ms"] > 0 else 0.0
+            kernels[r["kernel"]] = dict(bound="hbm", launches_per_step=r["launches"] / steps, avg_us=round(avg_us, 2),
+                                        ms_per_step=round(r["ms"] / steps, 4), achieved=round(rate, 1), unit="GB/s",
+                                        frac=round(rate / PEAK_HBM_GBS, 4),
+                                        frac_mfma=round(r["work"] / (r["ms"] * 1e-3) / 1e12 / PEAK_MFMA_F32_TFLOPS, 4) if r["ms"] > 0 else 0.0,
+                                        note="batch %d: bytes = the layer's weight matrix once (read for the input gradient, "
+                                             "written for the weight gradient)" % fc_batch)
+            continue
         rate = r["work"] / (r["ms"] * 1e-3) / (1e12 if mfma else 1e9) if r["ms"] > 0 else 0.0
         peak = PEAK_MFMA_F32_TFLOPS if mfma else PEAK_HBM_GBS
         kernels[r["kernel"]] = dict(bound="mfma" if mfma else "hbm", launches_per_step=r["launches"] / steps,
                                     avg_us=round(avg_us, 2), ms_per_step=round(r["ms"] / steps, 4),
                                     achieved=round(rate, 2 if mfma else 1), unit="TFLOP/s" if mfma else "GB/s",
                                     frac=round(rate / peak, 4))
+        if r["kernel"] in executed and r["work"] > 0:
+            k = kernels[r["kernel"]]
+            k["frac_ninetap"] = k["frac"]
+            k["work_ninetap_gflop_per_step"] = round(r["work"] / steps / 1e9, 3)
+            k["work_executed_gflop_per_step"] = round(executed[r["kernel"]] / steps / 1e9, 3)
+            k["achieved"] = round(rate * executed[r["kernel"]] / r["work"], 2)
+            k["frac"] = round(k["achieved"] / peak, 4)
+            k["frac_useful"] = round(rate * useful[r["kernel"]] / r["work"] / peak, 4)
         if r["kernel"] in big:
             kernels[r["kernel"]]["largest"] = big[r["kernel"]]
         if r["kernel"].endswith("/dense2x2"):
-            kernels[r["kernel"]]["note"] = ("3x3 windows on 2x2 maps as dense products: the work counted is the nine-tap "
-                                            "2*M*K*Cout, of which the kernel executes 16/36 (the rest multiplies padding)")
+            kernels[r["kernel"]]["note"] = ("3x3 windows on 2x2 maps as dense products: of the nine-tap 2*M*K*Cout the kernel "
+                                            "executes 16/36 (the rest multiplies padding)")
         if r["kernel"].endswith("/cell8x8"):
             kernels[r["kernel"]]["note"] = ("weight gradient of 3x3 windows on 8x8 maps, a reduction pair being one cell of two "
-                                            "images: the work counted is the nine-tap 2*M*K*Cout, of which the kernel executes "
-                                            "484/576 (the rest multiplies padding)")
+                                            "images: of the nine-tap 2*M*K*Cout the kernel executes 484/576 (the rest "
+                                            "multiplies padding)")
         if r["kernel"].endswith("/cell4x4"):
-            kernels[r["kernel"]]["note"] = ("3x3 windows on 4x4 maps, an MFMA block being one cell of 32 images: the work "
-                                            "counted is the nine-tap 2*M*K*Cout, of which the kernel executes 100/144 (the "
-                                            "rest multiplies padding)")
+            kernels[r["kernel"]]["note"] = ("3x3 windows on 4x4 maps, an MFMA block being one cell of 32 images: of the "
+                                            "nine-tap 2*M*K*Cout the kernel executes 100/144 (the rest multiplies padding)")
     return kernels
 
 
@@ -173,6 +238,7 @@ def gpu_leg(args):
     w = he_weights(model, rng).astype(np.float32)
     x, y = batch_inputs(model, batch, rng)
     gm = GpuModel(dev, model, w, x.astype(np.float32), y, batch)
+    conv_live = conv_live_fractions(model, batch)
     loss = gm.forward()  # untimed: produces z, probs and the loss errors
     # one plain copy of known size (64 Mi floats: 256 MiB read, 256 MiB written), outside the timed
     # region: the kernel that hardware traffic counters of the same run are scaled by
@@ -232,23 +298,32 @@ def gpu_leg(args):
         others = other_configs_leg(L, dev)
     dev.close()
 
-    kernels = kernel_table(rows, args.steps, launches)
+    kernels = kernel_table(rows, args.steps, launches, conv_live, batch)
     dom = max(rows, key=lambda r: r["ms"])
     dk = kernels[dom["kernel"]]
     roofline = dict(kernel=dom["kernel"], bound=dk["bound"], achieved=dk["achieved"],
                     peak=PEAK_MFMA_F32_TFLOPS if dk["bound"] == "mfma" else PEAK_HBM_GBS, unit=dk["unit"],
                     frac=dk["frac"], traffic=None, avg_launch_us=dk["avg_us"],
                     launches_per_step=dk["launches_per_step"])
+    for key in ("frac_ninetap", "frac_useful", "work_executed_gflop_per_step", "work_ninetap_gflop_per_step"):
+        if key in dk:
+            roofline[key] = dk[key]
     traffic, source, taken_at = measured_traffic(dom["kernel"])
     roofline["traffic"] = traffic
-    roofline["traffic_source"] = dict(file=source, counters_taken_at_commit=taken_at, this_tree=tree_commit(),
-                                      note="FETCH_SIZE / WRITE_SIZE of separate rocprofv3 --pmc runs of this program, "
-                                           "scaled by the calibration copy; not re-measured in this run")
+    # (a plain string: nested objects inside `roofline` do not survive every reader of this line)
+    roofline["traffic_source"] = ("%s: FETCH_SIZE / WRITE_SIZE of separate rocprofv3 --pmc runs of this program, scaled by the "
+                                  "calibration copy; counters taken at commit %s, this tree is %s; not re-measured in this run"
+                                  % (source, taken_at, tree_commit()))
     conv_rows = [r for r in rows if r["cls"] in ("conv_dw", "conv_dx")]
     conv_ms, conv_work = sum(r["ms"] for r in conv_rows), sum(r["work"] for r in conv_rows)
-    conv = dict(ms_per_step=round(conv_ms / args.steps, 4), gflop_per_step=round(conv_work / args.steps / 1e9, 2),
-                achieved=round(conv_work / (conv_ms * 1e-3) / 1e12, 2) if conv_ms else 0.0, unit="TFLOP/s")
+    conv_executed = sum(kernels[r["kernel"]].get("work_executed_gflop_per_step", r["work"] / args.steps / 1e9) for r in conv_rows)
+    conv = dict(ms_per_step=round(conv_ms / args.steps, 4), gflop_per_step_ninetap=round(conv_work / args.steps / 1e9, 2),
+                gflop_per_step_executed=round(conv_executed, 2), unit="TFLOP/s")
+    conv["achieved"] = round(conv_executed * 1e9 / (conv_ms / args.steps * 1e-3) / 1e12, 2) if conv_ms else 0.0
     conv["frac"] = round(conv["achieved"] / PEAK_MFMA_F32_TFLOPS, 4)
+    conv["frac_ninetap"] = round(conv_work / (conv_ms * 1e-3) / 1e12 / PEAK_MFMA_F32_TFLOPS, 4) if conv_ms else 0.0
+    conv["note"] = ("frac: multiply-adds the kernels execute; frac_ninetap: the window count 2*M*K*Cout of every layer, which "
+                    "includes products with the zero padding that the cell and dense kernels leave out")
     return dict(wall=wall, ms_events=ms_events.value, batch=batch, loss=loss, finite=finite,
                 device=name.value.decode(), compute_units=cus.value, roofline=roofline, kernels=kernels,
                 conv_backward_gemms=conv, kfac_factors=kfac, bandwidth_kernels=bandwidth, forward_ms=round(forward_ms, 4),
@@ -290,7 +365,7 @@ def other_configs_leg(L, dev, steps=10, only=None):
         dev.sync()
         L.check(L.hip.fitre_hip_profile_enable(0))
         rows = read_profile(L)
-        kernels = kernel_table(rows, steps, read_launches(L))
+        kernels = kernel_table(rows, steps, read_launches(L), conv_live_fractions(model, batch), batch)
         dom = max(rows, key=lambda r: r["ms"])
         dk = kernels[dom["kernel"]]
         out[name] = dict(images_per_s=round(batch * steps / dt, 1), ms_per_step=round(1e3 * dt / steps, 4),
