@@ -429,6 +429,24 @@ def bandwidth_leg(L, dev, batch, reps=20):
         out[name] = entry
         for p in (zhat, var, dpool, dact, dbn, bias, delta, ws):
             dev.free(p)
+    # What a plain copy reaches when nothing it touches is in a cache: 1 GiB read and 1 GiB written per pass, four
+    # times the memory-side cache.  The tensors of a backward pass are in that state (z comes from the forward pass,
+    # several hundred megabytes earlier); the layer-sized repeats above run partly out of the cache.
+    big = 1 << 28
+    src, dst = dev.zeros(big), dev.zeros(big)
+    L.check(hip.fitre_hip_copy(big, src, dst))
+    dev.sync()
+    L.check(hip.fitre_hip_profile_enable(1))
+    for _ in range(5):
+        L.check(hip.fitre_hip_copy(big, src, dst))
+    dev.sync()
+    L.check(hip.fitre_hip_profile_enable(0))
+    r = {r["cls"]: r for r in read_profile(L)}["blas1"]
+    t = r["ms"] * 1e-3 / r["launches"]
+    out["copy_1GiB_uncached"] = dict(us=round(t * 1e6, 2), achieved=round(8.0 * big / t / 1e9, 1), unit="GB/s",
+                                     frac=round(8.0 * big / t / 1e9 / PEAK_HBM_GBS, 4))
+    dev.free(src)
+    dev.free(dst)
     return out
 
 

@@ -7,6 +7,7 @@
 #include "conv_quad.h"
 #include "conv_thin.h"
 #include "linear_small.h"
+#include "linear_tail.h"
 
 namespace fitre {
 
@@ -917,6 +918,126 @@ int fitre_hip_linear_weight_grad(int in, int out, int n, const float *delta, con
 	int rc = gemm_ex(0, 1, out, in, n, 1.f, delta, out, zin, in, 0.f, dW, out, nullptr, 0, FITRE_KC_FC_GEMM, ws, wsBytes);
 	if (rc || !db) return rc;
 	return fitre_hip_row_sum(delta, out, n, db);
+}
+
+static int tail_samples(int n) { return n >= 512 ? kTailMaxSamples : 4; }
+static bool tail_in_ranges(int n) { return n > kSmallGemmMaxK; }
+
+int fitre_hip_fc_tail_fits(int layers, const fitre_fc_tail_layer *l, int n)
+{
+	if (!l || layers < 1 || layers > kTailMaxLayers || n < 1 || n > 65536) return 0;
+	long upper = 0;
+	for (int f = 0; f < layers; f++) {
+		if (l[f].in < 1 || l[f].out < 1 || l[f].in > kTailMaxDim || l[f].out > kTailMaxDim) return 0;
+		if (f > 0 && l[f].in != l[f - 1].out) return 0;
+		if (!(tail_in_ranges(n) ? small_gemm_ranges_fit(l[f].out, l[f].in, n) : small_gemm_fits(l[f].out, l[f].in, n))) return 0;
+		if (f > 0) upper += (long)l[f].in * l[f].out;
+	}
+	return upper <= kTailUpperFloats;
+}
+
+size_t fitre_hip_fc_tail_workspace(int layers, const fitre_fc_tail_layer *l, int n)
+{
+	if (!fitre_hip_fc_tail_fits(layers, l, n)) return 0;
+	size_t total = 256;
+	if (tail_in_ranges(n))
+		for (int f = 0; f < layers; f++) total += small_gemm_ranges_workspace(l[f].out, l[f].in, n);
+	return total;
+}
+
+int fitre_hip_fc_tail_backward(int layers, const fitre_fc_tail_layer *l, int n, const float *delta, int extA, int extB, float *features,
+                               void *ws, size_t wsBytes)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(fitre_hip_fc_tail_fits(layers, l, n), "fitre_hip_fc_tail_backward: the layers do not fit (at most %d layers of at most %d units)",
+	              kTailMaxLayers, kTailMaxDim);
+	FITRE_REQUIRE(delta && features, "fitre_hip_fc_tail_backward: null pointer");
+	const bool permute = extA > 0 || extB > 0;
+	FITRE_REQUIRE(!permute || (extA > 0 && extB > 0 && l[0].in % (extA * extB) == 0),
+	              "fitre_hip_fc_tail_backward: %d inputs are not whole %d x %d maps", l[0].in, extA, extB);
+	const bool ranges = tail_in_ranges(n);
+	const size_t need = fitre_hip_fc_tail_workspace(layers, l, n);
+	if (ranges && (!ws || wsBytes < need || (((uintptr_t)ws) & 3) != 0))
+		return fail(FITRE_E_WORKSPACE, "fitre_hip_fc_tail_backward: workspace of %zu bytes is smaller than the %zu required", wsBytes, need);
+	FcTailParams p{};
+	p.layers = layers, p.n = n, p.ns = tail_samples(n);
+	p.extA = permute ? extA : 0, p.extB = permute ? extB : 0;
+	p.delta = delta, p.features = features;
+	int maxDim = 1, upperLds = 0;
+	double chainFlops = 0.0;
+	for (int f = 0; f < layers; f++) {
+		FITRE_REQUIRE(l[f].W && l[f].zin && l[f].slot && l[f].dW && l[f].slot != delta, "fitre_hip_fc_tail_backward: null or aliased pointer in layer %d", f);
+		const bool derivative = l[f].act != CNN_ACT_NONE && l[f].act != ACT_LINEAR && l[f].act >= 0;
+		FITRE_REQUIRE(!derivative || (l[f].zPost && l[f].zPre), "fitre_hip_fc_tail_backward: layer %d has an activation but no z", f);
+		FcTailLayer &d = p.l[f];
+		d.in = l[f].in, d.out = l[f].out, d.act = l[f].act;
+		d.W = l[f].W, d.zPre = l[f].zPre, d.zPost = l[f].zPost, d.slot = l[f].slot;
+		d.outMagic = (unsigned)((1ull << 32) / (unsigned)d.out) + 1u;
+		if (f > 0) {
+			d.firstWeight = p.upperWeights, d.ldsBase = upperLds;
+			p.upperWeights += d.in * d.out, upperLds += d.in * (d.out + 1);
+		}
+		maxDim = d.in > maxDim ? d.in : maxDim;
+		maxDim = d.out > maxDim ? d.out : maxDim;
+		chainFlops += 2.0 * (double)d.in * d.out * n;
+	}
+	p.maxDim = maxDim;
+	const int groups = (n + p.ns - 1) / p.ns;
+	// parts of the lowest layer: each fits a workgroup's registers, and together with the groups they fill the chip
+	const long lowest = (long)l[0].in * l[0].out;
+	int parts = (int)((lowest + kTailPartFloats - 1) / kTailPartFloats);
+	const int cus = device_compute_units() > 0 ? device_compute_units() : 256;
+	const int fill = (cus + groups - 1) / groups;
+	parts = parts < fill ? fill : parts;
+	parts = parts > l[0].in ? l[0].in : parts;
+	p.partInputs = (l[0].in + parts - 1) / parts;
+	while ((long)p.partInputs * l[0].out > kTailPartFloats) p.partInputs--; // rounding up must not pass the registers
+	parts = (l[0].in + p.partInputs - 1) / p.partInputs;
+	const int lowLds = p.partInputs * (l[0].out + 1);
+	const size_t ldsBytes = sizeof(float) * ((size_t)2 * kTailMaxSamples * (maxDim + 1) + (upperLds > lowLds ? upperLds : lowLds) + 64);
+	static bool attributeSet = false;
+	if (!attributeSet) {
+		FITRE_HIP_TRY(hipFuncSetAttribute((const void *)fc_tail_chain_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+		attributeSet = true;
+	}
+	{
+		LaunchScope scope(FITRE_KC_FC_GEMM, chainFlops, 0);
+		fc_tail_chain_kernel<<<dim3((unsigned)groups, (unsigned)parts), 256, ldsBytes, stream()>>>(p);
+	}
+	// every layer's delta * zin' and delta * 1
+	SmallGemmBatch b{};
+	SmallReduceBatch r{};
+	b.count = r.count = layers;
+	const int nRanges = ranges ? (n + kSmallRange - 1) / kSmallRange : 1;
+	r.ranges = nRanges;
+	float *part = (float *)ws;
+	for (int f = 0; f < layers; f++) {
+		SmallGemmParams &q = b.p[f];
+		q.M = l[f].out, q.N = l[f].in, q.K = n;
+		q.A = l[f].slot, q.sAm = 1, q.sAk = l[f].out;
+		q.B = l[f].zin, q.sBk = l[f].in, q.sBn = 1;
+		q.C = l[f].dW, q.ldc = l[f].out, q.alpha = 1.f, q.beta = 0.f;
+		q.act = -1;
+		q.rowSums = l[f].db;
+		b.gridX[f] = (q.M + kSmallTile - 1) / kSmallTile, b.gridY[f] = (q.N + kSmallTile - 1) / kSmallTile;
+		b.first[f + 1] = b.first[f] + b.gridX[f] * b.gridY[f] * nRanges;
+		if (ranges) {
+			q.kChunk = kSmallRange, q.partial = part;
+			q.rowSums = l[f].db ? part : nullptr; // only its being non-null matters to the kernel in this mode
+			r.M[f] = q.M, r.N[f] = q.N, r.partial[f] = part, r.C[f] = l[f].dW, r.rowSums[f] = l[f].db, r.alpha[f] = 1.f;
+			r.first[f + 1] = r.first[f] + (long)q.M * q.N + q.M;
+			part += (size_t)nRanges * ((size_t)q.M * q.N + q.M);
+		}
+	}
+	{
+		LaunchScope scope(FITRE_KC_FC_GEMM, chainFlops, 0);
+		small_gemm_batch_kernel<<<(unsigned)b.first[layers], 256, 0, stream()>>>(b);
+	}
+	if (ranges) {
+		LaunchScope scope(FITRE_KC_SPLITK_REDUCE, 4.0 * (double)r.first[layers] * (nRanges + 1));
+		small_gemm_batch_reduce_kernel<<<(unsigned)((r.first[layers] + 255) / 256), 256, 0, stream()>>>(r);
+	}
+	return check_launch("fc_tail_chain_kernel");
 }
 
 } // extern "C"

@@ -53,19 +53,20 @@ __device__ __forceinline__ float act_backward_value(int actFun, float d, float z
 	}
 }
 
-__global__ void __launch_bounds__(256) small_gemm_kernel(const SmallGemmParams p)
+// one workgroup's block (bx, by) of the result over reduction range bz
+__device__ __forceinline__ void small_gemm_block(const SmallGemmParams &p, const int bx, const int by, const int bz)
 {
 	__shared__ float As[kSmallDepth][kSmallTile + 1]; // [k][m]
 	__shared__ float Bs[kSmallDepth][kSmallTile + 1]; // [k][n]
 	const int tid = threadIdx.x;
-	const int m0 = blockIdx.x * kSmallTile, n0 = blockIdx.y * kSmallTile;
+	const int m0 = bx * kSmallTile, n0 = by * kSmallTile;
 	const int tm = tid & 15, tn = tid >> 4;
 	// loads run along whichever index is contiguous in memory; all of a block's loads are in flight together
 	const bool aAlongM = p.sAm == 1, bAlongN = p.sBn == 1;
 	constexpr int kPer = kSmallDepth * kSmallTile / 256; // elements of each operand a thread loads per block
 	float acc00 = 0.f, acc01 = 0.f, acc10 = 0.f, acc11 = 0.f, rs0 = 0.f, rs1 = 0.f;
-	const bool sums = p.rowSums != nullptr && blockIdx.y == 0 && tn == 0;
-	const int kBeg = p.kChunk > 0 ? (int)blockIdx.z * p.kChunk : 0;
+	const bool sums = p.rowSums != nullptr && by == 0 && tn == 0;
+	const int kBeg = p.kChunk > 0 ? bz * p.kChunk : 0;
 	const int kEnd = (p.kChunk > 0 && kBeg + p.kChunk < p.K) ? kBeg + p.kChunk : p.K;
 	for (int k0 = kBeg; k0 < kEnd; k0 += kSmallDepth) {
 		float av[kPer], bv[kPer];
@@ -77,7 +78,7 @@ __global__ void __launch_bounds__(256) small_gemm_kernel(const SmallGemmParams p
 			const bool aok = (m0 + am < p.M) & (k0 + ak < kEnd), bok = (n0 + bn < p.N) & (k0 + bk < kEnd);
 			av[i] = aok ? p.A[(long)(m0 + am) * p.sAm + (long)(k0 + ak) * p.sAk] : 0.f;
 			bv[i] = bok ? p.B[(long)(k0 + bk) * p.sBk + (long)(n0 + bn) * p.sBn] : 0.f;
-			if (p.copyB != nullptr && blockIdx.x == 0 && bok) p.copyB[(long)(k0 + bk) * p.sBk + (long)(n0 + bn) * p.sBn] = bv[i];
+			if (p.copyB != nullptr && bx == 0 && bok) p.copyB[(long)(k0 + bk) * p.sBk + (long)(n0 + bn) * p.sBn] = bv[i];
 		}
 		__syncthreads(); // the previous block's readers are done
 #pragma unroll
@@ -100,7 +101,7 @@ __global__ void __launch_bounds__(256) small_gemm_kernel(const SmallGemmParams p
 		}
 	}
 	if (p.kChunk > 0) { // raw sums of this reduction range
-		float *part = p.partial + (size_t)blockIdx.z * ((size_t)p.M * p.N + p.M);
+		float *part = p.partial + (size_t)bz * ((size_t)p.M * p.N + p.M);
 		if (sums) {
 			if (m0 + tm < p.M) part[(size_t)p.M * p.N + m0 + tm] = rs0;
 			if (m0 + tm + 16 < p.M) part[(size_t)p.M * p.N + m0 + tm + 16] = rs1;
@@ -140,6 +141,53 @@ __global__ void __launch_bounds__(256) small_gemm_kernel(const SmallGemmParams p
 	store(m0 + tm + 16, n0 + tn, acc10);
 	store(m0 + tm, n0 + tn + 16, acc01);
 	store(m0 + tm + 16, n0 + tn + 16, acc11);
+}
+
+__global__ void __launch_bounds__(256) small_gemm_kernel(const SmallGemmParams p)
+{
+	small_gemm_block(p, (int)blockIdx.x, (int)blockIdx.y, (int)blockIdx.z);
+}
+
+// several independent products as one launch: the blocks of product j are blockIdx.x in [first[j], first[j + 1])
+constexpr int kSmallBatch = 4;
+struct SmallGemmBatch {
+	int count;
+	int first[kSmallBatch + 1];
+	int gridX[kSmallBatch], gridY[kSmallBatch];
+	SmallGemmParams p[kSmallBatch];
+};
+__global__ void __launch_bounds__(256) small_gemm_batch_kernel(const SmallGemmBatch b)
+{
+	const int block = (int)blockIdx.x;
+	int j = 0;
+	while (j + 1 < b.count && block >= b.first[j + 1]) j++;
+	const int local = block - b.first[j];
+	const int bx = local % b.gridX[j], rest = local / b.gridX[j];
+	small_gemm_block(b.p[j], bx, rest % b.gridY[j], rest / b.gridY[j]);
+}
+
+// the second launch of a batch whose reductions were cut into ranges: every product's sums in range order, in double
+struct SmallReduceBatch {
+	int count, ranges;
+	long first[kSmallBatch + 1]; // results (M * N + M) of the products before j
+	int M[kSmallBatch], N[kSmallBatch];
+	const float *partial[kSmallBatch];
+	float *C[kSmallBatch], *rowSums[kSmallBatch];
+	float alpha[kSmallBatch];
+};
+__global__ void __launch_bounds__(256) small_gemm_batch_reduce_kernel(const SmallReduceBatch b)
+{
+	const long at = (long)blockIdx.x * blockDim.x + threadIdx.x;
+	if (at >= b.first[b.count]) return;
+	int j = 0;
+	while (j + 1 < b.count && at >= b.first[j + 1]) j++;
+	const long i = at - b.first[j];
+	const long mn = (long)b.M[j] * b.N[j], per = mn + b.M[j];
+	const float *part = b.partial[j];
+	double acc = 0.0;
+	for (int r = 0; r < b.ranges; r++) acc += (double)part[(size_t)r * per + i];
+	if (i < mn) b.C[j][i] = b.alpha[j] * (float)acc; // ldc == M
+	else if (b.rowSums[j]) b.rowSums[j][i - mn] = (float)acc;
 }
 
 // C = alpha * (sum of the ranges' partial results, in range order, in double) and the row sums likewise

@@ -1,0 +1,152 @@
+// The backward pass of a whole tail of small fully connected layers in two launches (three at a large batch) instead of
+// two per layer (LeNet's 400-120-84-10: six launches of 6-10 us each: functions/cnn_backward.cu:100-254 runs these steps
+// layer by layer).
+//
+//   1. the chain of deltas.  It does not couple samples, so a workgroup owns a few samples and walks the layers top down
+//      on its own: delta_f (after the activation derivative) into its dx slot and into LDS, delta_{f-1} = f'(.) .* (W_f'
+//      delta_f) from weights staged in LDS.  The lowest layer has the most weights and nothing below it waits for
+//      all of its outputs at once, so its inputs are cut into parts that different workgroups take (each repeats the
+//      few thousand multiply-adds of the layers above); a workgroup requests its part of those weights first and uses
+//      them last, so their latency passes behind the upper layers.  The result goes to the convolution layout.
+//   2. every layer's weight and bias gradient, delta_f * zin_f' and delta_f * 1, as ONE launch of the small product
+//      kernel over the blocks of all layers (a long batch is cut into ranges, added by a third launch in range order).
+// The order of every sum is fixed by the shapes alone.
+#pragma once
+#include "linear_small.h"
+
+namespace fitre {
+
+constexpr int kTailMaxLayers = 4;
+constexpr int kTailMaxDim = 1024;         // inputs / outputs of a layer
+constexpr int kTailMaxSamples = 8;        // samples of a group
+constexpr int kTailPartFloats = 48 * 256; // weights of the lowest layer a workgroup takes, held in registers until used
+constexpr int kTailUpperFloats = 48 * 256; // weights of all layers above the lowest together, likewise
+
+struct FcTailLayer {
+	int in, out;
+	int act;                   // this layer's activation
+	unsigned outMagic;         // e / out == __umulhi(e, outMagic) for e < 2^20
+	int ldsBase;               // where its weights sit in LDS as [input][out + 1] (layers above the lowest)
+	int firstWeight;           // weights of the layers 1 .. f - 1 (its place in the registers that prefetch them)
+	const float *W;            // out x in, column-major
+	const float *zPre, *zPost; // its output before / after the activation, out x n
+	float *slot;               // receives delta (after the activation derivative), out x n
+};
+
+struct FcTailParams {
+	int layers, n, ns;
+	int extA, extB; // the lowest layer's inputs are whole extA x extB maps: its input gradient goes to [c][n][a][b]
+	FcTailLayer l[kTailMaxLayers];
+	const float *delta; // at the top layer's output, before its activation derivative
+	float *features;
+	int maxDim;
+	int partInputs;   // inputs of the lowest layer per blockIdx.y
+	int upperWeights; // weights of the layers above the lowest
+};
+
+__device__ __forceinline__ int tail_div(int e, int out, unsigned magic) { return out == 1 ? e : (int)__umulhi((unsigned)e, magic); }
+
+__global__ void __launch_bounds__(256) fc_tail_chain_kernel(const FcTailParams p)
+{
+	extern __shared__ float lds[];
+	const int ldd = p.maxDim + 1;
+	float *dcur = lds, *dnext = lds + kTailMaxSamples * ldd, *wbuf = dnext + kTailMaxSamples * ldd;
+	const int tid = threadIdx.x;
+	const int s0 = blockIdx.x * p.ns;
+	const int cnt = (p.n - s0 < p.ns) ? p.n - s0 : p.ns;
+	const bool first = blockIdx.y == 0; // the workgroup that writes the slots of the layers above the lowest
+	// every weight this workgroup multiplies by is requested before anything waits: its part of the lowest layer ...
+	const FcTailLayer &low = p.l[0];
+	const int pi0 = blockIdx.y * p.partInputs;
+	const int pni = (low.in - pi0 < p.partInputs) ? low.in - pi0 : p.partInputs;
+	float wlow[kTailPartFloats / 256], wup[kTailUpperFloats / 256];
+	{
+		const float *src = low.W + (long)pi0 * low.out;
+		const int count = pni * low.out;
+#pragma unroll
+		for (int t = 0; t < kTailPartFloats / 256; t++) wlow[t] = (tid + 256 * t < count) ? src[tid + 256 * t] : 0.f;
+	}
+	// ... and the layers above it, whole
+#pragma unroll
+	for (int t = 0; t < kTailUpperFloats / 256; t++) {
+		const int e = tid + 256 * t;
+		// which layer: static indices, so that the argument block stays in scalar registers
+		const float *src = p.l[1].W;
+		int base = 0;
+		if (p.layers > 2 && e >= p.l[2].firstWeight) src = p.l[2].W, base = p.l[2].firstWeight;
+		if (p.layers > 3 && e >= p.l[3].firstWeight) src = p.l[3].W, base = p.l[3].firstWeight;
+		wup[t] = e < p.upperWeights ? src[e - base] : 0.f;
+	}
+#pragma unroll
+	for (int t = 0; t < kTailUpperFloats / 256; t++) {
+		const int e = tid + 256 * t;
+		int base = 0, out = p.l[1].out, to = p.l[1].ldsBase;
+		unsigned magic = p.l[1].outMagic;
+		if (p.layers > 2 && e >= p.l[2].firstWeight) base = p.l[2].firstWeight, out = p.l[2].out, to = p.l[2].ldsBase, magic = p.l[2].outMagic;
+		if (p.layers > 3 && e >= p.l[3].firstWeight) base = p.l[3].firstWeight, out = p.l[3].out, to = p.l[3].ldsBase, magic = p.l[3].outMagic;
+		const int k = e - base;
+		if (e < p.upperWeights) wbuf[to + k + tail_div(k, out, magic)] = wup[t]; // [i][o] with rows out + 1 apart
+	}
+	const int planeAB = p.extA * p.extB;
+	// the layers top down; unrolled so that every index into the argument block is a constant
+#pragma unroll
+	for (int f = kTailMaxLayers - 1; f >= 0; f--) {
+		if (f >= p.layers) continue;
+		const FcTailLayer &lay = p.l[f];
+		const FcTailLayer &under = p.l[f > 0 ? f - 1 : 0];
+		const bool below = f > 0;
+		if (f == p.layers - 1) { // delta at the top, times its activation derivative
+			const bool derivative = lay.act != CNN_ACT_NONE && lay.act != ACT_LINEAR && lay.act >= 0;
+			for (int e = tid; e < lay.out * cnt; e += 256) {
+				const int s = tail_div(e, lay.out, lay.outMagic), o = e - s * lay.out;
+				const long at = (long)(s0 + s) * lay.out + o;
+				float v = p.delta[at];
+				if (derivative) v = act_backward_value(lay.act, v, lay.zPre[at], lay.zPost[at]);
+				dcur[s * ldd + o] = v;
+				if (first) lay.slot[at] = v;
+			}
+		}
+		const int in = lay.in, out = lay.out, ldw = out + 1;
+		const bool derivative = below && under.act != CNN_ACT_NONE && under.act != ACT_LINEAR && under.act >= 0;
+		const int i0 = below ? 0 : pi0, ni = below ? in : pni;
+		const float *wl = wbuf + (below ? lay.ldsBase : 0);
+		__syncthreads(); // dcur and the staged weights are complete; the layer above has been read
+		if (!below) {
+			// the lowest layer's part takes the place of the layers above it
+			const int count = pni * out;
+#pragma unroll
+			for (int t = 0; t < kTailPartFloats / 256; t++) {
+				const int e = tid + 256 * t;
+				if (e < count) wbuf[e + tail_div(e, out, lay.outMagic)] = wlow[t];
+			}
+			__syncthreads();
+		}
+		// (i, s) = f'(.) * sum over o of W(o, i) delta(o, s)
+		for (int e = tid; e < ni * cnt; e += 256) {
+			const int s = e / ni, ii = e - s * ni;
+			const int i = i0 + ii;
+			const long at = (long)(s0 + s) * in + i;
+			float zi = 0.f, zo = 0.f;
+			if (derivative) zi = under.zPre[at], zo = under.zPost[at]; // on their way while the sum runs
+			const float *w = wl + ii * ldw, *d = dcur + s * ldd;
+			float acc = 0.f;
+#pragma unroll 8
+			for (int o = 0; o < out; o++) acc = fmaf(w[o], d[o], acc);
+			if (below) {
+				if (derivative) acc = act_backward_value(under.act, acc, zi, zo);
+				dnext[s * ldd + i] = acc;
+				if (first) under.slot[at] = acc;
+			} else if (p.extA > 0) {
+				const int c = i / planeAB, r = i - c * planeAB;
+				const int b = r / p.extA, a = r - b * p.extA;
+				p.features[(((long)c * p.n + (s0 + s)) * p.extA + a) * p.extB + b] = acc;
+			} else {
+				p.features[at] = acc;
+			}
+		}
+		float *t = dcur;
+		dcur = dnext, dnext = t;
+	}
+}
+
+} // namespace fitre

@@ -117,9 +117,22 @@ static size_t backward_chain_ws_bytes(const CNN_MODEL *model, int batch)
 	return backward_dx_ws_bytes(model, batch) + backward_bn_ws_bytes(model, batch);
 }
 
+/* the linear layers as the fused tail sees them (shapes only; tail_layers fills in the pointers); 0 when they do not fit it */
+static int tail_shapes(const CNN_MODEL *model, int n, fitre_fc_tail_layer *tail)
+{
+	if (model->lLayers < 1 || model->lLayers > 4) return 0;
+	for (int f = 0; f < model->lLayers; f++) {
+		fitre_fc_tail_layer t = { model->fcLayer[f].in, model->fcLayer[f].out, model->fcLayer[f].actFun, NULL, NULL, NULL, NULL, NULL, NULL, NULL };
+		tail[f] = t;
+	}
+	return fitre_hip_fc_tail_fits(model->lLayers, tail, n);
+}
+
 static size_t backward_side_ws_bytes(const CNN_MODEL *model, int batch)
 {
 	size_t need = 256;
+	fitre_fc_tail_layer tail[4];
+	if (tail_shapes(model, batch, tail)) need = max_sz(need, fitre_hip_fc_tail_workspace(model->lLayers, tail, batch));
 	for (int i = 0; i < model->cLayers; i++) {
 		fitre_conv_shape s = conv_shape(&model->convLayer[i], batch);
 		need = max_sz(need, fitre_hip_conv_weight_grad_workspace(&s));
@@ -348,7 +361,24 @@ void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, 
 	real *features = (real *)ws;
 	int extA, extB;
 	feature_extent(model, &extA, &extB);
-	for (int f = model->lLayers - 1; f >= 0; f--) {
+	fitre_fc_tail_layer tail[4];
+	const int fusedTail = tail_shapes(model, n, tail);
+	if (fusedTail) {
+		/* small layers (LeNet's 400-120-84-10): the whole tail in two launches on the chain's lane -- every delta into its
+		 * slot, every weight and bias gradient, and the first convolution-side delta */
+		for (int f = 0; f < model->lLayers; f++) {
+			const FC_LAYER *l = &model->fcLayer[f];
+			real *zl = z + zOffsets[f + nc + 1];
+			tail[f].W = weights + wOffsets[f + nc];
+			tail[f].zPre = zl + l->offset, tail[f].zPost = zl;
+			tail[f].zin = z + zOffsets[f + nc] + ((f == 0) ? last->outputOffset : 0);
+			tail[f].slot = dx + zOffsets[f + nc + 1];
+			tail[f].dW = gradient + wOffsets[f + nc];
+			tail[f].db = (model->bias != 0) ? gradient + bOffsets[f + nc] : NULL;
+		}
+		HIP_CALL(fitre_hip_fc_tail_backward(model->lLayers, tail, n, delta, extA, extB, features, sideWs, sideBytes));
+	}
+	for (int f = fusedTail ? -1 : model->lLayers - 1; f >= 0; f--) {
 		const FC_LAYER *l = &model->fcLayer[f];
 		real *zl = z + zOffsets[f + nc + 1];
 		real *slot = dx + zOffsets[f + nc + 1];

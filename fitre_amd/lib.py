@@ -122,6 +122,9 @@ HIP_API = {
     "fitre_hip_linear_weight_grad_workspace": (sz, [i32, i32, i32]),
     "fitre_hip_linear_input_grad": (i32, [i32, i32, i32, vp, vp, i32, vp, vp, i32, i32, vp, vp, vp, sz, vp]),
     "fitre_hip_linear_weight_grad": (i32, [i32, i32, i32, vp, vp, vp, vp, vp, sz]),
+    "fitre_hip_fc_tail_fits": (i32, [i32, vp, i32]),
+    "fitre_hip_fc_tail_workspace": (sz, [i32, vp, i32]),
+    "fitre_hip_fc_tail_backward": (i32, [i32, vp, i32, vp, i32, i32, vp, vp, sz]),
     "fitre_hip_lane_select": (i32, [i32]),
     "fitre_hip_lane_wait": (i32, [i32, i32]),
     "fitre_hip_lanes_enable": (i32, [i32]),

@@ -146,3 +146,9 @@ class fitre_matrix(C.Structure):
     """Operand of the float64 products (include/fitre_hip.h)."""
     _fields_ = [("data", C.c_void_p), ("rowStride", C.c_long), ("colStride", C.c_long), ("kind", C.c_int),
                 ("onesRow", C.c_long), ("onesCol", C.c_long), ("onesValue", C.c_double)]
+
+
+class fitre_fc_tail_layer(C.Structure):
+    """One layer of fitre_hip_fc_tail_backward (include/fitre_hip.h)."""
+    _fields_ = [("in_", C.c_int), ("out", C.c_int), ("act", C.c_int), ("W", C.c_void_p), ("zPre", C.c_void_p),
+                ("zPost", C.c_void_p), ("zin", C.c_void_p), ("slot", C.c_void_p), ("dW", C.c_void_p), ("db", C.c_void_p)]

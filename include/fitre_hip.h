@@ -421,6 +421,30 @@ int fitre_hip_linear_input_grad(int in, int out, int n, const float *W, const fl
 int fitre_hip_linear_weight_grad(int in, int out, int n, const float *delta, const float *zin, float *dW, float *db,
                                  void *ws, size_t wsBytes);
 
+/* The backward products of a whole tail of small fully connected layers (layers[0] the lowest) in two launches (three
+ * when the batch is above 512): every layer's delta (after its activation derivative) into its slot, dW = delta * zin',
+ * db = delta * 1, and the lowest layer's input gradient W' * delta into `features` -- in a convolution layer's layout
+ * [channel][sample][a][b] when extA, extB > 0 (the permutation of fitre_hip_fc_to_conv), in x n otherwise.  The same
+ * bits as the per-layer entry points above give for layers this small (functions/cnn_backward.cu:100-254 for every
+ * layer of the tail): every sum runs in the same order.  delta: at the top layer's output (out x n), before that
+ * layer's activation derivative.  _fits: at most four layers of at most 1024 units, each of them small in the sense
+ * of fitre_hip_linear_is_small (or, above 512 samples, within the ranged weight gradient's limits), the layers above
+ * the lowest holding at most 12288 weights together.  Workspace:
+ * fitre_hip_fc_tail_workspace bytes (only read above 512 samples; ws may be NULL otherwise). */
+typedef struct fitre_fc_tail_layer {
+	int in, out;
+	int act;                   /* activation of this layer (CNN_ACT_NONE / ACT_LINEAR / negative: none) */
+	const float *W;            /* out x in, column-major */
+	const float *zPre, *zPost; /* its output before / after the activation, out x n (unused without an activation) */
+	const float *zin;          /* its input, in x n */
+	float *slot;               /* receives delta, out x n */
+	float *dW, *db;            /* out x in, out (db may be NULL) */
+} fitre_fc_tail_layer;
+int fitre_hip_fc_tail_fits(int layers, const fitre_fc_tail_layer *l, int n);
+size_t fitre_hip_fc_tail_workspace(int layers, const fitre_fc_tail_layer *l, int n);
+int fitre_hip_fc_tail_backward(int layers, const fitre_fc_tail_layer *l, int n, const float *delta, int extA, int extB,
+                               float *features, void *ws, size_t wsBytes);
+
 /* ---- Kronecker factors of the KFAC curvature approximation --------------------------------------
  * Each factor is a dense symmetric matrix, written in full (row-major == column-major).  The
  * products are symmetric, so only the tiles on and above the diagonal are computed.

@@ -145,3 +145,114 @@ def test_linear_arguments_are_checked(dev):
     assert hip.fitre_hip_linear_weight_grad(4, 4, 0, p, p, p, None, None, 0) == 2
     assert hip.fitre_hip_linear_weight_grad(4, 4, 4, p, None, p, None, None, 0) == 2
     dev.free(p)
+
+
+# layer widths bottom-up (the first is the tail's input), samples, activations per layer, (extA, extB) of the input maps
+TAILS = [
+    ((400, 120, 84, 10), 128, (CNN_ACT_RELU, CNN_ACT_RELU, CNN_ACT_NONE), (5, 5)),       # LeNet at batch 128
+    ((400, 120, 84, 10), 1024, (CNN_ACT_RELU, CNN_ACT_RELU, CNN_ACT_NONE), (5, 5)),      # groups of eight samples
+    ((36, 7), 5, (CNN_ACT_SWISH,), (3, 2)),                                                # one layer, an activation on top, ragged group
+    ((64, 33, 17, 9, 3), 67, (CNN_ACT_ELU, CNN_ACT_SOFTPLUS, CNN_ACT_SWISH, CNN_ACT_NONE), (0, 0)),   # four layers, no permutation
+    ((1024, 250), 9, (-1,), (4, 4)),                                                       # the widest input, weights staged in many chunks
+]
+
+
+@pytest.mark.parametrize("bias", [True, False])
+@pytest.mark.parametrize("dims,n,acts,ext", TAILS)
+def test_tail_of_small_layers_in_two_launches(dev, dims, n, acts, ext, bias):
+    """fitre_hip_fc_tail_backward against the chain of per-layer formulas in float64: every layer's delta, weight and bias
+    gradient and the lowest layer's input gradient (in the convolution layout when the inputs are maps)."""
+    from fitre_amd.structs import fitre_fc_tail_layer
+    layers = len(dims) - 1
+    rng = np.random.default_rng(sum(dims) + n)
+    Ws = [rng.standard_normal((dims[f + 1], dims[f])) / np.sqrt(dims[f]) for f in range(layers)]
+    zin0 = rng.standard_normal((dims[0], n)).astype(np.float32)
+    zpre, zpost, x = [], [], zin0.astype(np.float64)
+    for f in range(layers):                       # a forward pass in float64, stored as floats
+        pre = (Ws[f].astype(np.float32).astype(np.float64) @ x).astype(np.float32)
+        post = forward_act(acts[f], pre.astype(np.float64)).astype(np.float32)
+        zpre.append(pre), zpost.append(post)
+        x = post.astype(np.float64)
+    top = rng.standard_normal((dims[-1], n)).astype(np.float32)
+    # the reference chain
+    want_delta, want_dw, want_db = [None] * layers, [None] * layers, [None] * layers
+    d = top.astype(np.float64) * derivative(acts[-1], zpre[-1].astype(np.float64), zpost[-1].astype(np.float64))
+    for f in range(layers - 1, -1, -1):
+        want_delta[f] = d
+        inp = zin0 if f == 0 else zpost[f - 1]
+        want_dw[f] = d @ inp.astype(np.float64).T
+        want_db[f] = d.sum(axis=1)
+        below = Ws[f].astype(np.float32).astype(np.float64).T @ d
+        if f > 0:
+            below = below * derivative(acts[f - 1], zpre[f - 1].astype(np.float64), zpost[f - 1].astype(np.float64))
+        d = below
+    want_features = d                                              # dims[0] x n
+    col = lambda m: np.ascontiguousarray(m.T)                      # column-major upload of a (rows x cols) matrix
+    bufs = []
+    def up(a):
+        p = dev.upload(a)
+        bufs.append(p)
+        return p
+    arr = (fitre_fc_tail_layer * layers)()
+    slots, dws, dbs = [], [], []
+    pz0 = up(col(zin0))
+    pposts = [up(col(z)) for z in zpost]
+    for f in range(layers):
+        slots.append(up(np.full(dims[f + 1] * n, np.nan, np.float32)))
+        dws.append(up(np.full(dims[f + 1] * dims[f], np.nan, np.float32)))
+        dbs.append(up(np.full(dims[f + 1], np.nan, np.float32)))
+        arr[f] = fitre_fc_tail_layer(dims[f], dims[f + 1], acts[f], up(col(Ws[f].astype(np.float32))).value, up(col(zpre[f])).value,
+                                     pposts[f].value, (pz0 if f == 0 else pposts[f - 1]).value, slots[f].value, dws[f].value,
+                                     dbs[f].value if bias else None)
+    assert hip.fitre_hip_fc_tail_fits(layers, arr, n) == 1
+    nb = hip.fitre_hip_fc_tail_workspace(layers, arr, n)
+    ws = up(np.zeros(nb // 4 + 1, np.float32))
+    ptop = up(col(top))
+    feat = up(np.full(dims[0] * n, np.nan, np.float32))
+    ok(hip.fitre_hip_fc_tail_backward(layers, arr, n, ptop, ext[0], ext[1], feat, ws, nb))
+    for f in range(layers):
+        assert rel_err(dev.download(slots[f], dims[f + 1] * n).reshape(n, dims[f + 1]).T, want_delta[f]) < TOL, ("delta", f)
+        assert rel_err(dev.download(dws[f], dims[f + 1] * dims[f]).reshape(dims[f], dims[f + 1]).T, want_dw[f]) < TOL, ("dW", f)
+        if bias:
+            assert rel_err(dev.download(dbs[f], dims[f + 1]), want_db[f]) < TOL, ("db", f)
+    got = dev.download(feat, dims[0] * n)
+    if ext[0] > 0:      # row m = (c * extB + b) * extA + a of sample s -> [c][s][a][b]
+        a_, b_ = ext
+        c_ = dims[0] // (a_ * b_)
+        want = want_features.reshape(c_, b_, a_, n).transpose(0, 3, 2, 1).reshape(-1)
+    else:
+        want = want_features.T.reshape(-1)
+    assert rel_err(got, want) < TOL
+    # a second call gives the same bits
+    first = [dev.download(q, k) for q, k in zip(dws, [dims[f + 1] * dims[f] for f in range(layers)])]
+    ok(hip.fitre_hip_fc_tail_backward(layers, arr, n, ptop, ext[0], ext[1], feat, ws, nb))
+    for q, k, a in zip(dws, [dims[f + 1] * dims[f] for f in range(layers)], first):
+        np.testing.assert_array_equal(dev.download(q, k), a)
+    # and the per-layer entry points give those bits too: every sum runs in the same order
+    feat_bits = dev.download(feat, dims[0] * n)
+    for f in range(layers):
+        dw2, db2 = up(np.zeros(dims[f + 1] * dims[f], np.float32)), up(np.zeros(dims[f + 1], np.float32))
+        nb2 = hip.fitre_hip_linear_weight_grad_workspace(dims[f], dims[f + 1], n)
+        ws2 = up(np.zeros(nb2 // 4 + 1, np.float32))
+        ok(hip.fitre_hip_linear_weight_grad(dims[f], dims[f + 1], n, slots[f], pz0 if f == 0 else pposts[f - 1], dw2,
+                                            db2 if bias else None, ws2, nb2))
+        np.testing.assert_array_equal(dev.download(dw2, dims[f + 1] * dims[f]), dev.download(dws[f], dims[f + 1] * dims[f]))
+        if bias:
+            np.testing.assert_array_equal(dev.download(db2, dims[f + 1]), dev.download(dbs[f], dims[f + 1]))
+    feat2 = up(np.zeros(dims[0] * n, np.float32))
+    ok(hip.fitre_hip_linear_input_grad(dims[0], dims[1], n, arr[0].W, slots[0], -1, None, None, ext[0], ext[1], feat2, None, None, 0, None))
+    np.testing.assert_array_equal(dev.download(feat2, dims[0] * n), feat_bits)
+    for p in bufs:
+        dev.free(p)
+
+
+def test_tail_rejects_what_does_not_fit(dev):
+    from fitre_amd.structs import fitre_fc_tail_layer
+    arr = (fitre_fc_tail_layer * 2)()
+    arr[0] = fitre_fc_tail_layer(9216, 4096, CNN_ACT_RELU, None, None, None, None, None, None, None)
+    arr[1] = fitre_fc_tail_layer(4096, 1000, CNN_ACT_NONE, None, None, None, None, None, None, None)
+    assert hip.fitre_hip_fc_tail_fits(2, arr, 64) == 0 and hip.fitre_hip_fc_tail_workspace(2, arr, 64) == 0
+    arr[0] = fitre_fc_tail_layer(100, 50, CNN_ACT_RELU, None, None, None, None, None, None, None)
+    arr[1] = fitre_fc_tail_layer(60, 10, CNN_ACT_NONE, None, None, None, None, None, None, None)   # 60 inputs after 50 outputs
+    assert hip.fitre_hip_fc_tail_fits(2, arr, 64) == 0
+    assert hip.fitre_hip_fc_tail_backward(2, arr, 64, None, 0, 0, None, None, 0) == 2
