@@ -8,6 +8,7 @@
 #include "conv_thin.h"
 #include "linear_small.h"
 #include "linear_tail.h"
+#include "linear_skinny.h"
 
 namespace fitre {
 
@@ -914,6 +915,10 @@ int fitre_hip_linear_weight_grad(int in, int out, int n, const float *delta, con
 		p.act = -1;
 		p.rowSums = db;
 		return launch_small_gemm_ranges(p, FITRE_KC_FC_GEMM, ws);
+	}
+	if (skinny_dw_fits(in, out, n)) {
+		const int cus = device_compute_units() > 0 ? device_compute_units() : 256;
+		return launch_skinny_dw(in, out, n, delta, zin, dW, db, cus);
 	}
 	int rc = gemm_ex(0, 1, out, in, n, 1.f, delta, out, zin, in, 0.f, dW, out, nullptr, 0, FITRE_KC_FC_GEMM, ws, wsBytes);
 	if (rc || !db) return rc;

@@ -37,6 +37,9 @@ def forward_act(act, zi):
 # kernel); AlexNet-like layers (the engine) and long reductions over small results (ranges of the batch + a second launch)
 SMALL = [(84, 10, 128), (120, 84, 128), (400, 120, 128), (33, 31, 65), (1, 1, 1), (64, 32, 32), (100, 7, 500), (4096, 100, 96)]
 LARGE = [(1024, 512, 64), (400, 120, 1024), (4096, 1000, 64), (84, 10, 1024), (120, 84, 3000), (33, 7, 8192)]
+# wide layers at a batch of at most 64: the weight gradient that keeps the whole reduction in registers (AlexNet's first
+# linear layer at batch 64, an even batch below 64, ragged edges on either side, the smallest batch)
+SKINNY = [(9216, 4096, 64), (4096, 4096, 62), (1000, 4104, 10), (4100, 1000, 2)]
 
 
 @pytest.mark.parametrize("act", [CNN_ACT_RELU, CNN_ACT_SWISH, CNN_ACT_SOFTPLUS, CNN_ACT_ELU, CNN_ACT_NONE, -1])
@@ -95,7 +98,7 @@ def test_input_gradient_in_the_convolution_layout(dev, channels, ext_a, ext_b, n
 
 
 @pytest.mark.parametrize("bias", [True, False])
-@pytest.mark.parametrize("n_in,n_out,n", SMALL + LARGE)
+@pytest.mark.parametrize("n_in,n_out,n", SMALL + LARGE + SKINNY)
 def test_weight_and_bias_gradient(dev, n_in, n_out, n, bias):
     rng = np.random.default_rng(n_in * 3 + n_out * 5 + n)
     d = rng.standard_normal(n_out * n).astype(np.float32)
