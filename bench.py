@@ -38,13 +38,14 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK_MFMA_F32_TFLOPS = 157.3
+PEAK_MFMA_F64_TFLOPS = 78.6
 PEAK_HBM_GBS = 8000.0
 
 KC = dict(conv_dw=0, conv_dx=1, conv_fwd=2, fc_gemm=3, splitk_reduce=4, bn_bwd=5, bn_fwd=6, pool_bwd=7, pool_fwd=8,
           act_bwd=9, act_fwd=10, bias_grad=11, softmax=12, permute=13, blas1=14, pool_act_bwd=15, kfac_factor=16,
           spd_inverse=17)
 MFMA_CLASSES = ("conv_dw", "conv_dx", "conv_fwd", "fc_gemm", "kfac_factor", "spd_inverse")
-TILES = {0: "", 1: "64x64", 2: "64x128", 3: "128x64", 4: "128x128", 5: "96x128", 6: "dense2x2", 7: "cell4x4", 8: "cell8x8"}
+TILES = {0: "", 1: "64x64", 2: "64x128", 3: "128x64", 4: "128x128", 5: "96x128", 6: "dense2x2", 7: "cell4x4", 8: "cell8x8", 9: "skinny"}
 
 
 def measured_traffic(kernel):
@@ -147,6 +148,11 @@ def kernel_table(rows, steps, launches=None, conv_live=None, fc_batch=None):
                                         frac_mfma=round(r["work"] / (r["ms"] * 1e-3) / 1e12 / PEAK_MFMA_F32_TFLOPS, 4) if r["ms"] > 0 else 0.0,
                                         note="batch %d: bytes = the layer's weight matrix once (read for the input gradient, "
                                              "written for the weight gradient)" % fc_batch)
+            if r["kernel"] in big:   # per-launch work is in FLOP; the same conversion to bytes
+                kernels[r["kernel"]]["largest"] = [dict(e, work=2.0 * e["work"] / fc_batch,
+                                                        achieved=round(2.0 * e["work"] / fc_batch / (e["avg_us"] * 1e-6) / 1e9, 1),
+                                                        frac=round(2.0 * e["work"] / fc_batch / (e["avg_us"] * 1e-6) / 1e9 / PEAK_HBM_GBS, 4))
+                                                   for e in big[r["kernel"]]]
             continue
         rate = r["work"] / (r["ms"] * 1e-3) / (1e12 if mfma else 1e9) if r["ms"] > 0 else 0.0
         peak = PEAK_MFMA_F32_TFLOPS if mfma else PEAK_HBM_GBS
@@ -509,6 +515,22 @@ def kfac_leg(L, dev, gm, model, batch, passes):
     inverses()
     dev.sync()
     out["factors_and_inverses_ms"] = round(1e3 * (time.perf_counter() - t0), 3)
+    # the same pass once more with launch accounting: its float64 products and leaf factorisations
+    L.check(L.hip.fitre_hip_profile_enable(1))
+    inverses()
+    dev.sync()
+    L.check(L.hip.fitre_hip_profile_enable(0))
+    rows64 = [r for r in read_profile(L) if r["cls"] in ("kfac_factor", "spd_inverse")]
+    ms64, work64 = sum(r["ms"] for r in rows64), sum(r["work"] for r in rows64)
+    out["factors_and_inverses"] = dict(
+        arithmetic="f64 (v_mfma_f64_16x16x4f64): factors accumulated, factorised and inverted in double; inverses stored as float "
+                   "pairs; input-side factors with few positions behind them kept in low-rank form",
+        launches=int(sum(r["launches"] for r in rows64)), kernel_ms=round(ms64, 3), gflop=round(work64 / 1e9, 1),
+        achieved=round(work64 / (out["factors_and_inverses_ms"] * 1e-3) / 1e12, 2), unit="TFLOP/s", bound="mfma_f64",
+        peak=PEAK_MFMA_F64_TFLOPS, frac=round(work64 / (out["factors_and_inverses_ms"] * 1e-3) / 1e12 / PEAK_MFMA_F64_TFLOPS, 4),
+        note="work as accounted per launch (2MNK per product, MNK for a symmetric result, 2n^3/3 per 64-order leaf; zero blocks of "
+             "triangular operands are skipped but counted); achieved = that work / the pass's wall time over four streams; "
+             "kernel_ms sums the launches of all streams")
     L.cnn.computeNaturalGradient(C.byref(model), C.byref(info), ws2, None)
     dev.sync()
     t0 = time.perf_counter()

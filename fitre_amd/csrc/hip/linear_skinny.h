@@ -161,7 +161,7 @@ static inline int launch_skinny_dw(int in, int out, int n, const float *delta, c
 	groups = (p.inBlocks + p.inBlocksPerGroup - 1) / p.inBlocksPerGroup;
 	const bool vec = (out & 3) == 0 && (((uintptr_t)dW) & 15) == 0;
 	const dim3 grid((unsigned)outBlocks, (unsigned)groups);
-	LaunchScope scope(FITRE_KC_FC_GEMM, 2.0 * (double)in * out * n, 0);
+	LaunchScope scope(FITRE_KC_FC_GEMM, 2.0 * (double)in * out * n, 9);
 	if (vec) {
 		constexpr size_t ldsBytes = sizeof(float) * 128 * kSkinnyLd;
 		static bool attributeSet = false;

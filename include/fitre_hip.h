@@ -104,8 +104,9 @@ int fitre_hip_profile_read(int kernelClass, long *launches, double *milliseconds
  * one: 0 = not tiled, 1 = 64x64, 2 = 64x128, 3 = 128x64, 4 = 128x128, 5 = 96x128 (channel rows x contiguous columns);
  * 6 and 7 are the 3x3 convolution kernels that leave out the arithmetic on the padding: 6 = the dense per-image form
  * on 2x2 maps, 7 = the cell form on 4x4 maps, 8 = the cell form of the weight gradient on 8x8 maps (their work is
- * still counted as the nine-tap 2*M*K*Cout). */
-#define FITRE_TILE_VARIANTS 9
+ * still counted as the nine-tap 2*M*K*Cout); 9 = the weight gradient of a wide linear layer at a batch of at most 64
+ * (the whole reduction in registers). */
+#define FITRE_TILE_VARIANTS 10
 int fitre_hip_profile_read_tile(int kernelClass, int tile, long *launches, double *milliseconds, double *work);
 /* The accounted launches one by one, in issue order since the last fitre_hip_profile_enable(1) (at most 65 536
  * are kept): class, tile variant, duration and algorithmic work of launch `index` < *count. */

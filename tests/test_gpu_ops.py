@@ -51,6 +51,19 @@ def test_level1(dev):
         dev.free(dx_), dev.free(dy_)
 
 
+def test_copy_of_a_vector_larger_than_the_caches(dev):
+    """fitre_hip_copy from 64 MiB on takes a streaming kernel of its own: same bits, nothing written past the end (a
+    length that is not a multiple of the 1024 vectors a workgroup moves)."""
+    n = (16 << 20) + 4 * 1000
+    x = np.random.default_rng(11).integers(0, 1 << 30, n + 8).astype(np.float32)
+    src, dst = dev.upload(x), dev.upload(np.full(n + 8, -1.0, np.float32))
+    ok(hip.fitre_hip_copy(n, src, dst))
+    got = dev.download(dst, n + 8)
+    np.testing.assert_array_equal(got[:n], x[:n])
+    assert (got[n:] == -1.0).all()
+    dev.free(src), dev.free(dst)
+
+
 def test_elementwise_helpers(dev):
     rng = np.random.default_rng(2)
     n = 4099
