@@ -120,7 +120,7 @@ static size_t backward_chain_ws_bytes(const CNN_MODEL *model, int batch)
 /* the linear layers as the fused tail sees them (shapes only; tail_layers fills in the pointers); 0 when they do not fit it */
 static int tail_shapes(const CNN_MODEL *model, int n, fitre_fc_tail_layer *tail)
 {
-	if (model->lLayers < 1 || model->lLayers > 4) return 0;
+	if (model->lLayers < 2 || model->lLayers > 4) return 0; /* one layer alone: the two per-layer launches are the shorter way */
 	for (int f = 0; f < model->lLayers; f++) {
 		fitre_fc_tail_layer t = { model->fcLayer[f].in, model->fcLayer[f].out, model->fcLayer[f].actFun, NULL, NULL, NULL, NULL, NULL, NULL, NULL };
 		tail[f] = t;

@@ -87,7 +87,15 @@ long kfacInverseMemRequired(CNN_MODEL *model, int samples);
  * accumulated, factored and inverted in float64 on the device and the inverse is stored in the caller's n x n reals
  * as a PAIR of floats per element: the inverse rounded to float on and above the diagonal, the rounding remainder
  * below it (FITRE_MAT_SYM_PAIR, fitre_hip.h).  The upper triangle alone is the float inverse; computeNaturalGradient,
- * the only reader of these arrays in the reference (solvers/kfac_natural_gradient.cu:55-56), takes the pairs. */
+ * the only reader of these arrays in the reference (solvers/kfac_natural_gradient.cu:55-56), takes the pairs.
+ * An input-side factor with few positions behind it (2 * positions <= order, positions = samples * outH * outW of a
+ * convolution layer resp. samples of a linear layer: VGG-11's layers on 2x2 maps at batch 256, its linear layer) is
+ * not inverted at its own order: with A = alpha R R' (R: order x positions),
+ *     (A + s I)^-1 = (I - alpha R S^-1 R') / s,   S = s I + alpha R' R   (order = positions),
+ * and the slot holds, in its n x n words: word 0 = 0xF15EED12 (as a float a negative number, which no diagonal entry
+ * of a positive definite inverse is), word 1 = positions, word 2 = order, words 3, 4 = row / column stride of R in
+ * words, words 5-6 = alpha and 7-8 = s as doubles, word 9 = the word offset of S^-1; R as floats from word 64 on;
+ * S^-1 (positions x positions doubles) at that offset.  computeNaturalGradient reads either form. */
 /* The three trailing arguments are the reference's vendor handles (cublasHandle_t, cudaStream_t,
  * cusolverDnHandle_t, solvers/kfac_inverses.h:28-34), kept so that its solver source compiles against this
  * header unchanged; they are opaque pointers and are ignored (the device layer owns its streams). */
