@@ -152,7 +152,7 @@ __device__ __forceinline__ double dg_value(const DgRaw<KIND> &v, int n, int r, i
 // KA / KB: operand kinds (compile-time: the loads of the float and double kinds are one add and one load per element,
 // their offsets computed once per thread).  blockIdx.x: tile (row-major over tilesM x tilesN), blockIdx.y: split.
 template <int TM, int TN, int BK, int KA, int KB>
-__global__ void __launch_bounds__(256) dgemm_kernel(const DgemmArgs g)
+__device__ __forceinline__ void dgemm_tile(const DgemmArgs &g, const int tile, const int split, const int tiles)
 {
 	// An operand's slice sits in LDS as [k][row], rows TM + 16 doubles apart (a row offset of 16 mod 32: the four k rows of a
 	// fragment read hit different banks), when its lanes run along the rows; as [row][k], rows BK + 1 doubles apart, when
@@ -166,7 +166,7 @@ __global__ void __launch_bounds__(256) dgemm_kernel(const DgemmArgs g)
 	double *As = lds, *Bs = lds + 2 * BUFA; // two buffers each
 	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 	const int wm = wave >> 1, wn = wave & 1;
-	const int tile = blockIdx.x, ti = tile / g.tilesN, tj = tile - ti * g.tilesN;
+	const int ti = tile / g.tilesN, tj = tile - ti * g.tilesN;
 	if ((g.flags & kDgMirror) && tj < ti) return;
 	const int i0 = ti * TM, j0 = tj * TN;
 	int kb = 0, ke = g.K;
@@ -179,7 +179,7 @@ __global__ void __launch_bounds__(256) dgemm_kernel(const DgemmArgs g)
 	if (g.splits > 1) {
 		int chunk = (ke - kb + g.splits - 1) / g.splits;
 		chunk = (chunk + BK - 1) / BK * BK;
-		k0 = kb + (int)blockIdx.y * chunk;
+		k0 = kb + split * chunk;
 		k1 = min(ke, k0 + chunk);
 	}
 
@@ -305,7 +305,7 @@ __global__ void __launch_bounds__(256) dgemm_kernel(const DgemmArgs g)
 	if (g.splits > 1) {
 		// partial tile, element e of thread tid at [e][tid]: coalesced for the reduction kernel, which has the same mapping
 		constexpr int ACC = MI * NI * 4;
-		double *dst = g.partials + ((size_t)blockIdx.y * gridDim.x + tile) * (size_t)(ACC * 256) + tid;
+		double *dst = g.partials + ((size_t)split * tiles + tile) * (size_t)(ACC * 256) + tid;
 #pragma unroll
 		for (int mi = 0; mi < MI; mi++)
 #pragma unroll
@@ -325,6 +325,20 @@ __global__ void __launch_bounds__(256) dgemm_kernel(const DgemmArgs g)
 				            ti == tj);
 }
 
+template <int TM, int TN, int BK, int KA, int KB>
+__global__ void __launch_bounds__(256) dgemm_kernel(const DgemmArgs g)
+{
+	dgemm_tile<TM, TN, BK, KA, KB>(g, (int)blockIdx.x, (int)blockIdx.y, (int)gridDim.x);
+}
+
+// two unsplit products that do not depend on each other as one launch: the first `tiles1` workgroups take the first
+template <int TM, int TN, int BK, int KA, int KB>
+__global__ void __launch_bounds__(256) dgemm_pair_kernel(const DgemmArgs g1, const DgemmArgs g2, int tiles1)
+{
+	if ((int)blockIdx.x < tiles1) dgemm_tile<TM, TN, BK, KA, KB>(g1, (int)blockIdx.x, 0, tiles1);
+	else dgemm_tile<TM, TN, BK, KA, KB>(g2, (int)blockIdx.x - tiles1, 0, (int)gridDim.x - tiles1);
+}
+
 // adds the partial tiles of the splits in split order and stores the result (one workgroup per tile)
 template <int TM, int TN>
 __global__ void __launch_bounds__(256) dgemm_reduce_kernel(const DgemmArgs g)
@@ -337,7 +351,8 @@ __global__ void __launch_bounds__(256) dgemm_reduce_kernel(const DgemmArgs g)
 	const int i0 = ti * TM, j0 = tj * TN;
 	const bool mirrorToo = (g.flags & kDgMirror) && tj > ti && g.C.kind != FITRE_MAT_SYM_PAIR;
 	const size_t tiles = gridDim.x;
-	for (int e = 0; e < ACC; e++) {
+#pragma unroll 8
+	for (int e = 0; e < ACC; e++) { // eight elements' loads in flight; every sum in split order
 		double sum = 0.0;
 		for (int s = 0; s < g.splits; s++) sum += g.partials[((size_t)s * tiles + tile) * (size_t)(ACC * 256) + (size_t)e * 256 + tid];
 		const int mi = e / (NI * 4), ni = (e / 4) % NI, r = e & 3;
@@ -454,8 +469,16 @@ size_t dgemm_workspace(long M, long N, long K, int flags)
 }
 
 // C(M x N) = alpha * A(M x K) * B(K x N) + beta * C (+ diagAdd on the diagonal), on the selected lane
-int dgemm(long M, long N, long K, double alpha, DMat A, DMat B, double beta, DOut C, double diagAdd, int flags, int kernelClass,
-          void *ws, size_t wsBytes)
+struct DgemmLaunch {
+	DgemmArgs g;
+	DgemmPlan p;
+	double flops;
+	float *diagRemainder;
+	int kernelClass;
+};
+
+static int dgemm_setup(long M, long N, long K, double alpha, DMat A, DMat B, double beta, DOut C, double diagAdd, int flags, int kernelClass,
+                       void *ws, size_t wsBytes, DgemmLaunch *out)
 {
 	FITRE_REQUIRE(M > 0 && N > 0 && K > 0 && M < (1l << 30) && N < (1l << 30) && K < (1l << 30), "float64 product: shape %ld x %ld x %ld", M, N, K);
 	FITRE_REQUIRE(A.p && B.p && C.p, "float64 product: null pointer");
@@ -509,13 +532,55 @@ int dgemm(long M, long N, long K, double alpha, DMat A, DMat B, double beta, DOu
 	g.bytesA = (uint32_t)bytesA, g.bytesB = (uint32_t)bytesB;
 	FITRE_REQUIRE(A.rs >= 0 && A.cs >= 0 && B.rs >= 0 && B.cs >= 0, "float64 product: negative stride");
 	FITRE_REQUIRE(A.onesCol < 0 && B.onesRow < 0, "float64 product: a constant row / column along the reduction is not supported");
-	const dim3 grid((unsigned)(p.tilesM * p.tilesN), (unsigned)p.splits);
-	const double flops = ((flags & kDgMirror) ? 1.0 : 2.0) * (double)M * (double)N * (double)K;
-	LaunchScope scope(kernelClass, flops);
-	int rc = launch_dgemm(g, p, grid);
+	out->g = g, out->p = p, out->diagRemainder = diagRemainder, out->kernelClass = kernelClass;
+	out->flops = ((flags & kDgMirror) ? 1.0 : 2.0) * (double)M * (double)N * (double)K;
+	return FITRE_OK;
+}
+
+static int dgemm_issue(const DgemmLaunch &l)
+{
+	const dim3 grid((unsigned)(l.p.tilesM * l.p.tilesN), (unsigned)l.p.splits);
+	LaunchScope scope(l.kernelClass, l.flops);
+	int rc = launch_dgemm(l.g, l.p, grid);
 	if (rc) return rc;
-	if (diagRemainder) pair_fold_diagonal_kernel<<<blocks_for(M, 256), 256, 0, stream()>>>((float *)C.p, C.cs, (int)M, diagRemainder);
+	if (l.diagRemainder)
+		pair_fold_diagonal_kernel<<<blocks_for(l.g.M, 256), 256, 0, stream()>>>((float *)l.g.C.p, l.g.C.cs, l.g.M, l.diagRemainder);
 	return check_launch("float64 product");
+}
+
+// Two products that do not depend on each other: one launch when both are unsplit products of doubles on the small tile
+// (the nodes at the lower levels of the inverse's recursion, which last about as long as a launch costs), else one
+// after the other.
+static int dgemm_issue_pair(const DgemmLaunch &a, const DgemmLaunch &b)
+{
+	const bool together = a.p.splits == 1 && b.p.splits == 1 && a.p.tile == 64 && b.p.tile == 64 && a.g.A.kind == FITRE_MAT_F64 &&
+	                      a.g.B.kind == FITRE_MAT_F64 && b.g.A.kind == FITRE_MAT_F64 && b.g.B.kind == FITRE_MAT_F64 && !a.diagRemainder &&
+	                      !b.diagRemainder;
+	if (!together) {
+		int rc = dgemm_issue(a);
+		return rc ? rc : dgemm_issue(b);
+	}
+	constexpr int T = 64, BK = 32;
+	constexpr size_t perOperand = (BK * (T + 16) > T * (BK + 1)) ? BK * (T + 16) : T * (BK + 1);
+	constexpr size_t ldsBytes = (size_t)4 * perOperand * sizeof(double);
+	static bool attributeSet = false;
+	if (!attributeSet) {
+		FITRE_HIP_TRY(hipFuncSetAttribute((const void *)dgemm_pair_kernel<T, T, BK, FITRE_MAT_F64, FITRE_MAT_F64>,
+		                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes));
+		attributeSet = true;
+	}
+	const int tiles1 = a.p.tilesM * a.p.tilesN, tiles2 = b.p.tilesM * b.p.tilesN;
+	LaunchScope scope(a.kernelClass, a.flops + b.flops);
+	dgemm_pair_kernel<T, T, BK, FITRE_MAT_F64, FITRE_MAT_F64><<<(unsigned)(tiles1 + tiles2), 256, ldsBytes, stream()>>>(a.g, b.g, tiles1);
+	return check_launch("float64 product pair");
+}
+
+int dgemm(long M, long N, long K, double alpha, DMat A, DMat B, double beta, DOut C, double diagAdd, int flags, int kernelClass,
+          void *ws, size_t wsBytes)
+{
+	DgemmLaunch l;
+	int rc = dgemm_setup(M, N, K, alpha, A, B, beta, C, diagAdd, flags, kernelClass, ws, wsBytes, &l);
+	return rc ? rc : dgemm_issue(l);
 }
 
 // ---- leaf of the inverse: a diagonal block of order <= 64, one workgroup, float64 in registers -----------------------
@@ -698,11 +763,15 @@ static int dchol_and_inverse(const DInverseRun &r, int r0, int blocks, int nn, i
 	// L21(m x n1) = A21 * X11^T: B(k, j) = X11(j, k), zero for k > j
 	rc = dgemm(m, n1, n1, 1.0, dmat64(A21, 1, n), dmat64(X11, n, 1), 0.0, DOut{ L21, 1, m, FITRE_MAT_F64 }, 0.0, kDgBUpper, KC, r.gws, r.gBytes);
 	if (rc) return rc;
-	// A22 -= L21 L21^T
-	rc = dgemm(m, m, n1, -1.0, dmat64(L21, 1, m), dmat64(L21, m, 1), 1.0, DOut{ A22, 1, n, FITRE_MAT_F64 }, 0.0, kDgMirror, KC, r.gws, r.gBytes);
+	// A22 -= L21 L21^T and T2(m x n1) = L21 * X11 (B(k, j) = X11(k, j), zero for k < j): neither reads what the other writes
+	DgemmLaunch update, inner;
+	rc = dgemm_setup(m, m, n1, -1.0, dmat64(L21, 1, m), dmat64(L21, m, 1), 1.0, DOut{ A22, 1, n, FITRE_MAT_F64 }, 0.0, kDgMirror, KC, r.gws, r.gBytes,
+	                 &update);
 	if (rc) return rc;
-	// T2(m x n1) = L21 * X11: B(k, j) = X11(k, j), zero for k < j
-	rc = dgemm(m, n1, n1, 1.0, dmat64(L21, 1, m), dmat64(X11, 1, n), 0.0, DOut{ T2, 1, m, FITRE_MAT_F64 }, 0.0, kDgBLower, KC, r.gws, r.gBytes);
+	rc = dgemm_setup(m, n1, n1, 1.0, dmat64(L21, 1, m), dmat64(X11, 1, n), 0.0, DOut{ T2, 1, m, FITRE_MAT_F64 }, 0.0, kDgBLower, KC, r.gws, r.gBytes,
+	                 &inner);
+	if (rc) return rc;
+	rc = dgemm_issue_pair(update, inner);
 	if (rc) return rc;
 	rc = dchol_and_inverse(r, r1, blocks - b1, m, depth + 1);
 	if (rc) return rc;
