@@ -402,6 +402,13 @@ static DgemmPlan plan_dgemm(long M, long N, long K, int flags, bool pairOperand 
 		const long deepest = K / 256 > 0 ? K / 256 : 1;
 		if (splits > deepest) splits = deepest;
 		if (splits > 64) splits = 64;
+	} else if (!(flags & kDgMirror) && K >= 2048 && live < 2 * cus) {
+		// A deep reduction on a grid below one round of workgroups (two are resident per compute unit): as many splits as
+		// bring the grid to about a round (measured on 2305 x 2304 x 2304: 0.88 -> 0.73 ms with two, 4609 x 512 x 4609: 0.90
+		// -> 0.67 ms with three; symmetric products do not gain).
+		splits = (2 * cus + live / 2) / live;
+		if (splits > 4) splits = 4;
+		while (splits > 1 && K / splits < 1024) splits--;
 	}
 	p.splits = (int)splits;
 	return p;
@@ -907,6 +914,48 @@ int fitre_hip_write_header(void *dst, const unsigned int *words, int count)
 	for (int i = 0; i < count; i++) h.w[i] = words[i];
 	write_header_kernel<<<1, 64, 0, stream()>>>((uint32_t *)dst, h, count);
 	return check_launch("write_header_kernel");
+}
+
+// the dense double matrix a float pair stands for, 32 x 32 tiles: a tile and its mirror image are both read along their
+// columns (coalesced) and meet in LDS
+__global__ void __launch_bounds__(256) pair_decode_kernel(const float *P, long ld, int n, double *out, long ldo)
+{
+	__shared__ float U[32][33], V[32][33];
+	const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+	const int r0 = blockIdx.y * 32, c0 = blockIdx.x * 32;
+#pragma unroll
+	for (int k = 0; k < 4; k++) {
+		const int j = ty + 8 * k;
+		U[j][tx] = (r0 + tx < n && c0 + j < n) ? P[(long)(c0 + j) * ld + r0 + tx] : 0.f; // P(r0 + tx, c0 + j)
+		V[j][tx] = (c0 + tx < n && r0 + j < n) ? P[(long)(r0 + j) * ld + c0 + tx] : 0.f; // P(c0 + tx, r0 + j)
+	}
+	__syncthreads();
+#pragma unroll
+	for (int k = 0; k < 4; k++) {
+		const int j = ty + 8 * k, r = r0 + tx, c = c0 + j;
+		if (r >= n || c >= n) continue;
+		const float here = U[j][tx], mirrored = V[tx][j]; // P(r, c), P(c, r)
+		const int a = r < c ? r : c, b = r < c ? c : r;
+		float hi = r <= c ? here : mirrored;
+		uint32_t lo = __float_as_uint(r <= c ? mirrored : here);
+		if (a == b) {
+			lo = 0u;
+			if (n >= 3) lo = __float_as_uint(P[(a + 1 < n) ? (long)a * ld + a + 1 : (long)(n - 1)]) << 16;
+		} else if (n >= 3 && (b == a + 1 || (a == 0 && b == n - 1))) {
+			lo &= 0xFFFF0000u;
+		}
+		out[(long)c * ldo + r] = (double)hi + (double)__uint_as_float(lo);
+	}
+}
+
+int fitre_hip_pair_to_f64(const float *pairs, long ld, int n, double *out, long ldOut)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(pairs && out && n > 0 && ld >= n && ldOut >= n, "fitre_hip_pair_to_f64: bad argument");
+	LaunchScope scope(FITRE_KC_BLAS1, 12.0 * (double)n * n);
+	const unsigned tiles = (unsigned)((n + 31) / 32);
+	pair_decode_kernel<<<dim3(tiles, tiles), 256, 0, stream()>>>(pairs, ld, n, out, ldOut);
+	return check_launch("pair_decode_kernel");
 }
 
 int fitre_hip_widen_shift(const float *matrix, int n, double shift, double *out)

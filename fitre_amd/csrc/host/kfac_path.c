@@ -522,6 +522,38 @@ void computeOmegaZAndLambdaDelta(KFAC_CURVATURE_INFO *kfac_info, CNN_MODEL *mode
 
 /* ---- natural gradient ---------------------------------------------------------------------- */
 
+static fitre_matrix mat_of_pair(const real *slot, int order)
+{
+	fitre_matrix m = { slot, order, order, FITRE_MAT_SYM_PAIR, -1, -1, 0.0 };
+	return m;
+}
+
+/* A float-pair inverse from this order on is decoded into doubles once per layer and the products read the copy
+ * (fitre_hip_pair_to_f64): the pair operand costs two loads per element, one of them across the rows. */
+#define NG_DECODE_ORDER 128
+
+/* doubles for the largest decoded inverse of one side */
+static size_t decoded_bytes(const CNN_MODEL *model, int inputSide)
+{
+	const int b = model->bias != 0 ? 1 : 0;
+	size_t n = 0;
+	for (int l = 0; l < model->cLayers; l++) {
+		const CONV_LAYER *c = &model->convLayer[l];
+		n = max_sz(n, inputSide ? (size_t)(c->inChannels * c->kSize * c->kSize + b) : (size_t)c->outChannels);
+	}
+	for (int l = 0; l < model->lLayers; l++) n = max_sz(n, inputSide ? (size_t)(model->fcLayer[l].in + b) : (size_t)model->fcLayer[l].out);
+	return n >= NG_DECODE_ORDER ? round_up(n * n * sizeof(double), 256) : 0;
+}
+
+/* the operand a product reads a stored float-pair inverse through: the pairs themselves, or their decoded copy */
+static fitre_matrix pair_operand(const real *slot, int order, double *decoded)
+{
+	if (order < NG_DECODE_ORDER || !decoded) return mat_of_pair(slot, order);
+	HIP_CALL(fitre_hip_pair_to_f64(slot, order, order, decoded, order));
+	fitre_matrix m = { decoded, 1, order, FITRE_MAT_F64, -1, -1, 0.0 };
+	return m;
+}
+
 static size_t natural_gradient_bytes(const CNN_MODEL *model, size_t *matBytes)
 {
 	size_t mat = 256, ws = 256;
@@ -539,8 +571,9 @@ static size_t natural_gradient_bytes(const CNN_MODEL *model, size_t *matBytes)
 		ws = max_sz(ws, max_sz(fitre_hip_gemm_f64_workspace(o, k, o, 0), fitre_hip_gemm_f64_workspace(o, k, k, 0)));
 	}
 	*matBytes = round_up(mat, 256);
-	/* [wb | u | zt | t1 | t2 | headers | product workspace]; t1, t2 (low-rank form: positions x Cout, positions <= order / 2) */
-	return 5 * *matBytes + KFAC_INFO_BYTES + round_up(ws, 256) + 256;
+	/* [wb | u | zt | t1 | t2 | headers | decoded Omega^-1 | decoded Lambda^-1 | product workspace]; t1, t2 (low-rank form:
+	 * positions x Cout, positions <= order / 2) */
+	return 5 * *matBytes + KFAC_INFO_BYTES + decoded_bytes(model, 1) + decoded_bytes(model, 0) + round_up(ws, 256) + 256;
 }
 
 long kfacNaturalGradientMemRequired(CNN_MODEL *model)
@@ -565,12 +598,12 @@ typedef struct omega_form {
 /* result (rows x cols, `out`) = Omega^-1 applied to u (doubles) from the left (conv: Omega^-1 * u, u order x cols) or
  * from the right (linear: u * Omega^-1, u rows x order), for either form of the stored inverse */
 static void apply_omega(const OMEGA_FORM *form, const real *slot, int order, int other, int fromLeft, const double *u,
-                        const fitre_matrix *out, double *t1, double *t2, void *ws, size_t wsBytes)
+                        const fitre_matrix *out, double *t1, double *t2, double *decoded, void *ws, size_t wsBytes)
 {
 	const long ldu = fromLeft ? order : other;
 	const fitre_matrix um = mat_of(u, 1, ldu, FITRE_MAT_F64);
 	if (!form->lowrank) {
-		const fitre_matrix omega = mat_of(slot, order, order, FITRE_MAT_SYM_PAIR);
+		const fitre_matrix omega = pair_operand(slot, order, decoded);
 		if (fromLeft)
 			HIP_CALL(fitre_hip_gemm_f64(order, other, order, 1.0, &omega, &um, 0.0, out, 0.0, 0, ws, wsBytes));
 		else
@@ -609,8 +642,11 @@ void computeNaturalGradient(CNN_MODEL *model, KFAC_CURVATURE_INFO *kfacInfo, rea
 	real *wb = (real *)base, *zt = (real *)(base + 2 * matBytes);
 	double *u = (double *)(base + matBytes), *t1 = (double *)(base + 3 * matBytes), *t2 = (double *)(base + 4 * matBytes);
 	unsigned int *headers = (unsigned int *)(base + 5 * matBytes);
-	void *ws = base + 5 * matBytes + KFAC_INFO_BYTES;
-	const size_t wsBytes = total - 5 * matBytes - KFAC_INFO_BYTES - 256;
+	const size_t omegaBytes = decoded_bytes(model, 1), lambdaBytes = decoded_bytes(model, 0);
+	double *omegaDec = omegaBytes ? (double *)(base + 5 * matBytes + KFAC_INFO_BYTES) : NULL;
+	double *lambdaDec = lambdaBytes ? (double *)(base + 5 * matBytes + KFAC_INFO_BYTES + omegaBytes) : NULL;
+	void *ws = base + 5 * matBytes + KFAC_INFO_BYTES + omegaBytes + lambdaBytes;
+	const size_t wsBytes = total - 5 * matBytes - KFAC_INFO_BYTES - omegaBytes - lambdaBytes - 256;
 
 	/* which form every input-side inverse is stored in: the heads of the slots, with one copy */
 	OMEGA_FORM forms[MAX_LAYERS];
@@ -642,7 +678,7 @@ void computeNaturalGradient(CNN_MODEL *model, KFAC_CURVATURE_INFO *kfacInfo, rea
 	for (int c = 0; c < nc; c++) {
 		const CONV_LAYER *l = &model->convLayer[c];
 		const int K = l->inChannels * l->kSize * l->kSize, O = l->outChannels, R = K + bias;
-		const fitre_matrix lambda = mat_of(kfacInfo->LambdaGInv + lambdaOff[c], O, O, FITRE_MAT_SYM_PAIR);
+		const fitre_matrix lambda = pair_operand(kfacInfo->LambdaGInv + lambdaOff[c], O, lambdaDec);
 		const real *v = vec + wOffsets[c];
 		real *ng = nGradient + wOffsets[c];
 		const real *mat = v;
@@ -655,12 +691,12 @@ void computeNaturalGradient(CNN_MODEL *model, KFAC_CURVATURE_INFO *kfacInfo, rea
 		HIP_CALL(fitre_hip_gemm_f64(R, O, O, 1.0, &g, &lambda, 0.0, &um, 0.0, 0, ws, wsBytes));
 		if (bias) {
 			const fitre_matrix out = mat_of(zt, 1, R, FITRE_MAT_F32);
-			apply_omega(&forms[c], kfacInfo->OmegaZInv + omegaOff[c], R, O, 1, u, &out, t1, t2, ws, wsBytes);
+			apply_omega(&forms[c], kfacInfo->OmegaZInv + omegaOff[c], R, O, 1, u, &out, t1, t2, omegaDec, ws, wsBytes);
 			HIP_CALL(fitre_hip_copy_2d(ng, K, zt, R, K, O));
 			HIP_CALL(fitre_hip_copy_2d(nGradient + bOffsets[c], 1, zt + K, R, 1, O));
 		} else {
 			const fitre_matrix out = mat_of(ng, 1, R, FITRE_MAT_F32);
-			apply_omega(&forms[c], kfacInfo->OmegaZInv + omegaOff[c], R, O, 1, u, &out, t1, t2, ws, wsBytes);
+			apply_omega(&forms[c], kfacInfo->OmegaZInv + omegaOff[c], R, O, 1, u, &out, t1, t2, omegaDec, ws, wsBytes);
 		}
 	}
 	/* Linear layers: the gradient block [W | b] already is the out x (in + 1) matrix
@@ -668,11 +704,11 @@ void computeNaturalGradient(CNN_MODEL *model, KFAC_CURVATURE_INFO *kfacInfo, rea
 	for (int f = 0; f < model->lLayers; f++) {
 		const FC_LAYER *l = &model->fcLayer[f];
 		const int R = l->in + bias, O = l->out;
-		const fitre_matrix lambda = mat_of(kfacInfo->LambdaGInv + lambdaOff[nc + f], O, O, FITRE_MAT_SYM_PAIR);
+		const fitre_matrix lambda = pair_operand(kfacInfo->LambdaGInv + lambdaOff[nc + f], O, lambdaDec);
 		const fitre_matrix g = mat_of(vec + wOffsets[nc + f], 1, O, FITRE_MAT_F32), um = mat_of(u, 1, O, FITRE_MAT_F64);
 		const fitre_matrix out = mat_of(nGradient + wOffsets[nc + f], 1, O, FITRE_MAT_F32);
 		HIP_CALL(fitre_hip_gemm_f64(O, R, O, 1.0, &lambda, &g, 0.0, &um, 0.0, 0, ws, wsBytes));
-		apply_omega(&forms[nc + f], kfacInfo->OmegaZInv + omegaOff[nc + f], R, O, 0, u, &out, t1, t2, ws, wsBytes);
+		apply_omega(&forms[nc + f], kfacInfo->OmegaZInv + omegaOff[nc + f], R, O, 0, u, &out, t1, t2, omegaDec, ws, wsBytes);
 	}
 	HIP_CALL(fitre_hip_sync());
 }

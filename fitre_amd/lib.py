@@ -158,6 +158,7 @@ HIP_API = {
     "fitre_hip_spd_inverse_f64_workspace": (sz, [i32]),
     "fitre_hip_spd_inverse_f64_queued": (i32, [vp, i32, vp, i32, vp, sz, vp]),
     "fitre_hip_widen_shift": (i32, [vp, i32, f64, vp]),
+    "fitre_hip_pair_to_f64": (i32, [vp, lng, i32, vp, lng]),
     "fitre_hip_kfac_conv_input_factor_f64_workspace": (sz, [vp, i32]),
     "fitre_hip_kfac_conv_input_factor_f64": (i32, [vp, vp, i32, f64, vp, vp, sz]),
     "fitre_hip_kfac_conv_output_factor_f64": (i32, [vp, vp, f64, vp, vp, sz]),

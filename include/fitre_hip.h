@@ -612,6 +612,10 @@ int fitre_hip_kfac_fc_input_rows(const float *z, int in, int samples, int withBi
  * count (at most 16) words written to the head of a device array.  Stream-ordered. */
 int fitre_hip_gather_headers(const void *const *arrays, int count, void *out);
 int fitre_hip_write_header(void *dst, const unsigned int *words, int count);
+/* out (n x n doubles, leading dimension ldOut, both triangles) = the symmetric matrix that the float pair `pairs` (order n,
+ * leading dimension ld, FITRE_MAT_SYM_PAIR) stands for.  A product that reads a large float-pair operand many times is
+ * faster on the decoded copy (coalesced reads, the large tile); no counterpart in the reference. */
+int fitre_hip_pair_to_f64(const float *pairs, long ld, int n, double *out, long ldOut);
 /* out(n x n doubles) = matrix(n x n floats) + shift * I */
 int fitre_hip_widen_shift(const float *matrix, int n, double shift, double *out);
 /* The four Kronecker factors above accumulated in float64 and written as n x n doubles, with `shift` (the damping) added

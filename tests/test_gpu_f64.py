@@ -118,6 +118,24 @@ def test_gemm_f64_float_pair_operand(dev, n, m):
         dev.free(p)
 
 
+@pytest.mark.parametrize("n", [1, 2, 3, 31, 33, 100, 577])
+def test_float_pair_decoded_on_the_device(dev, n):
+    """fitre_hip_pair_to_f64 gives, bit for bit, the doubles the host decoder reads out of the same words (both triangles,
+    the shared words beside the diagonal included), into a result with a leading dimension of its own."""
+    rng = np.random.default_rng(n)
+    q = rng.standard_normal((n, n))
+    words = pair_encode(q @ q.T * 1e3 + np.eye(n))
+    ld = n + 3
+    pp = dev.upload(words.T.copy())                              # column-major
+    out = dev.upload(np.full(ld * n, -7.0), dtype=np.float64)
+    L.check(hip.fitre_hip_pair_to_f64(pp, n, n, out, ld))
+    got = dev.download(out, ld * n, dtype=np.float64).reshape(n, ld)
+    np.testing.assert_array_equal(got[:, :n].T, pair_decode(words))
+    assert (got[:, n:] == -7.0).all()
+    assert hip.fitre_hip_pair_to_f64(pp, n - 1, n, out, ld) == 2
+    dev.free(pp), dev.free(out)
+
+
 @pytest.mark.parametrize("flag", ["a_lower", "a_upper", "b_lower", "b_upper", "both"])
 @pytest.mark.parametrize("n", [100, 333])
 def test_gemm_f64_triangular_ranges(dev, flag, n):
