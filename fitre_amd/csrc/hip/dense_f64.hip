@@ -339,24 +339,46 @@ __global__ void __launch_bounds__(256) dgemm_pair_kernel(const DgemmArgs g1, con
 	else dgemm_tile<TM, TN, BK, KA, KB>(g2, (int)blockIdx.x - tiles1, 0, (int)gridDim.x - tiles1);
 }
 
-// adds the partial tiles of the splits in split order and stores the result (one workgroup per tile)
+// adds the partial tiles of the splits in split order and stores the result: blockIdx.x = tile, blockIdx.y = which
+// kDgReduceElements of a thread's elements (a tile with hundreds of splits behind it is shared by several workgroups)
+constexpr int kDgReduceElements = 4;
 template <int TM, int TN>
 __global__ void __launch_bounds__(256) dgemm_reduce_kernel(const DgemmArgs g)
 {
 	constexpr int WTM = TM / 2, WTN = TN / 2, MI = WTM / 16, NI = WTN / 16, ACC = MI * NI * 4;
+	static_assert(ACC % kDgReduceElements == 0, "elements per thread");
 	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 	const int wm = wave >> 1, wn = wave & 1;
 	const int tile = blockIdx.x, ti = tile / g.tilesN, tj = tile - ti * g.tilesN;
 	if ((g.flags & kDgMirror) && tj < ti) return;
 	const int i0 = ti * TM, j0 = tj * TN;
 	const bool mirrorToo = (g.flags & kDgMirror) && tj > ti && g.C.kind != FITRE_MAT_SYM_PAIR;
-	const size_t tiles = gridDim.x;
-#pragma unroll 8
-	for (int e = 0; e < ACC; e++) { // eight elements' loads in flight; every sum in split order
-		double sum = 0.0;
-		for (int s = 0; s < g.splits; s++) sum += g.partials[((size_t)s * tiles + tile) * (size_t)(ACC * 256) + (size_t)e * 256 + tid];
+	const size_t tiles = gridDim.x, perSplit = tiles * (size_t)(ACC * 256);
+	const int e0 = (int)blockIdx.y * kDgReduceElements;
+	const double *base = g.partials + (size_t)tile * (size_t)(ACC * 256) + (size_t)e0 * 256 + tid;
+	double sum[kDgReduceElements];
+#pragma unroll
+	for (int e = 0; e < kDgReduceElements; e++) sum[e] = 0.0;
+	int s = 0;
+	for (; s + 4 <= g.splits; s += 4) { // sixteen loads in flight; every sum in split order
+		double v[4][kDgReduceElements];
+#pragma unroll
+		for (int u = 0; u < 4; u++)
+#pragma unroll
+			for (int e = 0; e < kDgReduceElements; e++) v[u][e] = base[(size_t)(s + u) * perSplit + (size_t)e * 256];
+#pragma unroll
+		for (int u = 0; u < 4; u++)
+#pragma unroll
+			for (int e = 0; e < kDgReduceElements; e++) sum[e] += v[u][e];
+	}
+	for (; s < g.splits; s++)
+#pragma unroll
+		for (int e = 0; e < kDgReduceElements; e++) sum[e] += base[(size_t)s * perSplit + (size_t)e * 256];
+#pragma unroll
+	for (int k = 0; k < kDgReduceElements; k++) {
+		const int e = e0 + k;
 		const int mi = e / (NI * 4), ni = (e / 4) % NI, r = e & 3;
-		dgemm_store(g, i0 + wm * WTM + mi * 16 + 4 * r + (lane >> 4), j0 + wn * WTN + ni * 16 + (lane & 15), sum, mirrorToo, ti == tj);
+		dgemm_store(g, i0 + wm * WTM + mi * 16 + 4 * r + (lane >> 4), j0 + wn * WTN + ni * 16 + (lane & 15), sum[k], mirrorToo, ti == tj);
 	}
 }
 
@@ -401,7 +423,7 @@ static DgemmPlan plan_dgemm(long M, long N, long K, int flags, bool pairOperand 
 		splits = (2 * cus + live - 1) / live;
 		const long deepest = K / 256 > 0 ? K / 256 : 1;
 		if (splits > deepest) splits = deepest;
-		if (splits > 64) splits = 64;
+		if (splits > 512) splits = 512;
 	} else if (!(flags & kDgMirror) && K >= 2048 && live < 2 * cus) {
 		// A deep reduction on a grid below one round of workgroups (two are resident per compute unit): as many splits as
 		// bring the grid to about a round (measured on 2305 x 2304 x 2304: 0.88 -> 0.73 ms with two, 4609 x 512 x 4609: 0.90
@@ -439,7 +461,7 @@ static int launch_dgemm_kinds(const DgemmArgs &g, const DgemmPlan &p, dim3 grid)
 		attributeSet = true;
 	}
 	dgemm_kernel<T, T, BK, KA, KB><<<grid, 256, ldsBytes, stream()>>>(g);
-	if (p.splits > 1) dgemm_reduce_kernel<T, T><<<grid.x, 256, 0, stream()>>>(g);
+	if (p.splits > 1) dgemm_reduce_kernel<T, T><<<dim3(grid.x, (T / 32) * (T / 32) * 4 / kDgReduceElements), 256, 0, stream()>>>(g);
 	return FITRE_OK;
 }
 
