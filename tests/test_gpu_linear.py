@@ -156,7 +156,9 @@ TAILS = [
     ((400, 120, 84, 10), 1024, (CNN_ACT_RELU, CNN_ACT_RELU, CNN_ACT_NONE), (5, 5)),      # groups of eight samples
     ((36, 7), 5, (CNN_ACT_SWISH,), (3, 2)),                                                # one layer, an activation on top, ragged group
     ((64, 33, 17, 9, 3), 67, (CNN_ACT_ELU, CNN_ACT_SOFTPLUS, CNN_ACT_SWISH, CNN_ACT_NONE), (0, 0)),   # four layers, no permutation
-    ((1024, 250), 9, (-1,), (4, 4)),                                                       # the widest input, weights staged in many chunks
+    ((1024, 250), 9, (-1,), (4, 4)),                                                       # the widest input: one layer in many parts
+    ((300, 96, 124, 3), 777, (CNN_ACT_RELU, CNN_ACT_ELU, CNN_ACT_NONE), (5, 2)),           # a ragged batch above 512 (ranges + reduction), 12276 weights above the lowest layer
+    ((1000, 3, 2), 70, (CNN_ACT_SWISH, CNN_ACT_NONE), (0, 0)),                             # very few output units under many inputs
 ]
 
 
@@ -259,3 +261,10 @@ def test_tail_rejects_what_does_not_fit(dev):
     arr[1] = fitre_fc_tail_layer(60, 10, CNN_ACT_NONE, None, None, None, None, None, None, None)   # 60 inputs after 50 outputs
     assert hip.fitre_hip_fc_tail_fits(2, arr, 64) == 0
     assert hip.fitre_hip_fc_tail_backward(2, arr, 64, None, 0, 0, None, None, 0) == 2
+    # the layers above the lowest hold at most 12288 weights together
+    arr3 = (fitre_fc_tail_layer * 3)()
+    for top, fits in ((32, 1), (33, 0)):
+        arr3[0] = fitre_fc_tail_layer(200, 64, CNN_ACT_RELU, None, None, None, None, None, None, None)
+        arr3[1] = fitre_fc_tail_layer(64, 128, CNN_ACT_RELU, None, None, None, None, None, None, None)       # 8192
+        arr3[2] = fitre_fc_tail_layer(128, top, CNN_ACT_NONE, None, None, None, None, None, None, None)              # 4096 / 4224
+        assert hip.fitre_hip_fc_tail_fits(3, arr3, 64) == fits, top
