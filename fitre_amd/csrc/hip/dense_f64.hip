@@ -151,9 +151,12 @@ __device__ __forceinline__ double dg_value(const DgRaw<KIND> &v, int n, int r, i
 // accumulator, C(i = 4 r + l / 16, j = l % 16).
 // KA / KB: operand kinds (compile-time: the loads of the float and double kinds are one add and one load per element,
 // their offsets computed once per thread).  blockIdx.x: tile (row-major over tilesM x tilesN), blockIdx.y: split.
-template <int TM, int TN, int BK, int KA, int KB>
+// AKC / BKC: whether the operand is contiguous along the reduction (1), along its rows (0), or decided at run time (-1):
+// with the layout known at compile time every LDS offset of the loop is an immediate.
+template <int TM, int TN, int BK, int KA, int KB, int AKC, int BKC>
 __device__ __forceinline__ void dgemm_tile(const DgemmArgs &g, const int tile, const int split, const int tiles)
 {
+	const bool aKC = AKC < 0 ? (g.aKContig != 0) : (AKC != 0), bKC = BKC < 0 ? (g.bKContig != 0) : (BKC != 0);
 	// An operand's slice sits in LDS as [k][row], rows TM + 16 doubles apart (a row offset of 16 mod 32: the four k rows of a
 	// fragment read hit different banks), when its lanes run along the rows; as [row][k], rows BK + 1 doubles apart, when
 	// they run along k (a k-contiguous operand): the stores of a wave are then contiguous runs of BK doubles, and the
@@ -193,12 +196,12 @@ __device__ __forceinline__ void dgemm_tile(const DgemmArgs &g, const int tile, c
 	// with the lanes along the direction in which the operand is contiguous; its place in LDS and (float / double
 	// operands) its byte offset in memory at reduction index 0 are affine in q as well.
 	constexpr int SA = KA == FITRE_MAT_F64 ? 8 : 4, SB = KB == FITRE_MAT_F64 ? 8 : 4;
-	const int kq0A = g.aKContig ? tid % BK : tid / TM, kStepA = g.aKContig ? 0 : 256 / TM;
-	const int row0A = g.aKContig ? tid / BK : tid % TM, rowStepA = g.aKContig ? 256 / BK : 0;
-	const int kq0B = g.bKContig ? tid % BK : tid / TN, kStepB = g.bKContig ? 0 : 256 / TN;
-	const int row0B = g.bKContig ? tid / BK : tid % TN, rowStepB = g.bKContig ? 256 / BK : 0;
-	const int ldsRowA = g.aKContig ? LDK : 1, ldsKA = g.aKContig ? 1 : LDA; // LDS strides along the rows / along k
-	const int ldsRowB = g.bKContig ? LDK : 1, ldsKB = g.bKContig ? 1 : LDB;
+	const int kq0A = aKC ? tid % BK : tid / TM, kStepA = aKC ? 0 : 256 / TM;
+	const int row0A = aKC ? tid / BK : tid % TM, rowStepA = aKC ? 256 / BK : 0;
+	const int kq0B = bKC ? tid % BK : tid / TN, kStepB = bKC ? 0 : 256 / TN;
+	const int row0B = bKC ? tid / BK : tid % TN, rowStepB = bKC ? 256 / BK : 0;
+	const int ldsRowA = aKC ? LDK : 1, ldsKA = aKC ? 1 : LDA; // LDS strides along the rows / along k
+	const int ldsRowB = bKC ? LDK : 1, ldsKB = bKC ? 1 : LDB;
 	const int lds0A = kq0A * ldsKA + row0A * ldsRowA, ldsStepA = kStepA * ldsKA + rowStepA * ldsRowA;
 	const int lds0B = kq0B * ldsKB + row0B * ldsRowB, ldsStepB = kStepB * ldsKB + rowStepB * ldsRowB;
 	const int stepA = (int)g.A.cs, stepB = (int)g.B.rs; // elements per reduction index
@@ -281,6 +284,14 @@ __device__ __forceinline__ void dgemm_tile(const DgemmArgs &g, const int tile, c
 #pragma unroll
 				for (int ni = 0; ni < NI; ni++) acc[mi][ni] = __builtin_amdgcn_mfma_f64_16x16x4f64(a[mi], b[ni], acc[mi][ni], 0, 0, 0);
 		}
+		// the accumulators stay in the accumulation registers from slice to slice (left alone, the compiler carries them
+		// through the loop in vector registers and copies all of them in and out around every slice)
+		if constexpr (TM == 128) {
+#pragma unroll
+			for (int mi = 0; mi < MI; mi++)
+#pragma unroll
+				for (int ni = 0; ni < NI; ni++) asm volatile("" : "+a"(acc[mi][ni]));
+		}
 	};
 
 	if (k0 < k1) {
@@ -325,18 +336,18 @@ __device__ __forceinline__ void dgemm_tile(const DgemmArgs &g, const int tile, c
 				            ti == tj);
 }
 
-template <int TM, int TN, int BK, int KA, int KB>
-__global__ void __launch_bounds__(256) dgemm_kernel(const DgemmArgs g)
+template <int TM, int TN, int BK, int KA, int KB, int AKC, int BKC>
+__global__ void __launch_bounds__(256, (TM == 64 ? 2 : 1)) dgemm_kernel(const DgemmArgs g)
 {
-	dgemm_tile<TM, TN, BK, KA, KB>(g, (int)blockIdx.x, (int)blockIdx.y, (int)gridDim.x);
+	dgemm_tile<TM, TN, BK, KA, KB, AKC, BKC>(g, (int)blockIdx.x, (int)blockIdx.y, (int)gridDim.x);
 }
 
 // two unsplit products that do not depend on each other as one launch: the first `tiles1` workgroups take the first
 template <int TM, int TN, int BK, int KA, int KB>
-__global__ void __launch_bounds__(256) dgemm_pair_kernel(const DgemmArgs g1, const DgemmArgs g2, int tiles1)
+__global__ void __launch_bounds__(256, 2) dgemm_pair_kernel(const DgemmArgs g1, const DgemmArgs g2, int tiles1)
 {
-	if ((int)blockIdx.x < tiles1) dgemm_tile<TM, TN, BK, KA, KB>(g1, (int)blockIdx.x, 0, tiles1);
-	else dgemm_tile<TM, TN, BK, KA, KB>(g2, (int)blockIdx.x - tiles1, 0, (int)gridDim.x - tiles1);
+	if ((int)blockIdx.x < tiles1) dgemm_tile<TM, TN, BK, KA, KB, -1, -1>(g1, (int)blockIdx.x, 0, tiles1);
+	else dgemm_tile<TM, TN, BK, KA, KB, -1, -1>(g2, (int)blockIdx.x - tiles1, 0, (int)gridDim.x - tiles1);
 }
 
 // adds the partial tiles of the splits in split order and stores the result: blockIdx.x = tile, blockIdx.y = which
@@ -450,19 +461,35 @@ static DMat transposed(const DMat &m)
 	return t;
 }
 
-template <int T, int BK, int KA, int KB>
-static int launch_dgemm_kinds(const DgemmArgs &g, const DgemmPlan &p, dim3 grid)
+template <int T, int BK, int KA, int KB, int AKC, int BKC>
+static int launch_dgemm_layout(const DgemmArgs &g, const DgemmPlan &p, dim3 grid)
 {
 	constexpr size_t perOperand = (BK * (T + 16) > T * (BK + 1)) ? BK * (T + 16) : T * (BK + 1);
 	constexpr size_t ldsBytes = (size_t)4 * perOperand * sizeof(double);
 	static bool attributeSet = false; // dynamic LDS above 64 KB has to be allowed once per kernel
 	if (!attributeSet) {
-		FITRE_HIP_TRY(hipFuncSetAttribute((const void *)dgemm_kernel<T, T, BK, KA, KB>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes));
+		FITRE_HIP_TRY(hipFuncSetAttribute((const void *)dgemm_kernel<T, T, BK, KA, KB, AKC, BKC>, hipFuncAttributeMaxDynamicSharedMemorySize,
+		                                  (int)ldsBytes));
 		attributeSet = true;
 	}
-	dgemm_kernel<T, T, BK, KA, KB><<<grid, 256, ldsBytes, stream()>>>(g);
+	dgemm_kernel<T, T, BK, KA, KB, AKC, BKC><<<grid, 256, ldsBytes, stream()>>>(g);
 	if (p.splits > 1) dgemm_reduce_kernel<T, T><<<dim3(grid.x, (T / 32) * (T / 32) * 4 / kDgReduceElements), 256, 0, stream()>>>(g);
 	return FITRE_OK;
+}
+
+// Operands of one kind on both sides (the products of the inverse, the factor products) get a kernel per layout pair;
+// the mixed products keep the layout as a run-time value.
+template <int T, int BK, int KA, int KB>
+static int launch_dgemm_kinds(const DgemmArgs &g, const DgemmPlan &p, dim3 grid)
+{
+	if constexpr (KA == KB && KA != FITRE_MAT_SYM_PAIR) {
+		if (g.aKContig && g.bKContig) return launch_dgemm_layout<T, BK, KA, KB, 1, 1>(g, p, grid);
+		if (g.aKContig) return launch_dgemm_layout<T, BK, KA, KB, 1, 0>(g, p, grid);
+		if (g.bKContig) return launch_dgemm_layout<T, BK, KA, KB, 0, 1>(g, p, grid);
+		return launch_dgemm_layout<T, BK, KA, KB, 0, 0>(g, p, grid);
+	} else {
+		return launch_dgemm_layout<T, BK, KA, KB, -1, -1>(g, p, grid);
+	}
 }
 
 template <int KA, int KB>
