@@ -407,39 +407,35 @@ __global__ void __launch_bounds__(256) pair_fold_diagonal_kernel(float *pairs, l
 }
 
 struct DgemmPlan {
-	int tile;   // 128 or 64
+	int tile;   // 64
 	int splits;
 	int tilesM, tilesN;
 };
 
-// The 128 x 128 tile as soon as its workgroups fill half the chip (it does four times the work of the small tile per
-// operand byte: measured 44 TFLOP/s against 28), the 64 x 64 tile below that; a grid that still leaves most compute units
-// idle splits the reduction, down to 256 steps per split.
+// Tiles and reduction splits of a product.  One tile size: 64 x 64 with slices of 32 -- two of its workgroups share a
+// compute unit (two waves per SIMD), which a 128 x 128 tile's 512 registers per lane do not allow, and that beats the large
+// tile's better ratio of arithmetic to LDS traffic everywhere (4096^3: 49-52 against 46-48 TFLOP/s; a symmetric order-4609
+// factor over 4096 positions: 1.9 against 2.75 ms).  Splits, each rule from a sweep on the box: a grid far below the chip
+// splits down to 256 reduction steps per split; a deep reduction on a grid of less than two rounds of workgroups splits in
+// two to four (order-2305 factors: 2.46 -> 2.0 ms and 0.64 -> 0.53 ms; order 1153: 1.32 -> 0.67 ms; 4609 x 512 x 4609:
+// 0.67 -> 0.51 ms).
 static DgemmPlan plan_dgemm(long M, long N, long K, int flags, bool pairOperand = false)
 {
+	(void)pairOperand;
 	DgemmPlan p;
 	const int cus = device_compute_units() > 0 ? device_compute_units() : 256;
-	auto count = [&](int t) {
-		const long tm = (M + t - 1) / t, tn = (N + t - 1) / t;
-		return (flags & kDgMirror) ? tm * (tm + 1) / 2 : tm * tn;
-	};
-	// (a float-pair operand costs two loads and a decode per element: its products are faster on the small tile's shorter
-	// register lists, measured 1.3 against 2.1 ms for 4609 x 512 x 4609)
-	p.tile = (2 * count(128) >= cus && !(pairOperand && count(128) < 2 * cus)) ? 128 : 64;
+	p.tile = 64;
 	p.tilesM = (int)((M + p.tile - 1) / p.tile);
 	p.tilesN = (int)((N + p.tile - 1) / p.tile);
-	const long live = count(p.tile);
+	const long live = (flags & kDgMirror) ? (long)p.tilesM * (p.tilesM + 1) / 2 : (long)p.tilesM * p.tilesN;
 	long splits = 1;
 	if (2 * live < cus) {
 		splits = (2 * cus + live - 1) / live;
 		const long deepest = K / 256 > 0 ? K / 256 : 1;
 		if (splits > deepest) splits = deepest;
 		if (splits > 512) splits = 512;
-	} else if (!(flags & kDgMirror) && K >= 2048 && live < 2 * cus) {
-		// A deep reduction on a grid below one round of workgroups (two are resident per compute unit): as many splits as
-		// bring the grid to about a round (measured on 2305 x 2304 x 2304: 0.88 -> 0.73 ms with two, 4609 x 512 x 4609: 0.90
-		// -> 0.67 ms with three; symmetric products do not gain).
-		splits = (2 * cus + live / 2) / live;
+	} else if (K >= 2048 && live < 4 * cus) {
+		splits = (6 * cus + live / 2) / live;
 		if (splits > 4) splits = 4;
 		while (splits > 1 && K / splits < 1024) splits--;
 	}
@@ -495,9 +491,7 @@ static int launch_dgemm_kinds(const DgemmArgs &g, const DgemmPlan &p, dim3 grid)
 template <int KA, int KB>
 static int launch_dgemm_tiles(const DgemmArgs &g, const DgemmPlan &p, dim3 grid)
 {
-	if (p.tile == 128) return launch_dgemm_kinds<128, 16, KA, KB>(g, p, grid);
-	// the small tile takes slices of 32: the products at the bottom of the inverse's recursion (reduction 64) then have all
-	// their loads in flight at once
+	// slices of 32: the products at the bottom of the inverse's recursion (reduction 64) then have all their loads in flight at once
 	return launch_dgemm_kinds<64, 32, KA, KB>(g, p, grid);
 }
 
