@@ -720,6 +720,104 @@ __global__ void __launch_bounds__(256) dchol_leaf_kernel(const double *W, long l
 	}
 }
 
+// ---- a node of two leaves as one launch -----------------------------------------------------------------------------
+//
+// The node of the recursion that joins two 64-order blocks (the second may be smaller) is two leaf factorisations and four
+// 64 x 64 x 64 products, six dependent launches of 16 to 28 us each; here one workgroup does all of it without leaving
+// the compute unit: leaf of A11 in registers, X11 to memory and to LDS; L21 = A21 X11^T, T2 = L21 X11 and L21 L21^T on the
+// matrix pipes from LDS (a wave owns sixteen rows); leaf of A22 - L21 L21^T; X21 = -X22 T2.  Same arithmetic and the same
+// order of every sum as the separate launches up to the blocking of the products.
+constexpr int kNodeLd = kDLeaf + 1; // row stride of the 64 x 64 blocks in LDS (doubles)
+constexpr int kNodeBlock = kDLeaf * kNodeLd;
+
+// C = A * B (transposedB: C = A * B^T) for this wave's sixteen rows, all 64 columns; A, B, C are 64 x 64 blocks in LDS
+template <bool TRANSPOSED_B>
+__device__ __forceinline__ void node_product(const double *A, const double *B, v4d (&acc)[4], int wave, int lane)
+{
+	const int l16 = lane & 15, kq = lane >> 4;
+#pragma unroll
+	for (int nb = 0; nb < 4; nb++) acc[nb] = v4d{ 0.0, 0.0, 0.0, 0.0 };
+#pragma unroll 4
+	for (int kk = 0; kk < kDLeaf / 4; kk++) {
+		const int k = 4 * kk + kq;
+		const double a = A[(16 * wave + l16) * kNodeLd + k];
+#pragma unroll
+		for (int nb = 0; nb < 4; nb++) {
+			const double b = TRANSPOSED_B ? B[(16 * nb + l16) * kNodeLd + k] : B[k * kNodeLd + 16 * nb + l16];
+			acc[nb] = __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, acc[nb], 0, 0, 0);
+		}
+	}
+}
+
+// register r of block nb holds C(16 wave + 4 r + lane / 16, 16 nb + lane % 16)
+__device__ __forceinline__ void node_store_lds(double *C, const v4d (&acc)[4], int wave, int lane)
+{
+#pragma unroll
+	for (int nb = 0; nb < 4; nb++)
+#pragma unroll
+		for (int r = 0; r < 4; r++) C[(16 * wave + 4 * r + (lane >> 4)) * kNodeLd + 16 * nb + (lane & 15)] = acc[nb][r];
+}
+
+__global__ void __launch_bounds__(256) dnode_pair_kernel(const double *W, long ld, int r0, int m, double *X, int *info)
+{
+	extern __shared__ double nodeLds[];
+	double *Xs = nodeLds, *As = Xs + kNodeBlock, *Ls = As + kNodeBlock, *Ts = Ls + kNodeBlock; // X11 / X22, A21 / L21 L21^T, L21, T2
+	__shared__ double Lcol[2 * kDLeaf], Ycol[2 * kDLeaf];
+	const int tid = threadIdx.x, i = tid & 63, q = tid >> 6, lane = tid & 63, wave = tid >> 6;
+	const int r1 = r0 + kDLeaf;
+	double w[16], y[16];
+	// A21(i, k) = W(r1 + i, r0 + k): on its way while the first leaf runs
+	double a21[16];
+#pragma unroll
+	for (int t = 0; t < 16; t++) a21[t] = i < m ? W[(size_t)(r0 + 4 * t + q) * ld + r1 + i] : 0.0;
+	for (int pass = 0; pass < 2; pass++) {
+		const int k0 = pass ? r1 : r0, nn = pass ? m : kDLeaf;
+		const double *blk = W + (size_t)k0 * ld + k0;
+#pragma unroll
+		for (int t = 0; t < 16; t++) {
+			const int c = 4 * t + q;
+			double v = (i == c) ? 1.0 : 0.0; // beyond the block: identity, which factors to itself
+			if (i < nn && c <= i) v = blk[(size_t)c * ld + i] - (pass ? As[i * kNodeLd + c] : 0.0);
+			w[t] = v;
+			y[t] = (i == c) ? 1.0 : 0.0;
+		}
+		dleaf_steps<0>(w, y, Lcol, Ycol, i, q, k0, info);
+		// X(i, r) = Y(r, i) for r <= i: to memory, and the whole block (zeros above the diagonal) to LDS
+		double *xblk = X + (size_t)k0 * ld + k0;
+#pragma unroll
+		for (int t = 0; t < 16; t++) {
+			const int r = 4 * t + q;
+			if (i < nn && r <= i) xblk[(size_t)r * ld + i] = y[t];
+			Xs[i * kNodeLd + r] = (i < nn && r < nn) ? y[t] : 0.0;
+		}
+		if (pass == 0) {
+#pragma unroll
+			for (int t = 0; t < 16; t++) As[i * kNodeLd + 4 * t + q] = a21[t];
+			__syncthreads();
+			v4d acc[4];
+			node_product<true>(As, Xs, acc, wave, lane); // L21 = A21 X11^T
+			node_store_lds(Ls, acc, wave, lane);
+			__syncthreads();
+			node_product<false>(Ls, Xs, acc, wave, lane); // T2 = L21 X11
+			node_store_lds(Ts, acc, wave, lane);
+			node_product<true>(Ls, Ls, acc, wave, lane); // L21 L21^T, which the second leaf takes off A22
+			node_store_lds(As, acc, wave, lane);          // (A21 has been read by every wave: the barrier above)
+			__syncthreads();
+		}
+	}
+	__syncthreads();
+	// X21 = -X22 T2, rows i < m, to X(r1 + i, r0 + j)
+	v4d acc[4];
+	node_product<false>(Xs, Ts, acc, wave, lane);
+#pragma unroll
+	for (int nb = 0; nb < 4; nb++)
+#pragma unroll
+		for (int r = 0; r < 4; r++) {
+			const int row = 16 * wave + 4 * r + (lane >> 4), col = 16 * nb + (lane & 15);
+			if (row < m) X[(size_t)(r0 + col) * ld + r1 + row] = -acc[nb][r];
+		}
+}
+
 __global__ void __launch_bounds__(256) dfill_zero_kernel(double *p, long n)
 {
 	const long stride = (long)gridDim.x * blockDim.x;
@@ -801,6 +899,18 @@ static int dchol_and_inverse(const DInverseRun &r, int r0, int blocks, int nn, i
 		LaunchScope scope(KC, 2.0 * nn * (double)nn * nn / 3.0);
 		dchol_leaf_kernel<<<1, 256, 0, stream()>>>(r.W, n, r0, nn, r.X, r.dInfo);
 		return check_launch("dchol_leaf_kernel");
+	}
+	if (blocks == 2) {
+		constexpr size_t ldsBytes = sizeof(double) * 4 * kNodeBlock;
+		static bool attributeSet = false;
+		if (!attributeSet) {
+			FITRE_HIP_TRY(hipFuncSetAttribute((const void *)dnode_pair_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes));
+			attributeSet = true;
+		}
+		const int m = nn - kDLeaf;
+		LaunchScope scope(KC, 2.0 * (2.0 * kDLeaf * (double)kDLeaf * kDLeaf / 3.0) + 8.0 * kDLeaf * (double)kDLeaf * m);
+		dnode_pair_kernel<<<1, 256, ldsBytes, stream()>>>(r.W, n, r0, m, r.X, r.dInfo);
+		return check_launch("dnode_pair_kernel");
 	}
 	FITRE_REQUIRE(depth < kDMaxDepth, "float64 inverse: recursion deeper than %d", kDMaxDepth);
 	const int b1 = blocks / 2, n1 = b1 * kDLeaf, m = nn - n1, r1 = r0 + n1;
