@@ -928,17 +928,28 @@ int fitre_hip_linear_weight_grad(int in, int out, int n, const float *delta, con
 static int tail_samples(int n) { return n >= 512 ? kTailMaxSamples : 4; }
 static bool tail_in_ranges(int n) { return n > kSmallGemmMaxK; }
 
+// floats of LDS left for a workgroup's part of the lowest layer beside the two delta buffers and the upper layers
+static long tail_low_floats(int layers, const fitre_fc_tail_layer *l, long upperLds)
+{
+	int maxDim = 1;
+	for (int f = 0; f < layers; f++) {
+		maxDim = l[f].in > maxDim ? l[f].in : maxDim;
+		maxDim = l[f].out > maxDim ? l[f].out : maxDim;
+	}
+	return 160 * 1024 / 4 - 64 - 2L * kTailMaxSamples * (maxDim + 1) - upperLds;
+}
+
 int fitre_hip_fc_tail_fits(int layers, const fitre_fc_tail_layer *l, int n)
 {
 	if (!l || layers < 1 || layers > kTailMaxLayers || n < 1 || n > 65536) return 0;
-	long upper = 0;
+	long upperLds = 0;
 	for (int f = 0; f < layers; f++) {
 		if (l[f].in < 1 || l[f].out < 1 || l[f].in > kTailMaxDim || l[f].out > kTailMaxDim) return 0;
 		if (f > 0 && l[f].in != l[f - 1].out) return 0;
 		if (!(tail_in_ranges(n) ? small_gemm_ranges_fit(l[f].out, l[f].in, n) : small_gemm_fits(l[f].out, l[f].in, n))) return 0;
-		if (f > 0) upper += (long)l[f].in * l[f].out;
+		if (f > 0) upperLds += (long)l[f].in * (l[f].out + 1);
 	}
-	return upper <= kTailUpperFloats;
+	return upperLds <= kTailUpperLds && tail_low_floats(layers, l, upperLds) >= l[0].out + 1; // the layers above the lowest sit in LDS whole
 }
 
 size_t fitre_hip_fc_tail_workspace(int layers, const fitre_fc_tail_layer *l, int n)
@@ -978,28 +989,25 @@ int fitre_hip_fc_tail_backward(int layers, const fitre_fc_tail_layer *l, int n, 
 		d.in = l[f].in, d.out = l[f].out, d.act = l[f].act;
 		d.W = l[f].W, d.zPre = l[f].zPre, d.zPost = l[f].zPost, d.slot = l[f].slot;
 		d.outMagic = (unsigned)((1ull << 32) / (unsigned)d.out) + 1u;
-		if (f > 0) {
-			d.firstWeight = p.upperWeights, d.ldsBase = upperLds;
-			p.upperWeights += d.in * d.out, upperLds += d.in * (d.out + 1);
-		}
+		if (f > 0) d.ldsBase = upperLds, upperLds += d.in * (d.out + 1);
 		maxDim = d.in > maxDim ? d.in : maxDim;
 		maxDim = d.out > maxDim ? d.out : maxDim;
 		chainFlops += 2.0 * (double)d.in * d.out * n;
 	}
 	p.maxDim = maxDim;
 	const int groups = (n + p.ns - 1) / p.ns;
-	// parts of the lowest layer: each fits a workgroup's registers, and together with the groups they fill the chip
-	const long lowest = (long)l[0].in * l[0].out;
-	int parts = (int)((lowest + kTailPartFloats - 1) / kTailPartFloats);
+	// parts of the lowest layer: each fits its share of LDS, and together with the groups they fill the chip
+	const int mostRows = (int)(tail_low_floats(layers, l, upperLds) / (l[0].out + 1));
+	int parts = (l[0].in + mostRows - 1) / mostRows;
 	const int cus = device_compute_units() > 0 ? device_compute_units() : 256;
 	const int fill = (cus + groups - 1) / groups;
 	parts = parts < fill ? fill : parts;
 	parts = parts > l[0].in ? l[0].in : parts;
 	p.partInputs = (l[0].in + parts - 1) / parts;
-	while ((long)p.partInputs * l[0].out > kTailPartFloats) p.partInputs--; // rounding up must not pass the registers
+	if (p.partInputs > mostRows) p.partInputs = mostRows;
 	parts = (l[0].in + p.partInputs - 1) / p.partInputs;
-	const int lowLds = p.partInputs * (l[0].out + 1);
-	const size_t ldsBytes = sizeof(float) * ((size_t)2 * kTailMaxSamples * (maxDim + 1) + (upperLds > lowLds ? upperLds : lowLds) + 64);
+	p.lowBase = upperLds;
+	const size_t ldsBytes = sizeof(float) * ((size_t)2 * kTailMaxSamples * (maxDim + 1) + upperLds + (size_t)p.partInputs * (l[0].out + 1) + 64);
 	static bool attributeSet = false;
 	if (!attributeSet) {
 		FITRE_HIP_TRY(hipFuncSetAttribute((const void *)fc_tail_chain_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
@@ -1007,7 +1015,7 @@ int fitre_hip_fc_tail_backward(int layers, const fitre_fc_tail_layer *l, int n, 
 	}
 	{
 		LaunchScope scope(FITRE_KC_FC_GEMM, chainFlops, 0);
-		fc_tail_chain_kernel<<<dim3((unsigned)groups, (unsigned)parts), 256, ldsBytes, stream()>>>(p);
+		fc_tail_chain_kernel<<<dim3((unsigned)groups, (unsigned)parts), kTailThreads, ldsBytes, stream()>>>(p);
 	}
 	// every layer's delta * zin' and delta * 1
 	SmallGemmBatch b{};

@@ -6,28 +6,29 @@
 //      on its own: delta_f (after the activation derivative) into its dx slot and into LDS, delta_{f-1} = f'(.) .* (W_f'
 //      delta_f) from weights staged in LDS.  The lowest layer has the most weights and nothing below it waits for
 //      all of its outputs at once, so its inputs are cut into parts that different workgroups take (each repeats the
-//      few thousand multiply-adds of the layers above); a workgroup requests its part of those weights first and uses
-//      them last, so their latency passes behind the upper layers.  The result goes to the convolution layout.
+//      few thousand multiply-adds of the layers above).  A workgroup has sixteen waves, so that a wave's share of the
+//      weight rows is a dozen loads, all in flight at once.  The result goes to the convolution layout.
 //   2. every layer's weight and bias gradient, delta_f * zin_f' and delta_f * 1, as ONE launch of the small product
 //      kernel over the blocks of all layers (a long batch is cut into ranges, added by a third launch in range order).
 // The order of every sum is fixed by the shapes alone.
 #pragma once
+#include "gemm_engine.h"
 #include "linear_small.h"
 
 namespace fitre {
 
 constexpr int kTailMaxLayers = 4;
-constexpr int kTailMaxDim = 1024;         // inputs / outputs of a layer
-constexpr int kTailMaxSamples = 8;        // samples of a group
-constexpr int kTailPartFloats = 48 * 256; // weights of the lowest layer a workgroup takes, held in registers until used
-constexpr int kTailUpperFloats = 48 * 256; // weights of all layers above the lowest together, likewise
+constexpr int kTailMaxDim = 1024;   // inputs / outputs of a layer
+constexpr int kTailMaxSamples = 8;  // samples of a group
+constexpr int kTailThreads = 1024;  // sixteen waves: a wave's share of the weight rows is short enough for all its loads to be in flight
+constexpr int kTailWaves = kTailThreads / 64;
+constexpr int kTailUpperLds = 16384; // floats of LDS for the weights of the layers above the lowest
 
 struct FcTailLayer {
 	int in, out;
 	int act;                   // this layer's activation
 	unsigned outMagic;         // e / out == __umulhi(e, outMagic) for e < 2^20
 	int ldsBase;               // where its weights sit in LDS as [input][out + 1] (layers above the lowest)
-	int firstWeight;           // weights of the layers 1 .. f - 1 (its place in the registers that prefetch them)
 	const float *W;            // out x in, column-major
 	const float *zPre, *zPost; // its output before / after the activation, out x n
 	float *slot;               // receives delta (after the activation derivative), out x n
@@ -40,53 +41,47 @@ struct FcTailParams {
 	const float *delta; // at the top layer's output, before its activation derivative
 	float *features;
 	int maxDim;
-	int partInputs;   // inputs of the lowest layer per blockIdx.y
-	int upperWeights; // weights of the layers above the lowest
+	int partInputs; // inputs of the lowest layer per blockIdx.y
+	int lowBase;    // where the lowest layer's part sits in LDS
 };
 
 __device__ __forceinline__ int tail_div(int e, int out, unsigned magic) { return out == 1 ? e : (int)__umulhi((unsigned)e, magic); }
 
-__global__ void __launch_bounds__(256) fc_tail_chain_kernel(const FcTailParams p)
+// rows [row0, row0 + rows) of W (an input per row, its `out` output units contiguous) to LDS as [row][out + 1]: a wave
+// moves whole rows, the lanes along a row
+__device__ __forceinline__ void tail_stage_rows(const float *W, int out, int row0, int rows, float *dst, int wave, int lane)
+{
+	const int ldw = out + 1;
+	for (int c0 = 0; c0 < out; c0 += 64) {
+		const int col = c0 + lane;
+		const bool ok = col < out;
+		const float *src = W + (long)row0 * out + col;
+#pragma unroll 8
+		for (int r = wave; r < rows; r += kTailWaves) {
+			const float v = ok ? src[(long)r * out] : 0.f;
+			if (ok) dst[r * ldw + col] = v;
+		}
+	}
+}
+
+__global__ void __launch_bounds__(kTailThreads) fc_tail_chain_kernel(const FcTailParams p)
 {
 	extern __shared__ float lds[];
 	const int ldd = p.maxDim + 1;
 	float *dcur = lds, *dnext = lds + kTailMaxSamples * ldd, *wbuf = dnext + kTailMaxSamples * ldd;
-	const int tid = threadIdx.x;
+	const int tid = threadIdx.x, lane = tid & 63;
+	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 	const int s0 = blockIdx.x * p.ns;
 	const int cnt = (p.n - s0 < p.ns) ? p.n - s0 : p.ns;
 	const bool first = blockIdx.y == 0; // the workgroup that writes the slots of the layers above the lowest
-	// every weight this workgroup multiplies by is requested before anything waits: its part of the lowest layer ...
+	// every weight this workgroup multiplies by goes to LDS first: the layers above the lowest, whole, and its part of the lowest
 	const FcTailLayer &low = p.l[0];
 	const int pi0 = blockIdx.y * p.partInputs;
 	const int pni = (low.in - pi0 < p.partInputs) ? low.in - pi0 : p.partInputs;
-	float wlow[kTailPartFloats / 256], wup[kTailUpperFloats / 256];
-	{
-		const float *src = low.W + (long)pi0 * low.out;
-		const int count = pni * low.out;
 #pragma unroll
-		for (int t = 0; t < kTailPartFloats / 256; t++) wlow[t] = (tid + 256 * t < count) ? src[tid + 256 * t] : 0.f;
-	}
-	// ... and the layers above it, whole
-#pragma unroll
-	for (int t = 0; t < kTailUpperFloats / 256; t++) {
-		const int e = tid + 256 * t;
-		// which layer: static indices, so that the argument block stays in scalar registers
-		const float *src = p.l[1].W;
-		int base = 0;
-		if (p.layers > 2 && e >= p.l[2].firstWeight) src = p.l[2].W, base = p.l[2].firstWeight;
-		if (p.layers > 3 && e >= p.l[3].firstWeight) src = p.l[3].W, base = p.l[3].firstWeight;
-		wup[t] = e < p.upperWeights ? src[e - base] : 0.f;
-	}
-#pragma unroll
-	for (int t = 0; t < kTailUpperFloats / 256; t++) {
-		const int e = tid + 256 * t;
-		int base = 0, out = p.l[1].out, to = p.l[1].ldsBase;
-		unsigned magic = p.l[1].outMagic;
-		if (p.layers > 2 && e >= p.l[2].firstWeight) base = p.l[2].firstWeight, out = p.l[2].out, to = p.l[2].ldsBase, magic = p.l[2].outMagic;
-		if (p.layers > 3 && e >= p.l[3].firstWeight) base = p.l[3].firstWeight, out = p.l[3].out, to = p.l[3].ldsBase, magic = p.l[3].outMagic;
-		const int k = e - base;
-		if (e < p.upperWeights) wbuf[to + k + tail_div(k, out, magic)] = wup[t]; // [i][o] with rows out + 1 apart
-	}
+	for (int f = kTailMaxLayers - 1; f >= 1; f--)
+		if (f < p.layers) tail_stage_rows(p.l[f].W, p.l[f].out, 0, p.l[f].in, wbuf + p.l[f].ldsBase, wave, lane);
+	tail_stage_rows(low.W, low.out, pi0, pni, wbuf + p.lowBase, wave, lane);
 	const int planeAB = p.extA * p.extB;
 	// the layers top down; unrolled so that every index into the argument block is a constant
 #pragma unroll
@@ -97,7 +92,7 @@ __global__ void __launch_bounds__(256) fc_tail_chain_kernel(const FcTailParams p
 		const bool below = f > 0;
 		if (f == p.layers - 1) { // delta at the top, times its activation derivative
 			const bool derivative = lay.act != CNN_ACT_NONE && lay.act != ACT_LINEAR && lay.act >= 0;
-			for (int e = tid; e < lay.out * cnt; e += 256) {
+			for (int e = tid; e < lay.out * cnt; e += kTailThreads) {
 				const int s = tail_div(e, lay.out, lay.outMagic), o = e - s * lay.out;
 				const long at = (long)(s0 + s) * lay.out + o;
 				float v = p.delta[at];
@@ -109,20 +104,10 @@ __global__ void __launch_bounds__(256) fc_tail_chain_kernel(const FcTailParams p
 		const int in = lay.in, out = lay.out, ldw = out + 1;
 		const bool derivative = below && under.act != CNN_ACT_NONE && under.act != ACT_LINEAR && under.act >= 0;
 		const int i0 = below ? 0 : pi0, ni = below ? in : pni;
-		const float *wl = wbuf + (below ? lay.ldsBase : 0);
+		const float *wl = wbuf + (below ? lay.ldsBase : p.lowBase);
 		__syncthreads(); // dcur and the staged weights are complete; the layer above has been read
-		if (!below) {
-			// the lowest layer's part takes the place of the layers above it
-			const int count = pni * out;
-#pragma unroll
-			for (int t = 0; t < kTailPartFloats / 256; t++) {
-				const int e = tid + 256 * t;
-				if (e < count) wbuf[e + tail_div(e, out, lay.outMagic)] = wlow[t];
-			}
-			__syncthreads();
-		}
 		// (i, s) = f'(.) * sum over o of W(o, i) delta(o, s)
-		for (int e = tid; e < ni * cnt; e += 256) {
+		for (int e = tid; e < ni * cnt; e += kTailThreads) {
 			const int s = e / ni, ii = e - s * ni;
 			const int i = i0 + ii;
 			const long at = (long)(s0 + s) * in + i;

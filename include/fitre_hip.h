@@ -429,8 +429,8 @@ int fitre_hip_linear_weight_grad(int in, int out, int n, const float *delta, con
  * bits as the per-layer entry points above give for layers this small (functions/cnn_backward.cu:100-254 for every
  * layer of the tail): every sum runs in the same order.  delta: at the top layer's output (out x n), before that
  * layer's activation derivative.  _fits: at most four layers of at most 1024 units, each of them small in the sense
- * of fitre_hip_linear_is_small (or, above 512 samples, within the ranged weight gradient's limits), the layers above
- * the lowest holding at most 12288 weights together.  Workspace:
+ * of fitre_hip_linear_is_small (or, above 512 samples, within the ranged weight gradient's limits), the layers above the
+ * lowest together within 16384 floats of LDS (the sum of in * (out + 1)).  Workspace:
  * fitre_hip_fc_tail_workspace bytes (only read above 512 samples; ws may be NULL otherwise). */
 typedef struct fitre_fc_tail_layer {
 	int in, out;

@@ -261,10 +261,10 @@ def test_tail_rejects_what_does_not_fit(dev):
     arr[1] = fitre_fc_tail_layer(60, 10, CNN_ACT_NONE, None, None, None, None, None, None, None)   # 60 inputs after 50 outputs
     assert hip.fitre_hip_fc_tail_fits(2, arr, 64) == 0
     assert hip.fitre_hip_fc_tail_backward(2, arr, 64, None, 0, 0, None, None, 0) == 2
-    # the layers above the lowest hold at most 12288 weights together
+    # the layers above the lowest sit in LDS whole: the sum of in * (out + 1) at most 16384 floats
     arr3 = (fitre_fc_tail_layer * 3)()
-    for top, fits in ((32, 1), (33, 0)):
+    for top, fits in ((62, 1), (63, 0)):
         arr3[0] = fitre_fc_tail_layer(200, 64, CNN_ACT_RELU, None, None, None, None, None, None, None)
-        arr3[1] = fitre_fc_tail_layer(64, 128, CNN_ACT_RELU, None, None, None, None, None, None, None)       # 8192
-        arr3[2] = fitre_fc_tail_layer(128, top, CNN_ACT_NONE, None, None, None, None, None, None, None)              # 4096 / 4224
+        arr3[1] = fitre_fc_tail_layer(64, 128, CNN_ACT_RELU, None, None, None, None, None, None, None)      # 64 * 129 = 8256
+        arr3[2] = fitre_fc_tail_layer(128, top, CNN_ACT_NONE, None, None, None, None, None, None, None)     # 128 * 63 = 8064, 128 * 64 = 8192
         assert hip.fitre_hip_fc_tail_fits(3, arr3, 64) == fits, top
