@@ -635,14 +635,15 @@ int dgemm(long M, long N, long K, double alpha, DMat A, DMat B, double beta, DOu
 
 // ---- leaf of the inverse: a diagonal block of order <= 64, one workgroup, float64 in registers -----------------------
 //
-// One sweep of 64 steps, one barrier each, does the Cholesky factorisation W = L L^T (right-looking) and the inverse of
+// One sweep of 64 steps, a barrier every four, does the Cholesky factorisation W = L L^T (right-looking) and the inverse of
 // the factor together: the column operations that turn L^T into the identity (scale column j by 1 / l_jj, then column
 // k -= column j * l_kj for k > j) turn the identity into Y = L^-T, and step j of them needs exactly column j of L, which
 // step j of the factorisation has just produced.  Thread (i, q) = (lane, wave) keeps row i of the trailing matrix --
 // W(i, k) for k = 4 t + q -- and column i of Y -- Y(r, i) for r = 4 t + q -- in registers, 16 doubles each; what a step
-// needs from other threads (column j of W, column j of Y) goes through two small LDS vectors, double-buffered by the
-// parity of the step, and is read back wave-uniformly (broadcasts).  The steps are unrolled by template recursion, so
-// that every register index and every loop bound is a constant.
+// needs from other threads: column j of W goes through LDS, four columns (a register of each wave) at a time, and is read
+// back one row per lane, so that the entries a thread multiplies by are lanes of one register; column j of Y (rows r =
+// 4 t + q) is lane j of the same wave's registers.  The steps are unrolled by template recursion, so that every
+// register index, lane index and loop bound is a constant or wave-uniform.
 constexpr int kDLeaf = 64;
 
 __device__ __forceinline__ double rsqrt_f64(double a)
@@ -655,49 +656,85 @@ __device__ __forceinline__ double rsqrt_f64(double a)
 // Step J.  Entries of a row right of the diagonal (k > i) are never read, so the trailing update runs over them
 // unmasked; what has to be masked is folded into the multiplier (zero where a thread must not update), which keeps
 // the step free of branches and of selects on loaded values.
-template <int J>
-__device__ __forceinline__ void dleaf_steps(double (&w)[16], double (&y)[16], double *Lcol, double *Ycol, int i, int q, int k0, int *info)
+// a double of another lane of the wave (the lane index is wave-uniform)
+__device__ __forceinline__ double lane_value(double v, int lane)
 {
-	constexpr int jb = J >> 2, js = J & 3;
-	double *lc = Lcol + (J & 1) * kDLeaf, *yc = Ycol + (J & 1) * kDLeaf;
-	if (q == js) lc[i] = w[jb]; // column J of the trailing matrix (rows >= J are read)
-	if (i == J) {
+	const int lo = __builtin_amdgcn_readlane(__double2loint(v), lane), hi = __builtin_amdgcn_readlane(__double2hiint(v), lane);
+	return __hiloint2double(hi, lo);
+}
+
+// Step S of panel JB (column J = 4 JB + S).  c[]: the panel's four columns, one row per lane, every thread updating
+// them alike.  Entries of a row right of the diagonal (k > i) are never read, so the trailing update runs over them
+// unmasked; what has to be masked is folded into the multiplier (zero where a thread must not update), which keeps
+// the step free of branches and of selects on loaded values.
+template <int JB, int S>
+__device__ __forceinline__ void dleaf_step(double (&w)[16], double (&y)[16], double (&c)[4], double &dOwn, int &bad, int i, int q)
+{
+	constexpr int J = 4 * JB + S;
+	const double li = c[S];
+	const double ajj = lane_value(li, J);
+	double lk[16 - JB], yr[JB + 1], lc[4];
 #pragma unroll
-		for (int t = 0; t <= jb; t++) yc[4 * t + q] = y[t]; // column J of Y, rows <= J
-	}
-	__syncthreads();
-	const double ajj = lc[J], li = lc[i];
-	double lk[16 - jb], yr[jb + 1];
+	for (int t = JB + 1; t < 16; t++) lk[t - JB] = lane_value(li, 4 * t + q);
 #pragma unroll
-	for (int t = jb; t < 16; t++) lk[t - jb] = lc[4 * t + q];
+	for (int u = S + 1; u < 4; u++) lc[u] = lane_value(li, 4 * JB + u);
 #pragma unroll
-	for (int t = 0; t <= jb; t++) yr[t] = yc[4 * t + q];
-	if (!(ajj > 0.0) && i == 0 && q == 0) atomicCAS(info, 0, k0 + J + 1);
+	for (int t = 0; t <= JB; t++) yr[t] = lane_value(y[t], J);
+	if (!(ajj > 0.0) && bad == 0) bad = J + 1; // wave-uniform
 	const double d = rsqrt_f64(ajj);
 	const double m = li * (d * d);              // l_iJ / l_JJ
 	const double mw = (i > J) ? m : 0.0;        // rows below the pivot row take the update
-	// trailing matrix: W(i, k) -= l_iJ l_kJ for k > J
-	w[jb] = __builtin_fma((q > js) ? -mw : 0.0, lk[0], w[jb]);
+	if (i == J) dOwn = d;                       // column J of Y is final but for this factor (row J of X)
+	// trailing matrix: W(i, k) -= l_iJ l_kJ for k > J: the rest of the panel first (the next pivot is in it)
 #pragma unroll
-	for (int t = jb + 1; t < 16; t++) w[t] = __builtin_fma(-mw, lk[t - jb], w[t]);
-	// Y: column i -= column J * l_iJ / l_JJ for i > J, rows r <= J; column J itself is scaled and final (row J of X)
-	const double sc = (i == J) ? d : 1.0;
+	for (int u = S + 1; u < 4; u++) c[u] = __builtin_fma(-mw, lc[u], c[u]);
 #pragma unroll
-	for (int t = 0; t < jb; t++) y[t] = __builtin_fma(-mw, yr[t], y[t]) * sc;
-	y[jb] = __builtin_fma((q <= js) ? -mw : 0.0, yr[jb], y[jb]) * sc;
+	for (int t = JB + 1; t < 16; t++) w[t] = __builtin_fma(-mw, lk[t - JB], w[t]);
+	// Y: column i -= column J * l_iJ / l_JJ for i > J, rows r <= J
+#pragma unroll
+	for (int t = 0; t < JB; t++) y[t] = __builtin_fma(-mw, yr[t], y[t]);
+	y[JB] = __builtin_fma((q <= S) ? -mw : 0.0, yr[JB], y[JB]);
 	// the updates stay in this step: left to itself the compiler postpones them until a value is needed and keeps
 	// the operands of every postponed step alive
 #pragma unroll
-	for (int t = jb; t < 16; t++) asm volatile("" : "+v"(w[t]));
+	for (int t = JB + 1; t < 16; t++) asm volatile("" : "+v"(w[t]));
 #pragma unroll
-	for (int t = 0; t <= jb; t++) asm volatile("" : "+v"(y[t]));
-	if constexpr (J + 1 < kDLeaf) dleaf_steps<J + 1>(w, y, Lcol, Ycol, i, q, k0, info);
+	for (int t = 0; t <= JB; t++) asm volatile("" : "+v"(y[t]));
+}
+
+// Panel JB: columns 4 JB .. 4 JB + 3 of the trailing matrix are register JB of the four waves; they go through LDS once
+// (double-buffered by the parity of the panel) and every wave then runs the panel's four steps on its own.
+template <int JB>
+__device__ __forceinline__ void dleaf_panels(double (&w)[16], double (&y)[16], double &dOwn, int &bad, double *panel, int i, int q)
+{
+	double *pc = panel + (JB & 1) * 4 * kDLeaf;
+	pc[q * kDLeaf + i] = w[JB];
+	__syncthreads();
+	double c[4];
+#pragma unroll
+	for (int u = 0; u < 4; u++) c[u] = pc[u * kDLeaf + i];
+	dleaf_step<JB, 0>(w, y, c, dOwn, bad, i, q);
+	dleaf_step<JB, 1>(w, y, c, dOwn, bad, i, q);
+	dleaf_step<JB, 2>(w, y, c, dOwn, bad, i, q);
+	dleaf_step<JB, 3>(w, y, c, dOwn, bad, i, q);
+	if constexpr (JB + 1 < 16) dleaf_panels<JB + 1>(w, y, dOwn, bad, panel, i, q);
+}
+
+// the whole leaf: L is consumed column by column, Y = L^-T comes out; i = lane, q = wave (uniform); panel: 8 * kDLeaf doubles
+__device__ __forceinline__ void dleaf_run(double (&w)[16], double (&y)[16], double *panel, int i, int q, int k0, int *info)
+{
+	double dOwn = 1.0;
+	int bad = 0;
+	dleaf_panels<0>(w, y, dOwn, bad, panel, i, q);
+#pragma unroll
+	for (int t = 0; t < 16; t++) y[t] *= dOwn;
+	if (bad != 0 && i == 0 && q == 0) atomicCAS(info, 0, k0 + bad);
 }
 
 __global__ void __launch_bounds__(256) dchol_leaf_kernel(const double *W, long ld, int k0, int nn, double *X, int *info)
 {
-	__shared__ double Lcol[2 * kDLeaf], Ycol[2 * kDLeaf];
-	const int tid = threadIdx.x, i = tid & 63, q = tid >> 6;
+	__shared__ double Lcol[8 * kDLeaf];
+	const int tid = threadIdx.x, i = tid & 63, q = __builtin_amdgcn_readfirstlane(tid >> 6);
 	const double *blk = W + (size_t)k0 * ld + k0;
 	double w[16], y[16];
 #pragma unroll
@@ -708,7 +745,7 @@ __global__ void __launch_bounds__(256) dchol_leaf_kernel(const double *W, long l
 		w[t] = v;
 		y[t] = (i == c) ? 1.0 : 0.0;
 	}
-	dleaf_steps<0>(w, y, Lcol, Ycol, i, q, k0, info);
+	dleaf_run(w, y, Lcol, i, q, k0, info);
 	// X(i, r) = Y(r, i) for r <= i
 	double *xblk = X + (size_t)k0 * ld + k0;
 	if (i < nn) {
@@ -762,8 +799,8 @@ __global__ void __launch_bounds__(256) dnode_pair_kernel(const double *W, long l
 {
 	extern __shared__ double nodeLds[];
 	double *Xs = nodeLds, *As = Xs + kNodeBlock, *Ls = As + kNodeBlock, *Ts = Ls + kNodeBlock; // X11 / X22, A21 / L21 L21^T, L21, T2
-	__shared__ double Lcol[2 * kDLeaf], Ycol[2 * kDLeaf];
-	const int tid = threadIdx.x, i = tid & 63, q = tid >> 6, lane = tid & 63, wave = tid >> 6;
+	__shared__ double Lcol[8 * kDLeaf];
+	const int tid = threadIdx.x, i = tid & 63, q = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, wave = tid >> 6;
 	const int r1 = r0 + kDLeaf;
 	double w[16], y[16];
 	// A21(i, k) = W(r1 + i, r0 + k): on its way while the first leaf runs
@@ -781,7 +818,7 @@ __global__ void __launch_bounds__(256) dnode_pair_kernel(const double *W, long l
 			w[t] = v;
 			y[t] = (i == c) ? 1.0 : 0.0;
 		}
-		dleaf_steps<0>(w, y, Lcol, Ycol, i, q, k0, info);
+		dleaf_run(w, y, Lcol, i, q, k0, info);
 		// X(i, r) = Y(r, i) for r <= i: to memory, and the whole block (zeros above the diagonal) to LDS
 		double *xblk = X + (size_t)k0 * ld + k0;
 #pragma unroll
