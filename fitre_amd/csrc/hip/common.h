@@ -1,6 +1,7 @@
 // Shared plumbing of the gfx950 device layer: status reporting, the launch
 // stream, per-class launch accounting, wave64 reductions and fast division.
 #pragma once
+#include <float.h>
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stdio.h>
@@ -169,6 +170,57 @@ __device__ __forceinline__ void act_derivatives(int actFun, float zi, float zo, 
 	default: f1 = 1.f, f2 = 0.f; break;
 	}
 }
+
+// f'(x) alone, in the form the pooling / activation kernels multiply a gradient by
+__device__ __forceinline__ float act_derivative(int actFun, float zi, float zo)
+{
+	switch (actFun) {
+	case ACT_LOGISTIC: return zo * (1.f - zo);
+	case ACT_TANH: return (1.f + zo) * (1.f - zo);
+	case CNN_ACT_SOFTPLUS: return 1.f / (1.f + expf(-zi));
+	case CNN_ACT_SWISH: {
+		float t = 1.f / (1.f + expf(-zi));
+		return zo + t * (1.f - zo);
+	}
+	case CNN_ACT_RELU: return zo > 0.f ? 1.f : 0.f;
+	case CNN_ACT_ELU: return zo < 0.f ? zo + 1.f : 1.f;
+	default: return 1.f;
+	}
+}
+
+// strict-> scan of four values in order, starting below every finite float
+__device__ __forceinline__ int scan2x2(float v0, float v1, float v2, float v3)
+{
+	float best = -FLT_MAX;
+	int arg = -1;
+	if (v0 > best) { best = v0; arg = 0; }
+	if (v1 > best) { best = v1; arg = 1; }
+	if (v2 > best) { best = v2; arg = 2; }
+	if (v3 > best) { best = v3; arg = 3; }
+	return arg;
+}
+
+static inline bool act_known(int actFun)
+{
+	switch (actFun) {
+	case ACT_LOGISTIC:
+	case ACT_TANH:
+	case ACT_LINEAR:
+	case CNN_ACT_NONE:
+	case CNN_ACT_SOFTPLUS:
+	case CNN_ACT_ELU:
+	case CNN_ACT_RELU:
+	case CNN_ACT_SWISH: return true;
+	default: return false;
+	}
+}
+static inline bool act_needs_zin(int actFun) { return actFun == CNN_ACT_SOFTPLUS || actFun == CNN_ACT_SWISH; }
+static inline bool act_needs_zout(int actFun)
+{
+	return actFun == ACT_LOGISTIC || actFun == ACT_TANH || actFun == CNN_ACT_SWISH || actFun == CNN_ACT_RELU ||
+	       actFun == CNN_ACT_ELU;
+}
+
 
 // ---- per-class launch accounting ------------------------------------------
 // A LaunchScope brackets the launches made while it is alive with two events

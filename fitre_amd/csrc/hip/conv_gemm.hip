@@ -685,6 +685,42 @@ int fitre_hip_conv_input_grad(const fitre_conv_shape *s, const float *delta, con
 	return launch_gemm<FlipWeightKContig, PatchRowContig>(pa, pb, out, I, J, R, plan, ws, wsBytes, FITRE_KC_CONV_DX, conv_flops(s));
 }
 
+// ---- the input gradient taken on through the 2 x 2 max pool and the activation of the layer below ------------------
+static bool input_grad_takes_thin(const fitre_conv_shape *s)
+{
+	return s->stride == 1 && s->padding < s->ksize && !quad_eligible(s) && !c3_pos_eligible(s, true) && thin_dx_eligible(s);
+}
+
+int fitre_hip_conv_input_grad_folds_pool(const fitre_conv_shape *s)
+{
+	if (!s || s->samples <= 0 || s->inChannels <= 0 || s->outChannels <= 0 || s->inA <= 0 || s->inB <= 0 || s->ksize <= 0 || s->stride != 1 ||
+	    s->padding < 0 || s->outA != s->inA + 2 * s->padding - s->ksize + 1 || s->outB != s->inB + 2 * s->padding - s->ksize + 1 || s->outA <= 0 ||
+	    s->outB <= 0)
+		return 0;
+	return (input_grad_takes_thin(s) && thin_dx_fold_eligible(s)) ? 1 : 0;
+}
+
+int fitre_hip_conv_input_grad_pool_act(const fitre_conv_shape *s, const float *delta, const float *w, float *dx, int actFun, const float *z_in,
+                                       const float *z_act, float *dxPool, float *dxAct, void *ws, size_t wsBytes)
+{
+	FITRE_NEED_INIT();
+	int rc = check_conv("fitre_hip_conv_input_grad_pool_act", s);
+	if (rc) return rc;
+	FITRE_REQUIRE(delta && w && dx && z_act && dxAct, "fitre_hip_conv_input_grad_pool_act: null pointer");
+	FITRE_REQUIRE(act_known(actFun), "fitre_hip_conv_input_grad_pool_act: unknown activation code %d", actFun);
+	FITRE_REQUIRE(!act_needs_zin(actFun) || z_in, "fitre_hip_conv_input_grad_pool_act: activation %d needs z_in", actFun);
+	const bool aligned = ((((uintptr_t)z_act) | ((uintptr_t)dxAct) | ((uintptr_t)dxPool) | ((uintptr_t)(act_needs_zin(actFun) ? z_in : nullptr))) & 15) == 0;
+	if (fitre_hip_conv_input_grad_folds_pool(s) && aligned) {
+		const ThinPoolFold fold{ act_needs_zin(actFun) ? z_in : nullptr, z_act, dxPool, dxAct, actFun };
+		return launch_thin_dx(s, delta, w, dx, &fold);
+	}
+	// any other shape: the two steps one after the other
+	rc = fitre_hip_conv_input_grad(s, delta, w, dx, ws, wsBytes);
+	if (rc) return rc;
+	return fitre_hip_pool_act_backward(MAX_POOL, actFun, dx, z_in, z_act, s->inChannels, s->samples, 2 * s->inA, 2 * s->inB, 2, 2, 0, s->inA, s->inB,
+	                                   dxPool, dxAct);
+}
+
 // ---- sums of two products of one shape (the R operator's pairs) ---------------------------------------------------
 int fitre_hip_conv_pair_supported(const fitre_conv_shape *s, int kind)
 {
@@ -961,8 +997,42 @@ size_t fitre_hip_fc_tail_workspace(int layers, const fitre_fc_tail_layer *l, int
 	return total;
 }
 
+struct TailFold {
+	int act;
+	const float *zIn, *zAct;
+	float *dxPool, *dxAct;
+};
+static int fc_tail_run(int layers, const fitre_fc_tail_layer *l, int n, const float *delta, int extA, int extB, float *features, void *ws,
+                       size_t wsBytes, const TailFold *fold);
+
 int fitre_hip_fc_tail_backward(int layers, const fitre_fc_tail_layer *l, int n, const float *delta, int extA, int extB, float *features,
                                void *ws, size_t wsBytes)
+{
+	return fc_tail_run(layers, l, n, delta, extA, extB, features, ws, wsBytes, nullptr);
+}
+
+int fitre_hip_fc_tail_backward_pool_act(int layers, const fitre_fc_tail_layer *l, int n, const float *delta, int extA, int extB, float *features,
+                                        int actFun, const float *z_in, const float *z_act, float *dxPool, float *dxAct, void *ws, size_t wsBytes)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(extA > 0 && extB > 0, "fitre_hip_fc_tail_backward_pool_act: the lowest layer's inputs must be %d x %d maps", extA, extB);
+	FITRE_REQUIRE(z_act && dxAct, "fitre_hip_fc_tail_backward_pool_act: null pointer");
+	FITRE_REQUIRE(act_known(actFun), "fitre_hip_fc_tail_backward_pool_act: unknown activation code %d", actFun);
+	FITRE_REQUIRE(!act_needs_zin(actFun) || z_in, "fitre_hip_fc_tail_backward_pool_act: activation %d needs z_in", actFun);
+	const float *zi = act_needs_zin(actFun) ? z_in : nullptr;
+	if (((((uintptr_t)z_act) | ((uintptr_t)dxAct) | ((uintptr_t)dxPool) | ((uintptr_t)zi)) & 7) == 0) {
+		const TailFold fold{ actFun, zi, z_act, dxPool, dxAct };
+		return fc_tail_run(layers, l, n, delta, extA, extB, features, ws, wsBytes, &fold);
+	}
+	int rc = fc_tail_run(layers, l, n, delta, extA, extB, features, ws, wsBytes, nullptr);
+	if (rc) return rc;
+	FITRE_REQUIRE(l[0].in % (extA * extB) == 0, "fitre_hip_fc_tail_backward_pool_act: %d inputs are not whole maps", l[0].in);
+	return fitre_hip_pool_act_backward(MAX_POOL, actFun, features, z_in, z_act, l[0].in / (extA * extB), n, 2 * extA, 2 * extB, 2, 2, 0, extA, extB,
+	                                   dxPool, dxAct);
+}
+
+static int fc_tail_run(int layers, const fitre_fc_tail_layer *l, int n, const float *delta, int extA, int extB, float *features, void *ws,
+                       size_t wsBytes, const TailFold *fold)
 {
 	FITRE_NEED_INIT();
 	FITRE_REQUIRE(fitre_hip_fc_tail_fits(layers, l, n), "fitre_hip_fc_tail_backward: the layers do not fit (at most %d layers of at most %d units)",
@@ -979,6 +1049,18 @@ int fitre_hip_fc_tail_backward(int layers, const fitre_fc_tail_layer *l, int n, 
 	p.layers = layers, p.n = n, p.ns = tail_samples(n);
 	p.extA = permute ? extA : 0, p.extB = permute ? extB : 0;
 	p.delta = delta, p.features = features;
+	p.foldAct = -2;
+	if (fold) {
+		p.foldAct = (fold->act == CNN_ACT_NONE || fold->act == ACT_LINEAR || fold->act < 0) ? -1 : fold->act;
+		p.foldZIn = fold->zIn, p.foldZAct = fold->zAct, p.foldDxPool = fold->dxPool, p.foldDxAct = fold->dxAct;
+		// which of its kernels fitre_hip_pool_act_backward would take for these maps: the one for rows of whole 16-byte
+		// groups stores the gradient, the others add it to zero
+		p.foldDirect = ((2 * extB) % 4 == 0 &&
+		                ((((uintptr_t)fold->zAct) | ((uintptr_t)fold->dxAct) | ((uintptr_t)fold->dxPool) | ((uintptr_t)fold->zIn)) & 15) == 0 &&
+		                (((uintptr_t)features) & 7) == 0)
+		                   ? 1
+		                   : 0;
+	}
 	int maxDim = 1, upperLds = 0;
 	double chainFlops = 0.0;
 	for (int f = 0; f < layers; f++) {

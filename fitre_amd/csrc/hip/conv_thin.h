@@ -49,9 +49,24 @@ struct ThinConvParams {
 constexpr int kThinDxCells = 4; // cells of a row per thread
 __host__ __device__ inline int thin_dx_row_words(int inB, int ks) { return (((inB + 3) & ~3) + ks - 1 + 3) & ~3; }
 
-template <int KS>
+//
+// FOLD: the layer below ends in a 2 x 2 / stride 2 max pool (no padding) behind an activation, and this gradient is taken
+// on through both in the same launch (functions/cnn_backward.cu:560-640 does them as steps of their own): a thread's four
+// cells are four windows of the map below, two rows of eight cells, which it routes and scales exactly as
+// maxpool2_backward_kernel does -- the first largest cell of a window in memory order takes the gradient, then times
+// f'(.).  inB is even, so a pair of windows is one 16-byte group of each row.
+struct ThinPoolFold {
+	const float *zIn;  // the activation's input where its derivative needs it, else null
+	const float *zAct; // the activation's output = the pool's input, [Cin][N][2 inA][2 inB]
+	float *dxPool;     // gradient at the pool's input, or null
+	float *dxAct;      // gradient at the activation's input
+	int actFun;
+};
+
+template <int KS, bool FOLD>
 __global__ void __launch_bounds__(256)
-thin_input_grad_kernel(const ThinConvParams p, const float *__restrict__ w, const float *__restrict__ delta, float *__restrict__ dx)
+thin_input_grad_kernel(const ThinConvParams p, const float *__restrict__ w, const float *__restrict__ delta, float *__restrict__ dx,
+                       const ThinPoolFold fold)
 {
 	extern __shared__ __align__(16) float thin_lds[];
 	const int tid = threadIdx.x;
@@ -99,6 +114,21 @@ thin_input_grad_kernel(const ThinConvParams p, const float *__restrict__ w, cons
 		// delta[a - ta + p][b - tb + p] is the bordered cell [a + (k - 1 - ta)][b + (k - 1 - tb)]
 		const float *d0 = thin_lds + (int)a * PB + b0;
 		const float *wci = w + (size_t)ci * taps;
+		// the map below, on its way while the sums run
+		const int bigB = 2 * p.inB;
+		const size_t below = ((size_t)ci * p.samples + n) * (size_t)(4 * cells) + (size_t)(2 * (int)a) * bigB + 2 * b0;
+		float4 zo[2][2], zi[2][2];
+		if constexpr (FOLD) {
+#pragma unroll
+			for (int h = 0; h < 2; h++)
+#pragma unroll
+				for (int r = 0; r < 2; r++) {
+					zo[h][r] = make_float4(0.f, 0.f, 0.f, 0.f);
+					if (live && b0 + 2 * h < p.inB) zo[h][r] = *reinterpret_cast<const float4 *>(fold.zAct + below + (size_t)r * bigB + 4 * h);
+					zi[h][r] = zo[h][r];
+					if (fold.zIn && live && b0 + 2 * h < p.inB) zi[h][r] = *reinterpret_cast<const float4 *>(fold.zIn + below + (size_t)r * bigB + 4 * h);
+				}
+		}
 		float acc[kThinDxCells] = { 0.f, 0.f, 0.f, 0.f };
 		for (int co = 0; co < p.cout; co++) {
 			const float *wk = wci + (size_t)co * p.cin * taps;
@@ -136,6 +166,40 @@ thin_input_grad_kernel(const ThinConvParams p, const float *__restrict__ w, cons
 #pragma unroll
 			for (int jj = 0; jj < kThinDxCells; jj++)
 				if (b0 + jj < p.inB) out[jj] = acc[jj];
+			if constexpr (FOLD) {
+#pragma unroll
+				for (int h = 0; h < 2; h++) {
+					if (b0 + 2 * h >= p.inB) continue;
+					const float4 r0 = zo[h][0], r1 = zo[h][1];
+					float4 g0 = make_float4(0.f, 0.f, 0.f, 0.f), g1 = g0;
+					int arg = scan2x2(r0.x, r0.y, r1.x, r1.y);
+					if (arg == 0) g0.x = acc[2 * h];
+					else if (arg == 1) g0.y = acc[2 * h];
+					else if (arg == 2) g1.x = acc[2 * h];
+					else if (arg == 3) g1.y = acc[2 * h];
+					arg = scan2x2(r0.z, r0.w, r1.z, r1.w);
+					if (arg == 0) g0.z = acc[2 * h + 1];
+					else if (arg == 1) g0.w = acc[2 * h + 1];
+					else if (arg == 2) g1.z = acc[2 * h + 1];
+					else if (arg == 3) g1.w = acc[2 * h + 1];
+					const size_t at = below + 4 * h;
+					if (fold.dxPool) {
+						*reinterpret_cast<float4 *>(fold.dxPool + at) = g0;
+						*reinterpret_cast<float4 *>(fold.dxPool + at + bigB) = g1;
+					}
+					const float4 i0 = zi[h][0], i1 = zi[h][1];
+					g0.x *= act_derivative(fold.actFun, i0.x, r0.x);
+					g0.y *= act_derivative(fold.actFun, i0.y, r0.y);
+					g0.z *= act_derivative(fold.actFun, i0.z, r0.z);
+					g0.w *= act_derivative(fold.actFun, i0.w, r0.w);
+					g1.x *= act_derivative(fold.actFun, i1.x, r1.x);
+					g1.y *= act_derivative(fold.actFun, i1.y, r1.y);
+					g1.z *= act_derivative(fold.actFun, i1.z, r1.z);
+					g1.w *= act_derivative(fold.actFun, i1.w, r1.w);
+					*reinterpret_cast<float4 *>(fold.dxAct + at) = g0;
+					*reinterpret_cast<float4 *>(fold.dxAct + at + bigB) = g1;
+				}
+			}
 		}
 	}
 }
@@ -338,7 +402,9 @@ static inline bool thin_dx_eligible(const fitre_conv_shape *s)
 	return s->stride == 1 && s->padding <= s->ksize - 1 && s->inChannels <= kThinMaxChannels && s->outChannels <= 32 &&
 	       s->ksize <= 7 && s->inChannels * s->outChannels <= 256 && thin_dx_lds_floats(s) <= kThinDxLdsFloats;
 }
-static int launch_thin_dx(const fitre_conv_shape *s, const float *delta, const float *w, float *dx)
+// the pool / activation fold on top: whole 16-byte groups of the map below
+static inline bool thin_dx_fold_eligible(const fitre_conv_shape *s) { return thin_dx_eligible(s) && s->inB % 2 == 0; }
+static int launch_thin_dx(const fitre_conv_shape *s, const float *delta, const float *w, float *dx, const ThinPoolFold *fold = nullptr)
 {
 	ThinConvParams p = thin_params(s);
 	// enough workgroups for two per compute unit where the batch alone does not give them
@@ -350,9 +416,16 @@ static int launch_thin_dx(const fitre_conv_shape *s, const float *delta, const f
 	const dim3 grid((unsigned)s->samples, (unsigned)groupsY);
 	const size_t lds = sizeof(float) * (size_t)thin_dx_lds_floats(s);
 	LaunchScope scope(FITRE_KC_CONV_DX, conv_flops(s), 0);
-	if (s->ksize == 5) thin_input_grad_kernel<5><<<grid, 256, lds, stream()>>>(p, w, delta, dx);
-	else if (s->ksize == 3) thin_input_grad_kernel<3><<<grid, 256, lds, stream()>>>(p, w, delta, dx);
-	else thin_input_grad_kernel<0><<<grid, 256, lds, stream()>>>(p, w, delta, dx);
+	if (fold) {
+		if (s->ksize == 5) thin_input_grad_kernel<5, true><<<grid, 256, lds, stream()>>>(p, w, delta, dx, *fold);
+		else if (s->ksize == 3) thin_input_grad_kernel<3, true><<<grid, 256, lds, stream()>>>(p, w, delta, dx, *fold);
+		else thin_input_grad_kernel<0, true><<<grid, 256, lds, stream()>>>(p, w, delta, dx, *fold);
+	} else {
+		const ThinPoolFold none{};
+		if (s->ksize == 5) thin_input_grad_kernel<5, false><<<grid, 256, lds, stream()>>>(p, w, delta, dx, none);
+		else if (s->ksize == 3) thin_input_grad_kernel<3, false><<<grid, 256, lds, stream()>>>(p, w, delta, dx, none);
+		else thin_input_grad_kernel<0, false><<<grid, 256, lds, stream()>>>(p, w, delta, dx, none);
+	}
 	return check_launch("thin_input_grad_kernel");
 }
 

@@ -135,21 +135,6 @@ __device__ __forceinline__ float pool_gather(const float *dmap, const float *zma
 	return acc;
 }
 
-__device__ __forceinline__ float act_derivative(int actFun, float zi, float zo)
-{
-	switch (actFun) {
-	case ACT_LOGISTIC: return zo * (1.f - zo);
-	case ACT_TANH: return (1.f + zo) * (1.f - zo);
-	case CNN_ACT_SOFTPLUS: return 1.f / (1.f + expf(-zi));
-	case CNN_ACT_SWISH: {
-		float t = 1.f / (1.f + expf(-zi));
-		return zo + t * (1.f - zo);
-	}
-	case CNN_ACT_RELU: return zo > 0.f ? 1.f : 0.f;
-	case CNN_ACT_ELU: return zo < 0.f ? zo + 1.f : 1.f;
-	default: return 1.f;
-	}
-}
 
 // One thread per input cell.  POOL: 0 max, 1 average, 2 none.  FUSE_ACT: also
 // write dxAct = gradient * f'(.).
@@ -477,17 +462,6 @@ static int maps_per_group(int cells, int windows, long maps)
 	return (int)(fit < 1 ? 1 : fit);
 }
 
-// strict-> scan of four values in order, starting below every finite float
-__device__ __forceinline__ int scan2x2(float v0, float v1, float v2, float v3)
-{
-	float best = -FLT_MAX;
-	int arg = -1;
-	if (v0 > best) { best = v0; arg = 0; }
-	if (v1 > best) { best = v1; arg = 1; }
-	if (v2 > best) { best = v2; arg = 2; }
-	if (v3 > best) { best = v3; arg = 3; }
-	return arg;
-}
 
 // pool_routed_kernel for 2x2 / stride 2 / no padding windows on maps with B % 4 == 0 and A even: one thread per pair of
 // pooled cells adjacent along B, i.e. a 2 x 4 patch of z and of the values, moved with 16-byte accesses.
@@ -566,27 +540,6 @@ maxpool2_backward_kernel(const float *delta, const float *z_in, const float *z_a
 			*reinterpret_cast<float4 *>(dxAct + inOff + inB) = g1;
 		}
 	}
-}
-
-static bool act_known(int actFun)
-{
-	switch (actFun) {
-	case ACT_LOGISTIC:
-	case ACT_TANH:
-	case ACT_LINEAR:
-	case CNN_ACT_NONE:
-	case CNN_ACT_SOFTPLUS:
-	case CNN_ACT_ELU:
-	case CNN_ACT_RELU:
-	case CNN_ACT_SWISH: return true;
-	default: return false;
-	}
-}
-static bool act_needs_zin(int actFun) { return actFun == CNN_ACT_SOFTPLUS || actFun == CNN_ACT_SWISH; }
-static bool act_needs_zout(int actFun)
-{
-	return actFun == ACT_LOGISTIC || actFun == ACT_TANH || actFun == CNN_ACT_SWISH || actFun == CNN_ACT_RELU ||
-	       actFun == CNN_ACT_ELU;
 }
 
 static int check_pool_shape(const char *fn, int channels, int samples, int inA, int inB, int ksize, int stride,

@@ -43,6 +43,13 @@ struct FcTailParams {
 	int maxDim;
 	int partInputs; // inputs of the lowest layer per blockIdx.y
 	int lowBase;    // where the lowest layer's part sits in LDS
+	// foldAct >= -1: the maps below end in an activation (-1: none) and a 2 x 2 / stride 2 max pool whose output the lowest
+	// layer reads; its input gradient then goes on through both, exactly as maxpool_map_backward_kernel takes it (the first
+	// largest cell of a window in memory order gets the gradient, then times f'(.)); foldAct == -2: no fold
+	int foldAct;
+	int foldDirect; // the gradient is stored as it is (else as 0 + gradient, the sum over the windows a cell is the maximum of)
+	const float *foldZIn, *foldZAct; // [C][n][2 extA][2 extB]; foldZIn null where the derivative does not need it
+	float *foldDxPool, *foldDxAct;   // foldDxPool may be null
 };
 
 __device__ __forceinline__ int tail_div(int e, int out, unsigned magic) { return out == 1 ? e : (int)__umulhi((unsigned)e, magic); }
@@ -125,6 +132,29 @@ __global__ void __launch_bounds__(kTailThreads) fc_tail_chain_kernel(const FcTai
 				const int c = i / planeAB, r = i - c * planeAB;
 				const int b = r / p.extA, a = r - b * p.extA;
 				p.features[(((long)c * p.n + (s0 + s)) * p.extA + a) * p.extB + b] = acc;
+				if (p.foldAct != -2) {
+					const int bigB = 2 * p.extB;
+					const long at0 = (((long)c * p.n + (s0 + s)) * (2 * p.extA) + 2 * a) * bigB + 2 * b;
+					const float2 r0 = *reinterpret_cast<const float2 *>(p.foldZAct + at0);
+					const float2 r1 = *reinterpret_cast<const float2 *>(p.foldZAct + at0 + bigB);
+					float2 i0 = r0, i1 = r1;
+					if (p.foldZIn) {
+						i0 = *reinterpret_cast<const float2 *>(p.foldZIn + at0);
+						i1 = *reinterpret_cast<const float2 *>(p.foldZIn + at0 + bigB);
+					}
+					const int arg = scan2x2(r0.x, r0.y, r1.x, r1.y);
+					const float g = p.foldDirect ? acc : 0.f + acc;
+					float2 g0 = make_float2(arg == 0 ? g : 0.f, arg == 1 ? g : 0.f), g1 = make_float2(arg == 2 ? g : 0.f, arg == 3 ? g : 0.f);
+					if (p.foldDxPool) {
+						*reinterpret_cast<float2 *>(p.foldDxPool + at0) = g0;
+						*reinterpret_cast<float2 *>(p.foldDxPool + at0 + bigB) = g1;
+					}
+					const int fa = p.foldAct < 0 ? CNN_ACT_NONE : p.foldAct;
+					g0.x *= act_derivative(fa, i0.x, r0.x), g0.y *= act_derivative(fa, i0.y, r0.y);
+					g1.x *= act_derivative(fa, i1.x, r1.x), g1.y *= act_derivative(fa, i1.y, r1.y);
+					*reinterpret_cast<float2 *>(p.foldDxAct + at0) = g0;
+					*reinterpret_cast<float2 *>(p.foldDxAct + at0 + bigB) = g1;
+				}
 			} else {
 				p.features[at] = acc;
 			}

@@ -363,6 +363,7 @@ void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, 
 	feature_extent(model, &extA, &extB);
 	fitre_fc_tail_layer tail[4];
 	const int fusedTail = tail_shapes(model, n, tail);
+	int tailFoldedPool = 0;
 	if (fusedTail) {
 		/* small layers (LeNet's 400-120-84-10): the whole tail in two launches on the chain's lane -- every delta into its
 		 * slot, every weight and bias gradient, and the first convolution-side delta */
@@ -376,7 +377,19 @@ void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, 
 			tail[f].dW = gradient + wOffsets[f + nc];
 			tail[f].db = (model->bias != 0) ? gradient + bOffsets[f + nc] : NULL;
 		}
-		HIP_CALL(fitre_hip_fc_tail_backward(model->lLayers, tail, n, delta, extA, extB, features, sideWs, sideBytes));
+		const POOL_LAYER *pl = &model->poolLayer[nc - 1];
+		if (!has_bn(last) && pl->type == MAX_POOL && pl->pSize == 2 && pl->stride == 2 && pl->padding == 0 && pl->width == 2 * extA &&
+		    pl->height == 2 * extB && pl->outWidth == extA && pl->outHeight == extB) {
+			/* the top convolution layer's pool and activation steps ride on the launch that produces their delta */
+			const real *slabT = z + zOffsets[nc];
+			real *dslabT = dx + zOffsets[nc];
+			HIP_CALL(fitre_hip_fc_tail_backward_pool_act(model->lLayers, tail, n, delta, extA, extB, features, model->actFuns[nc - 1], slabT,
+			                                             slabT + last->activationOffset, dslabT, dslabT + last->activationOffset, sideWs,
+			                                             sideBytes));
+			tailFoldedPool = 1;
+		} else {
+			HIP_CALL(fitre_hip_fc_tail_backward(model->lLayers, tail, n, delta, extA, extB, features, sideWs, sideBytes));
+		}
 	}
 	for (int f = fusedTail ? -1 : model->lLayers - 1; f >= 0; f--) {
 		const FC_LAYER *l = &model->fcLayer[f];
@@ -420,6 +433,7 @@ void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, 
 	/* delta as the layer above left it: a plain tensor, or the unsummed split partials of its input
 	 * gradient (summed by the pool / activation pass below while it reads them) */
 	fitre_split_view dview = { features, 1, 0 };
+	int poolFolded = tailFoldedPool;
 	for (int c = nc - 1; c >= 0; c--) {
 		const CONV_LAYER *l = &model->convLayer[c];
 		const POOL_LAYER *p = &model->poolLayer[c];
@@ -444,7 +458,11 @@ void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, 
 			actOut = delta_new;
 		}
 		const real *cur;
-		if (has_bn(l)) {
+		if (poolFolded) {
+			/* the layer above's input gradient went on through this layer's pool and activation in its own launch */
+			poolFolded = 0;
+			cur = dslab + l->activationOffset;
+		} else if (has_bn(l)) {
 			/* pool backward -> dx slab + 0; times f'(.) -> dx slab + activationOffset; batch-norm backward ->
 			 * dx slab + batchNormOffset, its column sums being the bias gradient */
 			HIP_CALL(fitre_hip_pool_act_bn_backward(p->type, act, dview.base, dview.splits, dview.stride, actIn,
@@ -478,7 +496,20 @@ void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, 
 				HIP_CALL(fitre_hip_conv_input_grad_split_prepared(&shape, cur, weights + wOffsets[c], prepared[c], delta, ws, wsBytes,
 				                                                  &dview));
 			} else {
-				HIP_CALL(fitre_hip_conv_input_grad(&shape, cur, weights + wOffsets[c], delta, ws, wsBytes));
+				const CONV_LAYER *lb = &model->convLayer[c - 1];
+				const POOL_LAYER *pb = &model->poolLayer[c - 1];
+				if (pb->type == MAX_POOL && pb->pSize == 2 && pb->stride == 2 && pb->padding == 0 && pb->width == 2 * shape.inA &&
+				    pb->height == 2 * shape.inB && pb->outWidth == shape.inA && pb->outHeight == shape.inB &&
+				    fitre_hip_conv_input_grad_folds_pool(&shape)) {
+					const real *slabB = z + zOffsets[c];
+					real *dslabB = dx + zOffsets[c];
+					HIP_CALL(fitre_hip_conv_input_grad_pool_act(&shape, cur, weights + wOffsets[c], delta, model->actFuns[c - 1], slabB,
+					                                            slabB + lb->activationOffset, dslabB, dslabB + lb->activationOffset, ws,
+					                                            wsBytes));
+					poolFolded = 1;
+				} else {
+					HIP_CALL(fitre_hip_conv_input_grad(&shape, cur, weights + wOffsets[c], delta, ws, wsBytes));
+				}
 				dview.base = delta, dview.splits = 1, dview.stride = 0;
 			}
 		}

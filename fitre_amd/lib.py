@@ -116,6 +116,8 @@ HIP_API = {
     "fitre_hip_conv_weight_bias_grad": (i32, [pshape, vp, vp, vp, vp, vp, sz]),
     "fitre_hip_conv_input_grad_workspace": (sz, [pshape]),
     "fitre_hip_conv_input_grad": (i32, [pshape, vp, vp, vp, vp, sz]),
+    "fitre_hip_conv_input_grad_folds_pool": (i32, [pshape]),
+    "fitre_hip_conv_input_grad_pool_act": (i32, [pshape, vp, vp, vp, i32, vp, vp, vp, vp, vp, sz]),
     "fitre_hip_gemm_workspace": (sz, [i32, i32, i32]),
     "fitre_hip_gemm": (i32, [i32, i32, i32, i32, i32, f32, vp, i32, vp, i32, f32, vp, i32, vp, vp, sz]),
     "fitre_hip_linear_is_small": (i32, [i32, i32, i32]),
@@ -125,6 +127,7 @@ HIP_API = {
     "fitre_hip_fc_tail_fits": (i32, [i32, vp, i32]),
     "fitre_hip_fc_tail_workspace": (sz, [i32, vp, i32]),
     "fitre_hip_fc_tail_backward": (i32, [i32, vp, i32, vp, i32, i32, vp, vp, sz]),
+    "fitre_hip_fc_tail_backward_pool_act": (i32, [i32, vp, i32, vp, i32, i32, vp, i32, vp, vp, vp, vp, vp, sz]),
     "fitre_hip_lane_select": (i32, [i32]),
     "fitre_hip_lane_wait": (i32, [i32, i32]),
     "fitre_hip_lanes_enable": (i32, [i32]),

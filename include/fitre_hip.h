@@ -347,6 +347,16 @@ int fitre_hip_conv_weight_bias_grad(const fitre_conv_shape *s, const float *x, c
 size_t fitre_hip_conv_input_grad_workspace(const fitre_conv_shape *s);
 int fitre_hip_conv_input_grad(const fitre_conv_shape *s, const float *delta, const float *w, float *dx,
                               void *ws, size_t wsBytes);
+/* The same, taken on through the layer below where that ends in an activation and a 2 x 2 / stride 2 max pool without
+ * padding (its maps are 2 inA x 2 inB): dx as above, dxPool (may be NULL) and dxAct as fitre_hip_pool_act_backward(MAX_POOL,
+ * actFun, dx, z_in, z_act, Cin, N, 2 inA, 2 inB, 2, 2, 0, inA, inB, dxPool, dxAct) leaves them, the same bits.  One
+ * launch where fitre_hip_conv_input_grad_folds_pool says 1 (few channels, inB even) and the tensors are 16-byte aligned,
+ * else the two steps one after the other.  functions/cnn_backward.cu:560-640 runs the pool and activation steps of a
+ * layer as launches of their own behind the convolution step of the layer above. */
+int fitre_hip_conv_input_grad_folds_pool(const fitre_conv_shape *s);
+int fitre_hip_conv_input_grad_pool_act(const fitre_conv_shape *s, const float *delta, const float *w, float *dx, int actFun,
+                                       const float *z_in, const float *z_act, float *dxPool, float *dxAct, void *ws,
+                                       size_t wsBytes);
 /* Sums of two products of one shape in one launch, for the R operator of the Hessian-vector product
  * (functions/cnn_hv_forward.cu, cnn_hv_backward.cu: every convolution there is a sum of two):
  *   forward_pair:      y  = conv(x1, w1) + conv(x2, w2) + bias
@@ -445,6 +455,13 @@ int fitre_hip_fc_tail_fits(int layers, const fitre_fc_tail_layer *l, int n);
 size_t fitre_hip_fc_tail_workspace(int layers, const fitre_fc_tail_layer *l, int n);
 int fitre_hip_fc_tail_backward(int layers, const fitre_fc_tail_layer *l, int n, const float *delta, int extA, int extB,
                                float *features, void *ws, size_t wsBytes);
+/* The same where the lowest layer reads the output of a 2 x 2 / stride 2 max pool (no padding) behind an activation:
+ * features as above, then dxPool (may be NULL) and dxAct as fitre_hip_pool_act_backward(MAX_POOL, actFun, features, z_in,
+ * z_act, C, n, 2 extA, 2 extB, 2, 2, 0, extA, extB, dxPool, dxAct) leaves them, the same bits, from the launch that
+ * writes features when the four tensors are 8-byte aligned.  extA, extB > 0. */
+int fitre_hip_fc_tail_backward_pool_act(int layers, const fitre_fc_tail_layer *l, int n, const float *delta, int extA,
+                                        int extB, float *features, int actFun, const float *z_in, const float *z_act,
+                                        float *dxPool, float *dxAct, void *ws, size_t wsBytes);
 
 /* ---- Kronecker factors of the KFAC curvature approximation --------------------------------------
  * Each factor is a dense symmetric matrix, written in full (row-major == column-major).  The

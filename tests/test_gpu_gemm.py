@@ -350,3 +350,74 @@ def test_gemm(dev, oracle64, M, N, K, ta, tb):
     assert rel_err(dev.download(pc, ldc * N).reshape(N, ldc)[:, :M], want) < TOL
     for q in (pa, pb, pc, ws):
         dev.free(q)
+
+
+# N, Cin, Cout, A, B, k, pad, whether it is one launch: the input gradient of this layer taken on through the 2 x 2 max pool and the activation of
+# the layer below (maps of 2A x 2B)
+FOLD_CASES = [
+    (2, 6, 16, 14, 14, 5, 0, 1),     # LeNet conv2 above conv1's pool: 14 = three groups of four cells and a half one
+    (3, 4, 8, 6, 10, 5, 2, 1),       # rectangular, padded
+    (3, 4, 8, 6, 10, 3, 1, 0),       # a shape the 3 x 3 kernels take: the two steps one after the other
+    (5, 3, 5, 3, 2, 3, 1, 1),        # a row is half a group
+    (2, 16, 16, 12, 12, 5, 2, 1),    # the most channels the kernel takes
+    (2, 3, 5, 7, 7, 3, 1, 0),        # odd extent: the two steps one after the other
+    (2, 64, 128, 8, 8, 3, 1, 0),     # a layer of the 3 x 3 kernels: likewise
+]
+
+
+@pytest.mark.parametrize("case", FOLD_CASES)
+@pytest.mark.parametrize("act", [1, 3, 6, 0])  # filled in below: codes from fitre_amd.structs
+def test_input_gradient_through_pool_and_activation(dev, case, act):
+    """fitre_hip_conv_input_grad_pool_act against fitre_hip_conv_input_grad followed by
+    fitre_hip_pool_act_backward: dx, dxPool and dxAct bit for bit, also without dxPool."""
+    from fitre_amd.structs import ACT_LOGISTIC, CNN_ACT_NONE, CNN_ACT_RELU, CNN_ACT_SWISH, MAX_POOL
+    act = {1: CNN_ACT_RELU, 3: CNN_ACT_SWISH, 6: ACT_LOGISTIC, 0: CNN_ACT_NONE}[act]
+    N, Cin, Cout, A, B, k, p, one_launch = case
+    shape = conv_shape(N, Cin, Cout, A, B, k, 1, p)
+    rng = np.random.default_rng(sum(case) + 31 * act)
+    w = (rng.standard_normal(Cout * Cin * k * k) / np.sqrt(Cin * k * k)).astype(np.float32)
+    d = rng.standard_normal(Cout * N * shape.outA * shape.outB).astype(np.float32)
+    big = Cin * N * 4 * A * B
+    z_in = rng.standard_normal(big).astype(np.float32)
+    if act == CNN_ACT_RELU:
+        z_act = np.maximum(z_in, 0).astype(np.float32)  # whole windows of equal zeros: the first cell takes the gradient
+    elif act == ACT_LOGISTIC:
+        z_act = (1.0 / (1.0 + np.exp(-z_in.astype(np.float64)))).astype(np.float32)
+    elif act == CNN_ACT_SWISH:
+        z_act = (z_in.astype(np.float64) / (1.0 + np.exp(-z_in.astype(np.float64)))).astype(np.float32)
+    else:
+        z_act = z_in.copy()
+    pw, pd, pzi, pza = dev.upload(w), dev.upload(d), dev.upload(z_in), dev.upload(z_act)
+    nb = hip.fitre_hip_conv_input_grad_workspace(C.byref(shape))
+    ws = dev.alloc(max(nb, 256))
+    small = Cin * N * A * B
+    dx0, pool0, act0 = dev.zeros(small), dev.zeros(big), dev.zeros(big)
+    L.check(hip.fitre_hip_conv_input_grad(C.byref(shape), pd, pw, dx0, ws, nb))
+    L.check(hip.fitre_hip_pool_act_backward(MAX_POOL, act, dx0, pzi, pza, Cin, N, 2 * A, 2 * B, 2, 2, 0, A, B, pool0, act0))
+    want = [dev.download(dx0, small), dev.download(pool0, big), dev.download(act0, big)]
+    folds = hip.fitre_hip_conv_input_grad_folds_pool(C.byref(shape))
+    assert folds == one_launch
+    for with_pool in (True, False):
+        dx1, pool1, act1 = dev.zeros(small), dev.zeros(big), dev.zeros(big)
+        L.check(hip.fitre_hip_conv_input_grad_pool_act(C.byref(shape), pd, pw, dx1, act, pzi, pza, pool1 if with_pool else None, act1, ws, nb))
+        got = [dev.download(dx1, small), dev.download(pool1, big), dev.download(act1, big)]
+        assert np.array_equal(got[0], want[0])
+        assert np.array_equal(got[2], want[2])
+        if with_pool:
+            assert np.array_equal(got[1], want[1])
+        else:
+            assert not got[1].any()
+        for q in (dx1, pool1, act1):
+            dev.free(q)
+    assert want[2].any()
+    for q in (pw, pd, pzi, pza, ws, dx0, pool0, act0):
+        dev.free(q)
+
+
+def test_input_gradient_through_pool_refuses_bad_arguments(dev):
+    shape = conv_shape(2, 6, 16, 14, 14, 5, 1, 0)
+    p = dev.zeros(64)
+    assert hip.fitre_hip_conv_input_grad_pool_act(C.byref(shape), p, p, p, 1, None, None, None, p, None, 0) == 2   # no z_act
+    assert hip.fitre_hip_conv_input_grad_pool_act(C.byref(shape), p, p, p, 12345, None, p, None, p, None, 0) == 2  # unknown activation
+    assert hip.fitre_hip_conv_input_grad_folds_pool(None) == 0
+    dev.free(p)

@@ -247,6 +247,28 @@ def test_tail_of_small_layers_in_two_launches(dev, dims, n, acts, ext, bias):
     feat2 = up(np.zeros(dims[0] * n, np.float32))
     ok(hip.fitre_hip_linear_input_grad(dims[0], dims[1], n, arr[0].W, slots[0], -1, None, None, ext[0], ext[1], feat2, None, None, 0, None))
     np.testing.assert_array_equal(dev.download(feat2, dims[0] * n), feat_bits)
+    if ext[0] > 0:
+        # the input maps as the output of a 2 x 2 max pool behind an activation: the same launch takes the gradient on
+        # through both, with the bits fitre_hip_pool_act_backward leaves
+        from fitre_amd.structs import MAX_POOL
+        a_, b_ = ext
+        c_ = dims[0] // (a_ * b_)
+        big = c_ * n * 4 * a_ * b_
+        for act in (CNN_ACT_RELU, CNN_ACT_SWISH, CNN_ACT_NONE):
+            zi = rng.standard_normal(big).astype(np.float32)
+            za = forward_act(act, zi.astype(np.float64)).astype(np.float32)
+            pzi, pza = up(zi), up(za)
+            pool0, act0, pool1, act1 = (up(np.full(big, np.nan, np.float32)) for _ in range(4))
+            ok(hip.fitre_hip_pool_act_backward(MAX_POOL, act, feat, pzi, pza, c_, n, 2 * a_, 2 * b_, 2, 2, 0, a_, b_, pool0, act0))
+            feat3 = up(np.zeros(dims[0] * n, np.float32))
+            ok(hip.fitre_hip_fc_tail_backward_pool_act(layers, arr, n, ptop, a_, b_, feat3, act, pzi, pza, pool1, act1, ws, nb))
+            np.testing.assert_array_equal(dev.download(feat3, dims[0] * n), feat_bits)
+            np.testing.assert_array_equal(dev.download(pool1, big).view(np.uint32), dev.download(pool0, big).view(np.uint32))
+            np.testing.assert_array_equal(dev.download(act1, big).view(np.uint32), dev.download(act0, big).view(np.uint32))
+            # without the pool's own slot
+            act2 = up(np.full(big, np.nan, np.float32))
+            ok(hip.fitre_hip_fc_tail_backward_pool_act(layers, arr, n, ptop, a_, b_, feat3, act, pzi, pza, None, act2, ws, nb))
+            np.testing.assert_array_equal(dev.download(act2, big).view(np.uint32), dev.download(act0, big).view(np.uint32))
     for p in bufs:
         dev.free(p)
 
@@ -261,6 +283,7 @@ def test_tail_rejects_what_does_not_fit(dev):
     arr[1] = fitre_fc_tail_layer(60, 10, CNN_ACT_NONE, None, None, None, None, None, None, None)   # 60 inputs after 50 outputs
     assert hip.fitre_hip_fc_tail_fits(2, arr, 64) == 0
     assert hip.fitre_hip_fc_tail_backward(2, arr, 64, None, 0, 0, None, None, 0) == 2
+    assert hip.fitre_hip_fc_tail_backward_pool_act(2, arr, 64, None, 0, 0, None, CNN_ACT_RELU, None, None, None, None, None, 0) == 2
     # the layers above the lowest sit in LDS whole: the sum of in * (out + 1) at most 16384 floats
     arr3 = (fitre_fc_tail_layer * 3)()
     for top, fits in ((62, 1), (63, 0)):
