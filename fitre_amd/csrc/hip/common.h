@@ -127,12 +127,15 @@ void conv_gemm_release();
 
 // ---- wave priority of the bandwidth-bound kernels ---------------------------
 // The short memory-bound kernels of the delta chain run beside chip-filling matrix kernels of the other
-// lane.  Measured on the VGG-11 batch-256 backward pass: raising the priority of the memory-bound waves
-// (FITRE_WAVE_PRIORITY=3) makes the pass 3 % slower -- the pass is bound by the matrix pipes, and every issue
-// slot the other kernels win is one the matrix kernels lose -- while raising the matrix kernels' waves
-// (FITRE_MATRIX_WAVE_PRIORITY=2) gains 0.4 %.  Hence the defaults: 0 and 2.
+// lane, on the registers those leave free on every SIMD (the weight-gradient kernels are held to three waves of at
+// most 152 registers for that).  Measured on the VGG-11 batch-256 backward pass: with the memory-bound waves at the
+// top priority (FITRE_WAVE_PRIORITY=3) the pass is 1.5 % shorter than with none -- they issue a few instructions per
+// 16 bytes and then wait for memory, so the matrix waves lose little, and the chain behind them moves on sooner; the
+// matrix kernels' waves at 2 instead of 0 (FITRE_MATRIX_WAVE_PRIORITY) gain 0.4 %.  (While the largest
+// weight-gradient kernel still filled the register file, the memory-bound kernels beside it only ran in its tail,
+// and raising them cost 3 %.)
 #ifndef FITRE_WAVE_PRIORITY
-#define FITRE_WAVE_PRIORITY 0
+#define FITRE_WAVE_PRIORITY 3
 #endif
 #define FITRE_RAISE_WAVE_PRIORITY()                                                                  \
 	do {                                                                                             \

@@ -230,6 +230,9 @@ conv3x3_dw_cell_kernel(const Conv3x3Params p, const float *delta, uint32_t delta
 // opposite corners}, {down, up, up-right}, {left, right, down-left}: 81 / 77 / 84 live pairs on an upper half,
 // 81 / 84 / 77 on a lower one, against 96 steps of the nine-tap kernel.
 // ---------------------------------------------------------------------------------
+#ifndef FITRE_CELL8_CHUNK
+#define FITRE_CELL8_CHUNK 4
+#endif
 constexpr int kCell8Map = 8;
 constexpr int kCell8Half = 32;                 // cells of half a map
 constexpr int kCell8SrcCells = 5 * kCell8Map;  // source cells per image and half
@@ -251,6 +254,9 @@ __device__ __forceinline__ void cell8_dw_steps(const float *aBase, const float *
 			live[j] = sa >= 0 && sa < kCell8Map && sb >= 0 && sb < kCell8Map;
 			src[j] = (sa - (LOWER ? 3 : 0)) * kCell8Map + sb; // word inside the image's five source rows
 		}
+#if FITRE_CELL8_CHUNK > 0
+		if (cell % FITRE_CELL8_CHUNK == 0 && cell > 0) __builtin_amdgcn_sched_barrier(0);
+#endif
 		if (!(live[0] || live[1] || live[2])) continue;
 		const float fa = aBase[cell];
 #pragma unroll
