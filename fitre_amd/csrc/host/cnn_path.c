@@ -256,9 +256,13 @@ real cnnForward(CNN_MODEL *model, DEVICE_DATASET *data, SCRATCH_AREA *scratch, r
 }
 
 /* Multiply-adds of the convolution layers' two gradient products: what decides whether a pass is long enough for
- * the lanes to pay.  Ordering two lanes costs the host two runtime calls per dependency, about as long as a
- * kernel of LeNet at batch 128 runs, so a pass of such kernels is faster queued on one lane (measured: 0.136 ms
- * against 0.167 ms); from about LeNet at batch 1024 on the overlap wins. */
+ * the lanes to pay.  Ordering two lanes costs the host two runtime calls per dependency, a few microseconds each:
+ * a pass of LeNet at batch 128 (1.5e8, kernels of 5 to 17 us) takes the same time either way (0.092 ms) and stays on
+ * one lane; LeNet with batch norm at batch 1024 (1.2e9) takes 0.217 ms on two lanes against 0.227 on one, AlexNet
+ * at batch 64 2.82 against 2.90 ms, VGG-11 with batch norm at batch 256 1.37 against 1.52 ms.  (While the largest
+ * weight-gradient kernels filled the register file, two lanes lost on networks with little pooling / batch-norm
+ * traffic per multiply-add, such as AlexNet, and a second limit kept those on one lane; the kernels of the delta
+ * chain now find room beside every weight gradient and the limit is gone.) */
 static double backward_conv_work(const CNN_MODEL *model, int n)
 {
 	double macs = 0;
@@ -268,29 +272,14 @@ static double backward_conv_work(const CNN_MODEL *model, int n)
 	}
 	return macs;
 }
-/* What the lanes can hide is the chain's bandwidth-bound steps (pooling, activation, batch norm: about 28 bytes per
- * activation with batch norm, 16 without) behind the weight gradients' matrix work.  Where a pass has little of
- * them per multiply-add, two matrix kernels side by side only get in each other's way: AlexNet at batch 64 (about
- * 400 FLOP per such byte) takes 2.94 ms on one lane and 3.04 ms on two, VGG-11 with batch norm at batch 256 (about
- * 140) 1.52 ms against 1.39 ms. */
-static double backward_flop_per_elementwise_byte(const CNN_MODEL *model, int n)
-{
-	double bytes = 0;
-	for (int c = 0; c < model->cLayers; c++) {
-		const CONV_LAYER *l = &model->convLayer[c];
-		bytes += (double)n * l->outHeight * l->outWidth * l->outChannels * (has_bn(l) ? 28.0 : 16.0);
-	}
-	return bytes > 0 ? 2.0 * backward_conv_work(model, n) / bytes : 0.0;
-}
-#define LANE_WORK_THRESHOLD 2.0e9
-#define LANE_INTENSITY_LIMIT 250.0
-/* -1: by the two limits above (fitted on LeNet, VGG-11 and AlexNet); 0: one lane; 1: lanes, whatever the network */
+#define LANE_WORK_THRESHOLD 1.0e9
+/* -1: by the limit above (fitted on LeNet, VGG-11 and AlexNet); 0: one lane; 1: lanes, whatever the network */
 static int g_backward_lanes = -1;
 void fitreSetBackwardLanes(int mode) { g_backward_lanes = mode < 0 ? -1 : (mode ? 1 : 0); }
 int fitreBackwardUsesLanes(CNN_MODEL *model, int batchSize)
 {
 	if (g_backward_lanes >= 0) return g_backward_lanes;
-	return backward_conv_work(model, batchSize) >= LANE_WORK_THRESHOLD && backward_flop_per_elementwise_byte(model, batchSize) < LANE_INTENSITY_LIMIT;
+	return backward_conv_work(model, batchSize) >= LANE_WORK_THRESHOLD;
 }
 #define LANE_SELECT(lane_) do { if (lanes) HIP_CALL(fitre_hip_lane_select(lane_)); } while (0)
 #define LANE_WAIT(waiter_, signaller_) do { if (lanes) HIP_CALL(fitre_hip_lane_wait(waiter_, signaller_)); } while (0)

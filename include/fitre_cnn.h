@@ -95,8 +95,8 @@ void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, 
  * the first offending layer; cnnBackward and cnnHv call it before their first launch and exit(-1) with a message. */
 int fitreBackwardUnsupportedLayer(const CNN_MODEL *model);
 /* cnnBackward queues a pass on one stream or spreads it over the device layer's lanes (weight gradients beside the
- * chain of input gradients); by default it decides from the network's convolution work and its arithmetic per
- * byte of pooling / activation / batch-norm traffic, limits fitted on LeNet, VGG-11 and AlexNet.  mode 0: always one
+ * chain of input gradients); by default it decides from the network's convolution work (one lane below 1e9
+ * multiply-adds per pass, a limit fitted on LeNet, VGG-11 and AlexNet).  mode 0: always one
  * lane, 1: always the lanes, -1: the default rule.  The results do not depend on it, bit for bit.  No counterpart in
  * the reference (one stream).  fitreBackwardUsesLanes: what a pass of this model and batch would do now.
  * Weights, z and delta must be complete on lane 0 when cnnBackward is called; the other lanes order themselves behind it. */

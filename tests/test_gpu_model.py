@@ -246,9 +246,9 @@ def test_vgg11_full_size_one_lane_gives_the_same_bits(vgg_full, dev):
 
 @pytest.mark.parametrize("name", ["lenet_bn_b1024", "alexnet_b64", "vgg11_no_bn_b32"])
 def test_forced_lanes_give_the_same_bits(dev, name):
-    """Networks on the other side of cnnBackward's two lane limits (LeNet + batch norm: too little work; AlexNet: too much
-    arithmetic per elementwise byte; a VGG-11 without batch norm at a small batch in between) and the override
-    fitreSetBackwardLanes: one lane and the lanes give the same gradient and dx, bit for bit."""
+    """Networks on either side of cnnBackward's lane limit and without the batch-norm steps the lanes were built around
+    (LeNet + batch norm at batch 1024: just above it; AlexNet; a VGG-11 without batch norm at a small batch) and the
+    override fitreSetBackwardLanes: one lane and the lanes give the same gradient and dx, bit for bit."""
     from helpers import GpuModel, batch_inputs, build_alexnet, build_lenet, build_vgg11, he_weights
     if name == "lenet_bn_b1024":
         batch, model = 1024, build_lenet(1024, bn=True)
