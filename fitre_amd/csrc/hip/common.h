@@ -94,6 +94,8 @@ int lane();           // its index (0 .. kMaxLanes - 1)
 int lane_compute_units();     // compute units a kernel launched on the selected lane can occupy
 int lane_compute_units_min(); // the smallest such count over the lanes
 int device_compute_units();
+int weight_grad_units();      // compute units the 3 x 3 weight gradients are planned for (fitre_hip_weight_grad_share)
+int share_of_units(int cus, int eighths); // that many eighths of `cus`, in whole groups of eight
 bool ready();
 int current_device();            // the device fitre_hip_init selected, -1 before
 // Per-device set-up of the file that holds the batch-norm kernels (address of its static scratch

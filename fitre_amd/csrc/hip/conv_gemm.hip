@@ -162,9 +162,11 @@ static BlockPlan c3_pos_plan(const fitre_conv_shape *s, bool dx, int cus = 0, in
 	double blockUs = (9.0 * kC3CB / 2.0) * (it / 32.0) * 64.0 / 2400.0; // MFMA steps x blocks per wave x 64 cycles
 	return plan_blocks(tiles, pairs * cred / kC3CB, blockUs, it == 64 ? 3 : 2, I, J, cus);
 }
+// cus == 0: the units fitre_hip_weight_grad_share leaves these kernels (all of the lane's, or three quarters where the
+// caller runs them beside a chain of other kernels)
 static BlockPlan c3_dw_plan(const fitre_conv_shape *s, int cus = 0, int pairs = 1)
 {
-	if (cus <= 0) cus = lane_compute_units();
+	if (cus <= 0) cus = weight_grad_units();
 	long J = (long)s->samples * s->inA * s->inB;
 	long tiles = ((s->inChannels + kC3DwCin - 1) / kC3DwCin) * ((s->outChannels + kC3Tile - 1) / kC3Tile);
 	double stageUs = (kC3Stage / 2.0) * 9.0 * 64.0 / 2400.0; // three waves per SIMD, three MFMAs per step each
@@ -180,7 +182,12 @@ static size_t c3_pos_workspace(const fitre_conv_shape *s, bool dx, int pairs = 1
 static size_t c3_dw_workspace(const fitre_conv_shape *s, int pairs = 1)
 {
 	size_t a = c3_dw_plan(s, device_compute_units(), pairs).wsBytes, b = c3_dw_plan(s, lane_compute_units_min(), pairs).wsBytes;
-	return a > b ? a : b;
+	a = a > b ? a : b;
+	for (int eighths = 4; eighths < 8; eighths++) {
+		const size_t c = c3_dw_plan(s, share_of_units(lane_compute_units_min(), eighths), pairs).wsBytes;
+		a = a > c ? a : c;
+	}
+	return a;
 }
 
 // leftSplits (may be null): when the product is split, skip the reduction launch, leave the partial

@@ -23,6 +23,7 @@ static bool g_lanes_on = true;
 // planners size their grids for the lane's share.  Off unless asked for: on the gradient path
 // it measured within noise of two unmasked lanes.
 static int g_lane_cus[kLanes] = { 256, 256, 256, 256 };
+static int g_dw_eighths = 8; // share of the compute units the 3 x 3 weight gradients are planned for
 constexpr int kJoinEvents = 64;
 static hipEvent_t g_join[kJoinEvents];
 static int g_join_next = 0;
@@ -79,6 +80,12 @@ int lane_compute_units_min()
 	return m;
 }
 int device_compute_units() { return g_lane_cus[0]; }
+int share_of_units(int cus, int eighths)
+{
+	const int share = (cus * eighths / 8) & ~7;
+	return share >= 8 ? share : cus;
+}
+int weight_grad_units() { return g_dw_eighths < 8 ? share_of_units(g_lane_cus[g_lane], g_dw_eighths) : g_lane_cus[g_lane]; }
 bool ready() { return g_ready; }
 int current_device() { return g_ready ? g_device : -1; }
 
@@ -264,6 +271,14 @@ int fitre_hip_lanes_enable(int on)
 	g_lanes_on = (on != 0);
 	g_lane = 0;
 	g_stream = g_lanes[0];
+	return FITRE_OK;
+}
+
+int fitre_hip_weight_grad_share(int eighths)
+{
+	FITRE_NEED_INIT();
+	FITRE_REQUIRE(eighths >= 4 && eighths <= 8, "fitre_hip_weight_grad_share: %d eighths (4 to 8)", eighths);
+	g_dw_eighths = eighths;
 	return FITRE_OK;
 }
 

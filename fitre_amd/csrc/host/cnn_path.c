@@ -273,6 +273,39 @@ static double backward_conv_work(const CNN_MODEL *model, int n)
 	return macs;
 }
 #define LANE_WORK_THRESHOLD 1.0e9
+/* The chain's bandwidth-bound steps (pooling, activation, batch norm: about 28 bytes per activation with batch norm, 16
+ * without) of layer c - 1 run beside the weight gradient of layer c on lane 1, and the next input gradient waits for
+ * them.  Where they are many per multiply-add of that weight gradient, it is planned for fewer compute units and the
+ * chain has the rest of the chip to itself (fitre_hip_weight_grad_share).  Measured on VGG-11 with batch norm at batch
+ * 256, bytes per thousand FLOP / best share: layer 1 49 / six eighths, layer 2 24 and layer 4 12 / seven or six
+ * eighths (equal within the noise), layers 3 and 5 6 and 3 / the whole chip; the pass 1.32 against 1.37 ms.  A pass with
+ * few such bytes overall (AlexNet at batch 64: about 400 FLOP per byte against 140) keeps the whole chip for every weight
+ * gradient: 2.82 against 3.00 ms with the shares.  The share depends on the network alone, not on whether the lanes are
+ * in use, so that one lane and two give the same bits. */
+static double elementwise_bytes(const CONV_LAYER *l, int n)
+{
+	return (double)n * l->outHeight * l->outWidth * l->outChannels * (has_bn(l) ? 28.0 : 16.0);
+}
+static double backward_flop_per_elementwise_byte(const CNN_MODEL *model, int n)
+{
+	double bytes = 0;
+	for (int c = 0; c < model->cLayers; c++) bytes += elementwise_bytes(&model->convLayer[c], n);
+	return bytes > 0 ? 2.0 * backward_conv_work(model, n) / bytes : 0.0;
+}
+#define SHARE_INTENSITY_LIMIT 250.0
+static int backward_shares_chip(const CNN_MODEL *model, int n)
+{
+	return backward_conv_work(model, n) >= LANE_WORK_THRESHOLD && backward_flop_per_elementwise_byte(model, n) < SHARE_INTENSITY_LIMIT;
+}
+/* eighths of the compute units the weight gradient of layer c is planned for */
+static int weight_grad_eighths(const CNN_MODEL *model, int n, int c)
+{
+	if (c < 1) return 8;
+	const CONV_LAYER *l = &model->convLayer[c];
+	const double flops = 2.0 * n * l->outHeight * l->outWidth * (double)l->outChannels * l->inChannels * l->kSize * l->kSize;
+	const double perKiloFlop = 1000.0 * elementwise_bytes(&model->convLayer[c - 1], n) / flops;
+	return perKiloFlop >= 40.0 ? 6 : (perKiloFlop >= 10.0 ? 7 : 8);
+}
 /* -1: by the limit above (fitted on LeNet, VGG-11 and AlexNet); 0: one lane; 1: lanes, whatever the network */
 static int g_backward_lanes = -1;
 void fitreSetBackwardLanes(int mode) { g_backward_lanes = mode < 0 ? -1 : (mode ? 1 : 0); }
@@ -315,6 +348,7 @@ void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, 
 		exit(-1);
 	}
 	const CONV_LAYER *last = &model->convLayer[nc - 1];
+	const int sharesChip = backward_shares_chip(model, n);
 
 	/* Weight copies of the layers whose input gradient reads one: they depend on the weights only, so lane 2 makes
 	 * them while the chain works through the linear layers. */
@@ -515,11 +549,13 @@ void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, 
 		}
 		/* without batch norm the bias gradient is taken here as well (with batch norm it is a by-product of its
 		 * backward pass above); nothing in the chain reads either */
+		HIP_CALL(fitre_hip_weight_grad_share(sharesChip ? weight_grad_eighths(model, n, c) : 8));
 		HIP_CALL(fitre_hip_conv_weight_bias_grad(&shape, input, cur, gradient + wOffsets[c],
 		                                         (!has_bn(l) && model->bias != 0) ? gradient + bOffsets[c] : NULL, sideWs,
 		                                         sideBytes));
 		if (beside) LANE_SELECT(0);
 	}
+	HIP_CALL(fitre_hip_weight_grad_share(8));
 	HIP_CALL(fitre_hip_sync());
 }
 

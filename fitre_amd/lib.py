@@ -130,6 +130,7 @@ HIP_API = {
     "fitre_hip_fc_tail_backward_pool_act": (i32, [i32, vp, i32, vp, i32, i32, vp, i32, vp, vp, vp, vp, vp, sz]),
     "fitre_hip_lane_select": (i32, [i32]),
     "fitre_hip_lane_wait": (i32, [i32, i32]),
+    "fitre_hip_weight_grad_share": (i32, [i32]),
     "fitre_hip_lanes_enable": (i32, [i32]),
     "fitre_hip_activation_rop_backward": (i32, [i32, vp, vp, vp, vp, vp, vp, lng]),
     "fitre_hip_pool_forward_routed": (i32, [i32, vp, vp] + [i32] * 9 + [vp]),

@@ -55,6 +55,13 @@ int fitre_hip_lane_select(int lane);
  * kernel tracer whose per-kernel durations should not overlap); on = 1 (the default) restores lanes. */
 int fitre_hip_lanes_enable(int on);
 int fitre_hip_lane_wait(int waiter, int signaller);
+/* The 3 x 3 weight gradients (fitre_hip_conv_weight_grad and its relatives on maps up to 32 cells wide) are cut into
+ * workgroups for `eighths` eighths of the compute units (4 to 8; 8, the default: all of them), so that the rest of the
+ * chip stays free for whatever the caller runs beside them on another lane.  The setting changes how a reduction is
+ * split, hence the last bits of a result: a caller that wants the same bits with and without lanes keeps it the same
+ * in both.  cnnBackward sets it per layer from the network (include/fitre_cnn.h) and restores 8.  No counterpart in
+ * the reference (one stream). */
+int fitre_hip_weight_grad_share(int eighths);
 
 /* ---------------- memory (device/cuda_utils.c; device/cuda_utils.h:15-26) ---------------- */
 int fitre_hip_malloc(void **ptr, size_t bytes);

@@ -421,3 +421,17 @@ def test_input_gradient_through_pool_refuses_bad_arguments(dev):
     assert hip.fitre_hip_conv_input_grad_pool_act(C.byref(shape), p, p, p, 12345, None, p, None, p, None, 0) == 2  # unknown activation
     assert hip.fitre_hip_conv_input_grad_folds_pool(None) == 0
     dev.free(p)
+
+
+@pytest.mark.parametrize("eighths", [8, 7, 6, 4])
+def test_weight_gradient_planned_for_a_share_of_the_chip(dev, oracle64, eighths):
+    """fitre_hip_weight_grad_share: the 3 x 3 weight gradients cut for fewer compute units (another split of the
+    reduction) stay within the tolerance of the float64 oracle; the setting is refused outside 4 to 8 eighths."""
+    try:
+        L.check(hip.fitre_hip_weight_grad_share(eighths))
+        for case in [(64, 128, 256, 8, 8, 3, 1, 1), (32, 64, 128, 16, 16, 3, 1, 1), (32, 256, 512, 4, 4, 3, 1, 1)]:
+            got, want = run_conv(dev, oracle64, case, "dw")
+            assert rel_err(got, want) < TOL, case
+    finally:
+        L.check(hip.fitre_hip_weight_grad_share(8))
+    assert hip.fitre_hip_weight_grad_share(3) == 2 and hip.fitre_hip_weight_grad_share(9) == 2
