@@ -692,6 +692,31 @@ int fitre_hip_conv_input_grad(const fitre_conv_shape *s, const float *delta, con
 	return launch_gemm<FlipWeightKContig, PatchRowContig>(pa, pb, out, I, J, R, plan, ws, wsBytes, FITRE_KC_CONV_DX, conv_flops(s));
 }
 
+// ---- the reductions of several small layers' weight gradients in one launch ----------------------------------------
+int fitre_hip_thin_reduce_defer(int on)
+{
+	FITRE_NEED_INIT();
+	if (!on) {
+		const int rc = thin_reduce_flush();
+		if (rc) return rc;
+	}
+	g_thin_reduce_deferred = (on != 0);
+	return FITRE_OK;
+}
+
+size_t fitre_hip_thin_reduce_bytes(const fitre_conv_shape *s)
+{
+	if (!s || s->samples <= 0 || s->inChannels <= 0 || s->outChannels <= 0 || s->inA <= 0 || s->inB <= 0 || s->ksize <= 0 || s->stride <= 0) return 0;
+	if (quad_eligible(s) || c3_dw_eligible(s) || thin_dw_eligible(s) || !thin_dw_general_eligible(s)) return 0;
+	return (thin_dw_general_workspace(s) + 255) & ~(size_t)255;
+}
+
+int fitre_hip_thin_reduce_flush(void)
+{
+	FITRE_NEED_INIT();
+	return thin_reduce_flush();
+}
+
 // ---- the input gradient taken on through the 2 x 2 max pool and the activation of the layer below ------------------
 static bool input_grad_takes_thin(const fitre_conv_shape *s)
 {

@@ -327,12 +327,17 @@ thin_weight_grad_kernel(const ThinConvParams p, const float *__restrict__ x, con
 
 // dW[c][k] (k < K) and db[c] (k = K) = sum over the workgroups' blocks, in workgroup order: sixteen phases each add
 // every sixteenth block in double precision and are combined in phase order.
-__global__ void __launch_bounds__(256) thin_dw_reduce_kernel(const float *partial, int groups, int cout, int K, float *dW, float *db)
+struct ThinReduceJob {
+	const float *partial;
+	int groups, cout, K;
+	float *dW, *db;
+};
+__device__ __forceinline__ void thin_dw_reduce_block(const float *partial, int groups, int cout, int K, float *dW, float *db, int block)
 {
 	__shared__ double part[16][17];
 	const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
 	const int total = cout * (K + 1);
-	const int idx = blockIdx.x * 16 + tx;
+	const int idx = block * 16 + tx;
 	double acc = 0.0;
 	if (idx < total)
 		for (int s = ty; s < groups; s += 16) acc += (double)partial[(size_t)s * total + idx];
@@ -346,6 +351,27 @@ __global__ void __launch_bounds__(256) thin_dw_reduce_kernel(const float *partia
 		if (kk < K) dW[(size_t)c * K + kk] = (float)sum;
 		else if (db) db[c] = (float)sum;
 	}
+}
+__global__ void __launch_bounds__(256) thin_dw_reduce_kernel(const float *partial, int groups, int cout, int K, float *dW, float *db)
+{
+	thin_dw_reduce_block(partial, groups, cout, K, dW, db, blockIdx.x);
+}
+// The reductions of several layers in one launch (each workgroup finds its layer by its index): the same sums in the
+// same order as one launch per layer.
+constexpr int kThinReduceJobs = 4;
+struct ThinReduceBatch {
+	ThinReduceJob job[kThinReduceJobs];
+	int first[kThinReduceJobs + 1]; // first workgroup of each job
+	int jobs;
+};
+__global__ void __launch_bounds__(256) thin_dw_reduce_batch_kernel(const ThinReduceBatch b)
+{
+	const int block = blockIdx.x;
+	// constant indices only: a run-time index into the argument block would copy it to scratch memory
+	if (b.jobs > 3 && block >= b.first[3]) thin_dw_reduce_block(b.job[3].partial, b.job[3].groups, b.job[3].cout, b.job[3].K, b.job[3].dW, b.job[3].db, block - b.first[3]);
+	else if (b.jobs > 2 && block >= b.first[2]) thin_dw_reduce_block(b.job[2].partial, b.job[2].groups, b.job[2].cout, b.job[2].K, b.job[2].dW, b.job[2].db, block - b.first[2]);
+	else if (b.jobs > 1 && block >= b.first[1]) thin_dw_reduce_block(b.job[1].partial, b.job[1].groups, b.job[1].cout, b.job[1].K, b.job[1].dW, b.job[1].db, block - b.first[1]);
+	else thin_dw_reduce_block(b.job[0].partial, b.job[0].groups, b.job[0].cout, b.job[0].K, b.job[0].dW, b.job[0].db, block);
 }
 
 // Words per row of the weight gradient's bordered input in LDS.  The lanes of a wave are consecutive patch indices
@@ -471,6 +497,28 @@ static inline size_t thin_dw_general_workspace(const fitre_conv_shape *s)
 {
 	return sizeof(float) * 2 * (size_t)device_compute_units() * s->outChannels * (s->inChannels * s->ksize * s->ksize + 1);
 }
+// Reductions held back so that several layers' share one launch (fitre_hip_thin_reduce_defer / _flush)
+static bool g_thin_reduce_deferred = false;
+static ThinReduceBatch g_thin_reduce = {};
+static double g_thin_reduce_bytes = 0.0;
+static int thin_reduce_flush()
+{
+	if (g_thin_reduce.jobs == 0) return FITRE_OK;
+	{
+		LaunchScope scope(FITRE_KC_SPLITK_REDUCE, g_thin_reduce_bytes);
+		if (g_thin_reduce.jobs == 1) {
+			const ThinReduceJob &j = g_thin_reduce.job[0];
+			thin_dw_reduce_kernel<<<(unsigned)g_thin_reduce.first[1], 256, 0, stream()>>>(j.partial, j.groups, j.cout, j.K, j.dW, j.db);
+		} else {
+			thin_dw_reduce_batch_kernel<<<(unsigned)g_thin_reduce.first[g_thin_reduce.jobs], 256, 0, stream()>>>(g_thin_reduce);
+		}
+	}
+	g_thin_reduce.jobs = 0;
+	g_thin_reduce.first[0] = 0;
+	g_thin_reduce_bytes = 0.0;
+	return check_launch("thin_dw_reduce_batch_kernel");
+}
+
 // db may be null
 static int launch_thin_dw_general(const fitre_conv_shape *s, const float *x, const float *delta, float *dW, float *db, void *ws)
 {
@@ -490,10 +538,23 @@ static int launch_thin_dw_general(const fitre_conv_shape *s, const float *x, con
 		if (thin_dw_pad(s->outChannels) == 8) thin_weight_grad_kernel<8><<<pl.groups, 512, lds, stream()>>>(p, x, delta, (float *)ws);
 		else thin_weight_grad_kernel<16><<<pl.groups, 512, lds, stream()>>>(p, x, delta, (float *)ws);
 	}
+	const ThinReduceJob job{ (const float *)ws, pl.groups, s->outChannels, K, dW, db };
+	if (g_thin_reduce_deferred) {
+		// the caller keeps this workspace untouched until fitre_hip_thin_reduce_flush()
+		if (g_thin_reduce.jobs == kThinReduceJobs) {
+			const int rc = thin_reduce_flush();
+			if (rc) return rc;
+		}
+		const int j = g_thin_reduce.jobs++;
+		g_thin_reduce.job[j] = job;
+		g_thin_reduce.first[j + 1] = g_thin_reduce.first[j] + (s->outChannels * (K + 1) + 15) / 16;
+		g_thin_reduce_bytes += 4.0 * (double)s->outChannels * (K + 1) * (pl.groups + 1);
+		return check_launch("thin_weight_grad_kernel");
+	}
 	{
 		const int total = s->outChannels * (K + 1);
 		LaunchScope scope(FITRE_KC_SPLITK_REDUCE, 4.0 * (double)total * (pl.groups + 1));
-		thin_dw_reduce_kernel<<<(total + 15) / 16, 256, 0, stream()>>>((const float *)ws, pl.groups, s->outChannels, K, dW, db);
+		thin_dw_reduce_kernel<<<(total + 15) / 16, 256, 0, stream()>>>(job.partial, job.groups, job.cout, job.K, job.dW, job.db);
 	}
 	return check_launch("thin_weight_grad_kernel");
 }

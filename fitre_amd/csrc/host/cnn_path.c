@@ -133,9 +133,11 @@ static size_t backward_side_ws_bytes(const CNN_MODEL *model, int batch)
 	size_t need = 256;
 	fitre_fc_tail_layer tail[4];
 	if (tail_shapes(model, batch, tail)) need = max_sz(need, fitre_hip_fc_tail_workspace(model->lLayers, tail, batch));
+	size_t held = 0; /* layers whose reduction is held back until the end of the pass keep their blocks: a slice each */
 	for (int i = 0; i < model->cLayers; i++) {
 		fitre_conv_shape s = conv_shape(&model->convLayer[i], batch);
 		need = max_sz(need, fitre_hip_conv_weight_grad_workspace(&s));
+		held += fitre_hip_thin_reduce_bytes(&s);
 		if (!has_bn(&model->convLayer[i]))
 			need = max_sz(need, fitre_hip_channel_sum_workspace(model->convLayer[i].outChannels,
 			                                                    (long)batch * model->convLayer[i].outWidth * model->convLayer[i].outHeight));
@@ -144,7 +146,7 @@ static size_t backward_side_ws_bytes(const CNN_MODEL *model, int batch)
 		const FC_LAYER *f = &model->fcLayer[i];
 		need = max_sz(need, fitre_hip_linear_weight_grad_workspace(f->in, f->out, batch));
 	}
-	return (need + 255) & ~(size_t)255;
+	return ((need + 255) & ~(size_t)255) + held;
 }
 
 /* Rearranged weight copies that some input gradients multiply by (fitre_hip_conv_input_grad_prepare): made at the
@@ -456,6 +458,11 @@ void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, 
 	/* delta as the layer above left it: a plain tensor, or the unsummed split partials of its input
 	 * gradient (summed by the pool / activation pass below while it reads them) */
 	fitre_split_view dview = { features, 1, 0 };
+	/* The weight gradients of layers with very few channels end in a short reduction launch each: they are held back and
+	 * made as one launch at the end of the pass.  Until then such a layer's blocks stay in a slice of lane 1's workspace of
+	 * their own, and the layers after it work in what follows the slices. */
+	size_t sideHeld = 0;
+	HIP_CALL(fitre_hip_thin_reduce_defer(1));
 	int poolFolded = tailFoldedPool;
 	for (int c = nc - 1; c >= 0; c--) {
 		const CONV_LAYER *l = &model->convLayer[c];
@@ -551,8 +558,10 @@ void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, 
 		 * backward pass above); nothing in the chain reads either */
 		HIP_CALL(fitre_hip_weight_grad_share(sharesChip ? weight_grad_eighths(model, n, c) : 8));
 		HIP_CALL(fitre_hip_conv_weight_bias_grad(&shape, input, cur, gradient + wOffsets[c],
-		                                         (!has_bn(l) && model->bias != 0) ? gradient + bOffsets[c] : NULL, sideWs,
-		                                         sideBytes));
+		                                         (!has_bn(l) && model->bias != 0) ? gradient + bOffsets[c] : NULL,
+		                                         (char *)sideWs + sideHeld, sideBytes - sideHeld));
+		sideHeld += fitre_hip_thin_reduce_bytes(&shape);
+		if (c == 0) HIP_CALL(fitre_hip_thin_reduce_defer(0)); /* every held reduction, on the lane their blocks were made on */
 		if (beside) LANE_SELECT(0);
 	}
 	HIP_CALL(fitre_hip_weight_grad_share(8));

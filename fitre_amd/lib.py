@@ -114,6 +114,9 @@ HIP_API = {
     "fitre_hip_conv_weight_grad": (i32, [pshape, vp, vp, vp, vp, sz]),
     "fitre_hip_conv_weight_bias_grad_workspace": (sz, [pshape]),
     "fitre_hip_conv_weight_bias_grad": (i32, [pshape, vp, vp, vp, vp, vp, sz]),
+    "fitre_hip_thin_reduce_bytes": (sz, [pshape]),
+    "fitre_hip_thin_reduce_defer": (i32, [i32]),
+    "fitre_hip_thin_reduce_flush": (i32, []),
     "fitre_hip_conv_input_grad_workspace": (sz, [pshape]),
     "fitre_hip_conv_input_grad": (i32, [pshape, vp, vp, vp, vp, sz]),
     "fitre_hip_conv_input_grad_folds_pool": (i32, [pshape]),

@@ -346,6 +346,17 @@ int fitre_hip_conv_weight_grad(const fitre_conv_shape *s, const float *x, const 
  * 662-689), for layers without batch norm: one pass over delta where the layer has few channels, else
  * fitre_hip_channel_sum followed by fitre_hip_conv_weight_grad.  db may be NULL (then this is
  * fitre_hip_conv_weight_grad). */
+/* Layers with very few channels (LeNet's) leave their weight gradient as per-workgroup blocks that a second, short launch
+ * adds up.  fitre_hip_thin_reduce_defer(1): from now on that second launch is held back (up to four layers; a fifth
+ * flushes first) and fitre_hip_thin_reduce_flush() -- or fitre_hip_thin_reduce_defer(0) -- makes them all in ONE launch
+ * on the lane selected then: the same sums in the same order.  While a layer's reduction is held back its workspace must
+ * stay untouched and its dW / db are not yet written: give every such call a workspace of its own.  Layers of other
+ * shapes are not affected.  No counterpart in the reference. */
+/* fitre_hip_thin_reduce_bytes: 0 for a shape whose weight gradient has no such second launch, else the bytes at the
+ * head of its workspace that must stay untouched while it is held back. */
+size_t fitre_hip_thin_reduce_bytes(const fitre_conv_shape *s);
+int fitre_hip_thin_reduce_defer(int on);
+int fitre_hip_thin_reduce_flush(void);
 size_t fitre_hip_conv_weight_bias_grad_workspace(const fitre_conv_shape *s);
 int fitre_hip_conv_weight_bias_grad(const fitre_conv_shape *s, const float *x, const float *delta, float *dW,
                                     float *db, void *ws, size_t wsBytes);

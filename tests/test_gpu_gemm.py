@@ -435,3 +435,49 @@ def test_weight_gradient_planned_for_a_share_of_the_chip(dev, oracle64, eighths)
     finally:
         L.check(hip.fitre_hip_weight_grad_share(8))
     assert hip.fitre_hip_weight_grad_share(3) == 2 and hip.fitre_hip_weight_grad_share(9) == 2
+
+
+def test_held_back_reductions_of_small_layers_are_one_launch_with_the_same_bits(dev):
+    """fitre_hip_thin_reduce_defer / _flush: the weight and bias gradients of two LeNet-sized layers with their reductions
+    held back and made together equal, bit for bit, what the two calls write on their own; nothing is written before the
+    flush; shapes of other kernels report no bytes to keep."""
+    cases = [(8, 3, 6, 32, 32, 5, 1, 0), (8, 6, 16, 14, 14, 5, 1, 0)]
+    rng = np.random.default_rng(99)
+    data = []
+    for N, Cin, Cout, A, B, k, s, p in cases:
+        shape = conv_shape(N, Cin, Cout, A, B, k, s, p)
+        keep = hip.fitre_hip_thin_reduce_bytes(C.byref(shape))
+        assert keep > 0
+        x = rng.standard_normal(Cin * N * A * B).astype(np.float32)
+        d = rng.standard_normal(Cout * N * shape.outA * shape.outB).astype(np.float32)
+        nb = hip.fitre_hip_conv_weight_bias_grad_workspace(C.byref(shape))
+        assert nb >= 0 and keep <= max(nb, keep)
+        data.append((shape, dev.upload(x), dev.upload(d), Cout * Cin * k * k, Cout, max(nb, keep)))
+    assert hip.fitre_hip_thin_reduce_bytes(C.byref(conv_shape(4, 64, 128, 8, 8, 3, 1, 1))) == 0
+    want = []
+    for shape, px, pd, nw, nbias, nb in data:
+        ws, dw, db = dev.alloc(nb), dev.zeros(nw), dev.zeros(nbias)
+        L.check(hip.fitre_hip_conv_weight_bias_grad(C.byref(shape), px, pd, dw, db, ws, nb))
+        want.append((dev.download(dw, nw).view(np.uint32), dev.download(db, nbias).view(np.uint32)))
+        for q in (ws, dw, db):
+            dev.free(q)
+    held = []
+    L.check(hip.fitre_hip_thin_reduce_defer(1))
+    try:
+        for shape, px, pd, nw, nbias, nb in data:
+            ws, dw, db = dev.alloc(nb), dev.upload(np.full(nw, 7.0, np.float32)), dev.upload(np.full(nbias, 7.0, np.float32))
+            L.check(hip.fitre_hip_conv_weight_bias_grad(C.byref(shape), px, pd, dw, db, ws, nb))
+            held.append((ws, dw, db, nw, nbias))
+        dev.sync()
+        for ws, dw, db, nw, nbias in held:
+            assert (dev.download(dw, nw) == 7.0).all() and (dev.download(db, nbias) == 7.0).all()
+        L.check(hip.fitre_hip_thin_reduce_flush())
+    finally:
+        L.check(hip.fitre_hip_thin_reduce_defer(0))
+    for (ws, dw, db, nw, nbias), (wdw, wdb) in zip(held, want):
+        np.testing.assert_array_equal(dev.download(dw, nw).view(np.uint32), wdw)
+        np.testing.assert_array_equal(dev.download(db, nbias).view(np.uint32), wdb)
+        for q in (ws, dw, db):
+            dev.free(q)
+    for shape, px, pd, nw, nbias, nb in data:
+        dev.free(px), dev.free(pd)
