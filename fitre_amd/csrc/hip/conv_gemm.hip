@@ -599,8 +599,10 @@ size_t fitre_hip_conv_weight_grad_workspace(const fitre_conv_shape *s)
 
 int fitre_hip_conv_weight_grad_runs_beside(const fitre_conv_shape *s)
 {
-	if (!s) return 0;
-	return (quad_eligible(s) || c3_dw_eligible(s) || thin_dw_eligible(s) || thin_dw_general_eligible(s)) ? 1 : 0;
+	// Every weight gradient does by now.  Those on the general tile engine (5 x 5 and 11 x 11 windows) used to stay in line,
+	// because beside the chain's matrix kernels both lost more than the overlap gained; with the chain's bandwidth kernels
+	// finding room and priority beside a matrix kernel the balance has turned: AlexNet at batch 64 2.83 -> 2.69 ms.
+	return s ? 1 : 0;
 }
 
 int fitre_hip_conv_weight_grad(const fitre_conv_shape *s, const float *x, const float *delta, float *dW, void *ws, size_t wsBytes)

@@ -546,8 +546,8 @@ void cnnBackward(CNN_MODEL *model, DEVICE_DATASET *data, real *devPtr, real *z, 
 				dview.base = delta, dview.splits = 1, dview.stride = 0;
 			}
 		}
-		/* A weight gradient on the general tile engine stays in line: beside the next layer's matrix kernels both would
-		 * lose more than the overlap gains.  Its workspace is lane 1's, so the lanes are ordered around it. */
+		/* A weight gradient the device layer does not want beside other matrix kernels (none by now) stays in line; its
+		 * workspace is lane 1's, so the lanes are ordered around it. */
 		if (!beside) LANE_WAIT(1, 0);
 		if (beside) {
 			LANE_SELECT(1);

@@ -333,12 +333,10 @@ int fitre_hip_conv_forward(const fitre_conv_shape *s, const float *x, const floa
 /* dW[Cout][Cin*k*k] = sum over (n,a,b) of patch(x) * delta.  Replaces im2col + GEMM of
  * functions/cnn_backward.cu:771-783. */
 size_t fitre_hip_conv_weight_grad_workspace(const fitre_conv_shape *s);
-/* 1 when this shape's weight gradient runs on a kernel built to share the compute units with other work (the 3x3
- * kernel: one workgroup per compute unit with register room left; the dense and direct forms), 0 when it runs on the
- * general tile engine, whose workgroups want the compute units to themselves: beside another matrix kernel both
- * lose more than the overlap gains (AlexNet batch 64: 3.27 ms per pass with every weight gradient on a second lane,
- * 3.08 ms with the general-engine ones in line).  cnnBackward puts a weight gradient on its second lane only when
- * this says 1. */
+/* Whether cnnBackward should put this shape's weight gradient on its second lane, beside the chain of input gradients:
+ * 1 for every shape by now.  (Weight gradients on the general tile engine used to stay in line -- AlexNet batch 64 then
+ * took 3.27 ms with them on the second lane against 3.08 in line; since the chain's bandwidth kernels find room and
+ * priority beside a matrix kernel it is 2.69 against 2.83 ms the other way round.) */
 int fitre_hip_conv_weight_grad_runs_beside(const fitre_conv_shape *s);
 int fitre_hip_conv_weight_grad(const fitre_conv_shape *s, const float *x, const float *delta, float *dW,
                                void *ws, size_t wsBytes);
