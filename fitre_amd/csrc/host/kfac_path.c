@@ -286,10 +286,15 @@ static void inverse_pass_run(const CNN_MODEL *model, int samples, real *devPtr, 
 	INVERSE_JOB jobs[KFAC_MAX_ITEMS];
 	for (int i = 0; i < count; i++) {
 		jobs[i].item = i;
-		/* a chain of launches whose length grows with the order, plus the arithmetic */
+		/* Milliseconds alone on the chip, fitted to measurements: the inverse is a chain of launches whose length grows
+		 * with the order (0.42 / 1.12 / 2.46 / 6.86 ms at order 512 / 1153 / 2305 / 4609) plus the arithmetic; the factor is
+		 * a symmetric product over the positions (1.9 ms for order 4609 over 4096 positions).  With the chain's share
+		 * underrated (as an earlier form had it) every small matrix of a pass landed on one lane, which then finished last. */
 		const int lowrank = items[i].rows != NULL && lowrank_eligible(items[i].order, items[i].positions);
 		const double n = lowrank ? (double)items[i].positions : (double)items[i].order;
-		jobs[i].cost = n * (200.0 + n * n * 1e-3) + (lowrank ? 2e-3 * n * n * items[i].order : 0.0);
+		const double order = (double)items[i].order, positions = (double)(items[i].positions > 0 ? items[i].positions : 0);
+		jobs[i].cost = 0.82e-3 * n + 3.15e-11 * n * n * n +
+		               (lowrank ? 1.0e-10 * n * n * order : 2.2e-11 * order * order * positions);
 	}
 	qsort(jobs, (size_t)count, sizeof(INVERSE_JOB), job_by_cost);
 	double load[KFAC_LANES] = { 0, 0, 0, 0 };
