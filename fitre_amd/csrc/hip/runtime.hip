@@ -195,25 +195,8 @@ int fitre_hip_init(int device)
 	int cus = 0;
 	FITRE_HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device));
 	if (cus <= 0 || cus > 1024) return fail(FITRE_E_DEVICE, "fitre_hip_init: device reports %d compute units", cus);
-	FITRE_HIP_TRY(hipStreamCreate(&g_lanes[0])); // default priority
-	g_lane_cus[0] = cus;
-	// Lane 1 masked: the first `share` bits of the mask; the driver deals mask bits round-robin to
-	// the XCDs, so every XCD keeps the same number of compute units.
-	int share = cus;
-	if (const char *env = getenv("FITRE_LANE1_CUS")) share = atoi(env);
-	share -= share % 8;
-	if (share >= 8 && share < cus) {
-		uint32_t mask[32];
-		memset(mask, 0, sizeof(mask));
-		for (int b = 0; b < share; b++) mask[b / 32] |= 1u << (b % 32);
-		FITRE_HIP_TRY(hipExtStreamCreateWithCUMask(&g_lanes[1], (uint32_t)((cus + 31) / 32), mask));
-		g_lane_cus[1] = share;
-	} else {
-		FITRE_HIP_TRY(hipStreamCreate(&g_lanes[1]));
-		g_lane_cus[1] = cus;
-	}
-	for (int i = 2; i < kLanes; i++) {
-		FITRE_HIP_TRY(hipStreamCreate(&g_lanes[i]));
+	for (int i = 0; i < kLanes; i++) {
+		FITRE_HIP_TRY(hipStreamCreate(&g_lanes[i])); // default priority
 		g_lane_cus[i] = cus;
 	}
 	for (int i = 0; i < kJoinEvents; i++) FITRE_HIP_TRY(hipEventCreateWithFlags(&g_join[i], hipEventDisableTiming));
