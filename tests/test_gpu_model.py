@@ -379,3 +379,45 @@ def test_alexnet_full_size_against_the_oracle(dev, oracle64):
     """AlexNet at 3 x 224 x 224, batch 64, 1000 classes against the float64 oracle: 11x11 / stride 4 and 5x5
     convolutions, 3/2 max pooling, FC 9216-4096-4096-1000."""
     compare_with_oracle(dev, oracle64, build_alexnet(64), 64, seed=22)
+
+
+def test_backward_pass_leaves_the_device_layer_settings_as_it_found_them(vgg_full, dev):
+    """cnnBackward plans some weight gradients for a share of the chip and holds small layers' reductions back while it runs;
+    after it returns the device layer is back at its defaults: a weight gradient called directly gives the bits it gives
+    with the share set to the whole chip explicitly, and a small layer's call writes its result at once."""
+    from helpers import conv_shape
+    gm, w = vgg_full
+    gm.forward()
+    gm.backward()
+    hip = L.hip
+    rng = np.random.default_rng(5)
+    # a 3 x 3 layer the share would apply to
+    shape = conv_shape(32, 64, 128, 16, 16, 3, 1, 1)
+    x = dev.upload(rng.standard_normal(64 * 32 * 256).astype(np.float32))
+    d = dev.upload(rng.standard_normal(128 * 32 * 256).astype(np.float32))
+    nb = hip.fitre_hip_conv_weight_grad_workspace(C.byref(shape))
+    ws, dw = dev.alloc(nb), dev.zeros(128 * 64 * 9)
+    L.check(hip.fitre_hip_conv_weight_grad(C.byref(shape), x, d, dw, ws, nb))
+    after = dev.download(dw, 128 * 64 * 9).view(np.uint32)
+    L.check(hip.fitre_hip_weight_grad_share(8))
+    L.check(hip.fitre_hip_conv_weight_grad(C.byref(shape), x, d, dw, ws, nb))
+    np.testing.assert_array_equal(dev.download(dw, 128 * 64 * 9).view(np.uint32), after)
+    for q in (x, d, ws, dw):
+        dev.free(q)
+    # a LeNet-sized layer: the reduction is not held back
+    lenet = build_lenet(16, bn=False)
+    wl = he_weights(lenet, rng).astype(np.float32)
+    xl, yl = batch_inputs(lenet, 16, rng)
+    g2 = GpuModel(dev, lenet, wl, xl.astype(np.float32), yl, 16)
+    g2.forward()
+    g2.backward()
+    g2.release()
+    shape = conv_shape(8, 3, 6, 32, 32, 5, 1, 0)
+    x = dev.upload(rng.standard_normal(3 * 8 * 1024).astype(np.float32))
+    d = dev.upload(rng.standard_normal(6 * 8 * 28 * 28).astype(np.float32))
+    nb = max(hip.fitre_hip_conv_weight_bias_grad_workspace(C.byref(shape)), 256)
+    ws, dw, db = dev.alloc(nb), dev.upload(np.full(6 * 75, np.nan, np.float32)), dev.upload(np.full(6, np.nan, np.float32))
+    L.check(hip.fitre_hip_conv_weight_bias_grad(C.byref(shape), x, d, dw, db, ws, nb))
+    assert np.isfinite(dev.download(dw, 6 * 75)).all() and np.isfinite(dev.download(db, 6)).all()
+    for q in (x, d, ws, dw, db):
+        dev.free(q)
