@@ -99,6 +99,14 @@ def test_lenet_bn_batch1024(dev, oracle64):
     compare_with_oracle(dev, oracle64, build_lenet(1024, bn=True), 1024, seed=12)
 
 
+def test_lenet_batch1024_on_two_lanes(dev, oracle64):
+    """Without batch norm and above the lane limit: the pooling steps folded into the launches above them, the weight
+    gradients on the second lane and their reductions held back to one launch, against the oracle."""
+    model = build_lenet(1024, bn=False)
+    assert L.cnn.fitreBackwardUsesLanes(C.byref(model), 1024) == 1
+    compare_with_oracle(dev, oracle64, model, 1024, seed=13)
+
+
 def test_vgg11_bn_reduced_batch(dev, oracle64):
     # the benchmark network at its real layer shapes; batch trimmed so that the oracle takes seconds
     compare_with_oracle(dev, oracle64, build_vgg11(16, bn=True), 16, seed=13)
@@ -244,7 +252,7 @@ def test_vgg11_full_size_one_lane_gives_the_same_bits(vgg_full, dev):
         L.check(L.hip.fitre_hip_lanes_enable(1))
 
 
-@pytest.mark.parametrize("name", ["lenet_bn_b1024", "alexnet_b64", "vgg11_no_bn_b32"])
+@pytest.mark.parametrize("name", ["lenet_bn_b1024", "lenet_b1024", "alexnet_b64", "vgg11_no_bn_b32"])
 def test_forced_lanes_give_the_same_bits(dev, name):
     """Networks on either side of cnnBackward's lane limit and without the batch-norm steps the lanes were built around
     (LeNet + batch norm at batch 1024: just above it; AlexNet; a VGG-11 without batch norm at a small batch) and the
@@ -252,6 +260,8 @@ def test_forced_lanes_give_the_same_bits(dev, name):
     from helpers import GpuModel, batch_inputs, build_alexnet, build_lenet, build_vgg11, he_weights
     if name == "lenet_bn_b1024":
         batch, model = 1024, build_lenet(1024, bn=True)
+    elif name == "lenet_b1024":  # without batch norm: folded pooling steps and held-back reductions, on two lanes
+        batch, model = 1024, build_lenet(1024, bn=False)
     elif name == "alexnet_b64":
         batch, model = 64, build_alexnet(64)
     else:
